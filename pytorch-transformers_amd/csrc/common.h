@@ -1,0 +1,94 @@
+// Shared device helpers for the gfx950 kernels: bfloat16 bits, typed loads and
+// stores, wave and block reductions, and the error channel of the C entry points.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define PTA_WAVE 64
+#define PTA_PAGE 64  // tokens per cache page; must equal cache.paged.PAGE_SIZE
+
+enum PtaDtype { PTA_F32 = 0, PTA_BF16 = 1 };
+
+// fused query_key_value row orders (see config.falcon)
+enum PtaQkvLayout { PTA_QKV_GROUPED = 0, PTA_QKV_TAIL = 1, PTA_QKV_INTERLEAVED = 2 };
+
+enum PtaAct { PTA_ACT_NONE = 0, PTA_ACT_GELU = 1 };
+
+typedef uint16_t bf16_t;  // raw bits of a bfloat16
+
+__host__ __device__ __forceinline__ float bf16_bits_to_f32(bf16_t v) {
+    union { uint32_t u; float f; } c;
+    c.u = ((uint32_t)v) << 16;
+    return c.f;
+}
+
+// round to nearest, ties to even; NaN stays NaN
+__host__ __device__ __forceinline__ bf16_t f32_to_bf16_bits(float f) {
+    union { uint32_t u; float f; } c;
+    c.f = f;
+    uint32_t u = c.u;
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x0040u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (bf16_t)(u >> 16);
+}
+
+__host__ __device__ __forceinline__ float round_to_bf16(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
+
+template <typename T> struct Io;
+template <> struct Io<float> {
+    static __device__ __forceinline__ float ld(const float* p) { return *p; }
+    static __device__ __forceinline__ void st(float* p, float v) { *p = v; }
+    static __device__ __forceinline__ float round(float v) { return v; }
+};
+template <> struct Io<bf16_t> {
+    static __device__ __forceinline__ float ld(const bf16_t* p) { return bf16_bits_to_f32(*p); }
+    static __device__ __forceinline__ void st(bf16_t* p, float v) { *p = f32_to_bf16_bits(v); }
+    static __device__ __forceinline__ float round(float v) { return round_to_bf16(v); }
+};
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+
+// Sum over a block of up to 1024 threads; every thread gets the result.  `red`
+// is LDS of at least 16 floats.  The order of additions depends on the block
+// size only.
+__device__ __forceinline__ float block_sum(float v, float* red) {
+    v = wave_sum(v);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    __syncthreads();
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    float t = 0.f;
+    for (int i = 0; i < nw; ++i) t += red[i];
+    return t;
+}
+__device__ __forceinline__ float block_max(float v, float* red) {
+    v = wave_max(v);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    __syncthreads();
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    float t = red[0];
+    for (int i = 1; i < nw; ++i) t = fmaxf(t, red[i]);
+    return t;
+}
+
+// exact GELU, 0.5 x (1 + erf(x / sqrt 2))  (src/transformers/activations.py:59-78)
+__device__ __forceinline__ float gelu_erf(float x) { return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f)); }
+
+// ---- host side ---------------------------------------------------------
+// Entry points return 0 on success; otherwise pta_last_error() holds the reason.
+int pta_fail(const char* fmt, ...);
+int pta_check_launch(const char* what);
+
+#define PTA_REQUIRE(cond, ...) \
+    do { if (!(cond)) return pta_fail(__VA_ARGS__); } while (0)

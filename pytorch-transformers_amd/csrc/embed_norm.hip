@@ -1,0 +1,117 @@
+// Embedding lookup and LayerNorm for gfx950.
+//
+// LayerNorm: one workgroup per row, statistics in 32-bit, two passes over the
+// row for the variance (mean first, then squared distances), so the result
+// does not depend on which other rows are in the launch.  One pass over x can
+// feed two affine outputs (the ln_attn / ln_mlp pair of the parallel block),
+// and rows can be gathered by index (the final norm runs on wanted rows only).
+#include "common.h"
+#include "pta_kernels.h"
+
+template <typename T>
+__global__ void embed_kernel(T* __restrict__ out, const T* __restrict__ table, const int* __restrict__ ids,
+                             int H) {
+    const int m = blockIdx.x;
+    const long row = ids[m];
+    const T* src = table + row * (long)H;
+    T* dst = out + (long)m * H;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) dst[i] = src[i];
+}
+
+extern "C" int pta_embed(void* out, const void* table, const int* ids, int M, int H, int dtype, void* stream) {
+    PTA_REQUIRE(M > 0 && H > 0, "embed: M=%d H=%d must be positive", M, H);
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == PTA_F32)
+        hipLaunchKernelGGL(embed_kernel<float>, dim3(M), dim3(256), 0, s, (float*)out, (const float*)table, ids, H);
+    else if (dtype == PTA_BF16)
+        hipLaunchKernelGGL(embed_kernel<bf16_t>, dim3(M), dim3(256), 0, s, (bf16_t*)out, (const bf16_t*)table, ids, H);
+    else
+        return pta_fail("embed: unknown dtype %d", dtype);
+    return pta_check_launch("embed");
+}
+
+// y = (x - mean) / sqrt(var + eps) * w + b, biased variance (torch.nn.LayerNorm as built at
+// src/transformers/models/falcon/modeling_falcon.py:603-612, :843).  w and b are 32-bit.
+template <typename T>
+__global__ void layernorm_kernel(T* __restrict__ out1, T* __restrict__ out2, const T* __restrict__ x,
+                                 const int* __restrict__ rows, const float* __restrict__ w1,
+                                 const float* __restrict__ b1, const float* __restrict__ w2,
+                                 const float* __restrict__ b2, int H, float eps) {
+    __shared__ float red[16];
+    const int m = blockIdx.x;
+    const long src_row = rows ? (long)rows[m] : (long)m;
+    const T* xr = x + src_row * H;
+    float s = 0.f;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) s += Io<T>::ld(xr + i);
+    const float mean = block_sum(s, red) / (float)H;
+    float q = 0.f;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        const float d = Io<T>::ld(xr + i) - mean;
+        q += d * d;
+    }
+    const float var = block_sum(q, red) / (float)H;
+    const float rstd = 1.0f / sqrtf(var + eps);
+    T* o1 = out1 + (long)m * H;
+    T* o2 = out2 ? out2 + (long)m * H : nullptr;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        const float n = (Io<T>::ld(xr + i) - mean) * rstd;
+        Io<T>::st(o1 + i, n * w1[i] + b1[i]);
+        if (o2) Io<T>::st(o2 + i, n * w2[i] + b2[i]);
+    }
+}
+
+extern "C" int pta_layernorm(void* out1, void* out2, const void* x, const int* rows, const float* w1,
+                             const float* b1, const float* w2, const float* b2, int M, int H, float eps,
+                             int dtype, void* stream) {
+    PTA_REQUIRE(M > 0 && H > 0, "layernorm: M=%d H=%d must be positive", M, H);
+    PTA_REQUIRE(out1 && x && w1 && b1, "layernorm: null pointer");
+    PTA_REQUIRE(!out2 || (w2 && b2), "layernorm: a second output needs its own weight and bias");
+    hipStream_t s = (hipStream_t)stream;
+    const int threads = H >= 2048 ? 512 : 256;
+    if (dtype == PTA_F32)
+        hipLaunchKernelGGL(layernorm_kernel<float>, dim3(M), dim3(threads), 0, s, (float*)out1, (float*)out2,
+                           (const float*)x, rows, w1, b1, w2, b2, H, eps);
+    else if (dtype == PTA_BF16)
+        hipLaunchKernelGGL(layernorm_kernel<bf16_t>, dim3(M), dim3(threads), 0, s, (bf16_t*)out1, (bf16_t*)out2,
+                           (const bf16_t*)x, rows, w1, b1, w2, b2, H, eps);
+    else
+        return pta_fail("layernorm: unknown dtype %d", dtype);
+    return pta_check_launch("layernorm");
+}
+
+// In place on y [M, N]: y = act(round(y + bias)) + add1 + add2, the part of a linear layer
+// that follows a library matrix product.  The reference adds the bias as an op of its own, so
+// the sum is rounded to the storage type before the activation
+// (src/transformers/models/falcon/modeling_falcon.py:67-72).
+template <typename T>
+__global__ void epilogue_kernel(T* __restrict__ y, const float* __restrict__ bias, const T* __restrict__ add1,
+                                const T* __restrict__ add2, long total, int N, int act) {
+    const long stride = (long)gridDim.x * blockDim.x;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        float v = Io<T>::ld(y + i);
+        if (bias) v = Io<T>::round(v + bias[i % N]);
+        if (act == PTA_ACT_GELU) v = gelu_erf(v);
+        if (add1) v += Io<T>::ld(add1 + i);
+        if (add2) v += Io<T>::ld(add2 + i);
+        Io<T>::st(y + i, v);
+    }
+}
+
+extern "C" int pta_epilogue(void* y, const float* bias, const void* add1, const void* add2, int M, int N, int act,
+                            int dtype, void* stream) {
+    PTA_REQUIRE(M > 0 && N > 0, "epilogue: M=%d N=%d must be positive", M, N);
+    PTA_REQUIRE(act == PTA_ACT_NONE || act == PTA_ACT_GELU, "epilogue: unknown activation %d", act);
+    const long total = (long)M * N;
+    long blocks = (total + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == PTA_F32)
+        hipLaunchKernelGGL(epilogue_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, s, (float*)y, bias,
+                           (const float*)add1, (const float*)add2, total, N, act);
+    else if (dtype == PTA_BF16)
+        hipLaunchKernelGGL(epilogue_kernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, s, (bf16_t*)y, bias,
+                           (const bf16_t*)add1, (const bf16_t*)add2, total, N, act);
+    else
+        return pta_fail("epilogue: unknown dtype %d", dtype);
+    return pta_check_launch("epilogue");
+}

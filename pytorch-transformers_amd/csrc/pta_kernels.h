@@ -1,0 +1,64 @@
+// C entry points of the gfx950 kernel library (libpta_kernels.so).
+//
+// Conventions: every pointer is device memory unless it says "host"; `dtype` is
+// 0 for 32-bit float and 1 for bfloat16 and names the type of activations,
+// matrices and cache; norm weights and biases are always 32-bit; integer
+// arrays are int32; `stream` is a hipStream_t.  Activations are row-major
+// [tokens, features].  A function returns 0, or non-zero after storing a message
+// that pta_last_error() returns; shapes are checked on the host before a launch.
+//
+// Cache pools have the layout [page, kv_head, 64, head_dim]; `block_table` is
+// [sequences in the step, bt_stride] and lists each sequence's pages in order.
+#pragma once
+
+#include <stdint.h>
+
+#define PTA_ABI_VERSION 1
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char* pta_last_error(void);
+int pta_abi_version(void);
+int pta_page_size(void);
+
+// out[m, :] = table[ids[m], :]
+int pta_embed(void* out, const void* table, const int* ids, int M, int H, int dtype, void* stream);
+
+// out1 = LN(x[rows]) * w1 + b1, and out2 with (w2, b2) if out2 is not null; rows may be null (identity)
+int pta_layernorm(void* out1, void* out2, const void* x, const int* rows, const float* w1, const float* b1,
+                  const float* w2, const float* b2, int M, int H, float eps, int dtype, void* stream);
+
+// in place: y = act(round(y + bias)) + add1 + add2; bias, add1, add2 may be null
+int pta_epilogue(void* y, const float* bias, const void* add1, const void* add2, int M, int N, int act, int dtype,
+                 void* stream);
+
+// split fused qkv rows, add bias, rotate q and k (inv_freq null: no rotation), write q and append k, v
+int pta_qkv_rope_cache(void* q_out, const void* fused, const float* bias, const float* inv_freq, float cs_scale,
+                       const int* token_pos, const int* token_seq, const int* block_table, int bt_stride,
+                       void* k_pool, void* v_pool, int M, int nh, int nkv, int d, int layout, int write_cache,
+                       int dtype, void* stream);
+
+// causal attention of M tokens over their sequences' cache, 32-bit arithmetic
+int pta_attn_generic(void* out, const void* q, const void* k_pool, const void* v_pool, const int* block_table,
+                     int bt_stride, const int* token_seq, const int* token_pos, const float* slopes, int M, int nh,
+                     int nkv, int d, float scale, int dtype, void* stream);
+
+// C = act(A . W^T + bias) + add1 + add2, all 32-bit, fixed summation order
+int pta_gemm_f32(float* C, const float* A, const float* W, const float* bias, const float* add1, const float* add2,
+                 int M, int N, int K, int act, void* stream);
+
+// processors in the reference's order, then argmax (do_sample 0) or a draw; `work` [R, V] receives the
+// processed scores; hist/hist_off (tokens seen, per row), eos/suppress, uniforms may be null
+int pta_sample(int* out_tok, float* work, const float* logits, int R, int V, int do_sample, float temperature,
+               int top_k, float top_p, float min_p, float penalty, const int* hist, const int* hist_off,
+               const int* eos, int n_eos, const int* suppress, int remove_invalid, int renorm, uint64_t seed,
+               const int* rng_seq, const int* rng_step, const float* uniforms, void* stream);
+
+// host function: the uniform number in [0, 1) that pta_sample draws for (seed, sequence, step)
+float pta_philox_uniform(uint64_t seed, uint32_t seq, uint32_t step);
+
+#ifdef __cplusplus
+}
+#endif

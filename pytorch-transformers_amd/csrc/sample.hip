@@ -1,0 +1,314 @@
+// Next-token choice on the GPU: the reference's logits processors in their order, then argmax or
+// a draw from the softmax, one workgroup per row of 32-bit logits.
+//
+// Order (src/transformers/generation/utils.py:926-1097): repetition penalty, EOS suppression
+// (minimum length), removal of invalid values, then for sampling temperature, top-k, top-p, min-p;
+// then softmax and a draw (:3274-3279) or argmax.  Formulas: src/transformers/generation/logits_process.py
+// :337-343 (penalty), :144-151 (EOS), :1618-1626 (invalid), :286-289 (temperature), :505-518 (top-k),
+// :452-465 (top-p), :578-595 (min-p), :1762-1764 (renormalise).
+//
+// Thresholds are found without sorting: the k-th largest score by a radix search on counts, the
+// top-p cut by a radix search on probability mass held in 40-bit fixed point, so that both are
+// sums of integers and do not depend on the order in which threads add.  The draw inverts the
+// cumulative distribution in index order with a fixed summation order, from a uniform number of a
+// counter-based generator keyed by (seed, sequence, step): a sequence draws the same token alone or
+// in any batch.
+#include "common.h"
+#include "pta_kernels.h"
+
+#include <float.h>
+
+#define S_THREADS 1024
+
+__device__ __forceinline__ uint32_t order_key(float f) {
+    const uint32_t u = __float_as_uint(f);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+// Philox4x32-10 (Salmon et al. 2011), one block of four 32-bit words
+__device__ __forceinline__ void philox4x32_10(uint32_t c[4], uint32_t k0, uint32_t k1) {
+#pragma unroll
+    for (int r = 0; r < 10; ++r) {
+        const uint64_t p0 = (uint64_t)0xD2511F53u * c[0];
+        const uint64_t p1 = (uint64_t)0xCD9E8D57u * c[2];
+        const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c[1] ^ k0;
+        const uint32_t n1 = (uint32_t)p1;
+        const uint32_t n2 = (uint32_t)(p0 >> 32) ^ c[3] ^ k1;
+        const uint32_t n3 = (uint32_t)p0;
+        c[0] = n0; c[1] = n1; c[2] = n2; c[3] = n3;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+}
+
+__device__ __forceinline__ float uniform_of(uint64_t seed, uint32_t seq, uint32_t step) {
+    uint32_t c[4] = {seq, step, 0u, 0u};
+    philox4x32_10(c, (uint32_t)seed, (uint32_t)(seed >> 32));
+    return (float)(c[0] >> 8) * (1.0f / 16777216.0f);  // 24 bits, [0, 1)
+}
+
+extern "C" float pta_philox_uniform(uint64_t seed, uint32_t seq, uint32_t step);
+
+struct ArgBest { float v; int i; };
+
+// largest value, lowest index among equals; every thread gets the result
+__device__ __forceinline__ ArgBest block_argmax(float v, int i, float* red_v, int* red_i) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(v, o, 64);
+        const int oi = __shfl_xor(i, o, 64);
+        if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; }
+    }
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    __syncthreads();
+    if (lane == 0) { red_v[wave] = v; red_i[wave] = i; }
+    __syncthreads();
+    ArgBest b = {red_v[0], red_i[0]};
+    for (int w = 1; w < nw; ++w)
+        if (red_v[w] > b.v || (red_v[w] == b.v && red_i[w] < b.i)) { b.v = red_v[w]; b.i = red_i[w]; }
+    return b;
+}
+
+#define MASS_ONE 1099511627776.0f /* 2^40 */
+
+__global__ __launch_bounds__(S_THREADS) void sample_kernel(
+    int* __restrict__ out_tok, float* __restrict__ work, const float* __restrict__ logits, int V, int do_sample,
+    float temperature, int top_k, float top_p, float min_p, float penalty, const int* __restrict__ hist,
+    const int* __restrict__ hist_off, const int* __restrict__ eos, int n_eos, const int* __restrict__ suppress,
+    int remove_invalid, int renorm, uint64_t seed, const int* __restrict__ rng_seq, const int* __restrict__ rng_step,
+    const float* __restrict__ uniforms) {
+    __shared__ float red[16];
+    __shared__ int red_i[16];
+    __shared__ uint32_t cnt[256];
+    __shared__ unsigned long long mass[256];
+    __shared__ float csum[S_THREADS];
+    __shared__ uint32_t sh_bin, sh_remaining, sh_all;
+    __shared__ unsigned long long sh_cum;
+    __shared__ int sh_pick;
+    __shared__ float sh_target;
+
+    const int row = blockIdx.x, tid = threadIdx.x;
+    float* w = work + (long)row * V;
+    const float* l = logits + (long)row * V;
+
+    for (int i = tid; i < V; i += S_THREADS) w[i] = l[i];
+    __syncthreads();
+    if (hist_off && penalty != 1.0f) {
+        for (int t = hist_off[row] + tid; t < hist_off[row + 1]; t += S_THREADS) {
+            const int tok = hist[t];
+            if (tok >= 0 && tok < V) {
+                const float v = l[tok];
+                w[tok] = v < 0.f ? v * penalty : v / penalty;
+            }
+        }
+        __syncthreads();
+    }
+    if (suppress && suppress[row]) {
+        for (int e = tid; e < n_eos; e += S_THREADS)
+            if (eos[e] >= 0 && eos[e] < V) w[eos[e]] = -INFINITY;
+        __syncthreads();
+    }
+    if (remove_invalid) {
+        for (int i = tid; i < V; i += S_THREADS) {
+            float v = w[i];
+            if (v != v) v = 0.f;
+            else if (v == INFINITY) v = FLT_MAX;
+            else if (v == -INFINITY) v = -FLT_MAX;
+            w[i] = v;
+        }
+        __syncthreads();
+    }
+
+    if (do_sample) {
+        if (temperature != 1.0f) {
+            for (int i = tid; i < V; i += S_THREADS) w[i] = w[i] / temperature;
+            __syncthreads();
+        }
+        if (top_k > 0 && top_k < V) {
+            // key of the k-th largest score, one byte at a time from the top
+            uint32_t prefix = 0, maskbits = 0;
+            if (tid == 0) sh_remaining = (uint32_t)top_k;
+            for (int shift = 24; shift >= 0; shift -= 8) {
+                if (tid < 256) cnt[tid] = 0;
+                __syncthreads();
+                for (int i = tid; i < V; i += S_THREADS) {
+                    const uint32_t k = order_key(w[i]);
+                    if ((k & maskbits) == prefix) atomicAdd(&cnt[(k >> shift) & 255u], 1u);
+                }
+                __syncthreads();
+                if (tid == 0) {
+                    uint32_t rem = sh_remaining;
+                    int b = 255;
+                    while (b > 0 && cnt[b] < rem) { rem -= cnt[b]; --b; }
+                    sh_bin = (uint32_t)b;
+                    sh_remaining = rem;
+                }
+                __syncthreads();
+                prefix |= sh_bin << shift;
+                maskbits |= 255u << shift;
+            }
+            for (int i = tid; i < V; i += S_THREADS)
+                if (order_key(w[i]) < prefix) w[i] = -INFINITY;
+            __syncthreads();
+        }
+        if (top_p < 1.0f) {
+            float mx = -INFINITY;
+            int mi = 0x7fffffff;
+            for (int i = tid; i < V; i += S_THREADS)
+                if (w[i] > mx) { mx = w[i]; mi = i; }
+            const ArgBest best = block_argmax(mx, mi, red, red_i);
+            float s = 0.f;
+            for (int i = tid; i < V; i += S_THREADS) s += expf(w[i] - best.v);
+            const float Z = block_sum(s, red);
+            const unsigned long long T = (unsigned long long)((double)(1.0f - top_p) * (double)MASS_ONE);
+            uint32_t prefix = 0, maskbits = 0;
+            if (tid == 0) { sh_cum = 0ull; sh_all = 0u; }
+            for (int shift = 24; shift >= 0; shift -= 8) {
+                if (tid < 256) mass[tid] = 0ull;
+                __syncthreads();
+                for (int i = tid; i < V; i += S_THREADS) {
+                    const uint32_t k = order_key(w[i]);
+                    if ((k & maskbits) == prefix) {
+                        const unsigned long long q = (unsigned long long)(expf(w[i] - best.v) / Z * MASS_ONE + 0.5f);
+                        if (q) atomicAdd(&mass[(k >> shift) & 255u], q);
+                    }
+                }
+                __syncthreads();
+                if (tid == 0) {
+                    unsigned long long cum = sh_cum;
+                    int b = 0;
+                    while (b < 256 && cum + mass[b] <= T) { cum += mass[b]; ++b; }
+                    if (b == 256) { sh_all = 1u; b = 255; }
+                    sh_bin = (uint32_t)b;
+                    sh_cum = cum;
+                }
+                __syncthreads();
+                if (sh_all) break;
+                prefix |= sh_bin << shift;
+                maskbits |= 255u << shift;
+            }
+            // prefix: the lowest key that stays.  If everything could go, the largest score stays.
+            const uint32_t keep_from = sh_all ? order_key(best.v) : prefix;
+            for (int i = tid; i < V; i += S_THREADS)
+                if (order_key(w[i]) < keep_from) w[i] = -INFINITY;
+            __syncthreads();
+            if (!sh_all && tid == 0) {
+                // equal scores at the cut: in ascending stable order the first of them go while they fit
+                const float vcut = __uint_as_float((prefix & 0x80000000u) ? (prefix & 0x7fffffffu) : ~prefix);
+                const unsigned long long q = (unsigned long long)(expf(vcut - best.v) / Z * MASS_ONE + 0.5f);
+                unsigned long long r = q ? (T - sh_cum) / q : 0ull;
+                if (r > 0) {
+                    // never the last one: one token at least stays
+                    int last = -1;
+                    for (int i = 0; i < V; ++i) if (order_key(w[i]) == prefix) last = i;
+                    for (int i = 0; i < V && r > 0; ++i)
+                        if (i != last && order_key(w[i]) == prefix) { w[i] = -INFINITY; --r; }
+                }
+            }
+            __syncthreads();
+        }
+        if (min_p > 0.0f) {
+            float mx = -INFINITY;
+            for (int i = tid; i < V; i += S_THREADS) mx = fmaxf(mx, w[i]);
+            mx = block_max(mx, red);
+            float s = 0.f;
+            for (int i = tid; i < V; i += S_THREADS) s += expf(w[i] - mx);
+            const float Z = block_sum(s, red);
+            const float thr = min_p * (1.0f / Z);
+            for (int i = tid; i < V; i += S_THREADS)
+                if (w[i] != mx && expf(w[i] - mx) / Z < thr) w[i] = -INFINITY;
+            __syncthreads();
+        }
+    }
+
+    // choose
+    float mx = -INFINITY;
+    int mi = 0x7fffffff;
+    for (int i = tid; i < V; i += S_THREADS)
+        if (w[i] > mx) { mx = w[i]; mi = i; }
+    const ArgBest best = block_argmax(mx, mi, red, red_i);
+    int chosen = best.i;
+    float Z = 0.f;
+    if (do_sample || renorm) {
+        const int chunk = (V + S_THREADS - 1) / S_THREADS;
+        const int lo = min(V, tid * chunk), hi = min(V, lo + chunk);
+        float s = 0.f;
+        for (int i = lo; i < hi; ++i) s += expf(w[i] - best.v);
+        csum[tid] = s;
+        __syncthreads();
+        if (tid == 0) {
+            float total = 0.f;
+            for (int t = 0; t < S_THREADS; ++t) total += csum[t];
+            red[0] = total;
+            if (do_sample) {
+                const float u = uniforms ? uniforms[row] : uniform_of(seed, (uint32_t)rng_seq[row], (uint32_t)rng_step[row]);
+                const float target = u * total;
+                float acc = 0.f;
+                int pick = -1, last_nonzero = 0;
+                for (int t = 0; t < S_THREADS; ++t) {
+                    if (csum[t] > 0.f) last_nonzero = t;
+                    if (pick < 0 && acc + csum[t] > target) { pick = t; sh_target = target - acc; }
+                    if (pick < 0) acc += csum[t];
+                }
+                if (pick < 0) { pick = last_nonzero; sh_target = INFINITY; }
+                sh_pick = pick;
+            }
+        }
+        __syncthreads();
+        Z = red[0];
+        if (do_sample && tid == sh_pick) {
+            float acc = 0.f;
+            int tok = -1, last = lo;
+            for (int i = lo; i < hi; ++i) {
+                const float e = expf(w[i] - best.v);
+                if (e > 0.f) last = i;
+                acc += e;
+                if (acc > sh_target) { tok = i; break; }
+            }
+            out_tok[row] = tok >= 0 ? tok : last;
+        }
+    }
+    if (!do_sample && tid == 0) out_tok[row] = chosen;
+    if (renorm) {
+        __syncthreads();
+        const float lse = best.v + logf(Z);
+        for (int i = tid; i < V; i += S_THREADS) w[i] = w[i] - lse;
+    }
+}
+
+extern "C" int pta_sample(int* out_tok, float* work, const float* logits, int R, int V, int do_sample,
+                          float temperature, int top_k, float top_p, float min_p, float penalty, const int* hist,
+                          const int* hist_off, const int* eos, int n_eos, const int* suppress, int remove_invalid,
+                          int renorm, uint64_t seed, const int* rng_seq, const int* rng_step, const float* uniforms,
+                          void* stream) {
+    PTA_REQUIRE(R > 0 && V > 0, "sample: rows=%d vocab=%d must be positive", R, V);
+    PTA_REQUIRE(out_tok && work && logits, "sample: null pointer");
+    PTA_REQUIRE(!do_sample || temperature > 0.f, "sample: temperature must be > 0, got %g", (double)temperature);
+    PTA_REQUIRE(top_p >= 0.f && top_p <= 1.f, "sample: top_p must be in [0, 1], got %g", (double)top_p);
+    PTA_REQUIRE(min_p >= 0.f && min_p <= 1.f, "sample: min_p must be in [0, 1], got %g", (double)min_p);
+    PTA_REQUIRE(penalty > 0.f, "sample: repetition penalty must be > 0, got %g", (double)penalty);
+    PTA_REQUIRE(!do_sample || uniforms || (rng_seq && rng_step), "sample: sampling needs uniforms or rng counters");
+    PTA_REQUIRE(n_eos == 0 || eos, "sample: eos ids missing");
+    hipLaunchKernelGGL(sample_kernel, dim3(R), dim3(S_THREADS), 0, (hipStream_t)stream, out_tok, work, logits, V,
+                       do_sample, temperature, top_k, top_p, min_p, penalty, hist, hist_off, eos, n_eos, suppress,
+                       remove_invalid, renorm, seed, rng_seq, rng_step, uniforms);
+    return pta_check_launch("sample");
+}
+
+// the same generator on the host, for tests and for callers that want the number itself
+extern "C" float pta_philox_uniform(uint64_t seed, uint32_t seq, uint32_t step) {
+    uint32_t c[4] = {seq, step, 0u, 0u};
+    uint32_t k0 = (uint32_t)seed, k1 = (uint32_t)(seed >> 32);
+    for (int r = 0; r < 10; ++r) {
+        const uint64_t p0 = (uint64_t)0xD2511F53u * c[0];
+        const uint64_t p1 = (uint64_t)0xCD9E8D57u * c[2];
+        const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c[1] ^ k0;
+        const uint32_t n1 = (uint32_t)p1;
+        const uint32_t n2 = (uint32_t)(p0 >> 32) ^ c[3] ^ k1;
+        const uint32_t n3 = (uint32_t)p0;
+        c[0] = n0; c[1] = n1; c[2] = n2; c[3] = n3;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+    return (float)(c[0] >> 8) * (1.0f / 16777216.0f);
+}

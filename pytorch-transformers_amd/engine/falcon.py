@@ -1,0 +1,52 @@
+"""The Falcon architecture as a list of parts: the builder registered for ``model_type: falcon``.
+
+Tensor names are the checkpoint's (module tree of
+src/transformers/models/falcon/modeling_falcon.py:826-850, :588-612, :221-267, :565-578, :1165-1171,
+base prefix ``transformer.`` :782).  Which norms a block has follows the decoder layer's constructor
+and forward (:599-612, :630-666); see ``config.falcon.FalconConfig.norm_scheme``.
+"""
+from __future__ import annotations
+
+from ..config.falcon import NORMS_DUAL, NORMS_SEQUENTIAL, FalconConfig
+from ..config.registry import register
+from ..parts import (AlibiPositions, AttentionMixer, DenseFeedForward, Embedding, LayerNorm, OutputHead,
+                     ParallelBlock, RotaryPositions, SequentialBlock)
+from .spec import CACHE_FULL, CacheGroupSpec, LayerCall, ModelSpec
+
+KV_GROUP = "kv"
+
+
+def build_falcon(cfg: FalconConfig) -> ModelSpec:
+    H, L, eps = cfg.hidden_size, cfg.num_hidden_layers, cfg.layer_norm_epsilon
+    if cfg.alibi:
+        positions = AlibiPositions(cfg.num_attention_heads)
+    else:
+        factor = float(cfg.rope_scaling["factor"]) if cfg.rope_type == "linear" else 1.0
+        positions = RotaryPositions(cfg.head_dim, cfg.rope_theta, scaling_factor=factor)
+    blocks = []
+    for i in range(L):
+        p = f"transformer.h.{i}"
+        mixer = AttentionMixer(f"{p}.self_attention", H, cfg.num_attention_heads, cfg.kv_heads, cfg.head_dim,
+                               cfg.qkv_layout, cfg.bias, positions)
+        ffn = DenseFeedForward(f"{p}.mlp", H, cfg.ffn_hidden_size, cfg.bias, cfg.activation)
+        if cfg.norm_scheme == NORMS_SEQUENTIAL:
+            block = SequentialBlock(mixer, ffn, LayerNorm(f"{p}.input_layernorm", H, eps),
+                                    LayerNorm(f"{p}.post_attention_layernorm", H, eps))
+        elif cfg.norm_scheme == NORMS_DUAL:
+            block = ParallelBlock(mixer, ffn, LayerNorm(f"{p}.ln_attn", H, eps), LayerNorm(f"{p}.ln_mlp", H, eps))
+        else:
+            block = ParallelBlock(mixer, ffn, LayerNorm(f"{p}.input_layernorm", H, eps))
+        blocks.append(block)
+    embed_name = "transformer.word_embeddings"
+    return ModelSpec(
+        config=cfg,
+        embedding=Embedding(embed_name, cfg.vocab_size, H),
+        blocks=blocks,
+        order=[LayerCall(i, KV_GROUP, i) for i in range(L)],
+        final_norm=LayerNorm("transformer.ln_f", H, eps),
+        head=OutputHead("lm_head", cfg.vocab_size, H, f"{embed_name}.weight" if cfg.tie_word_embeddings else None),
+        cache_groups=[CacheGroupSpec(KV_GROUP, CACHE_FULL, L, cfg.kv_heads, cfg.head_dim)],
+    )
+
+
+register("falcon", FalconConfig, build_falcon, exist_ok=True)

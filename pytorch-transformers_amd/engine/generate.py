@@ -1,0 +1,165 @@
+"""The generation loop: batches of unequal prompts, stop tokens, sequences that end earlier.
+
+What the reference's ``generate`` and ``_sample`` do
+(src/transformers/generation/utils.py:1908-2401, :3139-3324), on top of the step function:
+
+* prompts of a batch go through one step together, unpadded, then every live sequence brings one
+  token per step; the reference pads on the left and masks (:2036-2059);
+* a sequence that produced a stop token (kept in its output, stopping_criteria.py:446-467) or
+  reached its length leaves the batch and gives its slot back at once; the reference keeps
+  feeding it padding until all rows are done (:3282-3291);
+* requests beyond ``batch_size`` run as further batches on the same cache, whose slots and pages
+  are used again.
+
+The loop decides on the host and needs from the model only ``new_cache``, ``step`` and a sampler,
+so its decisions are tested without a GPU.
+"""
+from __future__ import annotations
+
+import dataclasses
+import time
+from typing import Callable, List, Optional, Sequence, Union
+
+from ..config.generation import GenerationConfig
+
+PAGE = 64
+
+
+@dataclasses.dataclass
+class GenerateOutput:
+    """``return_dict_in_generate=True`` (src/transformers/generation/utils.py:3314-3322)."""
+
+    sequences: List[List[int]]
+    scores: Optional[List[List]] = None  # per sequence, per new token: processed scores [vocab]
+    logits: Optional[List[List]] = None  # per sequence, per new token: raw logits [vocab]
+
+
+def _round_up(n: int, m: int) -> int:
+    return (n + m - 1) // m * m
+
+
+def resolve_lengths(cfg: GenerationConfig, prompt_lens: Sequence[int]):
+    """New tokens per sequence and the padded length the reference's length rules count from.
+
+    ``max_new_tokens`` wins over ``max_length`` (:1461); the reference measures lengths on the
+    left-padded batch, so every row gets the same number of new tokens; a prompt that already
+    fills ``max_length`` is an error (:1409-1415).
+    """
+    longest = max(prompt_lens)
+    if cfg.max_new_tokens is not None:
+        new = int(cfg.max_new_tokens)
+    else:
+        new = int(cfg.max_length) - longest
+        if new <= 0:
+            raise ValueError(
+                f"Input length of input_ids is {longest}, but `max_length` is set to {cfg.max_length}. This can "
+                "lead to unexpected behavior. You should consider increasing `max_length` or, better yet, setting "
+                "`max_new_tokens`.")
+    return new, longest
+
+
+def generate(model, prompts: Sequence[Sequence[int]], generation_config: Optional[GenerationConfig] = None, *,
+             batch_size: Optional[int] = None, sampler=None, streamer=None, cache=None,
+             rng_ids: Optional[Sequence[int]] = None, **kwargs) -> Union[List[List[int]], GenerateOutput]:
+    """Generate for every prompt (a list of token ids); returns prompt + new tokens per prompt.
+
+    ``generation_config`` defaults to the model's; keyword arguments override its fields
+    (:1543-1545).  ``streamer`` is called as ``streamer(index, token)`` for every new token and
+    ``streamer.end()`` if it has one.  ``rng_ids`` name each prompt's random stream (default: its
+    index), so that a prompt draws the same tokens in any batch.
+    """
+    cfg = generation_config or getattr(model, "generation_config", None) or GenerationConfig()
+    if kwargs:
+        cfg = cfg.updated(**kwargs)
+    prompts = [list(map(int, p)) for p in prompts]
+    if not prompts:
+        return GenerateOutput([]) if cfg.return_dict_in_generate else []
+    bos = cfg.bos_token_id
+    for i, p in enumerate(prompts):
+        if not p:  # an empty prompt starts from BOS (:547-577)
+            if bos is None:
+                raise ValueError(f"prompt {i} is empty and no bos_token_id is set")
+            prompts[i] = [int(bos)]
+    n_ret = cfg.num_return_sequences
+    if n_ret > 1:  # :2244-2249, :716-748
+        prompts = [p for p in prompts for _ in range(n_ret)]
+    ids = list(rng_ids) if rng_ids is not None else list(range(len(prompts)))
+    if n_ret > 1 and rng_ids is not None:
+        ids = [r * n_ret + j for r in rng_ids for j in range(n_ret)]
+    if len(ids) != len(prompts):
+        raise ValueError("rng_ids must name one stream per prompt")
+
+    batch_size = batch_size or len(prompts)
+    batches = [list(range(b, min(b + batch_size, len(prompts)))) for b in range(0, len(prompts), batch_size)]
+    need = 0
+    for b in batches:
+        new, _ = resolve_lengths(cfg, [len(prompts[i]) for i in b])
+        need = max(need, sum(_round_up(len(prompts[i]) + new, PAGE) for i in b))
+    if cache is None:
+        cache = model.new_cache(need, max_slots=batch_size)
+    if sampler is None:
+        from ..sampling.sampler import Sampler
+
+        sampler = Sampler(cfg, model.vocab_size, model.device)
+
+    eos = set(cfg.eos_token_ids)
+    want_scores, want_logits = bool(cfg.output_scores), bool(cfg.output_logits)
+    out_tokens: List[List[int]] = [[] for _ in prompts]
+    out_scores = [[] for _ in prompts] if want_scores else None
+    out_logits = [[] for _ in prompts] if want_logits else None
+    t0 = time.time()
+
+    for batch in batches:
+        new_budget, padded_len = resolve_lengths(cfg, [len(prompts[i]) for i in batch])
+        slot_of = {i: cache.alloc() for i in batch}
+        live = list(batch)
+        feed = {i: prompts[i] for i in batch}
+        step_no = 0
+        try:
+            while live:
+                logits = model.step(cache, [slot_of[i] for i in live], [feed[i] for i in live], "last")
+                # EOS is masked while the minimum lengths are not reached (logits_process.py:144-151, :214-223)
+                too_short = (padded_len + step_no < (cfg.min_length or 0)) or (step_no < (cfg.min_new_tokens or 0))
+                tokens, scores = sampler.sample(
+                    logits, rng_seq=[ids[i] for i in live], rng_step=[step_no] * len(live),
+                    histories=[prompts[i] + out_tokens[i] for i in live], suppress_eos=[too_short] * len(live))
+                step_no += 1
+                timed_out = cfg.max_time is not None and (time.time() - t0) > cfg.max_time  # stopping_criteria.py:87-107
+                still = []
+                for row, i in enumerate(live):
+                    tok = int(tokens[row])
+                    out_tokens[i].append(tok)
+                    if want_scores:
+                        out_scores[i].append(scores[row].clone())
+                    if want_logits:
+                        out_logits[i].append(logits[row].clone())
+                    if streamer is not None:
+                        streamer(i, tok)
+                    if tok in eos or step_no >= new_budget or timed_out:
+                        cache.free(slot_of.pop(i))
+                    else:
+                        feed[i] = [tok]
+                        still.append(i)
+                live = still
+        finally:
+            for i in list(slot_of):
+                cache.free(slot_of.pop(i))
+    if streamer is not None and hasattr(streamer, "end"):
+        streamer.end()
+    sequences = [p + t for p, t in zip(prompts, out_tokens)]
+    if cfg.return_dict_in_generate:
+        return GenerateOutput(sequences, out_scores, out_logits)
+    return sequences
+
+
+def pad_sequences(sequences: Sequence[Sequence[int]], prompt_lens: Sequence[int], pad_token_id: int):
+    """The reference's rectangular return value: prompts padded on the left to the longest prompt, new
+    tokens padded on the right after a row ended (src/transformers/generation/utils.py:3282-3286)."""
+    import torch
+
+    longest = max(prompt_lens)
+    width = longest + max(len(s) - n for s, n in zip(sequences, prompt_lens))
+    out = torch.full((len(sequences), width), int(pad_token_id), dtype=torch.long)
+    for r, (s, n) in enumerate(zip(sequences, prompt_lens)):
+        out[r, longest - n:longest - n + len(s)] = torch.as_tensor(list(s), dtype=torch.long)
+    return out

@@ -1,0 +1,167 @@
+"""A causal language model put together from a ModelSpec, and its one step function.
+
+The reference's forward pass takes a padded batch, a cache object, a mask and positions and returns
+the logits of the last ``num_logits_to_keep`` places of every row
+(src/transformers/models/falcon/modeling_falcon.py:1185-1254, :864-1011).  ``CausalLM.step`` takes,
+for each sequence of a batch, its slot, the tokens it brings and the places whose logits are
+wanted; it runs exactly those tokens from the cache, appends their keys and values, and returns the
+wanted rows as 32-bit logits.  Whole prompts, single decoded tokens and any cut in between are the
+same call.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache.paged import PagedCache
+from ..config.registry import AutoConfig, lookup
+from ..parts.base import StepContext
+from ..weights.loader import load_weights
+from ..weights.random_init import random_tensors
+from .spec import ModelSpec
+from .step import StepPlan, Want, plan_step
+
+_DTYPES = {"float32": torch.float32, "fp32": torch.float32, "bfloat16": torch.bfloat16, "bf16": torch.bfloat16,
+           torch.float32: torch.float32, torch.bfloat16: torch.bfloat16}
+
+
+def resolve_dtype(dtype) -> torch.dtype:
+    try:
+        return _DTYPES[dtype]
+    except KeyError:
+        raise ValueError(f"dtype must be 'float32' or 'bfloat16', got {dtype!r}") from None
+
+
+def _require_gpu(device) -> torch.device:
+    device = torch.device(device)
+    if device.type != "cuda" or not torch.cuda.is_available():
+        raise RuntimeError(
+            f"the engine runs on an AMD GPU through its HIP kernels and has no CPU path (device={device}, "
+            f"torch.cuda.is_available()={torch.cuda.is_available()})")
+    return device
+
+
+class CausalLM:
+    def __init__(self, spec: ModelSpec, tensors: Dict[str, torch.Tensor], dtype: torch.dtype, device):
+        spec.validate()
+        self.spec = spec
+        self.config = spec.config
+        self.dtype = dtype
+        self.device = torch.device(device)
+        self.vocab_size = spec.head.vocab_size
+        for part in spec.parts():
+            part.load_all(tensors)
+        self._move_constants()
+        self.generation_config = None
+
+    def _move_constants(self) -> None:
+        seen = set()
+
+        def walk(p):
+            if id(p) in seen:
+                return
+            seen.add(id(p))
+            if hasattr(p, "to"):
+                p.to(self.device)
+            for c in p.children():
+                walk(c)
+
+        for part in self.spec.parts():
+            walk(part)
+
+    # construction ----------------------------------------------------------
+    @classmethod
+    def from_pretrained(cls, folder: str, dtype="bfloat16", device="cuda:0", strict: bool = True) -> "CausalLM":
+        from ..config.generation import GenerationConfig
+
+        device = _require_gpu(device)
+        dtype = resolve_dtype(dtype)
+        config = AutoConfig.from_pretrained(folder)
+        _, builder = lookup(config.model_type)
+        spec = builder(config)
+        tensors = load_weights(folder, spec.tensor_specs(), dtype, device, strict=strict)
+        model = cls(spec, tensors, dtype, device)
+        model.generation_config = GenerationConfig.from_pretrained(folder, config)
+        return model
+
+    @classmethod
+    def from_config(cls, config, seed: int = 0, dtype="bfloat16", device="cuda:0", std: Optional[float] = None,
+                    noise: Optional[float] = None) -> "CausalLM":
+        """Random weights drawn on the device; nothing is written to disk."""
+        from ..config.generation import GenerationConfig
+
+        device = _require_gpu(device)
+        dtype = resolve_dtype(dtype)
+        _, builder = lookup(config.model_type)
+        spec = builder(config)
+        std = float(getattr(config, "initializer_range", 0.02) if std is None else std)
+        specs = spec.tensor_specs()
+        tensors = random_tensors(specs, seed, std, noise=noise, device=device, compute_dtype=dtype)
+        for s in specs:
+            if s.name not in tensors and s.tied_to is not None:
+                tensors[s.name] = tensors[s.tied_to]
+        model = cls(spec, tensors, dtype, device)
+        model.generation_config = GenerationConfig.from_model_config(config)
+        return model
+
+    # cache -------------------------------------------------------------------
+    def new_cache(self, max_tokens: int, max_slots: Optional[int] = None) -> PagedCache:
+        """A cache for at most ``max_tokens`` live tokens (each sequence's count rounded up to a page)."""
+        return PagedCache(self.spec.cache_groups, max_tokens, self.dtype, self.device, max_slots=max_slots)
+
+    # the step ------------------------------------------------------------------
+    def make_context(self, plan: StepPlan, cache: PagedCache):
+        """Upload a plan's arrays in one buffer and wrap the views."""
+        n, M, R = plan.n_seqs, plan.n_tokens, int(plan.logit_rows.shape[0])
+        pieces = [plan.token_ids, plan.token_seq, plan.token_pos, plan.cu_tokens,
+                  np.asarray(plan.starts, dtype=np.int32), np.asarray(plan.slots, dtype=np.int32), plan.logit_rows]
+        names = list(plan.block_tables)
+        pieces += [plan.block_tables[g].reshape(-1) for g in names]
+        sizes = [int(p.shape[0]) for p in pieces]
+        dev = torch.from_numpy(np.concatenate(pieces)).to(self.device)
+        views = torch.split(dev, sizes)
+        tables = {g: views[7 + i].view(plan.block_tables[g].shape) for i, g in enumerate(names)}
+        ctx = StepContext(dtype=self.dtype, device=self.device, n_seqs=n, n_tokens=M, token_seq=views[1],
+                          token_pos=views[2], cu_tokens=views[3], seq_start=views[4], seq_slot=views[5],
+                          block_tables=tables, cache=cache, slots=plan.slots, new_tokens=plan.new_tokens,
+                          starts=plan.starts, is_decode=plan.is_decode, max_len=plan.max_len)
+        return ctx, views[0], (views[6] if R else None)
+
+    def forward_tokens(self, ctx: StepContext, token_ids: torch.Tensor, logit_rows: Optional[torch.Tensor]):
+        """Embedding, the layers in their run order, final norm and head on the wanted rows."""
+        x = self.spec.embedding.forward(token_ids)
+        blocks = self.spec.blocks
+        for call in self.spec.order:
+            x = blocks[call.block].forward(x, ctx, call)
+        if logit_rows is None:
+            return None
+        if self.spec.final_norm is not None:
+            h = self.spec.final_norm.forward(x, rows=logit_rows)
+        else:
+            h = x.index_select(0, logit_rows.long())
+        return self.spec.head.forward(h)
+
+    @torch.no_grad()
+    def step(self, cache: PagedCache, slots: Sequence[int], tokens: Sequence[Sequence[int]],
+             want: Want = "last") -> torch.Tensor:
+        """Run the given tokens of the given sequences; return logits ``[wanted places, vocab]`` in 32-bit.
+
+        ``want`` is ``"last"``, ``"all"``, ``"none"`` or, per sequence, the places among its tokens
+        of this step whose logits are asked for.  Rows come in the order of the sequences and of
+        their places.
+        """
+        plan = plan_step(cache, slots, tokens, want, self.vocab_size)
+        ctx, ids, rows = self.make_context(plan, cache)
+        logits = self.forward_tokens(ctx, ids, rows)
+        cache.commit(plan.slots, plan.new_tokens)
+        if logits is None:
+            return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
+        return logits
+
+    # generation (see engine.generate) -----------------------------------------------
+    def generate(self, prompts, generation_config=None, **kwargs):
+        from .generate import generate
+
+        return generate(self, prompts, generation_config, **kwargs)

@@ -1,0 +1,253 @@
+"""Python face of the HIP kernel library: loading, argument checks, one function per kernel.
+
+There is no CPU fallback.  A function given a tensor that is not on a GPU, or
+called when the library cannot be loaded, raises.  Shapes, strides and types are
+checked here, before a pointer reaches a kernel.  Kernels run on torch's current
+stream, so they order with torch's own work and are recorded by a HIP graph
+capture like it.
+"""
+from __future__ import annotations
+
+import ctypes
+import importlib.util
+import os
+import threading
+from typing import Optional
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+F32, BF16 = 0, 1
+QKV_LAYOUT_CODES = {"grouped": 0, "tail": 1, "interleaved": 2}
+ACT_CODES = {None: 0, "none": 0, "gelu": 1}
+ABI_VERSION = 1
+
+_lib = None
+_lock = threading.Lock()
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _build_module():
+    spec = importlib.util.spec_from_file_location("_pta_csrc_build", os.path.join(_HERE, "csrc", "build.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def load_library(build_if_missing: bool = True):
+    """Load libpta_kernels.so, compiling it first if no current build exists."""
+    global _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        b = _build_module()
+        path = b.find_library(require_current=True)
+        if path is None:
+            if not build_if_missing:
+                raise KernelError("libpta_kernels.so is not built (run __graft_entry__.build())")
+            path = b.build(verbose=True)
+        lib = ctypes.CDLL(path)
+        lib.pta_last_error.restype = ctypes.c_char_p
+        if lib.pta_abi_version() != ABI_VERSION:
+            raise KernelError(f"{path} has ABI {lib.pta_abi_version()}, this package needs {ABI_VERSION}; rebuild it")
+        _lib = lib
+        return lib
+
+
+def library_path() -> Optional[str]:
+    return _build_module().find_library(require_current=True)
+
+
+def _call(name: str, *args) -> None:
+    lib = load_library()
+    rc = getattr(lib, name)(*args)
+    if rc != 0:
+        raise KernelError(lib.pta_last_error().decode("utf-8", "replace"))
+
+
+def _stream() -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def dtype_code(dt: torch.dtype) -> int:
+    if dt == torch.float32:
+        return F32
+    if dt == torch.bfloat16:
+        return BF16
+    raise KernelError(f"dtype {dt} is not supported; use torch.float32 or torch.bfloat16")
+
+
+def _ptr(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _need(t: torch.Tensor, name: str, dtype=None, shape=None) -> None:
+    if not isinstance(t, torch.Tensor):
+        raise KernelError(f"{name} must be a tensor")
+    if not t.is_cuda:
+        raise KernelError(f"{name} is on {t.device}; the kernels run on the GPU only and there is no CPU fallback")
+    if not t.is_contiguous():
+        raise KernelError(f"{name} must be contiguous, got strides {t.stride()} for shape {tuple(t.shape)}")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{name} must be {dtype}, got {t.dtype}")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise KernelError(f"{name} must have shape {tuple(shape)}, got {tuple(t.shape)}")
+
+
+# ---------------------------------------------------------------------------
+def embed(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[m] = table[ids[m]].  The caller has checked that ids lie in [0, rows)."""
+    _need(table, "table")
+    V, H = table.shape
+    _need(ids, "ids", torch.int32)
+    M = ids.numel()
+    if out is None:
+        out = torch.empty((M, H), dtype=table.dtype, device=table.device)
+    _need(out, "out", table.dtype, (M, H))
+    _call("pta_embed", _ptr(out), _ptr(table), _ptr(ids), M, H, dtype_code(table.dtype), _stream())
+    return out
+
+
+def layernorm(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float, *, w2=None, b2=None,
+              rows: Optional[torch.Tensor] = None):
+    """LayerNorm of the rows of x (or of x[rows]); with (w2, b2) a second affine output of the same pass."""
+    _need(x, "x")
+    H = x.shape[-1]
+    _need(w, "weight", torch.float32, (H,))
+    _need(b, "bias", torch.float32, (H,))
+    if rows is not None:
+        _need(rows, "rows", torch.int32)
+        M = rows.numel()
+    else:
+        M = x.shape[0]
+    if x.dim() != 2:
+        raise KernelError(f"x must be [tokens, features], got {tuple(x.shape)}")
+    out1 = torch.empty((M, H), dtype=x.dtype, device=x.device)
+    out2 = None
+    if w2 is not None:
+        _need(w2, "weight2", torch.float32, (H,))
+        _need(b2, "bias2", torch.float32, (H,))
+        out2 = torch.empty((M, H), dtype=x.dtype, device=x.device)
+    if M == 0:
+        return (out1, out2) if w2 is not None else out1
+    _call("pta_layernorm", _ptr(out1), _ptr(out2), _ptr(x), _ptr(rows), _ptr(w), _ptr(b), _ptr(w2), _ptr(b2), M, H,
+          ctypes.c_float(eps), dtype_code(x.dtype), _stream())
+    return (out1, out2) if w2 is not None else out1
+
+
+def epilogue_(y: torch.Tensor, bias=None, act=None, add1=None, add2=None) -> torch.Tensor:
+    """In place: y = act(round(y + bias)) + add1 + add2."""
+    _need(y, "y")
+    M, N = y.shape
+    if bias is not None:
+        _need(bias, "bias", torch.float32, (N,))
+    for name, a in (("add1", add1), ("add2", add2)):
+        if a is not None:
+            _need(a, name, y.dtype, (M, N))
+    _call("pta_epilogue", _ptr(y), _ptr(bias), _ptr(add1), _ptr(add2), M, N, ACT_CODES[act], dtype_code(y.dtype),
+          _stream())
+    return y
+
+
+def qkv_rope_cache(fused: torch.Tensor, bias, inv_freq, cs_scale: float, token_pos, token_seq, block_table,
+                   k_pool, v_pool, nh: int, nkv: int, d: int, layout: str, write_cache: bool = True) -> torch.Tensor:
+    """Queries [M, nh, d] from the fused rows; keys and values go to the cache pages."""
+    _need(fused, "fused")
+    M = fused.shape[0]
+    _need(fused, "fused", None, (M, (nh + 2 * nkv) * d))
+    dt = fused.dtype
+    if bias is not None:
+        _need(bias, "bias", torch.float32, ((nh + 2 * nkv) * d,))
+    if inv_freq is not None:
+        _need(inv_freq, "inv_freq", torch.float32, (d // 2,))
+    _need(token_pos, "token_pos", torch.int32, (M,))
+    _need(token_seq, "token_seq", torch.int32, (M,))
+    _need(block_table, "block_table", torch.int32)
+    if block_table.dim() != 2:
+        raise KernelError("block_table must be [sequences, pages]")
+    for name, pool in (("k_pool", k_pool), ("v_pool", v_pool)):
+        _need(pool, name, dt)
+        if pool.dim() != 4 or pool.shape[1] != nkv or pool.shape[2] != 64 or pool.shape[3] != d:
+            raise KernelError(f"{name} must be [pages, {nkv}, 64, {d}], got {tuple(pool.shape)}")
+    q = torch.empty((M, nh, d), dtype=dt, device=fused.device)
+    _call("pta_qkv_rope_cache", _ptr(q), _ptr(fused), _ptr(bias), _ptr(inv_freq), ctypes.c_float(cs_scale),
+          _ptr(token_pos), _ptr(token_seq), _ptr(block_table), block_table.shape[1], _ptr(k_pool), _ptr(v_pool), M,
+          nh, nkv, d, QKV_LAYOUT_CODES[layout], int(write_cache), dtype_code(dt), _stream())
+    return q
+
+
+def attn_generic(q: torch.Tensor, k_pool, v_pool, block_table, token_seq, token_pos, slopes, scale: float):
+    """Causal attention of every token over its sequence's cache; out [M, nh*d]."""
+    _need(q, "q")
+    M, nh, d = q.shape
+    nkv = k_pool.shape[1]
+    for name, pool in (("k_pool", k_pool), ("v_pool", v_pool)):
+        _need(pool, name, q.dtype)
+        if pool.dim() != 4 or pool.shape[1] != nkv or pool.shape[2] != 64 or pool.shape[3] != d:
+            raise KernelError(f"{name} must be [pages, {nkv}, 64, {d}], got {tuple(pool.shape)}")
+    _need(block_table, "block_table", torch.int32)
+    _need(token_seq, "token_seq", torch.int32, (M,))
+    _need(token_pos, "token_pos", torch.int32, (M,))
+    if slopes is not None:
+        _need(slopes, "slopes", torch.float32, (nh,))
+    out = torch.empty((M, nh * d), dtype=q.dtype, device=q.device)
+    _call("pta_attn_generic", _ptr(out), _ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(block_table),
+          block_table.shape[1], _ptr(token_seq), _ptr(token_pos), _ptr(slopes), M, nh, nkv, d, ctypes.c_float(scale),
+          dtype_code(q.dtype), _stream())
+    return out
+
+
+def gemm_f32(a: torch.Tensor, w: torch.Tensor, bias=None, act=None, add1=None, add2=None) -> torch.Tensor:
+    """act(a @ w.T + bias) + add1 + add2 in true 32-bit with a fixed summation order."""
+    _need(a, "a", torch.float32)
+    _need(w, "w", torch.float32)
+    M, K = a.shape
+    N = w.shape[0]
+    if w.shape[1] != K:
+        raise KernelError(f"a is [{M}, {K}] but w is {tuple(w.shape)}; w must be [N, {K}]")
+    if bias is not None:
+        _need(bias, "bias", torch.float32, (N,))
+    for name, t in (("add1", add1), ("add2", add2)):
+        if t is not None:
+            _need(t, name, torch.float32, (M, N))
+    out = torch.empty((M, N), dtype=torch.float32, device=a.device)
+    _call("pta_gemm_f32", _ptr(out), _ptr(a), _ptr(w), _ptr(bias), _ptr(add1), _ptr(add2), M, N, K, ACT_CODES[act],
+          _stream())
+    return out
+
+
+def attention(q: torch.Tensor, k_pool, v_pool, block_table, ctx, slopes, scale: float) -> torch.Tensor:
+    """Attention of a step's tokens over the cache: picks the kernel for the step's shape and type."""
+    return attn_generic(q, k_pool, v_pool, block_table, ctx.token_seq, ctx.token_pos, slopes, scale)
+
+
+def sample(logits: torch.Tensor, *, do_sample: bool, temperature: float = 1.0, top_k: int = 0, top_p: float = 1.0,
+           min_p: float = 0.0, penalty: float = 1.0, hist=None, hist_off=None, eos=None, suppress=None,
+           remove_invalid: bool = False, renorm: bool = False, seed: int = 0, rng_seq=None, rng_step=None,
+           uniforms=None):
+    """Processors and choice for every row of ``logits`` [R, V] (32-bit); returns (tokens int32 [R], scores [R, V])."""
+    _need(logits, "logits", torch.float32)
+    if logits.dim() != 2:
+        raise KernelError(f"logits must be [rows, vocab], got {tuple(logits.shape)}")
+    R, V = logits.shape
+    for name, t, n in (("hist_off", hist_off, R + 1), ("suppress", suppress, R), ("rng_seq", rng_seq, R),
+                       ("rng_step", rng_step, R)):
+        if t is not None:
+            _need(t, name, torch.int32, (n,))
+    if hist is not None:
+        _need(hist, "hist", torch.int32)
+    if eos is not None:
+        _need(eos, "eos", torch.int32)
+    if uniforms is not None:
+        _need(uniforms, "uniforms", torch.float32, (R,))
+    work = torch.empty_like(logits)
+    out = torch.empty((R,), dtype=torch.int32, device=logits.device)
+    _call("pta_sample", _ptr(out), _ptr(work), _ptr(logits), R, V, int(bool(do_sample)), ctypes.c_float(temperature),
+          int(top_k), ctypes.c_float(top_p), ctypes.c_float(min_p), ctypes.c_float(penalty), _ptr(hist), _ptr(hist_off),
+          _ptr(eos), 0 if eos is None else int(eos.numel()), _ptr(suppress), int(bool(remove_invalid)),
+          int(bool(renorm)), ctypes.c_uint64(int(seed) & (2 ** 64 - 1)), _ptr(rng_seq), _ptr(rng_step), _ptr(uniforms),
+          _stream())
+    return out, work

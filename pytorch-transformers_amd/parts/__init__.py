@@ -1,0 +1,12 @@
+"""Parts that models are put together from: mixers, feed-forwards, norms, position encodings, blocks."""
+from .base import Part, StepContext, make_part, register_part, registered_parts
+from .linear import Embedding, Linear, OutputHead
+from .norms import LayerNorm
+from .positions import AlibiPositions, NoPositions, RotaryPositions, alibi_slopes
+from .attention import AttentionMixer
+from .feedforward import DenseFeedForward
+from .blocks import ParallelBlock, SequentialBlock
+
+__all__ = ["Part", "StepContext", "make_part", "register_part", "registered_parts", "Embedding", "Linear",
+           "OutputHead", "LayerNorm", "AlibiPositions", "NoPositions", "RotaryPositions", "alibi_slopes",
+           "AttentionMixer", "DenseFeedForward", "ParallelBlock", "SequentialBlock"]

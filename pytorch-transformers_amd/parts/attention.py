@@ -1,0 +1,56 @@
+"""Attention as a token mixer: fused projection, heads, positions, cache, scores, output projection.
+
+Follows ``FalconAttention.forward``
+(src/transformers/models/falcon/modeling_falcon.py:326-458) on its default
+branch (``scaled_dot_product_attention``, :371-386 and :407-422), with these
+differences of layout, none of value: tokens of all sequences lie end to end
+instead of in a padded batch; keys and values are kept once per KV head (the
+reference broadcasts them to every query head before caching, :286-289); the
+causal mask is implied by each token's position instead of being a tensor.
+"""
+from __future__ import annotations
+
+import math
+from typing import List, Optional, Sequence
+
+import torch
+
+from .. import ops
+from .base import Part, StepContext, register_part
+from .linear import Linear
+
+
+class AttentionMixer(Part):
+    def __init__(self, name: str, hidden_size: int, num_heads: int, kv_heads: int, head_dim: int, qkv_layout: str,
+                 bias: bool, positions: Part, qkv_name: str = "query_key_value", out_name: str = "dense"):
+        if num_heads % kv_heads:
+            raise ValueError(f"heads ({num_heads}) must be a multiple of kv heads ({kv_heads})")
+        if qkv_layout not in ops.QKV_LAYOUT_CODES:
+            raise ValueError(f"unknown qkv layout {qkv_layout!r}")
+        self.name = name
+        self.hidden_size = hidden_size
+        self.num_heads = num_heads
+        self.kv_heads = kv_heads
+        self.head_dim = head_dim
+        self.qkv_layout = qkv_layout
+        self.positions = positions
+        self.scale = 1.0 / math.sqrt(head_dim)  # modeling_falcon.py:250
+        self.qkv = Linear(f"{name}.{qkv_name}", hidden_size, (num_heads + 2 * kv_heads) * head_dim, bias)
+        self.out = Linear(f"{name}.{out_name}", num_heads * head_dim, hidden_size, bias)
+
+    def children(self) -> Sequence[Part]:
+        return (self.qkv, self.out, self.positions)
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, call, residual: Optional[torch.Tensor] = None):
+        k_pool, v_pool = ctx.cache.kv_layer(call.cache_group, call.cache_layer)
+        table = ctx.block_tables[call.cache_group]
+        fused = self.qkv(x, apply_bias=False)
+        inv_freq, cs_scale = self.positions.rotation()
+        q = ops.qkv_rope_cache(fused, self.qkv.bias, inv_freq, cs_scale, ctx.token_pos, ctx.token_seq, table,
+                               k_pool, v_pool, self.num_heads, self.kv_heads, self.head_dim, self.qkv_layout,
+                               write_cache=call.write_cache)
+        o = ops.attention(q, k_pool, v_pool, table, ctx, self.positions.score_bias(), self.scale)
+        return self.out(o, add1=residual)
+
+
+register_part("mixer", "attention", AttentionMixer)

@@ -1,0 +1,112 @@
+"""Interfaces of the parts a model is put together from, and the table of part kinds.
+
+A part is built from sizes and constants only; it never sees a model
+configuration and does not know which model it is in.  Every part
+
+* lists the tensors it needs (``tensor_specs``) under the names the weight file
+  uses, and takes them from a dict by those names (``load``);
+* works on activations ``[tokens, features]`` of all sequences of a step laid
+  end to end; which token belongs to which sequence, and where it stands, is in
+  the :class:`StepContext`.
+
+Kinds and their ``forward``:
+
+=============  ==================================================================
+mixer          ``forward(x, ctx, call, residual=None) -> [tokens, hidden]``; reads
+               and writes the cache layer that ``call`` names (keys and values, or
+               a state table); ``residual`` is added to the result if given
+feed_forward   ``forward(x, ctx, add1=None, add2=None) -> [tokens, hidden]``
+norm           ``forward(x, rows=None) -> [tokens, hidden]`` (``rows``: int32
+               indices of the rows to take); ``forward_pair(x, other)`` may fuse
+               two norms of the same input
+positions      ``rotation() -> (inv_freq or None, scale)`` for queries and keys,
+               ``score_bias() -> per-head slopes or None`` for attention scores
+block          ``forward(x, ctx, call) -> x``: the arrangement of the above
+=============  ==================================================================
+"""
+from __future__ import annotations
+
+import dataclasses
+from typing import Any, Dict, List, Optional, Sequence
+
+import torch
+
+from ..engine.spec import TensorSpec
+
+_KINDS = ("mixer", "feed_forward", "norm", "positions", "block")
+_TABLE: Dict[str, Dict[str, type]] = {k: {} for k in _KINDS}
+
+
+def register_part(kind: str, name: str, cls: type, *, exist_ok: bool = False) -> type:
+    if kind not in _TABLE:
+        raise ValueError(f"unknown part kind {kind!r}; kinds: {_KINDS}")
+    if not exist_ok and name in _TABLE[kind]:
+        raise ValueError(f"{kind} {name!r} is already registered")
+    _TABLE[kind][name] = cls
+    return cls
+
+
+def make_part(kind: str, name: str, **params):
+    try:
+        cls = _TABLE[kind][name]
+    except KeyError:
+        raise ValueError(f"no {kind} named {name!r}; registered: {sorted(_TABLE.get(kind, {}))}") from None
+    return cls(**params)
+
+
+def registered_parts(kind: str) -> List[str]:
+    return sorted(_TABLE[kind])
+
+
+class Part:
+    """Base of all parts: tensors by name."""
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return []
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        """Take this part's tensors out of ``tensors`` (already on the device, in device types)."""
+
+    def children(self) -> Sequence["Part"]:
+        return ()
+
+    def all_tensor_specs(self) -> List[TensorSpec]:
+        out = list(self.tensor_specs())
+        for c in self.children():
+            out.extend(c.all_tensor_specs())
+        return out
+
+    def load_all(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.load(tensors)
+        for c in self.children():
+            c.load_all(tensors)
+
+
+@dataclasses.dataclass
+class StepContext:
+    """What one step's tokens are: built once per step by the engine, read by every part."""
+
+    dtype: torch.dtype
+    device: torch.device
+    n_seqs: int
+    n_tokens: int
+    #: per token: index of its sequence in this step, and its position in that sequence
+    token_seq: torch.Tensor
+    token_pos: torch.Tensor
+    #: per sequence: first token's offset in the step (n_seqs + 1 entries), cached length before the step
+    cu_tokens: torch.Tensor
+    seq_start: torch.Tensor
+    #: per sequence: its slot (row of state tables)
+    seq_slot: torch.Tensor
+    #: per paged cache group: [n_seqs, pages] page ids
+    block_tables: Dict[str, torch.Tensor]
+    cache: Any
+    #: host copies, for launch geometry
+    slots: List[int]
+    new_tokens: List[int]
+    starts: List[int]
+    #: True if every sequence brings exactly one token
+    is_decode: bool = False
+    #: upper bound of any sequence's length after this step, used to size launches
+    max_len: int = 0
+    extras: Dict[str, Any] = dataclasses.field(default_factory=dict)

@@ -1,0 +1,31 @@
+"""Feed-forward parts.  ``DenseFeedForward``: ``down(act(up(x)))``, no gate, no experts
+(``FalconMLP`` src/transformers/models/falcon/modeling_falcon.py:565-578; ``gelu`` is the exact erf
+form, src/transformers/activations.py:59-78)."""
+from __future__ import annotations
+
+from typing import Sequence
+
+import torch
+
+from .base import Part, StepContext, register_part
+from .linear import Linear
+
+
+class DenseFeedForward(Part):
+    def __init__(self, name: str, hidden_size: int, ffn_size: int, bias: bool, activation: str = "gelu",
+                 up_name: str = "dense_h_to_4h", down_name: str = "dense_4h_to_h"):
+        if activation != "gelu":
+            raise ValueError(f"activation {activation!r} is not built; only 'gelu'")
+        self.name = name
+        self.activation = activation
+        self.up = Linear(f"{name}.{up_name}", hidden_size, ffn_size, bias)
+        self.down = Linear(f"{name}.{down_name}", ffn_size, hidden_size, bias)
+
+    def children(self) -> Sequence[Part]:
+        return (self.up, self.down)
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, add1=None, add2=None) -> torch.Tensor:
+        return self.down(self.up(x, act=self.activation), add1=add1, add2=add2)
+
+
+register_part("feed_forward", "dense", DenseFeedForward)

@@ -1,0 +1,94 @@
+"""Linear layers, the embedding table and the output head.
+
+``y = x @ W.T``, then ``+ b`` as a second operation whose result is rounded to the
+storage type, as the reference does on purpose
+(src/transformers/models/falcon/modeling_falcon.py:64-72).  In 32-bit the whole
+layer, with activation and residual additions, is one hand-written kernel with a
+fixed summation order.  In bfloat16 the matrix product is the vendor library's
+(as the reference's is torch's), followed by one fused kernel for bias,
+activation and additions.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from .. import ops
+from ..engine.spec import INIT_NORMAL, INIT_ZERO_NOISE, MATRIX, VECTOR, TensorSpec
+from .base import Part
+
+
+class Linear(Part):
+    def __init__(self, name: str, in_features: int, out_features: int, bias: bool):
+        self.name = name
+        self.in_features = in_features
+        self.out_features = out_features
+        self.has_bias = bias
+        self.weight: Optional[torch.Tensor] = None
+        self.bias: Optional[torch.Tensor] = None
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        specs = [TensorSpec(self.name + ".weight", (self.out_features, self.in_features), MATRIX, INIT_NORMAL)]
+        if self.has_bias:
+            specs.append(TensorSpec(self.name + ".bias", (self.out_features,), VECTOR, INIT_ZERO_NOISE))
+        return specs
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.weight = tensors[self.name + ".weight"]
+        self.bias = tensors[self.name + ".bias"] if self.has_bias else None
+
+    def __call__(self, x: torch.Tensor, *, act: Optional[str] = None, add1=None, add2=None,
+                 apply_bias: bool = True) -> torch.Tensor:
+        """``act(x @ W.T + b) + add1 + add2``; with ``apply_bias=False`` the caller adds the bias itself."""
+        bias = self.bias if apply_bias else None
+        if x.dtype == torch.float32:
+            return ops.gemm_f32(x, self.weight, bias, act, add1, add2)
+        y = torch.mm(x, self.weight.t())
+        if bias is not None or act is not None or add1 is not None or add2 is not None:
+            ops.epilogue_(y, bias, act, add1, add2)
+        return y
+
+
+class Embedding(Part):
+    """``h[t] = E[id_t]``, no scaling (src/transformers/models/falcon/modeling_falcon.py:835, :895-896)."""
+
+    def __init__(self, name: str, vocab_size: int, hidden_size: int):
+        self.name = name
+        self.vocab_size = vocab_size
+        self.hidden_size = hidden_size
+        self.weight: Optional[torch.Tensor] = None
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [TensorSpec(self.name + ".weight", (self.vocab_size, self.hidden_size), MATRIX, INIT_NORMAL)]
+
+    def load(self, tensors) -> None:
+        self.weight = tensors[self.name + ".weight"]
+
+    def forward(self, ids: torch.Tensor) -> torch.Tensor:
+        return ops.embed(self.weight, ids)
+
+
+class OutputHead(Part):
+    """``logits = h @ W.T`` in 32-bit, no bias; ``W`` is the embedding table when tied
+    (src/transformers/models/falcon/modeling_falcon.py:1163-1168, :1230; the reference casts the
+    rows it samples from to 32-bit, src/transformers/generation/utils.py:3247)."""
+
+    def __init__(self, name: str, vocab_size: int, hidden_size: int, tied_to: Optional[str]):
+        self.name = name
+        self.vocab_size = vocab_size
+        self.hidden_size = hidden_size
+        self.tied_to = tied_to
+        self.weight: Optional[torch.Tensor] = None
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [TensorSpec(self.name + ".weight", (self.vocab_size, self.hidden_size), MATRIX, INIT_NORMAL,
+                           tied_to=self.tied_to)]
+
+    def load(self, tensors) -> None:
+        self.weight = tensors[self.name + ".weight"]
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        if h.dtype == torch.float32:
+            return ops.gemm_f32(h, self.weight)
+        return torch.mm(h, self.weight.t(), out_dtype=torch.float32)

@@ -1,0 +1,40 @@
+"""Norms.  ``LayerNorm``: mean and biased variance over the features, affine always
+(``torch.nn.LayerNorm`` as built at src/transformers/models/falcon/modeling_falcon.py:603-612, :843)."""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from .. import ops
+from ..engine.spec import INIT_ONE_NOISE, INIT_ZERO_NOISE, VECTOR, TensorSpec
+from .base import Part, register_part
+
+
+class LayerNorm(Part):
+    def __init__(self, name: str, hidden_size: int, eps: float):
+        self.name = name
+        self.hidden_size = hidden_size
+        self.eps = float(eps)
+        self.weight: Optional[torch.Tensor] = None
+        self.bias: Optional[torch.Tensor] = None
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [TensorSpec(self.name + ".weight", (self.hidden_size,), VECTOR, INIT_ONE_NOISE),
+                TensorSpec(self.name + ".bias", (self.hidden_size,), VECTOR, INIT_ZERO_NOISE)]
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.weight = tensors[self.name + ".weight"]
+        self.bias = tensors[self.name + ".bias"]
+
+    def forward(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        return ops.layernorm(x, self.weight, self.bias, self.eps, rows=rows)
+
+    def forward_pair(self, x: torch.Tensor, other: "Part"):
+        """``(self(x), other(x))``; one pass over x when both are LayerNorms with one eps."""
+        if isinstance(other, LayerNorm) and other.eps == self.eps:
+            return ops.layernorm(x, self.weight, self.bias, self.eps, w2=other.weight, b2=other.bias)
+        return self.forward(x), other.forward(x)
+
+
+register_part("norm", "layernorm", LayerNorm)

@@ -1,0 +1,68 @@
+"""Choosing the next token of every sequence of a step, on the GPU.
+
+One kernel per step applies the processors that the generation options switch on, in the
+reference's order (src/transformers/generation/utils.py:926-1097), and takes the argmax or a draw
+(:3274-3279).  Draws come from a counter-based generator keyed by (seed, sequence id, step), not
+from a global generator as in the reference (:3277), so a sequence's tokens do not depend on which
+other sequences share its batch.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from .. import ops
+from ..config.generation import GenerationConfig
+
+
+class Sampler:
+    def __init__(self, config: GenerationConfig, vocab_size: int, device):
+        self.config = config
+        self.vocab_size = vocab_size
+        self.device = torch.device(device)
+        self.eos_ids = [e for e in config.eos_token_ids]
+        self._eos_dev = (torch.tensor(self.eos_ids, dtype=torch.int32, device=self.device)
+                         if self.eos_ids else None)
+        c = config
+        self.do_sample = bool(c.do_sample)
+        self.temperature = float(c.temperature) if (c.do_sample and c.temperature is not None) else 1.0
+        self.top_k = int(c.top_k) if (c.do_sample and c.top_k) else 0
+        self.top_p = float(c.top_p) if (c.do_sample and c.top_p is not None) else 1.0
+        self.min_p = float(c.min_p) if (c.do_sample and c.min_p is not None) else 0.0
+        self.penalty = float(c.repetition_penalty) if c.repetition_penalty is not None else 1.0
+
+    def sample(self, logits: torch.Tensor, *, rng_seq: Sequence[int], rng_step: Sequence[int],
+               histories: Optional[Sequence[Sequence[int]]] = None, suppress_eos: Optional[Sequence[bool]] = None,
+               uniforms: Optional[Sequence[float]] = None) -> Tuple[List[int], torch.Tensor]:
+        """Tokens for the rows of ``logits`` and the processed scores ``[rows, vocab]``."""
+        R = logits.shape[0]
+        use_hist = self.penalty != 1.0 and histories is not None
+        pieces = [np.asarray(rng_seq, dtype=np.int32), np.asarray(rng_step, dtype=np.int32),
+                  np.asarray([1 if s else 0 for s in (suppress_eos or [False] * R)], dtype=np.int32)]
+        if use_hist:
+            off = np.zeros(R + 1, dtype=np.int32)
+            off[1:] = np.cumsum([len(h) for h in histories])
+            flat = (np.concatenate([np.asarray(h, dtype=np.int32) for h in histories])
+                    if off[-1] else np.zeros(0, dtype=np.int32))
+            pieces += [off, flat]
+        dev = torch.from_numpy(np.concatenate(pieces)).to(self.device)
+        views = torch.split(dev, [int(p.shape[0]) for p in pieces])
+        u = (torch.tensor(list(uniforms), dtype=torch.float32, device=self.device) if uniforms is not None else None)
+        tokens, scores = ops.sample(
+            logits, do_sample=self.do_sample, temperature=self.temperature, top_k=self.top_k, top_p=self.top_p,
+            min_p=self.min_p, penalty=self.penalty, hist=views[4] if use_hist else None,
+            hist_off=views[3] if use_hist else None, eos=self._eos_dev,
+            suppress=views[2] if (self._eos_dev is not None and suppress_eos is not None and any(suppress_eos)) else None,
+            remove_invalid=self.config.remove_invalid_values, renorm=self.config.renormalize_logits,
+            seed=self.config.seed, rng_seq=views[0], rng_step=views[1], uniforms=u)
+        return tokens.tolist(), scores
+
+
+def philox_uniform(seed: int, seq: int, step: int) -> float:
+    """The uniform number in [0, 1) that the kernel draws for (seed, sequence id, step)."""
+    lib = ops.load_library()
+    lib.pta_philox_uniform.restype = ctypes.c_float
+    return float(lib.pta_philox_uniform(ctypes.c_uint64(seed & (2 ** 64 - 1)), ctypes.c_uint32(seq), ctypes.c_uint32(step)))

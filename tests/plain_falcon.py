@@ -1,0 +1,326 @@
+"""A plain, slow Falcon: whole sequences, no cache, one function per part.
+
+Written from the reference's formulas (each function cites file:line under
+/root/reference); it imports nothing from the engine, reads ``config.json`` as
+a dict and the weights with safetensors' own loader.  Arithmetic is float64 by
+default, so what the 32-bit engine is compared with is closer to exact than the
+engine itself; the places where the reference rounds on purpose (ALiBi's
+bfloat16 slopes) are reproduced.
+
+A sequence is a list of token ids; every function works on one sequence.
+"""
+from __future__ import annotations
+
+import json
+import math
+import os
+from typing import Dict, List, Optional, Sequence
+
+import torch
+
+DT = torch.float64
+
+
+# --- files -----------------------------------------------------------------
+def read_model(folder: str, dtype=DT):
+    """config.json as a dict, tensors by name (src/transformers/modeling_utils.py:3680-3695, :493-560)."""
+    from safetensors.torch import load_file
+
+    with open(os.path.join(folder, "config.json")) as f:
+        cfg = json.load(f)
+    single = os.path.join(folder, "model.safetensors")
+    if os.path.isfile(single):
+        tensors = load_file(single)
+    else:
+        with open(os.path.join(folder, "model.safetensors.index.json")) as f:
+            wm = json.load(f)["weight_map"]
+        tensors = {}
+        for shard in sorted(set(wm.values())):
+            tensors.update(load_file(os.path.join(folder, shard)))
+    return cfg, {k: v.to(dtype) for k, v in tensors.items()}
+
+
+def cfg_defaults(cfg: dict) -> dict:
+    """Defaults of FalconConfig (src/transformers/models/falcon/configuration_falcon.py:144-200)."""
+    c = dict(vocab_size=65024, hidden_size=4544, num_hidden_layers=32, num_attention_heads=71,
+             num_ln_in_parallel_attn=None, layer_norm_epsilon=1e-5, num_kv_heads=None, alibi=False,
+             new_decoder_architecture=False, multi_query=True, parallel_attn=True, bias=False,
+             rope_theta=10000.0, rope_scaling=None, ffn_hidden_size=None, tie_word_embeddings=True)
+    c.update(cfg)
+    if c["num_kv_heads"] is None:  # :184
+        c["num_kv_heads"] = c["num_attention_heads"]
+    if c["ffn_hidden_size"] is None:  # :195-198
+        c["ffn_hidden_size"] = 4 * c["hidden_size"]
+    if c["num_ln_in_parallel_attn"] is None and c["new_decoder_architecture"]:  # modeling_falcon.py:599-600
+        c["num_ln_in_parallel_attn"] = 2
+    return c
+
+
+# --- parts -------------------------------------------------------------------
+def layer_norm(x, w, b, eps):
+    """torch.nn.LayerNorm over the last axis, biased variance
+    (constructed at src/transformers/models/falcon/modeling_falcon.py:603-612, :843)."""
+    mean = x.mean(-1, keepdim=True)
+    var = ((x - mean) ** 2).mean(-1, keepdim=True)
+    return (x - mean) / torch.sqrt(var + eps) * w + b
+
+
+def gelu(x):
+    """Exact GELU (src/transformers/activations.py:59-78, the non-approximate branch)."""
+    return 0.5 * x * (1.0 + torch.erf(x / math.sqrt(2.0)))
+
+
+def linear(x, w, b=None):
+    """FalconLinear: x @ W.T, then + b (src/transformers/models/falcon/modeling_falcon.py:67-72)."""
+    y = x @ w.T
+    return y if b is None else y + b
+
+
+def rope_inv_freq(head_dim: int, theta: float, factor: float = 1.0):
+    """inv_freq = 1 / theta^(2i/d) in 32-bit (src/transformers/modeling_rope_utils.py:67);
+    linear scaling divides by the factor (:108)."""
+    inv = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.int64).float() / head_dim))
+    return inv / factor if factor != 1.0 else inv
+
+
+def rope_cos_sin(positions, inv_freq, dtype=DT):
+    """angles = position * inv_freq in 32-bit, doubled along the last axis
+    (src/transformers/models/falcon/modeling_falcon.py:155-164)."""
+    freqs = positions.float()[:, None] * inv_freq.float()[None, :]
+    emb = torch.cat((freqs, freqs), dim=-1)
+    return emb.to(dtype).cos(), emb.to(dtype).sin()
+
+
+def rotate_half(x):
+    """(-x2, x1) of the two halves of the last axis (src/transformers/models/falcon/modeling_falcon.py:76-80)."""
+    h = x.shape[-1] // 2
+    return torch.cat((-x[..., h:], x[..., :h]), dim=-1)
+
+
+def apply_rope(x, cos, sin):
+    """x*cos + rotate_half(x)*sin; x is [T, heads, d], cos/sin [T, d]
+    (src/transformers/models/falcon/modeling_falcon.py:104-108)."""
+    return x * cos[:, None, :] + rotate_half(x) * sin[:, None, :]
+
+
+def alibi_slopes(nh: int):
+    """src/transformers/models/falcon/modeling_falcon.py:175-188, in 32-bit."""
+    n2 = 2 ** math.floor(math.log2(nh))
+    base = torch.tensor(2 ** (-(2 ** -(math.log2(n2) - 3))), dtype=torch.float32)
+    slopes = torch.pow(base, torch.arange(1, 1 + n2, dtype=torch.int32))
+    if n2 != nh:
+        extra_base = torch.tensor(2 ** (-(2 ** -(math.log2(2 * n2) - 3))), dtype=torch.float32)
+        rem = min(n2, nh - n2)
+        slopes = torch.cat([slopes, torch.pow(extra_base, torch.arange(1, 1 + 2 * rem, 2, dtype=torch.int32))])
+    return slopes
+
+
+def alibi_bias(nh: int, n_keys: int, head_dim: int, dtype=DT):
+    """[heads, keys]: bf16(slope) * position formed in bfloat16 (:196-198), then / sqrt(d) in the
+    model's type (:1078-1085)."""
+    pos = torch.arange(n_keys, dtype=torch.int64)
+    alibi = alibi_slopes(nh)[:, None].bfloat16() * pos[None, :]  # bfloat16 result, as in the reference
+    return alibi.to(dtype) / math.sqrt(head_dim)
+
+
+def split_heads(fused, c):
+    """[T, Qout] -> q [T, nh, d], k and v [T, nkv, d]
+    (src/transformers/models/falcon/modeling_falcon.py:269-298; the reference then broadcasts k, v
+    to every query head, :286-289, which `attention` does by indexing)."""
+    T = fused.shape[0]
+    nh = c["num_attention_heads"]
+    d = c["hidden_size"] // nh
+    if c["new_decoder_architecture"]:
+        nkv = c["num_kv_heads"]
+        qkv = fused.view(T, nkv, nh // nkv + 2, d)
+        return qkv[:, :, :-2].reshape(T, nh, d), qkv[:, :, -2], qkv[:, :, -1]
+    if not c["multi_query"]:
+        qkv = fused.view(T, nh, 3, d)
+        return qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2]
+    qkv = fused.view(T, nh + 2, d)
+    return qkv[:, :-2], qkv[:, [-2]], qkv[:, [-1]]
+
+
+def attention_scores_softmax(q, k, v, bias=None):
+    """Causal softmax(q k^T / sqrt(d) + bias) v for one sequence; q [T, nh, d], k, v [T, nkv, d]
+    (src/transformers/models/falcon/modeling_falcon.py:371-386 / :407-422 with the mask of :1138-1153:
+    key j is visible to query t iff j <= t)."""
+    T, nh, d = q.shape
+    nkv = k.shape[1]
+    g = nh // nkv
+    out = torch.empty_like(q)
+    mask = torch.full((T, T), float("-inf"), dtype=q.dtype).triu(1)
+    for h in range(nh):
+        s = q[:, h] @ k[:, h // g].T / math.sqrt(d)
+        if bias is not None:
+            s = s + bias[h][None, :]
+        p = torch.softmax(s + mask, dim=-1)
+        out[:, h] = p @ v[:, h // g]
+    return out.reshape(T, nh * d)
+
+
+def self_attention(x, w, prefix, c, positions):
+    """FalconAttention.forward (src/transformers/models/falcon/modeling_falcon.py:326-458)."""
+    nh = c["num_attention_heads"]
+    d = c["hidden_size"] // nh
+    fused = linear(x, w[prefix + "query_key_value.weight"], w.get(prefix + "query_key_value.bias"))
+    q, k, v = split_heads(fused, c)
+    bias = None
+    if c["alibi"]:
+        bias = alibi_bias(nh, x.shape[0], d, x.dtype)
+    else:
+        rs = c.get("rope_scaling")
+        factor = 1.0
+        if rs is not None and rs.get("rope_type", rs.get("type")) == "linear":
+            factor = float(rs["factor"])
+        cos, sin = rope_cos_sin(positions, rope_inv_freq(d, float(c["rope_theta"]), factor), x.dtype)
+        q, k = apply_rope(q, cos, sin), apply_rope(k, cos, sin)
+    o = attention_scores_softmax(q, k, v, bias)
+    return linear(o, w[prefix + "dense.weight"], w.get(prefix + "dense.bias"))
+
+
+def mlp(x, w, prefix):
+    """FalconMLP (src/transformers/models/falcon/modeling_falcon.py:575-578)."""
+    u = linear(x, w[prefix + "dense_h_to_4h.weight"], w.get(prefix + "dense_h_to_4h.bias"))
+    return linear(gelu(u), w[prefix + "dense_4h_to_h.weight"], w.get(prefix + "dense_4h_to_h.bias"))
+
+
+def decoder_layer(x, w, i, c, positions):
+    """FalconDecoderLayer.forward (src/transformers/models/falcon/modeling_falcon.py:614-683)."""
+    p = f"transformer.h.{i}."
+    eps = c["layer_norm_epsilon"]
+    residual = x
+    if c["new_decoder_architecture"] and c["num_ln_in_parallel_attn"] == 2:  # :630-632
+        attn_in = layer_norm(x, w[p + "ln_attn.weight"], w[p + "ln_attn.bias"], eps)
+        mlp_in = layer_norm(x, w[p + "ln_mlp.weight"], w[p + "ln_mlp.bias"], eps)
+    else:  # :634
+        attn_in = layer_norm(x, w[p + "input_layernorm.weight"], w[p + "input_layernorm.bias"], eps)
+        mlp_in = None
+    attn = self_attention(attn_in, w, p + "self_attention.", c, positions)
+    if not c["new_decoder_architecture"]:
+        if c["parallel_attn"]:  # :649-650
+            mlp_in = attn_in
+        else:  # :652-659
+            residual = residual + attn
+            mlp_in = layer_norm(residual, w[p + "post_attention_layernorm.weight"],
+                                w[p + "post_attention_layernorm.bias"], eps)
+    if c["new_decoder_architecture"] and c["parallel_attn"] and c["num_ln_in_parallel_attn"] == 1:  # :661-666
+        mlp_in = attn_in
+    out = mlp(mlp_in, w, p + "mlp.")
+    if c["new_decoder_architecture"] or c["parallel_attn"]:  # :673-674
+        out = out + attn
+    return residual + out  # :676
+
+
+def forward(cfg: dict, w: Dict[str, torch.Tensor], token_ids: Sequence[int]):
+    """Logits [T, V] of one whole sequence (FalconModel.forward :864-1011, head :1230)."""
+    c = cfg_defaults(cfg)
+    ids = torch.as_tensor(list(token_ids), dtype=torch.long)
+    x = w["transformer.word_embeddings.weight"][ids]  # :895-896
+    positions = torch.arange(len(ids))
+    for i in range(c["num_hidden_layers"]):
+        x = decoder_layer(x, w, i, c, positions)
+    x = layer_norm(x, w["transformer.ln_f.weight"], w["transformer.ln_f.bias"], c["layer_norm_epsilon"])  # :992
+    head = w["lm_head.weight"] if "lm_head.weight" in w else w["transformer.word_embeddings.weight"]  # tied :1163
+    return x @ head.T
+
+
+# --- generation ---------------------------------------------------------------
+def repetition_penalty(scores, seen_ids, penalty):
+    """src/transformers/generation/logits_process.py:337-343."""
+    out = scores.clone()
+    idx = torch.as_tensor(sorted(set(int(t) for t in seen_ids)), dtype=torch.long)
+    s = scores[idx]
+    out[idx] = torch.where(s < 0, s * penalty, s / penalty)
+    return out
+
+
+def suppress(scores, ids):
+    """EOS scores to -inf while the minimum length is not reached (logits_process.py:144-151, :214-223)."""
+    out = scores.clone()
+    out[torch.as_tensor(list(ids), dtype=torch.long)] = float("-inf")
+    return out
+
+
+def temperature(scores, t):
+    """logits_process.py:286-289."""
+    return scores / t
+
+
+def top_k(scores, k, min_tokens_to_keep=1):
+    """logits_process.py:505-518."""
+    k = min(max(k, min_tokens_to_keep), scores.shape[-1])
+    kth = torch.topk(scores, k)[0][-1]
+    return scores.masked_fill(scores < kth, float("-inf"))
+
+
+def top_p(scores, p, min_tokens_to_keep=1):
+    """logits_process.py:452-465."""
+    sorted_logits, sorted_idx = torch.sort(scores, descending=False, stable=True)
+    cum = sorted_logits.softmax(-1).cumsum(-1)
+    remove = cum <= (1 - p)
+    remove[-min_tokens_to_keep:] = False
+    mask = torch.zeros_like(remove)
+    mask[sorted_idx] = remove
+    return scores.masked_fill(mask, float("-inf"))
+
+
+def min_p(scores, mp, min_tokens_to_keep=1):
+    """logits_process.py:578-595."""
+    probs = torch.softmax(scores, -1)
+    remove = probs < mp * probs.max()
+    order = torch.argsort(scores, descending=True)
+    r = remove[order]
+    r[:min_tokens_to_keep] = False
+    mask = torch.zeros_like(remove)
+    mask[order] = r
+    return scores.masked_fill(mask, float("-inf"))
+
+
+def process(scores, history, *, do_sample, temperature_=1.0, top_k_=0, top_p_=1.0, min_p_=None,
+            repetition_penalty_=1.0, suppress_ids=()):
+    """Processors in the order the reference builds them (src/transformers/generation/utils.py:926-1097):
+    repetition penalty, minimum length, then (sampling only) temperature, top-k, top-p, min-p."""
+    s = scores
+    if repetition_penalty_ is not None and repetition_penalty_ != 1.0:
+        s = repetition_penalty(s, history, repetition_penalty_)
+    if suppress_ids:
+        s = suppress(s, suppress_ids)
+    if do_sample:
+        if temperature_ is not None and temperature_ != 1.0:
+            s = temperature(s, temperature_)
+        if top_k_:
+            s = top_k(s, top_k_)
+        if top_p_ is not None and top_p_ < 1.0:
+            s = top_p(s, top_p_)
+        if min_p_ is not None:
+            s = min_p(s, min_p_)
+    return s
+
+
+def pick(scores, u: Optional[float]):
+    """argmax, or the token whose interval of the cumulative distribution holds ``u``
+    (the reference draws with torch.multinomial, src/transformers/generation/utils.py:3274-3279;
+    a given uniform number makes the draw repeatable)."""
+    if u is None:
+        return int(torch.argmax(scores))
+    cdf = torch.softmax(scores.double(), -1).cumsum(-1)
+    return int(min(torch.searchsorted(cdf, torch.tensor(u, dtype=torch.float64), right=True), scores.shape[-1] - 1))
+
+
+def generate(cfg, w, prompt: Sequence[int], max_new_tokens: int, *, eos_ids=(), min_new_tokens=0,
+             uniforms: Optional[Sequence[float]] = None, **proc) -> List[int]:
+    """One sequence, recomputed whole at every step (no cache); returns the new tokens, EOS included
+    (loop of src/transformers/generation/utils.py:3220-3296, stop test stopping_criteria.py:446-467)."""
+    seq = list(prompt)
+    new = []
+    for step in range(max_new_tokens):
+        logits = forward(cfg, w, seq)[-1].float()
+        s = process(logits, seq, do_sample=uniforms is not None,
+                    suppress_ids=tuple(eos_ids) if len(new) < min_new_tokens else (), **proc)
+        tok = pick(s, None if uniforms is None else uniforms[step])
+        seq.append(tok)
+        new.append(tok)
+        if tok in eos_ids:
+            break
+    return new

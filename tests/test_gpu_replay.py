@@ -1,0 +1,127 @@
+"""Engine against the plain implementation, for every way of cutting the work (GPU)."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import helpers
+from helpers import REL_BF16, REL_F32
+from tiny import TINY, write_model
+
+pytestmark = pytest.mark.gpu
+
+LENGTHS = {"A": [5, 11, 17, 40, 70, 33], "B": [1, 7, 20, 33, 65, 129], "C": [64, 3, 47, 90, 128, 66],
+           "D": [37, 12, 80, 5, 64, 100], "E": [9, 50, 130, 3, 64, 77]}
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    root = str(tmp_path_factory.mktemp("models"))
+    return {name: write_model(name, root) for name in TINY}
+
+
+@pytest.fixture(scope="module")
+def plain_cache():
+    return {}
+
+
+def _plain(folders, plain_cache, name):
+    if name not in plain_cache:
+        reqs = helpers.make_requests(TINY[name]["vocab_size"], LENGTHS[name], seed=100 + ord(name))
+        plain_cache[name] = (reqs, helpers.plain_logits(folders[name], reqs))
+    return plain_cache[name]
+
+
+def _replayer(folder, dtype, max_tokens=2048):
+    from pytorch_transformers_amd import AutoModelForCausalLM
+    from pytorch_transformers_amd.engine.replay import Replayer
+
+    model = AutoModelForCausalLM.from_pretrained(folder, dtype=dtype)
+    return Replayer(model, max_tokens)
+
+
+@pytest.mark.parametrize("dtype,rel", [("float32", REL_F32), ("bfloat16", REL_BF16)])
+@pytest.mark.parametrize("name", sorted(TINY))
+def test_schedules_match_plain(folders, plain_cache, name, dtype, rel):
+    """Whole / last 32 one by one / unequal batches with slot reuse: all equal the plain logits."""
+    reqs, want = _plain(folders, plain_cache, name)
+    rp = _replayer(folders[name], dtype)
+    results = {}
+    for sched_name, records in (("whole", helpers.schedule_whole(reqs)),
+                                ("tail32", helpers.schedule_tail(reqs, 32)),
+                                ("batches", helpers.schedule_batches(reqs, 4)),
+                                ("batches-again", helpers.schedule_batches(reqs, 3, decode=(20, 2, 7)))):
+        got = helpers.run_schedule(rp, records)
+        assert not rp.slots and not rp.cache.live_slots(), "slots left behind"
+        assert rp.cache.free_pages() == rp.cache.num_pages, "pages left behind"
+        for rid in reqs:
+            helpers.assert_close(got[rid], want[rid], rel, f"{name} {dtype} {sched_name} {rid} (len {len(reqs[rid])})")
+        results[sched_name] = got
+    if dtype == "float32":
+        # fixed summation orders: how the tokens were cut and batched changes no bit
+        for sched_name in ("tail32", "batches", "batches-again"):
+            for rid in reqs:
+                assert torch.equal(results[sched_name][rid], results["whole"][rid]), \
+                    f"{name} float32: {sched_name} differs from whole for {rid}"
+
+
+@pytest.mark.parametrize("dtype,rel", [("float32", REL_F32), ("bfloat16", REL_BF16)])
+@pytest.mark.parametrize("name", ["C", "E"])
+def test_long_decoding(folders, name, dtype, rel):
+    """A short prompt, then hundreds of tokens one by one (past several pages; ALiBi past position 256)."""
+    n = 330
+    reqs = helpers.make_requests(TINY[name]["vocab_size"], [n], seed=7)
+    want = helpers.plain_logits(folders[name], reqs)
+    rp = _replayer(folders[name], dtype, max_tokens=512)
+    got = helpers.run_schedule(rp, helpers.schedule_tail(reqs, n - 3))
+    helpers.assert_close(got["r0"], want["r0"], rel, f"{name} {dtype} long decoding")
+
+
+@pytest.mark.parametrize("dtype,rel", [("float32", REL_F32), ("bfloat16", REL_BF16)])
+def test_first_tokens(folders, dtype, rel):
+    """The first tokens of a sequence, fed one at a time from an empty slot."""
+    reqs = helpers.make_requests(TINY["A"]["vocab_size"], [6], seed=11)
+    want = helpers.plain_logits(folders["A"], reqs)
+    rp = _replayer(folders["A"], dtype, max_tokens=64)
+    got = helpers.run_schedule(rp, helpers.schedule_tail(reqs, 100))
+    helpers.assert_close(got["r0"], want["r0"], rel, f"A {dtype} first tokens")
+
+
+def test_cache_full_is_an_error(folders):
+    from pytorch_transformers_amd.cache import CacheFull
+
+    rp = _replayer(folders["A"], "float32", max_tokens=128)
+    rp.run({"step": 0, "entries": [{"id": "a", "tokens": list(range(100)), "want": []}], "end": []})
+    with pytest.raises(CacheFull):
+        rp.run({"step": 1, "entries": [{"id": "b", "tokens": list(range(100)), "want": []}], "end": []})
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(folders, tmp_path, dtype):
+    """bin/trace_run as a program: stdin records, files of logits, 'done' lines."""
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    reqs = helpers.make_requests(TINY["A"]["vocab_size"], [19, 40], seed=5)
+    records = helpers.schedule_batches(reqs, 2, decode=(4, 9))
+    out = tmp_path / "out"
+    p = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folders["A"], "--dtype", dtype,
+                        "--out", str(out), "--max-tokens", "128"],
+                       input="".join(json.dumps(r) + "\n" for r in records), capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert p.stdout.split("\n")[:-1] == [f"done {r['step']}" for r in records]
+    want = helpers.plain_logits(folders["A"], reqs)
+    V = TINY["A"]["vocab_size"]
+    fed = {rid: 0 for rid in reqs}
+    for r in records:
+        arr = np.fromfile(out / f"{r['step']}.f32", dtype="<f4").reshape(-1, V)
+        row = 0
+        for e in r["entries"]:
+            for pl in e["want"]:
+                helpers.assert_close(torch.from_numpy(arr[row]), want[e["id"]][fed[e["id"]] + pl],
+                                     REL_F32 if dtype == "float32" else REL_BF16, f"trace_run step {r['step']}")
+                row += 1
+            fed[e["id"]] += len(e["tokens"])
+        assert row == arr.shape[0]

@@ -1,0 +1,45 @@
+"""Tiny Falcon configurations for tests.  Together they differ in every size and option:
+head counts and groups, head sizes, widths and vocabularies that are no power of two, number of
+layers, eps, the three fused-QKV row orders, the three norm arrangements, bias, rotary (two
+thetas, linear scaling) and ALiBi (power-of-two and other head counts), tied and untied heads."""
+import os
+
+TINY = {
+    # new architecture, grouped QKV, two norms, rotary
+    "A": dict(model_type="falcon", num_hidden_layers=2, hidden_size=64, num_attention_heads=4, num_kv_heads=2,
+              ffn_hidden_size=256, vocab_size=512, rope_theta=10000.0, max_position_embeddings=128,
+              layer_norm_epsilon=1e-5, new_decoder_architecture=True, parallel_attn=True,
+              num_ln_in_parallel_attn=2, bias=False, alibi=False, tie_word_embeddings=True, initializer_range=0.02),
+    # RW style: per-head q,k,v rows, sequential norms, bias, ALiBi with 6 heads (not a power of two)
+    "B": dict(model_type="falcon", num_hidden_layers=3, hidden_size=144, num_attention_heads=6,
+              ffn_hidden_size=576, vocab_size=1000, max_position_embeddings=256, layer_norm_epsilon=1e-6,
+              new_decoder_architecture=False, multi_query=False, parallel_attn=False, bias=True, alibi=True,
+              tie_word_embeddings=True, initializer_range=0.02),
+    # 7B style: one KV head at the tail, one norm, 7 heads
+    "C": dict(model_type="falcon", num_hidden_layers=2, hidden_size=112, num_attention_heads=7,
+              ffn_hidden_size=320, vocab_size=777, rope_theta=10000.0, max_position_embeddings=512,
+              layer_norm_epsilon=1e-5, new_decoder_architecture=False, multi_query=True, parallel_attn=True,
+              bias=False, alibi=False, tie_word_embeddings=True, initializer_range=0.02),
+    # 11B style: new architecture with one norm, wide heads, large theta, untied head, linear rope scaling
+    "D": dict(model_type="falcon", num_hidden_layers=2, hidden_size=256, num_attention_heads=2, num_kv_heads=1,
+              ffn_hidden_size=384, vocab_size=300, rope_theta=500042.0, max_position_embeddings=8192,
+              layer_norm_epsilon=1e-5, new_decoder_architecture=True, parallel_attn=True,
+              num_ln_in_parallel_attn=1, bias=True, alibi=False, tie_word_embeddings=False,
+              rope_scaling={"rope_type": "linear", "factor": 2.0}, initializer_range=0.02),
+    # ALiBi with 20 heads: slopes that bfloat16 rounds, and (in long tests) positions past 256
+    "E": dict(model_type="falcon", num_hidden_layers=1, hidden_size=320, num_attention_heads=20,
+              ffn_hidden_size=160, vocab_size=211, max_position_embeddings=1024, layer_norm_epsilon=1e-5,
+              new_decoder_architecture=False, multi_query=False, parallel_attn=True, bias=False, alibi=True,
+              tie_word_embeddings=True, initializer_range=0.02),
+}
+
+SEEDS = {"A": 0, "B": 1, "C": 2, "D": 3, "E": 4}
+
+
+def write_model(name: str, folder: str, noise: float = 0.1) -> str:
+    """Write tiny model ``name`` with the framework's random-weights mode; returns the folder."""
+    from pytorch_transformers_amd.config import AutoConfig
+    from pytorch_transformers_amd.weights import write_random_model
+
+    cfg = AutoConfig.from_dict(TINY[name])
+    return write_random_model(os.path.join(folder, name), cfg, SEEDS[name], noise=noise)
