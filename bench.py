@@ -1,0 +1,170 @@
+"""Decode and prefill throughput at Falcon-7B layer sizes with random weights, on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one decode step of the batch (model step from the cache plus the greedy choice of the
+next token, fed back).  The default run: batch 8, prompts of 1,024 synthetic token ids, decoding
+towards a context of 2,048.  One JSON line is printed: decode tokens a second as ``value``, the
+prefill of 2,048 tokens under ``prefill``, the decode step's HBM roofline under ``roofline`` and
+decode at batch 1 and 64 under ``points``.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X, published
+PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}  # dense MFMA, published
+
+
+def falcon7b_config(layers):
+    from pytorch_transformers_amd import FalconConfig
+
+    # configs[2] of BASELINE.json: Falcon-7B layer sizes
+    return FalconConfig(vocab_size=65024, hidden_size=4544, num_hidden_layers=layers, num_attention_heads=71,
+                        multi_query=True, new_decoder_architecture=False, parallel_attn=True, bias=False, alibi=False,
+                        ffn_hidden_size=18176, rope_theta=10000.0, layer_norm_epsilon=1e-5,
+                        max_position_embeddings=2048, tie_word_embeddings=True)
+
+
+def weight_bytes(cfg, elem):
+    H, F, Q = cfg.hidden_size, cfg.ffn_hidden_size, cfg.qkv_out_dim
+    per_layer = (Q * H + H * H + 2 * F * H) * elem
+    return cfg.num_hidden_layers * per_layer + cfg.vocab_size * H * elem
+
+
+def kv_bytes_per_token(cfg, elem):
+    return cfg.num_hidden_layers * 2 * cfg.kv_heads * cfg.head_dim * elem
+
+
+def prefill_flops(cfg, T):
+    H, F, Q = cfg.hidden_size, cfg.ffn_hidden_size, cfg.qkv_out_dim
+    linear = 2.0 * T * (Q * H + H * H + 2 * F * H) * cfg.num_hidden_layers
+    attn = 2.0 * cfg.head_dim * cfg.num_attention_heads * T * (T + 1) * cfg.num_hidden_layers
+    head = 2.0 * cfg.vocab_size * H
+    return linear + attn + head
+
+
+def run_decode(model, sampler_cls, gen_cfg, batch, prompt_len, steps, warmup, seed=0):
+    """Prefill ``batch`` prompts, then time ``steps`` decode steps; returns (seconds, mean context)."""
+    import torch
+
+    g = torch.Generator().manual_seed(seed)
+    prompts = torch.randint(0, model.vocab_size, (batch, prompt_len), generator=g).tolist()
+    total = prompt_len + warmup + steps + 1
+    cache = model.new_cache(batch * ((total + 63) // 64 * 64), max_slots=batch)
+    sampler = sampler_cls(gen_cfg, model.vocab_size, model.device)
+    slots = [cache.alloc() for _ in range(batch)]
+    logits = model.step(cache, slots, prompts, "last")
+    rng = list(range(batch))
+    tokens, _ = sampler.sample(logits, rng_seq=rng, rng_step=[0] * batch)
+
+    def one(k):
+        nonlocal tokens
+        lg = model.step(cache, slots, [[t] for t in tokens], "last")
+        tokens, _ = sampler.sample(lg, rng_seq=rng, rng_step=[k] * batch)
+
+    for k in range(warmup):
+        one(k)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(steps):
+        one(warmup + k)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    mean_ctx = prompt_len + warmup + (steps + 1) / 2.0
+    for s in slots:
+        cache.free(s)
+    del cache
+    return dt, mean_ctx
+
+
+def run_prefill(model, T, reps=3, seed=1):
+    import torch
+
+    g = torch.Generator().manual_seed(seed)
+    prompt = torch.randint(0, model.vocab_size, (T,), generator=g).tolist()
+    cache = model.new_cache((T + 63) // 64 * 64, max_slots=1)
+    best = None
+    for r in range(reps + 1):
+        slot = cache.alloc()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        model.step(cache, [slot], [prompt], "last")
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        cache.free(slot)
+        if r > 0:  # the first run warms the library's kernel selection
+            best = dt if best is None else min(best, dt)
+    return best
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--prompt-len", type=int, default=1024)
+    ap.add_argument("--layers", type=int, default=32, help="fewer than 32 only where memory or time needs it")
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / batch 64 / prefill measurements")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    import torch
+
+    from pytorch_transformers_amd import AutoModelForCausalLM, GenerationConfig, ops
+    from pytorch_transformers_amd.sampling import Sampler
+
+    ops.load_library()
+    cfg = falcon7b_config(args.layers)
+    dtype = "bfloat16" if args.dtype == "bf16" else "float32"
+    elem = 2 if args.dtype == "bf16" else 4
+    model = AutoModelForCausalLM.from_config(cfg, seed=0, dtype=dtype, device="cuda:0")
+    gen_cfg = GenerationConfig(do_sample=False, eos_token_id=None)
+
+    dt, mean_ctx = run_decode(model, Sampler, gen_cfg, args.batch, args.prompt_len, args.steps, args.warmup)
+    ms = dt / args.steps * 1e3
+    value = args.batch * args.steps / dt
+    step_bytes = weight_bytes(cfg, elem) + args.batch * mean_ctx * kv_bytes_per_token(cfg, elem)
+    achieved = step_bytes / (ms * 1e-3) / 1e9
+
+    out = {
+        "metric": "falcon7b_decode_tokens_per_second", "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
+        "data": "synthetic token ids, random weights N(0, 0.02)",
+        "config": {"model": "falcon-7b layer sizes", "layers": args.layers, "layers_of_config": 32,
+                   "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.kv_heads,
+                   "head_dim": cfg.head_dim, "ffn": cfg.ffn_hidden_size, "vocab": cfg.vocab_size,
+                   "global_batch": args.batch, "prompt_len": args.prompt_len, "seq_len": 2048,
+                   "decode": "greedy", "parallelism": "single"},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+    }
+    if not args.no_points:
+        T = 2048
+        pt = run_prefill(model, T)
+        flops = prefill_flops(cfg, T)
+        out["prefill"] = {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3),
+                          "frac": round(flops / pt / (PEAK_TFLOPS[args.dtype] * 1e12), 4)}
+        points = {}
+        for b in (1, 64):
+            steps_b = max(16, args.steps // 2)
+            d, _ = run_decode(model, Sampler, gen_cfg, b, args.prompt_len, steps_b, 8)
+            points[f"decode_b{b}"] = round(b * steps_b / d, 2)
+        out["points"] = points
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
