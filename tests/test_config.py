@@ -1,0 +1,147 @@
+"""Configuration and registry (no GPU)."""
+import json
+
+import pytest
+
+from pytorch_transformers_amd.config import (AutoConfig, ConfigError, FalconConfig, GenerationConfig, known_model_types,
+                                             lookup, register, unregister)
+from pytorch_transformers_amd.config.base import ModelConfig
+from tiny import TINY
+
+
+def test_defaults_are_falcon_7b():
+    # src/transformers/models/falcon/configuration_falcon.py:144-170
+    c = FalconConfig()
+    assert (c.vocab_size, c.hidden_size, c.num_hidden_layers, c.num_attention_heads) == (65024, 4544, 32, 71)
+    assert c.num_kv_heads == 71 and c.kv_heads == 1  # multi_query: one KV head exists in the weights
+    assert c.ffn_hidden_size == 4 * 4544 and c.head_dim == 64 and c.rotary and not c.alibi
+    assert c.qkv_layout == "tail" and c.qkv_out_dim == 4544 + 2 * 64 and c.norm_scheme == "single"
+    assert c.layer_norm_epsilon == 1e-5 and c.rope_theta == 10000.0 and c.bos_token_id == 11 and c.eos_token_id == 11
+    assert c.tie_word_embeddings is True and c.activation == "gelu" and c.max_position_embeddings == 2048
+
+
+def test_layouts_and_norm_schemes():
+    a = AutoConfig.from_dict(TINY["A"])
+    assert (a.qkv_layout, a.norm_scheme, a.kv_heads, a.qkv_out_dim, a.num_ln_in_parallel_attn) == ("grouped", "dual", 2, 128, 2)
+    b = AutoConfig.from_dict(TINY["B"])
+    assert (b.qkv_layout, b.norm_scheme, b.kv_heads, b.qkv_out_dim, b.head_dim) == ("interleaved", "sequential", 6, 432, 24)
+    d = AutoConfig.from_dict(TINY["D"])
+    assert (d.qkv_layout, d.norm_scheme, d.rope_type) == ("grouped", "single", "linear")
+    # 40B-like: new architecture ignores multi_query
+    c = FalconConfig(hidden_size=512, num_attention_heads=8, num_kv_heads=2, new_decoder_architecture=True, multi_query=True)
+    assert c.kv_heads == 2 and c.norm_scheme == "dual"
+
+
+def test_aliases_and_legacy_keys():
+    c = AutoConfig.from_dict({"model_type": "RefinedWeb", "n_embed": 128, "n_head": 8, "n_layer": 3, "n_head_kv": 2})
+    assert (c.hidden_size, c.num_attention_heads, c.num_hidden_layers, c.num_kv_heads) == (128, 8, 3, 2)
+    assert c.new_decoder_architecture is True
+    c = AutoConfig.from_dict({"model_type": "RefinedWebModel", "n_head": 4, "hidden_size": 64})
+    assert c.new_decoder_architecture is False and c.multi_query is True
+
+
+def test_unknown_keys_are_kept_and_round_trip(tmp_path):
+    d = dict(TINY["A"], some_future_key=[1, 2], architectures=["FalconForCausalLM"], torch_dtype="bfloat16")
+    c = AutoConfig.from_dict(d)
+    assert c.extra == {"some_future_key": [1, 2]}
+    c.save_pretrained(str(tmp_path))
+    again = AutoConfig.from_pretrained(str(tmp_path))
+    assert again == c and again.to_dict()["some_future_key"] == [1, 2]
+    assert json.load(open(tmp_path / "config.json"))["model_type"] == "falcon"
+
+
+@pytest.mark.parametrize("bad,match", [
+    (dict(hidden_size=100, num_attention_heads=7), "divisible"),
+    (dict(new_decoder_architecture=True, parallel_attn=False), "parallel_attn"),
+    (dict(new_decoder_architecture=False, parallel_attn=True, num_ln_in_parallel_attn=2), "num_ln_in_parallel_attn"),
+    (dict(new_decoder_architecture=False, multi_query=False, num_kv_heads=2, num_attention_heads=8, hidden_size=64), "multi_query=false"),
+    (dict(new_decoder_architecture=True, num_attention_heads=8, num_kv_heads=3, hidden_size=64), "multiple"),
+    (dict(activation="relu"), "activation"),
+    (dict(hidden_size=66, num_attention_heads=22), "even head size"),
+    (dict(rope_scaling={"rope_type": "yarn", "factor": 2.0}), "not built"),
+    (dict(rope_scaling={"type": "bogus", "factor": 2.0}), "unknown"),
+    (dict(rope_scaling={"type": "linear", "factor": 0.5}), "factor"),
+    (dict(alibi=True, rope_scaling={"type": "linear", "factor": 2.0}), "alibi"),
+    (dict(vocab_size=0), "positive"),
+    (dict(layer_norm_epsilon=0.0), "epsilon"),
+])
+def test_invalid_combinations_are_rejected(bad, match):
+    with pytest.raises(ConfigError, match=match):
+        FalconConfig(**bad)
+
+
+def test_odd_head_size_is_fine_with_alibi():
+    assert FalconConfig(hidden_size=66, num_attention_heads=22, alibi=True).head_dim == 3
+
+
+def test_registry():
+    assert "falcon" in known_model_types()
+    with pytest.raises(ConfigError, match="not registered.*falcon"):
+        AutoConfig.from_dict({"model_type": "llama"})
+    with pytest.raises(ConfigError, match="model_type"):
+        AutoConfig.from_dict({"hidden_size": 8})
+    with pytest.raises(ValueError, match="already registered"):
+        register("falcon", FalconConfig, lambda c: None)
+
+    import dataclasses
+
+    @dataclasses.dataclass
+    class ToyConfig(ModelConfig):
+        model_type = "toy-registry-test"
+        width: int = 8
+
+    with pytest.raises(ValueError, match="must equal"):
+        register("other-name", ToyConfig, lambda c: None)
+    register("toy-registry-test", ToyConfig, lambda c: ("built", c.width))
+    try:
+        cfg = AutoConfig.from_dict({"model_type": "toy-registry-test", "width": 5, "tie_word_embeddings": False})
+        assert isinstance(cfg, ToyConfig) and cfg.width == 5 and cfg.tie_word_embeddings is False
+        assert lookup("toy-registry-test")[1](cfg) == ("built", 5)
+    finally:
+        unregister("toy-registry-test")
+
+
+def test_falcon_builder_lists_the_checkpoint_tensors():
+    _, builder = lookup("falcon")
+    names = {s.name: s for s in builder(AutoConfig.from_dict(TINY["A"])).tensor_specs()}
+    assert names["transformer.h.1.self_attention.query_key_value.weight"].shape == (128, 64)
+    assert names["transformer.h.0.ln_attn.weight"].shape == (64,) and "transformer.h.0.ln_mlp.bias" in names
+    assert "transformer.h.0.input_layernorm.weight" not in names
+    assert names["lm_head.weight"].tied_to == "transformer.word_embeddings.weight"
+    assert not any(n.endswith("query_key_value.bias") for n in names)
+    names_b = {s.name: s for s in builder(AutoConfig.from_dict(TINY["B"])).tensor_specs()}
+    assert names_b["transformer.h.2.self_attention.query_key_value.bias"].shape == (432,)
+    assert "transformer.h.0.post_attention_layernorm.weight" in names_b and "transformer.ln_f.bias" in names_b
+    assert names_b["transformer.h.0.mlp.dense_4h_to_h.weight"].shape == (144, 576)
+    names_d = {s.name: s for s in builder(AutoConfig.from_dict(TINY["D"])).tensor_specs()}
+    assert names_d["lm_head.weight"].tied_to is None
+
+
+def test_generation_config():
+    g = GenerationConfig()
+    # src/transformers/generation/configuration_utils.py:391-507
+    assert (g.max_length, g.max_new_tokens, g.do_sample, g.temperature, g.top_k, g.top_p, g.repetition_penalty) == \
+        (20, None, False, 1.0, 50, 1.0, 1.0)
+    assert GenerationConfig(eos_token_id=[3, 5]).eos_token_ids == [3, 5] and GenerationConfig(eos_token_id=7).eos_token_ids == [7]
+    with pytest.raises(ValueError, match="strictly positive float"):
+        GenerationConfig(do_sample=True, temperature=0.0)
+    with pytest.raises(ValueError, match="top_p"):
+        GenerationConfig(do_sample=True, top_p=1.5)
+    with pytest.raises(ValueError, match="num_return_sequences"):
+        GenerationConfig(do_sample=False, num_return_sequences=2)
+    with pytest.raises(ValueError, match="num_beams"):
+        GenerationConfig(num_beams=4)
+    with pytest.raises(ValueError, match="max_new_tokens"):
+        GenerationConfig(max_new_tokens=0)
+    with pytest.raises(ValueError, match="unknown generation option"):
+        g.updated(bogus=1)
+    assert g.updated(max_new_tokens=5).max_new_tokens == 5 and g.max_new_tokens is None
+    fm = GenerationConfig.from_model_config(FalconConfig())
+    assert (fm.bos_token_id, fm.eos_token_id, fm.pad_token_id) == (11, 11, None)
+
+
+def test_generation_config_from_folder(tmp_path):
+    (tmp_path / "generation_config.json").write_text(json.dumps(
+        {"eos_token_id": 2, "bos_token_id": 1, "do_sample": True, "temperature": 0.7, "transformers_version": "4.33"}))
+    g = GenerationConfig.from_pretrained(str(tmp_path))
+    assert (g.eos_token_id, g.do_sample, g.temperature) == (2, True, 0.7)

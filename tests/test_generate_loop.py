@@ -1,0 +1,186 @@
+"""The generation loop's decisions, with a scripted model and sampler in place of the GPU (no GPU)."""
+import pytest
+import torch
+
+from pytorch_transformers_amd.cache import PagedCache
+from pytorch_transformers_amd.config import GenerationConfig
+from pytorch_transformers_amd.engine.generate import GenerateOutput, generate, pad_sequences, resolve_lengths
+from pytorch_transformers_amd.engine.spec import CACHE_FULL, CacheGroupSpec
+
+V = 50
+
+
+class ScriptedModel:
+    """The next token of a sequence is (sum of its tokens so far) % V; records every step."""
+
+    vocab_size = V
+    device = torch.device("cpu")
+    generation_config = None
+
+    def __init__(self):
+        self.steps = []
+        self.seen = {}
+        self.caches = []
+
+    def new_cache(self, max_tokens, max_slots=None):
+        c = PagedCache([CacheGroupSpec("kv", CACHE_FULL, 1, 1, 16)], max_tokens, torch.float32, "cpu", max_slots=max_slots)
+        self.caches.append(c)
+        return c
+
+    def step(self, cache, slots, tokens, want):
+        assert want == "last"
+        cache.reserve(slots, [len(t) for t in tokens])
+        rows = []
+        for s, t in zip(slots, tokens):
+            if cache.length(s) == 0:
+                self.seen[s] = []
+            else:
+                assert len(t) == 1, "after its prompt a sequence brings one token a step"
+            self.seen[s] = self.seen[s] + list(t)
+            row = torch.zeros(V)
+            row[sum(self.seen[s]) % V] = 5.0
+            rows.append(row)
+        cache.commit(slots, [len(t) for t in tokens])
+        cache.check_consistent()
+        self.steps.append((list(slots), [list(t) for t in tokens]))
+        return torch.stack(rows)
+
+
+class ArgmaxSampler:
+    def __init__(self, eos=()):
+        self.calls = []
+        self.eos = list(eos)
+
+    def sample(self, logits, *, rng_seq, rng_step, histories, suppress_eos, uniforms=None):
+        self.calls.append(dict(rng_seq=list(rng_seq), rng_step=list(rng_step), suppress=list(suppress_eos),
+                               histories=[list(h) for h in histories]))
+        scores = logits.clone()
+        for r, sup in enumerate(suppress_eos):
+            if sup:
+                scores[r, self.eos] = float("-inf")
+        return scores.argmax(-1).tolist(), scores
+
+
+def expected(prompt, n, eos=()):
+    seq = list(prompt)
+    for _ in range(n):
+        seq.append(sum(seq) % V)
+        if seq[-1] in eos:
+            break
+    return seq
+
+
+def test_unequal_prompts_each_get_their_tokens():
+    m = ScriptedModel()
+    prompts = [[1, 2, 3], [4], [5, 6, 7, 8, 9, 10, 11]]
+    out = generate(m, prompts, GenerationConfig(max_new_tokens=4), sampler=ArgmaxSampler())
+    assert out == [expected(p, 4) for p in prompts]
+    assert m.steps[0][1] == prompts  # prompts go through one step together, unpadded
+    assert all(len(t) == 1 for _, toks in m.steps[1:] for t in toks)
+    assert len(m.steps) == 4  # prompt step + 3 single-token steps (the 4th token needs no further step)
+    assert not m.caches[0].live_slots() and m.caches[0].free_pages() == m.caches[0].num_pages
+
+
+def test_eos_ends_a_sequence_early_keeps_the_token_and_frees_the_slot():
+    m = ScriptedModel()
+    prompts = [[1, 2, 3], [20, 5]]
+    # sequence 0: 6, 12, 24, 48 ...; sequence 1: 25, 0, 0 ...  -> EOS 12 stops sequence 0 after two tokens
+    out = generate(m, prompts, GenerationConfig(max_new_tokens=5, eos_token_id=12), sampler=ArgmaxSampler([12]))
+    assert out[0] == [1, 2, 3, 6, 12] and out[1] == expected([20, 5], 5)
+    assert [len(s) for s, _ in m.steps] == [2, 2, 1, 1, 1]  # the batch shrinks at once
+    assert not m.caches[0].live_slots()
+    # a list of stop tokens
+    out = generate(ScriptedModel(), prompts, GenerationConfig(max_new_tokens=5, eos_token_id=[99, 25]),
+                   sampler=ArgmaxSampler([99, 25]))
+    assert out[1] == [20, 5, 25]
+
+
+def test_min_new_tokens_and_min_length_suppress_eos():
+    s = ArgmaxSampler([6])
+    generate(ScriptedModel(), [[1, 2, 3]], GenerationConfig(max_new_tokens=4, eos_token_id=6, min_new_tokens=2), sampler=s)
+    # 6 is masked twice (the argmax falls to token 0), then allowed, chosen, and ends the sequence
+    assert [c["suppress"][0] for c in s.calls] == [True, True, False]
+    s = ArgmaxSampler([6])
+    # min_length counts the (longest) prompt: 3 + new < 5 for the first two choices
+    generate(ScriptedModel(), [[1, 2, 3]], GenerationConfig(max_new_tokens=4, eos_token_id=6, min_length=5), sampler=s)
+    assert [c["suppress"][0] for c in s.calls] == [True, True, False]
+
+
+def test_max_length_counts_from_the_longest_prompt():
+    assert resolve_lengths(GenerationConfig(max_length=10), [3, 7]) == (3, 7)
+    assert resolve_lengths(GenerationConfig(max_length=10, max_new_tokens=2), [3, 7]) == (2, 7)
+    with pytest.raises(ValueError, match="max_length"):
+        resolve_lengths(GenerationConfig(max_length=7), [3, 7])
+    out = generate(ScriptedModel(), [[1, 2, 3], [4] * 7], GenerationConfig(max_length=10), sampler=ArgmaxSampler())
+    assert [len(o) for o in out] == [6, 10]
+
+
+def test_batches_run_one_after_another_on_one_cache():
+    m = ScriptedModel()
+    prompts = [[i + 1, i + 2] for i in range(7)]
+    out = generate(m, prompts, GenerationConfig(max_new_tokens=3), batch_size=3, sampler=ArgmaxSampler())
+    assert out == [expected(p, 3) for p in prompts]
+    assert len(m.caches) == 1 and m.caches[0].max_slots == 3
+    starts = [toks for _, toks in m.steps if len(toks[0]) == 2]
+    assert [len(t) for t in starts] == [3, 3, 1]  # three batches
+    used = {s for slots, _ in m.steps for s in slots}
+    assert used == {0, 1, 2}  # slots are used again
+
+
+def test_rng_streams_follow_the_prompt_not_the_batch():
+    s = ArgmaxSampler()
+    generate(ScriptedModel(), [[1], [2], [3]], GenerationConfig(max_new_tokens=2, do_sample=True), batch_size=2, sampler=s)
+    assert [c["rng_seq"] for c in s.calls] == [[0, 1], [0, 1], [2], [2]]
+    assert [c["rng_step"] for c in s.calls] == [[0, 0], [1, 1], [0], [1]]
+    s = ArgmaxSampler()
+    generate(ScriptedModel(), [[3]], GenerationConfig(max_new_tokens=1, do_sample=True), rng_ids=[2], sampler=s)
+    assert s.calls[0]["rng_seq"] == [2]
+    s = ArgmaxSampler()
+    out = generate(ScriptedModel(), [[1], [2]], GenerationConfig(max_new_tokens=1, do_sample=True, num_return_sequences=2), sampler=s)
+    assert len(out) == 4 and s.calls[0]["rng_seq"] == [0, 1, 2, 3] and out[0][:1] == out[1][:1] == [1]
+
+
+def test_histories_streamer_and_outputs():
+    s = ArgmaxSampler()
+    seen = []
+
+    class Streamer:
+        ended = False
+
+        def __call__(self, i, tok):
+            seen.append((i, tok))
+
+        def end(self):
+            self.ended = True
+
+    st = Streamer()
+    out = generate(ScriptedModel(), [[1, 2], [7]], GenerationConfig(max_new_tokens=2, return_dict_in_generate=True,
+                                                                    output_scores=True, output_logits=True),
+                   sampler=s, streamer=st)
+    assert isinstance(out, GenerateOutput) and out.sequences == [[1, 2, 3, 6], [7, 7, 14]]
+    assert s.calls[1]["histories"] == [[1, 2, 3], [7, 7]]  # prompt and new tokens, for the repetition penalty
+    assert seen == [(0, 3), (1, 7), (0, 6), (1, 14)] and st.ended
+    assert len(out.scores[0]) == 2 and out.logits[1][0].shape == (V,)
+
+
+def test_empty_prompt_starts_from_bos_and_slots_return_on_error():
+    out = generate(ScriptedModel(), [[]], GenerationConfig(max_new_tokens=1, bos_token_id=9), sampler=ArgmaxSampler())
+    assert out == [[9, 9]]
+    with pytest.raises(ValueError, match="empty"):
+        generate(ScriptedModel(), [[]], GenerationConfig(max_new_tokens=1), sampler=ArgmaxSampler())
+
+    class Boom(ScriptedModel):
+        def step(self, *a, **k):
+            if len(self.steps) == 1:
+                raise RuntimeError("boom")
+            return super().step(*a, **k)
+
+    m = Boom()
+    with pytest.raises(RuntimeError, match="boom"):
+        generate(m, [[1], [2]], GenerationConfig(max_new_tokens=3), sampler=ArgmaxSampler())
+    assert not m.caches[0].live_slots() and m.caches[0].free_pages() == m.caches[0].num_pages
+
+
+def test_pad_sequences_matches_the_reference_layout():
+    t = pad_sequences([[1, 2, 3, 9, 9], [4, 8]], [3, 1], pad_token_id=0)
+    assert t.tolist() == [[1, 2, 3, 9, 9], [0, 0, 4, 8, 0]]

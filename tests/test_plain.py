@@ -1,0 +1,308 @@
+"""What pins the plain implementation besides the reference's text (no GPU).
+
+Vectors that the reference's own tests hold, special cases that reduce to a torch routine, and
+invariants; each is chosen so that a plausible mistake fails it (named in the test's docstring).
+"""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import plain_falcon as P
+from tiny import TINY, write_model
+
+D = torch.float64
+
+
+def rnd(*shape, seed=0):
+    return torch.randn(*shape, dtype=D, generator=torch.Generator().manual_seed(seed))
+
+
+# --- norm, activation ----------------------------------------------------------------------
+def test_layer_norm_is_torchs():
+    """Fails for unbiased variance, eps outside the root, or a missing affine term."""
+    x, w, b = rnd(5, 48) * 3 + 1, rnd(48, seed=1), rnd(48, seed=2)
+    for eps in (1e-5, 1e-2):
+        torch.testing.assert_close(P.layer_norm(x, w, b, eps), F.layer_norm(x, (48,), w, b, eps))
+    torch.testing.assert_close(P.layer_norm(x + 7.5, w, b, 1e-5), P.layer_norm(x, w, b, 1e-5))
+    y = P.layer_norm(x, torch.ones(48, dtype=D), torch.zeros(48, dtype=D), 1e-12)
+    torch.testing.assert_close(y.mean(-1), torch.zeros(5, dtype=D), atol=1e-12, rtol=0)
+    torch.testing.assert_close((y ** 2).mean(-1), torch.ones(5, dtype=D))
+
+
+def test_gelu_is_the_erf_form():
+    """The reference's vector (tests/utils/test_activations.py:29-33); fails for the tanh form."""
+    x = torch.tensor([-100, -1, -0.1, 0, 0.1, 1.0, 100], dtype=D)
+    torch.testing.assert_close(P.gelu(x), F.gelu(x))
+    assert not torch.allclose(P.gelu(x), F.gelu(x, approximate="tanh"), atol=1e-6, rtol=0)
+
+
+# --- rotary ---------------------------------------------------------------------------------
+def test_rope_inv_freq_vector():
+    """tests/utils/test_modeling_rope_utils.py:133-166: d=128, theta=1e4."""
+    inv = P.rope_inv_freq(128, 10000.0)
+    expected = torch.tensor([10.0 ** (-i / 16.0) for i in range(64)])
+    torch.testing.assert_close(inv, expected, rtol=1e-4, atol=0)
+    assert inv.dtype == torch.float32 and abs(float(inv[1]) - 8.6596e-01) < 1e-4 and abs(float(inv[63]) - 1.1548e-04) < 1e-7
+    torch.testing.assert_close(P.rope_inv_freq(128, 10000.0, 4.0), inv / 4.0)  # linear scaling (:168-194)
+
+
+def test_rope_hand_case_pairs_and_sign():
+    """Pairs are (i, i + d/2), not (2i, 2i+1); the lower half gets -sin.  d=4, position 1."""
+    x = torch.tensor([[[1.0, 2.0, 3.0, 4.0]]], dtype=D)
+    inv = torch.tensor([1.0, 0.5])
+    cos, sin = P.rope_cos_sin(torch.tensor([1]), inv)
+    out = P.apply_rope(x, cos, sin)[0, 0]
+    c0, s0, c1, s1 = math.cos(1.0), math.sin(1.0), math.cos(0.5), math.sin(0.5)
+    want = torch.tensor([1 * c0 - 3 * s0, 2 * c1 - 4 * s1, 3 * c0 + 1 * s0, 4 * c1 + 2 * s1], dtype=D)
+    torch.testing.assert_close(out, want, rtol=1e-6, atol=1e-7)
+
+
+def test_rope_invariants():
+    """Position 0 is the identity; pair norms are kept; <R_m q, R_n k> depends on m - n only; the
+    cos/sin of a short range are the prefix of a long one (tests/models/falcon/test_modeling_falcon.py:470-475);
+    linear scaling by f maps position x to x / f (:485-488)."""
+    d = 32
+    inv = P.rope_inv_freq(d, 10000.0)
+    q, k = rnd(1, 3, d), rnd(1, 3, d, seed=1)
+    c0, s0 = P.rope_cos_sin(torch.tensor([0]), inv)
+    torch.testing.assert_close(P.apply_rope(q, c0, s0), q)
+    pos = torch.tensor([0, 3, 4, 10, 11, 17])
+    cos, sin = P.rope_cos_sin(pos, inv)
+    qq = P.apply_rope(q.expand(6, 3, d), cos, sin)
+    kk = P.apply_rope(k.expand(6, 3, d), cos, sin)
+    pair_norm = lambda t: t[..., :d // 2] ** 2 + t[..., d // 2:] ** 2
+    torch.testing.assert_close(pair_norm(qq), pair_norm(q.expand(6, 3, d)), rtol=1e-6, atol=1e-9)
+    dot = lambda a, b: float((qq[a, 0] * kk[b, 0]).sum())
+    assert abs(dot(2, 1) - dot(4, 3)) < 1e-5 and abs(dot(3, 1) - dot(5, 3)) < 1e-5  # distances 1 and 7
+    assert abs(dot(2, 1) - dot(1, 2)) > 1e-3  # ... and the sign of the distance matters
+    cl, sl = P.rope_cos_sin(torch.arange(40), inv)
+    cs, ss = P.rope_cos_sin(torch.arange(9), inv)
+    assert torch.equal(cl[:9], cs) and torch.equal(sl[:9], ss)
+    c2, s2 = P.rope_cos_sin(torch.tensor([10]), P.rope_inv_freq(d, 10000.0, 2.0))
+    c1, s1 = P.rope_cos_sin(torch.tensor([5]), inv)
+    torch.testing.assert_close(c2, c1, rtol=1e-6, atol=1e-7)
+    torch.testing.assert_close(s2, s1, rtol=1e-6, atol=1e-7)
+
+
+# --- ALiBi -----------------------------------------------------------------------------------
+def test_alibi_slopes():
+    """Power-of-two head counts: 2^(-8(i+1)/n).  Six heads: the four of n=4, then odd powers of the
+    n=8 base.  Fails for a wrong base or for taking the extra slopes at even powers."""
+    for n in (4, 8, 16):
+        torch.testing.assert_close(P.alibi_slopes(n), torch.tensor([2.0 ** (-8.0 * (i + 1) / n) for i in range(n)]))
+    torch.testing.assert_close(P.alibi_slopes(6), torch.tensor([1 / 4, 1 / 16, 1 / 64, 1 / 256, 1 / 2, 1 / 8]))
+    s20 = P.alibi_slopes(20)
+    torch.testing.assert_close(s20[16:], torch.tensor([2.0 ** (-0.25 * p) for p in (1, 3, 5, 7)]))
+
+
+def test_alibi_bias_is_rounded_like_the_reference():
+    """slope x position is formed in bfloat16 (modeling_falcon.py:196-198): exact for 6 heads at
+    small positions, visibly rounded for 20 heads and for positions past 256."""
+    b6 = P.alibi_bias(6, 10, 24)
+    torch.testing.assert_close(b6[4], torch.arange(10, dtype=D) * 0.5 / math.sqrt(24))
+    b20 = P.alibi_bias(20, 400, 16)
+    exact = P.alibi_slopes(20).double()[:, None] * torch.arange(400, dtype=D)[None, :] / 4.0
+    assert float((b20 - exact).abs().max()) > 1e-3
+    s_bf = P.alibi_slopes(20).bfloat16().double()
+    p_bf = torch.arange(400).bfloat16().double()
+    prod = (s_bf[:, None] * p_bf[None, :]).bfloat16().double()  # each product has <= 16 significant bits: exact in float64
+    torch.testing.assert_close(b20, prod / 4.0)
+    assert float(p_bf[301]) != 301.0  # positions past 256 are themselves rounded
+
+
+def test_alibi_key_bias_equals_relative_bias():
+    """Softmax ignores a per-query constant: slope*j == -slope*(t - j).  Zero slopes: no positions."""
+    T, d = 7, 8
+    q, k, v = rnd(T, 1, d), rnd(T, 1, d, seed=1), rnd(T, 1, d, seed=2)
+    slope = 0.3
+    key_bias = (slope * torch.arange(T, dtype=D))[None, :]
+    out_key = P.attention_scores_softmax(q, k, v, key_bias)
+    rel = torch.stack([-slope * (t - torch.arange(T, dtype=D)) for t in range(T)])  # [T, T]
+    s = (q[:, 0] @ k[:, 0].T) / math.sqrt(d) + rel + torch.full((T, T), float("-inf"), dtype=D).triu(1)
+    torch.testing.assert_close(out_key, torch.softmax(s, -1) @ v[:, 0])
+    torch.testing.assert_close(P.attention_scores_softmax(q, k, v, torch.zeros(1, T, dtype=D)),
+                               P.attention_scores_softmax(q, k, v, None))
+
+
+# --- fused projection layouts, attention ---------------------------------------------------------
+def _cfg(**kw):
+    return P.cfg_defaults(dict(kw))
+
+
+def test_split_heads_three_layouts():
+    """Hand-indexed rows for each order; fails if k and v are swapped or groups are interleaved wrongly."""
+    T, d = 3, 4
+    # grouped: 6 heads in 2 groups of 3: [q0 q1 q2 k0 v0 | q3 q4 q5 k1 v1]
+    c = _cfg(hidden_size=24, num_attention_heads=6, num_kv_heads=2, new_decoder_architecture=True)
+    fused = torch.arange(T * 10 * d, dtype=D).view(T, 10 * d)
+    q, k, v = P.split_heads(fused, c)
+    blocks = fused.view(T, 10, d)
+    assert torch.equal(q, blocks[:, [0, 1, 2, 5, 6, 7]]) and torch.equal(k, blocks[:, [3, 8]]) and torch.equal(v, blocks[:, [4, 9]])
+    # tail: [q0..q5 k v]
+    c = _cfg(hidden_size=24, num_attention_heads=6, multi_query=True)
+    fused = torch.arange(T * 8 * d, dtype=D).view(T, 8 * d)
+    q, k, v = P.split_heads(fused, c)
+    blocks = fused.view(T, 8, d)
+    assert torch.equal(q, blocks[:, :6]) and torch.equal(k, blocks[:, [6]]) and torch.equal(v, blocks[:, [7]])
+    # interleaved: [q0 k0 v0 q1 k1 v1 ...]
+    c = _cfg(hidden_size=24, num_attention_heads=6, multi_query=False)
+    fused = torch.arange(T * 18 * d, dtype=D).view(T, 18 * d)
+    q, k, v = P.split_heads(fused, c)
+    blocks = fused.view(T, 18, d)
+    assert torch.equal(q, blocks[:, 0::3]) and torch.equal(k, blocks[:, 1::3]) and torch.equal(v, blocks[:, 2::3])
+
+
+def test_attention_is_sdpa_and_groups_are_repeated_heads():
+    """No rotation, no bias: one sequence equals torch's scaled_dot_product_attention(is_causal=True);
+    grouped KV equals full heads on repeated keys and values (modeling_falcon.py:286-289)."""
+    T, nh, nkv, d = 9, 6, 2, 8
+    q, k, v = rnd(T, nh, d), rnd(T, nkv, d, seed=1), rnd(T, nkv, d, seed=2)
+    out = P.attention_scores_softmax(q, k, v)
+    kr, vr = k.repeat_interleave(nh // nkv, 1), v.repeat_interleave(nh // nkv, 1)
+    ref = F.scaled_dot_product_attention(q.transpose(0, 1)[None], kr.transpose(0, 1)[None], vr.transpose(0, 1)[None],
+                                         is_causal=True)[0].transpose(0, 1).reshape(T, nh * d)
+    torch.testing.assert_close(out, ref)
+    torch.testing.assert_close(P.attention_scores_softmax(q, kr, vr), out)
+    # one token: the output is its value; equal keys: the running mean of values
+    torch.testing.assert_close(P.attention_scores_softmax(q[:1], k[:1], v[:1]).view(nh, d), vr[0])
+    same_k = k[:1].expand(T, nkv, d)
+    mean = torch.cumsum(vr, 0) / torch.arange(1, T + 1, dtype=D)[:, None, None]
+    torch.testing.assert_close(P.attention_scores_softmax(q, same_k, v), mean.reshape(T, nh * d))
+
+
+# --- the whole model ----------------------------------------------------------------------------
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    root = str(tmp_path_factory.mktemp("plain"))
+    return {n: P.read_model(write_model(n, root)) for n in TINY}
+
+
+@pytest.mark.parametrize("name", sorted(TINY))
+def test_causality_and_prefix(models, name):
+    """Logits at a position do not change with later tokens; fails for a mask off by one."""
+    cfg, w = models[name]
+    ids = [(7 * i + 3) % cfg["vocab_size"] for i in range(20)]
+    full = P.forward(cfg, w, ids)
+    torch.testing.assert_close(P.forward(cfg, w, ids[:11]), full[:11], rtol=1e-9, atol=1e-9)
+    changed = list(ids)
+    changed[15] = (changed[15] + 1) % cfg["vocab_size"]
+    other = P.forward(cfg, w, changed)
+    torch.testing.assert_close(other[:15], full[:15], rtol=1e-9, atol=1e-9)
+    assert not torch.allclose(other[15:], full[15:], atol=1e-6)
+    assert full.shape == (20, cfg["vocab_size"])
+
+
+def test_residual_arrangements(models):
+    """Parallel block with the feed-forward's output matrix zeroed is x + attention; with the
+    attention's output matrix zeroed it is x + feed-forward (fails for a norm in the wrong branch)."""
+    cfg, w = models["C"]
+    c = P.cfg_defaults(cfg)
+    x = rnd(6, c["hidden_size"])
+    pos = torch.arange(6)
+    p = "transformer.h.0."
+    ln = P.layer_norm(x, w[p + "input_layernorm.weight"], w[p + "input_layernorm.bias"], c["layer_norm_epsilon"])
+    attn = P.self_attention(ln, w, p + "self_attention.", c, pos)
+    w0 = dict(w); w0[p + "mlp.dense_4h_to_h.weight"] = torch.zeros_like(w[p + "mlp.dense_4h_to_h.weight"])
+    torch.testing.assert_close(P.decoder_layer(x, w0, 0, c, pos), x + attn)
+    w1 = dict(w); w1[p + "self_attention.dense.weight"] = torch.zeros_like(w[p + "self_attention.dense.weight"])
+    torch.testing.assert_close(P.decoder_layer(x, w1, 0, c, pos), x + P.mlp(ln, w, p + "mlp."))
+    # sequential (B): the feed-forward reads the norm of x + attention, with the second norm's parameters
+    cfg, w = models["B"]
+    c = P.cfg_defaults(cfg)
+    x = rnd(5, c["hidden_size"])
+    pos = torch.arange(5)
+    a = P.self_attention(P.layer_norm(x, w[p + "input_layernorm.weight"], w[p + "input_layernorm.bias"], 1e-6), w,
+                         p + "self_attention.", c, pos)
+    r = x + a
+    want = r + P.mlp(P.layer_norm(r, w[p + "post_attention_layernorm.weight"], w[p + "post_attention_layernorm.bias"], 1e-6),
+                     w, p + "mlp.")
+    torch.testing.assert_close(P.decoder_layer(x, w, 0, c, pos), want)
+
+
+def test_two_equal_norms_are_one_norm(models):
+    """New architecture with ln_attn == ln_mlp equals the one-norm variant with that norm."""
+    cfg, w = models["A"]
+    w2 = dict(w)
+    for i in range(cfg["num_hidden_layers"]):
+        for s in ("weight", "bias"):
+            w2[f"transformer.h.{i}.ln_mlp.{s}"] = w[f"transformer.h.{i}.ln_attn.{s}"]
+            w2[f"transformer.h.{i}.input_layernorm.{s}"] = w[f"transformer.h.{i}.ln_attn.{s}"]
+    ids = list(range(3, 15))
+    one = dict(cfg, num_ln_in_parallel_attn=1)
+    torch.testing.assert_close(P.forward(cfg, w2, ids), P.forward(one, w2, ids))
+    assert not torch.allclose(P.forward(cfg, w, ids), P.forward(cfg, w2, ids), atol=1e-6)
+
+
+def test_tied_head(models):
+    cfg, w = models["A"]
+    ids = list(range(10))
+    untied = dict(w); untied["lm_head.weight"] = w["transformer.word_embeddings.weight"].clone()
+    torch.testing.assert_close(P.forward(cfg, w, ids), P.forward(dict(cfg, tie_word_embeddings=False), untied, ids))
+
+
+# --- processors and the choice -----------------------------------------------------------------------
+def test_processors_on_the_references_vectors():
+    """tests/generation/test_logits_process.py: :183-205 penalty, :235-271 top-k, :273-309 top-p, :311-355 min-p."""
+    s = torch.full((10,), 0.1); s[0] = -0.1
+    out = P.repetition_penalty(s, [0, 1], 2.0)
+    assert abs(float(out[0]) + 0.2) < 1e-7 and abs(float(out[1]) - 0.05) < 1e-7 and float(out[2]) == pytest.approx(0.1)
+    s = torch.full((10,), 0.1); s[5] = 0.4
+    out = P.repetition_penalty(s, [5, 0], 2.0)
+    assert float(out[0]) == pytest.approx(0.05) and float(out[5]) == pytest.approx(0.2)
+    assert float(s[5]) == pytest.approx(0.4)  # inputs are not changed in place
+
+    ramp = torch.arange(10.0)
+    assert torch.isinf(P.top_k(ramp, 3)).tolist() == 7 * [True] + 3 * [False]
+    ramp2 = ramp.clone(); ramp2[:5] += 10
+    assert torch.isinf(P.top_k(ramp2, 3)).tolist() == 2 * [True] + 3 * [False] + 5 * [True]
+    assert int(torch.isinf(P.top_k(torch.arange(5.0), 1, min_tokens_to_keep=3)).sum()) == 2
+
+    dist = torch.log(torch.tensor([[0.3, 0.1, 0.1, 0.5], [0.15, 0.3, 0.3, 0.25]]))
+    torch.testing.assert_close(torch.exp(P.top_p(dist[1], 0.8)), torch.tensor([0.0, 0.3, 0.3, 0.25]), atol=1e-3, rtol=0)
+    torch.testing.assert_close(torch.exp(P.top_p(dist[0], 0.79)), torch.tensor([0.3, 0.0, 0.0, 0.5]), atol=1e-3, rtol=0)
+    # of two equal scores at the cut, the first in ascending stable order goes
+    torch.testing.assert_close(torch.exp(P.top_p(dist[0], 0.85)), torch.tensor([0.3, 0.0, 0.1, 0.5]), atol=1e-3, rtol=0)
+    ramp = torch.arange(10.0) - 5
+    assert int((P.top_p(ramp, 0.9, min_tokens_to_keep=2) != float("-inf")).sum()) == 3
+    assert int((P.top_p(ramp * 100, 0.9, min_tokens_to_keep=2) != float("-inf")).sum()) == 2
+
+    dist = torch.log(torch.tensor([[0.9, 0.0274, 0.047, 0.0274], [0.15, 0.3, 0.3, 0.25], [0.97, 0.01, 0.01, 0.01]]))
+    want = torch.tensor([[0.9, 0.0, 0.047, 0.0], [0.15, 0.3, 0.3, 0.25], [0.97, 0.0, 0.0, 0.0]])
+    for r in range(3):
+        torch.testing.assert_close(torch.exp(P.min_p(dist[r], 0.05)), want[r], atol=1e-3, rtol=0)
+    assert int((P.min_p(ramp, 0.9, min_tokens_to_keep=2) != float("-inf")).sum()) == 2
+
+    # temperature (:148-181): uniform stays uniform, peaks sharpen below 1 and flatten above
+    s = torch.full((20,), 0.05); s[5] = 0.15; s[10] = -0.35
+    p, sharp, smooth = (torch.softmax(t, -1) for t in (s, P.temperature(s, 0.5), P.temperature(s, 1.3)))
+    assert sharp.max() > p.max() > smooth.max() and sharp.min() < p.min() < smooth.min()
+
+    assert torch.isinf(P.suppress(torch.zeros(6), [2, 4])).tolist() == [False, False, True, False, True, False]
+
+
+def test_processing_order_and_pick():
+    """Penalty before temperature, top-k before top-p (generation/utils.py:926-1097); argmax and
+    inverse-CDF choice."""
+    s = torch.tensor([2.0, 1.0, 0.75, -1.0])
+    out = P.process(s, [0], do_sample=True, temperature_=0.5, top_k_=2, repetition_penalty_=4.0)
+    # 2.0 / 4 = 0.5 falls behind 0.75 before top-k looks; top-k first would have kept token 0
+    assert out.tolist() == [float("-inf"), 2.0, 1.5, float("-inf")]
+    assert P.pick(s, None) == 0
+    probs = torch.softmax(s.double(), -1).cumsum(-1)
+    assert P.pick(s, 0.0) == 0 and P.pick(s, float(probs[0]) + 1e-9) == 1 and P.pick(s, 0.999999) == 3
+    greedy = P.process(s, [], do_sample=False, temperature_=0.5, top_k_=1)
+    assert torch.equal(greedy, s)  # warpers are not applied without sampling
+
+
+def test_generate_stops_at_eos_and_keeps_it(models):
+    cfg, w = models["A"]
+    free = P.generate(cfg, w, [1, 2, 3], 8)
+    assert len(free) == 8
+    eos = free[3]
+    first = free.index(eos)
+    stopped = P.generate(cfg, w, [1, 2, 3], 8, eos_ids=(eos,))
+    assert stopped == free[:first + 1]
+    held = P.generate(cfg, w, [1, 2, 3], 8, eos_ids=(eos,), min_new_tokens=first + 2)
+    assert len(held) > first + 1 and eos not in held[:first + 2]

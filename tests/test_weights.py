@@ -1,0 +1,139 @@
+"""Weight files: layouts, errors, dtypes, random-weights mode (no GPU: tensors are placed on the CPU)."""
+import json
+import os
+
+import pytest
+import torch
+
+from pytorch_transformers_amd.config import AutoConfig, lookup
+from pytorch_transformers_amd.weights import (WeightsError, load_weights, random_tensors, save_weights,
+                                              write_random_model)
+from tiny import TINY
+
+
+def _specs(name):
+    cfg = AutoConfig.from_dict(TINY[name])
+    return cfg, lookup("falcon")[1](cfg).tensor_specs()
+
+
+def _rewrite(folder, fn):
+    from safetensors.torch import load_file, save_file
+
+    path = os.path.join(folder, "model.safetensors")
+    t = load_file(path)
+    fn(t)
+    save_file(t, path, metadata={"format": "pt"})
+
+
+def test_random_model_loads_and_is_reproducible(tmp_path):
+    cfg, specs = _specs("A")
+    f1 = write_random_model(str(tmp_path / "m1"), cfg, seed=3)
+    f2 = write_random_model(str(tmp_path / "m2"), cfg, seed=3)
+    f3 = write_random_model(str(tmp_path / "m3"), cfg, seed=4)
+    w1, w2, w3 = (load_weights(f, specs, torch.float32, "cpu") for f in (f1, f2, f3))
+    assert set(w1) == {s.name for s in specs}
+    assert all(torch.equal(w1[k], w2[k]) for k in w1)
+    assert not torch.equal(w1["transformer.h.0.mlp.dense_h_to_4h.weight"], w3["transformer.h.0.mlp.dense_h_to_4h.weight"])
+    assert os.path.isfile(os.path.join(f1, "config.json"))
+    # the file is bfloat16; the tied head is absent from it and shares the embedding's storage
+    from safetensors.torch import load_file
+    raw = load_file(os.path.join(f1, "model.safetensors"))
+    assert "lm_head.weight" not in raw and all(t.dtype == torch.bfloat16 for t in raw.values())
+    assert w1["lm_head.weight"].data_ptr() == w1["transformer.word_embeddings.weight"].data_ptr()
+    # norms and biases are not the reference's ones and zeros, so that an affine term in the wrong place shows
+    assert float((w1["transformer.h.0.ln_attn.weight"] - 1).abs().max()) > 1e-3
+    assert float(w1["transformer.h.0.ln_attn.bias"].abs().max()) > 1e-3
+    std = float(w1["transformer.word_embeddings.weight"].std())
+    assert 0.015 < std < 0.025
+
+
+def test_device_types(tmp_path):
+    cfg, specs = _specs("B")
+    f = write_random_model(str(tmp_path / "m"), cfg, seed=1, store_dtype=torch.float32)
+    w = load_weights(f, specs, torch.bfloat16, "cpu")
+    assert w["transformer.h.0.mlp.dense_h_to_4h.weight"].dtype == torch.bfloat16  # matrices: the compute type
+    assert w["transformer.h.0.mlp.dense_h_to_4h.bias"].dtype == torch.float32  # vectors stay 32-bit
+    assert w["transformer.ln_f.weight"].dtype == torch.float32
+    from safetensors.torch import load_file
+    raw = load_file(os.path.join(f, "model.safetensors"))
+    assert torch.equal(w["transformer.ln_f.weight"], raw["transformer.ln_f.weight"])  # unchanged, not rounded
+    m = "transformer.h.1.self_attention.dense.weight"
+    assert torch.equal(w[m], raw[m].to(torch.bfloat16))  # round to nearest even
+    w32 = load_weights(f, specs, torch.float32, "cpu")
+    assert torch.equal(w32[m], raw[m])
+
+
+def test_one_error_lists_everything(tmp_path):
+    cfg, specs = _specs("A")
+    f = write_random_model(str(tmp_path / "m"), cfg, seed=0)
+
+    def damage(t):
+        del t["transformer.h.0.mlp.dense_4h_to_h.weight"]
+        del t["transformer.ln_f.bias"]
+        t["transformer.h.9.extra.weight"] = torch.zeros(3)
+        t["transformer.h.1.self_attention.dense.weight"] = torch.zeros(64, 32, dtype=torch.bfloat16)
+        t["transformer.h.1.ln_mlp.weight"] = torch.zeros(64, dtype=torch.int32)
+
+    _rewrite(f, damage)
+    with pytest.raises(WeightsError) as e:
+        load_weights(f, specs, torch.float32, "cpu")
+    err = e.value
+    assert err.missing == ["transformer.h.0.mlp.dense_4h_to_h.weight", "transformer.ln_f.bias"]
+    assert err.unexpected == ["transformer.h.9.extra.weight"]
+    assert err.wrong_shape == [("transformer.h.1.self_attention.dense.weight", (64, 32), (64, 64))]
+    assert [w[0] for w in err.wrong_type] == ["transformer.h.1.ln_mlp.weight"]
+    msg = str(err)
+    for part in ("missing tensors (2)", "unexpected tensors (1)", "wrong shapes (1)", "file has (64, 32), model needs (64, 64)",
+                 "wrong types (1)"):
+        assert part in msg, msg
+
+
+def test_unexpected_only_warns_when_not_strict_and_stale_inv_freq_is_ignored(tmp_path):
+    cfg, specs = _specs("A")
+    f = write_random_model(str(tmp_path / "m"), cfg, seed=0)
+    _rewrite(f, lambda t: t.update({"transformer.h.0.self_attention.rotary_emb.inv_freq": torch.zeros(8)}))
+    load_weights(f, specs, torch.float32, "cpu")  # modeling_utils.py:4529-4532
+    _rewrite(f, lambda t: t.update({"something.else": torch.zeros(2)}))
+    with pytest.raises(WeightsError, match="unexpected"):
+        load_weights(f, specs, torch.float32, "cpu")
+    with pytest.warns(UserWarning, match="something.else"):
+        load_weights(f, specs, torch.float32, "cpu", strict=False)
+
+
+def test_untied_head_is_required_and_tied_head_may_be_present(tmp_path):
+    cfg, specs = _specs("D")  # untied
+    f = write_random_model(str(tmp_path / "d"), cfg, seed=0)
+    w = load_weights(f, specs, torch.float32, "cpu")
+    assert w["lm_head.weight"].data_ptr() != w["transformer.word_embeddings.weight"].data_ptr()
+    _rewrite(f, lambda t: t.pop("lm_head.weight"))
+    with pytest.raises(WeightsError, match="missing tensors.*lm_head.weight"):
+        load_weights(f, specs, torch.float32, "cpu")
+    cfg, specs = _specs("A")  # tied, with an explicit copy in the file
+    f = write_random_model(str(tmp_path / "a"), cfg, seed=0)
+    _rewrite(f, lambda t: t.update({"lm_head.weight": t["transformer.word_embeddings.weight"].clone()}))
+    w = load_weights(f, specs, torch.float32, "cpu")
+    assert torch.equal(w["lm_head.weight"], w["transformer.word_embeddings.weight"])
+
+
+def test_sharded_and_unprefixed_files(tmp_path):
+    cfg, specs = _specs("C")
+    tensors = random_tensors(specs, 5, 0.02)
+    one = str(tmp_path / "one")
+    save_weights(one, tensors)
+    sharded = str(tmp_path / "sharded")
+    paths = save_weights(sharded, tensors, shards=3)
+    assert len(paths) == 3 and os.path.isfile(os.path.join(sharded, "model.safetensors.index.json"))
+    index = json.load(open(os.path.join(sharded, "model.safetensors.index.json")))
+    assert set(index["weight_map"]) == set(tensors)
+    bare = str(tmp_path / "bare")  # saved from the base model: no "transformer." prefix (modeling_utils.py:4495-4512)
+    save_weights(bare, {k[len("transformer."):] if k.startswith("transformer.") else k: v for k, v in tensors.items()})
+    a, b, c = (load_weights(f, specs, torch.float32, "cpu") for f in (one, sharded, bare))
+    assert all(torch.equal(a[k], b[k]) and torch.equal(a[k], c[k]) for k in a)
+
+
+def test_missing_files(tmp_path):
+    cfg, specs = _specs("A")
+    with pytest.raises(FileNotFoundError, match="model.safetensors"):
+        load_weights(str(tmp_path), specs, torch.float32, "cpu")
+    with pytest.raises(FileNotFoundError, match="config.json"):
+        AutoConfig.from_pretrained(str(tmp_path))
