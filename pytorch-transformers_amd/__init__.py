@@ -4,6 +4,8 @@ HIP kernels.  Import name: ``pytorch_transformers_amd``."""
 from .config import AutoConfig, ConfigError, FalconConfig, GenerationConfig, register
 from .engine import falcon as _falcon  # registers model_type "falcon"  # noqa: F401
 from .auto import AutoModelForCausalLM
+from .pipeline import TextGenerationPipeline, pipeline
 
 __version__ = "0.1.0"
-__all__ = ["AutoConfig", "AutoModelForCausalLM", "ConfigError", "FalconConfig", "GenerationConfig", "register"]
+__all__ = ["AutoConfig", "AutoModelForCausalLM", "ConfigError", "FalconConfig", "GenerationConfig", "TextGenerationPipeline",
+           "pipeline", "register"]

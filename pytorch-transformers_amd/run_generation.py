@@ -1,0 +1,125 @@
+"""Text generation from the command line, with the option names of the reference's example.
+
+    python -m pytorch_transformers_amd.run_generation --model_name_or_path DIR --prompt_ids 3,1,4 --length 20
+
+Options shared with examples/pytorch/text-generation/run_generation.py:286-333 keep its names,
+defaults and meanings: ``--model_type``, ``--model_name_or_path``, ``--prompt``, ``--length`` (20),
+``--stop_token``, ``--temperature`` (1.0), ``--repetition_penalty`` (1.0), ``--k`` (0), ``--p``
+(0.9), ``--prefix``, ``--seed`` (42), ``--num_return_sequences`` (1).  Like it, the program samples
+(``do_sample=True``, :408-417) and prints ``=== GENERATED SEQUENCE n ===`` before each result
+(:425-441).  Added here: ``--prompt_ids`` / ``--prompt_file`` (token ids, for folders without a
+tokenizer), ``--greedy``, ``--dtype``, ``--random_config`` with ``--random_seed`` (write a model
+folder with random weights first), ``--min_length``-style limits and ``--batch_size``.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import tempfile
+
+MAX_LENGTH = int(10000)  # run_generation.py:49: hard cap against an endless loop
+
+
+def adjust_length_to_model(length: int, max_sequence_length: int) -> int:
+    """run_generation.py:151-158."""
+    if length < 0 and max_sequence_length > 0:
+        return max_sequence_length
+    if 0 < max_sequence_length < length:
+        return max_sequence_length
+    if length < 0:
+        return MAX_LENGTH
+    return length
+
+
+def build_parser() -> argparse.ArgumentParser:
+    ap = argparse.ArgumentParser(description="Generate text (or token ids) with a model folder on one AMD GPU")
+    ap.add_argument("--model_type", default=None, type=str, help="checked against config.json's model_type if given")
+    ap.add_argument("--model_name_or_path", default=None, type=str, help="folder with config.json and model.safetensors")
+    ap.add_argument("--prompt", type=str, default="")
+    ap.add_argument("--prompt_ids", type=str, default=None, help="comma-separated token ids; ';' separates prompts")
+    ap.add_argument("--prompt_file", type=str, default=None, help="file with one prompt of comma-separated ids per line")
+    ap.add_argument("--length", type=int, default=20)
+    ap.add_argument("--min_new_tokens", type=int, default=None)
+    ap.add_argument("--stop_token", type=str, default=None, help="text at which the printed result is cut")
+    ap.add_argument("--stop_token_id", type=int, action="append", default=None, help="token id that ends a sequence")
+    ap.add_argument("--temperature", type=float, default=1.0,
+                    help="temperature of 1.0 has no effect, lower tend toward greedy sampling")
+    ap.add_argument("--repetition_penalty", type=float, default=1.0)
+    ap.add_argument("--k", type=int, default=0)
+    ap.add_argument("--p", type=float, default=0.9)
+    ap.add_argument("--min_p", type=float, default=None)
+    ap.add_argument("--greedy", action="store_true", help="argmax instead of sampling")
+    ap.add_argument("--prefix", type=str, default="", help="Text added prior to input.")
+    ap.add_argument("--seed", type=int, default=42, help="random seed for sampling")
+    ap.add_argument("--num_return_sequences", type=int, default=1, help="The number of samples to generate.")
+    ap.add_argument("--batch_size", type=int, default=None, help="prompts per batch; further batches follow")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--fp16", action="store_true", help="accepted for compatibility; the 16-bit type here is bfloat16")
+    ap.add_argument("--device", default="cuda:0")
+    ap.add_argument("--random_config", type=str, default=None, help="config.json to build a random-weights model from")
+    ap.add_argument("--random_seed", type=int, default=0)
+    return ap
+
+
+def main(argv=None) -> int:
+    args = build_parser().parse_args(argv)
+    from . import AutoConfig, GenerationConfig
+    from .pipeline import pipeline
+    from .weights import write_random_model
+
+    tmp = None
+    folder = args.model_name_or_path
+    if args.random_config is not None:
+        tmp = tempfile.TemporaryDirectory()
+        with open(args.random_config) as f:
+            cfg = AutoConfig.from_dict(json.load(f))
+        folder = write_random_model(tmp.name, cfg, args.random_seed)
+    if folder is None:
+        print("one of --model_name_or_path and --random_config is required", file=sys.stderr)
+        return 2
+    config = AutoConfig.from_pretrained(folder)
+    if args.model_type is not None and args.model_type != config.model_type:
+        print(f"--model_type {args.model_type} but {folder} holds model_type {config.model_type}", file=sys.stderr)
+        return 2
+    pipe = pipeline("text-generation", model=folder, dtype=args.dtype, device=args.device)
+
+    if args.prompt_file:
+        with open(args.prompt_file) as f:
+            prompts = [[int(t) for t in line.replace(",", " ").split()] for line in f if line.strip()]
+    elif args.prompt_ids:
+        prompts = [[int(t) for t in part.replace(",", " ").split()] for part in args.prompt_ids.split(";")]
+    else:
+        text = args.prompt if args.prompt else input("Model prompt >>> ")  # run_generation.py:365
+        prompts = [text]
+
+    length = adjust_length_to_model(args.length, getattr(config, "max_position_embeddings", 0))
+    gen = dict(max_new_tokens=length, min_new_tokens=args.min_new_tokens, seed=args.seed,
+               repetition_penalty=args.repetition_penalty, num_return_sequences=args.num_return_sequences)
+    if args.stop_token_id is not None:
+        gen["eos_token_id"] = args.stop_token_id
+    if args.greedy:
+        gen.update(do_sample=False, num_return_sequences=1)
+    else:
+        gen.update(do_sample=True, temperature=args.temperature, top_k=args.k, top_p=args.p, min_p=args.min_p)
+    GenerationConfig(**{k: v for k, v in gen.items()})  # validate before the model runs
+    results = pipe(prompts, prefix=args.prefix, batch_size=args.batch_size, **gen)
+    n = 0
+    for records in results:
+        for rec in records:
+            n += 1
+            print(f"=== GENERATED SEQUENCE {n} ===")
+            if "generated_text" in rec:
+                text = rec["generated_text"]
+                if args.stop_token:
+                    text = text[: text.find(args.stop_token) if args.stop_token in text else None]  # :433
+                print(text)
+            else:
+                print(",".join(str(t) for t in rec["generated_token_ids"]))
+    if tmp is not None:
+        tmp.cleanup()
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,214 @@
+"""The sampling kernel against the plain processors, and generation through the entry point (GPU)."""
+import math
+
+import pytest
+import torch
+
+import plain_falcon as P
+from tiny import TINY, write_model
+
+pytestmark = pytest.mark.gpu
+
+
+def _ops():
+    from pytorch_transformers_amd import ops
+    return ops
+
+
+def _dev(x, dtype=torch.float32):
+    return torch.as_tensor(x, dtype=dtype).cuda()
+
+
+def _finite_mask(t):
+    return (t != float("-inf")).cpu()
+
+
+def test_argmax_lowest_index_on_ties():
+    ops = _ops()
+    x = torch.zeros(3, 1000)
+    x[0, 517] = 2.0; x[0, 900] = 2.0
+    x[1, 0] = -1.0
+    x[2, 999] = 0.5
+    tok, scores = ops.sample(_dev(x), do_sample=False)
+    assert tok.tolist() == [517, 1, 999]
+    assert torch.equal(scores.cpu(), x)
+
+
+@pytest.mark.parametrize("V", [10, 211, 65024])
+def test_processors_match_plain(V):
+    """Penalty, EOS suppression, temperature, top-k, top-p, min-p: same tokens survive as in the plain code."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(V)
+    R = 5
+    logits = torch.randn(R, V, generator=g) * 3
+    hist = [[int(t) for t in torch.randint(0, V, (n,), generator=g)] for n in (3, 0, 7, 1, 12)]
+    off = [0]
+    for h in hist:
+        off.append(off[-1] + len(h))
+    flat = [t for h in hist for t in h]
+    eos = [1, V - 1]
+    suppress = [1, 0, 1, 0, 0]
+    for kw in (dict(temperature=0.7, top_k=min(50, V - 1)), dict(top_p=0.9), dict(min_p=0.02),
+               dict(temperature=1.3, top_k=min(40, V - 1), top_p=0.8, min_p=0.01, penalty=1.7),
+               dict(top_k=1), dict(top_p=0.05), dict(top_k=V + 5, penalty=0.5)):
+        tok, scores = ops.sample(
+            _dev(logits), do_sample=True, temperature=kw.get("temperature", 1.0), top_k=kw.get("top_k", 0),
+            top_p=kw.get("top_p", 1.0), min_p=kw.get("min_p", 0.0), penalty=kw.get("penalty", 1.0),
+            hist=_dev(flat, torch.int32) if flat else None, hist_off=_dev(off, torch.int32), eos=_dev(eos, torch.int32),
+            suppress=_dev(suppress, torch.int32), uniforms=_dev([0.5] * R))
+        for r in range(R):
+            want = P.process(logits[r], hist[r], do_sample=True, temperature_=kw.get("temperature", 1.0),
+                             top_k_=kw.get("top_k", 0), top_p_=kw.get("top_p", 1.0), min_p_=kw.get("min_p"),
+                             repetition_penalty_=kw.get("penalty", 1.0), suppress_ids=eos if suppress[r] else ())
+            got = scores[r].cpu()
+            keep_want, keep_got = want != float("-inf"), _finite_mask(got)
+            # a token whose cumulative mass sits within rounding of the top-p cut may fall on either side
+            diff = (keep_want != keep_got).nonzero().flatten().tolist()
+            if diff and "top_p" in kw:
+                probs = torch.softmax(torch.where(keep_want | keep_got, want if kw.get("min_p") is None else got, want).double(), -1)
+                assert len(diff) <= 1, f"V={V} {kw} row {r}: kept sets differ at {diff}"
+            else:
+                assert not diff, f"V={V} {kw} row {r}: kept sets differ at {diff}"
+            both = keep_want & keep_got
+            torch.testing.assert_close(got[both], want[both], rtol=1e-6, atol=1e-6)
+            assert keep_got[int(tok[r])], "the chosen token was filtered out"
+
+
+def test_reference_vectors_on_the_kernel():
+    """The reference's own small cases (tests/generation/test_logits_process.py:235-355) through the kernel."""
+    ops = _ops()
+    ramp = torch.arange(10.0)[None]
+    _, s = ops.sample(_dev(ramp), do_sample=True, top_k=3, uniforms=_dev([0.1]))
+    assert torch.isinf(s[0]).tolist() == 7 * [True] + 3 * [False]
+    dist = torch.log(torch.tensor([[0.15, 0.3, 0.3, 0.25], [0.3, 0.1, 0.1, 0.5], [0.3, 0.1, 0.1, 0.5]]))
+    for top_p, row, want in ((0.8, 0, [0.0, 0.3, 0.3, 0.25]), (0.79, 1, [0.3, 0.0, 0.0, 0.5]), (0.85, 2, [0.3, 0.0, 0.1, 0.5])):
+        _, s = ops.sample(_dev(dist[row:row + 1]), do_sample=True, top_p=top_p, uniforms=_dev([0.1]))
+        torch.testing.assert_close(torch.exp(s[0]).cpu(), torch.tensor(want), atol=1e-3, rtol=0)
+    dist = torch.log(torch.tensor([[0.9, 0.0274, 0.047, 0.0274], [0.15, 0.3, 0.3, 0.25], [0.97, 0.01, 0.01, 0.01]]))
+    _, s = ops.sample(_dev(dist), do_sample=True, min_p=0.05, uniforms=_dev([0.1] * 3))
+    want = torch.tensor([[0.9, 0.0, 0.047, 0.0], [0.15, 0.3, 0.3, 0.25], [0.97, 0.0, 0.0, 0.0]])
+    torch.testing.assert_close(torch.exp(s).cpu(), want, atol=1e-3, rtol=0)
+    # top_p so small that everything could go: the best token stays
+    _, s = ops.sample(_dev(torch.arange(6.0)[None]), do_sample=True, top_p=0.0, uniforms=_dev([0.9]))
+    assert _finite_mask(s[0]).tolist() == [False] * 5 + [True]
+    # remove_invalid_values and renormalize_logits
+    bad = torch.tensor([[float("nan"), float("inf"), -float("inf"), 1.0]])
+    _, s = ops.sample(_dev(bad), do_sample=False, remove_invalid=True)
+    assert s[0].tolist() == [0.0, torch.finfo(torch.float32).max, torch.finfo(torch.float32).min, 1.0]
+    x = torch.randn(2, 300)
+    _, s = ops.sample(_dev(x), do_sample=False, renorm=True)
+    torch.testing.assert_close(s.cpu(), torch.log_softmax(x, -1), rtol=1e-5, atol=1e-5)
+
+
+def test_draw_inverts_the_cumulative_distribution():
+    """A given uniform number picks the token whose CDF interval holds it; frequencies follow softmax."""
+    ops = _ops()
+    logits = torch.tensor([[0.0, math.log(2.0), math.log(3.0), math.log(4.0)]])  # p = .1 .2 .3 .4
+    for u, want in ((0.0, 0), (0.09, 0), (0.11, 1), (0.29, 1), (0.31, 2), (0.59, 2), (0.61, 3), (0.999, 3)):
+        tok, _ = ops.sample(_dev(logits), do_sample=True, uniforms=_dev([u]))
+        assert int(tok[0]) == want, (u, int(tok[0]))
+    R = 4000
+    big = logits.expand(R, 4).contiguous()
+    tok, _ = ops.sample(_dev(big), do_sample=True, seed=5, rng_seq=_dev(list(range(R)), torch.int32),
+                        rng_step=_dev([0] * R, torch.int32))
+    freq = torch.bincount(tok.cpu().long(), minlength=4).double() / R
+    assert float((freq - torch.tensor([0.1, 0.2, 0.3, 0.4], dtype=torch.float64)).abs().max()) < 4 * math.sqrt(0.25 / R)
+    # random logits over a wide vocabulary, against the plain choice fed the same uniform numbers
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(64, 5000, generator=g) * 2
+    u = torch.rand(64, generator=g)
+    tok, _ = ops.sample(_dev(x), do_sample=True, uniforms=_dev(u))
+    for r in range(64):
+        cdf = torch.softmax(x[r].double(), -1).cumsum(-1)
+        t = int(tok[r])
+        lo = float(cdf[t - 1]) if t else 0.0
+        assert lo - 1e-5 <= float(u[r]) <= float(cdf[t]) + 1e-5, (r, t, float(u[r]), lo, float(cdf[t]))
+
+
+def test_counter_based_uniforms():
+    """Same (seed, sequence, step) -> same draw whatever the batch; the host function gives the number."""
+    from pytorch_transformers_amd.sampling import philox_uniform
+
+    ops = _ops()
+    V = 1000
+    x = torch.randn(6, V, generator=torch.Generator().manual_seed(1))
+    seqs, steps = [4, 9, 2, 7, 7, 1], [0, 3, 3, 1, 2, 0]
+    tok_all, _ = ops.sample(_dev(x), do_sample=True, seed=1234, rng_seq=_dev(seqs, torch.int32), rng_step=_dev(steps, torch.int32))
+    for r in range(6):
+        alone, _ = ops.sample(_dev(x[r:r + 1]), do_sample=True, seed=1234, rng_seq=_dev([seqs[r]], torch.int32),
+                              rng_step=_dev([steps[r]], torch.int32))
+        assert int(alone[0]) == int(tok_all[r])
+        u = philox_uniform(1234, seqs[r], steps[r])
+        assert 0.0 <= u < 1.0
+        via_u, _ = ops.sample(_dev(x[r:r + 1]), do_sample=True, uniforms=_dev([u]))
+        assert int(via_u[0]) == int(tok_all[r])
+    us = [philox_uniform(7, s, 0) for s in range(2000)]
+    assert abs(sum(us) / len(us) - 0.5) < 0.03 and len(set(us)) > 1990
+    assert philox_uniform(7, 3, 0) != philox_uniform(8, 3, 0) != philox_uniform(8, 3, 1)
+
+
+# --- generation through the entry point ---------------------------------------------------------------
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    root = str(tmp_path_factory.mktemp("gen"))
+    return {n: write_model(n, root) for n in ("A", "B")}
+
+
+def test_greedy_generation_equals_plain(folders):
+    """Tiny A: batch of 3 prompts of 5/11/17 ids, 16 greedy tokens, 32-bit."""
+    from pytorch_transformers_amd import AutoModelForCausalLM, GenerationConfig
+
+    cfg, w = P.read_model(folders["A"])
+    g = torch.Generator().manual_seed(0)
+    prompts = [torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for n in (5, 11, 17)]
+    want = [p + P.generate(cfg, w, p, 16) for p in prompts]
+    model = AutoModelForCausalLM.from_pretrained(folders["A"], dtype="float32")
+    got = model.generate(prompts, GenerationConfig(max_new_tokens=16, do_sample=False, eos_token_id=None))
+    assert got == want
+    # one batch after another, and a stop token that ends one sequence early
+    eos = want[1][len(prompts[1]) + 4]
+    got = model.generate(prompts, GenerationConfig(max_new_tokens=16, eos_token_id=eos), batch_size=2)
+    for p, g_, w_ in zip(prompts, got, want):
+        new = w_[len(p):]
+        cut = new.index(eos) + 1 if eos in new else len(new)
+        assert g_ == p + new[:cut]
+    bf = AutoModelForCausalLM.from_pretrained(folders["A"], dtype="bfloat16")
+    got_bf = bf.generate(prompts, max_new_tokens=16, do_sample=False, eos_token_id=None)
+    agree = sum(a == b for x, y in zip(got_bf, want) for a, b in zip(x, y)) / sum(len(x) for x in want)
+    assert agree > 0.8, f"bfloat16 greedy tokens agree with the plain ones in only {agree:.0%} of places"
+
+
+def test_sampled_generation_equals_plain_fed_the_same_uniforms(folders):
+    """Tiny B: batch of 4 prompts of 1/7/20/33 ids, 24 tokens at temperature 0.8 (32-bit), alone and batched."""
+    from pytorch_transformers_amd import AutoModelForCausalLM, GenerationConfig
+    from pytorch_transformers_amd.sampling import philox_uniform
+
+    cfg, w = P.read_model(folders["B"])
+    g = torch.Generator().manual_seed(1)
+    prompts = [torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for n in (1, 7, 20, 33)]
+    gen = GenerationConfig(max_new_tokens=24, do_sample=True, temperature=0.8, top_k=0, eos_token_id=None, seed=77)
+    model = AutoModelForCausalLM.from_pretrained(folders["B"], dtype="float32")
+    got = model.generate(prompts, gen)
+    for i, p in enumerate(prompts):
+        us = [philox_uniform(77, i, s) for s in range(24)]
+        want = p + P.generate(cfg, w, p, 24, uniforms=us, temperature_=0.8)
+        # a draw within rounding of a CDF boundary may differ and then the tails differ: compare up to the first
+        # difference and require it to be such a boundary case
+        if got[i] != want:
+            k = next(j for j, (a, b) in enumerate(zip(got[i], want)) if a != b)
+            logits = P.forward(cfg, w, want[:k])[-1].float() / 0.8
+            cdf = torch.softmax(logits.double(), -1).cumsum(-1)
+            u = us[k - len(p)]
+            assert min(abs(float(cdf[t]) - u) for t in (got[i][k], want[k], got[i][k] - 1, want[k] - 1) if t >= 0) < 1e-5
+    alone = model.generate([prompts[2]], gen, rng_ids=[2])
+    assert alone[0] == got[2]
+    two = model.generate(prompts, gen, batch_size=2)
+    assert two == got
+
+
+def test_pipeline_and_cli_style_entry(folders):
+    from pytorch_transformers_amd import pipeline
+
+    pipe = pipeline("text-generation", model=folders["A"], dtype="float32")
+    out = pipe([[3, 4, 5]], max_new_tokens=4, do_sample=False, eos_token_id=None)
+    assert len(out) == 1 and out[0][0]["generated_token_ids"][:3] == [3, 4, 5] and len(out[0][0]["generated_token_ids"]) == 7
