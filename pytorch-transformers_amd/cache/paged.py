@@ -16,7 +16,8 @@ ends and are handed out again; nothing is zeroed, because a slot's length says
 what is valid.  Groups of kind ``state`` own a ``[max_slots, *shape]`` table per
 layer that is zeroed when a slot is handed out.
 
-K and V pools have the layout ``[layer, page, kv_head, page_size, head_dim]``.
+The K pool has the layout ``[layer, page, kv_head, page_size, head_dim]``, the V pool
+``[layer, page, kv_head, head_dim, page_size]``.
 """
 from __future__ import annotations
 
@@ -83,9 +84,12 @@ class _Group:
         self.state: Optional[torch.Tensor] = None
         self.pages: Optional[_FreeList] = None
         if spec.kind == CACHE_FULL:
-            shape = (spec.num_layers, num_pages, spec.kv_heads, page_size, spec.head_dim)
-            self.k = torch.empty(shape, dtype=dtype, device=device)
-            self.v = torch.empty(shape, dtype=dtype, device=device)
+            # values are held transposed inside a page so that the attention kernels read eight
+            # consecutive positions of one feature in one load
+            self.k = torch.zeros((spec.num_layers, num_pages, spec.kv_heads, page_size, spec.head_dim),
+                                 dtype=dtype, device=device)
+            self.v = torch.zeros((spec.num_layers, num_pages, spec.kv_heads, spec.head_dim, page_size),
+                                 dtype=dtype, device=device)
             self.pages = _FreeList(num_pages, f"page of cache group {spec.name!r}")
         elif spec.kind == CACHE_STATE:
             sd = spec.state_dtype or torch.float32

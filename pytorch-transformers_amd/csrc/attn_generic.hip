@@ -60,7 +60,7 @@ __global__ void attn_generic_kernel(T* __restrict__ out, const T* __restrict__ q
             const int dim = lane + r * PTA_WAVE;
             if (dim < d) {
                 float a = acc[r] * corr;
-                for (int jj = 0; jj < cnt; ++jj) a += p_s[jj] * Io<T>::ld(vp + (long)jj * d + dim);
+                for (int jj = 0; jj < cnt; ++jj) a += p_s[jj] * Io<T>::ld(vp + (long)dim * PTA_PAGE + jj);
                 acc[r] = a;
             }
         }

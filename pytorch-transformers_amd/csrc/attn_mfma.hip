@@ -1,0 +1,290 @@
+// Causal attention over the paged cache on the matrix cores, bfloat16 in, 32-bit softmax and
+// accumulation: the prefill kernel and the decode kernel are the same code.
+//
+// Work is laid out in *columns*: a column is one (new token, query head) pair of one KV head of one
+// sequence, ordered token-major.  Heads that share a KV head therefore sit side by side and read
+// its keys and values once: with one KV head for 71 query heads, a decode step's 71 columns are five
+// tiles of 16 that share every key load.  A wave owns CT column tiles and walks the keys 32 at a
+// time:
+//
+//   S^T[32 keys x 16 cols]  = K[32 x d] . Q^T[d x 16]         (A = key rows, B = query columns)
+//   online softmax over keys, per column (statistics in 32-bit, four lanes hold a column)
+//   O^T[d x 16 cols]       += V^T[d x 32 keys] . P^T[32 x 16]  (A = value pages, stored transposed)
+//
+// The score tile's accumulator layout (lane: column = lane % 16, four consecutive rows at
+// (lane / 16) * 4) is turned into the B operand of the second product without leaving registers:
+// key rows are assigned to the two 16-row score tiles so that a lane ends up with the eight
+// consecutive keys 8 * (lane / 16) .. + 7 of the block, which is what the B operand wants.
+//
+// Decoding splits a long context over several waves (split_size keys each, a function of the
+// context alone); each writes an unnormalised partial result with its running maximum and sum, and
+// attn_combine merges them in split order.  Prefill uses one wave per column group and no split.
+//
+// score = q . k / sqrt(d) + alibi, alibi = bf16(bf16(slope) * bf16(key position)) / sqrt(d)
+// (src/transformers/models/falcon/modeling_falcon.py:371-386, :407-422, :196-198, :1078-1085).
+#include "common.h"
+#include "pta_kernels.h"
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+union AFrag {
+    uint4 u;
+    bf16x8_t v;
+};
+
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+}
+
+template <int DT, int CT>
+__global__ __launch_bounds__(64) void attn_mfma_kernel(
+    bf16_t* __restrict__ out, float* __restrict__ po, float* __restrict__ pm, float* __restrict__ pl,
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
+    const int* __restrict__ block_table, int bt_stride, const int* __restrict__ cu_tokens,
+    const int* __restrict__ seq_start, const float* __restrict__ slopes, int nh, int nkv, float scale, float sqrt_d,
+    int split_size, int n_splits) {
+    constexpr int D = DT * 16;
+    constexpr int DS = (DT + 1) / 2;   // 32-wide steps over the head dimension
+    constexpr int CHUNKS = D / 8;      // 16-byte chunks in a row of d elements
+    const int lane = threadIdx.x, c = lane & 15, gq = lane >> 4;
+    const int seq = blockIdx.z / n_splits, split = blockIdx.z % n_splits;
+    const int kvh = blockIdx.y, g = nh / nkv;
+    const int t0 = cu_tokens[seq], n_new = cu_tokens[seq + 1] - t0, start = seq_start[seq];
+    const int ncols = n_new * g, col0 = blockIdx.x * (16 * CT);
+    if (col0 >= ncols) return;
+    const int last_col = min(ncols, col0 + 16 * CT) - 1;
+    const int max_qpos = start + last_col / g;
+    const int kv_len = start + n_new;
+    const int k_begin = n_splits > 1 ? split * split_size : 0;
+    const int k_end = n_splits > 1 ? min(max_qpos + 1, k_begin + split_size) : max_qpos + 1;
+    const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
+
+    int qpos[CT], tok[CT], head[CT];
+    float slope[CT];
+    AFrag qf[CT][DS];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        const int col = col0 + ct * 16 + c;
+        const int colc = min(col, ncols - 1);
+        const int t = colc / g;
+        tok[ct] = t0 + t;
+        head[ct] = kvh * g + colc % g;
+        qpos[ct] = col < ncols ? start + t : -1;  // -1: every key is masked for a column that does not exist
+        slope[ct] = slopes ? slopes[head[ct]] : 0.f;
+        const bf16_t* qp = q + ((long)tok[ct] * nh + head[ct]) * D;
+#pragma unroll
+        for (int ds = 0; ds < DS; ++ds) {
+            const int chunk = ds * 4 + gq;
+            qf[ct][ds].u = *reinterpret_cast<const uint4*>(qp + min(chunk, CHUNKS - 1) * 8);
+            if (chunk >= CHUNKS) qf[ct][ds].u = zero4;
+        }
+    }
+
+    f32x4_t oacc[DT][CT];
+    float m_run[CT], l_run[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        m_run[ct] = -INFINITY;
+        l_run[ct] = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) oacc[dt][ct] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
+
+    const int* bt = block_table + (long)seq * bt_stride;
+    for (int kb = k_begin; kb < k_end; kb += 32) {
+        const long page = bt[kb >> 6];
+        const int in_page = kb & 63;
+        const bf16_t* kpage = k_pool + (page * nkv + kvh) * (long)(PTA_PAGE * D);
+        const bf16_t* vpage = v_pool + (page * nkv + kvh) * (long)(PTA_PAGE * D);
+
+        // key rows: tile tt, row r holds key 8*(r/4) + 4*tt + r%4 of the block
+        AFrag kf[2][DS];
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt) {
+            const bf16_t* kp = kpage + (long)(in_page + 8 * (c >> 2) + 4 * tt + (c & 3)) * D;
+#pragma unroll
+            for (int ds = 0; ds < DS; ++ds) {
+                const int chunk = ds * 4 + gq;
+                kf[tt][ds].u = *reinterpret_cast<const uint4*>(kp + min(chunk, CHUNKS - 1) * 8);
+                if (chunk >= CHUNKS) kf[tt][ds].u = zero4;
+            }
+        }
+        // value rows: feature dt*16 + c, keys 8*gq .. 8*gq+7 of the block
+        AFrag vf[DT];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+            vf[dt].u = *reinterpret_cast<const uint4*>(vpage + (long)(dt * 16 + c) * PTA_PAGE + in_page + gq * 8);
+        if (kb + 32 > kv_len) {
+            // positions past the sequence's end were never written; whatever lies there must not reach
+            // the sum, not even with weight zero
+            const int kbase = kb + gq * 8;
+            uint32_t mk[4];
+#pragma unroll
+            for (int w = 0; w < 4; ++w)
+                mk[w] = (kbase + 2 * w < kv_len ? 0x0000ffffu : 0u) | (kbase + 2 * w + 1 < kv_len ? 0xffff0000u : 0u);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                vf[dt].u.x &= mk[0]; vf[dt].u.y &= mk[1]; vf[dt].u.z &= mk[2]; vf[dt].u.w &= mk[3];
+            }
+        }
+
+        f32x4_t sacc[2][CT];
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) {
+                sacc[tt][ct] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ds = 0; ds < DS; ++ds)
+                    sacc[tt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[tt][ds].v, qf[ct][ds].v, sacc[tt][ct], 0, 0, 0);
+            }
+
+        AFrag pf[CT];
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            float s[8];
+            float mx = -INFINITY;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int key = kb + 8 * gq + j;  // j = 4*tt + e
+                float v = sacc[j >> 2][ct][j & 3] * scale;
+                if (slopes) v += round_to_bf16(slope[ct] * round_to_bf16((float)key)) / sqrt_d;
+                s[j] = key <= qpos[ct] ? v : -INFINITY;
+                mx = fmaxf(mx, s[j]);
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float m_new = fmaxf(m_run[ct], mx);
+            const float m_use = m_new == -INFINITY ? 0.f : m_new;
+            const float corr = expf(m_run[ct] - m_use);
+            float p[8], psum = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                p[j] = expf(s[j] - m_use);
+                psum += p[j];
+            }
+            l_run[ct] = l_run[ct] * corr + psum;
+            m_run[ct] = m_new;
+            pf[ct].u = make_uint4(pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7]));
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                oacc[dt][ct][0] *= corr; oacc[dt][ct][1] *= corr; oacc[dt][ct][2] *= corr; oacc[dt][ct][3] *= corr;
+            }
+        }
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct)
+                oacc[dt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt].v, pf[ct].v, oacc[dt][ct], 0, 0, 0);
+    }
+
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        float l = l_run[ct];
+        l += __shfl_xor(l, 16, 64);
+        l += __shfl_xor(l, 32, 64);
+        if (qpos[ct] < 0) continue;
+        const long row = (long)tok[ct] * nh + head[ct];
+        if (n_splits == 1) {
+            const float inv = 1.0f / l;
+            bf16_t* o = out + row * D;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                uint2 w;
+                w.x = pack_bf16(oacc[dt][ct][0] * inv, oacc[dt][ct][1] * inv);
+                w.y = pack_bf16(oacc[dt][ct][2] * inv, oacc[dt][ct][3] * inv);
+                *reinterpret_cast<uint2*>(o + dt * 16 + gq * 4) = w;
+            }
+        } else {
+            float* o = po + (row * n_splits + split) * D;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+                *reinterpret_cast<float4*>(o + dt * 16 + gq * 4) =
+                    make_float4(oacc[dt][ct][0], oacc[dt][ct][1], oacc[dt][ct][2], oacc[dt][ct][3]);
+            if (gq == 0) {
+                pm[row * n_splits + split] = m_run[ct];
+                pl[row * n_splits + split] = l;
+            }
+        }
+    }
+}
+
+// out[row, :] = sum_s w_s po[row, s, :] / sum_s w_s pl[row, s], w_s = exp(pm[row, s] - max_s pm), splits in order
+__global__ void attn_combine_kernel(bf16_t* __restrict__ out, const float* __restrict__ po, const float* __restrict__ pm,
+                                    const float* __restrict__ pl, int D, int n_splits) {
+    const long row = blockIdx.x;
+    const float* m = pm + row * n_splits;
+    const float* l = pl + row * n_splits;
+    float mx = -INFINITY;
+    for (int s = 0; s < n_splits; ++s) mx = fmaxf(mx, m[s]);
+    float L = 0.f;
+    for (int s = 0; s < n_splits; ++s) L += (m[s] == -INFINITY ? 0.f : expf(m[s] - mx)) * l[s];
+    const float inv = 1.0f / L;
+    for (int dd = threadIdx.x; dd < D; dd += blockDim.x) {
+        float acc = 0.f;
+        for (int s = 0; s < n_splits; ++s) {
+            const float w = m[s] == -INFINITY ? 0.f : expf(m[s] - mx);
+            acc += w * po[(row * n_splits + s) * D + dd];
+        }
+        out[row * D + dd] = f32_to_bf16_bits(acc * inv);
+    }
+}
+
+template <int DT, int CT>
+static void launch_attn(bf16_t* out, float* po, float* pm, float* pl, const bf16_t* q, const bf16_t* k_pool,
+                        const bf16_t* v_pool, const int* block_table, int bt_stride, const int* cu_tokens,
+                        const int* seq_start, const float* slopes, int n_seqs, int max_new, int nh, int nkv, float scale,
+                        int split_size, int n_splits, hipStream_t s) {
+    const int g = nh / nkv;
+    const dim3 grid((max_new * g + 16 * CT - 1) / (16 * CT), nkv, n_seqs * n_splits);
+    hipLaunchKernelGGL((attn_mfma_kernel<DT, CT>), grid, dim3(64), 0, s, out, po, pm, pl, q, k_pool, v_pool, block_table,
+                       bt_stride, cu_tokens, seq_start, slopes, nh, nkv, scale, sqrtf((float)(DT * 16)), split_size,
+                       n_splits);
+}
+
+extern "C" int pta_attn_mfma_supported(int d) { return d % 16 == 0 && ((d >= 16 && d <= 128) || d == 256); }
+
+extern "C" int pta_attn_mfma(void* out, const void* q, const void* k_pool, const void* v_pool, const int* block_table,
+                             int bt_stride, const int* cu_tokens, const int* seq_start, const float* slopes, int n_seqs,
+                             int max_new, int M, int nh, int nkv, int d, float scale, int split_size, int n_splits,
+                             float* po, float* pm, float* pl, void* stream) {
+    PTA_REQUIRE(n_seqs > 0 && max_new > 0 && M > 0 && nh > 0 && nkv > 0, "attn_mfma: sizes must be positive");
+    PTA_REQUIRE(nh % nkv == 0, "attn_mfma: heads (%d) must be a multiple of kv heads (%d)", nh, nkv);
+    PTA_REQUIRE(pta_attn_mfma_supported(d), "attn_mfma: head size %d is not built (16..128 in steps of 16, or 256)", d);
+    PTA_REQUIRE(n_splits >= 1, "attn_mfma: n_splits must be at least 1");
+    PTA_REQUIRE(n_splits == 1 || (split_size > 0 && split_size % 64 == 0 && po && pm && pl),
+                "attn_mfma: splitting needs a split size that is a multiple of 64 and buffers for partial results");
+    PTA_REQUIRE((long)n_seqs * n_splits <= 65535 && nkv <= 65535, "attn_mfma: too many sequences x splits for one launch");
+    PTA_REQUIRE(((uintptr_t)q % 16) == 0 && ((uintptr_t)k_pool % 16) == 0 && ((uintptr_t)v_pool % 16) == 0 &&
+                    ((uintptr_t)out % 8) == 0, "attn_mfma: pointers must be 16-byte aligned");
+    hipStream_t s = (hipStream_t)stream;
+#define PTA_ATTN_CASE(DT_, CT_)                                                                                     \
+    case DT_:                                                                                                       \
+        launch_attn<DT_, CT_>((bf16_t*)out, po, pm, pl, (const bf16_t*)q, (const bf16_t*)k_pool,                    \
+                              (const bf16_t*)v_pool, block_table, bt_stride, cu_tokens, seq_start, slopes, n_seqs,  \
+                              max_new, nh, nkv, scale, split_size, n_splits, s);                                    \
+        break;
+    switch (d / 16) {
+        PTA_ATTN_CASE(1, 4)
+        PTA_ATTN_CASE(2, 4)
+        PTA_ATTN_CASE(3, 4)
+        PTA_ATTN_CASE(4, 4)
+        PTA_ATTN_CASE(5, 2)
+        PTA_ATTN_CASE(6, 2)
+        PTA_ATTN_CASE(7, 2)
+        PTA_ATTN_CASE(8, 2)
+        PTA_ATTN_CASE(16, 1)
+        default:
+            return pta_fail("attn_mfma: head size %d is not built", d);
+    }
+#undef PTA_ATTN_CASE
+    int rc = pta_check_launch("attn_mfma");
+    if (rc) return rc;
+    if (n_splits > 1) {
+        hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)((long)M * nh)), dim3(64), 0, s, (bf16_t*)out, po, pm, pl, d,
+                           n_splits);
+        rc = pta_check_launch("attn_combine");
+    }
+    return rc;
+}

@@ -1,0 +1,212 @@
+// y[M,N] = act(x[M,K] . W[N,K]^T + bias) + add1 + add2 for few rows (M <= 64), bfloat16 in,
+// 32-bit accumulation on the matrix cores.  This is the decode step's linear layer: the work is
+// reading W once from HBM, so the kernel is laid out for that, not for the arithmetic.
+//
+// A workgroup of S waves owns 16*RT rows of W and all of K.  Its waves take the 64-element K-steps
+// round robin (wave w: steps w, w + S, ...), so neighbouring waves read neighbouring 128-byte lines
+// of the same rows.  A wave works in stages of U steps and always has the next stage's loads in
+// flight while the matrix cores consume the current one (two register buffers), so every wave
+// keeps 2*U*RT KB of W on its way from HBM for as long as it runs.  W rows are the A operand of
+// v_mfma_f32_16x16x32_bf16 (lane: row = lane % 16, eight consecutive k at (lane / 16) * 8, one
+// 16-byte load straight from global memory), x rows are the B operand (same shape, read through
+// the caches; x is small).  The S partial tiles are summed through LDS in wave order, then bias,
+// activation and additions are applied and the tile is stored.  S is chosen from N and K alone, so
+// the order of summation never depends on M or on what else is in the batch.
+#include "common.h"
+#include "pta_kernels.h"
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+union Frag {
+    uint4 u;
+    bf16x8_t v;
+};
+
+template <typename OutT> struct OutIo;
+template <> struct OutIo<float> {
+    static __device__ __forceinline__ float round(float v) { return v; }
+    static __device__ __forceinline__ void st(float* p, float v) { *p = v; }
+};
+template <> struct OutIo<bf16_t> {
+    static __device__ __forceinline__ float round(float v) { return round_to_bf16(v); }
+    static __device__ __forceinline__ void st(bf16_t* p, float v) { *p = f32_to_bf16_bits(v); }
+};
+
+template <int MT, int RT, int U>
+struct Stage {
+    Frag a[U][2][RT];
+    Frag b[U][2][MT];
+    uint32_t keep[U][2];  // all ones if the chunk lies inside K, else zero
+};
+
+// Loads are unconditional: the address is clamped into the row, and the data of a chunk past K is
+// masked to zero only when it is used.  A load under a branch, or a mask applied here, would make
+// the wave wait for loads it has just issued, and the two stages would no longer overlap.
+template <int MT, int RT, int U>
+__device__ __forceinline__ void load_stage(Stage<MT, RT, U>& st, const bf16_t* const (&wrow)[RT],
+                                           const bf16_t* const (&xrow)[MT], int first_step, int S, int g, int K) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const int k0 = (first_step + u * S) * 64 + g * 8;  // K % 8 == 0: a chunk of 8 is inside K or outside it
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+            const int k = k0 + hf * 32;
+            const int kc = min(k, K - 8);
+            st.keep[u][hf] = k < K ? 0xffffffffu : 0u;
+#pragma unroll
+            for (int t = 0; t < RT; ++t) st.a[u][hf][t].u = *reinterpret_cast<const uint4*>(wrow[t] + kc);
+#pragma unroll
+            for (int t = 0; t < MT; ++t) st.b[u][hf][t].u = *reinterpret_cast<const uint4*>(xrow[t] + kc);
+        }
+    }
+}
+
+template <int MT, int RT, int U>
+__device__ __forceinline__ void compute_stage(const Stage<MT, RT, U>& st, f32x4_t (&acc)[RT][MT]) {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                Frag a = st.a[u][hf][rt];
+                const uint32_t keep = st.keep[u][hf];
+                a.u.x &= keep; a.u.y &= keep; a.u.z &= keep; a.u.w &= keep;
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+                    acc[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, st.b[u][hf][mt].v, acc[rt][mt], 0, 0, 0);
+            }
+}
+
+template <int MT, int RT, int U, typename OutT>
+__global__ __launch_bounds__(512) void gemm_skinny_kernel(
+    OutT* __restrict__ y, const bf16_t* __restrict__ x, const bf16_t* __restrict__ W, const float* __restrict__ bias,
+    const bf16_t* __restrict__ add1, const bf16_t* __restrict__ add2, int M, int N, int K, int act) {
+    extern __shared__ f32x4_t part[];  // [S][RT][MT][64]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, S = blockDim.x >> 6;
+    const int r = lane & 15, g = lane >> 4;
+    const int n0 = blockIdx.x * (16 * RT);
+    const bf16_t* wrow[RT];
+#pragma unroll
+    for (int t = 0; t < RT; ++t) wrow[t] = W + (long)min(n0 + t * 16 + r, N - 1) * K;
+    const bf16_t* xrow[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) xrow[t] = x + (long)min(t * 16 + r, M - 1) * K;
+
+    f32x4_t acc[RT][MT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[rt][mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    const int nsteps = (K + 63) >> 6;
+    Stage<MT, RT, U> s0, s1;
+    load_stage<MT, RT, U>(s0, wrow, xrow, wave, S, g, K);
+    // the scheduling barriers keep the compiler from sinking a stage's loads down to their first
+    // use, which would shrink what is in flight to a load or two
+    for (int step = wave; step < nsteps; step += 2 * U * S) {
+        load_stage<MT, RT, U>(s1, wrow, xrow, step + U * S, S, g, K);
+        __builtin_amdgcn_sched_barrier(0);
+        compute_stage<MT, RT, U>(s0, acc);
+        __builtin_amdgcn_sched_barrier(0);
+        load_stage<MT, RT, U>(s0, wrow, xrow, step + 2 * U * S, S, g, K);
+        __builtin_amdgcn_sched_barrier(0);
+        compute_stage<MT, RT, U>(s1, acc);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) part[((wave * RT + rt) * MT + mt) * 64 + lane] = acc[rt][mt];
+    __syncthreads();
+
+    // item (rt, mt, ln): outputs of row m = mt*16 + ln%16, columns n0 + rt*16 + (ln/16)*4 + 0..3
+    for (int item = threadIdx.x; item < RT * MT * 64; item += blockDim.x) {
+        const int ln = item & 63, mt = (item >> 6) % MT, rt = (item >> 6) / MT;
+        f32x4_t sum = part[(rt * MT + mt) * 64 + ln];
+        for (int w = 1; w < S; ++w) {
+            const f32x4_t p = part[((w * RT + rt) * MT + mt) * 64 + ln];
+            sum[0] += p[0]; sum[1] += p[1]; sum[2] += p[2]; sum[3] += p[3];
+        }
+        const int m = mt * 16 + (ln & 15);
+        if (m >= M) continue;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int n = n0 + rt * 16 + (ln >> 4) * 4 + i;
+            if (n < N) {
+                float v = OutIo<OutT>::round(sum[i]);
+                if (bias) v = OutIo<OutT>::round(v + bias[n]);
+                if (act == PTA_ACT_GELU) v = gelu_erf(v);
+                const long o = (long)m * N + n;
+                if (add1) v += bf16_bits_to_f32(add1[o]);
+                if (add2) v += bf16_bits_to_f32(add2[o]);
+                OutIo<OutT>::st(y + o, v);
+            }
+        }
+    }
+}
+
+// Waves per workgroup, i.e. how many ways K is split.  Measured on MI355X: long streams per wave beat
+// many short ones, so K is split only when N alone gives too few waves.  It depends on N only, never
+// on M or on the tile variant, so the order of summation is the same for every batch.
+static int pick_split(int N) {
+    const int groups = (N + 31) / 32;
+    if (groups >= 512) return 1;
+    if (groups >= 128) return 2;
+    if (groups >= 32) return 4;
+    return 8;
+}
+
+template <int MT, int RT, int U, typename OutT>
+static void launch_cfg(OutT* y, const bf16_t* x, const bf16_t* W, const float* bias, const bf16_t* add1,
+                       const bf16_t* add2, int M, int N, int K, int act, int S, hipStream_t s) {
+    const int rows = 16 * RT;
+    if (S <= 0) S = pick_split(N);
+    const dim3 grid((N + rows - 1) / rows), block(S * 64);
+    const size_t lds = (size_t)S * RT * MT * 64 * sizeof(f32x4_t);
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, U, OutT>), grid, block, lds, s, y, x, W, bias, add1, add2, M, N, K,
+                       act);
+}
+
+template <typename OutT>
+static int launch_skinny(OutT* y, const bf16_t* x, const bf16_t* W, const float* bias, const bf16_t* add1,
+                         const bf16_t* add2, int M, int N, int K, int act, int variant, int S, hipStream_t s) {
+    // variant: row tiles per wave and steps per stage; 0: chosen here
+    if (M <= 16) {
+        if (variant == 0) variant = 2;
+        if (variant == 1) launch_cfg<1, 1, 4, OutT>(y, x, W, bias, add1, add2, M, N, K, act, S, s);
+        else if (variant == 2) launch_cfg<1, 2, 2, OutT>(y, x, W, bias, add1, add2, M, N, K, act, S, s);
+        else if (variant == 3) launch_cfg<1, 4, 1, OutT>(y, x, W, bias, add1, add2, M, N, K, act, S, s);
+        else launch_cfg<1, 4, 2, OutT>(y, x, W, bias, add1, add2, M, N, K, act, S, s);
+    } else if (M <= 32) {
+        if (variant == 3 || variant == 4) launch_cfg<2, 4, 1, OutT>(y, x, W, bias, add1, add2, M, N, K, act, S, s);
+        else launch_cfg<2, 2, 1, OutT>(y, x, W, bias, add1, add2, M, N, K, act, S, s);
+    } else if (M <= 48) {
+        launch_cfg<3, 2, 1, OutT>(y, x, W, bias, add1, add2, M, N, K, act, S, s);
+    } else {
+        if (variant == 3 || variant == 4) launch_cfg<4, 4, 1, OutT>(y, x, W, bias, add1, add2, M, N, K, act, S, s);
+        else launch_cfg<4, 2, 1, OutT>(y, x, W, bias, add1, add2, M, N, K, act, S, s);
+    }
+    return pta_check_launch("gemm_skinny_bf16");
+}
+
+extern "C" int pta_gemm_skinny_bf16(void* y, const void* x, const void* W, const float* bias, const void* add1,
+                                    const void* add2, int M, int N, int K, int act, int out_f32, int variant,
+                                    int waves, void* stream) {
+    PTA_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_skinny_bf16: sizes must be positive (M=%d N=%d K=%d)", M, N, K);
+    PTA_REQUIRE(M <= 64, "gemm_skinny_bf16: at most 64 rows, got %d (use the library product)", M);
+    PTA_REQUIRE(K % 8 == 0, "gemm_skinny_bf16: K=%d must be a multiple of 8 (16-byte loads)", K);
+    PTA_REQUIRE(y && x && W, "gemm_skinny_bf16: null pointer");
+    PTA_REQUIRE(((uintptr_t)x % 16) == 0 && ((uintptr_t)W % 16) == 0, "gemm_skinny_bf16: x and W must be 16-byte aligned");
+    PTA_REQUIRE(act == PTA_ACT_NONE || act == PTA_ACT_GELU, "gemm_skinny_bf16: unknown activation %d", act);
+    PTA_REQUIRE(variant >= 0 && variant <= 4, "gemm_skinny_bf16: unknown variant %d", variant);
+    PTA_REQUIRE(waves == 0 || (waves >= 1 && waves <= 8 && (waves & (waves - 1)) == 0),
+                "gemm_skinny_bf16: waves per workgroup must be 0 (choose) or a power of two up to 8, got %d", waves);
+    hipStream_t s = (hipStream_t)stream;
+    if (out_f32)
+        return launch_skinny<float>((float*)y, (const bf16_t*)x, (const bf16_t*)W, bias, (const bf16_t*)add1,
+                                    (const bf16_t*)add2, M, N, K, act, variant, waves, s);
+    return launch_skinny<bf16_t>((bf16_t*)y, (const bf16_t*)x, (const bf16_t*)W, bias, (const bf16_t*)add1,
+                                 (const bf16_t*)add2, M, N, K, act, variant, waves, s);
+}

@@ -7,8 +7,9 @@
 // [tokens, features].  A function returns 0, or non-zero after storing a message
 // that pta_last_error() returns; shapes are checked on the host before a launch.
 //
-// Cache pools have the layout [page, kv_head, 64, head_dim]; `block_table` is
-// [sequences in the step, bt_stride] and lists each sequence's pages in order.
+// Key pools have the layout [page, kv_head, 64, head_dim]; value pools are transposed within a page,
+// [page, kv_head, head_dim, 64].  `block_table` is [sequences in the step, bt_stride] and lists each
+// sequence's pages in order.
 #pragma once
 
 #include <stdint.h>
@@ -45,9 +46,24 @@ int pta_attn_generic(void* out, const void* q, const void* k_pool, const void* v
                      int bt_stride, const int* token_seq, const int* token_pos, const float* slopes, int M, int nh,
                      int nkv, int d, float scale, int dtype, void* stream);
 
+// the same attention for bfloat16 on the matrix cores; cu_tokens [n_seqs + 1] and seq_start [n_seqs] say
+// which tokens are whose and how long each sequence was before the step; max_new bounds a sequence's new
+// tokens.  n_splits > 1 (decode): keys are cut into ranges of split_size, partial results go to
+// po [M, nh, n_splits, d], pm and pl [M, nh, n_splits] (32-bit) and are merged in split order.
+int pta_attn_mfma_supported(int d);
+int pta_attn_mfma(void* out, const void* q, const void* k_pool, const void* v_pool, const int* block_table,
+                  int bt_stride, const int* cu_tokens, const int* seq_start, const float* slopes, int n_seqs,
+                  int max_new, int M, int nh, int nkv, int d, float scale, int split_size, int n_splits, float* po,
+                  float* pm, float* pl, void* stream);
+
 // C = act(A . W^T + bias) + add1 + add2, all 32-bit, fixed summation order
 int pta_gemm_f32(float* C, const float* A, const float* W, const float* bias, const float* add1, const float* add2,
                  int M, int N, int K, int act, void* stream);
+
+// y = act(x . W^T + bias) + add1 + add2 for M <= 64 rows of bfloat16; y is bfloat16, or 32-bit if out_f32.
+// variant and waves are tuning knobs (0: chosen from N and K): row tiles per wave, waves per workgroup
+int pta_gemm_skinny_bf16(void* y, const void* x, const void* W, const float* bias, const void* add1, const void* add2,
+                         int M, int N, int K, int act, int out_f32, int variant, int waves, void* stream);
 
 // processors in the reference's order, then argmax (do_sample 0) or a draw; `work` [R, V] receives the
 // processed scores; hist/hist_off (tokens seen, per row), eos/suppress, uniforms may be null

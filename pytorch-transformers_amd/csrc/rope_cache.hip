@@ -8,6 +8,7 @@
 //   interleaved  per head h: q_h, k_h, v_h
 // Rotation pairs element i with i + d/2 (rotate_half, :76-80; apply :104-108); the angle is
 // position * inv_freq[i], taken in 32-bit (:155-164).  Keys are stored rotated (:350-358).
+// Key pages are [kv_head][64 positions][d]; value pages are transposed, [kv_head][d][64 positions].
 #include "common.h"
 #include "pta_kernels.h"
 
@@ -41,13 +42,18 @@ __global__ void qkv_rope_cache_kernel(T* __restrict__ q_out, const T* __restrict
 
     const int pos = token_pos[m];
     T* dst;
+    long dst_stride = 1;  // values are stored transposed, [d][64], so that eight keys of one feature are contiguous
     if (kind == 0) {
         dst = q_out + ((long)m * nh + head) * d;
     } else {
         const int seq = token_seq[m];
         const long page = block_table[(long)seq * bt_stride + pos / PTA_PAGE];
-        T* pool = kind == 1 ? k_pool : v_pool;
-        dst = pool + ((page * nkv + head) * PTA_PAGE + (pos % PTA_PAGE)) * (long)d;
+        if (kind == 1) {
+            dst = k_pool + ((page * nkv + head) * PTA_PAGE + (pos % PTA_PAGE)) * (long)d;
+        } else {
+            dst = v_pool + (page * nkv + head) * (long)PTA_PAGE * d + (pos % PTA_PAGE);
+            dst_stride = PTA_PAGE;
+        }
     }
 
     if (kind != 2 && inv_freq) {
@@ -64,7 +70,7 @@ __global__ void qkv_rope_cache_kernel(T* __restrict__ q_out, const T* __restrict
         for (int i = threadIdx.x; i < d; i += blockDim.x) {
             float a = Io<T>::ld(src + i);
             if (bsrc) a = Io<T>::round(a + bsrc[i]);
-            Io<T>::st(dst + i, a);
+            Io<T>::st(dst + i * dst_stride, a);
         }
     }
 }

@@ -97,6 +97,16 @@ def _need(t: torch.Tensor, name: str, dtype=None, shape=None) -> None:
         raise KernelError(f"{name} must have shape {tuple(shape)}, got {tuple(t.shape)}")
 
 
+def _need_pools(k_pool, v_pool, dtype, nkv: int, d: int) -> None:
+    """Key pages are [pages, kv_heads, 64, d]; value pages are transposed, [pages, kv_heads, d, 64]."""
+    _need(k_pool, "k_pool", dtype)
+    _need(v_pool, "v_pool", dtype)
+    if tuple(k_pool.shape[1:]) != (nkv, 64, d) or k_pool.dim() != 4:
+        raise KernelError(f"k_pool must be [pages, {nkv}, 64, {d}], got {tuple(k_pool.shape)}")
+    if tuple(v_pool.shape) != (k_pool.shape[0], nkv, d, 64):
+        raise KernelError(f"v_pool must be [{k_pool.shape[0]}, {nkv}, {d}, 64], got {tuple(v_pool.shape)}")
+
+
 # ---------------------------------------------------------------------------
 def embed(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out[m] = table[ids[m]].  The caller has checked that ids lie in [0, rows)."""
@@ -168,10 +178,7 @@ def qkv_rope_cache(fused: torch.Tensor, bias, inv_freq, cs_scale: float, token_p
     _need(block_table, "block_table", torch.int32)
     if block_table.dim() != 2:
         raise KernelError("block_table must be [sequences, pages]")
-    for name, pool in (("k_pool", k_pool), ("v_pool", v_pool)):
-        _need(pool, name, dt)
-        if pool.dim() != 4 or pool.shape[1] != nkv or pool.shape[2] != 64 or pool.shape[3] != d:
-            raise KernelError(f"{name} must be [pages, {nkv}, 64, {d}], got {tuple(pool.shape)}")
+    _need_pools(k_pool, v_pool, dt, nkv, d)
     q = torch.empty((M, nh, d), dtype=dt, device=fused.device)
     _call("pta_qkv_rope_cache", _ptr(q), _ptr(fused), _ptr(bias), _ptr(inv_freq), ctypes.c_float(cs_scale),
           _ptr(token_pos), _ptr(token_seq), _ptr(block_table), block_table.shape[1], _ptr(k_pool), _ptr(v_pool), M,
@@ -184,10 +191,7 @@ def attn_generic(q: torch.Tensor, k_pool, v_pool, block_table, token_seq, token_
     _need(q, "q")
     M, nh, d = q.shape
     nkv = k_pool.shape[1]
-    for name, pool in (("k_pool", k_pool), ("v_pool", v_pool)):
-        _need(pool, name, q.dtype)
-        if pool.dim() != 4 or pool.shape[1] != nkv or pool.shape[2] != 64 or pool.shape[3] != d:
-            raise KernelError(f"{name} must be [pages, {nkv}, 64, {d}], got {tuple(pool.shape)}")
+    _need_pools(k_pool, v_pool, q.dtype, nkv, d)
     _need(block_table, "block_table", torch.int32)
     _need(token_seq, "token_seq", torch.int32, (M,))
     _need(token_pos, "token_pos", torch.int32, (M,))
@@ -219,8 +223,55 @@ def gemm_f32(a: torch.Tensor, w: torch.Tensor, bias=None, act=None, add1=None, a
     return out
 
 
+ATTN_SPLIT_KEYS = 256  # keys per wave when a decode step's context is split; a constant, so that the
+# partition of a context depends on its length alone
+
+
+def attn_mfma_ok(q: torch.Tensor) -> bool:
+    """Whether the matrix-core attention kernel takes these queries (bfloat16, head size built)."""
+    return q.dtype == torch.bfloat16 and bool(load_library().pta_attn_mfma_supported(int(q.shape[2])))
+
+
+def attn_mfma(q: torch.Tensor, k_pool, v_pool, block_table, cu_tokens, seq_start, slopes, scale: float, *,
+              max_new: int, n_splits: int = 1, split_size: int = ATTN_SPLIT_KEYS) -> torch.Tensor:
+    """Causal attention of a step's tokens over the cache on the matrix cores; out [M, nh*d].
+
+    ``max_new`` bounds the new tokens of any sequence of the step; with ``n_splits > 1`` the keys
+    are split into ranges of ``split_size`` and ``n_splits * split_size`` bounds every context."""
+    _need(q, "q", torch.bfloat16)
+    M, nh, d = q.shape
+    nkv = k_pool.shape[1]
+    _need_pools(k_pool, v_pool, q.dtype, nkv, d)
+    _need(block_table, "block_table", torch.int32)
+    n_seqs = block_table.shape[0]
+    _need(cu_tokens, "cu_tokens", torch.int32, (n_seqs + 1,))
+    _need(seq_start, "seq_start", torch.int32, (n_seqs,))
+    if slopes is not None:
+        _need(slopes, "slopes", torch.float32, (nh,))
+    out = torch.empty((M, nh * d), dtype=q.dtype, device=q.device)
+    po = pm = pl = None
+    if n_splits > 1:
+        po = torch.empty((M, nh, n_splits, d), dtype=torch.float32, device=q.device)
+        pm = torch.empty((M, nh, n_splits), dtype=torch.float32, device=q.device)
+        pl = torch.empty((M, nh, n_splits), dtype=torch.float32, device=q.device)
+    _call("pta_attn_mfma", _ptr(out), _ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(block_table), block_table.shape[1],
+          _ptr(cu_tokens), _ptr(seq_start), _ptr(slopes), n_seqs, int(max_new), M, nh, nkv, d, ctypes.c_float(scale),
+          int(split_size), int(n_splits), _ptr(po), _ptr(pm), _ptr(pl), _stream())
+    return out
+
+
 def attention(q: torch.Tensor, k_pool, v_pool, block_table, ctx, slopes, scale: float) -> torch.Tensor:
-    """Attention of a step's tokens over the cache: picks the kernel for the step's shape and type."""
+    """Attention of a step's tokens over the cache: picks the kernel for the step's shape and type.
+
+    bfloat16 with a head size the matrix-core kernel is built for: that kernel, with the context
+    split over several waves when every sequence brings one token; anything else: the 32-bit
+    kernel."""
+    if attn_mfma_ok(q):
+        n_splits = 1
+        if ctx.is_decode and ctx.max_len > ATTN_SPLIT_KEYS:
+            n_splits = (ctx.max_len + ATTN_SPLIT_KEYS - 1) // ATTN_SPLIT_KEYS
+        return attn_mfma(q, k_pool, v_pool, block_table, ctx.cu_tokens, ctx.seq_start, slopes, scale,
+                         max_new=max(ctx.new_tokens), n_splits=n_splits)
     return attn_generic(q, k_pool, v_pool, block_table, ctx.token_seq, ctx.token_pos, slopes, scale)
 
 
@@ -251,3 +302,38 @@ def sample(logits: torch.Tensor, *, do_sample: bool, temperature: float = 1.0, t
           int(bool(renorm)), ctypes.c_uint64(int(seed) & (2 ** 64 - 1)), _ptr(rng_seq), _ptr(rng_step), _ptr(uniforms),
           _stream())
     return out, work
+
+
+SKINNY_MAX_ROWS = 64
+
+
+def gemm_skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether the decode kernel takes this product and is the faster choice for it.
+
+    It takes at most 64 rows of bfloat16 with K a multiple of 8.  Measured on MI355X against the
+    vendor library at Falcon-7B shapes: up to 16 rows it wins everywhere; from 17 to 64 rows only
+    where K is long against N (the feed-forward's second matrix)."""
+    if not (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and 0 < x.shape[0] <= SKINNY_MAX_ROWS
+            and x.shape[1] % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0):
+        return False
+    return x.shape[0] <= 16 or w.shape[1] >= 2 * w.shape[0]
+
+
+def gemm_skinny_bf16(x: torch.Tensor, w: torch.Tensor, bias=None, act=None, add1=None, add2=None,
+                     out_f32: bool = False, variant: int = 0, waves: int = 0) -> torch.Tensor:
+    """act(x @ w.T + bias) + add1 + add2 for at most 64 rows of bfloat16, 32-bit accumulation."""
+    _need(x, "x", torch.bfloat16)
+    _need(w, "w", torch.bfloat16)
+    M, K = x.shape
+    N = w.shape[0]
+    if w.shape[1] != K:
+        raise KernelError(f"x is [{M}, {K}] but w is {tuple(w.shape)}; w must be [N, {K}]")
+    if bias is not None:
+        _need(bias, "bias", torch.float32, (N,))
+    for name, t in (("add1", add1), ("add2", add2)):
+        if t is not None:
+            _need(t, name, torch.bfloat16, (M, N))
+    out = torch.empty((M, N), dtype=torch.float32 if out_f32 else torch.bfloat16, device=x.device)
+    _call("pta_gemm_skinny_bf16", _ptr(out), _ptr(x), _ptr(w), _ptr(bias), _ptr(add1), _ptr(add2), M, N, K,
+          ACT_CODES[act], int(out_f32), int(variant), int(waves), _stream())
+    return out

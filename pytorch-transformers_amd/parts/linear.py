@@ -4,8 +4,10 @@
 storage type, as the reference does on purpose
 (src/transformers/models/falcon/modeling_falcon.py:64-72).  In 32-bit the whole
 layer, with activation and residual additions, is one hand-written kernel with a
-fixed summation order.  In bfloat16 the matrix product is the vendor library's
-(as the reference's is torch's), followed by one fused kernel for bias,
+fixed summation order.  In bfloat16, steps of at most 64 tokens (decoding) run a
+hand-written kernel that streams the weights once and applies bias, activation
+and additions in its epilogue; larger steps use the vendor library's matrix
+product (as the reference uses torch's), followed by one fused kernel for bias,
 activation and additions.
 """
 from __future__ import annotations
@@ -44,6 +46,8 @@ class Linear(Part):
         bias = self.bias if apply_bias else None
         if x.dtype == torch.float32:
             return ops.gemm_f32(x, self.weight, bias, act, add1, add2)
+        if ops.gemm_skinny_ok(x, self.weight):
+            return ops.gemm_skinny_bf16(x, self.weight, bias, act, add1, add2)
         y = torch.mm(x, self.weight.t())
         if bias is not None or act is not None or add1 is not None or add2 is not None:
             ops.epilogue_(y, bias, act, add1, add2)
@@ -91,4 +95,6 @@ class OutputHead(Part):
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         if h.dtype == torch.float32:
             return ops.gemm_f32(h, self.weight)
+        if ops.gemm_skinny_ok(h, self.weight):
+            return ops.gemm_skinny_bf16(h, self.weight, out_f32=True)
         return torch.mm(h, self.weight.t(), out_dtype=torch.float32)

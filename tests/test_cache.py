@@ -19,7 +19,7 @@ def test_shapes_and_capacity():
     c = _cache(1000)
     assert c.num_pages == 16 and c.max_slots == 16  # 1000 tokens round up to 16 pages of 64
     k, v = c.kv_layer("kv", 1)
-    assert k.shape == (16, 2, 64, 16) and v.shape == k.shape
+    assert k.shape == (16, 2, 64, 16) and v.shape == (16, 2, 16, 64)  # value pages are transposed
     assert c.bytes_per_token() == 2 * 2 * 2 * 16 * 4
 
 

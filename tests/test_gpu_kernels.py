@@ -1,0 +1,300 @@
+"""Each kernel alone against a plain torch computation, at sizes other than the tiny models' (GPU)."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import plain_falcon as P
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def _ops():
+    from pytorch_transformers_amd import ops
+    return ops
+
+
+def _rand(*shape, seed=0, dtype=torch.float32, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).cuda()
+
+
+def _tol(dtype):
+    return dict(rtol=2e-5, atol=2e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embed(dtype):
+    ops = _ops()
+    table = _rand(1000, 72, dtype=dtype)
+    ids = torch.tensor([0, 999, 5, 5, 123], dtype=torch.int32).cuda()
+    assert torch.equal(ops.embed(table, ids), table[ids.long()])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H", [48, 1000, 4544])
+def test_layernorm(dtype, H):
+    ops = _ops()
+    x = _rand(7, H, dtype=dtype, scale=3.0) + 1.5
+    w, b, w2, b2 = (_rand(H, seed=s) for s in (1, 2, 3, 4))
+    ref = F.layer_norm(x.float(), (H,), w, b, 1e-5)
+    torch.testing.assert_close(ops.layernorm(x, w, b, 1e-5).float(), ref, **_tol(dtype))
+    o1, o2 = ops.layernorm(x, w, b, 1e-3, w2=w2, b2=b2)
+    torch.testing.assert_close(o1.float(), F.layer_norm(x.float(), (H,), w, b, 1e-3), **_tol(dtype))
+    torch.testing.assert_close(o2.float(), F.layer_norm(x.float(), (H,), w2, b2, 1e-3), **_tol(dtype))
+    rows = torch.tensor([6, 0, 3], dtype=torch.int32).cuda()
+    torch.testing.assert_close(ops.layernorm(x, w, b, 1e-5, rows=rows).float(), ref[rows.long()], **_tol(dtype))
+    # a row's result does not depend on the rows around it
+    assert torch.equal(ops.layernorm(x[2:3].contiguous(), w, b, 1e-5), ops.layernorm(x, w, b, 1e-5)[2:3])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_epilogue(dtype):
+    ops = _ops()
+    y, a1, a2 = (_rand(5, 130, seed=s, dtype=dtype) for s in (0, 1, 2))
+    bias = _rand(130, seed=3)
+    rnd = (lambda t: t) if dtype == torch.float32 else (lambda t: t.bfloat16().float())
+    want = F.gelu(rnd(y.float() + bias)) + a1.float() + a2.float()
+    got = ops.epilogue_(y.clone(), bias, "gelu", a1, a2)
+    torch.testing.assert_close(got.float(), want, **_tol(dtype))
+    torch.testing.assert_close(ops.epilogue_(y.clone(), None, None, a1, None).float(), y.float() + a1.float(), **_tol(dtype))
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 16, 8), (5, 100, 33), (64, 64, 16), (130, 257, 129), (17, 4544, 300)])
+def test_gemm_f32(M, N, K):
+    ops = _ops()
+    a, w, bias, a1, a2 = _rand(M, K), _rand(N, K, seed=1), _rand(N, seed=2), _rand(M, N, seed=3), _rand(M, N, seed=4)
+    want = (a.double() @ w.double().T)
+    torch.testing.assert_close(ops.gemm_f32(a, w).double(), want, rtol=1e-5, atol=1e-5 * math.sqrt(K))
+    full = F.gelu(want + bias.double()) + a1.double() + a2.double()
+    torch.testing.assert_close(ops.gemm_f32(a, w, bias, "gelu", a1, a2).double(), full, rtol=1e-5, atol=1e-5 * math.sqrt(K))
+    # bitwise the same for a row alone and in the batch
+    r = M // 2
+    assert torch.equal(ops.gemm_f32(a[r:r + 1].contiguous(), w, bias), ops.gemm_f32(a, w, bias)[r:r + 1])
+
+
+@pytest.mark.parametrize("M", [1, 3, 8, 16, 17, 32, 33, 48, 49, 64])
+@pytest.mark.parametrize("N,K", [(16, 64), (100, 200), (4544, 4544), (250, 18176 // 4)])
+def test_gemm_skinny_bf16(M, N, K):
+    ops = _ops()
+    x = _rand(M, K, dtype=torch.bfloat16)
+    w = _rand(N, K, seed=1, dtype=torch.bfloat16, scale=0.05)
+    bias, a1, a2 = _rand(N, seed=2), _rand(M, N, seed=3, dtype=torch.bfloat16), _rand(M, N, seed=4, dtype=torch.bfloat16)
+    prod = x.double() @ w.double().T
+    scale = float(prod.abs().max())
+    got32 = ops.gemm_skinny_bf16(x, w, out_f32=True)
+    assert float((got32.double() - prod).abs().max()) <= 2e-5 * scale + 1e-6, "32-bit output: only accumulation error"
+    got = ops.gemm_skinny_bf16(x, w, bias, "gelu", a1, a2)
+    want = F.gelu((prod.float().bfloat16().float() + bias).bfloat16().float()) + a1.float() + a2.float()
+    torch.testing.assert_close(got.float(), want, rtol=2e-2, atol=2e-2 * max(1.0, scale))
+    assert ops.gemm_skinny_ok(x, w) == (M <= 16 or K >= 2 * N)  # where it is also the faster choice
+    # a row alone gives the same bits as in the batch
+    r = M - 1
+    alone = ops.gemm_skinny_bf16(x[r:r + 1].contiguous(), w, out_f32=True)
+    assert torch.equal(alone, got32[r:r + 1])
+
+
+def test_gemm_skinny_refuses_what_it_cannot_do():
+    ops = _ops()
+    x, w = _rand(65, 64, dtype=torch.bfloat16), _rand(32, 64, dtype=torch.bfloat16)
+    assert not ops.gemm_skinny_ok(x, w)
+    with pytest.raises(ops.KernelError, match="at most 64 rows"):
+        ops.gemm_skinny_bf16(x, w)
+    x, w = _rand(4, 60, dtype=torch.bfloat16), _rand(32, 60, dtype=torch.bfloat16)
+    assert not ops.gemm_skinny_ok(x, w)
+    with pytest.raises(ops.KernelError, match="multiple of 8"):
+        ops.gemm_skinny_bf16(x, w)
+    with pytest.raises(ops.KernelError, match="no CPU fallback"):
+        ops.gemm_skinny_bf16(x.cpu(), w.cpu())
+
+
+# --- rotation, head split, cache write, attention ------------------------------------------------------
+def _cache_setup(n_seqs, lens, nkv, d, dtype, n_pages=64, seed=0):
+    """Scattered pages for every sequence; returns pools, block table and the page lists."""
+    g = torch.Generator().manual_seed(seed)
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    lists, at = [], 0
+    for L in lens:
+        n = (L + 63) // 64
+        lists.append(perm[at:at + n]); at += n
+    width = max(len(l) for l in lists)
+    bt = torch.zeros(n_seqs, width, dtype=torch.int32)
+    for i, l in enumerate(lists):
+        bt[i, :len(l)] = torch.tensor(l, dtype=torch.int32)
+    # unwritten positions hold NaN: a kernel that lets them into a sum, even with weight zero, shows
+    k_pool = torch.full((n_pages, nkv, 64, d), float("nan"), dtype=dtype).cuda()
+    v_pool = torch.full((n_pages, nkv, d, 64), float("nan"), dtype=dtype).cuda()  # values: transposed pages
+    return k_pool, v_pool, bt.cuda(), lists
+
+
+def _gather(pool, pages, L, transposed=False):
+    """[L, nkv, d] of a sequence from its pages."""
+    x = pool[torch.tensor(pages).long().cuda()]  # [p, nkv, 64, d], or [p, nkv, d, 64] for values
+    if transposed:
+        x = x.transpose(2, 3)
+    return x.permute(0, 2, 1, 3).reshape(-1, x.shape[1], x.shape[3])[:L]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("layout,nh,nkv,d", [("grouped", 6, 2, 32), ("tail", 7, 1, 64), ("interleaved", 5, 5, 24),
+                                             ("grouped", 8, 8, 16), ("grouped", 4, 1, 128)])
+@pytest.mark.parametrize("rotary", [True, False])
+def test_qkv_rope_cache(dtype, layout, nh, nkv, d, rotary):
+    """Against the plain split and rotation; keys and values land at (page, position) of their sequence."""
+    ops = _ops()
+    starts, news = [70, 0, 127], [3, 66, 1]
+    lens = [s + n for s, n in zip(starts, news)]
+    k_pool, v_pool, bt, lists = _cache_setup(3, lens, nkv, d, dtype)
+    M = sum(news)
+    fused = _rand(M, (nh + 2 * nkv) * d, dtype=dtype)
+    bias = _rand((nh + 2 * nkv) * d, seed=9)
+    token_seq = torch.tensor([i for i, n in enumerate(news) for _ in range(n)], dtype=torch.int32).cuda()
+    token_pos = torch.tensor([s + j for s, n in zip(starts, news) for j in range(n)], dtype=torch.int32).cuda()
+    inv = P.rope_inv_freq(d, 500042.0, 2.0).cuda() if rotary else None
+    q = ops.qkv_rope_cache(fused, bias, inv, 1.0, token_pos, token_seq, bt, k_pool, v_pool, nh, nkv, d, layout)
+
+    c = dict(num_attention_heads=nh, hidden_size=nh * d, num_kv_heads=nkv,
+             new_decoder_architecture=layout == "grouped", multi_query=layout == "tail")
+    rnd = (lambda t: t) if dtype == torch.float32 else (lambda t: t.bfloat16().double())
+    x = rnd(fused.double().cpu() + bias.double().cpu())
+    wq, wk, wv = P.split_heads(x, c)
+    if rotary:
+        cos, sin = P.rope_cos_sin(token_pos.cpu(), inv.cpu())
+        wq, wk = P.apply_rope(wq, cos, sin), P.apply_rope(wk, cos, sin)
+    tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(q.double().cpu(), wq, **tol)
+    at = 0
+    for i, (s, n) in enumerate(zip(starts, news)):
+        gk, gv = _gather(k_pool, lists[i], lens[i]), _gather(v_pool, lists[i], lens[i], transposed=True)
+        torch.testing.assert_close(gk[s:].double().cpu(), wk[at:at + n].contiguous(), **tol)
+        torch.testing.assert_close(gv[s:].double().cpu(), wv[at:at + n].contiguous(), **tol)
+        assert torch.isnan(gk[:s].float()).all(), "positions before the step's tokens must not be written"
+        at += n
+    # write_cache=False leaves the cache alone
+    k2 = k_pool.clone()
+    ops.qkv_rope_cache(fused * 2, bias, inv, 1.0, token_pos, token_seq, bt, k_pool, v_pool, nh, nkv, d, layout, write_cache=False)
+    assert torch.equal(torch.nan_to_num(k2.float()), torch.nan_to_num(k_pool.float()))
+
+
+def _attn_case(ops, fn, dtype, nh, nkv, d, starts, news, slopes=None, seed=0, boost=None):
+    """Fill a cache with random keys and values, run ``fn`` for the new tokens, compare with plain attention."""
+    lens = [s + n for s, n in zip(starts, news)]
+    n_pages = sum((L + 63) // 64 for L in lens) + 3
+    k_pool, v_pool, bt, lists = _cache_setup(len(lens), lens, nkv, d, dtype, n_pages=n_pages, seed=seed)
+    g = torch.Generator().manual_seed(seed + 1)
+    ks, vs, qs = [], [], []
+    for i, L in enumerate(lens):
+        k = torch.randn(L, nkv, d, generator=g).to(dtype)
+        v = torch.randn(L, nkv, d, generator=g).to(dtype)
+        q = torch.randn(news[i], nh, d, generator=g).to(dtype)
+        if boost is not None and boost[i] is not None:
+            # one far key stands out for the last query: the output must be (almost) that key's value
+            j = boost[i]
+            k[j] = 0
+            k[j, :, 0] = 6.0
+            q[-1] = 0
+            q[-1, :, 0] = 6.0 * math.sqrt(d)
+        ks.append(k); vs.append(v); qs.append(q)
+        for p, page in enumerate(lists[i]):
+            n = min(64, L - p * 64)
+            k_pool[page, :, :n] = k[p * 64:p * 64 + n].transpose(0, 1).cuda()
+            v_pool[page, :, :, :n] = v[p * 64:p * 64 + n].permute(1, 2, 0).cuda()
+    q_all = torch.cat(qs).cuda()
+    token_seq = torch.tensor([i for i, n in enumerate(news) for _ in range(n)], dtype=torch.int32).cuda()
+    token_pos = torch.tensor([s + j for s, n in zip(starts, news) for j in range(n)], dtype=torch.int32).cuda()
+    got = fn(q_all, k_pool, v_pool, bt, token_seq, token_pos, slopes, 1.0 / math.sqrt(d), starts, news)
+    at = 0
+    worst = 0.0
+    for i, (s, n) in enumerate(zip(starts, news)):
+        L = lens[i]
+        bias = None
+        if slopes is not None:
+            bias = P.alibi_bias(nh, L, d)
+        # plain attention of the whole sequence needs a query per position: only the new rows are compared
+        q_full = torch.zeros(L, nh, d, dtype=torch.float64)
+        q_full[s:] = qs[i].double()
+        want = P.attention_scores_softmax(q_full, ks[i].double(), vs[i].double(), bias)[s:]
+        g_ = got[at:at + n].double().cpu()
+        tol = 2e-5 if dtype == torch.float32 else 2e-2
+        err = float((g_ - want).abs().max())
+        assert err <= tol * max(1.0, float(want.abs().max())), f"sequence {i} (start {s}, {n} new): max diff {err:.3e}"
+        worst = max(worst, err)
+        if boost is not None and boost[i] is not None:
+            far = vs[i][boost[i]].double().repeat_interleave(nh // nkv, 0).reshape(-1)
+            assert float((g_[-1] - far).abs().max()) < 0.05, "the boosted far key does not dominate"
+        at += n
+    return worst
+
+
+def _generic(ops):
+    def fn(q, k_pool, v_pool, bt, token_seq, token_pos, slopes, scale, starts, news):
+        return ops.attn_generic(q, k_pool, v_pool, bt, token_seq, token_pos, slopes, scale)
+    return fn
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,d", [(7, 1, 64), (6, 2, 32), (3, 3, 24), (4, 2, 128), (2, 1, 256)])
+def test_attn_generic(dtype, nh, nkv, d):
+    """Prompts, single tokens and chunks over an existing cache in one launch; page edges at 64, 128."""
+    ops = _ops()
+    _attn_case(ops, _generic(ops), dtype, nh, nkv, d, starts=[0, 63, 200, 0, 127], news=[70, 1, 5, 1, 2])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attn_generic_far_key_and_alibi(dtype):
+    ops = _ops()
+    _attn_case(ops, _generic(ops), dtype, 4, 2, 32, starts=[700, 0, 300], news=[1, 650, 3], boost=[5, 64, 299])
+    from pytorch_transformers_amd.parts import AlibiPositions
+    for nh in (6, 20):
+        slopes = AlibiPositions(nh).slopes.cuda()
+        _attn_case(ops, _generic(ops), dtype, nh, nh, 16, starts=[0, 290], news=[40, 30], slopes=slopes)
+
+
+def _mfma(ops, n_splits_for=None):
+    def fn(q, k_pool, v_pool, bt, token_seq, token_pos, slopes, scale, starts, news):
+        cu = torch.tensor([0] + list(torch.tensor(news).cumsum(0)), dtype=torch.int32).cuda()
+        st = torch.tensor(starts, dtype=torch.int32).cuda()
+        n_splits = 1
+        if n_splits_for is not None:
+            n_splits = (max(s + n for s, n in zip(starts, news)) + n_splits_for - 1) // n_splits_for
+        return ops.attn_mfma(q, k_pool, v_pool, bt, cu, st, slopes, scale, max_new=max(news), n_splits=n_splits,
+                             split_size=n_splits_for or 256)
+    return fn
+
+
+@pytest.mark.parametrize("nh,nkv,d", [(71, 1, 64), (7, 1, 64), (6, 2, 32), (3, 3, 16), (4, 2, 128), (2, 1, 256),
+                                      (5, 5, 48), (8, 2, 80), (4, 4, 96), (2, 2, 112), (32, 8, 128)])
+def test_attn_mfma_prefill_and_chunks(nh, nkv, d):
+    """Whole prompts, single tokens and chunks over an existing cache in one launch (bfloat16 matrix cores)."""
+    ops = _ops()
+    assert ops.attn_mfma_ok(torch.empty(1, nh, d, dtype=torch.bfloat16).cuda())
+    _attn_case(ops, _mfma(ops), torch.bfloat16, nh, nkv, d, starts=[0, 63, 200, 0, 127, 31], news=[70, 1, 5, 1, 2, 40])
+
+
+@pytest.mark.parametrize("nh,nkv,d", [(71, 1, 64), (6, 2, 32), (3, 3, 16), (8, 2, 128), (2, 1, 256)])
+@pytest.mark.parametrize("split", [64, 256])
+def test_attn_mfma_decode_split(nh, nkv, d, split):
+    """One token per sequence, contexts of very different lengths, keys split over waves and merged."""
+    ops = _ops()
+    _attn_case(ops, _mfma(ops, split), torch.bfloat16, nh, nkv, d, starts=[0, 63, 64, 700, 255, 256, 1], news=[1] * 7)
+
+
+def test_attn_mfma_far_key_alibi_and_refusals():
+    ops = _ops()
+    _attn_case(ops, _mfma(ops), torch.bfloat16, 4, 2, 32, starts=[700, 0, 300], news=[1, 650, 3], boost=[5, 64, 299])
+    _attn_case(ops, _mfma(ops, 128), torch.bfloat16, 4, 2, 32, starts=[700, 900, 300], news=[1, 1, 1], boost=[5, 64, 299])
+    from pytorch_transformers_amd.parts import AlibiPositions
+    for nh in (6, 20):
+        slopes = AlibiPositions(nh).slopes.cuda()
+        _attn_case(ops, _mfma(ops), torch.bfloat16, nh, nh, 16, starts=[0, 290], news=[40, 30], slopes=slopes)
+        _attn_case(ops, _mfma(ops, 64), torch.bfloat16, nh, nh, 16, starts=[39, 319], news=[1, 1], slopes=slopes)
+    assert not ops.attn_mfma_ok(torch.empty(1, 2, 24, dtype=torch.bfloat16).cuda())  # head size 24: the 32-bit kernel runs
+    assert not ops.attn_mfma_ok(torch.empty(1, 2, 64, dtype=torch.float32).cuda())
+    with pytest.raises(ops.KernelError, match="head size 144 is not built"):
+        q = torch.zeros(1, 1, 144, dtype=torch.bfloat16).cuda()
+        ops.attn_mfma(q, torch.zeros(1, 1, 64, 144, dtype=torch.bfloat16).cuda(), torch.zeros(1, 1, 144, 64, dtype=torch.bfloat16).cuda(),
+                      torch.zeros(1, 1, dtype=torch.int32).cuda(), torch.tensor([0, 1], dtype=torch.int32).cuda(),
+                      torch.zeros(1, dtype=torch.int32).cuda(), None, 1.0, max_new=1)
