@@ -5,7 +5,7 @@
 // sequence, ordered token-major.  Heads that share a KV head therefore sit side by side and read
 // its keys and values once: with one KV head for 71 query heads, a decode step's 71 columns are five
 // tiles of 16 that share every key load.  A wave owns CT column tiles and walks the keys 32 at a
-// time:
+// time, always with the next block's keys and values already on their way:
 //
 //   S^T[32 keys x 16 cols]  = K[32 x d] . Q^T[d x 16]         (A = key rows, B = query columns)
 //   online softmax over keys, per column (statistics in 32-bit, four lanes hold a column)
@@ -37,6 +37,37 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
     return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
 }
 
+template <int DT>
+struct KvBlock {
+    AFrag k[2][(DT + 1) / 2];
+    AFrag v[DT];
+};
+
+// Keys and values of the 32-key block at kb, straight into matrix-operand registers.  Nothing here
+// depends on the loaded data, so the loads of the next block stay in flight while this one is used.
+template <int DT>
+__device__ __forceinline__ void load_block(KvBlock<DT>& b, int kb, const int* __restrict__ bt,
+                                           const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
+                                           int nkv, int kvh, int c, int gq) {
+    constexpr int D = DT * 16, DS = (DT + 1) / 2, CHUNKS = D / 8;
+    const long page = bt[kb >> 6];
+    const int in_page = kb & 63;
+    const bf16_t* kpage = k_pool + (page * nkv + kvh) * (long)(PTA_PAGE * D);
+    const bf16_t* vpage = v_pool + (page * nkv + kvh) * (long)(PTA_PAGE * D);
+    // key rows: tile tt, row r holds key 8*(r/4) + 4*tt + r%4 of the block
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+        const bf16_t* kp = kpage + (long)(in_page + 8 * (c >> 2) + 4 * tt + (c & 3)) * D;
+#pragma unroll
+        for (int ds = 0; ds < DS; ++ds)
+            b.k[tt][ds].u = *reinterpret_cast<const uint4*>(kp + min(ds * 4 + gq, CHUNKS - 1) * 8);
+    }
+    // value rows: feature dt*16 + c, keys 8*gq .. 8*gq+7 of the block
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+        b.v[dt].u = *reinterpret_cast<const uint4*>(vpage + (long)(dt * 16 + c) * PTA_PAGE + in_page + gq * 8);
+}
+
 template <int DT, int CT>
 __global__ __launch_bounds__(64) void attn_mfma_kernel(
     bf16_t* __restrict__ out, float* __restrict__ po, float* __restrict__ pm, float* __restrict__ pl,
@@ -58,7 +89,10 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(
     const int kv_len = start + n_new;
     const int k_begin = n_splits > 1 ? split * split_size : 0;
     const int k_end = n_splits > 1 ? min(max_qpos + 1, k_begin + split_size) : max_qpos + 1;
+    const int kb_last = (kv_len - 1) & ~31;  // the last block that has a page
     const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
+    // in the last 32-wide step of an odd number of 16-wide tiles, the upper half of the lanes has no data
+    const uint32_t tail_keep = (DT % 2 == 1 && (DS - 1) * 4 + gq >= CHUNKS) ? 0u : 0xffffffffu;
 
     int qpos[CT], tok[CT], head[CT];
     float slope[CT];
@@ -92,43 +126,31 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(
     }
 
     const int* bt = block_table + (long)seq * bt_stride;
-    for (int kb = k_begin; kb < k_end; kb += 32) {
-        const long page = bt[kb >> 6];
-        const int in_page = kb & 63;
-        const bf16_t* kpage = k_pool + (page * nkv + kvh) * (long)(PTA_PAGE * D);
-        const bf16_t* vpage = v_pool + (page * nkv + kvh) * (long)(PTA_PAGE * D);
 
-        // key rows: tile tt, row r holds key 8*(r/4) + 4*tt + r%4 of the block
-        AFrag kf[2][DS];
-#pragma unroll
-        for (int tt = 0; tt < 2; ++tt) {
-            const bf16_t* kp = kpage + (long)(in_page + 8 * (c >> 2) + 4 * tt + (c & 3)) * D;
-#pragma unroll
-            for (int ds = 0; ds < DS; ++ds) {
-                const int chunk = ds * 4 + gq;
-                kf[tt][ds].u = *reinterpret_cast<const uint4*>(kp + min(chunk, CHUNKS - 1) * 8);
-                if (chunk >= CHUNKS) kf[tt][ds].u = zero4;
-            }
-        }
-        // value rows: feature dt*16 + c, keys 8*gq .. 8*gq+7 of the block
-        AFrag vf[DT];
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-            vf[dt].u = *reinterpret_cast<const uint4*>(vpage + (long)(dt * 16 + c) * PTA_PAGE + in_page + gq * 8);
-        if (kb + 32 > kv_len) {
-            // positions past the sequence's end were never written; whatever lies there must not reach
-            // the sum, not even with weight zero
+    // scores, softmax update and value product of the block at kb (a block past k_end changes nothing)
+    auto use_block = [&](KvBlock<DT>& b, int kb) {
+        if (kb + 32 > kv_len || kb >= k_end) {
+            // positions past the sequence's end were never written; whatever lies there must not reach the
+            // sum, not even with weight zero.  A block past this wave's range was loaded from a clamped
+            // address and is dropped whole.
             const int kbase = kb + gq * 8;
+            const int lim = kb >= k_end ? 0 : kv_len;
             uint32_t mk[4];
 #pragma unroll
             for (int w = 0; w < 4; ++w)
-                mk[w] = (kbase + 2 * w < kv_len ? 0x0000ffffu : 0u) | (kbase + 2 * w + 1 < kv_len ? 0xffff0000u : 0u);
+                mk[w] = (kbase + 2 * w < lim ? 0x0000ffffu : 0u) | (kbase + 2 * w + 1 < lim ? 0xffff0000u : 0u);
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
-                vf[dt].u.x &= mk[0]; vf[dt].u.y &= mk[1]; vf[dt].u.z &= mk[2]; vf[dt].u.w &= mk[3];
+                b.v[dt].u.x &= mk[0]; b.v[dt].u.y &= mk[1]; b.v[dt].u.z &= mk[2]; b.v[dt].u.w &= mk[3];
             }
         }
-
+        if (DT % 2 == 1) {
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt) {
+                b.k[tt][DS - 1].u.x &= tail_keep; b.k[tt][DS - 1].u.y &= tail_keep;
+                b.k[tt][DS - 1].u.z &= tail_keep; b.k[tt][DS - 1].u.w &= tail_keep;
+            }
+        }
         f32x4_t sacc[2][CT];
 #pragma unroll
         for (int tt = 0; tt < 2; ++tt)
@@ -137,20 +159,20 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(
                 sacc[tt][ct] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int ds = 0; ds < DS; ++ds)
-                    sacc[tt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[tt][ds].v, qf[ct][ds].v, sacc[tt][ct], 0, 0, 0);
+                    sacc[tt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b.k[tt][ds].v, qf[ct][ds].v, sacc[tt][ct], 0, 0, 0);
             }
-
         AFrag pf[CT];
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
             float s[8];
             float mx = -INFINITY;
+            const int lim = min(qpos[ct] + 1, k_end);  // keys below this count for the column
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const int key = kb + 8 * gq + j;  // j = 4*tt + e
                 float v = sacc[j >> 2][ct][j & 3] * scale;
                 if (slopes) v += round_to_bf16(slope[ct] * round_to_bf16((float)key)) / sqrt_d;
-                s[j] = key <= qpos[ct] ? v : -INFINITY;
+                s[j] = key < lim ? v : -INFINITY;
                 mx = fmaxf(mx, s[j]);
             }
             mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
@@ -176,7 +198,22 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct)
-                oacc[dt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt].v, pf[ct].v, oacc[dt][ct], 0, 0, 0);
+                oacc[dt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b.v[dt].v, pf[ct].v, oacc[dt][ct], 0, 0, 0);
+    };
+
+    // two register buffers: while one block is used, the next one's loads are in flight.  Addresses past
+    // the last block are clamped to it, and such a block is dropped in use_block.
+    KvBlock<DT> b0, b1;
+    if (k_begin < k_end) load_block<DT>(b0, min(k_begin, kb_last), bt, k_pool, v_pool, nkv, kvh, c, gq);
+    for (int kb = k_begin; kb < k_end; kb += 64) {
+        load_block<DT>(b1, min(kb + 32, kb_last), bt, k_pool, v_pool, nkv, kvh, c, gq);
+        __builtin_amdgcn_sched_barrier(0);
+        use_block(b0, kb);
+        __builtin_amdgcn_sched_barrier(0);
+        load_block<DT>(b0, min(kb + 64, kb_last), bt, k_pool, v_pool, nkv, kvh, c, gq);
+        __builtin_amdgcn_sched_barrier(0);
+        use_block(b1, kb + 32);
+        __builtin_amdgcn_sched_barrier(0);
     }
 
 #pragma unroll
@@ -197,11 +234,13 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(
                 *reinterpret_cast<uint2*>(o + dt * 16 + gq * 4) = w;
             }
         } else {
-            float* o = po + (row * n_splits + split) * D;
+            if (k_begin < k_end) {  // a range past the column's keys has nothing to add: only its marker is written
+                float* o = po + (row * n_splits + split) * D;
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
-                *reinterpret_cast<float4*>(o + dt * 16 + gq * 4) =
-                    make_float4(oacc[dt][ct][0], oacc[dt][ct][1], oacc[dt][ct][2], oacc[dt][ct][3]);
+                for (int dt = 0; dt < DT; ++dt)
+                    *reinterpret_cast<float4*>(o + dt * 16 + gq * 4) =
+                        make_float4(oacc[dt][ct][0], oacc[dt][ct][1], oacc[dt][ct][2], oacc[dt][ct][3]);
+            }
             if (gq == 0) {
                 pm[row * n_splits + split] = m_run[ct];
                 pl[row * n_splits + split] = l;
@@ -210,23 +249,40 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(
     }
 }
 
-// out[row, :] = sum_s w_s po[row, s, :] / sum_s w_s pl[row, s], w_s = exp(pm[row, s] - max_s pm), splits in order
-__global__ void attn_combine_kernel(bf16_t* __restrict__ out, const float* __restrict__ po, const float* __restrict__ pm,
-                                    const float* __restrict__ pl, int D, int n_splits) {
+// out[row, :] = sum_s w_s po[row, s, :] / sum_s w_s pl[row, s], w_s = exp(pm[row, s] - max_s pm), splits in
+// order.  A split whose maximum is -inf (a range past the row's keys) has weight zero and is not read.
+__global__ __launch_bounds__(64) void attn_combine_kernel(bf16_t* __restrict__ out, const float* __restrict__ po,
+                                                          const float* __restrict__ pm, const float* __restrict__ pl,
+                                                          int D, int n_splits) {
+    __shared__ float w_s[1024];
     const long row = blockIdx.x;
+    const int lane = threadIdx.x;
     const float* m = pm + row * n_splits;
     const float* l = pl + row * n_splits;
     float mx = -INFINITY;
-    for (int s = 0; s < n_splits; ++s) mx = fmaxf(mx, m[s]);
+    for (int s = lane; s < n_splits; s += 64) mx = fmaxf(mx, m[s]);
+    mx = wave_max(mx);
     float L = 0.f;
-    for (int s = 0; s < n_splits; ++s) L += (m[s] == -INFINITY ? 0.f : expf(m[s] - mx)) * l[s];
+    int used = 0;
+    for (int s0 = 0; s0 < n_splits; s0 += 64) {  // lanes in order, chunks in order: a fixed summation order
+        const int s = s0 + lane;
+        float w = 0.f;
+        if (s < n_splits && m[s] != -INFINITY) { w = expf(m[s] - mx); used = s + 1; }
+        if (s < n_splits) w_s[s] = w;
+        L += wave_sum(w * (s < n_splits ? l[s] : 0.f));
+    }
+    used = (int)wave_max((float)used);
+    __syncthreads();
     const float inv = 1.0f / L;
-    for (int dd = threadIdx.x; dd < D; dd += blockDim.x) {
+    for (int dd = lane; dd < D; dd += 64) {
         float acc = 0.f;
-        for (int s = 0; s < n_splits; ++s) {
-            const float w = m[s] == -INFINITY ? 0.f : expf(m[s] - mx);
-            acc += w * po[(row * n_splits + s) * D + dd];
+        const float* p = po + row * (long)n_splits * D + dd;
+        int s = 0;
+        for (; s + 4 <= used; s += 4) {
+            const float v0 = p[(long)s * D], v1 = p[(long)(s + 1) * D], v2 = p[(long)(s + 2) * D], v3 = p[(long)(s + 3) * D];
+            acc += w_s[s] * v0; acc += w_s[s + 1] * v1; acc += w_s[s + 2] * v2; acc += w_s[s + 3] * v3;
         }
+        for (; s < used; ++s) acc += w_s[s] * p[(long)s * D];
         out[row * D + dd] = f32_to_bf16_bits(acc * inv);
     }
 }
@@ -252,18 +308,26 @@ extern "C" int pta_attn_mfma(void* out, const void* q, const void* k_pool, const
     PTA_REQUIRE(n_seqs > 0 && max_new > 0 && M > 0 && nh > 0 && nkv > 0, "attn_mfma: sizes must be positive");
     PTA_REQUIRE(nh % nkv == 0, "attn_mfma: heads (%d) must be a multiple of kv heads (%d)", nh, nkv);
     PTA_REQUIRE(pta_attn_mfma_supported(d), "attn_mfma: head size %d is not built (16..128 in steps of 16, or 256)", d);
-    PTA_REQUIRE(n_splits >= 1, "attn_mfma: n_splits must be at least 1");
+    PTA_REQUIRE(n_splits >= 1 && n_splits <= 1024, "attn_mfma: n_splits must be 1..1024, got %d", n_splits);
     PTA_REQUIRE(n_splits == 1 || (split_size > 0 && split_size % 64 == 0 && po && pm && pl),
                 "attn_mfma: splitting needs a split size that is a multiple of 64 and buffers for partial results");
     PTA_REQUIRE((long)n_seqs * n_splits <= 65535 && nkv <= 65535, "attn_mfma: too many sequences x splits for one launch");
     PTA_REQUIRE(((uintptr_t)q % 16) == 0 && ((uintptr_t)k_pool % 16) == 0 && ((uintptr_t)v_pool % 16) == 0 &&
                     ((uintptr_t)out % 8) == 0, "attn_mfma: pointers must be 16-byte aligned");
     hipStream_t s = (hipStream_t)stream;
+    // one token per sequence (decode): one column tile per wave, so that the tiles of a KV head run side
+    // by side; prompts: several tiles per wave, so that a key block is loaded once for all of them
+    const bool narrow = max_new == 1;
 #define PTA_ATTN_CASE(DT_, CT_)                                                                                     \
     case DT_:                                                                                                       \
-        launch_attn<DT_, CT_>((bf16_t*)out, po, pm, pl, (const bf16_t*)q, (const bf16_t*)k_pool,                    \
-                              (const bf16_t*)v_pool, block_table, bt_stride, cu_tokens, seq_start, slopes, n_seqs,  \
-                              max_new, nh, nkv, scale, split_size, n_splits, s);                                    \
+        if (narrow)                                                                                                 \
+            launch_attn<DT_, 1>((bf16_t*)out, po, pm, pl, (const bf16_t*)q, (const bf16_t*)k_pool,                  \
+                                (const bf16_t*)v_pool, block_table, bt_stride, cu_tokens, seq_start, slopes, n_seqs, \
+                                max_new, nh, nkv, scale, split_size, n_splits, s);                                  \
+        else                                                                                                        \
+            launch_attn<DT_, CT_>((bf16_t*)out, po, pm, pl, (const bf16_t*)q, (const bf16_t*)k_pool,                \
+                                  (const bf16_t*)v_pool, block_table, bt_stride, cu_tokens, seq_start, slopes,      \
+                                  n_seqs, max_new, nh, nkv, scale, split_size, n_splits, s);                        \
         break;
     switch (d / 16) {
         PTA_ATTN_CASE(1, 4)

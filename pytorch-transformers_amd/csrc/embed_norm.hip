@@ -60,6 +60,49 @@ __global__ void layernorm_kernel(T* __restrict__ out1, T* __restrict__ out2, con
     }
 }
 
+// The same, for rows of at most LN_THREADS * LN_VPT features: the row is read once and held in
+// registers, in the same thread-strided order, so the statistics are the same bits as above.
+#define LN_THREADS 512
+#define LN_VPT 16
+template <typename T>
+__global__ __launch_bounds__(LN_THREADS) void layernorm_reg_kernel(
+    T* __restrict__ out1, T* __restrict__ out2, const T* __restrict__ x, const int* __restrict__ rows,
+    const float* __restrict__ w1, const float* __restrict__ b1, const float* __restrict__ w2,
+    const float* __restrict__ b2, int H, float eps) {
+    __shared__ float red[16];
+    const int m = blockIdx.x;
+    const long src_row = rows ? (long)rows[m] : (long)m;
+    const T* xr = x + src_row * H;
+    float xv[LN_VPT];
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < LN_VPT; ++j) {
+        const int i = threadIdx.x + j * LN_THREADS;
+        xv[j] = i < H ? Io<T>::ld(xr + i) : 0.f;
+        if (i < H) s += xv[j];
+    }
+    const float mean = block_sum(s, red) / (float)H;
+    float q = 0.f;
+#pragma unroll
+    for (int j = 0; j < LN_VPT; ++j) {
+        const int i = threadIdx.x + j * LN_THREADS;
+        if (i < H) { const float d = xv[j] - mean; q += d * d; }
+    }
+    const float var = block_sum(q, red) / (float)H;
+    const float rstd = 1.0f / sqrtf(var + eps);
+    T* o1 = out1 + (long)m * H;
+    T* o2 = out2 ? out2 + (long)m * H : nullptr;
+#pragma unroll
+    for (int j = 0; j < LN_VPT; ++j) {
+        const int i = threadIdx.x + j * LN_THREADS;
+        if (i < H) {
+            const float n = (xv[j] - mean) * rstd;
+            Io<T>::st(o1 + i, n * w1[i] + b1[i]);
+            if (o2) Io<T>::st(o2 + i, n * w2[i] + b2[i]);
+        }
+    }
+}
+
 extern "C" int pta_layernorm(void* out1, void* out2, const void* x, const int* rows, const float* w1,
                              const float* b1, const float* w2, const float* b2, int M, int H, float eps,
                              int dtype, void* stream) {
@@ -67,15 +110,21 @@ extern "C" int pta_layernorm(void* out1, void* out2, const void* x, const int* r
     PTA_REQUIRE(out1 && x && w1 && b1, "layernorm: null pointer");
     PTA_REQUIRE(!out2 || (w2 && b2), "layernorm: a second output needs its own weight and bias");
     hipStream_t s = (hipStream_t)stream;
+    const bool in_regs = H > 1024 && H <= LN_THREADS * LN_VPT;
     const int threads = H >= 2048 ? 512 : 256;
-    if (dtype == PTA_F32)
+    if (dtype != PTA_F32 && dtype != PTA_BF16) return pta_fail("layernorm: unknown dtype %d", dtype);
+    if (in_regs && dtype == PTA_F32)
+        hipLaunchKernelGGL(layernorm_reg_kernel<float>, dim3(M), dim3(LN_THREADS), 0, s, (float*)out1, (float*)out2,
+                           (const float*)x, rows, w1, b1, w2, b2, H, eps);
+    else if (in_regs)
+        hipLaunchKernelGGL(layernorm_reg_kernel<bf16_t>, dim3(M), dim3(LN_THREADS), 0, s, (bf16_t*)out1, (bf16_t*)out2,
+                           (const bf16_t*)x, rows, w1, b1, w2, b2, H, eps);
+    else if (dtype == PTA_F32)
         hipLaunchKernelGGL(layernorm_kernel<float>, dim3(M), dim3(threads), 0, s, (float*)out1, (float*)out2,
                            (const float*)x, rows, w1, b1, w2, b2, H, eps);
-    else if (dtype == PTA_BF16)
+    else
         hipLaunchKernelGGL(layernorm_kernel<bf16_t>, dim3(M), dim3(threads), 0, s, (bf16_t*)out1, (bf16_t*)out2,
                            (const bf16_t*)x, rows, w1, b1, w2, b2, H, eps);
-    else
-        return pta_fail("layernorm: unknown dtype %d", dtype);
     return pta_check_launch("layernorm");
 }
 

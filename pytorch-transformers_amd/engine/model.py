@@ -43,6 +43,93 @@ def _require_gpu(device) -> torch.device:
     return device
 
 
+GRAPH_LEN_STEP = 1024  # a decode graph serves contexts up to the next multiple of this
+
+
+class _DecodeGraph:
+    """One decode step of ``n`` sequences with contexts up to ``len_bound``, captured once and replayed.
+
+    A decode step launches some ten kernels a layer; issued one by one from Python they cost more
+    host time than the GPU needs to run them.  The captured graph reads everything that changes
+    from step to step (token ids, positions, slots, page lists) from one device buffer, which a
+    replay refreshes with a single copy from pinned host memory.  Launch shapes that depend on the
+    context (how many key ranges the attention is split into) are sized for ``len_bound``; ranges
+    past a sequence's end do no work.  A step with fewer than ``n`` sequences repeats its first
+    sequence in the spare rows: the same token at the same place writes the same keys and values
+    again, and the spare logits are dropped.
+    """
+
+    def __init__(self, model: "CausalLM", cache: PagedCache, n: int, len_bound: int):
+        self.model, self.cache, self.n, self.len_bound = model, cache, n, len_bound
+        self.width = len_bound // cache.page_size
+        self.groups = cache.paged_groups()
+        ar = np.arange(n, dtype=np.int32)
+        # token_ids, token_seq, token_pos, cu_tokens, seq_start, seq_slot, logit_rows, then one table per group
+        self.sizes = [n, n, n, n + 1, n, n, n] + [n * self.width] * len(self.groups)
+        total = sum(self.sizes)
+        self.host = torch.empty(total, dtype=torch.int32, pin_memory=True)
+        self.host_np = self.host.numpy()
+        self.offsets = np.concatenate([[0], np.cumsum(self.sizes)]).tolist()
+        self._put(1, ar)
+        self._put(3, np.arange(n + 1, dtype=np.int32))
+        self._put(6, ar)
+        self.dev = torch.zeros(total, dtype=torch.int32, device=model.device)
+        self.copied = torch.cuda.Event()
+        self.graph = None
+        self.logits = None
+
+    def _put(self, i: int, arr) -> None:
+        self.host_np[self.offsets[i]:self.offsets[i + 1]] = arr
+
+    def _fill(self, plan: StepPlan) -> None:
+        n, k = self.n, plan.n_seqs
+        pad = lambda a: np.concatenate([a, np.repeat(a[:1], n - k)]) if k < n else a
+        self.copied.synchronize()  # the last copy out of the pinned buffer is done
+        self._put(0, pad(plan.token_ids))
+        self._put(2, pad(plan.token_pos))
+        self._put(4, pad(np.asarray(plan.starts, dtype=np.int32)))
+        self._put(5, pad(np.asarray(plan.slots, dtype=np.int32)))
+        for gi, g in enumerate(self.groups):
+            t = np.zeros((n, self.width), dtype=np.int32)
+            src = plan.block_tables[g]
+            t[:k, :src.shape[1]] = src
+            if k < n:
+                t[k:] = t[0]
+            self._put(7 + gi, t.reshape(-1))
+        self.dev.copy_(self.host, non_blocking=True)
+        self.copied.record()
+
+    def _context(self):
+        v = torch.split(self.dev, self.sizes)
+        tables = {g: v[7 + i].view(self.n, self.width) for i, g in enumerate(self.groups)}
+        ctx = StepContext(dtype=self.model.dtype, device=self.model.device, n_seqs=self.n, n_tokens=self.n,
+                          token_seq=v[1], token_pos=v[2], cu_tokens=v[3], seq_start=v[4], seq_slot=v[5],
+                          block_tables=tables, cache=self.cache, slots=[], new_tokens=[1] * self.n, starts=[],
+                          is_decode=True, max_len=self.len_bound)
+        return ctx, v[0], v[6]
+
+    def run(self, plan: StepPlan) -> torch.Tensor:
+        self._fill(plan)
+        if self.graph is None:
+            ctx, ids, rows = self._context()
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):  # once outside capture: libraries set themselves up
+                self.model.forward_tokens(ctx, ids, rows)
+            torch.cuda.current_stream().wait_stream(side)
+            self.graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(self.graph):
+                self.logits = self.model.forward_tokens(ctx, ids, rows)
+        self.graph.replay()
+        k = plan.n_seqs
+        rows = plan.logit_rows
+        if rows.shape[0] == k:  # one row per sequence, in order: the first k rows as they are
+            return self.logits[:k]
+        if rows.shape[0] == 0:
+            return self.logits[:0]
+        return self.logits.index_select(0, torch.from_numpy(rows.astype(np.int64)).to(self.logits.device))
+
+
 class CausalLM:
     def __init__(self, spec: ModelSpec, tensors: Dict[str, torch.Tensor], dtype: torch.dtype, device):
         spec.validate()
@@ -55,6 +142,8 @@ class CausalLM:
             part.load_all(tensors)
         self._move_constants()
         self.generation_config = None
+        #: run steps in which every sequence brings one token as replays of a captured HIP graph
+        self.use_graphs = bool(spec.supports_graphs)
 
     def _move_constants(self) -> None:
         seen = set()
@@ -143,6 +232,18 @@ class CausalLM:
             h = x.index_select(0, logit_rows.long())
         return self.spec.head.forward(h)
 
+    # decode steps as HIP graphs ---------------------------------------------------------
+    def _graph_for(self, cache: PagedCache, plan: StepPlan) -> "_DecodeGraph":
+        n = plan.n_seqs
+        n_bucket = n if n <= 8 else (n + 7) // 8 * 8
+        len_bound = (plan.max_len + GRAPH_LEN_STEP - 1) // GRAPH_LEN_STEP * GRAPH_LEN_STEP
+        graphs = cache.__dict__.setdefault("_decode_graphs", {})
+        key = (id(self), n_bucket, len_bound)
+        g = graphs.get(key)
+        if g is None:
+            g = graphs[key] = _DecodeGraph(self, cache, n_bucket, len_bound)
+        return g
+
     @torch.no_grad()
     def step(self, cache: PagedCache, slots: Sequence[int], tokens: Sequence[Sequence[int]],
              want: Want = "last") -> torch.Tensor:
@@ -153,6 +254,10 @@ class CausalLM:
         their places.
         """
         plan = plan_step(cache, slots, tokens, want, self.vocab_size)
+        if self.use_graphs and plan.is_decode:
+            logits = self._graph_for(cache, plan).run(plan)
+            cache.commit(plan.slots, plan.new_tokens)
+            return logits
         ctx, ids, rows = self.make_context(plan, cache)
         logits = self.forward_tokens(ctx, ids, rows)
         cache.commit(plan.slots, plan.new_tokens)

@@ -74,6 +74,9 @@ class ModelSpec:
     final_norm: Any  # parts norm or None
     head: Any  # parts.OutputHead
     cache_groups: List[CacheGroupSpec]
+    #: False if a part reads the step's host-side lists (``ctx.slots`` ...) while it runs: such a step
+    #: cannot be captured into a graph and replayed with other values
+    supports_graphs: bool = True
 
     def parts(self) -> Sequence[Any]:
         out = [self.embedding, *self.blocks]

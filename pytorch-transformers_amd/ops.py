@@ -223,7 +223,7 @@ def gemm_f32(a: torch.Tensor, w: torch.Tensor, bias=None, act=None, add1=None, a
     return out
 
 
-ATTN_SPLIT_KEYS = 256  # keys per wave when a decode step's context is split; a constant, so that the
+ATTN_SPLIT_KEYS = int(os.environ.get("PTA_ATTN_SPLIT", "64"))  # keys per wave when a decode step's context is split; a constant, so that the
 # partition of a context depends on its length alone
 
 

@@ -125,3 +125,32 @@ def test_trace_run_program(folders, tmp_path, dtype):
                 row += 1
             fed[e["id"]] += len(e["tokens"])
         assert row == arr.shape[0]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_graph_replays_equal_eager_steps(folders, name, dtype):
+    """Decode steps replayed from a captured graph give the bits of the same steps launched one by one,
+    on every replay, with eager work (prompts of other batches, frees) and synchronisation in between."""
+    from pytorch_transformers_amd import AutoModelForCausalLM
+    from pytorch_transformers_amd.engine.replay import Replayer
+
+    reqs = helpers.make_requests(TINY[name]["vocab_size"], [40, 9, 70, 33, 17, 64, 5, 21, 90, 12], seed=3)
+    records = helpers.schedule_batches(reqs, 4, decode=(12, 5, 30, 9)) + \
+        [dict(r, step=r["step"] + 1000) for r in helpers.schedule_batches(reqs, 10, decode=(7, 3))]
+    outs = {}
+    for graphs in (False, True):
+        model = AutoModelForCausalLM.from_pretrained(folders[name], dtype=dtype)
+        model.use_graphs = graphs
+        rp = Replayer(model, 4096)
+        outs[graphs] = []
+        for rec in records:
+            logits = rp.run(rec)
+            outs[graphs].append(None if logits is None else logits.clone())
+            torch.cuda.synchronize()
+        if graphs:
+            assert getattr(rp.cache, "_decode_graphs", None), "no graph was captured"
+    for rec, a, b in zip(records, outs[False], outs[True]):
+        assert (a is None) == (b is None)
+        if a is not None:
+            assert torch.equal(a, b), f"step {rec['step']}: graph replay differs from eager launch"
