@@ -1,0 +1,306 @@
+"""Each part alone against the plain functions, and a toy architecture with a state-holding mixer that
+is defined here, registered, built and stepped without touching the framework's files (GPU)."""
+import dataclasses
+import math
+
+import pytest
+import torch
+
+import helpers
+import plain_falcon as P
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [(torch.float32, 3e-5), (torch.bfloat16, 3e-2)]
+
+
+def _rand(*shape, seed=0, scale=1.0):
+    return torch.randn(*shape, generator=torch.Generator().manual_seed(seed)) * scale
+
+
+def _fill(part, dtype, seed=0, std=0.05):
+    """Random tensors for a part, as the device would hold them; returns (device dict, float64 dict)."""
+    from pytorch_transformers_amd.weights.loader import device_dtype_for
+    from pytorch_transformers_amd.weights.random_init import init_tensor
+
+    dev, ref = {}, {}
+    for s in part.all_tensor_specs():
+        t = init_tensor(s, seed, std, noise=0.2, dtype=torch.bfloat16)
+        dev[s.name] = t.to(device_dtype_for(s, dtype)).cuda()
+        ref[s.name] = t.double()
+    part.load_all(dev)
+    return dev, ref
+
+
+def _ctx(cache, slots, new_tokens, dtype):
+    """A StepContext for sequences that bring ``new_tokens`` tokens each (pages reserved, not committed)."""
+    import numpy as np
+
+    from pytorch_transformers_amd.engine.step import plan_step
+    from pytorch_transformers_amd.parts.base import StepContext
+
+    plan = plan_step(cache, slots, [[0] * n for n in new_tokens], "all", 10)
+    i32 = lambda a: torch.as_tensor(np.asarray(a), dtype=torch.int32).cuda()
+    return StepContext(dtype=dtype, device=torch.device("cuda:0"), n_seqs=plan.n_seqs, n_tokens=plan.n_tokens,
+                       token_seq=i32(plan.token_seq), token_pos=i32(plan.token_pos), cu_tokens=i32(plan.cu_tokens),
+                       seq_start=i32(plan.starts), seq_slot=i32(plan.slots),
+                       block_tables={g: i32(t) for g, t in plan.block_tables.items()}, cache=cache, slots=plan.slots,
+                       new_tokens=plan.new_tokens, starts=plan.starts, is_decode=plan.is_decode, max_len=plan.max_len), plan
+
+
+def _close(got, want, rel, what):
+    got, want = got.double().cpu(), want.double()
+    scale = max(1.0, float(want.abs().max()))
+    err = float((got - want).abs().max())
+    assert err <= rel * scale, f"{what}: max |diff| {err:.3e} > {rel} x {scale:.3e}"
+
+
+@pytest.mark.parametrize("dtype,rel", DTYPES)
+def test_layernorm_linear_embedding_head(dtype, rel):
+    from pytorch_transformers_amd.parts import Embedding, LayerNorm, Linear, OutputHead
+
+    H = 200
+    x = _rand(9, H).bfloat16()
+    ln, ln2 = LayerNorm("n1", H, 1e-5), LayerNorm("n2", H, 1e-5)
+    (_, r1), (_, r2) = _fill(ln, dtype, 1), _fill(ln2, dtype, 2)
+    want1 = P.layer_norm(x.double(), r1["n1.weight"], r1["n1.bias"], 1e-5)
+    _close(ln.forward(x.to(dtype).cuda()), want1, rel, "LayerNorm")
+    a, b = ln.forward_pair(x.to(dtype).cuda(), ln2)
+    _close(a, want1, rel, "LayerNorm pair, first")
+    _close(b, P.layer_norm(x.double(), r2["n2.weight"], r2["n2.bias"], 1e-5), rel, "LayerNorm pair, second")
+    rows = torch.tensor([8, 0], dtype=torch.int32).cuda()
+    _close(ln.forward(x.to(dtype).cuda(), rows=rows), want1[[8, 0]], rel, "LayerNorm on chosen rows")
+
+    for M in (3, 100):  # few rows: the decode kernel in bfloat16; many: the library product plus epilogue
+        x = _rand(M, H, seed=M).bfloat16()
+        lin = Linear("lin", H, 72, bias=True)
+        _, r = _fill(lin, dtype, 3)
+        add = _rand(M, 72, seed=5).bfloat16()
+        want = P.gelu(P.linear(x.double(), r["lin.weight"], r["lin.bias"])) + add.double()
+        _close(lin(x.to(dtype).cuda(), act="gelu", add1=add.to(dtype).cuda()), want, rel, f"Linear, {M} rows")
+        _close(lin(x.to(dtype).cuda(), apply_bias=False), x.double() @ r["lin.weight"].T, rel, "Linear without bias")
+
+    emb = Embedding("emb", 50, H)
+    _, r = _fill(emb, dtype, 4)
+    ids = torch.tensor([3, 49, 0, 3], dtype=torch.int32).cuda()
+    _close(emb.forward(ids), r["emb.weight"][[3, 49, 0, 3]], 0.0, "Embedding")
+    head = OutputHead("head", 50, H, tied_to=None)
+    _, r = _fill(head, dtype, 5)
+    for M in (2, 70):
+        h = _rand(M, H, seed=7).bfloat16()
+        out = head.forward(h.to(dtype).cuda())
+        assert out.dtype == torch.float32
+        _close(out, h.double() @ r["head.weight"].T, rel, f"OutputHead, {M} rows")
+
+
+def test_positions():
+    from pytorch_transformers_amd.parts import AlibiPositions, NoPositions, RotaryPositions
+
+    r = RotaryPositions(64, 500042.0, scaling_factor=4.0)
+    inv, scale = r.rotation()
+    assert torch.equal(inv, P.rope_inv_freq(64, 500042.0, 4.0)) and scale == 1.0 and r.score_bias() is None
+    for nh in (6, 20, 64):
+        a = AlibiPositions(nh)
+        assert torch.equal(a.score_bias(), P.alibi_slopes(nh).bfloat16().float()) and a.rotation() == (None, 1.0)
+    assert NoPositions().rotation() == (None, 1.0) and NoPositions().score_bias() is None
+
+
+@pytest.mark.parametrize("dtype,rel", DTYPES)
+@pytest.mark.parametrize("layout,nh,nkv,d,alibi,bias", [("grouped", 6, 2, 32, False, False), ("tail", 5, 1, 64, False, True),
+                                                        ("interleaved", 3, 3, 24, True, True)])
+def test_attention_mixer_and_blocks(dtype, rel, layout, nh, nkv, d, alibi, bias):
+    """The mixer alone (whole prompt, then a chunk, then single tokens), and both block arrangements around it."""
+    from pytorch_transformers_amd.cache import PagedCache
+    from pytorch_transformers_amd.engine.spec import CACHE_FULL, CacheGroupSpec, LayerCall
+    from pytorch_transformers_amd.parts import (AlibiPositions, AttentionMixer, DenseFeedForward, LayerNorm, ParallelBlock,
+                                                RotaryPositions, SequentialBlock)
+
+    H, F, T = nh * d, 3 * nh * d + 8, 75
+    pos = AlibiPositions(nh) if alibi else RotaryPositions(d, 10000.0)
+    pos.to("cuda:0")
+    mixer = AttentionMixer("transformer.h.0.self_attention", H, nh, nkv, d, layout, bias, pos)
+    ffn = DenseFeedForward("transformer.h.0.mlp", H, F, bias)
+    n1, n2 = LayerNorm("transformer.h.0.input_layernorm", H, 1e-5), LayerNorm("transformer.h.0.post_attention_layernorm", H, 1e-5)
+    n3, n4 = LayerNorm("transformer.h.0.ln_attn", H, 1e-5), LayerNorm("transformer.h.0.ln_mlp", H, 1e-5)
+    ref = {}
+    for i, part in enumerate((mixer, ffn, n1, n2, n3, n4)):
+        ref.update(_fill(part, dtype, 10 + i)[1])
+    c = P.cfg_defaults(dict(hidden_size=H, num_attention_heads=nh, num_kv_heads=nkv, alibi=alibi, bias=bias,
+                            new_decoder_architecture=layout == "grouped", multi_query=layout == "tail",
+                            ffn_hidden_size=F))
+    x = _rand(T, H, seed=1).bfloat16()
+    positions = torch.arange(T)
+    want_mixer = P.self_attention(x.double(), ref, "transformer.h.0.self_attention.", c, positions)
+    call = LayerCall(0, "kv", 0)
+
+    def run(fn, cuts):
+        cache = PagedCache([CacheGroupSpec("kv", CACHE_FULL, 1, nkv, d)], 256, dtype, "cuda:0")
+        slot = cache.alloc()
+        outs, at = [], 0
+        for n in cuts:
+            ctx, plan = _ctx(cache, [slot], [n], dtype)
+            outs.append(fn(x[at:at + n].to(dtype).cuda(), ctx))
+            cache.commit([slot], [n])
+            at += n
+        return torch.cat(outs)
+
+    cuts = [40, 30, 1, 1, 1, 1, 1]
+    _close(run(lambda xs, ctx: mixer.forward(xs, ctx, call), [T]), want_mixer, rel, "mixer, whole")
+    _close(run(lambda xs, ctx: mixer.forward(xs, ctx, call), cuts), want_mixer, rel, "mixer, cut")
+    res = run(lambda xs, ctx: mixer.forward(xs, ctx, call, residual=xs), cuts)
+    _close(res, want_mixer + x.double(), rel, "mixer with residual")
+
+    # blocks: each arrangement is a decoder layer of the plain implementation with the matching flags
+    for block, flags in ((ParallelBlock(mixer, ffn, n1), dict(parallel_attn=True, new_decoder_architecture=False)),
+                         (SequentialBlock(mixer, ffn, n1, n2), dict(parallel_attn=False, new_decoder_architecture=False)),
+                         (ParallelBlock(mixer, ffn, n3, n4), dict(parallel_attn=True, new_decoder_architecture=True,
+                                                                  num_ln_in_parallel_attn=2))):
+        if flags["new_decoder_architecture"] != (layout == "grouped"):
+            continue  # the fused row order belongs to the architecture flag in the plain code
+        cc = P.cfg_defaults(dict(c, **flags))
+        want = P.decoder_layer(x.double(), ref, 0, cc, positions)
+        _close(run(lambda xs, ctx: block.forward(xs, ctx, call), cuts), want, rel, f"{type(block).__name__} {flags}")
+
+
+# --- a toy architecture, defined in the test -------------------------------------------------------------
+def _define_toy():
+    from pytorch_transformers_amd.config.base import ModelConfig
+    from pytorch_transformers_amd.engine.spec import (CACHE_FULL, CACHE_STATE, INIT_NORMAL, MATRIX, CacheGroupSpec,
+                                                      LayerCall, ModelSpec, TensorSpec)
+    from pytorch_transformers_amd.parts import (AttentionMixer, DenseFeedForward, Embedding, LayerNorm, NoPositions,
+                                                OutputHead, ParallelBlock, Part, SequentialBlock, register_part)
+
+    @dataclasses.dataclass
+    class ToyConfig(ModelConfig):
+        model_type = "toy-decay"
+        vocab_size: int = 97
+        width: int = 48
+        layers: int = 3
+        decay: float = 0.8
+
+    class DecayMixer(Part):
+        """y_t = s_t @ W, s_t = decay * s_{t-1} + x_t: a running state per sequence instead of keys and values."""
+
+        def __init__(self, name, width, decay):
+            self.name, self.width, self.decay = name, width, decay
+
+        def tensor_specs(self):
+            return [TensorSpec(self.name + ".weight", (self.width, self.width), MATRIX, INIT_NORMAL)]
+
+        def load(self, tensors):
+            self.weight = tensors[self.name + ".weight"]
+
+        def forward(self, x, ctx, call, residual=None):
+            table = ctx.cache.state_layer(call.cache_group, call.cache_layer)  # [slots, width], 32-bit
+            out = torch.empty_like(x)
+            at = 0
+            for slot, n in zip(ctx.slots, ctx.new_tokens):
+                s = table[slot].clone()
+                for t in range(at, at + n):
+                    s = self.decay * s + x[t].float()
+                    out[t] = (s @ self.weight.float().T).to(x.dtype)
+                table[slot] = s
+                at += n
+            return out if residual is None else out + residual
+
+    register_part("mixer", "decay", DecayMixer, exist_ok=True)
+
+    def build_toy(cfg):
+        blocks, order = [], []
+        for i in range(cfg.layers):
+            p = f"toy.h.{i}"
+            ffn = DenseFeedForward(f"{p}.mlp", cfg.width, 2 * cfg.width, bias=False)
+            if i == 1:  # one attention layer among the state layers: two cache groups in one model
+                mixer = AttentionMixer(f"{p}.attn", cfg.width, 3, 1, 16, "tail", False, NoPositions())
+                blocks.append(ParallelBlock(mixer, ffn, LayerNorm(f"{p}.norm", cfg.width, 1e-5)))
+                order.append(LayerCall(i, "kv", 0))
+            else:
+                mixer = DecayMixer(f"{p}.decay", cfg.width, cfg.decay)
+                blocks.append(SequentialBlock(mixer, ffn, LayerNorm(f"{p}.n1", cfg.width, 1e-5), LayerNorm(f"{p}.n2", cfg.width, 1e-5)))
+                order.append(LayerCall(i, "state", len([c for c in order if c.cache_group == "state"])))
+        order.append(LayerCall(0, "state", cfg.layers - 1))  # block 0 runs a second time, on a state layer of its own
+        return ModelSpec(config=cfg, embedding=Embedding("toy.embed", cfg.vocab_size, cfg.width), blocks=blocks, order=order,
+                         final_norm=LayerNorm("toy.final", cfg.width, 1e-5),
+                         head=OutputHead("toy.head", cfg.vocab_size, cfg.width, "toy.embed.weight"),
+                         cache_groups=[CacheGroupSpec("kv", CACHE_FULL, 1, 1, 16),
+                                       CacheGroupSpec("state", CACHE_STATE, cfg.layers, state_shape=(cfg.width,))],
+                         supports_graphs=False)  # the toy mixer reads the step's host lists
+
+    return ToyConfig, build_toy
+
+
+def _plain_toy(cfg, w, ids):
+    """The toy model whole, in float64, from the same tensors."""
+    x = w["toy.embed.weight"][torch.as_tensor(ids)]
+    T = len(ids)
+
+    def decay_mixer(h, name):
+        s, out = torch.zeros(cfg.width, dtype=torch.float64), []
+        for t in range(T):
+            s = cfg.decay * s + h[t]
+            out.append(s @ w[name + ".weight"].T)
+        return torch.stack(out)
+
+    def ffn(h, p):
+        return P.gelu(h @ w[p + ".mlp.dense_h_to_4h.weight"].T) @ w[p + ".mlp.dense_4h_to_h.weight"].T
+
+    def ln(h, name):
+        return P.layer_norm(h, w[name + ".weight"], w[name + ".bias"], 1e-5)
+
+    def state_block(h, i):
+        p = f"toy.h.{i}"
+        r = h + decay_mixer(ln(h, p + ".n1"), p + ".decay")
+        return r + ffn(ln(r, p + ".n2"), p)
+
+    for i in list(range(cfg.layers)) + [0]:
+        p = f"toy.h.{i}"
+        if i == 1:
+            a = ln(x, p + ".norm")
+            fused = a @ w[p + ".attn.query_key_value.weight"].T
+            qkv = fused.view(T, 5, 16)
+            o = P.attention_scores_softmax(qkv[:, :3], qkv[:, [3]], qkv[:, [4]])
+            x = x + (ffn(a, p) + o @ w[p + ".attn.dense.weight"].T)
+        else:
+            x = state_block(x, i)
+    return ln(x, "toy.final") @ w["toy.embed.weight"].T
+
+
+@pytest.mark.parametrize("dtype,rel", [("float32", helpers.REL_F32), ("bfloat16", helpers.REL_BF16)])
+def test_toy_architecture_with_a_state_mixer(tmp_path, dtype, rel):
+    """Register, write random weights, load, replay whole / one by one / in unequal batches with slot
+    reuse, and generate: all through the framework's own entry points."""
+    from safetensors.torch import load_file
+
+    from pytorch_transformers_amd import AutoModelForCausalLM
+    from pytorch_transformers_amd.config import AutoConfig, register, unregister
+    from pytorch_transformers_amd.engine.replay import Replayer
+    from pytorch_transformers_amd.weights import write_random_model
+
+    ToyConfig, build_toy = _define_toy()
+    register("toy-decay", ToyConfig, build_toy, exist_ok=True)
+    try:
+        cfg = ToyConfig(decay=0.7, layers=3)
+        folder = write_random_model(str(tmp_path / "toy"), cfg, seed=5, std=0.08, noise=0.1)
+        assert isinstance(AutoConfig.from_pretrained(folder), ToyConfig)
+        model = AutoModelForCausalLM.from_pretrained(folder, dtype=dtype)
+        assert not model.use_graphs
+        w = {k: v.double() for k, v in load_file(f"{folder}/model.safetensors").items()}
+        reqs = helpers.make_requests(cfg.vocab_size, [9, 30, 70, 3, 41], seed=2)
+        want = {rid: _plain_toy(cfg, w, toks).float() for rid, toks in reqs.items()}
+        rp = Replayer(model, 1024, max_slots=8)
+        for name, records in (("whole", helpers.schedule_whole(reqs)), ("tail", helpers.schedule_tail(reqs, 8)),
+                              ("batches", helpers.schedule_batches(reqs, 3)), ("batches again", helpers.schedule_batches(reqs, 2))):
+            got = helpers.run_schedule(rp, records)
+            for rid in reqs:
+                helpers.assert_close(got[rid], want[rid], rel, f"toy {dtype} {name} {rid}")
+        # a slot that is used again starts from zero state: a stale state would change these logits
+        assert not rp.cache.live_slots()
+        if dtype == "float32":
+            out = model.generate([reqs["r0"], reqs["r3"]], max_new_tokens=5, do_sample=False, eos_token_id=None)
+            for seq, rid in zip(out, ("r0", "r3")):
+                toks = list(reqs[rid])
+                for _ in range(5):
+                    toks.append(int(_plain_toy(cfg, w, toks)[-1].argmax()))
+                assert seq == toks
+    finally:
+        unregister("toy-decay")
