@@ -25,6 +25,8 @@
 #include "common.h"
 #include "pta_kernels.h"
 
+#include <stdlib.h>
+
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
@@ -33,9 +35,17 @@ union AFrag {
     bf16x8_t v;
 };
 
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+
+// two 32-bit floats to two bfloat16 (round to nearest even) in one instruction
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-    return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+    union { bf16x2_t b; uint32_t u; } c;
+    c.b = __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t);
+    return c.u;
 }
+
+#define PTA_LOG2E 1.4426950408889634f
 
 template <int DT>
 struct KvBlock {
@@ -73,7 +83,7 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(
     bf16_t* __restrict__ out, float* __restrict__ po, float* __restrict__ pm, float* __restrict__ pl,
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
     const int* __restrict__ block_table, int bt_stride, const int* __restrict__ cu_tokens,
-    const int* __restrict__ seq_start, const float* __restrict__ slopes, int nh, int nkv, float scale, float sqrt_d,
+    const int* __restrict__ seq_start, const float* __restrict__ slopes, int nh, int nkv, float scale, float alibi_mul,
     int split_size, int n_splits) {
     constexpr int D = DT * 16;
     constexpr int DS = (DT + 1) / 2;   // 32-wide steps over the head dimension
@@ -82,7 +92,9 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(
     const int seq = blockIdx.z / n_splits, split = blockIdx.z % n_splits;
     const int kvh = blockIdx.y, g = nh / nkv;
     const int t0 = cu_tokens[seq], n_new = cu_tokens[seq + 1] - t0, start = seq_start[seq];
-    const int ncols = n_new * g, col0 = blockIdx.x * (16 * CT);
+    // column groups are handed out last first: late tokens see the most keys, and the longest work
+    // should start first so that the launch ends evenly
+    const int ncols = n_new * g, col0 = (gridDim.x - 1 - blockIdx.x) * (16 * CT);
     if (col0 >= ncols) return;
     const int last_col = min(ncols, col0 + 16 * CT) - 1;
     const int max_qpos = start + last_col / g;
@@ -90,6 +102,8 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(
     const int k_begin = n_splits > 1 ? split * split_size : 0;
     const int k_end = n_splits > 1 ? min(max_qpos + 1, k_begin + split_size) : max_qpos + 1;
     const int kb_last = (kv_len - 1) & ~31;  // the last block that has a page
+    // below this key index no column of this wave masks anything (columns are ordered by token)
+    const int min_lim = min(start + col0 / g + 1, k_end);
     const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
     // in the last 32-wide step of an odd number of 16-wide tiles, the upper half of the lanes has no data
     const uint32_t tail_keep = (DT % 2 == 1 && (DS - 1) * 4 + gq >= CHUNKS) ? 0u : 0xffffffffu;
@@ -161,6 +175,9 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(
                 for (int ds = 0; ds < DS; ++ds)
                     sacc[tt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b.k[tt][ds].v, qf[ct][ds].v, sacc[tt][ct], 0, 0, 0);
             }
+        // Scores are kept in units of log 2 (the scale carries log2 e), so that the exponential is the
+        // hardware's exp2.  A block that lies wholly below every column's limit needs no masking.
+        const bool interior = kb + 32 <= min_lim;
         AFrag pf[CT];
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
@@ -171,28 +188,31 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(
             for (int j = 0; j < 8; ++j) {
                 const int key = kb + 8 * gq + j;  // j = 4*tt + e
                 float v = sacc[j >> 2][ct][j & 3] * scale;
-                if (slopes) v += round_to_bf16(slope[ct] * round_to_bf16((float)key)) / sqrt_d;
-                s[j] = key < lim ? v : -INFINITY;
+                if (slopes) v += round_to_bf16(slope[ct] * round_to_bf16((float)key)) * alibi_mul;
+                s[j] = (interior || key < lim) ? v : -INFINITY;
                 mx = fmaxf(mx, s[j]);
             }
             mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
             mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
             const float m_new = fmaxf(m_run[ct], mx);
             const float m_use = m_new == -INFINITY ? 0.f : m_new;
-            const float corr = expf(m_run[ct] - m_use);
             float p[8], psum = 0.f;
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                p[j] = expf(s[j] - m_use);
+                p[j] = __builtin_amdgcn_exp2f(s[j] - m_use);
                 psum += p[j];
             }
-            l_run[ct] = l_run[ct] * corr + psum;
-            m_run[ct] = m_new;
             pf[ct].u = make_uint4(pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7]));
+            if (__any(m_new > m_run[ct])) {  // the running maximum moved for some column: rescale what was summed
+                const float corr = __builtin_amdgcn_exp2f(m_run[ct] - m_use);
+                l_run[ct] *= corr;
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                oacc[dt][ct][0] *= corr; oacc[dt][ct][1] *= corr; oacc[dt][ct][2] *= corr; oacc[dt][ct][3] *= corr;
+                for (int dt = 0; dt < DT; ++dt) {
+                    oacc[dt][ct][0] *= corr; oacc[dt][ct][1] *= corr; oacc[dt][ct][2] *= corr; oacc[dt][ct][3] *= corr;
+                }
             }
+            l_run[ct] += psum;
+            m_run[ct] = m_new;
         }
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
@@ -249,7 +269,7 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(
     }
 }
 
-// out[row, :] = sum_s w_s po[row, s, :] / sum_s w_s pl[row, s], w_s = exp(pm[row, s] - max_s pm), splits in
+// out[row, :] = sum_s w_s po[row, s, :] / sum_s w_s pl[row, s], w_s = 2^(pm[row, s] - max_s pm), splits in
 // order.  A split whose maximum is -inf (a range past the row's keys) has weight zero and is not read.
 __global__ __launch_bounds__(64) void attn_combine_kernel(bf16_t* __restrict__ out, const float* __restrict__ po,
                                                           const float* __restrict__ pm, const float* __restrict__ pl,
@@ -267,7 +287,7 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(bf16_t* __restrict__ o
     for (int s0 = 0; s0 < n_splits; s0 += 64) {  // lanes in order, chunks in order: a fixed summation order
         const int s = s0 + lane;
         float w = 0.f;
-        if (s < n_splits && m[s] != -INFINITY) { w = expf(m[s] - mx); used = s + 1; }
+        if (s < n_splits && m[s] != -INFINITY) { w = __builtin_amdgcn_exp2f(m[s] - mx); used = s + 1; }
         if (s < n_splits) w_s[s] = w;
         L += wave_sum(w * (s < n_splits ? l[s] : 0.f));
     }
@@ -295,8 +315,8 @@ static void launch_attn(bf16_t* out, float* po, float* pm, float* pl, const bf16
     const int g = nh / nkv;
     const dim3 grid((max_new * g + 16 * CT - 1) / (16 * CT), nkv, n_seqs * n_splits);
     hipLaunchKernelGGL((attn_mfma_kernel<DT, CT>), grid, dim3(64), 0, s, out, po, pm, pl, q, k_pool, v_pool, block_table,
-                       bt_stride, cu_tokens, seq_start, slopes, nh, nkv, scale, sqrtf((float)(DT * 16)), split_size,
-                       n_splits);
+                       bt_stride, cu_tokens, seq_start, slopes, nh, nkv, scale * PTA_LOG2E,
+                       PTA_LOG2E / sqrtf((float)(DT * 16)), split_size, n_splits);
 }
 
 extern "C" int pta_attn_mfma_supported(int d) { return d % 16 == 0 && ((d >= 16 && d <= 128) || d == 256); }
@@ -318,9 +338,17 @@ extern "C" int pta_attn_mfma(void* out, const void* q, const void* k_pool, const
     // one token per sequence (decode): one column tile per wave, so that the tiles of a KV head run side
     // by side; prompts: several tiles per wave, so that a key block is loaded once for all of them
     const bool narrow = max_new == 1;
+    // column tiles per wave for prompts.  Measured at Falcon-7B sizes (2,048 tokens, 71 heads on one KV
+    // head): 2 tiles 148 us a layer, 4 tiles 195 us, 1 tile 270 us: fewer tiles balance the causal
+    // triangle better, more tiles re-read keys less.  PTA_ATTN_CT overrides for tuning.
+    static const int ct_env = getenv("PTA_ATTN_CT") ? atoi(getenv("PTA_ATTN_CT")) : 2;
 #define PTA_ATTN_CASE(DT_, CT_)                                                                                     \
     case DT_:                                                                                                       \
-        if (narrow)                                                                                                 \
+        if (!narrow && ct_env == 2 && CT_ > 2)                                                                      \
+            launch_attn<DT_, 2>((bf16_t*)out, po, pm, pl, (const bf16_t*)q, (const bf16_t*)k_pool,                  \
+                                (const bf16_t*)v_pool, block_table, bt_stride, cu_tokens, seq_start, slopes, n_seqs, \
+                                max_new, nh, nkv, scale, split_size, n_splits, s);                                  \
+        else if (narrow || ct_env == 1)                                                                             \
             launch_attn<DT_, 1>((bf16_t*)out, po, pm, pl, (const bf16_t*)q, (const bf16_t*)k_pool,                  \
                                 (const bf16_t*)v_pool, block_table, bt_stride, cu_tokens, seq_start, slopes, n_seqs, \
                                 max_new, nh, nkv, scale, split_size, n_splits, s);                                  \

@@ -8,8 +8,8 @@
 // flight while the matrix cores consume the current one (two register buffers), so every wave
 // keeps 2*U*RT KB of W on its way from HBM for as long as it runs.  W rows are the A operand of
 // v_mfma_f32_16x16x32_bf16 (lane: row = lane % 16, eight consecutive k at (lane / 16) * 8, one
-// 16-byte load straight from global memory), x rows are the B operand (same shape, read through
-// the caches; x is small).  The S partial tiles are summed through LDS in wave order, then bias,
+// 16-byte load straight from global memory), x rows are the B operand (same shape, buffer loads whose
+// bounds are the M real rows, so the padding rows of the tile read zeros and cost no traffic).  The S partial tiles are summed through LDS in wave order, then bias,
 // activation and additions are applied and the tile is stored.  S is chosen from N and K alone, so
 // the order of summation never depends on M or on what else is in the batch.
 #include "common.h"
@@ -18,9 +18,12 @@
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
+typedef int i32x4_t __attribute__((ext_vector_type(4)));
+
 union Frag {
     uint4 u;
     bf16x8_t v;
+    i32x4_t i;
 };
 
 template <typename OutT> struct OutIo;
@@ -45,7 +48,7 @@ struct Stage {
 // the wave wait for loads it has just issued, and the two stages would no longer overlap.
 template <int MT, int RT, int U>
 __device__ __forceinline__ void load_stage(Stage<MT, RT, U>& st, const bf16_t* const (&wrow)[RT],
-                                           const bf16_t* const (&xrow)[MT], int first_step, int S, int g, int K) {
+                                           __amdgpu_buffer_rsrc_t xres, int r, int first_step, int S, int g, int K) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const int k0 = (first_step + u * S) * 64 + g * 8;  // K % 8 == 0: a chunk of 8 is inside K or outside it
@@ -57,7 +60,8 @@ __device__ __forceinline__ void load_stage(Stage<MT, RT, U>& st, const bf16_t* c
 #pragma unroll
             for (int t = 0; t < RT; ++t) st.a[u][hf][t].u = *reinterpret_cast<const uint4*>(wrow[t] + kc);
 #pragma unroll
-            for (int t = 0; t < MT; ++t) st.b[u][hf][t].u = *reinterpret_cast<const uint4*>(xrow[t] + kc);
+            for (int t = 0; t < MT; ++t)  // a row past M lies outside the buffer's bounds: it reads zeros and costs no traffic
+                st.b[u][hf][t].i = __builtin_amdgcn_raw_buffer_load_b128(xres, ((t * 16 + r) * K + kc) * 2, 0, 0);
         }
     }
 }
@@ -90,9 +94,8 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(
     const bf16_t* wrow[RT];
 #pragma unroll
     for (int t = 0; t < RT; ++t) wrow[t] = W + (long)min(n0 + t * 16 + r, N - 1) * K;
-    const bf16_t* xrow[MT];
-#pragma unroll
-    for (int t = 0; t < MT; ++t) xrow[t] = x + (long)min(t * 16 + r, M - 1) * K;
+    // x through a buffer descriptor whose bounds are the M real rows (0x00020000: 32-bit raw data format)
+    __amdgpu_buffer_rsrc_t xres = __builtin_amdgcn_make_buffer_rsrc((void*)x, 0, M * K * 2, 0x00020000);
 
     f32x4_t acc[RT][MT];
 #pragma unroll
@@ -102,15 +105,15 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(
 
     const int nsteps = (K + 63) >> 6;
     Stage<MT, RT, U> s0, s1;
-    load_stage<MT, RT, U>(s0, wrow, xrow, wave, S, g, K);
+    load_stage<MT, RT, U>(s0, wrow, xres, r, wave, S, g, K);
     // the scheduling barriers keep the compiler from sinking a stage's loads down to their first
     // use, which would shrink what is in flight to a load or two
     for (int step = wave; step < nsteps; step += 2 * U * S) {
-        load_stage<MT, RT, U>(s1, wrow, xrow, step + U * S, S, g, K);
+        load_stage<MT, RT, U>(s1, wrow, xres, r, step + U * S, S, g, K);
         __builtin_amdgcn_sched_barrier(0);
         compute_stage<MT, RT, U>(s0, acc);
         __builtin_amdgcn_sched_barrier(0);
-        load_stage<MT, RT, U>(s0, wrow, xrow, step + 2 * U * S, S, g, K);
+        load_stage<MT, RT, U>(s0, wrow, xres, r, step + 2 * U * S, S, g, K);
         __builtin_amdgcn_sched_barrier(0);
         compute_stage<MT, RT, U>(s1, acc);
         __builtin_amdgcn_sched_barrier(0);
@@ -198,6 +201,7 @@ extern "C" int pta_gemm_skinny_bf16(void* y, const void* x, const void* W, const
     PTA_REQUIRE(M <= 64, "gemm_skinny_bf16: at most 64 rows, got %d (use the library product)", M);
     PTA_REQUIRE(K % 8 == 0, "gemm_skinny_bf16: K=%d must be a multiple of 8 (16-byte loads)", K);
     PTA_REQUIRE(y && x && W, "gemm_skinny_bf16: null pointer");
+    PTA_REQUIRE((long)M * K * 2 < (1L << 31), "gemm_skinny_bf16: x is too large for 32-bit buffer offsets");
     PTA_REQUIRE(((uintptr_t)x % 16) == 0 && ((uintptr_t)W % 16) == 0, "gemm_skinny_bf16: x and W must be 16-byte aligned");
     PTA_REQUIRE(act == PTA_ACT_NONE || act == PTA_ACT_GELU, "gemm_skinny_bf16: unknown activation %d", act);
     PTA_REQUIRE(variant >= 0 && variant <= 4, "gemm_skinny_bf16: unknown variant %d", variant);

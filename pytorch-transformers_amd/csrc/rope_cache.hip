@@ -9,69 +9,75 @@
 // Rotation pairs element i with i + d/2 (rotate_half, :76-80; apply :104-108); the angle is
 // position * inv_freq[i], taken in 32-bit (:155-164).  Keys are stored rotated (:350-358).
 // Key pages are [kv_head][64 positions][d]; value pages are transposed, [kv_head][d][64 positions].
+//
+// One workgroup per token: the d/2 cosines and sines of the token's position are computed once into
+// LDS and used by every head; then the threads walk (head, element) items of the whole fused row.
 #include "common.h"
 #include "pta_kernels.h"
 
+#define RC_THREADS 256
+
 template <typename T>
-__global__ void qkv_rope_cache_kernel(T* __restrict__ q_out, const T* __restrict__ fused,
-                                      const float* __restrict__ bias, const float* __restrict__ inv_freq,
-                                      float cs_scale, const int* __restrict__ token_pos,
-                                      const int* __restrict__ token_seq, const int* __restrict__ block_table,
-                                      int bt_stride, T* __restrict__ k_pool, T* __restrict__ v_pool, int nh, int nkv,
-                                      int d, int layout, int write_cache) {
-    const int m = blockIdx.x;
-    const int slot = blockIdx.y;  // 0..nh-1 queries, then nkv keys, then nkv values
-    const int g = nh / nkv;
-    int kind, head;  // kind 0 q, 1 k, 2 v
-    if (slot < nh) { kind = 0; head = slot; }
-    else if (slot < nh + nkv) { kind = 1; head = slot - nh; }
-    else { kind = 2; head = slot - nh - nkv; }
-    if (kind != 0 && !write_cache) return;
-
-    int src_head;  // index of the d-wide row block inside the fused row
-    if (layout == PTA_QKV_GROUPED) {
-        src_head = kind == 0 ? (head / g) * (g + 2) + (head % g) : head * (g + 2) + g + (kind - 1);
-    } else if (layout == PTA_QKV_TAIL) {
-        src_head = kind == 0 ? head : nh + (kind - 1);
-    } else {
-        src_head = head * 3 + kind;
-    }
-    const long qout = (long)(nh + 2 * nkv) * d;
-    const T* src = fused + (long)m * qout + (long)src_head * d;
-    const float* bsrc = bias ? bias + (long)src_head * d : nullptr;
-
+__global__ __launch_bounds__(RC_THREADS) void qkv_rope_cache_kernel(
+    T* __restrict__ q_out, const T* __restrict__ fused, const float* __restrict__ bias,
+    const float* __restrict__ inv_freq, float cs_scale, const int* __restrict__ token_pos,
+    const int* __restrict__ token_seq, const int* __restrict__ block_table, int bt_stride, T* __restrict__ k_pool,
+    T* __restrict__ v_pool, int nh, int nkv, int d, int layout, int write_cache) {
+    __shared__ float cos_s[128], sin_s[128];
+    const int m = blockIdx.x, tid = threadIdx.x;
+    const int g = nh / nkv, half = d >> 1;
     const int pos = token_pos[m];
-    T* dst;
-    long dst_stride = 1;  // values are stored transposed, [d][64], so that eight keys of one feature are contiguous
-    if (kind == 0) {
-        dst = q_out + ((long)m * nh + head) * d;
-    } else {
-        const int seq = token_seq[m];
-        const long page = block_table[(long)seq * bt_stride + pos / PTA_PAGE];
-        if (kind == 1) {
-            dst = k_pool + ((page * nkv + head) * PTA_PAGE + (pos % PTA_PAGE)) * (long)d;
-        } else {
-            dst = v_pool + (page * nkv + head) * (long)PTA_PAGE * d + (pos % PTA_PAGE);
-            dst_stride = PTA_PAGE;
-        }
-    }
-
-    if (kind != 2 && inv_freq) {
-        const int half = d >> 1;
-        for (int i = threadIdx.x; i < half; i += blockDim.x) {
-            float a = Io<T>::ld(src + i), b = Io<T>::ld(src + i + half);
-            if (bsrc) { a = Io<T>::round(a + bsrc[i]); b = Io<T>::round(b + bsrc[i + half]); }
+    if (inv_freq) {
+        for (int i = tid; i < half; i += RC_THREADS) {
             const float ang = (float)pos * inv_freq[i];
-            const float c = cosf(ang) * cs_scale, s = sinf(ang) * cs_scale;
-            Io<T>::st(dst + i, a * c - b * s);
-            Io<T>::st(dst + i + half, b * c + a * s);
+            cos_s[i] = cosf(ang) * cs_scale;
+            sin_s[i] = sinf(ang) * cs_scale;
         }
-    } else {
-        for (int i = threadIdx.x; i < d; i += blockDim.x) {
-            float a = Io<T>::ld(src + i);
-            if (bsrc) a = Io<T>::round(a + bsrc[i]);
-            Io<T>::st(dst + i * dst_stride, a);
+        __syncthreads();
+    }
+    long page = 0;
+    if (write_cache) page = block_table[(long)token_seq[m] * bt_stride + pos / PTA_PAGE];
+    const int in_page = pos % PTA_PAGE;
+    const long qout = (long)(nh + 2 * nkv) * d;
+    const T* row = fused + (long)m * qout;
+    const int n_slots = write_cache ? nh + 2 * nkv : nh;  // queries, then keys, then values
+
+    // rotated items: (slot < nh + nkv, pair i < half); plain items: every element of a slot
+    const int rot_slots = inv_freq ? min(n_slots, nh + nkv) : 0;
+    for (int item = tid; item < rot_slots * half; item += RC_THREADS) {
+        const int slot = item / half, i = item - slot * half;
+        const int kind = slot < nh ? 0 : 1, head = slot < nh ? slot : slot - nh;
+        int src_head;
+        if (layout == PTA_QKV_GROUPED) src_head = kind == 0 ? (head / g) * (g + 2) + (head % g) : head * (g + 2) + g;
+        else if (layout == PTA_QKV_TAIL) src_head = kind == 0 ? head : nh;
+        else src_head = head * 3 + kind;
+        const T* src = row + (long)src_head * d;
+        float a = Io<T>::ld(src + i), b = Io<T>::ld(src + i + half);
+        if (bias) {
+            a = Io<T>::round(a + bias[(long)src_head * d + i]);
+            b = Io<T>::round(b + bias[(long)src_head * d + i + half]);
         }
+        const float c = cos_s[i], s = sin_s[i];
+        T* dst = kind == 0 ? q_out + ((long)m * nh + head) * d
+                           : k_pool + ((page * nkv + head) * PTA_PAGE + in_page) * (long)d;
+        Io<T>::st(dst + i, a * c - b * s);
+        Io<T>::st(dst + i + half, b * c + a * s);
+    }
+    for (int item = tid + rot_slots * d; item < n_slots * d; item += RC_THREADS) {
+        const int slot = item / d, i = item - slot * d;
+        int kind, head;
+        if (slot < nh) { kind = 0; head = slot; }
+        else if (slot < nh + nkv) { kind = 1; head = slot - nh; }
+        else { kind = 2; head = slot - nh - nkv; }
+        int src_head;
+        if (layout == PTA_QKV_GROUPED) src_head = kind == 0 ? (head / g) * (g + 2) + (head % g) : head * (g + 2) + g + (kind - 1);
+        else if (layout == PTA_QKV_TAIL) src_head = kind == 0 ? head : nh + (kind - 1);
+        else src_head = head * 3 + kind;
+        float a = Io<T>::ld(row + (long)src_head * d + i);
+        if (bias) a = Io<T>::round(a + bias[(long)src_head * d + i]);
+        if (kind == 0) Io<T>::st(q_out + ((long)m * nh + head) * d + i, a);
+        else if (kind == 1) Io<T>::st(k_pool + ((page * nkv + head) * PTA_PAGE + in_page) * (long)d + i, a);
+        else Io<T>::st(v_pool + ((page * nkv + head) * (long)d + i) * PTA_PAGE + in_page, a);
     }
 }
 
@@ -84,17 +90,15 @@ extern "C" int pta_qkv_rope_cache(void* q_out, const void* fused, const float* b
     PTA_REQUIRE(layout >= 0 && layout <= 2, "qkv_rope_cache: unknown layout %d", layout);
     PTA_REQUIRE(layout != PTA_QKV_TAIL || nkv == 1, "qkv_rope_cache: the tail layout has one kv head, got %d", nkv);
     PTA_REQUIRE(layout != PTA_QKV_INTERLEAVED || nkv == nh, "qkv_rope_cache: the interleaved layout needs kv heads == heads");
-    PTA_REQUIRE(!inv_freq || d % 2 == 0, "qkv_rope_cache: rotation needs an even head size, got %d", d);
+    PTA_REQUIRE(!inv_freq || (d % 2 == 0 && d <= 256), "qkv_rope_cache: rotation needs an even head size up to 256, got %d", d);
     PTA_REQUIRE(!write_cache || (k_pool && v_pool && block_table && token_seq), "qkv_rope_cache: null cache pointer");
-    PTA_REQUIRE(nh + 2 * nkv <= 65535, "qkv_rope_cache: too many heads for one launch");
     hipStream_t s = (hipStream_t)stream;
-    dim3 grid(M, nh + 2 * nkv);
     if (dtype == PTA_F32)
-        hipLaunchKernelGGL(qkv_rope_cache_kernel<float>, grid, dim3(64), 0, s, (float*)q_out, (const float*)fused,
-                           bias, inv_freq, cs_scale, token_pos, token_seq, block_table, bt_stride, (float*)k_pool,
-                           (float*)v_pool, nh, nkv, d, layout, write_cache);
+        hipLaunchKernelGGL(qkv_rope_cache_kernel<float>, dim3(M), dim3(RC_THREADS), 0, s, (float*)q_out,
+                           (const float*)fused, bias, inv_freq, cs_scale, token_pos, token_seq, block_table, bt_stride,
+                           (float*)k_pool, (float*)v_pool, nh, nkv, d, layout, write_cache);
     else if (dtype == PTA_BF16)
-        hipLaunchKernelGGL(qkv_rope_cache_kernel<bf16_t>, grid, dim3(64), 0, s, (bf16_t*)q_out,
+        hipLaunchKernelGGL(qkv_rope_cache_kernel<bf16_t>, dim3(M), dim3(RC_THREADS), 0, s, (bf16_t*)q_out,
                            (const bf16_t*)fused, bias, inv_freq, cs_scale, token_pos, token_seq, block_table,
                            bt_stride, (bf16_t*)k_pool, (bf16_t*)v_pool, nh, nkv, d, layout, write_cache);
     else
