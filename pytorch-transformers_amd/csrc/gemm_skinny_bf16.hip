@@ -181,7 +181,8 @@ static int launch_skinny(OutT* y, const bf16_t* x, const bf16_t* W, const float*
         if (variant == 1) launch_cfg<1, 1, 4, OutT>(y, x, W, bias, add1, add2, M, N, K, act, S, s);
         else if (variant == 2) launch_cfg<1, 2, 2, OutT>(y, x, W, bias, add1, add2, M, N, K, act, S, s);
         else if (variant == 3) launch_cfg<1, 4, 1, OutT>(y, x, W, bias, add1, add2, M, N, K, act, S, s);
-        else launch_cfg<1, 4, 2, OutT>(y, x, W, bias, add1, add2, M, N, K, act, S, s);
+        else if (variant == 4) launch_cfg<1, 4, 2, OutT>(y, x, W, bias, add1, add2, M, N, K, act, S, s);
+        else launch_cfg<1, 2, 4, OutT>(y, x, W, bias, add1, add2, M, N, K, act, S, s);
     } else if (M <= 32) {
         if (variant == 3 || variant == 4) launch_cfg<2, 4, 1, OutT>(y, x, W, bias, add1, add2, M, N, K, act, S, s);
         else launch_cfg<2, 2, 1, OutT>(y, x, W, bias, add1, add2, M, N, K, act, S, s);
@@ -204,7 +205,7 @@ extern "C" int pta_gemm_skinny_bf16(void* y, const void* x, const void* W, const
     PTA_REQUIRE((long)M * K * 2 < (1L << 31), "gemm_skinny_bf16: x is too large for 32-bit buffer offsets");
     PTA_REQUIRE(((uintptr_t)x % 16) == 0 && ((uintptr_t)W % 16) == 0, "gemm_skinny_bf16: x and W must be 16-byte aligned");
     PTA_REQUIRE(act == PTA_ACT_NONE || act == PTA_ACT_GELU, "gemm_skinny_bf16: unknown activation %d", act);
-    PTA_REQUIRE(variant >= 0 && variant <= 4, "gemm_skinny_bf16: unknown variant %d", variant);
+    PTA_REQUIRE(variant >= 0 && variant <= 5, "gemm_skinny_bf16: unknown variant %d", variant);
     PTA_REQUIRE(waves == 0 || (waves >= 1 && waves <= 8 && (waves & (waves - 1)) == 0),
                 "gemm_skinny_bf16: waves per workgroup must be 0 (choose) or a power of two up to 8, got %d", waves);
     hipStream_t s = (hipStream_t)stream;

@@ -44,7 +44,9 @@ __global__ __launch_bounds__(RC_THREADS) void qkv_rope_cache_kernel(
 
     // rotated items: (slot < nh + nkv, pair i < half); plain items: every element of a slot
     const int rot_slots = inv_freq ? min(n_slots, nh + nkv) : 0;
-    for (int item = tid; item < rot_slots * half; item += RC_THREADS) {
+    // gridDim.y workgroups share a token's items (a decode step has few tokens and many heads)
+    const int stride = RC_THREADS * gridDim.y, first = tid + blockIdx.y * RC_THREADS;
+    for (int item = first; item < rot_slots * half; item += stride) {
         const int slot = item / half, i = item - slot * half;
         const int kind = slot < nh ? 0 : 1, head = slot < nh ? slot : slot - nh;
         int src_head;
@@ -63,7 +65,7 @@ __global__ __launch_bounds__(RC_THREADS) void qkv_rope_cache_kernel(
         Io<T>::st(dst + i, a * c - b * s);
         Io<T>::st(dst + i + half, b * c + a * s);
     }
-    for (int item = tid + rot_slots * d; item < n_slots * d; item += RC_THREADS) {
+    for (int item = first + rot_slots * d; item < n_slots * d; item += stride) {
         const int slot = item / d, i = item - slot * d;
         int kind, head;
         if (slot < nh) { kind = 0; head = slot; }
@@ -93,12 +95,14 @@ extern "C" int pta_qkv_rope_cache(void* q_out, const void* fused, const float* b
     PTA_REQUIRE(!inv_freq || (d % 2 == 0 && d <= 256), "qkv_rope_cache: rotation needs an even head size up to 256, got %d", d);
     PTA_REQUIRE(!write_cache || (k_pool && v_pool && block_table && token_seq), "qkv_rope_cache: null cache pointer");
     hipStream_t s = (hipStream_t)stream;
+    int slices = 1;  // enough workgroups to occupy the chip when the step has few tokens
+    while (slices < 16 && M * slices < 512 && slices * RC_THREADS < (nh + 2 * nkv) * d) slices *= 2;
     if (dtype == PTA_F32)
-        hipLaunchKernelGGL(qkv_rope_cache_kernel<float>, dim3(M), dim3(RC_THREADS), 0, s, (float*)q_out,
+        hipLaunchKernelGGL(qkv_rope_cache_kernel<float>, dim3(M, slices), dim3(RC_THREADS), 0, s, (float*)q_out,
                            (const float*)fused, bias, inv_freq, cs_scale, token_pos, token_seq, block_table, bt_stride,
                            (float*)k_pool, (float*)v_pool, nh, nkv, d, layout, write_cache);
     else if (dtype == PTA_BF16)
-        hipLaunchKernelGGL(qkv_rope_cache_kernel<bf16_t>, dim3(M), dim3(RC_THREADS), 0, s, (bf16_t*)q_out,
+        hipLaunchKernelGGL(qkv_rope_cache_kernel<bf16_t>, dim3(M, slices), dim3(RC_THREADS), 0, s, (bf16_t*)q_out,
                            (const bf16_t*)fused, bias, inv_freq, cs_scale, token_pos, token_seq, block_table,
                            bt_stride, (bf16_t*)k_pool, (bf16_t*)v_pool, nh, nkv, d, layout, write_cache);
     else

@@ -109,4 +109,6 @@ class StepContext:
     is_decode: bool = False
     #: upper bound of any sequence's length after this step, used to size launches
     max_len: int = 0
+    #: a second stream on which a block may run work that does not depend on its mixer (None: do not)
+    side_stream: Any = None
     extras: Dict[str, Any] = dataclasses.field(default_factory=dict)

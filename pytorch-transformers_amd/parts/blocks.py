@@ -8,7 +8,8 @@ parallel    ``x + (ffn(norm_ffn(x)) + mixer(norm_mixer(x)))``; with one norm bot
             feed-forward plus mixer first (:673-674), then the residual (:676).
 sequential  ``r = x + mixer(norm_in(x))``; ``r + ffn(norm_post(r))`` (:652-659, :676).
 
-The additions ride in the last matrix product's epilogue of each branch.
+The additions ride in the last matrix product's epilogue of each branch.  In the parallel block the
+feed-forward's first product does not depend on the mixer, so it may run beside it on a second stream.
 """
 from __future__ import annotations
 
@@ -34,8 +35,20 @@ class ParallelBlock(Part):
             a = m = self.norm_mixer.forward(x)
         else:
             a, m = self.norm_mixer.forward_pair(x, self.norm_ffn)
+        side = ctx.side_stream
+        if side is None or not hasattr(self.feed_forward, "forward_up"):
+            mixed = self.mixer.forward(a, ctx, call)
+            return self.feed_forward.forward(m, ctx, add1=mixed, add2=x)
+        # The feed-forward's first product needs only the norm, not the mixer: it runs on a second
+        # stream beside projection, rotation, attention and output projection, and the two meet at the
+        # feed-forward's second product, whose epilogue sums the branches and the residual.
+        main = torch.cuda.current_stream()
+        side.wait_stream(main)
+        with torch.cuda.stream(side):
+            h = self.feed_forward.forward_up(m, ctx)
         mixed = self.mixer.forward(a, ctx, call)
-        return self.feed_forward.forward(m, ctx, add1=mixed, add2=x)
+        main.wait_stream(side)
+        return self.feed_forward.forward_down(h, ctx, add1=mixed, add2=x)
 
 
 class SequentialBlock(Part):

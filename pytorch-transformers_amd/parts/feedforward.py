@@ -27,5 +27,13 @@ class DenseFeedForward(Part):
     def forward(self, x: torch.Tensor, ctx: StepContext, add1=None, add2=None) -> torch.Tensor:
         return self.down(self.up(x, act=self.activation), add1=add1, add2=add2)
 
+    # The two halves on their own: a block whose feed-forward does not read the mixer's output can run
+    # the first half beside the mixer.
+    def forward_up(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        return self.up(x, act=self.activation)
+
+    def forward_down(self, h: torch.Tensor, ctx: StepContext, add1=None, add2=None) -> torch.Tensor:
+        return self.down(h, add1=add1, add2=add2)
+
 
 register_part("feed_forward", "dense", DenseFeedForward)
