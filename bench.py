@@ -114,6 +114,8 @@ def main():
     ap.add_argument("--layers", type=int, default=32, help="fewer than 32 only where memory or time needs it")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / batch 64 / prefill measurements")
+    ap.add_argument("--only-prefill", action="store_true",
+                    help="run the 2,048-token prefill alone and print its record (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -130,6 +132,12 @@ def main():
     elem = 2 if args.dtype == "bf16" else 4
     model = AutoModelForCausalLM.from_config(cfg, seed=0, dtype=dtype, device="cuda:0")
     gen_cfg = GenerationConfig(do_sample=False, eos_token_id=None)
+    if args.only_prefill:
+        pt = run_prefill(model, 2048)
+        print(json.dumps({"prefill": {"value": round(2048 / pt, 1), "tokens": 2048, "ms": round(pt * 1e3, 3),
+                                      "frac": round(prefill_flops(cfg, 2048) / pt / (PEAK_TFLOPS[args.dtype] * 1e12), 4)},
+                          "layers": args.layers, "dtype": args.dtype}))
+        return 0
 
     dt, mean_ctx = run_decode(model, Sampler, gen_cfg, args.batch, args.prompt_len, args.steps, args.warmup)
     ms = dt / args.steps * 1e3
