@@ -223,8 +223,10 @@ def gemm_f32(a: torch.Tensor, w: torch.Tensor, bias=None, act=None, add1=None, a
     return out
 
 
-ATTN_SPLIT_KEYS = int(os.environ.get("PTA_ATTN_SPLIT", "64"))  # keys per wave when a decode step's context is split; a constant, so that the
-# partition of a context depends on its length alone
+# a decode step's context is split into ranges of ATTN_SPLIT_KEYS keys, one wave each, or of the next
+# power-of-two multiple that keeps the launch at ATTN_SPLIT_WAVES waves or fewer
+ATTN_SPLIT_KEYS = int(os.environ.get("PTA_ATTN_SPLIT", "64"))
+ATTN_SPLIT_WAVES = int(os.environ.get("PTA_ATTN_WAVES", "2048"))
 
 
 def attn_mfma_ok(q: torch.Tensor) -> bool:
@@ -260,6 +262,24 @@ def attn_mfma(q: torch.Tensor, k_pool, v_pool, block_table, cu_tokens, seq_start
     return out
 
 
+def decode_split_size(n_seqs: int, n_heads: int, n_kv_heads: int, max_len: int) -> int:
+    """Keys per wave of a split decode launch: ``ATTN_SPLIT_KEYS``, doubled until the launch has at most
+    ``ATTN_SPLIT_WAVES`` waves (many short waves cost more in start-up than they win in parallelism).
+
+    The batch counts by its next power of two and the context by its next multiple of 1,024, so that a
+    captured step, which is sized for a padded batch and a length bound, splits exactly as the same
+    step run directly."""
+    n = 1
+    while n < n_seqs:
+        n *= 2
+    bound = (max_len + 1023) // 1024 * 1024
+    tiles = n * n_kv_heads * ((n_heads // n_kv_heads + 15) // 16)
+    size = ATTN_SPLIT_KEYS
+    while size < bound and tiles * (bound // size) > ATTN_SPLIT_WAVES:
+        size *= 2
+    return size
+
+
 def attention(q: torch.Tensor, k_pool, v_pool, block_table, ctx, slopes, scale: float) -> torch.Tensor:
     """Attention of a step's tokens over the cache: picks the kernel for the step's shape and type.
 
@@ -267,11 +287,12 @@ def attention(q: torch.Tensor, k_pool, v_pool, block_table, ctx, slopes, scale: 
     split over several waves when every sequence brings one token; anything else: the 32-bit
     kernel."""
     if attn_mfma_ok(q):
-        n_splits = 1
+        n_splits, size = 1, ATTN_SPLIT_KEYS
         if ctx.is_decode and ctx.max_len > ATTN_SPLIT_KEYS:
-            n_splits = (ctx.max_len + ATTN_SPLIT_KEYS - 1) // ATTN_SPLIT_KEYS
+            size = decode_split_size(ctx.n_seqs, q.shape[1], k_pool.shape[1], ctx.max_len)
+            n_splits = (ctx.max_len + size - 1) // size
         return attn_mfma(q, k_pool, v_pool, block_table, ctx.cu_tokens, ctx.seq_start, slopes, scale,
-                         max_new=max(ctx.new_tokens), n_splits=n_splits)
+                         max_new=max(ctx.new_tokens), n_splits=n_splits, split_size=size)
     return attn_generic(q, k_pool, v_pool, block_table, ctx.token_seq, ctx.token_pos, slopes, scale)
 
 
