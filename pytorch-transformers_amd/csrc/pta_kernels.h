@@ -65,6 +65,14 @@ int pta_gemm_f32(float* C, const float* A, const float* W, const float* bias, co
 int pta_gemm_skinny_bf16(void* y, const void* x, const void* W, const float* bias, const void* add1, const void* add2,
                          int M, int N, int K, int act, int out_f32, int variant, int waves, void* stream);
 
+// The same product for a batch of up to 64 rows that shares x through LDS and may split K over workgroups:
+// `part` is a 32-bit workspace [parts, M, N], needed when parts > 1.  rt (row tiles per wave), parts,
+// stage_blocks (64-element blocks of K per stage) and depth (stages in flight) are tuning knobs (0: chosen from N and K); pta_gemm_splitk_parts tells the choice of parts.
+int pta_gemm_splitk_bf16(void* y, float* part, const void* x, const void* W, const float* bias, const void* add1,
+                         const void* add2, int M, int N, int K, int act, int out_f32, int rt, int parts,
+                         int stage_blocks, int depth, void* stream);
+int pta_gemm_splitk_parts(int N, int K);
+
 // processors in the reference's order, then argmax (do_sample 0) or a draw; `work` [R, V] receives the
 // processed scores; hist/hist_off (tokens seen, per row), eos/suppress, uniforms may be null
 int pta_sample(int* out_tok, float* work, const float* logits, int R, int V, int do_sample, float temperature,

@@ -328,16 +328,47 @@ def sample(logits: torch.Tensor, *, do_sample: bool, temperature: float = 1.0, t
 SKINNY_MAX_ROWS = 64
 
 
-def gemm_skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
-    """Whether the decode kernel takes this product and is the faster choice for it.
+def gemm_splitk_bf16(x: torch.Tensor, w: torch.Tensor, bias=None, act=None, add1=None, add2=None,
+                     out_f32: bool = False, rt: int = 0, parts: int = 0, stage_blocks: int = 0,
+                     depth: int = 0) -> torch.Tensor:
+    """act(x @ w.T + bias) + add1 + add2 for a batch of at most 64 rows of bfloat16: x shared through LDS,
+    K split over workgroups where N gives too few of them."""
+    _need(x, "x", torch.bfloat16)
+    _need(w, "w", torch.bfloat16)
+    M, K = x.shape
+    N = w.shape[0]
+    if w.dim() != 2 or w.shape[1] != K:
+        raise KernelError(f"x is [{M}, {K}] but w is {tuple(w.shape)}; w must be [N, {K}]")
+    if bias is not None:
+        _need(bias, "bias", torch.float32, (N,))
+    for name, t in (("add1", add1), ("add2", add2)):
+        if t is not None:
+            _need(t, name, torch.bfloat16, (M, N))
+    if parts == 0:
+        parts = int(load_library().pta_gemm_splitk_parts(N, K))
+    part = torch.empty((parts, M, N), dtype=torch.float32, device=x.device) if parts > 1 else None
+    out = torch.empty((M, N), dtype=torch.float32 if out_f32 else torch.bfloat16, device=x.device)
+    _call("pta_gemm_splitk_bf16", _ptr(out), _ptr(part), _ptr(x), _ptr(w), _ptr(bias), _ptr(add1), _ptr(add2), M, N, K,
+          ACT_CODES[act], int(out_f32), int(rt), int(parts), int(stage_blocks), int(depth), _stream())
+    return out
 
-    It takes at most 64 rows of bfloat16 with K a multiple of 8.  Measured on MI355X against the
-    vendor library at Falcon-7B shapes: up to 16 rows it wins everywhere; from 17 to 64 rows only
-    where K is long against N (the feed-forward's second matrix)."""
-    if not (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and 0 < x.shape[0] <= SKINNY_MAX_ROWS
-            and x.shape[1] % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0):
-        return False
-    return x.shape[0] <= 16 or w.shape[1] >= 2 * w.shape[0]
+
+def _bf16_rows_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
+    return (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.shape[1] % 8 == 0
+            and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+
+
+def gemm_skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether the kernel for few rows takes this product and is the faster choice for it: bfloat16 with K a
+    multiple of 8 and at most 16 rows (measured on MI355X against the vendor library at Falcon-7B shapes)."""
+    return _bf16_rows_ok(x, w) and 0 < x.shape[0] <= 16
+
+
+def gemm_splitk_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether the kernel for a decode batch of 17 to 64 rows is the faster choice.  Measured at Falcon-7B
+    shapes: it beats the vendor library except where N is long against K (the feed-forward's first matrix
+    and the output head), which give the library enough row tiles to fill the chip."""
+    return _bf16_rows_ok(x, w) and 16 < x.shape[0] <= SKINNY_MAX_ROWS and w.shape[0] < 2 * w.shape[1]
 
 
 def gemm_skinny_bf16(x: torch.Tensor, w: torch.Tensor, bias=None, act=None, add1=None, add2=None,

@@ -90,17 +90,44 @@ def test_gemm_skinny_bf16(M, N, K):
     got = ops.gemm_skinny_bf16(x, w, bias, "gelu", a1, a2)
     want = F.gelu((prod.float().bfloat16().float() + bias).bfloat16().float()) + a1.float() + a2.float()
     torch.testing.assert_close(got.float(), want, rtol=2e-2, atol=2e-2 * max(1.0, scale))
-    assert ops.gemm_skinny_ok(x, w) == (M <= 16 or K >= 2 * N)  # where it is also the faster choice
+    assert ops.gemm_skinny_ok(x, w) == (M <= 16)  # where it is also the faster choice
     # a row alone gives the same bits as in the batch
     r = M - 1
     alone = ops.gemm_skinny_bf16(x[r:r + 1].contiguous(), w, out_f32=True)
     assert torch.equal(alone, got32[r:r + 1])
 
 
+@pytest.mark.parametrize("M", [1, 9, 17, 32, 33, 50, 64])
+@pytest.mark.parametrize("N,K,parts,rt,sb,depth", [(16, 64, 0, 0, 0, 0), (100, 200, 0, 0, 0, 0), (100, 200, 3, 2, 2, 2),
+                                                   (4544, 4544, 0, 0, 0, 0), (250, 18176 // 4, 5, 1, 2, 4),
+                                                   (1000, 1096, 1, 2, 2, 4), (333, 2056, 4, 1, 2, 2)])
+def test_gemm_splitk_bf16(M, N, K, parts, rt, sb, depth):
+    """The batch product with x shared through LDS: every row tile count, stage depth and split of K."""
+    ops = _ops()
+    x = _rand(M, K, dtype=torch.bfloat16)
+    w = _rand(N, K, seed=1, dtype=torch.bfloat16, scale=0.05)
+    bias, a1, a2 = _rand(N, seed=2), _rand(M, N, seed=3, dtype=torch.bfloat16), _rand(M, N, seed=4, dtype=torch.bfloat16)
+    prod = x.double() @ w.double().T
+    scale = float(prod.abs().max())
+    kw = dict(parts=parts, rt=rt, stage_blocks=sb, depth=depth)
+    got32 = ops.gemm_splitk_bf16(x, w, out_f32=True, **kw)
+    assert float((got32.double() - prod).abs().max()) <= 2e-5 * scale + 1e-6, "32-bit output: only accumulation error"
+    got = ops.gemm_splitk_bf16(x, w, bias, "gelu", a1, a2, **kw)
+    want = F.gelu((prod.float().bfloat16().float() + bias).bfloat16().float()) + a1.float() + a2.float()
+    torch.testing.assert_close(got.float(), want, rtol=2e-2, atol=2e-2 * max(1.0, scale))
+    # a row alone gives the same bits as in the batch: the split of K does not depend on M
+    r = M - 1
+    alone = ops.gemm_splitk_bf16(x[r:r + 1].contiguous(), w, out_f32=True, **kw)
+    assert torch.equal(alone, got32[r:r + 1])
+
+
 def test_gemm_skinny_refuses_what_it_cannot_do():
     ops = _ops()
     x, w = _rand(65, 64, dtype=torch.bfloat16), _rand(32, 64, dtype=torch.bfloat16)
-    assert not ops.gemm_skinny_ok(x, w)
+    assert not ops.gemm_skinny_ok(x, w) and not ops.gemm_splitk_ok(x, w)
+    assert ops.gemm_splitk_ok(x[:17].contiguous(), w) and not ops.gemm_splitk_ok(x[:16].contiguous(), w)
+    with pytest.raises(ops.KernelError, match="at most 64 rows"):
+        ops.gemm_splitk_bf16(x, w)
     with pytest.raises(ops.KernelError, match="at most 64 rows"):
         ops.gemm_skinny_bf16(x, w)
     x, w = _rand(4, 60, dtype=torch.bfloat16), _rand(32, 60, dtype=torch.bfloat16)
