@@ -9,7 +9,8 @@
 // memory into the A operand registers, one stage ahead of the matrix cores, as in the kernel for
 // few rows.  K is split over gridDim.y workgroups when N alone gives too few of them to occupy the
 // chip; each writes its 32-bit partial tile to `part`, and a second small kernel adds the partials
-// in the order of the ranges and applies bias, activation and additions.  The split is chosen from N
+// in the order of the ranges and applies bias, activation and additions; with reduce = 0 the partials
+// are the result, and the kernel that reads them next adds them in the same order.  The split is chosen from N
 // and K alone, so the order of summation does not depend on the batch.
 //
 // Chunks of x past the workgroup's K range, or rows past M, are read through a buffer descriptor at
@@ -34,7 +35,7 @@ template <int MT, int RT, int U, int D>
 __global__ __launch_bounds__(SK_THREADS) void gemm_splitk_kernel(
     void* __restrict__ y, float* __restrict__ part, const bf16_t* __restrict__ x, const bf16_t* __restrict__ W,
     const float* __restrict__ bias, const bf16_t* __restrict__ add1, const bf16_t* __restrict__ add2, int M, int N,
-    int K, int act, int out_f32, int blocks_per_part) {
+    int K, int act, int out_f32, int blocks_per_part, int direct) {
     constexpr int KS = U * 64;                       // elements of K per stage
     constexpr int MP = MT * 16;                      // rows of x, padded to whole tiles
     constexpr int LDW = KS + 8;                      // LDS row stride: 16 bytes of padding keep 16-byte reads off each other's banks
@@ -130,7 +131,6 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_splitk_kernel(
     }
 
     // lane: row m = mt*16 + r of x, columns n_base + t*16 + g*4 + 0..3
-    const bool direct = gridDim.y == 1;
 #pragma unroll
     for (int t = 0; t < RT; ++t)
 #pragma unroll
@@ -191,11 +191,21 @@ static int pick_parts(int N, int K, int rt) {
     return max(1, min(P, 16));
 }
 
-extern "C" int pta_gemm_splitk_parts(int N, int K) { return pick_parts(N, K, pick_rt(N)); }
+// ranges that are not empty when K is cut into `parts` ranges of whole 64-element blocks
+static int effective_parts(int K, int parts) {
+    const int nkb = (K + 63) / 64, per = (nkb + parts - 1) / parts;
+    return (nkb + per - 1) / per;
+}
+
+extern "C" int pta_gemm_splitk_parts(int N, int K, int parts, int rt) {
+    if (N <= 0 || K <= 0) return 0;
+    if (rt <= 0) rt = pick_rt(N);
+    return effective_parts(K, parts > 0 ? parts : pick_parts(N, K, rt));
+}
 
 template <int MT, int RT, int U, int D>
 static int launch_cfg(void* y, float* part, const bf16_t* x, const bf16_t* W, const float* bias, const bf16_t* add1,
-                      const bf16_t* add2, int M, int N, int K, int act, int out_f32, int P, hipStream_t s) {
+                      const bf16_t* add2, int M, int N, int K, int act, int out_f32, int P, int reduce, hipStream_t s) {
     const int nkb = (K + 63) / 64;
     const int per = (nkb + P - 1) / P;
     const int parts = (nkb + per - 1) / per;  // ranges that are not empty
@@ -210,8 +220,9 @@ static int launch_cfg(void* y, float* part, const bf16_t* x, const bf16_t* W, co
         }
     }
     const dim3 grid((N + 64 * RT - 1) / (64 * RT), parts);
-    hipLaunchKernelGGL(kern, grid, dim3(SK_THREADS), lds, s, y, part, x, W, bias, add1, add2, M, N, K, act, out_f32, per);
-    if (parts > 1) {
+    hipLaunchKernelGGL(kern, grid, dim3(SK_THREADS), lds, s, y, part, x, W, bias, add1, add2, M, N, K, act, out_f32, per,
+                       (int)(reduce && parts == 1));
+    if (reduce && parts > 1) {
         const long MN = (long)M * N;
         hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((MN + 255) / 256)), dim3(256), 0, s, y, part, bias,
                            add1, add2, MN, N, parts, act, out_f32);
@@ -222,22 +233,22 @@ static int launch_cfg(void* y, float* part, const bf16_t* x, const bf16_t* W, co
 template <int RT, int U, int D>
 static int launch_rows(int MT, void* y, float* part, const bf16_t* x, const bf16_t* W, const float* bias,
                        const bf16_t* add1, const bf16_t* add2, int M, int N, int K, int act, int out_f32, int P,
-                       hipStream_t s) {
+                       int reduce, hipStream_t s) {
     switch (MT) {
-        case 1: return launch_cfg<1, RT, U, D>(y, part, x, W, bias, add1, add2, M, N, K, act, out_f32, P, s);
-        case 2: return launch_cfg<2, RT, U, D>(y, part, x, W, bias, add1, add2, M, N, K, act, out_f32, P, s);
-        case 3: return launch_cfg<3, RT, U, D>(y, part, x, W, bias, add1, add2, M, N, K, act, out_f32, P, s);
-        default: return launch_cfg<4, RT, U, D>(y, part, x, W, bias, add1, add2, M, N, K, act, out_f32, P, s);
+        case 1: return launch_cfg<1, RT, U, D>(y, part, x, W, bias, add1, add2, M, N, K, act, out_f32, P, reduce, s);
+        case 2: return launch_cfg<2, RT, U, D>(y, part, x, W, bias, add1, add2, M, N, K, act, out_f32, P, reduce, s);
+        case 3: return launch_cfg<3, RT, U, D>(y, part, x, W, bias, add1, add2, M, N, K, act, out_f32, P, reduce, s);
+        default: return launch_cfg<4, RT, U, D>(y, part, x, W, bias, add1, add2, M, N, K, act, out_f32, P, reduce, s);
     }
 }
 
 extern "C" int pta_gemm_splitk_bf16(void* y, float* part, const void* x, const void* W, const float* bias,
                                     const void* add1, const void* add2, int M, int N, int K, int act, int out_f32,
-                                    int rt, int parts, int stage_blocks, int depth, void* stream) {
+                                    int rt, int parts, int stage_blocks, int depth, int reduce, void* stream) {
     PTA_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_splitk_bf16: sizes must be positive (M=%d N=%d K=%d)", M, N, K);
     PTA_REQUIRE(M <= 64, "gemm_splitk_bf16: at most 64 rows, got %d (use the library product)", M);
     PTA_REQUIRE(K % 8 == 0 && K >= 8, "gemm_splitk_bf16: K=%d must be a multiple of 8 (16-byte loads)", K);
-    PTA_REQUIRE(y && x && W, "gemm_splitk_bf16: null pointer");
+    PTA_REQUIRE(x && W && (y || !reduce), "gemm_splitk_bf16: null pointer");
     PTA_REQUIRE((long)M * K * 2 < 0x7ffffff0L, "gemm_splitk_bf16: x is too large for 32-bit buffer offsets");
     PTA_REQUIRE(((uintptr_t)x % 16) == 0 && ((uintptr_t)W % 16) == 0, "gemm_splitk_bf16: x and W must be 16-byte aligned");
     PTA_REQUIRE(act == PTA_ACT_NONE || act == PTA_ACT_GELU, "gemm_splitk_bf16: unknown activation %d", act);
@@ -249,14 +260,15 @@ extern "C" int pta_gemm_splitk_bf16(void* y, float* part, const void* x, const v
     if (rt == 0) rt = pick_rt(N);
     if (parts == 0) parts = pick_parts(N, K, rt);
     if (stage_blocks == 0) stage_blocks = 2;
-    PTA_REQUIRE(parts == 1 || part, "gemm_splitk_bf16: %d ranges of K need the workspace for partial sums", parts);
+    PTA_REQUIRE((parts == 1 && reduce) || part, "gemm_splitk_bf16: %d ranges of K need the workspace for partial sums", parts);
+    parts = effective_parts(K, parts);  // what the caller's workspace must hold
     hipStream_t s = (hipStream_t)stream;
     const int MT = (M + 15) / 16;
     const bf16_t *xb = (const bf16_t*)x, *wb = (const bf16_t*)W, *a1 = (const bf16_t*)add1, *a2 = (const bf16_t*)add2;
     if (depth == 0) depth = 2;  // measured: more stages in flight per wave do not pay, more workgroups do
 #define SK_CASE(RT_, U_, D_)                                                                                      \
     if (rt == RT_ && stage_blocks == U_ && depth == D_)                                                           \
-        return launch_rows<RT_, U_, D_>(MT, y, part, xb, wb, bias, a1, a2, M, N, K, act, out_f32, parts, s);
+        return launch_rows<RT_, U_, D_>(MT, y, part, xb, wb, bias, a1, a2, M, N, K, act, out_f32, parts, reduce, s);
     SK_CASE(1, 2, 2) SK_CASE(1, 2, 4) SK_CASE(2, 2, 2) SK_CASE(2, 2, 4)
 #undef SK_CASE
     return pta_fail("gemm_splitk_bf16: no kernel for rt=%d stage_blocks=%d depth=%d", rt, stage_blocks, depth);

@@ -1,0 +1,161 @@
+// The residual sum and the LayerNorm that reads it, in one pass over bfloat16 rows.
+//
+//   v    = A + B + add1 + add2          (terms that are absent are skipped; at least one is given)
+//   x    = round(v)                     -> out_x, if wanted
+//   out1 = LN(x) * w1 + b1              -> if wanted; out2 with (w2, b2) likewise
+//
+// A and B are matrix products that their kernels left as 32-bit partial sums over ranges of K,
+// [parts, rows, H]; each is summed in the order of its ranges, rounded to bfloat16, and its bias is
+// added and rounded again: what the epilogue of a product that ran whole would have stored.  B comes
+// first in the sum, then A, then the bfloat16 addends, as in the epilogue of the block's last product
+// (feed-forward plus mixer first, then the residual).  `rows` selects source rows (the final norm reads
+// only the rows whose logits are wanted).
+//
+// One workgroup of 512 threads per row; a thread holds up to two chunks of eight features in registers
+// (H <= 8192, H % 8 == 0), loaded and stored sixteen bytes at a time.  Norm weights are loaded before the
+// reductions so that their latency hides behind them.  Mean and biased variance in 32-bit, variance
+// from the centred values.
+#include "common.h"
+#include "pta_kernels.h"
+
+#define NS_THREADS 512
+#define NS_CHUNKS 2
+
+__device__ __forceinline__ void unpack8(const uint4& u, float (&f)[8]) {
+    const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        f[2 * p] = bf16_bits_to_f32((bf16_t)(w[p] & 0xffffu));
+        f[2 * p + 1] = bf16_bits_to_f32((bf16_t)(w[p] >> 16));
+    }
+}
+__device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
+    uint32_t w[4];
+#pragma unroll
+    for (int p = 0; p < 4; ++p) w[p] = (uint32_t)f32_to_bf16_bits(f[2 * p]) | ((uint32_t)f32_to_bf16_bits(f[2 * p + 1]) << 16);
+    return make_uint4(w[0], w[1], w[2], w[3]);
+}
+__device__ __forceinline__ void load8f(const float* p, float (&f)[8]) {
+    const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+    f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+}
+
+// round(sum of the parts in order), then the bias added and rounded
+__device__ __forceinline__ void product_value(const float* part, int P, long part_stride, const float* bias, long at,
+                                              int i, float (&out)[8]) {
+    load8f(part + at, out);
+    for (int p = 1; p < P; ++p) {
+        float t[8];
+        load8f(part + p * part_stride + at, t);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) out[e] += t[e];
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) out[e] = round_to_bf16(out[e]);
+    if (bias) {
+        float b[8];
+        load8f(bias + i, b);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) out[e] = round_to_bf16(out[e] + b[e]);
+    }
+}
+
+__global__ __launch_bounds__(NS_THREADS) void layernorm_sum_kernel(
+    bf16_t* __restrict__ out_x, bf16_t* __restrict__ out1, bf16_t* __restrict__ out2, const float* __restrict__ pa,
+    int Pa, const float* __restrict__ bias_a, const float* __restrict__ pb, int Pb, const float* __restrict__ bias_b,
+    const bf16_t* __restrict__ add1, const bf16_t* __restrict__ add2, const int* __restrict__ rows,
+    const float* __restrict__ w1, const float* __restrict__ b1, const float* __restrict__ w2,
+    const float* __restrict__ b2, int M_in, int H, float eps) {
+    __shared__ float red[16];
+    const int m = blockIdx.x;
+    const long src = rows ? (long)rows[m] : (long)m;
+    const long part_stride = (long)M_in * H;
+    float v[NS_CHUNKS][8];
+    float gw1[NS_CHUNKS][8], gb1[NS_CHUNKS][8], gw2[NS_CHUNKS][8], gb2[NS_CHUNKS][8];
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < NS_CHUNKS; ++j) {
+        const int i = (threadIdx.x + j * NS_THREADS) * 8;
+        if (i >= H) continue;
+        const long at = src * H + i;
+        if (out1) { load8f(w1 + i, gw1[j]); load8f(b1 + i, gb1[j]); }
+        if (out2) { load8f(w2 + i, gw2[j]); load8f(b2 + i, gb2[j]); }
+        bool any = false;
+        if (pb) { product_value(pb, Pb, part_stride, bias_b, at, i, v[j]); any = true; }
+        if (pa) {
+            float t[8];
+            product_value(pa, Pa, part_stride, bias_a, at, i, t);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[j][e] = any ? v[j][e] + t[e] : t[e];
+            any = true;
+        }
+        if (add1) {
+            float t[8];
+            unpack8(*reinterpret_cast<const uint4*>(add1 + at), t);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[j][e] = any ? v[j][e] + t[e] : t[e];
+            any = true;
+        }
+        if (add2) {
+            float t[8];
+            unpack8(*reinterpret_cast<const uint4*>(add2 + at), t);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[j][e] = any ? v[j][e] + t[e] : t[e];
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            v[j][e] = round_to_bf16(v[j][e]);
+            s += v[j][e];
+        }
+        if (out_x) *reinterpret_cast<uint4*>(out_x + (long)m * H + i) = pack8(v[j]);
+    }
+    if (!out1) return;
+    const float mean = block_sum(s, red) / (float)H;
+    float q = 0.f;
+#pragma unroll
+    for (int j = 0; j < NS_CHUNKS; ++j) {
+        const int i = (threadIdx.x + j * NS_THREADS) * 8;
+        if (i >= H) continue;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { const float d = v[j][e] - mean; q += d * d; }
+    }
+    const float var = block_sum(q, red) / (float)H;
+    const float rstd = 1.0f / sqrtf(var + eps);
+#pragma unroll
+    for (int j = 0; j < NS_CHUNKS; ++j) {
+        const int i = (threadIdx.x + j * NS_THREADS) * 8;
+        if (i >= H) continue;
+        float o[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = (v[j][e] - mean) * rstd * gw1[j][e] + gb1[j][e];
+        *reinterpret_cast<uint4*>(out1 + (long)m * H + i) = pack8(o);
+        if (out2) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = (v[j][e] - mean) * rstd * gw2[j][e] + gb2[j][e];
+            *reinterpret_cast<uint4*>(out2 + (long)m * H + i) = pack8(o);
+        }
+    }
+}
+
+extern "C" int pta_layernorm_sum_ok(int H) { return H > 0 && H % 8 == 0 && H <= NS_THREADS * NS_CHUNKS * 8; }
+
+extern "C" int pta_layernorm_sum(void* out_x, void* out1, void* out2, const float* pa, int Pa, const float* bias_a,
+                                 const float* pb, int Pb, const float* bias_b, const void* add1, const void* add2,
+                                 const int* rows, const float* w1, const float* b1, const float* w2, const float* b2,
+                                 int M_in, int M, int H, float eps, void* stream) {
+    PTA_REQUIRE(M > 0 && M_in > 0 && H > 0, "layernorm_sum: M=%d M_in=%d H=%d must be positive", M, M_in, H);
+    PTA_REQUIRE(pta_layernorm_sum_ok(H), "layernorm_sum: H=%d must be a multiple of 8 up to %d", H,
+                NS_THREADS * NS_CHUNKS * 8);
+    PTA_REQUIRE(pa || pb || add1 || add2, "layernorm_sum: nothing to sum");
+    PTA_REQUIRE((!pa || Pa > 0) && (!pb || Pb > 0), "layernorm_sum: a product needs at least one part");
+    PTA_REQUIRE(out_x || out1, "layernorm_sum: no output wanted");
+    PTA_REQUIRE(!out1 || (w1 && b1), "layernorm_sum: the norm needs weight and bias");
+    PTA_REQUIRE(!out2 || (out1 && w2 && b2), "layernorm_sum: a second output needs the first, and its own weight and bias");
+    PTA_REQUIRE(rows || M == M_in, "layernorm_sum: without row selection M (%d) must equal M_in (%d)", M, M_in);
+    const void* ptrs[] = {out_x, out1, out2, pa, pb, add1, add2, bias_a, bias_b, w1, b1, w2, b2};
+    for (const void* p : ptrs) PTA_REQUIRE(((uintptr_t)p % 16) == 0, "layernorm_sum: pointers must be 16-byte aligned");
+    hipLaunchKernelGGL(layernorm_sum_kernel, dim3(M), dim3(NS_THREADS), 0, (hipStream_t)stream, (bf16_t*)out_x,
+                       (bf16_t*)out1, (bf16_t*)out2, pa, Pa, bias_a, pb, Pb, bias_b, (const bf16_t*)add1,
+                       (const bf16_t*)add2, rows, w1, b1, w2, b2, M_in, H, eps);
+    return pta_check_launch("layernorm_sum");
+}

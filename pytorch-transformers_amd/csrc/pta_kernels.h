@@ -31,6 +31,15 @@ int pta_embed(void* out, const void* table, const int* ids, int M, int H, int dt
 int pta_layernorm(void* out1, void* out2, const void* x, const int* rows, const float* w1, const float* b1,
                   const float* w2, const float* b2, int M, int H, float eps, int dtype, void* stream);
 
+// bfloat16 rows: x = round(A + B + add1 + add2) with A, B products left as 32-bit partial sums [P, M_in, H]
+// (summed in order, rounded, bias added and rounded); out_x = x, out1 = LN(x) * w1 + b1, out2 likewise, each
+// if not null; rows (may be null) selects the M source rows out of M_in
+int pta_layernorm_sum(void* out_x, void* out1, void* out2, const float* pa, int Pa, const float* bias_a,
+                      const float* pb, int Pb, const float* bias_b, const void* add1, const void* add2,
+                      const int* rows, const float* w1, const float* b1, const float* w2, const float* b2, int M_in,
+                      int M, int H, float eps, void* stream);
+int pta_layernorm_sum_ok(int H);
+
 // in place: y = act(round(y + bias)) + add1 + add2; bias, add1, add2 may be null
 int pta_epilogue(void* y, const float* bias, const void* add1, const void* add2, int M, int N, int act, int dtype,
                  void* stream);
@@ -66,12 +75,15 @@ int pta_gemm_skinny_bf16(void* y, const void* x, const void* W, const float* bia
                          int M, int N, int K, int act, int out_f32, int variant, int waves, void* stream);
 
 // The same product for a batch of up to 64 rows that shares x through LDS and may split K over workgroups:
-// `part` is a 32-bit workspace [parts, M, N], needed when parts > 1.  rt (row tiles per wave), parts,
-// stage_blocks (64-element blocks of K per stage) and depth (stages in flight) are tuning knobs (0: chosen from N and K); pta_gemm_splitk_parts tells the choice of parts.
+// `part` is a 32-bit workspace [parts, M, N], needed when parts > 1 or reduce = 0.  rt (row tiles per wave),
+// parts, stage_blocks (64-element blocks of K per stage) and depth (stages in flight) are tuning knobs (0:
+// chosen from N and K alone); pta_gemm_splitk_parts tells the number of ranges that choice gives.
+// With reduce = 0 the product is left as the partial sums (y may be null; bias, act and additions are not
+// applied).  Ranges that would be empty are dropped: ceil(nkb / ceil(nkb / parts)) remain, nkb = ceil(K / 64).
 int pta_gemm_splitk_bf16(void* y, float* part, const void* x, const void* W, const float* bias, const void* add1,
                          const void* add2, int M, int N, int K, int act, int out_f32, int rt, int parts,
-                         int stage_blocks, int depth, void* stream);
-int pta_gemm_splitk_parts(int N, int K);
+                         int stage_blocks, int depth, int reduce, void* stream);
+int pta_gemm_splitk_parts(int N, int K, int parts, int rt);
 
 // processors in the reference's order, then argmax (do_sample 0) or a draw; `work` [R, V] receives the
 // processed scores; hist/hist_off (tokens seen, per row), eos/suppress, uniforms may be null

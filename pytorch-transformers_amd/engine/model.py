@@ -17,7 +17,7 @@ import torch
 
 from ..cache.paged import PagedCache
 from ..config.registry import AutoConfig, lookup
-from ..parts.base import StepContext
+from ..parts.base import ResidualSum, StepContext, as_tensor
 from ..weights.loader import load_weights
 from ..weights.random_init import random_tensors
 from .spec import ModelSpec
@@ -238,13 +238,18 @@ class CausalLM:
         x = self.spec.embedding.forward(token_ids)
         blocks = self.spec.blocks
         for call in self.spec.order:
-            x = blocks[call.block].forward(x, ctx, call)
+            block = blocks[call.block]
+            if isinstance(x, ResidualSum) and not getattr(block, "accepts_sum", False):
+                x = x.tensor()
+            x = block.forward(x, ctx, call)
         if logit_rows is None:
             return None
-        if self.spec.final_norm is not None:
-            h = self.spec.final_norm.forward(x, rows=logit_rows)
+        norm = self.spec.final_norm
+        if isinstance(x, ResidualSum) and norm is not None and hasattr(norm, "forward_sum"):
+            h = norm.forward_sum(x, rows=logit_rows, want_x=False)[1]
         else:
-            h = x.index_select(0, logit_rows.long())
+            x = as_tensor(x)
+            h = norm.forward(x, rows=logit_rows) if norm is not None else x.index_select(0, logit_rows.long())
         return self.spec.head.forward(h)
 
     # decode steps as HIP graphs ---------------------------------------------------------

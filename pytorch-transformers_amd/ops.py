@@ -344,13 +344,97 @@ def gemm_splitk_bf16(x: torch.Tensor, w: torch.Tensor, bias=None, act=None, add1
     for name, t in (("add1", add1), ("add2", add2)):
         if t is not None:
             _need(t, name, torch.bfloat16, (M, N))
-    if parts == 0:
-        parts = int(load_library().pta_gemm_splitk_parts(N, K))
+    parts = int(load_library().pta_gemm_splitk_parts(N, K, int(parts), int(rt)))
     part = torch.empty((parts, M, N), dtype=torch.float32, device=x.device) if parts > 1 else None
     out = torch.empty((M, N), dtype=torch.float32 if out_f32 else torch.bfloat16, device=x.device)
     _call("pta_gemm_splitk_bf16", _ptr(out), _ptr(part), _ptr(x), _ptr(w), _ptr(bias), _ptr(add1), _ptr(add2), M, N, K,
-          ACT_CODES[act], int(out_f32), int(rt), int(parts), int(stage_blocks), int(depth), _stream())
+          ACT_CODES[act], int(out_f32), int(rt), int(parts), int(stage_blocks), int(depth), 1, _stream())
     return out
+
+
+def gemm_splitk_partial(x: torch.Tensor, w: torch.Tensor, rt: int = 0, parts: int = 0) -> torch.Tensor:
+    """x @ w.T left as 32-bit partial sums over ranges of K, [ranges, M, N]: for a kernel that adds them
+    in order while it reads them (``layernorm_sum``)."""
+    _need(x, "x", torch.bfloat16)
+    _need(w, "w", torch.bfloat16)
+    M, K = x.shape
+    N = w.shape[0]
+    if w.dim() != 2 or w.shape[1] != K:
+        raise KernelError(f"x is [{M}, {K}] but w is {tuple(w.shape)}; w must be [N, {K}]")
+    parts = int(load_library().pta_gemm_splitk_parts(N, K, int(parts), int(rt)))
+    part = torch.empty((parts, M, N), dtype=torch.float32, device=x.device)
+    _call("pta_gemm_splitk_bf16", None, _ptr(part), _ptr(x), _ptr(w), None, None, None, M, N, K, 0, 0, int(rt),
+          int(parts), 0, 0, 0, _stream())
+    return part
+
+
+def gemm_partial_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether leaving x @ w.T as partial sums for the next norm pays: up to 64 rows, and either K long against
+    N (any batch: the kernel for few rows has too few row tiles there) or a batch past 16 rows."""
+    if not (_bf16_rows_ok(x, w) and 0 < x.shape[0] <= SKINNY_MAX_ROWS and w.shape[0] % 8 == 0):
+        return False
+    return w.shape[1] >= 2 * w.shape[0] or (x.shape[0] > 16 and w.shape[0] < 2 * w.shape[1])
+
+
+def layernorm_sum_ok(H: int) -> bool:
+    return bool(load_library().pta_layernorm_sum_ok(int(H)))
+
+
+def layernorm_sum(terms, H: int, *, w=None, b=None, eps: float = 0.0, w2=None, b2=None, rows=None,
+                  want_x: bool = True):
+    """The sum of ``terms`` rounded to bfloat16 and, with (w, b), its LayerNorm: ``(x, out1, out2)``.
+
+    A term is a bfloat16 tensor [M, H] or a pair (partial sums [P, M, H] in 32-bit, bias or None) of a
+    product left unreduced; at most two of each, products first.  A product is valued as its own epilogue
+    would have stored it; the terms are added in the order given."""
+    prods = [t for t in terms if isinstance(t, tuple)]
+    adds = [t for t in terms if not isinstance(t, tuple)]
+    if len(prods) > 2 or len(adds) > 2 or not terms:
+        raise KernelError(f"layernorm_sum takes one to four terms, at most two products and two tensors; got {len(terms)}")
+    if any(isinstance(t, tuple) for t in terms[len(prods):]):
+        raise KernelError("layernorm_sum: products must come before tensors in the list of terms")
+    M_in = None
+    for part, bias in prods:
+        _need(part, "partial sums", torch.float32)
+        if part.dim() != 3 or part.shape[2] != H:
+            raise KernelError(f"partial sums must be [parts, rows, {H}], got {tuple(part.shape)}")
+        if bias is not None:
+            _need(bias, "bias", torch.float32, (H,))
+        M_in = part.shape[1] if M_in is None else M_in
+        if part.shape[1] != M_in:
+            raise KernelError("terms differ in their number of rows")
+    for a in adds:
+        _need(a, "addend", torch.bfloat16)
+        M_in = a.shape[0] if M_in is None else M_in
+        if tuple(a.shape) != (M_in, H):
+            raise KernelError(f"addend must be [{M_in}, {H}], got {tuple(a.shape)}")
+    ref = prods[0][0] if prods else adds[0]
+    if rows is not None:
+        _need(rows, "rows", torch.int32)
+        M = rows.numel()
+    else:
+        M = M_in
+    dev = ref.device
+    norm = w is not None
+    if norm:
+        _need(w, "weight", torch.float32, (H,))
+        _need(b, "bias", torch.float32, (H,))
+    if w2 is not None:
+        _need(w2, "weight2", torch.float32, (H,))
+        _need(b2, "bias2", torch.float32, (H,))
+    out_x = torch.empty((M, H), dtype=torch.bfloat16, device=dev) if want_x else None
+    out1 = torch.empty((M, H), dtype=torch.bfloat16, device=dev) if norm else None
+    out2 = torch.empty((M, H), dtype=torch.bfloat16, device=dev) if norm and w2 is not None else None
+    if M == 0:
+        return out_x, out1, out2
+    pb, bb = prods[0] if prods else (None, None)  # the kernel adds B first, then A
+    pa, ba = prods[1] if len(prods) > 1 else (None, None)
+    a1 = adds[0] if adds else None
+    a2 = adds[1] if len(adds) > 1 else None
+    _call("pta_layernorm_sum", _ptr(out_x), _ptr(out1), _ptr(out2), _ptr(pa), 0 if pa is None else pa.shape[0], _ptr(ba),
+          _ptr(pb), 0 if pb is None else pb.shape[0], _ptr(bb), _ptr(a1), _ptr(a2), _ptr(rows), _ptr(w), _ptr(b),
+          _ptr(w2), _ptr(b2), M_in, M, H, ctypes.c_float(eps), _stream())
+    return out_x, out1, out2
 
 
 def _bf16_rows_ok(x: torch.Tensor, w: torch.Tensor) -> bool:

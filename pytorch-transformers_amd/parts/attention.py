@@ -41,7 +41,12 @@ class AttentionMixer(Part):
     def children(self) -> Sequence[Part]:
         return (self.qkv, self.out, self.positions)
 
-    def forward(self, x: torch.Tensor, ctx: StepContext, call, residual: Optional[torch.Tensor] = None):
+    can_defer = True
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, call, residual: Optional[torch.Tensor] = None,
+                defer: bool = False):
+        """Attention of the step's tokens over the cache, projected out, plus ``residual``.  With ``defer``
+        the output projection may come back as a ``PartialProduct``, without the residual."""
         k_pool, v_pool = ctx.cache.kv_layer(call.cache_group, call.cache_layer)
         table = ctx.block_tables[call.cache_group]
         fused = self.qkv(x, apply_bias=False)
@@ -50,6 +55,10 @@ class AttentionMixer(Part):
                                k_pool, v_pool, self.num_heads, self.kv_heads, self.head_dim, self.qkv_layout,
                                write_cache=call.write_cache)
         o = ops.attention(q, k_pool, v_pool, table, ctx, self.positions.score_bias(), self.scale)
+        if defer:
+            p = self.out.partial(o)
+            if p is not None:
+                return p
         return self.out(o, add1=residual)
 
 

@@ -23,6 +23,14 @@ positions      ``rotation() -> (inv_freq or None, scale)`` for queries and keys,
                ``score_bias() -> per-head slopes or None`` for attention scores
 block          ``forward(x, ctx, call) -> x``: the arrangement of the above
 =============  ==================================================================
+
+Optional, for parts that set ``can_defer = True``: a mixer or feed-forward called
+with ``defer=True`` may leave its last product unreduced and return a
+:class:`PartialProduct` (mixer, residual not added) or a :class:`ResidualSum`
+(feed-forward, its addends included); a norm with ``forward_sum(sum, rows=None,
+other=None, want_x=True) -> (x, normed, normed_other)`` forms such a sum while it
+normalises it; a block with ``accepts_sum = True`` takes a ``ResidualSum`` as its
+input.  Everything else receives plain tensors.
 """
 from __future__ import annotations
 
@@ -80,6 +88,49 @@ class Part:
         self.load(tensors)
         for c in self.children():
             c.load_all(tensors)
+
+
+@dataclasses.dataclass
+class PartialProduct:
+    """A matrix product that its kernel left as 32-bit partial sums over ranges of K, ``[ranges, tokens,
+    features]``, with the bias still to be added.  Whoever reads it adds the ranges in order, rounds, and adds
+    the bias: the value the product's own epilogue would have stored."""
+
+    parts: torch.Tensor
+    bias: Optional[torch.Tensor] = None
+
+    def term(self):
+        return (self.parts, self.bias)
+
+
+class ResidualSum:
+    """The residual stream as a sum that is not formed yet: products first, then tensors, added in that
+    order and rounded once.  A block may return it in place of a tensor; the norm that reads it next forms
+    the sum in the same pass (``forward_sum``), and ``tensor()`` forms it for anyone else."""
+
+    def __init__(self, terms: Sequence[Any]):
+        self.terms = [t for t in terms if t is not None]
+        first = self.terms[0]
+        self.features = (first.parts if isinstance(first, PartialProduct) else first).shape[-1]
+
+    def kernel_terms(self):
+        return [t.term() if isinstance(t, PartialProduct) else t for t in self.terms]
+
+    def tensor(self) -> torch.Tensor:
+        from .. import ops
+
+        if len(self.terms) == 1 and not isinstance(self.terms[0], PartialProduct):
+            return self.terms[0]
+        return ops.layernorm_sum(self.kernel_terms(), self.features)[0]
+
+
+def as_tensor(x):
+    """A tensor from what a part may hand on: a tensor, a ``PartialProduct`` or a ``ResidualSum``."""
+    if isinstance(x, PartialProduct):
+        return ResidualSum([x]).tensor()
+    if isinstance(x, ResidualSum):
+        return x.tensor()
+    return x
 
 
 @dataclasses.dataclass

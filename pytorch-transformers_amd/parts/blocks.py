@@ -8,7 +8,8 @@ parallel    ``x + (ffn(norm_ffn(x)) + mixer(norm_mixer(x)))``; with one norm bot
             feed-forward plus mixer first (:673-674), then the residual (:676).
 sequential  ``r = x + mixer(norm_in(x))``; ``r + ffn(norm_post(r))`` (:652-659, :676).
 
-The additions ride in the last matrix product's epilogue of each branch.  In the parallel block the
+The additions ride in the last matrix product's epilogue of each branch, or, in steps of few tokens,
+the products stay unreduced and the next norm forms the sum while it reads it (``ResidualSum``).  In the parallel block the
 feed-forward's first product does not depend on the mixer, so it may run beside it on a second stream.
 """
 from __future__ import annotations
@@ -17,10 +18,28 @@ from typing import Optional, Sequence
 
 import torch
 
-from .base import Part, StepContext, register_part
+from .base import Part, PartialProduct, ResidualSum, StepContext, register_part
+
+
+def _can_defer(part: Part) -> bool:
+    return bool(getattr(part, "can_defer", False))
+
+
+def _normed(x, norm: Part, other: Optional[Part] = None):
+    """``(x as a tensor, norm(x), other(x) or None)`` for a block input that may be a sum not formed yet."""
+    if isinstance(x, ResidualSum):
+        if hasattr(norm, "forward_sum"):
+            return norm.forward_sum(x, other=other)
+        x = x.tensor()
+    if other is None:
+        return x, norm.forward(x), None
+    a, m = norm.forward_pair(x, other)
+    return x, a, m
 
 
 class ParallelBlock(Part):
+    accepts_sum = True
+
     def __init__(self, mixer: Part, feed_forward: Part, norm_mixer: Part, norm_ffn: Optional[Part] = None):
         self.mixer = mixer
         self.feed_forward = feed_forward
@@ -30,13 +49,18 @@ class ParallelBlock(Part):
     def children(self) -> Sequence[Part]:
         return tuple(p for p in (self.norm_mixer, self.norm_ffn, self.mixer, self.feed_forward) if p is not None)
 
-    def forward(self, x: torch.Tensor, ctx: StepContext, call) -> torch.Tensor:
-        if self.norm_ffn is None:
-            a = m = self.norm_mixer.forward(x)
-        else:
-            a, m = self.norm_mixer.forward_pair(x, self.norm_ffn)
+    def forward(self, x, ctx: StepContext, call):
+        x, a, m = _normed(x, self.norm_mixer, self.norm_ffn)
+        if m is None:
+            m = a
         side = ctx.side_stream
         if side is None or not hasattr(self.feed_forward, "forward_up"):
+            # where the parts can, the last products stay unreduced and the next norm forms
+            # feed-forward + mixer + residual while it reads them
+            if _can_defer(self.feed_forward):
+                mixed = self.mixer.forward(a, ctx, call, defer=True) if _can_defer(self.mixer) else \
+                    self.mixer.forward(a, ctx, call)
+                return self.feed_forward.forward(m, ctx, add1=mixed, add2=x, defer=True)
             mixed = self.mixer.forward(a, ctx, call)
             return self.feed_forward.forward(m, ctx, add1=mixed, add2=x)
         # The feed-forward's first product needs only the norm, not the mixer: it runs on a second
@@ -52,6 +76,8 @@ class ParallelBlock(Part):
 
 
 class SequentialBlock(Part):
+    accepts_sum = True
+
     def __init__(self, mixer: Part, feed_forward: Part, norm_in: Part, norm_post: Part):
         self.mixer = mixer
         self.feed_forward = feed_forward
@@ -61,9 +87,18 @@ class SequentialBlock(Part):
     def children(self) -> Sequence[Part]:
         return (self.norm_in, self.norm_post, self.mixer, self.feed_forward)
 
-    def forward(self, x: torch.Tensor, ctx: StepContext, call) -> torch.Tensor:
-        r = self.mixer.forward(self.norm_in.forward(x), ctx, call, residual=x)
-        return self.feed_forward.forward(self.norm_post.forward(r), ctx, add1=r)
+    def forward(self, x, ctx: StepContext, call):
+        x, a, _ = _normed(x, self.norm_in)
+        if _can_defer(self.mixer):
+            r = self.mixer.forward(a, ctx, call, residual=x, defer=True)
+            if isinstance(r, PartialProduct):
+                r = ResidualSum([r, x])
+        else:
+            r = self.mixer.forward(a, ctx, call, residual=x)
+        r, m, _ = _normed(r, self.norm_post)
+        if _can_defer(self.feed_forward):
+            return self.feed_forward.forward(m, ctx, add1=r, defer=True)
+        return self.feed_forward.forward(m, ctx, add1=r)
 
 
 register_part("block", "parallel", ParallelBlock)

@@ -7,7 +7,7 @@ from typing import Sequence
 
 import torch
 
-from .base import Part, StepContext, register_part
+from .base import Part, ResidualSum, StepContext, as_tensor, register_part
 from .linear import Linear
 
 
@@ -24,8 +24,16 @@ class DenseFeedForward(Part):
     def children(self) -> Sequence[Part]:
         return (self.up, self.down)
 
-    def forward(self, x: torch.Tensor, ctx: StepContext, add1=None, add2=None) -> torch.Tensor:
-        return self.down(self.up(x, act=self.activation), add1=add1, add2=add2)
+    can_defer = True
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, add1=None, add2=None, defer: bool = False):
+        """``down(act(up(x))) + add1 + add2``; with ``defer`` the sum may come back unformed."""
+        h = self.up(x, act=self.activation)
+        if defer:
+            p = self.down.partial(h)
+            if p is not None:
+                return ResidualSum([p, add1, add2])
+        return self.down(h, add1=as_tensor(add1), add2=as_tensor(add2))
 
     # The two halves on their own: a block whose feed-forward does not read the mixer's output can run
     # the first half beside the mixer.
@@ -33,7 +41,7 @@ class DenseFeedForward(Part):
         return self.up(x, act=self.activation)
 
     def forward_down(self, h: torch.Tensor, ctx: StepContext, add1=None, add2=None) -> torch.Tensor:
-        return self.down(h, add1=add1, add2=add2)
+        return self.down(h, add1=as_tensor(add1), add2=as_tensor(add2))
 
 
 register_part("feed_forward", "dense", DenseFeedForward)

@@ -18,7 +18,7 @@ import torch
 
 from .. import ops
 from ..engine.spec import INIT_NORMAL, INIT_ZERO_NOISE, MATRIX, VECTOR, TensorSpec
-from .base import Part
+from .base import PartialProduct, Part
 
 
 class Linear(Part):
@@ -54,6 +54,12 @@ class Linear(Part):
         if bias is not None or act is not None or add1 is not None or add2 is not None:
             ops.epilogue_(y, bias, act, add1, add2)
         return y
+
+    def partial(self, x: torch.Tensor) -> Optional[PartialProduct]:
+        """The product left as partial sums for the next norm to add, where that pays; else None."""
+        if x.dtype == torch.bfloat16 and ops.gemm_partial_ok(x, self.weight) and ops.layernorm_sum_ok(self.out_features):
+            return PartialProduct(ops.gemm_splitk_partial(x, self.weight), self.bias)
+        return None
 
 
 class Embedding(Part):

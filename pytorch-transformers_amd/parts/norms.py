@@ -8,7 +8,7 @@ import torch
 
 from .. import ops
 from ..engine.spec import INIT_ONE_NOISE, INIT_ZERO_NOISE, VECTOR, TensorSpec
-from .base import Part, register_part
+from .base import Part, ResidualSum, register_part
 
 
 class LayerNorm(Part):
@@ -35,6 +35,22 @@ class LayerNorm(Part):
         if isinstance(other, LayerNorm) and other.eps == self.eps:
             return ops.layernorm(x, self.weight, self.bias, self.eps, w2=other.weight, b2=other.bias)
         return self.forward(x), other.forward(x)
+
+
+    def forward_sum(self, total: ResidualSum, rows: Optional[torch.Tensor] = None, other: Optional["Part"] = None,
+                    want_x: bool = True):
+        """``(x, self(x), other(x))`` for the unformed sum ``total``: x is formed, rounded and normalised in
+        one pass.  Falls back to forming the sum first where the fused kernel does not take the width."""
+        pair = isinstance(other, LayerNorm) and other.eps == self.eps
+        if total.features == self.hidden_size and ops.layernorm_sum_ok(self.hidden_size) and (other is None or pair):
+            return ops.layernorm_sum(total.kernel_terms(), self.hidden_size, w=self.weight, b=self.bias, eps=self.eps,
+                                     w2=other.weight if pair else None, b2=other.bias if pair else None, rows=rows,
+                                     want_x=want_x)
+        x = total.tensor()
+        if other is None:
+            return x, self.forward(x, rows=rows), None
+        a, m = self.forward_pair(x, other)
+        return x, a, m
 
 
 register_part("norm", "layernorm", LayerNorm)

@@ -121,6 +121,70 @@ def test_gemm_splitk_bf16(M, N, K, parts, rt, sb, depth):
     assert torch.equal(alone, got32[r:r + 1])
 
 
+@pytest.mark.parametrize("H", [64, 200, 4544, 8192])
+@pytest.mark.parametrize("case", ["plain", "two products", "product and tensors", "rows", "sum only"])
+def test_layernorm_sum(H, case):
+    """The fused residual sum and LayerNorm against the same steps one by one in 32-bit."""
+    ops = _ops()
+    M = 5
+    bf = lambda t: t.bfloat16()
+    pa, pb = _rand(3, M, H, seed=1), _rand(2, M, H, seed=2)
+    ba = _rand(H, seed=3)
+    x1, x2 = bf(_rand(M, H, seed=4)), bf(_rand(M, H, seed=5))
+    w, b, w2, b2 = _rand(H, seed=6) + 1.0, _rand(H, seed=7), _rand(H, seed=8) + 1.0, _rand(H, seed=9)
+    value = lambda p, bias: (bf(bf(p.sum(0)).float() + bias).float() if bias is not None else bf(p.sum(0)).float())
+    rows = None
+    if case == "plain":
+        terms, want = [x1], x1.float()
+    elif case == "two products":
+        terms, want = [(pb, None), (pa, ba), x1], value(pb, None) + value(pa, ba) + x1.float()
+    elif case == "product and tensors":
+        terms, want = [(pa, ba), x1, x2], value(pa, ba) + x1.float() + x2.float()
+    elif case == "rows":
+        rows = torch.tensor([4, 0, 4], dtype=torch.int32).cuda()
+        terms, want = [(pb, None), x2], (value(pb, None) + x2.float())[rows.long()]
+    else:
+        terms, want = [(pb, None), x1, x2], value(pb, None) + x1.float() + x2.float()
+    want = bf(want)
+    if case == "sum only":
+        x, o1, o2 = ops.layernorm_sum(terms, H)
+        assert o1 is None and o2 is None
+        assert torch.equal(x, want)
+        return
+    x, o1, o2 = ops.layernorm_sum(terms, H, w=w, b=b, eps=1e-5, w2=w2, b2=b2, rows=rows)
+    assert torch.equal(x, want), "the sum is formed in the stated order and rounded once"
+    for o, (ww, bb) in ((o1, (w, b)), (o2, (w2, b2))):
+        ref = F.layer_norm(want.float(), (H,), ww, bb, 1e-5)
+        torch.testing.assert_close(o.float(), ref, rtol=1e-2, atol=1e-2)
+    x_none, o1b, _ = ops.layernorm_sum(terms, H, w=w, b=b, eps=1e-5, rows=rows, want_x=False)
+    assert x_none is None and torch.equal(o1b, o1)
+
+
+def test_layernorm_sum_refuses_what_it_cannot_do():
+    ops = _ops()
+    assert not ops.layernorm_sum_ok(100) and not ops.layernorm_sum_ok(8200) and ops.layernorm_sum_ok(8192)
+    x = _rand(2, 100, dtype=torch.bfloat16)
+    with pytest.raises(ops.KernelError, match="multiple of 8"):
+        ops.layernorm_sum([x], 100)
+    x = _rand(2, 64, dtype=torch.bfloat16)
+    with pytest.raises(ops.KernelError, match="products must come before"):
+        ops.layernorm_sum([x, (_rand(1, 2, 64), None)], 64)
+
+
+def test_partial_product_equals_the_reduced_one():
+    """Partial sums added by the norm kernel give the bits the product's own reduction stores."""
+    ops = _ops()
+    M, N, K = 9, 328, 2056
+    x, w = _rand(M, K, dtype=torch.bfloat16), _rand(N, K, seed=1, dtype=torch.bfloat16, scale=0.05)
+    bias, a1 = _rand(N, seed=2), _rand(M, N, seed=3, dtype=torch.bfloat16)
+    whole = ops.gemm_splitk_bf16(x, w, bias, None, a1)
+    part = ops.gemm_splitk_partial(x, w)
+    assert part.shape[0] > 1 and part.shape[1:] == (M, N)
+    assert ops.gemm_partial_ok(x, w)  # K is long against N
+    formed = ops.layernorm_sum([(part, bias), a1], N)[0]
+    assert torch.equal(formed, whole)
+
+
 def test_gemm_skinny_refuses_what_it_cannot_do():
     ops = _ops()
     x, w = _rand(65, 64, dtype=torch.bfloat16), _rand(32, 64, dtype=torch.bfloat16)

@@ -112,6 +112,7 @@ def test_attention_mixer_and_blocks(dtype, rel, layout, nh, nkv, d, alibi, bias)
     """The mixer alone (whole prompt, then a chunk, then single tokens), and both block arrangements around it."""
     from pytorch_transformers_amd.cache import PagedCache
     from pytorch_transformers_amd.engine.spec import CACHE_FULL, CacheGroupSpec, LayerCall
+    from pytorch_transformers_amd.parts.base import as_tensor
     from pytorch_transformers_amd.parts import (AlibiPositions, AttentionMixer, DenseFeedForward, LayerNorm, ParallelBlock,
                                                 RotaryPositions, SequentialBlock)
 
@@ -159,7 +160,7 @@ def test_attention_mixer_and_blocks(dtype, rel, layout, nh, nkv, d, alibi, bias)
             continue  # the fused row order belongs to the architecture flag in the plain code
         cc = P.cfg_defaults(dict(c, **flags))
         want = P.decoder_layer(x.double(), ref, 0, cc, positions)
-        _close(run(lambda xs, ctx: block.forward(xs, ctx, call), cuts), want, rel, f"{type(block).__name__} {flags}")
+        _close(run(lambda xs, ctx: as_tensor(block.forward(xs, ctx, call)), cuts), want, rel, f"{type(block).__name__} {flags}")
 
 
 # --- a toy architecture, defined in the test -------------------------------------------------------------
