@@ -83,14 +83,34 @@ __device__ __forceinline__ void compute_stage(const Stage<MT, RT, U>& st, f32x4_
             }
 }
 
+// One product of a launch: a launch may carry two that share M and K (a block's two input projections),
+// so that the second one's workgroups fill the chip while the first one's drain.
+struct SkinnyProblem {
+    void* y;
+    const bf16_t* x;
+    const bf16_t* W;
+    const float* bias;
+    const bf16_t* add1;
+    const bf16_t* add2;
+    int N;
+    int act;
+    int blocks;  // workgroups of this product
+};
+
 template <int MT, int RT, int U, typename OutT>
-__global__ __launch_bounds__(512) void gemm_skinny_kernel(
-    OutT* __restrict__ y, const bf16_t* __restrict__ x, const bf16_t* __restrict__ W, const float* __restrict__ bias,
-    const bf16_t* __restrict__ add1, const bf16_t* __restrict__ add2, int M, int N, int K, int act) {
+__global__ __launch_bounds__(512) void gemm_skinny_kernel(SkinnyProblem pa, SkinnyProblem pb, int M, int K) {
     extern __shared__ f32x4_t part[];  // [S][RT][MT][64]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, S = blockDim.x >> 6;
     const int r = lane & 15, g = lane >> 4;
-    const int n0 = blockIdx.x * (16 * RT);
+    const bool second = (int)blockIdx.x >= pa.blocks;
+    OutT* __restrict__ y = (OutT*)(second ? pb.y : pa.y);
+    const bf16_t* __restrict__ x = second ? pb.x : pa.x;
+    const bf16_t* __restrict__ W = second ? pb.W : pa.W;
+    const float* __restrict__ bias = second ? pb.bias : pa.bias;
+    const bf16_t* __restrict__ add1 = second ? pb.add1 : pa.add1;
+    const bf16_t* __restrict__ add2 = second ? pb.add2 : pa.add2;
+    const int N = second ? pb.N : pa.N, act = second ? pb.act : pa.act;
+    const int n0 = ((int)blockIdx.x - (second ? pa.blocks : 0)) * (16 * RT);
     const bf16_t* wrow[RT];
 #pragma unroll
     for (int t = 0; t < RT; ++t) wrow[t] = W + (long)min(n0 + t * 16 + r, N - 1) * K;
@@ -162,56 +182,72 @@ static int pick_split(int N) {
 }
 
 template <int MT, int RT, int U, typename OutT>
-static void launch_cfg(OutT* y, const bf16_t* x, const bf16_t* W, const float* bias, const bf16_t* add1,
-                       const bf16_t* add2, int M, int N, int K, int act, int S, hipStream_t s) {
+static void launch_cfg(SkinnyProblem a, SkinnyProblem b, int M, int K, int S, hipStream_t s) {
     const int rows = 16 * RT;
-    if (S <= 0) S = pick_split(N);
-    const dim3 grid((N + rows - 1) / rows), block(S * 64);
+    if (S <= 0) S = pick_split(a.N + b.N);
+    a.blocks = (a.N + rows - 1) / rows;
+    b.blocks = (b.N + rows - 1) / rows;
+    const dim3 grid(a.blocks + b.blocks), block(S * 64);
     const size_t lds = (size_t)S * RT * MT * 64 * sizeof(f32x4_t);
-    hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, U, OutT>), grid, block, lds, s, y, x, W, bias, add1, add2, M, N, K,
-                       act);
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, U, OutT>), grid, block, lds, s, a, b, M, K);
 }
 
 template <typename OutT>
-static int launch_skinny(OutT* y, const bf16_t* x, const bf16_t* W, const float* bias, const bf16_t* add1,
-                         const bf16_t* add2, int M, int N, int K, int act, int variant, int S, hipStream_t s) {
+static int launch_skinny(SkinnyProblem a, SkinnyProblem b, int M, int K, int variant, int S, hipStream_t s) {
     // variant: row tiles per wave and steps per stage; 0: chosen here
     if (M <= 16) {
         if (variant == 0) variant = 2;
-        if (variant == 1) launch_cfg<1, 1, 4, OutT>(y, x, W, bias, add1, add2, M, N, K, act, S, s);
-        else if (variant == 2) launch_cfg<1, 2, 2, OutT>(y, x, W, bias, add1, add2, M, N, K, act, S, s);
-        else if (variant == 3) launch_cfg<1, 4, 1, OutT>(y, x, W, bias, add1, add2, M, N, K, act, S, s);
-        else if (variant == 4) launch_cfg<1, 4, 2, OutT>(y, x, W, bias, add1, add2, M, N, K, act, S, s);
-        else launch_cfg<1, 2, 4, OutT>(y, x, W, bias, add1, add2, M, N, K, act, S, s);
+        if (variant == 1) launch_cfg<1, 1, 4, OutT>(a, b, M, K, S, s);
+        else if (variant == 2) launch_cfg<1, 2, 2, OutT>(a, b, M, K, S, s);
+        else if (variant == 3) launch_cfg<1, 4, 1, OutT>(a, b, M, K, S, s);
+        else if (variant == 4) launch_cfg<1, 4, 2, OutT>(a, b, M, K, S, s);
+        else launch_cfg<1, 2, 4, OutT>(a, b, M, K, S, s);
     } else if (M <= 32) {
-        if (variant == 3 || variant == 4) launch_cfg<2, 4, 1, OutT>(y, x, W, bias, add1, add2, M, N, K, act, S, s);
-        else launch_cfg<2, 2, 1, OutT>(y, x, W, bias, add1, add2, M, N, K, act, S, s);
+        if (variant == 3 || variant == 4) launch_cfg<2, 4, 1, OutT>(a, b, M, K, S, s);
+        else launch_cfg<2, 2, 1, OutT>(a, b, M, K, S, s);
     } else if (M <= 48) {
-        launch_cfg<3, 2, 1, OutT>(y, x, W, bias, add1, add2, M, N, K, act, S, s);
+        launch_cfg<3, 2, 1, OutT>(a, b, M, K, S, s);
     } else {
-        if (variant == 3 || variant == 4) launch_cfg<4, 4, 1, OutT>(y, x, W, bias, add1, add2, M, N, K, act, S, s);
-        else launch_cfg<4, 2, 1, OutT>(y, x, W, bias, add1, add2, M, N, K, act, S, s);
+        if (variant == 3 || variant == 4) launch_cfg<4, 4, 1, OutT>(a, b, M, K, S, s);
+        else launch_cfg<4, 2, 1, OutT>(a, b, M, K, S, s);
     }
     return pta_check_launch("gemm_skinny_bf16");
+}
+
+static int check_skinny(const char* what, const void* y, const void* x, const void* W, int M, int N, int K, int act) {
+    PTA_REQUIRE(M > 0 && N > 0 && K > 0, "%s: sizes must be positive (M=%d N=%d K=%d)", what, M, N, K);
+    PTA_REQUIRE(M <= 64, "%s: at most 64 rows, got %d (use the library product)", what, M);
+    PTA_REQUIRE(K % 8 == 0, "%s: K=%d must be a multiple of 8 (16-byte loads)", what, K);
+    PTA_REQUIRE(y && x && W, "%s: null pointer", what);
+    PTA_REQUIRE((long)M * K * 2 < (1L << 31), "%s: x is too large for 32-bit buffer offsets", what);
+    PTA_REQUIRE(((uintptr_t)x % 16) == 0 && ((uintptr_t)W % 16) == 0, "%s: x and W must be 16-byte aligned", what);
+    PTA_REQUIRE(act == PTA_ACT_NONE || act == PTA_ACT_GELU, "%s: unknown activation %d", what, act);
+    return 0;
 }
 
 extern "C" int pta_gemm_skinny_bf16(void* y, const void* x, const void* W, const float* bias, const void* add1,
                                     const void* add2, int M, int N, int K, int act, int out_f32, int variant,
                                     int waves, void* stream) {
-    PTA_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_skinny_bf16: sizes must be positive (M=%d N=%d K=%d)", M, N, K);
-    PTA_REQUIRE(M <= 64, "gemm_skinny_bf16: at most 64 rows, got %d (use the library product)", M);
-    PTA_REQUIRE(K % 8 == 0, "gemm_skinny_bf16: K=%d must be a multiple of 8 (16-byte loads)", K);
-    PTA_REQUIRE(y && x && W, "gemm_skinny_bf16: null pointer");
-    PTA_REQUIRE((long)M * K * 2 < (1L << 31), "gemm_skinny_bf16: x is too large for 32-bit buffer offsets");
-    PTA_REQUIRE(((uintptr_t)x % 16) == 0 && ((uintptr_t)W % 16) == 0, "gemm_skinny_bf16: x and W must be 16-byte aligned");
-    PTA_REQUIRE(act == PTA_ACT_NONE || act == PTA_ACT_GELU, "gemm_skinny_bf16: unknown activation %d", act);
+    if (check_skinny("gemm_skinny_bf16", y, x, W, M, N, K, act)) return 1;
     PTA_REQUIRE(variant >= 0 && variant <= 5, "gemm_skinny_bf16: unknown variant %d", variant);
     PTA_REQUIRE(waves == 0 || (waves >= 1 && waves <= 8 && (waves & (waves - 1)) == 0),
                 "gemm_skinny_bf16: waves per workgroup must be 0 (choose) or a power of two up to 8, got %d", waves);
     hipStream_t s = (hipStream_t)stream;
-    if (out_f32)
-        return launch_skinny<float>((float*)y, (const bf16_t*)x, (const bf16_t*)W, bias, (const bf16_t*)add1,
-                                    (const bf16_t*)add2, M, N, K, act, variant, waves, s);
-    return launch_skinny<bf16_t>((bf16_t*)y, (const bf16_t*)x, (const bf16_t*)W, bias, (const bf16_t*)add1,
-                                 (const bf16_t*)add2, M, N, K, act, variant, waves, s);
+    const SkinnyProblem a{y, (const bf16_t*)x, (const bf16_t*)W, bias, (const bf16_t*)add1, (const bf16_t*)add2, N, act, 0};
+    const SkinnyProblem none{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0};
+    if (out_f32) return launch_skinny<float>(a, none, M, K, variant, waves, s);
+    return launch_skinny<bf16_t>(a, none, M, K, variant, waves, s);
+}
+
+// Two products of one launch: y1 = act1(x1 . W1^T + bias1), y2 = act2(x2 . W2^T + bias2), both [M, *] in
+// bfloat16 with one K.  The waves per workgroup follow N1 + N2, so a product's bits differ from those of
+// its own launch, but not with M or with what else is in the batch.
+extern "C" int pta_gemm_skinny_pair_bf16(void* y1, const void* x1, const void* W1, const float* bias1, int N1, int act1,
+                                         void* y2, const void* x2, const void* W2, const float* bias2, int N2, int act2,
+                                         int M, int K, void* stream) {
+    if (check_skinny("gemm_skinny_pair_bf16", y1, x1, W1, M, N1, K, act1)) return 1;
+    if (check_skinny("gemm_skinny_pair_bf16", y2, x2, W2, M, N2, K, act2)) return 1;
+    const SkinnyProblem a{y1, (const bf16_t*)x1, (const bf16_t*)W1, bias1, nullptr, nullptr, N1, act1, 0};
+    const SkinnyProblem b{y2, (const bf16_t*)x2, (const bf16_t*)W2, bias2, nullptr, nullptr, N2, act2, 0};
+    return launch_skinny<bf16_t>(a, b, M, K, 0, 0, (hipStream_t)stream);
 }

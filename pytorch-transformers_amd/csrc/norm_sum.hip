@@ -11,15 +11,15 @@
 // (feed-forward plus mixer first, then the residual).  `rows` selects source rows (the final norm reads
 // only the rows whose logits are wanted).
 //
-// One workgroup of 512 threads per row; a thread holds up to two chunks of eight features in registers
+// One workgroup of 1024 threads per row; a thread holds a chunk of eight features in registers
 // (H <= 8192, H % 8 == 0), loaded and stored sixteen bytes at a time.  Norm weights are loaded before the
 // reductions so that their latency hides behind them.  Mean and biased variance in 32-bit, variance
 // from the centred values.
 #include "common.h"
 #include "pta_kernels.h"
 
-#define NS_THREADS 512
-#define NS_CHUNKS 2
+#define NS_THREADS 1024
+#define NS_CHUNKS 1
 
 __device__ __forceinline__ void unpack8(const uint4& u, float (&f)[8]) {
     const uint32_t w[4] = {u.x, u.y, u.z, u.w};
@@ -40,23 +40,28 @@ __device__ __forceinline__ void load8f(const float* p, float (&f)[8]) {
     f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
 }
 
-// round(sum of the parts in order), then the bias added and rounded
+// round(sum of the parts in order), then the bias added and rounded.  The parts are loaded four at a
+// time before they are added, so that their latencies overlap.
 __device__ __forceinline__ void product_value(const float* part, int P, long part_stride, const float* bias, long at,
                                               int i, float (&out)[8]) {
-    load8f(part + at, out);
-    for (int p = 1; p < P; ++p) {
-        float t[8];
-        load8f(part + p * part_stride + at, t);
+    float bv[8];
+    if (bias) load8f(bias + i, bv);
+    for (int p0 = 0; p0 < P; p0 += 4) {
+        float t[4][8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) out[e] += t[e];
+        for (int u = 0; u < 4; ++u) load8f(part + (long)min(p0 + u, P - 1) * part_stride + at, t[u]);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (p0 + u >= P) continue;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) out[e] = (p0 + u == 0) ? t[u][e] : out[e] + t[u][e];
+        }
     }
 #pragma unroll
     for (int e = 0; e < 8; ++e) out[e] = round_to_bf16(out[e]);
     if (bias) {
-        float b[8];
-        load8f(bias + i, b);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) out[e] = round_to_bf16(out[e] + b[e]);
+        for (int e = 0; e < 8; ++e) out[e] = round_to_bf16(out[e] + bv[e]);
     }
 }
 

@@ -74,6 +74,11 @@ int pta_gemm_f32(float* C, const float* A, const float* W, const float* bias, co
 int pta_gemm_skinny_bf16(void* y, const void* x, const void* W, const float* bias, const void* add1, const void* add2,
                          int M, int N, int K, int act, int out_f32, int variant, int waves, void* stream);
 
+// two such products of one launch, both [M, *] in bfloat16 with one K (a block's two input projections)
+int pta_gemm_skinny_pair_bf16(void* y1, const void* x1, const void* W1, const float* bias1, int N1, int act1, void* y2,
+                              const void* x2, const void* W2, const float* bias2, int N2, int act2, int M, int K,
+                              void* stream);
+
 // The same product for a batch of up to 64 rows that shares x through LDS and may split K over workgroups:
 // `part` is a 32-bit workspace [parts, M, N], needed when parts > 1 or reduce = 0.  rt (row tiles per wave),
 // parts, stage_blocks (64-element blocks of K per stage) and depth (stages in flight) are tuning knobs (0:

@@ -328,6 +328,27 @@ def sample(logits: torch.Tensor, *, do_sample: bool, temperature: float = 1.0, t
 SKINNY_MAX_ROWS = 64
 
 
+def gemm_skinny_pair_bf16(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tensor, w2: torch.Tensor, bias1=None, act1=None,
+                          bias2=None, act2=None):
+    """(act1(x1 @ w1.T + bias1), act2(x2 @ w2.T + bias2)) in one launch: few rows, one K, bfloat16."""
+    for name, t in (("x1", x1), ("w1", w1), ("x2", x2), ("w2", w2)):
+        _need(t, name, torch.bfloat16)
+    M, K = x1.shape
+    if tuple(x2.shape) != (M, K) or w1.dim() != 2 or w2.dim() != 2 or w1.shape[1] != K or w2.shape[1] != K:
+        raise KernelError(f"a pair shares M and K: x1 {tuple(x1.shape)}, x2 {tuple(x2.shape)}, w1 {tuple(w1.shape)}, "
+                          f"w2 {tuple(w2.shape)}")
+    N1, N2 = w1.shape[0], w2.shape[0]
+    if bias1 is not None:
+        _need(bias1, "bias1", torch.float32, (N1,))
+    if bias2 is not None:
+        _need(bias2, "bias2", torch.float32, (N2,))
+    y1 = torch.empty((M, N1), dtype=torch.bfloat16, device=x1.device)
+    y2 = torch.empty((M, N2), dtype=torch.bfloat16, device=x1.device)
+    _call("pta_gemm_skinny_pair_bf16", _ptr(y1), _ptr(x1), _ptr(w1), _ptr(bias1), N1, ACT_CODES[act1], _ptr(y2), _ptr(x2),
+          _ptr(w2), _ptr(bias2), N2, ACT_CODES[act2], M, K, _stream())
+    return y1, y2
+
+
 def gemm_splitk_bf16(x: torch.Tensor, w: torch.Tensor, bias=None, act=None, add1=None, add2=None,
                      out_f32: bool = False, rt: int = 0, parts: int = 0, stage_blocks: int = 0,
                      depth: int = 0) -> torch.Tensor:

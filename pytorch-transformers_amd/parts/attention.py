@@ -43,13 +43,18 @@ class AttentionMixer(Part):
 
     can_defer = True
 
+    def input_projection(self):
+        """The first product of ``forward`` and how it is called: a block may run it together with another
+        part's and hand the result back as ``projected``."""
+        return self.qkv, {"apply_bias": False}
+
     def forward(self, x: torch.Tensor, ctx: StepContext, call, residual: Optional[torch.Tensor] = None,
-                defer: bool = False):
+                defer: bool = False, projected: Optional[torch.Tensor] = None):
         """Attention of the step's tokens over the cache, projected out, plus ``residual``.  With ``defer``
         the output projection may come back as a ``PartialProduct``, without the residual."""
         k_pool, v_pool = ctx.cache.kv_layer(call.cache_group, call.cache_layer)
         table = ctx.block_tables[call.cache_group]
-        fused = self.qkv(x, apply_bias=False)
+        fused = projected if projected is not None else self.qkv(x, apply_bias=False)
         inv_freq, cs_scale = self.positions.rotation()
         q = ops.qkv_rope_cache(fused, self.qkv.bias, inv_freq, cs_scale, ctx.token_pos, ctx.token_seq, table,
                                k_pool, v_pool, self.num_heads, self.kv_heads, self.head_dim, self.qkv_layout,

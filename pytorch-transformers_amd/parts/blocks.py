@@ -19,6 +19,7 @@ from typing import Optional, Sequence
 import torch
 
 from .base import Part, PartialProduct, ResidualSum, StepContext, register_part
+from .linear import Linear
 
 
 def _can_defer(part: Part) -> bool:
@@ -57,12 +58,20 @@ class ParallelBlock(Part):
         if side is None or not hasattr(self.feed_forward, "forward_up"):
             # where the parts can, the last products stay unreduced and the next norm forms
             # feed-forward + mixer + residual while it reads them
+            kw_mixer, kw_ffn = {}, {}
+            # both branches start with a product of the norm's output: one launch for the two in small steps
+            if hasattr(self.mixer, "input_projection") and hasattr(self.feed_forward, "input_projection"):
+                (lin_a, kw_a), (lin_m, kw_m) = self.mixer.input_projection(), self.feed_forward.input_projection()
+                both = Linear.pair(lin_a, a, kw_a, lin_m, m, kw_m)
+                if both is not None:
+                    kw_mixer["projected"], kw_ffn["projected"] = both
             if _can_defer(self.feed_forward):
-                mixed = self.mixer.forward(a, ctx, call, defer=True) if _can_defer(self.mixer) else \
-                    self.mixer.forward(a, ctx, call)
-                return self.feed_forward.forward(m, ctx, add1=mixed, add2=x, defer=True)
-            mixed = self.mixer.forward(a, ctx, call)
-            return self.feed_forward.forward(m, ctx, add1=mixed, add2=x)
+                if _can_defer(self.mixer):
+                    kw_mixer["defer"] = True
+                mixed = self.mixer.forward(a, ctx, call, **kw_mixer)
+                return self.feed_forward.forward(m, ctx, add1=mixed, add2=x, defer=True, **kw_ffn)
+            mixed = self.mixer.forward(a, ctx, call, **kw_mixer)
+            return self.feed_forward.forward(m, ctx, add1=mixed, add2=x, **kw_ffn)
         # The feed-forward's first product needs only the norm, not the mixer: it runs on a second
         # stream beside projection, rotation, attention and output projection, and the two meet at the
         # feed-forward's second product, whose epilogue sums the branches and the residual.

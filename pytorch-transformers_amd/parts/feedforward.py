@@ -26,9 +26,13 @@ class DenseFeedForward(Part):
 
     can_defer = True
 
-    def forward(self, x: torch.Tensor, ctx: StepContext, add1=None, add2=None, defer: bool = False):
+    def input_projection(self):
+        """The first product of ``forward`` and how it is called (see ``AttentionMixer.input_projection``)."""
+        return self.up, {"act": self.activation}
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, add1=None, add2=None, defer: bool = False, projected=None):
         """``down(act(up(x))) + add1 + add2``; with ``defer`` the sum may come back unformed."""
-        h = self.up(x, act=self.activation)
+        h = projected if projected is not None else self.up(x, act=self.activation)
         if defer:
             p = self.down.partial(h)
             if p is not None:

@@ -55,6 +55,19 @@ class Linear(Part):
             ops.epilogue_(y, bias, act, add1, add2)
         return y
 
+    @staticmethod
+    def pair(first: "Linear", x1: torch.Tensor, kw1: dict, second: "Linear", x2: torch.Tensor, kw2: dict):
+        """``(first(x1, **kw1), second(x2, **kw2))`` in one launch where the kernel for few rows takes both
+        (same rows, same K, no additions); else None."""
+        if not (x1.dtype == torch.bfloat16 and x1.shape == x2.shape and ops.gemm_skinny_ok(x1, first.weight)
+                and ops.gemm_skinny_ok(x2, second.weight)):
+            return None
+        if any(k not in ("act", "apply_bias") for k in list(kw1) + list(kw2)):
+            return None
+        b1 = first.bias if kw1.get("apply_bias", True) else None
+        b2 = second.bias if kw2.get("apply_bias", True) else None
+        return ops.gemm_skinny_pair_bf16(x1, first.weight, x2, second.weight, b1, kw1.get("act"), b2, kw2.get("act"))
+
     def partial(self, x: torch.Tensor) -> Optional[PartialProduct]:
         """The product left as partial sums for the next norm to add, where that pays; else None."""
         if x.dtype == torch.bfloat16 and ops.gemm_partial_ok(x, self.weight) and ops.layernorm_sum_ok(self.out_features):

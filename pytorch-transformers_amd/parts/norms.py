@@ -27,12 +27,22 @@ class LayerNorm(Part):
         self.weight = tensors[self.name + ".weight"]
         self.bias = tensors[self.name + ".bias"]
 
+    def _wide_loads(self, x: torch.Tensor) -> bool:
+        # bfloat16 rows of a width the sixteen-byte kernel takes: the one that also forms residual sums
+        return x.dtype == torch.bfloat16 and ops.layernorm_sum_ok(self.hidden_size)
+
     def forward(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        if self._wide_loads(x):
+            return ops.layernorm_sum([x], self.hidden_size, w=self.weight, b=self.bias, eps=self.eps, rows=rows,
+                                     want_x=False)[1]
         return ops.layernorm(x, self.weight, self.bias, self.eps, rows=rows)
 
     def forward_pair(self, x: torch.Tensor, other: "Part"):
         """``(self(x), other(x))``; one pass over x when both are LayerNorms with one eps."""
         if isinstance(other, LayerNorm) and other.eps == self.eps:
+            if self._wide_loads(x):
+                return ops.layernorm_sum([x], self.hidden_size, w=self.weight, b=self.bias, eps=self.eps,
+                                         w2=other.weight, b2=other.bias, want_x=False)[1:]
             return ops.layernorm(x, self.weight, self.bias, self.eps, w2=other.weight, b2=other.bias)
         return self.forward(x), other.forward(x)
 

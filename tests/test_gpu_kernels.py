@@ -185,6 +185,25 @@ def test_partial_product_equals_the_reduced_one():
     assert torch.equal(formed, whole)
 
 
+def test_gemm_skinny_pair():
+    """Two products of one launch equal the products on their own up to summation order."""
+    ops = _ops()
+    M, K, N1, N2 = 7, 328, 100, 530
+    x1, x2 = _rand(M, K, dtype=torch.bfloat16), _rand(M, K, seed=5, dtype=torch.bfloat16)
+    w1, w2 = _rand(N1, K, seed=1, dtype=torch.bfloat16, scale=0.05), _rand(N2, K, seed=2, dtype=torch.bfloat16, scale=0.05)
+    b2 = _rand(N2, seed=3)
+    y1, y2 = ops.gemm_skinny_pair_bf16(x1, w1, x2, w2, None, None, b2, "gelu")
+    torch.testing.assert_close(y1.float(), ops.gemm_skinny_bf16(x1, w1).float(), rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(y2.float(), ops.gemm_skinny_bf16(x2, w2, b2, "gelu").float(), rtol=2e-2, atol=2e-2)
+    want1 = (x1.double() @ w1.double().T).float()
+    torch.testing.assert_close(y1.float(), want1, rtol=2e-2, atol=2e-2 * float(want1.abs().max()))
+    # a row alone gives the same bits as in the batch
+    a1, a2 = ops.gemm_skinny_pair_bf16(x1[3:4].contiguous(), w1, x2[3:4].contiguous(), w2, None, None, b2, "gelu")
+    assert torch.equal(a1, y1[3:4]) and torch.equal(a2, y2[3:4])
+    with pytest.raises(ops.KernelError, match="shares M and K"):
+        ops.gemm_skinny_pair_bf16(x1, w1, x2[:3].contiguous(), w2)
+
+
 def test_gemm_skinny_refuses_what_it_cannot_do():
     ops = _ops()
     x, w = _rand(65, 64, dtype=torch.bfloat16), _rand(32, 64, dtype=torch.bfloat16)
