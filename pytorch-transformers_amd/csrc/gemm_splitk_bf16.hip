@@ -31,11 +31,25 @@ union Frag8 {
 
 #define SK_THREADS 256
 
+// One product of a launch.  A launch may carry two that share M (a block's two output projections, left
+// as partial sums): the workgroups of the second follow those of the first in a one-dimensional grid.
+struct SplitkProblem {
+    void* y;
+    float* part;
+    const bf16_t* x;
+    const bf16_t* W;
+    const float* bias;
+    const bf16_t* add1;
+    const bf16_t* add2;
+    int N, K, act, out_f32;
+    int blocks_per_part;  // 64-element blocks of K per range
+    int tiles;            // workgroups along N
+    int parts;            // ranges of K
+    int direct;           // one range and the epilogue in this kernel
+};
+
 template <int MT, int RT, int U, int D>
-__global__ __launch_bounds__(SK_THREADS) void gemm_splitk_kernel(
-    void* __restrict__ y, float* __restrict__ part, const bf16_t* __restrict__ x, const bf16_t* __restrict__ W,
-    const float* __restrict__ bias, const bf16_t* __restrict__ add1, const bf16_t* __restrict__ add2, int M, int N,
-    int K, int act, int out_f32, int blocks_per_part, int direct) {
+__global__ __launch_bounds__(SK_THREADS) void gemm_splitk_kernel(SplitkProblem pa, SplitkProblem pb, int M) {
     constexpr int KS = U * 64;                       // elements of K per stage
     constexpr int MP = MT * 16;                      // rows of x, padded to whole tiles
     constexpr int LDW = KS + 8;                      // LDS row stride: 16 bytes of padding keep 16-byte reads off each other's banks
@@ -47,9 +61,24 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_splitk_kernel(
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 15, g = lane >> 4;
-    const int n_base = blockIdx.x * (64 * RT) + wave * (16 * RT);
+    const int first_blocks = pa.tiles * pa.parts;
+    const bool second = (int)blockIdx.x >= first_blocks;
+    void* __restrict__ y = second ? pb.y : pa.y;
+    float* __restrict__ part = second ? pb.part : pa.part;
+    const bf16_t* __restrict__ x = second ? pb.x : pa.x;
+    const bf16_t* __restrict__ W = second ? pb.W : pa.W;
+    const float* __restrict__ bias = second ? pb.bias : pa.bias;
+    const bf16_t* __restrict__ add1 = second ? pb.add1 : pa.add1;
+    const bf16_t* __restrict__ add2 = second ? pb.add2 : pa.add2;
+    const int N = second ? pb.N : pa.N, K = second ? pb.K : pa.K, act = second ? pb.act : pa.act;
+    const int out_f32 = second ? pb.out_f32 : pa.out_f32, direct = second ? pb.direct : pa.direct;
+    const int blocks_per_part = second ? pb.blocks_per_part : pa.blocks_per_part;
+    const int tiles = second ? pb.tiles : pa.tiles;
+    const int idx = (int)blockIdx.x - (second ? first_blocks : 0);
+    const int tile = idx % tiles, range = idx / tiles;  // neighbours share a range of K: its x slice stays in L2
+    const int n_base = tile * (64 * RT) + wave * (16 * RT);
     const int nkb = (K + 63) >> 6;
-    const int kb0 = blockIdx.y * blocks_per_part, kb1 = min(kb0 + blocks_per_part, nkb);
+    const int kb0 = range * blocks_per_part, kb1 = min(kb0 + blocks_per_part, nkb);
     const int k_begin = kb0 * 64, k_end = min(kb1 * 64, K);
     const int nstages = (kb1 - kb0 + U - 1) / U;
 
@@ -139,9 +168,9 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_splitk_kernel(
             if (m >= M || n >= N) continue;
             const long o = (long)m * N + n;
             if (!direct) {
-                const long idx = (long)blockIdx.y * M * N + o;
-                float* dst = part + idx;
-                if (n + 3 < N && (idx & 3) == 0) *reinterpret_cast<f32x4_t*>(dst) = acc[t][mt];
+                const long at = (long)range * M * N + o;
+                float* dst = part + at;
+                if (n + 3 < N && (at & 3) == 0) *reinterpret_cast<f32x4_t*>(dst) = acc[t][mt];
                 else
                     for (int i = 0; i < 4 && n + i < N; ++i) dst[i] = acc[t][mt][i];
                 continue;
@@ -203,12 +232,23 @@ extern "C" int pta_gemm_splitk_parts(int N, int K, int parts, int rt) {
     return effective_parts(K, parts > 0 ? parts : pick_parts(N, K, rt));
 }
 
-template <int MT, int RT, int U, int D>
-static int launch_cfg(void* y, float* part, const bf16_t* x, const bf16_t* W, const float* bias, const bf16_t* add1,
-                      const bf16_t* add2, int M, int N, int K, int act, int out_f32, int P, int reduce, hipStream_t s) {
+static SplitkProblem make_problem(void* y, float* part, const void* x, const void* W, const float* bias,
+                                  const void* add1, const void* add2, int N, int K, int act, int out_f32, int rt,
+                                  int parts, int reduce) {
+    SplitkProblem p{};
+    p.y = y; p.part = part; p.x = (const bf16_t*)x; p.W = (const bf16_t*)W; p.bias = bias;
+    p.add1 = (const bf16_t*)add1; p.add2 = (const bf16_t*)add2;
+    p.N = N; p.K = K; p.act = act; p.out_f32 = out_f32;
     const int nkb = (K + 63) / 64;
-    const int per = (nkb + P - 1) / P;
-    const int parts = (nkb + per - 1) / per;  // ranges that are not empty
+    p.blocks_per_part = (nkb + parts - 1) / parts;
+    p.parts = (nkb + p.blocks_per_part - 1) / p.blocks_per_part;  // ranges that are not empty
+    p.tiles = (N + 64 * rt - 1) / (64 * rt);
+    p.direct = reduce && p.parts == 1;
+    return p;
+}
+
+template <int MT, int RT, int U, int D>
+static int launch_cfg(const SplitkProblem& a, const SplitkProblem& b, int M, int reduce, hipStream_t s) {
     const size_t lds = (size_t)2 * MT * 16 * (U * 64 + 8) * sizeof(bf16_t);
     auto kern = gemm_splitk_kernel<MT, RT, U, D>;
     if (lds > 64 * 1024) {
@@ -219,38 +259,41 @@ static int launch_cfg(void* y, float* part, const bf16_t* x, const bf16_t* W, co
             raised = true;
         }
     }
-    const dim3 grid((N + 64 * RT - 1) / (64 * RT), parts);
-    hipLaunchKernelGGL(kern, grid, dim3(SK_THREADS), lds, s, y, part, x, W, bias, add1, add2, M, N, K, act, out_f32, per,
-                       (int)(reduce && parts == 1));
-    if (reduce && parts > 1) {
-        const long MN = (long)M * N;
-        hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((MN + 255) / 256)), dim3(256), 0, s, y, part, bias,
-                           add1, add2, MN, N, parts, act, out_f32);
+    const dim3 grid(a.tiles * a.parts + b.tiles * b.parts);
+    hipLaunchKernelGGL(kern, grid, dim3(SK_THREADS), lds, s, a, b, M);
+    if (reduce && a.parts > 1) {
+        const long MN = (long)M * a.N;
+        hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((MN + 255) / 256)), dim3(256), 0, s, a.y, a.part,
+                           a.bias, a.add1, a.add2, MN, a.N, a.parts, a.act, a.out_f32);
     }
     return pta_check_launch("gemm_splitk_bf16");
 }
 
 template <int RT, int U, int D>
-static int launch_rows(int MT, void* y, float* part, const bf16_t* x, const bf16_t* W, const float* bias,
-                       const bf16_t* add1, const bf16_t* add2, int M, int N, int K, int act, int out_f32, int P,
-                       int reduce, hipStream_t s) {
+static int launch_rows(int MT, const SplitkProblem& a, const SplitkProblem& b, int M, int reduce, hipStream_t s) {
     switch (MT) {
-        case 1: return launch_cfg<1, RT, U, D>(y, part, x, W, bias, add1, add2, M, N, K, act, out_f32, P, reduce, s);
-        case 2: return launch_cfg<2, RT, U, D>(y, part, x, W, bias, add1, add2, M, N, K, act, out_f32, P, reduce, s);
-        case 3: return launch_cfg<3, RT, U, D>(y, part, x, W, bias, add1, add2, M, N, K, act, out_f32, P, reduce, s);
-        default: return launch_cfg<4, RT, U, D>(y, part, x, W, bias, add1, add2, M, N, K, act, out_f32, P, reduce, s);
+        case 1: return launch_cfg<1, RT, U, D>(a, b, M, reduce, s);
+        case 2: return launch_cfg<2, RT, U, D>(a, b, M, reduce, s);
+        case 3: return launch_cfg<3, RT, U, D>(a, b, M, reduce, s);
+        default: return launch_cfg<4, RT, U, D>(a, b, M, reduce, s);
     }
+}
+
+static int check_splitk(const char* what, const void* x, const void* W, int M, int N, int K) {
+    PTA_REQUIRE(M > 0 && N > 0 && K > 0, "%s: sizes must be positive (M=%d N=%d K=%d)", what, M, N, K);
+    PTA_REQUIRE(M <= 64, "%s: at most 64 rows, got %d (use the library product)", what, M);
+    PTA_REQUIRE(K % 8 == 0 && K >= 8, "%s: K=%d must be a multiple of 8 (16-byte loads)", what, K);
+    PTA_REQUIRE(x && W, "%s: null pointer", what);
+    PTA_REQUIRE((long)M * K * 2 < 0x7ffffff0L, "%s: x is too large for 32-bit buffer offsets", what);
+    PTA_REQUIRE(((uintptr_t)x % 16) == 0 && ((uintptr_t)W % 16) == 0, "%s: x and W must be 16-byte aligned", what);
+    return 0;
 }
 
 extern "C" int pta_gemm_splitk_bf16(void* y, float* part, const void* x, const void* W, const float* bias,
                                     const void* add1, const void* add2, int M, int N, int K, int act, int out_f32,
                                     int rt, int parts, int stage_blocks, int depth, int reduce, void* stream) {
-    PTA_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_splitk_bf16: sizes must be positive (M=%d N=%d K=%d)", M, N, K);
-    PTA_REQUIRE(M <= 64, "gemm_splitk_bf16: at most 64 rows, got %d (use the library product)", M);
-    PTA_REQUIRE(K % 8 == 0 && K >= 8, "gemm_splitk_bf16: K=%d must be a multiple of 8 (16-byte loads)", K);
-    PTA_REQUIRE(x && W && (y || !reduce), "gemm_splitk_bf16: null pointer");
-    PTA_REQUIRE((long)M * K * 2 < 0x7ffffff0L, "gemm_splitk_bf16: x is too large for 32-bit buffer offsets");
-    PTA_REQUIRE(((uintptr_t)x % 16) == 0 && ((uintptr_t)W % 16) == 0, "gemm_splitk_bf16: x and W must be 16-byte aligned");
+    if (check_splitk("gemm_splitk_bf16", x, W, M, N, K)) return 1;
+    PTA_REQUIRE(y || !reduce, "gemm_splitk_bf16: null pointer");
     PTA_REQUIRE(act == PTA_ACT_NONE || act == PTA_ACT_GELU, "gemm_splitk_bf16: unknown activation %d", act);
     PTA_REQUIRE(rt == 0 || rt == 1 || rt == 2, "gemm_splitk_bf16: row tiles per wave must be 0 (choose), 1 or 2, got %d", rt);
     PTA_REQUIRE(stage_blocks == 0 || stage_blocks == 2,
@@ -259,17 +302,28 @@ extern "C" int pta_gemm_splitk_bf16(void* y, float* part, const void* x, const v
     PTA_REQUIRE(parts >= 0 && parts <= 64, "gemm_splitk_bf16: parts must be 0 (choose) or 1..64, got %d", parts);
     if (rt == 0) rt = pick_rt(N);
     if (parts == 0) parts = pick_parts(N, K, rt);
-    if (stage_blocks == 0) stage_blocks = 2;
-    PTA_REQUIRE((parts == 1 && reduce) || part, "gemm_splitk_bf16: %d ranges of K need the workspace for partial sums", parts);
-    parts = effective_parts(K, parts);  // what the caller's workspace must hold
+    if (depth == 0) depth = 2;  // measured: more stages in flight per wave do not pay, more workgroups do
+    const SplitkProblem a = make_problem(y, part, x, W, bias, add1, add2, N, K, act, out_f32, rt, parts, reduce);
+    PTA_REQUIRE(a.direct || part, "gemm_splitk_bf16: %d ranges of K need the workspace for partial sums", a.parts);
+    const SplitkProblem none{};
     hipStream_t s = (hipStream_t)stream;
     const int MT = (M + 15) / 16;
-    const bf16_t *xb = (const bf16_t*)x, *wb = (const bf16_t*)W, *a1 = (const bf16_t*)add1, *a2 = (const bf16_t*)add2;
-    if (depth == 0) depth = 2;  // measured: more stages in flight per wave do not pay, more workgroups do
-#define SK_CASE(RT_, U_, D_)                                                                                      \
-    if (rt == RT_ && stage_blocks == U_ && depth == D_)                                                           \
-        return launch_rows<RT_, U_, D_>(MT, y, part, xb, wb, bias, a1, a2, M, N, K, act, out_f32, parts, reduce, s);
-    SK_CASE(1, 2, 2) SK_CASE(1, 2, 4) SK_CASE(2, 2, 2) SK_CASE(2, 2, 4)
-#undef SK_CASE
-    return pta_fail("gemm_splitk_bf16: no kernel for rt=%d stage_blocks=%d depth=%d", rt, stage_blocks, depth);
+    if (rt == 1 && depth == 2) return launch_rows<1, 2, 2>(MT, a, none, M, reduce, s);
+    if (rt == 1) return launch_rows<1, 2, 4>(MT, a, none, M, reduce, s);
+    if (depth == 2) return launch_rows<2, 2, 2>(MT, a, none, M, reduce, s);
+    return launch_rows<2, 2, 4>(MT, a, none, M, reduce, s);
+}
+
+// Two products of one launch, both left as partial sums: part1 [parts1, M, N1] of x1 . W1^T and part2
+// [parts2, M, N2] of x2 . W2^T, with the ranges pta_gemm_splitk_parts(N, K, 0, 1) gives for each.
+extern "C" int pta_gemm_splitk_pair_bf16(float* part1, const void* x1, const void* W1, int N1, int K1, float* part2,
+                                         const void* x2, const void* W2, int N2, int K2, int M, void* stream) {
+    if (check_splitk("gemm_splitk_pair_bf16", x1, W1, M, N1, K1)) return 1;
+    if (check_splitk("gemm_splitk_pair_bf16", x2, W2, M, N2, K2)) return 1;
+    PTA_REQUIRE(part1 && part2, "gemm_splitk_pair_bf16: null workspace");
+    const SplitkProblem a = make_problem(nullptr, part1, x1, W1, nullptr, nullptr, nullptr, N1, K1, 0, 0, 1,
+                                         pick_parts(N1, K1, 1), 0);
+    const SplitkProblem b = make_problem(nullptr, part2, x2, W2, nullptr, nullptr, nullptr, N2, K2, 0, 0, 1,
+                                         pick_parts(N2, K2, 1), 0);
+    return launch_rows<1, 2, 2>((M + 15) / 16, a, b, M, 0, (hipStream_t)stream);
 }

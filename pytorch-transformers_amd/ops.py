@@ -389,6 +389,31 @@ def gemm_splitk_partial(x: torch.Tensor, w: torch.Tensor, rt: int = 0, parts: in
     return part
 
 
+def gemm_splitk_pair_partial(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tensor, w2: torch.Tensor):
+    """(x1 @ w1.T, x2 @ w2.T), both left as 32-bit partial sums, in one launch; the products share M."""
+    for name, t in (("x1", x1), ("w1", w1), ("x2", x2), ("w2", w2)):
+        _need(t, name, torch.bfloat16)
+    M = x1.shape[0]
+    if x2.shape[0] != M or w1.dim() != 2 or w2.dim() != 2 or w1.shape[1] != x1.shape[1] or w2.shape[1] != x2.shape[1]:
+        raise KernelError(f"a pair shares M: x1 {tuple(x1.shape)}, w1 {tuple(w1.shape)}, x2 {tuple(x2.shape)}, "
+                          f"w2 {tuple(w2.shape)}")
+    lib = load_library()
+    (N1, K1), (N2, K2) = w1.shape, w2.shape
+    part1 = torch.empty((int(lib.pta_gemm_splitk_parts(N1, K1, 0, 1)), M, N1), dtype=torch.float32, device=x1.device)
+    part2 = torch.empty((int(lib.pta_gemm_splitk_parts(N2, K2, 0, 1)), M, N2), dtype=torch.float32, device=x1.device)
+    _call("pta_gemm_splitk_pair_bf16", _ptr(part1), _ptr(x1), _ptr(w1), N1, K1, _ptr(part2), _ptr(x2), _ptr(w2), N2, K2,
+          M, _stream())
+    return part1, part2
+
+
+def gemm_partial_pair_ok(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tensor, w2: torch.Tensor) -> bool:
+    """Whether two products onto the same features are best left as partial sums of one launch: up to 64
+    rows each, and at least one of them worth leaving so on its own."""
+    return (_bf16_rows_ok(x1, w1) and _bf16_rows_ok(x2, w2) and 0 < x1.shape[0] == x2.shape[0] <= SKINNY_MAX_ROWS
+            and w1.shape[0] == w2.shape[0] and w1.shape[0] % 8 == 0
+            and (gemm_partial_ok(x1, w1) or gemm_partial_ok(x2, w2)))
+
+
 def gemm_partial_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
     """Whether leaving x @ w.T as partial sums for the next norm pays: up to 64 rows, and either K long against
     N (any batch: the kernel for few rows has too few row tiles there) or a batch past 16 rows."""

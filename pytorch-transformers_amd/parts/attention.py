@@ -17,7 +17,7 @@ import torch
 
 from .. import ops
 from .base import Part, StepContext, register_part
-from .linear import Linear
+from .linear import Linear, PendingProjection
 
 
 class AttentionMixer(Part):
@@ -51,7 +51,7 @@ class AttentionMixer(Part):
     def forward(self, x: torch.Tensor, ctx: StepContext, call, residual: Optional[torch.Tensor] = None,
                 defer: bool = False, projected: Optional[torch.Tensor] = None):
         """Attention of the step's tokens over the cache, projected out, plus ``residual``.  With ``defer``
-        the output projection may come back as a ``PartialProduct``, without the residual."""
+        the output projection comes back not run (``PendingProjection``); the caller adds the residual."""
         k_pool, v_pool = ctx.cache.kv_layer(call.cache_group, call.cache_layer)
         table = ctx.block_tables[call.cache_group]
         fused = projected if projected is not None else self.qkv(x, apply_bias=False)
@@ -61,9 +61,7 @@ class AttentionMixer(Part):
                                write_cache=call.write_cache)
         o = ops.attention(q, k_pool, v_pool, table, ctx, self.positions.score_bias(), self.scale)
         if defer:
-            p = self.out.partial(o)
-            if p is not None:
-                return p
+            return PendingProjection(self.out, o)
         return self.out(o, add1=residual)
 
 

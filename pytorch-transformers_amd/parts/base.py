@@ -24,13 +24,16 @@ positions      ``rotation() -> (inv_freq or None, scale)`` for queries and keys,
 block          ``forward(x, ctx, call) -> x``: the arrangement of the above
 =============  ==================================================================
 
-Optional, for parts that set ``can_defer = True``: a mixer or feed-forward called
-with ``defer=True`` may leave its last product unreduced and return a
-:class:`PartialProduct` (mixer, residual not added) or a :class:`ResidualSum`
-(feed-forward, its addends included); a norm with ``forward_sum(sum, rows=None,
-other=None, want_x=True) -> (x, normed, normed_other)`` forms such a sum while it
-normalises it; a block with ``accepts_sum = True`` takes a ``ResidualSum`` as its
-input.  Everything else receives plain tensors.
+Optional: a mixer or feed-forward that sets ``can_defer = True`` and is called with
+``defer=True`` returns its last product not run, as a ``PendingProjection`` (the
+``Linear`` and its input; residual and additions are then the caller's), and one
+with ``input_projection()`` lets the block run its first product and hand the result
+in as ``projected``.  A block may so run two branches' products in one launch, and
+leave the last ones as 32-bit partial sums (:class:`PartialProduct`) in a
+:class:`ResidualSum` that it returns in place of a tensor.  A norm with
+``forward_sum(sum, rows=None, other=None, want_x=True) -> (x, normed, normed_other)``
+forms such a sum while it normalises it; a block with ``accepts_sum = True`` takes one
+as its input.  Everything else receives plain tensors.
 """
 from __future__ import annotations
 

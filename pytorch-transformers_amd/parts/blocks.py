@@ -19,7 +19,7 @@ from typing import Optional, Sequence
 import torch
 
 from .base import Part, PartialProduct, ResidualSum, StepContext, register_part
-from .linear import Linear
+from .linear import Linear, PendingProjection
 
 
 def _can_defer(part: Part) -> bool:
@@ -36,6 +36,22 @@ def _normed(x, norm: Part, other: Optional[Part] = None):
         return x, norm.forward(x), None
     a, m = norm.forward_pair(x, other)
     return x, a, m
+
+
+def _sum_parallel(ffn_out: PendingProjection, mixer_out: PendingProjection, x: torch.Tensor):
+    """feed-forward + mixer + residual, in that order, formed now or left to the next norm."""
+    both = PendingProjection.partial_pair(ffn_out, mixer_out)
+    if both is not None:
+        return ResidualSum([both[0], both[1], x])
+    p = ffn_out.partial()
+    if p is not None:
+        return ResidualSum([p, mixer_out.partial() or mixer_out.run(), x])
+    return ffn_out.run(add1=mixer_out.run(), add2=x)
+
+
+def _sum_sequential(out: PendingProjection, residual: torch.Tensor):
+    p = out.partial()
+    return ResidualSum([p, residual]) if p is not None else out.run(add1=residual)
 
 
 class ParallelBlock(Part):
@@ -56,8 +72,6 @@ class ParallelBlock(Part):
             m = a
         side = ctx.side_stream
         if side is None or not hasattr(self.feed_forward, "forward_up"):
-            # where the parts can, the last products stay unreduced and the next norm forms
-            # feed-forward + mixer + residual while it reads them
             kw_mixer, kw_ffn = {}, {}
             # both branches start with a product of the norm's output: one launch for the two in small steps
             if hasattr(self.mixer, "input_projection") and hasattr(self.feed_forward, "input_projection"):
@@ -65,11 +79,12 @@ class ParallelBlock(Part):
                 both = Linear.pair(lin_a, a, kw_a, lin_m, m, kw_m)
                 if both is not None:
                     kw_mixer["projected"], kw_ffn["projected"] = both
-            if _can_defer(self.feed_forward):
-                if _can_defer(self.mixer):
-                    kw_mixer["defer"] = True
-                mixed = self.mixer.forward(a, ctx, call, **kw_mixer)
-                return self.feed_forward.forward(m, ctx, add1=mixed, add2=x, defer=True, **kw_ffn)
+            if _can_defer(self.feed_forward) and _can_defer(self.mixer):
+                # the branches' last products: one launch of partial sums where that pays, which the
+                # next norm adds to the residual while it reads them
+                out_a = self.mixer.forward(a, ctx, call, defer=True, **kw_mixer)
+                out_m = self.feed_forward.forward(m, ctx, defer=True, **kw_ffn)
+                return _sum_parallel(out_m, out_a, x)
             mixed = self.mixer.forward(a, ctx, call, **kw_mixer)
             return self.feed_forward.forward(m, ctx, add1=mixed, add2=x, **kw_ffn)
         # The feed-forward's first product needs only the norm, not the mixer: it runs on a second
@@ -99,14 +114,12 @@ class SequentialBlock(Part):
     def forward(self, x, ctx: StepContext, call):
         x, a, _ = _normed(x, self.norm_in)
         if _can_defer(self.mixer):
-            r = self.mixer.forward(a, ctx, call, residual=x, defer=True)
-            if isinstance(r, PartialProduct):
-                r = ResidualSum([r, x])
+            r = _sum_sequential(self.mixer.forward(a, ctx, call, defer=True), x)
         else:
             r = self.mixer.forward(a, ctx, call, residual=x)
         r, m, _ = _normed(r, self.norm_post)
         if _can_defer(self.feed_forward):
-            return self.feed_forward.forward(m, ctx, add1=r, defer=True)
+            return _sum_sequential(self.feed_forward.forward(m, ctx, defer=True), r)
         return self.feed_forward.forward(m, ctx, add1=r)
 
 

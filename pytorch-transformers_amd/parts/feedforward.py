@@ -7,8 +7,8 @@ from typing import Sequence
 
 import torch
 
-from .base import Part, ResidualSum, StepContext, as_tensor, register_part
-from .linear import Linear
+from .base import Part, StepContext, as_tensor, register_part
+from .linear import Linear, PendingProjection
 
 
 class DenseFeedForward(Part):
@@ -31,12 +31,11 @@ class DenseFeedForward(Part):
         return self.up, {"act": self.activation}
 
     def forward(self, x: torch.Tensor, ctx: StepContext, add1=None, add2=None, defer: bool = False, projected=None):
-        """``down(act(up(x))) + add1 + add2``; with ``defer`` the sum may come back unformed."""
+        """``down(act(up(x))) + add1 + add2``.  With ``defer`` the second product comes back not run
+        (``PendingProjection``) and the caller sees to the additions."""
         h = projected if projected is not None else self.up(x, act=self.activation)
         if defer:
-            p = self.down.partial(h)
-            if p is not None:
-                return ResidualSum([p, add1, add2])
+            return PendingProjection(self.down, h)
         return self.down(h, add1=as_tensor(add1), add2=as_tensor(add2))
 
     # The two halves on their own: a block whose feed-forward does not read the mixer's output can run

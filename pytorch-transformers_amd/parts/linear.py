@@ -75,6 +75,32 @@ class Linear(Part):
         return None
 
 
+class PendingProjection:
+    """A part's last product, not run yet: the ``Linear`` and its input.  A mixer or feed-forward called
+    with ``defer=True`` returns it, and the block chooses how to run it: on its own with the additions in
+    its epilogue (``run``), left as partial sums for the next norm (``partial``), or together with the
+    other branch's in one launch (``partial_pair``)."""
+
+    def __init__(self, linear: Linear, x: torch.Tensor):
+        self.linear, self.x = linear, x
+
+    def run(self, add1=None, add2=None) -> torch.Tensor:
+        return self.linear(self.x, add1=add1, add2=add2)
+
+    def partial(self) -> Optional[PartialProduct]:
+        return self.linear.partial(self.x)
+
+    @staticmethod
+    def partial_pair(first: "PendingProjection", second: "PendingProjection"):
+        """Both as partial sums from one launch, or None where that does not apply."""
+        a, b = first, second
+        if not (a.x.dtype == torch.bfloat16 and ops.layernorm_sum_ok(a.linear.out_features)
+                and ops.gemm_partial_pair_ok(a.x, a.linear.weight, b.x, b.linear.weight)):
+            return None
+        pa, pb = ops.gemm_splitk_pair_partial(a.x, a.linear.weight, b.x, b.linear.weight)
+        return PartialProduct(pa, a.linear.bias), PartialProduct(pb, b.linear.bias)
+
+
 class Embedding(Part):
     """``h[t] = E[id_t]``, no scaling (src/transformers/models/falcon/modeling_falcon.py:835, :895-896)."""
 
