@@ -32,6 +32,25 @@ def falcon7b_config(layers):
                         max_position_embeddings=2048, tie_word_embeddings=True)
 
 
+def falcon_config(sizes, layers):
+    """Layer sizes of the published models; "7b" is the default run, the others are for comparison."""
+    from pytorch_transformers_amd import FalconConfig
+
+    if sizes == "7b":
+        return falcon7b_config(layers or 32), 32
+    if sizes == "11b":  # Falcon2-11B: 32 heads in 8 groups of head size 128, one norm
+        return FalconConfig(vocab_size=65024, hidden_size=4096, num_hidden_layers=layers or 60, num_attention_heads=32,
+                            num_kv_heads=8, new_decoder_architecture=True, num_ln_in_parallel_attn=1,
+                            parallel_attn=True, bias=False, alibi=False, ffn_hidden_size=16384, rope_theta=500042.0,
+                            layer_norm_epsilon=1e-5, max_position_embeddings=8192, tie_word_embeddings=False), 60
+    if sizes == "40b":  # Falcon-40B: 128 heads in 8 groups of head size 64, two norms
+        return FalconConfig(vocab_size=65024, hidden_size=8192, num_hidden_layers=layers or 60, num_attention_heads=128,
+                            num_kv_heads=8, new_decoder_architecture=True, num_ln_in_parallel_attn=2,
+                            parallel_attn=True, bias=False, alibi=False, ffn_hidden_size=32768, rope_theta=10000.0,
+                            layer_norm_epsilon=1e-5, max_position_embeddings=2048, tie_word_embeddings=False), 60
+    raise ValueError(sizes)
+
+
 def weight_bytes(cfg, elem):
     H, F, Q = cfg.hidden_size, cfg.ffn_hidden_size, cfg.qkv_out_dim
     per_layer = (Q * H + H * H + 2 * F * H) * elem
@@ -62,12 +81,12 @@ def run_decode(model, sampler_cls, gen_cfg, batch, prompt_len, steps, warmup, se
     slots = [cache.alloc() for _ in range(batch)]
     logits = model.step(cache, slots, prompts, "last")
     rng = list(range(batch))
-    tokens, _ = sampler.sample(logits, rng_seq=rng, rng_step=[0] * batch)
+    tokens, _ = sampler.sample(logits, rng_seq=rng, rng_step=[0] * batch, need_scores=False)
 
     def one(k):
         nonlocal tokens
         lg = model.step(cache, slots, [[t] for t in tokens], "last")
-        tokens, _ = sampler.sample(lg, rng_seq=rng, rng_step=[k] * batch)
+        tokens, _ = sampler.sample(lg, rng_seq=rng, rng_step=[k] * batch, need_scores=False)  # as generate() calls it
 
     for k in range(warmup):
         one(k)
@@ -111,7 +130,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--prompt-len", type=int, default=1024)
-    ap.add_argument("--layers", type=int, default=32, help="fewer than 32 only where memory or time needs it")
+    ap.add_argument("--layers", type=int, default=0, help="fewer than the model has only where memory or time needs it")
+    ap.add_argument("--sizes", default="7b", choices=["7b", "11b", "40b"],
+                    help="layer sizes: Falcon-7B (the default run), Falcon2-11B or Falcon-40B")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / batch 64 / prefill measurements")
     ap.add_argument("--only-prefill", action="store_true",
@@ -127,7 +148,8 @@ def main():
     from pytorch_transformers_amd.sampling import Sampler
 
     ops.load_library()
-    cfg = falcon7b_config(args.layers)
+    cfg, full_layers = falcon_config(args.sizes, args.layers)
+    args.layers = cfg.num_hidden_layers
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
     elem = 2 if args.dtype == "bf16" else 4
     model = AutoModelForCausalLM.from_config(cfg, seed=0, dtype=dtype, device="cuda:0")
@@ -146,11 +168,11 @@ def main():
     achieved = step_bytes / (ms * 1e-3) / 1e9
 
     out = {
-        "metric": "falcon7b_decode_tokens_per_second", "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1,
+        "metric": f"falcon{args.sizes}_decode_tokens_per_second", "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
         "data": "synthetic token ids, random weights N(0, 0.02)",
-        "config": {"model": "falcon-7b layer sizes", "layers": args.layers, "layers_of_config": 32,
+        "config": {"model": f"falcon-{args.sizes} layer sizes", "layers": args.layers, "layers_of_config": full_layers,
                    "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.kv_heads,
                    "head_dim": cfg.head_dim, "ffn": cfg.ffn_hidden_size, "vocab": cfg.vocab_size,
                    "global_batch": args.batch, "prompt_len": args.prompt_len, "seq_len": 2048,

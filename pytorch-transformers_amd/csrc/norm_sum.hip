@@ -11,8 +11,8 @@
 // (feed-forward plus mixer first, then the residual).  `rows` selects source rows (the final norm reads
 // only the rows whose logits are wanted).
 //
-// One workgroup of 1024 threads per row; a thread holds a chunk of eight features in registers
-// (H <= 8192, H % 8 == 0), loaded and stored sixteen bytes at a time.  Norm weights are loaded before the
+// One workgroup per row with a thread for every eight features (whole waves, at most 1024 threads:
+// H <= 8192, H % 8 == 0); a thread holds its chunk in registers, loaded and stored sixteen bytes at a time.  Norm weights are loaded before the
 // reductions so that their latency hides behind them.  Mean and biased variance in 32-bit, variance
 // from the centred values.
 #include "common.h"
@@ -159,7 +159,8 @@ extern "C" int pta_layernorm_sum(void* out_x, void* out1, void* out2, const floa
     PTA_REQUIRE(rows || M == M_in, "layernorm_sum: without row selection M (%d) must equal M_in (%d)", M, M_in);
     const void* ptrs[] = {out_x, out1, out2, pa, pb, add1, add2, bias_a, bias_b, w1, b1, w2, b2};
     for (const void* p : ptrs) PTA_REQUIRE(((uintptr_t)p % 16) == 0, "layernorm_sum: pointers must be 16-byte aligned");
-    hipLaunchKernelGGL(layernorm_sum_kernel, dim3(M), dim3(NS_THREADS), 0, (hipStream_t)stream, (bf16_t*)out_x,
+    const int threads = (H / 8 + 63) / 64 * 64;  // one chunk of eight features per thread, whole waves
+    hipLaunchKernelGGL(layernorm_sum_kernel, dim3(M), dim3(threads), 0, (hipStream_t)stream, (bf16_t*)out_x,
                        (bf16_t*)out1, (bf16_t*)out2, pa, Pa, bias_a, pb, Pb, bias_b, (const bf16_t*)add1,
                        (const bf16_t*)add2, rows, w1, b1, w2, b2, M_in, H, eps);
     return pta_check_launch("layernorm_sum");

@@ -101,6 +101,9 @@ int pta_sample(int* out_tok, float* work, const float* logits, int R, int V, int
                const int* eos, int n_eos, const int* suppress, int remove_invalid, int renorm, uint64_t seed,
                const int* rng_seq, const int* rng_step, const float* uniforms, void* stream);
 
+// out_tok[r] = index of the largest of logits[r, :], lowest index among equals (greedy choice, no processors)
+int pta_argmax(int* out_tok, const float* logits, int R, int V, void* stream);
+
 // host function: the uniform number in [0, 1) that pta_sample draws for (seed, sequence, step)
 float pta_philox_uniform(uint64_t seed, uint32_t seq, uint32_t step);
 

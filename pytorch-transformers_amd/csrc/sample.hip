@@ -69,6 +69,42 @@ __device__ __forceinline__ ArgBest block_argmax(float v, int i, float* red_v, in
     return b;
 }
 
+// Greedy choice with no processor in the way: the largest logit of each row, lowest index among equals,
+// read sixteen bytes at a time and never written back.
+__global__ __launch_bounds__(S_THREADS) void argmax_kernel(int* __restrict__ out_tok, const float* __restrict__ logits,
+                                                           int V) {
+    __shared__ float red[16];
+    __shared__ int red_i[16];
+    const int row = blockIdx.x, tid = threadIdx.x;
+    const float* l = logits + (long)row * V;
+    float mx = -INFINITY;
+    int mi = 0x7fffffff;
+    const int head = (int)((16 - ((uintptr_t)l & 15)) & 15) / 4;  // elements before the first 16-byte boundary
+    const int first = min(head, V), quads = (V - first) / 4;
+    if (tid < first && l[tid] > mx) { mx = l[tid]; mi = tid; }
+    const float4* l4 = reinterpret_cast<const float4*>(l + first);
+    for (int q = tid; q < quads; q += S_THREADS) {
+        const float4 v = l4[q];
+        const int i = first + q * 4;
+        if (v.x > mx) { mx = v.x; mi = i; }
+        if (v.y > mx) { mx = v.y; mi = i + 1; }
+        if (v.z > mx) { mx = v.z; mi = i + 2; }
+        if (v.w > mx) { mx = v.w; mi = i + 3; }
+    }
+    for (int i = first + quads * 4 + tid; i < V; i += S_THREADS)
+        if (l[i] > mx) { mx = l[i]; mi = i; }
+    // a thread meets its candidates in index order and keeps the first of equals; so does the reduction
+    const ArgBest best = block_argmax(mx, mi, red, red_i);
+    if (tid == 0) out_tok[row] = best.i;
+}
+
+extern "C" int pta_argmax(int* out_tok, const float* logits, int R, int V, void* stream) {
+    PTA_REQUIRE(R > 0 && V > 0, "argmax: R=%d V=%d must be positive", R, V);
+    PTA_REQUIRE(out_tok && logits, "argmax: null pointer");
+    hipLaunchKernelGGL(argmax_kernel, dim3(R), dim3(S_THREADS), 0, (hipStream_t)stream, out_tok, logits, V);
+    return pta_check_launch("argmax");
+}
+
 #define MASS_ONE 1099511627776.0f /* 2^40 */
 
 __global__ __launch_bounds__(S_THREADS) void sample_kernel(

@@ -299,12 +299,20 @@ def attention(q: torch.Tensor, k_pool, v_pool, block_table, ctx, slopes, scale: 
 def sample(logits: torch.Tensor, *, do_sample: bool, temperature: float = 1.0, top_k: int = 0, top_p: float = 1.0,
            min_p: float = 0.0, penalty: float = 1.0, hist=None, hist_off=None, eos=None, suppress=None,
            remove_invalid: bool = False, renorm: bool = False, seed: int = 0, rng_seq=None, rng_step=None,
-           uniforms=None):
-    """Processors and choice for every row of ``logits`` [R, V] (32-bit); returns (tokens int32 [R], scores [R, V])."""
+           uniforms=None, need_scores: bool = True):
+    """Processors and choice for every row of ``logits`` [R, V] (32-bit); returns (tokens int32 [R], scores [R, V]).
+
+    Without ``need_scores``, a greedy choice that no processor touches is a plain argmax and the scores
+    come back as None."""
     _need(logits, "logits", torch.float32)
     if logits.dim() != 2:
         raise KernelError(f"logits must be [rows, vocab], got {tuple(logits.shape)}")
     R, V = logits.shape
+    if (not need_scores and not do_sample and penalty == 1.0 and suppress is None and not remove_invalid
+            and not renorm):
+        out = torch.empty((R,), dtype=torch.int32, device=logits.device)
+        _call("pta_argmax", _ptr(out), _ptr(logits), R, V, _stream())
+        return out, None
     for name, t, n in (("hist_off", hist_off, R + 1), ("suppress", suppress, R), ("rng_seq", rng_seq, R),
                        ("rng_step", rng_step, R)):
         if t is not None:

@@ -36,8 +36,10 @@ class Sampler:
 
     def sample(self, logits: torch.Tensor, *, rng_seq: Sequence[int], rng_step: Sequence[int],
                histories: Optional[Sequence[Sequence[int]]] = None, suppress_eos: Optional[Sequence[bool]] = None,
-               uniforms: Optional[Sequence[float]] = None) -> Tuple[List[int], torch.Tensor]:
-        """Tokens for the rows of ``logits`` and the processed scores ``[rows, vocab]``."""
+               uniforms: Optional[Sequence[float]] = None,
+               need_scores: bool = True) -> Tuple[List[int], Optional[torch.Tensor]]:
+        """Tokens for the rows of ``logits`` and the processed scores ``[rows, vocab]`` (None if not needed
+        and the choice could be made without forming them)."""
         R = logits.shape[0]
         use_hist = self.penalty != 1.0 and histories is not None
         pieces = [np.asarray(rng_seq, dtype=np.int32), np.asarray(rng_step, dtype=np.int32),
@@ -57,7 +59,7 @@ class Sampler:
             hist_off=views[3] if use_hist else None, eos=self._eos_dev,
             suppress=views[2] if (self._eos_dev is not None and suppress_eos is not None and any(suppress_eos)) else None,
             remove_invalid=self.config.remove_invalid_values, renorm=self.config.renormalize_logits,
-            seed=self.config.seed, rng_seq=views[0], rng_step=views[1], uniforms=u)
+            seed=self.config.seed, rng_seq=views[0], rng_step=views[1], uniforms=u, need_scores=need_scores)
         return tokens.tolist(), scores
 
 

@@ -51,7 +51,7 @@ class ArgmaxSampler:
         self.calls = []
         self.eos = list(eos)
 
-    def sample(self, logits, *, rng_seq, rng_step, histories, suppress_eos, uniforms=None):
+    def sample(self, logits, *, rng_seq, rng_step, histories, suppress_eos, uniforms=None, need_scores=True):
         self.calls.append(dict(rng_seq=list(rng_seq), rng_step=list(rng_step), suppress=list(suppress_eos),
                                histories=[list(h) for h in histories]))
         scores = logits.clone()

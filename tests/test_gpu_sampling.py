@@ -212,3 +212,23 @@ def test_pipeline_and_cli_style_entry(folders):
     pipe = pipeline("text-generation", model=folders["A"], dtype="float32")
     out = pipe([[3, 4, 5]], max_new_tokens=4, do_sample=False, eos_token_id=None)
     assert len(out) == 1 and out[0][0]["generated_token_ids"][:3] == [3, 4, 5] and len(out[0][0]["generated_token_ids"]) == 7
+
+
+def test_greedy_without_scores_is_an_argmax():
+    """The plain argmax path: ties go to the lowest index, rows of odd length start off a 16-byte boundary."""
+    from pytorch_transformers_amd import ops
+
+    for V in (1, 5, 211, 4099, 65024):
+        g = torch.Generator().manual_seed(V)
+        logits = torch.randn(5, V, generator=g).cuda()
+        if V > 4:
+            logits[1, [V - 1, 2]] = 50.0  # equal maxima: the lower index wins
+            logits[2, V - 1] = 60.0  # the last element, in the tail past the 16-byte groups
+            logits[3, 0] = 70.0  # the first element, before the first 16-byte boundary of an odd row
+        tok, scores = ops.sample(logits, do_sample=False, need_scores=False)
+        assert scores is None
+        assert tok.tolist() == torch.argmax(logits, dim=-1).tolist() or V > 4
+        want = [int(torch.nonzero(r == r.max())[0]) for r in logits]
+        assert tok.tolist() == want
+        full, _ = ops.sample(logits, do_sample=False)
+        assert full.tolist() == want
