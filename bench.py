@@ -123,6 +123,26 @@ def run_prefill(model, T, reps=3, seed=1):
     return best
 
 
+MIXED = {"7b": (8, 1024, 1024, 128), "11b": (16, 128, 4096, 256), "40b": (32, 64, 1536, 512)}
+
+
+def run_mixed(model, batch, lo, hi, new, seed=2):
+    """One batch of prompts with seeded uniform lengths in [lo, hi] through ``generate`` (greedy, no stop
+    token): the whole request, prefill included.  Returns (seconds, prompt tokens)."""
+    import torch
+
+    g = torch.Generator().manual_seed(seed)
+    lens = torch.randint(lo, hi + 1, (batch,), generator=g).tolist()
+    prompts = [torch.randint(0, model.vocab_size, (n,), generator=g).tolist() for n in lens]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    out = model.generate(prompts, max_new_tokens=new, do_sample=False, eos_token_id=None)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    assert all(len(o) == len(p) + new for o, p in zip(out, prompts))
+    return dt, sum(lens)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -135,6 +155,9 @@ def main():
                     help="layer sizes: Falcon-7B (the default run), Falcon2-11B or Falcon-40B")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / batch 64 / prefill measurements")
+    ap.add_argument("--mixed", action="store_true",
+                    help="one batch of unequal prompts through generate(): 11b 16 x U[128,4096] + 256 new, "
+                         "40b 32 x U[64,1536] + 512 new; prints its own record")
     ap.add_argument("--only-prefill", action="store_true",
                     help="run the 2,048-token prefill alone and print its record (for profiling)")
     args = ap.parse_args()
@@ -154,6 +177,16 @@ def main():
     elem = 2 if args.dtype == "bf16" else 4
     model = AutoModelForCausalLM.from_config(cfg, seed=0, dtype=dtype, device="cuda:0")
     gen_cfg = GenerationConfig(do_sample=False, eos_token_id=None)
+    if args.mixed:
+        batch, lo, hi, new = MIXED[args.sizes]
+        run_mixed(model, 2, lo, min(hi, lo + 64), 4)  # builds what the first call builds
+        dt, prompt_tokens = run_mixed(model, batch, lo, hi, new)
+        print(json.dumps({"metric": f"falcon{args.sizes}_mixed_generated_tokens_per_second",
+                          "value": round(batch * new / dt, 1), "unit": "tokens/s", "seconds": round(dt, 3),
+                          "batch": batch, "prompt_tokens": prompt_tokens, "new_tokens_each": new,
+                          "prompt_lengths": f"U[{lo},{hi}]", "layers": args.layers, "dtype": args.dtype,
+                          "note": "whole requests, prefill included; greedy, no stop token"}))
+        return 0
     if args.only_prefill:
         pt = run_prefill(model, 2048)
         print(json.dumps({"prefill": {"value": round(2048 / pt, 1), "tokens": 2048, "ms": round(pt * 1e3, 3),
