@@ -78,8 +78,11 @@ __device__ __forceinline__ void load_block(KvBlock<DT>& b, int kb, const int* __
         b.v[dt].u = *reinterpret_cast<const uint4*>(vpage + (long)(dt * 16 + c) * PTA_PAGE + in_page + gq * 8);
 }
 
-template <int DT, int CT>
-__global__ __launch_bounds__(64) void attn_mfma_kernel(
+// W = 1: a workgroup is one wave, which loads its keys and values straight from global memory.
+// W = 4 (prompts): four waves with neighbouring column groups walk the keys together and share every
+// block through LDS, so that a block crosses the vector memory path once for 64 * CT columns.
+template <int DT, int CT, int W>
+__global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
     bf16_t* __restrict__ out, float* __restrict__ po, float* __restrict__ pm, float* __restrict__ pl,
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
     const int* __restrict__ block_table, int bt_stride, const int* __restrict__ cu_tokens,
@@ -88,19 +91,21 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(
     constexpr int D = DT * 16;
     constexpr int DS = (DT + 1) / 2;   // 32-wide steps over the head dimension
     constexpr int CHUNKS = D / 8;      // 16-byte chunks in a row of d elements
-    const int lane = threadIdx.x, c = lane & 15, gq = lane >> 4;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, gq = lane >> 4;
     const int seq = blockIdx.z / n_splits, split = blockIdx.z % n_splits;
     const int kvh = blockIdx.y, g = nh / nkv;
     const int t0 = cu_tokens[seq], n_new = cu_tokens[seq + 1] - t0, start = seq_start[seq];
     // column groups are handed out last first: late tokens see the most keys, and the longest work
     // should start first so that the launch ends evenly
-    const int ncols = n_new * g, col0 = (gridDim.x - 1 - blockIdx.x) * (16 * CT);
-    if (col0 >= ncols) return;
+    const int ncols = n_new * g, wg_col0 = (gridDim.x - 1 - blockIdx.x) * (16 * CT * W);
+    if (wg_col0 >= ncols) return;
+    const int col0 = wg_col0 + wave * (16 * CT);
+    const bool active = col0 < ncols;  // W > 1: a wave past the last column still loads and waits with the others
     const int last_col = min(ncols, col0 + 16 * CT) - 1;
     const int max_qpos = start + last_col / g;
     const int kv_len = start + n_new;
     const int k_begin = n_splits > 1 ? split * split_size : 0;
-    const int k_end = n_splits > 1 ? min(max_qpos + 1, k_begin + split_size) : max_qpos + 1;
+    const int k_end = !active ? 0 : n_splits > 1 ? min(max_qpos + 1, k_begin + split_size) : max_qpos + 1;
     const int kb_last = (kv_len - 1) & ~31;  // the last block that has a page
     // below this key index no column of this wave masks anything (columns are ordered by token)
     const int min_lim = min(start + col0 / g + 1, k_end);
@@ -192,10 +197,24 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(
                 s[j] = (interior || key < lim) ? v : -INFINITY;
                 mx = fmaxf(mx, s[j]);
             }
-            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-            const float m_new = fmaxf(m_run[ct], mx);
-            const float m_use = m_new == -INFINITY ? 0.f : m_new;
+            // The running maximum is only a reference point for the exponentials, shared by the four lanes of
+            // a column; it is brought up to the true maximum (an exchange between those lanes, and a
+            // rescale of what was summed) only when some score of the block lies more than 2^8 above it,
+            // which after the first blocks of a row is rare.  Weights stay below 2^8 and their rounding to
+            // bfloat16 is relative, so nothing is lost by a reference that lags.
+            if (__any(mx > m_run[ct] + 8.0f)) {
+                mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+                const float m_new = fmaxf(m_run[ct], mx);
+                const float corr = __builtin_amdgcn_exp2f(m_run[ct] - (m_new == -INFINITY ? 0.f : m_new));
+                l_run[ct] *= corr;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+                    oacc[dt][ct][0] *= corr; oacc[dt][ct][1] *= corr; oacc[dt][ct][2] *= corr; oacc[dt][ct][3] *= corr;
+                }
+                m_run[ct] = m_new;
+            }
+            const float m_use = m_run[ct] == -INFINITY ? 0.f : m_run[ct];
             float p[8], psum = 0.f;
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
@@ -203,16 +222,7 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(
                 psum += p[j];
             }
             pf[ct].u = make_uint4(pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7]));
-            if (__any(m_new > m_run[ct])) {  // the running maximum moved for some column: rescale what was summed
-                const float corr = __builtin_amdgcn_exp2f(m_run[ct] - m_use);
-                l_run[ct] *= corr;
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt) {
-                    oacc[dt][ct][0] *= corr; oacc[dt][ct][1] *= corr; oacc[dt][ct][2] *= corr; oacc[dt][ct][3] *= corr;
-                }
-            }
             l_run[ct] += psum;
-            m_run[ct] = m_new;
         }
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
@@ -221,19 +231,88 @@ __global__ __launch_bounds__(64) void attn_mfma_kernel(
                 oacc[dt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b.v[dt].v, pf[ct].v, oacc[dt][ct], 0, 0, 0);
     };
 
-    // two register buffers: while one block is used, the next one's loads are in flight.  Addresses past
-    // the last block are clamped to it, and such a block is dropped in use_block.
-    KvBlock<DT> b0, b1;
-    if (k_begin < k_end) load_block<DT>(b0, min(k_begin, kb_last), bt, k_pool, v_pool, nkv, kvh, c, gq);
-    for (int kb = k_begin; kb < k_end; kb += 64) {
-        load_block<DT>(b1, min(kb + 32, kb_last), bt, k_pool, v_pool, nkv, kvh, c, gq);
-        __builtin_amdgcn_sched_barrier(0);
-        use_block(b0, kb);
-        __builtin_amdgcn_sched_barrier(0);
-        load_block<DT>(b0, min(kb + 64, kb_last), bt, k_pool, v_pool, nkv, kvh, c, gq);
-        __builtin_amdgcn_sched_barrier(0);
-        use_block(b1, kb + 32);
-        __builtin_amdgcn_sched_barrier(0);
+    if constexpr (W == 1) {
+        // two register buffers: while one block is used, the next one's loads are in flight.  Addresses past
+        // the last block are clamped to it, and such a block is dropped in use_block.
+        KvBlock<DT> b0, b1;
+        if (k_begin < k_end) load_block<DT>(b0, min(k_begin, kb_last), bt, k_pool, v_pool, nkv, kvh, c, gq);
+        for (int kb = k_begin; kb < k_end; kb += 64) {
+            load_block<DT>(b1, min(kb + 32, kb_last), bt, k_pool, v_pool, nkv, kvh, c, gq);
+            __builtin_amdgcn_sched_barrier(0);
+            use_block(b0, kb);
+            __builtin_amdgcn_sched_barrier(0);
+            load_block<DT>(b0, min(kb + 64, kb_last), bt, k_pool, v_pool, nkv, kvh, c, gq);
+            __builtin_amdgcn_sched_barrier(0);
+            use_block(b1, kb + 32);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    } else {
+        // The workgroup's waves walk the keys of its last column together.  A block goes global memory ->
+        // registers (one block ahead) -> one of two LDS buffers -> each wave's operand registers.  Key rows
+        // are stored in the order the score tiles want them (tile tt, lane column c <-> key
+        // 8*(c/4) + 4*tt + c%4), so that sixteen lanes read sixteen consecutive LDS rows; the row
+        // strides (D*2 + 16 and 80 bytes) put those on distinct banks.
+        constexpr int KROW = D + 8, VROW = 40;                    // elements
+        constexpr int KPIECES = 4 * D, THREADS = 64 * W;          // 16-byte pieces of a 32-key block
+        constexpr int PER = (KPIECES + THREADS - 1) / THREADS;
+        __shared__ __attribute__((aligned(16))) bf16_t kbuf[2][32 * KROW];
+        __shared__ __attribute__((aligned(16))) bf16_t vbuf[2][D * VROW];
+        const int tid = threadIdx.x;
+        const int wg_last_col = min(ncols, wg_col0 + 16 * CT * W) - 1;
+        const int k_end_wg = start + wg_last_col / g + 1;
+        uint4 gk[PER], gv[PER];
+        auto gload = [&](int kb) {
+            kb = min(kb, kb_last);
+            const long page = bt[kb >> 6];
+            const int in_page = kb & 63;
+            const bf16_t* kpage = k_pool + (page * nkv + kvh) * (long)(PTA_PAGE * D);
+            const bf16_t* vpage = v_pool + (page * nkv + kvh) * (long)(PTA_PAGE * D);
+#pragma unroll
+            for (int j = 0; j < PER; ++j) {
+                const int p = min(tid + j * THREADS, KPIECES - 1);
+                gk[j] = *reinterpret_cast<const uint4*>(kpage + (long)(in_page + p / CHUNKS) * D + (p % CHUNKS) * 8);
+                gv[j] = *reinterpret_cast<const uint4*>(vpage + (long)(p >> 2) * PTA_PAGE + in_page + (p & 3) * 8);
+            }
+        };
+        auto sstore = [&](int buf) {
+#pragma unroll
+            for (int j = 0; j < PER; ++j) {
+                const int p = tid + j * THREADS;
+                if (p < KPIECES) {
+                    const int kk = p / CHUNKS;  // key of the block -> its row in operand order
+                    const int row = ((kk & 7) >> 2) * 16 + 4 * (kk >> 3) + (kk & 3);
+                    *reinterpret_cast<uint4*>(&kbuf[buf][row * KROW + (p % CHUNKS) * 8]) = gk[j];
+                    *reinterpret_cast<uint4*>(&vbuf[buf][(p >> 2) * VROW + (p & 3) * 8]) = gv[j];
+                }
+            }
+        };
+        auto lfetch = [&](KvBlock<DT>& b, int buf) {
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+                for (int ds = 0; ds < DS; ++ds)
+                    b.k[tt][ds].u = *reinterpret_cast<const uint4*>(
+                        &kbuf[buf][(tt * 16 + c) * KROW + min(ds * 4 + gq, CHUNKS - 1) * 8]);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+                b.v[dt].u = *reinterpret_cast<const uint4*>(&vbuf[buf][(dt * 16 + c) * VROW + gq * 8]);
+        };
+        gload(0);
+        sstore(0);
+        __syncthreads();
+        for (int kb = 0; kb < k_end_wg; kb += 32) {
+            const int buf = (kb >> 5) & 1;
+            gload(kb + 32);
+            __builtin_amdgcn_sched_barrier(0);
+            if (kb < k_end) {
+                KvBlock<DT> b;
+                lfetch(b, buf);
+                use_block(b, kb);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            sstore(buf ^ 1);
+            __syncthreads();
+        }
     }
 
 #pragma unroll
@@ -307,14 +386,14 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(bf16_t* __restrict__ o
     }
 }
 
-template <int DT, int CT>
+template <int DT, int CT, int W = 1>
 static void launch_attn(bf16_t* out, float* po, float* pm, float* pl, const bf16_t* q, const bf16_t* k_pool,
                         const bf16_t* v_pool, const int* block_table, int bt_stride, const int* cu_tokens,
                         const int* seq_start, const float* slopes, int n_seqs, int max_new, int nh, int nkv, float scale,
                         int split_size, int n_splits, hipStream_t s) {
     const int g = nh / nkv;
-    const dim3 grid((max_new * g + 16 * CT - 1) / (16 * CT), nkv, n_seqs * n_splits);
-    hipLaunchKernelGGL((attn_mfma_kernel<DT, CT>), grid, dim3(64), 0, s, out, po, pm, pl, q, k_pool, v_pool, block_table,
+    const dim3 grid((max_new * g + 16 * CT * W - 1) / (16 * CT * W), nkv, n_seqs * n_splits);
+    hipLaunchKernelGGL((attn_mfma_kernel<DT, CT, W>), grid, dim3(64 * W), 0, s, out, po, pm, pl, q, k_pool, v_pool, block_table,
                        bt_stride, cu_tokens, seq_start, slopes, nh, nkv, scale * PTA_LOG2E,
                        PTA_LOG2E / sqrtf((float)(DT * 16)), split_size, n_splits);
 }
@@ -336,26 +415,27 @@ extern "C" int pta_attn_mfma(void* out, const void* q, const void* k_pool, const
                     ((uintptr_t)out % 8) == 0, "attn_mfma: pointers must be 16-byte aligned");
     hipStream_t s = (hipStream_t)stream;
     // one token per sequence (decode): one column tile per wave, so that the tiles of a KV head run side
-    // by side; prompts: several tiles per wave, so that a key block is loaded once for all of them
+    // by side.  Prompts: four waves of two column tiles share each key block through LDS (head sizes up to
+    // 128; beyond, one wave per workgroup).  Measured at Falcon-7B sizes (2,048 tokens, 71 heads on one KV
+    // head), one wave per workgroup: 2 tiles 148 us a layer, 4 tiles 195 us, 1 tile 270 us (fewer tiles
+    // balance the causal triangle better, more tiles re-read keys less).  PTA_ATTN_CT and PTA_ATTN_W
+    // override for tuning.
     const bool narrow = max_new == 1;
-    // column tiles per wave for prompts.  Measured at Falcon-7B sizes (2,048 tokens, 71 heads on one KV
-    // head): 2 tiles 148 us a layer, 4 tiles 195 us, 1 tile 270 us: fewer tiles balance the causal
-    // triangle better, more tiles re-read keys less.  PTA_ATTN_CT overrides for tuning.
     static const int ct_env = getenv("PTA_ATTN_CT") ? atoi(getenv("PTA_ATTN_CT")) : 2;
-#define PTA_ATTN_CASE(DT_, CT_)                                                                                     \
-    case DT_:                                                                                                       \
-        if (!narrow && ct_env == 2 && CT_ > 2)                                                                      \
-            launch_attn<DT_, 2>((bf16_t*)out, po, pm, pl, (const bf16_t*)q, (const bf16_t*)k_pool,                  \
-                                (const bf16_t*)v_pool, block_table, bt_stride, cu_tokens, seq_start, slopes, n_seqs, \
-                                max_new, nh, nkv, scale, split_size, n_splits, s);                                  \
-        else if (narrow || ct_env == 1)                                                                             \
-            launch_attn<DT_, 1>((bf16_t*)out, po, pm, pl, (const bf16_t*)q, (const bf16_t*)k_pool,                  \
-                                (const bf16_t*)v_pool, block_table, bt_stride, cu_tokens, seq_start, slopes, n_seqs, \
-                                max_new, nh, nkv, scale, split_size, n_splits, s);                                  \
-        else                                                                                                        \
-            launch_attn<DT_, CT_>((bf16_t*)out, po, pm, pl, (const bf16_t*)q, (const bf16_t*)k_pool,                \
-                                  (const bf16_t*)v_pool, block_table, bt_stride, cu_tokens, seq_start, slopes,      \
-                                  n_seqs, max_new, nh, nkv, scale, split_size, n_splits, s);                        \
+    static const int w_env = getenv("PTA_ATTN_W") ? atoi(getenv("PTA_ATTN_W")) : 4;
+#define PTA_ATTN_ARGS                                                                                              \
+    (bf16_t*)out, po, pm, pl, (const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_table, bt_stride, \
+        cu_tokens, seq_start, slopes, n_seqs, max_new, nh, nkv, scale, split_size, n_splits, s
+#define PTA_ATTN_CASE(DT_, CT_)                                                                   \
+    case DT_:                                                                                     \
+        if (narrow || ct_env == 1) launch_attn<DT_, 1, 1>(PTA_ATTN_ARGS);                         \
+        else if (w_env == 4 && DT_ <= 8) {                                                        \
+            if constexpr (DT_ <= 8) {                                                             \
+                if (ct_env == 2 || CT_ < 2) launch_attn<DT_, (CT_ < 2 ? CT_ : 2), 4>(PTA_ATTN_ARGS); \
+                else launch_attn<DT_, CT_, 4>(PTA_ATTN_ARGS);                                     \
+            }                                                                                     \
+        } else if (ct_env == 2 && CT_ > 2) launch_attn<DT_, 2, 1>(PTA_ATTN_ARGS);                 \
+        else launch_attn<DT_, CT_, 1>(PTA_ATTN_ARGS);                                             \
         break;
     switch (d / 16) {
         PTA_ATTN_CASE(1, 4)
@@ -371,6 +451,7 @@ extern "C" int pta_attn_mfma(void* out, const void* q, const void* k_pool, const
             return pta_fail("attn_mfma: head size %d is not built", d);
     }
 #undef PTA_ATTN_CASE
+#undef PTA_ATTN_ARGS
     int rc = pta_check_launch("attn_mfma");
     if (rc) return rc;
     if (n_splits > 1) {
