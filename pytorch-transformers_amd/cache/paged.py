@@ -8,7 +8,9 @@ different shapes (``HybridCache`` :1626-1638) and fixed-size state lives in
 ``[layers, batch, ...]`` tables (``MambaCache`` :1813-1828).  A batch row is a
 sequence's place for the whole call and its true length is implied by padding.
 
-Here a sequence holds a *slot* (an integer) with an explicit length.  Each
+Here a sequence holds a *slot* (an integer) with an explicit length.  The bookkeeping (free lists,
+page lists, lengths) lives in the host runtime (``csrc/host/runtime_host.cpp``); this class owns the
+device tensors and is the runtime's Python face.  Each
 layer group owns a pool of pages of ``page_size`` tokens; a slot's keys and
 values are the pages its page list names, in order, so the position of a key is
 its index in the slot.  Slots and pages go back to free lists when a sequence
@@ -21,10 +23,12 @@ The K pool has the layout ``[layer, page, kv_head, page_size, head_dim]``, the V
 """
 from __future__ import annotations
 
+import ctypes
 from typing import Dict, List, Optional, Sequence
 
 import torch
 
+from .. import host
 from ..engine.spec import CACHE_FULL, CACHE_STATE, CACHE_WINDOW, CacheGroupSpec
 
 PAGE_SIZE = 64
@@ -38,42 +42,6 @@ class CacheFull(CacheError):
     """The pool has too few free pages (or no free slot) for what a step needs."""
 
 
-class _FreeList:
-    """Integers 0..n-1, handed out lowest first; returning one twice is an error."""
-
-    def __init__(self, n: int, what: str):
-        self.n = n
-        self.what = what
-        self._free = list(range(n - 1, -1, -1))  # pop() gives the lowest
-        self._held = [False] * n
-
-    def __len__(self):
-        return len(self._free)
-
-    def take(self) -> int:
-        if not self._free:
-            raise CacheFull(f"no free {self.what} (all {self.n} are held)")
-        i = self._free.pop()
-        self._held[i] = True
-        return i
-
-    def give(self, i: int) -> None:
-        if not (0 <= i < self.n):
-            raise CacheError(f"{self.what} {i} does not exist (0..{self.n - 1})")
-        if not self._held[i]:
-            raise CacheError(f"{self.what} {i} is freed twice (or was never handed out)")
-        self._held[i] = False
-        self._free.append(i)
-        # keep "lowest first" so that reuse is immediate and deterministic
-        self._free.sort(reverse=True)
-
-    def held(self, i: int) -> bool:
-        return 0 <= i < self.n and self._held[i]
-
-    def held_count(self) -> int:
-        return self.n - len(self._free)
-
-
 class _Group:
     """Storage of one layer group."""
 
@@ -82,7 +50,8 @@ class _Group:
         self.page_size = page_size
         self.k = self.v = None
         self.state: Optional[torch.Tensor] = None
-        self.pages: Optional[_FreeList] = None
+        self.paged = spec.kind == CACHE_FULL
+        self.index = -1  # among the paged groups, as the host runtime counts them
         if spec.kind == CACHE_FULL:
             # values are held transposed inside a page so that the attention kernels read eight
             # consecutive positions of one feature in one load
@@ -90,7 +59,6 @@ class _Group:
                                  dtype=dtype, device=device)
             self.v = torch.zeros((spec.num_layers, num_pages, spec.kv_heads, spec.head_dim, page_size),
                                  dtype=dtype, device=device)
-            self.pages = _FreeList(num_pages, f"page of cache group {spec.name!r}")
         elif spec.kind == CACHE_STATE:
             sd = spec.state_dtype or torch.float32
             self.state = torch.zeros((spec.num_layers, max_slots, *spec.state_shape), dtype=sd, device=device)
@@ -101,12 +69,9 @@ class _Group:
         else:
             raise CacheError(f"cache group {spec.name!r}: unknown kind {spec.kind!r}")
 
-    def pages_for(self, length: int) -> int:
-        return (length + self.page_size - 1) // self.page_size if self.pages is not None else 0
-
 
 class PagedCache:
-    """Slots, their lengths and page lists, and the device storage of every group."""
+    """Slots, their lengths and page lists (kept by the host runtime), and the device storage of every group."""
 
     def __init__(self, groups: Sequence[CacheGroupSpec], max_tokens: int, dtype: torch.dtype, device,
                  *, max_slots: Optional[int] = None, page_size: int = PAGE_SIZE):
@@ -120,81 +85,88 @@ class PagedCache:
         self.device = torch.device(device)
         self.groups: Dict[str, _Group] = {
             g.name: _Group(g, self.num_pages, self.max_slots, page_size, dtype, self.device) for g in groups}
-        self._slots = _FreeList(self.max_slots, "slot")
-        self._length: List[int] = [0] * self.max_slots
-        self._pages: Dict[str, List[List[int]]] = {
-            name: [[] for _ in range(self.max_slots)] for name, g in self.groups.items() if g.pages is not None}
+        self._paged = [name for name, g in self.groups.items() if g.paged]
+        for i, name in enumerate(self._paged):
+            self.groups[name].index = i
+        self._lib = host.load()
+        self._h = self._lib.ptah_cache_new(self.max_slots, page_size, len(self._paged),
+                                           host.int_array([self.num_pages] * len(self._paged)))
+        if not self._h:
+            raise CacheError(host.last_error())
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h:
+            self._lib.ptah_cache_delete(h)
+
+    def _raise(self, rc: int):
+        msg = host.last_error()
+        for i, name in enumerate(self._paged):  # the runtime knows groups by number
+            msg = msg.replace(f"group {i} ", f"group {name!r} ")
+        raise (CacheFull if rc == host.ERR_FULL else CacheError)(msg)
+
+    @property
+    def handle(self):
+        """The host runtime's handle of this cache (for ``plan_step``)."""
+        return self._h
 
     # slots -------------------------------------------------------------
     def alloc(self) -> int:
-        slot = self._slots.take()
-        self._length[slot] = 0
+        slot = self._lib.ptah_alloc(self._h)
+        if slot < 0:
+            self._raise(host.ERR_FULL)
         for g in self.groups.values():
             if g.state is not None:
                 g.state[:, slot].zero_()
         return slot
 
     def free(self, slot: int) -> None:
-        self._check(slot)
-        for name, table in self._pages.items():
-            pool = self.groups[name].pages
-            for p in table[slot]:
-                pool.give(p)
-            table[slot] = []
-        self._length[slot] = 0
-        self._slots.give(slot)
-
-    def _check(self, slot: int) -> None:
-        if not self._slots.held(slot):
-            raise CacheError(f"slot {slot} is not allocated")
+        rc = self._lib.ptah_free(self._h, int(slot))
+        if rc:
+            self._raise(rc)
 
     def length(self, slot: int) -> int:
-        self._check(slot)
-        return self._length[slot]
+        n = self._lib.ptah_length(self._h, int(slot))
+        if n < 0:
+            self._raise(host.ERR_CACHE)
+        return n
 
     def live_slots(self) -> List[int]:
-        return [s for s in range(self.max_slots) if self._slots.held(s)]
+        return [s for s in range(self.max_slots) if self._lib.ptah_is_live(self._h, s)]
 
     def free_pages(self, group: Optional[str] = None) -> int:
-        names = [group] if group is not None else list(self._pages)
-        return min((len(self.groups[n].pages) for n in names), default=self.num_pages)
+        names = [group] if group is not None else self._paged
+        return min((self._lib.ptah_free_pages(self._h, self.groups[n].index) for n in names), default=self.num_pages)
 
     def free_slots(self) -> int:
-        return len(self._slots)
+        return self._lib.ptah_free_slots(self._h)
 
     # growth ------------------------------------------------------------
     def reserve(self, slots: Sequence[int], new_tokens: Sequence[int]) -> None:
         """Give every slot the pages that ``new_tokens`` more tokens need; all or nothing."""
-        if len(set(slots)) != len(slots):
-            raise CacheError(f"a slot appears twice in one step: {list(slots)}")
-        for s in slots:
-            self._check(s)
-        for name, table in self._pages.items():
-            g = self.groups[name]
-            need = 0
-            for s, n in zip(slots, new_tokens):
-                need += max(0, g.pages_for(self._length[s] + n) - len(table[s]))
-            if need > len(g.pages):
-                raise CacheFull(
-                    f"cache group {name!r} needs {need} more pages of {self.page_size} tokens for this step, "
-                    f"{len(g.pages)} of {g.pages.n} are free")
-        for name, table in self._pages.items():
-            g = self.groups[name]
-            for s, n in zip(slots, new_tokens):
-                while len(table[s]) < g.pages_for(self._length[s] + n):
-                    table[s].append(g.pages.take())
+        rc = self._lib.ptah_reserve(self._h, len(slots), host.int_array([int(s) for s in slots]),
+                                    host.int_array([int(n) for n in new_tokens]))
+        if rc:
+            self._raise(rc)
 
     def commit(self, slots: Sequence[int], new_tokens: Sequence[int]) -> None:
         """The step has written ``new_tokens`` tokens of every slot."""
-        for s, n in zip(slots, new_tokens):
-            self._length[s] += n
+        rc = self._lib.ptah_commit(self._h, len(slots), host.int_array([int(s) for s in slots]),
+                                   host.int_array([int(n) for n in new_tokens]))
+        if rc:
+            self._raise(rc)
 
     def page_list(self, group: str, slot: int) -> List[int]:
-        self._check(slot)
-        return self._pages[group][slot]
+        gi = self.groups[group].index
+        n = self._lib.ptah_page_count(self._h, gi, int(slot))
+        if n < 0:
+            self._raise(host.ERR_CACHE)
+        out = (ctypes.c_int * max(1, n))()
+        self._lib.ptah_pages(self._h, gi, int(slot), out)
+        return list(out[:n])
 
     def paged_groups(self) -> List[str]:
-        return list(self._pages)
+        return list(self._paged)
 
     # storage -----------------------------------------------------------
     def kv_layer(self, group: str, layer: int):
@@ -213,20 +185,6 @@ class PagedCache:
 
     def check_consistent(self) -> None:
         """Every page is either free or in exactly one live slot's list; used by tests and debug runs."""
-        for name, table in self._pages.items():
-            g = self.groups[name]
-            seen = {}
-            for s in range(self.max_slots):
-                if table[s] and not self._slots.held(s):
-                    raise CacheError(f"freed slot {s} still lists pages {table[s]} in group {name!r}")
-                if self._slots.held(s) and len(table[s]) < g.pages_for(self._length[s]):
-                    raise CacheError(f"slot {s} has length {self._length[s]} but only {len(table[s])} pages")
-                for p in table[s]:
-                    if p in seen:
-                        raise CacheError(f"page {p} of group {name!r} is held by slots {seen[p]} and {s}")
-                    if not g.pages.held(p):
-                        raise CacheError(f"page {p} of group {name!r} is in slot {s}'s list and in the free list")
-                    seen[p] = s
-            if len(seen) != g.pages.held_count():
-                raise CacheError(
-                    f"group {name!r}: {g.pages.held_count()} pages are marked held, {len(seen)} are in slot lists")
+        rc = self._lib.ptah_check(self._h)
+        if rc:
+            self._raise(rc)

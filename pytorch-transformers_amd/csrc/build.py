@@ -1,4 +1,5 @@
-"""Compile the HIP sources in this folder into ``libpta_kernels.so`` for gfx950.
+"""Compile the HIP sources in this folder into ``libpta_kernels.so`` for gfx950, and the host runtime
+under ``host/`` (plain C++: slots, page lists, step layout) into ``libpta_host.so``.
 
 ``hipcc`` cross-compiles without a GPU.  Each ``.hip`` file becomes an object
 (in parallel), then all are linked.  The library lies next to the sources when
@@ -81,6 +82,79 @@ def find_library(require_current: bool = True):
     return None
 
 
+# ---- the host runtime: plain C++, no GPU code, needed on machines without a GPU too -------------
+HOST_LIB_NAME = "libpta_host.so"
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-Wall"]
+
+
+def host_sources():
+    return sorted(glob.glob(os.path.join(HERE, "host", "*.cpp")))
+
+
+def host_hash() -> str:
+    h = hashlib.sha256()
+    for p in host_sources():
+        h.update(os.path.basename(p).encode())
+        with open(p, "rb") as f:
+            h.update(f.read())
+    h.update(" ".join(HOST_FLAGS).encode())
+    return h.hexdigest()
+
+
+def host_lib_dirs():
+    out = [HERE]
+    try:
+        user = str(os.getuid())
+    except AttributeError:
+        user = "user"
+    out.append(os.path.join(tempfile.gettempdir(), f"pta_host_{user}_{host_hash()[:12]}"))
+    return out
+
+
+def find_host_library(require_current: bool = True):
+    want = host_hash()
+    for d in host_lib_dirs():
+        lib = os.path.join(d, HOST_LIB_NAME)
+        if not os.path.isfile(lib):
+            continue
+        if not require_current:
+            return lib
+        try:
+            with open(lib + ".hash") as f:
+                if f.read().strip() == want:
+                    return lib
+        except OSError:
+            pass
+    return None
+
+
+def host_compiler() -> str:
+    for cand in (os.environ.get("CXX"), shutil.which("g++"), shutil.which("c++"), shutil.which("clang++"),
+                 "/opt/rocm/llvm/bin/clang++"):
+        if cand and (os.path.isfile(cand) or shutil.which(cand)):
+            return cand
+    raise RuntimeError("no C++ compiler found for the host runtime (looked at $CXX, g++, c++, clang++)")
+
+
+def build_host(verbose: bool = True) -> str:
+    """Compile the host runtime (always) and return the library's path."""
+    target_dir = next((d for d in host_lib_dirs() if _writable(d)), None)
+    if target_dir is None:
+        raise RuntimeError(f"no writable folder for {HOST_LIB_NAME}: tried {host_lib_dirs()}")
+    lib = os.path.join(target_dir, HOST_LIB_NAME)
+    tmp = lib + f".tmp{os.getpid()}"
+    cmd = [host_compiler(), *HOST_FLAGS, "-o", tmp, *host_sources()]
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"host runtime failed to compile:\n{' '.join(cmd)}\n{r.stdout}")
+    os.replace(tmp, lib)
+    with open(lib + ".hash", "w") as f:
+        f.write(host_hash() + "\n")
+    if verbose:
+        print(f"[pta build] host runtime {lib}", file=sys.stderr, flush=True)
+    return lib
+
+
 def hipcc() -> str:
     for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
         if cand and os.path.isfile(cand):
@@ -137,4 +211,5 @@ def build(verbose: bool = True, jobs: int | None = None) -> str:
 
 
 if __name__ == "__main__":
+    print(build_host())
     print(build())

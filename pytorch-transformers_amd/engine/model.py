@@ -218,13 +218,9 @@ class CausalLM:
     def make_context(self, plan: StepPlan, cache: PagedCache):
         """Upload a plan's arrays in one buffer and wrap the views."""
         n, M, R = plan.n_seqs, plan.n_tokens, int(plan.logit_rows.shape[0])
-        pieces = [plan.token_ids, plan.token_seq, plan.token_pos, plan.cu_tokens,
-                  np.asarray(plan.starts, dtype=np.int32), np.asarray(plan.slots, dtype=np.int32), plan.logit_rows]
         names = list(plan.block_tables)
-        pieces += [plan.block_tables[g].reshape(-1) for g in names]
-        sizes = [int(p.shape[0]) for p in pieces]
-        dev = torch.from_numpy(np.concatenate(pieces)).to(self.device)
-        views = torch.split(dev, sizes)
+        dev = torch.from_numpy(plan.buffer).to(self.device)  # the host runtime laid the pieces out in one buffer
+        views = torch.split(dev, plan.sizes)
         tables = {g: views[7 + i].view(plan.block_tables[g].shape) for i, g in enumerate(names)}
         ctx = StepContext(dtype=self.dtype, device=self.device, n_seqs=n, n_tokens=M, token_seq=views[1],
                           token_pos=views[2], cu_tokens=views[3], seq_start=views[4], seq_slot=views[5],

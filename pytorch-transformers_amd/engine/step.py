@@ -8,6 +8,7 @@ rows.  All arrays go to the device in one int32 buffer.
 """
 from __future__ import annotations
 
+import ctypes
 import dataclasses
 from typing import Dict, List, Optional, Sequence, Union
 
@@ -32,6 +33,10 @@ class StepPlan:
     logit_rows: np.ndarray  # [R] indices into the M tokens
     rows_per_seq: List[int]
     block_tables: Dict[str, np.ndarray]  # group -> [n, pages]
+    #: all of the arrays above in one int32 buffer, in the order token_ids, token_seq, token_pos, cu_tokens,
+    #: starts, slots, logit_rows, then one page table per group; ``sizes`` are the pieces' lengths
+    buffer: Optional[np.ndarray] = None
+    sizes: Optional[List[int]] = None
 
     @property
     def n_seqs(self) -> int:
@@ -70,41 +75,55 @@ def normalize_want(want: Want, new_tokens: Sequence[int]) -> List[List[int]]:
     return want
 
 
+_WANT_MODES = {"none": 0, "last": 1, "all": 2}
+
+
 def plan_step(cache, slots: Sequence[int], tokens: Sequence[Sequence[int]], want: Want, vocab_size: int) -> StepPlan:
-    """Check a step's arguments, reserve cache pages for it and lay its arrays out."""
+    """Check a step's arguments, reserve cache pages for it and lay its arrays out (in the host runtime)."""
+    from .. import host
+    from ..cache.paged import CacheError, CacheFull
+
     slots = [int(s) for s in slots]
     if len(slots) == 0:
         raise StepError("a step needs at least one sequence")
     if len(tokens) != len(slots):
         raise StepError(f"{len(slots)} slots but {len(tokens)} token lists")
-    new_tokens = [len(t) for t in tokens]
-    for i, n in enumerate(new_tokens):
-        if n == 0:
-            raise StepError(f"sequence {i} (slot {slots[i]}) brings no tokens")
-    flat = np.concatenate([np.asarray(t, dtype=np.int64).reshape(-1) for t in tokens])
-    bad = np.nonzero((flat < 0) | (flat >= vocab_size))[0]
-    if bad.size:
-        raise StepError(f"token id {int(flat[bad[0]])} is outside the vocabulary [0, {vocab_size})")
-    wanted = normalize_want(want, new_tokens)
-
-    cache.reserve(slots, new_tokens)  # raises for unknown or repeated slots and for a full pool
-    starts = [cache.length(s) for s in slots]
-
     n = len(slots)
-    cu = np.zeros(n + 1, dtype=np.int32)
-    cu[1:] = np.cumsum(new_tokens)
-    token_seq = np.repeat(np.arange(n, dtype=np.int32), new_tokens)
-    token_pos = np.concatenate([np.arange(s, s + k, dtype=np.int32) for s, k in zip(starts, new_tokens)])
-    rows = [int(cu[i]) + int(p) for i, w in enumerate(wanted) for p in w]
-    tables = {}
-    for g in cache.paged_groups():
-        lists = [cache.page_list(g, s) for s in slots]
-        width = max(1, max(len(l) for l in lists))
-        t = np.zeros((n, width), dtype=np.int32)
-        for i, l in enumerate(lists):
-            t[i, :len(l)] = l
-        tables[g] = t
-    return StepPlan(slots=slots, new_tokens=new_tokens, starts=starts, token_ids=flat.astype(np.int32),
-                    token_seq=token_seq, token_pos=token_pos, cu_tokens=cu,
-                    logit_rows=np.asarray(rows, dtype=np.int32), rows_per_seq=[len(w) for w in wanted],
-                    block_tables=tables)
+    new_tokens = [len(t) for t in tokens]
+    flat = np.ascontiguousarray(np.concatenate([np.asarray(t, dtype=np.int64).reshape(-1) for t in tokens])
+                                if sum(new_tokens) else np.zeros(0, dtype=np.int64))
+    counts = places = None
+    if want is None or isinstance(want, str):
+        key = "none" if want is None else want
+        if key not in _WANT_MODES:
+            raise StepError(f"want must be 'last', 'all', 'none' or a list of places per sequence, got {want!r}")
+        mode = _WANT_MODES[key]
+    else:
+        want = [[int(p) for p in w] for w in want]
+        if len(want) != n:
+            raise StepError(f"want has {len(want)} entries for {n} sequences")
+        mode = 3
+        counts = host.int_array([len(w) for w in want])
+        places = host.int_array([p for w in want for p in w])
+    lib = host.load()
+    sizes = (ctypes.c_int * (7 + len(cache.paged_groups())))()
+    rc = lib.ptah_plan_step(cache.handle, n, host.int_array(slots), host.int_array(new_tokens),
+                            flat.ctypes.data_as(ctypes.POINTER(ctypes.c_longlong)), int(vocab_size), mode, counts,
+                            places, sizes)
+    if rc:
+        msg = host.last_error()
+        raise {host.ERR_STEP: StepError, host.ERR_FULL: CacheFull}.get(rc, CacheError)(msg)
+    sizes = list(sizes)
+    total = sum(sizes)
+    buf = np.ctypeslib.as_array(lib.ptah_plan_data(cache.handle), shape=(total,)).copy()  # the runtime reuses its buffer
+    views = np.split(buf, np.cumsum(sizes)[:-1])
+    M, R = sizes[0], sizes[6]
+    rows = views[6]
+    if mode == 3:
+        rows_per_seq = [len(w) for w in want]
+    else:
+        rows_per_seq = [0] * n if mode == 0 else [1] * n if mode == 1 else list(new_tokens)
+    tables = {g: views[7 + i].reshape(n, -1) for i, g in enumerate(cache.paged_groups())}
+    return StepPlan(slots=slots, new_tokens=new_tokens, starts=views[4].tolist(), token_ids=views[0], token_seq=views[1],
+                    token_pos=views[2], cu_tokens=views[3], logit_rows=rows, rows_per_seq=rows_per_seq,
+                    block_tables=tables, buffer=buf, sizes=sizes)
