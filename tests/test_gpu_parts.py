@@ -305,3 +305,152 @@ def test_toy_architecture_with_a_state_mixer(tmp_path, dtype, rel):
                 assert seq == toks
     finally:
         unregister("toy-decay")
+
+
+# --- a second toy: a routed feed-forward and a position encoding of its own, both defined here ------------
+def _define_routed_toy():
+    from pytorch_transformers_amd.config.base import ModelConfig
+    from pytorch_transformers_amd.engine.spec import (CACHE_FULL, INIT_NORMAL, MATRIX, CacheGroupSpec, LayerCall, ModelSpec,
+                                                      TensorSpec)
+    from pytorch_transformers_amd.parts import (AttentionMixer, DenseFeedForward, Embedding, LayerNorm, NoPositions,
+                                                OutputHead, ParallelBlock, Part, SequentialBlock, register_part)
+
+    @dataclasses.dataclass
+    class RoutedConfig(ModelConfig):
+        model_type = "toy-routed"
+        vocab_size: int = 131
+        width: int = 64
+        experts: int = 3
+        heads: int = 4
+
+    class HarmonicPositions(NoPositions):
+        """Rotation with frequencies 1/(j+1) instead of a geometric ladder: another position encoding that
+        feeds the same seam (``rotation()``), read by the framework's rotary kernel unchanged."""
+
+        def __init__(self, head_dim):
+            self.inv_freq = (1.0 / torch.arange(1, head_dim // 2 + 1, dtype=torch.float32)).contiguous()
+
+        def to(self, device):
+            self.inv_freq = self.inv_freq.to(device)
+
+        def rotation(self):
+            return self.inv_freq, 1.0
+
+    class RoutedFeedForward(Part):
+        """Each token goes to the expert its router scores highest (scores and softmax in 32-bit), and the
+        expert's output is weighted by that probability.  Experts are the framework's dense feed-forwards."""
+
+        def __init__(self, name, width, experts):
+            self.name, self.width = name, width
+            self.experts = [DenseFeedForward(f"{name}.experts.{e}", width, 2 * width, bias=True) for e in range(experts)]
+
+        def tensor_specs(self):
+            return [TensorSpec(self.name + ".router.weight", (len(self.experts), self.width), MATRIX, INIT_NORMAL)]
+
+        def load(self, tensors):
+            self.router = tensors[self.name + ".router.weight"]
+
+        def children(self):
+            return tuple(self.experts)
+
+        def forward(self, x, ctx, add1=None, add2=None):
+            probs = torch.softmax(x.float() @ self.router.float().T, dim=-1)
+            gate, pick = probs.max(dim=-1)
+            out = torch.zeros_like(x, dtype=torch.float32)
+            for e, expert in enumerate(self.experts):
+                rows = torch.nonzero(pick == e).flatten()
+                if rows.numel():
+                    y = expert.forward(x.index_select(0, rows).contiguous(), ctx)
+                    out.index_copy_(0, rows, y.float() * gate[rows, None])
+            for a in (add1, add2):
+                if a is not None:
+                    out = out + a.float()
+            return out.to(x.dtype)
+
+    register_part("positions", "harmonic", HarmonicPositions, exist_ok=True)
+    register_part("feed_forward", "routed", RoutedFeedForward, exist_ok=True)
+
+    def build(cfg):
+        d = cfg.width // cfg.heads
+        blocks = [
+            ParallelBlock(AttentionMixer("t.h.0.attn", cfg.width, cfg.heads, 2, d, "grouped", False, HarmonicPositions(d)),
+                          RoutedFeedForward("t.h.0.moe", cfg.width, cfg.experts), LayerNorm("t.h.0.norm", cfg.width, 1e-5)),
+            SequentialBlock(AttentionMixer("t.h.1.attn", cfg.width, cfg.heads, cfg.heads, d, "interleaved", True, NoPositions()),
+                            RoutedFeedForward("t.h.1.moe", cfg.width, cfg.experts), LayerNorm("t.h.1.n1", cfg.width, 1e-5),
+                            LayerNorm("t.h.1.n2", cfg.width, 1e-5)),
+        ]
+        return ModelSpec(config=cfg, embedding=Embedding("t.embed", cfg.vocab_size, cfg.width), blocks=blocks,
+                         order=[LayerCall(0, "grouped", 0), LayerCall(1, "full", 0)],
+                         final_norm=LayerNorm("t.final", cfg.width, 1e-5),
+                         head=OutputHead("t.head", cfg.vocab_size, cfg.width, "t.embed.weight"),
+                         # the two layers keep different numbers of heads: a cache group each, pages of their own
+                         cache_groups=[CacheGroupSpec("grouped", CACHE_FULL, 1, 2, d),
+                                       CacheGroupSpec("full", CACHE_FULL, 1, cfg.heads, d)],
+                         supports_graphs=False)  # routing looks at the data on the host
+
+    return RoutedConfig, build
+
+
+def _plain_routed(cfg, w, ids):
+    T, H, nh = len(ids), cfg.width, cfg.heads
+    d = H // nh
+    x = w["t.embed.weight"][torch.as_tensor(ids)]
+    ln = lambda h, n: P.layer_norm(h, w[n + ".weight"], w[n + ".bias"], 1e-5)
+
+    def moe(h, p):
+        probs = torch.softmax(h @ w[p + ".router.weight"].T, dim=-1)
+        gate, pick = probs.max(dim=-1)
+        out = torch.zeros_like(h)
+        for t in range(T):
+            e = f"{p}.experts.{int(pick[t])}"
+            u = P.gelu(h[t] @ w[e + ".dense_h_to_4h.weight"].T + w[e + ".dense_h_to_4h.bias"])
+            out[t] = gate[t] * (u @ w[e + ".dense_4h_to_h.weight"].T + w[e + ".dense_4h_to_h.bias"])
+        return out
+
+    # layer 0: parallel, grouped rows (2 groups of 2 heads), rotation with harmonic frequencies
+    a = ln(x, "t.h.0.norm")
+    f = (a @ w["t.h.0.attn.query_key_value.weight"].T).view(T, 2, 4, d)
+    q, k, v = f[:, :, :2].reshape(T, nh, d), f[:, :, 2], f[:, :, 3]
+    cos, sin = P.rope_cos_sin(torch.arange(T), 1.0 / torch.arange(1, d // 2 + 1, dtype=torch.float32))
+    o = P.attention_scores_softmax(P.apply_rope(q, cos, sin), P.apply_rope(k, cos, sin), v)
+    x = x + (moe(a, "t.h.0.moe") + o @ w["t.h.0.attn.dense.weight"].T)
+    # layer 1: sequential, interleaved rows with bias, no positions
+    a = ln(x, "t.h.1.n1")
+    f = (a @ w["t.h.1.attn.query_key_value.weight"].T + w["t.h.1.attn.query_key_value.bias"]).view(T, nh, 3, d)
+    o = P.attention_scores_softmax(f[:, :, 0], f[:, :, 1], f[:, :, 2])
+    r = x + o @ w["t.h.1.attn.dense.weight"].T + w["t.h.1.attn.dense.bias"]
+    x = r + moe(ln(r, "t.h.1.n2"), "t.h.1.moe")
+    return ln(x, "t.final") @ w["t.embed.weight"].T
+
+
+def test_toy_architecture_with_routing_and_its_own_positions(tmp_path):
+    """A feed-forward with a router and experts and a position encoding that the framework does not have,
+    both defined in this file, registered, built, loaded and stepped through every schedule (32-bit, where a
+    token that changed its expert would show)."""
+    from safetensors.torch import load_file
+
+    from pytorch_transformers_amd import AutoModelForCausalLM
+    from pytorch_transformers_amd.config import register, unregister
+    from pytorch_transformers_amd.engine.replay import Replayer
+    from pytorch_transformers_amd.parts import registered_parts
+    from pytorch_transformers_amd.weights import write_random_model
+
+    RoutedConfig, build = _define_routed_toy()
+    assert "routed" in registered_parts("feed_forward") and "harmonic" in registered_parts("positions")
+    register("toy-routed", RoutedConfig, build, exist_ok=True)
+    try:
+        cfg = RoutedConfig()
+        folder = write_random_model(str(tmp_path / "routed"), cfg, seed=9, std=0.2, noise=0.1)
+        w = {k: v.double() for k, v in load_file(f"{folder}/model.safetensors").items()}
+        assert sum(".experts." in k for k in w) == 2 * cfg.experts * 4 and "t.h.0.moe.router.weight" in w
+        model = AutoModelForCausalLM.from_pretrained(folder, dtype="float32")
+        reqs = helpers.make_requests(cfg.vocab_size, [11, 40, 70, 5], seed=4)
+        want = {rid: _plain_routed(cfg, w, toks).float() for rid, toks in reqs.items()}
+        rp = Replayer(model, 1024, max_slots=4)
+        for name, records in (("whole", helpers.schedule_whole(reqs)), ("tail", helpers.schedule_tail(reqs, 16)),
+                              ("batches", helpers.schedule_batches(reqs, 3))):
+            got = helpers.run_schedule(rp, records)
+            for rid in reqs:
+                helpers.assert_close(got[rid], want[rid], 5e-5, f"routed toy {name} {rid}")
+    finally:
+        unregister("toy-routed")
