@@ -1,0 +1,67 @@
+"""Falcon configurations drawn at random (fixed seeds) against the plain implementation (GPU).
+
+Sizes the tiny and the published configurations do not hit: head sizes from 16 to 256 that are and are not
+built for the matrix cores, head counts and groups that are no power of two, widths that are no multiple
+of 64, prime vocabularies, every norm arrangement and fused-row order the configuration allows.
+"""
+import os
+import random
+
+import pytest
+import torch
+
+import helpers
+from helpers import REL_BF16, REL_F32
+
+pytestmark = pytest.mark.gpu
+
+HEAD_SIZES = [16, 24, 32, 40, 48, 64, 80, 96, 112, 128, 256]
+VOCABS = [97, 211, 1009, 4099]
+
+
+def draw(seed: int) -> dict:
+    r = random.Random(seed)
+    d = r.choice(HEAD_SIZES)
+    new_arch = r.random() < 0.5
+    alibi = r.random() < 0.3
+    if new_arch:
+        nkv = r.choice([1, 2, 3])
+        nh = nkv * r.choice([1, 2, 3, 5])
+        extra = dict(new_decoder_architecture=True, num_kv_heads=nkv, parallel_attn=True,
+                     num_ln_in_parallel_attn=r.choice([1, 2]))
+    else:
+        nh = r.choice([1, 2, 3, 5, 7, 9])
+        extra = dict(new_decoder_architecture=False, multi_query=r.random() < 0.5, parallel_attn=r.random() < 0.6)
+    cfg = dict(model_type="falcon", num_hidden_layers=r.choice([1, 2, 3]), hidden_size=nh * d, num_attention_heads=nh,
+               ffn_hidden_size=r.choice([nh * d * 2 + 8, nh * d * 3, 200]), vocab_size=r.choice(VOCABS),
+               rope_theta=r.choice([10000.0, 500042.0]), max_position_embeddings=1024,
+               layer_norm_epsilon=r.choice([1e-5, 1e-6]), bias=r.random() < 0.5, alibi=alibi,
+               tie_word_embeddings=r.random() < 0.7, initializer_range=0.02, **extra)
+    if not alibi and r.random() < 0.3:
+        cfg["rope_scaling"] = {"rope_type": "linear", "factor": r.choice([2.0, 4.0])}
+    return cfg
+
+
+@pytest.mark.parametrize("seed", list(range(24)))
+def test_random_configuration_matches_plain(tmp_path, seed):
+    from pytorch_transformers_amd import AutoModelForCausalLM
+    from pytorch_transformers_amd.config import AutoConfig
+    from pytorch_transformers_amd.engine.replay import Replayer
+    from pytorch_transformers_amd.weights import write_random_model
+
+    raw = draw(seed)
+    print("configuration:", raw, flush=True)  # names the case before any kernel runs
+    cfg = AutoConfig.from_dict(raw)
+    folder = write_random_model(os.path.join(str(tmp_path), f"m{seed}"), cfg, seed=seed, noise=0.1)
+    reqs = helpers.make_requests(cfg.vocab_size, [3, 66, 37, 130], seed=seed)
+    want = helpers.plain_logits(folder, reqs)
+    for dtype, rel in (("float32", REL_F32), ("bfloat16", REL_BF16)):
+        model = AutoModelForCausalLM.from_pretrained(folder, dtype=dtype)
+        rp = Replayer(model, 1024)
+        for sched, records in (("whole", helpers.schedule_whole(reqs)), ("tail32", helpers.schedule_tail(reqs, 32)),
+                               ("batches", helpers.schedule_batches(reqs, 3, decode=(1, 20, 5)))):
+            got = helpers.run_schedule(rp, records)
+            for rid in reqs:
+                helpers.assert_close(got[rid], want[rid], rel, f"seed {seed} {dtype} {sched} {rid}")
+        del rp, model
+    torch.cuda.empty_cache()
