@@ -187,16 +187,23 @@ __global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
             float s[8];
-            float mx = -INFINITY;
-            const int lim = min(qpos[ct] + 1, k_end);  // keys below this count for the column
+            if (slopes) {  // one branch for the tile, not one per score
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int key = kb + 8 * gq + j;  // j = 4*tt + e
-                float v = sacc[j >> 2][ct][j & 3] * scale;
-                if (slopes) v += round_to_bf16(slope[ct] * round_to_bf16((float)key)) * alibi_mul;
-                s[j] = (interior || key < lim) ? v : -INFINITY;
-                mx = fmaxf(mx, s[j]);
+                for (int j = 0; j < 8; ++j) {
+                    const int key = kb + 8 * gq + j;  // j = 4*tt + e
+                    s[j] = sacc[j >> 2][ct][j & 3] * scale + round_to_bf16(slope[ct] * round_to_bf16((float)key)) * alibi_mul;
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) s[j] = sacc[j >> 2][ct][j & 3] * scale;
             }
+            if (!interior) {
+                const int lim = min(qpos[ct] + 1, k_end);  // keys below this count for the column
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (kb + 8 * gq + j >= lim) s[j] = -INFINITY;
+            }
+            float mx = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
             // The running maximum is only a reference point for the exponentials, shared by the four lanes of
             // a column; it is brought up to the true maximum (an exchange between those lanes, and a
             // rescale of what was summed) only when some score of the block lies more than 2^8 above it,

@@ -23,8 +23,10 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_NAME = "libpta_kernels.so"
 ARCH = "gfx950"
 # packed 32-bit float instructions are switched off for every kernel of this library
+# ... and matrix-core results go to ordinary vector registers: the kernels here do arithmetic on their
+# accumulators between products, and copies to and from the accumulation registers cost more than they save
 FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang",
-         "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
+         "-packed-fp32-ops", "-mllvm", "-amdgpu-mfma-vgpr-form", "-Wno-unused-command-line-argument"]
 
 
 def sources():
