@@ -208,6 +208,29 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(void* __restric
     else ((bf16_t*)y)[o] = f32_to_bf16_bits(v);
 }
 
+// the same for the two products of a pair launch, bfloat16 out, no additions
+__global__ __launch_bounds__(256) void gemm_splitk_reduce2_kernel(bf16_t* __restrict__ y1, const float* __restrict__ part1,
+                                                                  const float* __restrict__ bias1, long MN1, int N1, int P1,
+                                                                  int act1, bf16_t* __restrict__ y2,
+                                                                  const float* __restrict__ part2,
+                                                                  const float* __restrict__ bias2, long MN2, int N2, int P2,
+                                                                  int act2) {
+    long o = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const bool second = o >= MN1;
+    if (second) o -= MN1;
+    const long MN = second ? MN2 : MN1;
+    if (o >= MN) return;
+    const float* part = second ? part2 : part1;
+    const float* bias = second ? bias2 : bias1;
+    const int N = second ? N2 : N1, P = second ? P2 : P1, act = second ? act2 : act1;
+    float v = part[o];
+    for (int p = 1; p < P; ++p) v += part[(long)p * MN + o];
+    v = round_to_bf16(v);
+    if (bias) v = round_to_bf16(v + bias[(int)(o % N)]);
+    if (act == PTA_ACT_GELU) v = gelu_erf(v);
+    (second ? y2 : y1)[o] = f32_to_bf16_bits(v);
+}
+
 static int pick_rt(int N) { return N >= 16384 ? 2 : 1; }
 
 // Ranges of K (workgroups along gridDim.y): enough for about two workgroups per compute unit, but no
@@ -326,4 +349,23 @@ extern "C" int pta_gemm_splitk_pair_bf16(float* part1, const void* x1, const voi
     const SplitkProblem b = make_problem(nullptr, part2, x2, W2, nullptr, nullptr, nullptr, N2, K2, 0, 0, 1,
                                          pick_parts(N2, K2, 1), 0);
     return launch_rows<1, 2, 2>((M + 15) / 16, a, b, M, 0, (hipStream_t)stream);
+}
+
+// The same pair run to the end: y1 = act1(x1 . W1^T + bias1), y2 = act2(x2 . W2^T + bias2) in bfloat16; the two
+// products share the matrix launch and the launch that adds their partial sums.
+extern "C" int pta_gemm_splitk_pair_reduced_bf16(void* y1, float* part1, const void* x1, const void* W1,
+                                                 const float* bias1, int N1, int K1, int act1, void* y2, float* part2,
+                                                 const void* x2, const void* W2, const float* bias2, int N2, int K2,
+                                                 int act2, int M, void* stream) {
+    PTA_REQUIRE(y1 && y2, "gemm_splitk_pair_reduced_bf16: null output");
+    PTA_REQUIRE((act1 == PTA_ACT_NONE || act1 == PTA_ACT_GELU) && (act2 == PTA_ACT_NONE || act2 == PTA_ACT_GELU),
+                "gemm_splitk_pair_reduced_bf16: unknown activation");
+    const int rc = pta_gemm_splitk_pair_bf16(part1, x1, W1, N1, K1, part2, x2, W2, N2, K2, M, stream);
+    if (rc) return rc;
+    const long MN1 = (long)M * N1, MN2 = (long)M * N2;
+    const int P1 = effective_parts(K1, pick_parts(N1, K1, 1)), P2 = effective_parts(K2, pick_parts(N2, K2, 1));
+    hipLaunchKernelGGL(gemm_splitk_reduce2_kernel, dim3((unsigned)((MN1 + MN2 + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, (bf16_t*)y1, part1, bias1, MN1, N1, P1, act1, (bf16_t*)y2, part2, bias2, MN2, N2,
+                       P2, act2);
+    return pta_check_launch("gemm_splitk_pair_reduced_bf16");
 }

@@ -94,6 +94,11 @@ int pta_gemm_splitk_parts(int N, int K, int parts, int rt);
 int pta_gemm_splitk_pair_bf16(float* part1, const void* x1, const void* W1, int N1, int K1, float* part2,
                               const void* x2, const void* W2, int N2, int K2, int M, void* stream);
 
+// the same pair run to the end: y1 = act1(x1 . W1^T + bias1), y2 = act2(x2 . W2^T + bias2), bfloat16
+int pta_gemm_splitk_pair_reduced_bf16(void* y1, float* part1, const void* x1, const void* W1, const float* bias1, int N1,
+                                      int K1, int act1, void* y2, float* part2, const void* x2, const void* W2,
+                                      const float* bias2, int N2, int K2, int act2, int M, void* stream);
+
 // processors in the reference's order, then argmax (do_sample 0) or a draw; `work` [R, V] receives the
 // processed scores; hist/hist_off (tokens seen, per row), eos/suppress, uniforms may be null
 int pta_sample(int* out_tok, float* work, const float* logits, int R, int V, int do_sample, float temperature,

@@ -414,6 +414,31 @@ def gemm_splitk_pair_partial(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tenso
     return part1, part2
 
 
+def gemm_splitk_pair_bf16(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tensor, w2: torch.Tensor, bias1=None, act1=None,
+                          bias2=None, act2=None):
+    """(act1(x1 @ w1.T + bias1), act2(x2 @ w2.T + bias2)) for a batch of up to 64 rows: one matrix launch for
+    both products and one launch that adds their partial sums."""
+    for name, t in (("x1", x1), ("w1", w1), ("x2", x2), ("w2", w2)):
+        _need(t, name, torch.bfloat16)
+    M = x1.shape[0]
+    if x2.shape[0] != M or w1.dim() != 2 or w2.dim() != 2 or w1.shape[1] != x1.shape[1] or w2.shape[1] != x2.shape[1]:
+        raise KernelError(f"a pair shares M: x1 {tuple(x1.shape)}, w1 {tuple(w1.shape)}, x2 {tuple(x2.shape)}, "
+                          f"w2 {tuple(w2.shape)}")
+    lib = load_library()
+    (N1, K1), (N2, K2) = w1.shape, w2.shape
+    if bias1 is not None:
+        _need(bias1, "bias1", torch.float32, (N1,))
+    if bias2 is not None:
+        _need(bias2, "bias2", torch.float32, (N2,))
+    part1 = torch.empty((int(lib.pta_gemm_splitk_parts(N1, K1, 0, 1)), M, N1), dtype=torch.float32, device=x1.device)
+    part2 = torch.empty((int(lib.pta_gemm_splitk_parts(N2, K2, 0, 1)), M, N2), dtype=torch.float32, device=x1.device)
+    y1 = torch.empty((M, N1), dtype=torch.bfloat16, device=x1.device)
+    y2 = torch.empty((M, N2), dtype=torch.bfloat16, device=x1.device)
+    _call("pta_gemm_splitk_pair_reduced_bf16", _ptr(y1), _ptr(part1), _ptr(x1), _ptr(w1), _ptr(bias1), N1, K1,
+          ACT_CODES[act1], _ptr(y2), _ptr(part2), _ptr(x2), _ptr(w2), _ptr(bias2), N2, K2, ACT_CODES[act2], M, _stream())
+    return y1, y2
+
+
 def gemm_partial_pair_ok(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tensor, w2: torch.Tensor) -> bool:
     """Whether two products onto the same features are best left as partial sums of one launch: up to 64
     rows each, and at least one of them worth leaving so on its own."""
@@ -500,6 +525,11 @@ def gemm_skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
     """Whether the kernel for few rows takes this product and is the faster choice for it: bfloat16 with K a
     multiple of 8 and at most 16 rows (measured on MI355X against the vendor library at Falcon-7B shapes)."""
     return _bf16_rows_ok(x, w) and 0 < x.shape[0] <= 16
+
+
+def gemm_splitk_rows_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether the kernel for a decode batch takes this product at all (17 to 64 rows of bfloat16, K % 8 == 0)."""
+    return _bf16_rows_ok(x, w) and 16 < x.shape[0] <= SKINNY_MAX_ROWS
 
 
 def gemm_splitk_ok(x: torch.Tensor, w: torch.Tensor) -> bool:

@@ -57,16 +57,20 @@ class Linear(Part):
 
     @staticmethod
     def pair(first: "Linear", x1: torch.Tensor, kw1: dict, second: "Linear", x2: torch.Tensor, kw2: dict):
-        """``(first(x1, **kw1), second(x2, **kw2))`` in one launch where the kernel for few rows takes both
-        (same rows, same K, no additions); else None."""
-        if not (x1.dtype == torch.bfloat16 and x1.shape == x2.shape and ops.gemm_skinny_ok(x1, first.weight)
-                and ops.gemm_skinny_ok(x2, second.weight)):
+        """``(first(x1, **kw1), second(x2, **kw2))`` from one matrix launch, in steps small enough for the
+        decode kernels (same rows, no additions); else None."""
+        if not (x1.dtype == torch.bfloat16 and x1.shape[0] == x2.shape[0]):
             return None
         if any(k not in ("act", "apply_bias") for k in list(kw1) + list(kw2)):
             return None
         b1 = first.bias if kw1.get("apply_bias", True) else None
         b2 = second.bias if kw2.get("apply_bias", True) else None
-        return ops.gemm_skinny_pair_bf16(x1, first.weight, x2, second.weight, b1, kw1.get("act"), b2, kw2.get("act"))
+        args = (x1, first.weight, x2, second.weight, b1, kw1.get("act"), b2, kw2.get("act"))
+        if x1.shape == x2.shape and ops.gemm_skinny_ok(x1, first.weight) and ops.gemm_skinny_ok(x2, second.weight):
+            return ops.gemm_skinny_pair_bf16(*args)
+        if ops.gemm_splitk_rows_ok(x1, first.weight) and ops.gemm_splitk_rows_ok(x2, second.weight):
+            return ops.gemm_splitk_pair_bf16(*args)
+        return None
 
     def partial(self, x: torch.Tensor) -> Optional[PartialProduct]:
         """The product left as partial sums for the next norm to add, where that pays; else None."""

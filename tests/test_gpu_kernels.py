@@ -204,6 +204,20 @@ def test_gemm_skinny_pair():
         ops.gemm_skinny_pair_bf16(x1, w1, x2[:3].contiguous(), w2)
 
 
+def test_gemm_splitk_pair():
+    """Two products of one launch, run to the end, against the products on their own."""
+    ops = _ops()
+    M, K1, K2, N1, N2 = 40, 328, 264, 100, 530
+    x1, x2 = _rand(M, K1, dtype=torch.bfloat16), _rand(M, K2, seed=5, dtype=torch.bfloat16)
+    w1, w2 = _rand(N1, K1, seed=1, dtype=torch.bfloat16, scale=0.05), _rand(N2, K2, seed=2, dtype=torch.bfloat16, scale=0.05)
+    b2 = _rand(N2, seed=3)
+    y1, y2 = ops.gemm_splitk_pair_bf16(x1, w1, x2, w2, None, None, b2, "gelu")
+    assert torch.equal(y1, ops.gemm_splitk_bf16(x1, w1, rt=1)), "the same ranges in the same order: the same bits"
+    assert torch.equal(y2, ops.gemm_splitk_bf16(x2, w2, b2, "gelu", rt=1))
+    a1, a2 = ops.gemm_splitk_pair_bf16(x1[17:37].contiguous(), w1, x2[17:37].contiguous(), w2, None, None, b2, "gelu")
+    assert torch.equal(a1, y1[17:37]) and torch.equal(a2, y2[17:37])
+
+
 def test_gemm_skinny_refuses_what_it_cannot_do():
     ops = _ops()
     x, w = _rand(65, 64, dtype=torch.bfloat16), _rand(32, 64, dtype=torch.bfloat16)
