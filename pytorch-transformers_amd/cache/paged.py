@@ -15,7 +15,9 @@ layer group owns a pool of pages of ``page_size`` tokens; a slot's keys and
 values are the pages its page list names, in order, so the position of a key is
 its index in the slot.  Slots and pages go back to free lists when a sequence
 ends and are handed out again; nothing is zeroed, because a slot's length says
-what is valid.  Groups of kind ``state`` own a ``[max_slots, *shape]`` table per
+what is valid.  A group of kind ``window`` is laid out like a full one, but gives the pages that lie
+wholly behind its window back to its pool as a sequence grows (their places in the page list hold
+-1), so a long sequence holds about ``window / page_size`` pages of it.  Groups of kind ``state`` own a ``[max_slots, *shape]`` table per
 layer that is zeroed when a slot is handed out.
 
 The K pool has the layout ``[layer, page, kv_head, page_size, head_dim]``, the V pool
@@ -50,9 +52,12 @@ class _Group:
         self.page_size = page_size
         self.k = self.v = None
         self.state: Optional[torch.Tensor] = None
-        self.paged = spec.kind == CACHE_FULL
+        self.paged = spec.kind in (CACHE_FULL, CACHE_WINDOW)
+        self.window = int(spec.window or 0) if spec.kind == CACHE_WINDOW else 0
         self.index = -1  # among the paged groups, as the host runtime counts them
-        if spec.kind == CACHE_FULL:
+        if spec.kind == CACHE_WINDOW and self.window <= 0:
+            raise CacheError(f"cache group {spec.name!r}: kind 'window' needs a positive window, got {spec.window!r}")
+        if self.paged:
             # values are held transposed inside a page so that the attention kernels read eight
             # consecutive positions of one feature in one load
             self.k = torch.zeros((spec.num_layers, num_pages, spec.kv_heads, page_size, spec.head_dim),
@@ -62,10 +67,6 @@ class _Group:
         elif spec.kind == CACHE_STATE:
             sd = spec.state_dtype or torch.float32
             self.state = torch.zeros((spec.num_layers, max_slots, *spec.state_shape), dtype=sd, device=device)
-        elif spec.kind == CACHE_WINDOW:
-            raise CacheError(
-                f"cache group {spec.name!r}: kind 'window' is declared in the interface but no kernel reads a "
-                "ring of pages yet; use 'full'")
         else:
             raise CacheError(f"cache group {spec.name!r}: unknown kind {spec.kind!r}")
 
@@ -90,7 +91,8 @@ class PagedCache:
             self.groups[name].index = i
         self._lib = host.load()
         self._h = self._lib.ptah_cache_new(self.max_slots, page_size, len(self._paged),
-                                           host.int_array([self.num_pages] * len(self._paged)))
+                                           host.int_array([self.num_pages] * len(self._paged)),
+                                           host.int_array([self.groups[n].window for n in self._paged]))
         if not self._h:
             raise CacheError(host.last_error())
 

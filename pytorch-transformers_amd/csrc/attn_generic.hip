@@ -5,7 +5,7 @@
 // batch.  This is the engine's 32-bit path and the fallback for sizes the MFMA
 // kernels refuse.
 //
-// score[j] = q . k_j / sqrt(d) + alibi_j, keys 0 .. pos
+// score[j] = q . k_j / sqrt(d) + alibi_j, keys 0 .. pos (or the last `window` of them)
 // (src/transformers/models/falcon/modeling_falcon.py:371-386, :407-422).
 // alibi_j = bf16(bf16(slope_h) * bf16(j)) / sqrt(d): the reference forms slope x position in
 // bfloat16 even in a 32-bit model (:196-198) and divides by sqrt(d) when it folds the bias into
@@ -18,7 +18,7 @@ __global__ void attn_generic_kernel(T* __restrict__ out, const T* __restrict__ q
                                     const T* __restrict__ v_pool, const int* __restrict__ block_table,
                                     int bt_stride, const int* __restrict__ token_seq,
                                     const int* __restrict__ token_pos, const float* __restrict__ slopes, int nh,
-                                    int nkv, int d, float scale, float sqrt_d) {
+                                    int nkv, int d, float scale, float sqrt_d, int window) {
     __shared__ float q_s[256];
     __shared__ float p_s[PTA_PAGE];
     const int m = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
@@ -31,14 +31,16 @@ __global__ void attn_generic_kernel(T* __restrict__ out, const T* __restrict__ q
     __syncthreads();
     const float slope = slopes ? slopes[h] : 0.f;
 
+    // with a window the token sees keys first .. pos only; pages wholly before `first` may be gone
+    const int first = window > 0 ? max(0, nkeys - window) : 0;
     float m_run = -INFINITY, l_run = 0.f;
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int c0 = 0; c0 < nkeys; c0 += PTA_PAGE) {
+    for (int c0 = first / PTA_PAGE * PTA_PAGE; c0 < nkeys; c0 += PTA_PAGE) {
         const long page = bt[c0 / PTA_PAGE];
         const T* kp = k_pool + (page * nkv + kvh) * (long)PTA_PAGE * d;
         const T* vp = v_pool + (page * nkv + kvh) * (long)PTA_PAGE * d;
         const int j = c0 + lane;
-        const bool valid = j < nkeys;
+        const bool valid = j >= first && j < nkeys;
         float s = -INFINITY;
         if (valid) {
             const T* kr = kp + (long)lane * d;
@@ -60,7 +62,7 @@ __global__ void attn_generic_kernel(T* __restrict__ out, const T* __restrict__ q
             const int dim = lane + r * PTA_WAVE;
             if (dim < d) {
                 float a = acc[r] * corr;
-                for (int jj = 0; jj < cnt; ++jj) a += p_s[jj] * Io<T>::ld(vp + (long)dim * PTA_PAGE + jj);
+                for (int jj = max(0, first - c0); jj < cnt; ++jj) a += p_s[jj] * Io<T>::ld(vp + (long)dim * PTA_PAGE + jj);
                 acc[r] = a;
             }
         }
@@ -77,23 +79,24 @@ __global__ void attn_generic_kernel(T* __restrict__ out, const T* __restrict__ q
 
 extern "C" int pta_attn_generic(void* out, const void* q, const void* k_pool, const void* v_pool,
                                 const int* block_table, int bt_stride, const int* token_seq, const int* token_pos,
-                                const float* slopes, int M, int nh, int nkv, int d, float scale, int dtype,
+                                const float* slopes, int M, int nh, int nkv, int d, float scale, int window, int dtype,
                                 void* stream) {
     PTA_REQUIRE(M > 0 && nh > 0 && nkv > 0, "attn_generic: sizes must be positive (M=%d nh=%d nkv=%d)", M, nh, nkv);
     PTA_REQUIRE(nh % nkv == 0, "attn_generic: heads (%d) must be a multiple of kv heads (%d)", nh, nkv);
     PTA_REQUIRE(d > 0 && d <= 256, "attn_generic: head size %d is outside 1..256", d);
     PTA_REQUIRE(nh <= 65535, "attn_generic: at most 65535 heads, got %d", nh);
+    PTA_REQUIRE(window >= 0, "attn_generic: window must be 0 (none) or positive, got %d", window);
     hipStream_t s = (hipStream_t)stream;
     dim3 grid(M, nh);
     const float sqrt_d = sqrtf((float)d);
     if (dtype == PTA_F32)
         hipLaunchKernelGGL(attn_generic_kernel<float>, grid, dim3(PTA_WAVE), 0, s, (float*)out, (const float*)q,
                            (const float*)k_pool, (const float*)v_pool, block_table, bt_stride, token_seq, token_pos,
-                           slopes, nh, nkv, d, scale, sqrt_d);
+                           slopes, nh, nkv, d, scale, sqrt_d, window);
     else if (dtype == PTA_BF16)
         hipLaunchKernelGGL(attn_generic_kernel<bf16_t>, grid, dim3(PTA_WAVE), 0, s, (bf16_t*)out, (const bf16_t*)q,
                            (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_table, bt_stride, token_seq,
-                           token_pos, slopes, nh, nkv, d, scale, sqrt_d);
+                           token_pos, slopes, nh, nkv, d, scale, sqrt_d, window);
     else
         return pta_fail("attn_generic: unknown dtype %d", dtype);
     return pta_check_launch("attn_generic");

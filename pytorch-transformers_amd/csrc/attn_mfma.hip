@@ -87,7 +87,7 @@ __global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
     const int* __restrict__ block_table, int bt_stride, const int* __restrict__ cu_tokens,
     const int* __restrict__ seq_start, const float* __restrict__ slopes, int nh, int nkv, float scale, float alibi_mul,
-    int split_size, int n_splits) {
+    int split_size, int n_splits, int window) {
     constexpr int D = DT * 16;
     constexpr int DS = (DT + 1) / 2;   // 32-wide steps over the head dimension
     constexpr int CHUNKS = D / 8;      // 16-byte chunks in a row of d elements
@@ -104,8 +104,12 @@ __global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
     const int last_col = min(ncols, col0 + 16 * CT) - 1;
     const int max_qpos = start + last_col / g;
     const int kv_len = start + n_new;
-    const int k_begin = n_splits > 1 ? split * split_size : 0;
-    const int k_end = !active ? 0 : n_splits > 1 ? min(max_qpos + 1, k_begin + split_size) : max_qpos + 1;
+    // with a window a column at position t sees keys t - window + 1 .. t; this wave starts at the block of
+    // the first key its first column sees (earlier pages may be gone), and at its range's start if split
+    const int lo_first = window > 0 ? max(0, start + col0 / g - window + 1) : 0;   // lowest key any column sees
+    const int lo_last = window > 0 ? max(0, max_qpos - window + 1) : 0;            // lowest key the last column sees
+    const int k_begin = max(n_splits > 1 ? split * split_size : 0, lo_first & ~31);
+    const int k_end = !active ? 0 : n_splits > 1 ? min(max_qpos + 1, split * split_size + split_size) : max_qpos + 1;
     const int kb_last = (kv_len - 1) & ~31;  // the last block that has a page
     // below this key index no column of this wave masks anything (columns are ordered by token)
     const int min_lim = min(start + col0 / g + 1, k_end);
@@ -182,7 +186,7 @@ __global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
             }
         // Scores are kept in units of log 2 (the scale carries log2 e), so that the exponential is the
         // hardware's exp2.  A block that lies wholly below every column's limit needs no masking.
-        const bool interior = kb + 32 <= min_lim;
+        const bool interior = kb + 32 <= min_lim && kb >= lo_last;
         AFrag pf[CT];
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
@@ -198,10 +202,11 @@ __global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
                 for (int j = 0; j < 8; ++j) s[j] = sacc[j >> 2][ct][j & 3] * scale;
             }
             if (!interior) {
-                const int lim = min(qpos[ct] + 1, k_end);  // keys below this count for the column
+                const int lim = min(qpos[ct] + 1, k_end);  // keys below this, and from `lo` on, count for the column
+                const int lo = window > 0 ? qpos[ct] - window + 1 : 0;
 #pragma unroll
                 for (int j = 0; j < 8; ++j)
-                    if (kb + 8 * gq + j >= lim) s[j] = -INFINITY;
+                    if (kb + 8 * gq + j >= lim || kb + 8 * gq + j < lo) s[j] = -INFINITY;
             }
             float mx = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
             // The running maximum is only a reference point for the exponentials, shared by the four lanes of
@@ -267,6 +272,7 @@ __global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
         const int tid = threadIdx.x;
         const int wg_last_col = min(ncols, wg_col0 + 16 * CT * W) - 1;
         const int k_end_wg = start + wg_last_col / g + 1;
+        const int k_begin_wg = window > 0 ? max(0, start + wg_col0 / g - window + 1) & ~31 : 0;
         uint4 gk[PER], gv[PER];
         auto gload = [&](int kb) {
             kb = min(kb, kb_last);
@@ -304,14 +310,14 @@ __global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
             for (int dt = 0; dt < DT; ++dt)
                 b.v[dt].u = *reinterpret_cast<const uint4*>(&vbuf[buf][(dt * 16 + c) * VROW + gq * 8]);
         };
-        gload(0);
-        sstore(0);
+        gload(k_begin_wg);
+        sstore((k_begin_wg >> 5) & 1);
         __syncthreads();
-        for (int kb = 0; kb < k_end_wg; kb += 32) {
+        for (int kb = k_begin_wg; kb < k_end_wg; kb += 32) {
             const int buf = (kb >> 5) & 1;
             gload(kb + 32);
             __builtin_amdgcn_sched_barrier(0);
-            if (kb < k_end) {
+            if (kb < k_end && kb >= k_begin) {
                 KvBlock<DT> b;
                 lfetch(b, buf);
                 use_block(b, kb);
@@ -386,9 +392,11 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(bf16_t* __restrict__ o
         int s = 0;
         for (; s + 4 <= used; s += 4) {
             const float v0 = p[(long)s * D], v1 = p[(long)(s + 1) * D], v2 = p[(long)(s + 2) * D], v3 = p[(long)(s + 3) * D];
-            acc += w_s[s] * v0; acc += w_s[s + 1] * v1; acc += w_s[s + 2] * v2; acc += w_s[s + 3] * v3;
+            // a range with weight zero was never written (past the row's keys, or before its window)
+            acc += w_s[s] != 0.f ? w_s[s] * v0 : 0.f; acc += w_s[s + 1] != 0.f ? w_s[s + 1] * v1 : 0.f;
+            acc += w_s[s + 2] != 0.f ? w_s[s + 2] * v2 : 0.f; acc += w_s[s + 3] != 0.f ? w_s[s + 3] * v3 : 0.f;
         }
-        for (; s < used; ++s) acc += w_s[s] * p[(long)s * D];
+        for (; s < used; ++s) acc += w_s[s] != 0.f ? w_s[s] * p[(long)s * D] : 0.f;
         out[row * D + dd] = f32_to_bf16_bits(acc * inv);
     }
 }
@@ -397,12 +405,12 @@ template <int DT, int CT, int W = 1>
 static void launch_attn(bf16_t* out, float* po, float* pm, float* pl, const bf16_t* q, const bf16_t* k_pool,
                         const bf16_t* v_pool, const int* block_table, int bt_stride, const int* cu_tokens,
                         const int* seq_start, const float* slopes, int n_seqs, int max_new, int nh, int nkv, float scale,
-                        int split_size, int n_splits, hipStream_t s) {
+                        int split_size, int n_splits, int window, hipStream_t s) {
     const int g = nh / nkv;
     const dim3 grid((max_new * g + 16 * CT * W - 1) / (16 * CT * W), nkv, n_seqs * n_splits);
     hipLaunchKernelGGL((attn_mfma_kernel<DT, CT, W>), grid, dim3(64 * W), 0, s, out, po, pm, pl, q, k_pool, v_pool, block_table,
                        bt_stride, cu_tokens, seq_start, slopes, nh, nkv, scale * PTA_LOG2E,
-                       PTA_LOG2E / sqrtf((float)(DT * 16)), split_size, n_splits);
+                       PTA_LOG2E / sqrtf((float)(DT * 16)), split_size, n_splits, window);
 }
 
 extern "C" int pta_attn_mfma_supported(int d) { return d % 16 == 0 && ((d >= 16 && d <= 128) || d == 256); }
@@ -410,11 +418,12 @@ extern "C" int pta_attn_mfma_supported(int d) { return d % 16 == 0 && ((d >= 16 
 extern "C" int pta_attn_mfma(void* out, const void* q, const void* k_pool, const void* v_pool, const int* block_table,
                              int bt_stride, const int* cu_tokens, const int* seq_start, const float* slopes, int n_seqs,
                              int max_new, int M, int nh, int nkv, int d, float scale, int split_size, int n_splits,
-                             float* po, float* pm, float* pl, void* stream) {
+                             float* po, float* pm, float* pl, int window, void* stream) {
     PTA_REQUIRE(n_seqs > 0 && max_new > 0 && M > 0 && nh > 0 && nkv > 0, "attn_mfma: sizes must be positive");
     PTA_REQUIRE(nh % nkv == 0, "attn_mfma: heads (%d) must be a multiple of kv heads (%d)", nh, nkv);
     PTA_REQUIRE(pta_attn_mfma_supported(d), "attn_mfma: head size %d is not built (16..128 in steps of 16, or 256)", d);
     PTA_REQUIRE(n_splits >= 1 && n_splits <= 1024, "attn_mfma: n_splits must be 1..1024, got %d", n_splits);
+    PTA_REQUIRE(window >= 0, "attn_mfma: window must be 0 (none) or positive, got %d", window);
     PTA_REQUIRE(n_splits == 1 || (split_size > 0 && split_size % 64 == 0 && po && pm && pl),
                 "attn_mfma: splitting needs a split size that is a multiple of 64 and buffers for partial results");
     PTA_REQUIRE((long)n_seqs * n_splits <= 65535 && nkv <= 65535, "attn_mfma: too many sequences x splits for one launch");
@@ -432,7 +441,7 @@ extern "C" int pta_attn_mfma(void* out, const void* q, const void* k_pool, const
     static const int w_env = getenv("PTA_ATTN_W") ? atoi(getenv("PTA_ATTN_W")) : 4;
 #define PTA_ATTN_ARGS                                                                                              \
     (bf16_t*)out, po, pm, pl, (const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_table, bt_stride, \
-        cu_tokens, seq_start, slopes, n_seqs, max_new, nh, nkv, scale, split_size, n_splits, s
+        cu_tokens, seq_start, slopes, n_seqs, max_new, nh, nkv, scale, split_size, n_splits, window, s
 #define PTA_ATTN_CASE(DT_, CT_)                                                                   \
     case DT_:                                                                                     \
         if (narrow || ct_env == 1) launch_attn<DT_, 1, 1>(PTA_ATTN_ARGS);                         \

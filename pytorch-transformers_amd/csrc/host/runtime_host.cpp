@@ -67,7 +67,8 @@ struct FreeList {
 
 struct Group {
     FreeList pages;
-    std::vector<std::vector<int>> lists;  // per slot
+    std::vector<std::vector<int>> lists;  // per slot: page of every 64 positions, -1 where a window has moved on
+    int window = 0;                        // 0: all keys are kept; w: a token sees the last w positions only
 };
 
 struct Cache {
@@ -79,6 +80,11 @@ struct Cache {
     std::vector<int> plan_sizes;
 
     int pages_for(int len) const { return (len + page_size - 1) / page_size; }
+    // the first page a sequence of this length still reads: its next token, at position len, sees keys from
+    // len - window + 1 on
+    int first_needed(const Group& g, int len) const {
+        return g.window > 0 ? std::max(0, len - g.window + 1) / page_size : 0;
+    }
 };
 
 }  // namespace
@@ -87,9 +93,9 @@ extern "C" {
 
 const char* ptah_last_error() { return g_error.c_str(); }
 
-int ptah_abi_version() { return 1; }
+int ptah_abi_version() { return 2; }
 
-void* ptah_cache_new(int max_slots, int page_size, int n_groups, const int* group_pages) {
+void* ptah_cache_new(int max_slots, int page_size, int n_groups, const int* group_pages, const int* group_windows) {
     if (max_slots <= 0 || page_size <= 0 || n_groups < 0) {
         fail(ERR_CACHE, "cache: max_slots=%d page_size=%d groups=%d", max_slots, page_size, n_groups);
         return nullptr;
@@ -102,6 +108,7 @@ void* ptah_cache_new(int max_slots, int page_size, int n_groups, const int* grou
     for (int g = 0; g < n_groups; ++g) {
         c->groups[g].pages.init(group_pages[g]);
         c->groups[g].lists.assign(max_slots, {});
+        c->groups[g].window = group_windows ? std::max(0, group_windows[g]) : 0;
     }
     return c;
 }
@@ -126,7 +133,7 @@ int ptah_free(void* h, int slot) {
     if (!c->slots.is_held(slot)) return fail(ERR_CACHE, "slot %d is not allocated", slot);
     for (size_t g = 0; g < c->groups.size(); ++g) {
         for (int p : c->groups[g].lists[slot])
-            if (!c->groups[g].pages.give(p)) return fail(ERR_CACHE, "page %d of group %zu is freed twice", p, g);
+            if (p >= 0 && !c->groups[g].pages.give(p)) return fail(ERR_CACHE, "page %d of group %zu is freed twice", p, g);
         c->groups[g].lists[slot].clear();
     }
     c->length[slot] = 0;
@@ -159,6 +166,20 @@ int ptah_reserve(void* h, int n, const int* slots, const int* new_tokens) {
         if (!c->slots.is_held(slots[i])) return fail(ERR_CACHE, "slot %d is not allocated", slots[i]);
         for (int j = 0; j < i; ++j)
             if (slots[j] == slots[i]) return fail(ERR_CACHE, "a slot appears twice in one step: %d", slots[i]);
+    }
+    // pages that a window has left behind go back to the pool first: no later step reads them, whether
+    // this one is accepted or not
+    for (Group& gr : c->groups) {
+        if (gr.window <= 0) continue;
+        for (int i = 0; i < n; ++i) {
+            std::vector<int>& l = gr.lists[slots[i]];
+            const int keep_from = std::min((int)l.size(), c->first_needed(gr, c->length[slots[i]]));
+            for (int k = 0; k < keep_from; ++k)
+                if (l[k] >= 0) {
+                    gr.pages.give(l[k]);
+                    l[k] = -1;
+                }
+        }
     }
     for (size_t g = 0; g < c->groups.size(); ++g) {
         Group& gr = c->groups[g];
@@ -216,7 +237,9 @@ int ptah_check(void* h) {
             if (!l.empty() && !live) return fail(ERR_CACHE, "freed slot %d still lists %zu pages in group %zu", s, l.size(), g);
             if (live && (int)l.size() < c->pages_for(c->length[s]))
                 return fail(ERR_CACHE, "slot %d has length %d but only %zu pages", s, c->length[s], l.size());
-            for (int p : l) {
+            for (size_t k = 0; k < l.size(); ++k) {
+                const int p = l[k];
+                if (p == -1 && live && (int)k < c->first_needed(gr, c->length[s])) continue;  // behind the window
                 if (p < 0 || p >= gr.pages.size()) return fail(ERR_CACHE, "slot %d lists page %d, which does not exist", s, p);
                 if (owner[p] >= 0) return fail(ERR_CACHE, "page %d of group %zu is held by slots %d and %d", p, g, owner[p], s);
                 if (!gr.pages.is_held(p))
@@ -303,7 +326,7 @@ int ptah_plan_step(void* h, int n, const int* slots, const int* new_tokens, cons
     for (int g = 0; g < G; ++g) {
         for (int i = 0; i < n; ++i) {
             const std::vector<int>& l = c->groups[g].lists[slots[i]];
-            std::copy(l.begin(), l.end(), table + (long)i * width[g]);
+            for (size_t k = 0; k < l.size(); ++k) table[(long)i * width[g] + k] = std::max(0, l[k]);  // a hole is never read
         }
         table += (long)n * width[g];
     }

@@ -51,9 +51,10 @@ int pta_qkv_rope_cache(void* q_out, const void* fused, const float* bias, const 
                        int dtype, void* stream);
 
 // causal attention of M tokens over their sequences' cache, 32-bit arithmetic
+// window: 0, or the number of last positions a token sees (itself included)
 int pta_attn_generic(void* out, const void* q, const void* k_pool, const void* v_pool, const int* block_table,
                      int bt_stride, const int* token_seq, const int* token_pos, const float* slopes, int M, int nh,
-                     int nkv, int d, float scale, int dtype, void* stream);
+                     int nkv, int d, float scale, int window, int dtype, void* stream);
 
 // the same attention for bfloat16 on the matrix cores; cu_tokens [n_seqs + 1] and seq_start [n_seqs] say
 // which tokens are whose and how long each sequence was before the step; max_new bounds a sequence's new
@@ -63,7 +64,7 @@ int pta_attn_mfma_supported(int d);
 int pta_attn_mfma(void* out, const void* q, const void* k_pool, const void* v_pool, const int* block_table,
                   int bt_stride, const int* cu_tokens, const int* seq_start, const float* slopes, int n_seqs,
                   int max_new, int M, int nh, int nkv, int d, float scale, int split_size, int n_splits, float* po,
-                  float* pm, float* pl, void* stream);
+                  float* pm, float* pl, int window, void* stream);
 
 // C = act(A . W^T + bias) + add1 + add2, all 32-bit, fixed summation order
 int pta_gemm_f32(float* C, const float* A, const float* W, const float* bias, const float* add1, const float* add2,

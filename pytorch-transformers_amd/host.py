@@ -12,7 +12,7 @@ import os
 import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-ABI_VERSION = 1
+ABI_VERSION = 2
 OK, ERR_STEP, ERR_CACHE, ERR_FULL = 0, 1, 2, 3
 
 _lib = None
@@ -40,7 +40,7 @@ def load():
             raise RuntimeError(f"{path} has ABI {lib.ptah_abi_version()}, this package needs {ABI_VERSION}; rebuild it")
         lib.ptah_last_error.restype = ctypes.c_char_p
         lib.ptah_cache_new.restype = ctypes.c_void_p
-        lib.ptah_cache_new.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, _P_INT]
+        lib.ptah_cache_new.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, _P_INT, _P_INT]
         lib.ptah_cache_delete.argtypes = [ctypes.c_void_p]
         lib.ptah_cache_delete.restype = None
         for name in ("ptah_alloc", "ptah_free_slots", "ptah_check"):

@@ -186,8 +186,10 @@ def qkv_rope_cache(fused: torch.Tensor, bias, inv_freq, cs_scale: float, token_p
     return q
 
 
-def attn_generic(q: torch.Tensor, k_pool, v_pool, block_table, token_seq, token_pos, slopes, scale: float):
-    """Causal attention of every token over its sequence's cache; out [M, nh*d]."""
+def attn_generic(q: torch.Tensor, k_pool, v_pool, block_table, token_seq, token_pos, slopes, scale: float,
+                 window: int = 0):
+    """Causal attention of every token over its sequence's cache (the last ``window`` positions of it, itself
+    included, if ``window`` > 0); out [M, nh*d]."""
     _need(q, "q")
     M, nh, d = q.shape
     nkv = k_pool.shape[1]
@@ -200,7 +202,7 @@ def attn_generic(q: torch.Tensor, k_pool, v_pool, block_table, token_seq, token_
     out = torch.empty((M, nh * d), dtype=q.dtype, device=q.device)
     _call("pta_attn_generic", _ptr(out), _ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(block_table),
           block_table.shape[1], _ptr(token_seq), _ptr(token_pos), _ptr(slopes), M, nh, nkv, d, ctypes.c_float(scale),
-          dtype_code(q.dtype), _stream())
+          int(window), dtype_code(q.dtype), _stream())
     return out
 
 
@@ -235,7 +237,7 @@ def attn_mfma_ok(q: torch.Tensor) -> bool:
 
 
 def attn_mfma(q: torch.Tensor, k_pool, v_pool, block_table, cu_tokens, seq_start, slopes, scale: float, *,
-              max_new: int, n_splits: int = 1, split_size: int = ATTN_SPLIT_KEYS) -> torch.Tensor:
+              max_new: int, n_splits: int = 1, split_size: int = ATTN_SPLIT_KEYS, window: int = 0) -> torch.Tensor:
     """Causal attention of a step's tokens over the cache on the matrix cores; out [M, nh*d].
 
     ``max_new`` bounds the new tokens of any sequence of the step; with ``n_splits > 1`` the keys
@@ -258,7 +260,7 @@ def attn_mfma(q: torch.Tensor, k_pool, v_pool, block_table, cu_tokens, seq_start
         pl = torch.empty((M, nh, n_splits), dtype=torch.float32, device=q.device)
     _call("pta_attn_mfma", _ptr(out), _ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(block_table), block_table.shape[1],
           _ptr(cu_tokens), _ptr(seq_start), _ptr(slopes), n_seqs, int(max_new), M, nh, nkv, d, ctypes.c_float(scale),
-          int(split_size), int(n_splits), _ptr(po), _ptr(pm), _ptr(pl), _stream())
+          int(split_size), int(n_splits), _ptr(po), _ptr(pm), _ptr(pl), int(window), _stream())
     return out
 
 
@@ -280,7 +282,7 @@ def decode_split_size(n_seqs: int, n_heads: int, n_kv_heads: int, max_len: int) 
     return size
 
 
-def attention(q: torch.Tensor, k_pool, v_pool, block_table, ctx, slopes, scale: float) -> torch.Tensor:
+def attention(q: torch.Tensor, k_pool, v_pool, block_table, ctx, slopes, scale: float, window: int = 0) -> torch.Tensor:
     """Attention of a step's tokens over the cache: picks the kernel for the step's shape and type.
 
     bfloat16 with a head size the matrix-core kernel is built for: that kernel, with the context
@@ -292,8 +294,8 @@ def attention(q: torch.Tensor, k_pool, v_pool, block_table, ctx, slopes, scale: 
             size = decode_split_size(ctx.n_seqs, q.shape[1], k_pool.shape[1], ctx.max_len)
             n_splits = (ctx.max_len + size - 1) // size
         return attn_mfma(q, k_pool, v_pool, block_table, ctx.cu_tokens, ctx.seq_start, slopes, scale,
-                         max_new=max(ctx.new_tokens), n_splits=n_splits, split_size=size)
-    return attn_generic(q, k_pool, v_pool, block_table, ctx.token_seq, ctx.token_pos, slopes, scale)
+                         max_new=max(ctx.new_tokens), n_splits=n_splits, split_size=size, window=window)
+    return attn_generic(q, k_pool, v_pool, block_table, ctx.token_seq, ctx.token_pos, slopes, scale, window)
 
 
 def sample(logits: torch.Tensor, *, do_sample: bool, temperature: float = 1.0, top_k: int = 0, top_p: float = 1.0,

@@ -22,7 +22,8 @@ from .linear import Linear, PendingProjection
 
 class AttentionMixer(Part):
     def __init__(self, name: str, hidden_size: int, num_heads: int, kv_heads: int, head_dim: int, qkv_layout: str,
-                 bias: bool, positions: Part, qkv_name: str = "query_key_value", out_name: str = "dense"):
+                 bias: bool, positions: Part, qkv_name: str = "query_key_value", out_name: str = "dense",
+                 window: int = 0):
         if num_heads % kv_heads:
             raise ValueError(f"heads ({num_heads}) must be a multiple of kv heads ({kv_heads})")
         if qkv_layout not in ops.QKV_LAYOUT_CODES:
@@ -34,6 +35,9 @@ class AttentionMixer(Part):
         self.head_dim = head_dim
         self.qkv_layout = qkv_layout
         self.positions = positions
+        #: 0, or how many of the last positions a token attends to (itself included); its cache group is then
+        #: of kind ``window`` with the same number, and gives back the pages that fall behind
+        self.window = int(window)
         self.scale = 1.0 / math.sqrt(head_dim)  # modeling_falcon.py:250
         self.qkv = Linear(f"{name}.{qkv_name}", hidden_size, (num_heads + 2 * kv_heads) * head_dim, bias)
         self.out = Linear(f"{name}.{out_name}", num_heads * head_dim, hidden_size, bias)
@@ -59,7 +63,7 @@ class AttentionMixer(Part):
         q = ops.qkv_rope_cache(fused, self.qkv.bias, inv_freq, cs_scale, ctx.token_pos, ctx.token_seq, table,
                                k_pool, v_pool, self.num_heads, self.kv_heads, self.head_dim, self.qkv_layout,
                                write_cache=call.write_cache)
-        o = ops.attention(q, k_pool, v_pool, table, ctx, self.positions.score_bias(), self.scale)
+        o = ops.attention(q, k_pool, v_pool, table, ctx, self.positions.score_bias(), self.scale, self.window)
         if defer:
             return PendingProjection(self.out, o)
         return self.out(o, add1=residual)

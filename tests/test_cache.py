@@ -63,8 +63,8 @@ def test_errors():
     c2.alloc()
     with pytest.raises(CacheFull, match="no free slot"):
         c2.alloc()
-    with pytest.raises(CacheError, match="window"):
-        _cache(groups=(CacheGroupSpec("w", CACHE_WINDOW, 1, 1, 16, window=32),))
+    with pytest.raises(CacheError, match="positive window"):
+        _cache(groups=(CacheGroupSpec("w", CACHE_WINDOW, 1, 1, 16),))
 
 
 def test_reserve_is_all_or_nothing():
@@ -132,3 +132,28 @@ def test_plan_step_lays_tokens_end_to_end():
                         (([a, b], [[1]], "last"), "token lists"), (([a], [[1]], "first"), "want must be")):
         with pytest.raises(StepError, match=match):
             plan_step(c, *args, vocab_size=10)
+
+
+def test_a_window_group_gives_back_the_pages_behind_its_window():
+    """A group that keeps the last 100 positions holds two or three pages per sequence however long it grows;
+    the full group beside it keeps them all.  Holes in the page list are never below the first page the
+    next token reads."""
+    c = _cache(64 * 16, groups=(KV, CacheGroupSpec("near", CACHE_WINDOW, 1, 1, 16, window=100)), max_slots=2)
+    s = c.alloc()
+    c.reserve([s], [300]); c.commit([s], [300])  # a long prompt needs all its pages while it runs
+    assert c.page_list("near", s) == [0, 1, 2, 3, 4] and c.page_list("kv", s) == [0, 1, 2, 3, 4]
+    c.reserve([s], [1])  # the token at 300 sees 201..300: pages 0, 1, 2 (positions 0..191) are behind it
+    assert c.page_list("near", s) == [-1, -1, -1, 3, 4] and c.free_pages("near") == 14 and c.free_pages("kv") == 11
+    c.commit([s], [1]); c.check_consistent()
+    for _ in range(400):
+        c.reserve([s], [1]); c.commit([s], [1])
+    c.check_consistent()
+    held = [p for p in c.page_list("near", s) if p >= 0]
+    assert 2 <= len(held) <= 3 and len(c.page_list("kv", s)) == 11 and c.free_pages("kv") == 5
+    assert c.page_list("near", s)[-1] >= 0 and c.length(s) == 701
+    t = c.alloc()  # pages that came back are handed out again, lowest first
+    c.reserve([t], [10])
+    assert c.page_list("near", t) == [0]
+    c.free(s); c.free(t)
+    assert c.free_pages("near") == 16 and c.free_pages("kv") == 16
+    c.check_consistent()

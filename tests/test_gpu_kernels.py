@@ -303,8 +303,22 @@ def test_qkv_rope_cache(dtype, layout, nh, nkv, d, rotary):
     assert torch.equal(torch.nan_to_num(k2.float()), torch.nan_to_num(k_pool.float()))
 
 
-def _attn_case(ops, fn, dtype, nh, nkv, d, starts, news, slopes=None, seed=0, boost=None):
-    """Fill a cache with random keys and values, run ``fn`` for the new tokens, compare with plain attention."""
+def _windowed_attention(q, k, v, window):
+    """Plain attention in which query t sees keys t - window + 1 .. t; q [T, nh, d], k, v [T, nkv, d]."""
+    T, nh, d = q.shape
+    g = nh // k.shape[1]
+    t = torch.arange(T)
+    seen = (t[None, :] <= t[:, None]) & (t[None, :] > t[:, None] - window)
+    out = torch.empty_like(q)
+    for h in range(nh):
+        s = (q[:, h] @ k[:, h // g].T / math.sqrt(d)).masked_fill(~seen, float("-inf"))
+        out[:, h] = torch.softmax(s, dim=-1) @ v[:, h // g]
+    return out.reshape(T, nh * d)
+
+
+def _attn_case(ops, fn, dtype, nh, nkv, d, starts, news, slopes=None, seed=0, boost=None, window=0):
+    """Fill a cache with random keys and values, run ``fn`` for the new tokens, compare with plain attention.
+    With a window, the pages that lie wholly behind every new token's window hold NaN: they may be gone."""
     lens = [s + n for s, n in zip(starts, news)]
     n_pages = sum((L + 63) // 64 for L in lens) + 3
     k_pool, v_pool, bt, lists = _cache_setup(len(lens), lens, nkv, d, dtype, n_pages=n_pages, seed=seed)
@@ -324,12 +338,15 @@ def _attn_case(ops, fn, dtype, nh, nkv, d, starts, news, slopes=None, seed=0, bo
         ks.append(k); vs.append(v); qs.append(q)
         for p, page in enumerate(lists[i]):
             n = min(64, L - p * 64)
+            if window and (p + 1) * 64 <= starts[i] - window + 1:
+                continue  # behind the window of the first new token: left as NaN
             k_pool[page, :, :n] = k[p * 64:p * 64 + n].transpose(0, 1).cuda()
             v_pool[page, :, :, :n] = v[p * 64:p * 64 + n].permute(1, 2, 0).cuda()
     q_all = torch.cat(qs).cuda()
     token_seq = torch.tensor([i for i, n in enumerate(news) for _ in range(n)], dtype=torch.int32).cuda()
     token_pos = torch.tensor([s + j for s, n in zip(starts, news) for j in range(n)], dtype=torch.int32).cuda()
-    got = fn(q_all, k_pool, v_pool, bt, token_seq, token_pos, slopes, 1.0 / math.sqrt(d), starts, news)
+    kw = {"window": window} if window else {}
+    got = fn(q_all, k_pool, v_pool, bt, token_seq, token_pos, slopes, 1.0 / math.sqrt(d), starts, news, **kw)
     at = 0
     worst = 0.0
     for i, (s, n) in enumerate(zip(starts, news)):
@@ -340,7 +357,10 @@ def _attn_case(ops, fn, dtype, nh, nkv, d, starts, news, slopes=None, seed=0, bo
         # plain attention of the whole sequence needs a query per position: only the new rows are compared
         q_full = torch.zeros(L, nh, d, dtype=torch.float64)
         q_full[s:] = qs[i].double()
-        want = P.attention_scores_softmax(q_full, ks[i].double(), vs[i].double(), bias)[s:]
+        if window:
+            want = _windowed_attention(q_full, ks[i].double(), vs[i].double(), window)[s:]
+        else:
+            want = P.attention_scores_softmax(q_full, ks[i].double(), vs[i].double(), bias)[s:]
         g_ = got[at:at + n].double().cpu()
         tol = 2e-5 if dtype == torch.float32 else 2e-2
         err = float((g_ - want).abs().max())
@@ -354,8 +374,8 @@ def _attn_case(ops, fn, dtype, nh, nkv, d, starts, news, slopes=None, seed=0, bo
 
 
 def _generic(ops):
-    def fn(q, k_pool, v_pool, bt, token_seq, token_pos, slopes, scale, starts, news):
-        return ops.attn_generic(q, k_pool, v_pool, bt, token_seq, token_pos, slopes, scale)
+    def fn(q, k_pool, v_pool, bt, token_seq, token_pos, slopes, scale, starts, news, window=0):
+        return ops.attn_generic(q, k_pool, v_pool, bt, token_seq, token_pos, slopes, scale, window)
     return fn
 
 
@@ -378,14 +398,14 @@ def test_attn_generic_far_key_and_alibi(dtype):
 
 
 def _mfma(ops, n_splits_for=None):
-    def fn(q, k_pool, v_pool, bt, token_seq, token_pos, slopes, scale, starts, news):
+    def fn(q, k_pool, v_pool, bt, token_seq, token_pos, slopes, scale, starts, news, window=0):
         cu = torch.tensor([0] + list(torch.tensor(news).cumsum(0)), dtype=torch.int32).cuda()
         st = torch.tensor(starts, dtype=torch.int32).cuda()
         n_splits = 1
         if n_splits_for is not None:
             n_splits = (max(s + n for s, n in zip(starts, news)) + n_splits_for - 1) // n_splits_for
         return ops.attn_mfma(q, k_pool, v_pool, bt, cu, st, slopes, scale, max_new=max(news), n_splits=n_splits,
-                             split_size=n_splits_for or 256)
+                             split_size=n_splits_for or 256, window=window)
     return fn
 
 
@@ -404,6 +424,20 @@ def test_attn_mfma_decode_split(nh, nkv, d, split):
     """One token per sequence, contexts of very different lengths, keys split over waves and merged."""
     ops = _ops()
     _attn_case(ops, _mfma(ops, split), torch.bfloat16, nh, nkv, d, starts=[0, 63, 64, 700, 255, 256, 1], news=[1] * 7)
+
+
+@pytest.mark.parametrize("window", [1, 33, 64, 100, 200])
+def test_attention_with_a_window(window):
+    """Each token sees its last `window` positions only; pages behind the window hold NaN and are not read.
+    Prompts longer than the window, chunks over a cache, decode steps with and without split ranges."""
+    ops = _ops()
+    starts, news = [0, 63, 300, 0, 127, 500], [70, 1, 5, 1, 2, 150]
+    for dtype in DTYPES:
+        _attn_case(ops, _generic(ops), dtype, 6, 2, 32, starts, news, window=window)
+    for nh, nkv, d in ((6, 2, 32), (71, 1, 64), (4, 4, 128)):
+        _attn_case(ops, _mfma(ops), torch.bfloat16, nh, nkv, d, starts, news, window=window)
+        _attn_case(ops, _mfma(ops, 64), torch.bfloat16, nh, nkv, d, [0, 63, 64, 700, 255, 256, 1], [1] * 7, window=window)
+        _attn_case(ops, _mfma(ops, 256), torch.bfloat16, nh, nkv, d, [900, 30], [1, 1], window=window)
 
 
 def test_attn_mfma_far_key_alibi_and_refusals():

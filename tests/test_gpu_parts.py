@@ -454,3 +454,100 @@ def test_toy_architecture_with_routing_and_its_own_positions(tmp_path):
                 helpers.assert_close(got[rid], want[rid], 5e-5, f"routed toy {name} {rid}")
     finally:
         unregister("toy-routed")
+
+
+# --- a third toy: a layer that attends to a window of the last positions, with a cache group of its own ---
+def _define_window_toy(window):
+    from pytorch_transformers_amd.config.base import ModelConfig
+    from pytorch_transformers_amd.engine.spec import CACHE_FULL, CACHE_WINDOW, CacheGroupSpec, LayerCall, ModelSpec
+    from pytorch_transformers_amd.parts import (AttentionMixer, DenseFeedForward, Embedding, LayerNorm, OutputHead,
+                                                ParallelBlock, RotaryPositions)
+
+    @dataclasses.dataclass
+    class WindowConfig(ModelConfig):
+        model_type = "toy-window"
+        vocab_size: int = 113
+        width: int = 64
+        heads: int = 2
+
+    def build(cfg):
+        d = cfg.width // cfg.heads
+        def block(i, win):
+            mixer = AttentionMixer(f"t.h.{i}.attn", cfg.width, cfg.heads, 1, d, "tail", False, RotaryPositions(d, 10000.0),
+                                   window=win)
+            return ParallelBlock(mixer, DenseFeedForward(f"t.h.{i}.mlp", cfg.width, 2 * cfg.width, bias=False),
+                                 LayerNorm(f"t.h.{i}.norm", cfg.width, 1e-5))
+        return ModelSpec(config=cfg, embedding=Embedding("t.embed", cfg.vocab_size, cfg.width),
+                         blocks=[block(0, window), block(1, 0)], order=[LayerCall(0, "near", 0), LayerCall(1, "all", 0)],
+                         final_norm=LayerNorm("t.final", cfg.width, 1e-5),
+                         head=OutputHead("t.head", cfg.vocab_size, cfg.width, "t.embed.weight"),
+                         cache_groups=[CacheGroupSpec("near", CACHE_WINDOW, 1, 1, d, window=window),
+                                       CacheGroupSpec("all", CACHE_FULL, 1, 1, d)])
+
+    return WindowConfig, build
+
+
+def _plain_window_toy(cfg, w, ids, window):
+    T, H, nh = len(ids), cfg.width, cfg.heads
+    d = H // nh
+    x = w["t.embed.weight"][torch.as_tensor(ids)]
+    cos, sin = P.rope_cos_sin(torch.arange(T), P.rope_inv_freq(d, 10000.0))
+    t = torch.arange(T)
+    for i, win in ((0, window), (1, 0)):
+        p = f"t.h.{i}"
+        a = P.layer_norm(x, w[p + ".norm.weight"], w[p + ".norm.bias"], 1e-5)
+        f = (a @ w[p + ".attn.query_key_value.weight"].T).view(T, nh + 2, d)
+        q, k, v = P.apply_rope(f[:, :nh], cos, sin), P.apply_rope(f[:, nh:nh + 1], cos, sin), f[:, nh + 1:]
+        seen = t[None, :] <= t[:, None]
+        if win:
+            seen = seen & (t[None, :] > t[:, None] - win)
+        o = torch.empty(T, nh, d, dtype=x.dtype)
+        for h in range(nh):
+            s = (q[:, h] @ k[:, 0].T / math.sqrt(d)).masked_fill(~seen, float("-inf"))
+            o[:, h] = torch.softmax(s, dim=-1) @ v[:, 0]
+        mlp = P.gelu(a @ w[p + ".mlp.dense_h_to_4h.weight"].T) @ w[p + ".mlp.dense_4h_to_h.weight"].T
+        x = x + (mlp + o.reshape(T, H) @ w[p + ".attn.dense.weight"].T)
+    return P.layer_norm(x, w["t.final.weight"], w["t.final.bias"], 1e-5) @ w["t.embed.weight"].T
+
+
+@pytest.mark.parametrize("dtype,rel", [("float32", helpers.REL_F32), ("bfloat16", helpers.REL_BF16)])
+def test_toy_architecture_with_a_window_layer(tmp_path, dtype, rel):
+    """One layer sees the last 40 positions and keeps them in a cache group of kind `window`, the other sees
+    everything: every schedule against the plain model, and the window group gives its pages back."""
+    from safetensors.torch import load_file
+
+    from pytorch_transformers_amd import AutoModelForCausalLM
+    from pytorch_transformers_amd.config import register, unregister
+    from pytorch_transformers_amd.engine.replay import Replayer
+    from pytorch_transformers_amd.weights import write_random_model
+
+    window = 40
+    WindowConfig, build = _define_window_toy(window)
+    register("toy-window", WindowConfig, build, exist_ok=True)
+    try:
+        cfg = WindowConfig()
+        folder = write_random_model(str(tmp_path / "window"), cfg, seed=3, std=0.15, noise=0.1)
+        w = {k: v.double() for k, v in load_file(f"{folder}/model.safetensors").items()}
+        model = AutoModelForCausalLM.from_pretrained(folder, dtype=dtype)
+        reqs = helpers.make_requests(cfg.vocab_size, [9, 150, 70, 41, 230], seed=6)
+        want = {rid: _plain_window_toy(cfg, w, toks, window).float() for rid, toks in reqs.items()}
+        rp = Replayer(model, 1024, max_slots=4)
+        for name, records in (("whole", helpers.schedule_whole(reqs)), ("tail", helpers.schedule_tail(reqs, 32)),
+                              ("batches", helpers.schedule_batches(reqs, 3, decode=(3, 60, 1)))):
+            got = helpers.run_schedule(rp, records)
+            for rid in reqs:
+                helpers.assert_close(got[rid], want[rid], rel, f"window toy {dtype} {name} {rid}")
+        # decoding far past the window (as captured graphs where the model allows them): the window group holds
+        # a page or two, the full group all of them
+        cache = model.new_cache(1024, max_slots=1)
+        slot = cache.alloc()
+        toks = reqs["r4"]
+        model.step(cache, [slot], [toks[:50]], "none")
+        for t in toks[50:]:
+            logits = model.step(cache, [slot], [[t]], "last")
+        helpers.assert_close(logits[0].float().cpu()[None], want["r4"][-1:], rel, f"window toy {dtype} long decode")
+        held = [p for p in cache.page_list("near", slot) if p >= 0]
+        assert len(held) <= 2 and len(cache.page_list("all", slot)) == 4
+        cache.check_consistent()
+    finally:
+        unregister("toy-window")
