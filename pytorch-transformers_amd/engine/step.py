@@ -55,26 +55,6 @@ class StepPlan:
         return max(s + n for s, n in zip(self.starts, self.new_tokens))
 
 
-def normalize_want(want: Want, new_tokens: Sequence[int]) -> List[List[int]]:
-    """``"last"``, ``"all"``, ``None`` (nothing) or explicit places per sequence -> lists of places."""
-    if want is None or want == "none":
-        return [[] for _ in new_tokens]
-    if want == "last":
-        return [[n - 1] for n in new_tokens]
-    if want == "all":
-        return [list(range(n)) for n in new_tokens]
-    if isinstance(want, str):
-        raise StepError(f"want must be 'last', 'all', 'none' or a list of places per sequence, got {want!r}")
-    want = [list(w) for w in want]
-    if len(want) != len(new_tokens):
-        raise StepError(f"want has {len(want)} entries for {len(new_tokens)} sequences")
-    for i, (w, n) in enumerate(zip(want, new_tokens)):
-        for p in w:
-            if not (0 <= int(p) < n):
-                raise StepError(f"sequence {i} wants the logits at place {p}, but brings {n} tokens")
-    return want
-
-
 _WANT_MODES = {"none": 0, "last": 1, "all": 2}
 
 

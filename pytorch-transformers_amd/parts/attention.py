@@ -11,7 +11,7 @@ causal mask is implied by each token's position instead of being a tensor.
 from __future__ import annotations
 
 import math
-from typing import List, Optional, Sequence
+from typing import Optional, Sequence
 
 import torch
 

@@ -18,7 +18,7 @@ from typing import Optional, Sequence
 
 import torch
 
-from .base import Part, PartialProduct, ResidualSum, StepContext, register_part
+from .base import Part, ResidualSum, StepContext, register_part
 from .linear import Linear, PendingProjection
 
 
