@@ -81,14 +81,16 @@ __device__ __forceinline__ void load_block(KvBlock<DT>& b, int kb, const int* __
 // W = 1: a workgroup is one wave, which loads its keys and values straight from global memory.
 // W = 4 (prompts): four waves with neighbouring column groups walk the keys together and share every
 // block through LDS, so that a block crosses the vector memory path once for 64 * CT columns.
-template <int DT, int CT, int W>
+// WIN: the launch has a window (a kernel of its own, so that launches without one pay nothing for it).
+template <int DT, int CT, int W, bool WIN>
 __global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
     bf16_t* __restrict__ out, float* __restrict__ po, float* __restrict__ pm, float* __restrict__ pl,
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
     const int* __restrict__ block_table, int bt_stride, const int* __restrict__ cu_tokens,
     const int* __restrict__ seq_start, const float* __restrict__ slopes, int nh, int nkv, float scale, float alibi_mul,
-    int split_size, int n_splits, int window) {
+    int split_size, int n_splits, int window_arg) {
     constexpr int D = DT * 16;
+    const int window = WIN ? window_arg : 0;
     constexpr int DS = (DT + 1) / 2;   // 32-wide steps over the head dimension
     constexpr int CHUNKS = D / 8;      // 16-byte chunks in a row of d elements
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, gq = lane >> 4;
@@ -346,7 +348,10 @@ __global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
                 *reinterpret_cast<uint2*>(o + dt * 16 + gq * 4) = w;
             }
         } else {
-            if (k_begin < k_end) {  // a range past the column's keys has nothing to add: only its marker is written
+            // a range past the column's keys has nothing to add: only its marker is written, and the combine
+            // does not read past the last range that has one.  A range before a window is followed by ranges
+            // that count, so it is read with weight zero and must hold numbers: the (zero) sums are written.
+            if (k_begin < k_end || WIN) {
                 float* o = po + (row * n_splits + split) * D;
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt)
@@ -392,11 +397,9 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(bf16_t* __restrict__ o
         int s = 0;
         for (; s + 4 <= used; s += 4) {
             const float v0 = p[(long)s * D], v1 = p[(long)(s + 1) * D], v2 = p[(long)(s + 2) * D], v3 = p[(long)(s + 3) * D];
-            // a range with weight zero was never written (past the row's keys, or before its window)
-            acc += w_s[s] != 0.f ? w_s[s] * v0 : 0.f; acc += w_s[s + 1] != 0.f ? w_s[s + 1] * v1 : 0.f;
-            acc += w_s[s + 2] != 0.f ? w_s[s + 2] * v2 : 0.f; acc += w_s[s + 3] != 0.f ? w_s[s + 3] * v3 : 0.f;
+            acc += w_s[s] * v0; acc += w_s[s + 1] * v1; acc += w_s[s + 2] * v2; acc += w_s[s + 3] * v3;
         }
-        for (; s < used; ++s) acc += w_s[s] != 0.f ? w_s[s] * p[(long)s * D] : 0.f;
+        for (; s < used; ++s) acc += w_s[s] * p[(long)s * D];
         out[row * D + dd] = f32_to_bf16_bits(acc * inv);
     }
 }
@@ -408,7 +411,8 @@ static void launch_attn(bf16_t* out, float* po, float* pm, float* pl, const bf16
                         int split_size, int n_splits, int window, hipStream_t s) {
     const int g = nh / nkv;
     const dim3 grid((max_new * g + 16 * CT * W - 1) / (16 * CT * W), nkv, n_seqs * n_splits);
-    hipLaunchKernelGGL((attn_mfma_kernel<DT, CT, W>), grid, dim3(64 * W), 0, s, out, po, pm, pl, q, k_pool, v_pool, block_table,
+    auto kern = window > 0 ? attn_mfma_kernel<DT, CT, W, true> : attn_mfma_kernel<DT, CT, W, false>;
+    hipLaunchKernelGGL(kern, grid, dim3(64 * W), 0, s, out, po, pm, pl, q, k_pool, v_pool, block_table,
                        bt_stride, cu_tokens, seq_start, slopes, nh, nkv, scale * PTA_LOG2E,
                        PTA_LOG2E / sqrtf((float)(DT * 16)), split_size, n_splits, window);
 }
