@@ -82,6 +82,20 @@ def test_long_decoding(folders, name, dtype, rel):
 
 
 @pytest.mark.parametrize("dtype,rel", [("float32", REL_F32), ("bfloat16", REL_BF16)])
+def test_decoding_across_the_length_bound_of_a_captured_step(folders, dtype, rel):
+    """Three sequences of unequal lengths decode together across position 1,024, where the captured decode
+    step is replaced by one sized for longer contexts (more key ranges, another page-table width), and the
+    shortest leaves the batch on the way."""
+    lens = [1075, 1010, 700]
+    reqs = helpers.make_requests(TINY["D"]["vocab_size"], lens, seed=11)
+    want = helpers.plain_logits(folders["D"], reqs)
+    rp = _replayer(folders["D"], dtype, max_tokens=3 * 1088)
+    got = helpers.run_schedule(rp, helpers.schedule_batches(reqs, 3, decode=(90, 40, 12)))
+    for rid in reqs:
+        helpers.assert_close(got[rid], want[rid], rel, f"D {dtype} across 1024 {rid}")
+
+
+@pytest.mark.parametrize("dtype,rel", [("float32", REL_F32), ("bfloat16", REL_BF16)])
 def test_first_tokens(folders, dtype, rel):
     """The first tokens of a sequence, fed one at a time from an empty slot."""
     reqs = helpers.make_requests(TINY["A"]["vocab_size"], [6], seed=11)
