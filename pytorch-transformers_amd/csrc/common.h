@@ -82,6 +82,22 @@ __device__ __forceinline__ float block_max(float v, float* red) {
     return t;
 }
 
+// eight bfloat16 in sixteen bytes <-> eight floats
+__device__ __forceinline__ void unpack8(const uint4& u, float (&f)[8]) {
+    const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        f[2 * p] = bf16_bits_to_f32((bf16_t)(w[p] & 0xffffu));
+        f[2 * p + 1] = bf16_bits_to_f32((bf16_t)(w[p] >> 16));
+    }
+}
+__device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
+    uint32_t w[4];
+#pragma unroll
+    for (int p = 0; p < 4; ++p) w[p] = (uint32_t)f32_to_bf16_bits(f[2 * p]) | ((uint32_t)f32_to_bf16_bits(f[2 * p + 1]) << 16);
+    return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
 // exact GELU, 0.5 x (1 + erf(x / sqrt 2))  (src/transformers/activations.py:59-78)
 __device__ __forceinline__ float gelu_erf(float x) { return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f)); }
 

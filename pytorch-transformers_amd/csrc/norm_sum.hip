@@ -20,20 +20,6 @@
 #define NS_THREADS 1024  // at most
 #define NS_MAX_H (NS_THREADS * 8)
 
-__device__ __forceinline__ void unpack8(const uint4& u, float (&f)[8]) {
-    const uint32_t w[4] = {u.x, u.y, u.z, u.w};
-#pragma unroll
-    for (int p = 0; p < 4; ++p) {
-        f[2 * p] = bf16_bits_to_f32((bf16_t)(w[p] & 0xffffu));
-        f[2 * p + 1] = bf16_bits_to_f32((bf16_t)(w[p] >> 16));
-    }
-}
-__device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
-    uint32_t w[4];
-#pragma unroll
-    for (int p = 0; p < 4; ++p) w[p] = (uint32_t)f32_to_bf16_bits(f[2 * p]) | ((uint32_t)f32_to_bf16_bits(f[2 * p + 1]) << 16);
-    return make_uint4(w[0], w[1], w[2], w[3]);
-}
 __device__ __forceinline__ void load8f(const float* p, float (&f)[8]) {
     const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
     f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;

@@ -46,6 +46,39 @@ __global__ __launch_bounds__(RC_THREADS) void qkv_rope_cache_kernel(
     const int rot_slots = inv_freq ? min(n_slots, nh + nkv) : 0;
     // gridDim.y workgroups share a token's items (a decode step has few tokens and many heads)
     const int stride = RC_THREADS * gridDim.y, first = tid + blockIdx.y * RC_THREADS;
+    if (sizeof(T) == 2 && (d & 15) == 0) {
+        // bfloat16 with halves that are multiples of eight: eight pairs per item, sixteen bytes per access
+        const int h8 = half >> 3;
+        for (int item = first; item < rot_slots * h8; item += stride) {
+            const int slot = item / h8, i = (item - slot * h8) * 8;
+            const int kind = slot < nh ? 0 : 1, head = slot < nh ? slot : slot - nh;
+            int src_head;
+            if (layout == PTA_QKV_GROUPED) src_head = kind == 0 ? (head / g) * (g + 2) + (head % g) : head * (g + 2) + g;
+            else if (layout == PTA_QKV_TAIL) src_head = kind == 0 ? head : nh;
+            else src_head = head * 3 + kind;
+            const bf16_t* src = (const bf16_t*)row + (long)src_head * d;
+            float a[8], b[8], lo[8], hi[8];
+            unpack8(*reinterpret_cast<const uint4*>(src + i), a);
+            unpack8(*reinterpret_cast<const uint4*>(src + i + half), b);
+            if (bias) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    a[e] = round_to_bf16(a[e] + bias[(long)src_head * d + i + e]);
+                    b[e] = round_to_bf16(b[e] + bias[(long)src_head * d + i + half + e]);
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float c = cos_s[i + e], s = sin_s[i + e];
+                lo[e] = a[e] * c - b[e] * s;
+                hi[e] = b[e] * c + a[e] * s;
+            }
+            bf16_t* dst = kind == 0 ? (bf16_t*)q_out + ((long)m * nh + head) * d
+                                    : (bf16_t*)k_pool + ((page * nkv + head) * PTA_PAGE + in_page) * (long)d;
+            *reinterpret_cast<uint4*>(dst + i) = pack8(lo);
+            *reinterpret_cast<uint4*>(dst + i + half) = pack8(hi);
+        }
+    } else {
     for (int item = first; item < rot_slots * half; item += stride) {
         const int slot = item / half, i = item - slot * half;
         const int kind = slot < nh ? 0 : 1, head = slot < nh ? slot : slot - nh;
@@ -64,6 +97,7 @@ __global__ __launch_bounds__(RC_THREADS) void qkv_rope_cache_kernel(
                            : k_pool + ((page * nkv + head) * PTA_PAGE + in_page) * (long)d;
         Io<T>::st(dst + i, a * c - b * s);
         Io<T>::st(dst + i + half, b * c + a * s);
+    }
     }
     for (int item = first + rot_slots * d; item < n_slots * d; item += stride) {
         const int slot = item / d, i = item - slot * d;
@@ -94,6 +128,9 @@ extern "C" int pta_qkv_rope_cache(void* q_out, const void* fused, const float* b
     PTA_REQUIRE(layout != PTA_QKV_INTERLEAVED || nkv == nh, "qkv_rope_cache: the interleaved layout needs kv heads == heads");
     PTA_REQUIRE(!inv_freq || (d % 2 == 0 && d <= 256), "qkv_rope_cache: rotation needs an even head size up to 256, got %d", d);
     PTA_REQUIRE(!write_cache || (k_pool && v_pool && block_table && token_seq), "qkv_rope_cache: null cache pointer");
+    PTA_REQUIRE(dtype != PTA_BF16 || d % 16 != 0 ||
+                    (((uintptr_t)fused | (uintptr_t)q_out | (uintptr_t)k_pool) % 16) == 0,
+                "qkv_rope_cache: bfloat16 rows are moved sixteen bytes at a time and must be aligned so");
     hipStream_t s = (hipStream_t)stream;
     int slices = 1;  // enough workgroups to occupy the chip when the step has few tokens
     while (slices < 16 && M * slices < 512 && slices * RC_THREADS < (nh + 2 * nkv) * d) slices *= 2;
