@@ -336,4 +336,65 @@ int ptah_plan_step(void* h, int n, const int* slots, const int* new_tokens, cons
 
 const int* ptah_plan_data(void* h) { return static_cast<Cache*>(h)->plan.data(); }
 
+// The common step of decoding, without the general planner's detours: every sequence brings one token and
+// wants its logits.  Checks the step, reserves its pages and reports the longest context after it.
+int ptah_decode_prepare(void* h, int n, const int* slots, const long long* tokens, int vocab, int* max_len_out) {
+    Cache* c = static_cast<Cache*>(h);
+    if (n <= 0) return fail(ERR_STEP, "a step needs at least one sequence");
+    for (int i = 0; i < n; ++i)
+        if (tokens[i] < 0 || tokens[i] >= vocab)
+            return fail(ERR_STEP, "token id %lld is outside the vocabulary [0, %d)", tokens[i], vocab);
+    std::vector<int> ones(n, 1);
+    const int rc = ptah_reserve(h, n, slots, ones.data());
+    if (rc) return rc;
+    int longest = 0;
+    for (int i = 0; i < n; ++i) longest = std::max(longest, c->length[slots[i]] + 1);
+    *max_len_out = longest;
+    return OK;
+}
+
+// ... and lays it out for a captured decode step of n_rows >= n sequences whose page tables are `width` pages
+// wide, straight into the buffer that is copied to the device:
+//   token_ids | token_seq | token_pos [n_rows each] | cu_tokens [n_rows + 1] | seq_start | seq_slot |
+//   logit_rows [n_rows each] | one page table [n_rows, width] per paged group
+// Rows past n repeat sequence 0 (the same token at the same place writes the same keys and values again).
+int ptah_decode_fill(void* h, int n, const int* slots, const long long* tokens, int n_rows, int width, int32_t* out) {
+    Cache* c = static_cast<Cache*>(h);
+    if (n <= 0 || n_rows < n) return fail(ERR_STEP, "decode layout for %d rows cannot hold %d sequences", n_rows, n);
+    int32_t *ids = out, *seq = ids + n_rows, *pos = seq + n_rows, *cu = pos + n_rows, *start = cu + n_rows + 1;
+    int32_t *slot = start + n_rows, *rows = slot + n_rows, *table = rows + n_rows;
+    for (int r = 0; r < n_rows; ++r) {
+        const int i = r < n ? r : 0;
+        const int len = c->length[slots[i]];
+        ids[r] = (int32_t)tokens[i];
+        seq[r] = r;
+        pos[r] = len;
+        cu[r] = r;
+        start[r] = len;
+        slot[r] = slots[i];
+        rows[r] = r;
+    }
+    cu[n_rows] = n_rows;
+    for (const Group& gr : c->groups) {
+        for (int r = 0; r < n_rows; ++r) {
+            const std::vector<int>& l = gr.lists[slots[r < n ? r : 0]];
+            if ((int)l.size() > width) return fail(ERR_STEP, "a sequence holds %zu pages, the layout has room for %d", l.size(), width);
+            int32_t* row = table + (long)r * width;
+            for (size_t k = 0; k < l.size(); ++k) row[k] = std::max(0, l[k]);
+            for (int k = (int)l.size(); k < width; ++k) row[k] = 0;
+        }
+        table += (long)n_rows * width;
+    }
+    return OK;
+}
+
+// every listed slot grew by one token
+int ptah_commit_ones(void* h, int n, const int* slots) {
+    Cache* c = static_cast<Cache*>(h);
+    for (int i = 0; i < n; ++i)
+        if (!c->slots.is_held(slots[i])) return fail(ERR_CACHE, "slot %d is not allocated", slots[i]);
+    for (int i = 0; i < n; ++i) c->length[slots[i]] += 1;
+    return OK;
+}
+
 }  // extern "C"

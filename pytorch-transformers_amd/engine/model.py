@@ -12,16 +12,19 @@ from __future__ import annotations
 
 from typing import Dict, Optional, Sequence
 
+import ctypes
+
 import numpy as np
 import torch
 
+from .. import host
 from ..cache.paged import PagedCache
 from ..config.registry import AutoConfig, lookup
 from ..parts.base import ResidualSum, StepContext, as_tensor
 from ..weights.loader import load_weights
 from ..weights.random_init import random_tensors
 from .spec import ModelSpec
-from .step import StepPlan, Want, plan_step
+from .step import StepError, StepPlan, Want, plan_step
 
 _DTYPES = {"float32": torch.float32, "fp32": torch.float32, "bfloat16": torch.bfloat16, "bf16": torch.bfloat16,
            torch.float32: torch.float32, torch.bfloat16: torch.bfloat16}
@@ -110,6 +113,29 @@ class _DecodeGraph:
 
     def run(self, plan: StepPlan) -> torch.Tensor:
         self._fill(plan)
+        self._replay()
+        k = plan.n_seqs
+        rows = plan.logit_rows
+        if rows.shape[0] == k:  # one row per sequence, in order: the first k rows as they are
+            return self.logits[:k]
+        if rows.shape[0] == 0:
+            return self.logits[:0]
+        return self.logits.index_select(0, torch.from_numpy(rows.astype(np.int64)).to(self.logits.device))
+
+    def run_last(self, n: int, slots_c, tokens_c) -> torch.Tensor:
+        """The common case, laid out by the host runtime straight into the pinned buffer: ``n`` sequences, one
+        token each (C arrays), the logits of each."""
+        self.copied.synchronize()  # the last copy out of the pinned buffer is done
+        lib = host.load()
+        rc = lib.ptah_decode_fill(self.cache.handle, n, slots_c, tokens_c, self.n, self.width, self.host.data_ptr())
+        if rc:
+            raise StepError(host.last_error())
+        self.dev.copy_(self.host, non_blocking=True)
+        self.copied.record()
+        self._replay()
+        return self.logits[:n]
+
+    def _replay(self) -> None:
         if self.graph is None:
             ctx, ids, rows = self._context()
             side = torch.cuda.Stream()
@@ -121,13 +147,6 @@ class _DecodeGraph:
             with torch.cuda.graph(self.graph):
                 self.logits = self.model.forward_tokens(ctx, ids, rows)
         self.graph.replay()
-        k = plan.n_seqs
-        rows = plan.logit_rows
-        if rows.shape[0] == k:  # one row per sequence, in order: the first k rows as they are
-            return self.logits[:k]
-        if rows.shape[0] == 0:
-            return self.logits[:0]
-        return self.logits.index_select(0, torch.from_numpy(rows.astype(np.int64)).to(self.logits.device))
 
 
 class CausalLM:
@@ -250,9 +269,11 @@ class CausalLM:
 
     # decode steps as HIP graphs ---------------------------------------------------------
     def _graph_for(self, cache: PagedCache, plan: StepPlan) -> "_DecodeGraph":
-        n = plan.n_seqs
+        return self._graph_for_sizes(cache, plan.n_seqs, plan.max_len)
+
+    def _graph_for_sizes(self, cache: PagedCache, n: int, max_len: int) -> "_DecodeGraph":
         n_bucket = n if n <= 8 else (n + 7) // 8 * 8
-        len_bound = (plan.max_len + GRAPH_LEN_STEP - 1) // GRAPH_LEN_STEP * GRAPH_LEN_STEP
+        len_bound = (max_len + GRAPH_LEN_STEP - 1) // GRAPH_LEN_STEP * GRAPH_LEN_STEP
         graphs = cache.__dict__.setdefault("_decode_graphs", {})
         key = (id(self), n_bucket, len_bound)
         g = graphs.get(key)
@@ -269,6 +290,8 @@ class CausalLM:
         of this step whose logits are asked for.  Rows come in the order of the sequences and of
         their places.
         """
+        if self.use_graphs and want == "last" and len(tokens) == len(slots) and all(len(t) == 1 for t in tokens):
+            return self._decode_last(cache, slots, tokens)
         plan = plan_step(cache, slots, tokens, want, self.vocab_size)
         if self.use_graphs and plan.is_decode:
             logits = self._graph_for(cache, plan).run(plan)
@@ -279,6 +302,26 @@ class CausalLM:
         cache.commit(plan.slots, plan.new_tokens)
         if logits is None:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
+        return logits
+
+    def _decode_last(self, cache: PagedCache, slots: Sequence[int], tokens: Sequence[Sequence[int]]) -> torch.Tensor:
+        """One token per sequence, the logits of each, as a replay of a captured step: the host runtime checks
+        the step, reserves pages and writes the step's integers straight into the buffer that is copied to
+        the device."""
+        from ..cache.paged import CacheError, CacheFull
+
+        n = len(slots)
+        if n == 0:
+            raise StepError("a step needs at least one sequence")
+        lib = host.load()
+        slots_c = (ctypes.c_int * n)(*[int(s) for s in slots])
+        tokens_c = (ctypes.c_longlong * n)(*[int(t[0]) for t in tokens])
+        longest = ctypes.c_int(0)
+        rc = lib.ptah_decode_prepare(cache.handle, n, slots_c, tokens_c, self.vocab_size, ctypes.byref(longest))
+        if rc:
+            raise {host.ERR_STEP: StepError, host.ERR_FULL: CacheFull}.get(rc, CacheError)(host.last_error())
+        logits = self._graph_for_sizes(cache, n, longest.value).run_last(n, slots_c, tokens_c)
+        lib.ptah_commit_ones(cache.handle, n, slots_c)
         return logits
 
     # generation (see engine.generate) -----------------------------------------------

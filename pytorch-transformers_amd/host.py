@@ -53,6 +53,10 @@ def load():
         lib.ptah_pages.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, _P_INT]
         lib.ptah_plan_step.argtypes = [ctypes.c_void_p, ctypes.c_int, _P_INT, _P_INT, _P_LL, ctypes.c_int, ctypes.c_int,
                                        _P_INT, _P_INT, _P_INT]
+        lib.ptah_decode_prepare.argtypes = [ctypes.c_void_p, ctypes.c_int, _P_INT, _P_LL, ctypes.c_int, _P_INT]
+        lib.ptah_decode_fill.argtypes = [ctypes.c_void_p, ctypes.c_int, _P_INT, _P_LL, ctypes.c_int, ctypes.c_int,
+                                         ctypes.c_void_p]
+        lib.ptah_commit_ones.argtypes = [ctypes.c_void_p, ctypes.c_int, _P_INT]
         lib.ptah_plan_data.argtypes = [ctypes.c_void_p]
         lib.ptah_plan_data.restype = _P_INT
         _lib = lib

@@ -41,6 +41,11 @@ class Sampler:
         """Tokens for the rows of ``logits`` and the processed scores ``[rows, vocab]`` (None if not needed
         and the choice could be made without forming them)."""
         R = logits.shape[0]
+        suppress = self._eos_dev is not None and suppress_eos is not None and any(suppress_eos)
+        if (not need_scores and not self.do_sample and self.penalty == 1.0 and not suppress
+                and not self.config.remove_invalid_values and not self.config.renormalize_logits):
+            # greedy with no processor in the way: nothing to upload, one argmax kernel
+            return ops.sample(logits, do_sample=False, need_scores=False)[0].tolist(), None
         use_hist = self.penalty != 1.0 and histories is not None
         pieces = [np.asarray(rng_seq, dtype=np.int32), np.asarray(rng_step, dtype=np.int32),
                   np.asarray([1 if s else 0 for s in (suppress_eos or [False] * R)], dtype=np.int32)]
