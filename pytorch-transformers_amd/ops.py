@@ -337,6 +337,75 @@ def sample(logits: torch.Tensor, *, do_sample: bool, temperature: float = 1.0, t
 
 SKINNY_MAX_ROWS = 64
 
+# ---- the vendor library's product for many rows, cut along M where that is faster -----------------------
+# The library picks a kernel per (M, N, K) from a table, and on this hardware its choices are uneven in M:
+# at Falcon-7B shapes 2,048 rows of the feed-forward's first product take longer than 2,304, and 4,096 rows of
+# its second one almost as long as 8,192.  So for every weight shape the product is timed once at a ladder of
+# row counts, and a product of M rows runs as the cheapest sequence of those pieces (each written straight
+# into its rows of the result).  PTA_MM_CHUNKS=0 switches this off.
+MM_LADDER = (256, 512, 768, 1024, 1536, 2048, 3072, 4096, 6144, 8192)
+MM_CHUNKS = os.environ.get("PTA_MM_CHUNKS", "1") != "0"
+_mm_times: dict = {}  # (N, K) -> {rows: microseconds}
+_mm_plans: dict = {}  # (N, K, M) -> [rows, ...]
+
+
+def _mm_measure(x: torch.Tensor, w: torch.Tensor, rows: int, out: torch.Tensor) -> float:
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for _ in range(2):  # the library's first calls of a shape set it up
+        torch.mm(x[:rows], w.t(), out=out[:rows])
+    start.record()
+    for _ in range(3):
+        torch.mm(x[:rows], w.t(), out=out[:rows])
+    end.record()
+    end.synchronize()
+    return start.elapsed_time(end) / 3 * 1e3
+
+
+def _mm_plan(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor):
+    M, (N, K) = x.shape[0], w.shape
+    bucket = (M + 63) // 64  # row counts within 64 of each other share a plan: one timing of the whole product
+    plan = _mm_plans.get((N, K, bucket))
+    if plan is not None:
+        return plan[:-1] + [M - sum(plan[:-1])]
+    times = _mm_times.setdefault((N, K), {})
+    for rows in MM_LADDER:
+        if rows <= M and rows not in times:
+            times[rows] = _mm_measure(x, w, rows, out)
+    if M not in times:
+        times[M] = _mm_measure(x, w, M, out)  # the product as it is
+    # cheapest way to cover M rows with pieces of the ladder; what is left over rides on the last piece
+    units, rest = divmod(M, 256)
+    best = [(0.0, [])] + [None] * units
+    for u in range(1, units + 1):
+        for rows in MM_LADDER:
+            k = rows // 256
+            if k <= u and rows in times and best[u - k] is not None:
+                cand = best[u - k][0] + times[rows]
+                if best[u] is None or cand < best[u][0]:
+                    best[u] = (cand, best[u - k][1] + [rows])
+    cost, pieces = best[units]
+    if rest:
+        pieces = pieces[:-1] + [pieces[-1] + rest]
+        cost *= M / (M - rest)
+    plan = pieces if len(pieces) > 1 and cost < 0.97 * times[M] else [M]
+    _mm_plans[(N, K, bucket)] = plan
+    return plan
+
+
+def library_mm(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """``x @ w.T`` in bfloat16 through the vendor library, in the pieces along M that were measured fastest."""
+    M, N = x.shape[0], w.shape[0]
+    if not MM_CHUNKS or M < 512 or torch.cuda.is_current_stream_capturing():
+        return torch.mm(x, w.t())
+    out = torch.empty((M, N), dtype=x.dtype, device=x.device)
+    plan = _mm_plan(x, w, out)
+    at = 0
+    for rows in plan:
+        torch.mm(x[at:at + rows], w.t(), out=out[at:at + rows])
+        at += rows
+    return out
+
+
 
 def gemm_skinny_pair_bf16(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tensor, w2: torch.Tensor, bias1=None, act1=None,
                           bias2=None, act2=None):

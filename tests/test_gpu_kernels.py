@@ -218,6 +218,30 @@ def test_gemm_splitk_pair():
     assert torch.equal(a1, y1[17:37]) and torch.equal(a2, y2[17:37])
 
 
+def test_library_mm_in_pieces():
+    """The vendor library's product cut along M: forced here by made-up timings, since what is faster is the
+    machine's business; the pieces cover every row once and the result is the library's."""
+    ops = _ops()
+    N, K = 136, 264
+    w = _rand(N, K, seed=1, dtype=torch.bfloat16, scale=0.05)
+    ops._mm_times[(N, K)] = {256: 1.0, 512: 50.0, 1000: 1e6, 1030: 1e6}  # pieces of 256 look cheapest
+    try:
+        for M in (1000, 1030, 700):
+            x = _rand(M, K, seed=M, dtype=torch.bfloat16)
+            y = ops.library_mm(x, w)
+            plan = ops._mm_plans[(N, K, (M + 63) // 64)]
+            if M != 700:
+                assert len(plan) > 1 and sum(plan) == M and all(p >= 256 for p in plan), plan
+            torch.testing.assert_close(y.float(), torch.mm(x, w.t()).float(), rtol=2e-2, atol=2e-2)
+        # another row count of the same bucket reuses the plan, its last piece adjusted
+        x = _rand(1001, K, seed=7, dtype=torch.bfloat16)
+        torch.testing.assert_close(ops.library_mm(x, w).float(), torch.mm(x, w.t()).float(), rtol=2e-2, atol=2e-2)
+    finally:
+        ops._mm_times.pop((N, K), None)
+        for key in [k for k in ops._mm_plans if k[:2] == (N, K)]:
+            ops._mm_plans.pop(key)
+
+
 def test_gemm_skinny_refuses_what_it_cannot_do():
     ops = _ops()
     x, w = _rand(65, 64, dtype=torch.bfloat16), _rand(32, 64, dtype=torch.bfloat16)
