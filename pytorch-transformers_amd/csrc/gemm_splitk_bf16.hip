@@ -337,17 +337,36 @@ extern "C" int pta_gemm_splitk_bf16(void* y, float* part, const void* x, const v
     return launch_rows<2, 2, 4>(MT, a, none, M, reduce, s);
 }
 
+// Ranges of K for the two products of a pair launch: the one with more work is cut as it would be on its own,
+// the other into ranges of about the same length, so that the launch's workgroups are of a size and the
+// smaller product leaves no more partial sums than it must.
+static void pick_pair_parts(int N1, int K1, int N2, int K2, int* p1, int* p2) {
+    const bool first_big = (long)N1 * K1 >= (long)N2 * K2;
+    const int Nb = first_big ? N1 : N2, Kb = first_big ? K1 : K2, Ns = first_big ? N2 : N1, Ks = first_big ? K2 : K1;
+    const int pb = pick_parts(Nb, Kb, 1);
+    const int range = (Kb + pb - 1) / pb;
+    const int ps = max(1, min(pick_parts(Ns, Ks, 1), (Ks + range / 2) / range));
+    *p1 = effective_parts(K1, first_big ? pb : ps);
+    *p2 = effective_parts(K2, first_big ? ps : pb);
+}
+
+extern "C" int pta_gemm_splitk_pair_parts(int N1, int K1, int N2, int K2, int* p1, int* p2) {
+    if (N1 <= 0 || K1 <= 0 || N2 <= 0 || K2 <= 0) return pta_fail("gemm_splitk_pair_parts: sizes must be positive");
+    pick_pair_parts(N1, K1, N2, K2, p1, p2);
+    return 0;
+}
+
 // Two products of one launch, both left as partial sums: part1 [parts1, M, N1] of x1 . W1^T and part2
-// [parts2, M, N2] of x2 . W2^T, with the ranges pta_gemm_splitk_parts(N, K, 0, 1) gives for each.
+// [parts2, M, N2] of x2 . W2^T, with the ranges pta_gemm_splitk_pair_parts gives.
 extern "C" int pta_gemm_splitk_pair_bf16(float* part1, const void* x1, const void* W1, int N1, int K1, float* part2,
                                          const void* x2, const void* W2, int N2, int K2, int M, void* stream) {
     if (check_splitk("gemm_splitk_pair_bf16", x1, W1, M, N1, K1)) return 1;
     if (check_splitk("gemm_splitk_pair_bf16", x2, W2, M, N2, K2)) return 1;
     PTA_REQUIRE(part1 && part2, "gemm_splitk_pair_bf16: null workspace");
-    const SplitkProblem a = make_problem(nullptr, part1, x1, W1, nullptr, nullptr, nullptr, N1, K1, 0, 0, 1,
-                                         pick_parts(N1, K1, 1), 0);
-    const SplitkProblem b = make_problem(nullptr, part2, x2, W2, nullptr, nullptr, nullptr, N2, K2, 0, 0, 1,
-                                         pick_parts(N2, K2, 1), 0);
+    int p1, p2;
+    pick_pair_parts(N1, K1, N2, K2, &p1, &p2);
+    const SplitkProblem a = make_problem(nullptr, part1, x1, W1, nullptr, nullptr, nullptr, N1, K1, 0, 0, 1, p1, 0);
+    const SplitkProblem b = make_problem(nullptr, part2, x2, W2, nullptr, nullptr, nullptr, N2, K2, 0, 0, 1, p2, 0);
     return launch_rows<1, 2, 2>((M + 15) / 16, a, b, M, 0, (hipStream_t)stream);
 }
 
@@ -363,7 +382,8 @@ extern "C" int pta_gemm_splitk_pair_reduced_bf16(void* y1, float* part1, const v
     const int rc = pta_gemm_splitk_pair_bf16(part1, x1, W1, N1, K1, part2, x2, W2, N2, K2, M, stream);
     if (rc) return rc;
     const long MN1 = (long)M * N1, MN2 = (long)M * N2;
-    const int P1 = effective_parts(K1, pick_parts(N1, K1, 1)), P2 = effective_parts(K2, pick_parts(N2, K2, 1));
+    int P1, P2;
+    pick_pair_parts(N1, K1, N2, K2, &P1, &P2);
     hipLaunchKernelGGL(gemm_splitk_reduce2_kernel, dim3((unsigned)((MN1 + MN2 + 255) / 256)), dim3(256), 0,
                        (hipStream_t)stream, (bf16_t*)y1, part1, bias1, MN1, N1, P1, act1, (bf16_t*)y2, part2, bias2, MN2, N2,
                        P2, act2);

@@ -91,7 +91,8 @@ int pta_gemm_splitk_bf16(void* y, float* part, const void* x, const void* W, con
                          int stage_blocks, int depth, int reduce, void* stream);
 int pta_gemm_splitk_parts(int N, int K, int parts, int rt);
 // two products of one launch, both left as partial sums: part1 [parts1, M, N1], part2 [parts2, M, N2], with the
-// ranges pta_gemm_splitk_parts(N, K, 0, 1) gives for each
+// ranges pta_gemm_splitk_pair_parts gives
+int pta_gemm_splitk_pair_parts(int N1, int K1, int N2, int K2, int* parts1, int* parts2);
 int pta_gemm_splitk_pair_bf16(float* part1, const void* x1, const void* W1, int N1, int K1, float* part2,
                               const void* x2, const void* W2, int N2, int K2, int M, void* stream);
 

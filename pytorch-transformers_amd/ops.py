@@ -468,6 +468,13 @@ def gemm_splitk_partial(x: torch.Tensor, w: torch.Tensor, rt: int = 0, parts: in
     return part
 
 
+def gemm_splitk_pair_parts(N1: int, K1: int, N2: int, K2: int):
+    """How many ranges of K each product of a pair launch is cut into."""
+    p1, p2 = ctypes.c_int(0), ctypes.c_int(0)
+    _call("pta_gemm_splitk_pair_parts", int(N1), int(K1), int(N2), int(K2), ctypes.byref(p1), ctypes.byref(p2))
+    return p1.value, p2.value
+
+
 def gemm_splitk_pair_partial(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tensor, w2: torch.Tensor):
     """(x1 @ w1.T, x2 @ w2.T), both left as 32-bit partial sums, in one launch; the products share M."""
     for name, t in (("x1", x1), ("w1", w1), ("x2", x2), ("w2", w2)):
@@ -478,8 +485,9 @@ def gemm_splitk_pair_partial(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tenso
                           f"w2 {tuple(w2.shape)}")
     lib = load_library()
     (N1, K1), (N2, K2) = w1.shape, w2.shape
-    part1 = torch.empty((int(lib.pta_gemm_splitk_parts(N1, K1, 0, 1)), M, N1), dtype=torch.float32, device=x1.device)
-    part2 = torch.empty((int(lib.pta_gemm_splitk_parts(N2, K2, 0, 1)), M, N2), dtype=torch.float32, device=x1.device)
+    p1, p2 = gemm_splitk_pair_parts(N1, K1, N2, K2)
+    part1 = torch.empty((p1, M, N1), dtype=torch.float32, device=x1.device)
+    part2 = torch.empty((p2, M, N2), dtype=torch.float32, device=x1.device)
     _call("pta_gemm_splitk_pair_bf16", _ptr(part1), _ptr(x1), _ptr(w1), N1, K1, _ptr(part2), _ptr(x2), _ptr(w2), N2, K2,
           M, _stream())
     return part1, part2
@@ -501,8 +509,9 @@ def gemm_splitk_pair_bf16(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tensor, 
         _need(bias1, "bias1", torch.float32, (N1,))
     if bias2 is not None:
         _need(bias2, "bias2", torch.float32, (N2,))
-    part1 = torch.empty((int(lib.pta_gemm_splitk_parts(N1, K1, 0, 1)), M, N1), dtype=torch.float32, device=x1.device)
-    part2 = torch.empty((int(lib.pta_gemm_splitk_parts(N2, K2, 0, 1)), M, N2), dtype=torch.float32, device=x1.device)
+    p1, p2 = gemm_splitk_pair_parts(N1, K1, N2, K2)
+    part1 = torch.empty((p1, M, N1), dtype=torch.float32, device=x1.device)
+    part2 = torch.empty((p2, M, N2), dtype=torch.float32, device=x1.device)
     y1 = torch.empty((M, N1), dtype=torch.bfloat16, device=x1.device)
     y2 = torch.empty((M, N2), dtype=torch.bfloat16, device=x1.device)
     _call("pta_gemm_splitk_pair_reduced_bf16", _ptr(y1), _ptr(part1), _ptr(x1), _ptr(w1), _ptr(bias1), N1, K1,

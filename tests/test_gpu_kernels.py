@@ -212,8 +212,9 @@ def test_gemm_splitk_pair():
     w1, w2 = _rand(N1, K1, seed=1, dtype=torch.bfloat16, scale=0.05), _rand(N2, K2, seed=2, dtype=torch.bfloat16, scale=0.05)
     b2 = _rand(N2, seed=3)
     y1, y2 = ops.gemm_splitk_pair_bf16(x1, w1, x2, w2, None, None, b2, "gelu")
-    assert torch.equal(y1, ops.gemm_splitk_bf16(x1, w1, rt=1)), "the same ranges in the same order: the same bits"
-    assert torch.equal(y2, ops.gemm_splitk_bf16(x2, w2, b2, "gelu", rt=1))
+    p1, p2 = ops.gemm_splitk_pair_parts(N1, K1, N2, K2)
+    assert torch.equal(y1, ops.gemm_splitk_bf16(x1, w1, rt=1, parts=p1)), "the same ranges in the same order: the same bits"
+    assert torch.equal(y2, ops.gemm_splitk_bf16(x2, w2, b2, "gelu", rt=1, parts=p2))
     a1, a2 = ops.gemm_splitk_pair_bf16(x1[17:37].contiguous(), w1, x2[17:37].contiguous(), w2, None, None, b2, "gelu")
     assert torch.equal(a1, y1[17:37]) and torch.equal(a2, y2[17:37])
 
