@@ -179,7 +179,7 @@ def main():
     gen_cfg = GenerationConfig(do_sample=False, eos_token_id=None)
     if args.mixed:
         batch, lo, hi, new = MIXED[args.sizes]
-        run_mixed(model, 2, lo, min(hi, lo + 64), 4)  # builds what the first call builds
+        run_mixed(model, batch, lo, hi, 2)  # builds and tunes what the first call of these shapes builds and tunes
         dt, prompt_tokens = run_mixed(model, batch, lo, hi, new)
         print(json.dumps({"metric": f"falcon{args.sizes}_mixed_generated_tokens_per_second",
                           "value": round(batch * new / dt, 1), "unit": "tokens/s", "seconds": round(dt, 3),

@@ -19,6 +19,8 @@
 #include "common.h"
 #include "pta_kernels.h"
 
+#include <stdlib.h>
+
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef int i32x4_t __attribute__((ext_vector_type(4)));
@@ -233,20 +235,28 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce2_kernel(bf16_t* __rest
 
 static int pick_rt(int N) { return N >= 16384 ? 2 : 1; }
 
-// Ranges of K (workgroups along gridDim.y): enough for about two workgroups per compute unit, but no
-// range shorter than 512 elements and no more partial sums than about a sixth of W's bytes at 64 rows.
-static int pick_parts(int N, int K, int rt) {
-    const int groups = (N + 64 * rt - 1) / (64 * rt);
-    int P = (512 + groups - 1) / groups;
-    P = min(P, max(1, K / 512));
-    P = min(P, max(1, K / 900));
-    return max(1, min(P, 16));
-}
-
 // ranges that are not empty when K is cut into `parts` ranges of whole 64-element blocks
 static int effective_parts(int K, int parts) {
     const int nkb = (K + 63) / 64, per = (nkb + parts - 1) / parts;
     return (nkb + per - 1) / per;
+}
+
+// Ranges of K (workgroups along gridDim.y).  Measured at Falcon-7B to Falcon-40B shapes: a workgroup does best
+// with a range of about 2,304 elements (some 290 KB of weights for its 64 rows), and a launch with at least
+// some 512 workgroups; no range is shorter than 512 elements, and there are at most 16.
+#define SK_RANGE 2304
+static int splitk_target() {
+    static const int target = getenv("PTA_SPLITK_WGS") ? atoi(getenv("PTA_SPLITK_WGS")) : 512;
+    return target;
+}
+static int clamp_parts(int P, int K) { return max(1, min(min(P, 16), max(1, K / 512))); }
+
+// with many row tiles the ranges may be longer: fewer partial sums for the same number of workgroups
+static int range_for(int groups) { return SK_RANGE * max(1, groups / 64); }
+
+static int pick_parts(int N, int K, int rt) {
+    const int groups = (N + 64 * rt - 1) / (64 * rt), range = range_for(groups);
+    return clamp_parts(max((splitk_target() + groups - 1) / groups, (K + range / 2) / range), K);
 }
 
 extern "C" int pta_gemm_splitk_parts(int N, int K, int parts, int rt) {
@@ -337,17 +347,20 @@ extern "C" int pta_gemm_splitk_bf16(void* y, float* part, const void* x, const v
     return launch_rows<2, 2, 4>(MT, a, none, M, reduce, s);
 }
 
-// Ranges of K for the two products of a pair launch: the one with more work is cut as it would be on its own,
-// the other into ranges of about the same length, so that the launch's workgroups are of a size and the
-// smaller product leaves no more partial sums than it must.
+// Ranges of K for the two products of a pair launch: each by its own length, and more of both if the launch
+// would have too few workgroups.
 static void pick_pair_parts(int N1, int K1, int N2, int K2, int* p1, int* p2) {
-    const bool first_big = (long)N1 * K1 >= (long)N2 * K2;
-    const int Nb = first_big ? N1 : N2, Kb = first_big ? K1 : K2, Ns = first_big ? N2 : N1, Ks = first_big ? K2 : K1;
-    const int pb = pick_parts(Nb, Kb, 1);
-    const int range = (Kb + pb - 1) / pb;
-    const int ps = max(1, min(pick_parts(Ns, Ks, 1), (Ks + range / 2) / range));
-    *p1 = effective_parts(K1, first_big ? pb : ps);
-    *p2 = effective_parts(K2, first_big ? ps : pb);
+    const int g1 = (N1 + 63) / 64, g2 = (N2 + 63) / 64;
+    const int range = range_for(min(g1, g2));
+    int a = clamp_parts((K1 + range / 2) / range, K1), b = clamp_parts((K2 + range / 2) / range, K2);
+    const int total = g1 * a + g2 * b;
+    if (total < splitk_target()) {
+        const int more = (splitk_target() + total - 1) / total;
+        a = clamp_parts(a * more, K1);
+        b = clamp_parts(b * more, K2);
+    }
+    *p1 = effective_parts(K1, a);
+    *p2 = effective_parts(K2, b);
 }
 
 extern "C" int pta_gemm_splitk_pair_parts(int N1, int K1, int N2, int K2, int* p1, int* p2) {

@@ -351,14 +351,13 @@ _mm_plans: dict = {}  # (N, K, M) -> [rows, ...]
 
 def _mm_measure(x: torch.Tensor, w: torch.Tensor, rows: int, out: torch.Tensor) -> float:
     start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    for _ in range(2):  # the library's first calls of a shape set it up
-        torch.mm(x[:rows], w.t(), out=out[:rows])
+    torch.mm(x[:rows], w.t(), out=out[:rows])  # the library's first call of a shape sets it up
     start.record()
-    for _ in range(3):
+    for _ in range(2):
         torch.mm(x[:rows], w.t(), out=out[:rows])
     end.record()
     end.synchronize()
-    return start.elapsed_time(end) / 3 * 1e3
+    return start.elapsed_time(end) / 2 * 1e3
 
 
 def _mm_plan(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor):
@@ -371,7 +370,8 @@ def _mm_plan(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor):
     for rows in MM_LADDER:
         if rows <= M and rows not in times:
             times[rows] = _mm_measure(x, w, rows, out)
-    if M not in times:
+    whole = M <= MM_LADDER[-1]  # beyond the ladder the product always runs in pieces: timing it whole costs too much
+    if whole and M not in times:
         times[M] = _mm_measure(x, w, M, out)  # the product as it is
     # cheapest way to cover M rows with pieces of the ladder; what is left over rides on the last piece
     units, rest = divmod(M, 256)
@@ -387,7 +387,7 @@ def _mm_plan(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor):
     if rest:
         pieces = pieces[:-1] + [pieces[-1] + rest]
         cost *= M / (M - rest)
-    plan = pieces if len(pieces) > 1 and cost < 0.97 * times[M] else [M]
+    plan = pieces if not whole or (len(pieces) > 1 and cost < 0.97 * times[M]) else [M]
     _mm_plans[(N, K, bucket)] = plan
     return plan
 
