@@ -404,25 +404,55 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(bf16_t* __restrict__ o
     }
 }
 
-template <int DT, int CT, int W = 1>
-static void launch_attn(bf16_t* out, float* po, float* pm, float* pl, const bf16_t* q, const bf16_t* k_pool,
-                        const bf16_t* v_pool, const int* block_table, int bt_stride, const int* cu_tokens,
-                        const int* seq_start, const float* slopes, int n_seqs, int max_new, int nh, int nkv, float scale,
-                        int split_size, int n_splits, int window, hipStream_t s) {
-    const int g = nh / nkv;
-    const dim3 grid((max_new * g + 16 * CT * W - 1) / (16 * CT * W), nkv, n_seqs * n_splits);
-    auto kern = window > 0 ? attn_mfma_kernel<DT, CT, W, true> : attn_mfma_kernel<DT, CT, W, false>;
-    hipLaunchKernelGGL(kern, grid, dim3(64 * W), 0, s, out, po, pm, pl, q, k_pool, v_pool, block_table,
-                       bt_stride, cu_tokens, seq_start, slopes, nh, nkv, scale * PTA_LOG2E,
-                       PTA_LOG2E / sqrtf((float)(DT * 16)), split_size, n_splits, window);
+struct AttnLaunch {
+    bf16_t* out; float *po, *pm, *pl;
+    const bf16_t *q, *k_pool, *v_pool;
+    const int* block_table; int bt_stride;
+    const int *cu_tokens, *seq_start; const float* slopes;
+    int n_seqs, max_new, nh, nkv; float scale;
+    int split_size, n_splits, window;
+    hipStream_t s;
+};
+
+template <int DT, int CT, int W>
+static void launch_attn(const AttnLaunch& a) {
+    const int g = a.nh / a.nkv;
+    const dim3 grid((a.max_new * g + 16 * CT * W - 1) / (16 * CT * W), a.nkv, a.n_seqs * a.n_splits);
+    auto kern = a.window > 0 ? attn_mfma_kernel<DT, CT, W, true> : attn_mfma_kernel<DT, CT, W, false>;
+    hipLaunchKernelGGL(kern, grid, dim3(64 * W), 0, a.s, a.out, a.po, a.pm, a.pl, a.q, a.k_pool, a.v_pool, a.block_table,
+                       a.bt_stride, a.cu_tokens, a.seq_start, a.slopes, a.nh, a.nkv, a.scale * PTA_LOG2E,
+                       PTA_LOG2E / sqrtf((float)(DT * 16)), a.split_size, a.n_splits, a.window);
+}
+
+// column tiles (of sixteen query heads of one KV head) that one wave of a decode launch holds at most:
+// what the head size leaves registers for
+constexpr int decode_max_tiles(int dt) { return dt <= 4 ? 5 : dt <= 8 ? 4 : 1; }
+
+// one token per sequence: one wave per workgroup with `tiles` column tiles
+template <int DT, int CT = 1>
+static void launch_decode(const AttnLaunch& a, int tiles) {
+    if constexpr (CT <= decode_max_tiles(DT)) {
+        if (tiles == CT) launch_attn<DT, CT, 1>(a);
+        else launch_decode<DT, CT + 1>(a, tiles);
+    }
+}
+
+// prompts: four waves of two column tiles share each key block through LDS (head sizes up to 128;
+// beyond, one wave per workgroup)
+template <int DT>
+static void launch_prompt(const AttnLaunch& a) {
+    if constexpr (DT <= 8) launch_attn<DT, 2, 4>(a);
+    else launch_attn<DT, 1, 1>(a);
 }
 
 extern "C" int pta_attn_mfma_supported(int d) { return d % 16 == 0 && ((d >= 16 && d <= 128) || d == 256); }
 
+extern "C" int pta_attn_decode_max_tiles(int d) { return decode_max_tiles(d / 16); }
+
 extern "C" int pta_attn_mfma(void* out, const void* q, const void* k_pool, const void* v_pool, const int* block_table,
                              int bt_stride, const int* cu_tokens, const int* seq_start, const float* slopes, int n_seqs,
                              int max_new, int M, int nh, int nkv, int d, float scale, int split_size, int n_splits,
-                             float* po, float* pm, float* pl, int window, void* stream) {
+                             float* po, float* pm, float* pl, int window, int decode_tiles, void* stream) {
     PTA_REQUIRE(n_seqs > 0 && max_new > 0 && M > 0 && nh > 0 && nkv > 0, "attn_mfma: sizes must be positive");
     PTA_REQUIRE(nh % nkv == 0, "attn_mfma: heads (%d) must be a multiple of kv heads (%d)", nh, nkv);
     PTA_REQUIRE(pta_attn_mfma_supported(d), "attn_mfma: head size %d is not built (16..128 in steps of 16, or 256)", d);
@@ -434,44 +464,42 @@ extern "C" int pta_attn_mfma(void* out, const void* q, const void* k_pool, const
     PTA_REQUIRE(((uintptr_t)q % 16) == 0 && ((uintptr_t)k_pool % 16) == 0 && ((uintptr_t)v_pool % 16) == 0 &&
                     ((uintptr_t)out % 8) == 0, "attn_mfma: pointers must be 16-byte aligned");
     hipStream_t s = (hipStream_t)stream;
-    // one token per sequence (decode): one column tile per wave, so that the tiles of a KV head run side
-    // by side.  Prompts: four waves of two column tiles share each key block through LDS (head sizes up to
-    // 128; beyond, one wave per workgroup).  Measured at Falcon-7B sizes (2,048 tokens, 71 heads on one KV
+    // Prompts: four waves of two column tiles share each key block through LDS (head sizes up to 128;
+    // beyond, one wave per workgroup).  Measured at Falcon-7B sizes (2,048 tokens, 71 heads on one KV
     // head), one wave per workgroup: 2 tiles 148 us a layer, 4 tiles 195 us, 1 tile 270 us (fewer tiles
-    // balance the causal triangle better, more tiles re-read keys less).  PTA_ATTN_CT and PTA_ATTN_W
-    // override for tuning.
+    // balance the causal triangle better, more tiles re-read keys less).
+    // One token per sequence (decode): one wave per workgroup, which holds `decode_tiles` column tiles of
+    // its KV head (at most what the head size leaves registers for).  More tiles: the keys cross the memory
+    // path fewer times; fewer: shorter waves, more of them (71 heads on one KV head, 2,048 keys: 64
+    // sequences 39.5 us a layer with one tile, 27.5 us with five; 8 sequences 14.6 and 18.5 us).
     const bool narrow = max_new == 1;
-    static const int ct_env = getenv("PTA_ATTN_CT") ? atoi(getenv("PTA_ATTN_CT")) : 2;
-    static const int w_env = getenv("PTA_ATTN_W") ? atoi(getenv("PTA_ATTN_W")) : 4;
-#define PTA_ATTN_ARGS                                                                                              \
-    (bf16_t*)out, po, pm, pl, (const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_table, bt_stride, \
-        cu_tokens, seq_start, slopes, n_seqs, max_new, nh, nkv, scale, split_size, n_splits, window, s
-#define PTA_ATTN_CASE(DT_, CT_)                                                                   \
-    case DT_:                                                                                     \
-        if (narrow || ct_env == 1) launch_attn<DT_, 1, 1>(PTA_ATTN_ARGS);                         \
-        else if (w_env == 4 && DT_ <= 8) {                                                        \
-            if constexpr (DT_ <= 8) {                                                             \
-                if (ct_env == 2 || CT_ < 2) launch_attn<DT_, (CT_ < 2 ? CT_ : 2), 4>(PTA_ATTN_ARGS); \
-                else launch_attn<DT_, CT_, 4>(PTA_ATTN_ARGS);                                     \
-            }                                                                                     \
-        } else if (ct_env == 2 && CT_ > 2) launch_attn<DT_, 2, 1>(PTA_ATTN_ARGS);                 \
-        else launch_attn<DT_, CT_, 1>(PTA_ATTN_ARGS);                                             \
+    const int dct_most = std::min((nh / nkv + 15) / 16, pta_attn_decode_max_tiles(d));
+    PTA_REQUIRE(decode_tiles >= 0 && decode_tiles <= dct_most,
+                "attn_mfma: %d column tiles per decode wave; these sizes allow 1..%d (0: as many as that)", decode_tiles,
+                dct_most);
+    const int dct = decode_tiles > 0 ? decode_tiles : dct_most;
+    const AttnLaunch a{(bf16_t*)out, po, pm, pl, (const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool,
+                       block_table, bt_stride, cu_tokens, seq_start, slopes, n_seqs, max_new, nh, nkv, scale,
+                       split_size, n_splits, window, s};
+#define PTA_ATTN_CASE(DT_)                                        \
+    case DT_:                                                     \
+        if (narrow) launch_decode<DT_>(a, dct);                   \
+        else launch_prompt<DT_>(a);                               \
         break;
     switch (d / 16) {
-        PTA_ATTN_CASE(1, 4)
-        PTA_ATTN_CASE(2, 4)
-        PTA_ATTN_CASE(3, 4)
-        PTA_ATTN_CASE(4, 4)
-        PTA_ATTN_CASE(5, 2)
-        PTA_ATTN_CASE(6, 2)
-        PTA_ATTN_CASE(7, 2)
-        PTA_ATTN_CASE(8, 2)
-        PTA_ATTN_CASE(16, 1)
+        PTA_ATTN_CASE(1)
+        PTA_ATTN_CASE(2)
+        PTA_ATTN_CASE(3)
+        PTA_ATTN_CASE(4)
+        PTA_ATTN_CASE(5)
+        PTA_ATTN_CASE(6)
+        PTA_ATTN_CASE(7)
+        PTA_ATTN_CASE(8)
+        PTA_ATTN_CASE(16)
         default:
             return pta_fail("attn_mfma: head size %d is not built", d);
     }
 #undef PTA_ATTN_CASE
-#undef PTA_ATTN_ARGS
     int rc = pta_check_launch("attn_mfma");
     if (rc) return rc;
     if (n_splits > 1) {

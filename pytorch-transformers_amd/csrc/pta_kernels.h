@@ -60,11 +60,15 @@ int pta_attn_generic(void* out, const void* q, const void* k_pool, const void* v
 // which tokens are whose and how long each sequence was before the step; max_new bounds a sequence's new
 // tokens.  n_splits > 1 (decode): keys are cut into ranges of split_size, partial results go to
 // po [M, nh, n_splits, d], pm and pl [M, nh, n_splits] (32-bit) and are merged in split order.
+// decode_tiles (max_new == 1): column tiles that one wave holds, 1..min(tiles of a KV head, what
+// pta_attn_decode_max_tiles gives), or 0 for that most.
 int pta_attn_mfma_supported(int d);
+// Column tiles (sixteen query heads of one KV head) that one wave of a decode launch can hold at this head size.
+int pta_attn_decode_max_tiles(int d);
 int pta_attn_mfma(void* out, const void* q, const void* k_pool, const void* v_pool, const int* block_table,
                   int bt_stride, const int* cu_tokens, const int* seq_start, const float* slopes, int n_seqs,
                   int max_new, int M, int nh, int nkv, int d, float scale, int split_size, int n_splits, float* po,
-                  float* pm, float* pl, int window, void* stream);
+                  float* pm, float* pl, int window, int decode_tiles, void* stream);
 
 // C = act(A . W^T + bias) + add1 + add2, all 32-bit, fixed summation order
 int pta_gemm_f32(float* C, const float* A, const float* W, const float* bias, const float* add1, const float* add2,

@@ -9,6 +9,7 @@ capture like it.
 from __future__ import annotations
 
 import ctypes
+import functools
 import importlib.util
 import os
 import threading
@@ -225,11 +226,11 @@ def gemm_f32(a: torch.Tensor, w: torch.Tensor, bias=None, act=None, add1=None, a
     return out
 
 
-# a decode step's context is split into ranges of ATTN_SPLIT_KEYS keys, one wave each, or of the next
-# power-of-two multiple that keeps the launch at ATTN_SPLIT_WAVES waves or fewer
-ATTN_SPLIT_KEYS = int(os.environ.get("PTA_ATTN_SPLIT", "64"))
-ATTN_SPLIT_WAVES = int(os.environ.get("PTA_ATTN_WAVES", "2048"))
-
+# The smallest range of keys that one wave of a split decode launch walks (PTA_ATTN_SPLIT and PTA_ATTN_TILES
+# pin the cut of a decode launch for tuning: keys per wave, column tiles per wave).
+ATTN_SPLIT_KEYS = 128
+ATTN_FORCE_SPLIT = int(os.environ.get("PTA_ATTN_SPLIT", "0"))
+ATTN_FORCE_TILES = int(os.environ.get("PTA_ATTN_TILES", "0"))
 
 def attn_mfma_ok(q: torch.Tensor) -> bool:
     """Whether the matrix-core attention kernel takes these queries (bfloat16, head size built)."""
@@ -237,11 +238,14 @@ def attn_mfma_ok(q: torch.Tensor) -> bool:
 
 
 def attn_mfma(q: torch.Tensor, k_pool, v_pool, block_table, cu_tokens, seq_start, slopes, scale: float, *,
-              max_new: int, n_splits: int = 1, split_size: int = ATTN_SPLIT_KEYS, window: int = 0) -> torch.Tensor:
+              max_new: int, n_splits: int = 1, split_size: int = ATTN_SPLIT_KEYS, window: int = 0,
+              decode_tiles: int = 0) -> torch.Tensor:
     """Causal attention of a step's tokens over the cache on the matrix cores; out [M, nh*d].
 
     ``max_new`` bounds the new tokens of any sequence of the step; with ``n_splits > 1`` the keys
-    are split into ranges of ``split_size`` and ``n_splits * split_size`` bounds every context."""
+    are split into ranges of ``split_size`` and ``n_splits * split_size`` bounds every context.
+    ``decode_tiles``: groups of sixteen heads of one KV head that a wave holds when ``max_new`` is 1
+    (0: as many as the head size allows)."""
     _need(q, "q", torch.bfloat16)
     M, nh, d = q.shape
     nkv = k_pool.shape[1]
@@ -260,26 +264,73 @@ def attn_mfma(q: torch.Tensor, k_pool, v_pool, block_table, cu_tokens, seq_start
         pl = torch.empty((M, nh, n_splits), dtype=torch.float32, device=q.device)
     _call("pta_attn_mfma", _ptr(out), _ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(block_table), block_table.shape[1],
           _ptr(cu_tokens), _ptr(seq_start), _ptr(slopes), n_seqs, int(max_new), M, nh, nkv, d, ctypes.c_float(scale),
-          int(split_size), int(n_splits), _ptr(po), _ptr(pm), _ptr(pl), int(window), _stream())
+          int(split_size), int(n_splits), _ptr(po), _ptr(pm), _ptr(pl), int(window), int(decode_tiles), _stream())
     return out
 
 
-def decode_split_size(n_seqs: int, n_heads: int, n_kv_heads: int, max_len: int) -> int:
-    """Keys per wave of a split decode launch: ``ATTN_SPLIT_KEYS``, doubled until the launch has at most
-    ``ATTN_SPLIT_WAVES`` waves (many short waves cost more in start-up than they win in parallelism).
+@functools.lru_cache(maxsize=None)
+def _decode_plan(n: int, n_heads: int, n_kv_heads: int, head_dim: int, bound: int, most_tiles: int):
+    """The cheapest cut of a decode launch of ``n`` sequences of up to ``bound`` keys, by a model of its time.
+
+    A wave holds ``t`` groups of sixteen heads of one KV head and walks ``size`` keys in blocks of 32.  In
+    microseconds, fitted to launches with cold caches at three head shapes (71 heads on 1 KV head of 64; 32 on
+    8 of 128; 128 on 8 of 64), 1 to 64 sequences of 1,100 to 8,192 keys, every cut (the model's choice is
+    within 9 % of the best measured cut everywhere, and mostly equal to it):
+
+    - a wave takes 0.24 + 0.20 t + 0.15 (head_dim / 64 - 1) per block, and waves beyond what the chip
+      holds at once (1,024 SIMDs, as many waves each as 512 registers allow) wait for a whole round;
+    - the keys and values stream at 4.3 TB/s, and again at 8.3 TB/s for every further wave that shares
+      a KV head;
+    - ranges cost 2 + 0.085 per range, and their partial sums (32-bit, written and read) move at 3.7 TB/s.
+
+    The contexts of a step that is sized for ``bound`` lie in its last 1,024, so the time is taken at
+    ``bound - 512`` keys."""
+    groups = (n_heads // n_kv_heads + 15) // 16
+    dt = head_dim / 16.0
+    keys = bound - 512
+    kv_mb = n * keys * n_kv_heads * head_dim * 4 / 1e6
+    best = None
+    for t in range(1, most_tiles + 1):
+        if ATTN_FORCE_TILES and t != min(ATTN_FORCE_TILES, most_tiles):
+            continue
+        sharing = (groups + t - 1) // t
+        resident = 1024 * max(1, int(512 // ((38 + 11.5 * dt) + (26 + 8 * dt) * t)))
+        block_us = 0.24 + 0.20 * t + 0.15 * (head_dim / 64.0 - 1.0)
+        size = min(ATTN_SPLIT_KEYS, ATTN_FORCE_SPLIT) if ATTN_FORCE_SPLIT else ATTN_SPLIT_KEYS
+        while True:
+            whole = size >= bound
+            if (bound + size - 1) // size <= 1024 and (not ATTN_FORCE_SPLIT or size == ATTN_FORCE_SPLIT or
+                                                       (whole and size < ATTN_FORCE_SPLIT)):
+                ranges = (keys + size - 1) // size
+                waves = n * n_kv_heads * sharing * ranges
+                wave_us = min(size, keys) / 32 * block_us * ((waves + resident - 1) // resident)
+                stream_us = kv_mb / 4.3 + kv_mb * (sharing - 1) / 8.3
+                part_us = 0.0 if whole else 2.0 + 0.085 * ranges + n * n_heads * ranges * head_dim * 8 / 1e6 / 3.7
+                cost = max(wave_us, stream_us) + part_us
+                if best is None or cost < best[0]:
+                    best = (cost, t, size)
+            if whole:
+                break
+            size *= 2
+    if best is None:
+        raise KernelError(f"no cut of a decode launch over {bound} keys with PTA_ATTN_SPLIT={ATTN_FORCE_SPLIT}")
+    return best[1], best[2]
+
+
+def decode_plan(n_seqs: int, n_heads: int, n_kv_heads: int, head_dim: int, max_len: int):
+    """How a decode launch is cut: (column tiles per wave, keys per wave); a size that covers the
+    context means one wave per sequence and head group, which writes the result itself.
 
     The batch counts by its next power of two and the context by its next multiple of 1,024, so that a
-    captured step, which is sized for a padded batch and a length bound, splits exactly as the same
+    captured step, which is sized for a padded batch and a length bound, is cut exactly as the same
     step run directly."""
     n = 1
     while n < n_seqs:
         n *= 2
     bound = (max_len + 1023) // 1024 * 1024
-    tiles = n * n_kv_heads * ((n_heads // n_kv_heads + 15) // 16)
-    size = ATTN_SPLIT_KEYS
-    while size < bound and tiles * (bound // size) > ATTN_SPLIT_WAVES:
-        size *= 2
-    return size
+    groups = (n_heads // n_kv_heads + 15) // 16
+    most = min(groups, int(load_library().pta_attn_decode_max_tiles(head_dim)))
+    return _decode_plan(n, n_heads, n_kv_heads, head_dim, bound, most)
 
 
 def attention(q: torch.Tensor, k_pool, v_pool, block_table, ctx, slopes, scale: float, window: int = 0) -> torch.Tensor:
@@ -289,12 +340,13 @@ def attention(q: torch.Tensor, k_pool, v_pool, block_table, ctx, slopes, scale: 
     split over several waves when every sequence brings one token; anything else: the 32-bit
     kernel."""
     if attn_mfma_ok(q):
-        n_splits, size = 1, ATTN_SPLIT_KEYS
-        if ctx.is_decode and ctx.max_len > ATTN_SPLIT_KEYS:
-            size = decode_split_size(ctx.n_seqs, q.shape[1], k_pool.shape[1], ctx.max_len)
+        n_splits, size, tiles = 1, ATTN_SPLIT_KEYS, 0
+        if ctx.is_decode:
+            tiles, size = decode_plan(ctx.n_seqs, q.shape[1], k_pool.shape[1], q.shape[2], ctx.max_len)
             n_splits = (ctx.max_len + size - 1) // size
         return attn_mfma(q, k_pool, v_pool, block_table, ctx.cu_tokens, ctx.seq_start, slopes, scale,
-                         max_new=max(ctx.new_tokens), n_splits=n_splits, split_size=size, window=window)
+                         max_new=max(ctx.new_tokens), n_splits=n_splits, split_size=size, window=window,
+                         decode_tiles=tiles)
     return attn_generic(q, k_pool, v_pool, block_table, ctx.token_seq, ctx.token_pos, slopes, scale, window)
 
 

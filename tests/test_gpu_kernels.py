@@ -422,7 +422,7 @@ def test_attn_generic_far_key_and_alibi(dtype):
         _attn_case(ops, _generic(ops), dtype, nh, nh, 16, starts=[0, 290], news=[40, 30], slopes=slopes)
 
 
-def _mfma(ops, n_splits_for=None):
+def _mfma(ops, n_splits_for=None, tiles=0):
     def fn(q, k_pool, v_pool, bt, token_seq, token_pos, slopes, scale, starts, news, window=0):
         cu = torch.tensor([0] + list(torch.tensor(news).cumsum(0)), dtype=torch.int32).cuda()
         st = torch.tensor(starts, dtype=torch.int32).cuda()
@@ -430,7 +430,7 @@ def _mfma(ops, n_splits_for=None):
         if n_splits_for is not None:
             n_splits = (max(s + n for s, n in zip(starts, news)) + n_splits_for - 1) // n_splits_for
         return ops.attn_mfma(q, k_pool, v_pool, bt, cu, st, slopes, scale, max_new=max(news), n_splits=n_splits,
-                             split_size=n_splits_for or 256, window=window)
+                             split_size=n_splits_for or 256, window=window, decode_tiles=tiles)
     return fn
 
 
@@ -449,6 +449,41 @@ def test_attn_mfma_decode_split(nh, nkv, d, split):
     """One token per sequence, contexts of very different lengths, keys split over waves and merged."""
     ops = _ops()
     _attn_case(ops, _mfma(ops, split), torch.bfloat16, nh, nkv, d, starts=[0, 63, 64, 700, 255, 256, 1], news=[1] * 7)
+
+
+@pytest.mark.parametrize("nh,nkv,d,tiles", [(71, 1, 64, 1), (71, 1, 64, 2), (71, 1, 64, 3), (71, 1, 64, 5), (40, 1, 32, 3),
+                                            (128, 2, 128, 4), (128, 2, 128, 3), (66, 2, 16, 2), (17, 1, 256, 1)])
+def test_attn_mfma_decode_tiles(nh, nkv, d, tiles):
+    """One token per sequence with many heads on a KV head: a wave holds `tiles` groups of sixteen of them,
+    the last group partly filled; with split ranges and without, with and without ALiBi and a window."""
+    ops = _ops()
+    from pytorch_transformers_amd.parts import AlibiPositions
+    starts = [0, 63, 64, 700, 255, 256, 1]
+    for split in (None, 128):
+        _attn_case(ops, _mfma(ops, split, tiles), torch.bfloat16, nh, nkv, d, starts=starts, news=[1] * 7)
+    if d == 64:
+        slopes = AlibiPositions(nh).slopes.cuda()
+        _attn_case(ops, _mfma(ops, 128, tiles), torch.bfloat16, nh, nkv, d, starts=starts, news=[1] * 7, slopes=slopes)
+        _attn_case(ops, _mfma(ops, 128, tiles), torch.bfloat16, nh, nkv, d, starts=starts, news=[1] * 7, window=100)
+    most = min((nh // nkv + 15) // 16, 5 if d <= 64 else 4 if d <= 128 else 1)
+    with pytest.raises(ops.KernelError, match="column tiles per decode wave"):
+        _attn_case(ops, _mfma(ops, None, most + 1), torch.bfloat16, nh, nkv, d, starts=[5], news=[1])
+
+
+def test_decode_plan():
+    """The cut of a decode launch: whole tiles within what the head size allows, a range size that is a
+    multiple of the page, the same for every batch and context of one captured step's bucket."""
+    ops = _ops()
+    for nh, nkv, d in ((71, 1, 64), (32, 8, 128), (128, 8, 64), (6, 2, 32), (2, 1, 256)):
+        groups = (nh // nkv + 15) // 16
+        for n in (1, 3, 8, 33, 64):
+            for length in (1, 100, 1024, 1025, 2049, 8192, 100000):
+                tiles, size = ops.decode_plan(n, nh, nkv, d, length)
+                assert 1 <= tiles <= groups and size % 64 == 0 and size >= 128
+                assert (length + size - 1) // size <= 1024
+                bucket_n = 1 << (n - 1).bit_length()
+                bucket_len = (length + 1023) // 1024 * 1024
+                assert (tiles, size) == ops.decode_plan(bucket_n, nh, nkv, d, bucket_len)
 
 
 @pytest.mark.parametrize("window", [1, 33, 64, 100, 200])
