@@ -93,7 +93,7 @@ extern "C" {
 
 const char* ptah_last_error() { return g_error.c_str(); }
 
-int ptah_abi_version() { return 2; }
+int ptah_abi_version() { return 3; }
 
 void* ptah_cache_new(int max_slots, int page_size, int n_groups, const int* group_pages, const int* group_windows) {
     if (max_slots <= 0 || page_size <= 0 || n_groups < 0) {
@@ -337,8 +337,10 @@ int ptah_plan_step(void* h, int n, const int* slots, const int* new_tokens, cons
 const int* ptah_plan_data(void* h) { return static_cast<Cache*>(h)->plan.data(); }
 
 // The common step of decoding, without the general planner's detours: every sequence brings one token and
-// wants its logits.  Checks the step, reserves its pages and reports the longest context after it.
-int ptah_decode_prepare(void* h, int n, const int* slots, const long long* tokens, int vocab, int* max_len_out) {
+// wants its logits.  Checks the step, reserves its pages and reports the longest context after it and the
+// sum of all of them.
+int ptah_decode_prepare(void* h, int n, const int* slots, const long long* tokens, int vocab, int* max_len_out,
+                        long long* total_len_out) {
     Cache* c = static_cast<Cache*>(h);
     if (n <= 0) return fail(ERR_STEP, "a step needs at least one sequence");
     for (int i = 0; i < n; ++i)
@@ -348,8 +350,13 @@ int ptah_decode_prepare(void* h, int n, const int* slots, const long long* token
     const int rc = ptah_reserve(h, n, slots, ones.data());
     if (rc) return rc;
     int longest = 0;
-    for (int i = 0; i < n; ++i) longest = std::max(longest, c->length[slots[i]] + 1);
+    long long total = 0;
+    for (int i = 0; i < n; ++i) {
+        longest = std::max(longest, c->length[slots[i]] + 1);
+        total += c->length[slots[i]] + 1;
+    }
     *max_len_out = longest;
+    *total_len_out = total;
     return OK;
 }
 

@@ -46,11 +46,23 @@ def _require_gpu(device) -> torch.device:
     return device
 
 
-GRAPH_LEN_STEP = 1024  # a decode graph serves contexts up to the next multiple of this
+GRAPH_LEN_STEP = 1024  # a decode graph serves contexts up to the next multiple of this ...
+GRAPH_MEAN_STEP = 512  # ... whose mean is at most a multiple of this
+
+
+def _len_bound(max_len: int) -> int:
+    return (max_len + GRAPH_LEN_STEP - 1) // GRAPH_LEN_STEP * GRAPH_LEN_STEP
+
+
+def mean_len_bound(total_len: int, n_seqs: int, len_bound: int) -> int:
+    """The bucket of a step's mean context: its next multiple of ``GRAPH_MEAN_STEP``, at most ``len_bound``."""
+    mean = -(-int(total_len) // max(1, int(n_seqs)))
+    return min(len_bound, -(-mean // GRAPH_MEAN_STEP) * GRAPH_MEAN_STEP)
 
 
 class _DecodeGraph:
-    """One decode step of ``n`` sequences with contexts up to ``len_bound``, captured once and replayed.
+    """One decode step of ``n`` sequences with contexts up to ``len_bound`` (``mean_bound`` on average),
+    captured once and replayed.
 
     A decode step launches some ten kernels a layer; issued one by one from Python they cost more
     host time than the GPU needs to run them.  The captured graph reads everything that changes
@@ -62,8 +74,9 @@ class _DecodeGraph:
     again, and the spare logits are dropped.
     """
 
-    def __init__(self, model: "CausalLM", cache: PagedCache, n: int, len_bound: int):
+    def __init__(self, model: "CausalLM", cache: PagedCache, n: int, len_bound: int, mean_bound: int = 0):
         self.model, self.cache, self.n, self.len_bound = model, cache, n, len_bound
+        self.mean_bound = mean_bound or len_bound
         self.width = len_bound // cache.page_size
         self.groups = cache.paged_groups()
         ar = np.arange(n, dtype=np.int32)
@@ -108,7 +121,8 @@ class _DecodeGraph:
         ctx = StepContext(dtype=self.model.dtype, device=self.model.device, n_seqs=self.n, n_tokens=self.n,
                           token_seq=v[1], token_pos=v[2], cu_tokens=v[3], seq_start=v[4], seq_slot=v[5],
                           block_tables=tables, cache=self.cache, slots=[], new_tokens=[1] * self.n, starts=[],
-                          is_decode=True, max_len=self.len_bound, side_stream=self.model._side_stream(self.n))
+                          is_decode=True, max_len=self.len_bound, mean_len=self.mean_bound,
+                          side_stream=self.model._side_stream(self.n))
         return ctx, v[0], v[6]
 
     def run(self, plan: StepPlan) -> torch.Tensor:
@@ -245,6 +259,7 @@ class CausalLM:
                           token_pos=views[2], cu_tokens=views[3], seq_start=views[4], seq_slot=views[5],
                           block_tables=tables, cache=cache, slots=plan.slots, new_tokens=plan.new_tokens,
                           starts=plan.starts, is_decode=plan.is_decode, max_len=plan.max_len,
+                          mean_len=mean_len_bound(plan.total_len, n, _len_bound(plan.max_len)),
                           side_stream=self._side_stream(plan.n_tokens))
         return ctx, views[0], (views[6] if R else None)
 
@@ -269,16 +284,17 @@ class CausalLM:
 
     # decode steps as HIP graphs ---------------------------------------------------------
     def _graph_for(self, cache: PagedCache, plan: StepPlan) -> "_DecodeGraph":
-        return self._graph_for_sizes(cache, plan.n_seqs, plan.max_len)
+        return self._graph_for_sizes(cache, plan.n_seqs, plan.max_len, plan.total_len)
 
-    def _graph_for_sizes(self, cache: PagedCache, n: int, max_len: int) -> "_DecodeGraph":
+    def _graph_for_sizes(self, cache: PagedCache, n: int, max_len: int, total_len: int) -> "_DecodeGraph":
         n_bucket = n if n <= 8 else (n + 7) // 8 * 8
-        len_bound = (max_len + GRAPH_LEN_STEP - 1) // GRAPH_LEN_STEP * GRAPH_LEN_STEP
+        len_bound = _len_bound(max_len)
+        mean_bound = mean_len_bound(total_len, n, len_bound)
         graphs = cache.__dict__.setdefault("_decode_graphs", {})
-        key = (id(self), n_bucket, len_bound)
+        key = (id(self), n_bucket, len_bound, mean_bound)
         g = graphs.get(key)
         if g is None:
-            g = graphs[key] = _DecodeGraph(self, cache, n_bucket, len_bound)
+            g = graphs[key] = _DecodeGraph(self, cache, n_bucket, len_bound, mean_bound)
         return g
 
     @torch.no_grad()
@@ -316,11 +332,12 @@ class CausalLM:
         lib = host.load()
         slots_c = (ctypes.c_int * n)(*[int(s) for s in slots])
         tokens_c = (ctypes.c_longlong * n)(*[int(t[0]) for t in tokens])
-        longest = ctypes.c_int(0)
-        rc = lib.ptah_decode_prepare(cache.handle, n, slots_c, tokens_c, self.vocab_size, ctypes.byref(longest))
+        longest, total = ctypes.c_int(0), ctypes.c_longlong(0)
+        rc = lib.ptah_decode_prepare(cache.handle, n, slots_c, tokens_c, self.vocab_size, ctypes.byref(longest),
+                                     ctypes.byref(total))
         if rc:
             raise {host.ERR_STEP: StepError, host.ERR_FULL: CacheFull}.get(rc, CacheError)(host.last_error())
-        logits = self._graph_for_sizes(cache, n, longest.value).run_last(n, slots_c, tokens_c)
+        logits = self._graph_for_sizes(cache, n, longest.value, total.value).run_last(n, slots_c, tokens_c)
         lib.ptah_commit_ones(cache.handle, n, slots_c)
         return logits
 

@@ -54,6 +54,10 @@ class StepPlan:
     def max_len(self) -> int:
         return max(s + n for s, n in zip(self.starts, self.new_tokens))
 
+    @property
+    def total_len(self) -> int:
+        return sum(s + n for s, n in zip(self.starts, self.new_tokens))
+
 
 _WANT_MODES = {"none": 0, "last": 1, "all": 2}
 

@@ -269,8 +269,9 @@ def attn_mfma(q: torch.Tensor, k_pool, v_pool, block_table, cu_tokens, seq_start
 
 
 @functools.lru_cache(maxsize=None)
-def _decode_plan(n: int, n_heads: int, n_kv_heads: int, head_dim: int, bound: int, most_tiles: int):
-    """The cheapest cut of a decode launch of ``n`` sequences of up to ``bound`` keys, by a model of its time.
+def _decode_plan(n: int, n_heads: int, n_kv_heads: int, head_dim: int, bound: int, mean: int, most_tiles: int):
+    """The cheapest cut of a decode launch of ``n`` sequences of up to ``bound`` keys, ``mean`` on average,
+    by a model of its time.
 
     A wave holds ``t`` groups of sixteen heads of one KV head and walks ``size`` keys in blocks of 32.  In
     microseconds, fitted to launches with cold caches at three head shapes (71 heads on 1 KV head of 64; 32 on
@@ -283,12 +284,14 @@ def _decode_plan(n: int, n_heads: int, n_kv_heads: int, head_dim: int, bound: in
       a KV head;
     - ranges cost 2 + 0.085 per range, and their partial sums (32-bit, written and read) move at 3.7 TB/s.
 
-    The contexts of a step that is sized for ``bound`` lie in its last 1,024, so the time is taken at
-    ``bound - 512`` keys."""
+    The longest context of a step that is sized for ``bound`` lies in its last 1,024 and the mean in the 512
+    below ``mean``, so the longest wave's time is taken at ``bound - 512`` keys and the traffic at
+    ``mean - 256`` keys a sequence."""
     groups = (n_heads // n_kv_heads + 15) // 16
     dt = head_dim / 16.0
     keys = bound - 512
-    kv_mb = n * keys * n_kv_heads * head_dim * 4 / 1e6
+    mean_keys = min(keys, mean - 256)
+    kv_mb = n * mean_keys * n_kv_heads * head_dim * 4 / 1e6
     best = None
     for t in range(1, most_tiles + 1):
         if ATTN_FORCE_TILES and t != min(ATTN_FORCE_TILES, most_tiles):
@@ -301,7 +304,7 @@ def _decode_plan(n: int, n_heads: int, n_kv_heads: int, head_dim: int, bound: in
             whole = size >= bound
             if (bound + size - 1) // size <= 1024 and (not ATTN_FORCE_SPLIT or size == ATTN_FORCE_SPLIT or
                                                        (whole and size < ATTN_FORCE_SPLIT)):
-                ranges = (keys + size - 1) // size
+                ranges = (mean_keys + size - 1) // size
                 waves = n * n_kv_heads * sharing * ranges
                 wave_us = min(size, keys) / 32 * block_us * ((waves + resident - 1) // resident)
                 stream_us = kv_mb / 4.3 + kv_mb * (sharing - 1) / 8.3
@@ -317,20 +320,21 @@ def _decode_plan(n: int, n_heads: int, n_kv_heads: int, head_dim: int, bound: in
     return best[1], best[2]
 
 
-def decode_plan(n_seqs: int, n_heads: int, n_kv_heads: int, head_dim: int, max_len: int):
+def decode_plan(n_seqs: int, n_heads: int, n_kv_heads: int, head_dim: int, max_len: int, mean_len: int = 0):
     """How a decode launch is cut: (column tiles per wave, keys per wave); a size that covers the
     context means one wave per sequence and head group, which writes the result itself.
 
-    The batch counts by its next power of two and the context by its next multiple of 1,024, so that a
-    captured step, which is sized for a padded batch and a length bound, is cut exactly as the same
-    step run directly."""
+    The batch counts by its next power of two, the longest context by its next multiple of 1,024 and the
+    mean context (``mean_len``; 0: as the longest) by its next multiple of 512, so that a captured step,
+    which is sized for a padded batch and such bounds, is cut exactly as the same step run directly."""
     n = 1
     while n < n_seqs:
         n *= 2
     bound = (max_len + 1023) // 1024 * 1024
     groups = (n_heads // n_kv_heads + 15) // 16
     most = min(groups, int(load_library().pta_attn_decode_max_tiles(head_dim)))
-    return _decode_plan(n, n_heads, n_kv_heads, head_dim, bound, most)
+    mean = min(bound, (mean_len + 511) // 512 * 512) if mean_len > 0 else bound
+    return _decode_plan(n, n_heads, n_kv_heads, head_dim, bound, mean, most)
 
 
 def attention(q: torch.Tensor, k_pool, v_pool, block_table, ctx, slopes, scale: float, window: int = 0) -> torch.Tensor:
@@ -342,7 +346,8 @@ def attention(q: torch.Tensor, k_pool, v_pool, block_table, ctx, slopes, scale: 
     if attn_mfma_ok(q):
         n_splits, size, tiles = 1, ATTN_SPLIT_KEYS, 0
         if ctx.is_decode:
-            tiles, size = decode_plan(ctx.n_seqs, q.shape[1], k_pool.shape[1], q.shape[2], ctx.max_len)
+            tiles, size = decode_plan(ctx.n_seqs, q.shape[1], k_pool.shape[1], q.shape[2], ctx.max_len,
+                                      getattr(ctx, "mean_len", 0))
             n_splits = (ctx.max_len + size - 1) // size
         return attn_mfma(q, k_pool, v_pool, block_table, ctx.cu_tokens, ctx.seq_start, slopes, scale,
                          max_new=max(ctx.new_tokens), n_splits=n_splits, split_size=size, window=window,

@@ -484,6 +484,10 @@ def test_decode_plan():
                 bucket_n = 1 << (n - 1).bit_length()
                 bucket_len = (length + 1023) // 1024 * 1024
                 assert (tiles, size) == ops.decode_plan(bucket_n, nh, nkv, d, bucket_len)
+                for mean in (1, length // 3 + 1, length):
+                    cut = ops.decode_plan(n, nh, nkv, d, length, mean)
+                    assert cut == ops.decode_plan(bucket_n, nh, nkv, d, bucket_len, min(bucket_len, (mean + 511) // 512 * 512))
+                    assert 1 <= cut[0] <= groups and cut[1] % 64 == 0 and (length + cut[1] - 1) // cut[1] <= 1024
 
 
 @pytest.mark.parametrize("window", [1, 33, 64, 100, 200])
