@@ -21,7 +21,7 @@ from ..engine.spec import INIT_NORMAL, INIT_ZERO_NOISE, MATRIX, VECTOR, TensorSp
 from .base import PartialProduct, Part
 
 
-PAIR_MAX_WEIGHTS = 160 * 1024 * 1024  # elements of both matrices of a pair launch at 17 to 64 rows
+PAIR_MAX_WEIGHTS = 160 * 1024 * 1024  # elements of both matrices of a pair launch at 49 to 64 rows
 
 
 class Linear(Part):
@@ -71,9 +71,10 @@ class Linear(Part):
         args = (x1, first.weight, x2, second.weight, b1, kw1.get("act"), b2, kw2.get("act"))
         if x1.shape == x2.shape and ops.gemm_skinny_ok(x1, first.weight) and ops.gemm_skinny_ok(x2, second.weight):
             return ops.gemm_skinny_pair_bf16(*args)
-        # 17 to 64 rows: measured at Falcon-7B and Falcon2-11B sizes the pair beats the products on their own;
-        # at Falcon-40B sizes the vendor library's product for the feed-forward input is the faster one
-        small = first.weight.numel() + second.weight.numel() <= PAIR_MAX_WEIGHTS
+        # 17 to 64 rows: measured at Falcon-7B and Falcon2-11B sizes the pair beats the products on their own; at
+        # Falcon-40B sizes it does up to 48 rows (32 rows: 20.8 against 23.0 ms a step), beyond them the vendor
+        # library's product for the feed-forward input is the faster one (64 rows: 23.3 against 24.3 ms)
+        small = x1.shape[0] <= 48 or first.weight.numel() + second.weight.numel() <= PAIR_MAX_WEIGHTS
         if small and ops.gemm_splitk_rows_ok(x1, first.weight) and ops.gemm_splitk_rows_ok(x2, second.weight):
             return ops.gemm_splitk_pair_bf16(*args)
         return None
