@@ -13,6 +13,8 @@ from __future__ import annotations
 from typing import Dict, Optional, Sequence
 
 import ctypes
+import gc
+import weakref
 
 import numpy as np
 import torch
@@ -72,10 +74,16 @@ class _DecodeGraph:
     past a sequence's end do no work.  A step with fewer than ``n`` sequences repeats its first
     sequence in the spare rows: the same token at the same place writes the same keys and values
     again, and the spare logits are dropped.
+
+    The cache owns its graphs and a graph refers to its cache weakly: with no cycle between them a cache
+    that is dropped takes its graphs along at once.  A graph may not be destroyed while another one is
+    being captured (the runtime refuses every such call during a capture, and the refusal, raised in a
+    destructor, ends the process), and Python's collector of cycles runs when it pleases; for the same
+    reason it is switched off while a capture lasts.
     """
 
     def __init__(self, model: "CausalLM", cache: PagedCache, n: int, len_bound: int, mean_bound: int = 0):
-        self.model, self.cache, self.n, self.len_bound = model, cache, n, len_bound
+        self.model, self._cache, self.n, self.len_bound = model, weakref.ref(cache), n, len_bound
         self.mean_bound = mean_bound or len_bound
         self.width = len_bound // cache.page_size
         self.groups = cache.paged_groups()
@@ -93,6 +101,13 @@ class _DecodeGraph:
         self.copied = torch.cuda.Event()
         self.graph = None
         self.logits = None
+
+    @property
+    def cache(self) -> PagedCache:
+        cache = self._cache()
+        if cache is None:
+            raise StepError("this decode graph's cache is gone")
+        return cache
 
     def _put(self, i: int, arr) -> None:
         self.host_np[self.offsets[i]:self.offsets[i + 1]] = arr
@@ -157,9 +172,16 @@ class _DecodeGraph:
             with torch.cuda.stream(side):  # once outside capture: libraries set themselves up
                 self.model.forward_tokens(ctx, ids, rows)
             torch.cuda.current_stream().wait_stream(side)
-            self.graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(self.graph):
-                self.logits = self.model.forward_tokens(ctx, ids, rows)
+            graph = torch.cuda.CUDAGraph()
+            collecting = gc.isenabled()
+            gc.disable()  # no finalizer of a dead cycle may call into the runtime while the capture lasts
+            try:
+                with torch.cuda.graph(graph):
+                    self.logits = self.model.forward_tokens(ctx, ids, rows)
+            finally:
+                if collecting:
+                    gc.enable()
+            self.graph = graph
         self.graph.replay()
 
 

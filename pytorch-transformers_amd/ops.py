@@ -276,13 +276,14 @@ def _decode_plan(n: int, n_heads: int, n_kv_heads: int, head_dim: int, bound: in
     A wave holds ``t`` groups of sixteen heads of one KV head and walks ``size`` keys in blocks of 32.  In
     microseconds, fitted to launches with cold caches at three head shapes (71 heads on 1 KV head of 64; 32 on
     8 of 128; 128 on 8 of 64), 1 to 64 sequences of 1,100 to 8,192 keys, every cut (the model's choice is
-    within 9 % of the best measured cut everywhere, and mostly equal to it):
+    within a tenth of the best measured cut nearly everywhere, and mostly equal to it):
 
-    - a wave takes 0.24 + 0.20 t + 0.15 (head_dim / 64 - 1) per block, and waves beyond what the chip
+    - a wave takes 0.22 + 0.21 t + 0.15 (head_dim / 64 - 1) per block, and waves beyond what the chip
       holds at once (1,024 SIMDs, as many waves each as 512 registers allow) wait for a whole round;
-    - the keys and values stream at 4.3 TB/s, and again at 8.3 TB/s for every further wave that shares
+    - the keys and values stream at 5.1 TB/s, and again at 7.2 TB/s for every further wave that shares
       a KV head;
-    - ranges cost 2 + 0.085 per range, and their partial sums (32-bit, written and read) move at 3.7 TB/s.
+    - the launch takes the 4.2-norm of those two times (the larger one, and more where they are close);
+    - ranges cost 2.2 + 0.1 per range, and their partial sums (32-bit, written and read) move at 3.5 TB/s.
 
     The longest context of a step that is sized for ``bound`` lies in its last 1,024 and the mean in the 512
     below ``mean``, so the longest wave's time is taken at ``bound - 512`` keys and the traffic at
@@ -298,7 +299,7 @@ def _decode_plan(n: int, n_heads: int, n_kv_heads: int, head_dim: int, bound: in
             continue
         sharing = (groups + t - 1) // t
         resident = 1024 * max(1, int(512 // ((38 + 11.5 * dt) + (26 + 8 * dt) * t)))
-        block_us = 0.24 + 0.20 * t + 0.15 * (head_dim / 64.0 - 1.0)
+        block_us = 0.22 + 0.21 * t + 0.15 * (head_dim / 64.0 - 1.0)
         size = min(ATTN_SPLIT_KEYS, ATTN_FORCE_SPLIT) if ATTN_FORCE_SPLIT else ATTN_SPLIT_KEYS
         while True:
             whole = size >= bound
@@ -307,9 +308,9 @@ def _decode_plan(n: int, n_heads: int, n_kv_heads: int, head_dim: int, bound: in
                 ranges = (mean_keys + size - 1) // size
                 waves = n * n_kv_heads * sharing * ranges
                 wave_us = min(size, keys) / 32 * block_us * ((waves + resident - 1) // resident)
-                stream_us = kv_mb / 4.3 + kv_mb * (sharing - 1) / 8.3
-                part_us = 0.0 if whole else 2.0 + 0.085 * ranges + n * n_heads * ranges * head_dim * 8 / 1e6 / 3.7
-                cost = max(wave_us, stream_us) + part_us
+                stream_us = kv_mb / 5.1 + kv_mb * (sharing - 1) / 7.2
+                part_us = 0.0 if whole else 2.2 + 0.1 * ranges + n * n_heads * ranges * head_dim * 8 / 1e6 / 3.5
+                cost = (wave_us ** 4.2 + stream_us ** 4.2) ** (1 / 4.2) + part_us
                 if best is None or cost < best[0]:
                     best = (cost, t, size)
             if whole:

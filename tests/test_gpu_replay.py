@@ -168,3 +168,35 @@ def test_graph_replays_equal_eager_steps(folders, name, dtype):
         assert (a is None) == (b is None)
         if a is not None:
             assert torch.equal(a, b), f"step {rec['step']}: graph replay differs from eager launch"
+
+
+def test_a_dropped_cache_takes_its_graphs_along(folders):
+    """A cache and the decode steps captured for it form no reference cycle: dropping the cache frees them at
+    once, never later from the collector of cycles (which could then run while another step is captured, when
+    the runtime permits no graph to be destroyed), and captures of later caches go on working."""
+    import gc
+    import weakref
+
+    from pytorch_transformers_amd import AutoModelForCausalLM
+
+    model = AutoModelForCausalLM.from_pretrained(folders["A"], dtype="bfloat16")
+    assert model.use_graphs
+    gc.collect()
+    gc.disable()
+    try:
+        refs = []
+        for n in (2, 3):  # the second round captures while the first round's cache is already gone
+            cache = model.new_cache(1024, max_slots=4)
+            slots = [cache.alloc() for _ in range(n)]
+            model.step(cache, slots, [[1, 2, 3]] * n, "last")
+            model.step(cache, slots, [[4]] * n, "last")
+            graphs = list(cache._decode_graphs.values())
+            assert graphs and graphs[0].graph is not None
+            refs.append((weakref.ref(cache), weakref.ref(graphs[0])))
+            del graphs
+            for s in slots:
+                cache.free(s)
+            del cache
+            assert refs[-1][0]() is None and refs[-1][1]() is None, "the cache or its graph outlives its last reference"
+    finally:
+        gc.enable()
