@@ -136,8 +136,7 @@ class _DecodeGraph:
         ctx = StepContext(dtype=self.model.dtype, device=self.model.device, n_seqs=self.n, n_tokens=self.n,
                           token_seq=v[1], token_pos=v[2], cu_tokens=v[3], seq_start=v[4], seq_slot=v[5],
                           block_tables=tables, cache=self.cache, slots=[], new_tokens=[1] * self.n, starts=[],
-                          is_decode=True, max_len=self.len_bound, mean_len=self.mean_bound,
-                          side_stream=self.model._side_stream(self.n))
+                          is_decode=True, max_len=self.len_bound, mean_len=self.mean_bound)
         return ctx, v[0], v[6]
 
     def run(self, plan: StepPlan) -> torch.Tensor:
@@ -199,11 +198,6 @@ class CausalLM:
         self.generation_config = None
         #: run steps in which every sequence brings one token as replays of a captured HIP graph
         self.use_graphs = bool(spec.supports_graphs)
-        #: run a block's independent branches on two streams in steps of at most this many tokens.
-        #: Off: the first GPU run with it on ended in a host-side abort whose cause is not established.
-        self.overlap_branches = False
-        self.overlap_max_tokens = 256
-        self._side = None
 
     def _move_constants(self) -> None:
         seen = set()
@@ -219,15 +213,6 @@ class CausalLM:
 
         for part in self.spec.parts():
             walk(part)
-
-    def _side_stream(self, n_tokens: int):
-        """The second stream for independent branches of a block, for steps small enough to leave the
-        chip room for two kernels at once (large steps fill it with one)."""
-        if not self.overlap_branches or n_tokens > self.overlap_max_tokens:
-            return None
-        if self._side is None:
-            self._side = torch.cuda.Stream()
-        return self._side
 
     # construction ----------------------------------------------------------
     @classmethod
@@ -281,8 +266,7 @@ class CausalLM:
                           token_pos=views[2], cu_tokens=views[3], seq_start=views[4], seq_slot=views[5],
                           block_tables=tables, cache=cache, slots=plan.slots, new_tokens=plan.new_tokens,
                           starts=plan.starts, is_decode=plan.is_decode, max_len=plan.max_len,
-                          mean_len=mean_len_bound(plan.total_len, n, _len_bound(plan.max_len)),
-                          side_stream=self._side_stream(plan.n_tokens))
+                          mean_len=mean_len_bound(plan.total_len, n, _len_bound(plan.max_len)))
         return ctx, views[0], (views[6] if R else None)
 
     def forward_tokens(self, ctx: StepContext, token_ids: torch.Tensor, logit_rows: Optional[torch.Tensor]):

@@ -166,6 +166,4 @@ class StepContext:
     #: upper bound of the sequences' mean length after this step (0: not known, take ``max_len``); launches
     #: may be shaped by it, but no result depends on it
     mean_len: int = 0
-    #: a second stream on which a block may run work that does not depend on its mixer (None: do not)
-    side_stream: Any = None
     extras: Dict[str, Any] = dataclasses.field(default_factory=dict)

@@ -9,8 +9,7 @@ parallel    ``x + (ffn(norm_ffn(x)) + mixer(norm_mixer(x)))``; with one norm bot
 sequential  ``r = x + mixer(norm_in(x))``; ``r + ffn(norm_post(r))`` (:652-659, :676).
 
 The additions ride in the last matrix product's epilogue of each branch, or, in steps of few tokens,
-the products stay unreduced and the next norm forms the sum while it reads it (``ResidualSum``).  In the parallel block the
-feed-forward's first product does not depend on the mixer, so it may run beside it on a second stream.
+the products stay unreduced and the next norm forms the sum while it reads it (``ResidualSum``).
 """
 from __future__ import annotations
 
@@ -70,33 +69,21 @@ class ParallelBlock(Part):
         x, a, m = _normed(x, self.norm_mixer, self.norm_ffn)
         if m is None:
             m = a
-        side = ctx.side_stream
-        if side is None or not hasattr(self.feed_forward, "forward_up"):
-            kw_mixer, kw_ffn = {}, {}
-            # both branches start with a product of the norm's output: one launch for the two in small steps
-            if hasattr(self.mixer, "input_projection") and hasattr(self.feed_forward, "input_projection"):
-                (lin_a, kw_a), (lin_m, kw_m) = self.mixer.input_projection(), self.feed_forward.input_projection()
-                both = Linear.pair(lin_a, a, kw_a, lin_m, m, kw_m)
-                if both is not None:
-                    kw_mixer["projected"], kw_ffn["projected"] = both
-            if _can_defer(self.feed_forward) and _can_defer(self.mixer):
-                # the branches' last products: one launch of partial sums where that pays, which the
-                # next norm adds to the residual while it reads them
-                out_a = self.mixer.forward(a, ctx, call, defer=True, **kw_mixer)
-                out_m = self.feed_forward.forward(m, ctx, defer=True, **kw_ffn)
-                return _sum_parallel(out_m, out_a, x)
-            mixed = self.mixer.forward(a, ctx, call, **kw_mixer)
-            return self.feed_forward.forward(m, ctx, add1=mixed, add2=x, **kw_ffn)
-        # The feed-forward's first product needs only the norm, not the mixer: it runs on a second
-        # stream beside projection, rotation, attention and output projection, and the two meet at the
-        # feed-forward's second product, whose epilogue sums the branches and the residual.
-        main = torch.cuda.current_stream()
-        side.wait_stream(main)
-        with torch.cuda.stream(side):
-            h = self.feed_forward.forward_up(m, ctx)
-        mixed = self.mixer.forward(a, ctx, call)
-        main.wait_stream(side)
-        return self.feed_forward.forward_down(h, ctx, add1=mixed, add2=x)
+        kw_mixer, kw_ffn = {}, {}
+        # both branches start with a product of the norm's output: one launch for the two in small steps
+        if hasattr(self.mixer, "input_projection") and hasattr(self.feed_forward, "input_projection"):
+            (lin_a, kw_a), (lin_m, kw_m) = self.mixer.input_projection(), self.feed_forward.input_projection()
+            both = Linear.pair(lin_a, a, kw_a, lin_m, m, kw_m)
+            if both is not None:
+                kw_mixer["projected"], kw_ffn["projected"] = both
+        if _can_defer(self.feed_forward) and _can_defer(self.mixer):
+            # the branches' last products: one launch of partial sums where that pays, which the
+            # next norm adds to the residual while it reads them
+            out_a = self.mixer.forward(a, ctx, call, defer=True, **kw_mixer)
+            out_m = self.feed_forward.forward(m, ctx, defer=True, **kw_ffn)
+            return _sum_parallel(out_m, out_a, x)
+        mixed = self.mixer.forward(a, ctx, call, **kw_mixer)
+        return self.feed_forward.forward(m, ctx, add1=mixed, add2=x, **kw_ffn)
 
 
 class SequentialBlock(Part):

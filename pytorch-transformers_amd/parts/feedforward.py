@@ -38,13 +38,5 @@ class DenseFeedForward(Part):
             return PendingProjection(self.down, h)
         return self.down(h, add1=as_tensor(add1), add2=as_tensor(add2))
 
-    # The two halves on their own: a block whose feed-forward does not read the mixer's output can run
-    # the first half beside the mixer.
-    def forward_up(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
-        return self.up(x, act=self.activation)
-
-    def forward_down(self, h: torch.Tensor, ctx: StepContext, add1=None, add2=None) -> torch.Tensor:
-        return self.down(h, add1=as_tensor(add1), add2=as_tensor(add2))
-
 
 register_part("feed_forward", "dense", DenseFeedForward)

@@ -79,9 +79,12 @@ class Linear(Part):
             return ops.gemm_splitk_pair_bf16(*args)
         return None
 
+    def can_partial(self, x: torch.Tensor) -> bool:
+        return x.dtype == torch.bfloat16 and ops.gemm_partial_ok(x, self.weight) and ops.layernorm_sum_ok(self.out_features)
+
     def partial(self, x: torch.Tensor) -> Optional[PartialProduct]:
         """The product left as partial sums for the next norm to add, where that pays; else None."""
-        if x.dtype == torch.bfloat16 and ops.gemm_partial_ok(x, self.weight) and ops.layernorm_sum_ok(self.out_features):
+        if self.can_partial(x):
             return PartialProduct(ops.gemm_splitk_partial(x, self.weight), self.bias)
         return None
 
