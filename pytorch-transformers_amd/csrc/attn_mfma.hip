@@ -27,6 +27,9 @@
 
 #include <stdlib.h>
 
+#include <algorithm>
+#include <cmath>
+
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
@@ -88,7 +91,7 @@ __global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
     const int* __restrict__ block_table, int bt_stride, const int* __restrict__ cu_tokens,
     const int* __restrict__ seq_start, const float* __restrict__ slopes, int nh, int nkv, float scale, float alibi_mul,
-    int split_size, int n_splits, int window_arg) {
+    int split_size, int n_splits, int window_arg, int paired) {
     constexpr int D = DT * 16;
     const int window = WIN ? window_arg : 0;
     constexpr int DS = (DT + 1) / 2;   // 32-wide steps over the head dimension
@@ -97,9 +100,19 @@ __global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
     const int seq = blockIdx.z / n_splits, split = blockIdx.z % n_splits;
     const int kvh = blockIdx.y, g = nh / nkv;
     const int t0 = cu_tokens[seq], n_new = cu_tokens[seq + 1] - t0, start = seq_start[seq];
-    // column groups are handed out last first: late tokens see the most keys, and the longest work
-    // should start first so that the launch ends evenly
-    const int ncols = n_new * g, wg_col0 = (gridDim.x - 1 - blockIdx.x) * (16 * CT * W);
+    const int ncols = n_new * g, n_groups = (ncols + 16 * CT * W - 1) / (16 * CT * W);
+    // Column groups are handed out last first: late tokens see the most keys, and the longest work should
+    // start first so that the launch ends evenly.  A paired launch has half the workgroups, and each takes a
+    // late group and then the early group that mirrors it: under the causal mask the two together see as
+    // many keys as any other pair, so a launch whose workgroups are all resident at once ends evenly too.
+    for (int pass = 0; pass <= paired; ++pass) {
+    int group = (int)(gridDim.x - 1 - blockIdx.x);
+    if (paired) {
+        const int late = n_groups - 1 - (int)blockIdx.x, early = (int)blockIdx.x;
+        if (late < early || (pass == 1 && late == early)) return;
+        group = pass == 0 ? late : early;
+    }
+    const int wg_col0 = group * (16 * CT * W);
     if (wg_col0 >= ncols) return;
     const int col0 = wg_col0 + wave * (16 * CT);
     const bool active = col0 < ncols;  // W > 1: a wave past the last column still loads and waits with the others
@@ -275,31 +288,36 @@ __global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
         const int wg_last_col = min(ncols, wg_col0 + 16 * CT * W) - 1;
         const int k_end_wg = start + wg_last_col / g + 1;
         const int k_begin_wg = window > 0 ? max(0, start + wg_col0 / g - window + 1) & ~31 : 0;
-        uint4 gk[PER], gv[PER];
+        static_assert(PER <= 2, "a thread moves at most two pieces of keys and two of values per block");
+        // the pieces in flight are plain variables, not an array: an array that lambdas index stays in
+        // scratch memory at the larger head sizes, and every block then waits for its loads at once
+        uint4 gk0, gk1, gv0, gv1;
         auto gload = [&](int kb) {
             kb = min(kb, kb_last);
             const long page = bt[kb >> 6];
             const int in_page = kb & 63;
             const bf16_t* kpage = k_pool + (page * nkv + kvh) * (long)(PTA_PAGE * D);
             const bf16_t* vpage = v_pool + (page * nkv + kvh) * (long)(PTA_PAGE * D);
-#pragma unroll
-            for (int j = 0; j < PER; ++j) {
-                const int p = min(tid + j * THREADS, KPIECES - 1);
-                gk[j] = *reinterpret_cast<const uint4*>(kpage + (long)(in_page + p / CHUNKS) * D + (p % CHUNKS) * 8);
-                gv[j] = *reinterpret_cast<const uint4*>(vpage + (long)(p >> 2) * PTA_PAGE + in_page + (p & 3) * 8);
+            const int p0 = min(tid, KPIECES - 1);
+            gk0 = *reinterpret_cast<const uint4*>(kpage + (long)(in_page + p0 / CHUNKS) * D + (p0 % CHUNKS) * 8);
+            gv0 = *reinterpret_cast<const uint4*>(vpage + (long)(p0 >> 2) * PTA_PAGE + in_page + (p0 & 3) * 8);
+            if constexpr (PER > 1) {
+                const int p1 = min(tid + THREADS, KPIECES - 1);
+                gk1 = *reinterpret_cast<const uint4*>(kpage + (long)(in_page + p1 / CHUNKS) * D + (p1 % CHUNKS) * 8);
+                gv1 = *reinterpret_cast<const uint4*>(vpage + (long)(p1 >> 2) * PTA_PAGE + in_page + (p1 & 3) * 8);
+            }
+        };
+        auto put = [&](int buf, int p, const uint4& k, const uint4& v) {
+            if (p < KPIECES) {
+                const int kk = p / CHUNKS;  // key of the block -> its row in operand order
+                const int row = ((kk & 7) >> 2) * 16 + 4 * (kk >> 3) + (kk & 3);
+                *reinterpret_cast<uint4*>(&kbuf[buf][row * KROW + (p % CHUNKS) * 8]) = k;
+                *reinterpret_cast<uint4*>(&vbuf[buf][(p >> 2) * VROW + (p & 3) * 8]) = v;
             }
         };
         auto sstore = [&](int buf) {
-#pragma unroll
-            for (int j = 0; j < PER; ++j) {
-                const int p = tid + j * THREADS;
-                if (p < KPIECES) {
-                    const int kk = p / CHUNKS;  // key of the block -> its row in operand order
-                    const int row = ((kk & 7) >> 2) * 16 + 4 * (kk >> 3) + (kk & 3);
-                    *reinterpret_cast<uint4*>(&kbuf[buf][row * KROW + (p % CHUNKS) * 8]) = gk[j];
-                    *reinterpret_cast<uint4*>(&vbuf[buf][(p >> 2) * VROW + (p & 3) * 8]) = gv[j];
-                }
-            }
+            put(buf, tid, gk0, gv0);
+            if constexpr (PER > 1) put(buf, tid + THREADS, gk1, gv1);
         };
         auto lfetch = [&](KvBlock<DT>& b, int buf) {
 #pragma unroll
@@ -364,6 +382,7 @@ __global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
             }
         }
     }
+    }  // pass
 }
 
 // out[row, :] = sum_s w_s po[row, s, :] / sum_s w_s pl[row, s], w_s = 2^(pm[row, s] - max_s pm), splits in
@@ -411,17 +430,20 @@ struct AttnLaunch {
     const int *cu_tokens, *seq_start; const float* slopes;
     int n_seqs, max_new, nh, nkv; float scale;
     int split_size, n_splits, window;
+    int paired;  // workgroups take two column groups each, a late one and the early one that mirrors it
     hipStream_t s;
 };
 
 template <int DT, int CT, int W>
 static void launch_attn(const AttnLaunch& a) {
     const int g = a.nh / a.nkv;
-    const dim3 grid((a.max_new * g + 16 * CT * W - 1) / (16 * CT * W), a.nkv, a.n_seqs * a.n_splits);
+    const int groups = (a.max_new * g + 16 * CT * W - 1) / (16 * CT * W);
+    const int paired = a.paired && groups > 1 ? 1 : 0;
+    const dim3 grid(paired ? (groups + 1) / 2 : groups, a.nkv, a.n_seqs * a.n_splits);
     auto kern = a.window > 0 ? attn_mfma_kernel<DT, CT, W, true> : attn_mfma_kernel<DT, CT, W, false>;
     hipLaunchKernelGGL(kern, grid, dim3(64 * W), 0, a.s, a.out, a.po, a.pm, a.pl, a.q, a.k_pool, a.v_pool, a.block_table,
                        a.bt_stride, a.cu_tokens, a.seq_start, a.slopes, a.nh, a.nkv, a.scale * PTA_LOG2E,
-                       PTA_LOG2E / sqrtf((float)(DT * 16)), a.split_size, a.n_splits, a.window);
+                       PTA_LOG2E / sqrtf((float)(DT * 16)), a.split_size, a.n_splits, a.window, paired);
 }
 
 // column tiles (of sixteen query heads of one KV head) that one wave of a decode launch holds at most:
@@ -473,6 +495,18 @@ extern "C" int pta_attn_mfma(void* out, const void* q, const void* k_pool, const
     // path fewer times; fewer: shorter waves, more of them (71 heads on one KV head, 2,048 keys: 64
     // sequences 39.5 us a layer with one tile, 27.5 us with five; 8 sequences 14.6 and 18.5 us).
     const bool narrow = max_new == 1;
+    // Prompts: whether workgroups take a late and an early column group each.  Paired workgroups all do the
+    // same work, which ends a launch evenly if their number fills the compute units evenly; unpaired ones are
+    // twice as many and of all lengths, which the longest-first order spreads well over any number of units.
+    // In units of a mean workgroup's work a unit's share is max(n / units, 2) unpaired and 2 ceil(n / 2 / units)
+    // paired; measured at 2,048 tokens, pairs win where the two are equal (32 heads on 8 KV heads of 128:
+    // 102 -> 86 us a layer; 128 on 8 of 64: 172 -> 152) and lose where they are not (71 on 1 of 64: 75 -> 93).
+    static const int pair_env = getenv("PTA_ATTN_PAIR") ? atoi(getenv("PTA_ATTN_PAIR")) : -1;
+    int paired = 0;
+    if (!narrow) {
+        const double wgs = std::ceil((double)M * (nh / nkv) / (d <= 128 ? 128 : 16)) * nkv, units = pta_compute_units();
+        paired = pair_env >= 0 ? pair_env : 2.0 * std::ceil(wgs / 2.0 / units) <= 1.1 * std::max(wgs / units, 2.0);
+    }
     const int dct_most = std::min((nh / nkv + 15) / 16, pta_attn_decode_max_tiles(d));
     PTA_REQUIRE(decode_tiles >= 0 && decode_tiles <= dct_most,
                 "attn_mfma: %d column tiles per decode wave; these sizes allow 1..%d (0: as many as that)", decode_tiles,
@@ -480,7 +514,7 @@ extern "C" int pta_attn_mfma(void* out, const void* q, const void* k_pool, const
     const int dct = decode_tiles > 0 ? decode_tiles : dct_most;
     const AttnLaunch a{(bf16_t*)out, po, pm, pl, (const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool,
                        block_table, bt_stride, cu_tokens, seq_start, slopes, n_seqs, max_new, nh, nkv, scale,
-                       split_size, n_splits, window, s};
+                       split_size, n_splits, window, paired, s};
 #define PTA_ATTN_CASE(DT_)                                        \
     case DT_:                                                     \
         if (narrow) launch_decode<DT_>(a, dct);                   \

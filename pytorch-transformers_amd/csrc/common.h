@@ -105,6 +105,7 @@ __device__ __forceinline__ float gelu_erf(float x) { return 0.5f * x * (1.0f + e
 // Entry points return 0 on success; otherwise pta_last_error() holds the reason.
 int pta_fail(const char* fmt, ...);
 int pta_check_launch(const char* what);
+int pta_compute_units();
 
 #define PTA_REQUIRE(cond, ...) \
     do { if (!(cond)) return pta_fail(__VA_ARGS__); } while (0)

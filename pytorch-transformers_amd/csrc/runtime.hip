@@ -21,6 +21,18 @@ int pta_check_launch(const char* what) {
     return 0;
 }
 
+// compute units of the current device (asked once per device; 256 if the runtime will not say)
+int pta_compute_units() {
+    static int units[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (units[dev] == 0) {
+        int n = 0;
+        units[dev] = (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) ? n : 256;
+    }
+    return units[dev];
+}
+
 extern "C" const char* pta_last_error(void) { return g_error; }
 
 extern "C" int pta_abi_version(void) { return PTA_ABI_VERSION; }
