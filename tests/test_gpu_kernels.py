@@ -160,6 +160,26 @@ def test_layernorm_sum(H, case):
     assert x_none is None and torch.equal(o1b, o1)
 
 
+@pytest.mark.parametrize("H", [64, 200, 4544, 5000, 8192])
+@pytest.mark.parametrize("M", [512, 515, 1031])
+def test_layernorm_sum_of_many_rows(H, M):
+    """From 512 rows on a wave takes a row (the arrangement for prompts): one or two tensors, with and without
+    the sum as an output, one or two norms; rows beyond a multiple of four and widths that leave lanes idle."""
+    ops = _ops()
+    x1, x2 = _rand(M, H, seed=4, dtype=torch.bfloat16), _rand(M, H, seed=5, dtype=torch.bfloat16)
+    w, b, w2, b2 = _rand(H, seed=6) + 1.0, _rand(H, seed=7), _rand(H, seed=8) + 1.0, _rand(H, seed=9)
+    for terms, want in (([x1], x1), ([x1, x2], (x1.float() + x2.float()).bfloat16())):
+        x, o1, o2 = ops.layernorm_sum(terms, H, w=w, b=b, eps=1e-5, w2=w2, b2=b2)
+        assert torch.equal(x, want)
+        for o, (ww, bb) in ((o1, (w, b)), (o2, (w2, b2))):
+            torch.testing.assert_close(o.float(), F.layer_norm(want.float(), (H,), ww, bb, 1e-5), rtol=1e-2, atol=1e-2)
+        x_none, o1b, o2b = ops.layernorm_sum(terms, H, w=w, b=b, eps=1e-5, want_x=False)
+        assert x_none is None and o2b is None and torch.equal(o1b, o1)
+        few = ops.layernorm_sum([t[:7] for t in terms], H, w=w, b=b, eps=1e-5)[1]  # a workgroup per row
+        torch.testing.assert_close(o1[:7].float(), few.float(), rtol=1e-2, atol=1e-2)
+    assert torch.equal(ops.layernorm_sum([x1, x2], H)[0], (x1.float() + x2.float()).bfloat16())
+
+
 def test_layernorm_sum_refuses_what_it_cannot_do():
     ops = _ops()
     assert not ops.layernorm_sum_ok(100) and not ops.layernorm_sum_ok(8200) and ops.layernorm_sum_ok(8192)
