@@ -9,10 +9,16 @@
 //
 // Thresholds are found without sorting: the k-th largest score by a radix search on counts, the
 // top-p cut by a radix search on probability mass held in 40-bit fixed point, so that both are
-// sums of integers and do not depend on the order in which threads add.  The draw inverts the
-// cumulative distribution in index order with a fixed summation order, from a uniform number of a
-// counter-based generator keyed by (seed, sequence, step): a sequence draws the same token alone or
-// in any batch.
+// sums of integers and do not depend on the order in which threads add.  The searches run over short
+// candidate lists where they can (LDS atomics of 65,000 scores that share a few exponent bytes take
+// tens of microseconds a pass): the k-th largest of the threads' maxima is a lower bound of the k-th
+// largest score, so the scores at or above it are few and hold the threshold; the top-p cut lies among
+// the scores that still have mass after top-k, or among those above the 512th largest thread maximum
+// if the mass below them fits into 1 - p.  Where a list would overflow, or the cut lies below it, the
+// same searches run over the whole row.  The draw inverts the cumulative distribution in index order
+// with a fixed summation order (a wave per sixteenth of the row, sums of lanes, then of waves), from
+// a uniform number of a counter-based generator keyed by (seed, sequence, step): a sequence draws the
+// same token alone or in any batch.
 #include "common.h"
 #include "pta_kernels.h"
 
@@ -106,6 +112,121 @@ extern "C" int pta_argmax(int* out_tok, const float* logits, int R, int V, void*
 }
 
 #define MASS_ONE 1099511627776.0f /* 2^40 */
+#define S_CAP 2048  // candidates a list holds
+
+struct SampleShared {
+    float red[16];
+    int red_i[16];
+    unsigned long long red_q[16];
+    float seg[S_THREADS / 64];
+    uint32_t cnt[256];
+    unsigned long long mass[256];
+    uint32_t tkey[S_THREADS];  // the threads' largest scores as keys
+    uint32_t cand_key[S_CAP];
+    unsigned long long cand_q[S_CAP];
+    uint32_t bin, remaining, all, n_cand;
+    unsigned long long cum;
+};
+
+__device__ __forceinline__ unsigned long long wave_sum_u64(unsigned long long v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+// every thread gets the sum; integers, so any order gives the same bits
+__device__ __forceinline__ unsigned long long block_sum_u64(unsigned long long v, unsigned long long* red) {
+    v = wave_sum_u64(v);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    __syncthreads();
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    unsigned long long t = 0;
+    for (int i = 0; i < S_THREADS / 64; ++i) t += red[i];
+    return t;
+}
+
+// inclusive sums over the block's threads in thread order (integers)
+__device__ __forceinline__ unsigned long long block_scan_u64(unsigned long long v, unsigned long long* red) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const unsigned long long up = __shfl_up(v, o, 64);
+        if (lane >= o) v += up;
+    }
+    __syncthreads();
+    if (lane == 63) red[wave] = v;
+    __syncthreads();
+    for (int w = 0; w < wave; ++w) v += red[w];
+    return v;
+}
+
+// Key of the `want`-th largest (1-based, want <= n) of the n keys of a list in LDS: one byte of the key at a
+// time from the top, counts per byte value, the bin picked by all threads together.  Every thread gets it.
+__device__ __forceinline__ uint32_t list_kth_largest(SampleShared& sh, const uint32_t* keys, int n, uint32_t want) {
+    const int tid = threadIdx.x;
+    uint32_t prefix = 0, maskbits = 0, rem = want;
+    for (int shift = 24; shift >= 0; shift -= 8) {
+        __syncthreads();
+        if (tid < 256) sh.cnt[tid] = 0;
+        __syncthreads();
+        for (int c = tid; c < n; c += S_THREADS) {
+            const uint32_t k = keys[c];
+            if ((k & maskbits) == prefix) atomicAdd(&sh.cnt[(k >> shift) & 255u], 1u);
+        }
+        __syncthreads();
+        // thread t < 256 stands for bin 255 - t: the inclusive sum counts the keys in its bin and above
+        const uint32_t mine = tid < 256 ? sh.cnt[255 - tid] : 0u;
+        const uint32_t from_top = (uint32_t)block_scan_u64(mine, sh.red_q);
+        if (tid < 256 && from_top >= rem && from_top - mine < rem) {
+            sh.bin = (uint32_t)(255 - tid);
+            sh.remaining = rem - (from_top - mine);
+        }
+        __syncthreads();
+        prefix |= sh.bin << shift;
+        maskbits |= 255u << shift;
+        rem = sh.remaining;
+    }
+    __syncthreads();
+    return prefix;
+}
+
+// The top-p cut over the list of (key, mass) in LDS, `low` being the mass of the scores below every key of
+// the list (low <= T): the lowest key whose mass, with everything below it, passes T.  Returns false if none
+// does (everything could go); else `key` is that key and `below` the mass below it.
+__device__ __forceinline__ bool list_mass_cut(SampleShared& sh, int n, unsigned long long low, unsigned long long T,
+                                              uint32_t& key, unsigned long long& below) {
+    const int tid = threadIdx.x;
+    uint32_t prefix = 0, maskbits = 0;
+    unsigned long long cum = low;
+    for (int shift = 24; shift >= 0; shift -= 8) {
+        __syncthreads();
+        if (tid < 256) sh.mass[tid] = 0ull;
+        if (tid == 0) sh.bin = 256u;
+        __syncthreads();
+        for (int c = tid; c < n; c += S_THREADS) {
+            const uint32_t k = sh.cand_key[c];
+            const unsigned long long q = sh.cand_q[c];
+            if ((k & maskbits) == prefix && q) atomicAdd(&sh.mass[(k >> shift) & 255u], q);
+        }
+        __syncthreads();
+        const unsigned long long mine = tid < 256 ? sh.mass[tid] : 0ull;
+        const unsigned long long upto = block_scan_u64(mine, sh.red_q);  // mass of bins 0 .. tid
+        if (tid < 256 && cum + upto > T && cum + upto - mine <= T) {      // the first bin that passes T
+            sh.bin = (uint32_t)tid;
+            sh.cum = cum + upto - mine;
+        }
+        __syncthreads();
+        if (sh.bin == 256u) return false;
+        prefix |= sh.bin << shift;
+        maskbits |= 255u << shift;
+        cum = sh.cum;
+    }
+    __syncthreads();
+    key = prefix;
+    below = cum;
+    return true;
+}
 
 __global__ __launch_bounds__(S_THREADS) void sample_kernel(
     int* __restrict__ out_tok, float* __restrict__ work, const float* __restrict__ logits, int V, int do_sample,
@@ -113,15 +234,16 @@ __global__ __launch_bounds__(S_THREADS) void sample_kernel(
     const int* __restrict__ hist_off, const int* __restrict__ eos, int n_eos, const int* __restrict__ suppress,
     int remove_invalid, int renorm, uint64_t seed, const int* __restrict__ rng_seq, const int* __restrict__ rng_step,
     const float* __restrict__ uniforms) {
-    __shared__ float red[16];
-    __shared__ int red_i[16];
-    __shared__ uint32_t cnt[256];
-    __shared__ unsigned long long mass[256];
-    __shared__ float csum[S_THREADS];
-    __shared__ uint32_t sh_bin, sh_remaining, sh_all;
-    __shared__ unsigned long long sh_cum;
-    __shared__ int sh_pick;
-    __shared__ float sh_target;
+    __shared__ SampleShared sh;
+    float* const red = sh.red;
+    int* const red_i = sh.red_i;
+    uint32_t* const cnt = sh.cnt;
+    unsigned long long* const mass = sh.mass;
+    uint32_t& sh_bin = sh.bin;
+    uint32_t& sh_remaining = sh.remaining;
+    uint32_t& sh_all = sh.all;
+    unsigned long long& sh_cum = sh.cum;
+    const int n_holding = min(V, S_THREADS);  // threads that hold scores
 
     const int row = blockIdx.x, tid = threadIdx.x;
     float* w = work + (long)row * V;
@@ -161,27 +283,53 @@ __global__ __launch_bounds__(S_THREADS) void sample_kernel(
             __syncthreads();
         }
         if (top_k > 0 && top_k < V) {
-            // key of the k-th largest score, one byte at a time from the top
             uint32_t prefix = 0, maskbits = 0;
-            if (tid == 0) sh_remaining = (uint32_t)top_k;
-            for (int shift = 24; shift >= 0; shift -= 8) {
-                if (tid < 256) cnt[tid] = 0;
+            bool found = false;
+            if (top_k <= n_holding) {
+                // the k-th largest of the threads' maxima bounds the k-th largest score from below: the scores
+                // at or above it are few, and the k-th largest of those is the threshold
+                float m = -INFINITY;
+                for (int i = tid; i < V; i += S_THREADS) m = fmaxf(m, w[i]);
+                sh.tkey[tid] = tid < V ? order_key(m) : 0u;
+                const uint32_t bound = list_kth_largest(sh, sh.tkey, S_THREADS, (uint32_t)top_k);
+                if (tid == 0) sh.n_cand = 0u;
                 __syncthreads();
                 for (int i = tid; i < V; i += S_THREADS) {
                     const uint32_t k = order_key(w[i]);
-                    if ((k & maskbits) == prefix) atomicAdd(&cnt[(k >> shift) & 255u], 1u);
+                    if (k >= bound) {
+                        const uint32_t at = atomicAdd(&sh.n_cand, 1u);
+                        if (at < S_CAP) sh.cand_key[at] = k;
+                    }
                 }
                 __syncthreads();
-                if (tid == 0) {
-                    uint32_t rem = sh_remaining;
-                    int b = 255;
-                    while (b > 0 && cnt[b] < rem) { rem -= cnt[b]; --b; }
-                    sh_bin = (uint32_t)b;
-                    sh_remaining = rem;
+                if (sh.n_cand <= S_CAP) {
+                    prefix = list_kth_largest(sh, sh.cand_key, (int)sh.n_cand, (uint32_t)top_k);
+                    found = true;
                 }
+            }
+            if (!found) {
+                // key of the k-th largest score over the whole row, one byte at a time from the top
                 __syncthreads();
-                prefix |= sh_bin << shift;
-                maskbits |= 255u << shift;
+                if (tid == 0) sh_remaining = (uint32_t)top_k;
+                for (int shift = 24; shift >= 0; shift -= 8) {
+                    if (tid < 256) cnt[tid] = 0;
+                    __syncthreads();
+                    for (int i = tid; i < V; i += S_THREADS) {
+                        const uint32_t k = order_key(w[i]);
+                        if ((k & maskbits) == prefix) atomicAdd(&cnt[(k >> shift) & 255u], 1u);
+                    }
+                    __syncthreads();
+                    if (tid == 0) {
+                        uint32_t rem = sh_remaining;
+                        int b = 255;
+                        while (b > 0 && cnt[b] < rem) { rem -= cnt[b]; --b; }
+                        sh_bin = (uint32_t)b;
+                        sh_remaining = rem;
+                    }
+                    __syncthreads();
+                    prefix |= sh_bin << shift;
+                    maskbits |= 255u << shift;
+                }
             }
             for (int i = tid; i < V; i += S_THREADS)
                 if (order_key(w[i]) < prefix) w[i] = -INFINITY;
@@ -190,38 +338,77 @@ __global__ __launch_bounds__(S_THREADS) void sample_kernel(
         if (top_p < 1.0f) {
             float mx = -INFINITY;
             int mi = 0x7fffffff;
-            for (int i = tid; i < V; i += S_THREADS)
-                if (w[i] > mx) { mx = w[i]; mi = i; }
+            unsigned long long finite = 0ull;
+            for (int i = tid; i < V; i += S_THREADS) {
+                const float x = w[i];
+                if (x > mx) { mx = x; mi = i; }
+                finite += x != -INFINITY ? 1ull : 0ull;
+            }
             const ArgBest best = block_argmax(mx, mi, red, red_i);
             float s = 0.f;
             for (int i = tid; i < V; i += S_THREADS) s += expf(w[i] - best.v);
             const float Z = block_sum(s, red);
             const unsigned long long T = (unsigned long long)((double)(1.0f - top_p) * (double)MASS_ONE);
-            uint32_t prefix = 0, maskbits = 0;
-            if (tid == 0) { sh_cum = 0ull; sh_all = 0u; }
-            for (int shift = 24; shift >= 0; shift -= 8) {
-                if (tid < 256) mass[tid] = 0ull;
-                __syncthreads();
-                for (int i = tid; i < V; i += S_THREADS) {
-                    const uint32_t k = order_key(w[i]);
-                    if ((k & maskbits) == prefix) {
-                        const unsigned long long q = (unsigned long long)(expf(w[i] - best.v) / Z * MASS_ONE + 0.5f);
-                        if (q) atomicAdd(&mass[(k >> shift) & 255u], q);
+            // The candidates: every score that is left if those are few (after top-k), else the scores from the
+            // 512th largest thread maximum up, if the mass of all the others fits into 1 - p.
+            const unsigned long long n_finite = block_sum_u64(finite, sh.red_q);
+            uint32_t from = order_key(-INFINITY) + 1u;
+            if (n_finite > S_CAP) {
+                sh.tkey[tid] = tid < V ? order_key(mx) : 0u;
+                from = list_kth_largest(sh, sh.tkey, S_THREADS, (uint32_t)min(512, n_holding));
+            }
+            __syncthreads();
+            if (tid == 0) sh.n_cand = 0u;
+            __syncthreads();
+            unsigned long long others = 0ull;
+            for (int i = tid; i < V; i += S_THREADS) {
+                const uint32_t k = order_key(w[i]);
+                if (k >= from) {
+                    const uint32_t at = atomicAdd(&sh.n_cand, 1u);
+                    if (at < S_CAP) {
+                        sh.cand_key[at] = k;
+                        sh.cand_q[at] = (unsigned long long)(expf(w[i] - best.v) / Z * MASS_ONE + 0.5f);
                     }
+                } else if (n_finite > S_CAP) {
+                    others += (unsigned long long)(expf(w[i] - best.v) / Z * MASS_ONE + 0.5f);
                 }
+            }
+            const unsigned long long low = block_sum_u64(others, sh.red_q);
+            uint32_t prefix = 0, maskbits = 0;
+            if (sh.n_cand <= S_CAP && low <= T) {
+                unsigned long long below = 0ull;
+                const bool cut = list_mass_cut(sh, (int)sh.n_cand, low, T, prefix, below);
                 __syncthreads();
-                if (tid == 0) {
-                    unsigned long long cum = sh_cum;
-                    int b = 0;
-                    while (b < 256 && cum + mass[b] <= T) { cum += mass[b]; ++b; }
-                    if (b == 256) { sh_all = 1u; b = 255; }
-                    sh_bin = (uint32_t)b;
-                    sh_cum = cum;
+                if (tid == 0) { sh_all = cut ? 0u : 1u; sh_cum = below; }
+                __syncthreads();
+            } else {
+                // the cut by mass over the whole row, one byte of the key at a time
+                __syncthreads();
+                if (tid == 0) { sh_cum = 0ull; sh_all = 0u; }
+                for (int shift = 24; shift >= 0; shift -= 8) {
+                    if (tid < 256) mass[tid] = 0ull;
+                    __syncthreads();
+                    for (int i = tid; i < V; i += S_THREADS) {
+                        const uint32_t k = order_key(w[i]);
+                        if ((k & maskbits) == prefix) {
+                            const unsigned long long q = (unsigned long long)(expf(w[i] - best.v) / Z * MASS_ONE + 0.5f);
+                            if (q) atomicAdd(&mass[(k >> shift) & 255u], q);
+                        }
+                    }
+                    __syncthreads();
+                    if (tid == 0) {
+                        unsigned long long cum = sh_cum;
+                        int b = 0;
+                        while (b < 256 && cum + mass[b] <= T) { cum += mass[b]; ++b; }
+                        if (b == 256) { sh_all = 1u; b = 255; }
+                        sh_bin = (uint32_t)b;
+                        sh_cum = cum;
+                    }
+                    __syncthreads();
+                    if (sh_all) break;
+                    prefix |= sh_bin << shift;
+                    maskbits |= 255u << shift;
                 }
-                __syncthreads();
-                if (sh_all) break;
-                prefix |= sh_bin << shift;
-                maskbits |= 255u << shift;
             }
             // prefix: the lowest key that stays.  If everything could go, the largest score stays.
             const uint32_t keep_from = sh_all ? order_key(best.v) : prefix;
@@ -266,42 +453,53 @@ __global__ __launch_bounds__(S_THREADS) void sample_kernel(
     int chosen = best.i;
     float Z = 0.f;
     if (do_sample || renorm) {
-        const int chunk = (V + S_THREADS - 1) / S_THREADS;
-        const int lo = min(V, tid * chunk), hi = min(V, lo + chunk);
+        // A wave per sixteenth of the row (a multiple of 64 scores): its lanes add every 64th exponential, the
+        // wave adds its lanes, and every thread adds the sixteen sums in order.
+        const int lane = tid & 63, wave = tid >> 6, n_waves = S_THREADS / 64;
+        const int span = ((V + n_waves - 1) / n_waves + 63) & ~63;
+        const int lo = min(V, wave * span), hi = min(V, lo + span);
         float s = 0.f;
-        for (int i = lo; i < hi; ++i) s += expf(w[i] - best.v);
-        csum[tid] = s;
+        for (int i = lo + lane; i < hi; i += 64) s += expf(w[i] - best.v);
+        s = wave_sum(s);
         __syncthreads();
-        if (tid == 0) {
-            float total = 0.f;
-            for (int t = 0; t < S_THREADS; ++t) total += csum[t];
-            red[0] = total;
-            if (do_sample) {
-                const float u = uniforms ? uniforms[row] : uniform_of(seed, (uint32_t)rng_seq[row], (uint32_t)rng_step[row]);
-                const float target = u * total;
-                float acc = 0.f;
-                int pick = -1, last_nonzero = 0;
-                for (int t = 0; t < S_THREADS; ++t) {
-                    if (csum[t] > 0.f) last_nonzero = t;
-                    if (pick < 0 && acc + csum[t] > target) { pick = t; sh_target = target - acc; }
-                    if (pick < 0) acc += csum[t];
+        if (lane == 0) sh.seg[wave] = s;
+        __syncthreads();
+        float total = 0.f;
+        for (int k = 0; k < n_waves; ++k) total += sh.seg[k];
+        Z = total;
+        if (do_sample) {
+            const float u = uniforms ? uniforms[row] : uniform_of(seed, (uint32_t)rng_seq[row], (uint32_t)rng_step[row]);
+            const float target = u * total;
+            // the sixteenth in which the cumulative sum passes the target, and what is left of the target there;
+            // if rounding leaves none, the last one that has mass, to its last token with mass
+            float acc = 0.f, left = INFINITY;
+            int pick = -1, last_nonzero = 0;
+            for (int k = 0; k < n_waves; ++k) {
+                if (sh.seg[k] > 0.f) last_nonzero = k;
+                if (pick < 0 && acc + sh.seg[k] > target) { pick = k; left = target - acc; }
+                if (pick < 0) acc += sh.seg[k];
+            }
+            if (pick < 0) pick = last_nonzero;
+            if (wave == pick) {
+                float before = 0.f;
+                int tok = -1, last = lo;
+                for (int i0 = lo; i0 < hi && tok < 0; i0 += 64) {
+                    const int i = i0 + lane;
+                    const float e = i < hi ? expf(w[i] - best.v) : 0.f;
+                    float incl = e;
+#pragma unroll
+                    for (int o = 1; o < 64; o <<= 1) {
+                        const float up = __shfl_up(incl, o, 64);
+                        if (lane >= o) incl += up;
+                    }
+                    const unsigned long long has_mass = __ballot(e > 0.f);
+                    const unsigned long long passed = __ballot(before + incl > left);
+                    if (has_mass) last = i0 + 63 - __clzll(has_mass);
+                    if (passed) tok = i0 + __ffsll((long long)passed) - 1;
+                    before += __shfl(incl, 63, 64);
                 }
-                if (pick < 0) { pick = last_nonzero; sh_target = INFINITY; }
-                sh_pick = pick;
+                if (lane == 0) out_tok[row] = tok >= 0 ? tok : last;
             }
-        }
-        __syncthreads();
-        Z = red[0];
-        if (do_sample && tid == sh_pick) {
-            float acc = 0.f;
-            int tok = -1, last = lo;
-            for (int i = lo; i < hi; ++i) {
-                const float e = expf(w[i] - best.v);
-                if (e > 0.f) last = i;
-                acc += e;
-                if (acc > sh_target) { tok = i; break; }
-            }
-            out_tok[row] = tok >= 0 ? tok : last;
         }
     }
     if (!do_sample && tid == 0) out_tok[row] = chosen;
