@@ -113,6 +113,7 @@ extern "C" int pta_argmax(int* out_tok, const float* logits, int R, int V, void*
 
 #define MASS_ONE 1099511627776.0f /* 2^40 */
 #define S_CAP 2048  // candidates a list holds
+#define S_SHORT 256  // candidates of the short way, which sorts them by counting
 
 struct SampleShared {
     float red[16];
@@ -126,6 +127,11 @@ struct SampleShared {
     unsigned long long cand_q[S_CAP];
     uint32_t bin, remaining, all, n_cand;
     unsigned long long cum;
+    // the short way (sample_short): scores seen before, scores that are left, and the survivors in index order
+    uint32_t seen[2048], left[2048];
+    uint32_t cand_idx[S_SHORT];
+    uint32_t s_key[S_SHORT], s_idx[S_SHORT], s_alive[S_SHORT];
+    uint32_t pick, last_mass;
 };
 
 __device__ __forceinline__ unsigned long long wave_sum_u64(unsigned long long v) {
@@ -228,12 +234,181 @@ __device__ __forceinline__ bool list_mass_cut(SampleShared& sh, int n, unsigned 
     return true;
 }
 
+// inclusive sums over the block's threads in thread order, with a fixed tree: inside a wave by doubling
+// steps, then the waves' totals in order
+__device__ __forceinline__ float block_scan_f32(float v, float* red) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const float up = __shfl_up(v, o, 64);
+        if (lane >= o) v += up;
+    }
+    __syncthreads();
+    if (lane == 63) red[wave] = v;
+    __syncthreads();
+    float before = 0.f;
+    for (int w = 0; w < wave; ++w) before += red[w];
+    return before + v;
+}
+
+__device__ __forceinline__ float key_value(uint32_t k) {
+    return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
+}
+
+// The short way for a draw with top-k, up to 65,536 scores: two passes over the row (one for the threads'
+// maxima, one that lists the scores at or above the bound they give), then everything on that list: the
+// k-th largest, the survivors in index order, the top-p cut by integer masses, min-p, the draw.  The row is
+// never written unless the processed scores are wanted.  Sums of exponentials run over the survivors in
+// index order with a fixed tree, so they can round differently from the sums over the whole row (whose
+// other terms are zero), but never depend on the batch.  Returns false, having written nothing, if the list
+// would have more than S_SHORT entries (many equal scores, or a large k): then the long way runs.
+__device__ __forceinline__ bool sample_short(
+    SampleShared& sh, int* __restrict__ out_tok, float* __restrict__ work, const float* __restrict__ l, int row, int V,
+    float temperature, int top_k, float top_p, float min_p, float penalty, const int* __restrict__ hist,
+    const int* __restrict__ hist_off, const int* __restrict__ eos, int n_eos, bool suppress_eos, int remove_invalid,
+    int renorm, float u) {
+    const int tid = threadIdx.x;
+    const bool penalize = hist_off && penalty != 1.0f;
+    if (penalize) {
+        for (int w = tid; w < 2048; w += S_THREADS) sh.seen[w] = 0u;
+        __syncthreads();
+        for (int t = hist_off[row] + tid; t < hist_off[row + 1]; t += S_THREADS) {
+            const int tok = hist[t];
+            if (tok >= 0 && tok < V) atomicOr(&sh.seen[tok >> 5], 1u << (tok & 31));
+        }
+        __syncthreads();
+    }
+    // the processed score of token i, with the operations of the long way in their order
+    auto score = [&](int i) {
+        float x = l[i];
+        if (penalize && ((sh.seen[i >> 5] >> (i & 31)) & 1u)) x = x < 0.f ? x * penalty : x / penalty;
+        if (suppress_eos)
+            for (int e = 0; e < n_eos; ++e)
+                if (eos[e] == i) x = -INFINITY;
+        if (remove_invalid) {
+            if (x != x) x = 0.f;
+            else if (x == INFINITY) x = FLT_MAX;
+            else if (x == -INFINITY) x = -FLT_MAX;
+        }
+        if (temperature != 1.0f) x = x / temperature;
+        return x;
+    };
+    float m = -INFINITY, mx = -INFINITY;
+    int mi = 0x7fffffff;
+    for (int i = tid; i < V; i += S_THREADS) {
+        const float x = score(i);
+        m = fmaxf(m, x);
+        if (x > mx) { mx = x; mi = i; }
+    }
+    sh.tkey[tid] = tid < V ? order_key(m) : 0u;
+    const ArgBest best = block_argmax(mx, mi, sh.red, sh.red_i);
+    const uint32_t bound = list_kth_largest(sh, sh.tkey, S_THREADS, (uint32_t)top_k);
+    if (tid == 0) sh.n_cand = 0u;
+    __syncthreads();
+    for (int i = tid; i < V; i += S_THREADS) {
+        const uint32_t k = order_key(score(i));
+        if (k >= bound) {
+            const uint32_t at = atomicAdd(&sh.n_cand, 1u);
+            if (at < S_SHORT) { sh.cand_key[at] = k; sh.cand_idx[at] = (uint32_t)i; }
+        }
+    }
+    __syncthreads();
+    const int n = (int)sh.n_cand;
+    if (n > S_SHORT) return false;
+    const uint32_t kth = list_kth_largest(sh, sh.cand_key, n, (uint32_t)top_k);
+    // survivors in index order: a survivor's place is the number of survivors before it
+    if (tid == 0) sh.n_cand = 0u;
+    __syncthreads();
+    if (tid < n && sh.cand_key[tid] >= kth) {
+        uint32_t place = 0;
+        for (int o = 0; o < n; ++o) place += (sh.cand_key[o] >= kth && sh.cand_idx[o] < sh.cand_idx[tid]) ? 1u : 0u;
+        sh.s_key[place] = sh.cand_key[tid];
+        sh.s_idx[place] = sh.cand_idx[tid];
+        sh.s_alive[place] = 1u;
+        atomicAdd(&sh.n_cand, 1u);
+    }
+    __syncthreads();
+    const int ns = (int)sh.n_cand;  // at least top_k
+    const bool mine = tid < ns;
+    const float x = mine ? key_value(sh.s_key[tid]) : -INFINITY;
+    if (top_p < 1.0f) {
+        const float e = mine ? expf(x - best.v) : 0.f;
+        const float incl = block_scan_f32(e, sh.red);
+        __syncthreads();
+        if (tid == ns - 1) sh.seg[0] = incl;
+        __syncthreads();
+        const float Z = sh.seg[0];
+        const unsigned long long T = (unsigned long long)((double)(1.0f - top_p) * (double)MASS_ONE);
+        if (mine) {
+            sh.cand_key[tid] = sh.s_key[tid];
+            sh.cand_q[tid] = (unsigned long long)(e / Z * MASS_ONE + 0.5f);
+        }
+        uint32_t cut = 0;
+        unsigned long long below = 0ull;
+        const bool found = list_mass_cut(sh, ns, 0ull, T, cut, below);
+        const uint32_t keep_from = found ? cut : order_key(best.v);  // if everything could go, the largest stays
+        __syncthreads();
+        if (mine && sh.s_key[tid] < keep_from) sh.s_alive[tid] = 0u;
+        if (found) {
+            // equal scores at the cut: in index order the first of them go while they fit, never the last
+            const unsigned long long q = (unsigned long long)(expf(key_value(cut) - best.v) / Z * MASS_ONE + 0.5f);
+            const unsigned long long r = q ? (T - below) / q : 0ull;
+            if (r > 0 && mine && sh.s_key[tid] == cut) {
+                uint32_t before = 0, ties = 0;
+                for (int o = 0; o < ns; ++o) {
+                    const bool tie = sh.s_key[o] == cut;
+                    ties += tie ? 1u : 0u;
+                    before += (tie && o < tid) ? 1u : 0u;
+                }
+                if (before < r && before != ties - 1) sh.s_alive[tid] = 0u;
+            }
+        }
+        __syncthreads();
+    }
+    if (min_p > 0.0f) {
+        const float e = (mine && sh.s_alive[tid]) ? expf(x - best.v) : 0.f;
+        const float incl = block_scan_f32(e, sh.red);
+        __syncthreads();
+        if (tid == ns - 1) sh.seg[0] = incl;
+        __syncthreads();
+        const float Z = sh.seg[0];
+        const float thr = min_p * (1.0f / Z);
+        if (mine && x != best.v && e / Z < thr) sh.s_alive[tid] = 0u;
+        __syncthreads();
+    }
+    // the draw over the survivors in index order
+    const float e = (mine && sh.s_alive[tid]) ? expf(x - best.v) : 0.f;
+    const float incl = block_scan_f32(e, sh.red);
+    __syncthreads();
+    if (tid == ns - 1) sh.seg[0] = incl;
+    if (tid == 0) { sh.pick = 0xffffffffu; sh.last_mass = 0u; }
+    __syncthreads();
+    const float total = sh.seg[0];
+    const float target = u * total;
+    if (mine && incl > target) atomicMin(&sh.pick, (uint32_t)tid);
+    if (mine && e > 0.f) atomicMax(&sh.last_mass, (uint32_t)tid);
+    __syncthreads();
+    if (tid == 0) out_tok[row] = (int)sh.s_idx[sh.pick != 0xffffffffu ? sh.pick : sh.last_mass];
+    if (work) {
+        // the processed scores: the survivors keep theirs, everything else is gone
+        for (int w = tid; w < 2048; w += S_THREADS) sh.left[w] = 0u;
+        __syncthreads();
+        if (mine && sh.s_alive[tid]) atomicOr(&sh.left[sh.s_idx[tid] >> 5], 1u << (sh.s_idx[tid] & 31));
+        __syncthreads();
+        const float lse = renorm ? best.v + logf(total) : 0.f;
+        float* w = work + (long)row * V;
+        for (int i = tid; i < V; i += S_THREADS)
+            w[i] = ((sh.left[i >> 5] >> (i & 31)) & 1u) ? score(i) - lse : -INFINITY;
+    }
+    return true;
+}
+
 __global__ __launch_bounds__(S_THREADS) void sample_kernel(
     int* __restrict__ out_tok, float* __restrict__ work, const float* __restrict__ logits, int V, int do_sample,
     float temperature, int top_k, float top_p, float min_p, float penalty, const int* __restrict__ hist,
     const int* __restrict__ hist_off, const int* __restrict__ eos, int n_eos, const int* __restrict__ suppress,
     int remove_invalid, int renorm, uint64_t seed, const int* __restrict__ rng_seq, const int* __restrict__ rng_step,
-    const float* __restrict__ uniforms) {
+    const float* __restrict__ uniforms, int want_scores) {
     __shared__ SampleShared sh;
     float* const red = sh.red;
     int* const red_i = sh.red_i;
@@ -249,6 +424,13 @@ __global__ __launch_bounds__(S_THREADS) void sample_kernel(
     float* w = work + (long)row * V;
     const float* l = logits + (long)row * V;
 
+    if (do_sample && top_k > 0 && top_k < V && top_k <= n_holding && top_k <= S_SHORT && V <= 65536) {
+        const float u = uniforms ? uniforms[row] : uniform_of(seed, (uint32_t)rng_seq[row], (uint32_t)rng_step[row]);
+        if (sample_short(sh, out_tok, want_scores ? work : nullptr, l, row, V, temperature, top_k, top_p, min_p, penalty,
+                         hist, hist_off, eos, n_eos, suppress && suppress[row], remove_invalid, renorm, u))
+            return;
+        __syncthreads();
+    }
     for (int i = tid; i < V; i += S_THREADS) w[i] = l[i];
     __syncthreads();
     if (hist_off && penalty != 1.0f) {
@@ -415,17 +597,28 @@ __global__ __launch_bounds__(S_THREADS) void sample_kernel(
             for (int i = tid; i < V; i += S_THREADS)
                 if (order_key(w[i]) < keep_from) w[i] = -INFINITY;
             __syncthreads();
-            if (!sh_all && tid == 0) {
-                // equal scores at the cut: in ascending stable order the first of them go while they fit
-                const float vcut = __uint_as_float((prefix & 0x80000000u) ? (prefix & 0x7fffffffu) : ~prefix);
+            if (!sh_all) {
+                // equal scores at the cut: in index order the first of them go while they fit, never the last one
+                // (one token at least stays).  Tiles of consecutive tokens, the tied ones numbered by a scan.
+                const float vcut = key_value(prefix);
                 const unsigned long long q = (unsigned long long)(expf(vcut - best.v) / Z * MASS_ONE + 0.5f);
-                unsigned long long r = q ? (T - sh_cum) / q : 0ull;
+                const unsigned long long r = q ? (T - sh_cum) / q : 0ull;
                 if (r > 0) {
-                    // never the last one: one token at least stays
-                    int last = -1;
-                    for (int i = 0; i < V; ++i) if (order_key(w[i]) == prefix) last = i;
-                    for (int i = 0; i < V && r > 0; ++i)
-                        if (i != last && order_key(w[i]) == prefix) { w[i] = -INFINITY; --r; }
+                    unsigned long long mine = 0ull;
+                    for (int i = tid; i < V; i += S_THREADS) mine += order_key(w[i]) == prefix ? 1ull : 0ull;
+                    const unsigned long long ties = block_sum_u64(mine, sh.red_q);
+                    unsigned long long before = 0ull;
+                    for (int i0 = 0; i0 < V && before < r; i0 += S_THREADS) {
+                        const int i = i0 + tid;
+                        const bool tie = i < V && order_key(w[i]) == prefix;
+                        const unsigned long long upto = block_scan_u64(tie ? 1ull : 0ull, sh.red_q);
+                        const unsigned long long place = before + upto - 1;  // of a tied score, from 0
+                        if (tie && place < r && place != ties - 1) w[i] = -INFINITY;
+                        __syncthreads();
+                        if (tid == S_THREADS - 1) sh_cum = upto;
+                        __syncthreads();
+                        before += sh_cum;
+                    }
                 }
             }
             __syncthreads();
@@ -514,7 +707,7 @@ extern "C" int pta_sample(int* out_tok, float* work, const float* logits, int R,
                           float temperature, int top_k, float top_p, float min_p, float penalty, const int* hist,
                           const int* hist_off, const int* eos, int n_eos, const int* suppress, int remove_invalid,
                           int renorm, uint64_t seed, const int* rng_seq, const int* rng_step, const float* uniforms,
-                          void* stream) {
+                          int want_scores, void* stream) {
     PTA_REQUIRE(R > 0 && V > 0, "sample: rows=%d vocab=%d must be positive", R, V);
     PTA_REQUIRE(out_tok && work && logits, "sample: null pointer");
     PTA_REQUIRE(!do_sample || temperature > 0.f, "sample: temperature must be > 0, got %g", (double)temperature);
@@ -525,7 +718,7 @@ extern "C" int pta_sample(int* out_tok, float* work, const float* logits, int R,
     PTA_REQUIRE(n_eos == 0 || eos, "sample: eos ids missing");
     hipLaunchKernelGGL(sample_kernel, dim3(R), dim3(S_THREADS), 0, (hipStream_t)stream, out_tok, work, logits, V,
                        do_sample, temperature, top_k, top_p, min_p, penalty, hist, hist_off, eos, n_eos, suppress,
-                       remove_invalid, renorm, seed, rng_seq, rng_step, uniforms);
+                       remove_invalid, renorm, seed, rng_seq, rng_step, uniforms, want_scores);
     return pta_check_launch("sample");
 }
 

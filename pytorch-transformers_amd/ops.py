@@ -389,8 +389,8 @@ def sample(logits: torch.Tensor, *, do_sample: bool, temperature: float = 1.0, t
           int(top_k), ctypes.c_float(top_p), ctypes.c_float(min_p), ctypes.c_float(penalty), _ptr(hist), _ptr(hist_off),
           _ptr(eos), 0 if eos is None else int(eos.numel()), _ptr(suppress), int(bool(remove_invalid)),
           int(bool(renorm)), ctypes.c_uint64(int(seed) & (2 ** 64 - 1)), _ptr(rng_seq), _ptr(rng_step), _ptr(uniforms),
-          _stream())
-    return out, work
+          int(bool(need_scores)), _stream())
+    return out, (work if need_scores else None)
 
 
 SKINNY_MAX_ROWS = 64

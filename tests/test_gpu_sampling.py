@@ -125,6 +125,44 @@ def test_draw_inverts_the_cumulative_distribution():
         assert lo - 1e-5 <= float(u[r]) <= float(cdf[t]) + 1e-5, (r, t, float(u[r]), lo, float(cdf[t]))
 
 
+def test_top_k_by_the_short_way_and_the_long_way():
+    """A draw with top-k runs on a short list of candidates, or over the whole row where the list would be long
+    (a large k, many equal scores at the threshold): both keep what the plain processors keep, tied scores
+    included, and draw the token whose interval of the survivors' cumulative distribution holds the number."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(7)
+    V, R = 65024, 6
+    logits = torch.randn(R, V, generator=g) * 3
+    logits[1, 100:900] = 50.0        # 800 equal scores at the top: more candidates than the short list holds
+    logits[2, 5000:5040] = 40.0      # 40 equal scores that straddle the k-th place
+    logits[3, :] = 0.25              # everything equal
+    logits[4, :] = -30.0             # ten equal scores at the top-p cut: the first four in index order go
+    logits[4, 7] = math.log(0.5)
+    logits[4, 100:110] = math.log(0.05)
+    u = torch.rand(R, generator=g)
+    for kw in (dict(top_k=50), dict(top_k=50, top_p=0.7, temperature=0.6), dict(top_k=300, top_p=0.9), dict(top_k=7, min_p=0.1),
+               dict(top_k=256, temperature=1.5), dict(top_k=1), dict(top_k=20, top_p=0.78), dict(top_k=300, top_p=0.78)):
+        tok, scores = ops.sample(_dev(logits), do_sample=True, temperature=kw.get("temperature", 1.0), top_k=kw["top_k"],
+                                 top_p=kw.get("top_p", 1.0), min_p=kw.get("min_p", 0.0), uniforms=_dev(u))
+        tok2, none = ops.sample(_dev(logits), do_sample=True, temperature=kw.get("temperature", 1.0), top_k=kw["top_k"],
+                                top_p=kw.get("top_p", 1.0), min_p=kw.get("min_p", 0.0), uniforms=_dev(u), need_scores=False)
+        assert none is None and tok2.tolist() == tok.tolist(), "the choice does not depend on whether the scores are wanted"
+        for r in range(R):
+            want = P.process(logits[r], [], do_sample=True, temperature_=kw.get("temperature", 1.0), top_k_=kw["top_k"],
+                             top_p_=kw.get("top_p", 1.0), min_p_=kw.get("min_p"), repetition_penalty_=1.0, suppress_ids=())
+            got = scores[r].cpu()
+            keep_want, keep_got = want != float("-inf"), _finite_mask(got)
+            diff = (keep_want != keep_got).nonzero().flatten().tolist()
+            assert len(diff) <= (1 if "top_p" in kw and r != 4 else 0), f"{kw} row {r}: kept sets differ at {diff[:10]}"
+            if r == 4 and kw.get("top_p") == 0.78:
+                assert keep_got.nonzero().flatten().tolist() == [7, 104, 105, 106, 107, 108, 109]
+            assert int(keep_got.sum()) >= min(kw["top_k"], 1)
+            cdf = torch.softmax(got.double(), -1).cumsum(-1)
+            t = int(tok[r])
+            lo = float(cdf[t - 1]) if t else 0.0
+            assert keep_got[t] and lo - 1e-5 <= float(u[r]) <= float(cdf[t]) + 1e-5, (kw, r, t, float(u[r]), lo, float(cdf[t]))
+
+
 def test_counter_based_uniforms():
     """Same (seed, sequence, step) -> same draw whatever the batch; the host function gives the number."""
     from pytorch_transformers_amd.sampling import philox_uniform
