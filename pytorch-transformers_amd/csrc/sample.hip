@@ -255,6 +255,66 @@ __device__ __forceinline__ float key_value(uint32_t k) {
     return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
 }
 
+// The processed score of a token before the thresholds: repetition penalty (tokens seen before are marked in
+// a bitmap in LDS, so vocabularies up to 65,536), EOS suppression, invalid values, temperature, in this order.
+struct Processed {
+    const float* l;
+    const uint32_t* seen;  // null: no penalty
+    const int* eos;
+    int n_eos;  // 0: no suppression
+    float penalty, temperature;
+    int remove_invalid;
+    __device__ __forceinline__ float operator()(int i) const { return of(i, l[i]); }
+    __device__ __forceinline__ float of(int i, float x) const {
+        if (seen && ((seen[i >> 5] >> (i & 31)) & 1u)) x = x < 0.f ? x * penalty : x / penalty;
+        for (int e = 0; e < n_eos; ++e)
+            if (eos[e] == i) x = -INFINITY;
+        if (remove_invalid) {
+            if (x != x) x = 0.f;
+            else if (x == INFINITY) x = FLT_MAX;
+            else if (x == -INFINITY) x = -FLT_MAX;
+        }
+        if (temperature != 1.0f) x = x / temperature;
+        return x;
+    }
+};
+
+// marks the tokens of the row's history in sh.seen; returns the bitmap, or null if there is no penalty
+__device__ __forceinline__ const uint32_t* mark_seen(SampleShared& sh, int row, int V, float penalty,
+                                                     const int* __restrict__ hist, const int* __restrict__ hist_off) {
+    if (!(hist_off && penalty != 1.0f)) return nullptr;
+    const int tid = threadIdx.x;
+    for (int w = tid; w < 2048; w += S_THREADS) sh.seen[w] = 0u;
+    __syncthreads();
+    for (int t = hist_off[row] + tid; t < hist_off[row + 1]; t += S_THREADS) {
+        const int tok = hist[t];
+        if (tok >= 0 && tok < V) atomicOr(&sh.seen[tok >> 5], 1u << (tok & 31));
+    }
+    __syncthreads();
+    return sh.seen;
+}
+
+// f(i, l[i]) for every score of a row, each thread in ascending order of i.  Sixteen bytes a load and four
+// loads in flight per thread: one load at a time leaves a pass waiting for memory most of its time.
+template <typename F>
+__device__ __forceinline__ void for_each_score(const float* __restrict__ l, int V, F&& f) {
+    const int tid = threadIdx.x;
+    if ((((uintptr_t)l) & 15) != 0) {
+        for (int i = tid; i < V; i += S_THREADS) f(i, l[i]);
+        return;
+    }
+    const float4* l4 = reinterpret_cast<const float4*>(l);
+    const int quads = V >> 2;
+    auto four = [&](int q, const float4& a) { f(4 * q, a.x); f(4 * q + 1, a.y); f(4 * q + 2, a.z); f(4 * q + 3, a.w); };
+    int q = tid;
+    for (; q + 3 * S_THREADS < quads; q += 4 * S_THREADS) {
+        const float4 a = l4[q], b = l4[q + S_THREADS], c = l4[q + 2 * S_THREADS], d = l4[q + 3 * S_THREADS];
+        four(q, a); four(q + S_THREADS, b); four(q + 2 * S_THREADS, c); four(q + 3 * S_THREADS, d);
+    }
+    for (; q < quads; q += S_THREADS) four(q, l4[q]);
+    for (int i = quads * 4 + tid; i < V; i += S_THREADS) f(i, l[i]);
+}
+
 // The short way for a draw with top-k, up to 65,536 scores: two passes over the row (one for the threads'
 // maxima, one that lists the scores at or above the bound they give), then everything on that list: the
 // k-th largest, the survivors in index order, the top-p cut by integer masses, min-p, the draw.  The row is
@@ -263,55 +323,30 @@ __device__ __forceinline__ float key_value(uint32_t k) {
 // other terms are zero), but never depend on the batch.  Returns false, having written nothing, if the list
 // would have more than S_SHORT entries (many equal scores, or a large k): then the long way runs.
 __device__ __forceinline__ bool sample_short(
-    SampleShared& sh, int* __restrict__ out_tok, float* __restrict__ work, const float* __restrict__ l, int row, int V,
-    float temperature, int top_k, float top_p, float min_p, float penalty, const int* __restrict__ hist,
-    const int* __restrict__ hist_off, const int* __restrict__ eos, int n_eos, bool suppress_eos, int remove_invalid,
-    int renorm, float u) {
+    SampleShared& sh, int* __restrict__ out_tok, float* __restrict__ work, const Processed& score, int row, int V,
+    int top_k, float top_p, float min_p, int renorm, float u) {
     const int tid = threadIdx.x;
-    const bool penalize = hist_off && penalty != 1.0f;
-    if (penalize) {
-        for (int w = tid; w < 2048; w += S_THREADS) sh.seen[w] = 0u;
-        __syncthreads();
-        for (int t = hist_off[row] + tid; t < hist_off[row + 1]; t += S_THREADS) {
-            const int tok = hist[t];
-            if (tok >= 0 && tok < V) atomicOr(&sh.seen[tok >> 5], 1u << (tok & 31));
-        }
-        __syncthreads();
-    }
-    // the processed score of token i, with the operations of the long way in their order
-    auto score = [&](int i) {
-        float x = l[i];
-        if (penalize && ((sh.seen[i >> 5] >> (i & 31)) & 1u)) x = x < 0.f ? x * penalty : x / penalty;
-        if (suppress_eos)
-            for (int e = 0; e < n_eos; ++e)
-                if (eos[e] == i) x = -INFINITY;
-        if (remove_invalid) {
-            if (x != x) x = 0.f;
-            else if (x == INFINITY) x = FLT_MAX;
-            else if (x == -INFINITY) x = -FLT_MAX;
-        }
-        if (temperature != 1.0f) x = x / temperature;
-        return x;
-    };
     float m = -INFINITY, mx = -INFINITY;
     int mi = 0x7fffffff;
-    for (int i = tid; i < V; i += S_THREADS) {
-        const float x = score(i);
+    bool any = false;
+    for_each_score(score.l, V, [&](int i, float raw) {
+        const float x = score.of(i, raw);
         m = fmaxf(m, x);
         if (x > mx) { mx = x; mi = i; }
-    }
-    sh.tkey[tid] = tid < V ? order_key(m) : 0u;
+        any = true;
+    });
+    sh.tkey[tid] = any ? order_key(m) : 0u;
     const ArgBest best = block_argmax(mx, mi, sh.red, sh.red_i);
     const uint32_t bound = list_kth_largest(sh, sh.tkey, S_THREADS, (uint32_t)top_k);
     if (tid == 0) sh.n_cand = 0u;
     __syncthreads();
-    for (int i = tid; i < V; i += S_THREADS) {
-        const uint32_t k = order_key(score(i));
+    for_each_score(score.l, V, [&](int i, float raw) {
+        const uint32_t k = order_key(score.of(i, raw));
         if (k >= bound) {
             const uint32_t at = atomicAdd(&sh.n_cand, 1u);
             if (at < S_SHORT) { sh.cand_key[at] = k; sh.cand_idx[at] = (uint32_t)i; }
         }
-    }
+    });
     __syncthreads();
     const int n = (int)sh.n_cand;
     if (n > S_SHORT) return false;
@@ -397,8 +432,9 @@ __device__ __forceinline__ bool sample_short(
         __syncthreads();
         const float lse = renorm ? best.v + logf(total) : 0.f;
         float* w = work + (long)row * V;
-        for (int i = tid; i < V; i += S_THREADS)
-            w[i] = ((sh.left[i >> 5] >> (i & 31)) & 1u) ? score(i) - lse : -INFINITY;
+        for_each_score(score.l, V, [&](int i, float raw) {
+            w[i] = ((sh.left[i >> 5] >> (i & 31)) & 1u) ? score.of(i, raw) - lse : -INFINITY;
+        });
     }
     return true;
 }
@@ -424,46 +460,68 @@ __global__ __launch_bounds__(S_THREADS) void sample_kernel(
     float* w = work + (long)row * V;
     const float* l = logits + (long)row * V;
 
-    if (do_sample && top_k > 0 && top_k < V && top_k <= n_holding && top_k <= S_SHORT && V <= 65536) {
-        const float u = uniforms ? uniforms[row] : uniform_of(seed, (uint32_t)rng_seq[row], (uint32_t)rng_step[row]);
-        if (sample_short(sh, out_tok, want_scores ? work : nullptr, l, row, V, temperature, top_k, top_p, min_p, penalty,
-                         hist, hist_off, eos, n_eos, suppress && suppress[row], remove_invalid, renorm, u))
-            return;
+    const bool suppress_eos = suppress && suppress[row];
+    ArgBest first_best = {-INFINITY, 0x7fffffff};
+    unsigned long long first_finite = 0ull;
+    float first_max = -INFINITY;  // the largest of the scores this thread saw in the first pass
+    bool have_first = false;
+    if (V <= 65536) {
+        const Processed score{l, mark_seen(sh, row, V, penalty, hist, hist_off), eos, suppress_eos ? n_eos : 0, penalty,
+                              do_sample ? temperature : 1.0f, remove_invalid};
+        if (do_sample && top_k > 0 && top_k < V && top_k <= n_holding && top_k <= S_SHORT) {
+            const float u = uniforms ? uniforms[row] : uniform_of(seed, (uint32_t)rng_seq[row], (uint32_t)rng_step[row]);
+            if (sample_short(sh, out_tok, want_scores ? work : nullptr, score, row, V, top_k, top_p, min_p, renorm, u)) return;
+            __syncthreads();
+        }
+        // every processor before the thresholds in one pass, which also finds the largest score (no threshold
+        // ever removes it) and counts the scores that are not gone
+        float mx = -INFINITY;
+        int mi = 0x7fffffff;
+        for_each_score(l, V, [&](int i, float raw) {
+            const float x = score.of(i, raw);
+            w[i] = x;
+            if (x > mx) { mx = x; mi = i; }
+            first_finite += x != -INFINITY ? 1ull : 0ull;
+        });
+        first_best = block_argmax(mx, mi, red, red_i);
+        first_max = mx;
+        have_first = true;
         __syncthreads();
-    }
-    for (int i = tid; i < V; i += S_THREADS) w[i] = l[i];
-    __syncthreads();
-    if (hist_off && penalty != 1.0f) {
-        for (int t = hist_off[row] + tid; t < hist_off[row + 1]; t += S_THREADS) {
-            const int tok = hist[t];
-            if (tok >= 0 && tok < V) {
-                const float v = l[tok];
-                w[tok] = v < 0.f ? v * penalty : v / penalty;
+    } else {
+        for (int i = tid; i < V; i += S_THREADS) w[i] = l[i];
+        __syncthreads();
+        if (hist_off && penalty != 1.0f) {
+            for (int t = hist_off[row] + tid; t < hist_off[row + 1]; t += S_THREADS) {
+                const int tok = hist[t];
+                if (tok >= 0 && tok < V) {
+                    const float v = l[tok];
+                    w[tok] = v < 0.f ? v * penalty : v / penalty;
+                }
             }
+            __syncthreads();
         }
-        __syncthreads();
-    }
-    if (suppress && suppress[row]) {
-        for (int e = tid; e < n_eos; e += S_THREADS)
-            if (eos[e] >= 0 && eos[e] < V) w[eos[e]] = -INFINITY;
-        __syncthreads();
-    }
-    if (remove_invalid) {
-        for (int i = tid; i < V; i += S_THREADS) {
-            float v = w[i];
-            if (v != v) v = 0.f;
-            else if (v == INFINITY) v = FLT_MAX;
-            else if (v == -INFINITY) v = -FLT_MAX;
-            w[i] = v;
+        if (suppress_eos) {
+            for (int e = tid; e < n_eos; e += S_THREADS)
+                if (eos[e] >= 0 && eos[e] < V) w[eos[e]] = -INFINITY;
+            __syncthreads();
         }
-        __syncthreads();
-    }
-
-    if (do_sample) {
-        if (temperature != 1.0f) {
+        if (remove_invalid) {
+            for (int i = tid; i < V; i += S_THREADS) {
+                float v = w[i];
+                if (v != v) v = 0.f;
+                else if (v == INFINITY) v = FLT_MAX;
+                else if (v == -INFINITY) v = -FLT_MAX;
+                w[i] = v;
+            }
+            __syncthreads();
+        }
+        if (do_sample && temperature != 1.0f) {
             for (int i = tid; i < V; i += S_THREADS) w[i] = w[i] / temperature;
             __syncthreads();
         }
+    }
+
+    if (do_sample) {
         if (top_k > 0 && top_k < V) {
             uint32_t prefix = 0, maskbits = 0;
             bool found = false;
@@ -520,13 +578,17 @@ __global__ __launch_bounds__(S_THREADS) void sample_kernel(
         if (top_p < 1.0f) {
             float mx = -INFINITY;
             int mi = 0x7fffffff;
-            unsigned long long finite = 0ull;
-            for (int i = tid; i < V; i += S_THREADS) {
-                const float x = w[i];
-                if (x > mx) { mx = x; mi = i; }
-                finite += x != -INFINITY ? 1ull : 0ull;
+            unsigned long long finite = first_finite;
+            const bool counted = have_first && !(top_k > 0 && top_k < V);  // nothing has gone since the first pass
+            if (!counted) {
+                finite = 0ull;
+                for (int i = tid; i < V; i += S_THREADS) {
+                    const float x = w[i];
+                    if (x > mx) { mx = x; mi = i; }
+                    finite += x != -INFINITY ? 1ull : 0ull;
+                }
             }
-            const ArgBest best = block_argmax(mx, mi, red, red_i);
+            const ArgBest best = have_first ? first_best : block_argmax(mx, mi, red, red_i);
             float s = 0.f;
             for (int i = tid; i < V; i += S_THREADS) s += expf(w[i] - best.v);
             const float Z = block_sum(s, red);
@@ -536,7 +598,8 @@ __global__ __launch_bounds__(S_THREADS) void sample_kernel(
             const unsigned long long n_finite = block_sum_u64(finite, sh.red_q);
             uint32_t from = order_key(-INFINITY) + 1u;
             if (n_finite > S_CAP) {
-                sh.tkey[tid] = tid < V ? order_key(mx) : 0u;
+                // (a thread that saw no score has the key of minus infinity, which is below every candidate)
+                sh.tkey[tid] = order_key(counted ? first_max : mx);
                 from = list_kth_largest(sh, sh.tkey, S_THREADS, (uint32_t)min(512, n_holding));
             }
             __syncthreads();
@@ -640,9 +703,10 @@ __global__ __launch_bounds__(S_THREADS) void sample_kernel(
     // choose
     float mx = -INFINITY;
     int mi = 0x7fffffff;
-    for (int i = tid; i < V; i += S_THREADS)
-        if (w[i] > mx) { mx = w[i]; mi = i; }
-    const ArgBest best = block_argmax(mx, mi, red, red_i);
+    if (!have_first)
+        for (int i = tid; i < V; i += S_THREADS)
+            if (w[i] > mx) { mx = w[i]; mi = i; }
+    const ArgBest best = have_first ? first_best : block_argmax(mx, mi, red, red_i);
     int chosen = best.i;
     float Z = 0.f;
     if (do_sample || renorm) {
@@ -652,7 +716,23 @@ __global__ __launch_bounds__(S_THREADS) void sample_kernel(
         const int span = ((V + n_waves - 1) / n_waves + 63) & ~63;
         const int lo = min(V, wave * span), hi = min(V, lo + span);
         float s = 0.f;
-        for (int i = lo + lane; i < hi; i += 64) s += expf(w[i] - best.v);
+        if ((((uintptr_t)(w + lo)) & 15) == 0) {
+            // sixteen bytes a load, four loads in flight per lane
+            const float4* w4 = reinterpret_cast<const float4*>(w + lo);
+            const int quads = (hi - lo) >> 2;
+            auto add4 = [&](const float4& a) {
+                s += expf(a.x - best.v); s += expf(a.y - best.v); s += expf(a.z - best.v); s += expf(a.w - best.v);
+            };
+            int q = lane;
+            for (; q + 192 < quads; q += 256) {
+                const float4 a = w4[q], b = w4[q + 64], c = w4[q + 128], d = w4[q + 192];
+                add4(a); add4(b); add4(c); add4(d);
+            }
+            for (; q < quads; q += 64) add4(w4[q]);
+            for (int i = lo + quads * 4 + lane; i < hi; i += 64) s += expf(w[i] - best.v);
+        } else {
+            for (int i = lo + lane; i < hi; i += 64) s += expf(w[i] - best.v);
+        }
         s = wave_sum(s);
         __syncthreads();
         if (lane == 0) sh.seg[wave] = s;
@@ -676,20 +756,26 @@ __global__ __launch_bounds__(S_THREADS) void sample_kernel(
             if (wave == pick) {
                 float before = 0.f;
                 int tok = -1, last = lo;
-                for (int i0 = lo; i0 < hi && tok < 0; i0 += 64) {
-                    const int i = i0 + lane;
-                    const float e = i < hi ? expf(w[i] - best.v) : 0.f;
-                    float incl = e;
+                for (int i0 = lo; i0 < hi && tok < 0; i0 += 256) {
+                    float x[4];  // four times 64 scores are loaded before the first of them is used
 #pragma unroll
-                    for (int o = 1; o < 64; o <<= 1) {
-                        const float up = __shfl_up(incl, o, 64);
-                        if (lane >= o) incl += up;
+                    for (int k = 0; k < 4; ++k) x[k] = i0 + 64 * k + lane < hi ? w[i0 + 64 * k + lane] : -INFINITY;
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        if (tok >= 0) break;
+                        const float e = expf(x[k] - best.v);
+                        float incl = e;
+#pragma unroll
+                        for (int o = 1; o < 64; o <<= 1) {
+                            const float up = __shfl_up(incl, o, 64);
+                            if (lane >= o) incl += up;
+                        }
+                        const unsigned long long has_mass = __ballot(e > 0.f);
+                        const unsigned long long passed = __ballot(before + incl > left);
+                        if (has_mass) last = i0 + 64 * k + 63 - __clzll(has_mass);
+                        if (passed) tok = i0 + 64 * k + __ffsll((long long)passed) - 1;
+                        before += __shfl(incl, 63, 64);
                     }
-                    const unsigned long long has_mass = __ballot(e > 0.f);
-                    const unsigned long long passed = __ballot(before + incl > left);
-                    if (has_mass) last = i0 + 63 - __clzll(has_mass);
-                    if (passed) tok = i0 + __ffsll((long long)passed) - 1;
-                    before += __shfl(incl, 63, 64);
                 }
                 if (lane == 0) out_tok[row] = tok >= 0 ? tok : last;
             }
