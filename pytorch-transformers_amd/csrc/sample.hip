@@ -89,14 +89,19 @@ __global__ __launch_bounds__(S_THREADS) void argmax_kernel(int* __restrict__ out
     const int first = min(head, V), quads = (V - first) / 4;
     if (tid < first && l[tid] > mx) { mx = l[tid]; mi = tid; }
     const float4* l4 = reinterpret_cast<const float4*>(l + first);
-    for (int q = tid; q < quads; q += S_THREADS) {
-        const float4 v = l4[q];
+    auto four = [&](int q, const float4& v) {
         const int i = first + q * 4;
         if (v.x > mx) { mx = v.x; mi = i; }
         if (v.y > mx) { mx = v.y; mi = i + 1; }
         if (v.z > mx) { mx = v.z; mi = i + 2; }
         if (v.w > mx) { mx = v.w; mi = i + 3; }
+    };
+    int q = tid;
+    for (; q + 3 * S_THREADS < quads; q += 4 * S_THREADS) {  // four loads in flight
+        const float4 a = l4[q], b = l4[q + S_THREADS], c = l4[q + 2 * S_THREADS], d = l4[q + 3 * S_THREADS];
+        four(q, a); four(q + S_THREADS, b); four(q + 2 * S_THREADS, c); four(q + 3 * S_THREADS, d);
     }
+    for (; q < quads; q += S_THREADS) four(q, l4[q]);
     for (int i = first + quads * 4 + tid; i < V; i += S_THREADS)
         if (l[i] > mx) { mx = l[i]; mi = i; }
     // a thread meets its candidates in index order and keeps the first of equals; so does the reduction
