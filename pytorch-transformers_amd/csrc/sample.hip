@@ -26,8 +26,9 @@
 
 #define S_THREADS 1024
 
+// a key that orders like the score; the two zeros are one score and get one key
 __device__ __forceinline__ uint32_t order_key(float f) {
-    const uint32_t u = __float_as_uint(f);
+    const uint32_t u = f == 0.f ? 0u : __float_as_uint(f);
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 

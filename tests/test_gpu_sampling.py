@@ -163,6 +163,50 @@ def test_top_k_by_the_short_way_and_the_long_way():
             assert keep_got[t] and lo - 1e-5 <= float(u[r]) <= float(cdf[t]) + 1e-5, (kw, r, t, float(u[r]), lo, float(cdf[t]))
 
 
+@pytest.mark.parametrize("V", [1, 2, 63, 65, 1000, 4100, 65536, 70001])
+def test_random_settings_match_plain(V):
+    """Random processor settings over vocabularies around the kernel's edges (one score, partly filled tiles,
+    the longest row of the short way, a row too long for it): the survivors are the plain code's and the
+    chosen token is the one whose interval of their cumulative distribution holds the uniform number."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(1000 + V)
+    R = 4
+    for trial in range(6):
+        logits = torch.randn(R, V, generator=g) * float(torch.rand((), generator=g) * 4 + 0.5)
+        if trial % 3 == 2 and V > 4:  # groups of equal scores
+            logits = (logits * 2).round() / 2
+        rnd = lambda: float(torch.rand((), generator=g))
+        kw = dict(temperature=0.5 + rnd() * 1.5 if rnd() < 0.7 else 1.0,
+                  top_k=int(rnd() * min(V, 300)) if rnd() < 0.7 else 0,
+                  top_p=0.3 + 0.69 * rnd() if rnd() < 0.6 else 1.0,
+                  min_p=0.2 * rnd() if rnd() < 0.3 else 0.0,
+                  penalty=0.5 + rnd() * 1.5 if rnd() < 0.5 else 1.0)
+        hist = [[int(t) for t in torch.randint(0, V, (n,), generator=g)] for n in (0, 5, 40, 300)]
+        off = [0]
+        for h in hist:
+            off.append(off[-1] + len(h))
+        flat = [t for h in hist for t in h]
+        u = torch.rand(R, generator=g)
+        tok, scores = ops.sample(_dev(logits), do_sample=True, temperature=kw["temperature"], top_k=kw["top_k"], top_p=kw["top_p"],
+                                 min_p=kw["min_p"], penalty=kw["penalty"], hist=_dev(flat, torch.int32),
+                                 hist_off=_dev(off, torch.int32), uniforms=_dev(u))
+        for r in range(R):
+            want = P.process(logits[r], hist[r], do_sample=True, temperature_=kw["temperature"], top_k_=kw["top_k"],
+                             top_p_=kw["top_p"], min_p_=kw["min_p"] or None, repetition_penalty_=kw["penalty"])
+            got = scores[r].cpu()
+            keep_want, keep_got = want != float("-inf"), _finite_mask(got)
+            diff = (keep_want != keep_got).nonzero().flatten().tolist()
+            # a token whose mass sits within rounding of the top-p cut or of the min-p threshold may fall on either side
+            loose = kw["top_p"] < 1.0 or kw["min_p"] > 0.0
+            assert len(diff) <= (2 if loose else 0), f"V={V} trial {trial} {kw} row {r}: kept sets differ at {diff[:10]}"
+            both = keep_want & keep_got
+            torch.testing.assert_close(got[both], want[both], rtol=1e-6, atol=1e-6)
+            cdf = torch.softmax(got.double(), -1).cumsum(-1)
+            t = int(tok[r])
+            lo = float(cdf[t - 1]) if t else 0.0
+            assert keep_got[t] and lo - 1e-5 <= float(u[r]) <= float(cdf[t]) + 1e-5, (V, trial, kw, r, t)
+
+
 def test_counter_based_uniforms():
     """Same (seed, sequence, step) -> same draw whatever the batch; the host function gives the number."""
     from pytorch_transformers_amd.sampling import philox_uniform
