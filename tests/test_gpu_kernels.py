@@ -510,6 +510,49 @@ def test_decode_plan():
                     assert 1 <= cut[0] <= groups and cut[1] % 64 == 0 and (length + cut[1] - 1) // cut[1] <= 1024
 
 
+@pytest.mark.parametrize("nh,nkv,d", [(71, 1, 64), (32, 8, 128), (128, 8, 64)])
+@pytest.mark.parametrize("n,lengths", [(8, "equal"), (64, "equal"), (16, "unequal"), (33, "unequal")])
+def test_decode_attention_as_planned(nh, nkv, d, n, lengths):
+    """A decode step's attention the way the engine cuts it at the published models' head shapes (groups of
+    heads per wave, keys per wave, with and without partial sums), against the 32-bit-arithmetic kernel."""
+    from types import SimpleNamespace
+
+    from pytorch_transformers_amd.engine.model import _len_bound, mean_len_bound
+
+    ops = _ops()
+    g = torch.Generator().manual_seed(n * 1000 + nh)
+    lens = [1100] * n if lengths == "equal" else [int(x) for x in torch.randint(100, 4400, (n,), generator=g)]
+    pages = [(L + 63) // 64 for L in lens]
+    width = max(pages)
+    k_pool = torch.randn(sum(pages), nkv, 64, d, generator=g).bfloat16().cuda()
+    v_pool = torch.randn(sum(pages), nkv, d, 64, generator=g).bfloat16().cuda()
+    bt = torch.zeros(n, width, dtype=torch.int32)
+    at = 0
+    for i, p in enumerate(pages):
+        bt[i, :p] = torch.arange(at, at + p, dtype=torch.int32)
+        at += p
+    q = torch.randn(n, nh, d, generator=g).bfloat16().cuda()
+    q[0] = 0
+    q[0, :, 0] = 6.0 * math.sqrt(d)          # sequence 0 looks at one far key only
+    k_pool[int(bt[0, 0]), :, 5] = 0
+    k_pool[int(bt[0, 0]), :, 5, 0] = 6.0
+    starts = [L - 1 for L in lens]
+    ctx = SimpleNamespace(is_decode=True, n_seqs=n, max_len=max(lens), new_tokens=[1] * n,
+                          mean_len=mean_len_bound(sum(lens), n, _len_bound(max(lens))),
+                          cu_tokens=torch.arange(n + 1, dtype=torch.int32).cuda(),
+                          seq_start=torch.tensor(starts, dtype=torch.int32).cuda(),
+                          token_seq=torch.arange(n, dtype=torch.int32).cuda(),
+                          token_pos=torch.tensor(starts, dtype=torch.int32).cuda())
+    scale = 1.0 / math.sqrt(d)
+    got = ops.attention(q, k_pool, v_pool, bt.cuda(), ctx, None, scale).float()
+    want = ops.attn_generic(q, k_pool, v_pool, bt.cuda(), ctx.token_seq, ctx.token_pos, None, scale).float()
+    assert float((got - want).abs().max()) <= 2e-2 * max(1.0, float(want.abs().max()))
+    far = v_pool[int(bt[0, 0]), :, :, 5].float().repeat_interleave(nh // nkv, 0).reshape(-1)
+    assert float((got[0] - far).abs().max()) < 0.05, "the far key does not dominate"
+    tiles, size = ops.decode_plan(n, nh, nkv, d, ctx.max_len, ctx.mean_len)
+    assert 1 <= tiles <= (nh // nkv + 15) // 16 and size % 64 == 0
+
+
 @pytest.mark.parametrize("window", [1, 33, 64, 100, 200])
 def test_attention_with_a_window(window):
     """Each token sees its last `window` positions only; pages behind the window hold NaN and are not read.
