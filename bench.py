@@ -25,7 +25,7 @@ PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}  # dense MFMA, published
 def falcon7b_config(layers):
     from pytorch_transformers_amd import FalconConfig
 
-    # configs[2] of BASELINE.json: Falcon-7B layer sizes
+    # the layer sizes of the published Falcon-7B configuration
     return FalconConfig(vocab_size=65024, hidden_size=4544, num_hidden_layers=layers, num_attention_heads=71,
                         multi_query=True, new_decoder_architecture=False, parallel_attn=True, bias=False, alibi=False,
                         ffn_hidden_size=18176, rope_theta=10000.0, layer_norm_epsilon=1e-5,
