@@ -128,33 +128,35 @@ extern "C" int pta_layernorm(void* out1, void* out2, const void* x, const int* r
     return pta_check_launch("layernorm");
 }
 
-// In place on y [M, N]: y = act(round(y + bias)) + add1 + add2, the part of a linear layer
+// In place on y [M, N] (rows ld apart): y = act(round(y + bias)) + add1 + add2, the part of a linear layer
 // that follows a library matrix product.  The reference adds the bias as an op of its own, so
 // the sum is rounded to the storage type before the activation
 // (src/transformers/models/falcon/modeling_falcon.py:67-72).
 template <typename T>
 __global__ void epilogue_kernel(T* __restrict__ y, const float* __restrict__ bias, const T* __restrict__ add1,
-                                const T* __restrict__ add2, long total, int N, int act) {
+                                const T* __restrict__ add2, long total, int N, long ld, int act) {
     const long stride = (long)gridDim.x * blockDim.x;
     for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-        float v = Io<T>::ld(y + i);
+        T* at = y + (i / N) * ld + i % N;
+        float v = Io<T>::ld(at);
         if (bias) v = Io<T>::round(v + bias[i % N]);
         if (act == PTA_ACT_GELU) v = gelu_erf(v);
         if (add1) v += Io<T>::ld(add1 + i);
         if (add2) v += Io<T>::ld(add2 + i);
-        Io<T>::st(y + i, v);
+        Io<T>::st(at, v);
     }
 }
 
 // The same on bfloat16 rows whose length is a multiple of 8: sixteen bytes per thread and access.
 __global__ void epilogue_bf16x8_kernel(bf16_t* __restrict__ y, const float* __restrict__ bias,
                                        const bf16_t* __restrict__ add1, const bf16_t* __restrict__ add2, long groups,
-                                       int N, int act) {
+                                       int N, long ld, int act) {
     const long stride = (long)gridDim.x * blockDim.x;
     for (long gi = (long)blockIdx.x * blockDim.x + threadIdx.x; gi < groups; gi += stride) {
         const long i = gi * 8;
         const int n = (int)(i % N);
-        uint4 yv = *reinterpret_cast<const uint4*>(y + i);
+        bf16_t* at = y + (i / N) * ld + n;
+        uint4 yv = *reinterpret_cast<const uint4*>(at);
         uint4 a1 = add1 ? *reinterpret_cast<const uint4*>(add1 + i) : make_uint4(0u, 0u, 0u, 0u);
         uint4 a2 = add2 ? *reinterpret_cast<const uint4*>(add2 + i) : make_uint4(0u, 0u, 0u, 0u);
         uint32_t* yw = reinterpret_cast<uint32_t*>(&yv);
@@ -174,21 +176,22 @@ __global__ void epilogue_bf16x8_kernel(bf16_t* __restrict__ y, const float* __re
             }
             yw[p] = (uint32_t)f32_to_bf16_bits(v[0]) | ((uint32_t)f32_to_bf16_bits(v[1]) << 16);
         }
-        *reinterpret_cast<uint4*>(y + i) = yv;
+        *reinterpret_cast<uint4*>(at) = yv;
     }
 }
 
-extern "C" int pta_epilogue(void* y, const float* bias, const void* add1, const void* add2, int M, int N, int act,
-                            int dtype, void* stream) {
+extern "C" int pta_epilogue(void* y, int ld_y, const float* bias, const void* add1, const void* add2, int M, int N,
+                            int act, int dtype, void* stream) {
     PTA_REQUIRE(M > 0 && N > 0, "epilogue: M=%d N=%d must be positive", M, N);
+    PTA_REQUIRE(ld_y >= N, "epilogue: rows of %d elements cannot lie %d apart", N, ld_y);
     PTA_REQUIRE(act == PTA_ACT_NONE || act == PTA_ACT_GELU, "epilogue: unknown activation %d", act);
-    if (dtype == PTA_BF16 && N % 8 == 0 && ((uintptr_t)y % 16) == 0 && ((uintptr_t)add1 % 16) == 0 &&
+    if (dtype == PTA_BF16 && N % 8 == 0 && ld_y % 8 == 0 && ((uintptr_t)y % 16) == 0 && ((uintptr_t)add1 % 16) == 0 &&
         ((uintptr_t)add2 % 16) == 0) {
         const long groups = (long)M * N / 8;
         long nb = (groups + 255) / 256;
         if (nb > 16384) nb = 16384;
         hipLaunchKernelGGL(epilogue_bf16x8_kernel, dim3((unsigned)nb), dim3(256), 0, (hipStream_t)stream, (bf16_t*)y, bias,
-                           (const bf16_t*)add1, (const bf16_t*)add2, groups, N, act);
+                           (const bf16_t*)add1, (const bf16_t*)add2, groups, N, ld_y, act);
         return pta_check_launch("epilogue");
     }
     const long total = (long)M * N;
@@ -197,10 +200,10 @@ extern "C" int pta_epilogue(void* y, const float* bias, const void* add1, const 
     hipStream_t s = (hipStream_t)stream;
     if (dtype == PTA_F32)
         hipLaunchKernelGGL(epilogue_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, s, (float*)y, bias,
-                           (const float*)add1, (const float*)add2, total, N, act);
+                           (const float*)add1, (const float*)add2, total, N, ld_y, act);
     else if (dtype == PTA_BF16)
         hipLaunchKernelGGL(epilogue_kernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, s, (bf16_t*)y, bias,
-                           (const bf16_t*)add1, (const bf16_t*)add2, total, N, act);
+                           (const bf16_t*)add1, (const bf16_t*)add2, total, N, ld_y, act);
     else
         return pta_fail("epilogue: unknown dtype %d", dtype);
     return pta_check_launch("epilogue");

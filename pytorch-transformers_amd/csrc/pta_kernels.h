@@ -41,11 +41,11 @@ int pta_layernorm_sum(void* out_x, void* out1, void* out2, const float* pa, int 
 int pta_layernorm_sum_ok(int H);
 
 // in place: y = act(round(y + bias)) + add1 + add2; bias, add1, add2 may be null
-int pta_epilogue(void* y, const float* bias, const void* add1, const void* add2, int M, int N, int act, int dtype,
-                 void* stream);
+int pta_epilogue(void* y, int ld_y, const float* bias, const void* add1, const void* add2, int M, int N, int act,
+                 int dtype, void* stream);
 
 // split fused qkv rows, add bias, rotate q and k (inv_freq null: no rotation), write q and append k, v
-int pta_qkv_rope_cache(void* q_out, const void* fused, const float* bias, const float* inv_freq, float cs_scale,
+int pta_qkv_rope_cache(void* q_out, const void* fused, int fused_ld, const float* bias, const float* inv_freq, float cs_scale,
                        const int* token_pos, const int* token_seq, const int* block_table, int bt_stride,
                        void* k_pool, void* v_pool, int M, int nh, int nkv, int d, int layout, int write_cache,
                        int dtype, void* stream);

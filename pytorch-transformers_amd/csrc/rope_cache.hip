@@ -19,7 +19,7 @@
 
 template <typename T>
 __global__ __launch_bounds__(RC_THREADS) void qkv_rope_cache_kernel(
-    T* __restrict__ q_out, const T* __restrict__ fused, const float* __restrict__ bias,
+    T* __restrict__ q_out, const T* __restrict__ fused, long fused_ld, const float* __restrict__ bias,
     const float* __restrict__ inv_freq, float cs_scale, const int* __restrict__ token_pos,
     const int* __restrict__ token_seq, const int* __restrict__ block_table, int bt_stride, T* __restrict__ k_pool,
     T* __restrict__ v_pool, int nh, int nkv, int d, int layout, int write_cache) {
@@ -39,7 +39,7 @@ __global__ __launch_bounds__(RC_THREADS) void qkv_rope_cache_kernel(
     if (write_cache) page = block_table[(long)token_seq[m] * bt_stride + pos / PTA_PAGE];
     const int in_page = pos % PTA_PAGE;
     const long qout = (long)(nh + 2 * nkv) * d;
-    const T* row = fused + (long)m * qout;
+    const T* row = fused + (long)m * fused_ld;  // rows of the fused projection may lie apart
     const int n_slots = write_cache ? nh + 2 * nkv : nh;  // queries, then keys, then values
 
     // rotated items: (slot < nh + nkv, pair i < half); plain items: every element of a slot
@@ -117,7 +117,7 @@ __global__ __launch_bounds__(RC_THREADS) void qkv_rope_cache_kernel(
     }
 }
 
-extern "C" int pta_qkv_rope_cache(void* q_out, const void* fused, const float* bias, const float* inv_freq,
+extern "C" int pta_qkv_rope_cache(void* q_out, const void* fused, int fused_ld, const float* bias, const float* inv_freq,
                                   float cs_scale, const int* token_pos, const int* token_seq,
                                   const int* block_table, int bt_stride, void* k_pool, void* v_pool, int M, int nh,
                                   int nkv, int d, int layout, int write_cache, int dtype, void* stream) {
@@ -128,19 +128,21 @@ extern "C" int pta_qkv_rope_cache(void* q_out, const void* fused, const float* b
     PTA_REQUIRE(layout != PTA_QKV_INTERLEAVED || nkv == nh, "qkv_rope_cache: the interleaved layout needs kv heads == heads");
     PTA_REQUIRE(!inv_freq || (d % 2 == 0 && d <= 256), "qkv_rope_cache: rotation needs an even head size up to 256, got %d", d);
     PTA_REQUIRE(!write_cache || (k_pool && v_pool && block_table && token_seq), "qkv_rope_cache: null cache pointer");
+    PTA_REQUIRE(fused_ld >= (long)(nh + 2 * nkv) * d, "qkv_rope_cache: fused rows of %ld elements cannot lie %d apart",
+                (long)(nh + 2 * nkv) * d, fused_ld);
     PTA_REQUIRE(dtype != PTA_BF16 || d % 16 != 0 ||
-                    (((uintptr_t)fused | (uintptr_t)q_out | (uintptr_t)k_pool) % 16) == 0,
+                    ((((uintptr_t)fused | (uintptr_t)q_out | (uintptr_t)k_pool) % 16) == 0 && fused_ld % 8 == 0),
                 "qkv_rope_cache: bfloat16 rows are moved sixteen bytes at a time and must be aligned so");
     hipStream_t s = (hipStream_t)stream;
     int slices = 1;  // enough workgroups to occupy the chip when the step has few tokens
     while (slices < 16 && M * slices < 512 && slices * RC_THREADS < (nh + 2 * nkv) * d) slices *= 2;
     if (dtype == PTA_F32)
         hipLaunchKernelGGL(qkv_rope_cache_kernel<float>, dim3(M, slices), dim3(RC_THREADS), 0, s, (float*)q_out,
-                           (const float*)fused, bias, inv_freq, cs_scale, token_pos, token_seq, block_table, bt_stride,
+                           (const float*)fused, fused_ld, bias, inv_freq, cs_scale, token_pos, token_seq, block_table, bt_stride,
                            (float*)k_pool, (float*)v_pool, nh, nkv, d, layout, write_cache);
     else if (dtype == PTA_BF16)
         hipLaunchKernelGGL(qkv_rope_cache_kernel<bf16_t>, dim3(M, slices), dim3(RC_THREADS), 0, s, (bf16_t*)q_out,
-                           (const bf16_t*)fused, bias, inv_freq, cs_scale, token_pos, token_seq, block_table,
+                           (const bf16_t*)fused, fused_ld, bias, inv_freq, cs_scale, token_pos, token_seq, block_table,
                            bt_stride, (bf16_t*)k_pool, (bf16_t*)v_pool, nh, nkv, d, layout, write_cache);
     else
         return pta_fail("qkv_rope_cache: unknown dtype %d", dtype);

@@ -194,6 +194,9 @@ class CausalLM:
         self.vocab_size = spec.head.vocab_size
         for part in spec.parts():
             part.load_all(tensors)
+        for part in spec.parts():  # layouts that a part wants for its weights once they are there
+            if hasattr(part, "after_load"):
+                part.after_load()
         self._move_constants()
         self.generation_config = None
         #: run steps in which every sequence brings one token as replays of a captured HIP graph

@@ -98,6 +98,18 @@ def _need(t: torch.Tensor, name: str, dtype=None, shape=None) -> None:
         raise KernelError(f"{name} must have shape {tuple(shape)}, got {tuple(t.shape)}")
 
 
+def _need_rows(t: torch.Tensor, name: str, dtype=None, shape=None) -> None:
+    """Like ``_need`` for a matrix whose rows may lie apart (a block of columns of a wider matrix)."""
+    if isinstance(t, torch.Tensor) and t.dim() == 2 and t.is_cuda and not t.is_contiguous() and t.stride(1) == 1 \
+            and t.stride(0) >= t.shape[1]:
+        if dtype is not None and t.dtype != dtype:
+            raise KernelError(f"{name} must be {dtype}, got {t.dtype}")
+        if shape is not None and tuple(t.shape) != tuple(shape):
+            raise KernelError(f"{name} must have shape {tuple(shape)}, got {tuple(t.shape)}")
+        return
+    _need(t, name, dtype, shape)
+
+
 def _need_pools(k_pool, v_pool, dtype, nkv: int, d: int) -> None:
     """Key pages are [pages, kv_heads, 64, d]; value pages are transposed, [pages, kv_heads, d, 64]."""
     _need(k_pool, "k_pool", dtype)
@@ -150,25 +162,24 @@ def layernorm(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float, *, 
 
 
 def epilogue_(y: torch.Tensor, bias=None, act=None, add1=None, add2=None) -> torch.Tensor:
-    """In place: y = act(round(y + bias)) + add1 + add2."""
-    _need(y, "y")
+    """In place: y = act(round(y + bias)) + add1 + add2.  The rows of y may lie apart."""
+    _need_rows(y, "y")
     M, N = y.shape
     if bias is not None:
         _need(bias, "bias", torch.float32, (N,))
     for name, a in (("add1", add1), ("add2", add2)):
         if a is not None:
             _need(a, name, y.dtype, (M, N))
-    _call("pta_epilogue", _ptr(y), _ptr(bias), _ptr(add1), _ptr(add2), M, N, ACT_CODES[act], dtype_code(y.dtype),
-          _stream())
+    _call("pta_epilogue", _ptr(y), int(y.stride(0)), _ptr(bias), _ptr(add1), _ptr(add2), M, N, ACT_CODES[act],
+          dtype_code(y.dtype), _stream())
     return y
 
 
 def qkv_rope_cache(fused: torch.Tensor, bias, inv_freq, cs_scale: float, token_pos, token_seq, block_table,
                    k_pool, v_pool, nh: int, nkv: int, d: int, layout: str, write_cache: bool = True) -> torch.Tensor:
-    """Queries [M, nh, d] from the fused rows; keys and values go to the cache pages."""
-    _need(fused, "fused")
+    """Queries [M, nh, d] from the fused rows (which may lie apart); keys and values go to the cache pages."""
     M = fused.shape[0]
-    _need(fused, "fused", None, (M, (nh + 2 * nkv) * d))
+    _need_rows(fused, "fused", None, (M, (nh + 2 * nkv) * d))
     dt = fused.dtype
     if bias is not None:
         _need(bias, "bias", torch.float32, ((nh + 2 * nkv) * d,))
@@ -181,7 +192,7 @@ def qkv_rope_cache(fused: torch.Tensor, bias, inv_freq, cs_scale: float, token_p
         raise KernelError("block_table must be [sequences, pages]")
     _need_pools(k_pool, v_pool, dt, nkv, d)
     q = torch.empty((M, nh, d), dtype=dt, device=fused.device)
-    _call("pta_qkv_rope_cache", _ptr(q), _ptr(fused), _ptr(bias), _ptr(inv_freq), ctypes.c_float(cs_scale),
+    _call("pta_qkv_rope_cache", _ptr(q), _ptr(fused), int(fused.stride(0)), _ptr(bias), _ptr(inv_freq), ctypes.c_float(cs_scale),
           _ptr(token_pos), _ptr(token_seq), _ptr(block_table), block_table.shape[1], _ptr(k_pool), _ptr(v_pool), M,
           nh, nkv, d, QKV_LAYOUT_CODES[layout], int(write_cache), dtype_code(dt), _stream())
     return q
@@ -403,19 +414,26 @@ SKINNY_MAX_ROWS = 64
 # into its rows of the result).  PTA_MM_CHUNKS=0 switches this off.
 MM_LADDER = (256, 512, 768, 1024, 1536, 2048, 3072, 4096, 6144, 8192)
 MM_CHUNKS = os.environ.get("PTA_MM_CHUNKS", "1") != "0"
+MM_JOIN = os.environ.get("PTA_MM_JOIN", "1") != "0"  # one product for two matrices of one input where it is faster
 _mm_times: dict = {}  # (N, K) -> {rows: microseconds}
 _mm_plans: dict = {}  # (N, K, M) -> [rows, ...]
+_mm_costs: dict = {}  # (N, K, M) -> microseconds of that plan, as measured piece by piece
+_mm_joined: dict = {}  # (N1, N2, K, M) -> whether one product with both matrices beats the two
 
 
 def _mm_measure(x: torch.Tensor, w: torch.Tensor, rows: int, out: torch.Tensor) -> float:
-    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    """Microseconds of ``x[:rows] @ w.T``: the fastest of five runs, each timed on its own (a mean over two runs
+    right after the library's set-up misjudged products by a tenth, enough to choose the slower plan)."""
     torch.mm(x[:rows], w.t(), out=out[:rows])  # the library's first call of a shape sets it up
-    start.record()
-    for _ in range(2):
+    best = float("inf")
+    for _ in range(5):
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
         torch.mm(x[:rows], w.t(), out=out[:rows])
-    end.record()
-    end.synchronize()
-    return start.elapsed_time(end) / 2 * 1e3
+        end.record()
+        end.synchronize()
+        best = min(best, start.elapsed_time(end) * 1e3)
+    return best
 
 
 def _mm_plan(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor):
@@ -447,7 +465,35 @@ def _mm_plan(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor):
         cost *= M / (M - rest)
     plan = pieces if not whole or (len(pieces) > 1 and cost < 0.97 * times[M]) else [M]
     _mm_plans[(N, K, bucket)] = plan
+    _mm_costs[(N, K, bucket)] = cost if plan is pieces else times[M]
     return plan
+
+
+def joined_mm_pays(x: torch.Tensor, joined: torch.Tensor, n_first: int) -> bool:
+    """Whether ``x @ joined.T`` in one library product beats the products with its first ``n_first`` rows and
+    with the rest on their own.  The library's kernel choice decides, so both ways are timed once per shape (at
+    Falcon-7B shapes, 2,048 rows: 308 us against 87 + 286; at Falcon2-11B shapes 311 against 80 + 179)."""
+    M, (N, K) = x.shape[0], joined.shape
+    if not MM_JOIN or not MM_CHUNKS or M < 512 or torch.cuda.is_current_stream_capturing():
+        return False
+    bucket = (M + 63) // 64
+    key = (n_first, N - n_first, K, bucket)
+    if key not in _mm_joined:
+        first, rest = joined[:n_first], joined[n_first:]
+        ways = (lambda: library_mm(x, joined), lambda: (library_mm(x, first), library_mm(x, rest)))
+        best = [float("inf"), float("inf")]
+        for run in ways:  # plans are made and the library set up before anything is timed
+            run()
+        for _ in range(4):  # the two ways in turn, each run timed on its own; the fastest of each counts
+            for i, run in enumerate(ways):
+                start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                start.record()
+                run()
+                end.record()
+                end.synchronize()
+                best[i] = min(best[i], start.elapsed_time(end))
+        _mm_joined[key] = best[0] < 0.98 * best[1]
+    return _mm_joined[key]
 
 
 def library_mm(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:

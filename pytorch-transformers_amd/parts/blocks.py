@@ -65,6 +65,12 @@ class ParallelBlock(Part):
     def children(self) -> Sequence[Part]:
         return tuple(p for p in (self.norm_mixer, self.norm_ffn, self.mixer, self.feed_forward) if p is not None)
 
+    def after_load(self) -> None:
+        """With one norm both branches start from the same input: their first matrices are laid out side by
+        side, so that prompts can run them as one product."""
+        if self.norm_ffn is None and hasattr(self.mixer, "input_projection") and hasattr(self.feed_forward, "input_projection"):
+            Linear.join(self.mixer.input_projection()[0], self.feed_forward.input_projection()[0])
+
     def forward(self, x, ctx: StepContext, call):
         x, a, m = _normed(x, self.norm_mixer, self.norm_ffn)
         if m is None:

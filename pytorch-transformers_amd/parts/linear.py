@@ -42,6 +42,26 @@ class Linear(Part):
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.weight = tensors[self.name + ".weight"]
         self.bias = tensors[self.name + ".bias"] if self.has_bias else None
+        self.joined = None  # (both matrices as one, the other Linear) after ``join``
+
+    @staticmethod
+    def join(first: "Linear", second: "Linear") -> bool:
+        """Lay the two weight matrices out as one, ``first``'s rows then ``second``'s, if they are bfloat16 with
+        one K: products of many rows with the same input can then run as one library product (``pair``).  The
+        matrices themselves become views of the joined one, so nothing is held twice."""
+        if first.joined is not None and first.joined[1] is second:
+            return True
+        a, b = first.weight, second.weight
+        if not (a is not None and b is not None and a.dtype == b.dtype == torch.bfloat16 and a.is_cuda
+                and a.device == b.device and a.dim() == b.dim() == 2 and a.shape[1] == b.shape[1]
+                and a.shape[0] % 8 == 0 and b.shape[0] % 8 == 0):
+            return False
+        both = torch.empty((a.shape[0] + b.shape[0], a.shape[1]), dtype=a.dtype, device=a.device)
+        both[:a.shape[0]].copy_(a)
+        both[a.shape[0]:].copy_(b)
+        first.weight, second.weight = both[:a.shape[0]], both[a.shape[0]:]
+        first.joined = (both, second)
+        return True
 
     def __call__(self, x: torch.Tensor, *, act: Optional[str] = None, add1=None, add2=None,
                  apply_bias: bool = True) -> torch.Tensor:
@@ -71,6 +91,16 @@ class Linear(Part):
         args = (x1, first.weight, x2, second.weight, b1, kw1.get("act"), b2, kw2.get("act"))
         if x1.shape == x2.shape and ops.gemm_skinny_ok(x1, first.weight) and ops.gemm_skinny_ok(x2, second.weight):
             return ops.gemm_skinny_pair_bf16(*args)
+        if (x1 is x2 and x1.shape[0] > ops.SKINNY_MAX_ROWS and first.joined is not None and first.joined[1] is second
+                and ops.joined_mm_pays(x1, first.joined[0], first.out_features)):
+            # many rows, one input, the matrices side by side in memory: one library product where it was measured
+            # faster than two; the results are blocks of columns of its output, each with its own epilogue
+            y = ops.library_mm(x1, first.joined[0])
+            y1, y2 = y[:, :first.out_features], y[:, first.out_features:]
+            for yi, bias, act in ((y1, b1, kw1.get("act")), (y2, b2, kw2.get("act"))):
+                if bias is not None or act is not None:
+                    ops.epilogue_(yi, bias, act)
+            return y1, y2
         # 17 to 64 rows: measured at Falcon-7B and Falcon2-11B sizes the pair beats the products on their own; at
         # Falcon-40B sizes it does up to 48 rows (32 rows: 20.8 against 23.0 ms a step), beyond them the vendor
         # library's product for the feed-forward input is the faster one (64 rows: 23.3 against 24.3 ms)

@@ -93,6 +93,40 @@ def test_layernorm_linear_embedding_head(dtype, rel):
         _close(out, h.double() @ r["head.weight"].T, rel, f"OutputHead, {M} rows")
 
 
+def test_joined_matrices_give_one_product_for_many_rows(monkeypatch):
+    """Two linear layers of one input whose matrices are laid out side by side: a prompt's rows can go through
+    one library product; the two results are blocks of columns of its output, each with its own epilogue, and
+    what reads them (the next product, the rotation kernel) takes rows that lie apart."""
+    from pytorch_transformers_amd import ops
+    from pytorch_transformers_amd.parts import Linear
+
+    H, N1, N2, M = 200, 72, 136, 600
+    first, second = Linear("a", H, N1, bias=True), Linear("b", H, N2, bias=False)
+    (_, r1), (_, r2) = _fill(first, torch.bfloat16, 1), _fill(second, torch.bfloat16, 2)
+    w1, w2 = first.weight.clone(), second.weight.clone()
+    assert Linear.join(first, second) and Linear.join(first, second)
+    assert torch.equal(first.weight, w1) and torch.equal(second.weight, w2)
+    assert first.weight.data_ptr() + first.weight.numel() * 2 == second.weight.data_ptr()
+    x = _rand(M, H, seed=3).bfloat16().cuda()
+    want1 = P.linear(x.double().cpu(), r1["a.weight"], r1["a.bias"])
+    want2 = P.gelu(x.double().cpu() @ r2["b.weight"].T)
+    for pays in (True, False):
+        monkeypatch.setattr(ops, "joined_mm_pays", lambda *a, **k: pays)
+        both = Linear.pair(first, x, {}, second, x, {"act": "gelu"})
+        if not pays:
+            assert both is None  # the block then runs the two on their own
+            continue
+        y1, y2 = both
+        assert y1.shape == (M, N1) and y2.shape == (M, N2) and not y2.is_contiguous()
+        _close(y1, want1, 2e-2, "first of the joined product")
+        _close(y2, want2, 2e-2, "second of the joined product, with its activation")
+        down = Linear("c", N2, 64, bias=False)
+        _, r3 = _fill(down, torch.bfloat16, 4)
+        _close(down(y2), y2.double().cpu() @ r3["c.weight"].T, 2e-2, "a product whose input rows lie apart")
+    monkeypatch.undo()
+    assert ops.joined_mm_pays(x, first.joined[0], N1) in (True, False)  # measured, either way
+
+
 def test_positions():
     from pytorch_transformers_amd.parts import AlibiPositions, NoPositions, RotaryPositions
 
