@@ -58,10 +58,6 @@ def load_library(build_if_missing: bool = True):
         return lib
 
 
-def library_path() -> Optional[str]:
-    return _build_module().find_library(require_current=True)
-
-
 def _call(name: str, *args) -> None:
     lib = load_library()
     rc = getattr(lib, name)(*args)
