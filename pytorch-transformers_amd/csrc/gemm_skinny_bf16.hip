@@ -15,6 +15,8 @@
 #include "common.h"
 #include "pta_kernels.h"
 
+#include <algorithm>
+
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
@@ -110,10 +112,12 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(SkinnyProblem pa, Skin
     const bf16_t* __restrict__ add1 = second ? pb.add1 : pa.add1;
     const bf16_t* __restrict__ add2 = second ? pb.add2 : pa.add2;
     const int N = second ? pb.N : pa.N, act = second ? pb.act : pa.act;
-    const int n0 = ((int)blockIdx.x - (second ? pa.blocks : 0)) * (16 * RT);
+    // the workgroups of a product share its rows evenly: this one has rows n0 .. n1 - 1, at most 16 * RT
+    const int blocks = second ? pb.blocks : pa.blocks, j = (int)blockIdx.x - (second ? pa.blocks : 0);
+    const int n0 = (int)((long)j * N / blocks), n1 = (int)((long)(j + 1) * N / blocks);
     const bf16_t* wrow[RT];
 #pragma unroll
-    for (int t = 0; t < RT; ++t) wrow[t] = W + (long)min(n0 + t * 16 + r, N - 1) * K;
+    for (int t = 0; t < RT; ++t) wrow[t] = W + (long)min(n0 + t * 16 + r, n1 - 1) * K;
     // x through a buffer descriptor whose bounds are the M real rows (0x00020000: 32-bit raw data format)
     __amdgpu_buffer_rsrc_t xres = __builtin_amdgcn_make_buffer_rsrc((void*)x, 0, M * K * 2, 0x00020000);
 
@@ -157,7 +161,7 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(SkinnyProblem pa, Skin
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int n = n0 + rt * 16 + (ln >> 4) * 4 + i;
-            if (n < N) {
+            if (n < n1) {
                 float v = OutIo<OutT>::round(sum[i]);
                 if (bias) v = OutIo<OutT>::round(v + bias[n]);
                 if (act == PTA_ACT_GELU) v = gelu_erf(v);
@@ -187,6 +191,20 @@ static void launch_cfg(SkinnyProblem a, SkinnyProblem b, int M, int K, int S, hi
     if (S <= 0) S = pick_split(a.N + b.N);
     a.blocks = (a.N + rows - 1) / rows;
     b.blocks = (b.N + rows - 1) / rows;
+    // A launch takes as long as the compute unit with the most workgroups: 714 workgroups on 256 units take
+    // the time of 768 (measured: 44.7 us for 22,848 rows, 45.5 us for 24,576).  So a launch with more
+    // workgroups than units gets a whole number of workgroups per unit, each with a little fewer rows.
+    const int units = pta_compute_units(), natural = a.blocks + b.blocks;
+    if (natural > units && natural % units != 0) {
+        const int total = (natural + units - 1) / units * units;
+        if (b.blocks == 0) {
+            a.blocks = total;
+        } else {
+            const int first = (int)((long)total * a.N / (a.N + b.N));
+            a.blocks = std::max(a.blocks, std::min(first, total - b.blocks));
+            b.blocks = total - a.blocks;
+        }
+    }
     const dim3 grid(a.blocks + b.blocks), block(S * 64);
     const size_t lds = (size_t)S * RT * MT * 64 * sizeof(f32x4_t);
     hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, U, OutT>), grid, block, lds, s, a, b, M, K);
