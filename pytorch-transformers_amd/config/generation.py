@@ -38,6 +38,9 @@ class GenerationConfig:
     top_k: Optional[int] = 50
     top_p: Optional[float] = 1.0
     min_p: Optional[float] = None
+    typical_p: Optional[float] = 1.0
+    epsilon_cutoff: Optional[float] = 0.0
+    eta_cutoff: Optional[float] = 0.0
     repetition_penalty: Optional[float] = 1.0
     renormalize_logits: bool = False
     remove_invalid_values: bool = False
@@ -83,7 +86,8 @@ class GenerationConfig:
                 raise ValueError(
                     "Greedy methods without beam search do not support `num_return_sequences` different than 1 "
                     f"(got {self.num_return_sequences}).")
-            for name, default in (("temperature", 1.0), ("top_p", 1.0), ("min_p", None)):
+            for name, default in (("temperature", 1.0), ("top_p", 1.0), ("min_p", None), ("typical_p", 1.0),
+                                  ("epsilon_cutoff", 0.0), ("eta_cutoff", 0.0)):
                 v = getattr(self, name)
                 if v is not None and v != default:
                     warnings.warn(
@@ -105,6 +109,8 @@ class GenerationConfig:
                 raise ValueError(f"`top_p` has to be a float > 0 and < 1, but is {self.top_p}")
             if self.min_p is not None and not (0 <= self.min_p <= 1.0):  # :568-570
                 raise ValueError(f"`min_p` has to be a float in the [0, 1] interval, but is {self.min_p}")
+            if self.typical_p is not None and self.typical_p < 1.0 and not (self.typical_p > 0):  # :651-653
+                raise ValueError(f"`typical_p` has to be a float > 0 and < 1, but is {self.typical_p}")
         rp = self.repetition_penalty
         if rp is not None and (not isinstance(rp, float) or not (rp > 0)):  # :329-331
             raise ValueError(f"`penalty` has to be a strictly positive float, but is {rp}")

@@ -447,10 +447,10 @@ __device__ __forceinline__ bool sample_short(
 
 __global__ __launch_bounds__(S_THREADS) void sample_kernel(
     int* __restrict__ out_tok, float* __restrict__ work, const float* __restrict__ logits, int V, int do_sample,
-    float temperature, int top_k, float top_p, float min_p, float penalty, const int* __restrict__ hist,
-    const int* __restrict__ hist_off, const int* __restrict__ eos, int n_eos, const int* __restrict__ suppress,
-    int remove_invalid, int renorm, uint64_t seed, const int* __restrict__ rng_seq, const int* __restrict__ rng_step,
-    const float* __restrict__ uniforms, int want_scores) {
+    float temperature, int top_k, float top_p, float min_p, float typical_p, float epsilon_cutoff, float eta_cutoff,
+    float penalty, const int* __restrict__ hist, const int* __restrict__ hist_off, const int* __restrict__ eos, int n_eos,
+    const int* __restrict__ suppress, int remove_invalid, int renorm, uint64_t seed, const int* __restrict__ rng_seq,
+    const int* __restrict__ rng_step, const float* __restrict__ uniforms, int want_scores) {
     __shared__ SampleShared sh;
     float* const red = sh.red;
     int* const red_i = sh.red_i;
@@ -474,7 +474,8 @@ __global__ __launch_bounds__(S_THREADS) void sample_kernel(
     if (V <= 65536) {
         const Processed score{l, mark_seen(sh, row, V, penalty, hist, hist_off), eos, suppress_eos ? n_eos : 0, penalty,
                               do_sample ? temperature : 1.0f, remove_invalid};
-        if (do_sample && top_k > 0 && top_k < V && top_k <= n_holding && top_k <= S_SHORT) {
+        const bool later_warpers = typical_p < 1.0f || epsilon_cutoff > 0.0f || eta_cutoff > 0.0f;  // the long way has them
+        if (do_sample && top_k > 0 && top_k < V && top_k <= n_holding && top_k <= S_SHORT && !later_warpers) {
             const float u = uniforms ? uniforms[row] : uniform_of(seed, (uint32_t)rng_seq[row], (uint32_t)rng_step[row]);
             if (sample_short(sh, out_tok, want_scores ? work : nullptr, score, row, V, top_k, top_p, min_p, renorm, u)) return;
             __syncthreads();
@@ -704,6 +705,90 @@ __global__ __launch_bounds__(S_THREADS) void sample_kernel(
                 if (w[i] != mx && expf(w[i] - mx) / Z < thr) w[i] = -INFINITY;
             __syncthreads();
         }
+        if (typical_p < 1.0f) {
+            // Locally typical sampling: the scores whose information content -log p lies nearest to the entropy
+            // stay, as many as it takes for their mass to reach typical_p.  The key of a score is its distance
+            // from the entropy (the smaller the better); the cut by mass goes over the keys one byte at a time,
+            // and equal distances at the cut all stay.  The most probable score is not safe here.
+            float mx = -INFINITY;
+            for (int i = tid; i < V; i += S_THREADS) mx = fmaxf(mx, w[i]);
+            mx = block_max(mx, red);
+            float s = 0.f;
+            for (int i = tid; i < V; i += S_THREADS) s += expf(w[i] - mx);
+            const float Z = block_sum(s, red);
+            const float logZ = logf(Z);
+            float h = 0.f;
+            for (int i = tid; i < V; i += S_THREADS)
+                if (w[i] != -INFINITY) h -= (w[i] - mx - logZ) * expf(w[i] - mx - logZ);
+            const float ent = block_sum(h, red);
+            auto typical_key = [&](float x) { return order_key(-fabsf(-(x - mx - logZ) - ent)); };
+            uint32_t kbest = 0u;
+            for (int i = tid; i < V; i += S_THREADS)
+                if (w[i] != -INFINITY) kbest = max(kbest, typical_key(w[i]));
+            __syncthreads();
+            if (tid == 0) { sh.pick = 0u; sh_cum = 0ull; sh_all = 0u; }
+            __syncthreads();
+            atomicMax(&sh.pick, kbest);
+            const unsigned long long T = (unsigned long long)((double)(1.0f - typical_p) * (double)MASS_ONE);
+            uint32_t prefix = 0, maskbits = 0;
+            for (int shift = 24; shift >= 0; shift -= 8) {
+                if (tid < 256) mass[tid] = 0ull;
+                __syncthreads();
+                for (int i = tid; i < V; i += S_THREADS) {
+                    if (w[i] == -INFINITY) continue;
+                    const uint32_t k = typical_key(w[i]);
+                    if ((k & maskbits) == prefix) {
+                        const unsigned long long q = (unsigned long long)(expf(w[i] - mx) / Z * MASS_ONE + 0.5f);
+                        if (q) atomicAdd(&mass[(k >> shift) & 255u], q);
+                    }
+                }
+                __syncthreads();
+                if (tid == 0) {
+                    unsigned long long cum = sh_cum;
+                    int b = 0;
+                    while (b < 256 && cum + mass[b] <= T) { cum += mass[b]; ++b; }
+                    if (b == 256) { sh_all = 1u; b = 255; }
+                    sh_bin = (uint32_t)b;
+                    sh_cum = cum;
+                }
+                __syncthreads();
+                if (sh_all) break;
+                prefix |= sh_bin << shift;
+                maskbits |= 255u << shift;
+            }
+            // prefix: the lowest key that stays.  If everything could go, the most typical score stays.
+            const uint32_t keep_from = sh_all ? sh.pick : prefix;
+            for (int i = tid; i < V; i += S_THREADS)
+                if (w[i] != -INFINITY && typical_key(w[i]) < keep_from) w[i] = -INFINITY;
+            have_first = false;
+            __syncthreads();
+        }
+        if (epsilon_cutoff > 0.0f || eta_cutoff > 0.0f) {
+            // probabilities below a bound go, the largest score always stays: the bound is epsilon itself, then
+            // min(eta, sqrt(eta) * exp(-entropy)) with the entropy of what epsilon left
+            for (int pass = 0; pass < 2; ++pass) {
+                const float eps = pass == 0 ? epsilon_cutoff : eta_cutoff;
+                if (!(eps > 0.0f)) continue;
+                float mx = -INFINITY;
+                for (int i = tid; i < V; i += S_THREADS) mx = fmaxf(mx, w[i]);
+                mx = block_max(mx, red);
+                float s = 0.f;
+                for (int i = tid; i < V; i += S_THREADS) s += expf(w[i] - mx);
+                const float Z = block_sum(s, red);
+                float bound = eps;
+                if (pass == 1) {
+                    const float logZ = logf(Z);
+                    float h = 0.f;
+                    for (int i = tid; i < V; i += S_THREADS)
+                        if (w[i] != -INFINITY) h -= (w[i] - mx - logZ) * (expf(w[i] - mx) / Z);
+                    const float ent = block_sum(h, red);
+                    bound = fminf(eps, sqrtf(eps) * expf(-ent));
+                }
+                for (int i = tid; i < V; i += S_THREADS)
+                    if (w[i] != mx && expf(w[i] - mx) / Z < bound) w[i] = -INFINITY;
+                __syncthreads();
+            }
+        }
     }
 
     // choose
@@ -796,7 +881,8 @@ __global__ __launch_bounds__(S_THREADS) void sample_kernel(
 }
 
 extern "C" int pta_sample(int* out_tok, float* work, const float* logits, int R, int V, int do_sample,
-                          float temperature, int top_k, float top_p, float min_p, float penalty, const int* hist,
+                          float temperature, int top_k, float top_p, float min_p, float typical_p,
+                          float epsilon_cutoff, float eta_cutoff, float penalty, const int* hist,
                           const int* hist_off, const int* eos, int n_eos, const int* suppress, int remove_invalid,
                           int renorm, uint64_t seed, const int* rng_seq, const int* rng_step, const float* uniforms,
                           int want_scores, void* stream) {
@@ -805,11 +891,16 @@ extern "C" int pta_sample(int* out_tok, float* work, const float* logits, int R,
     PTA_REQUIRE(!do_sample || temperature > 0.f, "sample: temperature must be > 0, got %g", (double)temperature);
     PTA_REQUIRE(top_p >= 0.f && top_p <= 1.f, "sample: top_p must be in [0, 1], got %g", (double)top_p);
     PTA_REQUIRE(min_p >= 0.f && min_p <= 1.f, "sample: min_p must be in [0, 1], got %g", (double)min_p);
+    PTA_REQUIRE(typical_p > 0.f && typical_p <= 1.f, "sample: typical_p must be in (0, 1] (1: off), got %g", (double)typical_p);
+    PTA_REQUIRE(epsilon_cutoff >= 0.f && epsilon_cutoff < 1.f, "sample: epsilon_cutoff must be in [0, 1) (0: off), got %g",
+                (double)epsilon_cutoff);
+    PTA_REQUIRE(eta_cutoff >= 0.f && eta_cutoff < 1.f, "sample: eta_cutoff must be in [0, 1) (0: off), got %g", (double)eta_cutoff);
     PTA_REQUIRE(penalty > 0.f, "sample: repetition penalty must be > 0, got %g", (double)penalty);
     PTA_REQUIRE(!do_sample || uniforms || (rng_seq && rng_step), "sample: sampling needs uniforms or rng counters");
     PTA_REQUIRE(n_eos == 0 || eos, "sample: eos ids missing");
     hipLaunchKernelGGL(sample_kernel, dim3(R), dim3(S_THREADS), 0, (hipStream_t)stream, out_tok, work, logits, V,
-                       do_sample, temperature, top_k, top_p, min_p, penalty, hist, hist_off, eos, n_eos, suppress,
+                       do_sample, temperature, top_k, top_p, min_p, typical_p, epsilon_cutoff, eta_cutoff, penalty, hist,
+                       hist_off, eos, n_eos, suppress,
                        remove_invalid, renorm, seed, rng_seq, rng_step, uniforms, want_scores);
     return pta_check_launch("sample");
 }

@@ -364,7 +364,8 @@ def attention(q: torch.Tensor, k_pool, v_pool, block_table, ctx, slopes, scale: 
 
 
 def sample(logits: torch.Tensor, *, do_sample: bool, temperature: float = 1.0, top_k: int = 0, top_p: float = 1.0,
-           min_p: float = 0.0, penalty: float = 1.0, hist=None, hist_off=None, eos=None, suppress=None,
+           min_p: float = 0.0, typical_p: float = 1.0, epsilon_cutoff: float = 0.0, eta_cutoff: float = 0.0,
+           penalty: float = 1.0, hist=None, hist_off=None, eos=None, suppress=None,
            remove_invalid: bool = False, renorm: bool = False, seed: int = 0, rng_seq=None, rng_step=None,
            uniforms=None, need_scores: bool = True):
     """Processors and choice for every row of ``logits`` [R, V] (32-bit); returns (tokens int32 [R], scores [R, V]).
@@ -393,7 +394,8 @@ def sample(logits: torch.Tensor, *, do_sample: bool, temperature: float = 1.0, t
     work = torch.empty_like(logits)
     out = torch.empty((R,), dtype=torch.int32, device=logits.device)
     _call("pta_sample", _ptr(out), _ptr(work), _ptr(logits), R, V, int(bool(do_sample)), ctypes.c_float(temperature),
-          int(top_k), ctypes.c_float(top_p), ctypes.c_float(min_p), ctypes.c_float(penalty), _ptr(hist), _ptr(hist_off),
+          int(top_k), ctypes.c_float(top_p), ctypes.c_float(min_p), ctypes.c_float(typical_p),
+          ctypes.c_float(epsilon_cutoff), ctypes.c_float(eta_cutoff), ctypes.c_float(penalty), _ptr(hist), _ptr(hist_off),
           _ptr(eos), 0 if eos is None else int(eos.numel()), _ptr(suppress), int(bool(remove_invalid)),
           int(bool(renorm)), ctypes.c_uint64(int(seed) & (2 ** 64 - 1)), _ptr(rng_seq), _ptr(rng_step), _ptr(uniforms),
           int(bool(need_scores)), _stream())

@@ -32,6 +32,10 @@ class Sampler:
         self.top_k = int(c.top_k) if (c.do_sample and c.top_k) else 0
         self.top_p = float(c.top_p) if (c.do_sample and c.top_p is not None) else 1.0
         self.min_p = float(c.min_p) if (c.do_sample and c.min_p is not None) else 0.0
+        self.typical_p = float(c.typical_p) if (c.do_sample and c.typical_p is not None and c.typical_p < 1.0) else 1.0
+        # the cut-offs apply strictly between 0 and 1 (src/transformers/generation/utils.py:1076-1087)
+        self.epsilon_cutoff = float(c.epsilon_cutoff) if (c.do_sample and c.epsilon_cutoff and 0.0 < c.epsilon_cutoff < 1.0) else 0.0
+        self.eta_cutoff = float(c.eta_cutoff) if (c.do_sample and c.eta_cutoff and 0.0 < c.eta_cutoff < 1.0) else 0.0
         self.penalty = float(c.repetition_penalty) if c.repetition_penalty is not None else 1.0
 
     def sample(self, logits: torch.Tensor, *, rng_seq: Sequence[int], rng_step: Sequence[int],
@@ -60,7 +64,8 @@ class Sampler:
         u = (torch.tensor(list(uniforms), dtype=torch.float32, device=self.device) if uniforms is not None else None)
         tokens, scores = ops.sample(
             logits, do_sample=self.do_sample, temperature=self.temperature, top_k=self.top_k, top_p=self.top_p,
-            min_p=self.min_p, penalty=self.penalty, hist=views[4] if use_hist else None,
+            min_p=self.min_p, typical_p=self.typical_p, epsilon_cutoff=self.epsilon_cutoff, eta_cutoff=self.eta_cutoff,
+            penalty=self.penalty, hist=views[4] if use_hist else None,
             hist_off=views[3] if use_hist else None, eos=self._eos_dev,
             suppress=views[2] if (self._eos_dev is not None and suppress_eos is not None and any(suppress_eos)) else None,
             remove_invalid=self.config.remove_invalid_values, renorm=self.config.renormalize_logits,

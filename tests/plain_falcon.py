@@ -277,10 +277,46 @@ def min_p(scores, mp, min_tokens_to_keep=1):
     return scores.masked_fill(mask, float("-inf"))
 
 
-def process(scores, history, *, do_sample, temperature_=1.0, top_k_=0, top_p_=1.0, min_p_=None,
-            repetition_penalty_=1.0, suppress_ids=()):
+def typical_p(scores, mass, min_tokens_to_keep=1):
+    """logits_process.py:663-683: tokens in the order of |(-log p) - entropy|, the nearest first; as many stay as
+    it takes for their mass to reach ``mass``, and every token as near as the last of them."""
+    logp = torch.log_softmax(scores, -1)
+    p = logp.exp()
+    entropy = -torch.nansum(logp * p)  # -inf * 0 is skipped
+    distance = ((-logp) - entropy).abs()
+    nearest_first = torch.argsort(distance, stable=True)
+    cum = scores[nearest_first].softmax(-1).cumsum(-1)
+    last = min(int((cum < mass).sum()), scores.shape[-1] - 1)
+    remove = distance > distance[nearest_first[last]]
+    remove[nearest_first[:min_tokens_to_keep]] = False
+    return scores.masked_fill(remove, float("-inf"))
+
+
+def _below_but_not_best(scores, probs, bound, min_tokens_to_keep=1):
+    best = torch.topk(scores, min(min_tokens_to_keep, scores.shape[-1]))[0][-1]
+    return scores.masked_fill((probs < bound) & (scores < best), float("-inf"))
+
+
+def epsilon_cutoff(scores, epsilon):
+    """logits_process.py:742-752: probabilities below ``epsilon`` go, the most probable token stays."""
+    return _below_but_not_best(scores, scores.softmax(-1), epsilon)
+
+
+def eta_cutoff(scores, epsilon):
+    """logits_process.py:825-837: the bound is min(epsilon, sqrt(epsilon) * exp(-entropy)); the entropy is that
+    of the normalised scores, a token that is already gone adding nothing."""
+    logp = torch.log_softmax(scores, -1)
+    probs = scores.softmax(-1)
+    entropy = -(logp.clamp(min=torch.finfo(scores.dtype).min) * probs).sum()
+    eta = min(epsilon, math.sqrt(epsilon) * math.exp(-float(entropy)))
+    return _below_but_not_best(scores, probs, eta)
+
+
+def process(scores, history, *, do_sample, temperature_=1.0, top_k_=0, top_p_=1.0, min_p_=None, typical_p_=None,
+            epsilon_cutoff_=None, eta_cutoff_=None, repetition_penalty_=1.0, suppress_ids=()):
     """Processors in the order the reference builds them (src/transformers/generation/utils.py:926-1097):
-    repetition penalty, minimum length, then (sampling only) temperature, top-k, top-p, min-p."""
+    repetition penalty, minimum length, then (sampling only) temperature, top-k, top-p, min-p, typical-p,
+    epsilon and eta cut-offs."""
     s = scores
     if repetition_penalty_ is not None and repetition_penalty_ != 1.0:
         s = repetition_penalty(s, history, repetition_penalty_)
@@ -295,6 +331,12 @@ def process(scores, history, *, do_sample, temperature_=1.0, top_k_=0, top_p_=1.
             s = top_p(s, top_p_)
         if min_p_ is not None:
             s = min_p(s, min_p_)
+        if typical_p_ is not None and typical_p_ < 1.0:
+            s = typical_p(s, typical_p_)
+        if epsilon_cutoff_ is not None and 0.0 < epsilon_cutoff_ < 1.0:
+            s = epsilon_cutoff(s, epsilon_cutoff_)
+        if eta_cutoff_ is not None and 0.0 < eta_cutoff_ < 1.0:
+            s = eta_cutoff(s, eta_cutoff_)
     return s
 
 

@@ -127,6 +127,9 @@ def test_generation_config():
         GenerationConfig(do_sample=True, temperature=0.0)
     with pytest.raises(ValueError, match="top_p"):
         GenerationConfig(do_sample=True, top_p=1.5)
+    with pytest.raises(ValueError, match="typical_p"):
+        GenerationConfig(do_sample=True, typical_p=0.0)
+    assert (g.typical_p, g.epsilon_cutoff, g.eta_cutoff) == (1.0, 0.0, 0.0)  # configuration_utils.py:423-425
     with pytest.raises(ValueError, match="num_return_sequences"):
         GenerationConfig(do_sample=False, num_return_sequences=2)
     with pytest.raises(ValueError, match="num_beams"):

@@ -88,6 +88,16 @@ def test_reference_vectors_on_the_kernel():
     _, s = ops.sample(_dev(dist), do_sample=True, min_p=0.05, uniforms=_dev([0.1] * 3))
     want = torch.tensor([[0.9, 0.0, 0.047, 0.0], [0.15, 0.3, 0.3, 0.25], [0.97, 0.0, 0.0, 0.0]])
     torch.testing.assert_close(torch.exp(s).cpu(), want, atol=1e-3, rtol=0)
+    # typical-p, epsilon and eta cut-offs (:357-378, :405-428, :445-468)
+    dist = torch.log(torch.tensor([[0.97, 0.01, 0.01, 0.01], [0.4, 0.2, 0.2, 0.2]]))
+    _, s = ops.sample(_dev(dist), do_sample=True, typical_p=0.5, uniforms=_dev([0.1] * 2))
+    torch.testing.assert_close(torch.exp(s).cpu(), torch.tensor([[0.97, 0.0, 0.0, 0.0], [0.0, 0.2, 0.2, 0.2]]), atol=1e-3, rtol=0)
+    dist = torch.log(torch.tensor([[0.87, 0.099, 0.001, 0.03], [0.4, 0.299, 0.101, 0.2]]))
+    _, s = ops.sample(_dev(dist), do_sample=True, epsilon_cutoff=0.1, uniforms=_dev([0.1] * 2))
+    torch.testing.assert_close(torch.exp(s).cpu(), torch.tensor([[0.87, 0.0, 0.0, 0.0], [0.4, 0.299, 0.101, 0.2]]), atol=1e-3, rtol=0)
+    dist = torch.log(torch.tensor([[0.0, 0.1, 0.8, 0.1], [0.01, 0.04, 0.9, 0.05]]))
+    _, s = ops.sample(_dev(dist), do_sample=True, eta_cutoff=0.0625, uniforms=_dev([0.1] * 2))
+    torch.testing.assert_close(torch.exp(s).cpu(), torch.tensor([[0.0, 0.1, 0.8, 0.1], [0.0, 0.0, 0.9, 0.0]]), atol=1e-3, rtol=0)
     # top_p so small that everything could go: the best token stays
     _, s = ops.sample(_dev(torch.arange(6.0)[None]), do_sample=True, top_p=0.0, uniforms=_dev([0.9]))
     assert _finite_mask(s[0]).tolist() == [False] * 5 + [True]
@@ -205,6 +215,46 @@ def test_random_settings_match_plain(V):
             t = int(tok[r])
             lo = float(cdf[t - 1]) if t else 0.0
             assert keep_got[t] and lo - 1e-5 <= float(u[r]) <= float(cdf[t]) + 1e-5, (V, trial, kw, r, t)
+
+
+@pytest.mark.parametrize("V", [5, 211, 4100, 65024, 70001])
+def test_typical_epsilon_eta_match_plain(V):
+    """The three later warpers alone, together, and behind top-k and top-p: the survivors are the plain code's
+    (a token within rounding of a bound may fall on either side), and the draw comes from among them, also
+    where typical-p has taken the likeliest token away."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(77 + V)
+    R = 4
+    for trial, kw in enumerate((dict(typical_p=0.9), dict(typical_p=0.2), dict(epsilon_cutoff=3e-4), dict(eta_cutoff=2e-3),
+                                dict(typical_p=0.95, epsilon_cutoff=1e-4, eta_cutoff=1e-3, temperature=0.8),
+                                dict(top_k=40, typical_p=0.6), dict(top_k=50, top_p=0.9, eta_cutoff=0.05, epsilon_cutoff=0.02),
+                                dict(typical_p=1e-6), dict(epsilon_cutoff=0.9), dict(eta_cutoff=0.9))):
+        logits = torch.randn(R, V, generator=g) * (1.0 + trial % 4)
+        logits[R - 1] = (logits[R - 1] * 2).round() / 2  # groups of equal scores
+        u = torch.rand(R, generator=g)
+        names = dict(temperature=1.0, top_k=0, top_p=1.0, typical_p=1.0, epsilon_cutoff=0.0, eta_cutoff=0.0)
+        names.update(kw)
+        names["top_k"] = min(names["top_k"], V)
+        tok, scores = ops.sample(_dev(logits), do_sample=True, uniforms=_dev(u), **names)
+        for r in range(R):
+            want = P.process(logits[r], [], do_sample=True, temperature_=names["temperature"], top_k_=names["top_k"],
+                             top_p_=names["top_p"], typical_p_=names["typical_p"], epsilon_cutoff_=names["epsilon_cutoff"],
+                             eta_cutoff_=names["eta_cutoff"])
+            got = scores[r].cpu()
+            keep_want, keep_got = want != float("-inf"), _finite_mask(got)
+            diff = (keep_want != keep_got).nonzero().flatten().tolist()
+            assert len(diff) <= 2, f"V={V} {kw} row {r}: kept sets differ at {diff[:10]} ({int(keep_want.sum())} kept)"
+            assert int(keep_got.sum()) >= 1
+            both = keep_want & keep_got
+            torch.testing.assert_close(got[both], want[both], rtol=1e-6, atol=1e-6)
+            cdf = torch.softmax(got.double(), -1).cumsum(-1)
+            t = int(tok[r])
+            lo = float(cdf[t - 1]) if t else 0.0
+            assert keep_got[t] and lo - 1e-5 <= float(u[r]) <= float(cdf[t]) + 1e-5, (V, kw, r, t)
+    # the likeliest token goes where it is far from typical, and the draw never returns it
+    x = torch.log(torch.tensor([[0.4] + [0.6 / 30] * 30]))
+    tok, s = ops.sample(_dev(x), do_sample=True, typical_p=0.5, uniforms=_dev([0.0]))
+    assert not _finite_mask(s[0])[0] and int(tok[0]) == 1
 
 
 def test_counter_based_uniforms():

@@ -274,6 +274,20 @@ def test_processors_on_the_references_vectors():
         torch.testing.assert_close(torch.exp(P.min_p(dist[r], 0.05)), want[r], atol=1e-3, rtol=0)
     assert int((P.min_p(ramp, 0.9, min_tokens_to_keep=2) != float("-inf")).sum()) == 2
 
+    # typical-p, epsilon and eta cut-offs (:357-378, :405-428, :445-468)
+    dist = torch.log(torch.tensor([[0.97, 0.01, 0.01, 0.01], [0.4, 0.2, 0.2, 0.2]]))
+    want = torch.tensor([[0.97, 0.0, 0.0, 0.0], [0.0, 0.2, 0.2, 0.2]])  # the likeliest token is not the typical one
+    for r in range(2):
+        torch.testing.assert_close(torch.exp(P.typical_p(dist[r], 0.5)), want[r], atol=1e-3, rtol=0)
+    dist = torch.log(torch.tensor([[0.87, 0.099, 0.001, 0.03], [0.4, 0.299, 0.101, 0.2]]))
+    want = torch.tensor([[0.87, 0.0, 0.0, 0.0], [0.4, 0.299, 0.101, 0.2]])
+    for r in range(2):
+        torch.testing.assert_close(torch.exp(P.epsilon_cutoff(dist[r], 0.1)), want[r], atol=1e-3, rtol=0)
+    dist = torch.log(torch.tensor([[0.0, 0.1, 0.8, 0.1], [0.01, 0.04, 0.9, 0.05]]))
+    want = torch.tensor([[0.0, 0.1, 0.8, 0.1], [0.0, 0.0, 0.9, 0.0]])
+    for r in range(2):
+        torch.testing.assert_close(torch.exp(P.eta_cutoff(dist[r], 0.0625)), want[r], atol=1e-3, rtol=0)
+
     # temperature (:148-181): uniform stays uniform, peaks sharpen below 1 and flatten above
     s = torch.full((20,), 0.05); s[5] = 0.15; s[10] = -0.35
     p, sharp, smooth = (torch.softmax(t, -1) for t in (s, P.temperature(s, 0.5), P.temperature(s, 1.3)))
