@@ -42,6 +42,10 @@ class GenerationConfig:
     epsilon_cutoff: Optional[float] = 0.0
     eta_cutoff: Optional[float] = 0.0
     repetition_penalty: Optional[float] = 1.0
+    no_repeat_ngram_size: Optional[int] = 0
+    bad_words_ids: Optional[List[List[int]]] = None
+    suppress_tokens: Optional[List[int]] = None
+    begin_suppress_tokens: Optional[List[int]] = None
     renormalize_logits: bool = False
     remove_invalid_values: bool = False
     # outputs
@@ -111,6 +115,17 @@ class GenerationConfig:
                 raise ValueError(f"`min_p` has to be a float in the [0, 1] interval, but is {self.min_p}")
             if self.typical_p is not None and self.typical_p < 1.0 and not (self.typical_p > 0):  # :651-653
                 raise ValueError(f"`typical_p` has to be a float > 0 and < 1, but is {self.typical_p}")
+        n = self.no_repeat_ngram_size
+        if n is not None and n != 0 and (not isinstance(n, int) or n < 0):  # logits_process.py:949-951
+            raise ValueError(f"`ngram_size` has to be a strictly positive integer, but is {n}")
+        bw = self.bad_words_ids
+        if bw is not None:  # logits_process.py:1288-1299
+            if not isinstance(bw, list) or len(bw) == 0:
+                raise ValueError(f"`bad_words_ids` has to be a non-empty list, but is {bw}.")
+            if any(not isinstance(w, list) for w in bw):
+                raise ValueError(f"`bad_words_ids` has to be a list of lists, but is {bw}.")
+            if any(len(w) == 0 or any((not isinstance(t, int) or t < 0) for t in w) for w in bw):
+                raise ValueError(f"Each list in `bad_words_ids` has to be a list of positive integers, but is {bw}.")
         rp = self.repetition_penalty
         if rp is not None and (not isinstance(rp, float) or not (rp > 0)):  # :329-331
             raise ValueError(f"`penalty` has to be a strictly positive float, but is {rp}")

@@ -108,11 +108,11 @@ int pta_gemm_splitk_pair_reduced_bf16(void* y1, float* part1, const void* x1, co
 // processors in the reference's order, then argmax (do_sample 0) or a draw; `work` [R, V] is scratch and,
 // with want_scores, receives the processed scores (without, its contents are unspecified);
 // typical_p 1, epsilon_cutoff 0 and eta_cutoff 0 switch those off; hist/hist_off (tokens seen, per row),
-// eos/suppress, uniforms may be null
+// ban/ban_off (tokens a row may not take, per row), eos/suppress, uniforms may be null
 int pta_sample(int* out_tok, float* work, const float* logits, int R, int V, int do_sample, float temperature,
                int top_k, float top_p, float min_p, float typical_p, float epsilon_cutoff, float eta_cutoff,
-               float penalty, const int* hist, const int* hist_off, const int* eos, int n_eos,
-               const int* suppress, int remove_invalid, int renorm, uint64_t seed,
+               float penalty, const int* hist, const int* hist_off, const int* ban, const int* ban_off,
+               const int* eos, int n_eos, const int* suppress, int remove_invalid, int renorm, uint64_t seed,
                const int* rng_seq, const int* rng_step, const float* uniforms, int want_scores, void* stream);
 
 // out_tok[r] = index of the largest of logits[r, :], lowest index among equals (greedy choice, no processors)

@@ -134,7 +134,7 @@ struct SampleShared {
     uint32_t bin, remaining, all, n_cand;
     unsigned long long cum;
     // the short way (sample_short): scores seen before, scores that are left, and the survivors in index order
-    uint32_t seen[2048], left[2048];
+    uint32_t seen[2048], left[2048], banned[2048];
     uint32_t cand_idx[S_SHORT];
     uint32_t s_key[S_SHORT], s_idx[S_SHORT], s_alive[S_SHORT];
     uint32_t pick, last_mass;
@@ -262,10 +262,12 @@ __device__ __forceinline__ float key_value(uint32_t k) {
 }
 
 // The processed score of a token before the thresholds: repetition penalty (tokens seen before are marked in
-// a bitmap in LDS, so vocabularies up to 65,536), EOS suppression, invalid values, temperature, in this order.
+// a bitmap in LDS, so vocabularies up to 65,536), the row's banned tokens (a second bitmap), EOS suppression,
+// invalid values, temperature, in this order.
 struct Processed {
     const float* l;
     const uint32_t* seen;  // null: no penalty
+    const uint32_t* banned;  // null: no token of this row is banned
     const int* eos;
     int n_eos;  // 0: no suppression
     float penalty, temperature;
@@ -273,6 +275,7 @@ struct Processed {
     __device__ __forceinline__ float operator()(int i) const { return of(i, l[i]); }
     __device__ __forceinline__ float of(int i, float x) const {
         if (seen && ((seen[i >> 5] >> (i & 31)) & 1u)) x = x < 0.f ? x * penalty : x / penalty;
+        if (banned && ((banned[i >> 5] >> (i & 31)) & 1u)) x = -INFINITY;
         for (int e = 0; e < n_eos; ++e)
             if (eos[e] == i) x = -INFINITY;
         if (remove_invalid) {
@@ -298,6 +301,21 @@ __device__ __forceinline__ const uint32_t* mark_seen(SampleShared& sh, int row, 
     }
     __syncthreads();
     return sh.seen;
+}
+
+// marks the row's banned tokens in sh.banned; returns the bitmap, or null if the row has none
+__device__ __forceinline__ const uint32_t* mark_banned(SampleShared& sh, int row, int V, const int* __restrict__ ban,
+                                                       const int* __restrict__ ban_off) {
+    if (!ban_off || ban_off[row + 1] == ban_off[row]) return nullptr;
+    const int tid = threadIdx.x;
+    for (int w = tid; w < 2048; w += S_THREADS) sh.banned[w] = 0u;
+    __syncthreads();
+    for (int t = ban_off[row] + tid; t < ban_off[row + 1]; t += S_THREADS) {
+        const int tok = ban[t];
+        if (tok >= 0 && tok < V) atomicOr(&sh.banned[tok >> 5], 1u << (tok & 31));
+    }
+    __syncthreads();
+    return sh.banned;
 }
 
 // f(i, l[i]) for every score of a row, each thread in ascending order of i.  Sixteen bytes a load and four
@@ -448,8 +466,9 @@ __device__ __forceinline__ bool sample_short(
 __global__ __launch_bounds__(S_THREADS) void sample_kernel(
     int* __restrict__ out_tok, float* __restrict__ work, const float* __restrict__ logits, int V, int do_sample,
     float temperature, int top_k, float top_p, float min_p, float typical_p, float epsilon_cutoff, float eta_cutoff,
-    float penalty, const int* __restrict__ hist, const int* __restrict__ hist_off, const int* __restrict__ eos, int n_eos,
-    const int* __restrict__ suppress, int remove_invalid, int renorm, uint64_t seed, const int* __restrict__ rng_seq,
+    float penalty, const int* __restrict__ hist, const int* __restrict__ hist_off, const int* __restrict__ ban,
+    const int* __restrict__ ban_off, const int* __restrict__ eos, int n_eos, const int* __restrict__ suppress,
+    int remove_invalid, int renorm, uint64_t seed, const int* __restrict__ rng_seq,
     const int* __restrict__ rng_step, const float* __restrict__ uniforms, int want_scores) {
     __shared__ SampleShared sh;
     float* const red = sh.red;
@@ -472,7 +491,8 @@ __global__ __launch_bounds__(S_THREADS) void sample_kernel(
     float first_max = -INFINITY;  // the largest of the scores this thread saw in the first pass
     bool have_first = false;
     if (V <= 65536) {
-        const Processed score{l, mark_seen(sh, row, V, penalty, hist, hist_off), eos, suppress_eos ? n_eos : 0, penalty,
+        const Processed score{l, mark_seen(sh, row, V, penalty, hist, hist_off), mark_banned(sh, row, V, ban, ban_off), eos,
+                              suppress_eos ? n_eos : 0, penalty,
                               do_sample ? temperature : 1.0f, remove_invalid};
         const bool later_warpers = typical_p < 1.0f || epsilon_cutoff > 0.0f || eta_cutoff > 0.0f;  // the long way has them
         if (do_sample && top_k > 0 && top_k < V && top_k <= n_holding && top_k <= S_SHORT && !later_warpers) {
@@ -505,6 +525,11 @@ __global__ __launch_bounds__(S_THREADS) void sample_kernel(
                     w[tok] = v < 0.f ? v * penalty : v / penalty;
                 }
             }
+            __syncthreads();
+        }
+        if (ban_off) {
+            for (int t = ban_off[row] + tid; t < ban_off[row + 1]; t += S_THREADS)
+                if (ban[t] >= 0 && ban[t] < V) w[ban[t]] = -INFINITY;
             __syncthreads();
         }
         if (suppress_eos) {
@@ -883,7 +908,8 @@ __global__ __launch_bounds__(S_THREADS) void sample_kernel(
 extern "C" int pta_sample(int* out_tok, float* work, const float* logits, int R, int V, int do_sample,
                           float temperature, int top_k, float top_p, float min_p, float typical_p,
                           float epsilon_cutoff, float eta_cutoff, float penalty, const int* hist,
-                          const int* hist_off, const int* eos, int n_eos, const int* suppress, int remove_invalid,
+                          const int* hist_off, const int* ban, const int* ban_off, const int* eos, int n_eos,
+                          const int* suppress, int remove_invalid,
                           int renorm, uint64_t seed, const int* rng_seq, const int* rng_step, const float* uniforms,
                           int want_scores, void* stream) {
     PTA_REQUIRE(R > 0 && V > 0, "sample: rows=%d vocab=%d must be positive", R, V);
@@ -898,10 +924,10 @@ extern "C" int pta_sample(int* out_tok, float* work, const float* logits, int R,
     PTA_REQUIRE(penalty > 0.f, "sample: repetition penalty must be > 0, got %g", (double)penalty);
     PTA_REQUIRE(!do_sample || uniforms || (rng_seq && rng_step), "sample: sampling needs uniforms or rng counters");
     PTA_REQUIRE(n_eos == 0 || eos, "sample: eos ids missing");
+    PTA_REQUIRE(!ban_off || ban, "sample: banned ids missing");
     hipLaunchKernelGGL(sample_kernel, dim3(R), dim3(S_THREADS), 0, (hipStream_t)stream, out_tok, work, logits, V,
                        do_sample, temperature, top_k, top_p, min_p, typical_p, epsilon_cutoff, eta_cutoff, penalty, hist,
-                       hist_off, eos, n_eos, suppress,
-                       remove_invalid, renorm, seed, rng_seq, rng_step, uniforms, want_scores);
+                       hist_off, ban, ban_off, eos, n_eos, suppress, remove_invalid, renorm, seed, rng_seq, rng_step, uniforms, want_scores);
     return pta_check_launch("sample");
 }
 

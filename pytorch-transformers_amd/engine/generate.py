@@ -123,6 +123,7 @@ def generate(model, prompts: Sequence[Sequence[int]], generation_config: Optiona
                 tokens, scores = sampler.sample(
                     logits, rng_seq=[ids[i] for i in live], rng_step=[step_no] * len(live),
                     histories=[prompts[i] + out_tokens[i] for i in live], suppress_eos=[too_short] * len(live),
+                    new_counts=[len(out_tokens[i]) for i in live],
                     need_scores=want_scores)
                 step_no += 1
                 timed_out = cfg.max_time is not None and (time.time() - t0) > cfg.max_time  # stopping_criteria.py:87-107

@@ -365,7 +365,7 @@ def attention(q: torch.Tensor, k_pool, v_pool, block_table, ctx, slopes, scale: 
 
 def sample(logits: torch.Tensor, *, do_sample: bool, temperature: float = 1.0, top_k: int = 0, top_p: float = 1.0,
            min_p: float = 0.0, typical_p: float = 1.0, epsilon_cutoff: float = 0.0, eta_cutoff: float = 0.0,
-           penalty: float = 1.0, hist=None, hist_off=None, eos=None, suppress=None,
+           penalty: float = 1.0, hist=None, hist_off=None, ban=None, ban_off=None, eos=None, suppress=None,
            remove_invalid: bool = False, renorm: bool = False, seed: int = 0, rng_seq=None, rng_step=None,
            uniforms=None, need_scores: bool = True):
     """Processors and choice for every row of ``logits`` [R, V] (32-bit); returns (tokens int32 [R], scores [R, V]).
@@ -376,17 +376,23 @@ def sample(logits: torch.Tensor, *, do_sample: bool, temperature: float = 1.0, t
     if logits.dim() != 2:
         raise KernelError(f"logits must be [rows, vocab], got {tuple(logits.shape)}")
     R, V = logits.shape
-    if (not need_scores and not do_sample and penalty == 1.0 and suppress is None and not remove_invalid
-            and not renorm):
+    if ban is not None and ban.numel() == 0:
+        ban = ban_off = None  # no row has a banned token
+    if (not need_scores and not do_sample and penalty == 1.0 and suppress is None and ban_off is None
+            and not remove_invalid and not renorm):
         out = torch.empty((R,), dtype=torch.int32, device=logits.device)
         _call("pta_argmax", _ptr(out), _ptr(logits), R, V, _stream())
         return out, None
-    for name, t, n in (("hist_off", hist_off, R + 1), ("suppress", suppress, R), ("rng_seq", rng_seq, R),
+    for name, t, n in (("hist_off", hist_off, R + 1), ("ban_off", ban_off, R + 1), ("suppress", suppress, R), ("rng_seq", rng_seq, R),
                        ("rng_step", rng_step, R)):
         if t is not None:
             _need(t, name, torch.int32, (n,))
     if hist is not None:
         _need(hist, "hist", torch.int32)
+    if ban_off is not None:
+        if ban is None:
+            raise KernelError("ban_off without ban")
+        _need(ban, "ban", torch.int32)
     if eos is not None:
         _need(eos, "eos", torch.int32)
     if uniforms is not None:
@@ -396,6 +402,7 @@ def sample(logits: torch.Tensor, *, do_sample: bool, temperature: float = 1.0, t
     _call("pta_sample", _ptr(out), _ptr(work), _ptr(logits), R, V, int(bool(do_sample)), ctypes.c_float(temperature),
           int(top_k), ctypes.c_float(top_p), ctypes.c_float(min_p), ctypes.c_float(typical_p),
           ctypes.c_float(epsilon_cutoff), ctypes.c_float(eta_cutoff), ctypes.c_float(penalty), _ptr(hist), _ptr(hist_off),
+          _ptr(ban), _ptr(ban_off),
           _ptr(eos), 0 if eos is None else int(eos.numel()), _ptr(suppress), int(bool(remove_invalid)),
           int(bool(renorm)), ctypes.c_uint64(int(seed) & (2 ** 64 - 1)), _ptr(rng_seq), _ptr(rng_step), _ptr(uniforms),
           int(bool(need_scores)), _stream())

@@ -16,6 +16,7 @@ import torch
 
 from .. import ops
 from ..config.generation import GenerationConfig
+from .bans import BanRules
 
 
 class Sampler:
@@ -37,16 +38,28 @@ class Sampler:
         self.epsilon_cutoff = float(c.epsilon_cutoff) if (c.do_sample and c.epsilon_cutoff and 0.0 < c.epsilon_cutoff < 1.0) else 0.0
         self.eta_cutoff = float(c.eta_cutoff) if (c.do_sample and c.eta_cutoff and 0.0 < c.eta_cutoff < 1.0) else 0.0
         self.penalty = float(c.repetition_penalty) if c.repetition_penalty is not None else 1.0
+        self.bans = BanRules(c.no_repeat_ngram_size, c.bad_words_ids, c.suppress_tokens, c.begin_suppress_tokens,
+                             self.eos_ids)
 
     def sample(self, logits: torch.Tensor, *, rng_seq: Sequence[int], rng_step: Sequence[int],
                histories: Optional[Sequence[Sequence[int]]] = None, suppress_eos: Optional[Sequence[bool]] = None,
-               uniforms: Optional[Sequence[float]] = None,
+               uniforms: Optional[Sequence[float]] = None, new_counts: Optional[Sequence[int]] = None,
                need_scores: bool = True) -> Tuple[List[int], Optional[torch.Tensor]]:
         """Tokens for the rows of ``logits`` and the processed scores ``[rows, vocab]`` (None if not needed
-        and the choice could be made without forming them)."""
+        and the choice could be made without forming them).  ``histories`` are the rows' ids so far (prompt and
+        new tokens) and ``new_counts`` how many of them are new; the repetition penalty and the options that forbid
+        tokens read them."""
         R = logits.shape[0]
         suppress = self._eos_dev is not None and suppress_eos is not None and any(suppress_eos)
-        if (not need_scores and not self.do_sample and self.penalty == 1.0 and not suppress
+        ban_lists = None
+        if self.bans:
+            if histories is None:
+                raise ValueError("options that forbid tokens by what was generated need the rows' histories")
+            counts = new_counts if new_counts is not None else [1] * R
+            ban_lists = [self.bans.banned(h, n) for h, n in zip(histories, counts)]
+            if not any(ban_lists):
+                ban_lists = None
+        if (not need_scores and not self.do_sample and self.penalty == 1.0 and not suppress and ban_lists is None
                 and not self.config.remove_invalid_values and not self.config.renormalize_logits):
             # greedy with no processor in the way: nothing to upload, one argmax kernel
             return ops.sample(logits, do_sample=False, need_scores=False)[0].tolist(), None
@@ -59,6 +72,11 @@ class Sampler:
             flat = (np.concatenate([np.asarray(h, dtype=np.int32) for h in histories])
                     if off[-1] else np.zeros(0, dtype=np.int32))
             pieces += [off, flat]
+        n_before = len(pieces)
+        if ban_lists is not None:
+            boff = np.zeros(R + 1, dtype=np.int32)
+            boff[1:] = np.cumsum([len(b) for b in ban_lists])
+            pieces += [boff, np.asarray([t for b in ban_lists for t in b], dtype=np.int32)]
         dev = torch.from_numpy(np.concatenate(pieces)).to(self.device)
         views = torch.split(dev, [int(p.shape[0]) for p in pieces])
         u = (torch.tensor(list(uniforms), dtype=torch.float32, device=self.device) if uniforms is not None else None)
@@ -66,7 +84,8 @@ class Sampler:
             logits, do_sample=self.do_sample, temperature=self.temperature, top_k=self.top_k, top_p=self.top_p,
             min_p=self.min_p, typical_p=self.typical_p, epsilon_cutoff=self.epsilon_cutoff, eta_cutoff=self.eta_cutoff,
             penalty=self.penalty, hist=views[4] if use_hist else None,
-            hist_off=views[3] if use_hist else None, eos=self._eos_dev,
+            hist_off=views[3] if use_hist else None, ban=views[n_before + 1] if ban_lists is not None else None,
+            ban_off=views[n_before] if ban_lists is not None else None, eos=self._eos_dev,
             suppress=views[2] if (self._eos_dev is not None and suppress_eos is not None and any(suppress_eos)) else None,
             remove_invalid=self.config.remove_invalid_values, renorm=self.config.renormalize_logits,
             seed=self.config.seed, rng_seq=views[0], rng_step=views[1], uniforms=u, need_scores=need_scores)

@@ -312,14 +312,45 @@ def eta_cutoff(scores, epsilon):
     return _below_but_not_best(scores, probs, eta)
 
 
+def no_repeat_ngram(scores, history, n):
+    """logits_process.py:840-903, :954-962: every n-gram of the ids so far, filed under its first n - 1 tokens;
+    what is filed under the last n - 1 ids may not come next."""
+    ids = list(history)
+    if len(ids) + 1 < n:
+        return scores
+    filed = {}
+    for j in range(len(ids) - n + 1):
+        gram = tuple(ids[j:j + n])
+        filed.setdefault(gram[:-1], []).append(gram[-1])
+    return suppress(scores, filed.get(tuple(ids[len(ids) + 1 - n:]), []))
+
+
+def no_bad_words(scores, history, bad_words, eos_ids=()):
+    """logits_process.py:1110-1140, :1270-1286: -inf for the last token of an entry whose other tokens end the ids
+    so far (one-token entries always); an entry that is an EOS token alone does not count."""
+    ids = list(history)
+    gone = []
+    for word in bad_words:
+        if len(word) == 1 and word[0] in eos_ids:
+            continue
+        if len(word) == 1 or (len(word) - 1 <= len(ids) and ids[len(ids) - (len(word) - 1):] == list(word[:-1])):
+            gone.append(word[-1])
+    return suppress(scores, gone)
+
+
 def process(scores, history, *, do_sample, temperature_=1.0, top_k_=0, top_p_=1.0, min_p_=None, typical_p_=None,
-            epsilon_cutoff_=None, eta_cutoff_=None, repetition_penalty_=1.0, suppress_ids=()):
+            epsilon_cutoff_=None, eta_cutoff_=None, repetition_penalty_=1.0, suppress_ids=(), no_repeat_ngram_size_=0,
+            bad_words_ids_=None, eos_ids_=()):
     """Processors in the order the reference builds them (src/transformers/generation/utils.py:926-1097):
-    repetition penalty, minimum length, then (sampling only) temperature, top-k, top-p, min-p, typical-p,
+    repetition penalty, no-repeat n-grams, bad words, minimum length, then (sampling only) temperature, top-k, top-p, min-p, typical-p,
     epsilon and eta cut-offs."""
     s = scores
     if repetition_penalty_ is not None and repetition_penalty_ != 1.0:
         s = repetition_penalty(s, history, repetition_penalty_)
+    if no_repeat_ngram_size_:
+        s = no_repeat_ngram(s, history, no_repeat_ngram_size_)
+    if bad_words_ids_:
+        s = no_bad_words(s, history, bad_words_ids_, eos_ids_)
     if suppress_ids:
         s = suppress(s, suppress_ids)
     if do_sample:

@@ -51,9 +51,10 @@ class ArgmaxSampler:
         self.calls = []
         self.eos = list(eos)
 
-    def sample(self, logits, *, rng_seq, rng_step, histories, suppress_eos, uniforms=None, need_scores=True):
+    def sample(self, logits, *, rng_seq, rng_step, histories, suppress_eos, uniforms=None, new_counts=None,
+               need_scores=True):
         self.calls.append(dict(rng_seq=list(rng_seq), rng_step=list(rng_step), suppress=list(suppress_eos),
-                               histories=[list(h) for h in histories]))
+                               histories=[list(h) for h in histories], new_counts=list(new_counts)))
         scores = logits.clone()
         for r, sup in enumerate(suppress_eos):
             if sup:

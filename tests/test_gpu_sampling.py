@@ -257,6 +257,63 @@ def test_typical_epsilon_eta_match_plain(V):
     assert not _finite_mask(s[0])[0] and int(tok[0]) == 1
 
 
+@pytest.mark.parametrize("V", [40, 65024, 70001])
+def test_banned_tokens_per_row(V):
+    """A list of tokens per row that may not be taken: gone from the scores and never chosen, greedy or drawn,
+    by the short way and the long way, with the other processors around them."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(V)
+    R = 4
+    logits = torch.randn(R, V, generator=g) * 2
+    best = logits.argmax(-1).tolist()
+    bans = [[best[0], 3], [], [best[2]] + list(range(10, 30)), [V - 1, 0, best[3]]]
+    off = [0]
+    for b in bans:
+        off.append(off[-1] + len(b))
+    flat = [t for b in bans for t in b]
+    kw_ban = dict(ban=_dev(flat, torch.int32), ban_off=_dev(off, torch.int32))
+    tok, scores = ops.sample(_dev(logits), do_sample=False, **kw_ban)
+    for r in range(R):
+        want = P.suppress(logits[r], bans[r])
+        assert torch.equal(scores[r].cpu(), want) and int(tok[r]) == int(want.argmax())
+    u = torch.rand(R, generator=g)
+    for kw in (dict(top_k=5), dict(top_k=0, top_p=0.9), dict(top_k=20, temperature=0.7, penalty=1.3)):
+        hist = [[best[r], 1, 2] for r in range(R)]
+        tok, scores = ops.sample(_dev(logits), do_sample=True, uniforms=_dev(u), temperature=kw.get("temperature", 1.0),
+                                 top_k=kw["top_k"], top_p=kw.get("top_p", 1.0), penalty=kw.get("penalty", 1.0),
+                                 hist=_dev([t for h in hist for t in h], torch.int32),
+                                 hist_off=_dev([0, 3, 6, 9, 12], torch.int32), **kw_ban)
+        for r in range(R):
+            want = P.process(P.suppress(logits[r], bans[r]), hist[r], do_sample=True, temperature_=kw.get("temperature", 1.0),
+                             top_k_=kw["top_k"], top_p_=kw.get("top_p", 1.0), repetition_penalty_=kw.get("penalty", 1.0))
+            keep_want, keep_got = want != float("-inf"), _finite_mask(scores[r])
+            assert int((keep_want != keep_got).sum()) <= (1 if "top_p" in kw else 0), (V, kw, r)
+            assert int(tok[r]) not in bans[r] and keep_got[int(tok[r])]
+
+
+def test_generation_without_repeated_ngrams_equals_plain(folders):
+    """Greedy generation with no_repeat_ngram_size and bad_words_ids against the plain loop: a tiny random model
+    repeats itself soon, so the option decides tokens."""
+    from pytorch_transformers_amd import AutoModelForCausalLM, GenerationConfig
+
+    cfg, w = P.read_model(folders["A"])
+    g = torch.Generator().manual_seed(5)
+    prompts = [torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for n in (3, 9)]
+    model = AutoModelForCausalLM.from_pretrained(folders["A"], dtype="float32")
+    free = [p + P.generate(cfg, w, p, 24) for p in prompts]
+    bad = [[free[0][len(prompts[0]) + 1]], free[1][len(prompts[1]) + 2:len(prompts[1]) + 4]]
+    for opts in (dict(no_repeat_ngram_size=1), dict(no_repeat_ngram_size=2), dict(bad_words_ids=bad),
+                 dict(no_repeat_ngram_size=3, bad_words_ids=bad)):
+        want = [p + P.generate(cfg, w, p, 24, no_repeat_ngram_size_=opts.get("no_repeat_ngram_size", 0),
+                               bad_words_ids_=opts.get("bad_words_ids")) for p in prompts]
+        got = model.generate(prompts, GenerationConfig(max_new_tokens=24, do_sample=False, eos_token_id=None, **opts))
+        assert got == want, opts
+        assert want != free, f"{opts} changed nothing: the test would not see the option"
+    new = want[0][len(prompts[0]):]
+    grams = [tuple(want[0][j:j + 3]) for j in range(len(want[0]) - 2)]
+    assert len(set(grams)) == len(grams) and bad[0][0] not in new
+
+
 def test_counter_based_uniforms():
     """Same (seed, sequence, step) -> same draw whatever the batch; the host function gives the number."""
     from pytorch_transformers_amd.sampling import philox_uniform

@@ -288,6 +288,15 @@ def test_processors_on_the_references_vectors():
     for r in range(2):
         torch.testing.assert_close(torch.exp(P.eta_cutoff(dist[r], 0.0625)), want[r], atol=1e-3, rtol=0)
 
+    # no-repeat n-grams and bad words (:485-508, :576-601)
+    flat = torch.zeros(3)
+    for ids, n, gone in (([1, 1, 2, 1], 2, [False, True, True]), ([0, 1, 0, 1], 2, [True, False, False]),
+                         ([1, 1, 2, 1], 3, [False, False, False]), ([0, 1, 0, 1], 3, [True, False, False])):
+        assert torch.isinf(P.no_repeat_ngram(flat, ids, n)).tolist() == gone
+    words = [[1], [4], [1, 0], [0, 1, 2], [1, 3, 1, 3]]
+    assert torch.isinf(P.no_bad_words(torch.zeros(5), [0, 1, 3, 1], words, eos_ids=[4])).tolist() == [True, True, False, True, False]
+    assert torch.isinf(P.no_bad_words(torch.zeros(5), [0, 1, 0, 1], words, eos_ids=[4])).tolist() == [True, True, True, False, False]
+
     # temperature (:148-181): uniform stays uniform, peaks sharpen below 1 and flatten above
     s = torch.full((20,), 0.05); s[5] = 0.15; s[10] = -0.35
     p, sharp, smooth = (torch.softmax(t, -1) for t in (s, P.temperature(s, 0.5), P.temperature(s, 1.3)))
