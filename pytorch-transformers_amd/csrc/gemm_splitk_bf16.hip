@@ -1,4 +1,4 @@
-// y[M,N] = act(x[M,K] . W[N,K]^T + bias) + add1 + add2 for a decode batch of up to 64 rows,
+// y[M,N] = act(x[M,K] . W[N,K]^T + bias) + add1 + add2 for a decode batch of up to 128 rows,
 // bfloat16 in, 32-bit accumulation on the matrix cores.
 //
 // With more than 16 rows the activations are no longer negligible beside the weights: a wave that
@@ -32,6 +32,8 @@ union Frag8 {
 };
 
 #define SK_THREADS 256
+#define SK_CHUNK_ROWS 128  // eight tiles of sixteen rows of x: what a workgroup holds
+#define SK_MAX_ROWS 256
 
 // One product of a launch.  A launch may carry two that share M (a block's two output projections, left
 // as partial sums): the workgroups of the second follow those of the first in a one-dimensional grid.
@@ -51,7 +53,8 @@ struct SplitkProblem {
 };
 
 template <int MT, int RT, int U, int D>
-__global__ __launch_bounds__(SK_THREADS) void gemm_splitk_kernel(SplitkProblem pa, SplitkProblem pb, int M) {
+__global__ __launch_bounds__(SK_THREADS) void gemm_splitk_kernel(SplitkProblem pa, SplitkProblem pb, int M, int chunks,
+                                                                 int chunk_rows) {
     constexpr int KS = U * 64;                       // elements of K per stage
     constexpr int MP = MT * 16;                      // rows of x, padded to whole tiles
     constexpr int LDW = KS + 8;                      // LDS row stride: 16 bytes of padding keep 16-byte reads off each other's banks
@@ -63,8 +66,24 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_splitk_kernel(SplitkProblem p
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 15, g = lane >> 4;
+    // More rows than a workgroup holds are cut into `chunks` chunks of `chunk_rows`; the workgroups that take the
+    // same rows of W for the chunks sit a multiple of eight apart in the grid, so that they start together on one
+    // die and all but the first find W in its cache.
     const int first_blocks = pa.tiles * pa.parts;
-    const bool second = (int)blockIdx.x >= first_blocks;
+    int block = (int)blockIdx.x, chunk = 0;
+    if (chunks > 1) {
+        const int per_chunk = (int)gridDim.x / chunks, whole = per_chunk / 8 * 8, rest = per_chunk - whole;
+        if (block < whole * chunks) {
+            chunk = (block >> 3) % chunks;
+            block = block / (8 * chunks) * 8 + (block & 7);
+        } else {
+            const int t = block - whole * chunks;
+            chunk = t / rest;
+            block = whole + t % rest;
+        }
+    }
+    const int m0 = chunk * chunk_rows, m_end = min(M, m0 + chunk_rows);
+    const bool second = block >= first_blocks;
     void* __restrict__ y = second ? pb.y : pa.y;
     float* __restrict__ part = second ? pb.part : pa.part;
     const bf16_t* __restrict__ x = second ? pb.x : pa.x;
@@ -76,7 +95,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_splitk_kernel(SplitkProblem p
     const int out_f32 = second ? pb.out_f32 : pa.out_f32, direct = second ? pb.direct : pa.direct;
     const int blocks_per_part = second ? pb.blocks_per_part : pa.blocks_per_part;
     const int tiles = second ? pb.tiles : pa.tiles;
-    const int idx = (int)blockIdx.x - (second ? first_blocks : 0);
+    const int idx = block - (second ? first_blocks : 0);
     const int tile = idx % tiles, range = idx / tiles;  // neighbours share a range of K: its x slice stays in L2
     const int n_base = tile * (64 * RT) + wave * (16 * RT);
     const int nkb = (K + 63) >> 6;
@@ -99,8 +118,8 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_splitk_kernel(SplitkProblem p
         const int k_stage = k_begin + stage * KS;
 #pragma unroll
         for (int j = 0; j < PIECES; ++j) {
-            const int q = tid + j * SK_THREADS, row = q / (KS / 8), k = k_stage + (q % (KS / 8)) * 8;
-            const int off = (k < k_end && row < M) ? (row * K + k) * 2 : 0x7ffffff0;
+            const int q = tid + j * SK_THREADS, row = m0 + q / (KS / 8), k = k_stage + (q % (KS / 8)) * 8;
+            const int off = (k < k_end && row < m_end) ? (row * K + k) * 2 : 0x7ffffff0;
             xr[j] = __builtin_amdgcn_raw_buffer_load_b128(xres, off, 0, 0);
         }
     };
@@ -166,8 +185,8 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_splitk_kernel(SplitkProblem p
     for (int t = 0; t < RT; ++t)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-            const int m = mt * 16 + r, n = n_base + t * 16 + g * 4;
-            if (m >= M || n >= N) continue;
+            const int m = m0 + mt * 16 + r, n = n_base + t * 16 + g * 4;
+            if (m >= m_end || n >= N) continue;
             const long o = (long)m * N + n;
             if (!direct) {
                 const long at = (long)range * M * N + o;
@@ -292,8 +311,10 @@ static int launch_cfg(const SplitkProblem& a, const SplitkProblem& b, int M, int
             raised = true;
         }
     }
-    const dim3 grid(a.tiles * a.parts + b.tiles * b.parts);
-    hipLaunchKernelGGL(kern, grid, dim3(SK_THREADS), lds, s, a, b, M);
+    // rows beyond the MT tiles of a workgroup go to further chunks of workgroups, all of the same size
+    const int chunks = (M + MT * 16 - 1) / (MT * 16), chunk_rows = ((M + chunks - 1) / chunks + 15) / 16 * 16;
+    const dim3 grid((a.tiles * a.parts + b.tiles * b.parts) * chunks);
+    hipLaunchKernelGGL(kern, grid, dim3(SK_THREADS), lds, s, a, b, M, chunks, chunk_rows);
     if (reduce && a.parts > 1) {
         const long MN = (long)M * a.N;
         hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((MN + 255) / 256)), dim3(256), 0, s, a.y, a.part,
@@ -302,19 +323,33 @@ static int launch_cfg(const SplitkProblem& a, const SplitkProblem& b, int M, int
     return pta_check_launch("gemm_splitk_bf16");
 }
 
+// sixteen-row tiles of x that a workgroup holds: all rows up to SK_CHUNK_ROWS, else an even share of them
+static int tiles_per_chunk(int M) {
+    const int chunks = (M + SK_CHUNK_ROWS - 1) / SK_CHUNK_ROWS;
+    return ((M + chunks - 1) / chunks + 15) / 16;
+}
+
 template <int RT, int U, int D>
 static int launch_rows(int MT, const SplitkProblem& a, const SplitkProblem& b, int M, int reduce, hipStream_t s) {
     switch (MT) {
         case 1: return launch_cfg<1, RT, U, D>(a, b, M, reduce, s);
         case 2: return launch_cfg<2, RT, U, D>(a, b, M, reduce, s);
         case 3: return launch_cfg<3, RT, U, D>(a, b, M, reduce, s);
-        default: return launch_cfg<4, RT, U, D>(a, b, M, reduce, s);
+        case 4: return launch_cfg<4, RT, U, D>(a, b, M, reduce, s);
+        default:
+            // 65 to 128 rows: two stages in flight only (four would not fit the registers)
+            if constexpr (D == 2) {
+                if (MT <= 6) return launch_cfg<6, RT, U, D>(a, b, M, reduce, s);
+                return launch_cfg<8, RT, U, D>(a, b, M, reduce, s);
+            } else {
+                return pta_fail("gemm_splitk_bf16: more than 64 rows run with two stages in flight, not %d", D);
+            }
     }
 }
 
 static int check_splitk(const char* what, const void* x, const void* W, int M, int N, int K) {
     PTA_REQUIRE(M > 0 && N > 0 && K > 0, "%s: sizes must be positive (M=%d N=%d K=%d)", what, M, N, K);
-    PTA_REQUIRE(M <= 64, "%s: at most 64 rows, got %d (use the library product)", what, M);
+    PTA_REQUIRE(M <= SK_MAX_ROWS, "%s: at most %d rows, got %d (use the library product)", what, SK_MAX_ROWS, M);
     PTA_REQUIRE(K % 8 == 0 && K >= 8, "%s: K=%d must be a multiple of 8 (16-byte loads)", what, K);
     PTA_REQUIRE(x && W, "%s: null pointer", what);
     PTA_REQUIRE((long)M * K * 2 < 0x7ffffff0L, "%s: x is too large for 32-bit buffer offsets", what);
@@ -335,12 +370,12 @@ extern "C" int pta_gemm_splitk_bf16(void* y, float* part, const void* x, const v
     PTA_REQUIRE(parts >= 0 && parts <= 64, "gemm_splitk_bf16: parts must be 0 (choose) or 1..64, got %d", parts);
     if (rt == 0) rt = pick_rt(N);
     if (parts == 0) parts = pick_parts(N, K, rt);
-    if (depth == 0) depth = 2;  // measured: more stages in flight per wave do not pay, more workgroups do
+    if (depth == 0 || M > 64) depth = 2;  // measured: more stages in flight per wave do not pay, more workgroups do
     const SplitkProblem a = make_problem(y, part, x, W, bias, add1, add2, N, K, act, out_f32, rt, parts, reduce);
     PTA_REQUIRE(a.direct || part, "gemm_splitk_bf16: %d ranges of K need the workspace for partial sums", a.parts);
     const SplitkProblem none{};
     hipStream_t s = (hipStream_t)stream;
-    const int MT = (M + 15) / 16;
+    const int MT = tiles_per_chunk(M);
     if (rt == 1 && depth == 2) return launch_rows<1, 2, 2>(MT, a, none, M, reduce, s);
     if (rt == 1) return launch_rows<1, 2, 4>(MT, a, none, M, reduce, s);
     if (depth == 2) return launch_rows<2, 2, 2>(MT, a, none, M, reduce, s);
@@ -380,7 +415,7 @@ extern "C" int pta_gemm_splitk_pair_bf16(float* part1, const void* x1, const voi
     pick_pair_parts(N1, K1, N2, K2, &p1, &p2);
     const SplitkProblem a = make_problem(nullptr, part1, x1, W1, nullptr, nullptr, nullptr, N1, K1, 0, 0, 1, p1, 0);
     const SplitkProblem b = make_problem(nullptr, part2, x2, W2, nullptr, nullptr, nullptr, N2, K2, 0, 0, 1, p2, 0);
-    return launch_rows<1, 2, 2>((M + 15) / 16, a, b, M, 0, (hipStream_t)stream);
+    return launch_rows<1, 2, 2>(tiles_per_chunk(M), a, b, M, 0, (hipStream_t)stream);
 }
 
 // The same pair run to the end: y1 = act1(x1 . W1^T + bias1), y2 = act2(x2 . W2^T + bias2) in bfloat16; the two

@@ -84,7 +84,7 @@ int pta_gemm_skinny_pair_bf16(void* y1, const void* x1, const void* W1, const fl
                               const void* x2, const void* W2, const float* bias2, int N2, int act2, int M, int K,
                               void* stream);
 
-// The same product for a batch of up to 64 rows that shares x through LDS and may split K over workgroups:
+// The same product for a batch of up to 128 rows that shares x through LDS and may split K over workgroups:
 // `part` is a 32-bit workspace [parts, M, N], needed when parts > 1 or reduce = 0.  rt (row tiles per wave),
 // parts, stage_blocks (64-element blocks of K per stage) and depth (stages in flight) are tuning knobs (0:
 // chosen from N and K alone); pta_gemm_splitk_parts tells the number of ranges that choice gives.

@@ -410,6 +410,70 @@ def sample(logits: torch.Tensor, *, do_sample: bool, temperature: float = 1.0, t
 
 
 SKINNY_MAX_ROWS = 64
+# rows up to which the decode batch kernel (x shared through LDS, K split over workgroups) stands in for the
+# vendor library's product, whose choices for 65 to 128 rows leave most of the chip idle (Falcon-7B sizes, 128
+# rows: 10.4 ms a step with the library)
+SPLITK_MAX_ROWS = int(os.environ.get("PTA_SPLITK_MAX_ROWS", "256"))
+SPLITK_MARGIN = float(os.environ.get("PTA_SPLITK_MARGIN", "0.95"))
+SPLITK_SURE_ROWS = 128  # up to here the kernel won at every shape measured; beyond, by the weight's own timing
+_splitk_limits: dict = {}  # (N, K) -> rows up to which the batch kernel beats the library's product
+
+
+def splitk_row_limit(*ws: torch.Tensor) -> int:
+    """Rows up to which the decode batch kernel is the faster way to the product with ``w`` (or, for two weights, to
+    the two products of a pair launch).  Up to 128 rows it always was (one chunk of rows per workgroup); with two
+    chunks it depends on how well the library does at the shape (at 256 rows it wins at Falcon-7B shapes, 9.5
+    against 11.4 ms a step, and loses at Falcon2-11B shapes, 22.1 against 20.2), so both are timed once per shape
+    at 192 and 256 rows."""
+    if SPLITK_MAX_ROWS <= SPLITK_SURE_ROWS:
+        return SPLITK_MAX_ROWS
+    key = tuple(tuple(w.shape) for w in ws)
+    limit = _splitk_limits.get(key)
+    if limit is None:
+        if torch.cuda.is_current_stream_capturing():
+            return SPLITK_SURE_ROWS  # nothing can be timed now; the next eager step decides
+        dev = ws[0].device
+        xs = [torch.randn((256, w.shape[1]), dtype=torch.float32, device=dev).to(torch.bfloat16) for w in ws]
+        outs = [torch.empty((256, w.shape[0]), dtype=torch.bfloat16, device=dev) for w in ws]
+        limit = SPLITK_SURE_ROWS
+        for rows in (192, 256):
+            if rows > SPLITK_MAX_ROWS:
+                break
+            xr = [x[:rows] for x in xs]
+
+            def kernel():
+                if len(ws) == 1:
+                    gemm_splitk_bf16(xr[0], ws[0])
+                else:
+                    gemm_splitk_pair_bf16(xr[0], ws[0], xr[1], ws[1])
+
+            def library():
+                for x, w, out in zip(xr, ws, outs):
+                    torch.mm(x, w.t(), out=out[:rows])
+
+            ways = (kernel, library)
+            best = [float("inf"), float("inf")]
+            for run in ways:
+                run()
+            for _ in range(4):
+                for i, run in enumerate(ways):
+                    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    start.record()
+                    run()
+                    end.record()
+                    end.synchronize()
+                    best[i] = min(best[i], start.elapsed_time(end))
+            if best[0] < SPLITK_MARGIN * best[1]:
+                limit = rows
+            else:
+                break
+        _splitk_limits[key] = limit
+    return limit
+
+
+def _splitk_rows(x: torch.Tensor, *ws: torch.Tensor) -> bool:
+    return x.shape[0] <= SPLITK_SURE_ROWS or x.shape[0] <= splitk_row_limit(*ws)
+
 
 # ---- the vendor library's product for many rows, cut along M where that is faster -----------------------
 # The library picks a kernel per (M, N, K) from a table, and on this hardware its choices are uneven in M:
@@ -540,7 +604,7 @@ def gemm_skinny_pair_bf16(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tensor, 
 def gemm_splitk_bf16(x: torch.Tensor, w: torch.Tensor, bias=None, act=None, add1=None, add2=None,
                      out_f32: bool = False, rt: int = 0, parts: int = 0, stage_blocks: int = 0,
                      depth: int = 0) -> torch.Tensor:
-    """act(x @ w.T + bias) + add1 + add2 for a batch of at most 64 rows of bfloat16: x shared through LDS,
+    """act(x @ w.T + bias) + add1 + add2 for a batch of at most 128 rows of bfloat16: x shared through LDS,
     K split over workgroups where N gives too few of them."""
     _need(x, "x", torch.bfloat16)
     _need(w, "w", torch.bfloat16)
@@ -604,7 +668,7 @@ def gemm_splitk_pair_partial(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tenso
 
 def gemm_splitk_pair_bf16(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tensor, w2: torch.Tensor, bias1=None, act1=None,
                           bias2=None, act2=None):
-    """(act1(x1 @ w1.T + bias1), act2(x2 @ w2.T + bias2)) for a batch of up to 64 rows: one matrix launch for
+    """(act1(x1 @ w1.T + bias1), act2(x2 @ w2.T + bias2)) for a batch of up to 128 rows: one matrix launch for
     both products and one launch that adds their partial sums."""
     for name, t in (("x1", x1), ("w1", w1), ("x2", x2), ("w2", w2)):
         _need(t, name, torch.bfloat16)
@@ -629,17 +693,18 @@ def gemm_splitk_pair_bf16(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tensor, 
 
 
 def gemm_partial_pair_ok(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tensor, w2: torch.Tensor) -> bool:
-    """Whether two products onto the same features are best left as partial sums of one launch: up to 64
+    """Whether two products onto the same features are best left as partial sums of one launch: up to 128
     rows each, and at least one of them worth leaving so on its own."""
-    return (_bf16_rows_ok(x1, w1) and _bf16_rows_ok(x2, w2) and 0 < x1.shape[0] == x2.shape[0] <= SKINNY_MAX_ROWS
+    return (_bf16_rows_ok(x1, w1) and _bf16_rows_ok(x2, w2) and 0 < x1.shape[0] == x2.shape[0] <= SPLITK_MAX_ROWS
+            and _splitk_rows(x1, w1, w2)
             and w1.shape[0] == w2.shape[0] and w1.shape[0] % 8 == 0
             and (gemm_partial_ok(x1, w1) or gemm_partial_ok(x2, w2)))
 
 
 def gemm_partial_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
-    """Whether leaving x @ w.T as partial sums for the next norm pays: up to 64 rows, and either K long against
+    """Whether leaving x @ w.T as partial sums for the next norm pays: up to 128 rows, and either K long against
     N (any batch: the kernel for few rows has too few row tiles there) or a batch past 16 rows."""
-    if not (_bf16_rows_ok(x, w) and 0 < x.shape[0] <= SKINNY_MAX_ROWS and w.shape[0] % 8 == 0):
+    if not (_bf16_rows_ok(x, w) and 0 < x.shape[0] <= SPLITK_MAX_ROWS and w.shape[0] % 8 == 0 and _splitk_rows(x, w)):
         return False
     return w.shape[1] >= 2 * w.shape[0] or (x.shape[0] > 16 and w.shape[0] < 2 * w.shape[1])
 
@@ -716,16 +781,19 @@ def gemm_skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
     return _bf16_rows_ok(x, w) and 0 < x.shape[0] <= 16
 
 
-def gemm_splitk_rows_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
-    """Whether the kernel for a decode batch takes this product at all (17 to 64 rows of bfloat16, K % 8 == 0)."""
-    return _bf16_rows_ok(x, w) and 16 < x.shape[0] <= SKINNY_MAX_ROWS
+def gemm_splitk_pair_ok(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tensor, w2: torch.Tensor) -> bool:
+    """Whether the two products run as a pair launch of the decode batch kernel (17 to 256 rows; beyond 128 only
+    where the pair was timed faster than the library's two products)."""
+    return (_bf16_rows_ok(x1, w1) and _bf16_rows_ok(x2, w2) and 16 < x1.shape[0] == x2.shape[0] <= SPLITK_MAX_ROWS
+            and _splitk_rows(x1, w1, w2))
 
 
 def gemm_splitk_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
-    """Whether the kernel for a decode batch of 17 to 64 rows is the faster choice.  Measured at Falcon-7B
+    """Whether the kernel for a decode batch of 17 to 128 rows is the faster choice.  Measured at Falcon-7B
     shapes: it beats the vendor library except where N is long against K (the feed-forward's first matrix
     and the output head), which give the library enough row tiles to fill the chip."""
-    return _bf16_rows_ok(x, w) and 16 < x.shape[0] <= SKINNY_MAX_ROWS and w.shape[0] < 2 * w.shape[1]
+    return (_bf16_rows_ok(x, w) and 16 < x.shape[0] <= SPLITK_MAX_ROWS and w.shape[0] < 2 * w.shape[1]
+            and _splitk_rows(x, w))
 
 
 def gemm_skinny_bf16(x: torch.Tensor, w: torch.Tensor, bias=None, act=None, add1=None, add2=None,

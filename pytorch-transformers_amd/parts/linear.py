@@ -4,9 +4,10 @@
 storage type, as the reference does on purpose
 (src/transformers/models/falcon/modeling_falcon.py:64-72).  In 32-bit the whole
 layer, with activation and residual additions, is one hand-written kernel with a
-fixed summation order.  In bfloat16, steps of at most 64 tokens (decoding) run a
-hand-written kernel that streams the weights once and applies bias, activation
-and additions in its epilogue; larger steps use the vendor library's matrix
+fixed summation order.  In bfloat16, steps of at most 128 tokens (decoding, short
+prompts), and up to 256 where that was timed faster, run a hand-written kernel
+that streams the weights once and applies bias, activation and additions in its
+epilogue; larger steps use the vendor library's matrix
 product (as the reference uses torch's), followed by one fused kernel for bias,
 activation and additions.
 """
@@ -21,7 +22,7 @@ from ..engine.spec import INIT_NORMAL, INIT_ZERO_NOISE, MATRIX, VECTOR, TensorSp
 from .base import PartialProduct, Part
 
 
-PAIR_MAX_WEIGHTS = 160 * 1024 * 1024  # elements of both matrices of a pair launch at 49 to 64 rows
+PAIR_MAX_WEIGHTS = 160 * 1024 * 1024  # elements of both matrices of a pair launch beyond 48 rows
 
 
 class Linear(Part):
@@ -91,7 +92,7 @@ class Linear(Part):
         args = (x1, first.weight, x2, second.weight, b1, kw1.get("act"), b2, kw2.get("act"))
         if x1.shape == x2.shape and ops.gemm_skinny_ok(x1, first.weight) and ops.gemm_skinny_ok(x2, second.weight):
             return ops.gemm_skinny_pair_bf16(*args)
-        if (x1 is x2 and x1.shape[0] > ops.SKINNY_MAX_ROWS and first.joined is not None and first.joined[1] is second
+        if (x1 is x2 and x1.shape[0] > ops.SPLITK_MAX_ROWS and first.joined is not None and first.joined[1] is second
                 and ops.joined_mm_pays(x1, first.joined[0], first.out_features)):
             # many rows, one input, the matrices side by side in memory: one library product where it was measured
             # faster than two; the results are blocks of columns of its output, each with its own epilogue
@@ -101,11 +102,11 @@ class Linear(Part):
                 if bias is not None or act is not None:
                     ops.epilogue_(yi, bias, act)
             return y1, y2
-        # 17 to 64 rows: measured at Falcon-7B and Falcon2-11B sizes the pair beats the products on their own; at
+        # 17 rows and more: measured at Falcon-7B and Falcon2-11B sizes the pair beats the products on their own; at
         # Falcon-40B sizes it does up to 48 rows (32 rows: 20.8 against 23.0 ms a step), beyond them the vendor
         # library's product for the feed-forward input is the faster one (64 rows: 23.3 against 24.3 ms)
         small = x1.shape[0] <= 48 or first.weight.numel() + second.weight.numel() <= PAIR_MAX_WEIGHTS
-        if small and ops.gemm_splitk_rows_ok(x1, first.weight) and ops.gemm_splitk_rows_ok(x2, second.weight):
+        if small and ops.gemm_splitk_pair_ok(x1, first.weight, x2, second.weight):
             return ops.gemm_splitk_pair_bf16(*args)
         return None
 

@@ -97,7 +97,7 @@ def test_gemm_skinny_bf16(M, N, K):
     assert torch.equal(alone, got32[r:r + 1])
 
 
-@pytest.mark.parametrize("M", [1, 9, 17, 32, 33, 50, 64])
+@pytest.mark.parametrize("M", [1, 9, 17, 32, 33, 50, 64, 65, 81, 96, 100, 128, 129, 200, 256])
 @pytest.mark.parametrize("N,K,parts,rt,sb,depth", [(16, 64, 0, 0, 0, 0), (100, 200, 0, 0, 0, 0), (100, 200, 3, 2, 2, 2),
                                                    (4544, 4544, 0, 0, 0, 0), (250, 18176 // 4, 5, 1, 2, 4),
                                                    (1000, 1096, 1, 2, 2, 4), (333, 2056, 4, 1, 2, 2)])
@@ -227,7 +227,7 @@ def test_gemm_skinny_pair():
 def test_gemm_splitk_pair():
     """Two products of one launch, run to the end, against the products on their own."""
     ops = _ops()
-    M, K1, K2, N1, N2 = 40, 328, 264, 100, 530
+    M, K1, K2, N1, N2 = 100, 328, 264, 100, 530
     x1, x2 = _rand(M, K1, dtype=torch.bfloat16), _rand(M, K2, seed=5, dtype=torch.bfloat16)
     w1, w2 = _rand(N1, K1, seed=1, dtype=torch.bfloat16, scale=0.05), _rand(N2, K2, seed=2, dtype=torch.bfloat16, scale=0.05)
     b2 = _rand(N2, seed=3)
@@ -265,13 +265,14 @@ def test_library_mm_in_pieces():
 
 def test_gemm_skinny_refuses_what_it_cannot_do():
     ops = _ops()
-    x, w = _rand(65, 64, dtype=torch.bfloat16), _rand(32, 64, dtype=torch.bfloat16)
+    x, w = _rand(257, 64, dtype=torch.bfloat16), _rand(32, 64, dtype=torch.bfloat16)
     assert not ops.gemm_skinny_ok(x, w) and not ops.gemm_splitk_ok(x, w)
     assert ops.gemm_splitk_ok(x[:17].contiguous(), w) and not ops.gemm_splitk_ok(x[:16].contiguous(), w)
-    with pytest.raises(ops.KernelError, match="at most 64 rows"):
+    assert ops.gemm_splitk_ok(x[:ops.SPLITK_MAX_ROWS].contiguous(), w)
+    with pytest.raises(ops.KernelError, match="at most 256 rows"):
         ops.gemm_splitk_bf16(x, w)
     with pytest.raises(ops.KernelError, match="at most 64 rows"):
-        ops.gemm_skinny_bf16(x, w)
+        ops.gemm_skinny_bf16(x[:65].contiguous(), w)
     x, w = _rand(4, 60, dtype=torch.bfloat16), _rand(32, 60, dtype=torch.bfloat16)
     assert not ops.gemm_skinny_ok(x, w)
     with pytest.raises(ops.KernelError, match="multiple of 8"):

@@ -127,6 +127,33 @@ def test_joined_matrices_give_one_product_for_many_rows(monkeypatch):
     assert ops.joined_mm_pays(x, first.joined[0], N1) in (True, False)  # measured, either way
 
 
+def test_rows_beyond_one_chunk_take_the_way_that_was_timed_faster(monkeypatch):
+    """129 to 256 rows: the decode batch kernel (two chunks of rows per launch) or the library's product, by a
+    timing per weight shape; both ways give the plain result, alone and as a pair launch."""
+    from pytorch_transformers_amd import ops
+    from pytorch_transformers_amd.parts import Linear
+
+    H, N1, N2, M = 264, 136, 200, 200
+    first, second = Linear("a", H, N1, bias=True), Linear("b", H, N2, bias=False)
+    (_, r1), (_, r2) = _fill(first, torch.bfloat16, 1), _fill(second, torch.bfloat16, 2)
+    x = _rand(M, H, seed=3).bfloat16().cuda()
+    want1 = P.linear(x.double().cpu(), r1["a.weight"], r1["a.bias"])
+    want2 = P.gelu(x.double().cpu() @ r2["b.weight"].T)
+    assert ops.splitk_row_limit(first.weight) in (128, 192, 256)  # measured, whichever
+    for limit in (256, 128):
+        monkeypatch.setattr(ops, "splitk_row_limit", lambda *ws: limit)
+        assert ops.gemm_splitk_ok(x, first.weight) == (limit == 256)
+        _close(first(x), want1, 2e-2, f"alone, limit {limit}")
+        both = Linear.pair(first, x, {}, second, x, {"act": "gelu"})
+        assert (both is not None) == (limit == 256)
+        if both is not None:
+            _close(both[0], want1, 2e-2, "first of the pair")
+            _close(both[1], want2, 2e-2, "second of the pair")
+    # at 128 rows and below nothing is timed: the kernel takes them
+    monkeypatch.setattr(ops, "splitk_row_limit", lambda *ws: 1 / 0)
+    assert ops.gemm_splitk_ok(x[:128].contiguous(), first.weight)
+
+
 def test_positions():
     from pytorch_transformers_amd.parts import AlibiPositions, NoPositions, RotaryPositions
 
