@@ -252,6 +252,20 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce2_kernel(bf16_t* __rest
     (second ? y2 : y1)[o] = f32_to_bf16_bits(v);
 }
 
+// The reduction on its own, for partial sums that something else made (the vendor library's batched product
+// over ranges of K): y[M, N] = act(sum over part[P, M, N] in order + bias) + add1 + add2.
+extern "C" int pta_gemm_reduce_parts(void* y, const float* part, const float* bias, const void* add1, const void* add2,
+                                     int M, int N, int P, int act, int out_f32, void* stream) {
+    PTA_REQUIRE(M > 0 && N > 0 && P > 0, "gemm_reduce_parts: sizes must be positive (M=%d N=%d P=%d)", M, N, P);
+    PTA_REQUIRE(y && part, "gemm_reduce_parts: null pointer");
+    PTA_REQUIRE(act == PTA_ACT_NONE || act == PTA_ACT_GELU, "gemm_reduce_parts: unknown activation %d", act);
+    const long MN = (long)M * N;
+    PTA_REQUIRE((MN + 255) / 256 < (1L << 31), "gemm_reduce_parts: too many elements for one launch");
+    hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((MN + 255) / 256)), dim3(256), 0, (hipStream_t)stream, y,
+                       part, bias, (const bf16_t*)add1, (const bf16_t*)add2, MN, N, P, act, out_f32);
+    return pta_check_launch("gemm_reduce_parts");
+}
+
 static int pick_rt(int N) { return N >= 16384 ? 2 : 1; }
 
 // ranges that are not empty when K is cut into `parts` ranges of whole 64-element blocks

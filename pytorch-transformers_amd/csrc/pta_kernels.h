@@ -97,6 +97,11 @@ int pta_gemm_splitk_parts(int N, int K, int parts, int rt);
 // two products of one launch, both left as partial sums: part1 [parts1, M, N1], part2 [parts2, M, N2], with the
 // ranges pta_gemm_splitk_pair_parts gives
 int pta_gemm_splitk_pair_parts(int N1, int K1, int N2, int K2, int* parts1, int* parts2);
+
+// y[M, N] = act(sum of part[P, M, N] over P, in order, + bias) + add1 + add2: the reduction of the products above
+// on its own, for 32-bit partial sums over ranges of K that the vendor library's batched product made
+int pta_gemm_reduce_parts(void* y, const float* part, const float* bias, const void* add1, const void* add2, int M,
+                          int N, int P, int act, int out_f32, void* stream);
 int pta_gemm_splitk_pair_bf16(float* part1, const void* x1, const void* W1, int N1, int K1, float* part2,
                               const void* x2, const void* W2, int N2, int K2, int M, void* stream);
 

@@ -419,6 +419,26 @@ SPLITK_SURE_ROWS = 128  # up to here the kernel won at every shape measured; bey
 _splitk_limits: dict = {}  # (N, K) -> rows up to which the batch kernel beats the library's product
 
 
+def _time_ways_cold(ways, device, rounds: int = 3):
+    """Milliseconds of each of ``ways`` (callables), the fastest of ``rounds`` runs each, taken in turn; before
+    every run half a gigabyte is written, so that the weights come from memory as they do in a model (timed back
+    to back, a product finds its matrix in the memory-side cache and every way looks alike)."""
+    flush = torch.empty(128 * 1024 * 1024, dtype=torch.float32, device=device)
+    best = [float("inf")] * len(ways)
+    for run in ways:  # plans are made and the library set up before anything is timed
+        run()
+    for _ in range(rounds):
+        for i, run in enumerate(ways):
+            flush.fill_(1.0)
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            run()
+            end.record()
+            end.synchronize()
+            best[i] = min(best[i], start.elapsed_time(end))
+    return best
+
+
 def splitk_row_limit(*ws: torch.Tensor) -> int:
     """Rows up to which the decode batch kernel is the faster way to the product with ``w`` (or, for two weights, to
     the two products of a pair launch).  Up to 128 rows it always was (one chunk of rows per workgroup); with two
@@ -451,18 +471,7 @@ def splitk_row_limit(*ws: torch.Tensor) -> int:
                 for x, w, out in zip(xr, ws, outs):
                     torch.mm(x, w.t(), out=out[:rows])
 
-            ways = (kernel, library)
-            best = [float("inf"), float("inf")]
-            for run in ways:
-                run()
-            for _ in range(4):
-                for i, run in enumerate(ways):
-                    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                    start.record()
-                    run()
-                    end.record()
-                    end.synchronize()
-                    best[i] = min(best[i], start.elapsed_time(end))
+            best = _time_ways_cold((kernel, library), dev)
             if best[0] < SPLITK_MARGIN * best[1]:
                 limit = rows
             else:
@@ -578,6 +587,54 @@ def library_mm(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
         at += rows
     return out
 
+
+
+# ---- the vendor library's product with K cut into a batch ------------------------------------------------
+# Where K is long against N (the feed-forward's second matrix) and the rows are a few hundred, the library's
+# kernel choice has too few tiles of the result to fill the chip: at Falcon-7B shapes 512 rows take 225 us, and
+# 112 us as a batch of two products over the halves of K (32-bit partial sums, added in order by the kernel
+# that also applies bias, activation and additions, so no epilogue launch follows).
+MM_KSPLIT = os.environ.get("PTA_MM_KSPLIT", "1") != "0"
+MM_KSPLIT_MAX_ROWS = 1536  # at 2,048 rows the batch gained nothing alone and lost 3 % in a model (Falcon-40B sizes)
+_mm_ksplit: dict = {}  # (N, K, row bucket) -> ranges of K (1: the plain product)
+
+
+def _k_batch(x: torch.Tensor, w: torch.Tensor, S: int) -> torch.Tensor:
+    M, K = x.shape
+    xb = x.unflatten(1, (S, K // S)).transpose(0, 1)   # [S, M, K/S], rows as far apart as x's
+    wb = w.unflatten(1, (S, K // S)).permute(1, 2, 0)  # [S, K/S, N]
+    return torch.bmm(xb, wb, out_dtype=torch.float32)
+
+
+def library_mm_ksplit(x: torch.Tensor, w: torch.Tensor, bias=None, act=None, add1=None, add2=None):
+    """``act(x @ w.T + bias) + add1 + add2`` through the library's batched product over ranges of K, where that
+    was timed faster than its plain product (once per shape, by 64 rows); else None."""
+    M, (N, K) = x.shape[0], w.shape
+    if (not MM_KSPLIT or K < 2 * N or not (SPLITK_MAX_ROWS < M <= MM_KSPLIT_MAX_ROWS) or K % 32 or x.stride(1) != 1
+            or not w.is_contiguous()):
+        return None
+    key = (N, K, (M + 63) // 64)
+    S = _mm_ksplit.get(key)
+    if S is None:
+        if torch.cuda.is_current_stream_capturing():
+            return None
+        ways = [(1, lambda: library_mm(x, w))] + [(s, (lambda s=s: _k_batch(x, w, s))) for s in (2, 4) if K % (s * 8) == 0]
+        best = _time_ways_cold([run for _, run in ways], x.device)
+        pick = min(range(len(ways)), key=lambda i: best[i])
+        S = ways[pick][0] if best[pick] < 0.9 * best[0] else 1
+        _mm_ksplit[key] = S
+    if S == 1:
+        return None
+    part = _k_batch(x, w, S)
+    if bias is not None:
+        _need(bias, "bias", torch.float32, (N,))
+    for name, a in (("add1", add1), ("add2", add2)):
+        if a is not None:
+            _need(a, name, torch.bfloat16, (M, N))
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    _call("pta_gemm_reduce_parts", _ptr(y), _ptr(part), _ptr(bias), _ptr(add1), _ptr(add2), M, N, S, ACT_CODES[act], 0,
+          _stream())
+    return y
 
 
 def gemm_skinny_pair_bf16(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tensor, w2: torch.Tensor, bias1=None, act1=None,

@@ -74,6 +74,9 @@ class Linear(Part):
             return ops.gemm_skinny_bf16(x, self.weight, bias, act, add1, add2)
         if ops.gemm_splitk_ok(x, self.weight):
             return ops.gemm_splitk_bf16(x, self.weight, bias, act, add1, add2)
+        y = ops.library_mm_ksplit(x, self.weight, bias, act, add1, add2)
+        if y is not None:
+            return y
         y = ops.library_mm(x, self.weight)
         if bias is not None or act is not None or add1 is not None or add2 is not None:
             ops.epilogue_(y, bias, act, add1, add2)

@@ -154,6 +154,34 @@ def test_rows_beyond_one_chunk_take_the_way_that_was_timed_faster(monkeypatch):
     assert ops.gemm_splitk_ok(x[:128].contiguous(), first.weight)
 
 
+def test_library_product_over_ranges_of_k():
+    """A few hundred rows with K long against N: the library's batched product over ranges of K, its 32-bit
+    partial sums added in order by the kernel that applies bias, activation and additions.  Which way is
+    faster is the machine's business, so the ranges are set by hand here; rows of x may lie apart."""
+    from pytorch_transformers_amd import ops
+    from pytorch_transformers_amd.parts import Linear
+
+    K, N, M = 640, 136, 300
+    lin = Linear("a", K, N, bias=True)
+    _, ref = _fill(lin, torch.bfloat16, 1)
+    wide = _rand(M, K + 64, seed=3).bfloat16().cuda()
+    x = wide[:, 64:]  # rows that lie apart, as a block of columns of a joined product
+    a1, a2 = _rand(M, N, seed=4).bfloat16().cuda(), _rand(M, N, seed=5).bfloat16().cuda()
+    want = P.gelu(P.linear(x.double().cpu(), ref["a.weight"], ref["a.bias"])) + a1.double().cpu() + a2.double().cpu()
+    key = (N, K, (M + 63) // 64)
+    try:
+        for S in (2, 4, 1):
+            ops._mm_ksplit[key] = S
+            got = ops.library_mm_ksplit(x, lin.weight, lin.bias, "gelu", a1, a2)
+            assert (got is None) == (S == 1)
+            _close(lin(x, act="gelu", add1=a1, add2=a2), want, 2e-2, f"{S} ranges of K")
+    finally:
+        ops._mm_ksplit.pop(key, None)
+    assert ops.library_mm_ksplit(x[:64], lin.weight) is None  # few rows go to the decode kernels
+    lin(x, act="gelu", add1=a1, add2=a2)  # timed, whichever way
+    assert ops._mm_ksplit.pop(key) in (1, 2, 4)
+
+
 def test_positions():
     from pytorch_transformers_amd.parts import AlibiPositions, NoPositions, RotaryPositions
 
