@@ -96,6 +96,21 @@ def test_decoding_across_the_length_bound_of_a_captured_step(folders, dtype, rel
 
 
 @pytest.mark.parametrize("dtype,rel", [("float32", REL_F32), ("bfloat16", REL_BF16)])
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_a_batch_of_150_sequences_that_thins_out(folders, name, dtype, rel):
+    """150 short requests decode together and leave a few at a time: the steps bring 150, 133, 117, ... 17 rows,
+    through every row count at which the matrix products change kernels (two chunks of rows, one, the kernels
+    for few rows)."""
+    lens = [6 + (7 * i) % 23 for i in range(150)]
+    reqs = helpers.make_requests(TINY[name]["vocab_size"], lens, seed=150)
+    want = helpers.plain_logits(folders[name], reqs)
+    rp = _replayer(folders[name], dtype, max_tokens=150 * 64)
+    got = helpers.run_schedule(rp, helpers.schedule_batches(reqs, 150, decode=(1, 2, 3, 4, 5, 6, 7, 8, 9)))
+    for rid in reqs:
+        helpers.assert_close(got[rid], want[rid], rel, f"{name} {dtype} batch of 150, {rid}")
+
+
+@pytest.mark.parametrize("dtype,rel", [("float32", REL_F32), ("bfloat16", REL_BF16)])
 def test_first_tokens(folders, dtype, rel):
     """The first tokens of a sequence, fed one at a time from an empty slot."""
     reqs = helpers.make_requests(TINY["A"]["vocab_size"], [6], seed=11)
