@@ -23,7 +23,7 @@ NORMS_SINGLE = "single"  # input_layernorm feeds attention and MLP
 NORMS_DUAL = "dual"  # ln_attn feeds attention, ln_mlp feeds the MLP
 NORMS_SEQUENTIAL = "sequential"  # input_layernorm, then post_attention_layernorm on x + attn
 
-ROPE_TYPES_BUILT = ("default", "linear")
+ROPE_TYPES_BUILT = ("default", "linear", "yarn", "llama3")  # the two others change with the length of the sequence
 ROPE_TYPES_KNOWN = ("default", "linear", "dynamic", "yarn", "longrope", "llama3")  # modeling_rope_utils.py:351-358
 
 
@@ -119,10 +119,27 @@ class FalconConfig(ModelConfig):
                     raise ConfigError(f"rope_scaling type {kind!r} is unknown; known: {ROPE_TYPES_KNOWN}")
                 if kind not in ROPE_TYPES_BUILT:
                     raise ConfigError(f"rope_scaling type {kind!r} is not built; built: {ROPE_TYPES_BUILT}")
-                if kind == "linear":
-                    f = self.rope_scaling.get("factor")
-                    if not isinstance(f, (int, float)) or isinstance(f, bool) or f < 1.0:  # modeling_rope_utils.py:392-394
-                        raise ConfigError(f"rope_scaling factor must be a number >= 1, got {f!r}")
+                def number(key, least=None, required=True):
+                    v = self.rope_scaling.get(key)
+                    if v is None and not required:
+                        return
+                    if not isinstance(v, (int, float)) or isinstance(v, bool) or (least is not None and v < least):
+                        raise ConfigError(f"rope_scaling {key} must be a number" + (f" >= {least}" if least is not None else "")
+                                          + f", got {v!r}")
+                if kind in ("linear", "yarn", "llama3"):
+                    number("factor", 1.0)  # modeling_rope_utils.py:392-394, :432-434, :512-514
+                if kind == "yarn":  # :424-450
+                    number("attention_factor", 0.0, required=False)
+                    number("beta_fast", required=False)
+                    number("beta_slow", required=False)
+                    if (self.rope_scaling.get("beta_fast") or 32) < (self.rope_scaling.get("beta_slow") or 1):
+                        raise ConfigError("rope_scaling beta_fast must not be less than beta_slow")
+                if kind == "llama3":  # :505-536
+                    number("low_freq_factor")
+                    number("high_freq_factor")
+                    number("original_max_position_embeddings", 1)
+                    if self.rope_scaling["high_freq_factor"] <= self.rope_scaling["low_freq_factor"]:
+                        raise ConfigError("rope_scaling high_freq_factor must be greater than low_freq_factor")
         elif self.rope_scaling is not None:  # configuration_falcon.py: alibi and rope scaling exclude each other
             raise ConfigError("rope_scaling is not supported together with alibi")
 

@@ -11,9 +11,27 @@ from ..config.falcon import NORMS_DUAL, NORMS_SEQUENTIAL, FalconConfig
 from ..config.registry import register
 from ..parts import (AlibiPositions, AttentionMixer, DenseFeedForward, Embedding, LayerNorm, OutputHead,
                      ParallelBlock, RotaryPositions, SequentialBlock)
+from ..parts.positions import llama3_frequencies, yarn_frequencies
 from .spec import CACHE_FULL, CacheGroupSpec, LayerCall, ModelSpec
 
 KV_GROUP = "kv"
+
+
+def rotary_positions(cfg: FalconConfig) -> RotaryPositions:
+    """The rotation that ``rope_scaling`` asks for (src/transformers/models/falcon/modeling_falcon.py:112-134)."""
+    rs, kind = cfg.rope_scaling or {}, cfg.rope_type
+    if kind == "linear":
+        return RotaryPositions(cfg.head_dim, cfg.rope_theta, scaling_factor=float(rs["factor"]))
+    if kind == "yarn":
+        inv, scale = yarn_frequencies(cfg.head_dim, cfg.rope_theta, float(rs["factor"]), cfg.max_position_embeddings,
+                                      float(rs.get("beta_fast") or 32), float(rs.get("beta_slow") or 1),
+                                      rs.get("attention_factor"))
+        return RotaryPositions(cfg.head_dim, cfg.rope_theta, attention_scaling=scale, inv_freq=inv)
+    if kind == "llama3":
+        inv = llama3_frequencies(cfg.head_dim, cfg.rope_theta, float(rs["factor"]), float(rs["low_freq_factor"]),
+                                 float(rs["high_freq_factor"]), int(rs["original_max_position_embeddings"]))
+        return RotaryPositions(cfg.head_dim, cfg.rope_theta, inv_freq=inv)
+    return RotaryPositions(cfg.head_dim, cfg.rope_theta)
 
 
 def build_falcon(cfg: FalconConfig) -> ModelSpec:
@@ -21,8 +39,7 @@ def build_falcon(cfg: FalconConfig) -> ModelSpec:
     if cfg.alibi:
         positions = AlibiPositions(cfg.num_attention_heads)
     else:
-        factor = float(cfg.rope_scaling["factor"]) if cfg.rope_type == "linear" else 1.0
-        positions = RotaryPositions(cfg.head_dim, cfg.rope_theta, scaling_factor=factor)
+        positions = rotary_positions(cfg)
     blocks = []
     for i in range(L):
         p = f"transformer.h.{i}"

@@ -29,16 +29,26 @@ class RotaryPositions(NoPositions):
     to be (src/transformers/models/falcon/modeling_falcon.py:155-164).
     """
 
-    def __init__(self, head_dim: int, theta: float, scaling_factor: float = 1.0, attention_scaling: float = 1.0):
+    def __init__(self, head_dim: int, theta: float, scaling_factor: float = 1.0, attention_scaling: float = 1.0,
+                 inv_freq: Optional[torch.Tensor] = None):
+        """``inv_freq`` given: a table of ``head_dim / 2`` frequencies of another scheme (``yarn_frequencies``,
+        ``llama3_frequencies``); cosines and sines are multiplied by ``attention_scaling``
+        (src/transformers/models/falcon/modeling_falcon.py:162-166)."""
         if head_dim % 2:
             raise ValueError(f"rotary positions need an even head size, got {head_dim}")
         self.head_dim = head_dim
         self.theta = float(theta)
         self.scaling_factor = float(scaling_factor)
         self.attention_scaling = float(attention_scaling)
-        inv = 1.0 / (self.theta ** (torch.arange(0, head_dim, 2, dtype=torch.int64).float() / head_dim))
-        if self.scaling_factor != 1.0:
-            inv = inv / self.scaling_factor
+        if inv_freq is not None:
+            if tuple(inv_freq.shape) != (head_dim // 2,):
+                raise ValueError(f"a frequency table for head size {head_dim} has {head_dim // 2} entries, got "
+                                 f"{tuple(inv_freq.shape)}")
+            inv = inv_freq.to(torch.float32)
+        else:
+            inv = default_frequencies(head_dim, self.theta)
+            if self.scaling_factor != 1.0:
+                inv = inv / self.scaling_factor
         self.inv_freq = inv.contiguous()
 
     def to(self, device) -> None:
@@ -46,6 +56,49 @@ class RotaryPositions(NoPositions):
 
     def rotation(self):
         return self.inv_freq, self.attention_scaling
+
+
+def default_frequencies(head_dim: int, theta: float) -> torch.Tensor:
+    """``1 / theta^(2i/d)`` in 32-bit (src/transformers/modeling_rope_utils.py:58-68)."""
+    return 1.0 / (float(theta) ** (torch.arange(0, head_dim, 2, dtype=torch.int64).float() / head_dim))
+
+
+def yarn_frequencies(head_dim: int, theta: float, factor: float, max_position_embeddings: int,
+                     beta_fast: float = 32.0, beta_slow: float = 1.0, attention_factor: Optional[float] = None):
+    """YaRN (src/transformers/modeling_rope_utils.py:163-239): frequencies that turn often within the trained
+    context stay, those that turn less than once are divided by ``factor``, and a linear ramp over the pair
+    index blends the two in between; returns (table, factor on cosines and sines)."""
+    scale = 0.1 * math.log(factor) + 1.0 if attention_factor is None else float(attention_factor)
+    half = head_dim // 2
+
+    def pair_with_turns(turns: float) -> float:  # the pair index whose frequency makes `turns` turns in the context
+        return head_dim * math.log(max_position_embeddings / (turns * 2 * math.pi)) / (2 * math.log(theta))
+
+    low = max(math.floor(pair_with_turns(beta_fast)), 0)
+    high = min(math.ceil(pair_with_turns(beta_slow)), head_dim - 1)
+    if low == high:
+        high += 0.001
+    ramp = torch.clamp((torch.arange(half, dtype=torch.float32) - low) / (high - low), 0, 1)
+    keep = 1.0 - ramp  # 1: the frequency as trained, 0: divided by the factor
+    turns_per_pos = theta ** (torch.arange(0, head_dim, 2).float() / head_dim)
+    inv = (1.0 / (factor * turns_per_pos)) * (1 - keep) + (1.0 / turns_per_pos) * keep
+    return inv, scale
+
+
+def llama3_frequencies(head_dim: int, theta: float, factor: float, low_freq_factor: float, high_freq_factor: float,
+                       original_max_position_embeddings: int) -> torch.Tensor:
+    """Llama 3.1's scheme (src/transformers/modeling_rope_utils.py:310-341): wavelengths beyond
+    ``original / low_freq_factor`` are stretched by ``factor``, those under ``original / high_freq_factor`` stay,
+    and in between the two are blended by where the wavelength lies."""
+    inv = default_frequencies(head_dim, theta)
+    wavelen = 2 * math.pi / inv
+    long_from = original_max_position_embeddings / low_freq_factor
+    short_to = original_max_position_embeddings / high_freq_factor
+    out = torch.where(wavelen > long_from, inv / factor, inv)
+    smooth = (original_max_position_embeddings / wavelen - low_freq_factor) / (high_freq_factor - low_freq_factor)
+    blended = (1 - smooth) * out / factor + smooth * out
+    middle = ~(wavelen < short_to) & ~(wavelen > long_from)
+    return torch.where(middle, blended, out)
 
 
 def alibi_slopes(num_heads: int) -> torch.Tensor:

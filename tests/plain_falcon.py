@@ -83,12 +83,53 @@ def rope_inv_freq(head_dim: int, theta: float, factor: float = 1.0):
     return inv / factor if factor != 1.0 else inv
 
 
-def rope_cos_sin(positions, inv_freq, dtype=DT):
+def rope_parameters(c):
+    """(inv_freq, factor on cos and sin) for a configuration's ``rope_scaling``
+    (src/transformers/modeling_rope_utils.py: default :58-68, linear :108, yarn :163-239, llama3 :310-341)."""
+    d = c["hidden_size"] // c["num_attention_heads"]
+    theta = float(c["rope_theta"])
+    rs = c.get("rope_scaling") or {}
+    kind = rs.get("rope_type", rs.get("type", "default"))
+    base = rope_inv_freq(d, theta)
+    if kind == "linear":
+        return base / float(rs["factor"]), 1.0
+    if kind == "yarn":
+        factor, ctx = float(rs["factor"]), c["max_position_embeddings"]
+        scale = rs.get("attention_factor")
+        if scale is None:
+            scale = 0.1 * math.log(factor) + 1.0
+        # pair index at which a frequency makes `rot` rotations over the trained context
+        where = lambda rot: (d * math.log(ctx / (rot * 2 * math.pi))) / (2 * math.log(theta))
+        lo = max(math.floor(where(rs.get("beta_fast") or 32)), 0)
+        hi = min(math.ceil(where(rs.get("beta_slow") or 1)), d - 1)
+        if lo == hi:
+            hi += 0.001
+        out = torch.empty(d // 2)
+        for i in range(d // 2):
+            ramp = min(max((i - lo) / (hi - lo), 0.0), 1.0)  # 0: as trained, 1: interpolated
+            out[i] = float(base[i]) / factor * ramp + float(base[i]) * (1 - ramp)
+        return out, float(scale)
+    if kind == "llama3":
+        factor, lo_f, hi_f = float(rs["factor"]), float(rs["low_freq_factor"]), float(rs["high_freq_factor"])
+        old = rs["original_max_position_embeddings"]
+        out = base.clone()
+        for i in range(d // 2):
+            wavelen = 2 * math.pi / float(base[i])
+            if wavelen > old / lo_f:
+                out[i] = base[i] / factor
+            elif not wavelen < old / hi_f:
+                smooth = (old / wavelen - lo_f) / (hi_f - lo_f)
+                out[i] = (1 - smooth) * base[i] / factor + smooth * base[i]
+        return out, 1.0
+    return base, 1.0
+
+
+def rope_cos_sin(positions, inv_freq, dtype=DT, scale=1.0):
     """angles = position * inv_freq in 32-bit, doubled along the last axis
     (src/transformers/models/falcon/modeling_falcon.py:155-164)."""
     freqs = positions.float()[:, None] * inv_freq.float()[None, :]
     emb = torch.cat((freqs, freqs), dim=-1)
-    return emb.to(dtype).cos(), emb.to(dtype).sin()
+    return (emb.cos() * scale).to(dtype), (emb.sin() * scale).to(dtype)
 
 
 def rotate_half(x):
@@ -169,11 +210,8 @@ def self_attention(x, w, prefix, c, positions):
     if c["alibi"]:
         bias = alibi_bias(nh, x.shape[0], d, x.dtype)
     else:
-        rs = c.get("rope_scaling")
-        factor = 1.0
-        if rs is not None and rs.get("rope_type", rs.get("type")) == "linear":
-            factor = float(rs["factor"])
-        cos, sin = rope_cos_sin(positions, rope_inv_freq(d, float(c["rope_theta"]), factor), x.dtype)
+        inv_freq, scale = rope_parameters(c)
+        cos, sin = rope_cos_sin(positions, inv_freq, x.dtype, scale)
         q, k = apply_rope(q, cos, sin), apply_rope(k, cos, sin)
     o = attention_scores_softmax(q, k, v, bias)
     return linear(o, w[prefix + "dense.weight"], w.get(prefix + "dense.bias"))

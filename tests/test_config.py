@@ -58,7 +58,13 @@ def test_unknown_keys_are_kept_and_round_trip(tmp_path):
     (dict(new_decoder_architecture=True, num_attention_heads=8, num_kv_heads=3, hidden_size=64), "multiple"),
     (dict(activation="relu"), "activation"),
     (dict(hidden_size=66, num_attention_heads=22), "even head size"),
-    (dict(rope_scaling={"rope_type": "yarn", "factor": 2.0}), "not built"),
+    (dict(rope_scaling={"rope_type": "dynamic", "factor": 2.0}), "not built"),
+    (dict(rope_scaling={"rope_type": "longrope", "factor": 2.0}), "not built"),
+    (dict(rope_scaling={"rope_type": "yarn", "factor": 0.5}), "factor"),
+    (dict(rope_scaling={"rope_type": "yarn", "factor": 2.0, "beta_fast": 1.0, "beta_slow": 4.0}), "beta_fast"),
+    (dict(rope_scaling={"rope_type": "llama3", "factor": 8.0}), "low_freq_factor"),
+    (dict(rope_scaling={"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 4.0, "high_freq_factor": 1.0,
+                        "original_max_position_embeddings": 512}), "high_freq_factor"),
     (dict(rope_scaling={"type": "bogus", "factor": 2.0}), "unknown"),
     (dict(rope_scaling={"type": "linear", "factor": 0.5}), "factor"),
     (dict(alibi=True, rope_scaling={"type": "linear", "factor": 2.0}), "alibi"),

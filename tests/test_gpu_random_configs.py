@@ -39,6 +39,12 @@ def draw(seed: int) -> dict:
                tie_word_embeddings=r.random() < 0.7, initializer_range=0.02, **extra)
     if not alibi and r.random() < 0.3:
         cfg["rope_scaling"] = {"rope_type": "linear", "factor": r.choice([2.0, 4.0])}
+    elif not alibi and r.random() < 0.4:
+        cfg["rope_scaling"] = r.choice([
+            {"rope_type": "yarn", "factor": 4.0},
+            {"rope_type": "yarn", "factor": 8.0, "beta_fast": 16.0, "beta_slow": 2.0, "attention_factor": 0.8},
+            {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+             "original_max_position_embeddings": 256}])
     return cfg
 
 

@@ -48,6 +48,54 @@ def test_rope_inv_freq_vector():
     torch.testing.assert_close(P.rope_inv_freq(128, 10000.0, 4.0), inv / 4.0)  # linear scaling (:168-194)
 
 
+YARN_SNAPSHOT = [  # tests/utils/test_modeling_rope_utils.py:235-252: d=128, theta=1e4, context 2048, factor 10
+    1.0000e+00, 8.6596e-01, 7.4989e-01, 6.4938e-01, 5.6234e-01, 4.8697e-01, 4.2170e-01, 3.6517e-01, 3.1623e-01, 2.7384e-01,
+    2.3714e-01, 2.0535e-01, 1.7783e-01, 1.5399e-01, 1.3335e-01, 1.1548e-01, 1.0000e-01, 8.3479e-02, 6.9590e-02, 5.7925e-02,
+    4.8136e-02, 3.9931e-02, 3.3061e-02, 2.7315e-02, 2.2515e-02, 1.8512e-02, 1.5177e-02, 1.2403e-02, 1.0101e-02, 8.1924e-03,
+    6.6143e-03, 5.3120e-03, 4.2400e-03, 3.3599e-03, 2.6396e-03, 2.0520e-03, 1.5746e-03, 1.1882e-03, 8.7713e-04, 6.2810e-04,
+    4.3007e-04, 2.7384e-04, 2.3714e-04, 2.0535e-04, 1.7783e-04, 1.5399e-04, 1.3335e-04, 1.1548e-04, 1.0000e-04, 8.6596e-05,
+    7.4989e-05, 6.4938e-05, 5.6234e-05, 4.8697e-05, 4.2170e-05, 3.6517e-05, 3.1623e-05, 2.7384e-05, 2.3714e-05, 2.0535e-05,
+    1.7783e-05, 1.5399e-05, 1.3335e-05, 1.1548e-05]
+LLAMA3_SNAPSHOT = [  # :372-389: the same, original context 2048, low 1, high 4, factor 10
+    1.0000e+00, 8.6596e-01, 7.4989e-01, 6.4938e-01, 5.6234e-01, 4.8697e-01, 4.2170e-01, 3.6517e-01, 3.1623e-01, 2.7384e-01,
+    2.3714e-01, 2.0535e-01, 1.7783e-01, 1.5399e-01, 1.3335e-01, 1.1548e-01, 1.0000e-01, 8.6596e-02, 7.4989e-02, 6.4938e-02,
+    5.6234e-02, 4.8697e-02, 4.2170e-02, 3.6517e-02, 3.1623e-02, 2.7384e-02, 2.3714e-02, 2.0535e-02, 1.7783e-02, 1.5399e-02,
+    1.3335e-02, 1.0730e-02, 7.7785e-03, 5.6009e-03, 3.9991e-03, 2.8248e-03, 1.9675e-03, 1.3449e-03, 8.9549e-04, 5.7363e-04,
+    3.4539e-04, 2.7384e-04, 2.3714e-04, 2.0535e-04, 1.7783e-04, 1.5399e-04, 1.3335e-04, 1.1548e-04, 1.0000e-04, 8.6596e-05,
+    7.4989e-05, 6.4938e-05, 5.6234e-05, 4.8697e-05, 4.2170e-05, 3.6517e-05, 3.1623e-05, 2.7384e-05, 2.3714e-05, 2.0535e-05,
+    1.7783e-05, 1.5399e-05, 1.3335e-05, 1.1548e-05]
+
+
+def test_yarn_and_llama3_frequencies_against_the_reference_snapshots():
+    """The plain tables and the engine's, both against the vectors the reference's tests hold, and the factor on
+    cosines and sines that yarn asks for (tests/utils/test_modeling_rope_utils.py:262-272, :401-412)."""
+    from pytorch_transformers_amd.parts.positions import llama3_frequencies, yarn_frequencies
+
+    base = dict(hidden_size=4096, num_attention_heads=32, rope_theta=10000.0, max_position_embeddings=2048)
+    yarn = {"rope_type": "yarn", "factor": 10.0, "beta_fast": 32, "beta_slow": 1}
+    l3 = {"rope_type": "llama3", "factor": 10.0, "original_max_position_embeddings": 2048, "low_freq_factor": 1,
+          "high_freq_factor": 4}
+    inv, scale = P.rope_parameters(dict(base, rope_scaling=yarn))
+    torch.testing.assert_close(inv, torch.tensor(YARN_SNAPSHOT), rtol=2e-4, atol=0)
+    assert scale == 0.1 * math.log(10.0) + 1.0
+    assert P.rope_parameters(dict(base, rope_scaling=dict(yarn, attention_factor=0.5)))[1] == 0.5
+    got, got_scale = yarn_frequencies(128, 10000.0, 10.0, 2048)
+    torch.testing.assert_close(got, inv, rtol=1e-6, atol=0)
+    assert got_scale == scale and yarn_frequencies(128, 10000.0, 10.0, 2048, attention_factor=0.5)[1] == 0.5
+    inv, scale = P.rope_parameters(dict(base, rope_scaling=l3))
+    torch.testing.assert_close(inv, torch.tensor(LLAMA3_SNAPSHOT), rtol=2e-4, atol=0)
+    assert scale == 1.0
+    torch.testing.assert_close(llama3_frequencies(128, 10000.0, 10.0, 1, 4, 2048), inv, rtol=1e-6, atol=0)
+    # every frequency lies between the trained one and the trained one divided by the factor (:279-287, :420-430)
+    plain = P.rope_inv_freq(128, 10000.0)
+    for table in (torch.tensor(YARN_SNAPSHOT), torch.tensor(LLAMA3_SNAPSHOT)):
+        assert bool(((table <= plain * (1 + 2e-4)) & (table >= plain / 10.0 * (1 - 2e-4))).all())
+    # a very large beta_fast leaves only the first frequency as trained (:289-298)
+    inv, _ = P.rope_parameters(dict(base, rope_scaling=dict(yarn, beta_fast=1000)))
+    assert float(inv[0]) == 1.0 and bool((inv[1:] < plain[1:]).all())
+    torch.testing.assert_close(inv[-20:], plain[-20:] / 10.0)
+
+
 def test_rope_hand_case_pairs_and_sign():
     """Pairs are (i, i + d/2), not (2i, 2i+1); the lower half gets -sin.  d=4, position 1."""
     x = torch.tensor([[[1.0, 2.0, 3.0, 4.0]]], dtype=D)
