@@ -23,6 +23,10 @@ NORMS_SINGLE = "single"  # input_layernorm feeds attention and MLP
 NORMS_DUAL = "dual"  # ln_attn feeds attention, ln_mlp feeds the MLP
 NORMS_SEQUENTIAL = "sequential"  # input_layernorm, then post_attention_layernorm on x + attn
 
+# src/transformers/activations.py:200-220, all but "laplace"
+ACTIVATIONS_BUILT = ("gelu", "gelu_10", "gelu_fast", "gelu_new", "gelu_python", "gelu_pytorch_tanh", "gelu_accurate",
+                     "leaky_relu", "linear", "mish", "quick_gelu", "relu", "relu2", "relu6", "sigmoid", "silu", "swish",
+                     "tanh")
 ROPE_TYPES_BUILT = ("default", "linear", "yarn", "llama3")  # the two others change with the length of the sequence
 ROPE_TYPES_KNOWN = ("default", "linear", "dynamic", "yarn", "longrope", "llama3")  # modeling_rope_utils.py:351-358
 
@@ -91,8 +95,8 @@ class FalconConfig(ModelConfig):
                 f"num_attention_heads={self.num_attention_heads})")
         if not (self.layer_norm_epsilon > 0):
             raise ConfigError(f"layer_norm_epsilon must be positive, got {self.layer_norm_epsilon!r}")
-        if self.activation != "gelu":
-            raise ConfigError(f"activation {self.activation!r} is not built; only 'gelu' (the exact erf form) is")
+        if self.activation not in ACTIVATIONS_BUILT:
+            raise ConfigError(f"activation {self.activation!r} is not built; built: {ACTIVATIONS_BUILT}")
         if self.num_ln_in_parallel_attn not in (None, 1, 2):
             raise ConfigError(f"num_ln_in_parallel_attn must be None, 1 or 2, got {self.num_ln_in_parallel_attn!r}")
         if self.new_decoder_architecture and not self.parallel_attn:

@@ -13,7 +13,23 @@ enum PtaDtype { PTA_F32 = 0, PTA_BF16 = 1 };
 // fused query_key_value row orders (see config.falcon)
 enum PtaQkvLayout { PTA_QKV_GROUPED = 0, PTA_QKV_TAIL = 1, PTA_QKV_INTERLEAVED = 2 };
 
-enum PtaAct { PTA_ACT_NONE = 0, PTA_ACT_GELU = 1 };
+// activations of an epilogue, by the reference's names (src/transformers/activations.py:200-220)
+enum PtaAct {
+    PTA_ACT_NONE = 0,        // "linear"
+    PTA_ACT_GELU = 1,        // "gelu", "gelu_python": the exact erf form
+    PTA_ACT_GELU_TANH = 2,   // "gelu_new", "gelu_pytorch_tanh", "gelu_fast", "gelu_accurate"
+    PTA_ACT_QUICK_GELU = 3,  // x * sigmoid(1.702 x)
+    PTA_ACT_RELU = 4,
+    PTA_ACT_RELU2 = 5,       // relu(x)^2
+    PTA_ACT_RELU6 = 6,
+    PTA_ACT_SILU = 7,        // "silu", "swish"
+    PTA_ACT_SIGMOID = 8,
+    PTA_ACT_TANH = 9,
+    PTA_ACT_LEAKY_RELU = 10, // slope 0.01
+    PTA_ACT_MISH = 11,       // x * tanh(softplus(x))
+    PTA_ACT_GELU_10 = 12,    // exact GELU clipped to [-10, 10]
+    PTA_ACT_COUNT = 13
+};
 
 typedef uint16_t bf16_t;  // raw bits of a bfloat16
 
@@ -101,11 +117,32 @@ __device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
 // exact GELU, 0.5 x (1 + erf(x / sqrt 2))  (src/transformers/activations.py:59-78)
 __device__ __forceinline__ float gelu_erf(float x) { return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f)); }
 
+// Every activation in 32-bit, rounded once by whoever stores it (src/transformers/activations.py:25-195; softplus
+// with torch's threshold of 20, beyond which it is the identity).
+__device__ __forceinline__ float apply_act(float x, int act) {
+    switch (act) {
+        case PTA_ACT_GELU: return gelu_erf(x);
+        case PTA_ACT_GELU_TANH: return 0.5f * x * (1.0f + tanhf(0.79788456080286535588f * (x + 0.044715f * x * x * x)));
+        case PTA_ACT_QUICK_GELU: return x / (1.0f + expf(-1.702f * x));
+        case PTA_ACT_RELU: return fmaxf(x, 0.f);
+        case PTA_ACT_RELU2: { const float r = fmaxf(x, 0.f); return r * r; }
+        case PTA_ACT_RELU6: return fminf(fmaxf(x, 0.f), 6.f);
+        case PTA_ACT_SILU: return x / (1.0f + expf(-x));
+        case PTA_ACT_SIGMOID: return 1.0f / (1.0f + expf(-x));
+        case PTA_ACT_TANH: return tanhf(x);
+        case PTA_ACT_LEAKY_RELU: return x >= 0.f ? x : 0.01f * x;
+        case PTA_ACT_MISH: return x * tanhf(x > 20.f ? x : log1pf(expf(x)));
+        case PTA_ACT_GELU_10: return fminf(fmaxf(gelu_erf(x), -10.f), 10.f);
+        default: return x;
+    }
+}
+
 // ---- host side ---------------------------------------------------------
 // Entry points return 0 on success; otherwise pta_last_error() holds the reason.
 int pta_fail(const char* fmt, ...);
 int pta_check_launch(const char* what);
 int pta_compute_units();
+static inline bool pta_act_known(int act) { return act >= 0 && act < PTA_ACT_COUNT; }
 
 #define PTA_REQUIRE(cond, ...) \
     do { if (!(cond)) return pta_fail(__VA_ARGS__); } while (0)

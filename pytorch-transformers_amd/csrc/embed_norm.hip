@@ -140,7 +140,7 @@ __global__ void epilogue_kernel(T* __restrict__ y, const float* __restrict__ bia
         T* at = y + (i / N) * ld + i % N;
         float v = Io<T>::ld(at);
         if (bias) v = Io<T>::round(v + bias[i % N]);
-        if (act == PTA_ACT_GELU) v = gelu_erf(v);
+        if (act) v = apply_act(v, act);
         if (add1) v += Io<T>::ld(add1 + i);
         if (add2) v += Io<T>::ld(add2 + i);
         Io<T>::st(at, v);
@@ -170,7 +170,7 @@ __global__ void epilogue_bf16x8_kernel(bf16_t* __restrict__ y, const float* __re
 #pragma unroll
             for (int e = 0; e < 2; ++e) {
                 if (bias) v[e] = round_to_bf16(v[e] + bias[n + 2 * p + e]);
-                if (act == PTA_ACT_GELU) v[e] = gelu_erf(v[e]);
+                if (act) v[e] = apply_act(v[e], act);
                 v[e] += x1[e];  // an absent addend was loaded as zeros
                 v[e] += x2[e];
             }
@@ -184,7 +184,7 @@ extern "C" int pta_epilogue(void* y, int ld_y, const float* bias, const void* ad
                             int act, int dtype, void* stream) {
     PTA_REQUIRE(M > 0 && N > 0, "epilogue: M=%d N=%d must be positive", M, N);
     PTA_REQUIRE(ld_y >= N, "epilogue: rows of %d elements cannot lie %d apart", N, ld_y);
-    PTA_REQUIRE(act == PTA_ACT_NONE || act == PTA_ACT_GELU, "epilogue: unknown activation %d", act);
+    PTA_REQUIRE(pta_act_known(act), "epilogue: unknown activation %d", act);
     if (dtype == PTA_BF16 && N % 8 == 0 && ld_y % 8 == 0 && ((uintptr_t)y % 16) == 0 && ((uintptr_t)add1 % 16) == 0 &&
         ((uintptr_t)add2 % 16) == 0) {
         const long groups = (long)M * N / 8;

@@ -60,7 +60,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(float* __restrict__ C, co
             if (gn >= N) continue;
             float v = acc[i][j];
             if (bias) v += bias[gn];
-            if (act == PTA_ACT_GELU) v = gelu_erf(v);
+            if (act) v = apply_act(v, act);
             const long o = (long)gm * N + gn;
             if (add1) v += add1[o];
             if (add2) v += add2[o];
@@ -73,7 +73,7 @@ extern "C" int pta_gemm_f32(float* C, const float* A, const float* W, const floa
                             const float* add2, int M, int N, int K, int act, void* stream) {
     PTA_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_f32: sizes must be positive (M=%d N=%d K=%d)", M, N, K);
     PTA_REQUIRE(C && A && W, "gemm_f32: null pointer");
-    PTA_REQUIRE(act == PTA_ACT_NONE || act == PTA_ACT_GELU, "gemm_f32: unknown activation %d", act);
+    PTA_REQUIRE(pta_act_known(act), "gemm_f32: unknown activation %d", act);
     const int gy = (M + G_BM - 1) / G_BM, gx = (N + G_BN - 1) / G_BN;
     PTA_REQUIRE(gy <= 65535, "gemm_f32: M=%d is too large for one launch", M);
     hipLaunchKernelGGL(gemm_f32_kernel, dim3(gx, gy), dim3(256), 0, (hipStream_t)stream, C, A, W, bias, add1, add2,

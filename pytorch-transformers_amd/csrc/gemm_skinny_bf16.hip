@@ -164,7 +164,7 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(SkinnyProblem pa, Skin
             if (n < n1) {
                 float v = OutIo<OutT>::round(sum[i]);
                 if (bias) v = OutIo<OutT>::round(v + bias[n]);
-                if (act == PTA_ACT_GELU) v = gelu_erf(v);
+                if (act) v = apply_act(v, act);
                 const long o = (long)m * N + n;
                 if (add1) v += bf16_bits_to_f32(add1[o]);
                 if (add2) v += bf16_bits_to_f32(add2[o]);
@@ -239,7 +239,7 @@ static int check_skinny(const char* what, const void* y, const void* x, const vo
     PTA_REQUIRE(y && x && W, "%s: null pointer", what);
     PTA_REQUIRE((long)M * K * 2 < (1L << 31), "%s: x is too large for 32-bit buffer offsets", what);
     PTA_REQUIRE(((uintptr_t)x % 16) == 0 && ((uintptr_t)W % 16) == 0, "%s: x and W must be 16-byte aligned", what);
-    PTA_REQUIRE(act == PTA_ACT_NONE || act == PTA_ACT_GELU, "%s: unknown activation %d", what, act);
+    PTA_REQUIRE(pta_act_known(act), "%s: unknown activation %d", what, act);
     return 0;
 }
 

@@ -200,7 +200,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_splitk_kernel(SplitkProblem p
                 float v = acc[t][mt][i];
                 if (!out_f32) v = round_to_bf16(v);
                 if (bias) { v += bias[n + i]; if (!out_f32) v = round_to_bf16(v); }
-                if (act == PTA_ACT_GELU) v = gelu_erf(v);
+                if (act) v = apply_act(v, act);
                 if (add1) v += bf16_bits_to_f32(add1[o + i]);
                 if (add2) v += bf16_bits_to_f32(add2[o + i]);
                 if (out_f32) ((float*)y)[o + i] = v;
@@ -222,7 +222,7 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(void* __restric
     const int n = (int)(o % N);
     if (!out_f32) v = round_to_bf16(v);
     if (bias) { v += bias[n]; if (!out_f32) v = round_to_bf16(v); }
-    if (act == PTA_ACT_GELU) v = gelu_erf(v);
+    if (act) v = apply_act(v, act);
     if (add1) v += bf16_bits_to_f32(add1[o]);
     if (add2) v += bf16_bits_to_f32(add2[o]);
     if (out_f32) ((float*)y)[o] = v;
@@ -248,7 +248,7 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce2_kernel(bf16_t* __rest
     for (int p = 1; p < P; ++p) v += part[(long)p * MN + o];
     v = round_to_bf16(v);
     if (bias) v = round_to_bf16(v + bias[(int)(o % N)]);
-    if (act == PTA_ACT_GELU) v = gelu_erf(v);
+    if (act) v = apply_act(v, act);
     (second ? y2 : y1)[o] = f32_to_bf16_bits(v);
 }
 
@@ -258,7 +258,7 @@ extern "C" int pta_gemm_reduce_parts(void* y, const float* part, const float* bi
                                      int M, int N, int P, int act, int out_f32, void* stream) {
     PTA_REQUIRE(M > 0 && N > 0 && P > 0, "gemm_reduce_parts: sizes must be positive (M=%d N=%d P=%d)", M, N, P);
     PTA_REQUIRE(y && part, "gemm_reduce_parts: null pointer");
-    PTA_REQUIRE(act == PTA_ACT_NONE || act == PTA_ACT_GELU, "gemm_reduce_parts: unknown activation %d", act);
+    PTA_REQUIRE(pta_act_known(act), "gemm_reduce_parts: unknown activation %d", act);
     const long MN = (long)M * N;
     PTA_REQUIRE((MN + 255) / 256 < (1L << 31), "gemm_reduce_parts: too many elements for one launch");
     hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((MN + 255) / 256)), dim3(256), 0, (hipStream_t)stream, y,
@@ -376,7 +376,7 @@ extern "C" int pta_gemm_splitk_bf16(void* y, float* part, const void* x, const v
                                     int rt, int parts, int stage_blocks, int depth, int reduce, void* stream) {
     if (check_splitk("gemm_splitk_bf16", x, W, M, N, K)) return 1;
     PTA_REQUIRE(y || !reduce, "gemm_splitk_bf16: null pointer");
-    PTA_REQUIRE(act == PTA_ACT_NONE || act == PTA_ACT_GELU, "gemm_splitk_bf16: unknown activation %d", act);
+    PTA_REQUIRE(pta_act_known(act), "gemm_splitk_bf16: unknown activation %d", act);
     PTA_REQUIRE(rt == 0 || rt == 1 || rt == 2, "gemm_splitk_bf16: row tiles per wave must be 0 (choose), 1 or 2, got %d", rt);
     PTA_REQUIRE(stage_blocks == 0 || stage_blocks == 2,
                 "gemm_splitk_bf16: 64-element blocks per stage must be 0 (choose) or 2, got %d", stage_blocks);
@@ -439,7 +439,7 @@ extern "C" int pta_gemm_splitk_pair_reduced_bf16(void* y1, float* part1, const v
                                                  const void* x2, const void* W2, const float* bias2, int N2, int K2,
                                                  int act2, int M, void* stream) {
     PTA_REQUIRE(y1 && y2, "gemm_splitk_pair_reduced_bf16: null output");
-    PTA_REQUIRE((act1 == PTA_ACT_NONE || act1 == PTA_ACT_GELU) && (act2 == PTA_ACT_NONE || act2 == PTA_ACT_GELU),
+    PTA_REQUIRE(pta_act_known(act1) && pta_act_known(act2),
                 "gemm_splitk_pair_reduced_bf16: unknown activation");
     const int rc = pta_gemm_splitk_pair_bf16(part1, x1, W1, N1, K1, part2, x2, W2, N2, K2, M, stream);
     if (rc) return rc;

@@ -20,7 +20,10 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 F32, BF16 = 0, 1
 QKV_LAYOUT_CODES = {"grouped": 0, "tail": 1, "interleaved": 2}
-ACT_CODES = {None: 0, "none": 0, "gelu": 1}
+# activations by the reference's names (src/transformers/activations.py:200-220) -> codes of csrc/common.h
+ACT_CODES = {None: 0, "none": 0, "linear": 0, "gelu": 1, "gelu_python": 1, "gelu_new": 2, "gelu_pytorch_tanh": 2,
+             "gelu_fast": 2, "gelu_accurate": 2, "quick_gelu": 3, "relu": 4, "relu2": 5, "relu6": 6, "silu": 7, "swish": 7,
+             "sigmoid": 8, "tanh": 9, "leaky_relu": 10, "mish": 11, "gelu_10": 12}
 ABI_VERSION = 1
 
 _lib = None

@@ -1,12 +1,14 @@
 """Feed-forward parts.  ``DenseFeedForward``: ``down(act(up(x)))``, no gate, no experts
-(``FalconMLP`` src/transformers/models/falcon/modeling_falcon.py:565-578; ``gelu`` is the exact erf
-form, src/transformers/activations.py:59-78)."""
+(``FalconMLP`` src/transformers/models/falcon/modeling_falcon.py:565-578).  The activation is one of the
+reference's by name (src/transformers/activations.py:200-220; ``gelu`` is the exact erf form, :59-78), applied
+in 32-bit in the epilogue of the first product."""
 from __future__ import annotations
 
 from typing import Sequence
 
 import torch
 
+from .. import ops
 from .base import Part, StepContext, as_tensor, register_part
 from .linear import Linear, PendingProjection
 
@@ -14,8 +16,8 @@ from .linear import Linear, PendingProjection
 class DenseFeedForward(Part):
     def __init__(self, name: str, hidden_size: int, ffn_size: int, bias: bool, activation: str = "gelu",
                  up_name: str = "dense_h_to_4h", down_name: str = "dense_4h_to_h"):
-        if activation != "gelu":
-            raise ValueError(f"activation {activation!r} is not built; only 'gelu'")
+        if activation not in ops.ACT_CODES:
+            raise ValueError(f"activation {activation!r} is not built; built: {sorted(k for k in ops.ACT_CODES if k)}")
         self.name = name
         self.activation = activation
         self.up = Linear(f"{name}.{up_name}", hidden_size, ffn_size, bias)

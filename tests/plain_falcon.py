@@ -217,10 +217,30 @@ def self_attention(x, w, prefix, c, positions):
     return linear(o, w[prefix + "dense.weight"], w.get(prefix + "dense.bias"))
 
 
-def mlp(x, w, prefix):
-    """FalconMLP (src/transformers/models/falcon/modeling_falcon.py:575-578)."""
+def activation(x, name):
+    """An activation by the reference's name (src/transformers/activations.py:25-195, table :200-220)."""
+    F = torch.nn.functional
+    if name in ("gelu", "gelu_python"):
+        return gelu(x)
+    if name in ("gelu_new", "gelu_accurate", "gelu_pytorch_tanh"):  # :56, :127, :46
+        return 0.5 * x * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (x + 0.044715 * torch.pow(x, 3.0))))
+    if name == "gelu_fast":  # :83
+        return 0.5 * x * (1.0 + torch.tanh(x * 0.7978845608 * (1.0 + 0.044715 * x * x)))
+    if name == "quick_gelu":  # :90
+        return x * torch.sigmoid(1.702 * x)
+    if name == "gelu_10":  # :113
+        return torch.clip(gelu(x), -10, 10)
+    table = {"relu": F.relu, "relu6": F.relu6, "silu": F.silu, "swish": F.silu, "sigmoid": torch.sigmoid,
+             "tanh": torch.tanh, "leaky_relu": F.leaky_relu, "mish": F.mish, "linear": lambda t: t,
+             "relu2": lambda t: torch.square(F.relu(t))}  # :172
+    return table[name](x)
+
+
+def mlp(x, w, prefix, act="gelu"):
+    """FalconMLP (src/transformers/models/falcon/modeling_falcon.py:575-578); ``act`` is the configuration's
+    ``activation`` (:568, ``get_activation``)."""
     u = linear(x, w[prefix + "dense_h_to_4h.weight"], w.get(prefix + "dense_h_to_4h.bias"))
-    return linear(gelu(u), w[prefix + "dense_4h_to_h.weight"], w.get(prefix + "dense_4h_to_h.bias"))
+    return linear(activation(u, act), w[prefix + "dense_4h_to_h.weight"], w.get(prefix + "dense_4h_to_h.bias"))
 
 
 def decoder_layer(x, w, i, c, positions):
@@ -244,7 +264,7 @@ def decoder_layer(x, w, i, c, positions):
                                 w[p + "post_attention_layernorm.bias"], eps)
     if c["new_decoder_architecture"] and c["parallel_attn"] and c["num_ln_in_parallel_attn"] == 1:  # :661-666
         mlp_in = attn_in
-    out = mlp(mlp_in, w, p + "mlp.")
+    out = mlp(mlp_in, w, p + "mlp.", c.get("activation", "gelu"))
     if c["new_decoder_architecture"] or c["parallel_attn"]:  # :673-674
         out = out + attn
     return residual + out  # :676

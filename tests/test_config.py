@@ -56,7 +56,8 @@ def test_unknown_keys_are_kept_and_round_trip(tmp_path):
     (dict(new_decoder_architecture=False, parallel_attn=True, num_ln_in_parallel_attn=2), "num_ln_in_parallel_attn"),
     (dict(new_decoder_architecture=False, multi_query=False, num_kv_heads=2, num_attention_heads=8, hidden_size=64), "multi_query=false"),
     (dict(new_decoder_architecture=True, num_attention_heads=8, num_kv_heads=3, hidden_size=64), "multiple"),
-    (dict(activation="relu"), "activation"),
+    (dict(activation="laplace"), "activation"),
+    (dict(activation="gelu_typo"), "activation"),
     (dict(hidden_size=66, num_attention_heads=22), "even head size"),
     (dict(rope_scaling={"rope_type": "dynamic", "factor": 2.0}), "not built"),
     (dict(rope_scaling={"rope_type": "longrope", "factor": 2.0}), "not built"),

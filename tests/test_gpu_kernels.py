@@ -239,6 +239,29 @@ def test_gemm_splitk_pair():
     assert torch.equal(a1, y1[17:37]) and torch.equal(a2, y2[17:37])
 
 
+def test_every_activation_in_every_epilogue():
+    """The reference's activations by name, in the epilogue of each product kernel and of the library's product,
+    in both types, against the plain table (values out to where relu6 and gelu_10 clip and softplus is linear)."""
+    ops = _ops()
+    M, N, K = 24, 72, 64
+    x = (torch.eye(K)[:M] * 1.0).cuda()  # row m picks column m of W: the product is W's own values
+    grid = torch.linspace(-30.0, 30.0, M * N).reshape(N, M).T.contiguous()  # pre-activations, spread over the rows
+    w = torch.zeros(N, K)
+    w[:, :M] = grid.T
+    for name in sorted(k for k in ops.ACT_CODES if k and k != "none"):
+        want = P.activation(grid.double(), name)
+        got32 = ops.gemm_f32(x, w.cuda(), None, name)
+        torch.testing.assert_close(got32.double().cpu(), want, rtol=2e-6, atol=2e-6, msg=lambda m: f"{name} float32: {m}")
+        xb, wb = x.bfloat16(), w.bfloat16().cuda()
+        wantb = P.activation(w.bfloat16().double().T[:M], name)
+        for what, got in (("few rows", ops.gemm_skinny_bf16(xb[:9].contiguous(), wb, None, name)),
+                          ("batch", ops.gemm_splitk_bf16(xb, wb, None, name)),
+                          ("epilogue", ops.epilogue_(torch.mm(xb, wb.t()), None, name))):
+            rows = got.shape[0]
+            torch.testing.assert_close(got.double().cpu(), wantb[:rows], rtol=1e-2, atol=1e-2,
+                                       msg=lambda m: f"{name} bfloat16 {what}: {m}")
+
+
 def test_library_mm_in_pieces():
     """The vendor library's product cut along M: forced here by made-up timings, since what is faster is the
     machine's business; the pieces cover every row once and the result is the library's."""
@@ -268,7 +291,7 @@ def test_gemm_skinny_refuses_what_it_cannot_do():
     x, w = _rand(257, 64, dtype=torch.bfloat16), _rand(32, 64, dtype=torch.bfloat16)
     assert not ops.gemm_skinny_ok(x, w) and not ops.gemm_splitk_ok(x, w)
     assert ops.gemm_splitk_ok(x[:17].contiguous(), w) and not ops.gemm_splitk_ok(x[:16].contiguous(), w)
-    assert ops.gemm_splitk_ok(x[:ops.SPLITK_MAX_ROWS].contiguous(), w)
+    assert ops.gemm_splitk_ok(x[:ops.SPLITK_SURE_ROWS].contiguous(), w)  # beyond that rows by a timing
     with pytest.raises(ops.KernelError, match="at most 256 rows"):
         ops.gemm_splitk_bf16(x, w)
     with pytest.raises(ops.KernelError, match="at most 64 rows"):

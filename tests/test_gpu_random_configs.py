@@ -45,6 +45,8 @@ def draw(seed: int) -> dict:
             {"rope_type": "yarn", "factor": 8.0, "beta_fast": 16.0, "beta_slow": 2.0, "attention_factor": 0.8},
             {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
              "original_max_position_embeddings": 256}])
+    if r.random() < 0.4:
+        cfg["activation"] = r.choice(["gelu_new", "silu", "relu", "quick_gelu", "gelu_pytorch_tanh", "relu2", "mish", "tanh"])
     return cfg
 
 
