@@ -54,7 +54,7 @@ struct SplitkProblem {
 
 template <int MT, int RT, int U, int D>
 __global__ __launch_bounds__(SK_THREADS) void gemm_splitk_kernel(SplitkProblem pa, SplitkProblem pb, int M, int chunks,
-                                                                 int chunk_rows) {
+                                                                 int chunk_rows, int rot_stride) {
     constexpr int KS = U * 64;                       // elements of K per stage
     constexpr int MP = MT * 16;                      // rows of x, padded to whole tiles
     constexpr int LDW = KS + 8;                      // LDS row stride: 16 bytes of padding keep 16-byte reads off each other's banks
@@ -114,8 +114,19 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_splitk_kernel(SplitkProblem p
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) acc[t][mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
+    // Where a row of W is a power of two long, workgroups that walk the same range of K in step ask the same few
+    // memory channels at the same time (N = 4,096, K = 16,384: a third slower than K = 16,448).  So each walks its
+    // range from a starting stage of its own and wraps round; stages past the last read nothing.  A feature's
+    // order of summation follows from N, K and the launch alone.
+    const int rot = rot_stride > 0 && nstages > 0 ? (int)(((long)tile * rot_stride) % nstages) : 0;
+    auto stage_k = [&](int stage) {
+        if (stage >= nstages) return k_end;
+        int at = stage + rot;
+        at -= at >= nstages ? nstages : 0;
+        return k_begin + at * KS;
+    };
     auto load_x = [&](int stage, i32x4_t(&xr)[PIECES]) {
-        const int k_stage = k_begin + stage * KS;
+        const int k_stage = stage_k(stage);
 #pragma unroll
         for (int j = 0; j < PIECES; ++j) {
             const int q = tid + j * SK_THREADS, row = m0 + q / (KS / 8), k = k_stage + (q % (KS / 8)) * 8;
@@ -131,7 +142,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_splitk_kernel(SplitkProblem p
         }
     };
     auto load_w = [&](int stage, Frag8(&wr)[STEPS][RT]) {
-        const int k_stage = k_begin + stage * KS + g * 8;
+        const int k_stage = stage_k(stage) + g * 8;
 #pragma unroll
         for (int j = 0; j < STEPS; ++j) {
             const int kc = min(k_stage + j * 32, k_end - 8);
@@ -328,7 +339,9 @@ static int launch_cfg(const SplitkProblem& a, const SplitkProblem& b, int M, int
     // rows beyond the MT tiles of a workgroup go to further chunks of workgroups, all of the same size
     const int chunks = (M + MT * 16 - 1) / (MT * 16), chunk_rows = ((M + chunks - 1) / chunks + 15) / 16 * 16;
     const dim3 grid((a.tiles * a.parts + b.tiles * b.parts) * chunks);
-    hipLaunchKernelGGL(kern, grid, dim3(SK_THREADS), lds, s, a, b, M, chunks, chunk_rows);
+    static const int rot_env = getenv("PTA_SPLITK_ROT") ? atoi(getenv("PTA_SPLITK_ROT")) : -1;
+    const int rot_stride = rot_env >= 0 ? rot_env : 1;
+    hipLaunchKernelGGL(kern, grid, dim3(SK_THREADS), lds, s, a, b, M, chunks, chunk_rows, rot_stride);
     if (reduce && a.parts > 1) {
         const long MN = (long)M * a.N;
         hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((MN + 255) / 256)), dim3(256), 0, s, a.y, a.part,
