@@ -175,7 +175,7 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(SkinnyProblem pa, Skin
             if (n < n1) {
                 float v = OutIo<OutT>::round(sum[i]);
                 if (bias) v = OutIo<OutT>::round(v + bias[n]);
-                if (act) v = apply_act(v, act);
+                if (act == PTA_ACT_GELU) v = gelu_erf(v);  // other activations run as a pass of their own
                 const long o = (long)m * N + n;
                 if (add1) v += bf16_bits_to_f32(add1[o]);
                 if (add2) v += bf16_bits_to_f32(add2[o]);
@@ -245,6 +245,8 @@ static int launch_skinny(SkinnyProblem a, SkinnyProblem b, int M, int K, int var
     return pta_check_launch("gemm_skinny_bf16");
 }
 
+static bool in_kernel(int act) { return act == PTA_ACT_NONE || act == PTA_ACT_GELU; }
+
 static int check_skinny(const char* what, const void* y, const void* x, const void* W, int M, int N, int K, int act) {
     PTA_REQUIRE(M > 0 && N > 0 && K > 0, "%s: sizes must be positive (M=%d N=%d K=%d)", what, M, N, K);
     PTA_REQUIRE(M <= 64, "%s: at most 64 rows, got %d (use the library product)", what, M);
@@ -264,8 +266,16 @@ extern "C" int pta_gemm_skinny_bf16(void* y, const void* x, const void* W, const
     PTA_REQUIRE(waves == 0 || (waves >= 1 && waves <= 8 && (waves & (waves - 1)) == 0),
                 "gemm_skinny_bf16: waves per workgroup must be 0 (choose) or a power of two up to 8, got %d", waves);
     hipStream_t s = (hipStream_t)stream;
-    const SkinnyProblem a{y, (const bf16_t*)x, (const bf16_t*)W, bias, (const bf16_t*)add1, (const bf16_t*)add2, N, act, 0};
     const SkinnyProblem none{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0};
+    if (!in_kernel(act)) {
+        // the kernel's epilogue knows the exact GELU only (every activation there would cost it its unrolled
+        // loops): the product with its bias first, then activation and additions as a pass over y
+        PTA_REQUIRE(!out_f32, "gemm_skinny_bf16: activation %d needs a bfloat16 result", act);
+        const SkinnyProblem plain{y, (const bf16_t*)x, (const bf16_t*)W, bias, nullptr, nullptr, N, PTA_ACT_NONE, 0};
+        if (launch_skinny<bf16_t>(plain, none, M, K, variant, waves, s)) return 1;
+        return pta_epilogue(y, N, nullptr, add1, add2, M, N, act, PTA_BF16, stream);
+    }
+    const SkinnyProblem a{y, (const bf16_t*)x, (const bf16_t*)W, bias, (const bf16_t*)add1, (const bf16_t*)add2, N, act, 0};
     if (out_f32) return launch_skinny<float>(a, none, M, K, variant, waves, s);
     return launch_skinny<bf16_t>(a, none, M, K, variant, waves, s);
 }
@@ -278,7 +288,10 @@ extern "C" int pta_gemm_skinny_pair_bf16(void* y1, const void* x1, const void* W
                                          int M, int K, void* stream) {
     if (check_skinny("gemm_skinny_pair_bf16", y1, x1, W1, M, N1, K, act1)) return 1;
     if (check_skinny("gemm_skinny_pair_bf16", y2, x2, W2, M, N2, K, act2)) return 1;
-    const SkinnyProblem a{y1, (const bf16_t*)x1, (const bf16_t*)W1, bias1, nullptr, nullptr, N1, act1, 0};
-    const SkinnyProblem b{y2, (const bf16_t*)x2, (const bf16_t*)W2, bias2, nullptr, nullptr, N2, act2, 0};
-    return launch_skinny<bf16_t>(a, b, M, K, 0, 0, (hipStream_t)stream);
+    const SkinnyProblem a{y1, (const bf16_t*)x1, (const bf16_t*)W1, bias1, nullptr, nullptr, N1, in_kernel(act1) ? act1 : 0, 0};
+    const SkinnyProblem b{y2, (const bf16_t*)x2, (const bf16_t*)W2, bias2, nullptr, nullptr, N2, in_kernel(act2) ? act2 : 0, 0};
+    if (launch_skinny<bf16_t>(a, b, M, K, 0, 0, (hipStream_t)stream)) return 1;
+    if (!in_kernel(act1) && pta_epilogue(y1, N1, nullptr, nullptr, nullptr, M, N1, act1, PTA_BF16, stream)) return 1;
+    if (!in_kernel(act2) && pta_epilogue(y2, N2, nullptr, nullptr, nullptr, M, N2, act2, PTA_BF16, stream)) return 1;
+    return 0;
 }

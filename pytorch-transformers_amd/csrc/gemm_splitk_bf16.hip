@@ -211,7 +211,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_splitk_kernel(SplitkProblem p
                 float v = acc[t][mt][i];
                 if (!out_f32) v = round_to_bf16(v);
                 if (bias) { v += bias[n + i]; if (!out_f32) v = round_to_bf16(v); }
-                if (act) v = apply_act(v, act);
+                if (act == PTA_ACT_GELU) v = gelu_erf(v);  // other activations: see pta_gemm_splitk_bf16
                 if (add1) v += bf16_bits_to_f32(add1[o + i]);
                 if (add2) v += bf16_bits_to_f32(add2[o + i]);
                 if (out_f32) ((float*)y)[o + i] = v;
@@ -398,15 +398,26 @@ extern "C" int pta_gemm_splitk_bf16(void* y, float* part, const void* x, const v
     if (rt == 0) rt = pick_rt(N);
     if (parts == 0) parts = pick_parts(N, K, rt);
     if (depth == 0 || M > 64) depth = 2;  // measured: more stages in flight per wave do not pay, more workgroups do
-    const SplitkProblem a = make_problem(y, part, x, W, bias, add1, add2, N, K, act, out_f32, rt, parts, reduce);
+    SplitkProblem a = make_problem(y, part, x, W, bias, add1, add2, N, K, act, out_f32, rt, parts, reduce);
     PTA_REQUIRE(a.direct || part, "gemm_splitk_bf16: %d ranges of K need the workspace for partial sums", a.parts);
+    // One range of K ends in the matrix kernel itself, whose epilogue knows the exact GELU only (every activation
+    // there would cost it its unrolled loops): another activation, and the additions after it, run as a pass over y.
+    const bool after = a.direct && act != PTA_ACT_NONE && act != PTA_ACT_GELU;
+    if (after) {
+        PTA_REQUIRE(!out_f32, "gemm_splitk_bf16: activation %d needs a bfloat16 result", act);
+        a.act = PTA_ACT_NONE;
+        a.add1 = a.add2 = nullptr;
+    }
     const SplitkProblem none{};
     hipStream_t s = (hipStream_t)stream;
     const int MT = tiles_per_chunk(M);
-    if (rt == 1 && depth == 2) return launch_rows<1, 2, 2>(MT, a, none, M, reduce, s);
-    if (rt == 1) return launch_rows<1, 2, 4>(MT, a, none, M, reduce, s);
-    if (depth == 2) return launch_rows<2, 2, 2>(MT, a, none, M, reduce, s);
-    return launch_rows<2, 2, 4>(MT, a, none, M, reduce, s);
+    int rc;
+    if (rt == 1 && depth == 2) rc = launch_rows<1, 2, 2>(MT, a, none, M, reduce, s);
+    else if (rt == 1) rc = launch_rows<1, 2, 4>(MT, a, none, M, reduce, s);
+    else if (depth == 2) rc = launch_rows<2, 2, 2>(MT, a, none, M, reduce, s);
+    else rc = launch_rows<2, 2, 4>(MT, a, none, M, reduce, s);
+    if (rc || !after) return rc;
+    return pta_epilogue(y, N, nullptr, add1, add2, M, N, act, PTA_BF16, stream);
 }
 
 // Ranges of K for the two products of a pair launch: each by its own length, and more of both if the launch
