@@ -219,7 +219,7 @@ static void launch_cfg(SkinnyProblem a, SkinnyProblem b, int M, int K, int S, hi
     const dim3 grid(a.blocks + b.blocks), block(S * 64);
     const size_t lds = (size_t)S * RT * MT * 64 * sizeof(f32x4_t);
     static const int rot_env = getenv("PTA_SKINNY_ROT") ? atoi(getenv("PTA_SKINNY_ROT")) : -1;
-    const int rot_stride = rot_env >= 0 ? rot_env : 5;
+    const int rot_stride = rot_env >= 0 ? rot_env : (K % 2048 == 0 ? 5 : 0);  // rows a multiple of 4 KB long
     hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, U, OutT>), grid, block, lds, s, a, b, M, K, rot_stride);
 }
 

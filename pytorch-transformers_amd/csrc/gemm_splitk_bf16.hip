@@ -52,7 +52,7 @@ struct SplitkProblem {
     int direct;           // one range and the epilogue in this kernel
 };
 
-template <int MT, int RT, int U, int D>
+template <int MT, int RT, int U, int D, bool ROT>
 __global__ __launch_bounds__(SK_THREADS) void gemm_splitk_kernel(SplitkProblem pa, SplitkProblem pb, int M, int chunks,
                                                                  int chunk_rows, int rot_stride) {
     constexpr int KS = U * 64;                       // elements of K per stage
@@ -118,8 +118,10 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_splitk_kernel(SplitkProblem p
     // memory channels at the same time (N = 4,096, K = 16,384: a third slower than K = 16,448).  So each walks its
     // range from a starting stage of its own and wraps round; stages past the last read nothing.  A feature's
     // order of summation follows from N, K and the launch alone.
-    const int rot = rot_stride > 0 && nstages > 0 ? (int)(((long)tile * rot_stride) % nstages) : 0;
+    // (ROT is a compile-time choice: the wrap costs the other shapes 5 % of this kernel at 17 to 32 rows.)
+    const int rot = ROT && nstages > 0 ? (int)(((long)tile * rot_stride) % nstages) : 0;
     auto stage_k = [&](int stage) {
+        if (!ROT) return k_begin + stage * KS;
         if (stage >= nstages) return k_end;
         int at = stage + rot;
         at -= at >= nstages ? nstages : 0;
@@ -327,20 +329,23 @@ static SplitkProblem make_problem(void* y, float* part, const void* x, const voi
 template <int MT, int RT, int U, int D>
 static int launch_cfg(const SplitkProblem& a, const SplitkProblem& b, int M, int reduce, hipStream_t s) {
     const size_t lds = (size_t)2 * MT * 16 * (U * 64 + 8) * sizeof(bf16_t);
-    auto kern = gemm_splitk_kernel<MT, RT, U, D>;
+    // rows of W a multiple of 4 KB long are the ones that crowd memory channels: there every workgroup starts at a
+    // stage of its own (PTA_SPLITK_ROT: stages between neighbours, 0 switches it off)
+    static const int rot_env = getenv("PTA_SPLITK_ROT") ? atoi(getenv("PTA_SPLITK_ROT")) : -1;
+    const int rot_stride = rot_env >= 0 ? rot_env : 1;
+    const bool rotate = rot_stride > 0 && (a.K % 2048 == 0 || (b.N > 0 && b.K % 2048 == 0));
+    auto kern = rotate ? gemm_splitk_kernel<MT, RT, U, D, true> : gemm_splitk_kernel<MT, RT, U, D, false>;
     if (lds > 64 * 1024) {
-        static bool raised = false;  // per instantiation
-        if (!raised) {
+        static bool raised[2] = {false, false};  // per instantiation
+        if (!raised[rotate]) {
             if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
                 return pta_fail("gemm_splitk_bf16: cannot have %zu bytes of LDS", lds);
-            raised = true;
+            raised[rotate] = true;
         }
     }
     // rows beyond the MT tiles of a workgroup go to further chunks of workgroups, all of the same size
     const int chunks = (M + MT * 16 - 1) / (MT * 16), chunk_rows = ((M + chunks - 1) / chunks + 15) / 16 * 16;
     const dim3 grid((a.tiles * a.parts + b.tiles * b.parts) * chunks);
-    static const int rot_env = getenv("PTA_SPLITK_ROT") ? atoi(getenv("PTA_SPLITK_ROT")) : -1;
-    const int rot_stride = rot_env >= 0 ? rot_env : 1;
     hipLaunchKernelGGL(kern, grid, dim3(SK_THREADS), lds, s, a, b, M, chunks, chunk_rows, rot_stride);
     if (reduce && a.parts > 1) {
         const long MN = (long)M * a.N;
