@@ -60,13 +60,16 @@ def resolve_lengths(cfg: GenerationConfig, prompt_lens: Sequence[int]):
 
 def generate(model, prompts: Sequence[Sequence[int]], generation_config: Optional[GenerationConfig] = None, *,
              batch_size: Optional[int] = None, sampler=None, streamer=None, cache=None,
-             rng_ids: Optional[Sequence[int]] = None, **kwargs) -> Union[List[List[int]], GenerateOutput]:
+             rng_ids: Optional[Sequence[int]] = None, tokenizer=None, **kwargs) -> Union[List[List[int]], GenerateOutput]:
     """Generate for every prompt (a list of token ids); returns prompt + new tokens per prompt.
 
     ``generation_config`` defaults to the model's; keyword arguments override its fields
     (:1543-1545).  ``streamer`` is called as ``streamer(index, token)`` for every new token and
     ``streamer.end()`` if it has one.  ``rng_ids`` name each prompt's random stream (default: its
-    index), so that a prompt draws the same tokens in any batch.
+    index), so that a prompt draws the same tokens in any batch.  ``tokenizer`` (anything with
+    ``decode(ids) -> str``) is needed for ``stop_strings`` only: a sequence ends with the token that
+    completes one of them in the text of its new tokens (src/transformers/generation/utils.py:1118-1125,
+    stopping_criteria.py:110-443; the token is kept, as the reference keeps it).
     """
     cfg = generation_config or getattr(model, "generation_config", None) or GenerationConfig()
     if kwargs:
@@ -103,6 +106,12 @@ def generate(model, prompts: Sequence[Sequence[int]], generation_config: Optiona
         sampler = Sampler(cfg, model.vocab_size, model.device)
 
     eos = set(cfg.eos_token_ids)
+    stop_strings = [cfg.stop_strings] if isinstance(cfg.stop_strings, str) else list(cfg.stop_strings or [])
+    if stop_strings and tokenizer is None:
+        raise ValueError(
+            "There are one or more stop strings, either in the arguments to `generate` or in the model's generation "
+            "config, but we could not locate a tokenizer. When generating with stop strings, you must pass the model's "
+            "tokenizer to the `tokenizer` argument of `generate`.")
     want_scores, want_logits = bool(cfg.output_scores), bool(cfg.output_logits)
     out_tokens: List[List[int]] = [[] for _ in prompts]
     out_scores = [[] for _ in prompts] if want_scores else None
@@ -137,7 +146,8 @@ def generate(model, prompts: Sequence[Sequence[int]], generation_config: Optiona
                         out_logits[i].append(logits[row].clone())
                     if streamer is not None:
                         streamer(i, tok)
-                    if tok in eos or step_no >= new_budget or timed_out:
+                    said_stop = bool(stop_strings) and _ends_with_stop(tokenizer, out_tokens[i], stop_strings)
+                    if tok in eos or step_no >= new_budget or timed_out or said_stop:
                         cache.free(slot_of.pop(i))
                     else:
                         feed[i] = [tok]
@@ -152,6 +162,14 @@ def generate(model, prompts: Sequence[Sequence[int]], generation_config: Optiona
     if cfg.return_dict_in_generate:
         return GenerateOutput(sequences, out_scores, out_logits)
     return sequences
+
+
+def _ends_with_stop(tokenizer, new_tokens: Sequence[int], stop_strings: Sequence[str]) -> bool:
+    """Whether the last token completed a stop string: the string lies in the text of the new tokens and not
+    wholly in the text before the last token."""
+    text = tokenizer.decode(list(new_tokens))
+    before = tokenizer.decode(list(new_tokens[:-1])) if len(new_tokens) > 1 else ""
+    return any(s and s in text and s not in before for s in stop_strings)
 
 
 def pad_sequences(sequences: Sequence[Sequence[int]], prompt_lens: Sequence[int], pad_token_id: int):

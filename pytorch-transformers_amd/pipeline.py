@@ -47,7 +47,7 @@ class TextGenerationPipeline:
         items = [prompts] if single else list(prompts)
         ids = [self._encode(p, prefix) for p in items]
         n_ret = int(generate_kwargs.get("num_return_sequences", 1))
-        seqs = self.model.generate(ids, batch_size=batch_size, **generate_kwargs)
+        seqs = self.model.generate(ids, batch_size=batch_size, tokenizer=self.tokenizer, **generate_kwargs)
         as_text = self.tokenizer is not None and not return_tensors and all(isinstance(p, str) for p in items)
         out = []
         for i, p in enumerate(ids):

@@ -182,6 +182,29 @@ def test_empty_prompt_starts_from_bos_and_slots_return_on_error():
     assert not m.caches[0].live_slots() and m.caches[0].free_pages() == m.caches[0].num_pages
 
 
+def test_stop_strings_need_a_tokenizer_and_end_a_sequence_with_the_completing_token():
+    """src/transformers/generation/utils.py:1118-1125: no tokenizer is an error; with one, a sequence ends with
+    the token that completes a stop string in the text of its new tokens (the token stays), the others go on."""
+    class Letters:
+        def decode(self, ids):
+            return "".join(chr(ord("a") + t % 26) for t in ids)
+
+    prompts = [[1, 2, 3], [4]]
+    free = [expected(p, 8) for p in prompts]
+    with pytest.raises(ValueError, match="tokenizer"):
+        generate(ScriptedModel(), prompts, GenerationConfig(max_new_tokens=8, stop_strings="ab"), sampler=ArgmaxSampler())
+    text = Letters().decode(free[0][3:])
+    stop = text[2:4]  # completed by the fourth new token of the first prompt
+    assert stop not in Letters().decode(free[1][1:]) and stop not in text[:3]
+    out = generate(ScriptedModel(), prompts, GenerationConfig(max_new_tokens=8, stop_strings=[stop, "zzzz"]),
+                   sampler=ArgmaxSampler(), tokenizer=Letters())
+    assert out[0] == free[0][:3 + 4] and out[1] == free[1]
+    # a stop string that the prompt holds does not count: only new tokens are read
+    out = generate(ScriptedModel(), [[0, 1]], GenerationConfig(max_new_tokens=3, stop_strings="ab"), sampler=ArgmaxSampler(),
+                   tokenizer=Letters())
+    assert len(out[0]) == 2 + 3 or "ab" in Letters().decode(out[0][2:])
+
+
 def test_pad_sequences_matches_the_reference_layout():
     t = pad_sequences([[1, 2, 3, 9, 9], [4, 8]], [3, 1], pad_token_id=0)
     assert t.tolist() == [[1, 2, 3, 9, 9], [0, 0, 4, 8, 0]]
