@@ -105,9 +105,27 @@ struct SkinnyProblem {
     int blocks;  // workgroups of this product
 };
 
-template <int MT, int RT, int U, typename OutT>
+// What becomes of the first product's rows when it is a fused query_key_value projection of a decode step:
+// instead of being stored they are split into heads, rotated and written as queries and into the cache pages
+// (what qkv_rope_cache does as a kernel of its own).  The rotation pairs feature i of a head with i + d/2, so a
+// workgroup takes sixteen features of a head's lower half as its first row tile and their partners as its second.
+struct QkvTail {
+    bf16_t* q_out;  // [M, heads, d]
+    const float* inv_freq;  // [d/2], or null: no rotation
+    float cs_scale;
+    const int* token_pos;
+    const int* token_seq;
+    const int* block_table;
+    int bt_stride;
+    bf16_t* k_pool;
+    bf16_t* v_pool;
+    int nh, nkv, d, layout, write_cache;
+};
+
+template <int MT, int RT, int U, typename OutT, bool TAIL = false>
 __global__ __launch_bounds__(512) void gemm_skinny_kernel(SkinnyProblem pa, SkinnyProblem pb, int M, int K,
-                                                          int rot_stride) {
+                                                          int rot_stride, QkvTail tail) {
+    static_assert(!TAIL || (RT == 2 && MT == 1 && sizeof(OutT) == 2), "the query_key_value tail: two row tiles, sixteen rows of x");
     extern __shared__ f32x4_t part[];  // [S][RT][MT][64]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, S = blockDim.x >> 6;
     const int r = lane & 15, g = lane >> 4;
@@ -123,8 +141,14 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(SkinnyProblem pa, Skin
     const int blocks = second ? pb.blocks : pa.blocks, j = (int)blockIdx.x - (second ? pa.blocks : 0);
     const int n0 = (int)((long)j * N / blocks), n1 = (int)((long)(j + 1) * N / blocks);
     const bf16_t* wrow[RT];
+    const bool tailed = TAIL && !second;
+    // with the tail: workgroup j has features s16*16 .. +15 of segment seg (a head's q, k or v) and their partners
+    const int per_seg = TAIL ? tail.d / 32 : 1, seg = j / per_seg, s16 = j % per_seg;
 #pragma unroll
-    for (int t = 0; t < RT; ++t) wrow[t] = W + (long)min(n0 + t * 16 + r, n1 - 1) * K;
+    for (int t = 0; t < RT; ++t) {
+        const int row = tailed ? seg * tail.d + t * (tail.d >> 1) + s16 * 16 + r : min(n0 + t * 16 + r, n1 - 1);
+        wrow[t] = W + (long)row * K;
+    }
     // x through a buffer descriptor whose bounds are the M real rows (0x00020000: 32-bit raw data format)
     __amdgpu_buffer_rsrc_t xres = __builtin_amdgcn_make_buffer_rsrc((void*)x, 0, M * K * 2, 0x00020000);
 
@@ -159,6 +183,82 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(SkinnyProblem pa, Skin
         for (int mt = 0; mt < MT; ++mt) part[((wave * RT + rt) * MT + mt) * 64 + lane] = acc[rt][mt];
     __syncthreads();
 
+    if constexpr (TAIL) {
+        if (tailed) {
+            // thread ln: token m = ln % 16, features i0 .. i0+3 of the segment's lower half and their partners
+            for (int ln = threadIdx.x; ln < 64; ln += blockDim.x) {
+                f32x4_t lo = part[ln], hi = part[64 + ln];
+                for (int w = 1; w < S; ++w) {
+                    const f32x4_t p = part[(w * 2) * 64 + ln], q = part[(w * 2 + 1) * 64 + ln];
+                    lo[0] += p[0]; lo[1] += p[1]; lo[2] += p[2]; lo[3] += p[3];
+                    hi[0] += q[0]; hi[1] += q[1]; hi[2] += q[2]; hi[3] += q[3];
+                }
+                const int m = ln & 15;
+                if (m >= M) continue;
+                const int d = tail.d, half = d >> 1, i0 = s16 * 16 + (ln >> 4) * 4, gq = tail.nh / tail.nkv;
+                int kind, head;  // 0 query, 1 key, 2 value
+                if (tail.layout == PTA_QKV_GROUPED) {
+                    const int grp = seg / (gq + 2), w = seg % (gq + 2);
+                    kind = w < gq ? 0 : w - gq + 1;
+                    head = w < gq ? grp * gq + w : grp;
+                } else if (tail.layout == PTA_QKV_TAIL) {
+                    kind = seg < tail.nh ? 0 : seg - tail.nh + 1;
+                    head = seg < tail.nh ? seg : 0;
+                } else {
+                    kind = seg % 3;
+                    head = seg / 3;
+                }
+                if (kind != 0 && !tail.write_cache) continue;
+                const int pos = tail.token_pos[m];
+                float a[4], b[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    a[e] = round_to_bf16(lo[e]);
+                    b[e] = round_to_bf16(hi[e]);
+                    if (bias) {
+                        a[e] = round_to_bf16(a[e] + bias[seg * d + i0 + e]);
+                        b[e] = round_to_bf16(b[e] + bias[seg * d + half + i0 + e]);
+                    }
+                }
+                if (tail.inv_freq && kind != 2) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float ang = (float)pos * tail.inv_freq[i0 + e];
+                        const float c = cosf(ang) * tail.cs_scale, sn = sinf(ang) * tail.cs_scale;
+                        const float x0 = a[e], x1 = b[e];
+                        a[e] = x0 * c - x1 * sn;
+                        b[e] = x1 * c + x0 * sn;
+                    }
+                }
+                uint2 pa4, pb4;
+                pa4.x = (uint32_t)f32_to_bf16_bits(a[0]) | ((uint32_t)f32_to_bf16_bits(a[1]) << 16);
+                pa4.y = (uint32_t)f32_to_bf16_bits(a[2]) | ((uint32_t)f32_to_bf16_bits(a[3]) << 16);
+                pb4.x = (uint32_t)f32_to_bf16_bits(b[0]) | ((uint32_t)f32_to_bf16_bits(b[1]) << 16);
+                pb4.y = (uint32_t)f32_to_bf16_bits(b[2]) | ((uint32_t)f32_to_bf16_bits(b[3]) << 16);
+                if (kind == 0) {
+                    bf16_t* dst = tail.q_out + ((long)m * tail.nh + head) * d + i0;
+                    *reinterpret_cast<uint2*>(dst) = pa4;
+                    *reinterpret_cast<uint2*>(dst + half) = pb4;
+                    continue;
+                }
+                const long page = tail.block_table[(long)tail.token_seq[m] * tail.bt_stride + pos / PTA_PAGE];
+                const int in_page = pos % PTA_PAGE;
+                if (kind == 1) {
+                    bf16_t* dst = tail.k_pool + ((page * tail.nkv + head) * PTA_PAGE + in_page) * (long)d + i0;
+                    *reinterpret_cast<uint2*>(dst) = pa4;
+                    *reinterpret_cast<uint2*>(dst + half) = pb4;
+                } else {
+                    bf16_t* dst = tail.v_pool + ((page * tail.nkv + head) * (long)d + i0) * PTA_PAGE + in_page;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        dst[(long)e * PTA_PAGE] = f32_to_bf16_bits(a[e]);
+                        dst[(long)(half + e) * PTA_PAGE] = f32_to_bf16_bits(b[e]);
+                    }
+                }
+            }
+            return;
+        }
+    }
     // item (rt, mt, ln): outputs of row m = mt*16 + ln%16, columns n0 + rt*16 + (ln/16)*4 + 0..3
     for (int item = threadIdx.x; item < RT * MT * 64; item += blockDim.x) {
         const int ln = item & 63, mt = (item >> 6) % MT, rt = (item >> 6) / MT;
@@ -220,7 +320,7 @@ static void launch_cfg(SkinnyProblem a, SkinnyProblem b, int M, int K, int S, hi
     const size_t lds = (size_t)S * RT * MT * 64 * sizeof(f32x4_t);
     static const int rot_env = getenv("PTA_SKINNY_ROT") ? atoi(getenv("PTA_SKINNY_ROT")) : -1;
     const int rot_stride = rot_env >= 0 ? rot_env : (K % 2048 == 0 ? 5 : 0);  // rows a multiple of 4 KB long
-    hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, U, OutT>), grid, block, lds, s, a, b, M, K, rot_stride);
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, RT, U, OutT>), grid, block, lds, s, a, b, M, K, rot_stride, QkvTail{});
 }
 
 template <typename OutT>
@@ -278,6 +378,47 @@ extern "C" int pta_gemm_skinny_bf16(void* y, const void* x, const void* W, const
     const SkinnyProblem a{y, (const bf16_t*)x, (const bf16_t*)W, bias, (const bf16_t*)add1, (const bf16_t*)add2, N, act, 0};
     if (out_f32) return launch_skinny<float>(a, none, M, K, variant, waves, s);
     return launch_skinny<bf16_t>(a, none, M, K, variant, waves, s);
+}
+
+// The pair launch of a decode step whose first product is a fused query_key_value projection: its rows never
+// reach memory as such; queries come out rotated in q_out [M, heads, d], keys (rotated) and values go to the
+// cache pages of their sequences, as pta_qkv_rope_cache would have left them.  Up to 16 rows, head sizes that are
+// multiples of 32.  The second product is y2 = act2(x2 . W2^T + bias2) as in the plain pair.
+extern "C" int pta_gemm_skinny_pair_qkv_bf16(void* q_out, const void* x1, const void* W1, const float* bias1,
+                                             const float* inv_freq, float cs_scale, const int* token_pos,
+                                             const int* token_seq, const int* block_table, int bt_stride, void* k_pool,
+                                             void* v_pool, int nh, int nkv, int d, int layout, int write_cache, void* y2,
+                                             const void* x2, const void* W2, const float* bias2, int N2, int act2, int M,
+                                             int K, void* stream) {
+    PTA_REQUIRE(nh > 0 && nkv > 0 && d > 0 && nh % nkv == 0, "gemm_skinny_pair_qkv_bf16: heads %d, kv heads %d, head size %d", nh, nkv, d);
+    const int N1 = (nh + 2 * nkv) * d;
+    if (check_skinny("gemm_skinny_pair_qkv_bf16", q_out, x1, W1, M, N1, K, PTA_ACT_NONE)) return 1;
+    if (check_skinny("gemm_skinny_pair_qkv_bf16", y2, x2, W2, M, N2, K, act2)) return 1;
+    PTA_REQUIRE(M <= 16, "gemm_skinny_pair_qkv_bf16: at most 16 rows, got %d", M);
+    PTA_REQUIRE(d % 32 == 0 && d <= 256, "gemm_skinny_pair_qkv_bf16: head size %d must be a multiple of 32 up to 256", d);
+    PTA_REQUIRE(layout >= 0 && layout <= 2, "gemm_skinny_pair_qkv_bf16: unknown layout %d", layout);
+    PTA_REQUIRE(layout != PTA_QKV_TAIL || nkv == 1, "gemm_skinny_pair_qkv_bf16: the tail layout has one kv head, got %d", nkv);
+    PTA_REQUIRE(layout != PTA_QKV_INTERLEAVED || nkv == nh, "gemm_skinny_pair_qkv_bf16: the interleaved layout needs kv heads == heads");
+    PTA_REQUIRE(token_pos, "gemm_skinny_pair_qkv_bf16: null token positions");
+    PTA_REQUIRE(!write_cache || (k_pool && v_pool && block_table && token_seq), "gemm_skinny_pair_qkv_bf16: null cache pointer");
+    PTA_REQUIRE((((uintptr_t)q_out | (uintptr_t)k_pool) % 8) == 0, "gemm_skinny_pair_qkv_bf16: outputs must be 8-byte aligned");
+    SkinnyProblem a{nullptr, (const bf16_t*)x1, (const bf16_t*)W1, bias1, nullptr, nullptr, N1, PTA_ACT_NONE, 0};
+    SkinnyProblem b{y2, (const bf16_t*)x2, (const bf16_t*)W2, bias2, nullptr, nullptr, N2, in_kernel(act2) ? act2 : 0, 0};
+    const QkvTail tail{(bf16_t*)q_out, inv_freq, cs_scale, token_pos, token_seq, block_table, bt_stride, (bf16_t*)k_pool,
+                       (bf16_t*)v_pool, nh, nkv, d, layout, write_cache};
+    // the first product's workgroups are bound to heads; the second one's fill the launch up to a whole number per unit
+    a.blocks = (nh + 2 * nkv) * (d / 32);
+    b.blocks = (N2 + 31) / 32;
+    const int units = pta_compute_units(), natural = a.blocks + b.blocks;
+    if (natural > units && natural % units != 0) b.blocks = (natural + units - 1) / units * units - a.blocks;
+    const int S = pick_split(N1 + N2);
+    static const int rot_env = getenv("PTA_SKINNY_ROT") ? atoi(getenv("PTA_SKINNY_ROT")) : -1;
+    const int rot_stride = rot_env >= 0 ? rot_env : (K % 2048 == 0 ? 5 : 0);
+    hipLaunchKernelGGL((gemm_skinny_kernel<1, 2, 2, bf16_t, true>), dim3(a.blocks + b.blocks), dim3(S * 64),
+                       (size_t)S * 2 * 64 * sizeof(f32x4_t), (hipStream_t)stream, a, b, M, K, rot_stride, tail);
+    if (pta_check_launch("gemm_skinny_pair_qkv_bf16")) return 1;
+    if (!in_kernel(act2)) return pta_epilogue(y2, N2, nullptr, nullptr, nullptr, M, N2, act2, PTA_BF16, stream);
+    return 0;
 }
 
 // Two products of one launch: y1 = act1(x1 . W1^T + bias1), y2 = act2(x2 . W2^T + bias2), both [M, *] in

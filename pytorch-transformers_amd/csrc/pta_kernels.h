@@ -84,6 +84,15 @@ int pta_gemm_skinny_pair_bf16(void* y1, const void* x1, const void* W1, const fl
                               const void* x2, const void* W2, const float* bias2, int N2, int act2, int M, int K,
                               void* stream);
 
+// the pair launch of a decode step (M <= 16) whose first product is a fused query_key_value projection: its rows
+// are split, rotated and written as queries [M, heads, d] and into the cache pages, as pta_qkv_rope_cache leaves
+// them; head sizes that are multiples of 32
+int pta_gemm_skinny_pair_qkv_bf16(void* q_out, const void* x1, const void* W1, const float* bias1,
+                                  const float* inv_freq, float cs_scale, const int* token_pos, const int* token_seq,
+                                  const int* block_table, int bt_stride, void* k_pool, void* v_pool, int nh, int nkv,
+                                  int d, int layout, int write_cache, void* y2, const void* x2, const void* W2,
+                                  const float* bias2, int N2, int act2, int M, int K, void* stream);
+
 // The same product for a batch of up to 128 rows that shares x through LDS and may split K over workgroups:
 // `part` is a 32-bit workspace [parts, M, N], needed when parts > 1 or reduce = 0.  rt (row tiles per wave),
 // parts, stage_blocks (64-element blocks of K per stage) and depth (stages in flight) are tuning knobs (0:

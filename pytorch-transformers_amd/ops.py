@@ -661,6 +661,51 @@ def gemm_skinny_pair_bf16(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tensor, 
     return y1, y2
 
 
+def gemm_skinny_pair_qkv_ok(x: torch.Tensor, w_qkv: torch.Tensor, w2: torch.Tensor, d: int) -> bool:
+    """Whether the pair launch for few rows can take a fused query_key_value projection to its end (rotation,
+    queries, cache pages): bfloat16, at most 16 rows, head sizes that are multiples of 32.  PTA_QKV_TAIL=0
+    switches it off."""
+    return (QKV_TAIL and gemm_skinny_ok(x, w_qkv) and gemm_skinny_ok(x, w2) and d % 32 == 0 and d <= 256
+            and w_qkv.shape[1] == w2.shape[1])
+
+
+QKV_TAIL = os.environ.get("PTA_QKV_TAIL", "1") != "0"
+
+
+def gemm_skinny_pair_qkv(x1: torch.Tensor, w_qkv: torch.Tensor, bias_qkv, inv_freq, cs_scale: float, token_pos,
+                         token_seq, block_table, k_pool, v_pool, nh: int, nkv: int, d: int, layout: str,
+                         write_cache: bool, x2: torch.Tensor, w2: torch.Tensor, bias2=None, act2=None):
+    """One launch for a decode step's two input products, the first a fused query_key_value projection taken to
+    its end: returns (queries [M, nh, d] rotated, act2(x2 @ w2.T + bias2)); keys and values are in the cache pages,
+    as ``qkv_rope_cache`` would have left them."""
+    for name, t in (("x1", x1), ("w_qkv", w_qkv), ("x2", x2), ("w2", w2)):
+        _need(t, name, torch.bfloat16)
+    M, K = x1.shape
+    N1, N2 = (nh + 2 * nkv) * d, w2.shape[0]
+    if tuple(x2.shape) != (M, K) or tuple(w_qkv.shape) != (N1, K) or w2.dim() != 2 or w2.shape[1] != K:
+        raise KernelError(f"a pair shares M and K: x1 {tuple(x1.shape)}, x2 {tuple(x2.shape)}, w_qkv {tuple(w_qkv.shape)} "
+                          f"(wanted [{N1}, {K}]), w2 {tuple(w2.shape)}")
+    if bias_qkv is not None:
+        _need(bias_qkv, "bias_qkv", torch.float32, (N1,))
+    if bias2 is not None:
+        _need(bias2, "bias2", torch.float32, (N2,))
+    if inv_freq is not None:
+        _need(inv_freq, "inv_freq", torch.float32, (d // 2,))
+    _need(token_pos, "token_pos", torch.int32, (M,))
+    _need(token_seq, "token_seq", torch.int32, (M,))
+    _need(block_table, "block_table", torch.int32)
+    if block_table.dim() != 2:
+        raise KernelError("block_table must be [sequences, pages]")
+    _need_pools(k_pool, v_pool, torch.bfloat16, nkv, d)
+    q = torch.empty((M, nh, d), dtype=torch.bfloat16, device=x1.device)
+    y2 = torch.empty((M, N2), dtype=torch.bfloat16, device=x1.device)
+    _call("pta_gemm_skinny_pair_qkv_bf16", _ptr(q), _ptr(x1), _ptr(w_qkv), _ptr(bias_qkv), _ptr(inv_freq),
+          ctypes.c_float(cs_scale), _ptr(token_pos), _ptr(token_seq), _ptr(block_table), block_table.shape[1], _ptr(k_pool),
+          _ptr(v_pool), nh, nkv, d, QKV_LAYOUT_CODES[layout], int(write_cache), _ptr(y2), _ptr(x2), _ptr(w2), _ptr(bias2),
+          N2, ACT_CODES[act2], M, K, _stream())
+    return q, y2
+
+
 def gemm_splitk_bf16(x: torch.Tensor, w: torch.Tensor, bias=None, act=None, add1=None, add2=None,
                      out_f32: bool = False, rt: int = 0, parts: int = 0, stage_blocks: int = 0,
                      depth: int = 0) -> torch.Tensor:

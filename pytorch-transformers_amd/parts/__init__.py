@@ -1,6 +1,6 @@
 """Parts that models are put together from: mixers, feed-forwards, norms, position encodings, blocks."""
 from .base import Part, StepContext, make_part, register_part, registered_parts
-from .linear import Embedding, Linear, OutputHead
+from .linear import Embedding, Linear, OutputHead, QkvTail, TailDone
 from .norms import LayerNorm
 from .positions import AlibiPositions, NoPositions, RotaryPositions, alibi_slopes
 from .attention import AttentionMixer

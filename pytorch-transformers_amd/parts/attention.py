@@ -17,7 +17,7 @@ import torch
 
 from .. import ops
 from .base import Part, StepContext, register_part
-from .linear import Linear, PendingProjection
+from .linear import Linear, PendingProjection, QkvTail, TailDone
 
 
 class AttentionMixer(Part):
@@ -52,17 +52,27 @@ class AttentionMixer(Part):
         part's and hand the result back as ``projected``."""
         return self.qkv, {"apply_bias": False}
 
+    def projection_tail(self, ctx: StepContext, call) -> QkvTail:
+        """What ``forward`` does with the first product's rows; a block that runs that product in a launch of its
+        own may hand this to the launch (``Linear.pair``)."""
+        k_pool, v_pool = ctx.cache.kv_layer(call.cache_group, call.cache_layer)
+        inv_freq, cs_scale = self.positions.rotation()
+        return QkvTail(self.qkv.bias, inv_freq, cs_scale, ctx.token_pos, ctx.token_seq, ctx.block_tables[call.cache_group],
+                       k_pool, v_pool, self.num_heads, self.kv_heads, self.head_dim, self.qkv_layout, call.write_cache)
+
     def forward(self, x: torch.Tensor, ctx: StepContext, call, residual: Optional[torch.Tensor] = None,
-                defer: bool = False, projected: Optional[torch.Tensor] = None):
+                defer: bool = False, projected=None):
         """Attention of the step's tokens over the cache, projected out, plus ``residual``.  With ``defer``
-        the output projection comes back not run (``PendingProjection``); the caller adds the residual."""
+        the output projection comes back not run (``PendingProjection``); the caller adds the residual.
+        ``projected``: the first product, run by the caller, or ``TailDone(queries)`` if its launch has also
+        rotated it and written the cache."""
         k_pool, v_pool = ctx.cache.kv_layer(call.cache_group, call.cache_layer)
         table = ctx.block_tables[call.cache_group]
-        fused = projected if projected is not None else self.qkv(x, apply_bias=False)
-        inv_freq, cs_scale = self.positions.rotation()
-        q = ops.qkv_rope_cache(fused, self.qkv.bias, inv_freq, cs_scale, ctx.token_pos, ctx.token_seq, table,
-                               k_pool, v_pool, self.num_heads, self.kv_heads, self.head_dim, self.qkv_layout,
-                               write_cache=call.write_cache)
+        if isinstance(projected, TailDone):
+            q = projected.value
+        else:
+            fused = projected if projected is not None else self.qkv(x, apply_bias=False)
+            q = self.projection_tail(ctx, call).run(fused)
         o = ops.attention(q, k_pool, v_pool, table, ctx, self.positions.score_bias(), self.scale, self.window)
         if defer:
             return PendingProjection(self.out, o)

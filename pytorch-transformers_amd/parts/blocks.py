@@ -79,7 +79,8 @@ class ParallelBlock(Part):
         # both branches start with a product of the norm's output: one launch for the two in small steps
         if hasattr(self.mixer, "input_projection") and hasattr(self.feed_forward, "input_projection"):
             (lin_a, kw_a), (lin_m, kw_m) = self.mixer.input_projection(), self.feed_forward.input_projection()
-            both = Linear.pair(lin_a, a, kw_a, lin_m, m, kw_m)
+            tail = self.mixer.projection_tail(ctx, call) if hasattr(self.mixer, "projection_tail") else None
+            both = Linear.pair(lin_a, a, kw_a, lin_m, m, kw_m, tail=tail)
             if both is not None:
                 kw_mixer["projected"], kw_ffn["projected"] = both
         if _can_defer(self.feed_forward) and _can_defer(self.mixer):

@@ -83,15 +83,24 @@ class Linear(Part):
         return y
 
     @staticmethod
-    def pair(first: "Linear", x1: torch.Tensor, kw1: dict, second: "Linear", x2: torch.Tensor, kw2: dict):
+    def pair(first: "Linear", x1: torch.Tensor, kw1: dict, second: "Linear", x2: torch.Tensor, kw2: dict, tail=None):
         """``(first(x1, **kw1), second(x2, **kw2))`` from one matrix launch, in steps small enough for the
-        decode kernels (same rows, no additions); else None."""
+        decode kernels (same rows, no additions); else None.  ``tail`` (a ``QkvTail``) says what the caller will
+        do with the first result; where the launch can do that itself, the first result comes back as
+        ``TailDone(queries)``."""
         if not (x1.dtype == torch.bfloat16 and x1.shape[0] == x2.shape[0]):
             return None
         if any(k not in ("act", "apply_bias") for k in list(kw1) + list(kw2)):
             return None
         b1 = first.bias if kw1.get("apply_bias", True) else None
         b2 = second.bias if kw2.get("apply_bias", True) else None
+        if (tail is not None and x1.shape == x2.shape and kw1.get("act") is None
+                and ops.gemm_skinny_pair_qkv_ok(x1, first.weight, second.weight, tail.head_dim)):
+            q, y2 = ops.gemm_skinny_pair_qkv(
+                x1, first.weight, tail.bias, tail.inv_freq, tail.cs_scale, tail.token_pos, tail.token_seq, tail.table,
+                tail.k_pool, tail.v_pool, tail.num_heads, tail.kv_heads, tail.head_dim, tail.layout, tail.write_cache,
+                x2, second.weight, b2, kw2.get("act"))
+            return TailDone(q), y2
         args = (x1, first.weight, x2, second.weight, b1, kw1.get("act"), b2, kw2.get("act"))
         if x1.shape == x2.shape and ops.gemm_skinny_ok(x1, first.weight) and ops.gemm_skinny_ok(x2, second.weight):
             return ops.gemm_skinny_pair_bf16(*args)
@@ -121,6 +130,31 @@ class Linear(Part):
         if self.can_partial(x):
             return PartialProduct(ops.gemm_splitk_partial(x, self.weight), self.bias)
         return None
+
+
+class QkvTail:
+    """What a mixer does with its fused query_key_value rows: bias, split into heads, rotation, queries out, keys
+    and values into the cache pages.  ``run`` does it as a kernel of its own; a pair launch that is given the tail
+    may do it in its epilogue instead (``Linear.pair``)."""
+
+    def __init__(self, bias, inv_freq, cs_scale, token_pos, token_seq, table, k_pool, v_pool, num_heads: int,
+                 kv_heads: int, head_dim: int, layout: str, write_cache: bool):
+        self.bias, self.inv_freq, self.cs_scale = bias, inv_freq, cs_scale
+        self.token_pos, self.token_seq, self.table, self.k_pool, self.v_pool = token_pos, token_seq, table, k_pool, v_pool
+        self.num_heads, self.kv_heads, self.head_dim, self.layout = num_heads, kv_heads, head_dim, layout
+        self.write_cache = write_cache
+
+    def run(self, fused: torch.Tensor) -> torch.Tensor:
+        return ops.qkv_rope_cache(fused, self.bias, self.inv_freq, self.cs_scale, self.token_pos, self.token_seq,
+                                  self.table, self.k_pool, self.v_pool, self.num_heads, self.kv_heads, self.head_dim,
+                                  self.layout, write_cache=self.write_cache)
+
+
+class TailDone:
+    """A first product whose tail the launch has already run: ``value`` is what the tail gives."""
+
+    def __init__(self, value: torch.Tensor):
+        self.value = value
 
 
 class PendingProjection:

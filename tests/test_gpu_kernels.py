@@ -372,6 +372,48 @@ def test_qkv_rope_cache(dtype, layout, nh, nkv, d, rotary):
     assert torch.equal(torch.nan_to_num(k2.float()), torch.nan_to_num(k_pool.float()))
 
 
+@pytest.mark.parametrize("layout,nh,nkv,d", [("grouped", 4, 2, 32), ("grouped", 8, 2, 128), ("tail", 7, 1, 64),
+                                             ("interleaved", 3, 3, 96), ("tail", 71, 1, 64)])
+@pytest.mark.parametrize("rotary,bias", [(True, True), (False, False), (True, False)])
+def test_pair_launch_takes_the_fused_qkv_rows_to_their_end(layout, nh, nkv, d, rotary, bias):
+    """The pair launch for few rows with the query_key_value tail in its epilogue against the same two products
+    followed by the kernel that splits, rotates and writes the cache: the same queries, the same pages (bit for bit
+    where K is not a multiple of 2,048, so that both walk K alike), nothing written where no token lies, and
+    nothing written at all with write_cache off."""
+    ops = _ops()
+    K, N2 = 264, 200
+    starts = [70, 0, 127, 5, 63]
+    M = len(starts)
+    lens = [s + 1 for s in starts]
+    N1 = (nh + 2 * nkv) * d
+    x = _rand(M, K, dtype=torch.bfloat16)
+    w1, w2 = _rand(N1, K, seed=1, dtype=torch.bfloat16, scale=0.05), _rand(N2, K, seed=2, dtype=torch.bfloat16, scale=0.05)
+    b1, b2 = (_rand(N1, seed=3) if bias else None), _rand(N2, seed=4)
+    token_seq = torch.arange(M, dtype=torch.int32).cuda()
+    token_pos = torch.tensor(starts, dtype=torch.int32).cuda()
+    inv = P.rope_inv_freq(d, 10000.0).cuda() if rotary else None
+    assert ops.gemm_skinny_pair_qkv_ok(x, w1, w2, d)
+    pools = []
+    for fused_way in (False, True):
+        k_pool, v_pool, bt, lists = _cache_setup(M, lens, nkv, d, torch.bfloat16)
+        if fused_way:
+            q, y2 = ops.gemm_skinny_pair_qkv(x, w1, b1, inv, 0.9, token_pos, token_seq, bt, k_pool, v_pool, nh, nkv, d,
+                                             layout, True, x, w2, b2, "gelu")
+        else:
+            fused, y2 = ops.gemm_skinny_pair_bf16(x, w1, x, w2, None, None, b2, "gelu")
+            q = ops.qkv_rope_cache(fused, b1, inv, 0.9, token_pos, token_seq, bt, k_pool, v_pool, nh, nkv, d, layout)
+        pools.append((q, y2, k_pool, v_pool))
+    (q0, y0, k0, v0), (q1, y1, k1, v1) = pools
+    assert torch.equal(y0, y1), "the second product does not know about the first one's tail"
+    assert torch.equal(q0, q1)
+    same = lambda a, b: torch.equal(torch.nan_to_num(a.float(), nan=-7.0), torch.nan_to_num(b.float(), nan=-7.0))
+    assert same(k0, k1) and same(v0, v1), "the same values at the same places of the pages, and nothing anywhere else"
+    before = k1.clone()
+    q2, _ = ops.gemm_skinny_pair_qkv(x, w1 * 2, b1, inv, 0.9, token_pos, token_seq, bt, k1, v1, nh, nkv, d, layout, False,
+                                     x, w2, b2, "gelu")
+    assert same(before, k1) and not torch.equal(q2, q1)
+
+
 def _windowed_attention(q, k, v, window):
     """Plain attention in which query t sees keys t - window + 1 .. t; q [T, nh, d], k, v [T, nkv, d]."""
     T, nh, d = q.shape
