@@ -14,6 +14,7 @@
 // the order of summation never depends on M or on what else is in the batch.
 #include "common.h"
 #include "pta_kernels.h"
+#include "qkv_tail.h"
 
 #include <stdlib.h>
 
@@ -105,23 +106,9 @@ struct SkinnyProblem {
     int blocks;  // workgroups of this product
 };
 
-// What becomes of the first product's rows when it is a fused query_key_value projection of a decode step:
-// instead of being stored they are split into heads, rotated and written as queries and into the cache pages
-// (what qkv_rope_cache does as a kernel of its own).  The rotation pairs feature i of a head with i + d/2, so a
-// workgroup takes sixteen features of a head's lower half as its first row tile and their partners as its second.
-struct QkvTail {
-    bf16_t* q_out;  // [M, heads, d]
-    const float* inv_freq;  // [d/2], or null: no rotation
-    float cs_scale;
-    const int* token_pos;
-    const int* token_seq;
-    const int* block_table;
-    int bt_stride;
-    bf16_t* k_pool;
-    bf16_t* v_pool;
-    int nh, nkv, d, layout, write_cache;
-};
-
+// With a QkvTail (qkv_tail.h) the first product's rows are not stored: they are split into heads, rotated and written
+// as queries and into the cache pages.  The rotation pairs feature i of a head with i + d/2, so a workgroup takes
+// sixteen features of a head's lower half as its first row tile and their partners as its second.
 template <int MT, int RT, int U, typename OutT, bool TAIL = false>
 __global__ __launch_bounds__(512) void gemm_skinny_kernel(SkinnyProblem pa, SkinnyProblem pb, int M, int K,
                                                           int rot_stride, QkvTail tail) {
@@ -195,19 +182,9 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(SkinnyProblem pa, Skin
                 }
                 const int m = ln & 15;
                 if (m >= M) continue;
-                const int d = tail.d, half = d >> 1, i0 = s16 * 16 + (ln >> 4) * 4, gq = tail.nh / tail.nkv;
+                const int d = tail.d, half = d >> 1, i0 = s16 * 16 + (ln >> 4) * 4;
                 int kind, head;  // 0 query, 1 key, 2 value
-                if (tail.layout == PTA_QKV_GROUPED) {
-                    const int grp = seg / (gq + 2), w = seg % (gq + 2);
-                    kind = w < gq ? 0 : w - gq + 1;
-                    head = w < gq ? grp * gq + w : grp;
-                } else if (tail.layout == PTA_QKV_TAIL) {
-                    kind = seg < tail.nh ? 0 : seg - tail.nh + 1;
-                    head = seg < tail.nh ? seg : 0;
-                } else {
-                    kind = seg % 3;
-                    head = seg / 3;
-                }
+                qkv_tail_segment(tail, seg, kind, head);
                 if (kind != 0 && !tail.write_cache) continue;
                 const int pos = tail.token_pos[m];
                 float a[4], b[4];

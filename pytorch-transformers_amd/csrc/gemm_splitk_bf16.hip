@@ -18,6 +18,7 @@
 // a stage past the end multiplies weights that are already in cache by zeros.
 #include "common.h"
 #include "pta_kernels.h"
+#include "qkv_tail.h"
 
 #include <stdlib.h>
 
@@ -279,6 +280,36 @@ extern "C" int pta_gemm_reduce_parts(void* y, const float* part, const float* bi
     return pta_check_launch("gemm_reduce_parts");
 }
 
+// The reduction of a pair launch whose first product is a fused query_key_value projection: a thread adds the
+// partial sums of one rotation pair (feature i of a segment's lower half and i + d/2) and takes it to its end
+// (qkv_tail.h); the second product as in gemm_splitk_reduce2_kernel.
+__global__ __launch_bounds__(256) void gemm_splitk_reduce2_qkv_kernel(QkvTail tail, const float* __restrict__ part1,
+                                                                      const float* __restrict__ bias1, long MN1, int N1,
+                                                                      int P1, bf16_t* __restrict__ y2,
+                                                                      const float* __restrict__ part2,
+                                                                      const float* __restrict__ bias2, long MN2, int N2,
+                                                                      int P2, int act2) {
+    long o = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long pairs = MN1 >> 1;
+    if (o < pairs) {
+        const int half = tail.d >> 1, per_row = N1 >> 1;
+        const int m = (int)(o / per_row), p = (int)(o % per_row), seg = p / half, i = p % half;
+        const long lo = (long)m * N1 + (long)seg * tail.d + i, hi = lo + half;
+        float a = part1[lo], b = part1[hi];
+        for (int q = 1; q < P1; ++q) { a += part1[(long)q * MN1 + lo]; b += part1[(long)q * MN1 + hi]; }
+        qkv_tail_pair(tail, bias1, m, seg, i, round_to_bf16(a), round_to_bf16(b));
+        return;
+    }
+    o -= pairs;
+    if (o >= MN2) return;
+    float v = part2[o];
+    for (int q = 1; q < P2; ++q) v += part2[(long)q * MN2 + o];
+    v = round_to_bf16(v);
+    if (bias2) v = round_to_bf16(v + bias2[(int)(o % N2)]);
+    if (act2) v = apply_act(v, act2);
+    y2[o] = f32_to_bf16_bits(v);
+}
+
 static int pick_rt(int N) { return N >= 16384 ? 2 : 1; }
 
 // ranges that are not empty when K is cut into `parts` ranges of whole 64-element blocks
@@ -479,4 +510,34 @@ extern "C" int pta_gemm_splitk_pair_reduced_bf16(void* y1, float* part1, const v
                        (hipStream_t)stream, (bf16_t*)y1, part1, bias1, MN1, N1, P1, act1, (bf16_t*)y2, part2, bias2, MN2, N2,
                        P2, act2);
     return pta_check_launch("gemm_splitk_pair_reduced_bf16");
+}
+
+// The same pair with the first product a fused query_key_value projection taken to its end: queries rotated in
+// q_out [M, heads, d], keys and values in the cache pages (as pta_qkv_rope_cache leaves them); even head sizes.
+extern "C" int pta_gemm_splitk_pair_reduced_qkv_bf16(void* q_out, float* part1, const void* x1, const void* W1,
+                                                     const float* bias1, int K1, const float* inv_freq, float cs_scale,
+                                                     const int* token_pos, const int* token_seq, const int* block_table,
+                                                     int bt_stride, void* k_pool, void* v_pool, int nh, int nkv, int d,
+                                                     int layout, int write_cache, void* y2, float* part2, const void* x2,
+                                                     const void* W2, const float* bias2, int N2, int K2, int act2, int M,
+                                                     void* stream) {
+    PTA_REQUIRE(nh > 0 && nkv > 0 && d > 0 && nh % nkv == 0, "gemm_splitk_pair_reduced_qkv_bf16: heads %d, kv heads %d, head size %d", nh, nkv, d);
+    PTA_REQUIRE(d % 2 == 0, "gemm_splitk_pair_reduced_qkv_bf16: head size %d must be even", d);
+    PTA_REQUIRE(layout >= 0 && layout <= 2, "gemm_splitk_pair_reduced_qkv_bf16: unknown layout %d", layout);
+    PTA_REQUIRE(layout != PTA_QKV_TAIL || nkv == 1, "gemm_splitk_pair_reduced_qkv_bf16: the tail layout has one kv head, got %d", nkv);
+    PTA_REQUIRE(layout != PTA_QKV_INTERLEAVED || nkv == nh, "gemm_splitk_pair_reduced_qkv_bf16: the interleaved layout needs kv heads == heads");
+    PTA_REQUIRE(q_out && y2 && token_pos, "gemm_splitk_pair_reduced_qkv_bf16: null pointer");
+    PTA_REQUIRE(!write_cache || (k_pool && v_pool && block_table && token_seq), "gemm_splitk_pair_reduced_qkv_bf16: null cache pointer");
+    PTA_REQUIRE(pta_act_known(act2), "gemm_splitk_pair_reduced_qkv_bf16: unknown activation %d", act2);
+    const int N1 = (nh + 2 * nkv) * d;
+    const int rc = pta_gemm_splitk_pair_bf16(part1, x1, W1, N1, K1, part2, x2, W2, N2, K2, M, stream);
+    if (rc) return rc;
+    const long MN1 = (long)M * N1, MN2 = (long)M * N2;
+    int P1, P2;
+    pick_pair_parts(N1, K1, N2, K2, &P1, &P2);
+    const QkvTail tail{(bf16_t*)q_out, inv_freq, cs_scale, token_pos, token_seq, block_table, bt_stride, (bf16_t*)k_pool,
+                       (bf16_t*)v_pool, nh, nkv, d, layout, write_cache};
+    hipLaunchKernelGGL(gemm_splitk_reduce2_qkv_kernel, dim3((unsigned)((MN1 / 2 + MN2 + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, tail, part1, bias1, MN1, N1, P1, (bf16_t*)y2, part2, bias2, MN2, N2, P2, act2);
+    return pta_check_launch("gemm_splitk_pair_reduced_qkv_bf16");
 }

@@ -107,6 +107,15 @@ int pta_gemm_splitk_parts(int N, int K, int parts, int rt);
 // ranges pta_gemm_splitk_pair_parts gives
 int pta_gemm_splitk_pair_parts(int N1, int K1, int N2, int K2, int* parts1, int* parts2);
 
+// the pair run to the end with the first product a fused query_key_value projection (N1 = (nh + 2 nkv) d rows of
+// W1): queries rotated in q_out [M, nh, d], keys and values in the cache pages, as pta_qkv_rope_cache leaves them
+int pta_gemm_splitk_pair_reduced_qkv_bf16(void* q_out, float* part1, const void* x1, const void* W1, const float* bias1,
+                                          int K1, const float* inv_freq, float cs_scale, const int* token_pos,
+                                          const int* token_seq, const int* block_table, int bt_stride, void* k_pool,
+                                          void* v_pool, int nh, int nkv, int d, int layout, int write_cache, void* y2,
+                                          float* part2, const void* x2, const void* W2, const float* bias2, int N2, int K2,
+                                          int act2, int M, void* stream);
+
 // y[M, N] = act(sum of part[P, M, N] over P, in order, + bias) + add1 + add2: the reduction of the products above
 // on its own, for 32-bit partial sums over ranges of K that the vendor library's batched product made
 int pta_gemm_reduce_parts(void* y, const float* part, const float* bias, const void* add1, const void* add2, int M,

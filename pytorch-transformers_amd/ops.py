@@ -797,6 +797,45 @@ def gemm_splitk_pair_bf16(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tensor, 
     return y1, y2
 
 
+def gemm_splitk_pair_qkv(x1: torch.Tensor, w_qkv: torch.Tensor, bias_qkv, inv_freq, cs_scale: float, token_pos,
+                         token_seq, block_table, k_pool, v_pool, nh: int, nkv: int, d: int, layout: str,
+                         write_cache: bool, x2: torch.Tensor, w2: torch.Tensor, bias2=None, act2=None):
+    """The pair launch of a decode batch (17 to 256 rows) with its first product a fused query_key_value projection
+    taken to its end by the launch that adds the partial sums: returns (queries [M, nh, d] rotated,
+    act2(x2 @ w2.T + bias2)); keys and values are in the cache pages, as ``qkv_rope_cache`` leaves them."""
+    for name, t in (("x1", x1), ("w_qkv", w_qkv), ("x2", x2), ("w2", w2)):
+        _need(t, name, torch.bfloat16)
+    M = x1.shape[0]
+    N1, (N2, K2), K1 = (nh + 2 * nkv) * d, w2.shape, x1.shape[1]
+    if x2.shape[0] != M or tuple(w_qkv.shape) != (N1, K1) or x2.shape[1] != K2:
+        raise KernelError(f"a pair shares M: x1 {tuple(x1.shape)}, w_qkv {tuple(w_qkv.shape)} (wanted [{N1}, {K1}]), "
+                          f"x2 {tuple(x2.shape)}, w2 {tuple(w2.shape)}")
+    if d % 2:
+        raise KernelError(f"head size {d} must be even")
+    if bias_qkv is not None:
+        _need(bias_qkv, "bias_qkv", torch.float32, (N1,))
+    if bias2 is not None:
+        _need(bias2, "bias2", torch.float32, (N2,))
+    if inv_freq is not None:
+        _need(inv_freq, "inv_freq", torch.float32, (d // 2,))
+    _need(token_pos, "token_pos", torch.int32, (M,))
+    _need(token_seq, "token_seq", torch.int32, (M,))
+    _need(block_table, "block_table", torch.int32)
+    if block_table.dim() != 2:
+        raise KernelError("block_table must be [sequences, pages]")
+    _need_pools(k_pool, v_pool, torch.bfloat16, nkv, d)
+    p1, p2 = gemm_splitk_pair_parts(N1, K1, N2, K2)
+    part1 = torch.empty((p1, M, N1), dtype=torch.float32, device=x1.device)
+    part2 = torch.empty((p2, M, N2), dtype=torch.float32, device=x1.device)
+    q = torch.empty((M, nh, d), dtype=torch.bfloat16, device=x1.device)
+    y2 = torch.empty((M, N2), dtype=torch.bfloat16, device=x1.device)
+    _call("pta_gemm_splitk_pair_reduced_qkv_bf16", _ptr(q), _ptr(part1), _ptr(x1), _ptr(w_qkv), _ptr(bias_qkv), K1,
+          _ptr(inv_freq), ctypes.c_float(cs_scale), _ptr(token_pos), _ptr(token_seq), _ptr(block_table),
+          block_table.shape[1], _ptr(k_pool), _ptr(v_pool), nh, nkv, d, QKV_LAYOUT_CODES[layout], int(write_cache),
+          _ptr(y2), _ptr(part2), _ptr(x2), _ptr(w2), _ptr(bias2), N2, K2, ACT_CODES[act2], M, _stream())
+    return q, y2
+
+
 def gemm_partial_pair_ok(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tensor, w2: torch.Tensor) -> bool:
     """Whether two products onto the same features are best left as partial sums of one launch: up to 128
     rows each, and at least one of them worth leaving so on its own."""

@@ -119,6 +119,13 @@ class Linear(Part):
         # library's product for the feed-forward input is the faster one (64 rows: 23.3 against 24.3 ms)
         small = x1.shape[0] <= 48 or first.weight.numel() + second.weight.numel() <= PAIR_MAX_WEIGHTS
         if small and ops.gemm_splitk_pair_ok(x1, first.weight, x2, second.weight):
+            if tail is not None and ops.QKV_TAIL and kw1.get("act") is None and tail.head_dim % 2 == 0:
+                # the launch that adds the partial sums takes the fused rows to their end as well
+                q, y2 = ops.gemm_splitk_pair_qkv(
+                    x1, first.weight, tail.bias, tail.inv_freq, tail.cs_scale, tail.token_pos, tail.token_seq, tail.table,
+                    tail.k_pool, tail.v_pool, tail.num_heads, tail.kv_heads, tail.head_dim, tail.layout, tail.write_cache,
+                    x2, second.weight, b2, kw2.get("act"))
+                return TailDone(q), y2
             return ops.gemm_splitk_pair_bf16(*args)
         return None
 

@@ -414,6 +414,44 @@ def test_pair_launch_takes_the_fused_qkv_rows_to_their_end(layout, nh, nkv, d, r
     assert same(before, k1) and not torch.equal(q2, q1)
 
 
+@pytest.mark.parametrize("layout,nh,nkv,d,M", [("grouped", 4, 2, 24, 40), ("grouped", 8, 2, 128, 17), ("tail", 7, 1, 64, 150),
+                                               ("interleaved", 3, 3, 96, 64)])
+@pytest.mark.parametrize("rotary,bias", [(True, True), (False, False)])
+def test_batch_pair_launch_takes_the_fused_qkv_rows_to_their_end(layout, nh, nkv, d, M, rotary, bias):
+    """The same for a decode batch of 17 to 256 rows, where the launch that adds the partial sums carries the
+    tail: the queries and pages of the two products followed by the kernel of its own, bit for bit."""
+    ops = _ops()
+    K1, K2, N2 = 264, 328, 200
+    g = torch.Generator().manual_seed(M)
+    starts = torch.randint(0, 190, (M,), generator=g).tolist()
+    lens = [s + 1 for s in starts]
+    N1 = (nh + 2 * nkv) * d
+    x1, x2 = _rand(M, K1, dtype=torch.bfloat16), _rand(M, K2, seed=7, dtype=torch.bfloat16)
+    w1, w2 = _rand(N1, K1, seed=1, dtype=torch.bfloat16, scale=0.05), _rand(N2, K2, seed=2, dtype=torch.bfloat16, scale=0.05)
+    b1, b2 = (_rand(N1, seed=3) if bias else None), _rand(N2, seed=4)
+    token_seq = torch.arange(M, dtype=torch.int32).cuda()
+    token_pos = torch.tensor(starts, dtype=torch.int32).cuda()
+    inv = P.rope_inv_freq(d, 10000.0).cuda() if rotary else None
+    pools = []
+    for fused_way in (False, True):
+        k_pool, v_pool, bt, lists = _cache_setup(M, lens, nkv, d, torch.bfloat16, n_pages=3 * M + 8)
+        if fused_way:
+            q, y2 = ops.gemm_splitk_pair_qkv(x1, w1, b1, inv, 1.0, token_pos, token_seq, bt, k_pool, v_pool, nh, nkv, d,
+                                             layout, True, x2, w2, b2, "gelu")
+        else:
+            fused, y2 = ops.gemm_splitk_pair_bf16(x1, w1, x2, w2, None, None, b2, "gelu")
+            q = ops.qkv_rope_cache(fused, b1, inv, 1.0, token_pos, token_seq, bt, k_pool, v_pool, nh, nkv, d, layout)
+        pools.append((q, y2, k_pool, v_pool))
+    (q0, y0, k0, v0), (q1, y1, k1, v1) = pools
+    same = lambda a, b: torch.equal(torch.nan_to_num(a.float(), nan=-7.0), torch.nan_to_num(b.float(), nan=-7.0))
+    assert torch.equal(y0, y1) and torch.equal(q0, q1)
+    assert same(k0, k1) and same(v0, v1), "the same values at the same places of the pages, and nothing anywhere else"
+    before = k1.clone()
+    ops.gemm_splitk_pair_qkv(x1, w1 * 2, b1, inv, 1.0, token_pos, token_seq, bt, k1, v1, nh, nkv, d, layout, False, x2, w2,
+                             b2, "gelu")
+    assert same(before, k1)
+
+
 def _windowed_attention(q, k, v, window):
     """Plain attention in which query t sees keys t - window + 1 .. t; q [T, nh, d], k, v [T, nkv, d]."""
     T, nh, d = q.shape
