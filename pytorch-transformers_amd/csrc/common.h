@@ -39,14 +39,21 @@ __host__ __device__ __forceinline__ float bf16_bits_to_f32(bf16_t v) {
     return c.f;
 }
 
-// round to nearest, ties to even; NaN stays NaN
+// round to nearest, ties to even; NaN stays NaN.  On the device this is gfx950's own conversion instruction
+// (one for two values where the compiler can pair them); the host spells the same rounding out.
 __host__ __device__ __forceinline__ bf16_t f32_to_bf16_bits(float f) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    union { __bf16 b; bf16_t u; } c;
+    c.b = (__bf16)f;
+    return c.u;
+#else
     union { uint32_t u; float f; } c;
     c.f = f;
     uint32_t u = c.u;
     if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x0040u);
     u += 0x7fffu + ((u >> 16) & 1u);
     return (bf16_t)(u >> 16);
+#endif
 }
 
 __host__ __device__ __forceinline__ float round_to_bf16(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
@@ -108,9 +115,15 @@ __device__ __forceinline__ void unpack8(const uint4& u, float (&f)[8]) {
     }
 }
 __device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
+    typedef __bf16 bf16_pair __attribute__((ext_vector_type(2)));
+    typedef float f32_pair __attribute__((ext_vector_type(2)));
     uint32_t w[4];
 #pragma unroll
-    for (int p = 0; p < 4; ++p) w[p] = (uint32_t)f32_to_bf16_bits(f[2 * p]) | ((uint32_t)f32_to_bf16_bits(f[2 * p + 1]) << 16);
+    for (int p = 0; p < 4; ++p) {
+        union { bf16_pair b; uint32_t u; } c;
+        c.b = __builtin_convertvector(f32_pair{f[2 * p], f[2 * p + 1]}, bf16_pair);  // one instruction for the two
+        w[p] = c.u;
+    }
     return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
