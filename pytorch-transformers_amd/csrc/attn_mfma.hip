@@ -48,6 +48,14 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
     return c.u;
 }
 
+// the largest of three in one instruction; written out because the compiler, asked for fmaxf of values that
+// come through a branch, first makes each of them canonical with an instruction of its own
+__device__ __forceinline__ float max3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
 #define PTA_LOG2E 1.4426950408889634f
 
 template <int DT>
@@ -212,10 +220,11 @@ __global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
                     const int key = kb + 8 * gq + j;  // j = 4*tt + e
                     s[j] = sacc[j >> 2][ct][j & 3] * scale + round_to_bf16(slope[ct] * round_to_bf16((float)key)) * alibi_mul;
                 }
-            } else {
+            } else {  // left unscaled: the scale rides in the one multiply-add in front of the exponential
 #pragma unroll
-                for (int j = 0; j < 8; ++j) s[j] = sacc[j >> 2][ct][j & 3] * scale;
+                for (int j = 0; j < 8; ++j) s[j] = sacc[j >> 2][ct][j & 3];
             }
+            const float s_mul = slopes ? 1.0f : scale;  // what s is still to be multiplied by (positive)
             if (!interior) {
                 const int lim = min(qpos[ct] + 1, k_end);  // keys below this, and from `lo` on, count for the column
                 const int lo = window > 0 ? qpos[ct] - window + 1 : 0;
@@ -223,7 +232,9 @@ __global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
                 for (int j = 0; j < 8; ++j)
                     if (kb + 8 * gq + j >= lim || kb + 8 * gq + j < lo) s[j] = -INFINITY;
             }
-            float mx = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
+            const float mx3 = max3(s[6], s[7], max3(s[0], s[1], s[2]));
+            float mx = max3(s[3], s[4], s[5]);
+            mx = max3(mx, mx3, mx3) * s_mul;
             // The running maximum is only a reference point for the exponentials, shared by the four lanes of
             // a column; it is brought up to the true maximum (an exchange between those lanes, and a
             // rescale of what was summed) only when some score of the block lies more than 2^8 above it,
@@ -242,12 +253,12 @@ __global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
                 m_run[ct] = m_new;
             }
             const float m_use = m_run[ct] == -INFINITY ? 0.f : m_run[ct];
-            float p[8], psum = 0.f;
+            float p[8];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                p[j] = __builtin_amdgcn_exp2f(s[j] - m_use);
-                psum += p[j];
-            }
+            for (int j = 0; j < 8; ++j) p[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[j], s_mul, -m_use));
+            float psum = p[0];
+#pragma unroll
+            for (int j = 1; j < 8; ++j) psum += p[j];
             pf[ct].u = make_uint4(pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7]));
             l_run[ct] += psum;
         }
