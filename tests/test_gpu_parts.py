@@ -133,6 +133,8 @@ def test_rows_beyond_one_chunk_take_the_way_that_was_timed_faster(monkeypatch):
     from pytorch_transformers_amd import ops
     from pytorch_transformers_amd.parts import Linear
 
+    if ops.SPLITK_MAX_ROWS < 256:
+        pytest.skip("capped by PTA_SPLITK_MAX_ROWS")
     H, N1, N2, M = 264, 136, 200, 200
     first, second = Linear("a", H, N1, bias=True), Linear("b", H, N2, bias=False)
     (_, r1), (_, r2) = _fill(first, torch.bfloat16, 1), _fill(second, torch.bfloat16, 2)
@@ -161,6 +163,8 @@ def test_library_product_over_ranges_of_k():
     from pytorch_transformers_amd import ops
     from pytorch_transformers_amd.parts import Linear
 
+    if not ops.MM_KSPLIT:
+        pytest.skip("switched off by PTA_MM_KSPLIT=0")
     K, N, M = 640, 136, 300
     lin = Linear("a", K, N, bias=True)
     _, ref = _fill(lin, torch.bfloat16, 1)
