@@ -312,6 +312,14 @@ def test_generation_without_repeated_ngrams_equals_plain(folders):
     new = want[0][len(prompts[0]):]
     grams = [tuple(want[0][j:j + 3]) for j in range(len(want[0]) - 2)]
     assert len(set(grams)) == len(grams) and bad[0][0] not in new
+    # suppress_tokens never come, begin_suppress_tokens do not come first
+    first, second = free[0][len(prompts[0])], free[0][len(prompts[0]) + 1]
+    got = model.generate(prompts[:1], GenerationConfig(max_new_tokens=24, do_sample=False, eos_token_id=None,
+                                                       suppress_tokens=[second], begin_suppress_tokens=[first]))
+    new = got[0][len(prompts[0]):]
+    assert second not in new and new[0] != first
+    want_first = int(P.suppress(P.forward(cfg, w, prompts[0])[-1].float(), [first, second]).argmax())
+    assert new[0] == want_first
 
 
 def test_counter_based_uniforms():
