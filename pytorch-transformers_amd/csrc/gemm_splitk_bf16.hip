@@ -512,6 +512,20 @@ extern "C" int pta_gemm_splitk_pair_reduced_bf16(void* y1, float* part1, const v
     return pta_check_launch("gemm_splitk_pair_reduced_bf16");
 }
 
+// what the launches that take fused query_key_value rows to their end ask of their arguments
+static int check_qkv_tail(const char* what, const void* q_out, const int* token_pos, const int* token_seq,
+                          const int* block_table, const void* k_pool, const void* v_pool, int nh, int nkv, int d,
+                          int layout, int write_cache) {
+    PTA_REQUIRE(nh > 0 && nkv > 0 && d > 0 && nh % nkv == 0, "%s: heads %d, kv heads %d, head size %d", what, nh, nkv, d);
+    PTA_REQUIRE(d % 2 == 0, "%s: head size %d must be even", what, d);
+    PTA_REQUIRE(layout >= 0 && layout <= 2, "%s: unknown layout %d", what, layout);
+    PTA_REQUIRE(layout != PTA_QKV_TAIL || nkv == 1, "%s: the tail layout has one kv head, got %d", what, nkv);
+    PTA_REQUIRE(layout != PTA_QKV_INTERLEAVED || nkv == nh, "%s: the interleaved layout needs kv heads == heads", what);
+    PTA_REQUIRE(q_out && token_pos, "%s: null pointer", what);
+    PTA_REQUIRE(!write_cache || (k_pool && v_pool && block_table && token_seq), "%s: null cache pointer", what);
+    return 0;
+}
+
 // The same pair with the first product a fused query_key_value projection taken to its end: queries rotated in
 // q_out [M, heads, d], keys and values in the cache pages (as pta_qkv_rope_cache leaves them); even head sizes.
 extern "C" int pta_gemm_splitk_pair_reduced_qkv_bf16(void* q_out, float* part1, const void* x1, const void* W1,
@@ -521,13 +535,10 @@ extern "C" int pta_gemm_splitk_pair_reduced_qkv_bf16(void* q_out, float* part1, 
                                                      int layout, int write_cache, void* y2, float* part2, const void* x2,
                                                      const void* W2, const float* bias2, int N2, int K2, int act2, int M,
                                                      void* stream) {
-    PTA_REQUIRE(nh > 0 && nkv > 0 && d > 0 && nh % nkv == 0, "gemm_splitk_pair_reduced_qkv_bf16: heads %d, kv heads %d, head size %d", nh, nkv, d);
-    PTA_REQUIRE(d % 2 == 0, "gemm_splitk_pair_reduced_qkv_bf16: head size %d must be even", d);
-    PTA_REQUIRE(layout >= 0 && layout <= 2, "gemm_splitk_pair_reduced_qkv_bf16: unknown layout %d", layout);
-    PTA_REQUIRE(layout != PTA_QKV_TAIL || nkv == 1, "gemm_splitk_pair_reduced_qkv_bf16: the tail layout has one kv head, got %d", nkv);
-    PTA_REQUIRE(layout != PTA_QKV_INTERLEAVED || nkv == nh, "gemm_splitk_pair_reduced_qkv_bf16: the interleaved layout needs kv heads == heads");
-    PTA_REQUIRE(q_out && y2 && token_pos, "gemm_splitk_pair_reduced_qkv_bf16: null pointer");
-    PTA_REQUIRE(!write_cache || (k_pool && v_pool && block_table && token_seq), "gemm_splitk_pair_reduced_qkv_bf16: null cache pointer");
+    if (check_qkv_tail("gemm_splitk_pair_reduced_qkv_bf16", q_out, token_pos, token_seq, block_table, k_pool, v_pool, nh,
+                       nkv, d, layout, write_cache))
+        return 1;
+    PTA_REQUIRE(y2, "gemm_splitk_pair_reduced_qkv_bf16: null pointer");
     PTA_REQUIRE(pta_act_known(act2), "gemm_splitk_pair_reduced_qkv_bf16: unknown activation %d", act2);
     const int N1 = (nh + 2 * nkv) * d;
     const int rc = pta_gemm_splitk_pair_bf16(part1, x1, W1, N1, K1, part2, x2, W2, N2, K2, M, stream);
@@ -540,4 +551,28 @@ extern "C" int pta_gemm_splitk_pair_reduced_qkv_bf16(void* q_out, float* part1, 
     hipLaunchKernelGGL(gemm_splitk_reduce2_qkv_kernel, dim3((unsigned)((MN1 / 2 + MN2 + 255) / 256)), dim3(256), 0,
                        (hipStream_t)stream, tail, part1, bias1, MN1, N1, P1, (bf16_t*)y2, part2, bias2, MN2, N2, P2, act2);
     return pta_check_launch("gemm_splitk_pair_reduced_qkv_bf16");
+}
+
+// A fused query_key_value projection on its own (17 to 256 rows), taken to its end by the launch that adds its
+// partial sums: part [pta_gemm_splitk_parts(N, K, 0, 0), M, N] is the workspace, N = (nh + 2 nkv) d.
+extern "C" int pta_gemm_splitk_reduced_qkv_bf16(void* q_out, float* part, const void* x, const void* W,
+                                                const float* bias, int K, const float* inv_freq, float cs_scale,
+                                                const int* token_pos, const int* token_seq, const int* block_table,
+                                                int bt_stride, void* k_pool, void* v_pool, int nh, int nkv, int d,
+                                                int layout, int write_cache, int M, void* stream) {
+    if (check_qkv_tail("gemm_splitk_reduced_qkv_bf16", q_out, token_pos, token_seq, block_table, k_pool, v_pool, nh, nkv,
+                       d, layout, write_cache))
+        return 1;
+    PTA_REQUIRE(part, "gemm_splitk_reduced_qkv_bf16: null workspace");
+    const int N = (nh + 2 * nkv) * d;
+    const int rc = pta_gemm_splitk_bf16(nullptr, part, x, W, nullptr, nullptr, nullptr, M, N, K, PTA_ACT_NONE, 0, 0, 0, 0,
+                                        0, 0, stream);
+    if (rc) return rc;
+    const long MN = (long)M * N;
+    const QkvTail tail{(bf16_t*)q_out, inv_freq, cs_scale, token_pos, token_seq, block_table, bt_stride, (bf16_t*)k_pool,
+                       (bf16_t*)v_pool, nh, nkv, d, layout, write_cache};
+    hipLaunchKernelGGL(gemm_splitk_reduce2_qkv_kernel, dim3((unsigned)((MN / 2 + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, tail, part, bias, MN, N, pta_gemm_splitk_parts(N, K, 0, 0), (bf16_t*)nullptr,
+                       (const float*)nullptr, (const float*)nullptr, 0L, 1, 1, 0);
+    return pta_check_launch("gemm_splitk_reduced_qkv_bf16");
 }

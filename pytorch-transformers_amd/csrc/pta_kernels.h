@@ -115,6 +115,11 @@ int pta_gemm_splitk_pair_reduced_qkv_bf16(void* q_out, float* part1, const void*
                                           void* v_pool, int nh, int nkv, int d, int layout, int write_cache, void* y2,
                                           float* part2, const void* x2, const void* W2, const float* bias2, int N2, int K2,
                                           int act2, int M, void* stream);
+// such a projection on its own: part [pta_gemm_splitk_parts(N, K, 0, 0), M, N] is the workspace
+int pta_gemm_splitk_reduced_qkv_bf16(void* q_out, float* part, const void* x, const void* W, const float* bias, int K,
+                                     const float* inv_freq, float cs_scale, const int* token_pos, const int* token_seq,
+                                     const int* block_table, int bt_stride, void* k_pool, void* v_pool, int nh, int nkv,
+                                     int d, int layout, int write_cache, int M, void* stream);
 
 // y[M, N] = act(sum of part[P, M, N] over P, in order, + bias) + add1 + add2: the reduction of the products above
 // on its own, for 32-bit partial sums over ranges of K that the vendor library's batched product made

@@ -836,6 +836,38 @@ def gemm_splitk_pair_qkv(x1: torch.Tensor, w_qkv: torch.Tensor, bias_qkv, inv_fr
     return q, y2
 
 
+def gemm_splitk_qkv(x: torch.Tensor, w_qkv: torch.Tensor, bias_qkv, inv_freq, cs_scale: float, token_pos, token_seq,
+                    block_table, k_pool, v_pool, nh: int, nkv: int, d: int, layout: str, write_cache: bool):
+    """A fused query_key_value projection of a decode batch (17 to 256 rows) on its own, taken to its end by the
+    launch that adds its partial sums: returns the queries [M, nh, d] rotated; keys and values are in the cache
+    pages, as ``qkv_rope_cache`` leaves them."""
+    _need(x, "x", torch.bfloat16)
+    _need(w_qkv, "w_qkv", torch.bfloat16)
+    M, K = x.shape
+    N = (nh + 2 * nkv) * d
+    if tuple(w_qkv.shape) != (N, K):
+        raise KernelError(f"w_qkv {tuple(w_qkv.shape)}: wanted [{N}, {K}] for x {tuple(x.shape)}")
+    if d % 2:
+        raise KernelError(f"head size {d} must be even")
+    if bias_qkv is not None:
+        _need(bias_qkv, "bias_qkv", torch.float32, (N,))
+    if inv_freq is not None:
+        _need(inv_freq, "inv_freq", torch.float32, (d // 2,))
+    _need(token_pos, "token_pos", torch.int32, (M,))
+    _need(token_seq, "token_seq", torch.int32, (M,))
+    _need(block_table, "block_table", torch.int32)
+    if block_table.dim() != 2:
+        raise KernelError("block_table must be [sequences, pages]")
+    _need_pools(k_pool, v_pool, torch.bfloat16, nkv, d)
+    part = torch.empty((int(load_library().pta_gemm_splitk_parts(N, K, 0, 0)), M, N), dtype=torch.float32, device=x.device)
+    q = torch.empty((M, nh, d), dtype=torch.bfloat16, device=x.device)
+    _call("pta_gemm_splitk_reduced_qkv_bf16", _ptr(q), _ptr(part), _ptr(x), _ptr(w_qkv), _ptr(bias_qkv), K,
+          _ptr(inv_freq), ctypes.c_float(cs_scale), _ptr(token_pos), _ptr(token_seq), _ptr(block_table),
+          block_table.shape[1], _ptr(k_pool), _ptr(v_pool), nh, nkv, d, QKV_LAYOUT_CODES[layout], int(write_cache), M,
+          _stream())
+    return q
+
+
 def gemm_partial_pair_ok(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tensor, w2: torch.Tensor) -> bool:
     """Whether two products onto the same features are best left as partial sums of one launch: up to 128
     rows each, and at least one of them worth leaving so on its own."""

@@ -68,6 +68,8 @@ class AttentionMixer(Part):
         rotated it and written the cache."""
         k_pool, v_pool = ctx.cache.kv_layer(call.cache_group, call.cache_layer)
         table = ctx.block_tables[call.cache_group]
+        if projected is None:
+            projected = self.qkv.with_tail(x, self.projection_tail(ctx, call))
         if isinstance(projected, TailDone):
             q = projected.value
         else:

@@ -82,6 +82,16 @@ class Linear(Part):
             ops.epilogue_(y, bias, act, add1, add2)
         return y
 
+    def with_tail(self, x: torch.Tensor, tail: "QkvTail") -> Optional["TailDone"]:
+        """This product as a fused query_key_value projection whose launch also runs ``tail`` (a decode batch of
+        17 rows and more, where the product is the split-K kernel's); else None, and the caller runs the two."""
+        if not (ops.QKV_TAIL and x.dtype == torch.bfloat16 and tail.head_dim % 2 == 0
+                and not ops.gemm_skinny_ok(x, self.weight) and ops.gemm_splitk_ok(x, self.weight)):
+            return None
+        return TailDone(ops.gemm_splitk_qkv(
+            x, self.weight, tail.bias, tail.inv_freq, tail.cs_scale, tail.token_pos, tail.token_seq, tail.table,
+            tail.k_pool, tail.v_pool, tail.num_heads, tail.kv_heads, tail.head_dim, tail.layout, tail.write_cache))
+
     @staticmethod
     def pair(first: "Linear", x1: torch.Tensor, kw1: dict, second: "Linear", x2: torch.Tensor, kw2: dict, tail=None):
         """``(first(x1, **kw1), second(x2, **kw2))`` from one matrix launch, in steps small enough for the

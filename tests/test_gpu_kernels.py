@@ -454,6 +454,44 @@ def test_batch_pair_launch_takes_the_fused_qkv_rows_to_their_end(layout, nh, nkv
     assert same(before, k1)
 
 
+@pytest.mark.parametrize("layout,nh,nkv,d,M,K", [("grouped", 4, 2, 24, 40, 264), ("grouped", 8, 2, 128, 17, 2560),
+                                                 ("tail", 7, 1, 64, 150, 1032), ("interleaved", 3, 3, 96, 256, 4104)])
+@pytest.mark.parametrize("rotary,bias", [(True, True), (False, False)])
+def test_batch_launch_takes_the_fused_qkv_rows_to_their_end(layout, nh, nkv, d, M, K, rotary, bias):
+    """A query_key_value projection on its own, 17 to 256 rows, one range of K and several: the launch that adds
+    the partial sums carries the tail, and gives the queries and pages of the product followed by the kernel of
+    its own, bit for bit; with write_cache off the pages stay as they are."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(M)
+    starts = torch.randint(0, 190, (M,), generator=g).tolist()
+    lens = [s + 1 for s in starts]
+    N = (nh + 2 * nkv) * d
+    x = _rand(M, K, dtype=torch.bfloat16)
+    w = _rand(N, K, seed=1, dtype=torch.bfloat16, scale=0.05)
+    b = _rand(N, seed=3) if bias else None
+    token_seq = torch.arange(M, dtype=torch.int32).cuda()
+    token_pos = torch.tensor(starts, dtype=torch.int32).cuda()
+    inv = P.rope_inv_freq(d, 10000.0).cuda() if rotary else None
+    pools = []
+    for fused_way in (False, True):
+        k_pool, v_pool, bt, lists = _cache_setup(M, lens, nkv, d, torch.bfloat16, n_pages=3 * M + 8)
+        if fused_way:
+            q = ops.gemm_splitk_qkv(x, w, b, inv, 1.0, token_pos, token_seq, bt, k_pool, v_pool, nh, nkv, d, layout, True)
+        else:
+            fused = ops.gemm_splitk_bf16(x, w)
+            q = ops.qkv_rope_cache(fused, b, inv, 1.0, token_pos, token_seq, bt, k_pool, v_pool, nh, nkv, d, layout)
+        pools.append((q, k_pool, v_pool))
+    (q0, k0, v0), (q1, k1, v1) = pools
+    same = lambda a, b: torch.equal(torch.nan_to_num(a.float(), nan=-7.0), torch.nan_to_num(b.float(), nan=-7.0))
+    assert torch.equal(q0, q1)
+    assert same(k0, k1) and same(v0, v1), "the same values at the same places of the pages, and nothing anywhere else"
+    before = k1.clone()
+    q2 = ops.gemm_splitk_qkv(x, w * 2, b, inv, 1.0, token_pos, token_seq, bt, k1, v1, nh, nkv, d, layout, False)
+    assert same(before, k1) and not torch.equal(q2, q1)
+    with pytest.raises(ops.KernelError, match="w_qkv"):
+        ops.gemm_splitk_qkv(x, w[:-8], b, inv, 1.0, token_pos, token_seq, bt, k1, v1, nh, nkv, d, layout, False)
+
+
 def _windowed_attention(q, k, v, window):
     """Plain attention in which query t sees keys t - window + 1 .. t; q [T, nh, d], k, v [T, nkv, d]."""
     T, nh, d = q.shape

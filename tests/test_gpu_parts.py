@@ -244,6 +244,16 @@ def test_attention_mixer_and_blocks(dtype, rel, layout, nh, nkv, d, alibi, bias)
     res = run(lambda xs, ctx: mixer.forward(xs, ctx, call, residual=xs), cuts)
     _close(res, want_mixer + x.double(), rel, "mixer with residual")
 
+    # which way the 40-row step above went: its product's launch carries the tail where that product is the
+    # split-K kernel's (bfloat16, fewer fused rows than twice the width), else the tail is a kernel of its own
+    from pytorch_transformers_amd import ops
+    from pytorch_transformers_amd.parts.linear import TailDone
+    cache = PagedCache([CacheGroupSpec("kv", CACHE_FULL, 1, nkv, d)], 256, dtype, "cuda:0")
+    ctx, _ = _ctx(cache, [cache.alloc()], [40], dtype)
+    done = mixer.qkv.with_tail(x[:40].to(dtype).cuda(), mixer.projection_tail(ctx, call))
+    carried = dtype == torch.bfloat16 and ops.QKV_TAIL and (nh + 2 * nkv) * d < 2 * H
+    assert isinstance(done, TailDone) if carried else done is None
+
     # blocks: each arrangement is a decoder layer of the plain implementation with the matching flags
     for block, flags in ((ParallelBlock(mixer, ffn, n1), dict(parallel_attn=True, new_decoder_architecture=False)),
                          (SequentialBlock(mixer, ffn, n1, n2), dict(parallel_attn=False, new_decoder_architecture=False)),
