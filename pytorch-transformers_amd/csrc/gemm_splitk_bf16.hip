@@ -22,6 +22,11 @@
 
 #include <stdlib.h>
 
+#include <array>
+#include <map>
+#include <mutex>
+#include <utility>
+
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef int i32x4_t __attribute__((ext_vector_type(4)));
@@ -331,9 +336,23 @@ static int clamp_parts(int P, int K) { return max(1, min(min(P, 16), max(1, K / 
 // with many row tiles the ranges may be longer: fewer partial sums for the same number of workgroups
 static int range_for(int groups) { return SK_RANGE * max(1, groups / 64); }
 
+// Among the counts near that rule's, the one with the least (rounds of workgroups on the chip's 256 compute units)
+// x (a workgroup's fixed cost + the length of its range).  Measured at 32 to 128 rows: a launch just over a whole
+// number of rounds pays for the last one in full (Falcon-40B's fused QKV, 144 row tiles: 4 ranges, 2.25 rounds, 81
+// us; 3 ranges, 1.69 rounds, 65 us; Falcon-7B's, 73 row tiles: 8 ranges 31.6 us, 7 ranges 27.6 us), and the fixed
+// cost of a workgroup (start, first loads, its tile of partial sums) is that of some 1,300 elements of K.
+#define SK_WG_FIXED 1300
 static int pick_parts(int N, int K, int rt) {
     const int groups = (N + 64 * rt - 1) / (64 * rt), range = range_for(groups);
-    return clamp_parts(max((splitk_target() + groups - 1) / groups, (K + range / 2) / range), K);
+    const int p0 = clamp_parts(max((splitk_target() + groups - 1) / groups, (K + range / 2) / range), K);
+    auto cost = [&](int p) { return (((long)groups * p + 255) / 256) * (SK_WG_FIXED + K / p); };
+    static const bool balance = !getenv("PTA_SPLITK_BALANCE") || atoi(getenv("PTA_SPLITK_BALANCE")) != 0;
+    int best = p0;
+    for (int p = max(1, p0 - 2); balance && p <= p0 + 2; ++p) {
+        if (clamp_parts(p, K) != p || effective_parts(K, p) != p || (long)groups * p < 384) continue;
+        if (cost(p) < cost(best)) best = p;
+    }
+    return best;
 }
 
 extern "C" int pta_gemm_splitk_parts(int N, int K, int parts, int rt) {
@@ -458,7 +477,38 @@ extern "C" int pta_gemm_splitk_bf16(void* y, float* part, const void* x, const v
 
 // Ranges of K for the two products of a pair launch: each by its own length, and more of both if the launch
 // would have too few workgroups.
+// Counts that a caller has fixed for the pairs of one shape: no rule tells which neighbour of its choice is the
+// fastest (Falcon2-11B's output and feed-forward-down pair at 64 rows: 2 and 7 ranges by the rule; 4 and 8 make the
+// decode step 7 % faster, 2 and 10 make it 3 % slower with as many workgroups), so the Python side times them once.
+static std::map<std::array<int, 4>, std::pair<int, int>> pair_parts_fixed;
+static std::mutex pair_parts_lock;
+
+static bool parts_valid(int K, int p) { return p >= 1 && clamp_parts(p, K) == p && effective_parts(K, p) == p; }
+
+// p1 = p2 = 0 forgets the shape; returns 1 (no error text) for counts that the kernel does not take
+extern "C" int pta_gemm_splitk_pair_fix_parts(int N1, int K1, int N2, int K2, int p1, int p2) {
+    if (N1 <= 0 || K1 <= 0 || N2 <= 0 || K2 <= 0) return 1;
+    std::lock_guard<std::mutex> hold(pair_parts_lock);
+    const std::array<int, 4> key{N1, K1, N2, K2};
+    if (p1 == 0 && p2 == 0) {
+        pair_parts_fixed.erase(key);
+        return 0;
+    }
+    if (!parts_valid(K1, p1) || !parts_valid(K2, p2)) return 1;
+    pair_parts_fixed[key] = {p1, p2};
+    return 0;
+}
+
 static void pick_pair_parts(int N1, int K1, int N2, int K2, int* p1, int* p2) {
+    {
+        std::lock_guard<std::mutex> hold(pair_parts_lock);
+        const auto it = pair_parts_fixed.find({N1, K1, N2, K2});
+        if (it != pair_parts_fixed.end()) {
+            *p1 = it->second.first;
+            *p2 = it->second.second;
+            return;
+        }
+    }
     const int g1 = (N1 + 63) / 64, g2 = (N2 + 63) / 64;
     const int range = range_for(min(g1, g2));
     int a = clamp_parts((K1 + range / 2) / range, K1), b = clamp_parts((K2 + range / 2) / range, K2);

@@ -125,6 +125,9 @@ int pta_gemm_splitk_reduced_qkv_bf16(void* q_out, float* part, const void* x, co
 // on its own, for 32-bit partial sums over ranges of K that the vendor library's batched product made
 int pta_gemm_reduce_parts(void* y, const float* part, const float* bias, const void* add1, const void* add2, int M,
                           int N, int P, int act, int out_f32, void* stream);
+// fixes the ranges of K (1..16 each, as pta_gemm_splitk_pair_parts then reports them) for every later pair launch
+// of this shape; 0, 0 returns the shape to the built-in rule; returns 1 for counts the kernel does not take
+int pta_gemm_splitk_pair_fix_parts(int N1, int K1, int N2, int K2, int p1, int p2);
 int pta_gemm_splitk_pair_bf16(float* part1, const void* x1, const void* W1, int N1, int K1, float* part2,
                               const void* x2, const void* W2, int N2, int K2, int M, void* stream);
 

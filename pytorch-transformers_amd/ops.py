@@ -753,6 +753,47 @@ def gemm_splitk_pair_parts(N1: int, K1: int, N2: int, K2: int):
     return p1.value, p2.value
 
 
+# Ranges of K for the pairs of a shape: the kernel library's rule gives a choice, and its neighbours are timed
+# once per shape, at 64 rows, with cold caches; one that is at least 3 % faster is kept for every later launch
+# (PTA_PAIR_TUNE=0 switches this off).
+PAIR_TUNE = os.environ.get("PTA_PAIR_TUNE", "1") != "0"
+PAIR_TUNE_MARGIN = 0.97
+_pair_parts_tuned: dict = {}  # (shape of w1, shape of w2) -> the counts in use
+
+
+def tune_pair_parts(w1: torch.Tensor, w2: torch.Tensor) -> None:
+    key = (tuple(w1.shape), tuple(w2.shape))
+    if not PAIR_TUNE or key in _pair_parts_tuned or torch.cuda.is_current_stream_capturing():
+        return  # under capture nothing can be timed: the next eager step decides
+    lib = load_library()
+    (N1, K1), (N2, K2) = w1.shape, w2.shape
+    a0, b0 = gemm_splitk_pair_parts(N1, K1, N2, K2)
+    fix = lambda c: lib.pta_gemm_splitk_pair_fix_parts(int(N1), int(K1), int(N2), int(K2), int(c[0]), int(c[1]))
+    cands = [(a0, b0)] + [(a, b) for a in range(max(1, a0 - 1), a0 + 3) for b in range(max(1, b0 - 2), b0 + 3)
+                          if (a, b) != (a0, b0)]
+    cands = [c for c in cands if fix(c) == 0]
+    xs = [torch.randn((64, K), dtype=torch.float32, device=w1.device).to(torch.bfloat16) for K in (K1, K2)]
+    parts = [[torch.empty((c[i], 64, N), dtype=torch.float32, device=w1.device) for i, N in enumerate((N1, N2))]
+             for c in cands]
+
+    def way(c, out):
+        def run():
+            fix(c)
+            _call("pta_gemm_splitk_pair_bf16", _ptr(out[0]), _ptr(xs[0]), _ptr(w1), int(N1), int(K1), _ptr(out[1]),
+                  _ptr(xs[1]), _ptr(w2), int(N2), int(K2), 64, _stream())
+        return run
+
+    try:
+        times = _time_ways_cold([way(c, out) for c, out in zip(cands, parts)], w1.device)
+    finally:
+        fix((0, 0))
+    best = min(range(len(cands)), key=lambda i: times[i])
+    chosen = cands[best] if times[best] < PAIR_TUNE_MARGIN * times[0] else cands[0]
+    if chosen != cands[0]:
+        fix(chosen)
+    _pair_parts_tuned[key] = chosen
+
+
 def gemm_splitk_pair_partial(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tensor, w2: torch.Tensor):
     """(x1 @ w1.T, x2 @ w2.T), both left as 32-bit partial sums, in one launch; the products share M."""
     for name, t in (("x1", x1), ("w1", w1), ("x2", x2), ("w2", w2)):
@@ -761,8 +802,8 @@ def gemm_splitk_pair_partial(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tenso
     if x2.shape[0] != M or w1.dim() != 2 or w2.dim() != 2 or w1.shape[1] != x1.shape[1] or w2.shape[1] != x2.shape[1]:
         raise KernelError(f"a pair shares M: x1 {tuple(x1.shape)}, w1 {tuple(w1.shape)}, x2 {tuple(x2.shape)}, "
                           f"w2 {tuple(w2.shape)}")
-    lib = load_library()
     (N1, K1), (N2, K2) = w1.shape, w2.shape
+    tune_pair_parts(w1, w2)
     p1, p2 = gemm_splitk_pair_parts(N1, K1, N2, K2)
     part1 = torch.empty((p1, M, N1), dtype=torch.float32, device=x1.device)
     part2 = torch.empty((p2, M, N2), dtype=torch.float32, device=x1.device)
@@ -787,6 +828,7 @@ def gemm_splitk_pair_bf16(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tensor, 
         _need(bias1, "bias1", torch.float32, (N1,))
     if bias2 is not None:
         _need(bias2, "bias2", torch.float32, (N2,))
+    tune_pair_parts(w1, w2)
     p1, p2 = gemm_splitk_pair_parts(N1, K1, N2, K2)
     part1 = torch.empty((p1, M, N1), dtype=torch.float32, device=x1.device)
     part2 = torch.empty((p2, M, N2), dtype=torch.float32, device=x1.device)
@@ -824,6 +866,7 @@ def gemm_splitk_pair_qkv(x1: torch.Tensor, w_qkv: torch.Tensor, bias_qkv, inv_fr
     if block_table.dim() != 2:
         raise KernelError("block_table must be [sequences, pages]")
     _need_pools(k_pool, v_pool, torch.bfloat16, nkv, d)
+    tune_pair_parts(w_qkv, w2)
     p1, p2 = gemm_splitk_pair_parts(N1, K1, N2, K2)
     part1 = torch.empty((p1, M, N1), dtype=torch.float32, device=x1.device)
     part2 = torch.empty((p2, M, N2), dtype=torch.float32, device=x1.device)

@@ -224,6 +224,42 @@ def test_gemm_skinny_pair():
         ops.gemm_skinny_pair_bf16(x1, w1, x2[:3].contiguous(), w2)
 
 
+def test_pair_ranges_are_timed_once_per_shape_and_kept():
+    """The ranges of K of a pair: the rule's choice or a timed neighbour of it, the same for every later launch of
+    the shape (so the workspace that is asked for fits, and a row alone has the bits it has in the batch), reported
+    by gemm_splitk_pair_parts; counts that the kernel does not take are refused; 0, 0 returns to the rule."""
+    ops = _ops()
+    lib = ops.load_library()
+    M, K1, K2, N1, N2 = 48, 2112, 4608, 320, 192
+    x1, x2 = _rand(M, K1, dtype=torch.bfloat16), _rand(M, K2, seed=5, dtype=torch.bfloat16)
+    w1, w2 = _rand(N1, K1, seed=1, dtype=torch.bfloat16, scale=0.05), _rand(N2, K2, seed=2, dtype=torch.bfloat16, scale=0.05)
+    rule = ops.gemm_splitk_pair_parts(N1, K1, N2, K2)
+    y1, y2 = ops.gemm_splitk_pair_bf16(x1, w1, x2, w2)
+    key = ((N1, K1), (N2, K2))
+    if ops.PAIR_TUNE:
+        kept = ops._pair_parts_tuned[key]
+        assert abs(kept[0] - rule[0]) <= 2 and abs(kept[1] - rule[1]) <= 2
+        assert ops.gemm_splitk_pair_parts(N1, K1, N2, K2) == kept
+    p1, p2 = ops.gemm_splitk_pair_parts(N1, K1, N2, K2)
+    assert torch.equal(y1, ops.gemm_splitk_bf16(x1, w1, rt=1, parts=p1)) and torch.equal(y2, ops.gemm_splitk_bf16(x2, w2, rt=1, parts=p2))
+    for y, x, w in ((y1, x1, w1), (y2, x2, w2)):
+        want = (x.double() @ w.double().T).float()
+        torch.testing.assert_close(y.float(), want, rtol=2e-2, atol=2e-2 * float(want.abs().max()))
+    a1, a2 = ops.gemm_splitk_pair_bf16(x1[20:37].contiguous(), w1, x2[20:37].contiguous(), w2)
+    assert torch.equal(a1, y1[20:37]) and torch.equal(a2, y2[20:37])
+    assert lib.pta_gemm_splitk_pair_fix_parts(N1, K1, N2, K2, 5, 2) == 1, "2,112 elements are no five ranges of 512 and more"
+    assert lib.pta_gemm_splitk_pair_fix_parts(N1, K1, N2, K2, 1, 17) == 1
+    try:
+        assert lib.pta_gemm_splitk_pair_fix_parts(N1, K1, N2, K2, 1, 3) == 0
+        assert ops.gemm_splitk_pair_parts(N1, K1, N2, K2) == (1, 3)
+        z1, z2 = ops.gemm_splitk_pair_bf16(x1, w1, x2, w2)
+        assert torch.equal(z1, ops.gemm_splitk_bf16(x1, w1, rt=1, parts=1)) and torch.equal(z2, ops.gemm_splitk_bf16(x2, w2, rt=1, parts=3))
+    finally:
+        assert lib.pta_gemm_splitk_pair_fix_parts(N1, K1, N2, K2, 0, 0) == 0
+        ops._pair_parts_tuned.pop(key, None)
+    assert ops.gemm_splitk_pair_parts(N1, K1, N2, K2) == rule
+
+
 def test_gemm_splitk_pair():
     """Two products of one launch, run to the end, against the products on their own."""
     ops = _ops()
