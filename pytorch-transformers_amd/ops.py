@@ -762,6 +762,8 @@ _pair_parts_tuned: dict = {}  # (shape of w1, shape of w2) -> the counts in use
 
 
 def tune_pair_parts(w1: torch.Tensor, w2: torch.Tensor) -> None:
+    """Once per pair of shapes: time the pair launch with the rule's ranges of K and with their neighbours, and fix
+    the fastest in the kernel library if it beats the rule's by the margin (``_pair_parts_tuned`` says which)."""
     key = (tuple(w1.shape), tuple(w2.shape))
     if not PAIR_TUNE or key in _pair_parts_tuned or torch.cuda.is_current_stream_capturing():
         return  # under capture nothing can be timed: the next eager step decides
