@@ -626,3 +626,52 @@ extern "C" int pta_gemm_splitk_reduced_qkv_bf16(void* q_out, float* part, const 
                        (const float*)nullptr, (const float*)nullptr, 0L, 1, 1, 0);
     return pta_check_launch("gemm_splitk_reduced_qkv_bf16");
 }
+
+// ---- the same product for callers that cannot allocate ---------------------------------------------------
+// The 32-bit partial sums of the ranges of K lie in a file-scope device array instead of a workspace that the
+// caller brings.  Every GPU holds its own copy of the array at its own address until the process ends; its
+// address is asked from the runtime once per device, with that device current, and only that address is ever
+// handed to a kernel or a runtime call (the array's name in host code is a stand-in, no device address).
+#define PTA_STATIC_PART_FLOATS (4 * 1024 * 1024)  // 16 MiB per GPU
+#define PTA_MAX_DEVICES 64
+static __device__ __align__(256) float scratch[PTA_STATIC_PART_FLOATS];
+static float* scratch_ptr[PTA_MAX_DEVICES] = {nullptr};
+static std::mutex scratch_lock;
+
+// the current device's copy of `scratch`; null after storing the reason
+static float* static_workspace() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= PTA_MAX_DEVICES) {
+        pta_fail("gemm_splitk_bf16_static: no current device (or more than %d devices)", PTA_MAX_DEVICES);
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> hold(scratch_lock);
+    if (!scratch_ptr[dev]) {
+        void* p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            pta_fail("gemm_splitk_bf16_static: the workspace's address on device %d is not known: %s", dev,
+                     hipGetErrorString(e));
+            return nullptr;
+        }
+        scratch_ptr[dev] = (float*)p;
+    }
+    return scratch_ptr[dev];
+}
+
+extern "C" long pta_gemm_splitk_static_floats(void) { return PTA_STATIC_PART_FLOATS; }
+
+extern "C" int pta_gemm_splitk_bf16_static(void* y, const void* x, const void* W, const float* bias, const void* add1,
+                                           const void* add2, int M, int N, int K, int act, int out_f32, void* stream) {
+    if (check_splitk("gemm_splitk_bf16_static", x, W, M, N, K)) return 1;
+    const long need = (long)pta_gemm_splitk_parts(N, K, 0, 0) * M * N;
+    PTA_REQUIRE(need <= (long)PTA_STATIC_PART_FLOATS,
+                "gemm_splitk_bf16_static: %d ranges of K x %d rows x %d features are %ld partial sums, the built-in "
+                "workspace holds %d (bring a workspace to pta_gemm_splitk_bf16 instead)",
+                pta_gemm_splitk_parts(N, K, 0, 0), M, N, need, PTA_STATIC_PART_FLOATS);
+    float* part = static_workspace();
+    if (!part) return 1;
+    // every partial sum that the reduction reads is written by this call's matrix launch first, so nothing of
+    // the array has to start at zero
+    return pta_gemm_splitk_bf16(y, part, x, W, bias, add1, add2, M, N, K, act, out_f32, 0, 0, 0, 0, 1, stream);
+}

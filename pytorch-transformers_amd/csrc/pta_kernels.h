@@ -136,6 +136,18 @@ int pta_gemm_splitk_pair_reduced_bf16(void* y1, float* part1, const void* x1, co
                                       int K1, int act1, void* y2, float* part2, const void* x2, const void* W2,
                                       const float* bias2, int N2, int K2, int act2, int M, void* stream);
 
+// pta_gemm_splitk_bf16 (rt, parts, stage_blocks, depth chosen, reduce = 1) for callers that cannot allocate device
+// memory: code under HIP graph capture, tight serving loops, harnesses that forbid it.  It has no counterpart in
+// the reference.  The partial sums lie in an array that the library holds on every GPU it runs on until the
+// process ends (pta_gemm_splitk_static_floats() 32-bit values, 16 MiB); a product whose ranges x M x N exceed that
+// is refused with a message.  The call allocates and frees nothing.  All calls on one GPU share that GPU's array,
+// which keeps the last call's contents (nothing in it has to start at zero: a call writes every partial sum
+// before it reads it): calls that overlap on one GPU (two streams, two threads) race and must be ordered by the
+// caller.
+int pta_gemm_splitk_bf16_static(void* y, const void* x, const void* W, const float* bias, const void* add1,
+                                const void* add2, int M, int N, int K, int act, int out_f32, void* stream);
+long pta_gemm_splitk_static_floats(void);
+
 // processors in the reference's order, then argmax (do_sample 0) or a draw; `work` [R, V] is scratch and,
 // with want_scores, receives the processed scores (without, its contents are unspecified);
 // typical_p 1, epsilon_cutoff 0 and eta_cutoff 0 switch those off; hist/hist_off (tokens seen, per row),
