@@ -1,8 +1,8 @@
 """Replaying a trace: requests named by ids, fed step by step through a model's step function.
 
 One record of a trace is a dict ``{"step": k, "entries": [{"id", "tokens", "want"}...], "end": [ids]}``.
-The requests of a step either all start or all go on; a request holds a cache slot from its first
-step until a record's ``end`` names it.  This is the whole of the program ``bin/trace_run`` apart
+A step may hold any mix: whole prompts, pieces of prompts and single tokens of requests that are
+already running; a request holds a cache slot from its first step until a record's ``end`` names it.  This is the whole of the program ``bin/trace_run`` apart
 from reading lines and writing files, and what the tests drive in-process.
 """
 from __future__ import annotations

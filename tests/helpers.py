@@ -60,6 +60,36 @@ def schedule_batches(reqs: Dict[str, List[int]], batch_size: int, decode: Sequen
     return out
 
 
+def schedule_staggered(reqs: Dict[str, List[int]], start_every: int = 2, decode: Sequence[int] = (6, 2, 11, 4),
+                       chunks: Sequence = (None, 5, 19, 1)) -> List[dict]:
+    """Requests join while others run: request i starts at step ``i * start_every``.  Its prompt (all but its last
+    ``decode[i]`` tokens) comes whole (``chunks[i]`` None) or in pieces of ``chunks[i]`` tokens over consecutive
+    steps, then one token a step.  So a step may hold single tokens of running requests beside whole or partial
+    prompts of new ones; requests end at different steps, and later ones take the slots and pages they gave back."""
+    ids = list(reqs)
+    todo = {}
+    for i, rid in enumerate(ids):
+        toks = reqs[rid]
+        head = max(1, len(toks) - decode[i % len(decode)])
+        size = chunks[i % len(chunks)] or head
+        pieces = [toks[a:min(a + size, head)] for a in range(0, head, size)] + [[t] for t in toks[head:]]
+        todo[rid] = (i * start_every, pieces)
+    out, k = [], 0
+    while any(pieces for _, pieces in todo.values()):
+        entries, end = [], []
+        for rid in ids:
+            start, pieces = todo[rid]
+            if k < start or not pieces:
+                continue
+            piece = pieces.pop(0)
+            entries.append({"id": rid, "tokens": piece, "want": list(range(len(piece)))})
+            if not pieces:
+                end.append(rid)
+        out.append({"step": k, "entries": entries, "end": end})
+        k += 1
+    return out
+
+
 def run_schedule(replayer, records: List[dict]) -> Dict[str, torch.Tensor]:
     """Replay ``records``; gather the logits of every wanted place per request, in position order."""
     got: Dict[str, Dict[int, torch.Tensor]] = {}

@@ -1,7 +1,7 @@
 """A plain, slow Falcon: whole sequences, no cache, one function per part.
 
-Written from the reference's formulas (each function cites file:line under
-/root/reference); it imports nothing from the engine, reads ``config.json`` as
+Written from the reference's formulas (each function cites file:line of the
+reference checkout); it imports nothing from the engine, reads ``config.json`` as
 a dict and the weights with safetensors' own loader.  Arithmetic is float64 by
 default, so what the 32-bit engine is compared with is closer to exact than the
 engine itself; the places where the reference rounds on purpose (ALiBi's
@@ -230,6 +230,8 @@ def activation(x, name):
         return x * torch.sigmoid(1.702 * x)
     if name == "gelu_10":  # :113
         return torch.clip(gelu(x), -10, 10)
+    if name == "laplace":  # :176-178
+        return 0.5 * (1.0 + torch.erf((x - 0.707107) / (0.282095 * math.sqrt(2.0))))
     table = {"relu": F.relu, "relu6": F.relu6, "silu": F.silu, "swish": F.silu, "sigmoid": torch.sigmoid,
              "tanh": torch.tanh, "leaky_relu": F.leaky_relu, "mish": F.mish, "linear": lambda t: t,
              "relu2": lambda t: torch.square(F.relu(t))}  # :172

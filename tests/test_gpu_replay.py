@@ -47,14 +47,17 @@ def _replayer(folder, dtype, max_tokens=2048):
 @pytest.mark.parametrize("dtype,rel", [("float32", REL_F32), ("bfloat16", REL_BF16)])
 @pytest.mark.parametrize("name", sorted(TINY))
 def test_schedules_match_plain(folders, plain_cache, name, dtype, rel):
-    """Whole / last 32 one by one / unequal batches with slot reuse: all equal the plain logits."""
+    """Whole / last 32 one by one / unequal batches with slot reuse / requests that join while others decode, with
+    prompts in pieces: all equal the plain logits."""
     reqs, want = _plain(folders, plain_cache, name)
     rp = _replayer(folders[name], dtype)
     results = {}
     for sched_name, records in (("whole", helpers.schedule_whole(reqs)),
                                 ("tail32", helpers.schedule_tail(reqs, 32)),
                                 ("batches", helpers.schedule_batches(reqs, 4)),
-                                ("batches-again", helpers.schedule_batches(reqs, 3, decode=(20, 2, 7)))):
+                                ("batches-again", helpers.schedule_batches(reqs, 3, decode=(20, 2, 7))),
+                                ("staggered", helpers.schedule_staggered(reqs)),
+                                ("staggered-again", helpers.schedule_staggered(reqs, 1, decode=(1, 30, 3), chunks=(7, None, 64)))):
         got = helpers.run_schedule(rp, records)
         assert not rp.slots and not rp.cache.live_slots(), "slots left behind"
         assert rp.cache.free_pages() == rp.cache.num_pages, "pages left behind"
@@ -63,7 +66,7 @@ def test_schedules_match_plain(folders, plain_cache, name, dtype, rel):
         results[sched_name] = got
     if dtype == "float32":
         # fixed summation orders: how the tokens were cut and batched changes no bit
-        for sched_name in ("tail32", "batches", "batches-again"):
+        for sched_name in ("tail32", "batches", "batches-again", "staggered", "staggered-again"):
             for rid in reqs:
                 assert torch.equal(results[sched_name][rid], results["whole"][rid]), \
                     f"{name} float32: {sched_name} differs from whole for {rid}"

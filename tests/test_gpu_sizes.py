@@ -46,13 +46,18 @@ def test_layer_sizes_match_plain(tmp_path, name):
     folder = write_random_model(os.path.join(str(tmp_path), name), cfg, seed=11, noise=0.1)
     reqs = helpers.make_requests(cfg.vocab_size, LENGTHS, seed=5)
     want = helpers.plain_logits(folder, reqs)
+    first_f32 = {}
     for dtype, rel in (("float32", REL_F32), ("bfloat16", REL_BF16)):
         model = AutoModelForCausalLM.from_pretrained(folder, dtype=dtype)
         rp = Replayer(model, 1024)
         for sched, records in (("whole", helpers.schedule_whole(reqs)), ("tail32", helpers.schedule_tail(reqs, 32)),
-                               ("batches", helpers.schedule_batches(reqs, 2, decode=(3, 9)))):
+                               ("batches", helpers.schedule_batches(reqs, 2, decode=(3, 9))),
+                               ("staggered", helpers.schedule_staggered(reqs, 2, decode=(6, 2, 11), chunks=(None, 5, 19)))):
             got = helpers.run_schedule(rp, records)
             for rid in reqs:
                 helpers.assert_close(got[rid], want[rid], rel, f"{name} {dtype} {sched} {rid}")
+                if dtype == "float32":
+                    first = first_f32.setdefault(rid, got[rid])
+                    assert torch.equal(got[rid], first), f"{name} float32: {sched} differs from whole for {rid}"
         del rp, model
         torch.cuda.empty_cache()

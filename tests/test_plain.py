@@ -38,6 +38,37 @@ def test_gelu_is_the_erf_form():
     assert not torch.allclose(P.gelu(x), F.gelu(x, approximate="tanh"), atol=1e-6, rtol=0)
 
 
+def test_hand_written_activations_against_torchs_own():
+    """The activations that the plain table spells out by hand, on the reference's vector
+    (tests/utils/test_activations.py:29-33) and on a denser one, each against a torch routine or an
+    independent spelling; fails for a wrong constant (1.702, 0.044715, sqrt(2/pi)), a missing clip, a cube
+    taken of the wrong term or a square in front of the relu."""
+    for x in (torch.tensor([-100, -1, -0.1, 0, 0.1, 1.0, 100], dtype=D), torch.linspace(-6, 6, 97, dtype=D)):
+        tanh_form = F.gelu(x, approximate="tanh")
+        for name in ("gelu_new", "gelu_pytorch_tanh", "gelu_accurate", "gelu_fast"):
+            torch.testing.assert_close(P.activation(x, name), tanh_form, rtol=1e-8, atol=1e-9)
+        torch.testing.assert_close(P.activation(x, "gelu_python"), F.gelu(x))
+        torch.testing.assert_close(P.activation(x, "quick_gelu"), x / (1 + torch.exp(-1.702 * x)))
+        torch.testing.assert_close(P.activation(x, "gelu_10"), torch.clamp(F.gelu(x), -10, 10))
+        torch.testing.assert_close(P.activation(x, "relu2"), torch.where(x > 0, x * x, torch.zeros_like(x)))
+        torch.testing.assert_close(P.activation(x, "silu"), x * torch.sigmoid(x))
+        torch.testing.assert_close(P.activation(x, "swish"), F.silu(x))
+        torch.testing.assert_close(P.activation(x, "mish"), x * torch.tanh(F.softplus(x)))
+        torch.testing.assert_close(P.activation(x, "leaky_relu"), torch.where(x > 0, x, 0.01 * x))
+        torch.testing.assert_close(P.activation(x, "relu6"), torch.clamp(x, 0, 6))
+        # the Laplace activation is the normal distribution function with mean 0.707107 and deviation 0.282095
+        # (src/transformers/activations.py:176-178)
+        normal = torch.distributions.Normal(torch.tensor(0.707107, dtype=D), torch.tensor(0.282095, dtype=D))
+        torch.testing.assert_close(P.activation(x, "laplace"), normal.cdf(x), rtol=1e-7, atol=1e-12)
+    x = torch.tensor([-100, -1, -0.1, 0, 0.1, 1.0, 100], dtype=D)
+    # tests/utils/test_activations.py:35-47: clipped at 10, equal to the exact form below the clip
+    y, y10 = P.activation(x, "gelu"), P.activation(x, "gelu_10")
+    assert float(y10.max()) == 10.0 and float(y.max()) == 100.0
+    torch.testing.assert_close(y10[:-1], y[:-1])
+    assert not torch.allclose(P.activation(x, "gelu_new"), y, atol=1e-6, rtol=0)  # :29-33
+    assert not torch.allclose(P.activation(x, "quick_gelu"), y, atol=1e-4, rtol=0)
+
+
 # --- rotary ---------------------------------------------------------------------------------
 def test_rope_inv_freq_vector():
     """tests/utils/test_modeling_rope_utils.py:133-166: d=128, theta=1e4."""
@@ -105,6 +136,27 @@ def test_rope_hand_case_pairs_and_sign():
     c0, s0, c1, s1 = math.cos(1.0), math.sin(1.0), math.cos(0.5), math.sin(0.5)
     want = torch.tensor([1 * c0 - 3 * s0, 2 * c1 - 4 * s1, 3 * c0 + 1 * s0, 4 * c1 + 2 * s1], dtype=D)
     torch.testing.assert_close(out, want, rtol=1e-6, atol=1e-7)
+
+
+def test_rope_is_a_complex_multiplication_of_half_split_pairs():
+    """An independent spelling: z_i = x[i] + j x[i + d/2] times e^{j pos inv_freq[i]}.  Fails for a flipped sign
+    of the sine (the conjugate rotation) and for interleaved pairs (2i, 2i + 1)."""
+    d, T = 16, 5
+    x = rnd(T, 3, d)
+    inv = P.rope_inv_freq(d, 10000.0)
+    pos = torch.tensor([0, 1, 7, 30, 200])
+    cos, sin = P.rope_cos_sin(pos, inv)
+    got = P.apply_rope(x, cos, sin)
+    ang = pos.float()[:, None] * inv[None, :]  # 32-bit angles, as the reference forms them
+    turn = torch.complex(torch.cos(ang).double(), torch.sin(ang).double())[:, None, :]
+    z = torch.complex(x[..., :d // 2], x[..., d // 2:]) * turn
+    torch.testing.assert_close(got, torch.cat((z.real, z.imag), dim=-1), rtol=1e-9, atol=1e-12)
+    z_conj = torch.complex(x[..., :d // 2], x[..., d // 2:]) * turn.conj()
+    assert not torch.allclose(got[1:], torch.cat((z_conj.real, z_conj.imag), dim=-1)[1:], atol=1e-3)
+    zi = torch.complex(x[..., 0::2], x[..., 1::2]) * turn  # the interleaved convention, which this is not
+    inter = torch.stack((zi.real, zi.imag), dim=-1).reshape(T, 3, d)
+    assert not torch.allclose(got[1:], inter[1:], atol=1e-3)
+    torch.testing.assert_close(got[0], x[0])
 
 
 def test_rope_invariants():
@@ -267,6 +319,48 @@ def test_residual_arrangements(models):
     want = r + P.mlp(P.layer_norm(r, w[p + "post_attention_layernorm.weight"], w[p + "post_attention_layernorm.bias"], 1e-6),
                      w, p + "mlp.")
     torch.testing.assert_close(P.decoder_layer(x, w, 0, c, pos), want)
+
+
+def test_sequential_block_by_special_cases(models):
+    """The sequential arrangement (modeling_falcon.py:652-659, :676) pinned without recomputing it the same way:
+    a silent attention (output matrix and bias zero) leaves x + mlp(post_norm(x)); a silent feed-forward leaves
+    x + attention(input_norm(x)), with no trace of the second norm; and the two norms are not interchangeable
+    (fails for a post norm applied to x instead of x + attention, or for the norms swapped)."""
+    cfg, w = models["B"]
+    c = P.cfg_defaults(cfg)
+    assert not c["parallel_attn"] and not c["new_decoder_architecture"]
+    p = "transformer.h.1."
+    eps = c["layer_norm_epsilon"]
+    x = rnd(7, c["hidden_size"], seed=5)
+    pos = torch.arange(7)
+    ln_in = lambda t, ww=w: P.layer_norm(t, ww[p + "input_layernorm.weight"], ww[p + "input_layernorm.bias"], eps)
+    ln_post = lambda t, ww=w: P.layer_norm(t, ww[p + "post_attention_layernorm.weight"], ww[p + "post_attention_layernorm.bias"], eps)
+
+    def silenced(*names):
+        out = dict(w)
+        for n in names:
+            out[p + n] = torch.zeros_like(w[p + n])
+        return out
+
+    no_attn = silenced("self_attention.dense.weight", "self_attention.dense.bias")
+    torch.testing.assert_close(P.decoder_layer(x, no_attn, 1, c, pos), x + P.mlp(ln_post(x), w, p + "mlp."))
+    no_ffn = silenced("mlp.dense_4h_to_h.weight", "mlp.dense_4h_to_h.bias")
+    attn = P.self_attention(ln_in(x), w, p + "self_attention.", c, pos)
+    torch.testing.assert_close(P.decoder_layer(x, no_ffn, 1, c, pos), x + attn)
+    changed = dict(no_ffn)  # ... whatever the second norm holds
+    changed[p + "post_attention_layernorm.weight"] = w[p + "post_attention_layernorm.weight"] * 3 + 1
+    torch.testing.assert_close(P.decoder_layer(x, changed, 1, c, pos), x + attn)
+    # the feed-forward reads the norm of x + attention: with attention on, the result is not
+    # x + attention + mlp(post_norm(x)) ...
+    full = P.decoder_layer(x, w, 1, c, pos)
+    assert not torch.allclose(full, x + attn + P.mlp(ln_post(x), w, p + "mlp."), atol=1e-6)
+    torch.testing.assert_close(full, (x + attn) + P.mlp(ln_post(x + attn), w, p + "mlp."))
+    # ... and swapping the two norms' parameters changes it
+    swapped = dict(w)
+    for s_ in ("weight", "bias"):
+        swapped[p + "input_layernorm." + s_] = w[p + "post_attention_layernorm." + s_]
+        swapped[p + "post_attention_layernorm." + s_] = w[p + "input_layernorm." + s_]
+    assert not torch.allclose(P.decoder_layer(x, swapped, 1, c, pos), full, atol=1e-6)
 
 
 def test_two_equal_norms_are_one_norm(models):
