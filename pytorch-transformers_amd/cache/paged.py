@@ -15,7 +15,10 @@ layer group owns a pool of pages of ``page_size`` tokens; a slot's keys and
 values are the pages its page list names, in order, so the position of a key is
 its index in the slot.  Slots and pages go back to free lists when a sequence
 ends and are handed out again; nothing is zeroed, because a slot's length says
-what is valid.  A group of kind ``window`` is laid out like a full one, but gives the pages that lie
+what is valid.  Beyond the pages and slots that sequences can hold, every pool has one more page and every
+state table one more row (``scratch_page``, ``scratch_slot``) that no sequence ever owns: rows that pad a
+step to a fixed batch size (a captured decode step) write there, so that padding touches no sequence's
+keys, values or state.  A group of kind ``window`` is laid out like a full one, but gives the pages that lie
 wholly behind its window back to its pool as a sequence grows (their places in the page list hold
 -1), so a long sequence holds about ``window / page_size`` pages of it.  Groups of kind ``state`` own a ``[max_slots, *shape]`` table per
 layer that is zeroed when a slot is handed out.
@@ -60,13 +63,15 @@ class _Group:
         if self.paged:
             # values are held transposed inside a page so that the attention kernels read eight
             # consecutive positions of one feature in one load
-            self.k = torch.zeros((spec.num_layers, num_pages, spec.kv_heads, page_size, spec.head_dim),
+            # (one page more than sequences can hold: the scratch page of padding rows)
+            self.k = torch.zeros((spec.num_layers, num_pages + 1, spec.kv_heads, page_size, spec.head_dim),
                                  dtype=dtype, device=device)
-            self.v = torch.zeros((spec.num_layers, num_pages, spec.kv_heads, spec.head_dim, page_size),
+            self.v = torch.zeros((spec.num_layers, num_pages + 1, spec.kv_heads, spec.head_dim, page_size),
                                  dtype=dtype, device=device)
         elif spec.kind == CACHE_STATE:
             sd = spec.state_dtype or torch.float32
-            self.state = torch.zeros((spec.num_layers, max_slots, *spec.state_shape), dtype=sd, device=device)
+            # (one row more than there are slots: the scratch slot of padding rows)
+            self.state = torch.zeros((spec.num_layers, max_slots + 1, *spec.state_shape), dtype=sd, device=device)
         else:
             raise CacheError(f"cache group {spec.name!r}: unknown kind {spec.kind!r}")
 
@@ -106,6 +111,16 @@ class PagedCache:
         for i, name in enumerate(self._paged):  # the runtime knows groups by number
             msg = msg.replace(f"group {i} ", f"group {name!r} ")
         raise (CacheFull if rc == host.ERR_FULL else CacheError)(msg)
+
+    @property
+    def scratch_slot(self) -> int:
+        """A row of every state table that no sequence owns: where padding rows of a step keep their state."""
+        return self.max_slots
+
+    @property
+    def scratch_page(self) -> int:
+        """A page of every pool that no sequence owns: where padding rows of a step write keys and values."""
+        return self.num_pages
 
     @property
     def handle(self):
@@ -177,6 +192,29 @@ class PagedCache:
 
     def state_layer(self, group: str, layer: int) -> torch.Tensor:
         return self.groups[group].state[layer]
+
+    # fixed-size state: copies out and back -------------------------------------------------
+    def snapshot_state(self, slot: int) -> Dict[str, torch.Tensor]:
+        """A copy of everything of fixed size that ``slot`` holds, per state group ``[layers, *shape]`` (the
+        reference clones its state tables when a sequence forks, src/transformers/cache_utils.py:1813-1847)."""
+        if not self._lib.ptah_is_live(self._h, int(slot)):
+            raise CacheError(f"slot {slot} is not allocated")
+        return {name: g.state[:, int(slot)].clone() for name, g in self.groups.items() if g.state is not None}
+
+    def restore_state(self, slot: int, snapshot: Dict[str, torch.Tensor]) -> None:
+        """Put a ``snapshot_state`` back into ``slot`` (the same slot later, or another one that is to go on from
+        that state)."""
+        if not self._lib.ptah_is_live(self._h, int(slot)):
+            raise CacheError(f"slot {slot} is not allocated")
+        names = {name for name, g in self.groups.items() if g.state is not None}
+        if set(snapshot) != names:
+            raise CacheError(f"the snapshot holds the state groups {sorted(snapshot)}, this cache has {sorted(names)}")
+        for name, t in snapshot.items():
+            dst = self.groups[name].state[:, int(slot)]
+            if tuple(t.shape) != tuple(dst.shape) or t.dtype != dst.dtype:
+                raise CacheError(f"state group {name!r}: the snapshot is {tuple(t.shape)} {t.dtype}, the slot holds "
+                                 f"{tuple(dst.shape)} {dst.dtype}")
+            dst.copy_(t)
 
     def bytes_per_token(self) -> int:
         total = 0

@@ -13,25 +13,40 @@ from __future__ import annotations
 
 import json
 import os
-from typing import Callable, Dict, Tuple, Type
+from typing import Callable, Dict, Sequence, Tuple, Type
 
 from .base import CONFIG_NAME, ConfigError, ModelConfig
 
 _REGISTRY: Dict[str, Tuple[Type[ModelConfig], Callable]] = {}
+_ALIASES: Dict[str, str] = {}  # other names a config.json may give an architecture -> its registered name
 
 
-def register(model_type: str, config_cls: Type[ModelConfig], builder: Callable, *, exist_ok: bool = False) -> None:
+def register(model_type: str, config_cls: Type[ModelConfig], builder: Callable, *, exist_ok: bool = False,
+             aliases: Sequence[str] = ()) -> None:
+    """Add an architecture.  ``aliases`` are further values of ``model_type`` that older files of the same
+    architecture carry; they are read as ``model_type``."""
     if not exist_ok and model_type in _REGISTRY:
         raise ValueError(f"model_type {model_type!r} is already registered")
+    for a in aliases:
+        if not exist_ok and (a in _REGISTRY or _ALIASES.get(a, model_type) != model_type):
+            raise ValueError(f"alias {a!r} of {model_type!r} is already taken")
     if getattr(config_cls, "model_type", None) != model_type:
         raise ValueError(
             f"{config_cls.__name__}.model_type is {getattr(config_cls, 'model_type', None)!r}, "
             f"it must equal the registered name {model_type!r}")  # configuration_auto.py:1110-1115
     _REGISTRY[model_type] = (config_cls, builder)
+    for a in aliases:
+        _ALIASES[a] = model_type
 
 
 def unregister(model_type: str) -> None:
     _REGISTRY.pop(model_type, None)
+    for a in [a for a, t in _ALIASES.items() if t == model_type]:
+        del _ALIASES[a]
+
+
+def resolve_alias(model_type: str) -> str:
+    return _ALIASES.get(model_type, model_type)
 
 
 def known_model_types():
@@ -48,10 +63,6 @@ def lookup(model_type: str) -> Tuple[Type[ModelConfig], Callable]:
         ) from None
 
 
-# old custom-code names of the architecture (convert_custom_code_checkpoint.py:38-40)
-_MODEL_TYPE_ALIASES = {"RefinedWebModel": "falcon", "RefinedWeb": "falcon"}
-
-
 class AutoConfig:
     """``AutoConfig.from_pretrained(folder)``: the typed configuration that config.json names."""
 
@@ -66,7 +77,7 @@ class AutoConfig:
         d = dict(d)
         if "model_type" not in d:
             raise ConfigError("config.json has no 'model_type' key; cannot choose an architecture")
-        d["model_type"] = _MODEL_TYPE_ALIASES.get(d["model_type"], d["model_type"])
+        d["model_type"] = resolve_alias(d["model_type"])
         cls, _ = lookup(d["model_type"])
         return cls.from_dict(d, **overrides)
 

@@ -93,7 +93,7 @@ extern "C" {
 
 const char* ptah_last_error() { return g_error.c_str(); }
 
-int ptah_abi_version() { return 3; }
+int ptah_abi_version() { return 4; }
 
 void* ptah_cache_new(int max_slots, int page_size, int n_groups, const int* group_pages, const int* group_windows) {
     if (max_slots <= 0 || page_size <= 0 || n_groups < 0) {
@@ -364,29 +364,35 @@ int ptah_decode_prepare(void* h, int n, const int* slots, const long long* token
 // wide, straight into the buffer that is copied to the device:
 //   token_ids | token_seq | token_pos [n_rows each] | cu_tokens [n_rows + 1] | seq_start | seq_slot |
 //   logit_rows [n_rows each] | one page table [n_rows, width] per paged group
-// Rows past n repeat sequence 0 (the same token at the same place writes the same keys and values again).
-int ptah_decode_fill(void* h, int n, const int* slots, const long long* tokens, int n_rows, int width, int32_t* out) {
+// Rows past n are padding: token 0 as the first token of a sequence of its own, which lives in pad_slot (a row of
+// the state tables that no sequence owns) and on pad_page (a page of every pool that no sequence owns), so that
+// padding touches no sequence's keys, values or state, whatever the layers keep there.
+int ptah_decode_fill(void* h, int n, const int* slots, const long long* tokens, int n_rows, int width, int pad_slot,
+                     int pad_page, int32_t* out) {
     Cache* c = static_cast<Cache*>(h);
     if (n <= 0 || n_rows < n) return fail(ERR_STEP, "decode layout for %d rows cannot hold %d sequences", n_rows, n);
     int32_t *ids = out, *seq = ids + n_rows, *pos = seq + n_rows, *cu = pos + n_rows, *start = cu + n_rows + 1;
     int32_t *slot = start + n_rows, *rows = slot + n_rows, *table = rows + n_rows;
     for (int r = 0; r < n_rows; ++r) {
-        const int i = r < n ? r : 0;
-        const int len = c->length[slots[i]];
-        ids[r] = (int32_t)tokens[i];
+        const int len = r < n ? c->length[slots[r]] : 0;
+        ids[r] = r < n ? (int32_t)tokens[r] : 0;
         seq[r] = r;
         pos[r] = len;
         cu[r] = r;
         start[r] = len;
-        slot[r] = slots[i];
+        slot[r] = r < n ? slots[r] : pad_slot;
         rows[r] = r;
     }
     cu[n_rows] = n_rows;
     for (const Group& gr : c->groups) {
         for (int r = 0; r < n_rows; ++r) {
-            const std::vector<int>& l = gr.lists[slots[r < n ? r : 0]];
-            if ((int)l.size() > width) return fail(ERR_STEP, "a sequence holds %zu pages, the layout has room for %d", l.size(), width);
             int32_t* row = table + (long)r * width;
+            if (r >= n) {
+                for (int k = 0; k < width; ++k) row[k] = pad_page;
+                continue;
+            }
+            const std::vector<int>& l = gr.lists[slots[r]];
+            if ((int)l.size() > width) return fail(ERR_STEP, "a sequence holds %zu pages, the layout has room for %d", l.size(), width);
             for (size_t k = 0; k < l.size(); ++k) row[k] = std::max(0, l[k]);
             for (int k = (int)l.size(); k < width; ++k) row[k] = 0;
         }

@@ -63,7 +63,10 @@ def build_falcon(cfg: FalconConfig) -> ModelSpec:
         final_norm=LayerNorm("transformer.ln_f", H, eps),
         head=OutputHead("lm_head", cfg.vocab_size, H, f"{embed_name}.weight" if cfg.tie_word_embeddings else None),
         cache_groups=[CacheGroupSpec(KV_GROUP, CACHE_FULL, L, cfg.kv_heads, cfg.head_dim)],
+        base_prefix="transformer.",  # src/transformers/models/falcon/modeling_falcon.py:782
     )
 
 
-register("falcon", FalconConfig, build_falcon, exist_ok=True)
+# "RefinedWeb" and "RefinedWebModel" are what the older custom-code checkpoints call the architecture
+# (src/transformers/models/falcon/convert_custom_code_checkpoint.py:38-40)
+register("falcon", FalconConfig, build_falcon, exist_ok=True, aliases=("RefinedWebModel", "RefinedWeb"))

@@ -22,8 +22,6 @@ from typing import List, Optional, Sequence, Union
 
 from ..config.generation import GenerationConfig
 
-PAGE = 64
-
 
 @dataclasses.dataclass
 class GenerateOutput:
@@ -95,9 +93,10 @@ def generate(model, prompts: Sequence[Sequence[int]], generation_config: Optiona
     batch_size = batch_size or len(prompts)
     batches = [list(range(b, min(b + batch_size, len(prompts)))) for b in range(0, len(prompts), batch_size)]
     need = 0
+    page = cache.page_size if cache is not None else getattr(model, "page_size", 64)
     for b in batches:
         new, _ = resolve_lengths(cfg, [len(prompts[i]) for i in b])
-        need = max(need, sum(_round_up(len(prompts[i]) + new, PAGE) for i in b))
+        need = max(need, sum(_round_up(len(prompts[i]) + new, page) for i in b))
     if cache is None:
         cache = model.new_cache(need, max_slots=batch_size)
     if sampler is None:

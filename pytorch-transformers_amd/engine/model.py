@@ -36,7 +36,25 @@ def resolve_dtype(dtype) -> torch.dtype:
     try:
         return _DTYPES[dtype]
     except KeyError:
-        raise ValueError(f"dtype must be 'float32' or 'bfloat16', got {dtype!r}") from None
+        raise ValueError(f"dtype must be 'float32', 'bfloat16' or 'auto', got {dtype!r}") from None
+
+
+def auto_dtype(config, folder: str) -> torch.dtype:
+    """What ``dtype="auto"`` means (src/transformers/modeling_utils.py:3996-4058): the configuration's
+    ``torch_dtype`` if it names one, else the type of the first floating-point tensor of the weight files.  The
+    engine computes in bfloat16 or in 32-bit: 16-bit floats of the other kind run as bfloat16, wider ones in 32-bit."""
+    from ..weights.loader import first_float_dtype
+
+    named = getattr(config, "torch_dtype", None)
+    if named is not None:
+        name = str(named).replace("torch.", "")
+        if name in ("bfloat16", "float16", "half"):
+            return torch.bfloat16
+        if name in ("float32", "float", "float64", "double"):
+            return torch.float32
+        raise ValueError(f"config.json names torch_dtype {named!r}, which the engine cannot compute in")
+    found = first_float_dtype(folder)
+    return torch.bfloat16 if found in (torch.bfloat16, torch.float16) else torch.float32
 
 
 def _require_gpu(device) -> torch.device:
@@ -71,9 +89,12 @@ class _DecodeGraph:
     from step to step (token ids, positions, slots, page lists) from one device buffer, which a
     replay refreshes with a single copy from pinned host memory.  Launch shapes that depend on the
     context (how many key ranges the attention is split into) are sized for ``len_bound``; ranges
-    past a sequence's end do no work.  A step with fewer than ``n`` sequences repeats its first
-    sequence in the spare rows: the same token at the same place writes the same keys and values
-    again, and the spare logits are dropped.
+    past a sequence's end do no work.  A step with fewer than ``n`` sequences fills the spare rows with
+    padding: token 0 as the first token of a sequence that lives in the cache's scratch slot and on its
+    scratch page, which no sequence owns, so padding changes no sequence's keys, values or state, whatever
+    the layers keep; the spare logits are dropped.  The first step of a graph's shape is launched directly
+    (its result is the step's result) and the graph is captured after it, which runs nothing: no step's
+    tokens go through the model twice.
 
     The cache owns its graphs and a graph refers to its cache weakly: with no cycle between them a cache
     that is dropped takes its graphs along at once.  A graph may not be destroyed while another one is
@@ -114,18 +135,18 @@ class _DecodeGraph:
 
     def _fill(self, plan: StepPlan) -> None:
         n, k = self.n, plan.n_seqs
-        pad = lambda a: np.concatenate([a, np.repeat(a[:1], n - k)]) if k < n else a
+        cache = self.cache
+        pad = lambda a, fill=0: np.concatenate([a, np.full(n - k, fill, dtype=np.int32)]) if k < n else a
         self.copied.synchronize()  # the last copy out of the pinned buffer is done
         self._put(0, pad(plan.token_ids))
         self._put(2, pad(plan.token_pos))
         self._put(4, pad(np.asarray(plan.starts, dtype=np.int32)))
-        self._put(5, pad(np.asarray(plan.slots, dtype=np.int32)))
+        self._put(5, pad(np.asarray(plan.slots, dtype=np.int32), cache.scratch_slot))
         for gi, g in enumerate(self.groups):
             t = np.zeros((n, self.width), dtype=np.int32)
             src = plan.block_tables[g]
             t[:k, :src.shape[1]] = src
-            if k < n:
-                t[k:] = t[0]
+            t[k:] = cache.scratch_page
             self._put(7 + gi, t.reshape(-1))
         self.dev.copy_(self.host, non_blocking=True)
         self.copied.record()
@@ -140,48 +161,52 @@ class _DecodeGraph:
         return ctx, v[0], v[6]
 
     def run(self, plan: StepPlan) -> torch.Tensor:
+        """The step's logits, in a tensor of their own (the graph's output buffer is written again by the next
+        replay)."""
         self._fill(plan)
-        self._replay()
+        logits = self._launch()
         k = plan.n_seqs
         rows = plan.logit_rows
         if rows.shape[0] == k:  # one row per sequence, in order: the first k rows as they are
-            return self.logits[:k]
+            return logits[:k].clone()
         if rows.shape[0] == 0:
-            return self.logits[:0]
-        return self.logits.index_select(0, torch.from_numpy(rows.astype(np.int64)).to(self.logits.device))
+            return logits[:0].clone()
+        return logits.index_select(0, torch.from_numpy(rows.astype(np.int64)).to(logits.device))
 
     def run_last(self, n: int, slots_c, tokens_c) -> torch.Tensor:
         """The common case, laid out by the host runtime straight into the pinned buffer: ``n`` sequences, one
         token each (C arrays), the logits of each."""
         self.copied.synchronize()  # the last copy out of the pinned buffer is done
         lib = host.load()
-        rc = lib.ptah_decode_fill(self.cache.handle, n, slots_c, tokens_c, self.n, self.width, self.host.data_ptr())
+        cache = self.cache
+        rc = lib.ptah_decode_fill(cache.handle, n, slots_c, tokens_c, self.n, self.width, cache.scratch_slot,
+                                  cache.scratch_page, self.host.data_ptr())
         if rc:
             raise StepError(host.last_error())
         self.dev.copy_(self.host, non_blocking=True)
         self.copied.record()
-        self._replay()
-        return self.logits[:n]
+        return self._launch()[:n].clone()
 
-    def _replay(self) -> None:
-        if self.graph is None:
-            ctx, ids, rows = self._context()
-            side = torch.cuda.Stream()
-            side.wait_stream(torch.cuda.current_stream())
-            with torch.cuda.stream(side):  # once outside capture: libraries set themselves up
-                self.model.forward_tokens(ctx, ids, rows)
-            torch.cuda.current_stream().wait_stream(side)
-            graph = torch.cuda.CUDAGraph()
-            collecting = gc.isenabled()
-            gc.disable()  # no finalizer of a dead cycle may call into the runtime while the capture lasts
-            try:
-                with torch.cuda.graph(graph):
-                    self.logits = self.model.forward_tokens(ctx, ids, rows)
-            finally:
-                if collecting:
-                    gc.enable()
-            self.graph = graph
-        self.graph.replay()
+    def _launch(self) -> torch.Tensor:
+        """Run the step that the device buffer now describes; returns the logits of all ``n`` rows (a buffer
+        that the next call writes again)."""
+        if self.graph is not None:
+            self.graph.replay()
+            return self.logits
+        # the first step of this shape: launched directly, which also lets libraries set themselves up outside a
+        # capture; its result is the step's result.  The capture that follows records launches and runs nothing.
+        logits = self.model.forward_tokens(*self._context())
+        graph = torch.cuda.CUDAGraph()
+        collecting = gc.isenabled()
+        gc.disable()  # no finalizer of a dead cycle may call into the runtime while the capture lasts
+        try:
+            with torch.cuda.graph(graph):
+                self.logits = self.model.forward_tokens(*self._context())  # a context of its own: nothing cached per step is shared
+        finally:
+            if collecting:
+                gc.enable()
+        self.graph = graph
+        return logits
 
 
 class CausalLM:
@@ -223,11 +248,11 @@ class CausalLM:
         from ..config.generation import GenerationConfig
 
         device = _require_gpu(device)
-        dtype = resolve_dtype(dtype)
         config = AutoConfig.from_pretrained(folder)
+        dtype = auto_dtype(config, folder) if dtype == "auto" else resolve_dtype(dtype)
         _, builder = lookup(config.model_type)
         spec = builder(config)
-        tensors = load_weights(folder, spec.tensor_specs(), dtype, device, strict=strict)
+        tensors = load_weights(folder, spec.tensor_specs(), dtype, device, base_prefix=spec.base_prefix, strict=strict)
         model = cls(spec, tensors, dtype, device)
         model.generation_config = GenerationConfig.from_pretrained(folder, config)
         return model
@@ -252,7 +277,49 @@ class CausalLM:
         model.generation_config = GenerationConfig.from_model_config(config)
         return model
 
+    # timed choices ---------------------------------------------------------------
+    @torch.no_grad()
+    def tune(self, prompt_lens: Sequence[int] = (2048,), batches: Sequence[int] = (8, 64), table=None) -> dict:
+        """Time, once, the choices between kernels that no rule decides, for prompts of ``prompt_lens`` tokens and
+        decode steps of ``batches`` sequences, and keep them for every later step of this process; returns the
+        table (``ops.tuning_table``).  With ``table`` given nothing is timed: its choices are taken instead.
+        Steps never time anything by themselves (unless PTA_TUNE=1 is set): untuned, they take the built-in
+        choice, and logits are the same bits in every process."""
+        from .. import ops
+
+        if table is not None:
+            ops.load_tuning(table)
+            return ops.tuning_table()
+        if self.dtype != torch.bfloat16:
+            return ops.tuning_table()  # the 32-bit path has one kernel per operation
+        graphs, self.use_graphs = self.use_graphs, False  # nothing can be timed inside a capture
+        need = max([int(t) for t in prompt_lens] + [0]) + 64 * max([int(b) for b in batches] + [1]) + 64
+        cache = self.new_cache(need)
+        try:
+            with ops.live_tuning():
+                for T in prompt_lens:
+                    slot = cache.alloc()
+                    self.step(cache, [slot], [[0] * int(T)], "last")
+                    cache.free(slot)
+                for b in batches:
+                    slots = [cache.alloc() for _ in range(int(b))]
+                    self.step(cache, slots, [[0]] * int(b), "last")  # one token each: the shape of a decode step
+                    for s_ in slots:
+                        cache.free(s_)
+            torch.cuda.synchronize()
+        finally:
+            self.use_graphs = graphs
+            ops.release_flush()
+        return ops.tuning_table()
+
     # cache -------------------------------------------------------------------
+    @property
+    def page_size(self) -> int:
+        """Tokens per cache page: a sequence's share of a cache is its length rounded up to this."""
+        from ..cache.paged import PAGE_SIZE
+
+        return PAGE_SIZE
+
     def new_cache(self, max_tokens: int, max_slots: Optional[int] = None) -> PagedCache:
         """A cache for at most ``max_tokens`` live tokens (each sequence's count rounded up to a page)."""
         return PagedCache(self.spec.cache_groups, max_tokens, self.dtype, self.device, max_slots=max_slots)

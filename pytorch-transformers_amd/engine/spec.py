@@ -74,6 +74,9 @@ class ModelSpec:
     final_norm: Any  # parts norm or None
     head: Any  # parts.OutputHead
     cache_groups: List[CacheGroupSpec]
+    #: what the checkpoint's tensor names start with when the whole model was saved, and lack when only its body
+    #: was (the reference's ``base_model_prefix`` plus a dot); "" if there is no such prefix
+    base_prefix: str = ""
     #: False if a part reads the step's host-side lists (``ctx.slots`` ...) while it runs: such a step
     #: cannot be captured into a graph and replayed with other values
     supports_graphs: bool = True

@@ -12,7 +12,7 @@ import os
 import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-ABI_VERSION = 3
+ABI_VERSION = 4
 OK, ERR_STEP, ERR_CACHE, ERR_FULL = 0, 1, 2, 3
 
 _lib = None
@@ -55,7 +55,7 @@ def load():
                                        _P_INT, _P_INT, _P_INT]
         lib.ptah_decode_prepare.argtypes = [ctypes.c_void_p, ctypes.c_int, _P_INT, _P_LL, ctypes.c_int, _P_INT, _P_LL]
         lib.ptah_decode_fill.argtypes = [ctypes.c_void_p, ctypes.c_int, _P_INT, _P_LL, ctypes.c_int, ctypes.c_int,
-                                         ctypes.c_void_p]
+                                         ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
         lib.ptah_commit_ones.argtypes = [ctypes.c_void_p, ctypes.c_int, _P_INT]
         lib.ptah_plan_data.argtypes = [ctypes.c_void_p]
         lib.ptah_plan_data.restype = _P_INT

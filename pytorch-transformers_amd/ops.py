@@ -313,7 +313,7 @@ def _decode_plan(n: int, n_heads: int, n_kv_heads: int, head_dim: int, bound: in
         size = min(ATTN_SPLIT_KEYS, ATTN_FORCE_SPLIT) if ATTN_FORCE_SPLIT else ATTN_SPLIT_KEYS
         while True:
             whole = size >= bound
-            if (bound + size - 1) // size <= 1024 and (not ATTN_FORCE_SPLIT or size == ATTN_FORCE_SPLIT or
+            if (bound + size - 1) // size <= 1024 and n * ((bound + size - 1) // size) <= 65535 and (not ATTN_FORCE_SPLIT or size == ATTN_FORCE_SPLIT or
                                                        (whole and size < ATTN_FORCE_SPLIT)):
                 ranges = (mean_keys + size - 1) // size
                 waves = n * n_kv_heads * sharing * ranges
@@ -412,21 +412,62 @@ def sample(logits: torch.Tensor, *, do_sample: bool, temperature: float = 1.0, t
     return out, (work if need_scores else None)
 
 
+# ---- choices that are timed, and when ---------------------------------------------------------------------
+# Some choices between two ways to the same product have no rule that holds across shapes (how many ranges of K
+# a pair launch is cut into, up to how many rows the decode batch kernel beats the vendor library, in which pieces
+# along M the library's product runs, whether two matrices of one input run as one product, whether K is cut into
+# a batch).  Each has a built-in default, and a table keyed by shape that overrides it.  The table is filled only
+# while timing is switched on: inside ``live_tuning()`` (``CausalLM.tune`` runs steps of given sizes in it), or in
+# every step with PTA_TUNE=1 in the environment.  With timing off (the default) a step allocates nothing for
+# measurements and times nothing, and its results depend on weights, tokens and schedule alone: two processes give
+# the same bits.  ``tuning_table()`` / ``load_tuning()`` carry a table from one process to another.
+TUNE_LIVE = os.environ.get("PTA_TUNE", "0") == "1"
+
+
+class live_tuning:
+    """Context in which choices that have no entry in the tuning table yet are timed at first use."""
+
+    def __enter__(self):
+        global TUNE_LIVE
+        self._old, TUNE_LIVE = TUNE_LIVE, True
+        return self
+
+    def __exit__(self, *exc):
+        global TUNE_LIVE
+        TUNE_LIVE = self._old
+        return False
+
+
+def _may_time() -> bool:
+    return TUNE_LIVE and not torch.cuda.is_current_stream_capturing()
+
+
 SKINNY_MAX_ROWS = 64
 # rows up to which the decode batch kernel (x shared through LDS, K split over workgroups) stands in for the
-# vendor library's product, whose choices for 65 to 128 rows leave most of the chip idle (Falcon-7B sizes, 128
-# rows: 10.4 ms a step with the library)
+# vendor library's product, whose choices for 65 to 128 rows leave most of the chip idle (K = 4,544 with N =
+# 4,672 and 18,176 in one product of 128 rows: 151 us, 1.4 TB/s of weights)
 SPLITK_MAX_ROWS = int(os.environ.get("PTA_SPLITK_MAX_ROWS", "256"))
 SPLITK_MARGIN = float(os.environ.get("PTA_SPLITK_MARGIN", "0.95"))
 SPLITK_SURE_ROWS = 128  # up to here the kernel won at every shape measured; beyond, by the weight's own timing
 _splitk_limits: dict = {}  # (N, K) -> rows up to which the batch kernel beats the library's product
 
 
+_flush = None  # half a gigabyte that is written between timed runs; held only while timing is on (``release_flush``)
+
+
+def release_flush() -> None:
+    global _flush
+    _flush = None
+
+
 def _time_ways_cold(ways, device, rounds: int = 3):
     """Milliseconds of each of ``ways`` (callables), the fastest of ``rounds`` runs each, taken in turn; before
     every run half a gigabyte is written, so that the weights come from memory as they do in a model (timed back
     to back, a product finds its matrix in the memory-side cache and every way looks alike)."""
-    flush = torch.empty(128 * 1024 * 1024, dtype=torch.float32, device=device)
+    global _flush
+    if _flush is None or _flush.device != device:
+        _flush = torch.empty(128 * 1024 * 1024, dtype=torch.float32, device=device)
+    flush = _flush
     best = [float("inf")] * len(ways)
     for run in ways:  # plans are made and the library set up before anything is timed
         run()
@@ -445,16 +486,16 @@ def _time_ways_cold(ways, device, rounds: int = 3):
 def splitk_row_limit(*ws: torch.Tensor) -> int:
     """Rows up to which the decode batch kernel is the faster way to the product with ``w`` (or, for two weights, to
     the two products of a pair launch).  Up to 128 rows it always was (one chunk of rows per workgroup); with two
-    chunks it depends on how well the library does at the shape (at 256 rows it wins at Falcon-7B shapes, 9.5
-    against 11.4 ms a step, and loses at Falcon2-11B shapes, 22.1 against 20.2), so both are timed once per shape
-    at 192 and 256 rows."""
+    chunks it depends on how well the library does at the shape (at 256 rows it wins with K = 4,544, 9.5 against
+    11.4 ms a step of 32 layers, and loses with K = 4,096, 22.1 against 20.2 ms of 60 layers), so both are timed once
+    per shape at 192 and 256 rows, when timing is on; without an entry the kernel stops at 128 rows."""
     if SPLITK_MAX_ROWS <= SPLITK_SURE_ROWS:
         return SPLITK_MAX_ROWS
     key = tuple(tuple(w.shape) for w in ws)
     limit = _splitk_limits.get(key)
     if limit is None:
-        if torch.cuda.is_current_stream_capturing():
-            return SPLITK_SURE_ROWS  # nothing can be timed now; the next eager step decides
+        if not _may_time():
+            return SPLITK_SURE_ROWS
         dev = ws[0].device
         xs = [torch.randn((256, w.shape[1]), dtype=torch.float32, device=dev).to(torch.bfloat16) for w in ws]
         outs = [torch.empty((256, w.shape[0]), dtype=torch.bfloat16, device=dev) for w in ws]
@@ -489,10 +530,10 @@ def _splitk_rows(x: torch.Tensor, *ws: torch.Tensor) -> bool:
 
 # ---- the vendor library's product for many rows, cut along M where that is faster -----------------------
 # The library picks a kernel per (M, N, K) from a table, and on this hardware its choices are uneven in M:
-# at Falcon-7B shapes 2,048 rows of the feed-forward's first product take longer than 2,304, and 4,096 rows of
-# its second one almost as long as 8,192.  So for every weight shape the product is timed once at a ladder of
-# row counts, and a product of M rows runs as the cheapest sequence of those pieces (each written straight
-# into its rows of the result).  PTA_MM_CHUNKS=0 switches this off.
+# with K = 4,544 and N = 18,176, 2,048 rows take longer than 2,304, and 4,096 rows of the product with the
+# transposed shape almost as long as 8,192.  So, when timing is on, the product is timed once per weight shape at
+# a ladder of row counts, and a product of M rows then runs as the cheapest sequence of those pieces (each written
+# straight into its rows of the result); without an entry it runs whole.  PTA_MM_CHUNKS=0 switches this off.
 MM_LADDER = (256, 512, 768, 1024, 1536, 2048, 3072, 4096, 6144, 8192)
 MM_CHUNKS = os.environ.get("PTA_MM_CHUNKS", "1") != "0"
 MM_JOIN = os.environ.get("PTA_MM_JOIN", "1") != "0"  # one product for two matrices of one input where it is faster
@@ -523,6 +564,8 @@ def _mm_plan(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor):
     plan = _mm_plans.get((N, K, bucket))
     if plan is not None:
         return plan[:-1] + [M - sum(plan[:-1])]
+    if not _may_time():
+        return [M]
     times = _mm_times.setdefault((N, K), {})
     for rows in MM_LADDER:
         if rows <= M and rows not in times:
@@ -552,14 +595,17 @@ def _mm_plan(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor):
 
 def joined_mm_pays(x: torch.Tensor, joined: torch.Tensor, n_first: int) -> bool:
     """Whether ``x @ joined.T`` in one library product beats the products with its first ``n_first`` rows and
-    with the rest on their own.  The library's kernel choice decides, so both ways are timed once per shape (at
-    Falcon-7B shapes, 2,048 rows: 308 us against 87 + 286; at Falcon2-11B shapes 311 against 80 + 179)."""
+    with the rest on their own.  The library's kernel choice decides, so both ways are timed once per shape when
+    timing is on (2,048 rows, K = 4,544, N = 4,672 + 18,176: 308 us against 87 + 286; K = 4,096, N = 6,144 + 16,384:
+    311 against 80 + 179); without an entry the two stay apart."""
     M, (N, K) = x.shape[0], joined.shape
-    if not MM_JOIN or not MM_CHUNKS or M < 512 or torch.cuda.is_current_stream_capturing():
+    if not MM_JOIN or not MM_CHUNKS or M < 512:
         return False
     bucket = (M + 63) // 64
     key = (n_first, N - n_first, K, bucket)
     if key not in _mm_joined:
+        if not _may_time():
+            return False
         first, rest = joined[:n_first], joined[n_first:]
         ways = (lambda: library_mm(x, joined), lambda: (library_mm(x, first), library_mm(x, rest)))
         best = [float("inf"), float("inf")]
@@ -580,7 +626,9 @@ def joined_mm_pays(x: torch.Tensor, joined: torch.Tensor, n_first: int) -> bool:
 def library_mm(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     """``x @ w.T`` in bfloat16 through the vendor library, in the pieces along M that were measured fastest."""
     M, N = x.shape[0], w.shape[0]
-    if not MM_CHUNKS or M < 512 or torch.cuda.is_current_stream_capturing():
+    if not MM_CHUNKS or M < 512:
+        return torch.mm(x, w.t())
+    if (N, w.shape[1], (M + 63) // 64) not in _mm_plans and not _may_time():
         return torch.mm(x, w.t())
     out = torch.empty((M, N), dtype=x.dtype, device=x.device)
     plan = _mm_plan(x, w, out)
@@ -594,11 +642,12 @@ def library_mm(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
 
 # ---- the vendor library's product with K cut into a batch ------------------------------------------------
 # Where K is long against N (the feed-forward's second matrix) and the rows are a few hundred, the library's
-# kernel choice has too few tiles of the result to fill the chip: at Falcon-7B shapes 512 rows take 225 us, and
-# 112 us as a batch of two products over the halves of K (32-bit partial sums, added in order by the kernel
-# that also applies bias, activation and additions, so no epilogue launch follows).
+# kernel choice has too few tiles of the result to fill the chip: with K = 18,176 and N = 4,544, 512 rows take 225
+# us, and 112 us as a batch of two products over the halves of K (32-bit partial sums, added in order by the kernel
+# that also applies bias, activation and additions, so no epilogue launch follows).  Timed once per shape when
+# timing is on; without an entry the plain product runs.
 MM_KSPLIT = os.environ.get("PTA_MM_KSPLIT", "1") != "0"
-MM_KSPLIT_MAX_ROWS = 1536  # at 2,048 rows the batch gained nothing alone and lost 3 % in a model (Falcon-40B sizes)
+MM_KSPLIT_MAX_ROWS = 1536  # at 2,048 rows the batch gained nothing alone and lost 3 % in a model (K = 32,768, N = 8,192)
 _mm_ksplit: dict = {}  # (N, K, row bucket) -> ranges of K (1: the plain product)
 
 
@@ -619,7 +668,7 @@ def library_mm_ksplit(x: torch.Tensor, w: torch.Tensor, bias=None, act=None, add
     key = (N, K, (M + 63) // 64)
     S = _mm_ksplit.get(key)
     if S is None:
-        if torch.cuda.is_current_stream_capturing():
+        if not _may_time():
             return None
         ways = [(1, lambda: library_mm(x, w))] + [(s, (lambda s=s: _k_batch(x, w, s))) for s in (2, 4) if K % (s * 8) == 0]
         best = _time_ways_cold([run for _, run in ways], x.device)
@@ -753,9 +802,9 @@ def gemm_splitk_pair_parts(N1: int, K1: int, N2: int, K2: int):
     return p1.value, p2.value
 
 
-# Ranges of K for the pairs of a shape: the kernel library's rule gives a choice, and its neighbours are timed
-# once per shape, at 64 rows, with cold caches; one that is at least 3 % faster is kept for every later launch
-# (PTA_PAIR_TUNE=0 switches this off).
+# Ranges of K for the pairs of a shape: the kernel library's rule gives a choice; when timing is on, its neighbours
+# are timed once per shape, at 64 rows, with cold caches, and one that is at least 3 % faster is kept for every
+# later launch (PTA_PAIR_TUNE=0 switches this off).
 PAIR_TUNE = os.environ.get("PTA_PAIR_TUNE", "1") != "0"
 PAIR_TUNE_MARGIN = 0.97
 _pair_parts_tuned: dict = {}  # (shape of w1, shape of w2) -> the counts in use
@@ -765,8 +814,8 @@ def tune_pair_parts(w1: torch.Tensor, w2: torch.Tensor) -> None:
     """Once per pair of shapes: time the pair launch with the rule's ranges of K and with their neighbours, and fix
     the fastest in the kernel library if it beats the rule's by the margin (``_pair_parts_tuned`` says which)."""
     key = (tuple(w1.shape), tuple(w2.shape))
-    if not PAIR_TUNE or key in _pair_parts_tuned or torch.cuda.is_current_stream_capturing():
-        return  # under capture nothing can be timed: the next eager step decides
+    if not PAIR_TUNE or key in _pair_parts_tuned or not _may_time():
+        return
     lib = load_library()
     (N1, K1), (N2, K2) = w1.shape, w2.shape
     a0, b0 = gemm_splitk_pair_parts(N1, K1, N2, K2)
@@ -794,6 +843,60 @@ def tune_pair_parts(w1: torch.Tensor, w2: torch.Tensor) -> None:
     if chosen != cands[0]:
         fix(chosen)
     _pair_parts_tuned[key] = chosen
+
+
+def tuning_table() -> dict:
+    """What has been timed so far, as plain data (JSON-able): give it to ``load_tuning`` in another process and
+    that process makes the same choices, hence the same bits."""
+    key = lambda t: ",".join("x".join(str(int(v)) for v in (p if isinstance(p, tuple) else (p,))) for p in t)
+    return {
+        "pair_parts": {key(k): list(v) for k, v in _pair_parts_tuned.items()},
+        "splitk_rows": {key(k): int(v) for k, v in _splitk_limits.items()},
+        "mm_plans": {key(k): list(v) for k, v in _mm_plans.items()},
+        "mm_joined": {key(k): bool(v) for k, v in _mm_joined.items()},
+        "mm_ksplit": {key(k): int(v) for k, v in _mm_ksplit.items()},
+    }
+
+
+def clear_tuning() -> None:
+    """Back to the built-in defaults for every shape."""
+    lib = load_library()
+    for (s1, s2) in list(_pair_parts_tuned):
+        lib.pta_gemm_splitk_pair_fix_parts(int(s1[0]), int(s1[1]), int(s2[0]), int(s2[1]), 0, 0)
+    for d in (_pair_parts_tuned, _splitk_limits, _mm_plans, _mm_costs, _mm_times, _mm_joined, _mm_ksplit):
+        d.clear()
+
+
+def load_tuning(table: dict) -> None:
+    """Take the choices of a table that ``tuning_table`` made (entries for other shapes stay as they are)."""
+    lib = load_library()
+    shapes = lambda k: tuple(tuple(int(v) for v in p.split("x")) for p in k.split(","))
+    flat = lambda k: tuple(int(p) for p in k.split(","))
+    for k, (a, b) in table.get("pair_parts", {}).items():
+        s1, s2 = shapes(k)
+        rule = gemm_splitk_pair_parts_rule(s1[0], s1[1], s2[0], s2[1])
+        if (int(a), int(b)) != rule and lib.pta_gemm_splitk_pair_fix_parts(s1[0], s1[1], s2[0], s2[1], int(a), int(b)):
+            raise KernelError(f"tuning table: {a} and {b} ranges of K are not valid for the pair {k}")
+        _pair_parts_tuned[(s1, s2)] = (int(a), int(b))
+    for k, v in table.get("splitk_rows", {}).items():
+        _splitk_limits[shapes(k)] = int(v)
+    for k, v in table.get("mm_plans", {}).items():
+        _mm_plans[flat(k)] = [int(r) for r in v]
+    for k, v in table.get("mm_joined", {}).items():
+        _mm_joined[flat(k)] = bool(v)
+    for k, v in table.get("mm_ksplit", {}).items():
+        _mm_ksplit[flat(k)] = int(v)
+
+
+def gemm_splitk_pair_parts_rule(N1: int, K1: int, N2: int, K2: int):
+    """The ranges of K that the kernel library's own rule gives a pair, whatever has been fixed for the shape."""
+    lib = load_library()
+    now = gemm_splitk_pair_parts(N1, K1, N2, K2)
+    lib.pta_gemm_splitk_pair_fix_parts(int(N1), int(K1), int(N2), int(K2), 0, 0)
+    rule = gemm_splitk_pair_parts(N1, K1, N2, K2)
+    if now != rule:
+        lib.pta_gemm_splitk_pair_fix_parts(int(N1), int(K1), int(N2), int(K2), int(now[0]), int(now[1]))
+    return rule
 
 
 def gemm_splitk_pair_partial(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tensor, w2: torch.Tensor):
@@ -998,7 +1101,7 @@ def _bf16_rows_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
 
 def gemm_skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
     """Whether the kernel for few rows takes this product and is the faster choice for it: bfloat16 with K a
-    multiple of 8 and at most 16 rows (measured on MI355X against the vendor library at Falcon-7B shapes)."""
+    multiple of 8 and at most 16 rows (measured on MI355X against the vendor library at K = 4,544 and K = 18,176)."""
     return _bf16_rows_ok(x, w) and 0 < x.shape[0] <= 16
 
 
@@ -1010,8 +1113,8 @@ def gemm_splitk_pair_ok(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tensor, w2
 
 
 def gemm_splitk_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
-    """Whether the kernel for a decode batch of 17 to 128 rows is the faster choice.  Measured at Falcon-7B
-    shapes: it beats the vendor library except where N is long against K (the feed-forward's first matrix
+    """Whether the kernel for a decode batch of 17 to 128 rows is the faster choice.  Measured at K = 4,544 and
+    K = 18,176: it beats the vendor library except where N is long against K (the feed-forward's first matrix
     and the output head), which give the library enough row tiles to fill the chip."""
     return (_bf16_rows_ok(x, w) and 16 < x.shape[0] <= SPLITK_MAX_ROWS and w.shape[0] < 2 * w.shape[1]
             and _splitk_rows(x, w))

@@ -93,6 +93,22 @@ def _strip_or_add_prefix(file_names: Iterable[str], wanted: Sequence[str], prefi
     return out
 
 
+def first_float_dtype(folder: str) -> Optional[torch.dtype]:
+    """The type of the first floating-point tensor of the weight files (what ``dtype="auto"`` falls back on,
+    src/transformers/modeling_utils.py:4030-4041), read from the files' headers."""
+    from safetensors import safe_open
+
+    names = {"F64": torch.float64, "F32": torch.float32, "F16": torch.float16, "BF16": torch.bfloat16}
+    files = resolve_files(folder)
+    for path in sorted(set(files.values())):
+        with safe_open(path, framework="pt") as f:
+            for k in f.keys():
+                dt = names.get(f.get_slice(k).get_dtype())
+                if dt is not None:
+                    return dt
+    return None
+
+
 def device_dtype_for(spec: TensorSpec, compute_dtype: torch.dtype) -> torch.dtype:
     if spec.kind == MATRIX:
         return compute_dtype
@@ -109,8 +125,10 @@ def place(spec: TensorSpec, t: torch.Tensor, compute_dtype: torch.dtype, device)
 
 
 def load_weights(folder: str, specs: Sequence[TensorSpec], compute_dtype: torch.dtype, device,
-                 *, base_prefix: str = "transformer.", strict: bool = True) -> Dict[str, torch.Tensor]:
-    """Read every tensor of ``specs`` from ``folder``; raise one WeightsError naming all problems."""
+                 *, base_prefix: str = "", strict: bool = True) -> Dict[str, torch.Tensor]:
+    """Read every tensor of ``specs`` from ``folder``; raise one WeightsError naming all problems.  ``base_prefix``
+    is what the model's tensor names start with when the whole model was saved; a file saved from the body alone
+    lacks it and loads too."""
     from safetensors import safe_open
 
     files = resolve_files(folder)

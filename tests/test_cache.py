@@ -19,7 +19,8 @@ def test_shapes_and_capacity():
     c = _cache(1000)
     assert c.num_pages == 16 and c.max_slots == 16  # 1000 tokens round up to 16 pages of 64
     k, v = c.kv_layer("kv", 1)
-    assert k.shape == (16, 2, 64, 16) and v.shape == (16, 2, 16, 64)  # value pages are transposed
+    # value pages are transposed; one page more than sequences can hold is the scratch page of padding rows
+    assert k.shape == (17, 2, 64, 16) and v.shape == (17, 2, 16, 64) and c.scratch_page == 16 and c.scratch_slot == 16
     assert c.bytes_per_token() == 2 * 2 * 2 * 16 * 4
 
 
@@ -78,13 +79,38 @@ def test_reserve_is_all_or_nothing():
 def test_state_groups_are_zeroed_on_alloc():
     st = CacheGroupSpec("s", CACHE_STATE, num_layers=2, state_shape=(3, 4))
     c = _cache(256, groups=(KV, st), max_slots=4)
-    assert c.state_layer("s", 0).shape == (4, 3, 4)
+    assert c.state_layer("s", 0).shape == (5, 3, 4)  # four slots and the scratch slot of padding rows
     a = c.alloc()
     c.state_layer("s", 1)[a] += 7.0
     c.free(a)
     b = c.alloc()
     assert b == a and float(c.state_layer("s", 1)[b].abs().sum()) == 0.0
     assert c.paged_groups() == ["kv"]
+
+
+def test_state_can_be_copied_out_and_put_back():
+    """A sequence's fixed-size state as a snapshot: put back into the same slot it undoes what came after, put
+    into another slot that one goes on from there; slots that are not allocated and snapshots of another shape
+    are refused."""
+    st = CacheGroupSpec("s", CACHE_STATE, num_layers=2, state_shape=(3,))
+    c = _cache(256, groups=(KV, st), max_slots=4)
+    a, b = c.alloc(), c.alloc()
+    c.state_layer("s", 0)[a] += 1.0
+    c.state_layer("s", 1)[a] += 2.0
+    snap = c.snapshot_state(a)
+    assert set(snap) == {"s"} and snap["s"].shape == (2, 3)
+    c.state_layer("s", 1)[a] += 5.0
+    assert float(snap["s"][1, 0]) == 2.0  # a copy, not a view
+    c.restore_state(a, snap)
+    assert c.state_layer("s", 1)[a].tolist() == [2.0, 2.0, 2.0]
+    c.restore_state(b, snap)
+    assert c.state_layer("s", 0)[b].tolist() == [1.0, 1.0, 1.0]
+    with pytest.raises(CacheError):
+        c.snapshot_state(3)
+    with pytest.raises(CacheError):
+        c.restore_state(b, {"s": snap["s"][:, :2]})
+    with pytest.raises(CacheError):
+        c.restore_state(b, {})
 
 
 def test_random_traffic_keeps_the_books_straight():

@@ -234,8 +234,12 @@ def test_pair_ranges_are_timed_once_per_shape_and_kept():
     x1, x2 = _rand(M, K1, dtype=torch.bfloat16), _rand(M, K2, seed=5, dtype=torch.bfloat16)
     w1, w2 = _rand(N1, K1, seed=1, dtype=torch.bfloat16, scale=0.05), _rand(N2, K2, seed=2, dtype=torch.bfloat16, scale=0.05)
     rule = ops.gemm_splitk_pair_parts(N1, K1, N2, K2)
-    y1, y2 = ops.gemm_splitk_pair_bf16(x1, w1, x2, w2)
     key = ((N1, K1), (N2, K2))
+    ops.gemm_splitk_pair_bf16(x1, w1, x2, w2)
+    assert ops.TUNE_LIVE or key not in ops._pair_parts_tuned, "a launch times nothing unless timing is switched on"
+    with ops.live_tuning():
+        y1, y2 = ops.gemm_splitk_pair_bf16(x1, w1, x2, w2)
+    ops.release_flush()
     if ops.PAIR_TUNE:
         kept = ops._pair_parts_tuned[key]
         assert abs(kept[0] - rule[0]) <= 2 and abs(kept[1] - rule[1]) <= 2
@@ -308,7 +312,10 @@ def test_library_mm_in_pieces():
     try:
         for M in (1000, 1030, 700):
             x = _rand(M, K, seed=M, dtype=torch.bfloat16)
-            y = ops.library_mm(x, w)
+            ops.library_mm(x, w)
+            assert ops.TUNE_LIVE or (N, K, (M + 63) // 64) not in ops._mm_plans, "no plan is made unless timing is on"
+            with ops.live_tuning():
+                y = ops.library_mm(x, w)
             plan = ops._mm_plans[(N, K, (M + 63) // 64)]
             if M != 700:
                 assert len(plan) > 1 and sum(plan) == M and all(p >= 256 for p in plan), plan
@@ -676,12 +683,14 @@ def test_decode_plan():
     ops = _ops()
     for nh, nkv, d in ((71, 1, 64), (32, 8, 128), (128, 8, 64), (6, 2, 32), (2, 1, 256)):
         groups = (nh // nkv + 15) // 16
-        for n in (1, 3, 8, 33, 64):
-            for length in (1, 100, 1024, 1025, 2049, 8192, 100000):
+        for n in (1, 3, 8, 33, 64, 128, 300, 512):
+            for length in (1, 100, 1024, 1025, 2049, 8192, 32768, 65536, 100000):
                 tiles, size = ops.decode_plan(n, nh, nkv, d, length)
                 assert 1 <= tiles <= groups and size % 64 == 0 and size >= 128
                 assert (length + size - 1) // size <= 1024
                 bucket_n = 1 << (n - 1).bit_length()
+                # the launch has one workgroup row per (sequence of the padded batch, range): the grid's limit
+                assert bucket_n * ((((length + 1023) // 1024 * 1024) + size - 1) // size) <= 65535
                 bucket_len = (length + 1023) // 1024 * 1024
                 assert (tiles, size) == ops.decode_plan(bucket_n, nh, nkv, d, bucket_len)
                 for mean in (1, length // 3 + 1, length):

@@ -124,7 +124,9 @@ def test_joined_matrices_give_one_product_for_many_rows(monkeypatch):
         _, r3 = _fill(down, torch.bfloat16, 4)
         _close(down(y2), y2.double().cpu() @ r3["c.weight"].T, 2e-2, "a product whose input rows lie apart")
     monkeypatch.undo()
-    assert ops.joined_mm_pays(x, first.joined[0], N1) in (True, False)  # measured, either way
+    assert ops.TUNE_LIVE or ops.joined_mm_pays(x, first.joined[0], N1) is False  # nothing is timed unless asked
+    with ops.live_tuning():
+        assert ops.joined_mm_pays(x, first.joined[0], N1) in (True, False)  # measured, either way
 
 
 def test_rows_beyond_one_chunk_take_the_way_that_was_timed_faster(monkeypatch):
@@ -141,7 +143,10 @@ def test_rows_beyond_one_chunk_take_the_way_that_was_timed_faster(monkeypatch):
     x = _rand(M, H, seed=3).bfloat16().cuda()
     want1 = P.linear(x.double().cpu(), r1["a.weight"], r1["a.bias"])
     want2 = P.gelu(x.double().cpu() @ r2["b.weight"].T)
-    assert ops.splitk_row_limit(first.weight) in (128, 192, 256)  # measured, whichever
+    assert ops.TUNE_LIVE or ops.splitk_row_limit(first.weight) == 128  # nothing is timed unless asked
+    with ops.live_tuning():
+        assert ops.splitk_row_limit(first.weight) in (128, 192, 256)  # measured, whichever
+    ops.release_flush()
     for limit in (256, 128):
         monkeypatch.setattr(ops, "splitk_row_limit", lambda *ws: limit)
         assert ops.gemm_splitk_ok(x, first.weight) == (limit == 256)
@@ -182,7 +187,11 @@ def test_library_product_over_ranges_of_k():
     finally:
         ops._mm_ksplit.pop(key, None)
     assert ops.library_mm_ksplit(x[:64], lin.weight) is None  # few rows go to the decode kernels
-    lin(x, act="gelu", add1=a1, add2=a2)  # timed, whichever way
+    lin(x, act="gelu", add1=a1, add2=a2)
+    assert ops.TUNE_LIVE or key not in ops._mm_ksplit  # nothing is timed unless asked
+    with ops.live_tuning():
+        lin(x, act="gelu", add1=a1, add2=a2)  # timed, whichever way
+    ops.release_flush()
     assert ops._mm_ksplit.pop(key) in (1, 2, 4)
 
 
@@ -267,7 +276,9 @@ def test_attention_mixer_and_blocks(dtype, rel, layout, nh, nkv, d, alibi, bias)
 
 
 # --- a toy architecture, defined in the test -------------------------------------------------------------
-def _define_toy():
+def _define_toy(device_decode: bool = False):
+    """``device_decode``: in steps of one token per sequence the mixer reads nothing but the step's device
+    arrays, so that such steps can be captured and replayed; the model then says ``supports_graphs=True``."""
     from pytorch_transformers_amd.config.base import ModelConfig
     from pytorch_transformers_amd.engine.spec import (CACHE_FULL, CACHE_STATE, INIT_NORMAL, MATRIX, CacheGroupSpec,
                                                       LayerCall, ModelSpec, TensorSpec)
@@ -296,6 +307,12 @@ def _define_toy():
 
         def forward(self, x, ctx, call, residual=None):
             table = ctx.cache.state_layer(call.cache_group, call.cache_layer)  # [slots, width], 32-bit
+            if device_decode and ctx.is_decode:
+                rows = ctx.seq_slot.long()  # one token per sequence: token t belongs to sequence t
+                s = self.decay * table.index_select(0, rows) + x.float()
+                table.index_copy_(0, rows, s)
+                out = (s @ self.weight.float().T).to(x.dtype)
+                return out if residual is None else out + residual
             out = torch.empty_like(x)
             at = 0
             for slot, n in zip(ctx.slots, ctx.new_tokens):
@@ -328,7 +345,7 @@ def _define_toy():
                          head=OutputHead("toy.head", cfg.vocab_size, cfg.width, "toy.embed.weight"),
                          cache_groups=[CacheGroupSpec("kv", CACHE_FULL, 1, 1, 16),
                                        CacheGroupSpec("state", CACHE_STATE, cfg.layers, state_shape=(cfg.width,))],
-                         supports_graphs=False)  # the toy mixer reads the step's host lists
+                         supports_graphs=device_decode)  # else the toy mixer reads the step's host lists
 
     return ToyConfig, build_toy
 
@@ -406,6 +423,45 @@ def test_toy_architecture_with_a_state_mixer(tmp_path, dtype, rel):
                 for _ in range(5):
                     toks.append(int(_plain_toy(cfg, w, toks)[-1].argmax()))
                 assert seq == toks
+    finally:
+        unregister("toy-decay")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_state_mixer_decodes_under_captured_steps(tmp_path, dtype):
+    """A model with a state group whose decode steps are captured and replayed gives the bits of the same steps
+    launched one by one: the first step of a shape runs once (not once to warm up and once as a replay), and the
+    rows that pad a batch to the captured size advance the scratch slot's state, never a sequence's.  Batches of
+    3, 5 and 11 sequences use padded shapes (4 rows; 8; 16), and sequences leave on the way."""
+    from pytorch_transformers_amd import AutoModelForCausalLM
+    from pytorch_transformers_amd.config import register, unregister
+    from pytorch_transformers_amd.engine.replay import Replayer
+    from pytorch_transformers_amd.weights import write_random_model
+
+    ToyConfig, build_toy = _define_toy(device_decode=True)
+    register("toy-decay", ToyConfig, build_toy, exist_ok=True)
+    try:
+        cfg = ToyConfig(decay=0.6, layers=3)
+        folder = write_random_model(str(tmp_path / "toy"), cfg, seed=6, std=0.08, noise=0.1)
+        reqs = helpers.make_requests(cfg.vocab_size, [9, 30, 70, 3, 41, 12, 25, 8, 19, 33, 50], seed=4)
+        records = helpers.schedule_batches(reqs, 3, decode=(5, 2, 8)) + \
+            [dict(r, step=r["step"] + 1000) for r in helpers.schedule_batches(reqs, 5, decode=(3, 7, 2, 6, 4))] + \
+            [dict(r, step=r["step"] + 2000) for r in helpers.schedule_batches(reqs, 11, decode=(2, 9, 4))]
+        outs = {}
+        for graphs in (False, True):
+            model = AutoModelForCausalLM.from_pretrained(folder, dtype=dtype)
+            assert model.use_graphs
+            model.use_graphs = graphs
+            rp = Replayer(model, 2048, max_slots=16)
+            outs[graphs] = [rp.run(rec) for rec in records]
+            torch.cuda.synchronize()
+            if graphs:
+                shapes = sorted(g.n for g in rp.cache._decode_graphs.values() if g.graph is not None)
+                assert len(shapes) >= 3 and shapes[-1] == 16, f"captured shapes: {shapes}"
+        for rec, a, b in zip(records, outs[False], outs[True]):
+            assert (a is None) == (b is None)
+            if a is not None:
+                assert torch.equal(a, b), f"step {rec['step']}: a captured step differs from the same step launched directly"
     finally:
         unregister("toy-decay")
 

@@ -123,6 +123,26 @@ def test_first_tokens(folders, dtype, rel):
     helpers.assert_close(got["r0"], want["r0"], rel, f"A {dtype} first tokens")
 
 
+def test_dtype_auto_follows_the_configuration_then_the_file(tmp_path):
+    """``dtype="auto"`` (src/transformers/modeling_utils.py:3996-4058): config.json's ``torch_dtype`` if it names
+    one, else the type of the first floating-point tensor of the file."""
+    from pytorch_transformers_amd import AutoModelForCausalLM
+    from pytorch_transformers_amd.config import AutoConfig
+    from pytorch_transformers_amd.weights import write_random_model
+
+    for i, (named, stored, want) in enumerate(((None, torch.float32, torch.float32), (None, torch.bfloat16, torch.bfloat16),
+                                               ("float32", torch.bfloat16, torch.float32),
+                                               ("bfloat16", torch.float32, torch.bfloat16),
+                                               ("float16", torch.float32, torch.bfloat16))):
+        cfg = AutoConfig.from_dict(dict(TINY["A"], torch_dtype=named))
+        folder = write_random_model(str(tmp_path / f"m{i}"), cfg, seed=1, store_dtype=stored)
+        model = AutoModelForCausalLM.from_pretrained(folder, dtype="auto")
+        assert model.dtype == want, f"torch_dtype={named}, file {stored}: got {model.dtype}"
+        assert model.spec.embedding.weight.dtype == want
+    with pytest.raises(ValueError):
+        AutoModelForCausalLM.from_pretrained(folder, dtype="int8")
+
+
 def test_cache_full_is_an_error(folders):
     from pytorch_transformers_amd.cache import CacheFull
 
@@ -157,6 +177,83 @@ def test_trace_run_program(folders, tmp_path, dtype):
                 row += 1
             fed[e["id"]] += len(e["tokens"])
         assert row == arr.shape[0]
+
+
+def test_two_processes_write_the_same_bfloat16_bits(folders, tmp_path):
+    """bfloat16 logits are a function of weights, tokens and schedule: two fresh processes of the replay program
+    write identical files.  The trace has a prompt long enough for the vendor library's product (300 rows), short
+    ones, a batch that decodes together and requests that join while others run."""
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    reqs = helpers.make_requests(TINY["C"]["vocab_size"], [300, 40, 7, 130], seed=9)
+    records = helpers.schedule_batches(reqs, 4, decode=(20, 9, 3, 14)) + \
+        [dict(r, step=r["step"] + 1000) for r in helpers.schedule_staggered(reqs, 2, decode=(4, 9, 2, 30), chunks=(None, 16, 1, 50))]
+    text = "".join(json.dumps(r) + "\n" for r in records)
+    outs = []
+    for run in range(2):
+        out = tmp_path / f"out{run}"
+        env = dict(os.environ, PTA_TUNE="0")
+        p = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folders["C"], "--dtype",
+                            "bfloat16", "--out", str(out), "--max-tokens", "1024"], input=text, capture_output=True,
+                           text=True, timeout=300, env=env)
+        assert p.returncode == 0, p.stderr[-2000:]
+        outs.append(out)
+    names = sorted(os.listdir(outs[0]))
+    assert names == sorted(os.listdir(outs[1])) and len(names) == len(records)
+    for name in names:
+        a, b = (np.fromfile(o / name, dtype="<u4") for o in outs)
+        assert np.array_equal(a, b), f"{name}: the two processes wrote different bits"
+
+
+def test_steps_time_nothing_unless_asked_and_a_table_carries_the_choices(folders):
+    """An untuned step makes no timed choice and keeps no half-gigabyte buffer; ``tune`` fills the table, the table
+    as plain data restores the same choices after they were forgotten, and logits follow the choices in use."""
+    from pytorch_transformers_amd import AutoModelForCausalLM, ops
+
+    model = AutoModelForCausalLM.from_pretrained(folders["C"], dtype="bfloat16")
+    ops.clear_tuning()
+    cache = model.new_cache(2048, max_slots=4)
+    slot = cache.alloc()
+    prompt = list(range(600))
+    before = model.step(cache, [slot], [prompt], "last").clone()
+    cache.free(slot)
+    assert ops._flush is None and not any(ops.tuning_table().values()), "a plain step timed something"
+    table = model.tune(prompt_lens=(600,), batches=(4, 40))
+    assert ops._flush is None, "the buffer for cold timings outlives tune()"
+    assert table["pair_parts"], "tune() of a parallel block times its pair launches"
+    import json as _json
+    table = _json.loads(_json.dumps(table))  # plain data
+    ops.clear_tuning()
+    assert not any(ops.tuning_table().values())
+    ops.load_tuning(table)
+    assert ops.tuning_table() == table
+    slot = cache.alloc()
+    tuned = model.step(cache, [slot], [prompt], "last").clone()
+    cache.free(slot)
+    ops.clear_tuning()
+    slot = cache.alloc()
+    again = model.step(cache, [slot], [prompt], "last").clone()
+    cache.free(slot)
+    assert torch.equal(before, again), "without a table the same step gives the same bits"
+    helpers.assert_close(tuned, before, 2e-2, "tuned against untuned logits")
+
+
+def test_logits_of_a_step_outlive_the_next_step(folders):
+    """What ``step`` returns is the caller's: the next step, replayed from the same captured graph, writes a
+    buffer of its own."""
+    from pytorch_transformers_amd import AutoModelForCausalLM
+
+    got = {}
+    for graphs in (False, True):
+        model = AutoModelForCausalLM.from_pretrained(folders["A"], dtype="bfloat16")
+        model.use_graphs = graphs
+        cache = model.new_cache(512, max_slots=2)
+        slots = [cache.alloc(), cache.alloc()]
+        model.step(cache, slots, [[1, 2, 3], [4, 5]], "last")
+        held = [model.step(cache, slots, [[6 + k], [9 + k]], "last") for k in range(4)]  # no clone by the caller
+        torch.cuda.synchronize()
+        got[graphs] = [h.clone() for h in held]
+    for k, (a, b) in enumerate(zip(got[False], got[True])):
+        assert torch.equal(a, b), f"the logits of step {k} were overwritten by a later replay"
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

@@ -127,8 +127,12 @@ def test_sharded_and_unprefixed_files(tmp_path):
     assert set(index["weight_map"]) == set(tensors)
     bare = str(tmp_path / "bare")  # saved from the base model: no "transformer." prefix (modeling_utils.py:4495-4512)
     save_weights(bare, {k[len("transformer."):] if k.startswith("transformer.") else k: v for k, v in tensors.items()})
-    a, b, c = (load_weights(f, specs, torch.float32, "cpu") for f in (one, sharded, bare))
+    prefix = lookup("falcon")[1](cfg).base_prefix
+    assert prefix == "transformer."  # the builder names it, the loader has no default of its own
+    a, b, c = (load_weights(f, specs, torch.float32, "cpu", base_prefix=prefix) for f in (one, sharded, bare))
     assert all(torch.equal(a[k], b[k]) and torch.equal(a[k], c[k]) for k in a)
+    with pytest.raises(WeightsError):
+        load_weights(bare, specs, torch.float32, "cpu")  # without the prefix the bare names are unexpected tensors
 
 
 def test_missing_files(tmp_path):
@@ -137,3 +141,17 @@ def test_missing_files(tmp_path):
         load_weights(str(tmp_path), specs, torch.float32, "cpu")
     with pytest.raises(FileNotFoundError, match="config.json"):
         AutoConfig.from_pretrained(str(tmp_path))
+
+
+def test_first_float_dtype_reads_the_headers(tmp_path):
+    """What ``dtype="auto"`` falls back on when config.json names no type: the first floating-point tensor's."""
+    from safetensors.torch import save_file
+
+    from pytorch_transformers_amd.weights.loader import first_float_dtype
+
+    for i, dt in enumerate((torch.float32, torch.bfloat16, torch.float16)):
+        folder = tmp_path / f"m{i}"
+        os.makedirs(folder)
+        save_file({"a.ids": torch.zeros(3, dtype=torch.int32), "b.weight": torch.zeros(2, 2, dtype=dt)},
+                  str(folder / "model.safetensors"), metadata={"format": "pt"})
+        assert first_float_dtype(str(folder)) == dt
