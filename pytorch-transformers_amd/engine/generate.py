@@ -30,6 +30,10 @@ class GenerateOutput:
     sequences: List[List[int]]
     scores: Optional[List[List]] = None  # per sequence, per new token: processed scores [vocab]
     logits: Optional[List[List]] = None  # per sequence, per new token: raw logits [vocab]
+    #: with ``keep_slots``: the cache that holds the sequences and each sequence's slot in it, for a later call
+    #: that goes on from there (the reference returns ``past_key_values`` for that, :3314-3322)
+    cache: Optional[object] = None
+    slots: Optional[List[int]] = None
 
 
 def _round_up(n: int, m: int) -> int:
@@ -58,7 +62,8 @@ def resolve_lengths(cfg: GenerationConfig, prompt_lens: Sequence[int]):
 
 def generate(model, prompts: Sequence[Sequence[int]], generation_config: Optional[GenerationConfig] = None, *,
              batch_size: Optional[int] = None, sampler=None, streamer=None, cache=None,
-             rng_ids: Optional[Sequence[int]] = None, tokenizer=None, **kwargs) -> Union[List[List[int]], GenerateOutput]:
+             rng_ids: Optional[Sequence[int]] = None, tokenizer=None, keep_slots: bool = False,
+             slots: Optional[Sequence[int]] = None, **kwargs) -> Union[List[List[int]], GenerateOutput]:
     """Generate for every prompt (a list of token ids); returns prompt + new tokens per prompt.
 
     ``generation_config`` defaults to the model's; keyword arguments override its fields
@@ -68,6 +73,13 @@ def generate(model, prompts: Sequence[Sequence[int]], generation_config: Optiona
     ``decode(ids) -> str``) is needed for ``stop_strings`` only: a sequence ends with the token that
     completes one of them in the text of its new tokens (src/transformers/generation/utils.py:1118-1125,
     stopping_criteria.py:110-443; the token is kept, as the reference keeps it).
+
+    ``keep_slots``: sequences keep their cache slots when they end instead of giving them back, and the result
+    is a ``GenerateOutput`` with ``cache`` and ``slots``.  A later call goes on from there when it is given that
+    cache, those ``slots`` and, as prompts, the whole sequences so far: only the tokens a slot does not hold yet
+    are run (the reference continues from a returned cache the same way, src/transformers/generation/utils.py
+    :349-481, tests/generation/test_utils.py:1775-1855).  Whoever keeps slots frees them (``cache.free``), or
+    hands them to a call without ``keep_slots``, which frees them when it ends.
     """
     cfg = generation_config or getattr(model, "generation_config", None) or GenerationConfig()
     if kwargs:
@@ -82,6 +94,19 @@ def generate(model, prompts: Sequence[Sequence[int]], generation_config: Optiona
                 raise ValueError(f"prompt {i} is empty and no bos_token_id is set")
             prompts[i] = [int(bos)]
     n_ret = cfg.num_return_sequences
+    if slots is not None:
+        slots = [int(s_) for s_ in slots]
+        if cache is None:
+            raise ValueError("slots to go on from need the cache they live in")
+        if n_ret > 1:
+            raise ValueError("a call that goes on from kept slots returns one sequence per slot")
+        if len(slots) != len(prompts) or len(set(slots)) != len(slots):
+            raise ValueError(f"{len(prompts)} prompts but slots {slots}: one slot of its own per prompt")
+        for p, s_ in zip(prompts, slots):
+            held = cache.length(s_)
+            if held >= len(p):
+                raise ValueError(f"slot {s_} already holds {held} tokens, the sequence given for it has {len(p)}: "
+                                 "give the whole sequence so far, which ends with a token that has not been run yet")
     if n_ret > 1:  # :2244-2249, :716-748
         prompts = [p for p in prompts for _ in range(n_ret)]
     ids = list(rng_ids) if rng_ids is not None else list(range(len(prompts)))
@@ -92,13 +117,14 @@ def generate(model, prompts: Sequence[Sequence[int]], generation_config: Optiona
 
     batch_size = batch_size or len(prompts)
     batches = [list(range(b, min(b + batch_size, len(prompts)))) for b in range(0, len(prompts), batch_size)]
-    need = 0
     page = cache.page_size if cache is not None else getattr(model, "page_size", 64)
+    per_batch = []
     for b in batches:
         new, _ = resolve_lengths(cfg, [len(prompts[i]) for i in b])
-        need = max(need, sum(_round_up(len(prompts[i]) + new, page) for i in b))
-    if cache is None:
-        cache = model.new_cache(need, max_slots=batch_size)
+        per_batch.append(sum(_round_up(len(prompts[i]) + new, page) for i in b))
+    if cache is None:  # kept slots stay held while later batches run
+        cache = model.new_cache(sum(per_batch) if keep_slots else max(per_batch),
+                                max_slots=len(prompts) if keep_slots else batch_size)
     if sampler is None:
         from ..sampling.sampler import Sampler
 
@@ -115,13 +141,24 @@ def generate(model, prompts: Sequence[Sequence[int]], generation_config: Optiona
     out_tokens: List[List[int]] = [[] for _ in prompts]
     out_scores = [[] for _ in prompts] if want_scores else None
     out_logits = [[] for _ in prompts] if want_logits else None
+    kept = [None] * len(prompts)
     t0 = time.time()
+
+    def done_with(i: int, slot: int) -> None:
+        if keep_slots:
+            kept[i] = slot
+        else:
+            cache.free(slot)
 
     for batch in batches:
         new_budget, padded_len = resolve_lengths(cfg, [len(prompts[i]) for i in batch])
-        slot_of = {i: cache.alloc() for i in batch}
+        if slots is not None:  # going on: each sequence's slot holds its first tokens already
+            slot_of = {i: slots[i] for i in batch}
+            feed = {i: prompts[i][cache.length(slots[i]):] for i in batch}
+        else:
+            slot_of = {i: cache.alloc() for i in batch}
+            feed = {i: prompts[i] for i in batch}
         live = list(batch)
-        feed = {i: prompts[i] for i in batch}
         step_no = 0
         try:
             while live:
@@ -147,17 +184,24 @@ def generate(model, prompts: Sequence[Sequence[int]], generation_config: Optiona
                         streamer(i, tok)
                     said_stop = bool(stop_strings) and _ends_with_stop(tokenizer, out_tokens[i], stop_strings)
                     if tok in eos or step_no >= new_budget or timed_out or said_stop:
-                        cache.free(slot_of.pop(i))
+                        done_with(i, slot_of.pop(i))
                     else:
                         feed[i] = [tok]
                         still.append(i)
                 live = still
-        finally:
-            for i in list(slot_of):
+        except BaseException:
+            for i in list(slot_of):  # a step failed: nothing of this batch can be gone on from
                 cache.free(slot_of.pop(i))
+            for i in batch:
+                if kept[i] is not None:
+                    cache.free(kept[i])
+                    kept[i] = None
+            raise
     if streamer is not None and hasattr(streamer, "end"):
         streamer.end()
     sequences = [p + t for p, t in zip(prompts, out_tokens)]
+    if keep_slots:
+        return GenerateOutput(sequences, out_scores, out_logits, cache=cache, slots=kept)
     if cfg.return_dict_in_generate:
         return GenerateOutput(sequences, out_scores, out_logits)
     return sequences

@@ -18,18 +18,17 @@ import json
 import sys
 import tempfile
 
-MAX_LENGTH = int(10000)  # run_generation.py:49: hard cap against an endless loop
-
-
-def adjust_length_to_model(length: int, max_sequence_length: int) -> int:
-    """run_generation.py:151-158."""
-    if length < 0 and max_sequence_length > 0:
-        return max_sequence_length
-    if 0 < max_sequence_length < length:
-        return max_sequence_length
+def new_token_budget(length: int, context: int, longest_prompt: int) -> int:
+    """New tokens for ``--length``.  The reference's example caps the request at the model's trained context and
+    reads a negative length as "as long as the model allows" (run_generation.py:151-158, :371-376).  Here the
+    sequence as a whole stays within the trained context where the configuration names one; nothing else limits
+    it, because the cache is sized for what is asked."""
+    room = max(1, context - longest_prompt) if context > 0 else None
     if length < 0:
-        return MAX_LENGTH
-    return length
+        if room is None:
+            raise ValueError("--length is negative and the configuration names no context length to fill")
+        return room
+    return length if room is None else min(length, room)
 
 
 def build_parser() -> argparse.ArgumentParser:
@@ -93,7 +92,8 @@ def main(argv=None) -> int:
         text = args.prompt if args.prompt else input("Model prompt >>> ")  # run_generation.py:365
         prompts = [text]
 
-    length = adjust_length_to_model(args.length, getattr(config, "max_position_embeddings", 0))
+    longest = max((len(p) for p in prompts if not isinstance(p, str)), default=0)
+    length = new_token_budget(args.length, int(getattr(config, "max_position_embeddings", 0) or 0), longest)
     gen = dict(max_new_tokens=length, min_new_tokens=args.min_new_tokens, seed=args.seed,
                repetition_penalty=args.repetition_penalty, num_return_sequences=args.num_return_sequences)
     if args.stop_token_id is not None:

@@ -208,3 +208,44 @@ def test_stop_strings_need_a_tokenizer_and_end_a_sequence_with_the_completing_to
 def test_pad_sequences_matches_the_reference_layout():
     t = pad_sequences([[1, 2, 3, 9, 9], [4, 8]], [3, 1], pad_token_id=0)
     assert t.tolist() == [[1, 2, 3, 9, 9], [0, 0, 4, 8, 0]]
+
+
+def test_kept_slots_go_on_in_a_later_call():
+    """Four new tokens at once equal three and then one from the kept slots (the reference's test of continuing
+    from a returned cache, tests/generation/test_utils.py:1775-1855); the later call runs only the tokens that
+    the slots do not hold, and whoever does not keep the slots gives them back."""
+    m = ScriptedModel()
+    prompts = [[1, 2, 3], [4], [5, 6, 7, 8]]
+    at_once = generate(m, prompts, GenerationConfig(max_new_tokens=4), sampler=ArgmaxSampler())
+    m2 = ScriptedModel()
+    first = generate(m2, prompts, GenerationConfig(max_new_tokens=3), sampler=ArgmaxSampler(), keep_slots=True,
+                     cache=m2.new_cache(64 * 8, max_slots=4))
+    assert isinstance(first, GenerateOutput) and sorted(first.slots) == [0, 1, 2]
+    cache = first.cache
+    assert sorted(cache.live_slots()) == [0, 1, 2]
+    assert [cache.length(s) for s in first.slots] == [len(seq) - 1 for seq in first.sequences]  # the last token is not run yet
+    steps_before = len(m2.steps)
+    more = generate(m2, first.sequences, GenerationConfig(max_new_tokens=1), sampler=ArgmaxSampler(), cache=cache,
+                    slots=first.slots)
+    assert more == at_once
+    assert m2.steps[steps_before:] == [(first.slots, [[seq[-1]] for seq in first.sequences])]  # one token each, no prompt again
+    assert cache.live_slots() == [] and cache.free_pages() == cache.num_pages
+    # one sequence ends early by its stop token and still keeps its slot; batches one after another keep all
+    m3 = ScriptedModel()
+    eos = expected(prompts[1], 2)[-1]
+    out = generate(m3, prompts, GenerationConfig(max_new_tokens=3, eos_token_id=eos), sampler=ArgmaxSampler(), keep_slots=True,
+                   batch_size=2)
+    assert len(out.sequences[1]) == len(prompts[1]) + 2 and all(s is not None for s in out.slots)
+    assert sorted(out.cache.live_slots()) == sorted(out.slots)
+    for s in out.slots:
+        out.cache.free(s)
+    # misuse is refused before anything runs
+    with pytest.raises(ValueError, match="cache"):
+        generate(m3, prompts, GenerationConfig(max_new_tokens=1), sampler=ArgmaxSampler(), slots=[0, 1, 2])
+    c = m3.new_cache(256, max_slots=2)
+    a = c.alloc()
+    c.reserve([a], [3]); c.commit([a], [3])
+    with pytest.raises(ValueError, match="already holds"):
+        generate(m3, [[1, 2, 3]], GenerationConfig(max_new_tokens=1), sampler=ArgmaxSampler(), cache=c, slots=[a])
+    with pytest.raises(ValueError, match="one slot"):
+        generate(m3, [[1, 2, 3, 4], [1, 2, 3, 4]], GenerationConfig(max_new_tokens=1), sampler=ArgmaxSampler(), cache=c, slots=[a, a])

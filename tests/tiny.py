@@ -36,10 +36,18 @@ TINY = {
 SEEDS = {"A": 0, "B": 1, "C": 2, "D": 3, "E": 4}
 
 
-def write_model(name: str, folder: str, noise: float = 0.1) -> str:
-    """Write tiny model ``name`` with the framework's random-weights mode; returns the folder."""
+LIVELY_STD = 0.2
+
+
+def write_model(name: str, folder: str, noise: float = 0.1, std=None) -> str:
+    """Write tiny model ``name`` with the framework's random-weights mode; returns the folder.
+
+    ``std`` (default: the configuration's ``initializer_range``, 0.02): with weights that small and a tied head a
+    tiny model's likeliest next token is its last token over and over, whatever its layers do; tests that compare
+    generated tokens pass ``LIVELY_STD``, with which greedy tokens keep changing."""
     from pytorch_transformers_amd.config import AutoConfig
     from pytorch_transformers_amd.weights import write_random_model
 
     cfg = AutoConfig.from_dict(TINY[name])
-    return write_random_model(os.path.join(folder, name), cfg, SEEDS[name], noise=noise)
+    sub = name if std is None else f"{name}-std{std}"
+    return write_random_model(os.path.join(folder, sub), cfg, SEEDS[name], noise=noise, std=std)
