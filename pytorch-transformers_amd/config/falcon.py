@@ -23,12 +23,12 @@ NORMS_SINGLE = "single"  # input_layernorm feeds attention and MLP
 NORMS_DUAL = "dual"  # ln_attn feeds attention, ln_mlp feeds the MLP
 NORMS_SEQUENTIAL = "sequential"  # input_layernorm, then post_attention_layernorm on x + attn
 
-# src/transformers/activations.py:200-220, all but "laplace"
+# src/transformers/activations.py:200-220
 ACTIVATIONS_BUILT = ("gelu", "gelu_10", "gelu_fast", "gelu_new", "gelu_python", "gelu_pytorch_tanh", "gelu_accurate",
-                     "leaky_relu", "linear", "mish", "quick_gelu", "relu", "relu2", "relu6", "sigmoid", "silu", "swish",
-                     "tanh")
-ROPE_TYPES_BUILT = ("default", "linear", "yarn", "llama3")  # the two others change with the length of the sequence
+                     "laplace", "leaky_relu", "linear", "mish", "quick_gelu", "relu", "relu2", "relu6", "sigmoid", "silu",
+                     "swish", "tanh")
 ROPE_TYPES_KNOWN = ("default", "linear", "dynamic", "yarn", "longrope", "llama3")  # modeling_rope_utils.py:351-358
+ROPE_TYPES_BUILT = ROPE_TYPES_KNOWN
 
 
 @dataclasses.dataclass
@@ -130,8 +130,24 @@ class FalconConfig(ModelConfig):
                     if not isinstance(v, (int, float)) or isinstance(v, bool) or (least is not None and v < least):
                         raise ConfigError(f"rope_scaling {key} must be a number" + (f" >= {least}" if least is not None else "")
                                           + f", got {v!r}")
-                if kind in ("linear", "yarn", "llama3"):
-                    number("factor", 1.0)  # modeling_rope_utils.py:392-394, :432-434, :512-514
+                if kind in ("linear", "dynamic", "yarn", "llama3"):
+                    number("factor", 1.0)  # modeling_rope_utils.py:392-394, :409-411, :432-434, :512-514
+                if kind == "dynamic" and self.head_dim <= 2:  # the stretched base has the exponent d / (d - 2) (:157)
+                    raise ConfigError("rope_scaling type 'dynamic' needs a head size above 2")
+                if kind == "longrope":  # :453-503
+                    half = self.head_dim // 2
+                    for key in ("short_factor", "long_factor"):
+                        v = self.rope_scaling.get(key)
+                        if (not isinstance(v, (list, tuple)) or len(v) != half
+                                or not all(isinstance(x, (int, float)) and not isinstance(x, bool) and x > 0 for x in v)):
+                            raise ConfigError(f"rope_scaling {key} must be a list of {half} positive numbers, got {v!r}")
+                    number("attention_factor", 0.0, required=False)
+                    original = self.extra.get("original_max_position_embeddings")
+                    if original is not None:
+                        if not isinstance(original, int) or isinstance(original, bool) or original <= 0:
+                            raise ConfigError(f"original_max_position_embeddings must be a positive integer, got {original!r}")
+                    elif self.rope_scaling.get("attention_factor") is None:
+                        number("factor", 1.0)
                 if kind == "yarn":  # :424-450
                     number("attention_factor", 0.0, required=False)
                     number("beta_fast", required=False)

@@ -10,7 +10,7 @@
 
 enum PtaDtype { PTA_F32 = 0, PTA_BF16 = 1 };
 
-// fused query_key_value row orders (see config.falcon)
+// orders of the rows of a fused query_key_value projection (described in rope_cache.hip)
 enum PtaQkvLayout { PTA_QKV_GROUPED = 0, PTA_QKV_TAIL = 1, PTA_QKV_INTERLEAVED = 2 };
 
 // activations of an epilogue, by the reference's names (src/transformers/activations.py:200-220)
@@ -28,7 +28,8 @@ enum PtaAct {
     PTA_ACT_LEAKY_RELU = 10, // slope 0.01
     PTA_ACT_MISH = 11,       // x * tanh(softplus(x))
     PTA_ACT_GELU_10 = 12,    // exact GELU clipped to [-10, 10]
-    PTA_ACT_COUNT = 13
+    PTA_ACT_LAPLACE = 13,    // the normal distribution function with mean 0.707107, deviation 0.282095
+    PTA_ACT_COUNT = 14
 };
 
 typedef uint16_t bf16_t;  // raw bits of a bfloat16
@@ -146,6 +147,7 @@ __device__ __forceinline__ float apply_act(float x, int act) {
         case PTA_ACT_LEAKY_RELU: return x >= 0.f ? x : 0.01f * x;
         case PTA_ACT_MISH: return x * tanhf(x > 20.f ? x : log1pf(expf(x)));
         case PTA_ACT_GELU_10: return fminf(fmaxf(gelu_erf(x), -10.f), 10.f);
+        case PTA_ACT_LAPLACE: return 0.5f * (1.0f + erff((x - 0.707107f) / (0.282095f * 1.41421356237309504880f)));
         default: return x;
     }
 }

@@ -198,9 +198,10 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(SkinnyProblem pa, Skin
                     }
                 }
                 if (tail.inv_freq && kind != 2) {
+                    const float* freq = qkv_tail_freq(tail, m);
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        const float ang = (float)pos * tail.inv_freq[i0 + e];
+                        const float ang = (float)pos * freq[i0 + e];
                         const float c = cosf(ang) * tail.cs_scale, sn = sinf(ang) * tail.cs_scale;
                         const float x0 = a[e], x1 = b[e];
                         a[e] = x0 * c - x1 * sn;
@@ -362,7 +363,8 @@ extern "C" int pta_gemm_skinny_bf16(void* y, const void* x, const void* W, const
 // cache pages of their sequences, as pta_qkv_rope_cache would have left them.  Up to 16 rows, head sizes that are
 // multiples of 32.  The second product is y2 = act2(x2 . W2^T + bias2) as in the plain pair.
 extern "C" int pta_gemm_skinny_pair_qkv_bf16(void* q_out, const void* x1, const void* W1, const float* bias1,
-                                             const float* inv_freq, float cs_scale, const int* token_pos,
+                                             const float* inv_freq, int inv_freq_ld, float cs_scale,
+                                             const int* token_pos,
                                              const int* token_seq, const int* block_table, int bt_stride, void* k_pool,
                                              void* v_pool, int nh, int nkv, int d, int layout, int write_cache, void* y2,
                                              const void* x2, const void* W2, const float* bias2, int N2, int act2, int M,
@@ -377,11 +379,13 @@ extern "C" int pta_gemm_skinny_pair_qkv_bf16(void* q_out, const void* x1, const 
     PTA_REQUIRE(layout != PTA_QKV_TAIL || nkv == 1, "gemm_skinny_pair_qkv_bf16: the tail layout has one kv head, got %d", nkv);
     PTA_REQUIRE(layout != PTA_QKV_INTERLEAVED || nkv == nh, "gemm_skinny_pair_qkv_bf16: the interleaved layout needs kv heads == heads");
     PTA_REQUIRE(token_pos, "gemm_skinny_pair_qkv_bf16: null token positions");
+    PTA_REQUIRE(inv_freq_ld == 0 || (inv_freq && token_seq && inv_freq_ld >= d / 2),
+                "gemm_skinny_pair_qkv_bf16: a frequency table per sequence needs the tokens' sequences and rows of %d", d / 2);
     PTA_REQUIRE(!write_cache || (k_pool && v_pool && block_table && token_seq), "gemm_skinny_pair_qkv_bf16: null cache pointer");
     PTA_REQUIRE((((uintptr_t)q_out | (uintptr_t)k_pool) % 8) == 0, "gemm_skinny_pair_qkv_bf16: outputs must be 8-byte aligned");
     SkinnyProblem a{nullptr, (const bf16_t*)x1, (const bf16_t*)W1, bias1, nullptr, nullptr, N1, PTA_ACT_NONE, 0};
     SkinnyProblem b{y2, (const bf16_t*)x2, (const bf16_t*)W2, bias2, nullptr, nullptr, N2, in_kernel(act2) ? act2 : 0, 0};
-    const QkvTail tail{(bf16_t*)q_out, inv_freq, cs_scale, token_pos, token_seq, block_table, bt_stride, (bf16_t*)k_pool,
+    const QkvTail tail{(bf16_t*)q_out, inv_freq, inv_freq_ld, cs_scale, token_pos, token_seq, block_table, bt_stride, (bf16_t*)k_pool,
                        (bf16_t*)v_pool, nh, nkv, d, layout, write_cache};
     // the first product's workgroups are bound to heads; the second one's fill the launch up to a whole number per unit
     a.blocks = (nh + 2 * nkv) * (d / 32);

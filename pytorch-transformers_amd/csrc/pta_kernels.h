@@ -14,7 +14,7 @@
 
 #include <stdint.h>
 
-#define PTA_ABI_VERSION 1
+#define PTA_ABI_VERSION 2
 
 #ifdef __cplusplus
 extern "C" {
@@ -44,8 +44,11 @@ int pta_layernorm_sum_ok(int H);
 int pta_epilogue(void* y, int ld_y, const float* bias, const void* add1, const void* add2, int M, int N, int act,
                  int dtype, void* stream);
 
-// split fused qkv rows, add bias, rotate q and k (inv_freq null: no rotation), write q and append k, v
-int pta_qkv_rope_cache(void* q_out, const void* fused, int fused_ld, const float* bias, const float* inv_freq, float cs_scale,
+// split fused qkv rows, add bias, rotate q and k (inv_freq null: no rotation), write q and append k, v.
+// inv_freq_ld (here and in the three launches below that rotate): 0 for one table [d/2] for all tokens, else a
+// table per sequence of the step, [sequences, inv_freq_ld], found through token_seq
+int pta_qkv_rope_cache(void* q_out, const void* fused, int fused_ld, const float* bias, const float* inv_freq,
+                       int inv_freq_ld, float cs_scale,
                        const int* token_pos, const int* token_seq, const int* block_table, int bt_stride,
                        void* k_pool, void* v_pool, int M, int nh, int nkv, int d, int layout, int write_cache,
                        int dtype, void* stream);
@@ -88,7 +91,8 @@ int pta_gemm_skinny_pair_bf16(void* y1, const void* x1, const void* W1, const fl
 // are split, rotated and written as queries [M, heads, d] and into the cache pages, as pta_qkv_rope_cache leaves
 // them; head sizes that are multiples of 32
 int pta_gemm_skinny_pair_qkv_bf16(void* q_out, const void* x1, const void* W1, const float* bias1,
-                                  const float* inv_freq, float cs_scale, const int* token_pos, const int* token_seq,
+                                  const float* inv_freq, int inv_freq_ld, float cs_scale, const int* token_pos,
+                                  const int* token_seq,
                                   const int* block_table, int bt_stride, void* k_pool, void* v_pool, int nh, int nkv,
                                   int d, int layout, int write_cache, void* y2, const void* x2, const void* W2,
                                   const float* bias2, int N2, int act2, int M, int K, void* stream);
@@ -110,16 +114,24 @@ int pta_gemm_splitk_pair_parts(int N1, int K1, int N2, int K2, int* parts1, int*
 // the pair run to the end with the first product a fused query_key_value projection (N1 = (nh + 2 nkv) d rows of
 // W1): queries rotated in q_out [M, nh, d], keys and values in the cache pages, as pta_qkv_rope_cache leaves them
 int pta_gemm_splitk_pair_reduced_qkv_bf16(void* q_out, float* part1, const void* x1, const void* W1, const float* bias1,
-                                          int K1, const float* inv_freq, float cs_scale, const int* token_pos,
+                                          int K1, const float* inv_freq, int inv_freq_ld, float cs_scale,
+                                          const int* token_pos,
                                           const int* token_seq, const int* block_table, int bt_stride, void* k_pool,
                                           void* v_pool, int nh, int nkv, int d, int layout, int write_cache, void* y2,
                                           float* part2, const void* x2, const void* W2, const float* bias2, int N2, int K2,
                                           int act2, int M, void* stream);
 // such a projection on its own: part [pta_gemm_splitk_parts(N, K, 0, 0), M, N] is the workspace
 int pta_gemm_splitk_reduced_qkv_bf16(void* q_out, float* part, const void* x, const void* W, const float* bias, int K,
-                                     const float* inv_freq, float cs_scale, const int* token_pos, const int* token_seq,
+                                     const float* inv_freq, int inv_freq_ld, float cs_scale, const int* token_pos,
+                                     const int* token_seq,
                                      const int* block_table, int bt_stride, void* k_pool, void* v_pool, int nh, int nkv,
                                      int d, int layout, int write_cache, int M, void* stream);
+
+// a frequency table per sequence of the step, out [n_seqs, d/2], for frequencies that follow the sequence's length
+// after the step (seq_start[s] + its tokens): 1 / base^(2i/d) with base = theta while that length is at most
+// max_pos, else theta * (factor * length / max_pos - (factor - 1))^(d / (d - 2))
+int pta_rope_dynamic_table(float* out, const int* seq_start, const int* cu_tokens, int n_seqs, int d, float theta,
+                           float factor, int max_pos, void* stream);
 
 // y[M, N] = act(sum of part[P, M, N] over P, in order, + bias) + add1 + add2: the reduction of the products above
 // on its own, for 32-bit partial sums over ranges of K that the vendor library's batched product made

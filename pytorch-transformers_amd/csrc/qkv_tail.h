@@ -8,6 +8,7 @@
 struct QkvTail {
     bf16_t* q_out;  // [M, heads, d]
     const float* inv_freq;  // [d/2], or null: no rotation
+    int inv_freq_ld;        // 0: one table for all tokens; else a table per sequence of the step, this many apart
     float cs_scale;
     const int* token_pos;
     const int* token_seq;
@@ -17,6 +18,11 @@ struct QkvTail {
     bf16_t* v_pool;
     int nh, nkv, d, layout, write_cache;
 };
+
+// the frequency table of token m
+__device__ __forceinline__ const float* qkv_tail_freq(const QkvTail& t, int m) {
+    return t.inv_freq + (t.inv_freq_ld ? (long)t.token_seq[m] * t.inv_freq_ld : 0L);
+}
 
 // segment `seg` of d features of the fused row: kind 0 query, 1 key, 2 value, and which head
 __device__ __forceinline__ void qkv_tail_segment(const QkvTail& t, int seg, int& kind, int& head) {
@@ -47,7 +53,7 @@ __device__ __forceinline__ void qkv_tail_pair(const QkvTail& t, const float* __r
         b = round_to_bf16(b + bias[seg * d + half + i]);
     }
     if (t.inv_freq && kind != 2) {
-        const float ang = (float)pos * t.inv_freq[i];
+        const float ang = (float)pos * qkv_tail_freq(t, m)[i];
         const float c = cosf(ang) * t.cs_scale, sn = sinf(ang) * t.cs_scale;
         const float x0 = a, x1 = b;
         a = x0 * c - x1 * sn;

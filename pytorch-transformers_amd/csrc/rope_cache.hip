@@ -20,7 +20,7 @@
 template <typename T>
 __global__ __launch_bounds__(RC_THREADS) void qkv_rope_cache_kernel(
     T* __restrict__ q_out, const T* __restrict__ fused, long fused_ld, const float* __restrict__ bias,
-    const float* __restrict__ inv_freq, float cs_scale, const int* __restrict__ token_pos,
+    const float* __restrict__ inv_freq, int inv_freq_ld, float cs_scale, const int* __restrict__ token_pos,
     const int* __restrict__ token_seq, const int* __restrict__ block_table, int bt_stride, T* __restrict__ k_pool,
     T* __restrict__ v_pool, int nh, int nkv, int d, int layout, int write_cache) {
     __shared__ float cos_s[128], sin_s[128];
@@ -28,8 +28,10 @@ __global__ __launch_bounds__(RC_THREADS) void qkv_rope_cache_kernel(
     const int g = nh / nkv, half = d >> 1;
     const int pos = token_pos[m];
     if (inv_freq) {
+        // one table for all tokens, or one per sequence of the step (frequencies that follow a sequence's length)
+        const float* freq = inv_freq + (inv_freq_ld ? (long)token_seq[m] * inv_freq_ld : 0L);
         for (int i = tid; i < half; i += RC_THREADS) {
-            const float ang = (float)pos * inv_freq[i];
+            const float ang = (float)pos * freq[i];
             cos_s[i] = cosf(ang) * cs_scale;
             sin_s[i] = sinf(ang) * cs_scale;
         }
@@ -118,7 +120,7 @@ __global__ __launch_bounds__(RC_THREADS) void qkv_rope_cache_kernel(
 }
 
 extern "C" int pta_qkv_rope_cache(void* q_out, const void* fused, int fused_ld, const float* bias, const float* inv_freq,
-                                  float cs_scale, const int* token_pos, const int* token_seq,
+                                  int inv_freq_ld, float cs_scale, const int* token_pos, const int* token_seq,
                                   const int* block_table, int bt_stride, void* k_pool, void* v_pool, int M, int nh,
                                   int nkv, int d, int layout, int write_cache, int dtype, void* stream) {
     PTA_REQUIRE(M > 0 && nh > 0 && nkv > 0 && d > 0, "qkv_rope_cache: sizes must be positive (M=%d nh=%d nkv=%d d=%d)", M, nh, nkv, d);
@@ -128,6 +130,8 @@ extern "C" int pta_qkv_rope_cache(void* q_out, const void* fused, int fused_ld, 
     PTA_REQUIRE(layout != PTA_QKV_INTERLEAVED || nkv == nh, "qkv_rope_cache: the interleaved layout needs kv heads == heads");
     PTA_REQUIRE(!inv_freq || (d % 2 == 0 && d <= 256), "qkv_rope_cache: rotation needs an even head size up to 256, got %d", d);
     PTA_REQUIRE(!write_cache || (k_pool && v_pool && block_table && token_seq), "qkv_rope_cache: null cache pointer");
+    PTA_REQUIRE(inv_freq_ld == 0 || (inv_freq && token_seq && inv_freq_ld >= d / 2),
+                "qkv_rope_cache: a frequency table per sequence needs the tokens' sequences and rows of %d", d / 2);
     PTA_REQUIRE(fused_ld >= (long)(nh + 2 * nkv) * d, "qkv_rope_cache: fused rows of %ld elements cannot lie %d apart",
                 (long)(nh + 2 * nkv) * d, fused_ld);
     PTA_REQUIRE(dtype != PTA_BF16 || d % 16 != 0 ||
@@ -138,13 +142,39 @@ extern "C" int pta_qkv_rope_cache(void* q_out, const void* fused, int fused_ld, 
     while (slices < 16 && M * slices < 512 && slices * RC_THREADS < (nh + 2 * nkv) * d) slices *= 2;
     if (dtype == PTA_F32)
         hipLaunchKernelGGL(qkv_rope_cache_kernel<float>, dim3(M, slices), dim3(RC_THREADS), 0, s, (float*)q_out,
-                           (const float*)fused, fused_ld, bias, inv_freq, cs_scale, token_pos, token_seq, block_table, bt_stride,
+                           (const float*)fused, fused_ld, bias, inv_freq, inv_freq_ld, cs_scale, token_pos, token_seq, block_table, bt_stride,
                            (float*)k_pool, (float*)v_pool, nh, nkv, d, layout, write_cache);
     else if (dtype == PTA_BF16)
         hipLaunchKernelGGL(qkv_rope_cache_kernel<bf16_t>, dim3(M, slices), dim3(RC_THREADS), 0, s, (bf16_t*)q_out,
-                           (const bf16_t*)fused, fused_ld, bias, inv_freq, cs_scale, token_pos, token_seq, block_table,
+                           (const bf16_t*)fused, fused_ld, bias, inv_freq, inv_freq_ld, cs_scale, token_pos, token_seq, block_table,
                            bt_stride, (bf16_t*)k_pool, (bf16_t*)v_pool, nh, nkv, d, layout, write_cache);
     else
         return pta_fail("qkv_rope_cache: unknown dtype %d", dtype);
     return pta_check_launch("qkv_rope_cache");
+}
+
+// Frequencies that follow each sequence's length (dynamic NTK scaling, src/transformers/modeling_rope_utils.py:112-160):
+// out[s, i] = 1 / base_s^(2i/d), base_s = theta * (factor * len_s / max_pos - (factor - 1))^(d / (d - 2)) once the
+// sequence's length after this step, len_s = seq_start[s] + its tokens of the step, exceeds max_pos, else theta.
+// Evaluated in double precision and rounded once.
+__global__ void rope_dynamic_table_kernel(float* __restrict__ out, const int* __restrict__ seq_start,
+                                          const int* __restrict__ cu_tokens, int n_seqs, int half, double theta,
+                                          double factor, int max_pos) {
+    const int s = blockIdx.x;
+    const int len = seq_start[s] + cu_tokens[s + 1] - cu_tokens[s];
+    const int d = 2 * half;
+    double base = theta;
+    if (len > max_pos) base = theta * pow(factor * (double)len / (double)max_pos - (factor - 1.0), (double)d / (double)(d - 2));
+    for (int i = threadIdx.x; i < half; i += blockDim.x) out[(long)s * half + i] = (float)(1.0 / pow(base, (double)(2 * i) / (double)d));
+}
+
+extern "C" int pta_rope_dynamic_table(float* out, const int* seq_start, const int* cu_tokens, int n_seqs, int d,
+                                      float theta, float factor, int max_pos, void* stream) {
+    PTA_REQUIRE(out && seq_start && cu_tokens, "rope_dynamic_table: null pointer");
+    PTA_REQUIRE(n_seqs > 0 && d > 2 && d % 2 == 0, "rope_dynamic_table: %d sequences, head size %d (even, more than 2)", n_seqs, d);
+    PTA_REQUIRE(theta > 0.f && factor >= 1.f && max_pos > 0, "rope_dynamic_table: theta %g, factor %g, positions %d", theta,
+                factor, max_pos);
+    hipLaunchKernelGGL(rope_dynamic_table_kernel, dim3(n_seqs), dim3(64), 0, (hipStream_t)stream, out, seq_start, cu_tokens,
+                       n_seqs, d / 2, (double)theta, (double)factor, max_pos);
+    return pta_check_launch("rope_dynamic_table");
 }

@@ -11,7 +11,7 @@ from ..config.falcon import NORMS_DUAL, NORMS_SEQUENTIAL, FalconConfig
 from ..config.registry import register
 from ..parts import (AlibiPositions, AttentionMixer, DenseFeedForward, Embedding, LayerNorm, OutputHead,
                      ParallelBlock, RotaryPositions, SequentialBlock)
-from ..parts.positions import llama3_frequencies, yarn_frequencies
+from ..parts.positions import llama3_frequencies, longrope_frequencies, yarn_frequencies
 from .spec import CACHE_FULL, CacheGroupSpec, LayerCall, ModelSpec
 
 KV_GROUP = "kv"
@@ -31,6 +31,14 @@ def rotary_positions(cfg: FalconConfig) -> RotaryPositions:
         inv = llama3_frequencies(cfg.head_dim, cfg.rope_theta, float(rs["factor"]), float(rs["low_freq_factor"]),
                                  float(rs["high_freq_factor"]), int(rs["original_max_position_embeddings"]))
         return RotaryPositions(cfg.head_dim, cfg.rope_theta, inv_freq=inv)
+    if kind == "dynamic":
+        return RotaryPositions(cfg.head_dim, cfg.rope_theta, dynamic_factor=float(rs["factor"]),
+                               trained_positions=cfg.max_position_embeddings)
+    if kind == "longrope":
+        inv, scale = longrope_frequencies(cfg.head_dim, cfg.rope_theta, rs["short_factor"], rs.get("factor"),
+                                          cfg.max_position_embeddings, cfg.extra.get("original_max_position_embeddings"),
+                                          rs.get("attention_factor"))
+        return RotaryPositions(cfg.head_dim, cfg.rope_theta, attention_scaling=scale, inv_freq=inv)
     return RotaryPositions(cfg.head_dim, cfg.rope_theta)
 
 

@@ -23,8 +23,8 @@ QKV_LAYOUT_CODES = {"grouped": 0, "tail": 1, "interleaved": 2}
 # activations by the reference's names (src/transformers/activations.py:200-220) -> codes of csrc/common.h
 ACT_CODES = {None: 0, "none": 0, "linear": 0, "gelu": 1, "gelu_python": 1, "gelu_new": 2, "gelu_pytorch_tanh": 2,
              "gelu_fast": 2, "gelu_accurate": 2, "quick_gelu": 3, "relu": 4, "relu2": 5, "relu6": 6, "silu": 7, "swish": 7,
-             "sigmoid": 8, "tanh": 9, "leaky_relu": 10, "mish": 11, "gelu_10": 12}
-ABI_VERSION = 1
+             "sigmoid": 8, "tanh": 9, "leaky_relu": 10, "mish": 11, "gelu_10": 12, "laplace": 13}
+ABI_VERSION = 2
 
 _lib = None
 _lock = threading.Lock()
@@ -174,24 +174,52 @@ def epilogue_(y: torch.Tensor, bias=None, act=None, add1=None, add2=None) -> tor
     return y
 
 
+def _freq_ld(inv_freq, d: int, n_seqs: Optional[int] = None) -> int:
+    """0 for one frequency table [d/2] for all tokens; for a table per sequence of the step, [sequences, d/2],
+    the distance between its rows."""
+    if inv_freq is None:
+        return 0
+    _need(inv_freq, "inv_freq", torch.float32)
+    if inv_freq.dim() == 1 and inv_freq.shape[0] == d // 2:
+        return 0
+    if inv_freq.dim() == 2 and inv_freq.shape[1] == d // 2 and (n_seqs is None or inv_freq.shape[0] == n_seqs):
+        return d // 2
+    raise KernelError(f"inv_freq must be [{d // 2}] or [sequences, {d // 2}], got {tuple(inv_freq.shape)}")
+
+
+def rope_dynamic_table(seq_start: torch.Tensor, cu_tokens: torch.Tensor, d: int, theta: float, factor: float,
+                       max_pos: int) -> torch.Tensor:
+    """A frequency table per sequence of the step, [sequences, d/2], for frequencies that follow the sequence's
+    length after the step: the trained ones up to ``max_pos`` tokens, beyond that those of a base stretched by
+    ``(factor * length / max_pos - (factor - 1)) ** (d / (d - 2))``."""
+    n = seq_start.numel()
+    _need(seq_start, "seq_start", torch.int32, (n,))
+    _need(cu_tokens, "cu_tokens", torch.int32, (n + 1,))
+    out = torch.empty((n, d // 2), dtype=torch.float32, device=seq_start.device)
+    _call("pta_rope_dynamic_table", _ptr(out), _ptr(seq_start), _ptr(cu_tokens), n, int(d), ctypes.c_float(theta),
+          ctypes.c_float(factor), int(max_pos), _stream())
+    return out
+
+
 def qkv_rope_cache(fused: torch.Tensor, bias, inv_freq, cs_scale: float, token_pos, token_seq, block_table,
                    k_pool, v_pool, nh: int, nkv: int, d: int, layout: str, write_cache: bool = True) -> torch.Tensor:
-    """Queries [M, nh, d] from the fused rows (which may lie apart); keys and values go to the cache pages."""
+    """Queries [M, nh, d] from the fused rows (which may lie apart); keys and values go to the cache pages.
+    ``inv_freq`` is one table [d/2], or one per sequence of the step, [sequences, d/2]."""
     M = fused.shape[0]
     _need_rows(fused, "fused", None, (M, (nh + 2 * nkv) * d))
     dt = fused.dtype
     if bias is not None:
         _need(bias, "bias", torch.float32, ((nh + 2 * nkv) * d,))
-    if inv_freq is not None:
-        _need(inv_freq, "inv_freq", torch.float32, (d // 2,))
     _need(token_pos, "token_pos", torch.int32, (M,))
     _need(token_seq, "token_seq", torch.int32, (M,))
     _need(block_table, "block_table", torch.int32)
     if block_table.dim() != 2:
         raise KernelError("block_table must be [sequences, pages]")
+    freq_ld = _freq_ld(inv_freq, d, block_table.shape[0])
     _need_pools(k_pool, v_pool, dt, nkv, d)
     q = torch.empty((M, nh, d), dtype=dt, device=fused.device)
-    _call("pta_qkv_rope_cache", _ptr(q), _ptr(fused), int(fused.stride(0)), _ptr(bias), _ptr(inv_freq), ctypes.c_float(cs_scale),
+    _call("pta_qkv_rope_cache", _ptr(q), _ptr(fused), int(fused.stride(0)), _ptr(bias), _ptr(inv_freq), freq_ld,
+          ctypes.c_float(cs_scale),
           _ptr(token_pos), _ptr(token_seq), _ptr(block_table), block_table.shape[1], _ptr(k_pool), _ptr(v_pool), M,
           nh, nkv, d, QKV_LAYOUT_CODES[layout], int(write_cache), dtype_code(dt), _stream())
     return q
@@ -738,17 +766,16 @@ def gemm_skinny_pair_qkv(x1: torch.Tensor, w_qkv: torch.Tensor, bias_qkv, inv_fr
         _need(bias_qkv, "bias_qkv", torch.float32, (N1,))
     if bias2 is not None:
         _need(bias2, "bias2", torch.float32, (N2,))
-    if inv_freq is not None:
-        _need(inv_freq, "inv_freq", torch.float32, (d // 2,))
     _need(token_pos, "token_pos", torch.int32, (M,))
     _need(token_seq, "token_seq", torch.int32, (M,))
     _need(block_table, "block_table", torch.int32)
     if block_table.dim() != 2:
         raise KernelError("block_table must be [sequences, pages]")
+    freq_ld = _freq_ld(inv_freq, d, block_table.shape[0])
     _need_pools(k_pool, v_pool, torch.bfloat16, nkv, d)
     q = torch.empty((M, nh, d), dtype=torch.bfloat16, device=x1.device)
     y2 = torch.empty((M, N2), dtype=torch.bfloat16, device=x1.device)
-    _call("pta_gemm_skinny_pair_qkv_bf16", _ptr(q), _ptr(x1), _ptr(w_qkv), _ptr(bias_qkv), _ptr(inv_freq),
+    _call("pta_gemm_skinny_pair_qkv_bf16", _ptr(q), _ptr(x1), _ptr(w_qkv), _ptr(bias_qkv), _ptr(inv_freq), freq_ld,
           ctypes.c_float(cs_scale), _ptr(token_pos), _ptr(token_seq), _ptr(block_table), block_table.shape[1], _ptr(k_pool),
           _ptr(v_pool), nh, nkv, d, QKV_LAYOUT_CODES[layout], int(write_cache), _ptr(y2), _ptr(x2), _ptr(w2), _ptr(bias2),
           N2, ACT_CODES[act2], M, K, _stream())
@@ -963,13 +990,12 @@ def gemm_splitk_pair_qkv(x1: torch.Tensor, w_qkv: torch.Tensor, bias_qkv, inv_fr
         _need(bias_qkv, "bias_qkv", torch.float32, (N1,))
     if bias2 is not None:
         _need(bias2, "bias2", torch.float32, (N2,))
-    if inv_freq is not None:
-        _need(inv_freq, "inv_freq", torch.float32, (d // 2,))
     _need(token_pos, "token_pos", torch.int32, (M,))
     _need(token_seq, "token_seq", torch.int32, (M,))
     _need(block_table, "block_table", torch.int32)
     if block_table.dim() != 2:
         raise KernelError("block_table must be [sequences, pages]")
+    freq_ld = _freq_ld(inv_freq, d, block_table.shape[0])
     _need_pools(k_pool, v_pool, torch.bfloat16, nkv, d)
     tune_pair_parts(w_qkv, w2)
     p1, p2 = gemm_splitk_pair_parts(N1, K1, N2, K2)
@@ -978,7 +1004,7 @@ def gemm_splitk_pair_qkv(x1: torch.Tensor, w_qkv: torch.Tensor, bias_qkv, inv_fr
     q = torch.empty((M, nh, d), dtype=torch.bfloat16, device=x1.device)
     y2 = torch.empty((M, N2), dtype=torch.bfloat16, device=x1.device)
     _call("pta_gemm_splitk_pair_reduced_qkv_bf16", _ptr(q), _ptr(part1), _ptr(x1), _ptr(w_qkv), _ptr(bias_qkv), K1,
-          _ptr(inv_freq), ctypes.c_float(cs_scale), _ptr(token_pos), _ptr(token_seq), _ptr(block_table),
+          _ptr(inv_freq), freq_ld, ctypes.c_float(cs_scale), _ptr(token_pos), _ptr(token_seq), _ptr(block_table),
           block_table.shape[1], _ptr(k_pool), _ptr(v_pool), nh, nkv, d, QKV_LAYOUT_CODES[layout], int(write_cache),
           _ptr(y2), _ptr(part2), _ptr(x2), _ptr(w2), _ptr(bias2), N2, K2, ACT_CODES[act2], M, _stream())
     return q, y2
@@ -999,18 +1025,17 @@ def gemm_splitk_qkv(x: torch.Tensor, w_qkv: torch.Tensor, bias_qkv, inv_freq, cs
         raise KernelError(f"head size {d} must be even")
     if bias_qkv is not None:
         _need(bias_qkv, "bias_qkv", torch.float32, (N,))
-    if inv_freq is not None:
-        _need(inv_freq, "inv_freq", torch.float32, (d // 2,))
     _need(token_pos, "token_pos", torch.int32, (M,))
     _need(token_seq, "token_seq", torch.int32, (M,))
     _need(block_table, "block_table", torch.int32)
     if block_table.dim() != 2:
         raise KernelError("block_table must be [sequences, pages]")
+    freq_ld = _freq_ld(inv_freq, d, block_table.shape[0])
     _need_pools(k_pool, v_pool, torch.bfloat16, nkv, d)
     part = torch.empty((int(load_library().pta_gemm_splitk_parts(N, K, 0, 0)), M, N), dtype=torch.float32, device=x.device)
     q = torch.empty((M, nh, d), dtype=torch.bfloat16, device=x.device)
     _call("pta_gemm_splitk_reduced_qkv_bf16", _ptr(q), _ptr(part), _ptr(x), _ptr(w_qkv), _ptr(bias_qkv), K,
-          _ptr(inv_freq), ctypes.c_float(cs_scale), _ptr(token_pos), _ptr(token_seq), _ptr(block_table),
+          _ptr(inv_freq), freq_ld, ctypes.c_float(cs_scale), _ptr(token_pos), _ptr(token_seq), _ptr(block_table),
           block_table.shape[1], _ptr(k_pool), _ptr(v_pool), nh, nkv, d, QKV_LAYOUT_CODES[layout], int(write_cache), M,
           _stream())
     return q

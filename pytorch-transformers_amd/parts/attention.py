@@ -56,7 +56,9 @@ class AttentionMixer(Part):
         """What ``forward`` does with the first product's rows; a block that runs that product in a launch of its
         own may hand this to the launch (``Linear.pair``)."""
         k_pool, v_pool = ctx.cache.kv_layer(call.cache_group, call.cache_layer)
-        inv_freq, cs_scale = self.positions.rotation()
+        # a position encoding whose rotation depends on the step (frequencies per sequence) offers rotation_for
+        inv_freq, cs_scale = (self.positions.rotation_for(ctx) if hasattr(self.positions, "rotation_for")
+                              else self.positions.rotation())
         return QkvTail(self.qkv.bias, inv_freq, cs_scale, ctx.token_pos, ctx.token_seq, ctx.block_tables[call.cache_group],
                        k_pool, v_pool, self.num_heads, self.kv_heads, self.head_dim, self.qkv_layout, call.write_cache)
 

@@ -20,7 +20,9 @@ norm           ``forward(x, rows=None) -> [tokens, hidden]`` (``rows``: int32
                indices of the rows to take); ``forward_pair(x, other)`` may fuse
                two norms of the same input
 positions      ``rotation() -> (inv_freq or None, scale)`` for queries and keys,
-               ``score_bias() -> per-head slopes or None`` for attention scores
+               ``score_bias() -> per-head slopes or None`` for attention scores;
+               optionally ``rotation_for(ctx) -> (table, scale)`` where the table may
+               have a row per sequence of the step (frequencies that follow a length)
 block          ``forward(x, ctx, call) -> x``: the arrangement of the above
 =============  ==================================================================
 

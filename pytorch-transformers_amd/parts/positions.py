@@ -30,16 +30,34 @@ class RotaryPositions(NoPositions):
     """
 
     def __init__(self, head_dim: int, theta: float, scaling_factor: float = 1.0, attention_scaling: float = 1.0,
-                 inv_freq: Optional[torch.Tensor] = None):
+                 inv_freq: Optional[torch.Tensor] = None, dynamic_factor: Optional[float] = None,
+                 trained_positions: Optional[int] = None):
         """``inv_freq`` given: a table of ``head_dim / 2`` frequencies of another scheme (``yarn_frequencies``,
-        ``llama3_frequencies``); cosines and sines are multiplied by ``attention_scaling``
-        (src/transformers/models/falcon/modeling_falcon.py:162-166)."""
+        ``llama3_frequencies``, ``longrope_frequencies``); cosines and sines are multiplied by
+        ``attention_scaling`` (src/transformers/models/falcon/modeling_falcon.py:162-166).
+
+        ``dynamic_factor`` with ``trained_positions``: dynamic NTK scaling
+        (src/transformers/modeling_rope_utils.py:112-160).  The frequencies of a sequence follow its own length:
+        up to ``trained_positions`` tokens they are the trained ones, beyond that those of the base
+        ``theta * (factor * length / trained - (factor - 1)) ** (d / (d - 2))``, taken anew in every step from
+        the length the sequence has after it.  Keys already in the cache keep the rotation of the step that
+        wrote them, as they do in the reference (:136-156 there rotates only what a forward pass is given).
+        The reference takes one length for a whole padded batch, the longest, and keeps the largest it has seen
+        until a call shorter than the trained context resets it (modeling_falcon.py:136-153); here each
+        sequence has its own, so that its logits do not depend on what else is in the batch: a sequence alone
+        gets what the reference gives a batch of one."""
         if head_dim % 2:
             raise ValueError(f"rotary positions need an even head size, got {head_dim}")
         self.head_dim = head_dim
         self.theta = float(theta)
         self.scaling_factor = float(scaling_factor)
         self.attention_scaling = float(attention_scaling)
+        self.dynamic_factor = None if dynamic_factor is None else float(dynamic_factor)
+        self.trained_positions = None if trained_positions is None else int(trained_positions)
+        if self.dynamic_factor is not None:
+            if self.trained_positions is None or self.trained_positions <= 0 or self.dynamic_factor < 1.0 or head_dim <= 2:
+                raise ValueError("dynamic frequencies need a factor >= 1, the trained context length and a head size "
+                                 f"above 2 (factor {dynamic_factor}, context {trained_positions}, head size {head_dim})")
         if inv_freq is not None:
             if tuple(inv_freq.shape) != (head_dim // 2,):
                 raise ValueError(f"a frequency table for head size {head_dim} has {head_dim // 2} entries, got "
@@ -56,6 +74,21 @@ class RotaryPositions(NoPositions):
 
     def rotation(self):
         return self.inv_freq, self.attention_scaling
+
+    def rotation_for(self, ctx):
+        """The frequencies for one step: the table, or with dynamic scaling one table per sequence of the step,
+        ``[sequences, head_dim / 2]``, made once per step on the device from the step's own arrays (so a captured
+        step makes it anew at every replay)."""
+        if self.dynamic_factor is None:
+            return self.rotation()
+        from .. import ops
+
+        key = ("rotary frequencies", id(self))
+        table = ctx.extras.get(key)
+        if table is None:
+            table = ctx.extras[key] = ops.rope_dynamic_table(ctx.seq_start, ctx.cu_tokens, self.head_dim, self.theta,
+                                                             self.dynamic_factor, self.trained_positions)
+        return table, self.attention_scaling
 
 
 def default_frequencies(head_dim: int, theta: float) -> torch.Tensor:
@@ -99,6 +132,32 @@ def llama3_frequencies(head_dim: int, theta: float, factor: float, low_freq_fact
     blended = (1 - smooth) * out / factor + smooth * out
     middle = ~(wavelen < short_to) & ~(wavelen > long_from)
     return torch.where(middle, blended, out)
+
+
+def longrope_frequencies(head_dim: int, theta: float, short_factor, factor: Optional[float],
+                         max_position_embeddings: int, original_max_position_embeddings: Optional[int] = None,
+                         attention_factor: Optional[float] = None):
+    """LongRoPE as the reference's Falcon runs it (src/transformers/modeling_rope_utils.py:242-302 called from
+    modeling_falcon.py:128, once, without a length): every trained frequency divided by its entry of
+    ``short_factor``; the table for long sequences (``long_factor``) is only ever taken by rotary modules that update
+    "dynamic" types (modeling_falcon.py:155-157 asks for that word in the type's name), so it is never used.
+    Returns (table, factor on cosines and sines): ``sqrt(1 + ln(factor) / ln(trained context))`` for a factor
+    above 1 unless ``attention_factor`` is given; with ``original_max_position_embeddings`` the factor is the
+    ratio of the two context lengths (:283-290)."""
+    short = torch.as_tensor([float(v) for v in short_factor], dtype=torch.float32)
+    if tuple(short.shape) != (head_dim // 2,):
+        raise ValueError(f"short_factor needs {head_dim // 2} entries, got {tuple(short.shape)}")
+    if original_max_position_embeddings:
+        trained = int(original_max_position_embeddings)
+        factor = max_position_embeddings / trained
+    else:
+        trained = int(max_position_embeddings)
+    if attention_factor is None:
+        if factor is None:
+            raise ValueError("longrope needs a factor, an attention_factor or original_max_position_embeddings")
+        attention_factor = 1.0 if factor <= 1.0 else math.sqrt(1 + math.log(factor) / math.log(trained))
+    inv = 1.0 / (short * float(theta) ** (torch.arange(0, head_dim, 2, dtype=torch.int64).float() / head_dim))
+    return inv, float(attention_factor)
 
 
 def alibi_slopes(num_heads: int) -> torch.Tensor:

@@ -113,6 +113,25 @@ def plain_logits(folder: str, reqs: Dict[str, List[int]]) -> Dict[str, torch.Ten
     return {rid: plain.forward(cfg, w, toks).float() for rid, toks in reqs.items()}
 
 
+def lengths_reached(reqs: Dict[str, List[int]], records: List[dict]) -> Dict[str, List[int]]:
+    """For every token of every request, the length its request had after the step that brought the token: what
+    frequencies that follow a sequence's length look at."""
+    out: Dict[str, List[int]] = {rid: [] for rid in reqs}
+    for rec in records:
+        for e in rec["entries"]:
+            n = len(out[e["id"]]) + len(e["tokens"])
+            out[e["id"]].extend([n] * len(e["tokens"]))
+    assert all(len(out[rid]) == len(reqs[rid]) for rid in reqs)
+    return out
+
+
+def plain_logits_as_fed(folder: str, reqs: Dict[str, List[int]], records: List[dict]) -> Dict[str, torch.Tensor]:
+    """The plain logits for a configuration whose result depends on the pieces a sequence was fed in."""
+    cfg, w = plain.read_model(folder)
+    lens = lengths_reached(reqs, records)
+    return {rid: plain.forward(cfg, w, toks, seq_lens=lens[rid]).float() for rid, toks in reqs.items()}
+
+
 def assert_close(got: torch.Tensor, want: torch.Tensor, rel: float, what: str) -> float:
     """max |got - want| <= rel * max |want|; returns the measured ratio."""
     assert got.shape == want.shape, f"{what}: shape {tuple(got.shape)} vs {tuple(want.shape)}"

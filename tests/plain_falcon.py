@@ -83,14 +83,40 @@ def rope_inv_freq(head_dim: int, theta: float, factor: float = 1.0):
     return inv / factor if factor != 1.0 else inv
 
 
-def rope_parameters(c):
+def rope_dynamic_inv_freq(head_dim: int, theta: float, factor: float, max_pos: int, seq_len: int):
+    """Dynamic NTK (src/transformers/modeling_rope_utils.py:149-158): up to the trained context the trained
+    frequencies, beyond it those of a stretched base; 32-bit arithmetic as there (the length arrives as an integer
+    tensor, src/transformers/models/falcon/modeling_falcon.py:142)."""
+    seq_len = seq_len if seq_len > max_pos else max_pos  # :152
+    n = torch.tensor(seq_len, dtype=torch.int64)
+    base = theta * ((factor * n / max_pos) - (factor - 1)) ** (head_dim / (head_dim - 2))  # :155
+    return 1.0 / (base ** (torch.arange(0, head_dim, 2, dtype=torch.int64).float() / head_dim))  # :156
+
+
+def rope_parameters(c, seq_len: Optional[int] = None):
     """(inv_freq, factor on cos and sin) for a configuration's ``rope_scaling``
-    (src/transformers/modeling_rope_utils.py: default :58-68, linear :108, yarn :163-239, llama3 :310-341)."""
+    (src/transformers/modeling_rope_utils.py: default :58-68, linear :108, dynamic :112-160, yarn :163-239,
+    longrope :242-302, llama3 :310-341).  ``seq_len`` matters to ``dynamic`` alone: Falcon's rotary module hands
+    the length to the types whose name holds "dynamic" and to no other
+    (src/transformers/models/falcon/modeling_falcon.py:155-157), so ``longrope`` always takes its short factors."""
     d = c["hidden_size"] // c["num_attention_heads"]
     theta = float(c["rope_theta"])
     rs = c.get("rope_scaling") or {}
     kind = rs.get("rope_type", rs.get("type", "default"))
     base = rope_inv_freq(d, theta)
+    if kind == "dynamic":
+        return rope_dynamic_inv_freq(d, theta, float(rs["factor"]), c["max_position_embeddings"], seq_len or 0), 1.0
+    if kind == "longrope":  # :276-300 with seq_len None
+        factor, scale = rs.get("factor"), rs.get("attention_factor")
+        trained = c["max_position_embeddings"]
+        if c.get("original_max_position_embeddings"):  # :283-287
+            trained = c["original_max_position_embeddings"]
+            factor = c["max_position_embeddings"] / trained
+        if scale is None:  # :290-294
+            scale = 1.0 if factor <= 1.0 else math.sqrt(1 + math.log(factor) / math.log(trained))
+        ext = torch.tensor(rs["short_factor"], dtype=torch.float32)
+        shape = torch.arange(0, d, 2, dtype=torch.int64).float() / d
+        return 1.0 / (ext * theta ** shape), float(scale)
     if kind == "linear":
         return base / float(rs["factor"]), 1.0
     if kind == "yarn":
@@ -200,8 +226,11 @@ def attention_scores_softmax(q, k, v, bias=None):
     return out.reshape(T, nh * d)
 
 
-def self_attention(x, w, prefix, c, positions):
-    """FalconAttention.forward (src/transformers/models/falcon/modeling_falcon.py:326-458)."""
+def self_attention(x, w, prefix, c, positions, seq_lens=None):
+    """FalconAttention.forward (src/transformers/models/falcon/modeling_falcon.py:326-458).  ``seq_lens``: for
+    every token the length its sequence had after the forward pass that brought the token (default: the whole
+    sequence at once); only frequencies that follow the length (``dynamic``) look at it, and what they rotated
+    stays as it was rotated then, like a key in the reference's cache."""
     nh = c["num_attention_heads"]
     d = c["hidden_size"] // nh
     fused = linear(x, w[prefix + "query_key_value.weight"], w.get(prefix + "query_key_value.bias"))
@@ -209,10 +238,17 @@ def self_attention(x, w, prefix, c, positions):
     bias = None
     if c["alibi"]:
         bias = alibi_bias(nh, x.shape[0], d, x.dtype)
-    else:
-        inv_freq, scale = rope_parameters(c)
+    elif seq_lens is None or (c.get("rope_scaling") or {}).get("rope_type", (c.get("rope_scaling") or {}).get("type")) != "dynamic":
+        inv_freq, scale = rope_parameters(c, x.shape[0])
         cos, sin = rope_cos_sin(positions, inv_freq, x.dtype, scale)
         q, k = apply_rope(q, cos, sin), apply_rope(k, cos, sin)
+    else:
+        q, k = q.clone(), k.clone()
+        for n in sorted(set(int(v) for v in seq_lens)):  # the tokens of one forward pass share its table
+            rows = torch.tensor([t for t, v in enumerate(seq_lens) if int(v) == n])
+            inv_freq, scale = rope_parameters(c, n)
+            cos, sin = rope_cos_sin(positions[rows], inv_freq, x.dtype, scale)
+            q[rows], k[rows] = apply_rope(q[rows], cos, sin), apply_rope(k[rows], cos, sin)
     o = attention_scores_softmax(q, k, v, bias)
     return linear(o, w[prefix + "dense.weight"], w.get(prefix + "dense.bias"))
 
@@ -245,7 +281,7 @@ def mlp(x, w, prefix, act="gelu"):
     return linear(activation(u, act), w[prefix + "dense_4h_to_h.weight"], w.get(prefix + "dense_4h_to_h.bias"))
 
 
-def decoder_layer(x, w, i, c, positions):
+def decoder_layer(x, w, i, c, positions, seq_lens=None):
     """FalconDecoderLayer.forward (src/transformers/models/falcon/modeling_falcon.py:614-683)."""
     p = f"transformer.h.{i}."
     eps = c["layer_norm_epsilon"]
@@ -256,7 +292,7 @@ def decoder_layer(x, w, i, c, positions):
     else:  # :634
         attn_in = layer_norm(x, w[p + "input_layernorm.weight"], w[p + "input_layernorm.bias"], eps)
         mlp_in = None
-    attn = self_attention(attn_in, w, p + "self_attention.", c, positions)
+    attn = self_attention(attn_in, w, p + "self_attention.", c, positions, seq_lens)
     if not c["new_decoder_architecture"]:
         if c["parallel_attn"]:  # :649-650
             mlp_in = attn_in
@@ -272,14 +308,15 @@ def decoder_layer(x, w, i, c, positions):
     return residual + out  # :676
 
 
-def forward(cfg: dict, w: Dict[str, torch.Tensor], token_ids: Sequence[int]):
-    """Logits [T, V] of one whole sequence (FalconModel.forward :864-1011, head :1230)."""
+def forward(cfg: dict, w: Dict[str, torch.Tensor], token_ids: Sequence[int], seq_lens: Optional[Sequence[int]] = None):
+    """Logits [T, V] of one whole sequence (FalconModel.forward :864-1011, head :1230).  ``seq_lens``: see
+    ``self_attention``; it says in which pieces the sequence was fed, for configurations that ask."""
     c = cfg_defaults(cfg)
     ids = torch.as_tensor(list(token_ids), dtype=torch.long)
     x = w["transformer.word_embeddings.weight"][ids]  # :895-896
     positions = torch.arange(len(ids))
     for i in range(c["num_hidden_layers"]):
-        x = decoder_layer(x, w, i, c, positions)
+        x = decoder_layer(x, w, i, c, positions, seq_lens)
     x = layer_norm(x, w["transformer.ln_f.weight"], w["transformer.ln_f.bias"], c["layer_norm_epsilon"])  # :992
     head = w["lm_head.weight"] if "lm_head.weight" in w else w["transformer.word_embeddings.weight"]  # tied :1163
     return x @ head.T

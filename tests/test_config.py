@@ -56,11 +56,16 @@ def test_unknown_keys_are_kept_and_round_trip(tmp_path):
     (dict(new_decoder_architecture=False, parallel_attn=True, num_ln_in_parallel_attn=2), "num_ln_in_parallel_attn"),
     (dict(new_decoder_architecture=False, multi_query=False, num_kv_heads=2, num_attention_heads=8, hidden_size=64), "multi_query=false"),
     (dict(new_decoder_architecture=True, num_attention_heads=8, num_kv_heads=3, hidden_size=64), "multiple"),
-    (dict(activation="laplace"), "activation"),
     (dict(activation="gelu_typo"), "activation"),
     (dict(hidden_size=66, num_attention_heads=22), "even head size"),
-    (dict(rope_scaling={"rope_type": "dynamic", "factor": 2.0}), "not built"),
-    (dict(rope_scaling={"rope_type": "longrope", "factor": 2.0}), "not built"),
+    (dict(rope_scaling={"rope_type": "dynamic", "factor": 0.5}), "factor"),
+    (dict(rope_scaling={"rope_type": "dynamic"}), "factor"),
+    (dict(hidden_size=8, num_attention_heads=4, rope_scaling={"rope_type": "dynamic", "factor": 2.0}), "head size above 2"),
+    (dict(rope_scaling={"rope_type": "longrope", "factor": 2.0}), "short_factor"),
+    (dict(hidden_size=64, num_attention_heads=4,
+          rope_scaling={"rope_type": "longrope", "factor": 2.0, "short_factor": [1.0] * 8, "long_factor": [1.0] * 7}), "long_factor"),
+    (dict(hidden_size=64, num_attention_heads=4,
+          rope_scaling={"rope_type": "longrope", "short_factor": [1.0] * 8, "long_factor": [1.0] * 8}), "factor"),
     (dict(rope_scaling={"rope_type": "yarn", "factor": 0.5}), "factor"),
     (dict(rope_scaling={"rope_type": "yarn", "factor": 2.0, "beta_fast": 1.0, "beta_slow": 4.0}), "beta_fast"),
     (dict(rope_scaling={"rope_type": "llama3", "factor": 8.0}), "low_freq_factor"),
@@ -75,6 +80,19 @@ def test_unknown_keys_are_kept_and_round_trip(tmp_path):
 def test_invalid_combinations_are_rejected(bad, match):
     with pytest.raises(ConfigError, match=match):
         FalconConfig(**bad)
+
+
+def test_every_rope_type_and_activation_of_the_reference_is_built():
+    """modeling_rope_utils.py:351-358 and activations.py:200-220: nothing that a Falcon config.json may name is refused."""
+    from pytorch_transformers_amd.config.falcon import ACTIVATIONS_BUILT, ROPE_TYPES_BUILT
+
+    assert set(ROPE_TYPES_BUILT) == {"default", "linear", "dynamic", "yarn", "longrope", "llama3"}
+    assert len(ACTIVATIONS_BUILT) == 19 and "laplace" in ACTIVATIONS_BUILT
+    FalconConfig(rope_scaling={"rope_type": "dynamic", "factor": 2.0})
+    FalconConfig(hidden_size=64, num_attention_heads=4,
+                 rope_scaling={"rope_type": "longrope", "short_factor": [1.0] * 8, "long_factor": [2.0] * 8, "attention_factor": 1.1})
+    AutoConfig.from_dict(dict(model_type="falcon", hidden_size=64, num_attention_heads=4, original_max_position_embeddings=512,
+                              rope_scaling={"rope_type": "longrope", "short_factor": [1.0] * 8, "long_factor": [2.0] * 8}))
 
 
 def test_odd_head_size_is_fine_with_alibi():

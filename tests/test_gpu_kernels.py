@@ -374,10 +374,42 @@ def _gather(pool, pages, L, transposed=False):
     return x.permute(0, 2, 1, 3).reshape(-1, x.shape[1], x.shape[3])[:L]
 
 
+def _freq(rotary, d, n_seqs, theta=10000.0, factor=1.0):
+    """None, one frequency table, or (rotary == "per sequence") a table per sequence, all rows different."""
+    if not rotary:
+        return None
+    inv = P.rope_inv_freq(d, theta, factor)
+    if rotary == "per sequence":
+        inv = torch.stack([inv / (1.0 + 0.37 * s) for s in range(n_seqs)])
+    return inv.cuda()
+
+
+def test_rope_dynamic_table():
+    """A frequency table per sequence from the lengths after the step, against the plain formula
+    (src/transformers/modeling_rope_utils.py:149-158): trained frequencies up to the trained context, stretched
+    beyond it, each sequence by its own length."""
+    ops = _ops()
+    starts, news = [0, 40, 47, 48, 300, 5000], [48, 9, 1, 1, 7, 1]
+    seq_start = torch.tensor(starts, dtype=torch.int32).cuda()
+    cu = torch.tensor([0] + list(torch.tensor(news).cumsum(0)), dtype=torch.int32).cuda()
+    for d, theta, factor, ctx in ((32, 10000.0, 4.0, 48), (128, 500042.0, 10.0, 48), (6, 10000.0, 2.0, 100)):
+        got = ops.rope_dynamic_table(seq_start, cu, d, theta, factor, ctx).cpu()
+        assert got.shape == (len(starts), d // 2)
+        for i, (s, n) in enumerate(zip(starts, news)):
+            want = P.rope_dynamic_inv_freq(d, theta, factor, ctx, s + n)
+            # the kernel rounds the double-precision value once; the plain formula is the reference's chain of
+            # 32-bit operations, each of which may be a unit or two in the last place off (2^-23 = 1.2e-7)
+            torch.testing.assert_close(got[i], want, rtol=2e-6, atol=0)
+            if s + n <= ctx:
+                torch.testing.assert_close(got[i], P.rope_inv_freq(d, theta), rtol=5e-7, atol=0)
+    with pytest.raises(ops.KernelError):
+        ops.rope_dynamic_table(seq_start, cu, 2, 10000.0, 2.0, 48)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("layout,nh,nkv,d", [("grouped", 6, 2, 32), ("tail", 7, 1, 64), ("interleaved", 5, 5, 24),
                                              ("grouped", 8, 8, 16), ("grouped", 4, 1, 128)])
-@pytest.mark.parametrize("rotary", [True, False])
+@pytest.mark.parametrize("rotary", [True, False, "per sequence"])
 def test_qkv_rope_cache(dtype, layout, nh, nkv, d, rotary):
     """Against the plain split and rotation; keys and values land at (page, position) of their sequence."""
     ops = _ops()
@@ -389,7 +421,7 @@ def test_qkv_rope_cache(dtype, layout, nh, nkv, d, rotary):
     bias = _rand((nh + 2 * nkv) * d, seed=9)
     token_seq = torch.tensor([i for i, n in enumerate(news) for _ in range(n)], dtype=torch.int32).cuda()
     token_pos = torch.tensor([s + j for s, n in zip(starts, news) for j in range(n)], dtype=torch.int32).cuda()
-    inv = P.rope_inv_freq(d, 500042.0, 2.0).cuda() if rotary else None
+    inv = _freq(rotary, d, 3, 500042.0, 2.0)
     q = ops.qkv_rope_cache(fused, bias, inv, 1.0, token_pos, token_seq, bt, k_pool, v_pool, nh, nkv, d, layout)
 
     c = dict(num_attention_heads=nh, hidden_size=nh * d, num_kv_heads=nkv,
@@ -397,7 +429,11 @@ def test_qkv_rope_cache(dtype, layout, nh, nkv, d, rotary):
     rnd = (lambda t: t) if dtype == torch.float32 else (lambda t: t.bfloat16().double())
     x = rnd(fused.double().cpu() + bias.double().cpu())
     wq, wk, wv = P.split_heads(x, c)
-    if rotary:
+    if rotary == "per sequence":  # every token by its own sequence's table
+        cs = [P.rope_cos_sin(token_pos.cpu()[t:t + 1], inv.cpu()[int(token_seq[t])]) for t in range(M)]
+        cos, sin = torch.cat([c for c, _ in cs]), torch.cat([s_ for _, s_ in cs])
+        wq, wk = P.apply_rope(wq, cos, sin), P.apply_rope(wk, cos, sin)
+    elif rotary:
         cos, sin = P.rope_cos_sin(token_pos.cpu(), inv.cpu())
         wq, wk = P.apply_rope(wq, cos, sin), P.apply_rope(wk, cos, sin)
     tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=1e-2, atol=1e-2)
@@ -417,7 +453,7 @@ def test_qkv_rope_cache(dtype, layout, nh, nkv, d, rotary):
 
 @pytest.mark.parametrize("layout,nh,nkv,d", [("grouped", 4, 2, 32), ("grouped", 8, 2, 128), ("tail", 7, 1, 64),
                                              ("interleaved", 3, 3, 96), ("tail", 71, 1, 64)])
-@pytest.mark.parametrize("rotary,bias", [(True, True), (False, False), (True, False)])
+@pytest.mark.parametrize("rotary,bias", [(True, True), (False, False), (True, False), ("per sequence", True)])
 def test_pair_launch_takes_the_fused_qkv_rows_to_their_end(layout, nh, nkv, d, rotary, bias):
     """The pair launch for few rows with the query_key_value tail in its epilogue against the same two products
     followed by the kernel that splits, rotates and writes the cache: the same queries, the same pages (bit for bit
@@ -436,7 +472,7 @@ def test_pair_launch_takes_the_fused_qkv_rows_to_their_end(layout, nh, nkv, d, r
     b1, b2 = (_rand(N1, seed=3) if bias else None), _rand(N2, seed=4)
     token_seq = torch.arange(M, dtype=torch.int32).cuda()
     token_pos = torch.tensor(starts, dtype=torch.int32).cuda()
-    inv = P.rope_inv_freq(d, 10000.0).cuda() if rotary else None
+    inv = _freq(rotary, d, M)
     assert ops.gemm_skinny_pair_qkv_ok(x, w1, w2, d)
     pools = []
     for fused_way in (False, True):
@@ -461,7 +497,7 @@ def test_pair_launch_takes_the_fused_qkv_rows_to_their_end(layout, nh, nkv, d, r
 
 @pytest.mark.parametrize("layout,nh,nkv,d,M", [("grouped", 4, 2, 24, 40), ("grouped", 8, 2, 128, 17), ("tail", 7, 1, 64, 150),
                                                ("interleaved", 3, 3, 96, 64)])
-@pytest.mark.parametrize("rotary,bias", [(True, True), (False, False)])
+@pytest.mark.parametrize("rotary,bias", [(True, True), (False, False), ("per sequence", False)])
 def test_batch_pair_launch_takes_the_fused_qkv_rows_to_their_end(layout, nh, nkv, d, M, rotary, bias):
     """The same for a decode batch of 17 to 256 rows, where the launch that adds the partial sums carries the
     tail: the queries and pages of the two products followed by the kernel of its own, bit for bit."""
@@ -476,7 +512,7 @@ def test_batch_pair_launch_takes_the_fused_qkv_rows_to_their_end(layout, nh, nkv
     b1, b2 = (_rand(N1, seed=3) if bias else None), _rand(N2, seed=4)
     token_seq = torch.arange(M, dtype=torch.int32).cuda()
     token_pos = torch.tensor(starts, dtype=torch.int32).cuda()
-    inv = P.rope_inv_freq(d, 10000.0).cuda() if rotary else None
+    inv = _freq(rotary, d, M)
     pools = []
     for fused_way in (False, True):
         k_pool, v_pool, bt, lists = _cache_setup(M, lens, nkv, d, torch.bfloat16, n_pages=3 * M + 8)
@@ -499,7 +535,7 @@ def test_batch_pair_launch_takes_the_fused_qkv_rows_to_their_end(layout, nh, nkv
 
 @pytest.mark.parametrize("layout,nh,nkv,d,M,K", [("grouped", 4, 2, 24, 40, 264), ("grouped", 8, 2, 128, 17, 2560),
                                                  ("tail", 7, 1, 64, 150, 1032), ("interleaved", 3, 3, 96, 256, 4104)])
-@pytest.mark.parametrize("rotary,bias", [(True, True), (False, False)])
+@pytest.mark.parametrize("rotary,bias", [(True, True), (False, False), ("per sequence", True)])
 def test_batch_launch_takes_the_fused_qkv_rows_to_their_end(layout, nh, nkv, d, M, K, rotary, bias):
     """A query_key_value projection on its own, 17 to 256 rows, one range of K and several: the launch that adds
     the partial sums carries the tail, and gives the queries and pages of the product followed by the kernel of
@@ -514,7 +550,7 @@ def test_batch_launch_takes_the_fused_qkv_rows_to_their_end(layout, nh, nkv, d, 
     b = _rand(N, seed=3) if bias else None
     token_seq = torch.arange(M, dtype=torch.int32).cuda()
     token_pos = torch.tensor(starts, dtype=torch.int32).cuda()
-    inv = P.rope_inv_freq(d, 10000.0).cuda() if rotary else None
+    inv = _freq(rotary, d, M)
     pools = []
     for fused_way in (False, True):
         k_pool, v_pool, bt, lists = _cache_setup(M, lens, nkv, d, torch.bfloat16, n_pages=3 * M + 8)

@@ -15,7 +15,7 @@ from tiny import TINY, write_model
 pytestmark = pytest.mark.gpu
 
 LENGTHS = {"A": [5, 11, 17, 40, 70, 33], "B": [1, 7, 20, 33, 65, 129], "C": [64, 3, 47, 90, 128, 66],
-           "D": [37, 12, 80, 5, 64, 100], "E": [9, 50, 130, 3, 64, 77]}
+           "D": [37, 12, 80, 5, 64, 100], "E": [9, 50, 130, 3, 64, 77], "F": [70, 2, 64, 31, 100, 65]}
 
 
 @pytest.fixture(scope="module")
@@ -70,6 +70,42 @@ def test_schedules_match_plain(folders, plain_cache, name, dtype, rel):
             for rid in reqs:
                 assert torch.equal(results[sched_name][rid], results["whole"][rid]), \
                     f"{name} float32: {sched_name} differs from whole for {rid}"
+
+
+@pytest.mark.parametrize("dtype,rel", [("float32", REL_F32), ("bfloat16", REL_BF16)])
+def test_frequencies_that_follow_each_sequences_length(tmp_path, dtype, rel):
+    """``rope_scaling: dynamic`` with a trained context of 48 positions: every piece of a sequence is rotated by the
+    frequencies of the length reached with it, each sequence by its own length whatever else the step holds, and
+    what is in the cache stays as it was rotated.  The plain logits are computed for the pieces of each schedule;
+    sequences that stay within the trained context equal the model without scaling."""
+    from pytorch_transformers_amd import AutoModelForCausalLM
+    from pytorch_transformers_amd.engine.replay import Replayer
+    from tiny import DYNAMIC, write_config
+
+    folder = write_config(DYNAMIC, str(tmp_path), "dyn", seed=6)
+    reqs = helpers.make_requests(DYNAMIC["vocab_size"], [30, 70, 100, 49, 48, 130], seed=21)
+    model = AutoModelForCausalLM.from_pretrained(folder, dtype=dtype)
+    rp = Replayer(model, 1024)
+    seen = {}
+    for sched_name, records in (("whole", helpers.schedule_whole(reqs)), ("tail32", helpers.schedule_tail(reqs, 32)),
+                                ("batches", helpers.schedule_batches(reqs, 4, decode=(3, 25, 1, 14))),
+                                ("staggered", helpers.schedule_staggered(reqs, 2, decode=(6, 2, 60, 4), chunks=(None, 40, 19, 1)))):
+        want = helpers.plain_logits_as_fed(folder, reqs, records)
+        got = helpers.run_schedule(rp, records)
+        for rid in reqs:
+            helpers.assert_close(got[rid], want[rid], rel, f"dynamic {dtype} {sched_name} {rid} (len {len(reqs[rid])})")
+        seen[sched_name] = got
+    if dtype == "float32":
+        # the schedules do differ where a sequence crossed the trained context in pieces ...
+        assert not torch.allclose(seen["tail32"]["r2"], seen["whole"]["r2"], atol=1e-4)
+        # ... and do not where it never left it: bitwise the same, and the unscaled model's logits
+        for rid in ("r0", "r4"):
+            for sched_name in ("tail32", "batches", "staggered"):
+                assert torch.equal(seen[sched_name][rid], seen["whole"][rid])
+        plain_folder = write_config(dict(DYNAMIC, rope_scaling=None), str(tmp_path), "plain", seed=6)
+        unscaled = helpers.plain_logits(plain_folder, {rid: reqs[rid] for rid in ("r0", "r4")})
+        for rid in ("r0", "r4"):
+            helpers.assert_close(seen["whole"][rid], unscaled[rid], rel, f"within the trained context, {rid}")
 
 
 @pytest.mark.parametrize("dtype,rel", [("float32", REL_F32), ("bfloat16", REL_BF16)])

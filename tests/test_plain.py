@@ -127,6 +127,82 @@ def test_yarn_and_llama3_frequencies_against_the_reference_snapshots():
     torch.testing.assert_close(inv[-20:], plain[-20:] / 10.0)
 
 
+DYNAMIC_SNAPSHOT = [  # tests/utils/test_modeling_rope_utils.py:184-199: d=128, theta=1e4, context 2048, factor 10, length 16384
+    1.0000e+00, 8.0931e-01, 6.5498e-01, 5.3008e-01, 4.2900e-01, 3.4720e-01, 2.8099e-01, 2.2741e-01, 1.8404e-01, 1.4895e-01,
+    1.2055e-01, 9.7558e-02, 7.8955e-02, 6.3899e-02, 5.1714e-02, 4.1853e-02, 3.3872e-02, 2.7413e-02, 2.2185e-02, 1.7955e-02,
+    1.4531e-02, 1.1760e-02, 9.5176e-03, 7.7027e-03, 6.2339e-03, 5.0451e-03, 4.0831e-03, 3.3045e-03, 2.6744e-03, 2.1644e-03,
+    1.7517e-03, 1.4176e-03, 1.1473e-03, 9.2852e-04, 7.5146e-04, 6.0817e-04, 4.9220e-04, 3.9834e-04, 3.2238e-04, 2.6091e-04,
+    2.1115e-04, 1.7089e-04, 1.3830e-04, 1.1193e-04, 9.0585e-05, 7.3312e-05, 5.9332e-05, 4.8018e-05, 3.8861e-05, 3.1451e-05,
+    2.5453e-05, 2.0600e-05, 1.6672e-05, 1.3492e-05, 1.0920e-05, 8.8374e-06, 7.1522e-06, 5.7883e-06, 4.6845e-06, 3.7912e-06,
+    3.0683e-06, 2.4832e-06, 2.0097e-06, 1.6265e-06]
+
+
+def test_dynamic_and_longrope_frequencies_against_the_references_tests():
+    """Dynamic NTK: the trained table up to the trained context whatever the factor, the reference's snapshot beyond
+    it, no plain division by the factor (tests/utils/test_modeling_rope_utils.py:201-225).  LongRoPE: the short
+    factors divide the trained table, and the factor on cosines and sines has the paper's default
+    (:300-365); fails for the long factors, a missing logarithm or the wrong context length in it."""
+    from pytorch_transformers_amd.parts.positions import longrope_frequencies
+
+    base = dict(hidden_size=4096, num_attention_heads=32, rope_theta=10000.0, max_position_embeddings=2048)
+    plain = P.rope_inv_freq(128, 10000.0)
+    for factor in (2.0, 10.0, 20.0):
+        c = dict(base, rope_scaling={"rope_type": "dynamic", "factor": factor})
+        for n in (None, 1, 2048):
+            inv, scale = P.rope_parameters(c, n)
+            assert scale == 1.0
+            torch.testing.assert_close(inv, plain)
+    inv, _ = P.rope_parameters(dict(base, rope_scaling={"rope_type": "dynamic", "factor": 10.0}), 16384)
+    torch.testing.assert_close(inv, torch.tensor(DYNAMIC_SNAPSHOT), rtol=2e-4, atol=0)
+    assert not torch.allclose(inv, plain / 10.0, rtol=1e-3)
+    assert bool((inv <= plain).all())  # tests/models/falcon/test_modeling_falcon.py:503
+    # cosines of a short range are the trained ones, of a long range not (:493-502 there)
+    c10 = dict(base, rope_scaling={"type": "dynamic", "factor": 10.0})
+    cs_short, _ = P.rope_cos_sin(torch.arange(10), P.rope_parameters(c10, 10)[0])
+    cs_plain, _ = P.rope_cos_sin(torch.arange(10), plain)
+    torch.testing.assert_close(cs_short, cs_plain)
+    cs_long, _ = P.rope_cos_sin(torch.arange(3072), P.rope_parameters(c10, 3072)[0])
+    assert not torch.allclose(cs_long, P.rope_cos_sin(torch.arange(3072), plain)[0], atol=1e-3)
+
+    short, long_ = [2.0] * 64, [float(i + 1) for i in range(64)]
+    for factor in (2.0, 10.0, 20.0):
+        rs = {"rope_type": "longrope", "factor": factor, "short_factor": short, "long_factor": long_}
+        inv, scale = P.rope_parameters(dict(base, rope_scaling=rs))
+        assert scale == math.sqrt(1 + math.log(factor) / math.log(2048))
+        torch.testing.assert_close(inv, plain / 2.0)
+        assert P.rope_parameters(dict(base, rope_scaling=dict(rs, attention_factor=0.5)))[1] == 0.5
+        got, got_scale = longrope_frequencies(128, 10000.0, short, factor, 2048)
+        torch.testing.assert_close(got, inv, rtol=1e-6, atol=0)
+        assert got_scale == scale and longrope_frequencies(128, 10000.0, short, factor, 2048, attention_factor=0.5)[1] == 0.5
+    rs = {"rope_type": "longrope", "factor": 1.0, "short_factor": short, "long_factor": long_}
+    assert P.rope_parameters(dict(base, rope_scaling=rs))[1] == 1.0
+    # a configuration that names the trained context takes the ratio of the two lengths as its factor
+    c = dict(base, max_position_embeddings=8192, original_max_position_embeddings=2048,
+             rope_scaling={"rope_type": "longrope", "short_factor": short, "long_factor": long_})
+    assert P.rope_parameters(c)[1] == math.sqrt(1 + math.log(4.0) / math.log(2048))
+    assert longrope_frequencies(128, 10000.0, short, None, 8192, 2048)[1] == P.rope_parameters(c)[1]
+
+
+def test_dynamic_frequencies_in_the_model(models_dynamic):
+    """Falcon's own test of scaling from the configuration (tests/models/falcon/test_modeling_falcon.py:424-455):
+    up to the trained context a model with dynamic scaling gives what it gives without, beyond it not; and fed in
+    pieces, every piece is rotated by the table of the length reached with it, earlier pieces staying as they were."""
+    cfg, w = models_dynamic
+    unscaled = dict(cfg, rope_scaling=None)
+    ctx = cfg["max_position_embeddings"]
+    short = [(5 * i + 1) % cfg["vocab_size"] for i in range(ctx)]
+    long_ = [(3 * i + 2) % cfg["vocab_size"] for i in range(ctx + ctx // 2)]
+    torch.testing.assert_close(P.forward(cfg, w, short), P.forward(unscaled, w, short))
+    whole = P.forward(cfg, w, long_)
+    assert not torch.allclose(whole, P.forward(unscaled, w, long_), atol=1e-5)
+    # the first `ctx` tokens as one piece, then one token at a time
+    lens = [ctx] * ctx + list(range(ctx + 1, len(long_) + 1))
+    pieces = P.forward(cfg, w, long_, seq_lens=lens)
+    torch.testing.assert_close(pieces[:ctx], P.forward(unscaled, w, long_[:ctx]))  # nothing was scaled yet
+    assert not torch.allclose(pieces[ctx:], whole[ctx:], atol=1e-5)  # the prompt's keys kept their rotation
+    torch.testing.assert_close(P.forward(cfg, w, long_, seq_lens=[len(long_)] * len(long_)), whole)
+
+
 def test_rope_hand_case_pairs_and_sign():
     """Pairs are (i, i + d/2), not (2i, 2i+1); the lower half gets -sin.  d=4, position 1."""
     x = torch.tensor([[[1.0, 2.0, 3.0, 4.0]]], dtype=D)
@@ -277,6 +353,13 @@ def test_attention_is_sdpa_and_groups_are_repeated_heads():
 def models(tmp_path_factory):
     root = str(tmp_path_factory.mktemp("plain"))
     return {n: P.read_model(write_model(n, root)) for n in TINY}
+
+
+@pytest.fixture(scope="module")
+def models_dynamic(tmp_path_factory):
+    from tiny import DYNAMIC, write_config
+
+    return P.read_model(write_config(DYNAMIC, str(tmp_path_factory.mktemp("plain-dyn")), "dyn", seed=6))
 
 
 @pytest.mark.parametrize("name", sorted(TINY))

@@ -33,7 +33,22 @@ TINY = {
               tie_word_embeddings=True, initializer_range=0.02),
 }
 
-SEEDS = {"A": 0, "B": 1, "C": 2, "D": 3, "E": 4}
+# frequencies that follow the sequence's length: a trained context of 48 positions, so that short tests cross it
+DYNAMIC = dict(model_type="falcon", num_hidden_layers=2, hidden_size=96, num_attention_heads=3, num_kv_heads=1,
+               ffn_hidden_size=136, vocab_size=211, rope_theta=10000.0, max_position_embeddings=48,
+               layer_norm_epsilon=1e-5, new_decoder_architecture=True, parallel_attn=True, num_ln_in_parallel_attn=1,
+               bias=False, alibi=False, tie_word_embeddings=True, initializer_range=0.02,
+               rope_scaling={"rope_type": "dynamic", "factor": 4.0})
+# LongRoPE: a factor per frequency, and a factor on cosines and sines
+LONGROPE = dict(model_type="falcon", num_hidden_layers=2, hidden_size=80, num_attention_heads=5,
+                ffn_hidden_size=96, vocab_size=97, rope_theta=500042.0, max_position_embeddings=64,
+                layer_norm_epsilon=1e-5, new_decoder_architecture=False, multi_query=True, parallel_attn=True,
+                bias=True, alibi=False, tie_word_embeddings=False, initializer_range=0.02,
+                rope_scaling={"rope_type": "longrope", "factor": 4.0, "short_factor": [1.0, 1.1, 1.3, 1.6, 2.0, 2.5, 3.1, 3.8],
+                              "long_factor": [1.0, 2.0, 3.0, 4.0, 5.0, 6.0, 7.0, 8.0]})
+
+TINY["F"] = LONGROPE
+SEEDS = {"A": 0, "B": 1, "C": 2, "D": 3, "E": 4, "F": 5}
 
 
 LIVELY_STD = 0.2
@@ -51,3 +66,11 @@ def write_model(name: str, folder: str, noise: float = 0.1, std=None) -> str:
     cfg = AutoConfig.from_dict(TINY[name])
     sub = name if std is None else f"{name}-std{std}"
     return write_random_model(os.path.join(folder, sub), cfg, SEEDS[name], noise=noise, std=std)
+
+
+def write_config(raw: dict, folder: str, name: str, seed: int, noise: float = 0.1, std=None) -> str:
+    """Write a model of the configuration ``raw`` (a dict as config.json holds it); returns the folder."""
+    from pytorch_transformers_amd.config import AutoConfig
+    from pytorch_transformers_amd.weights import write_random_model
+
+    return write_random_model(os.path.join(folder, name), AutoConfig.from_dict(raw), seed, noise=noise, std=std)
