@@ -26,18 +26,19 @@ __device__ __forceinline__ void load8f(const float* p, float (&f)[8]) {
     f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
 }
 
-// round(sum of the parts in order), then the bias added and rounded.  The parts are loaded four at a
-// time before they are added, so that their latencies overlap.
+// round(sum of the parts in order), then the bias added and rounded.  The parts are loaded eight at a
+// time before they are added, so that their latencies overlap (a row's workgroup runs on one compute unit,
+// and what it waits for is the number of round trips to memory, not the bytes).
 __device__ __forceinline__ void product_value(const float* part, int P, long part_stride, const float* bias, long at,
                                               int i, float (&out)[8]) {
     float bv[8];
     if (bias) load8f(bias + i, bv);
-    for (int p0 = 0; p0 < P; p0 += 4) {
-        float t[4][8];
+    for (int p0 = 0; p0 < P; p0 += 8) {
+        float t[8][8];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) load8f(part + (long)min(p0 + u, P - 1) * part_stride + at, t[u]);
+        for (int u = 0; u < 8; ++u) load8f(part + (long)min(p0 + u, P - 1) * part_stride + at, t[u]);
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < 8; ++u) {
             if (p0 + u >= P) continue;
 #pragma unroll
             for (int e = 0; e < 8; ++e) out[e] = (p0 + u == 0) ? t[u][e] : out[e] + t[u][e];

@@ -226,6 +226,10 @@ class CausalLM:
         self.generation_config = None
         #: run steps in which every sequence brings one token as replays of a captured HIP graph
         self.use_graphs = bool(spec.supports_graphs)
+        #: ``layer_hook(i, x)`` is called after entry ``i`` of the run order with the residual stream
+        #: ``[tokens, hidden]`` as a tensor (for dumps when a mismatch is being looked for); while it is set, steps
+        #: are launched directly, never replayed from a captured graph
+        self.layer_hook = None
 
     def _move_constants(self) -> None:
         seen = set()
@@ -343,11 +347,13 @@ class CausalLM:
         """Embedding, the layers in their run order, final norm and head on the wanted rows."""
         x = self.spec.embedding.forward(token_ids)
         blocks = self.spec.blocks
-        for call in self.spec.order:
+        for i, call in enumerate(self.spec.order):
             block = blocks[call.block]
             if isinstance(x, ResidualSum) and not getattr(block, "accepts_sum", False):
                 x = x.tensor()
             x = block.forward(x, ctx, call)
+            if self.layer_hook is not None:
+                self.layer_hook(i, as_tensor(x))  # a sum that is not formed yet is formed for the hook alone
         if logit_rows is None:
             return None
         norm = self.spec.final_norm
@@ -382,10 +388,11 @@ class CausalLM:
         of this step whose logits are asked for.  Rows come in the order of the sequences and of
         their places.
         """
-        if self.use_graphs and want == "last" and len(tokens) == len(slots) and all(len(t) == 1 for t in tokens):
+        graphs = self.use_graphs and self.layer_hook is None
+        if graphs and want == "last" and len(tokens) == len(slots) and all(len(t) == 1 for t in tokens):
             return self._decode_last(cache, slots, tokens)
         plan = plan_step(cache, slots, tokens, want, self.vocab_size)
-        if self.use_graphs and plan.is_decode:
+        if graphs and plan.is_decode:
             logits = self._graph_for(cache, plan).run(plan)
             cache.commit(plan.slots, plan.new_tokens)
             return logits

@@ -806,7 +806,7 @@ def gemm_splitk_bf16(x: torch.Tensor, w: torch.Tensor, bias=None, act=None, add1
     return out
 
 
-def gemm_splitk_partial(x: torch.Tensor, w: torch.Tensor, rt: int = 0, parts: int = 0) -> torch.Tensor:
+def gemm_splitk_partial(x: torch.Tensor, w: torch.Tensor, rt: int = 0, parts: int = 0, stage_blocks: int = 0) -> torch.Tensor:
     """x @ w.T left as 32-bit partial sums over ranges of K, [ranges, M, N]: for a kernel that adds them
     in order while it reads them (``layernorm_sum``)."""
     _need(x, "x", torch.bfloat16)
@@ -818,7 +818,7 @@ def gemm_splitk_partial(x: torch.Tensor, w: torch.Tensor, rt: int = 0, parts: in
     parts = int(load_library().pta_gemm_splitk_parts(N, K, int(parts), int(rt)))
     part = torch.empty((parts, M, N), dtype=torch.float32, device=x.device)
     _call("pta_gemm_splitk_bf16", None, _ptr(part), _ptr(x), _ptr(w), None, None, None, M, N, K, 0, 0, int(rt),
-          int(parts), 0, 0, 0, _stream())
+          int(parts), int(stage_blocks), 0, 0, _stream())
     return part
 
 

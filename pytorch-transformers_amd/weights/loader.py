@@ -134,9 +134,14 @@ def load_weights(folder: str, specs: Sequence[TensorSpec], compute_dtype: torch.
     files = resolve_files(folder)
     by_name = {s.name: s for s in specs}
     mapping = _strip_or_add_prefix(files.keys(), list(by_name), base_prefix)
+    # A tensor that is tied to another one is that other one, whatever the file holds under its name: the reference
+    # ties after it has loaded (src/transformers/modeling_utils.py:1858-1884 called from :4368), which overwrites a
+    # head that a file of a tied model carries.  The file's copy is neither read nor unexpected.
+    tied_in_file = {mapping.pop(s.name) for s in specs if s.tied_to is not None and s.name in mapping}
 
     used_file_names = set(mapping.values())
-    unexpected = sorted(k for k in files if k not in used_file_names and not k.endswith(_IGNORED_SUFFIXES))
+    unexpected = sorted(k for k in files if k not in used_file_names and k not in tied_in_file
+                        and not k.endswith(_IGNORED_SUFFIXES))
     missing = []
     for s in specs:
         if s.name in mapping:

@@ -308,15 +308,19 @@ def decoder_layer(x, w, i, c, positions, seq_lens=None):
     return residual + out  # :676
 
 
-def forward(cfg: dict, w: Dict[str, torch.Tensor], token_ids: Sequence[int], seq_lens: Optional[Sequence[int]] = None):
+def forward(cfg: dict, w: Dict[str, torch.Tensor], token_ids: Sequence[int], seq_lens: Optional[Sequence[int]] = None,
+            hidden: Optional[list] = None):
     """Logits [T, V] of one whole sequence (FalconModel.forward :864-1011, head :1230).  ``seq_lens``: see
-    ``self_attention``; it says in which pieces the sequence was fed, for configurations that ask."""
+    ``self_attention``; it says in which pieces the sequence was fed, for configurations that ask.  ``hidden``: a
+    list that receives the residual stream after every layer."""
     c = cfg_defaults(cfg)
     ids = torch.as_tensor(list(token_ids), dtype=torch.long)
     x = w["transformer.word_embeddings.weight"][ids]  # :895-896
     positions = torch.arange(len(ids))
     for i in range(c["num_hidden_layers"]):
         x = decoder_layer(x, w, i, c, positions, seq_lens)
+        if hidden is not None:
+            hidden.append(x)
     x = layer_norm(x, w["transformer.ln_f.weight"], w["transformer.ln_f.bias"], c["layer_norm_epsilon"])  # :992
     head = w["lm_head.weight"] if "lm_head.weight" in w else w["transformer.word_embeddings.weight"]  # tied :1163
     return x @ head.T

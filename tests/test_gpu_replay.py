@@ -190,13 +190,14 @@ def test_cache_full_is_an_error(folders):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_trace_run_program(folders, tmp_path, dtype):
-    """bin/trace_run as a program: stdin records, files of logits, 'done' lines."""
+    """bin/trace_run as a program: stdin records, files of logits, 'done' lines; with --dump-layers also the
+    residual stream after every layer, which equals the plain implementation's."""
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     reqs = helpers.make_requests(TINY["A"]["vocab_size"], [19, 40], seed=5)
     records = helpers.schedule_batches(reqs, 2, decode=(4, 9))
     out = tmp_path / "out"
     p = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folders["A"], "--dtype", dtype,
-                        "--out", str(out), "--max-tokens", "128"],
+                        "--out", str(out), "--max-tokens", "128", "--dump-layers", "--check-finite"],
                        input="".join(json.dumps(r) + "\n" for r in records), capture_output=True, text=True, timeout=300)
     assert p.returncode == 0, p.stderr[-2000:]
     assert p.stdout.split("\n")[:-1] == [f"done {r['step']}" for r in records]
@@ -213,6 +214,18 @@ def test_trace_run_program(folders, tmp_path, dtype):
                 row += 1
             fed[e["id"]] += len(e["tokens"])
         assert row == arr.shape[0]
+    # the dumps of the first step (both prompts, laid end to end) against the plain residual streams
+    cfg, w = helpers.plain.read_model(folders["A"])
+    H, rel = TINY["A"]["hidden_size"], (REL_F32 if dtype == "float32" else REL_BF16)
+    first = records[0]
+    hidden = {}
+    for e in first["entries"]:
+        hidden[e["id"]] = []
+        helpers.plain.forward(cfg, w, e["tokens"], hidden=hidden[e["id"]])
+    for layer in range(TINY["A"]["num_hidden_layers"]):
+        got = torch.from_numpy(np.fromfile(out / f"{first['step']}.layer{layer}.f32", dtype="<f4").reshape(-1, H))
+        want_rows = torch.cat([hidden[e["id"]][layer] for e in first["entries"]]).float()
+        helpers.assert_close(got, want_rows, rel, f"trace_run layer {layer} dump")
 
 
 def test_two_processes_write_the_same_bfloat16_bits(folders, tmp_path):

@@ -155,3 +155,18 @@ def test_first_float_dtype_reads_the_headers(tmp_path):
         save_file({"a.ids": torch.zeros(3, dtype=torch.int32), "b.weight": torch.zeros(2, 2, dtype=dt)},
                   str(folder / "model.safetensors"), metadata={"format": "pt"})
         assert first_float_dtype(str(folder)) == dt
+
+
+def test_a_tied_head_in_the_file_is_not_read(tmp_path):
+    """tie_word_embeddings=true: the head is the embedding table even if the file carries another tensor under the
+    head's name (the reference ties after loading, src/transformers/modeling_utils.py:1858-1884); untied, the file's
+    head is the head."""
+    cfg, specs = _specs("A")
+    f = write_random_model(str(tmp_path / "tied"), cfg, seed=3)
+    _rewrite(f, lambda t: t.__setitem__("lm_head.weight", torch.full_like(t["transformer.word_embeddings.weight"], 7.0)))
+    w = load_weights(f, specs, torch.float32, "cpu", base_prefix="transformer.")
+    assert w["lm_head.weight"] is w["transformer.word_embeddings.weight"]
+    cfg_u = AutoConfig.from_dict(dict(TINY["A"], tie_word_embeddings=False))
+    specs_u = lookup("falcon")[1](cfg_u).tensor_specs()
+    w = load_weights(f, specs_u, torch.float32, "cpu", base_prefix="transformer.")
+    assert float(w["lm_head.weight"][0, 0]) == 7.0
