@@ -5,8 +5,10 @@
 A step is one decode step of the batch (model step from the cache plus the greedy choice of the
 next token, fed back).  The default run: batch 8, prompts of 1,024 synthetic token ids, decoding
 towards a context of 2,048.  One JSON line is printed: decode tokens a second as ``value``, the
-prefill of 2,048 tokens under ``prefill``, the decode step's HBM roofline under ``roofline`` and
-decode at batch 1 and 64 under ``points``.
+prefill of 2,048 tokens under ``prefill``, the decode step's HBM roofline under ``roofline``,
+decode at batch 1 and 64 under ``points``, and under ``kernels`` the launches of a decode step at batch
+8 and 64 and of the prefill, each with its time (events around every launch of a step that is launched
+directly), the bytes it has to read or its arithmetic, and the fraction of the published peak.
 """
 import argparse
 import json
@@ -123,6 +125,84 @@ def run_prefill(model, T, reps=3, seed=1):
     return best
 
 
+KERNEL_LABELS = {
+    "pta_gemm_skinny_pair_qkv_bf16": "qkv+up (few rows; rotation and cache write in its epilogue)",
+    "pta_gemm_skinny_pair_bf16": "qkv+up (few rows)",
+    "pta_gemm_splitk_pair_reduced_qkv_bf16": "qkv+up (decode batch; reduction rotates and writes the cache)",
+    "pta_gemm_splitk_pair_reduced_bf16": "qkv+up (decode batch)",
+    "pta_gemm_splitk_pair_bf16": "dense+down (partial sums)",
+    "pta_gemm_splitk_bf16": "product, K split",
+    "pta_gemm_skinny_bf16": "lm_head / product of few rows",
+    "pta_layernorm_sum": "residual sum + LayerNorm",
+    "pta_attn_mfma": "attention over the cache (+ merge of key ranges)",
+    "library_mm": "vendor library products",
+    "pta_epilogue": "bias / activation / additions pass",
+    "pta_qkv_rope_cache": "split, rotation, cache write",
+}
+
+
+def kernel_figures(model, ops, dtype, step, attn_bytes=0.0, attn_flops=0.0):
+    """Per entry point of the kernel library: time of one step launched directly with events around every launch
+    (a captured step cannot hold events), the bytes it has to read or the arithmetic it does, and the achieved
+    rate as a fraction of the published peak.  ``step`` runs one step."""
+    import torch
+
+    graphs, model.use_graphs = model.use_graphs, False
+    try:
+        step()  # the shapes' first launch outside the timing
+        torch.cuda.synchronize()
+        ops.timing_hint.update(attn_bytes=attn_bytes, attn_flops=attn_flops)
+        ops.start_timing()
+        step()
+        raw = ops.stop_timing()
+    finally:
+        model.use_graphs = graphs
+    out = {}
+    for name, r in sorted(raw.items(), key=lambda kv: -kv[1]["us"]):
+        rec = {"what": KERNEL_LABELS.get(name, name), "calls": r["calls"], "us": round(r["us"], 1)}
+        if r["flops"] and r["flops"] / max(r["bytes"], 1.0) > 300:  # bound by arithmetic
+            tf = r["flops"] / r["us"] / 1e6
+            rec.update({"TFLOP/s": round(tf, 1), "frac": round(tf / PEAK_TFLOPS[dtype], 3)})
+        elif r["bytes"]:
+            gbs = r["bytes"] / r["us"] / 1e3
+            rec.update({"GB/s": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 3)})
+        out[name.replace("pta_", "")] = rec
+    return out
+
+
+def decode_kernels(model, ops, sampler_cls, gen_cfg, cfg, dtype, elem, batch, prompt_len):
+    """The kernels of one decode step of ``batch`` sequences at a context of ``prompt_len``."""
+    import torch
+
+    g = torch.Generator().manual_seed(3)
+    prompts = torch.randint(0, model.vocab_size, (batch, prompt_len), generator=g).tolist()
+    cache = model.new_cache(batch * ((prompt_len + 8 + 63) // 64 * 64), max_slots=batch)
+    slots = [cache.alloc() for _ in range(batch)]
+    model.step(cache, slots, prompts, "last")
+    per_layer_kv = batch * (prompt_len + 1) * 2 * cfg.kv_heads * cfg.head_dim * elem
+    figures = kernel_figures(model, ops, dtype, lambda: model.step(cache, slots, [[1]] * batch, "last"),
+                             attn_bytes=per_layer_kv)
+    for s_ in slots:
+        cache.free(s_)
+    return figures
+
+
+def prefill_kernels(model, ops, cfg, dtype, T):
+    import torch
+
+    g = torch.Generator().manual_seed(4)
+    prompt = torch.randint(0, model.vocab_size, (T,), generator=g).tolist()
+    cache = model.new_cache((T + 63) // 64 * 64 * 2, max_slots=2)
+
+    def step():
+        slot = cache.alloc()
+        model.step(cache, [slot], [prompt], "last")
+        cache.free(slot)
+
+    return kernel_figures(model, ops, dtype, step,
+                          attn_flops=2.0 * cfg.head_dim * cfg.num_attention_heads * T * (T + 1))
+
+
 MIXED = {"7b": (8, 1024, 1024, 128), "11b": (16, 128, 4096, 256), "40b": (32, 64, 1536, 512)}
 
 
@@ -140,6 +220,7 @@ def run_mixed(model, batch, lo, hi, new, seed=2):
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     assert all(len(o) == len(p) + new for o, p in zip(out, prompts))
+    run_mixed.lens = lens
     return dt, sum(lens)
 
 
@@ -183,10 +264,19 @@ def main():
             run_mixed(model, batch, lo, hi, 2)
         ops.release_flush()
         dt, prompt_tokens = run_mixed(model, batch, lo, hi, new)
+        # what the request has to do at the least: the prompts' arithmetic, and for every decode step all weights once
+        # and the live sequences' keys and values (a sequence of n prompt tokens is n + k long at step k)
+        flops = sum(prefill_flops(cfg, n) for n in run_mixed.lens)
+        kv = kv_bytes_per_token(cfg, elem)
+        decode_bytes = new * weight_bytes(cfg, elem) + sum(kv * (n * new + new * (new + 1) / 2) for n in run_mixed.lens)
+        floor = flops / (PEAK_TFLOPS[args.dtype] * 1e12) + decode_bytes / (HBM_PEAK_GBS * 1e9)
         print(json.dumps({"metric": f"falcon{args.sizes}_mixed_generated_tokens_per_second",
                           "value": round(batch * new / dt, 1), "unit": "tokens/s", "seconds": round(dt, 3),
                           "batch": batch, "prompt_tokens": prompt_tokens, "new_tokens_each": new,
                           "prompt_lengths": f"U[{lo},{hi}]", "layers": args.layers, "dtype": args.dtype,
+                          "roofline": {"bound": "prefill arithmetic + decode hbm", "prefill_tflop": round(flops / 1e12, 1),
+                                       "decode_gb": round(decode_bytes / 1e9, 1), "floor_s": round(floor, 3),
+                                       "frac": round(floor / dt, 4)},
                           "note": "whole requests, prefill included; greedy, no stop token"}))
         return 0
     # the choices between kernels that are timed rather than ruled, once, for the shapes measured below; the timed
@@ -230,6 +320,12 @@ def main():
             d, _ = run_decode(model, Sampler, gen_cfg, b, args.prompt_len, steps_b, 8)
             points[f"decode_b{b}"] = round(b * steps_b / d, 2)
         out["points"] = points
+        if args.dtype == "bf16":
+            out["kernels"] = {
+                f"decode_b{args.batch}": decode_kernels(model, ops, Sampler, gen_cfg, cfg, args.dtype, elem, args.batch, args.prompt_len),
+                "decode_b64": decode_kernels(model, ops, Sampler, gen_cfg, cfg, args.dtype, elem, 64, args.prompt_len),
+                "prefill_2048": prefill_kernels(model, ops, cfg, args.dtype, 2048),
+            }
     print(json.dumps(out))
     return 0
 

@@ -63,9 +63,92 @@ def load_library(build_if_missing: bool = True):
 
 def _call(name: str, *args) -> None:
     lib = load_library()
-    rc = getattr(lib, name)(*args)
+    if _timing is None or name in _HOST_ENTRIES:
+        rc = getattr(lib, name)(*args)
+    else:
+        with timed(name, *_entry_cost(name, args)):
+            rc = getattr(lib, name)(*args)
     if rc != 0:
         raise KernelError(lib.pta_last_error().decode("utf-8", "replace"))
+
+
+# ---- per-kernel timings for measurements ----------------------------------------------------------------------
+# With ``start_timing()`` every launch through this module (and the library products that ``timed`` wraps) is
+# bracketed by two events; ``stop_timing()`` returns, per entry point, calls, microseconds, the bytes it has to
+# read and the arithmetic it does.  Steps must then be launched directly (``model.use_graphs = False``): events
+# cannot be recorded into a captured step.  ``timing_hint`` carries what an entry point's arguments do not say
+# (how many cached keys and values an attention launch reads, the arithmetic of a prompt's attention).
+_timing = None
+_HOST_ENTRIES = ("pta_gemm_splitk_pair_parts",)  # entry points that launch nothing
+timing_hint = {"attn_bytes": 0, "attn_flops": 0}
+
+
+class timed:
+    def __init__(self, name: str, nbytes: float = 0.0, flops: float = 0.0):
+        self.name, self.nbytes, self.flops = name, nbytes, flops
+
+    def __enter__(self):
+        if _timing is not None:
+            self.start = torch.cuda.Event(enable_timing=True)
+            self.start.record()
+        return self
+
+    def __exit__(self, *exc):
+        if _timing is not None:
+            end = torch.cuda.Event(enable_timing=True)
+            end.record()
+            _timing.append((self.name, self.start, end, self.nbytes, self.flops))
+        return False
+
+
+def start_timing() -> None:
+    global _timing
+    _timing = []
+
+
+def stop_timing() -> dict:
+    """``{entry point: {"calls", "us", "bytes", "flops"}}`` of everything launched since ``start_timing``."""
+    global _timing
+    records, _timing = _timing or [], None
+    torch.cuda.synchronize()
+    out: dict = {}
+    for name, start, end, nbytes, flops in records:
+        r = out.setdefault(name, {"calls": 0, "us": 0.0, "bytes": 0.0, "flops": 0.0})
+        r["calls"] += 1
+        r["us"] += start.elapsed_time(end) * 1e3
+        r["bytes"] += nbytes
+        r["flops"] += flops
+    return out
+
+
+def _entry_cost(name: str, a) -> tuple:
+    """(bytes a launch has to read, arithmetic it does), from the entry point's own arguments: matrices count
+    once, activations and results of a few rows are left out."""
+    gemm = lambda M, N, K, elem=2: (float(N) * K * elem, 2.0 * M * N * K)
+    both = lambda x, y: (x[0] + y[0], x[1] + y[1])
+    if name == "pta_gemm_skinny_bf16":
+        return gemm(a[6], a[7], a[8])
+    if name == "pta_gemm_skinny_pair_bf16":
+        return both(gemm(a[12], a[4], a[13]), gemm(a[12], a[10], a[13]))
+    if name == "pta_gemm_skinny_pair_qkv_bf16":
+        return both(gemm(a[24], (a[13] + 2 * a[14]) * a[15], a[25]), gemm(a[24], a[22], a[25]))
+    if name == "pta_gemm_splitk_bf16":
+        return gemm(a[7], a[8], a[9])
+    if name == "pta_gemm_splitk_pair_bf16":
+        return both(gemm(a[10], a[3], a[4]), gemm(a[10], a[8], a[9]))
+    if name == "pta_gemm_splitk_pair_reduced_bf16":
+        return both(gemm(a[16], a[5], a[6]), gemm(a[16], a[13], a[14]))
+    if name == "pta_gemm_splitk_pair_reduced_qkv_bf16":
+        return both(gemm(a[28], (a[15] + 2 * a[16]) * a[17], a[5]), gemm(a[28], a[25], a[26]))
+    if name == "pta_gemm_splitk_reduced_qkv_bf16":
+        return gemm(a[20], (a[15] + 2 * a[16]) * a[17], a[5])
+    if name == "pta_gemm_f32":
+        return gemm(a[6], a[7], a[8], 4)
+    if name == "pta_layernorm_sum":
+        return ((a[4] + a[7]) * float(a[16]) * a[18] * 4, 0.0)
+    if name in ("pta_attn_mfma", "pta_attn_generic"):
+        return (float(timing_hint.get("attn_bytes", 0)), float(timing_hint.get("attn_flops", 0)))
+    return (0.0, 0.0)
 
 
 def _stream() -> ctypes.c_void_p:
@@ -654,17 +737,18 @@ def joined_mm_pays(x: torch.Tensor, joined: torch.Tensor, n_first: int) -> bool:
 def library_mm(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     """``x @ w.T`` in bfloat16 through the vendor library, in the pieces along M that were measured fastest."""
     M, N = x.shape[0], w.shape[0]
-    if not MM_CHUNKS or M < 512:
-        return torch.mm(x, w.t())
-    if (N, w.shape[1], (M + 63) // 64) not in _mm_plans and not _may_time():
-        return torch.mm(x, w.t())
-    out = torch.empty((M, N), dtype=x.dtype, device=x.device)
-    plan = _mm_plan(x, w, out)
-    at = 0
-    for rows in plan:
-        torch.mm(x[at:at + rows], w.t(), out=out[at:at + rows])
-        at += rows
-    return out
+    with timed("library_mm", float(w.numel()) * 2, 2.0 * M * N * w.shape[1]):
+        if not MM_CHUNKS or M < 512:
+            return torch.mm(x, w.t())
+        if (N, w.shape[1], (M + 63) // 64) not in _mm_plans and not _may_time():
+            return torch.mm(x, w.t())
+        out = torch.empty((M, N), dtype=x.dtype, device=x.device)
+        plan = _mm_plan(x, w, out)
+        at = 0
+        for rows in plan:
+            torch.mm(x[at:at + rows], w.t(), out=out[at:at + rows])
+            at += rows
+        return out
 
 
 
@@ -705,7 +789,8 @@ def library_mm_ksplit(x: torch.Tensor, w: torch.Tensor, bias=None, act=None, add
         _mm_ksplit[key] = S
     if S == 1:
         return None
-    part = _k_batch(x, w, S)
+    with timed("library_mm", float(w.numel()) * 2, 2.0 * M * N * K):
+        part = _k_batch(x, w, S)
     if bias is not None:
         _need(bias, "bias", torch.float32, (N,))
     for name, a in (("add1", add1), ("add2", add2)):

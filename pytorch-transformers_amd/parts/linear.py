@@ -243,4 +243,5 @@ class OutputHead(Part):
             return ops.gemm_f32(h, self.weight)
         if ops.gemm_skinny_ok(h, self.weight):
             return ops.gemm_skinny_bf16(h, self.weight, out_f32=True)
-        return torch.mm(h, self.weight.t(), out_dtype=torch.float32)
+        with ops.timed("library_mm", float(self.weight.numel()) * 2, 2.0 * h.shape[0] * self.weight.numel()):
+            return torch.mm(h, self.weight.t(), out_dtype=torch.float32)
