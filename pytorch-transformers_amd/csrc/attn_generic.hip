@@ -17,7 +17,7 @@ template <typename T>
 __global__ void attn_generic_kernel(T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ k_pool,
                                     const T* __restrict__ v_pool, const int* __restrict__ block_table,
                                     int bt_stride, const int* __restrict__ token_seq,
-                                    const int* __restrict__ token_pos, const float* __restrict__ slopes, int nh,
+                                    const int* __restrict__ token_pos, const float* __restrict__ slopes, int alibi_exact, int nh,
                                     int nkv, int d, float scale, float sqrt_d, int window) {
     __shared__ float q_s[256];
     __shared__ float p_s[PTA_PAGE];
@@ -47,7 +47,7 @@ __global__ void attn_generic_kernel(T* __restrict__ out, const T* __restrict__ q
             float dot = 0.f;
             for (int i = 0; i < d; ++i) dot += q_s[i] * Io<T>::ld(kr + i);
             s = dot * scale;
-            if (slopes) s += round_to_bf16(slope * round_to_bf16((float)j)) / sqrt_d;
+            if (slopes) s += (alibi_exact ? slope * (float)j : round_to_bf16(slope * round_to_bf16((float)j))) / sqrt_d;
         }
         const float m_new = fmaxf(m_run, wave_max(s));
         const float p = valid ? expf(s - m_new) : 0.f;
@@ -79,7 +79,7 @@ __global__ void attn_generic_kernel(T* __restrict__ out, const T* __restrict__ q
 
 extern "C" int pta_attn_generic(void* out, const void* q, const void* k_pool, const void* v_pool,
                                 const int* block_table, int bt_stride, const int* token_seq, const int* token_pos,
-                                const float* slopes, int M, int nh, int nkv, int d, float scale, int window, int dtype,
+                                const float* slopes, int alibi_exact, int M, int nh, int nkv, int d, float scale, int window, int dtype,
                                 void* stream) {
     PTA_REQUIRE(M > 0 && nh > 0 && nkv > 0, "attn_generic: sizes must be positive (M=%d nh=%d nkv=%d)", M, nh, nkv);
     PTA_REQUIRE(nh % nkv == 0, "attn_generic: heads (%d) must be a multiple of kv heads (%d)", nh, nkv);
@@ -92,11 +92,11 @@ extern "C" int pta_attn_generic(void* out, const void* q, const void* k_pool, co
     if (dtype == PTA_F32)
         hipLaunchKernelGGL(attn_generic_kernel<float>, grid, dim3(PTA_WAVE), 0, s, (float*)out, (const float*)q,
                            (const float*)k_pool, (const float*)v_pool, block_table, bt_stride, token_seq, token_pos,
-                           slopes, nh, nkv, d, scale, sqrt_d, window);
+                           slopes, alibi_exact, nh, nkv, d, scale, sqrt_d, window);
     else if (dtype == PTA_BF16)
         hipLaunchKernelGGL(attn_generic_kernel<bf16_t>, grid, dim3(PTA_WAVE), 0, s, (bf16_t*)out, (const bf16_t*)q,
                            (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_table, bt_stride, token_seq,
-                           token_pos, slopes, nh, nkv, d, scale, sqrt_d, window);
+                           token_pos, slopes, alibi_exact, nh, nkv, d, scale, sqrt_d, window);
     else
         return pta_fail("attn_generic: unknown dtype %d", dtype);
     return pta_check_launch("attn_generic");

@@ -102,7 +102,8 @@ __global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
     bf16_t* __restrict__ out, float* __restrict__ po, float* __restrict__ pm, float* __restrict__ pl,
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
     const int* __restrict__ block_table, int bt_stride, const int* __restrict__ cu_tokens,
-    const int* __restrict__ seq_start, const float* __restrict__ slopes, int nh, int nkv, float scale, float alibi_mul,
+    const int* __restrict__ seq_start, const float* __restrict__ slopes, int alibi_exact, int nh, int nkv, float scale,
+    float alibi_mul,
     int split_size, int n_splits, int window_arg, int paired) {
     constexpr int D = DT * 16;
     const int window = WIN ? window_arg : 0;
@@ -222,7 +223,8 @@ __global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                     const int key = kb + 8 * gq + j;  // j = 4*tt + e
-                    s[j] = sacc[j >> 2][ct][j & 3] * scale + round_to_bf16(slope[ct] * round_to_bf16((float)key)) * alibi_mul;
+                    const float bias = alibi_exact ? slope[ct] * (float)key : round_to_bf16(slope[ct] * round_to_bf16((float)key));
+                    s[j] = sacc[j >> 2][ct][j & 3] * scale + bias * alibi_mul;
                 }
             } else {  // left unscaled: the scale rides in the one multiply-add in front of the exponential
 #pragma unroll
@@ -447,7 +449,7 @@ struct AttnLaunch {
     bf16_t* out; float *po, *pm, *pl;
     const bf16_t *q, *k_pool, *v_pool;
     const int* block_table; int bt_stride;
-    const int *cu_tokens, *seq_start; const float* slopes;
+    const int *cu_tokens, *seq_start; const float* slopes; int alibi_exact;
     int n_seqs, max_new, nh, nkv; float scale;
     int split_size, n_splits, window;
     int paired;  // workgroups take two column groups each, a late one and the early one that mirrors it
@@ -462,7 +464,7 @@ static void launch_attn(const AttnLaunch& a) {
     const dim3 grid(paired ? (groups + 1) / 2 : groups, a.nkv, a.n_seqs * a.n_splits);
     auto kern = a.window > 0 ? attn_mfma_kernel<DT, CT, W, true> : attn_mfma_kernel<DT, CT, W, false>;
     hipLaunchKernelGGL(kern, grid, dim3(64 * W), 0, a.s, a.out, a.po, a.pm, a.pl, a.q, a.k_pool, a.v_pool, a.block_table,
-                       a.bt_stride, a.cu_tokens, a.seq_start, a.slopes, a.nh, a.nkv, a.scale * PTA_LOG2E,
+                       a.bt_stride, a.cu_tokens, a.seq_start, a.slopes, a.alibi_exact, a.nh, a.nkv, a.scale * PTA_LOG2E,
                        PTA_LOG2E / sqrtf((float)(DT * 16)), a.split_size, a.n_splits, a.window, paired);
 }
 
@@ -492,8 +494,8 @@ extern "C" int pta_attn_mfma_supported(int d) { return d % 16 == 0 && ((d >= 16 
 extern "C" int pta_attn_decode_max_tiles(int d) { return decode_max_tiles(d / 16); }
 
 extern "C" int pta_attn_mfma(void* out, const void* q, const void* k_pool, const void* v_pool, const int* block_table,
-                             int bt_stride, const int* cu_tokens, const int* seq_start, const float* slopes, int n_seqs,
-                             int max_new, int M, int nh, int nkv, int d, float scale, int split_size, int n_splits,
+                             int bt_stride, const int* cu_tokens, const int* seq_start, const float* slopes, int alibi_exact,
+                             int n_seqs, int max_new, int M, int nh, int nkv, int d, float scale, int split_size, int n_splits,
                              float* po, float* pm, float* pl, int window, int decode_tiles, void* stream) {
     PTA_REQUIRE(n_seqs > 0 && max_new > 0 && M > 0 && nh > 0 && nkv > 0, "attn_mfma: sizes must be positive");
     PTA_REQUIRE(nh % nkv == 0, "attn_mfma: heads (%d) must be a multiple of kv heads (%d)", nh, nkv);
@@ -533,7 +535,7 @@ extern "C" int pta_attn_mfma(void* out, const void* q, const void* k_pool, const
                 dct_most);
     const int dct = decode_tiles > 0 ? decode_tiles : dct_most;
     const AttnLaunch a{(bf16_t*)out, po, pm, pl, (const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool,
-                       block_table, bt_stride, cu_tokens, seq_start, slopes, n_seqs, max_new, nh, nkv, scale,
+                       block_table, bt_stride, cu_tokens, seq_start, slopes, alibi_exact, n_seqs, max_new, nh, nkv, scale,
                        split_size, n_splits, window, paired, s};
 #define PTA_ATTN_CASE(DT_)                                        \
     case DT_:                                                     \

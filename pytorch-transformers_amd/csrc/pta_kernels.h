@@ -14,7 +14,7 @@
 
 #include <stdint.h>
 
-#define PTA_ABI_VERSION 2
+#define PTA_ABI_VERSION 3
 
 #ifdef __cplusplus
 extern "C" {
@@ -55,8 +55,12 @@ int pta_qkv_rope_cache(void* q_out, const void* fused, int fused_ld, const float
 
 // causal attention of M tokens over their sequences' cache, 32-bit arithmetic
 // window: 0, or the number of last positions a token sees (itself included)
+// slopes (null: none): a bias slope[head] * key position / sqrt(d) on the scores; with alibi_exact = 0 the position
+// and the product are rounded to bfloat16 first, as the reference forms them, and the slopes given are expected
+// rounded too; with 1 nothing is rounded
 int pta_attn_generic(void* out, const void* q, const void* k_pool, const void* v_pool, const int* block_table,
-                     int bt_stride, const int* token_seq, const int* token_pos, const float* slopes, int M, int nh,
+                     int bt_stride, const int* token_seq, const int* token_pos, const float* slopes, int alibi_exact,
+                     int M, int nh,
                      int nkv, int d, float scale, int window, int dtype, void* stream);
 
 // the same attention for bfloat16 on the matrix cores; cu_tokens [n_seqs + 1] and seq_start [n_seqs] say
@@ -69,8 +73,8 @@ int pta_attn_mfma_supported(int d);
 // Column tiles (sixteen query heads of one KV head) that one wave of a decode launch can hold at this head size.
 int pta_attn_decode_max_tiles(int d);
 int pta_attn_mfma(void* out, const void* q, const void* k_pool, const void* v_pool, const int* block_table,
-                  int bt_stride, const int* cu_tokens, const int* seq_start, const float* slopes, int n_seqs,
-                  int max_new, int M, int nh, int nkv, int d, float scale, int split_size, int n_splits, float* po,
+                  int bt_stride, const int* cu_tokens, const int* seq_start, const float* slopes, int alibi_exact,
+                  int n_seqs, int max_new, int M, int nh, int nkv, int d, float scale, int split_size, int n_splits, float* po,
                   float* pm, float* pl, int window, int decode_tiles, void* stream);
 
 // C = act(A . W^T + bias) + add1 + add2, all 32-bit, fixed summation order

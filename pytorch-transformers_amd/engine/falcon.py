@@ -45,7 +45,8 @@ def rotary_positions(cfg: FalconConfig) -> RotaryPositions:
 def build_falcon(cfg: FalconConfig) -> ModelSpec:
     H, L, eps = cfg.hidden_size, cfg.num_hidden_layers, cfg.layer_norm_epsilon
     if cfg.alibi:
-        positions = AlibiPositions(cfg.num_attention_heads)
+        # ``alibi_bf16_compat`` is this library's own key (default true: the reference's rounding of the bias)
+        positions = AlibiPositions(cfg.num_attention_heads, bf16_compat=bool(cfg.extra.get("alibi_bf16_compat", True)))
     else:
         positions = rotary_positions(cfg)
     blocks = []

@@ -24,7 +24,7 @@ QKV_LAYOUT_CODES = {"grouped": 0, "tail": 1, "interleaved": 2}
 ACT_CODES = {None: 0, "none": 0, "linear": 0, "gelu": 1, "gelu_python": 1, "gelu_new": 2, "gelu_pytorch_tanh": 2,
              "gelu_fast": 2, "gelu_accurate": 2, "quick_gelu": 3, "relu": 4, "relu2": 5, "relu6": 6, "silu": 7, "swish": 7,
              "sigmoid": 8, "tanh": 9, "leaky_relu": 10, "mish": 11, "gelu_10": 12, "laplace": 13}
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _lib = None
 _lock = threading.Lock()
@@ -309,7 +309,7 @@ def qkv_rope_cache(fused: torch.Tensor, bias, inv_freq, cs_scale: float, token_p
 
 
 def attn_generic(q: torch.Tensor, k_pool, v_pool, block_table, token_seq, token_pos, slopes, scale: float,
-                 window: int = 0):
+                 window: int = 0, alibi_exact: bool = False):
     """Causal attention of every token over its sequence's cache (the last ``window`` positions of it, itself
     included, if ``window`` > 0); out [M, nh*d]."""
     _need(q, "q")
@@ -323,8 +323,8 @@ def attn_generic(q: torch.Tensor, k_pool, v_pool, block_table, token_seq, token_
         _need(slopes, "slopes", torch.float32, (nh,))
     out = torch.empty((M, nh * d), dtype=q.dtype, device=q.device)
     _call("pta_attn_generic", _ptr(out), _ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(block_table),
-          block_table.shape[1], _ptr(token_seq), _ptr(token_pos), _ptr(slopes), M, nh, nkv, d, ctypes.c_float(scale),
-          int(window), dtype_code(q.dtype), _stream())
+          block_table.shape[1], _ptr(token_seq), _ptr(token_pos), _ptr(slopes), int(bool(alibi_exact)), M, nh, nkv, d,
+          ctypes.c_float(scale), int(window), dtype_code(q.dtype), _stream())
     return out
 
 
@@ -360,7 +360,7 @@ def attn_mfma_ok(q: torch.Tensor) -> bool:
 
 def attn_mfma(q: torch.Tensor, k_pool, v_pool, block_table, cu_tokens, seq_start, slopes, scale: float, *,
               max_new: int, n_splits: int = 1, split_size: int = ATTN_SPLIT_KEYS, window: int = 0,
-              decode_tiles: int = 0) -> torch.Tensor:
+              decode_tiles: int = 0, alibi_exact: bool = False) -> torch.Tensor:
     """Causal attention of a step's tokens over the cache on the matrix cores; out [M, nh*d].
 
     ``max_new`` bounds the new tokens of any sequence of the step; with ``n_splits > 1`` the keys
@@ -384,7 +384,8 @@ def attn_mfma(q: torch.Tensor, k_pool, v_pool, block_table, cu_tokens, seq_start
         pm = torch.empty((M, nh, n_splits), dtype=torch.float32, device=q.device)
         pl = torch.empty((M, nh, n_splits), dtype=torch.float32, device=q.device)
     _call("pta_attn_mfma", _ptr(out), _ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(block_table), block_table.shape[1],
-          _ptr(cu_tokens), _ptr(seq_start), _ptr(slopes), n_seqs, int(max_new), M, nh, nkv, d, ctypes.c_float(scale),
+          _ptr(cu_tokens), _ptr(seq_start), _ptr(slopes), int(bool(alibi_exact)), n_seqs, int(max_new), M, nh, nkv, d,
+          ctypes.c_float(scale),
           int(split_size), int(n_splits), _ptr(po), _ptr(pm), _ptr(pl), int(window), int(decode_tiles), _stream())
     return out
 
@@ -459,7 +460,8 @@ def decode_plan(n_seqs: int, n_heads: int, n_kv_heads: int, head_dim: int, max_l
     return _decode_plan(n, n_heads, n_kv_heads, head_dim, bound, mean, most)
 
 
-def attention(q: torch.Tensor, k_pool, v_pool, block_table, ctx, slopes, scale: float, window: int = 0) -> torch.Tensor:
+def attention(q: torch.Tensor, k_pool, v_pool, block_table, ctx, slopes, scale: float, window: int = 0,
+              alibi_exact: bool = False) -> torch.Tensor:
     """Attention of a step's tokens over the cache: picks the kernel for the step's shape and type.
 
     bfloat16 with a head size the matrix-core kernel is built for: that kernel, with the context
@@ -473,8 +475,8 @@ def attention(q: torch.Tensor, k_pool, v_pool, block_table, ctx, slopes, scale: 
             n_splits = (ctx.max_len + size - 1) // size
         return attn_mfma(q, k_pool, v_pool, block_table, ctx.cu_tokens, ctx.seq_start, slopes, scale,
                          max_new=max(ctx.new_tokens), n_splits=n_splits, split_size=size, window=window,
-                         decode_tiles=tiles)
-    return attn_generic(q, k_pool, v_pool, block_table, ctx.token_seq, ctx.token_pos, slopes, scale, window)
+                         decode_tiles=tiles, alibi_exact=alibi_exact)
+    return attn_generic(q, k_pool, v_pool, block_table, ctx.token_seq, ctx.token_pos, slopes, scale, window, alibi_exact)
 
 
 def sample(logits: torch.Tensor, *, do_sample: bool, temperature: float = 1.0, top_k: int = 0, top_p: float = 1.0,

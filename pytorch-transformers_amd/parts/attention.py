@@ -77,7 +77,8 @@ class AttentionMixer(Part):
         else:
             fused = projected if projected is not None else self.qkv(x, apply_bias=False)
             q = self.projection_tail(ctx, call).run(fused)
-        o = ops.attention(q, k_pool, v_pool, table, ctx, self.positions.score_bias(), self.scale, self.window)
+        o = ops.attention(q, k_pool, v_pool, table, ctx, self.positions.score_bias(), self.scale, self.window,
+                          alibi_exact=bool(getattr(self.positions, "exact_bias", False)))
         if defer:
             return PendingProjection(self.out, o)
         return self.out(o, add1=residual)

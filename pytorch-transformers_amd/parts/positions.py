@@ -183,9 +183,16 @@ class AlibiPositions(NoPositions):
     attention kernels round the position and the product.
     """
 
-    def __init__(self, num_heads: int):
+    #: False: slopes, positions and their product are rounded to bfloat16 as the reference rounds them
+    exact_bias = False
+
+    def __init__(self, num_heads: int, bf16_compat: bool = True):
+        """``bf16_compat=False`` leaves the reference's numbers for the exact ``slope * position`` in 32-bit
+        (``alibi_bf16_compat: false`` in config.json); the default reproduces the reference."""
         self.num_heads = num_heads
-        self.slopes = alibi_slopes(num_heads).bfloat16().float().contiguous()
+        self.exact_bias = not bf16_compat
+        slopes = alibi_slopes(num_heads)
+        self.slopes = (slopes if self.exact_bias else slopes.bfloat16().float()).contiguous()
 
     def to(self, device) -> None:
         self.slopes = self.slopes.to(device)

@@ -182,10 +182,12 @@ def alibi_slopes(nh: int):
     return slopes
 
 
-def alibi_bias(nh: int, n_keys: int, head_dim: int, dtype=DT):
+def alibi_bias(nh: int, n_keys: int, head_dim: int, dtype=DT, bf16_compat: bool = True):
     """[heads, keys]: bf16(slope) * position formed in bfloat16 (:196-198), then / sqrt(d) in the
-    model's type (:1078-1085)."""
+    model's type (:1078-1085).  ``bf16_compat=False`` (not the reference): the exact product."""
     pos = torch.arange(n_keys, dtype=torch.int64)
+    if not bf16_compat:
+        return (alibi_slopes(nh)[:, None].to(dtype) * pos[None, :].to(dtype)) / math.sqrt(head_dim)
     alibi = alibi_slopes(nh)[:, None].bfloat16() * pos[None, :]  # bfloat16 result, as in the reference
     return alibi.to(dtype) / math.sqrt(head_dim)
 
@@ -237,7 +239,7 @@ def self_attention(x, w, prefix, c, positions, seq_lens=None):
     q, k, v = split_heads(fused, c)
     bias = None
     if c["alibi"]:
-        bias = alibi_bias(nh, x.shape[0], d, x.dtype)
+        bias = alibi_bias(nh, x.shape[0], d, x.dtype, bool(c.get("alibi_bf16_compat", True)))
     elif seq_lens is None or (c.get("rope_scaling") or {}).get("rope_type", (c.get("rope_scaling") or {}).get("type")) != "dynamic":
         inv_freq, scale = rope_parameters(c, x.shape[0])
         cos, sin = rope_cos_sin(positions, inv_freq, x.dtype, scale)

@@ -159,6 +159,28 @@ def test_first_tokens(folders, dtype, rel):
     helpers.assert_close(got["r0"], want["r0"], rel, f"A {dtype} first tokens")
 
 
+@pytest.mark.parametrize("dtype,rel", [("float32", REL_F32), ("bfloat16", REL_BF16)])
+def test_alibi_without_the_references_rounding(tmp_path, dtype, rel):
+    """``alibi_bf16_compat: false`` in config.json: the bias is the exact slope times position; the default keeps the
+    reference's bfloat16 rounding of both and of their product, and the two differ visibly past position 256."""
+    from pytorch_transformers_amd import AutoModelForCausalLM
+    from pytorch_transformers_amd.engine.replay import Replayer
+    from tiny import write_config
+
+    raw = dict(TINY["E"], alibi_bf16_compat=False)
+    folder = write_config(raw, str(tmp_path), "exact", seed=4)
+    reqs = helpers.make_requests(raw["vocab_size"], [330, 40], seed=8)
+    want = helpers.plain_logits(folder, reqs)
+    rp = Replayer(AutoModelForCausalLM.from_pretrained(folder, dtype=dtype), 1024)
+    for records in (helpers.schedule_whole(reqs), helpers.schedule_batches(reqs, 2, decode=(40, 5))):
+        got = helpers.run_schedule(rp, records)
+        for rid in reqs:
+            helpers.assert_close(got[rid], want[rid], rel, f"exact alibi {dtype} {rid}")
+    if dtype == "float32":
+        rounded = helpers.plain_logits(write_config(TINY["E"], str(tmp_path), "rounded", seed=4), reqs)
+        assert float((rounded["r0"] - want["r0"]).abs().max()) > 1e-3 * float(want["r0"].abs().max())
+
+
 def test_dtype_auto_follows_the_configuration_then_the_file(tmp_path):
     """``dtype="auto"`` (src/transformers/modeling_utils.py:3996-4058): config.json's ``torch_dtype`` if it names
     one, else the type of the first floating-point tensor of the file."""
