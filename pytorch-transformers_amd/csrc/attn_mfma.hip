@@ -308,8 +308,11 @@ __global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
         __shared__ __attribute__((aligned(16))) bf16_t vbuf[2][D * VROW];
         const int tid = threadIdx.x;
         const int wg_last_col = min(ncols, wg_col0 + 16 * CT * W) - 1;
-        const int k_end_wg = start + wg_last_col / g + 1;
-        const int k_begin_wg = window > 0 ? max(0, start + wg_col0 / g - window + 1) & ~31 : 0;
+        // (a launch that cuts the keys into ranges walks its own range only)
+        const int k_end_wg = n_splits > 1 ? min(start + wg_last_col / g + 1, split * split_size + split_size)
+                                          : start + wg_last_col / g + 1;
+        const int k_begin_wg = max(window > 0 ? max(0, start + wg_col0 / g - window + 1) & ~31 : 0,
+                                   n_splits > 1 ? split * split_size : 0);
         static_assert(PER <= 2, "a thread moves at most two pieces of keys and two of values per block");
         // the pieces in flight are plain variables, not an array: an array that lambdas index stays in
         // scratch memory at the larger head sizes, and every block then waits for its loads at once

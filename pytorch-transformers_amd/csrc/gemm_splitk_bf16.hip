@@ -480,13 +480,18 @@ extern "C" int pta_gemm_splitk_bf16(void* y, float* part, const void* x, const v
 // Counts that a caller has fixed for the pairs of one shape: no rule tells which neighbour of its choice is the
 // fastest (Falcon2-11B's output and feed-forward-down pair at 64 rows: 2 and 7 ranges by the rule; 4 and 8 make the
 // decode step 7 % faster, 2 and 10 make it 3 % slower with as many workgroups), so the Python side times them once.
-static std::map<std::array<int, 4>, std::pair<int, int>> pair_parts_fixed;
+struct PairChoice { int p1, p2, rt; };
+static std::map<std::array<int, 4>, PairChoice> pair_parts_fixed;
 static std::mutex pair_parts_lock;
 
 static bool parts_valid(int K, int p) { return p >= 1 && clamp_parts(p, K) == p && effective_parts(K, p) == p; }
 
-// p1 = p2 = 0 forgets the shape; returns 1 (no error text) for counts that the kernel does not take
-extern "C" int pta_gemm_splitk_pair_fix_parts(int N1, int K1, int N2, int K2, int p1, int p2) {
+// Fixes, for every later pair launch of this shape, the ranges of K of the two products and how many tiles of
+// sixteen rows of W a wave holds in steps of more than 32 rows (rt 1 or 2: 64 or 128 rows of W a workgroup; the
+// taller tile loads the activations half as often and has half as many workgroups).  p1 = p2 = 0 forgets the
+// shape.  Returns 1 (no error text) for counts that the kernel does not take.  The ranges decide the order of
+// summation; the tile height does not.
+extern "C" int pta_gemm_splitk_pair_fix(int N1, int K1, int N2, int K2, int p1, int p2, int rt) {
     if (N1 <= 0 || K1 <= 0 || N2 <= 0 || K2 <= 0) return 1;
     std::lock_guard<std::mutex> hold(pair_parts_lock);
     const std::array<int, 4> key{N1, K1, N2, K2};
@@ -494,19 +499,24 @@ extern "C" int pta_gemm_splitk_pair_fix_parts(int N1, int K1, int N2, int K2, in
         pair_parts_fixed.erase(key);
         return 0;
     }
-    if (!parts_valid(K1, p1) || !parts_valid(K2, p2)) return 1;
-    pair_parts_fixed[key] = {p1, p2};
+    if (!parts_valid(K1, p1) || !parts_valid(K2, p2) || (rt != 1 && rt != 2)) return 1;
+    pair_parts_fixed[key] = {p1, p2, rt};
     return 0;
 }
 
-static void pick_pair_parts(int N1, int K1, int N2, int K2, int* p1, int* p2) {
+extern "C" int pta_gemm_splitk_pair_fix_parts(int N1, int K1, int N2, int K2, int p1, int p2) {
+    return pta_gemm_splitk_pair_fix(N1, K1, N2, K2, p1, p2, 1);
+}
+
+// returns the row tiles per wave for steps of more than 32 rows
+static int pick_pair_parts(int N1, int K1, int N2, int K2, int* p1, int* p2) {
     {
         std::lock_guard<std::mutex> hold(pair_parts_lock);
         const auto it = pair_parts_fixed.find({N1, K1, N2, K2});
         if (it != pair_parts_fixed.end()) {
-            *p1 = it->second.first;
-            *p2 = it->second.second;
-            return;
+            *p1 = it->second.p1;
+            *p2 = it->second.p2;
+            return it->second.rt;
         }
     }
     const int g1 = (N1 + 63) / 64, g2 = (N2 + 63) / 64;
@@ -520,6 +530,7 @@ static void pick_pair_parts(int N1, int K1, int N2, int K2, int* p1, int* p2) {
     }
     *p1 = effective_parts(K1, a);
     *p2 = effective_parts(K2, b);
+    return 1;
 }
 
 extern "C" int pta_gemm_splitk_pair_parts(int N1, int K1, int N2, int K2, int* p1, int* p2) {
@@ -536,9 +547,10 @@ extern "C" int pta_gemm_splitk_pair_bf16(float* part1, const void* x1, const voi
     if (check_splitk("gemm_splitk_pair_bf16", x2, W2, M, N2, K2)) return 1;
     PTA_REQUIRE(part1 && part2, "gemm_splitk_pair_bf16: null workspace");
     int p1, p2;
-    pick_pair_parts(N1, K1, N2, K2, &p1, &p2);
-    const SplitkProblem a = make_problem(nullptr, part1, x1, W1, nullptr, nullptr, nullptr, N1, K1, 0, 0, 1, p1, 0);
-    const SplitkProblem b = make_problem(nullptr, part2, x2, W2, nullptr, nullptr, nullptr, N2, K2, 0, 0, 1, p2, 0);
+    const int rt = M > 32 ? pick_pair_parts(N1, K1, N2, K2, &p1, &p2) : (pick_pair_parts(N1, K1, N2, K2, &p1, &p2), 1);
+    const SplitkProblem a = make_problem(nullptr, part1, x1, W1, nullptr, nullptr, nullptr, N1, K1, 0, 0, rt, p1, 0);
+    const SplitkProblem b = make_problem(nullptr, part2, x2, W2, nullptr, nullptr, nullptr, N2, K2, 0, 0, rt, p2, 0);
+    if (rt == 2) return launch_rows<2, 2, 2>(tiles_per_chunk(M), a, b, M, 0, (hipStream_t)stream);
     return launch_rows<1, 2, 2>(tiles_per_chunk(M), a, b, M, 0, (hipStream_t)stream);
 }
 

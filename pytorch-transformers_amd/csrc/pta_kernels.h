@@ -144,6 +144,9 @@ int pta_gemm_reduce_parts(void* y, const float* part, const float* bias, const v
 // fixes the ranges of K (1..16 each, as pta_gemm_splitk_pair_parts then reports them) for every later pair launch
 // of this shape; 0, 0 returns the shape to the built-in rule; returns 1 for counts the kernel does not take
 int pta_gemm_splitk_pair_fix_parts(int N1, int K1, int N2, int K2, int p1, int p2);
+// the same, and how many tiles of sixteen rows of W a wave holds in steps of more than 32 rows (rt 1 or 2, i.e. 64
+// or 128 rows of W a workgroup); the ranges decide the order of summation, the tile height does not
+int pta_gemm_splitk_pair_fix(int N1, int K1, int N2, int K2, int p1, int p2, int rt);
 int pta_gemm_splitk_pair_bf16(float* part1, const void* x1, const void* W1, int N1, int K1, float* part2,
                               const void* x2, const void* W2, int N2, int K2, int M, void* stream);
 

@@ -921,39 +921,74 @@ def gemm_splitk_pair_parts(N1: int, K1: int, N2: int, K2: int):
 # later launch (PTA_PAIR_TUNE=0 switches this off).
 PAIR_TUNE = os.environ.get("PTA_PAIR_TUNE", "1") != "0"
 PAIR_TUNE_MARGIN = 0.97
+PAIR_TUNE_ROWS = int(os.environ.get("PTA_PAIR_TUNE_ROWS", "64"))  # rows of the timed launches (17 to 128)
 _pair_parts_tuned: dict = {}  # (shape of w1, shape of w2) -> the counts in use
 
 
 def tune_pair_parts(w1: torch.Tensor, w2: torch.Tensor) -> None:
-    """Once per pair of shapes: time the pair launch with the rule's ranges of K and with their neighbours, and fix
-    the fastest in the kernel library if it beats the rule's by the margin (``_pair_parts_tuned`` says which)."""
+    """Once per pair of shapes, while timing is on: time the pair launch with the rule's ranges of K, with their
+    neighbours, and with workgroups of 128 rows of W (which load the activations half as often, have half as many
+    workgroups and so want more ranges), at 64 rows with cold caches; keep the fastest in the kernel library if it
+    beats the rule's by the margin and is no slower than the rule's at 24 rows (where the tile height does not
+    apply, but the ranges do).  ``_pair_parts_tuned`` says what is in use: (ranges, ranges, row tiles per wave)."""
     key = (tuple(w1.shape), tuple(w2.shape))
     if not PAIR_TUNE or key in _pair_parts_tuned or not _may_time():
         return
     lib = load_library()
     (N1, K1), (N2, K2) = w1.shape, w2.shape
     a0, b0 = gemm_splitk_pair_parts(N1, K1, N2, K2)
-    fix = lambda c: lib.pta_gemm_splitk_pair_fix_parts(int(N1), int(K1), int(N2), int(K2), int(c[0]), int(c[1]))
-    cands = [(a0, b0)] + [(a, b) for a in range(max(1, a0 - 1), a0 + 3) for b in range(max(1, b0 - 2), b0 + 3)
-                          if (a, b) != (a0, b0)]
+    fix = lambda c: lib.pta_gemm_splitk_pair_fix(int(N1), int(K1), int(N2), int(K2), int(c[0]), int(c[1]), int(c[2]))
+    forget = lambda: lib.pta_gemm_splitk_pair_fix(int(N1), int(K1), int(N2), int(K2), 0, 0, 1)
+    cands = [(a0, b0, 1)] + [(a, b, 1) for a in range(max(1, a0 - 1), a0 + 3) for b in range(max(1, b0 - 2), b0 + 3)
+                             if (a, b) != (a0, b0)]
+    tall = lambda p: sorted({max(1, p - 1), p, p + 1, max(1, 2 * p - 1), 2 * p, 2 * p + 1})
+    cands += [(a, b, 2) for a in tall(a0) for b in tall(b0)]
     cands = [c for c in cands if fix(c) == 0]
-    xs = [torch.randn((64, K), dtype=torch.float32, device=w1.device).to(torch.bfloat16) for K in (K1, K2)]
-    parts = [[torch.empty((c[i], 64, N), dtype=torch.float32, device=w1.device) for i, N in enumerate((N1, N2))]
-             for c in cands]
+    xs = {rows: [torch.randn((rows, K), dtype=torch.float32, device=w1.device).to(torch.bfloat16) for K in (K1, K2)]
+          for rows in (PAIR_TUNE_ROWS, 24)}
+    most = [max(c[i] for c in cands) for i in (0, 1)]
+    parts = [torch.empty((most[i], PAIR_TUNE_ROWS, N), dtype=torch.float32, device=w1.device) for i, N in enumerate((N1, N2))]
+    # A launch is timed over several copies of the matrices in turn (more bytes than the memory-side cache holds),
+    # back to back between two events: every launch reads its matrices from memory, as in a model, and no gap of
+    # the host's lies inside the timed span.
+    copy_bytes = (w1.numel() + w2.numel()) * 2
+    n_copies = max(2, min(6, int(640e6 // copy_bytes) + 1))
+    copies = [(w1, w2)] + [(w1.clone(), w2.clone()) for _ in range(n_copies - 1)]
 
-    def way(c, out):
-        def run():
-            fix(c)
-            _call("pta_gemm_splitk_pair_bf16", _ptr(out[0]), _ptr(xs[0]), _ptr(w1), int(N1), int(K1), _ptr(out[1]),
-                  _ptr(xs[1]), _ptr(w2), int(N2), int(K2), 64, _stream())
-        return run
+    def timed_ways(chosen, rows, rounds=3):
+        best = [float("inf")] * len(chosen)
+        for r in range(rounds + 1):  # the first round warms up
+            for j, c in enumerate(chosen):
+                fix(c)
+                start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                start.record()
+                for a, b in copies:
+                    _call("pta_gemm_splitk_pair_bf16", _ptr(parts[0]), _ptr(xs[rows][0]), _ptr(a), int(N1), int(K1),
+                          _ptr(parts[1]), _ptr(xs[rows][1]), _ptr(b), int(N2), int(K2), rows, _stream())
+                end.record()
+                end.synchronize()
+                if r > 0:
+                    best[j] = min(best[j], start.elapsed_time(end) / len(copies))
+        return best
 
     try:
-        times = _time_ways_cold([way(c, out) for c, out in zip(cands, parts)], w1.device)
+        times = timed_ways(cands, PAIR_TUNE_ROWS)
+        order = sorted(range(len(cands)), key=lambda i: times[i])
+        short = [0] + [i for i in order if i != 0 and times[i] < PAIR_TUNE_MARGIN * times[0]][:3]
+        small = timed_ways([cands[i] for i in short], 24) if len(short) > 1 else [0.0]
     finally:
-        fix((0, 0))
-    best = min(range(len(cands)), key=lambda i: times[i])
-    chosen = cands[best] if times[best] < PAIR_TUNE_MARGIN * times[0] else cands[0]
+        forget()
+        del copies
+    if os.environ.get("PTA_TUNE_VERBOSE"):
+        print(f"[pta tune] pair {key}: rule {cands[0]} {times[0] * 1e3:.1f} us at {PAIR_TUNE_ROWS} rows; fastest " +
+              ", ".join(f"{cands[i]} {times[i] * 1e3:.1f}" for i in order[:6]) +
+              (f"; at 24 rows {[round(t * 1e3, 1) for t in small]} for {[cands[i] for i in short]}" if len(short) > 1 else ""),
+              flush=True)
+    chosen = cands[0]
+    for i, t24 in zip(short[1:], small[1:]):  # fastest first
+        if t24 <= 1.03 * small[0]:
+            chosen = cands[i]
+            break
     if chosen != cands[0]:
         fix(chosen)
     _pair_parts_tuned[key] = chosen
@@ -964,7 +999,7 @@ def tuning_table() -> dict:
     that process makes the same choices, hence the same bits."""
     key = lambda t: ",".join("x".join(str(int(v)) for v in (p if isinstance(p, tuple) else (p,))) for p in t)
     return {
-        "pair_parts": {key(k): list(v) for k, v in _pair_parts_tuned.items()},
+        "pair_parts": {key(k): list(v) for k, v in _pair_parts_tuned.items()},  # ranges, ranges, row tiles per wave
         "splitk_rows": {key(k): int(v) for k, v in _splitk_limits.items()},
         "mm_plans": {key(k): list(v) for k, v in _mm_plans.items()},
         "mm_joined": {key(k): bool(v) for k, v in _mm_joined.items()},
@@ -976,7 +1011,7 @@ def clear_tuning() -> None:
     """Back to the built-in defaults for every shape."""
     lib = load_library()
     for (s1, s2) in list(_pair_parts_tuned):
-        lib.pta_gemm_splitk_pair_fix_parts(int(s1[0]), int(s1[1]), int(s2[0]), int(s2[1]), 0, 0)
+        lib.pta_gemm_splitk_pair_fix(int(s1[0]), int(s1[1]), int(s2[0]), int(s2[1]), 0, 0, 1)
     for d in (_pair_parts_tuned, _splitk_limits, _mm_plans, _mm_costs, _mm_times, _mm_joined, _mm_ksplit):
         d.clear()
 
@@ -986,12 +1021,13 @@ def load_tuning(table: dict) -> None:
     lib = load_library()
     shapes = lambda k: tuple(tuple(int(v) for v in p.split("x")) for p in k.split(","))
     flat = lambda k: tuple(int(p) for p in k.split(","))
-    for k, (a, b) in table.get("pair_parts", {}).items():
+    for k, v in table.get("pair_parts", {}).items():
         s1, s2 = shapes(k)
+        a, b, rt = int(v[0]), int(v[1]), int(v[2]) if len(v) > 2 else 1
         rule = gemm_splitk_pair_parts_rule(s1[0], s1[1], s2[0], s2[1])
-        if (int(a), int(b)) != rule and lib.pta_gemm_splitk_pair_fix_parts(s1[0], s1[1], s2[0], s2[1], int(a), int(b)):
-            raise KernelError(f"tuning table: {a} and {b} ranges of K are not valid for the pair {k}")
-        _pair_parts_tuned[(s1, s2)] = (int(a), int(b))
+        if (a, b, rt) != rule + (1,) and lib.pta_gemm_splitk_pair_fix(s1[0], s1[1], s2[0], s2[1], a, b, rt):
+            raise KernelError(f"tuning table: {a} and {b} ranges of K with {rt} row tiles are not valid for the pair {k}")
+        _pair_parts_tuned[(s1, s2)] = (a, b, rt)
     for k, v in table.get("splitk_rows", {}).items():
         _splitk_limits[shapes(k)] = int(v)
     for k, v in table.get("mm_plans", {}).items():
@@ -1005,11 +1041,11 @@ def load_tuning(table: dict) -> None:
 def gemm_splitk_pair_parts_rule(N1: int, K1: int, N2: int, K2: int):
     """The ranges of K that the kernel library's own rule gives a pair, whatever has been fixed for the shape."""
     lib = load_library()
-    now = gemm_splitk_pair_parts(N1, K1, N2, K2)
-    lib.pta_gemm_splitk_pair_fix_parts(int(N1), int(K1), int(N2), int(K2), 0, 0)
+    kept = _pair_parts_tuned.get(((int(N1), int(K1)), (int(N2), int(K2))))
+    lib.pta_gemm_splitk_pair_fix(int(N1), int(K1), int(N2), int(K2), 0, 0, 1)
     rule = gemm_splitk_pair_parts(N1, K1, N2, K2)
-    if now != rule:
-        lib.pta_gemm_splitk_pair_fix_parts(int(N1), int(K1), int(N2), int(K2), int(now[0]), int(now[1]))
+    if kept is not None and tuple(kept) != rule + (1,):
+        lib.pta_gemm_splitk_pair_fix(int(N1), int(K1), int(N2), int(K2), int(kept[0]), int(kept[1]), int(kept[2]))
     return rule
 
 

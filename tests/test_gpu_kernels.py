@@ -241,9 +241,9 @@ def test_pair_ranges_are_timed_once_per_shape_and_kept():
         y1, y2 = ops.gemm_splitk_pair_bf16(x1, w1, x2, w2)
     ops.release_flush()
     if ops.PAIR_TUNE:
-        kept = ops._pair_parts_tuned[key]
-        assert abs(kept[0] - rule[0]) <= 2 and abs(kept[1] - rule[1]) <= 2
-        assert ops.gemm_splitk_pair_parts(N1, K1, N2, K2) == kept
+        kept = ops._pair_parts_tuned[key]  # ranges, ranges, row tiles per wave
+        assert kept[2] in (1, 2) and 1 <= kept[0] <= 2 * rule[0] + 1 and 1 <= kept[1] <= 2 * rule[1] + 1
+        assert ops.gemm_splitk_pair_parts(N1, K1, N2, K2) == kept[:2]
     p1, p2 = ops.gemm_splitk_pair_parts(N1, K1, N2, K2)
     assert torch.equal(y1, ops.gemm_splitk_bf16(x1, w1, rt=1, parts=p1)) and torch.equal(y2, ops.gemm_splitk_bf16(x2, w2, rt=1, parts=p2))
     for y, x, w in ((y1, x1, w1), (y2, x2, w2)):
@@ -258,6 +258,11 @@ def test_pair_ranges_are_timed_once_per_shape_and_kept():
         assert ops.gemm_splitk_pair_parts(N1, K1, N2, K2) == (1, 3)
         z1, z2 = ops.gemm_splitk_pair_bf16(x1, w1, x2, w2)
         assert torch.equal(z1, ops.gemm_splitk_bf16(x1, w1, rt=1, parts=1)) and torch.equal(z2, ops.gemm_splitk_bf16(x2, w2, rt=1, parts=3))
+        # workgroups of 128 rows of W instead of 64: other workgroups, the same ranges, the same bits
+        assert lib.pta_gemm_splitk_pair_fix(N1, K1, N2, K2, 1, 3, 2) == 0
+        t1, t2 = ops.gemm_splitk_pair_bf16(x1, w1, x2, w2)
+        assert torch.equal(t1, z1) and torch.equal(t2, z2)
+        assert lib.pta_gemm_splitk_pair_fix(N1, K1, N2, K2, 1, 3, 3) == 1
     finally:
         assert lib.pta_gemm_splitk_pair_fix_parts(N1, K1, N2, K2, 0, 0) == 0
         ops._pair_parts_tuned.pop(key, None)
