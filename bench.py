@@ -263,6 +263,10 @@ def main():
         with ops.live_tuning():  # the choices that are timed, for the shapes of this run; nothing of it is timed below
             run_mixed(model, batch, lo, hi, 2)
         ops.release_flush()
+        # ... and the decode attention's cut at the (longest, mean) contexts that the run passes through
+        lens = run_mixed.lens
+        model.tune(prompt_lens=(), batches=(batch,),
+                   contexts=sorted({(max(lens) + k, sum(lens) // len(lens) + k) for k in range(1, new + 1, 64)}))
         dt, prompt_tokens = run_mixed(model, batch, lo, hi, new)
         # what the request has to do at the least: the prompts' arithmetic, and for every decode step all weights once
         # and the live sequences' keys and values (a sequence of n prompt tokens is n + k long at step k)
@@ -281,7 +285,8 @@ def main():
         return 0
     # the choices between kernels that are timed rather than ruled, once, for the shapes measured below; the timed
     # steps themselves time nothing
-    model.tune(prompt_lens=(2048,), batches=sorted({args.batch, 1, 64}))
+    model.tune(prompt_lens=(2048,), batches=sorted({args.batch, 1, 64}),
+               contexts=sorted({args.prompt_len + 1, args.prompt_len + args.warmup + args.steps}))
     if args.only_prefill:
         pt = run_prefill(model, 2048)
         print(json.dumps({"prefill": {"value": round(2048 / pt, 1), "tokens": 2048, "ms": round(pt * 1e3, 3),

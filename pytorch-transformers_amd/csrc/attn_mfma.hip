@@ -16,9 +16,11 @@
 // key rows are assigned to the two 16-row score tiles so that a lane ends up with the eight
 // consecutive keys 8 * (lane / 16) .. + 7 of the block, which is what the B operand wants.
 //
-// Decoding splits a long context over several waves (split_size keys each, a function of the
-// context alone); each writes an unnormalised partial result with its running maximum and sum, and
-// attn_combine merges them in split order.  Prefill uses one wave per column group and no split.
+// Decoding splits a long context over several workgroups (split_size keys each); each writes an
+// unnormalised partial result with its running maximum and sum, and attn_combine merges them in split
+// order.  A workgroup is one wave, or four or eight that take its keys block by block in turn and merge
+// through LDS in the order of the waves; with the whole context in one workgroup there is no second
+// launch, but all of a sequence's keys then pass through one compute unit.  Prefill does not split.
 //
 // score = q . k / sqrt(d) + alibi, alibi = bf16(bf16(slope) * bf16(key position)) / sqrt(d)
 // (src/transformers/models/falcon/modeling_falcon.py:371-386, :407-422, :196-198, :1078-1085).
@@ -97,8 +99,10 @@ __device__ __forceinline__ void load_block(KvBlock<DT>& b, int kb, const int* __
 // W = 4 (prompts): four waves with neighbouring column groups walk the keys together and share every
 // block through LDS, so that a block crosses the vector memory path once for 64 * CT columns.
 // WIN: the launch has a window (a kernel of its own, so that launches without one pay nothing for it).
-template <int DT, int CT, int W, bool WIN>
-__global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
+// KS > 1 (one token per sequence): KS waves of a workgroup hold the same columns and take every KS-th block of the
+// workgroup's keys; their partial results meet in LDS, so that a context walked by KS waves needs no second launch.
+template <int DT, int CT, int W, bool WIN, int KS = 1>
+__global__ __launch_bounds__(64 * W * KS) void attn_mfma_kernel(
     bf16_t* __restrict__ out, float* __restrict__ po, float* __restrict__ pm, float* __restrict__ pl,
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
     const int* __restrict__ block_table, int bt_stride, const int* __restrict__ cu_tokens,
@@ -109,7 +113,10 @@ __global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
     const int window = WIN ? window_arg : 0;
     constexpr int DS = (DT + 1) / 2;   // 32-wide steps over the head dimension
     constexpr int CHUNKS = D / 8;      // 16-byte chunks in a row of d elements
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, gq = lane >> 4;
+    static_assert(KS == 1 || W == 1, "waves either share key blocks or divide them");
+    const int lane = threadIdx.x & 63, c = lane & 15, gq = lane >> 4;
+    const int wave = KS > 1 ? 0 : threadIdx.x >> 6;   // which columns of the workgroup
+    const int kw = KS > 1 ? threadIdx.x >> 6 : 0;     // which blocks of the keys
     const int seq = blockIdx.z / n_splits, split = blockIdx.z % n_splits;
     const int kvh = blockIdx.y, g = nh / nkv;
     const int t0 = cu_tokens[seq], n_new = cu_tokens[seq + 1] - t0, start = seq_start[seq];
@@ -280,18 +287,21 @@ __global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
         // has nothing else to hide the memory's latency behind).  Addresses past the last block are clamped to
         // it, and such a block is not used.
         constexpr int NB = DT <= 4 ? PTA_ATTN_DEPTH : 2;
+        constexpr int STEP = 32 * KS;  // from one block of this wave to its next
         KvBlock<DT> b[NB];
-        if (k_begin < k_end) {
+        const int k_first = k_begin + 32 * kw;
+        const int n_mine = k_first < k_end ? (k_end - k_first + STEP - 1) / STEP : 0;  // blocks of this wave
+        auto blk = [&](int j) { return j < n_mine ? min(k_first + STEP * j, kb_last) : kb_last; };
+        if (n_mine > 0) {
 #pragma unroll
-            for (int i = 0; i < NB - 1; ++i)
-                load_block<DT>(b[i], min(k_begin + 32 * i, kb_last), bt, k_pool, v_pool, nkv, kvh, c, gq);
+            for (int i = 0; i < NB - 1; ++i) load_block<DT>(b[i], blk(i), bt, k_pool, v_pool, nkv, kvh, c, gq);
         }
-        for (int kb = k_begin; kb < k_end; kb += 32 * NB) {
+        for (int j = 0; j < n_mine; j += NB) {
 #pragma unroll
             for (int i = 0; i < NB; ++i) {
-                load_block<DT>(b[(i + NB - 1) % NB], min(kb + 32 * (i + NB - 1), kb_last), bt, k_pool, v_pool, nkv, kvh, c, gq);
+                load_block<DT>(b[(i + NB - 1) % NB], blk(j + i + NB - 1), bt, k_pool, v_pool, nkv, kvh, c, gq);
                 __builtin_amdgcn_sched_barrier(0);
-                if (kb + 32 * i < k_end) use_block(b[i], kb + 32 * i);
+                if (j + i < n_mine) use_block(b[i], blk(j + i));
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -373,6 +383,63 @@ __global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
         }
     }
 
+    if constexpr (KS > 1) {
+        // every wave's sums, running maxima and unnormalised results go to LDS; then the (column tile, feature
+        // tile) pairs are dealt out to the waves, and each merges its pairs over the waves in their order
+        extern __shared__ __attribute__((aligned(16))) float ks_mem[];
+        float4* so = reinterpret_cast<float4*>(ks_mem);
+        float* sm = ks_mem + KS * CT * DT * 256;
+        float* sl = sm + KS * CT * 16;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            float l = l_run[ct];
+            l += __shfl_xor(l, 16, 64);
+            l += __shfl_xor(l, 32, 64);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+                so[((kw * CT + ct) * DT + dt) * 64 + lane] =
+                    make_float4(oacc[dt][ct][0], oacc[dt][ct][1], oacc[dt][ct][2], oacc[dt][ct][3]);
+            if (gq == 0) {
+                sm[(kw * CT + ct) * 16 + c] = m_run[ct];
+                sl[(kw * CT + ct) * 16 + c] = l;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                if ((ct * DT + dt) % KS != kw || qpos[ct] < 0) continue;
+                float mx = -INFINITY;
+#pragma unroll
+                for (int w = 0; w < KS; ++w) mx = fmaxf(mx, sm[(w * CT + ct) * 16 + c]);
+                float l = 0.f;
+                float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+                for (int w = 0; w < KS; ++w) {
+                    const float mw = sm[(w * CT + ct) * 16 + c];
+                    const float wgt = mw == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mw - mx);
+                    const float4 o = so[((w * CT + ct) * DT + dt) * 64 + lane];
+                    l += wgt * sl[(w * CT + ct) * 16 + c];
+                    acc.x += wgt * o.x; acc.y += wgt * o.y; acc.z += wgt * o.z; acc.w += wgt * o.w;
+                }
+                const long row = (long)tok[ct] * nh + head[ct];
+                if (n_splits == 1) {
+                    const float inv = 1.0f / l;
+                    uint2 w2;
+                    w2.x = pack_bf16(acc.x * inv, acc.y * inv);
+                    w2.y = pack_bf16(acc.z * inv, acc.w * inv);
+                    *reinterpret_cast<uint2*>(out + row * D + dt * 16 + gq * 4) = w2;
+                } else {
+                    *reinterpret_cast<float4*>(po + (row * n_splits + split) * D + dt * 16 + gq * 4) = acc;
+                    if (dt == 0 && gq == 0) {
+                        pm[row * n_splits + split] = mx;
+                        pl[row * n_splits + split] = l;
+                    }
+                }
+            }
+        }
+    } else {
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
         float l = l_run[ct];
@@ -406,6 +473,7 @@ __global__ __launch_bounds__(64 * W) void attn_mfma_kernel(
                 pl[row * n_splits + split] = l;
             }
         }
+    }
     }
     }  // pass
 }
@@ -456,32 +524,66 @@ struct AttnLaunch {
     int n_seqs, max_new, nh, nkv; float scale;
     int split_size, n_splits, window;
     int paired;  // workgroups take two column groups each, a late one and the early one that mirrors it
+    int waves;   // one token per sequence: waves of a workgroup that divide its keys among them
     hipStream_t s;
 };
 
-template <int DT, int CT, int W>
+// LDS in which KS waves of CT column tiles leave their partial results
+constexpr size_t key_split_lds(int dt, int ct, int ks) { return ks == 1 ? 0 : (size_t)ks * ct * (dt * 1024 + 128); }
+
+template <int DT, int CT, int W, int KS = 1>
 static void launch_attn(const AttnLaunch& a) {
     const int g = a.nh / a.nkv;
     const int groups = (a.max_new * g + 16 * CT * W - 1) / (16 * CT * W);
     const int paired = a.paired && groups > 1 ? 1 : 0;
     const dim3 grid(paired ? (groups + 1) / 2 : groups, a.nkv, a.n_seqs * a.n_splits);
-    auto kern = a.window > 0 ? attn_mfma_kernel<DT, CT, W, true> : attn_mfma_kernel<DT, CT, W, false>;
-    hipLaunchKernelGGL(kern, grid, dim3(64 * W), 0, a.s, a.out, a.po, a.pm, a.pl, a.q, a.k_pool, a.v_pool, a.block_table,
-                       a.bt_stride, a.cu_tokens, a.seq_start, a.slopes, a.alibi_exact, a.nh, a.nkv, a.scale * PTA_LOG2E,
-                       PTA_LOG2E / sqrtf((float)(DT * 16)), a.split_size, a.n_splits, a.window, paired);
+    auto kern = a.window > 0 ? attn_mfma_kernel<DT, CT, W, true, KS> : attn_mfma_kernel<DT, CT, W, false, KS>;
+    constexpr size_t lds = key_split_lds(DT, CT, KS);
+    if constexpr (lds > 64 * 1024) {  // more than a launch may ask for unless the kernel has been told, once per device
+        static bool told[64] = {};
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+        if (!told[dev]) {
+            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            told[dev] = true;
+        }
+    }
+    hipLaunchKernelGGL(kern, grid, dim3(64 * W * KS), lds, a.s, a.out, a.po, a.pm, a.pl, a.q, a.k_pool, a.v_pool,
+                       a.block_table, a.bt_stride, a.cu_tokens, a.seq_start, a.slopes, a.alibi_exact, a.nh, a.nkv,
+                       a.scale * PTA_LOG2E, PTA_LOG2E / sqrtf((float)(DT * 16)), a.split_size, a.n_splits, a.window, paired);
 }
 
 // column tiles (of sixteen query heads of one KV head) that one wave of a decode launch holds at most:
 // what the head size leaves registers for
 constexpr int decode_max_tiles(int dt) { return dt <= 4 ? 5 : dt <= 8 ? 4 : 1; }
 
-// one token per sequence: one wave per workgroup with `tiles` column tiles
-template <int DT, int CT = 1>
-static void launch_decode(const AttnLaunch& a, int tiles) {
-    if constexpr (CT <= decode_max_tiles(DT)) {
-        if (tiles == CT) launch_attn<DT, CT, 1>(a);
-        else launch_decode<DT, CT + 1>(a, tiles);
+// waves that may divide a workgroup's keys: one, or four or eight with up to two column tiles each (more tiles
+// gained nothing with more waves wherever that was measured, and every combination is a kernel to build)
+constexpr bool decode_waves_built(int dt, int ct, int ks) {
+    return ks == 1 || ((ks == 4 || ks == 8) && ct <= 2 && ct <= decode_max_tiles(dt) &&
+                       key_split_lds(dt, ct, ks) <= 144 * 1024);
+}
+
+template <int DT, int CT, int KS = 1>
+static bool launch_decode_waves(const AttnLaunch& a) {
+    if constexpr (KS <= 8) {
+        if (a.waves == KS) {
+            if constexpr (decode_waves_built(DT, CT, KS)) { launch_attn<DT, CT, 1, KS>(a); return true; }
+            return false;
+        }
+        return launch_decode_waves<DT, CT, KS * 2>(a);
     }
+    return false;
+}
+
+// one token per sequence: workgroups of `waves` waves with `tiles` column tiles
+template <int DT, int CT = 1>
+static bool launch_decode(const AttnLaunch& a, int tiles) {
+    if constexpr (CT <= decode_max_tiles(DT)) {
+        if (tiles == CT) return launch_decode_waves<DT, CT>(a);
+        return launch_decode<DT, CT + 1>(a, tiles);
+    }
+    return false;
 }
 
 // prompts: four waves of two column tiles share each key block through LDS (head sizes up to 128;
@@ -496,10 +598,15 @@ extern "C" int pta_attn_mfma_supported(int d) { return d % 16 == 0 && ((d >= 16 
 
 extern "C" int pta_attn_decode_max_tiles(int d) { return decode_max_tiles(d / 16); }
 
+extern "C" int pta_attn_decode_waves_ok(int d, int tiles, int waves) {
+    return pta_attn_mfma_supported(d) && tiles >= 1 && decode_waves_built(d / 16, tiles, waves);
+}
+
 extern "C" int pta_attn_mfma(void* out, const void* q, const void* k_pool, const void* v_pool, const int* block_table,
                              int bt_stride, const int* cu_tokens, const int* seq_start, const float* slopes, int alibi_exact,
                              int n_seqs, int max_new, int M, int nh, int nkv, int d, float scale, int split_size, int n_splits,
-                             float* po, float* pm, float* pl, int window, int decode_tiles, void* stream) {
+                             float* po, float* pm, float* pl, int window, int decode_tiles, int decode_waves,
+                             void* stream) {
     PTA_REQUIRE(n_seqs > 0 && max_new > 0 && M > 0 && nh > 0 && nkv > 0, "attn_mfma: sizes must be positive");
     PTA_REQUIRE(nh % nkv == 0, "attn_mfma: heads (%d) must be a multiple of kv heads (%d)", nh, nkv);
     PTA_REQUIRE(pta_attn_mfma_supported(d), "attn_mfma: head size %d is not built (16..128 in steps of 16, or 256)", d);
@@ -537,13 +644,17 @@ extern "C" int pta_attn_mfma(void* out, const void* q, const void* k_pool, const
                 "attn_mfma: %d column tiles per decode wave; these sizes allow 1..%d (0: as many as that)", decode_tiles,
                 dct_most);
     const int dct = decode_tiles > 0 ? decode_tiles : dct_most;
+    PTA_REQUIRE(!narrow || pta_attn_decode_waves_ok(d, dct, decode_waves),
+                "attn_mfma: %d waves on the keys of a workgroup with %d column tiles are not built for head size %d "
+                "(one wave, or four or eight with up to two tiles)", decode_waves, dct, d);
     const AttnLaunch a{(bf16_t*)out, po, pm, pl, (const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool,
                        block_table, bt_stride, cu_tokens, seq_start, slopes, alibi_exact, n_seqs, max_new, nh, nkv, scale,
-                       split_size, n_splits, window, paired, s};
+                       split_size, n_splits, window, paired, narrow ? decode_waves : 1, s};
 #define PTA_ATTN_CASE(DT_)                                        \
     case DT_:                                                     \
-        if (narrow) launch_decode<DT_>(a, dct);                   \
-        else launch_prompt<DT_>(a);                               \
+        if (!narrow) launch_prompt<DT_>(a);                       \
+        else if (!launch_decode<DT_>(a, dct))                     \
+            return pta_fail("attn_mfma: no kernel for %d waves and %d column tiles at head size %d", decode_waves, dct, d); \
         break;
     switch (d / 16) {
         PTA_ATTN_CASE(1)

@@ -14,7 +14,7 @@
 
 #include <stdint.h>
 
-#define PTA_ABI_VERSION 3
+#define PTA_ABI_VERSION 4
 
 #ifdef __cplusplus
 extern "C" {
@@ -72,10 +72,13 @@ int pta_attn_generic(void* out, const void* q, const void* k_pool, const void* v
 int pta_attn_mfma_supported(int d);
 // Column tiles (sixteen query heads of one KV head) that one wave of a decode launch can hold at this head size.
 int pta_attn_decode_max_tiles(int d);
+// decode_waves (max_new == 1): waves of a workgroup that take its range of keys block by block in turn and merge
+// their results in LDS (1, 4 or 8; pta_attn_decode_waves_ok says whether the combination with decode_tiles is built).
+int pta_attn_decode_waves_ok(int d, int tiles, int waves);
 int pta_attn_mfma(void* out, const void* q, const void* k_pool, const void* v_pool, const int* block_table,
                   int bt_stride, const int* cu_tokens, const int* seq_start, const float* slopes, int alibi_exact,
                   int n_seqs, int max_new, int M, int nh, int nkv, int d, float scale, int split_size, int n_splits, float* po,
-                  float* pm, float* pl, int window, int decode_tiles, void* stream);
+                  float* pm, float* pl, int window, int decode_tiles, int decode_waves, void* stream);
 
 // C = act(A . W^T + bias) + add1 + add2, all 32-bit, fixed summation order
 int pta_gemm_f32(float* C, const float* A, const float* W, const float* bias, const float* add1, const float* add2,

@@ -14,6 +14,7 @@ from typing import Dict, Optional, Sequence
 
 import ctypes
 import gc
+import os
 import weakref
 
 import numpy as np
@@ -283,10 +284,14 @@ class CausalLM:
 
     # timed choices ---------------------------------------------------------------
     @torch.no_grad()
-    def tune(self, prompt_lens: Sequence[int] = (2048,), batches: Sequence[int] = (8, 64), table=None) -> dict:
+    def tune(self, prompt_lens: Sequence[int] = (2048,), batches: Sequence[int] = (8, 64), table=None,
+             contexts: Sequence = ()) -> dict:
         """Time, once, the choices between kernels that no rule decides, for prompts of ``prompt_lens`` tokens and
         decode steps of ``batches`` sequences, and keep them for every later step of this process; returns the
-        table (``ops.tuning_table``).  With ``table`` given nothing is timed: its choices are taken instead.
+        table (``ops.tuning_table``).  With ``contexts`` the decode steps are also run at these context lengths,
+        each a number or a pair (longest, mean of the batch), over a cache that holds whatever it holds (only times
+        are taken): that is where the cut of the decode attention is timed.  With ``table`` given nothing is
+        timed: its choices are taken instead.
         Steps never time anything by themselves (unless PTA_TUNE=1 is set): untuned, they take the built-in
         choice, and logits are the same bits in every process."""
         from .. import ops
@@ -297,24 +302,92 @@ class CausalLM:
         if self.dtype != torch.bfloat16:
             return ops.tuning_table()  # the 32-bit path has one kernel per operation
         graphs, self.use_graphs = self.use_graphs, False  # nothing can be timed inside a capture
-        need = max([int(t) for t in prompt_lens] + [0]) + 64 * max([int(b) for b in batches] + [1]) + 64
+        page = self.page_size
+        pairs = sorted({(int(c), int(c)) if isinstance(c, int) else (int(c[0]), int(c[1])) for c in contexts})
+        most = max([int(b) for b in batches] + [1])
+        need = max([int(t) for t in prompt_lens] + [0]) + 64 * most + 64
+        need = max(need, most * ((max([c[0] for c in pairs] + [0]) + page) // page * page))
         cache = self.new_cache(need)
+        timed: set = set()  # decode launches whose cuts have been timed in this call
         try:
             with ops.live_tuning():
                 for T in prompt_lens:
                     slot = cache.alloc()
                     self.step(cache, [slot], [[0] * int(T)], "last")
                     cache.free(slot)
-                for b in batches:
-                    slots = [cache.alloc() for _ in range(int(b))]
-                    self.step(cache, slots, [[0]] * int(b), "last")  # one token each: the shape of a decode step
-                    for s_ in slots:
-                        cache.free(s_)
+                for b in (int(b) for b in batches):
+                    # one token each: the shape of a decode step; then the same with tokens before it in every
+                    # sequence, one sequence as long as the longest and the others such that the mean comes out
+                    for longest, mean in [(1, 1)] + pairs:
+                        rest = longest if b == 1 else max(1, min(longest, (mean * b - longest) // (b - 1)))
+                        before = [longest - 1] + [rest - 1] * (b - 1)
+                        slots = [cache.alloc() for _ in range(b)]
+                        grow = [(s_, n_) for s_, n_ in zip(slots, before) if n_ > 0]
+                        if grow:
+                            cache.reserve([s_ for s_, _ in grow], [n_ for _, n_ in grow])
+                            cache.commit([s_ for s_, _ in grow], [n_ for _, n_ in grow])
+                        ops.take_decode_keys()
+                        self.step(cache, slots, [[0]] * b, "last")
+                        if longest > 1 and graphs and os.environ.get("PTA_DECODE_TUNE", "1") != "0":
+                            self._time_decode_cuts(cache, slots, timed)
+                        for s_ in slots:
+                            cache.free(s_)
             torch.cuda.synchronize()
         finally:
             self.use_graphs = graphs
             ops.release_flush()
         return ops.tuning_table()
+
+    def _time_decode_cuts(self, cache: PagedCache, slots: Sequence[int], timed: set, replays: int = 8,
+                          rounds: int = 3) -> None:
+        """For the decode launches of the step that was just run with timing on: capture the next step of these
+        sequences once per candidate cut of the attention and keep the cut whose replays are fastest, if it beats
+        the rule's by more than noise.  Whole steps are timed because a cut's time alone, after a flush of the
+        caches, does not rank the cuts as a step does.  Nothing is committed: every replay writes the same
+        position again."""
+        from .. import ops
+
+        keys = ops.take_decode_keys()
+        if not keys:
+            return
+        b = len(slots)
+        plan = plan_step(cache, slots, [[0]] * b, "last", self.vocab_size)
+        n_bucket = b if b <= 8 else (b + 7) // 8 * 8
+        len_bound = _len_bound(plan.max_len)
+        mean_bound = mean_len_bound(plan.total_len, b, len_bound)
+
+        def step_ms() -> float:
+            g = _DecodeGraph(self, cache, n_bucket, len_bound, mean_bound)
+            g._fill(plan)
+            g._launch()  # directly, then captured
+            g._launch()
+            best = float("inf")
+            for _ in range(rounds):
+                start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                start.record()
+                for _ in range(replays):
+                    g._launch()
+                end.record()
+                end.synchronize()
+                best = min(best, start.elapsed_time(end) / replays)
+            return best
+
+        for key in keys:
+            if key in timed:
+                continue
+            timed.add(key)
+            cuts = ops.decode_plan_candidates(key)
+            times = []
+            for cut in cuts:
+                ops.set_decode_plan(key, cut)
+                times.append(step_ms())
+            best = min(range(len(cuts)), key=lambda i: times[i])
+            chosen = cuts[best] if times[best] < 0.985 * times[0] else None
+            ops.set_decode_plan(key, chosen)
+            if os.environ.get("PTA_TUNE_VERBOSE"):
+                print(f"[pta tune] decode attention {key}: " + " ".join(f"{c}:{t:.3f}" for c, t in zip(cuts, times))
+                      + f" ms a step -> {chosen or cuts[0]}", flush=True)
+        ops.take_decode_keys()  # the steps above asked too
 
     # cache -------------------------------------------------------------------
     @property

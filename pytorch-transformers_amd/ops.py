@@ -24,7 +24,7 @@ QKV_LAYOUT_CODES = {"grouped": 0, "tail": 1, "interleaved": 2}
 ACT_CODES = {None: 0, "none": 0, "linear": 0, "gelu": 1, "gelu_python": 1, "gelu_new": 2, "gelu_pytorch_tanh": 2,
              "gelu_fast": 2, "gelu_accurate": 2, "quick_gelu": 3, "relu": 4, "relu2": 5, "relu6": 6, "silu": 7, "swish": 7,
              "sigmoid": 8, "tanh": 9, "leaky_relu": 10, "mish": 11, "gelu_10": 12, "laplace": 13}
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 _lib = None
 _lock = threading.Lock()
@@ -360,7 +360,7 @@ def attn_mfma_ok(q: torch.Tensor) -> bool:
 
 def attn_mfma(q: torch.Tensor, k_pool, v_pool, block_table, cu_tokens, seq_start, slopes, scale: float, *,
               max_new: int, n_splits: int = 1, split_size: int = ATTN_SPLIT_KEYS, window: int = 0,
-              decode_tiles: int = 0, alibi_exact: bool = False) -> torch.Tensor:
+              decode_tiles: int = 0, decode_waves: int = 1, alibi_exact: bool = False) -> torch.Tensor:
     """Causal attention of a step's tokens over the cache on the matrix cores; out [M, nh*d].
 
     ``max_new`` bounds the new tokens of any sequence of the step; with ``n_splits > 1`` the keys
@@ -386,7 +386,8 @@ def attn_mfma(q: torch.Tensor, k_pool, v_pool, block_table, cu_tokens, seq_start
     _call("pta_attn_mfma", _ptr(out), _ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(block_table), block_table.shape[1],
           _ptr(cu_tokens), _ptr(seq_start), _ptr(slopes), int(bool(alibi_exact)), n_seqs, int(max_new), M, nh, nkv, d,
           ctypes.c_float(scale),
-          int(split_size), int(n_splits), _ptr(po), _ptr(pm), _ptr(pl), int(window), int(decode_tiles), _stream())
+          int(split_size), int(n_splits), _ptr(po), _ptr(pm), _ptr(pl), int(window), int(decode_tiles), int(decode_waves),
+          _stream())
     return out
 
 
@@ -443,21 +444,81 @@ def _decode_plan(n: int, n_heads: int, n_kv_heads: int, head_dim: int, bound: in
     return best[1], best[2]
 
 
-def decode_plan(n_seqs: int, n_heads: int, n_kv_heads: int, head_dim: int, max_len: int, mean_len: int = 0):
-    """How a decode launch is cut: (column tiles per wave, keys per wave); a size that covers the
-    context means one wave per sequence and head group, which writes the result itself.
+_decode_plans: dict = {}  # (batch, heads, KV heads, head size, longest, mean) as counted below -> a timed cut
 
-    The batch counts by its next power of two, the longest context by its next multiple of 1,024 and the
-    mean context (``mean_len``; 0: as the longest) by its next multiple of 512, so that a captured step,
-    which is sized for a padded batch and such bounds, is cut exactly as the same step run directly."""
+
+def _decode_key(n_seqs: int, n_heads: int, n_kv_heads: int, head_dim: int, max_len: int, mean_len: int):
     n = 1
     while n < n_seqs:
         n *= 2
     bound = (max_len + 1023) // 1024 * 1024
+    mean = min(bound, (mean_len + 511) // 512 * 512) if mean_len > 0 else bound
+    return (n, int(n_heads), int(n_kv_heads), int(head_dim), bound, mean)
+
+
+def decode_plan(n_seqs: int, n_heads: int, n_kv_heads: int, head_dim: int, max_len: int, mean_len: int = 0):
+    """How a decode launch is cut: (column tiles per wave, keys per workgroup, waves per workgroup); a size that
+    covers the context means one workgroup per sequence and head group, which writes the result itself.  The
+    waves of a workgroup take its keys block by block in turn and merge in LDS.
+
+    The batch counts by its next power of two, the longest context by its next multiple of 1,024 and the
+    mean context (``mean_len``; 0: as the longest) by its next multiple of 512, so that a captured step,
+    which is sized for a padded batch and such bounds, is cut exactly as the same step run directly.
+    A cut that was fixed for these counts (``set_decode_plan``; ``CausalLM.tune`` times whole steps with the cuts
+    of ``decode_plan_candidates``) goes before the rule, which has one wave per workgroup."""
+    key = _decode_key(n_seqs, n_heads, n_kv_heads, head_dim, max_len, mean_len)
+    kept = _decode_plans.get(key)
+    if kept is not None:
+        return kept
+    n, _, _, _, bound, mean = key
     groups = (n_heads // n_kv_heads + 15) // 16
     most = min(groups, int(load_library().pta_attn_decode_max_tiles(head_dim)))
-    mean = min(bound, (mean_len + 511) // 512 * 512) if mean_len > 0 else bound
-    return _decode_plan(n, n_heads, n_kv_heads, head_dim, bound, mean, most)
+    return _decode_plan(n, n_heads, n_kv_heads, head_dim, bound, mean, most) + (1,)
+
+
+_decode_keys_seen: set = set()  # what decode launches asked ``decode_plan`` for while timing was on
+
+
+def take_decode_keys() -> list:
+    """The (batch, head shape, context) counts of the decode launches since the last call, while timing was on."""
+    keys = sorted(_decode_keys_seen)
+    _decode_keys_seen.clear()
+    return keys
+
+
+def decode_plan_candidates(key) -> list:
+    """Cuts of the decode launch that ``key`` counts, the rule's first: its neighbours with one wave per
+    workgroup, and workgroups of four and eight waves over the whole context and over ranges of 512 and 1,024
+    keys.  A workgroup of several waves needs no second launch when it walks the whole context, but all its keys
+    pass through one compute unit; which wins depends on how many sequences and KV heads there are to fill the
+    chip.  Timed alone after a flush of the caches, these cuts rank differently than inside a step (the rule's
+    cut at 64 sequences, 8 KV heads of 64 and 1,100 keys: 42 us alone, 31 us in a step, where a cut with four
+    waves takes 34 us both times), so the caller times whole steps with each (``CausalLM.tune``)."""
+    n, nh, nkv, d, bound, mean = key
+    lib = load_library()
+    groups = (nh // nkv + 15) // 16
+    most = min(groups, int(lib.pta_attn_decode_max_tiles(d)))
+    rule = _decode_plan(n, nh, nkv, d, bound, mean, most) + (1,)
+    cuts = [rule]
+    want = [(rule[0], rule[1] * 2, 1), (rule[0], rule[1] // 2, 1), (max(1, rule[0] - 1), rule[1], 1),
+            (min(most, rule[0] + 1), rule[1], 1)]
+    want += [(t, size, w) for t in (1, min(2, most)) for w in (4, 8) for size in (bound, 1024, 512)]
+    for t, size, w in want:
+        size = min(size, bound)
+        splits = (bound + size - 1) // size
+        if (size < ATTN_SPLIT_KEYS or size % 64 or size // w < 64 or splits > 1024 or n * splits > 65535 or (t, size, w) in cuts
+                or not lib.pta_attn_decode_waves_ok(d, t, w)):
+            continue
+        cuts.append((t, size, w))
+    return cuts
+
+
+def set_decode_plan(key, cut=None) -> None:
+    """Fix the cut of the decode launches that ``key`` counts (None: back to the rule)."""
+    if cut is None:
+        _decode_plans.pop(tuple(key), None)
+    else:
+        _decode_plans[tuple(key)] = tuple(int(v) for v in cut)
 
 
 def attention(q: torch.Tensor, k_pool, v_pool, block_table, ctx, slopes, scale: float, window: int = 0,
@@ -468,14 +529,17 @@ def attention(q: torch.Tensor, k_pool, v_pool, block_table, ctx, slopes, scale: 
     split over several waves when every sequence brings one token; anything else: the 32-bit
     kernel."""
     if attn_mfma_ok(q):
-        n_splits, size, tiles = 1, ATTN_SPLIT_KEYS, 0
+        n_splits, size, tiles, waves = 1, ATTN_SPLIT_KEYS, 0, 1
         if ctx.is_decode:
-            tiles, size = decode_plan(ctx.n_seqs, q.shape[1], k_pool.shape[1], q.shape[2], ctx.max_len,
-                                      getattr(ctx, "mean_len", 0))
+            if window == 0 and _may_time():
+                _decode_keys_seen.add(_decode_key(ctx.n_seqs, q.shape[1], k_pool.shape[1], q.shape[2], ctx.max_len,
+                                                  getattr(ctx, "mean_len", 0)))
+            tiles, size, waves = decode_plan(ctx.n_seqs, q.shape[1], k_pool.shape[1], q.shape[2], ctx.max_len,
+                                             getattr(ctx, "mean_len", 0))
             n_splits = (ctx.max_len + size - 1) // size
         return attn_mfma(q, k_pool, v_pool, block_table, ctx.cu_tokens, ctx.seq_start, slopes, scale,
                          max_new=max(ctx.new_tokens), n_splits=n_splits, split_size=size, window=window,
-                         decode_tiles=tiles, alibi_exact=alibi_exact)
+                         decode_tiles=tiles, decode_waves=waves, alibi_exact=alibi_exact)
     return attn_generic(q, k_pool, v_pool, block_table, ctx.token_seq, ctx.token_pos, slopes, scale, window, alibi_exact)
 
 
@@ -565,7 +629,7 @@ SPLITK_SURE_ROWS = 128  # up to here the kernel won at every shape measured; bey
 _splitk_limits: dict = {}  # (N, K) -> rows up to which the batch kernel beats the library's product
 
 
-_flush = None  # half a gigabyte that is written between timed runs; held only while timing is on (``release_flush``)
+_flush = None  # half a gigabyte that is read between timed runs; held only while timing is on (``release_flush``)
 
 
 def release_flush() -> None:
@@ -575,18 +639,22 @@ def release_flush() -> None:
 
 def _time_ways_cold(ways, device, rounds: int = 3):
     """Milliseconds of each of ``ways`` (callables), the fastest of ``rounds`` runs each, taken in turn; before
-    every run half a gigabyte is written, so that the weights come from memory as they do in a model (timed back
-    to back, a product finds its matrix in the memory-side cache and every way looks alike)."""
+    every run half a gigabyte is read, so that the weights come from memory as they do in a model (timed back
+    to back, a product finds its matrix in the memory-side cache and every way looks alike).  Read, not
+    written: after half a gigabyte of writes the caches are full of lines that must go back to memory before
+    anything else comes in, which no step of a model leaves behind, and a kernel that streams from memory then
+    measures at little more than half its speed (decode attention over 144 MB of keys and values: 55 us after
+    writes, 31 us in a step)."""
     global _flush
     if _flush is None or _flush.device != device:
-        _flush = torch.empty(128 * 1024 * 1024, dtype=torch.float32, device=device)
+        _flush = torch.zeros(128 * 1024 * 1024, dtype=torch.float32, device=device)
     flush = _flush
     best = [float("inf")] * len(ways)
     for run in ways:  # plans are made and the library set up before anything is timed
         run()
     for _ in range(rounds):
         for i, run in enumerate(ways):
-            flush.fill_(1.0)
+            flush.sum()
             start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             start.record()
             run()
@@ -1004,6 +1072,7 @@ def tuning_table() -> dict:
         "mm_plans": {key(k): list(v) for k, v in _mm_plans.items()},
         "mm_joined": {key(k): bool(v) for k, v in _mm_joined.items()},
         "mm_ksplit": {key(k): int(v) for k, v in _mm_ksplit.items()},
+        "decode_plans": {key(k): list(v) for k, v in _decode_plans.items()},  # tiles, keys per workgroup, waves
     }
 
 
@@ -1012,7 +1081,7 @@ def clear_tuning() -> None:
     lib = load_library()
     for (s1, s2) in list(_pair_parts_tuned):
         lib.pta_gemm_splitk_pair_fix(int(s1[0]), int(s1[1]), int(s2[0]), int(s2[1]), 0, 0, 1)
-    for d in (_pair_parts_tuned, _splitk_limits, _mm_plans, _mm_costs, _mm_times, _mm_joined, _mm_ksplit):
+    for d in (_pair_parts_tuned, _splitk_limits, _mm_plans, _mm_costs, _mm_times, _mm_joined, _mm_ksplit, _decode_plans):
         d.clear()
 
 
@@ -1036,6 +1105,8 @@ def load_tuning(table: dict) -> None:
         _mm_joined[flat(k)] = bool(v)
     for k, v in table.get("mm_ksplit", {}).items():
         _mm_ksplit[flat(k)] = int(v)
+    for k, v in table.get("decode_plans", {}).items():
+        _decode_plans[flat(k)] = tuple(int(p) for p in v)
 
 
 def gemm_splitk_pair_parts_rule(N1: int, K1: int, N2: int, K2: int):

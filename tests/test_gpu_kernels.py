@@ -670,7 +670,7 @@ def test_attn_generic_far_key_and_alibi(dtype):
         _attn_case(ops, _generic(ops), dtype, nh, nh, 16, starts=[0, 290], news=[40, 30], slopes=slopes)
 
 
-def _mfma(ops, n_splits_for=None, tiles=0):
+def _mfma(ops, n_splits_for=None, tiles=0, waves=1):
     def fn(q, k_pool, v_pool, bt, token_seq, token_pos, slopes, scale, starts, news, window=0):
         cu = torch.tensor([0] + list(torch.tensor(news).cumsum(0)), dtype=torch.int32).cuda()
         st = torch.tensor(starts, dtype=torch.int32).cuda()
@@ -678,7 +678,7 @@ def _mfma(ops, n_splits_for=None, tiles=0):
         if n_splits_for is not None:
             n_splits = (max(s + n for s, n in zip(starts, news)) + n_splits_for - 1) // n_splits_for
         return ops.attn_mfma(q, k_pool, v_pool, bt, cu, st, slopes, scale, max_new=max(news), n_splits=n_splits,
-                             split_size=n_splits_for or 256, window=window, decode_tiles=tiles)
+                             split_size=n_splits_for or 256, window=window, decode_tiles=tiles, decode_waves=waves)
     return fn
 
 
@@ -718,6 +718,41 @@ def test_attn_mfma_decode_tiles(nh, nkv, d, tiles):
         _attn_case(ops, _mfma(ops, None, most + 1), torch.bfloat16, nh, nkv, d, starts=[5], news=[1])
 
 
+@pytest.mark.parametrize("nh,nkv,d,tiles", [(71, 1, 64, 1), (71, 1, 64, 2), (6, 2, 32, 1), (3, 3, 16, 1), (32, 8, 128, 1),
+                                            (40, 2, 128, 2), (17, 1, 256, 1), (5, 5, 48, 1), (20, 1, 80, 2), (9, 3, 112, 1)])
+@pytest.mark.parametrize("waves", [4, 8])
+def test_attn_mfma_decode_waves(nh, nkv, d, tiles, waves):
+    """One token per sequence, a workgroup of four or eight waves that take the keys block by block in turn and
+    merge in LDS: the whole context in one workgroup (no second launch), and ranges of 256 and 512 keys merged
+    afterwards as well; contexts shorter than the waves have blocks for, page edges, ALiBi, a window, and one
+    far key that must dominate whichever wave it falls to."""
+    ops = _ops()
+    from pytorch_transformers_amd.parts import AlibiPositions
+    assert ops.load_library().pta_attn_decode_waves_ok(d, tiles, waves)
+    starts = [0, 63, 64, 700, 255, 256, 1, 31, 32, 1500]
+    boost = [0, 40, None, 333, None, 17, None, None, 31, 1203]
+    for split in (None, 256, 512):
+        _attn_case(ops, _mfma(ops, split, tiles, waves), torch.bfloat16, nh, nkv, d, starts=starts, news=[1] * 10, boost=boost)
+    slopes = AlibiPositions(nh).slopes.cuda()
+    _attn_case(ops, _mfma(ops, None, tiles, waves), torch.bfloat16, nh, nkv, d, starts=starts, news=[1] * 10, slopes=slopes)
+    for window in (33, 100):
+        for split in (None, 256):
+            _attn_case(ops, _mfma(ops, split, tiles, waves), torch.bfloat16, nh, nkv, d, starts=starts, news=[1] * 10,
+                       window=window)
+
+
+def test_attn_mfma_decode_waves_refusals():
+    ops = _ops()
+    lib = ops.load_library()
+    assert not lib.pta_attn_decode_waves_ok(64, 3, 4) and not lib.pta_attn_decode_waves_ok(64, 1, 2)
+    assert not lib.pta_attn_decode_waves_ok(64, 1, 16) and lib.pta_attn_decode_waves_ok(64, 5, 1)
+    assert not lib.pta_attn_decode_waves_ok(256, 2, 4) and lib.pta_attn_decode_waves_ok(256, 1, 8)
+    with pytest.raises(ops.KernelError, match="waves on the keys of a workgroup"):
+        _attn_case(ops, _mfma(ops, None, 3, 4), torch.bfloat16, 71, 1, 64, starts=[5], news=[1])
+    with pytest.raises(ops.KernelError, match="waves on the keys of a workgroup"):
+        _attn_case(ops, _mfma(ops, None, 1, 2), torch.bfloat16, 71, 1, 64, starts=[5], news=[1])
+
+
 def test_decode_plan():
     """The cut of a decode launch: whole tiles within what the head size allows, a range size that is a
     multiple of the page, the same for every batch and context of one captured step's bucket."""
@@ -726,14 +761,14 @@ def test_decode_plan():
         groups = (nh // nkv + 15) // 16
         for n in (1, 3, 8, 33, 64, 128, 300, 512):
             for length in (1, 100, 1024, 1025, 2049, 8192, 32768, 65536, 100000):
-                tiles, size = ops.decode_plan(n, nh, nkv, d, length)
-                assert 1 <= tiles <= groups and size % 64 == 0 and size >= 128
+                tiles, size, waves = ops.decode_plan(n, nh, nkv, d, length)
+                assert 1 <= tiles <= groups and size % 64 == 0 and size >= 128 and waves == 1  # the rule: one wave
                 assert (length + size - 1) // size <= 1024
                 bucket_n = 1 << (n - 1).bit_length()
                 # the launch has one workgroup row per (sequence of the padded batch, range): the grid's limit
                 assert bucket_n * ((((length + 1023) // 1024 * 1024) + size - 1) // size) <= 65535
                 bucket_len = (length + 1023) // 1024 * 1024
-                assert (tiles, size) == ops.decode_plan(bucket_n, nh, nkv, d, bucket_len)
+                assert (tiles, size, 1) == ops.decode_plan(bucket_n, nh, nkv, d, bucket_len)
                 for mean in (1, length // 3 + 1, length):
                     cut = ops.decode_plan(n, nh, nkv, d, length, mean)
                     assert cut == ops.decode_plan(bucket_n, nh, nkv, d, bucket_len, min(bucket_len, (mean + 511) // 512 * 512))
@@ -779,8 +814,36 @@ def test_decode_attention_as_planned(nh, nkv, d, n, lengths):
     assert float((got - want).abs().max()) <= 2e-2 * max(1.0, float(want.abs().max()))
     far = v_pool[int(bt[0, 0]), :, :, 5].float().repeat_interleave(nh // nkv, 0).reshape(-1)
     assert float((got[0] - far).abs().max()) < 0.05, "the far key does not dominate"
-    tiles, size = ops.decode_plan(n, nh, nkv, d, ctx.max_len, ctx.mean_len)
-    assert 1 <= tiles <= (nh // nkv + 15) // 16 and size % 64 == 0
+    tiles, size, waves = ops.decode_plan(n, nh, nkv, d, ctx.max_len, ctx.mean_len)
+    assert 1 <= tiles <= (nh // nkv + 15) // 16 and size % 64 == 0 and waves == 1
+    # the same launch with every other cut that may be timed against the rule's: the same result within rounding;
+    # a fixed cut holds for the step's bucket and for no other, travels in the tuning table, and is forgotten with it
+    key = ops._decode_key(n, nh, nkv, d, ctx.max_len, ctx.mean_len)
+    cuts = ops.decode_plan_candidates(key)
+    assert cuts[0] == (tiles, size, 1) and len(set(cuts)) == len(cuts) > 3 and any(c[2] > 1 for c in cuts)
+    try:
+        with ops.live_tuning():
+            ops.take_decode_keys()
+            ops.attention(q, k_pool, v_pool, bt.cuda(), ctx, None, scale)
+            assert ops.take_decode_keys() == [key] and ops.take_decode_keys() == []
+        for cut in cuts[1:]:
+            assert ops.load_library().pta_attn_decode_waves_ok(d, cut[0], cut[2]) and cut[1] % 64 == 0
+            ops.set_decode_plan(key, cut)
+            assert ops.decode_plan(n, nh, nkv, d, ctx.max_len, ctx.mean_len) == cut
+            fixed = ops.attention(q, k_pool, v_pool, bt.cuda(), ctx, None, scale).float()
+            assert float((fixed - want).abs().max()) <= 2e-2 * max(1.0, float(want.abs().max())), cut
+            assert float((fixed[0] - far).abs().max()) < 0.05, cut
+        assert ops.decode_plan(n, nh, nkv, d, ctx.max_len + 2048, ctx.mean_len)[2] == 1  # another bucket: the rule
+        table = ops.tuning_table()
+        assert table["decode_plans"][",".join(str(v) for v in key)] == list(cuts[-1])
+        ops.clear_tuning()
+        assert ops.decode_plan(n, nh, nkv, d, ctx.max_len, ctx.mean_len) == cuts[0]
+        ops.load_tuning(table)
+        assert ops.decode_plan(n, nh, nkv, d, ctx.max_len, ctx.mean_len) == cuts[-1]
+        ops.set_decode_plan(key, None)
+        assert ops.decode_plan(n, nh, nkv, d, ctx.max_len, ctx.mean_len) == cuts[0]
+    finally:
+        ops.clear_tuning()
 
 
 @pytest.mark.parametrize("window", [1, 33, 64, 100, 200])

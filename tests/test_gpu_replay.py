@@ -308,6 +308,39 @@ def test_steps_time_nothing_unless_asked_and_a_table_carries_the_choices(folders
     helpers.assert_close(tuned, before, 2e-2, "tuned against untuned logits")
 
 
+def test_tune_times_whole_steps_with_each_cut_of_the_decode_attention(folders):
+    """``tune(contexts=...)`` replays captured decode steps at those contexts once per candidate cut of the attention
+    and leaves every bucket either at the rule's cut or at a candidate.  Decoding with every candidate fixed by hand
+    still matches the plain implementation, and forgetting the table restores the untuned bits."""
+    from pytorch_transformers_amd import AutoModelForCausalLM, ops
+    from pytorch_transformers_amd.engine.replay import Replayer
+
+    name = "C"
+    ops.clear_tuning()
+    model = AutoModelForCausalLM.from_pretrained(folders[name], dtype="bfloat16")
+    reqs = helpers.make_requests(TINY[name]["vocab_size"], [700], seed=11)
+    records = helpers.schedule_tail(reqs, 40)
+    want = helpers.plain_logits(folders[name], reqs)
+    run = lambda: helpers.run_schedule(Replayer(model, 1024), records)["r0"]
+    before = run()
+    helpers.assert_close(before, want["r0"], REL_BF16, "untuned")
+    try:
+        table = model.tune(prompt_lens=(), batches=(1, 3), contexts=(690, (700, 300)))
+        for k, cut in table["decode_plans"].items():
+            assert tuple(cut) in ops.decode_plan_candidates(tuple(int(v) for v in k.split(",")))[1:]
+        assert ops.take_decode_keys() == [] and ops._flush is None
+        cfg = model.config
+        key = ops._decode_key(1, cfg.num_attention_heads, cfg.kv_heads, cfg.head_dim, 700, 700)
+        cuts = ops.decode_plan_candidates(key)
+        assert any(c[2] > 1 for c in cuts)
+        for cut in cuts:
+            ops.set_decode_plan(key, cut)
+            helpers.assert_close(run(), want["r0"], REL_BF16, f"cut {cut}")
+    finally:
+        ops.clear_tuning()
+    assert torch.equal(run(), before)
+
+
 def test_logits_of_a_step_outlive_the_next_step(folders):
     """What ``step`` returns is the caller's: the next step, replayed from the same captured graph, writes a
     buffer of its own."""
