@@ -533,24 +533,88 @@ static int pick_pair_parts(int N1, int K1, int N2, int K2, int* p1, int* p2) {
     return 1;
 }
 
-extern "C" int pta_gemm_splitk_pair_parts(int N1, int K1, int N2, int K2, int* p1, int* p2) {
-    if (N1 <= 0 || K1 <= 0 || N2 <= 0 || K2 <= 0) return pta_fail("gemm_splitk_pair_parts: sizes must be positive");
-    pick_pair_parts(N1, K1, N2, K2, p1, p2);
+// Steps of 17 to 64 rows may run with the activations stationary (gemm_stationary_bf16.hip), which cuts K into
+// ranges of its own: few and long, since its workgroups are as many as the compute units whatever the ranges.
+// The rule: ranges about as long as the shorter K of the pair (between 2,048 and 8,192 elements), from 49 rows on.
+// Measured against the staged kernel at 64 rows, pairs of K = 4,544 with N = 4,672 + 18,176 and K = 4,544 +
+// 18,176 with N = 4,544: 51.8 against 58.2 us and 51.2 against 57.5 us; K = 4,096 / 16,384: 48.3 against 51.7 and
+// 44.7 against 53.9; K = 8,192 / 32,768: 155 against 179 and 157 against 171.  At 40 rows the two are within 5 % of
+// each other either way (three shapes of six go to each), at 32 rows the staged kernel wins.
+#define STATIONARY_FROM_ROWS 49
+#define STATIONARY_MAX_ROWS 64
+struct StationaryChoice { int q1, q2, from; };
+static std::map<std::array<int, 4>, StationaryChoice> pair_stationary_fixed;
+
+static StationaryChoice stationary_rule(int K1, int K2) {
+    const int target = max(2048, min(8192, min(K1, K2)));
+    auto parts = [&](int K) { return effective_parts(K, max(1, min(16, (K + target / 2) / target))); };
+    return {parts(K1), parts(K2), STATIONARY_FROM_ROWS};
+}
+
+// Fixes, for every later pair launch of this shape with from_rows to 64 rows, the ranges of K of the launch with
+// stationary activations (from_rows 17 to 65; 65: never that launch).  q1 = q2 = 0 forgets the shape.  Returns 1
+// (no error text) for counts that the kernel does not take.
+extern "C" int pta_gemm_splitk_pair_fix_stationary(int N1, int K1, int N2, int K2, int q1, int q2, int from_rows) {
+    if (N1 <= 0 || K1 <= 0 || N2 <= 0 || K2 <= 0) return 1;
+    std::lock_guard<std::mutex> hold(pair_parts_lock);
+    const std::array<int, 4> key{N1, K1, N2, K2};
+    if (q1 == 0 && q2 == 0) {
+        pair_stationary_fixed.erase(key);
+        return 0;
+    }
+    if (q1 < 1 || q2 < 1 || q1 > 16 || q2 > 16 || effective_parts(K1, q1) != q1 || effective_parts(K2, q2) != q2 ||
+        from_rows < 17 || from_rows > STATIONARY_MAX_ROWS + 1)
+        return 1;
+    pair_stationary_fixed[key] = {q1, q2, from_rows};
+    return 0;
+}
+
+// The ranges of a pair launch of M rows and its kind: 3 with stationary activations, else the tiles of sixteen
+// rows of W per wave of the staged kernel (1 or 2).  M = 0 asks for the staged kernel's ranges.
+static int pick_pair_parts_rows(int N1, int K1, int N2, int K2, int M, int* p1, int* p2) {
+    if (M > 16 && M <= STATIONARY_MAX_ROWS && K1 % 8 == 0 && K2 % 8 == 0) {
+        StationaryChoice c = stationary_rule(K1, K2);
+        {
+            std::lock_guard<std::mutex> hold(pair_parts_lock);
+            const auto it = pair_stationary_fixed.find({N1, K1, N2, K2});
+            if (it != pair_stationary_fixed.end()) c = it->second;
+        }
+        if (M >= c.from) {
+            *p1 = c.q1;
+            *p2 = c.q2;
+            return 3;
+        }
+    }
+    const int rt = pick_pair_parts(N1, K1, N2, K2, p1, p2);
+    return M > 32 ? rt : 1;
+}
+
+extern "C" int pta_gemm_splitk_pair_parts(int N1, int K1, int N2, int K2, int M, int* p1, int* p2) {
+    if (N1 <= 0 || K1 <= 0 || N2 <= 0 || K2 <= 0 || M < 0) return pta_fail("gemm_splitk_pair_parts: sizes must be positive");
+    pick_pair_parts_rows(N1, K1, N2, K2, M, p1, p2);
+    return 0;
+}
+
+extern "C" int pta_gemm_stationary_rule(int K1, int K2, int* q1, int* q2, int* from_rows) {
+    if (K1 <= 0 || K2 <= 0) return pta_fail("gemm_stationary_rule: sizes must be positive");
+    const StationaryChoice c = stationary_rule(K1, K2);
+    *q1 = c.q1; *q2 = c.q2; *from_rows = c.from;
     return 0;
 }
 
 // Two products of one launch, both left as partial sums: part1 [parts1, M, N1] of x1 . W1^T and part2
-// [parts2, M, N2] of x2 . W2^T, with the ranges pta_gemm_splitk_pair_parts gives.
+// [parts2, M, N2] of x2 . W2^T, with the ranges pta_gemm_splitk_pair_parts gives for M rows.
 extern "C" int pta_gemm_splitk_pair_bf16(float* part1, const void* x1, const void* W1, int N1, int K1, float* part2,
                                          const void* x2, const void* W2, int N2, int K2, int M, void* stream) {
     if (check_splitk("gemm_splitk_pair_bf16", x1, W1, M, N1, K1)) return 1;
     if (check_splitk("gemm_splitk_pair_bf16", x2, W2, M, N2, K2)) return 1;
     PTA_REQUIRE(part1 && part2, "gemm_splitk_pair_bf16: null workspace");
     int p1, p2;
-    const int rt = M > 32 ? pick_pair_parts(N1, K1, N2, K2, &p1, &p2) : (pick_pair_parts(N1, K1, N2, K2, &p1, &p2), 1);
-    const SplitkProblem a = make_problem(nullptr, part1, x1, W1, nullptr, nullptr, nullptr, N1, K1, 0, 0, rt, p1, 0);
-    const SplitkProblem b = make_problem(nullptr, part2, x2, W2, nullptr, nullptr, nullptr, N2, K2, 0, 0, rt, p2, 0);
-    if (rt == 2) return launch_rows<2, 2, 2>(tiles_per_chunk(M), a, b, M, 0, (hipStream_t)stream);
+    const int kind = pick_pair_parts_rows(N1, K1, N2, K2, M, &p1, &p2);
+    if (kind == 3) return pta_gemm_stationary_pair_bf16(part1, x1, W1, N1, K1, p1, part2, x2, W2, N2, K2, p2, M, stream);
+    const SplitkProblem a = make_problem(nullptr, part1, x1, W1, nullptr, nullptr, nullptr, N1, K1, 0, 0, kind, p1, 0);
+    const SplitkProblem b = make_problem(nullptr, part2, x2, W2, nullptr, nullptr, nullptr, N2, K2, 0, 0, kind, p2, 0);
+    if (kind == 2) return launch_rows<2, 2, 2>(tiles_per_chunk(M), a, b, M, 0, (hipStream_t)stream);
     return launch_rows<1, 2, 2>(tiles_per_chunk(M), a, b, M, 0, (hipStream_t)stream);
 }
 
@@ -567,7 +631,7 @@ extern "C" int pta_gemm_splitk_pair_reduced_bf16(void* y1, float* part1, const v
     if (rc) return rc;
     const long MN1 = (long)M * N1, MN2 = (long)M * N2;
     int P1, P2;
-    pick_pair_parts(N1, K1, N2, K2, &P1, &P2);
+    pick_pair_parts_rows(N1, K1, N2, K2, M, &P1, &P2);
     hipLaunchKernelGGL(gemm_splitk_reduce2_kernel, dim3((unsigned)((MN1 + MN2 + 255) / 256)), dim3(256), 0,
                        (hipStream_t)stream, (bf16_t*)y1, part1, bias1, MN1, N1, P1, act1, (bf16_t*)y2, part2, bias2, MN2, N2,
                        P2, act2);
@@ -611,7 +675,7 @@ extern "C" int pta_gemm_splitk_pair_reduced_qkv_bf16(void* q_out, float* part1, 
     if (rc) return rc;
     const long MN1 = (long)M * N1, MN2 = (long)M * N2;
     int P1, P2;
-    pick_pair_parts(N1, K1, N2, K2, &P1, &P2);
+    pick_pair_parts_rows(N1, K1, N2, K2, M, &P1, &P2);
     const QkvTail tail{(bf16_t*)q_out, inv_freq, inv_freq_ld, cs_scale, token_pos, token_seq, block_table, bt_stride, (bf16_t*)k_pool,
                        (bf16_t*)v_pool, nh, nkv, d, layout, write_cache};
     hipLaunchKernelGGL(gemm_splitk_reduce2_qkv_kernel, dim3((unsigned)((MN1 / 2 + MN2 + 255) / 256)), dim3(256), 0,

@@ -24,7 +24,7 @@ QKV_LAYOUT_CODES = {"grouped": 0, "tail": 1, "interleaved": 2}
 ACT_CODES = {None: 0, "none": 0, "linear": 0, "gelu": 1, "gelu_python": 1, "gelu_new": 2, "gelu_pytorch_tanh": 2,
              "gelu_fast": 2, "gelu_accurate": 2, "quick_gelu": 3, "relu": 4, "relu2": 5, "relu6": 6, "silu": 7, "swish": 7,
              "sigmoid": 8, "tanh": 9, "leaky_relu": 10, "mish": 11, "gelu_10": 12, "laplace": 13}
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 _lib = None
 _lock = threading.Lock()
@@ -79,7 +79,7 @@ def _call(name: str, *args) -> None:
 # cannot be recorded into a captured step.  ``timing_hint`` carries what an entry point's arguments do not say
 # (how many cached keys and values an attention launch reads, the arithmetic of a prompt's attention).
 _timing = None
-_HOST_ENTRIES = ("pta_gemm_splitk_pair_parts",)  # entry points that launch nothing
+_HOST_ENTRIES = ("pta_gemm_splitk_pair_parts", "pta_gemm_stationary_rule")  # entry points that launch nothing
 timing_hint = {"attn_bytes": 0, "attn_flops": 0}
 
 
@@ -977,11 +977,20 @@ def gemm_splitk_partial(x: torch.Tensor, w: torch.Tensor, rt: int = 0, parts: in
     return part
 
 
-def gemm_splitk_pair_parts(N1: int, K1: int, N2: int, K2: int):
-    """How many ranges of K each product of a pair launch is cut into."""
+def gemm_splitk_pair_parts(N1: int, K1: int, N2: int, K2: int, M: int = 0):
+    """How many ranges of K each product of a pair launch of ``M`` rows is cut into (0: by the kernel that walks
+    K in stages, whatever the rows; steps of 17 to 64 rows may run with the activations stationary, which has
+    ranges of its own)."""
     p1, p2 = ctypes.c_int(0), ctypes.c_int(0)
-    _call("pta_gemm_splitk_pair_parts", int(N1), int(K1), int(N2), int(K2), ctypes.byref(p1), ctypes.byref(p2))
+    _call("pta_gemm_splitk_pair_parts", int(N1), int(K1), int(N2), int(K2), int(M), ctypes.byref(p1), ctypes.byref(p2))
     return p1.value, p2.value
+
+
+def gemm_stationary_rule(K1: int, K2: int):
+    """(ranges, ranges, rows from which it is used) of the pair launch with stationary activations, by the rule."""
+    q1, q2, rows = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(0)
+    _call("pta_gemm_stationary_rule", int(K1), int(K2), ctypes.byref(q1), ctypes.byref(q2), ctypes.byref(rows))
+    return q1.value, q2.value, rows.value
 
 
 # Ranges of K for the pairs of a shape: the kernel library's rule gives a choice; when timing is on, its neighbours
@@ -991,6 +1000,9 @@ PAIR_TUNE = os.environ.get("PTA_PAIR_TUNE", "1") != "0"
 PAIR_TUNE_MARGIN = 0.97
 PAIR_TUNE_ROWS = int(os.environ.get("PTA_PAIR_TUNE_ROWS", "64"))  # rows of the timed launches (17 to 128)
 _pair_parts_tuned: dict = {}  # (shape of w1, shape of w2) -> the counts in use
+_pair_stationary_tuned: dict = {}  # (shape of w1, shape of w2) -> (ranges, ranges, rows from which) of the launch
+#                                    with stationary activations; 65 rows: never
+STATIONARY_NEVER = 65
 
 
 def tune_pair_parts(w1: torch.Tensor, w2: torch.Tensor) -> None:
@@ -998,7 +1010,10 @@ def tune_pair_parts(w1: torch.Tensor, w2: torch.Tensor) -> None:
     neighbours, and with workgroups of 128 rows of W (which load the activations half as often, have half as many
     workgroups and so want more ranges), at 64 rows with cold caches; keep the fastest in the kernel library if it
     beats the rule's by the margin and is no slower than the rule's at 24 rows (where the tile height does not
-    apply, but the ranges do).  ``_pair_parts_tuned`` says what is in use: (ranges, ranges, row tiles per wave)."""
+    apply, but the ranges do).  ``_pair_parts_tuned`` says what is in use: (ranges, ranges, row tiles per wave).
+    Then the launch with stationary activations is timed against the winner, with its rule's ranges and their
+    neighbours, at 64 and at 40 rows: it is used from 33 rows on, from 49 on, or never, by what those say
+    (``_pair_stationary_tuned``: ranges, ranges, rows from which)."""
     key = (tuple(w1.shape), tuple(w2.shape))
     if not PAIR_TUNE or key in _pair_parts_tuned or not _may_time():
         return
@@ -1007,14 +1022,20 @@ def tune_pair_parts(w1: torch.Tensor, w2: torch.Tensor) -> None:
     a0, b0 = gemm_splitk_pair_parts(N1, K1, N2, K2)
     fix = lambda c: lib.pta_gemm_splitk_pair_fix(int(N1), int(K1), int(N2), int(K2), int(c[0]), int(c[1]), int(c[2]))
     forget = lambda: lib.pta_gemm_splitk_pair_fix(int(N1), int(K1), int(N2), int(K2), 0, 0, 1)
+    fix_st = lambda c: lib.pta_gemm_splitk_pair_fix_stationary(int(N1), int(K1), int(N2), int(K2), int(c[0]), int(c[1]), int(c[2]))
+    q1, q2, from0 = gemm_stationary_rule(K1, K2)
+    fix_st((q1, q2, STATIONARY_NEVER))  # the launches timed first are the staged kernel's
     cands = [(a0, b0, 1)] + [(a, b, 1) for a in range(max(1, a0 - 1), a0 + 3) for b in range(max(1, b0 - 2), b0 + 3)
                              if (a, b) != (a0, b0)]
     tall = lambda p: sorted({max(1, p - 1), p, p + 1, max(1, 2 * p - 1), 2 * p, 2 * p + 1})
     cands += [(a, b, 2) for a in tall(a0) for b in tall(b0)]
     cands = [c for c in cands if fix(c) == 0]
     xs = {rows: [torch.randn((rows, K), dtype=torch.float32, device=w1.device).to(torch.bfloat16) for K in (K1, K2)]
-          for rows in (PAIR_TUNE_ROWS, 24)}
-    most = [max(c[i] for c in cands) for i in (0, 1)]
+          for rows in (PAIR_TUNE_ROWS, 24, 40)}
+    st_cands = [(q1, q2)] + [c for c in ((q1, 2 * q2), (2 * q1, 2 * q2), (q1, max(1, q2 // 2)), (2 * q1, q2))
+                             if c != (q1, q2) and fix_st(c + (STATIONARY_NEVER,)) == 0]
+    st_cands = list(dict.fromkeys(st_cands))
+    most = [max([c[i] for c in cands] + [c[i] for c in st_cands]) for i in (0, 1)]
     parts = [torch.empty((most[i], PAIR_TUNE_ROWS, N), dtype=torch.float32, device=w1.device) for i, N in enumerate((N1, N2))]
     # A launch is timed over several copies of the matrices in turn (more bytes than the memory-side cache holds),
     # back to back between two events: every launch reads its matrices from memory, as in a model, and no gap of
@@ -1023,7 +1044,7 @@ def tune_pair_parts(w1: torch.Tensor, w2: torch.Tensor) -> None:
     n_copies = max(2, min(6, int(640e6 // copy_bytes) + 1))
     copies = [(w1, w2)] + [(w1.clone(), w2.clone()) for _ in range(n_copies - 1)]
 
-    def timed_ways(chosen, rows, rounds=3):
+    def timed_ways(chosen, rows, rounds=3, fix=fix):
         best = [float("inf")] * len(chosen)
         for r in range(rounds + 1):  # the first round warms up
             for j, c in enumerate(chosen):
@@ -1046,7 +1067,6 @@ def tune_pair_parts(w1: torch.Tensor, w2: torch.Tensor) -> None:
         small = timed_ways([cands[i] for i in short], 24) if len(short) > 1 else [0.0]
     finally:
         forget()
-        del copies
     if os.environ.get("PTA_TUNE_VERBOSE"):
         print(f"[pta tune] pair {key}: rule {cands[0]} {times[0] * 1e3:.1f} us at {PAIR_TUNE_ROWS} rows; fastest " +
               ", ".join(f"{cands[i]} {times[i] * 1e3:.1f}" for i in order[:6]) +
@@ -1060,6 +1080,26 @@ def tune_pair_parts(w1: torch.Tensor, w2: torch.Tensor) -> None:
     if chosen != cands[0]:
         fix(chosen)
     _pair_parts_tuned[key] = chosen
+    # the launch with stationary activations against that choice, where both apply
+    stationary = (q1, q2, STATIONARY_NEVER)
+    if PAIR_TUNE_ROWS == 64:
+        try:
+            t64 = times[cands.index(chosen)]
+            s64 = timed_ways([c + (17,) for c in st_cands], 64, fix=fix_st)
+            best = min(range(len(st_cands)), key=lambda i: s64[i])
+            if s64[best] < 0.98 * t64:
+                fix_st(st_cands[best] + (STATIONARY_NEVER,))
+                t40 = timed_ways([chosen], 40)[0]
+                s40 = timed_ways([st_cands[best] + (17,)], 40, fix=fix_st)[0]
+                stationary = st_cands[best] + (33 if s40 < 0.98 * t40 else 49,)
+            if os.environ.get("PTA_TUNE_VERBOSE"):
+                print(f"[pta tune] pair {key} with stationary activations: " +
+                      ", ".join(f"{c} {t * 1e3:.1f}" for c, t in zip(st_cands, s64)) + f" us against {t64 * 1e3:.1f} at 64 rows"
+                      + (f"; {s40 * 1e3:.1f} against {t40 * 1e3:.1f} at 40 rows" if stationary[2] != STATIONARY_NEVER else "")
+                      + f" -> {stationary}", flush=True)
+        finally:
+            fix_st(stationary)
+    _pair_stationary_tuned[key] = stationary
 
 
 def tuning_table() -> dict:
@@ -1068,6 +1108,7 @@ def tuning_table() -> dict:
     key = lambda t: ",".join("x".join(str(int(v)) for v in (p if isinstance(p, tuple) else (p,))) for p in t)
     return {
         "pair_parts": {key(k): list(v) for k, v in _pair_parts_tuned.items()},  # ranges, ranges, row tiles per wave
+        "pair_stationary": {key(k): list(v) for k, v in _pair_stationary_tuned.items()},  # ranges, ranges, rows from
         "splitk_rows": {key(k): int(v) for k, v in _splitk_limits.items()},
         "mm_plans": {key(k): list(v) for k, v in _mm_plans.items()},
         "mm_joined": {key(k): bool(v) for k, v in _mm_joined.items()},
@@ -1081,7 +1122,9 @@ def clear_tuning() -> None:
     lib = load_library()
     for (s1, s2) in list(_pair_parts_tuned):
         lib.pta_gemm_splitk_pair_fix(int(s1[0]), int(s1[1]), int(s2[0]), int(s2[1]), 0, 0, 1)
-    for d in (_pair_parts_tuned, _splitk_limits, _mm_plans, _mm_costs, _mm_times, _mm_joined, _mm_ksplit, _decode_plans):
+    for (s1, s2) in list(_pair_stationary_tuned):
+        lib.pta_gemm_splitk_pair_fix_stationary(int(s1[0]), int(s1[1]), int(s2[0]), int(s2[1]), 0, 0, 0)
+    for d in (_pair_stationary_tuned, _pair_parts_tuned, _splitk_limits, _mm_plans, _mm_costs, _mm_times, _mm_joined, _mm_ksplit, _decode_plans):
         d.clear()
 
 
@@ -1097,6 +1140,11 @@ def load_tuning(table: dict) -> None:
         if (a, b, rt) != rule + (1,) and lib.pta_gemm_splitk_pair_fix(s1[0], s1[1], s2[0], s2[1], a, b, rt):
             raise KernelError(f"tuning table: {a} and {b} ranges of K with {rt} row tiles are not valid for the pair {k}")
         _pair_parts_tuned[(s1, s2)] = (a, b, rt)
+    for k, v in table.get("pair_stationary", {}).items():
+        s1, s2 = shapes(k)
+        if lib.pta_gemm_splitk_pair_fix_stationary(s1[0], s1[1], s2[0], s2[1], int(v[0]), int(v[1]), int(v[2])):
+            raise KernelError(f"tuning table: {list(v)} is not valid for the pair {k} with stationary activations")
+        _pair_stationary_tuned[(s1, s2)] = (int(v[0]), int(v[1]), int(v[2]))
     for k, v in table.get("splitk_rows", {}).items():
         _splitk_limits[shapes(k)] = int(v)
     for k, v in table.get("mm_plans", {}).items():
@@ -1130,7 +1178,7 @@ def gemm_splitk_pair_partial(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tenso
                           f"w2 {tuple(w2.shape)}")
     (N1, K1), (N2, K2) = w1.shape, w2.shape
     tune_pair_parts(w1, w2)
-    p1, p2 = gemm_splitk_pair_parts(N1, K1, N2, K2)
+    p1, p2 = gemm_splitk_pair_parts(N1, K1, N2, K2, M)
     part1 = torch.empty((p1, M, N1), dtype=torch.float32, device=x1.device)
     part2 = torch.empty((p2, M, N2), dtype=torch.float32, device=x1.device)
     _call("pta_gemm_splitk_pair_bf16", _ptr(part1), _ptr(x1), _ptr(w1), N1, K1, _ptr(part2), _ptr(x2), _ptr(w2), N2, K2,
@@ -1155,7 +1203,7 @@ def gemm_splitk_pair_bf16(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tensor, 
     if bias2 is not None:
         _need(bias2, "bias2", torch.float32, (N2,))
     tune_pair_parts(w1, w2)
-    p1, p2 = gemm_splitk_pair_parts(N1, K1, N2, K2)
+    p1, p2 = gemm_splitk_pair_parts(N1, K1, N2, K2, M)
     part1 = torch.empty((p1, M, N1), dtype=torch.float32, device=x1.device)
     part2 = torch.empty((p2, M, N2), dtype=torch.float32, device=x1.device)
     y1 = torch.empty((M, N1), dtype=torch.bfloat16, device=x1.device)
@@ -1192,7 +1240,7 @@ def gemm_splitk_pair_qkv(x1: torch.Tensor, w_qkv: torch.Tensor, bias_qkv, inv_fr
     freq_ld = _freq_ld(inv_freq, d, block_table.shape[0])
     _need_pools(k_pool, v_pool, torch.bfloat16, nkv, d)
     tune_pair_parts(w_qkv, w2)
-    p1, p2 = gemm_splitk_pair_parts(N1, K1, N2, K2)
+    p1, p2 = gemm_splitk_pair_parts(N1, K1, N2, K2, M)
     part1 = torch.empty((p1, M, N1), dtype=torch.float32, device=x1.device)
     part2 = torch.empty((p2, M, N2), dtype=torch.float32, device=x1.device)
     q = torch.empty((M, nh, d), dtype=torch.bfloat16, device=x1.device)
