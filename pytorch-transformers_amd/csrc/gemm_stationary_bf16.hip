@@ -17,8 +17,6 @@
 #include "common.h"
 #include "pta_kernels.h"
 
-#include <stdlib.h>
-
 #include <algorithm>
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
@@ -209,8 +207,9 @@ static int launch_stationary(const StationaryProblem& a, const StationaryProblem
 extern "C" int pta_gemm_stationary_groups(int N1, int K1, int parts1, int N2, int K2, int parts2, int* g1, int* g2) {
     if (N1 <= 0 || K1 <= 0 || N2 <= 0 || K2 <= 0 || parts1 <= 0 || parts2 <= 0)
         return pta_fail("gemm_stationary_groups: sizes must be positive");
-    static const double share = getenv("PTA_ST_UNITS") ? atof(getenv("PTA_ST_UNITS")) : 1.0;
-    const double units = pta_compute_units() * share, w1 = (double)N1 * K1, w2 = (double)N2 * K2;
+    // (half as many workgroups, which would read x half as often, take a third longer: a compute unit alone pulls
+    // no more than some 21 GB/s out of memory in this walk)
+    const double units = pta_compute_units(), w1 = (double)N1 * K1, w2 = (double)N2 * K2;
     const int need1 = ((N1 + 15) / 16 + ST_WAVES * ST_TMAX - 1) / (ST_WAVES * ST_TMAX);
     const int need2 = ((N2 + 15) / 16 + ST_WAVES * ST_TMAX - 1) / (ST_WAVES * ST_TMAX);
     *g1 = std::max(need1, std::max(1, (int)(units * w1 / (w1 + w2) / parts1 + 0.5)));
