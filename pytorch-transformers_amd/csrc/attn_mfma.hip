@@ -619,11 +619,11 @@ extern "C" int pta_attn_mfma(void* out, const void* q, const void* k_pool, const
                     ((uintptr_t)out % 8) == 0, "attn_mfma: pointers must be 16-byte aligned");
     hipStream_t s = (hipStream_t)stream;
     // Prompts: four waves of two column tiles share each key block through LDS (head sizes up to 128;
-    // beyond, one wave per workgroup).  Measured at Falcon-7B sizes (2,048 tokens, 71 heads on one KV
-    // head), one wave per workgroup: 2 tiles 148 us a layer, 4 tiles 195 us, 1 tile 270 us (fewer tiles
+    // beyond, one wave per workgroup).  Measured at 2,048 tokens, 71 heads on one KV
+    // head, one wave per workgroup: 2 tiles 148 us a layer, 4 tiles 195 us, 1 tile 270 us (fewer tiles
     // balance the causal triangle better, more tiles re-read keys less).
-    // One token per sequence (decode): one wave per workgroup, which holds `decode_tiles` column tiles of
-    // its KV head (at most what the head size leaves registers for).  More tiles: the keys cross the memory
+    // One token per sequence (decode): workgroups of `decode_waves` waves, each of which holds `decode_tiles` column
+    // tiles of its KV head (at most what the head size leaves registers for).  More tiles: the keys cross the memory
     // path fewer times; fewer: shorter waves, more of them (71 heads on one KV head, 2,048 keys: 64
     // sequences 39.5 us a layer with one tile, 27.5 us with five; 8 sequences 14.6 and 18.5 us).
     const bool narrow = max_new == 1;

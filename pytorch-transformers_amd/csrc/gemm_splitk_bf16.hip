@@ -323,7 +323,7 @@ static int effective_parts(int K, int parts) {
     return (nkb + per - 1) / per;
 }
 
-// Ranges of K (workgroups along gridDim.y).  Measured at Falcon-7B to Falcon-40B shapes: a workgroup does best
+// Ranges of K (workgroups along gridDim.y).  Measured at K = 4,096 to 32,768 and N = 4,096 to 32,768: a workgroup does best
 // with a range of about 2,304 elements (some 290 KB of weights for its 64 rows), and a launch with at least
 // some 512 workgroups; no range is shorter than 512 elements, and there are at most 16.
 #define SK_RANGE 2304
@@ -338,8 +338,8 @@ static int range_for(int groups) { return SK_RANGE * max(1, groups / 64); }
 
 // Among the counts near that rule's, the one with the least (rounds of workgroups on the chip's 256 compute units)
 // x (a workgroup's fixed cost + the length of its range).  Measured at 32 to 128 rows: a launch just over a whole
-// number of rounds pays for the last one in full (Falcon-40B's fused QKV, 144 row tiles: 4 ranges, 2.25 rounds, 81
-// us; 3 ranges, 1.69 rounds, 65 us; Falcon-7B's, 73 row tiles: 8 ranges 31.6 us, 7 ranges 27.6 us), and the fixed
+// number of rounds pays for the last one in full (N = 9,216 and K = 8,192, 144 row tiles: 4 ranges, 2.25 rounds, 81
+// us; 3 ranges, 1.69 rounds, 65 us; N = 4,672 and K = 4,544, 73 row tiles: 8 ranges 31.6 us, 7 ranges 27.6 us), and the fixed
 // cost of a workgroup (start, first loads, its tile of partial sums) is that of some 1,300 elements of K.
 #define SK_WG_FIXED 1300
 static int pick_parts(int N, int K, int rt) {
@@ -478,7 +478,7 @@ extern "C" int pta_gemm_splitk_bf16(void* y, float* part, const void* x, const v
 // Ranges of K for the two products of a pair launch: each by its own length, and more of both if the launch
 // would have too few workgroups.
 // Counts that a caller has fixed for the pairs of one shape: no rule tells which neighbour of its choice is the
-// fastest (Falcon2-11B's output and feed-forward-down pair at 64 rows: 2 and 7 ranges by the rule; 4 and 8 make the
+// fastest (N = 4,096 with K = 4,096 and 16,384 at 64 rows: 2 and 7 ranges by the rule; 4 and 8 make the
 // decode step 7 % faster, 2 and 10 make it 3 % slower with as many workgroups), so the Python side times them once.
 struct PairChoice { int p1, p2, rt; };
 static std::map<std::array<int, 4>, PairChoice> pair_parts_fixed;

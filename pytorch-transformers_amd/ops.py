@@ -1168,6 +1168,20 @@ def gemm_splitk_pair_parts_rule(N1: int, K1: int, N2: int, K2: int):
     return rule
 
 
+# Elements of both matrices of a pair launch up to which it beats the two products on their own beyond 48 rows.
+# Measured in whole decode steps: pairs of 104 M elements (K = 4,544, N = 4,672 + 18,176) and of 92 M (K = 4,096, N
+# = 6,144 + 16,384) win at every row count; a pair of 344 M (K = 8,192, N = 9,216 + 32,768) wins up to 48 rows (32
+# rows: 20.8 against 23.0 ms a step) and loses beyond them to the vendor library's product for the longer matrix
+# (64 rows: 24.3 against 23.3 ms).
+PAIR_MAX_WEIGHTS = 160 * 1024 * 1024
+PAIR_SURE_ROWS = 48
+
+
+def pair_launch_pays(rows: int, w1: torch.Tensor, w2: torch.Tensor) -> bool:
+    """Whether two products of ``rows`` rows (17 and more) run as one launch of the decode batch kernels."""
+    return rows <= PAIR_SURE_ROWS or w1.numel() + w2.numel() <= PAIR_MAX_WEIGHTS
+
+
 def gemm_splitk_pair_partial(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tensor, w2: torch.Tensor):
     """(x1 @ w1.T, x2 @ w2.T), both left as 32-bit partial sums, in one launch; the products share M."""
     for name, t in (("x1", x1), ("w1", w1), ("x2", x2), ("w2", w2)):

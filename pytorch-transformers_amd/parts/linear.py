@@ -22,9 +22,6 @@ from ..engine.spec import INIT_NORMAL, INIT_ZERO_NOISE, MATRIX, VECTOR, TensorSp
 from .base import PartialProduct, Part
 
 
-PAIR_MAX_WEIGHTS = 160 * 1024 * 1024  # elements of both matrices of a pair launch beyond 48 rows
-
-
 class Linear(Part):
     def __init__(self, name: str, in_features: int, out_features: int, bias: bool):
         self.name = name
@@ -124,11 +121,9 @@ class Linear(Part):
                 if bias is not None or act is not None:
                     ops.epilogue_(yi, bias, act)
             return y1, y2
-        # 17 rows and more: measured at Falcon-7B and Falcon2-11B sizes the pair beats the products on their own; at
-        # Falcon-40B sizes it does up to 48 rows (32 rows: 20.8 against 23.0 ms a step), beyond them the vendor
-        # library's product for the feed-forward input is the faster one (64 rows: 23.3 against 24.3 ms)
-        small = x1.shape[0] <= 48 or first.weight.numel() + second.weight.numel() <= PAIR_MAX_WEIGHTS
-        if small and ops.gemm_splitk_pair_ok(x1, first.weight, x2, second.weight):
+        # 17 rows and more: the pair launch where it beats the products on their own (``ops.pair_launch_pays``)
+        if ops.pair_launch_pays(x1.shape[0], first.weight, second.weight) and \
+                ops.gemm_splitk_pair_ok(x1, first.weight, x2, second.weight):
             if tail is not None and ops.QKV_TAIL and kw1.get("act") is None and tail.head_dim % 2 == 0:
                 # the launch that adds the partial sums takes the fused rows to their end as well
                 q, y2 = ops.gemm_splitk_pair_qkv(
