@@ -533,15 +533,16 @@ static int pick_pair_parts(int N1, int K1, int N2, int K2, int* p1, int* p2) {
     return 1;
 }
 
-// Steps of 17 to 64 rows may run with the activations stationary (gemm_stationary_bf16.hip), which cuts K into
+// Steps of 17 to 128 rows may run with the activations stationary (gemm_stationary_bf16.hip), which cuts K into
 // ranges of its own: few and long, since its workgroups are as many as the compute units whatever the ranges.
 // The rule: ranges about as long as the shorter K of the pair (between 2,048 and 8,192 elements), from 49 rows on.
 // Measured against the staged kernel at 64 rows, pairs of K = 4,544 with N = 4,672 + 18,176 and K = 4,544 +
 // 18,176 with N = 4,544: 51.8 against 58.2 us and 51.2 against 57.5 us; K = 4,096 / 16,384: 48.3 against 51.7 and
-// 44.7 against 53.9; K = 8,192 / 32,768: 155 against 179 and 157 against 171.  At 40 rows the two are within 5 % of
-// each other either way (three shapes of six go to each), at 32 rows the staged kernel wins.
+// 44.7 against 53.9; K = 8,192 / 32,768: 155 against 179 and 157 against 171; at 128 rows 59.5 against 75.4 and 60.4
+// against 72.6 (K = 4,544), 53.6 against 64.8 and 55.1 against 75.0 (K = 4,096 / 16,384).  At 40 rows the two are
+// within 5 % of each other either way (three shapes of six go to each), at 32 rows the staged kernel wins.
 #define STATIONARY_FROM_ROWS 49
-#define STATIONARY_MAX_ROWS 64
+#define STATIONARY_MAX_ROWS 128
 struct StationaryChoice { int q1, q2, from; };
 static std::map<std::array<int, 4>, StationaryChoice> pair_stationary_fixed;
 
@@ -552,7 +553,7 @@ static StationaryChoice stationary_rule(int K1, int K2) {
 }
 
 // Fixes, for every later pair launch of this shape with from_rows to 64 rows, the ranges of K of the launch with
-// stationary activations (from_rows 17 to 65; 65: never that launch).  q1 = q2 = 0 forgets the shape.  Returns 1
+// stationary activations (from_rows 17 to 129; 129: never that launch).  q1 = q2 = 0 forgets the shape.  Returns 1
 // (no error text) for counts that the kernel does not take.
 extern "C" int pta_gemm_splitk_pair_fix_stationary(int N1, int K1, int N2, int K2, int q1, int q2, int from_rows) {
     if (N1 <= 0 || K1 <= 0 || N2 <= 0 || K2 <= 0) return 1;

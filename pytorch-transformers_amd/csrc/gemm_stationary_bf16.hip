@@ -1,4 +1,4 @@
-// The two products of a pair launch for a decode batch of 17 to 64 rows, left as 32-bit partial sums, with the
+// The two products of a pair launch for a decode batch of 17 to 128 rows, left as 32-bit partial sums, with the
 // activations stationary: part[p, M, N] = x[M, range p of K] . W[N, range p of K]^T.
 //
 // The kernel that walks K in stages (gemm_splitk_bf16.hip) copies every stage's slice of x into LDS once per
@@ -31,7 +31,6 @@ union SFrag8 {
 
 #define ST_WAVES 8
 #define ST_THREADS (ST_WAVES * 64)
-#define ST_TMAX 3      // row tiles of W per wave
 #define ST_LDS_BYTES (152 * 1024)
 
 struct StationaryProblem {
@@ -47,7 +46,7 @@ struct StationaryProblem {
 // MT: sixteen-row tiles of x.  KP: elements of K per phase (a multiple of 64).  PF: 32-element steps of W in flight
 // per wave; it is even and divides the steps of a phase, so that a step's registers are known when the kernel is
 // compiled.  Every phase runs all its steps: past the range's end x is zero.
-template <int MT, int KP, int PF>
+template <int MT, int KP, int PF, int ST_TMAX>
 __global__ __launch_bounds__(ST_THREADS) void gemm_stationary_kernel(StationaryProblem pa, StationaryProblem pb, int M) {
     constexpr int MP = MT * 16;
     constexpr int LDW = KP + 8;  // 16 bytes of padding keep the sixteen rows of a 16-byte read on distinct banks
@@ -185,11 +184,11 @@ static StationaryProblem make_stationary(float* part, const void* x, const void*
     return p;
 }
 
-template <int MT, int KP, int PF>
+template <int MT, int KP, int PF, int TMAX>
 static int launch_stationary(const StationaryProblem& a, const StationaryProblem& b, int M, hipStream_t s) {
     constexpr size_t lds = (size_t)2 * MT * 16 * (KP + 8) * sizeof(bf16_t);
     static_assert(lds <= ST_LDS_BYTES, "two slices of x must fit the LDS of a compute unit");
-    auto kern = gemm_stationary_kernel<MT, KP, PF>;
+    auto kern = gemm_stationary_kernel<MT, KP, PF, TMAX>;
     if (lds > 64 * 1024) {
         static bool raised = false;
         if (!raised) {
@@ -204,14 +203,18 @@ static int launch_stationary(const StationaryProblem& a, const StationaryProblem
 
 // workgroups per range of K for the two products: together about one per compute unit, shared by the bytes of
 // the two matrices, and at least as many as the tiles a wave can hold ask for
-extern "C" int pta_gemm_stationary_groups(int N1, int K1, int parts1, int N2, int K2, int parts2, int* g1, int* g2) {
+// row tiles of W that a wave holds at most: what the sums of M rows leave registers for
+static int stationary_tmax(int M) { return M <= 64 ? 3 : 2; }
+
+extern "C" int pta_gemm_stationary_groups(int N1, int K1, int parts1, int N2, int K2, int parts2, int M, int* g1, int* g2) {
+    const int tmax = stationary_tmax(M);
     if (N1 <= 0 || K1 <= 0 || N2 <= 0 || K2 <= 0 || parts1 <= 0 || parts2 <= 0)
         return pta_fail("gemm_stationary_groups: sizes must be positive");
     // (half as many workgroups, which would read x half as often, take a third longer: a compute unit alone pulls
     // no more than some 21 GB/s out of memory in this walk)
     const double units = pta_compute_units(), w1 = (double)N1 * K1, w2 = (double)N2 * K2;
-    const int need1 = ((N1 + 15) / 16 + ST_WAVES * ST_TMAX - 1) / (ST_WAVES * ST_TMAX);
-    const int need2 = ((N2 + 15) / 16 + ST_WAVES * ST_TMAX - 1) / (ST_WAVES * ST_TMAX);
+    const int need1 = ((N1 + 15) / 16 + ST_WAVES * tmax - 1) / (ST_WAVES * tmax);
+    const int need2 = ((N2 + 15) / 16 + ST_WAVES * tmax - 1) / (ST_WAVES * tmax);
     *g1 = std::max(need1, std::max(1, (int)(units * w1 / (w1 + w2) / parts1 + 0.5)));
     *g2 = std::max(need2, std::max(1, (int)((units - (double)*g1 * parts1) / parts2 + 0.5)));
     return 0;
@@ -220,7 +223,7 @@ extern "C" int pta_gemm_stationary_groups(int N1, int K1, int parts1, int N2, in
 extern "C" int pta_gemm_stationary_pair_bf16(float* part1, const void* x1, const void* W1, int N1, int K1, int parts1,
                                              float* part2, const void* x2, const void* W2, int N2, int K2, int parts2,
                                              int M, void* stream) {
-    PTA_REQUIRE(M > 16 && M <= 64, "gemm_stationary_pair_bf16: 17 to 64 rows, got %d", M);
+    PTA_REQUIRE(M > 16 && M <= 128, "gemm_stationary_pair_bf16: 17 to 128 rows, got %d", M);
     PTA_REQUIRE(N1 > 0 && K1 > 0 && N2 > 0 && K2 > 0, "gemm_stationary_pair_bf16: sizes must be positive");
     PTA_REQUIRE(K1 % 8 == 0 && K2 % 8 == 0, "gemm_stationary_pair_bf16: K must be a multiple of 8 (16-byte loads)");
     PTA_REQUIRE(part1 && part2 && x1 && x2 && W1 && W2, "gemm_stationary_pair_bf16: null pointer");
@@ -230,13 +233,15 @@ extern "C" int pta_gemm_stationary_pair_bf16(float* part1, const void* x1, const
     for (const void* p : {x1, x2, W1, W2})
         PTA_REQUIRE(((uintptr_t)p % 16) == 0, "gemm_stationary_pair_bf16: x and W must be 16-byte aligned");
     int g1, g2;
-    if (pta_gemm_stationary_groups(N1, K1, parts1, N2, K2, parts2, &g1, &g2)) return 1;
+    if (pta_gemm_stationary_groups(N1, K1, parts1, N2, K2, parts2, M, &g1, &g2)) return 1;
     const StationaryProblem a = make_stationary(part1, x1, W1, N1, K1, parts1, g1);
     const StationaryProblem b = make_stationary(part2, x2, W2, N2, K2, parts2, g2);
     hipStream_t s = (hipStream_t)stream;
     switch ((M + 15) / 16) {
-        case 2: return launch_stationary<2, 1024, 8>(a, b, M, s);
-        case 3: return launch_stationary<3, 768, 8>(a, b, M, s);
-        default: return launch_stationary<4, 512, 8>(a, b, M, s);
+        case 2: return launch_stationary<2, 1024, 8, 3>(a, b, M, s);
+        case 3: return launch_stationary<3, 768, 8, 3>(a, b, M, s);
+        case 4: return launch_stationary<4, 512, 8, 3>(a, b, M, s);
+        case 5: case 6: return launch_stationary<6, 384, 6, 2>(a, b, M, s);
+        default: return launch_stationary<8, 256, 8, 2>(a, b, M, s);
     }
 }

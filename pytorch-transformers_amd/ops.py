@@ -979,7 +979,7 @@ def gemm_splitk_partial(x: torch.Tensor, w: torch.Tensor, rt: int = 0, parts: in
 
 def gemm_splitk_pair_parts(N1: int, K1: int, N2: int, K2: int, M: int = 0):
     """How many ranges of K each product of a pair launch of ``M`` rows is cut into (0: by the kernel that walks
-    K in stages, whatever the rows; steps of 17 to 64 rows may run with the activations stationary, which has
+    K in stages, whatever the rows; steps of 17 to 128 rows may run with the activations stationary, which has
     ranges of its own)."""
     p1, p2 = ctypes.c_int(0), ctypes.c_int(0)
     _call("pta_gemm_splitk_pair_parts", int(N1), int(K1), int(N2), int(K2), int(M), ctypes.byref(p1), ctypes.byref(p2))
@@ -1001,8 +1001,8 @@ PAIR_TUNE_MARGIN = 0.97
 PAIR_TUNE_ROWS = int(os.environ.get("PTA_PAIR_TUNE_ROWS", "64"))  # rows of the timed launches (17 to 128)
 _pair_parts_tuned: dict = {}  # (shape of w1, shape of w2) -> the counts in use
 _pair_stationary_tuned: dict = {}  # (shape of w1, shape of w2) -> (ranges, ranges, rows from which) of the launch
-#                                    with stationary activations; 65 rows: never
-STATIONARY_NEVER = 65
+#                                    with stationary activations (it runs up to 128 rows); 129 rows: never
+STATIONARY_NEVER = 129
 
 
 def tune_pair_parts(w1: torch.Tensor, w2: torch.Tensor) -> None:

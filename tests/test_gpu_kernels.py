@@ -269,7 +269,7 @@ def test_pair_ranges_are_timed_once_per_shape_and_kept():
     assert ops.gemm_splitk_pair_parts(N1, K1, N2, K2) == rule
 
 
-@pytest.mark.parametrize("M", [17, 32, 33, 47, 48, 49, 64])
+@pytest.mark.parametrize("M", [17, 32, 33, 47, 48, 49, 64, 65, 96, 100, 128])
 @pytest.mark.parametrize("shapes,parts", [(((1000, 520), (344, 1096)), (1, 1)), (((1000, 520), (344, 1096)), (2, 3)),
                                           (((40, 72), (1608, 2304)), (1, 2)), (((4672, 4544), (512, 8192)), (1, 2)),
                                           (((24, 8), (16, 4104)), (1, 16))])
@@ -300,7 +300,7 @@ def test_gemm_stationary_pair(M, shapes, parts):
 
 
 def test_gemm_stationary_pair_refusals_and_dispatch():
-    """Rows outside 17..64 and K that is no multiple of 8 are refused with a message; a pair launch of 49 to 64 rows
+    """Rows outside 17..128 are refused with a message; a pair launch of 49 to 128 rows
     runs with stationary activations and the ranges the library reports for those rows, one of 48 rows does not,
     and the rows from which it does can be fixed per shape and forgotten."""
     import ctypes
@@ -311,17 +311,17 @@ def test_gemm_stationary_pair_refusals_and_dispatch():
     P = lambda t: ctypes.c_void_p(t.data_ptr())
     stream = lambda: ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     w1, w2 = _rand(N1, K1, seed=1, dtype=torch.bfloat16, scale=0.05), _rand(N2, K2, seed=2, dtype=torch.bfloat16, scale=0.05)
-    for M in (16, 65):
+    for M in (16, 129):
         x1, x2 = _rand(M, K1, dtype=torch.bfloat16), _rand(M, K2, seed=5, dtype=torch.bfloat16)
         part = torch.empty(4, M, 328).cuda()
         assert lib.pta_gemm_stationary_pair_bf16(P(part), P(x1), P(w1), N1, K1, 1, P(part), P(x2), P(w2), N2, K2, 1, M, stream()) != 0
-        assert "17 to 64 rows" in lib.pta_last_error().decode()
+        assert "17 to 128 rows" in lib.pta_last_error().decode()
     q1, q2, rows = ops.gemm_stationary_rule(K1, K2)
     assert (q1, q2, rows) == (1, 2, 49)
     staged = ops.gemm_splitk_pair_parts(N1, K1, N2, K2)
-    assert ops.gemm_splitk_pair_parts(N1, K1, N2, K2, 48) == staged and ops.gemm_splitk_pair_parts(N1, K1, N2, K2, 65) == staged
-    assert ops.gemm_splitk_pair_parts(N1, K1, N2, K2, 49) == (q1, q2) == ops.gemm_splitk_pair_parts(N1, K1, N2, K2, 64)
-    for M in (48, 49, 64):
+    assert ops.gemm_splitk_pair_parts(N1, K1, N2, K2, 48) == staged and ops.gemm_splitk_pair_parts(N1, K1, N2, K2, 129) == staged
+    assert ops.gemm_splitk_pair_parts(N1, K1, N2, K2, 49) == (q1, q2) == ops.gemm_splitk_pair_parts(N1, K1, N2, K2, 128)
+    for M in (48, 49, 64, 100, 128):
         x1, x2 = _rand(M, K1, dtype=torch.bfloat16), _rand(M, K2, seed=5, dtype=torch.bfloat16)
         a, b = ops.gemm_splitk_pair_partial(x1, w1, x2, w2)
         assert (a.shape[0], b.shape[0]) == ops.gemm_splitk_pair_parts(N1, K1, N2, K2, M)
@@ -331,8 +331,9 @@ def test_gemm_stationary_pair_refusals_and_dispatch():
     try:
         assert lib.pta_gemm_splitk_pair_fix_stationary(N1, K1, N2, K2, 2, 4, 33) == 0
         assert ops.gemm_splitk_pair_parts(N1, K1, N2, K2, 33) == (2, 4) and ops.gemm_splitk_pair_parts(N1, K1, N2, K2, 32) == staged
-        assert lib.pta_gemm_splitk_pair_fix_stationary(N1, K1, N2, K2, 1, 1, 65) == 0
-        assert ops.gemm_splitk_pair_parts(N1, K1, N2, K2, 64) == staged
+        assert lib.pta_gemm_splitk_pair_fix_stationary(N1, K1, N2, K2, 1, 1, ops.STATIONARY_NEVER) == 0
+        assert ops.gemm_splitk_pair_parts(N1, K1, N2, K2, 64) == staged == ops.gemm_splitk_pair_parts(N1, K1, N2, K2, 128)
+        assert lib.pta_gemm_splitk_pair_fix_stationary(N1, K1, N2, K2, 1, 1, 130) != 0
         assert lib.pta_gemm_splitk_pair_fix_stationary(N1, K1, N2, K2, 1, 1, 16) != 0
         assert lib.pta_gemm_splitk_pair_fix_stationary(N1, K1, N2, K2, 0, 1, 33) != 0
     finally:
