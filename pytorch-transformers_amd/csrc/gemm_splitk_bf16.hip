@@ -533,56 +533,87 @@ static int pick_pair_parts(int N1, int K1, int N2, int K2, int* p1, int* p2) {
     return 1;
 }
 
-// Steps of 17 to 128 rows may run with the activations stationary (gemm_stationary_bf16.hip), which cuts K into
-// ranges of its own: few and long, since its workgroups are as many as the compute units whatever the ranges.
-// The rule: ranges about as long as the shorter K of the pair (between 2,048 and 8,192 elements), from 49 rows on.
-// Measured against the staged kernel at 64 rows, pairs of K = 4,544 with N = 4,672 + 18,176 and K = 4,544 +
-// 18,176 with N = 4,544: 51.8 against 58.2 us and 51.2 against 57.5 us; K = 4,096 / 16,384: 48.3 against 51.7 and
-// 44.7 against 53.9; K = 8,192 / 32,768: 155 against 179 and 157 against 171; at 128 rows 59.5 against 75.4 and 60.4
-// against 72.6 (K = 4,544), 53.6 against 64.8 and 55.1 against 75.0 (K = 4,096 / 16,384).  At 40 rows the two are
-// within 5 % of each other either way (three shapes of six go to each), at 32 rows the staged kernel wins.
-#define STATIONARY_FROM_ROWS 49
+// Steps of up to 128 rows may run with the activations stationary (gemm_stationary_bf16.hip), which cuts K into
+// ranges of its own, by the class of the step's rows (up to 16, 32, 64, 128).  The rule: ranges of about 1,400
+// elements, of the same length in both products, but no more of them than leave every wave at most the row tiles
+// it can hold with one workgroup per compute unit (past that the launch needs a second round of workgroups).
+// Measured against the staged kernel (us, staged -> stationary with the rule's ranges): K = 4,544 with N = 4,672
+// + 18,176 at 8 / 32 / 64 / 128 rows 45.3 -> 40.5, 47.1 -> 43.1, 58.2 -> 46.5, 75.4 -> 56.0; K = 4,544 + 18,176
+// with N = 4,544: 44.9 -> 41.6, 48.8 -> 44.9, 57.5 -> 48.0, 72.6 -> 55.6; K = 4,096 with N = 6,144 + 16,384: 42.3
+// -> 38.4, 45.6 -> 40.1, 51.7 -> 45.1, 64.8 -> 55.1; K = 8,192 with N = 9,216 + 32,768: 141.8 -> 137.5, 158.5 ->
+// 154.6, 178.9 -> 163.5, 188.7 -> 185.7.  Which count of ranges is fastest varies by a few percent around the
+// rule's (and at 128 rows of the last shape three ranges in two rounds beat one by a tenth), so the Python side
+// times the neighbours per class and fixes what wins, or the staged kernel where that wins.
 #define STATIONARY_MAX_ROWS 128
-struct StationaryChoice { int q1, q2, from; };
+#define STATIONARY_CLASSES 4
+#define STATIONARY_RANGE 1400
+static int stationary_class(int M) { return M <= 16 ? 0 : M <= 32 ? 1 : M <= 64 ? 2 : 3; }
+struct StationaryChoice { int q1[STATIONARY_CLASSES], q2[STATIONARY_CLASSES]; };  // 0: the staged kernel
 static std::map<std::array<int, 4>, StationaryChoice> pair_stationary_fixed;
 
-static StationaryChoice stationary_rule(int K1, int K2) {
-    const int target = max(2048, min(8192, min(K1, K2)));
-    auto parts = [&](int K) { return effective_parts(K, max(1, min(16, (K + target / 2) / target))); };
-    return {parts(K1), parts(K2), STATIONARY_FROM_ROWS};
+// Without a fixed choice the launch is used from 33 rows on (classes 2 and 3): below, the staged kernel with timed
+// ranges is as fast or faster at most shapes.
+#define STATIONARY_RULE_FROM_CLASS 2
+static void stationary_rule(int N1, int K1, int N2, int K2, int cls, int* q1, int* q2) {
+    const int kmin = min(K1, K2), f1 = max(1, (K1 + kmin / 2) / kmin), f2 = max(1, (K2 + kmin / 2) / kmin);
+    const long tiles = (long)((N1 + 15) / 16) * f1 + (long)((N2 + 15) / 16) * f2;
+    const long room = (long)pta_compute_units() * 8 * (cls == 3 ? 2 : 3);  // waves x row tiles a wave holds
+    int base = max(1, (kmin + STATIONARY_RANGE / 2) / STATIONARY_RANGE);
+    base = max(1, (int)min((long)base, room / max(1L, tiles)));
+    while (base > 1 && (base * f1 > 16 || base * f2 > 16)) --base;
+    *q1 = effective_parts(K1, min(16, base * f1));
+    *q2 = effective_parts(K2, min(16, base * f2));
 }
 
-// Fixes, for every later pair launch of this shape with from_rows to 64 rows, the ranges of K of the launch with
-// stationary activations (from_rows 17 to 129; 129: never that launch).  q1 = q2 = 0 forgets the shape.  Returns 1
-// (no error text) for counts that the kernel does not take.
-extern "C" int pta_gemm_splitk_pair_fix_stationary(int N1, int K1, int N2, int K2, int q1, int q2, int from_rows) {
+// Fixes, for every later pair launch of this shape with rows of class cls (0: up to 16 rows, 1: 32, 2: 64, 3:
+// 128), the ranges of K of the launch with stationary activations; q1 = q2 = 0: the staged kernel for the class;
+// cls = -1 forgets the shape.  Returns 1 (no error text) for counts that the kernel does not take.
+extern "C" int pta_gemm_splitk_pair_fix_stationary(int N1, int K1, int N2, int K2, int cls, int q1, int q2) {
     if (N1 <= 0 || K1 <= 0 || N2 <= 0 || K2 <= 0) return 1;
     std::lock_guard<std::mutex> hold(pair_parts_lock);
     const std::array<int, 4> key{N1, K1, N2, K2};
-    if (q1 == 0 && q2 == 0) {
+    if (cls == -1) {
         pair_stationary_fixed.erase(key);
         return 0;
     }
-    if (q1 < 1 || q2 < 1 || q1 > 16 || q2 > 16 || effective_parts(K1, q1) != q1 || effective_parts(K2, q2) != q2 ||
-        from_rows < 17 || from_rows > STATIONARY_MAX_ROWS + 1)
+    if (cls < 0 || cls >= STATIONARY_CLASSES) return 1;
+    const bool staged = q1 == 0 && q2 == 0;
+    if (!staged && (q1 < 1 || q2 < 1 || q1 > 16 || q2 > 16 || effective_parts(K1, q1) != q1 || effective_parts(K2, q2) != q2))
         return 1;
-    pair_stationary_fixed[key] = {q1, q2, from_rows};
+    auto it = pair_stationary_fixed.find(key);
+    if (it == pair_stationary_fixed.end()) {
+        StationaryChoice c{};
+        for (int i = STATIONARY_RULE_FROM_CLASS; i < STATIONARY_CLASSES; ++i) stationary_rule(N1, K1, N2, K2, i, &c.q1[i], &c.q2[i]);
+        it = pair_stationary_fixed.emplace(key, c).first;
+    }
+    it->second.q1[cls] = q1;
+    it->second.q2[cls] = q2;
     return 0;
 }
 
 // The ranges of a pair launch of M rows and its kind: 3 with stationary activations, else the tiles of sixteen
 // rows of W per wave of the staged kernel (1 or 2).  M = 0 asks for the staged kernel's ranges.
 static int pick_pair_parts_rows(int N1, int K1, int N2, int K2, int M, int* p1, int* p2) {
-    if (M > 16 && M <= STATIONARY_MAX_ROWS && K1 % 8 == 0 && K2 % 8 == 0) {
-        StationaryChoice c = stationary_rule(K1, K2);
+    if (M >= 1 && M <= STATIONARY_MAX_ROWS && K1 % 8 == 0 && K2 % 8 == 0) {
+        const int cls = stationary_class(M);
+        int q1, q2;
+        bool fixed = false;
         {
             std::lock_guard<std::mutex> hold(pair_parts_lock);
             const auto it = pair_stationary_fixed.find({N1, K1, N2, K2});
-            if (it != pair_stationary_fixed.end()) c = it->second;
+            if (it != pair_stationary_fixed.end()) {
+                q1 = it->second.q1[cls];
+                q2 = it->second.q2[cls];
+                fixed = true;
+            }
         }
-        if (M >= c.from) {
-            *p1 = c.q1;
-            *p2 = c.q2;
+        if (!fixed) {
+            q1 = q2 = 0;
+            if (cls >= STATIONARY_RULE_FROM_CLASS) stationary_rule(N1, K1, N2, K2, cls, &q1, &q2);
+        }
+        if (q1 > 0 && q2 > 0) {
+            *p1 = q1;
+            *p2 = q2;
             return 3;
         }
     }
@@ -596,10 +627,10 @@ extern "C" int pta_gemm_splitk_pair_parts(int N1, int K1, int N2, int K2, int M,
     return 0;
 }
 
-extern "C" int pta_gemm_stationary_rule(int K1, int K2, int* q1, int* q2, int* from_rows) {
-    if (K1 <= 0 || K2 <= 0) return pta_fail("gemm_stationary_rule: sizes must be positive");
-    const StationaryChoice c = stationary_rule(K1, K2);
-    *q1 = c.q1; *q2 = c.q2; *from_rows = c.from;
+extern "C" int pta_gemm_stationary_rule(int N1, int K1, int N2, int K2, int cls, int* q1, int* q2) {
+    if (N1 <= 0 || K1 <= 0 || N2 <= 0 || K2 <= 0 || cls < 0 || cls >= STATIONARY_CLASSES)
+        return pta_fail("gemm_stationary_rule: sizes must be positive and the class of rows 0 to %d", STATIONARY_CLASSES - 1);
+    stationary_rule(N1, K1, N2, K2, cls, q1, q2);
     return 0;
 }
 

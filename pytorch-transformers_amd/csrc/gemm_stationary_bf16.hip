@@ -46,7 +46,11 @@ struct StationaryProblem {
 // MT: sixteen-row tiles of x.  KP: elements of K per phase (a multiple of 64).  PF: 32-element steps of W in flight
 // per wave; it is even and divides the steps of a phase, so that a step's registers are known when the kernel is
 // compiled.  Every phase runs all its steps: past the range's end x is zero.
-template <int MT, int KP, int PF, int ST_TMAX>
+// SINGLE: the workgroup's whole range of K is one phase (the host has seen to it that it fits): one LDS buffer, and
+// after the first no barrier at all.  The barriers cost more than they look: the waves of a workgroup stream their
+// tiles at the pace memory gives each of them, and at every phase's end all wait for the slowest (K = 4,544 in
+// nine phases: 51 us; in one phase, at 8 rows, 42 us, which is what a kernel that only reads W in this walk takes).
+template <int MT, int KP, int PF, int ST_TMAX, bool SINGLE>
 __global__ __launch_bounds__(ST_THREADS) void gemm_stationary_kernel(StationaryProblem pa, StationaryProblem pb, int M) {
     constexpr int MP = MT * 16;
     constexpr int LDW = KP + 8;  // 16 bytes of padding keep the sixteen rows of a 16-byte read on distinct banks
@@ -54,7 +58,7 @@ __global__ __launch_bounds__(ST_THREADS) void gemm_stationary_kernel(StationaryP
     static_assert(STEPS % PF == 0 && PF % 2 == 0, "the loads in flight must divide a phase's steps and be even");
     constexpr int PIECES = MP * (KP / 8) / ST_THREADS;  // 16-byte pieces of a slice per thread
     static_assert(MP * (KP / 8) % ST_THREADS == 0, "a slice of x must divide over the threads");
-    extern __shared__ __attribute__((aligned(16))) bf16_t xs[];  // [2][MP][LDW]
+    extern __shared__ __attribute__((aligned(16))) bf16_t xs[];  // [2][MP][LDW], [MP][LDW] if SINGLE
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 15, g4 = lane >> 4;
@@ -70,7 +74,9 @@ __global__ __launch_bounds__(ST_THREADS) void gemm_stationary_kernel(StationaryP
     const int nkb = (K + 63) >> 6;
     const int kb0 = range * pr.blocks_per_part, kb1 = min(kb0 + pr.blocks_per_part, nkb);
     const int k_begin = kb0 * 64, k_end = min(kb1 * 64, K);
-    const int phases = (k_end - k_begin + KP - 1) / KP;
+    const int phases = SINGLE ? 1 : (k_end - k_begin + KP - 1) / KP;
+    // steps of a phase: all of them, or with one phase as many as the range has, in whole rounds of PF
+    const int nsteps = SINGLE ? min(STEPS, (((k_end - k_begin + 31) >> 5) + PF - 1) / PF * PF) : STEPS;
     const int n_tiles = (N + 15) >> 4;
     // this wave's tiles: group + groups * (wave + 8 j)
     const int t0 = group + groups * wave, t_stride = groups * ST_WAVES;
@@ -102,7 +108,7 @@ __global__ __launch_bounds__(ST_THREADS) void gemm_stationary_kernel(StationaryP
     auto prefetch = [&](SFrag8& dst) {
         const int k = min(k_begin + p_phase * KP + p_step * 32 + g4 * 8, k_end - 8);
         dst.u = *reinterpret_cast<const uint4*>(p_row + k);
-        if (++p_step >= STEPS) {
+        if (++p_step >= nsteps) {
             p_step = 0;
             if (++p_tile >= n_my) { p_tile = 0; ++p_phase; }
             p_row = W + (long)min((t0 + t_stride * p_tile) * 16 + r, N - 1) * K;
@@ -124,8 +130,10 @@ __global__ __launch_bounds__(ST_THREADS) void gemm_stationary_kernel(StationaryP
 
     for (int phase = 0; phase < phases; ++phase) {
         const int buf = phase & 1;
-        load_x(phase + 1);  // in flight while this phase's tiles run; zeros past the last phase
-        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (!SINGLE) {
+            load_x(phase + 1);  // in flight while this phase's tiles run; zeros past the last phase
+            __builtin_amdgcn_sched_barrier(0);
+        }
         // a step's B fragments are read from LDS while the step before it is on the matrix cores: two sets of
         // registers that alternate, and a scheduling barrier per step, without which the compiler reads all of a
         // round's fragments first and runs out of registers
@@ -139,11 +147,11 @@ __global__ __launch_bounds__(ST_THREADS) void gemm_stationary_kernel(StationaryP
 #pragma unroll
         for (int t = 0; t < ST_TMAX; ++t) {
             if (t >= n_my) break;
-            for (int s0 = 0; s0 < STEPS; s0 += PF) {
+            for (int s0 = 0; s0 < nsteps; s0 += PF) {
 #pragma unroll
                 for (int u = 0; u < PF; ++u) {
                     const int next = s0 + u + 1;
-                    read_b(b[(u + 1) & 1], next == STEPS ? 0 : next);  // the next tile starts at the slice's start
+                    read_b(b[(u + 1) & 1], next == nsteps ? 0 : next);  // the next tile starts at the slice's start
 #pragma unroll
                     for (int mt = 0; mt < MT; ++mt)
                         acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u].v, b[u & 1][mt], acc[t][mt], 0, 0, 0);
@@ -152,9 +160,11 @@ __global__ __launch_bounds__(ST_THREADS) void gemm_stationary_kernel(StationaryP
                 }
             }
         }
-        __builtin_amdgcn_sched_barrier(0);
-        store_x(buf ^ 1);
-        __syncthreads();
+        if constexpr (!SINGLE) {
+            __builtin_amdgcn_sched_barrier(0);
+            store_x(buf ^ 1);
+            __syncthreads();
+        }
     }
 
     // lane: row m = mt*16 + r of x, columns tile*16 + g4*4 + 0..3
@@ -184,11 +194,11 @@ static StationaryProblem make_stationary(float* part, const void* x, const void*
     return p;
 }
 
-template <int MT, int KP, int PF, int TMAX>
+template <int MT, int KP, int PF, int TMAX, bool SINGLE = false>
 static int launch_stationary(const StationaryProblem& a, const StationaryProblem& b, int M, hipStream_t s) {
-    constexpr size_t lds = (size_t)2 * MT * 16 * (KP + 8) * sizeof(bf16_t);
+    constexpr size_t lds = (size_t)(SINGLE ? 1 : 2) * MT * 16 * (KP + 8) * sizeof(bf16_t);
     static_assert(lds <= ST_LDS_BYTES, "two slices of x must fit the LDS of a compute unit");
-    auto kern = gemm_stationary_kernel<MT, KP, PF, TMAX>;
+    auto kern = gemm_stationary_kernel<MT, KP, PF, TMAX, SINGLE>;
     if (lds > 64 * 1024) {
         static bool raised = false;
         if (!raised) {
@@ -208,22 +218,37 @@ static int stationary_tmax(int M) { return M <= 64 ? 3 : 2; }
 
 extern "C" int pta_gemm_stationary_groups(int N1, int K1, int parts1, int N2, int K2, int parts2, int M, int* g1, int* g2) {
     const int tmax = stationary_tmax(M);
-    if (N1 <= 0 || K1 <= 0 || N2 <= 0 || K2 <= 0 || parts1 <= 0 || parts2 <= 0)
-        return pta_fail("gemm_stationary_groups: sizes must be positive");
-    // (half as many workgroups, which would read x half as often, take a third longer: a compute unit alone pulls
-    // no more than some 21 GB/s out of memory in this walk)
-    const double units = pta_compute_units(), w1 = (double)N1 * K1, w2 = (double)N2 * K2;
-    const int need1 = ((N1 + 15) / 16 + ST_WAVES * tmax - 1) / (ST_WAVES * tmax);
-    const int need2 = ((N2 + 15) / 16 + ST_WAVES * tmax - 1) / (ST_WAVES * tmax);
-    *g1 = std::max(need1, std::max(1, (int)(units * w1 / (w1 + w2) / parts1 + 0.5)));
-    *g2 = std::max(need2, std::max(1, (int)((units - (double)*g1 * parts1) / parts2 + 0.5)));
+    if (N1 <= 0 || K1 <= 0 || N2 <= 0 || K2 <= 0 || parts1 <= 0 || parts2 <= 0 || parts1 > 64 || parts2 > 64)
+        return pta_fail("gemm_stationary_groups: sizes must be positive, ranges 1 to 64");
+    // Workgroups per range for the two products: as many as the compute units in all and no more (a few workgroups
+    // over start when the first ones end and double the launch's time; half as many, which would read x half as
+    // often, take a third longer: a compute unit alone pulls no more than some 21 GB/s out of memory in this walk),
+    // shared so that the slower kind of workgroup, by its tiles per wave times the length of its range, is as
+    // fast as can be; more than the units only where the tiles a wave can hold ask for it.
+    const int units = pta_compute_units(), t1 = (N1 + 15) / 16, t2 = (N2 + 15) / 16;
+    const int need1 = (t1 + ST_WAVES * tmax - 1) / (ST_WAVES * tmax), need2 = (t2 + ST_WAVES * tmax - 1) / (ST_WAVES * tmax);
+    const double r1 = (double)K1 / parts1, r2 = (double)K2 / parts2;
+    double best = 0.0;
+    *g1 = need1;
+    *g2 = need2;
+    for (int a = need1; a == need1 || a * parts1 + need2 * parts2 <= units; ++a) {
+        const int b = std::max(need2, (units - a * parts1) / parts2);
+        const double rounds = (double)((a * parts1 + b * parts2 + units - 1) / units);
+        const double per1 = (double)((t1 + a - 1) / a) / ST_WAVES * r1, per2 = (double)((t2 + b - 1) / b) / ST_WAVES * r2;
+        const double cost = std::max(per1, per2) * rounds;
+        if (best == 0.0 || cost < best) {
+            best = cost;
+            *g1 = a;
+            *g2 = b;
+        }
+    }
     return 0;
 }
 
 extern "C" int pta_gemm_stationary_pair_bf16(float* part1, const void* x1, const void* W1, int N1, int K1, int parts1,
                                              float* part2, const void* x2, const void* W2, int N2, int K2, int parts2,
                                              int M, void* stream) {
-    PTA_REQUIRE(M > 16 && M <= 128, "gemm_stationary_pair_bf16: 17 to 128 rows, got %d", M);
+    PTA_REQUIRE(M >= 1 && M <= 128, "gemm_stationary_pair_bf16: 1 to 128 rows, got %d", M);
     PTA_REQUIRE(N1 > 0 && K1 > 0 && N2 > 0 && K2 > 0, "gemm_stationary_pair_bf16: sizes must be positive");
     PTA_REQUIRE(K1 % 8 == 0 && K2 % 8 == 0, "gemm_stationary_pair_bf16: K must be a multiple of 8 (16-byte loads)");
     PTA_REQUIRE(part1 && part2 && x1 && x2 && W1 && W2, "gemm_stationary_pair_bf16: null pointer");
@@ -237,7 +262,17 @@ extern "C" int pta_gemm_stationary_pair_bf16(float* part1, const void* x1, const
     const StationaryProblem a = make_stationary(part1, x1, W1, N1, K1, parts1, g1);
     const StationaryProblem b = make_stationary(part2, x2, W2, N2, K2, parts2, g2);
     hipStream_t s = (hipStream_t)stream;
+    // ranges of K that fit LDS whole run as one phase
+    const int longest = std::max(a.blocks_per_part, b.blocks_per_part) * 64;
     switch ((M + 15) / 16) {
+        case 1: if (longest <= 4608) return launch_stationary<1, 4608, 8, 3, true>(a, b, M, s); break;
+        case 2: if (longest <= 2304) return launch_stationary<2, 2304, 8, 3, true>(a, b, M, s); break;
+        case 3: if (longest <= 1536) return launch_stationary<3, 1536, 8, 3, true>(a, b, M, s); break;
+        case 4: if (longest <= 1152) return launch_stationary<4, 1152, 12, 3, true>(a, b, M, s); break;
+        default: break;
+    }
+    switch ((M + 15) / 16) {
+        case 1: return launch_stationary<1, 2048, 8, 3>(a, b, M, s);
         case 2: return launch_stationary<2, 1024, 8, 3>(a, b, M, s);
         case 3: return launch_stationary<3, 768, 8, 3>(a, b, M, s);
         case 4: return launch_stationary<4, 512, 8, 3>(a, b, M, s);

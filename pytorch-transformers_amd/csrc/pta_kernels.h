@@ -150,17 +150,18 @@ int pta_gemm_splitk_pair_fix_parts(int N1, int K1, int N2, int K2, int p1, int p
 // the same, and how many tiles of sixteen rows of W a wave holds in steps of more than 32 rows (rt 1 or 2, i.e. 64
 // or 128 rows of W a workgroup); the ranges decide the order of summation, the tile height does not
 int pta_gemm_splitk_pair_fix(int N1, int K1, int N2, int K2, int p1, int p2, int rt);
-// The same two partial products for 17 to 128 rows with the activations stationary (gemm_stationary_bf16.hip):
+// The same two partial products for 1 to 128 rows with the activations stationary (gemm_stationary_bf16.hip):
 // about one workgroup per compute unit, each wave keeping the sums of its row tiles in registers while the
 // workgroup walks its range of K in phases of LDS-resident slices of x.  parts1 and parts2 ranges of K
 // (part1 [parts1, M, N1], part2 [parts2, M, N2], ranges of whole 64-element blocks as in the launches above).
 int pta_gemm_stationary_groups(int N1, int K1, int parts1, int N2, int K2, int parts2, int M, int* g1, int* g2);
 int pta_gemm_stationary_pair_bf16(float* part1, const void* x1, const void* W1, int N1, int K1, int parts1, float* part2,
                                   const void* x2, const void* W2, int N2, int K2, int parts2, int M, void* stream);
-// fixes the ranges of K of the pair launch with stationary activations and the rows from which it is used, up to
-// 128 (17 to 129; 129: never); 0, 0 returns the shape to the rule (pta_gemm_stationary_rule); returns 1 for invalid counts
-int pta_gemm_splitk_pair_fix_stationary(int N1, int K1, int N2, int K2, int q1, int q2, int from_rows);
-int pta_gemm_stationary_rule(int K1, int K2, int* q1, int* q2, int* from_rows);
+// The pair launch with stationary activations has ranges of K of its own per class of rows (0: up to 16 rows, 1:
+// 32, 2: 64, 3: 128): pta_gemm_stationary_rule gives the rule's, pta_gemm_splitk_pair_fix_stationary fixes them for
+// a shape and class (0, 0: the staged kernel for that class; cls = -1 forgets the shape; returns 1 for invalid counts).
+int pta_gemm_splitk_pair_fix_stationary(int N1, int K1, int N2, int K2, int cls, int q1, int q2);
+int pta_gemm_stationary_rule(int N1, int K1, int N2, int K2, int cls, int* q1, int* q2);
 int pta_gemm_splitk_pair_bf16(float* part1, const void* x1, const void* W1, int N1, int K1, float* part2,
                               const void* x2, const void* W2, int N2, int K2, int M, void* stream);
 

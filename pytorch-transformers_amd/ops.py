@@ -986,11 +986,15 @@ def gemm_splitk_pair_parts(N1: int, K1: int, N2: int, K2: int, M: int = 0):
     return p1.value, p2.value
 
 
-def gemm_stationary_rule(K1: int, K2: int):
-    """(ranges, ranges, rows from which it is used) of the pair launch with stationary activations, by the rule."""
-    q1, q2, rows = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(0)
-    _call("pta_gemm_stationary_rule", int(K1), int(K2), ctypes.byref(q1), ctypes.byref(q2), ctypes.byref(rows))
-    return q1.value, q2.value, rows.value
+STATIONARY_CLASS_ROWS = (16, 32, 64, 128)  # a pair launch's rows count by the first of these that holds them
+
+
+def gemm_stationary_rule(N1: int, K1: int, N2: int, K2: int, cls: int):
+    """(ranges, ranges) of K of the pair launch with stationary activations for rows of class ``cls`` (the index
+    into ``STATIONARY_CLASS_ROWS``), by the rule."""
+    q1, q2 = ctypes.c_int(0), ctypes.c_int(0)
+    _call("pta_gemm_stationary_rule", int(N1), int(K1), int(N2), int(K2), int(cls), ctypes.byref(q1), ctypes.byref(q2))
+    return q1.value, q2.value
 
 
 # Ranges of K for the pairs of a shape: the kernel library's rule gives a choice; when timing is on, its neighbours
@@ -1000,9 +1004,8 @@ PAIR_TUNE = os.environ.get("PTA_PAIR_TUNE", "1") != "0"
 PAIR_TUNE_MARGIN = 0.97
 PAIR_TUNE_ROWS = int(os.environ.get("PTA_PAIR_TUNE_ROWS", "64"))  # rows of the timed launches (17 to 128)
 _pair_parts_tuned: dict = {}  # (shape of w1, shape of w2) -> the counts in use
-_pair_stationary_tuned: dict = {}  # (shape of w1, shape of w2) -> (ranges, ranges, rows from which) of the launch
-#                                    with stationary activations (it runs up to 128 rows); 129 rows: never
-STATIONARY_NEVER = 129
+_pair_stationary_tuned: dict = {}  # (shape of w1, shape of w2) -> per class of rows the (ranges, ranges) of the
+#                                    launch with stationary activations, (0, 0) where the staged kernel stays
 
 
 def tune_pair_parts(w1: torch.Tensor, w2: torch.Tensor) -> None:
@@ -1011,9 +1014,9 @@ def tune_pair_parts(w1: torch.Tensor, w2: torch.Tensor) -> None:
     workgroups and so want more ranges), at 64 rows with cold caches; keep the fastest in the kernel library if it
     beats the rule's by the margin and is no slower than the rule's at 24 rows (where the tile height does not
     apply, but the ranges do).  ``_pair_parts_tuned`` says what is in use: (ranges, ranges, row tiles per wave).
-    Then the launch with stationary activations is timed against the winner, with its rule's ranges and their
-    neighbours, at 64 and at 40 rows: it is used from 33 rows on, from 49 on, or never, by what those say
-    (``_pair_stationary_tuned``: ranges, ranges, rows from which)."""
+    Then, at 8, 32, 64 and 128 rows (one count per class of rows), the launch with stationary activations is timed
+    against the winner with one to six ranges of the shorter K (and as many times more of the longer): the
+    fastest is fixed for the class, or the staged kernel where that is not beaten by 2 % (``_pair_stationary_tuned``)."""
     key = (tuple(w1.shape), tuple(w2.shape))
     if not PAIR_TUNE or key in _pair_parts_tuned or not _may_time():
         return
@@ -1022,21 +1025,22 @@ def tune_pair_parts(w1: torch.Tensor, w2: torch.Tensor) -> None:
     a0, b0 = gemm_splitk_pair_parts(N1, K1, N2, K2)
     fix = lambda c: lib.pta_gemm_splitk_pair_fix(int(N1), int(K1), int(N2), int(K2), int(c[0]), int(c[1]), int(c[2]))
     forget = lambda: lib.pta_gemm_splitk_pair_fix(int(N1), int(K1), int(N2), int(K2), 0, 0, 1)
-    fix_st = lambda c: lib.pta_gemm_splitk_pair_fix_stationary(int(N1), int(K1), int(N2), int(K2), int(c[0]), int(c[1]), int(c[2]))
-    q1, q2, from0 = gemm_stationary_rule(K1, K2)
-    fix_st((q1, q2, STATIONARY_NEVER))  # the launches timed first are the staged kernel's
+    fix_st = lambda cls, c: lib.pta_gemm_splitk_pair_fix_stationary(int(N1), int(K1), int(N2), int(K2), int(cls), int(c[0]), int(c[1]))
+    for cls in range(len(STATIONARY_CLASS_ROWS)):
+        fix_st(cls, (0, 0))  # the launches timed first are the staged kernel's
     cands = [(a0, b0, 1)] + [(a, b, 1) for a in range(max(1, a0 - 1), a0 + 3) for b in range(max(1, b0 - 2), b0 + 3)
                              if (a, b) != (a0, b0)]
     tall = lambda p: sorted({max(1, p - 1), p, p + 1, max(1, 2 * p - 1), 2 * p, 2 * p + 1})
     cands += [(a, b, 2) for a in tall(a0) for b in tall(b0)]
     cands = [c for c in cands if fix(c) == 0]
     xs = {rows: [torch.randn((rows, K), dtype=torch.float32, device=w1.device).to(torch.bfloat16) for K in (K1, K2)]
-          for rows in (PAIR_TUNE_ROWS, 24, 40)}
-    st_cands = [(q1, q2)] + [c for c in ((q1, 2 * q2), (2 * q1, 2 * q2), (q1, max(1, q2 // 2)), (2 * q1, q2))
-                             if c != (q1, q2) and fix_st(c + (STATIONARY_NEVER,)) == 0]
-    st_cands = list(dict.fromkeys(st_cands))
-    most = [max([c[i] for c in cands] + [c[i] for c in st_cands]) for i in (0, 1)]
-    parts = [torch.empty((most[i], PAIR_TUNE_ROWS, N), dtype=torch.float32, device=w1.device) for i, N in enumerate((N1, N2))]
+          for rows in sorted({PAIR_TUNE_ROWS, 24, 8, 32, 64, 128})}
+    kmin = min(K1, K2)
+    f1, f2 = max(1, (K1 + kmin // 2) // kmin), max(1, (K2 + kmin // 2) // kmin)
+    st_cands = [(b * f1, b * f2) for b in (1, 2, 3, 4, 6) if b * f1 <= 16 and b * f2 <= 16 and fix_st(0, (b * f1, b * f2)) == 0]
+    fix_st(0, (0, 0))
+    most = [max([c[i] for c in cands] + [c[i] for c in st_cands] + [16]) for i in (0, 1)]
+    parts = [torch.empty((most[i], 128, N), dtype=torch.float32, device=w1.device) for i, N in enumerate((N1, N2))]
     # A launch is timed over several copies of the matrices in turn (more bytes than the memory-side cache holds),
     # back to back between two events: every launch reads its matrices from memory, as in a model, and no gap of
     # the host's lies inside the timed span.
@@ -1080,26 +1084,25 @@ def tune_pair_parts(w1: torch.Tensor, w2: torch.Tensor) -> None:
     if chosen != cands[0]:
         fix(chosen)
     _pair_parts_tuned[key] = chosen
-    # the launch with stationary activations against that choice, where both apply
-    stationary = (q1, q2, STATIONARY_NEVER)
-    if PAIR_TUNE_ROWS == 64:
-        try:
-            t64 = times[cands.index(chosen)]
-            s64 = timed_ways([c + (17,) for c in st_cands], 64, fix=fix_st)
-            best = min(range(len(st_cands)), key=lambda i: s64[i])
-            if s64[best] < 0.98 * t64:
-                fix_st(st_cands[best] + (STATIONARY_NEVER,))
-                t40 = timed_ways([chosen], 40)[0]
-                s40 = timed_ways([st_cands[best] + (17,)], 40, fix=fix_st)[0]
-                stationary = st_cands[best] + (33 if s40 < 0.98 * t40 else 49,)
+    # the launch with stationary activations against that choice, per class of rows
+    chosen_st = []
+    try:
+        for cls, rows in enumerate((8, 32, 64, 128)):
+            fix_st(cls, (0, 0))
+            t_staged = timed_ways([chosen], rows)[0]
+            t_st = timed_ways([(cls, c) for c in st_cands], rows, fix=lambda a: fix_st(a[0], a[1])) if st_cands else []
+            best = min(range(len(st_cands)), key=lambda i: t_st[i]) if st_cands else -1
+            keep = st_cands[best] if best >= 0 and t_st[best] < 0.98 * t_staged else (0, 0)
+            chosen_st.append(keep)
             if os.environ.get("PTA_TUNE_VERBOSE"):
-                print(f"[pta tune] pair {key} with stationary activations: " +
-                      ", ".join(f"{c} {t * 1e3:.1f}" for c, t in zip(st_cands, s64)) + f" us against {t64 * 1e3:.1f} at 64 rows"
-                      + (f"; {s40 * 1e3:.1f} against {t40 * 1e3:.1f} at 40 rows" if stationary[2] != STATIONARY_NEVER else "")
-                      + f" -> {stationary}", flush=True)
-        finally:
-            fix_st(stationary)
-    _pair_stationary_tuned[key] = stationary
+                print(f"[pta tune] pair {key} at {rows} rows: staged {t_staged * 1e3:.1f} us; stationary " +
+                      ", ".join(f"{c} {t * 1e3:.1f}" for c, t in zip(st_cands, t_st)) + f" -> {keep}", flush=True)
+    finally:
+        while len(chosen_st) < len(STATIONARY_CLASS_ROWS):
+            chosen_st.append((0, 0))
+        for cls, c in enumerate(chosen_st):
+            fix_st(cls, c)
+    _pair_stationary_tuned[key] = tuple(chosen_st)
 
 
 def tuning_table() -> dict:
@@ -1108,7 +1111,7 @@ def tuning_table() -> dict:
     key = lambda t: ",".join("x".join(str(int(v)) for v in (p if isinstance(p, tuple) else (p,))) for p in t)
     return {
         "pair_parts": {key(k): list(v) for k, v in _pair_parts_tuned.items()},  # ranges, ranges, row tiles per wave
-        "pair_stationary": {key(k): list(v) for k, v in _pair_stationary_tuned.items()},  # ranges, ranges, rows from
+        "pair_stationary": {key(k): [list(c) for c in v] for k, v in _pair_stationary_tuned.items()},  # per class of rows
         "splitk_rows": {key(k): int(v) for k, v in _splitk_limits.items()},
         "mm_plans": {key(k): list(v) for k, v in _mm_plans.items()},
         "mm_joined": {key(k): bool(v) for k, v in _mm_joined.items()},
@@ -1123,7 +1126,7 @@ def clear_tuning() -> None:
     for (s1, s2) in list(_pair_parts_tuned):
         lib.pta_gemm_splitk_pair_fix(int(s1[0]), int(s1[1]), int(s2[0]), int(s2[1]), 0, 0, 1)
     for (s1, s2) in list(_pair_stationary_tuned):
-        lib.pta_gemm_splitk_pair_fix_stationary(int(s1[0]), int(s1[1]), int(s2[0]), int(s2[1]), 0, 0, 0)
+        lib.pta_gemm_splitk_pair_fix_stationary(int(s1[0]), int(s1[1]), int(s2[0]), int(s2[1]), -1, 0, 0)
     for d in (_pair_stationary_tuned, _pair_parts_tuned, _splitk_limits, _mm_plans, _mm_costs, _mm_times, _mm_joined, _mm_ksplit, _decode_plans):
         d.clear()
 
@@ -1142,9 +1145,10 @@ def load_tuning(table: dict) -> None:
         _pair_parts_tuned[(s1, s2)] = (a, b, rt)
     for k, v in table.get("pair_stationary", {}).items():
         s1, s2 = shapes(k)
-        if lib.pta_gemm_splitk_pair_fix_stationary(s1[0], s1[1], s2[0], s2[1], int(v[0]), int(v[1]), int(v[2])):
-            raise KernelError(f"tuning table: {list(v)} is not valid for the pair {k} with stationary activations")
-        _pair_stationary_tuned[(s1, s2)] = (int(v[0]), int(v[1]), int(v[2]))
+        for cls, c in enumerate(v):
+            if lib.pta_gemm_splitk_pair_fix_stationary(s1[0], s1[1], s2[0], s2[1], cls, int(c[0]), int(c[1])):
+                raise KernelError(f"tuning table: {list(c)} is not valid for the pair {k} with stationary activations")
+        _pair_stationary_tuned[(s1, s2)] = tuple((int(c[0]), int(c[1])) for c in v)
     for k, v in table.get("splitk_rows", {}).items():
         _splitk_limits[shapes(k)] = int(v)
     for k, v in table.get("mm_plans", {}).items():

@@ -269,10 +269,11 @@ def test_pair_ranges_are_timed_once_per_shape_and_kept():
     assert ops.gemm_splitk_pair_parts(N1, K1, N2, K2) == rule
 
 
-@pytest.mark.parametrize("M", [17, 32, 33, 47, 48, 49, 64, 65, 96, 100, 128])
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 32, 33, 47, 48, 49, 64, 65, 96, 100, 128])
 @pytest.mark.parametrize("shapes,parts", [(((1000, 520), (344, 1096)), (1, 1)), (((1000, 520), (344, 1096)), (2, 3)),
                                           (((40, 72), (1608, 2304)), (1, 2)), (((4672, 4544), (512, 8192)), (1, 2)),
-                                          (((24, 8), (16, 4104)), (1, 16))])
+                                          (((24, 8), (16, 4104)), (1, 16)), (((1000, 4608), (40, 1152)), (1, 1)),
+                                          (((200, 1536), (48, 2304)), (1, 1)), (((4672, 4544), (4544, 4544)), (3, 3))])
 def test_gemm_stationary_pair(M, shapes, parts):
     """The pair launch with stationary activations, called on its own: every count of sixteen-row tiles of x, K
     that ends inside a block, a phase and a 32-element step, N that ends inside a tile, more row tiles than the
@@ -300,9 +301,9 @@ def test_gemm_stationary_pair(M, shapes, parts):
 
 
 def test_gemm_stationary_pair_refusals_and_dispatch():
-    """Rows outside 17..128 are refused with a message; a pair launch of 49 to 128 rows
-    runs with stationary activations and the ranges the library reports for those rows, one of 48 rows does not,
-    and the rows from which it does can be fixed per shape and forgotten."""
+    """Rows beyond 128 are refused with a message; a pair launch of up to 128 rows runs with stationary activations
+    and the ranges the library reports for the class of its rows; a class can be fixed to other ranges or to the
+    staged kernel per shape, and forgotten; partial sums add up to the product either way."""
     import ctypes
 
     ops = _ops()
@@ -311,34 +312,41 @@ def test_gemm_stationary_pair_refusals_and_dispatch():
     P = lambda t: ctypes.c_void_p(t.data_ptr())
     stream = lambda: ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     w1, w2 = _rand(N1, K1, seed=1, dtype=torch.bfloat16, scale=0.05), _rand(N2, K2, seed=2, dtype=torch.bfloat16, scale=0.05)
-    for M in (16, 129):
-        x1, x2 = _rand(M, K1, dtype=torch.bfloat16), _rand(M, K2, seed=5, dtype=torch.bfloat16)
-        part = torch.empty(4, M, 328).cuda()
+    for M in (0, 129):
+        x1, x2 = _rand(max(M, 1), K1, dtype=torch.bfloat16), _rand(max(M, 1), K2, seed=5, dtype=torch.bfloat16)
+        part = torch.empty(4, max(M, 1), 328).cuda()
         assert lib.pta_gemm_stationary_pair_bf16(P(part), P(x1), P(w1), N1, K1, 1, P(part), P(x2), P(w2), N2, K2, 1, M, stream()) != 0
-        assert "17 to 128 rows" in lib.pta_last_error().decode()
-    q1, q2, rows = ops.gemm_stationary_rule(K1, K2)
-    assert (q1, q2, rows) == (1, 2, 49)
+        assert "1 to 128 rows" in lib.pta_last_error().decode()
     staged = ops.gemm_splitk_pair_parts(N1, K1, N2, K2)
-    assert ops.gemm_splitk_pair_parts(N1, K1, N2, K2, 48) == staged and ops.gemm_splitk_pair_parts(N1, K1, N2, K2, 129) == staged
-    assert ops.gemm_splitk_pair_parts(N1, K1, N2, K2, 49) == (q1, q2) == ops.gemm_splitk_pair_parts(N1, K1, N2, K2, 128)
-    for M in (48, 49, 64, 100, 128):
+    rules = [ops.gemm_stationary_rule(N1, K1, N2, K2, cls) for cls in range(4)]
+    assert all(q1 >= 1 and q2 >= q1 for q1, q2 in rules), rules  # the longer K has at least as many ranges
+    for cls, top in enumerate(ops.STATIONARY_CLASS_ROWS):  # without a fixed choice: from 33 rows on
+        assert ops.gemm_splitk_pair_parts(N1, K1, N2, K2, top) == (rules[cls] if cls >= 2 else staged)
+    assert ops.gemm_splitk_pair_parts(N1, K1, N2, K2, 129) == staged
+
+    def check(M):
         x1, x2 = _rand(M, K1, dtype=torch.bfloat16), _rand(M, K2, seed=5, dtype=torch.bfloat16)
         a, b = ops.gemm_splitk_pair_partial(x1, w1, x2, w2)
         assert (a.shape[0], b.shape[0]) == ops.gemm_splitk_pair_parts(N1, K1, N2, K2, M)
         for part, x, w in ((a, x1, w1), (b, x2, w2)):
             want = x.double() @ w.double().T
             assert float((part.double().sum(0) - want).abs().max()) <= 2e-5 * float(want.abs().max())
+
+    for M in (1, 8, 16, 17, 48, 64, 100, 128, 129):
+        check(M)
+    fix = lib.pta_gemm_splitk_pair_fix_stationary
     try:
-        assert lib.pta_gemm_splitk_pair_fix_stationary(N1, K1, N2, K2, 2, 4, 33) == 0
-        assert ops.gemm_splitk_pair_parts(N1, K1, N2, K2, 33) == (2, 4) and ops.gemm_splitk_pair_parts(N1, K1, N2, K2, 32) == staged
-        assert lib.pta_gemm_splitk_pair_fix_stationary(N1, K1, N2, K2, 1, 1, ops.STATIONARY_NEVER) == 0
-        assert ops.gemm_splitk_pair_parts(N1, K1, N2, K2, 64) == staged == ops.gemm_splitk_pair_parts(N1, K1, N2, K2, 128)
-        assert lib.pta_gemm_splitk_pair_fix_stationary(N1, K1, N2, K2, 1, 1, 130) != 0
-        assert lib.pta_gemm_splitk_pair_fix_stationary(N1, K1, N2, K2, 1, 1, 16) != 0
-        assert lib.pta_gemm_splitk_pair_fix_stationary(N1, K1, N2, K2, 0, 1, 33) != 0
+        assert fix(N1, K1, N2, K2, 1, 2, 4) == 0
+        assert ops.gemm_splitk_pair_parts(N1, K1, N2, K2, 20) == (2, 4) and ops.gemm_splitk_pair_parts(N1, K1, N2, K2, 16) == staged
+        assert fix(N1, K1, N2, K2, 0, 1, 1) == 0 and ops.gemm_splitk_pair_parts(N1, K1, N2, K2, 8) == (1, 1)
+        assert fix(N1, K1, N2, K2, 2, 0, 0) == 0
+        assert ops.gemm_splitk_pair_parts(N1, K1, N2, K2, 64) == staged and ops.gemm_splitk_pair_parts(N1, K1, N2, K2, 65) == rules[3]
+        for M in (8, 20, 64):
+            check(M)
+        assert fix(N1, K1, N2, K2, 4, 1, 1) != 0 and fix(N1, K1, N2, K2, 1, 0, 1) != 0 and fix(N1, K1, N2, K2, 1, 17, 1) != 0
     finally:
-        lib.pta_gemm_splitk_pair_fix_stationary(N1, K1, N2, K2, 0, 0, 0)
-    assert ops.gemm_splitk_pair_parts(N1, K1, N2, K2, 64) == (q1, q2)
+        fix(N1, K1, N2, K2, -1, 0, 0)
+    assert ops.gemm_splitk_pair_parts(N1, K1, N2, K2, 64) == rules[2]
 
 
 def test_gemm_splitk_pair():
