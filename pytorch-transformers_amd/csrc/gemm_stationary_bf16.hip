@@ -18,6 +18,7 @@
 #include "pta_kernels.h"
 
 #include <algorithm>
+#include <type_traits>
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
@@ -128,43 +129,64 @@ __global__ __launch_bounds__(ST_THREADS) void gemm_stationary_kernel(StationaryP
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) acc[t][mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-    for (int phase = 0; phase < phases; ++phase) {
-        const int buf = phase & 1;
-        if constexpr (!SINGLE) {
-            load_x(phase + 1);  // in flight while this phase's tiles run; zeros past the last phase
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        // a step's B fragments are read from LDS while the step before it is on the matrix cores: two sets of
-        // registers that alternate, and a scheduling barrier per step, without which the compiler reads all of a
-        // round's fragments first and runs out of registers
-        bf16x8_t b[2][MT];
-        auto read_b = [&](bf16x8_t(&dst)[MT], int step) {
+    // The phases for a wave with NT tiles, NT known when the kernel is compiled: the next phase's slice of x is asked
+    // for at the start of the wave's last round of steps of the phase and written to LDS at the phase's end, so
+    // that the compiler can count the W loads that are younger than it (one round's) and lets the wave wait for
+    // the slice alone.  Asked for at the phase's start, a loop of unknown length lies between the slice's loads
+    // and their use, the count is unknown, and the wave waits for every load it has in flight, W rows included,
+    // at every phase's end.
+    auto run = [&](auto tiles_c) {
+        constexpr int NT = decltype(tiles_c)::value;
+        for (int phase = 0; phase < phases; ++phase) {
+            const int buf = phase & 1;
+            // a step's B fragments are read from LDS while the step before it is on the matrix cores: two sets of
+            // registers that alternate, and a scheduling barrier per step, without which the compiler reads all of
+            // a round's fragments first and runs out of registers
+            bf16x8_t b[2][MT];
+            auto read_b = [&](bf16x8_t(&dst)[MT], int step) {
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
-                dst[mt] = *reinterpret_cast<const bf16x8_t*>(&xs[(buf * MP + mt * 16 + r) * LDW + step * 32 + g4 * 8]);
-        };
-        read_b(b[0], 0);
+                for (int mt = 0; mt < MT; ++mt)
+                    dst[mt] = *reinterpret_cast<const bf16x8_t*>(&xs[(buf * MP + mt * 16 + r) * LDW + step * 32 + g4 * 8]);
+            };
+            if constexpr (NT == 0 && !SINGLE) load_x(phase + 1);
+            if constexpr (NT > 0) read_b(b[0], 0);
 #pragma unroll
-        for (int t = 0; t < ST_TMAX; ++t) {
-            if (t >= n_my) break;
-            for (int s0 = 0; s0 < nsteps; s0 += PF) {
+            for (int t = 0; t < NT; ++t) {
+                auto round = [&](int s0) {
 #pragma unroll
-                for (int u = 0; u < PF; ++u) {
-                    const int next = s0 + u + 1;
-                    read_b(b[(u + 1) & 1], next == nsteps ? 0 : next);  // the next tile starts at the slice's start
+                    for (int u = 0; u < PF; ++u) {
+                        const int next = s0 + u + 1;
+                        read_b(b[(u + 1) & 1], next == nsteps ? 0 : next);  // the next tile starts at the slice's start
 #pragma unroll
-                    for (int mt = 0; mt < MT; ++mt)
-                        acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u].v, b[u & 1][mt], acc[t][mt], 0, 0, 0);
-                    prefetch(w[u]);
-                    __builtin_amdgcn_sched_barrier(0);
+                        for (int mt = 0; mt < MT; ++mt)
+                            acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u].v, b[u & 1][mt], acc[t][mt], 0, 0, 0);
+                        prefetch(w[u]);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                };
+                for (int s0 = 0; s0 < nsteps - PF; s0 += PF) round(s0);
+                if constexpr (!SINGLE) {
+                    if (t == NT - 1) {
+                        load_x(phase + 1);  // zeros past the last phase
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
                 }
+                round(nsteps - PF);
+            }
+            if constexpr (!SINGLE) {
+                __builtin_amdgcn_sched_barrier(0);
+                store_x(buf ^ 1);
+                __syncthreads();
             }
         }
-        if constexpr (!SINGLE) {
-            __builtin_amdgcn_sched_barrier(0);
-            store_x(buf ^ 1);
-            __syncthreads();
-        }
+    };
+    switch (n_my) {
+        case 0: run(std::integral_constant<int, 0>{}); break;
+        case 1: run(std::integral_constant<int, 1>{}); break;
+        case 2: run(std::integral_constant<int, 2>{}); break;
+        default:
+            if constexpr (ST_TMAX >= 3) run(std::integral_constant<int, 3>{});
+            break;
     }
 
     // lane: row m = mt*16 + r of x, columns tile*16 + g4*4 + 0..3
