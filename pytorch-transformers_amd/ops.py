@@ -1015,8 +1015,8 @@ def tune_pair_parts(w1: torch.Tensor, w2: torch.Tensor) -> None:
     beats the rule's by the margin and is no slower than the rule's at 24 rows (where the tile height does not
     apply, but the ranges do).  ``_pair_parts_tuned`` says what is in use: (ranges, ranges, row tiles per wave).
     Then, at 8, 32, 64 and 128 rows (one count per class of rows), the launch with stationary activations is timed
-    against the winner with one to six ranges of the shorter K (and as many times more of the longer): the
-    fastest is fixed for the class, or the staged kernel where that is not beaten by 2 % (``_pair_stationary_tuned``)."""
+    against the winner with one to six ranges of the shorter K (and as many times more of the longer), each
+    charged for the partial sums that its ranges leave to be read: the fastest is fixed for the class, or the staged kernel where that is not beaten by 2 % (``_pair_stationary_tuned``)."""
     key = (tuple(w1.shape), tuple(w2.shape))
     if not PAIR_TUNE or key in _pair_parts_tuned or not _may_time():
         return
@@ -1089,13 +1089,17 @@ def tune_pair_parts(w1: torch.Tensor, w2: torch.Tensor) -> None:
     try:
         for cls, rows in enumerate((8, 32, 64, 128)):
             fix_st(cls, (0, 0))
-            t_staged = timed_ways([chosen], rows)[0]
+            # what reads the partial sums afterwards pays for every range (measured: some 8 TB/s worth of them), so
+            # a launch is charged for its ranges' bytes at that rate on top of its own time
+            slices_ms = lambda c: (c[0] * N1 + c[1] * N2) * rows * 4 / 8e12 * 1e3
+            t_staged = timed_ways([chosen], rows)[0] + slices_ms(chosen)
             t_st = timed_ways([(cls, c) for c in st_cands], rows, fix=lambda a: fix_st(a[0], a[1])) if st_cands else []
+            t_st = [t + slices_ms(c) for t, c in zip(t_st, st_cands)]
             best = min(range(len(st_cands)), key=lambda i: t_st[i]) if st_cands else -1
             keep = st_cands[best] if best >= 0 and t_st[best] < 0.98 * t_staged else (0, 0)
             chosen_st.append(keep)
             if os.environ.get("PTA_TUNE_VERBOSE"):
-                print(f"[pta tune] pair {key} at {rows} rows: staged {t_staged * 1e3:.1f} us; stationary " +
+                print(f"[pta tune] pair {key} at {rows} rows (with the reading of the partial sums): staged {t_staged * 1e3:.1f} us; stationary " +
                       ", ".join(f"{c} {t * 1e3:.1f}" for c, t in zip(st_cands, t_st)) + f" -> {keep}", flush=True)
     finally:
         while len(chosen_st) < len(STATIONARY_CLASS_ROWS):
