@@ -10,6 +10,7 @@
 //   S^T[32 keys x 16 cols]  = K[32 x d] . Q^T[d x 16]         (A = key rows, B = query columns)
 //   online softmax over keys, per column (statistics in 32-bit, four lanes hold a column)
 //   O^T[d x 16 cols]       += V^T[d x 32 keys] . P^T[32 x 16]  (A = value pages, stored transposed)
+//   l[16 cols]             += 1[16 x 32] . P^T[32 x 16]        (the sums of the weights, as they were rounded)
 //
 // The score tile's accumulator layout (lane: column = lane % 16, four consecutive rows at
 // (lane / 16) * 4) is turned into the B operand of the second product without leaving registers:
@@ -31,6 +32,7 @@
 
 #include <algorithm>
 #include <cmath>
+#include <type_traits>
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
@@ -101,8 +103,10 @@ __device__ __forceinline__ void load_block(KvBlock<DT>& b, int kb, const int* __
 // WIN: the launch has a window (a kernel of its own, so that launches without one pay nothing for it).
 // KS > 1 (one token per sequence): KS waves of a workgroup hold the same columns and take every KS-th block of the
 // workgroup's keys; their partial results meet in LDS, so that a context walked by KS waves needs no second launch.
-template <int DT, int CT, int W, bool WIN, int KS = 1>
-__global__ __launch_bounds__(64 * W * KS) void attn_mfma_kernel(
+// AL: whether there is ALiBi, known when the kernel is compiled (0: none, 1: there is) or looked up (2).
+// OCC: waves that a SIMD is to hold at least (the registers a wave may use follow from it; 1: as many as it likes).
+template <int DT, int CT, int W, bool WIN, int KS = 1, int AL = 2, int OCC = 1>
+__global__ __launch_bounds__(64 * W * KS, OCC) void attn_mfma_kernel(
     bf16_t* __restrict__ out, float* __restrict__ po, float* __restrict__ pm, float* __restrict__ pl,
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
     const int* __restrict__ block_table, int bt_stride, const int* __restrict__ cu_tokens,
@@ -115,7 +119,7 @@ __global__ __launch_bounds__(64 * W * KS) void attn_mfma_kernel(
     constexpr int CHUNKS = D / 8;      // 16-byte chunks in a row of d elements
     static_assert(KS == 1 || W == 1, "waves either share key blocks or divide them");
     const int lane = threadIdx.x & 63, c = lane & 15, gq = lane >> 4;
-    const int wave = KS > 1 ? 0 : threadIdx.x >> 6;   // which columns of the workgroup
+    const int wave = KS > 1 ? 0 : __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // which columns of the workgroup
     const int kw = KS > 1 ? threadIdx.x >> 6 : 0;     // which blocks of the keys
     const int seq = blockIdx.z / n_splits, split = blockIdx.z % n_splits;
     const int kvh = blockIdx.y, g = nh / nkv;
@@ -173,116 +177,157 @@ __global__ __launch_bounds__(64 * W * KS) void attn_mfma_kernel(
         }
     }
 
-    f32x4_t oacc[DT][CT];
-    float m_run[CT], l_run[CT];
+    // The sum of a column's weights is one more product: a tile of ones in the place of the values adds the
+    // block's (rounded) weights of every column into lacc, whose sixteen rows all hold the same sums.  The
+    // vector units, which bound this kernel, are spared eight additions a tile; the matrix cores take a ninth
+    // instruction beside eight.
+    f32x4_t oacc[DT][CT], lacc[CT];
+    float m_run[CT], m_raise[CT];  // m_raise: the raw score above which the running maximum is brought up
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
         m_run[ct] = -INFINITY;
-        l_run[ct] = 0.f;
+        m_raise[ct] = -INFINITY;
+        lacc[ct] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) oacc[dt][ct] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     }
+    AFrag ones;
+    ones.u = make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u);
 
     const int* bt = block_table + (long)seq * bt_stride;
 
-    // scores, softmax update and value product of the block at kb (a block past k_end changes nothing)
-    auto use_block = [&](KvBlock<DT>& b, int kb) {
-        if (kb + 32 > kv_len || kb >= k_end) {
-            // positions past the sequence's end were never written; whatever lies there must not reach the
-            // sum, not even with weight zero.  A block past this wave's range was loaded from a clamped
-            // address and is dropped whole.
-            const int kbase = kb + gq * 8;
-            const int lim = kb >= k_end ? 0 : kv_len;
-            uint32_t mk[4];
+    // AL says at compile time whether there is ALiBi (0: none, 1: there is; 2: whatever the launch brings), so
+    // that the kernels for prompts, which are bound by their instruction stream, branch on nothing in it.
+    const bool has_alibi = AL == 2 ? slopes != nullptr : AL == 1;
+    // Scores are kept in units of log 2 (the scale carries log2 e), so that the exponential is the hardware's
+    // exp2.  Without ALiBi the products are left unscaled, and the scale rides in the one multiply-add in front
+    // of the exponential: s_mul is what a settled score is still to be multiplied by (positive).
+    const float s_mul = has_alibi ? 1.0f : scale;
+
+    // The work on a block of 32 keys, in the four pieces that the loops below put together:
+    // the products S^T = K . Q^T of the block, raw
+    auto scores = [&](const AFrag (&k)[2][DS], f32x4_t (&sacc)[2][CT]) {
 #pragma unroll
-            for (int w = 0; w < 4; ++w)
-                mk[w] = (kbase + 2 * w < lim ? 0x0000ffffu : 0u) | (kbase + 2 * w + 1 < lim ? 0xffff0000u : 0u);
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                b.v[dt].u.x &= mk[0]; b.v[dt].u.y &= mk[1]; b.v[dt].u.z &= mk[2]; b.v[dt].u.w &= mk[3];
+        for (int tt = 0; tt < 2; ++tt) {
+            AFrag k_last = k[tt][DS - 1];
+            if (DT % 2 == 1) {
+                k_last.u.x &= tail_keep; k_last.u.y &= tail_keep; k_last.u.z &= tail_keep; k_last.u.w &= tail_keep;
             }
-        }
-        if (DT % 2 == 1) {
-#pragma unroll
-            for (int tt = 0; tt < 2; ++tt) {
-                b.k[tt][DS - 1].u.x &= tail_keep; b.k[tt][DS - 1].u.y &= tail_keep;
-                b.k[tt][DS - 1].u.z &= tail_keep; b.k[tt][DS - 1].u.w &= tail_keep;
-            }
-        }
-        f32x4_t sacc[2][CT];
-#pragma unroll
-        for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) {
-                sacc[tt][ct] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+                f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int ds = 0; ds < DS; ++ds)
-                    sacc[tt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b.k[tt][ds].v, qf[ct][ds].v, sacc[tt][ct], 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ds == DS - 1 ? k_last.v : k[tt][ds].v, qf[ct][ds].v, acc, 0, 0, 0);
+                sacc[tt][ct] = acc;
             }
-        // Scores are kept in units of log 2 (the scale carries log2 e), so that the exponential is the
-        // hardware's exp2.  A block that lies wholly below every column's limit needs no masking.
-        const bool interior = kb + 32 <= min_lim && kb >= lo_last;
-        AFrag pf[CT];
+        }
+    };
+    // what the products become before the exponentials: with ALiBi, scaled and biased; keys that a column does
+    // not see set to -inf; and the column's running maximum looked after.  MASKED = false is for a block that
+    // every column of the wave sees whole: no key of it is past the sequence's end, past a column's own position
+    // or before its window, and the code that would look is not there.
+    auto settle = [&](auto masked_tag, f32x4_t (&sacc)[2][CT], int kb, float (&mx)[CT]) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
+        const bool interior = !MASKED || (kb + 32 <= min_lim && kb >= lo_last);
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
-            float s[8];
-            if (slopes) {  // one branch for the tile, not one per score
+            if (has_alibi) {  // one branch for the tile, not one per score
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                     const int key = kb + 8 * gq + j;  // j = 4*tt + e
                     const float bias = alibi_exact ? slope[ct] * (float)key : round_to_bf16(slope[ct] * round_to_bf16((float)key));
-                    s[j] = sacc[j >> 2][ct][j & 3] * scale + bias * alibi_mul;
+                    sacc[j >> 2][ct][j & 3] = sacc[j >> 2][ct][j & 3] * scale + bias * alibi_mul;
                 }
-            } else {  // left unscaled: the scale rides in the one multiply-add in front of the exponential
-#pragma unroll
-                for (int j = 0; j < 8; ++j) s[j] = sacc[j >> 2][ct][j & 3];
             }
-            const float s_mul = slopes ? 1.0f : scale;  // what s is still to be multiplied by (positive)
-            if (!interior) {
+            if (MASKED && !interior) {
                 const int lim = min(qpos[ct] + 1, k_end);  // keys below this, and from `lo` on, count for the column
                 const int lo = window > 0 ? qpos[ct] - window + 1 : 0;
 #pragma unroll
                 for (int j = 0; j < 8; ++j)
-                    if (kb + 8 * gq + j >= lim || kb + 8 * gq + j < lo) s[j] = -INFINITY;
+                    if (kb + 8 * gq + j >= lim || kb + 8 * gq + j < lo) sacc[j >> 2][ct][j & 3] = -INFINITY;
             }
-            const float mx3 = max3(s[6], s[7], max3(s[0], s[1], s[2]));
-            float mx = max3(s[3], s[4], s[5]);
-            mx = max3(mx, mx3, mx3) * s_mul;
-            // The running maximum is only a reference point for the exponentials, shared by the four lanes of
-            // a column; it is brought up to the true maximum (an exchange between those lanes, and a
-            // rescale of what was summed) only when some score of the block lies more than 2^8 above it,
-            // which after the first blocks of a row is rare.  Weights stay below 2^8 and their rounding to
-            // bfloat16 is relative, so nothing is lost by a reference that lags.
-            if (__any(mx > m_run[ct] + 8.0f)) {
-                mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-                const float m_new = fmaxf(m_run[ct], mx);
-                const float corr = __builtin_amdgcn_exp2f(m_run[ct] - (m_new == -INFINITY ? 0.f : m_new));
-                l_run[ct] *= corr;
+            const f32x4_t s0 = sacc[0][ct], s1 = sacc[1][ct];
+            const float mx3 = max3(s1[2], s1[3], max3(s0[0], s0[1], s0[2]));
+            mx[ct] = max3(s0[3], s1[0], s1[1]);
+            mx[ct] = max3(mx[ct], mx3, mx3);
+        }
+    };
+    // The running maximum is only a reference point for the exponentials, shared by the four lanes of a column;
+    // it is brought up to the true maximum (an exchange between those lanes, and a rescale of what was summed)
+    // only when some score of the block lies more than 2^8 above it, which after the first blocks of a row is
+    // rare.  Weights stay below 2^8 and their rounding to bfloat16 is relative, so nothing is lost by a
+    // reference that lags.  mx: the largest settled score of each tile's block, per lane.
+    auto raise = [&](const float (&mx)[CT]) {
 #pragma unroll
-                for (int dt = 0; dt < DT; ++dt) {
-                    oacc[dt][ct][0] *= corr; oacc[dt][ct][1] *= corr; oacc[dt][ct][2] *= corr; oacc[dt][ct][3] *= corr;
-                }
-                m_run[ct] = m_new;
+        for (int ct = 0; ct < CT; ++ct) {
+            if (!__any(mx[ct] > m_raise[ct])) continue;
+            float m = mx[ct] * s_mul;
+            m = fmaxf(m, __shfl_xor(m, 16, 64));
+            m = fmaxf(m, __shfl_xor(m, 32, 64));
+            const float m_new = fmaxf(m_run[ct], m);
+            const float corr = __builtin_amdgcn_exp2f(m_run[ct] - (m_new == -INFINITY ? 0.f : m_new));
+            lacc[ct][0] *= corr;  // the one row of the sums that is read at the end
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                oacc[dt][ct][0] *= corr; oacc[dt][ct][1] *= corr; oacc[dt][ct][2] *= corr; oacc[dt][ct][3] *= corr;
             }
+            m_run[ct] = m_new;
+            m_raise[ct] = (m_new + 8.0f) / s_mul;
+        }
+    };
+    // the weights 2^(score - reference) of the block, rounded, as the second product's operand
+    auto weights = [&](const f32x4_t (&sacc)[2][CT], AFrag (&pf)[CT]) {
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
             const float m_use = m_run[ct] == -INFINITY ? 0.f : m_run[ct];
             float p[8];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) p[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[j], s_mul, -m_use));
-            float psum = p[0];
-#pragma unroll
-            for (int j = 1; j < 8; ++j) psum += p[j];
+            for (int j = 0; j < 8; ++j) p[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[j >> 2][ct][j & 3], s_mul, -m_use));
             pf[ct].u = make_uint4(pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7]));
-            l_run[ct] += psum;
         }
+    };
+    // sums of weights and O^T += V^T . P^T
+    auto values = [&](const AFrag (&v)[DT], const AFrag (&pf)[CT]) {
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+            lacc[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones.v, pf[ct].v, lacc[ct], 0, 0, 0);
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct)
-                oacc[dt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b.v[dt].v, pf[ct].v, oacc[dt][ct], 0, 0, 0);
+                oacc[dt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v[dt].v, pf[ct].v, oacc[dt][ct], 0, 0, 0);
+    };
+    const std::true_type masked_block;
+    const std::false_type whole_block;
+    // a key whose index is not below lim is taken out of eight values of consecutive keys from kbase on
+    auto keep_below = [&](uint4& v, int kbase, int lim) {
+        uint32_t mk[4];
+#pragma unroll
+        for (int w = 0; w < 4; ++w)
+            mk[w] = (kbase + 2 * w < lim ? 0x0000ffffu : 0u) | (kbase + 2 * w + 1 < lim ? 0xffff0000u : 0u);
+        v.x &= mk[0]; v.y &= mk[1]; v.z &= mk[2]; v.w &= mk[3];
     };
 
     if constexpr (W == 1) {
+        // all of a block at once (a block past k_end changes nothing)
+        auto use_block = [&](KvBlock<DT>& b, int kb) {
+            if (kb + 32 > kv_len || kb >= k_end) {
+                // positions past the sequence's end were never written; whatever lies there must not reach the
+                // sum, not even with weight zero.  A block past this wave's range was loaded from a clamped
+                // address and is dropped whole.
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) keep_below(b.v[dt].u, kb + gq * 8, kb >= k_end ? 0 : kv_len);
+            }
+            f32x4_t sacc[2][CT];
+            AFrag pf[CT];
+            float mx[CT];
+            scores(b.k, sacc);
+            settle(masked_block, sacc, kb, mx);
+            raise(mx);
+            weights(sacc, pf);
+            values(b.v, pf);
+        };
         // NB register buffers: while one block is used, the loads of the next NB - 1 are in flight (a wave alone
         // has nothing else to hide the memory's latency behind).  Addresses past the last block are clamped to
         // it, and such a block is not used.
@@ -306,79 +351,99 @@ __global__ __launch_bounds__(64 * W * KS) void attn_mfma_kernel(
             }
         }
     } else {
-        // The workgroup's waves walk the keys of its last column together.  A block goes global memory ->
-        // registers (one block ahead) -> one of two LDS buffers -> each wave's operand registers.  Key rows
-        // are stored in the order the score tiles want them (tile tt, lane column c <-> key
-        // 8*(c/4) + 4*tt + c%4), so that sixteen lanes read sixteen consecutive LDS rows; the row
-        // strides (D*2 + 16 and 80 bytes) put those on distinct banks.
-        constexpr int KROW = D + 8, VROW = 40;                    // elements
-        constexpr int KPIECES = 4 * D, THREADS = 64 * W;          // 16-byte pieces of a 32-key block
+        // The workgroup's waves walk the keys of its last column together, a stage of SK keys (one or two
+        // blocks) between barriers.  A stage goes global memory -> registers (one stage ahead) -> one of two
+        // LDS buffers -> each wave's operand registers.  Key rows are stored in the order the score tiles want
+        // them (within a block: tile tt, lane column c <-> key 8*(c/4) + 4*tt + c%4), so that sixteen lanes
+        // read sixteen consecutive LDS rows; the row strides (D*2 + 16 and SK*2 + 16 bytes) put those on
+        // distinct banks.  Small heads take a whole page per stage: half the barriers.
+        constexpr int SK = D <= 64 ? 64 : 32, NBK = SK / 32;
+        constexpr int KROW = D + 8, VROW = SK + 8;                // elements
+        constexpr int KPIECES = SK / 8 * D, THREADS = 64 * W;     // 16-byte pieces of a stage's keys (and values)
         constexpr int PER = (KPIECES + THREADS - 1) / THREADS;
-        __shared__ __attribute__((aligned(16))) bf16_t kbuf[2][32 * KROW];
+        constexpr int VCH = SK / 8;                               // pieces in a stage's row of values
+        __shared__ __attribute__((aligned(16))) bf16_t kbuf[2][SK * KROW];
         __shared__ __attribute__((aligned(16))) bf16_t vbuf[2][D * VROW];
         const int tid = threadIdx.x;
         const int wg_last_col = min(ncols, wg_col0 + 16 * CT * W) - 1;
         // (a launch that cuts the keys into ranges walks its own range only)
         const int k_end_wg = n_splits > 1 ? min(start + wg_last_col / g + 1, split * split_size + split_size)
                                           : start + wg_last_col / g + 1;
-        const int k_begin_wg = max(window > 0 ? max(0, start + wg_col0 / g - window + 1) & ~31 : 0,
+        const int k_begin_wg = max(window > 0 ? max(0, start + wg_col0 / g - window + 1) & ~(SK - 1) : 0,
                                    n_splits > 1 ? split * split_size : 0);
-        static_assert(PER <= 2, "a thread moves at most two pieces of keys and two of values per block");
+        const int ks_last = (kv_len - 1) & ~(SK - 1);  // the last stage that has a page
+        static_assert(PER <= 2, "a thread moves at most two pieces of keys and two of values per stage");
+        static_assert(PTA_PAGE % SK == 0, "a stage lies in one page");
         // the pieces in flight are plain variables, not an array: an array that lambdas index stays in
-        // scratch memory at the larger head sizes, and every block then waits for its loads at once
+        // scratch memory at the larger head sizes, and every stage then waits for its loads at once
         uint4 gk0, gk1, gv0, gv1;
-        auto gload = [&](int kb) {
-            kb = min(kb, kb_last);
-            const long page = bt[kb >> 6];
-            const int in_page = kb & 63;
-            const bf16_t* kpage = k_pool + (page * nkv + kvh) * (long)(PTA_PAGE * D);
-            const bf16_t* vpage = v_pool + (page * nkv + kvh) * (long)(PTA_PAGE * D);
-            const int p0 = min(tid, KPIECES - 1);
-            gk0 = *reinterpret_cast<const uint4*>(kpage + (long)(in_page + p0 / CHUNKS) * D + (p0 % CHUNKS) * 8);
-            gv0 = *reinterpret_cast<const uint4*>(vpage + (long)(p0 >> 2) * PTA_PAGE + in_page + (p0 & 3) * 8);
+        const int p0 = min(tid, KPIECES - 1), p1 = min(tid + THREADS, KPIECES - 1);
+        auto gload = [&](int ks) {  // keys and values of the stage at ks (clamped to the last one there is)
+            ks = min(ks, ks_last);
+            const long page = ((long)bt[ks >> 6] * nkv + kvh) * (long)(PTA_PAGE * D);
+            const bf16_t* kpage = k_pool + page + (long)(ks & 63) * D;
+            const bf16_t* vpage = v_pool + page + (ks & 63);
+            gk0 = *reinterpret_cast<const uint4*>(kpage + (long)(p0 / CHUNKS) * D + (p0 % CHUNKS) * 8);
+            gv0 = *reinterpret_cast<const uint4*>(vpage + (long)(p0 / VCH) * PTA_PAGE + (p0 % VCH) * 8);
             if constexpr (PER > 1) {
-                const int p1 = min(tid + THREADS, KPIECES - 1);
-                gk1 = *reinterpret_cast<const uint4*>(kpage + (long)(in_page + p1 / CHUNKS) * D + (p1 % CHUNKS) * 8);
-                gv1 = *reinterpret_cast<const uint4*>(vpage + (long)(p1 >> 2) * PTA_PAGE + in_page + (p1 & 3) * 8);
+                gk1 = *reinterpret_cast<const uint4*>(kpage + (long)(p1 / CHUNKS) * D + (p1 % CHUNKS) * 8);
+                gv1 = *reinterpret_cast<const uint4*>(vpage + (long)(p1 / VCH) * PTA_PAGE + (p1 % VCH) * 8);
             }
         };
-        auto put = [&](int buf, int p, const uint4& k, const uint4& v) {
+        // Positions past the sequence's end were never written; whatever lies there must not reach the sums, not
+        // even with weight zero: such values are cleared on their way into LDS.
+        auto put = [&](int buf, int p, const uint4& k, uint4 v, int ks) {
             if (p < KPIECES) {
-                const int kk = p / CHUNKS;  // key of the block -> its row in operand order
-                const int row = ((kk & 7) >> 2) * 16 + 4 * (kk >> 3) + (kk & 3);
+                const int kk = p / CHUNKS;  // key of the stage -> its row in operand order
+                const int row = (kk & ~31) + ((kk & 7) >> 2) * 16 + 4 * ((kk & 31) >> 3) + (kk & 3);
                 *reinterpret_cast<uint4*>(&kbuf[buf][row * KROW + (p % CHUNKS) * 8]) = k;
-                *reinterpret_cast<uint4*>(&vbuf[buf][(p >> 2) * VROW + (p & 3) * 8]) = v;
+                if (ks + SK > kv_len) keep_below(v, ks + (p % VCH) * 8, kv_len);
+                *reinterpret_cast<uint4*>(&vbuf[buf][(p / VCH) * VROW + (p % VCH) * 8]) = v;
             }
         };
-        auto sstore = [&](int buf) {
-            put(buf, tid, gk0, gv0);
-            if constexpr (PER > 1) put(buf, tid + THREADS, gk1, gv1);
+        auto sstore = [&](int ks) {  // into the buffer of the stage's number, whatever was loaded for it
+            const int buf = (ks / SK) & 1;
+            put(buf, tid, gk0, gv0, min(ks, ks_last));
+            if constexpr (PER > 1) put(buf, tid + THREADS, gk1, gv1, min(ks, ks_last));
         };
-        auto lfetch = [&](KvBlock<DT>& b, int buf) {
+        auto lfetch_k = [&](AFrag (&k)[2][DS], int kb) {  // the keys of the block at kb, from its stage's buffer
+            const bf16_t* kb_lds = &kbuf[(kb / SK) & 1][((kb & (SK - 1)) + c) * KROW];
 #pragma unroll
             for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
                 for (int ds = 0; ds < DS; ++ds)
-                    b.k[tt][ds].u = *reinterpret_cast<const uint4*>(
-                        &kbuf[buf][(tt * 16 + c) * KROW + min(ds * 4 + gq, CHUNKS - 1) * 8]);
+                    k[tt][ds].u = *reinterpret_cast<const uint4*>(kb_lds + tt * 16 * KROW + min(ds * 4 + gq, CHUNKS - 1) * 8);
+        };
+        auto lfetch_v = [&](AFrag (&v)[DT], int kb) {
+            const bf16_t* vb_lds = &vbuf[(kb / SK) & 1][c * VROW + (kb & (SK - 1)) + gq * 8];
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
-                b.v[dt].u = *reinterpret_cast<const uint4*>(&vbuf[buf][(dt * 16 + c) * VROW + gq * 8]);
+            for (int dt = 0; dt < DT; ++dt) v[dt].u = *reinterpret_cast<const uint4*>(vb_lds + dt * 16 * VROW);
         };
         gload(k_begin_wg);
-        sstore((k_begin_wg >> 5) & 1);
+        sstore(k_begin_wg);
         __syncthreads();
-        for (int kb = k_begin_wg; kb < k_end_wg; kb += 32) {
-            const int buf = (kb >> 5) & 1;
-            gload(kb + 32);
+        for (int ks = k_begin_wg; ks < k_end_wg; ks += SK) {
+            gload(ks + SK);
             __builtin_amdgcn_sched_barrier(0);
-            if (kb < k_end && kb >= k_begin) {
-                KvBlock<DT> b;
-                lfetch(b, buf);
-                use_block(b, kb);
+            // the blocks of the stage that are this wave's: a plain loop with one way through it, in which the
+            // compiler leaves the sums in their registers (two copies of the block's second half, one for the
+            // rare block that raises a maximum, made it move all of them in every block)
+            const int b_hi = min(ks + SK, k_end);
+            for (int kb = max(ks, k_begin); kb < b_hi; kb += 32) {
+                f32x4_t sacc[2][CT];
+                AFrag pf[CT], kf[2][DS], vf[DT];
+                float mx[CT];
+                lfetch_k(kf, kb);
+                scores(kf, sacc);
+                if (kb + 32 <= min_lim && kb >= lo_last) settle(whole_block, sacc, kb, mx);
+                else settle(masked_block, sacc, kb, mx);
+                raise(mx);
+                weights(sacc, pf);
+                lfetch_v(vf, kb);
+                values(vf, pf);
             }
             __builtin_amdgcn_sched_barrier(0);
-            sstore(buf ^ 1);
+            sstore(ks + SK);
             __syncthreads();
         }
     }
@@ -392,9 +457,7 @@ __global__ __launch_bounds__(64 * W * KS) void attn_mfma_kernel(
         float* sl = sm + KS * CT * 16;
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
-            float l = l_run[ct];
-            l += __shfl_xor(l, 16, 64);
-            l += __shfl_xor(l, 32, 64);
+            const float l = lacc[ct][0];
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
                 so[((kw * CT + ct) * DT + dt) * 64 + lane] =
@@ -442,9 +505,7 @@ __global__ __launch_bounds__(64 * W * KS) void attn_mfma_kernel(
     } else {
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
-        float l = l_run[ct];
-        l += __shfl_xor(l, 16, 64);
-        l += __shfl_xor(l, 32, 64);
+        const float l = lacc[ct][0];
         if (qpos[ct] < 0) continue;
         const long row = (long)tok[ct] * nh + head[ct];
         if (n_splits == 1) {
@@ -531,13 +592,17 @@ struct AttnLaunch {
 // LDS in which KS waves of CT column tiles leave their partial results
 constexpr size_t key_split_lds(int dt, int ct, int ks) { return ks == 1 ? 0 : (size_t)ks * ct * (dt * 1024 + 128); }
 
-template <int DT, int CT, int W, int KS = 1>
+template <int DT, int CT, int W, int KS = 1, int OCC = 1>
 static void launch_attn(const AttnLaunch& a) {
     const int g = a.nh / a.nkv;
     const int groups = (a.max_new * g + 16 * CT * W - 1) / (16 * CT * W);
     const int paired = a.paired && groups > 1 ? 1 : 0;
     const dim3 grid(paired ? (groups + 1) / 2 : groups, a.nkv, a.n_seqs * a.n_splits);
-    auto kern = a.window > 0 ? attn_mfma_kernel<DT, CT, W, true, KS> : attn_mfma_kernel<DT, CT, W, false, KS>;
+    // prompts: a kernel with ALiBi and one without; one token per sequence: one kernel that looks
+    constexpr int AL0 = W > 1 ? 0 : 2, AL1 = W > 1 ? 1 : 2;
+    auto kern = a.window > 0 ? attn_mfma_kernel<DT, CT, W, true, KS, AL0, OCC> : attn_mfma_kernel<DT, CT, W, false, KS, AL0, OCC>;
+    if (W > 1 && a.slopes)
+        kern = a.window > 0 ? attn_mfma_kernel<DT, CT, W, true, KS, AL1, OCC> : attn_mfma_kernel<DT, CT, W, false, KS, AL1, OCC>;
     constexpr size_t lds = key_split_lds(DT, CT, KS);
     if constexpr (lds > 64 * 1024) {  // more than a launch may ask for unless the kernel has been told, once per device
         static bool told[64] = {};
@@ -586,11 +651,14 @@ static bool launch_decode(const AttnLaunch& a, int tiles) {
     return false;
 }
 
-// prompts: four waves of two column tiles share each key block through LDS (head sizes up to 128;
-// beyond, one wave per workgroup)
+// prompts: four waves of two column tiles share each stage of keys through LDS (head sizes up to 128;
+// beyond, one wave per workgroup).  Heads up to 64 fit four waves a SIMD (measured at 8,192 tokens, 71 heads
+// on one KV head of 64: as many registers as the compiler likes, three waves, 800 us a layer; four waves 760;
+// a third column tile, 256 registers, two waves, 817).
 template <int DT>
 static void launch_prompt(const AttnLaunch& a) {
-    if constexpr (DT <= 8) launch_attn<DT, 2, 4>(a);
+    if constexpr (DT <= 4) launch_attn<DT, 2, 4, 1, 4>(a);
+    else if constexpr (DT <= 8) launch_attn<DT, 2, 4>(a);
     else launch_attn<DT, 1, 1>(a);
 }
 
@@ -618,10 +686,8 @@ extern "C" int pta_attn_mfma(void* out, const void* q, const void* k_pool, const
     PTA_REQUIRE(((uintptr_t)q % 16) == 0 && ((uintptr_t)k_pool % 16) == 0 && ((uintptr_t)v_pool % 16) == 0 &&
                     ((uintptr_t)out % 8) == 0, "attn_mfma: pointers must be 16-byte aligned");
     hipStream_t s = (hipStream_t)stream;
-    // Prompts: four waves of two column tiles share each key block through LDS (head sizes up to 128;
-    // beyond, one wave per workgroup).  Measured at 2,048 tokens, 71 heads on one KV
-    // head, one wave per workgroup: 2 tiles 148 us a layer, 4 tiles 195 us, 1 tile 270 us (fewer tiles
-    // balance the causal triangle better, more tiles re-read keys less).
+    // Prompts: four waves of two column tiles share each stage of keys through LDS (head sizes up to 128;
+    // beyond, one wave per workgroup).
     // One token per sequence (decode): workgroups of `decode_waves` waves, each of which holds `decode_tiles` column
     // tiles of its KV head (at most what the head size leaves registers for).  More tiles: the keys cross the memory
     // path fewer times; fewer: shorter waves, more of them (71 heads on one KV head, 2,048 keys: 64
@@ -631,13 +697,14 @@ extern "C" int pta_attn_mfma(void* out, const void* q, const void* k_pool, const
     // same work, which ends a launch evenly if their number fills the compute units evenly; unpaired ones are
     // twice as many and of all lengths, which the longest-first order spreads well over any number of units.
     // In units of a mean workgroup's work a unit's share is max(n / units, 2) unpaired and 2 ceil(n / 2 / units)
-    // paired; measured at 2,048 tokens, pairs win where the two are equal (32 heads on 8 KV heads of 128:
-    // 102 -> 86 us a layer; 128 on 8 of 64: 172 -> 152) and lose where they are not (71 on 1 of 64: 75 -> 93).
+    // paired; pairs win where the two are equal (32 heads on 8 KV heads of 128: 2,048 tokens 92 -> 77 us a layer,
+    // 8,192 tokens 787 -> 657; 128 on 8 of 64: 123 -> 103 and 1,264 -> 1,214) and lose where they are not (71 on
+    // 1 of 64: 68 -> 89, and 737 -> 766 where the two differ by 2 %).
     static const int pair_env = getenv("PTA_ATTN_PAIR") ? atoi(getenv("PTA_ATTN_PAIR")) : -1;
     int paired = 0;
     if (!narrow) {
         const double wgs = std::ceil((double)M * (nh / nkv) / (d <= 128 ? 128 : 16)) * nkv, units = pta_compute_units();
-        paired = pair_env >= 0 ? pair_env : 2.0 * std::ceil(wgs / 2.0 / units) <= 1.1 * std::max(wgs / units, 2.0);
+        paired = pair_env >= 0 ? pair_env : 2.0 * std::ceil(wgs / 2.0 / units) <= 1.01 * std::max(wgs / units, 2.0);
     }
     const int dct_most = std::min((nh / nkv + 15) / 16, pta_attn_decode_max_tiles(d));
     PTA_REQUIRE(decode_tiles >= 0 && decode_tiles <= dct_most,
