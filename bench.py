@@ -83,12 +83,14 @@ def run_decode(model, sampler_cls, gen_cfg, batch, prompt_len, steps, warmup, se
     slots = [cache.alloc() for _ in range(batch)]
     logits = model.step(cache, slots, prompts, "last")
     rng = list(range(batch))
-    tokens, _ = sampler.sample(logits, rng_seq=rng, rng_step=[0] * batch, need_scores=False)
+    pending, _ = sampler.sample(logits, rng_seq=rng, rng_step=[0] * batch, need_scores=False, ahead=True)
 
-    def one(k):
-        nonlocal tokens
-        lg = model.step(cache, slots, [[t] for t in tokens], "last")
-        tokens, _ = sampler.sample(lg, rng_seq=rng, rng_step=[k] * batch, need_scores=False)  # as generate() calls it
+    def one(k):  # as generate() runs a step: launched from the tokens on the device, which the host reads meanwhile
+        nonlocal pending
+        lg = model.step(cache, slots, pending, "last", own_logits=False)
+        chosen, _ = sampler.sample(lg, rng_seq=rng, rng_step=[k] * batch, need_scores=False, ahead=True)
+        pending.tolist()
+        pending = chosen
 
     for k in range(warmup):
         one(k)
@@ -96,6 +98,7 @@ def run_decode(model, sampler_cls, gen_cfg, batch, prompt_len, steps, warmup, se
     t0 = time.perf_counter()
     for k in range(steps):
         one(warmup + k)
+    pending.tolist()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     mean_ctx = prompt_len + warmup + (steps + 1) / 2.0

@@ -143,6 +143,11 @@ def generate(model, prompts: Sequence[Sequence[int]], generation_config: Optiona
     out_logits = [[] for _ in prompts] if want_logits else None
     kept = [None] * len(prompts)
     t0 = time.time()
+    # Steps ahead of the host: where nothing of a step's decisions needs more than the tokens themselves, the next
+    # step is launched from the tokens on the device before the host has read them.
+    ahead = (bool(getattr(model, "steps_ahead", False)) and getattr(sampler, "needs_histories", True) is False
+             and not want_scores and not want_logits and streamer is None and not stop_strings
+             and cfg.max_time is None and not keep_slots)
 
     def done_with(i: int, slot: int) -> None:
         if keep_slots:
@@ -161,6 +166,10 @@ def generate(model, prompts: Sequence[Sequence[int]], generation_config: Optiona
         live = list(batch)
         step_no = 0
         try:
+            if ahead:
+                _decode_ahead(model, cache, sampler, cfg, eos, ids, batch, slot_of, feed, out_tokens, new_budget,
+                              padded_len, done_with)
+                live = []
             while live:
                 logits = model.step(cache, [slot_of[i] for i in live], [feed[i] for i in live], "last")
                 # EOS is masked while the minimum lengths are not reached (logits_process.py:144-151, :214-223)
@@ -205,6 +214,61 @@ def generate(model, prompts: Sequence[Sequence[int]], generation_config: Optiona
     if cfg.return_dict_in_generate:
         return GenerateOutput(sequences, out_scores, out_logits)
     return sequences
+
+
+def _decode_ahead(model, cache, sampler, cfg, eos, ids, batch, slot_of, feed, out_tokens, new_budget, padded_len,
+                  done_with) -> None:
+    """One batch, with every step launched before the host has seen the tokens of the step before it.
+
+    The tokens of a step stay on the device (``sampler.sample(..., ahead=True)``) and the next step takes them
+    from there (``model.step`` with those tokens); while it runs the host reads the earlier tokens, appends them
+    and finds who has ended.  A sequence that ended on a stop token was part of one more step, whose row nobody
+    reads: its keys and values went into a slot that is given back, and whatever takes the slot's pages next is
+    launched later on the same stream.  A sequence that ends by its length is known beforehand and never takes
+    part in a step too many.  The tokens are those of the loop that waits after every step: a sequence's result
+    does not depend on what else is in its batch.
+    """
+    from ..cache.paged import CacheFull
+
+    def too_short(step: int) -> bool:  # as in the loop that waits: EOS is masked until the minimum lengths are reached
+        return (padded_len + step < (cfg.min_length or 0)) or (step < (cfg.min_new_tokens or 0))
+
+    def choose(logits, seqs, step):
+        return sampler.sample(logits, rng_seq=[ids[i] for i in seqs], rng_step=[step] * len(seqs),
+                              suppress_eos=[too_short(step)] * len(seqs), need_scores=False, ahead=True)[0]
+
+    step_no = 0  # the number of the token that `pending` holds for each of its sequences
+    seqs = list(batch)
+    pending = choose(model.step(cache, [slot_of[i] for i in seqs], [feed[i] for i in seqs], "last"), seqs, 0)
+    rows = list(range(len(seqs)))  # the rows of `pending` whose sequences live, as far as the host knows
+    while True:
+        nxt = None
+        if step_no + 1 < new_budget:  # (else every sequence ends with the pending token)
+            try:
+                logits = model.step(cache, [slot_of[i] for i in seqs], pending.take(rows), "last", own_logits=False)
+            except CacheFull:
+                logits = None  # no room to go on before knowing who has ended: wait for the tokens first
+            if logits is not None:
+                nxt = choose(logits, seqs, step_no + 1)
+        tokens = pending.tolist()
+        step_no += 1
+        on = []  # of the next step's rows, those whose sequences go on
+        for at, (row, i) in enumerate(zip(rows, seqs)):
+            tok = int(tokens[row])
+            out_tokens[i].append(tok)
+            if tok in eos or step_no >= new_budget:
+                done_with(i, slot_of.pop(i))
+            else:
+                on.append(at)
+        if not on:
+            return
+        survivors = [seqs[at] for at in on]
+        if nxt is None:  # the step that found no room: now with the sequences that are left, and their tokens
+            logits = model.step(cache, [slot_of[i] for i in survivors], [[out_tokens[i][-1]] for i in survivors], "last")
+            pending, rows = choose(logits, survivors, step_no), list(range(len(survivors)))
+        else:
+            pending, rows = nxt, on
+        seqs = survivors
 
 
 def _ends_with_stop(tokenizer, new_tokens: Sequence[int], stop_strings: Sequence[str]) -> bool:

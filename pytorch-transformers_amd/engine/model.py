@@ -174,9 +174,11 @@ class _DecodeGraph:
             return logits[:0].clone()
         return logits.index_select(0, torch.from_numpy(rows.astype(np.int64)).to(logits.device))
 
-    def run_last(self, n: int, slots_c, tokens_c) -> torch.Tensor:
+    def run_last(self, n: int, slots_c, tokens_c, ids: Optional[torch.Tensor] = None,
+                 own_logits: bool = True) -> torch.Tensor:
         """The common case, laid out by the host runtime straight into the pinned buffer: ``n`` sequences, one
-        token each (C arrays), the logits of each."""
+        token each (C arrays), the logits of each.  ``ids``: the tokens as a tensor on the device, which takes
+        the place of ``tokens_c`` there."""
         self.copied.synchronize()  # the last copy out of the pinned buffer is done
         lib = host.load()
         cache = self.cache
@@ -186,7 +188,10 @@ class _DecodeGraph:
             raise StepError(host.last_error())
         self.dev.copy_(self.host, non_blocking=True)
         self.copied.record()
-        return self._launch()[:n].clone()
+        if ids is not None:
+            self.dev[:n].copy_(ids)
+        logits = self._launch()[:n]
+        return logits.clone() if own_logits else logits
 
     def _launch(self) -> torch.Tensor:
         """Run the step that the device buffer now describes; returns the logits of all ``n`` rows (a buffer
@@ -389,6 +394,12 @@ class CausalLM:
                       + f" ms a step -> {chosen or cuts[0]}", flush=True)
         ops.take_decode_keys()  # the steps above asked too
 
+    @property
+    def steps_ahead(self) -> bool:
+        """Whether ``step`` can launch a step from tokens that are still on the device (a ``TokensAhead``) without
+        waiting for them: where steps of one token per sequence are replays of a captured step."""
+        return bool(self.use_graphs) and self.layer_hook is None
+
     # cache -------------------------------------------------------------------
     @property
     def page_size(self) -> int:
@@ -453,17 +464,29 @@ class CausalLM:
         return g
 
     @torch.no_grad()
-    def step(self, cache: PagedCache, slots: Sequence[int], tokens: Sequence[Sequence[int]],
-             want: Want = "last") -> torch.Tensor:
+    def step(self, cache: PagedCache, slots: Sequence[int], tokens, want: Want = "last",
+             own_logits: bool = True) -> torch.Tensor:
         """Run the given tokens of the given sequences; return logits ``[wanted places, vocab]`` in 32-bit.
 
         ``want`` is ``"last"``, ``"all"``, ``"none"`` or, per sequence, the places among its tokens
         of this step whose logits are asked for.  Rows come in the order of the sequences and of
         their places.
+
+        ``tokens`` is a list of token lists, or a ``TokensAhead``: one token per sequence, chosen by the last step
+        and still on the device, of which this step takes ``tokens.rows``; the step is then launched without a
+        wait for them.  ``own_logits=False`` lets a step of one token per sequence return its logits in the buffer
+        that the next such step writes again (for a caller that uses them at once).
         """
+        from ..sampling.ahead import TokensAhead
+
         graphs = self.use_graphs and self.layer_hook is None
+        if isinstance(tokens, TokensAhead):
+            if graphs and want == "last":
+                return self._decode_last(cache, slots, None, ahead=tokens, own_logits=own_logits)
+            seen = tokens.tolist()  # no captured step to launch them into: as any other tokens, once they are here
+            tokens = [[seen[r]] for r in (tokens.rows if tokens.rows is not None else range(len(seen)))]
         if graphs and want == "last" and len(tokens) == len(slots) and all(len(t) == 1 for t in tokens):
-            return self._decode_last(cache, slots, tokens)
+            return self._decode_last(cache, slots, tokens, own_logits=own_logits)
         plan = plan_step(cache, slots, tokens, want, self.vocab_size)
         if graphs and plan.is_decode:
             logits = self._graph_for(cache, plan).run(plan)
@@ -476,24 +499,30 @@ class CausalLM:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
         return logits
 
-    def _decode_last(self, cache: PagedCache, slots: Sequence[int], tokens: Sequence[Sequence[int]]) -> torch.Tensor:
+    def _decode_last(self, cache: PagedCache, slots: Sequence[int], tokens, ahead=None,
+                     own_logits: bool = True) -> torch.Tensor:
         """One token per sequence, the logits of each, as a replay of a captured step: the host runtime checks
         the step, reserves pages and writes the step's integers straight into the buffer that is copied to
-        the device."""
+        the device.  ``ahead``: the tokens are not ``tokens`` but rows of a tensor on the device, which are copied
+        into the step's buffer there."""
         from ..cache.paged import CacheError, CacheFull
 
         n = len(slots)
         if n == 0:
             raise StepError("a step needs at least one sequence")
+        if ahead is not None and n != (len(ahead.rows) if ahead.rows is not None else len(ahead)):
+            raise StepError(f"{n} sequences, but tokens ahead for "
+                            f"{len(ahead.rows) if ahead.rows is not None else len(ahead)}")
         lib = host.load()
         slots_c = (ctypes.c_int * n)(*[int(s) for s in slots])
-        tokens_c = (ctypes.c_longlong * n)(*[int(t[0]) for t in tokens])
+        tokens_c = (ctypes.c_longlong * n)() if ahead is not None else (ctypes.c_longlong * n)(*[int(t[0]) for t in tokens])
         longest, total = ctypes.c_int(0), ctypes.c_longlong(0)
         rc = lib.ptah_decode_prepare(cache.handle, n, slots_c, tokens_c, self.vocab_size, ctypes.byref(longest),
                                      ctypes.byref(total))
         if rc:
             raise {host.ERR_STEP: StepError, host.ERR_FULL: CacheFull}.get(rc, CacheError)(host.last_error())
-        logits = self._graph_for_sizes(cache, n, longest.value, total.value).run_last(n, slots_c, tokens_c)
+        logits = self._graph_for_sizes(cache, n, longest.value, total.value).run_last(
+            n, slots_c, tokens_c, ids=None if ahead is None else ahead.for_step(), own_logits=own_logits)
         lib.ptah_commit_ones(cache.handle, n, slots_c)
         return logits
 

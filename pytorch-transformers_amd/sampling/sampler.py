@@ -16,6 +16,7 @@ import torch
 
 from .. import ops
 from ..config.generation import GenerationConfig
+from .ahead import TokensAhead
 from .bans import BanRules
 
 
@@ -44,12 +45,15 @@ class Sampler:
     def sample(self, logits: torch.Tensor, *, rng_seq: Sequence[int], rng_step: Sequence[int],
                histories: Optional[Sequence[Sequence[int]]] = None, suppress_eos: Optional[Sequence[bool]] = None,
                uniforms: Optional[Sequence[float]] = None, new_counts: Optional[Sequence[int]] = None,
-               need_scores: bool = True) -> Tuple[List[int], Optional[torch.Tensor]]:
+               need_scores: bool = True, ahead: bool = False):
         """Tokens for the rows of ``logits`` and the processed scores ``[rows, vocab]`` (None if not needed
         and the choice could be made without forming them).  ``histories`` are the rows' ids so far (prompt and
         new tokens) and ``new_counts`` how many of them are new; the repetition penalty and the options that forbid
-        tokens read them."""
+        tokens read them.  ``ahead``: the tokens come back as a ``TokensAhead``, without a wait for the GPU
+        (only where ``needs_histories`` is false)."""
         R = logits.shape[0]
+        if ahead and self.needs_histories:
+            raise ValueError("tokens ahead of the host cannot be chosen by options that read the tokens so far")
         suppress = self._eos_dev is not None and suppress_eos is not None and any(suppress_eos)
         ban_lists = None
         if self.bans:
@@ -62,7 +66,8 @@ class Sampler:
         if (not need_scores and not self.do_sample and self.penalty == 1.0 and not suppress and ban_lists is None
                 and not self.config.remove_invalid_values and not self.config.renormalize_logits):
             # greedy with no processor in the way: nothing to upload, one argmax kernel
-            return ops.sample(logits, do_sample=False, need_scores=False)[0].tolist(), None
+            chosen = ops.sample(logits, do_sample=False, need_scores=False)[0]
+            return (TokensAhead(chosen) if ahead else chosen.tolist()), None
         use_hist = self.penalty != 1.0 and histories is not None
         pieces = [np.asarray(rng_seq, dtype=np.int32), np.asarray(rng_step, dtype=np.int32),
                   np.asarray([1 if s else 0 for s in (suppress_eos or [False] * R)], dtype=np.int32)]
@@ -77,9 +82,16 @@ class Sampler:
             boff = np.zeros(R + 1, dtype=np.int32)
             boff[1:] = np.cumsum([len(b) for b in ban_lists])
             pieces += [boff, np.asarray([t for b in ban_lists for t in b], dtype=np.int32)]
-        dev = torch.from_numpy(np.concatenate(pieces)).to(self.device)
+        staged = torch.from_numpy(np.concatenate(pieces))
+        # (ahead of the host nothing may wait for the stream: the copy starts from pinned memory and does not block)
+        dev = staged.pin_memory().to(self.device, non_blocking=True) if ahead else staged.to(self.device)
         views = torch.split(dev, [int(p.shape[0]) for p in pieces])
-        u = (torch.tensor(list(uniforms), dtype=torch.float32, device=self.device) if uniforms is not None else None)
+        if uniforms is None:
+            u = None
+        elif ahead:
+            u = torch.tensor(list(uniforms), dtype=torch.float32).pin_memory().to(self.device, non_blocking=True)
+        else:
+            u = torch.tensor(list(uniforms), dtype=torch.float32, device=self.device)
         tokens, scores = ops.sample(
             logits, do_sample=self.do_sample, temperature=self.temperature, top_k=self.top_k, top_p=self.top_p,
             min_p=self.min_p, typical_p=self.typical_p, epsilon_cutoff=self.epsilon_cutoff, eta_cutoff=self.eta_cutoff,
@@ -89,7 +101,12 @@ class Sampler:
             suppress=views[2] if (self._eos_dev is not None and suppress_eos is not None and any(suppress_eos)) else None,
             remove_invalid=self.config.remove_invalid_values, renorm=self.config.renormalize_logits,
             seed=self.config.seed, rng_seq=views[0], rng_step=views[1], uniforms=u, need_scores=need_scores)
-        return tokens.tolist(), scores
+        return (TokensAhead(tokens) if ahead else tokens.tolist()), scores
+
+    @property
+    def needs_histories(self) -> bool:
+        """Whether a choice reads the sequence's tokens so far (which the host then has to have seen)."""
+        return bool(self.bans) or self.penalty != 1.0
 
 
 def philox_uniform(seed: int, seq: int, step: int) -> float:

@@ -249,3 +249,119 @@ def test_kept_slots_go_on_in_a_later_call():
         generate(m3, [[1, 2, 3]], GenerationConfig(max_new_tokens=1), sampler=ArgmaxSampler(), cache=c, slots=[a])
     with pytest.raises(ValueError, match="one slot"):
         generate(m3, [[1, 2, 3, 4], [1, 2, 3, 4]], GenerationConfig(max_new_tokens=1), sampler=ArgmaxSampler(), cache=c, slots=[a, a])
+
+
+# ---- steps ahead of the host -------------------------------------------------------------------------------
+class FakeAhead:
+    """Stands in for tokens that are still on the device: the model may use the values, the host's reading is logged."""
+
+    def __init__(self, values, log):
+        self.values, self.log, self.rows = list(values), log, None
+        self.name = len([e for e in log if e[0] == "chosen"])
+        log.append(("chosen", self.name))
+
+    def __len__(self):
+        return len(self.values)
+
+    def take(self, rows):
+        self.rows = None if rows is None or list(rows) == list(range(len(self.values))) else list(rows)
+        return self
+
+    def tolist(self):
+        self.log.append(("read", self.name))
+        return list(self.values)
+
+
+class AheadModel(ScriptedModel):
+    steps_ahead = True
+
+    def __init__(self, log):
+        super().__init__()
+        self.log = log
+
+    def step(self, cache, slots, tokens, want, own_logits=True):
+        if isinstance(tokens, FakeAhead):
+            self.log.append(("step from", tokens.name))
+            picked = tokens.rows if tokens.rows is not None else range(len(tokens.values))
+            tokens = [[tokens.values[r]] for r in picked]
+        else:
+            self.log.append(("step", None))
+        return super().step(cache, slots, tokens, want)
+
+
+class AheadSampler(ArgmaxSampler):
+    needs_histories = False
+
+    def __init__(self, log, eos=()):
+        super().__init__(eos)
+        self.log = log
+
+    def sample(self, logits, *, rng_seq, rng_step, suppress_eos, need_scores=True, ahead=False, **_):
+        tokens, scores = super().sample(logits, rng_seq=rng_seq, rng_step=rng_step, histories=[[]] * len(rng_seq),
+                                        suppress_eos=suppress_eos, new_counts=[0] * len(rng_seq))
+        return (FakeAhead(tokens, self.log) if ahead else tokens), scores
+
+
+def test_steps_ahead_choose_the_same_tokens_and_wait_for_none_before_the_next_step_is_launched():
+    prompts = [[1, 2, 3], [20, 5], [7, 7, 7, 7], [9]]
+    for cfg, eos in ((GenerationConfig(max_new_tokens=5, eos_token_id=12), [12]),
+                     (GenerationConfig(max_new_tokens=6, eos_token_id=[25, 12], min_new_tokens=2), [25, 12]),
+                     (GenerationConfig(max_new_tokens=1), [])):
+        want = generate(ScriptedModel(), prompts, cfg, batch_size=3, sampler=ArgmaxSampler(eos))
+        log = []
+        m, s = AheadModel(log), AheadSampler(log, eos)
+        assert generate(m, prompts, cfg, batch_size=3, sampler=s) == want
+        assert not m.caches[0].live_slots() and m.caches[0].free_pages() == m.caches[0].num_pages
+        # the choices were asked for as in the loop that waits: same streams, steps and masks of EOS per sequence
+        waits = ArgmaxSampler(eos)
+        generate(ScriptedModel(), prompts, cfg, batch_size=3, sampler=waits)
+        per_seq = lambda calls: sorted((q, st, sup) for c in calls for q, st, sup in zip(c["rng_seq"], c["rng_step"], c["suppress"]))
+        assert set(per_seq(waits.calls)) <= set(per_seq(s.calls))  # (plus the rows that nobody read)
+        # every step after a batch's first was launched from tokens that the host had not read yet
+        for at, (what, name) in enumerate(log):
+            if what == "step from":
+                assert ("read", name) not in log[:at]
+        if cfg.max_new_tokens > 1:
+            assert any(what == "step from" for what, _ in log)
+
+
+def test_a_sequence_that_ends_on_a_stop_token_takes_part_in_one_step_too_many_and_one_that_ends_by_length_in_none():
+    log = []
+    m = AheadModel(log)
+    prompts = [[1, 2, 3], [20, 5]]
+    out = generate(m, prompts, GenerationConfig(max_new_tokens=5, eos_token_id=12), sampler=AheadSampler(log, [12]))
+    assert out[0] == [1, 2, 3, 6, 12] and out[1] == expected([20, 5], 5)
+    assert [len(s) for s, _ in m.steps] == [2, 2, 2, 1, 1]  # (the loop that waits: 2, 2, 1, 1, 1)
+    assert not m.caches[0].live_slots() and m.caches[0].free_pages() == m.caches[0].num_pages
+
+
+def test_a_step_ahead_that_finds_no_room_waits_for_the_tokens_and_goes_on_with_who_is_left():
+    a, b = [1] * 60, [2] * 62
+    eos = expected(a, 3)[-1]  # the third new token of the first sequence ends it
+    assert eos not in expected(b, 6)[len(b):]
+    cfg = GenerationConfig(max_new_tokens=6, eos_token_id=eos)
+    want = [expected(a, 3), expected(b, 6)]
+    for model, sampler in ((ScriptedModel(), ArgmaxSampler([eos])), (AheadModel([]), AheadSampler([], [eos]))):
+        # two pages of 64: the second sequence's 65th token finds a page only once the first sequence has given its own back
+        cache = model.new_cache(128, max_slots=2)
+        assert cache.page_size == 64 and cache.num_pages == 2
+        assert generate(model, [a, b], cfg, sampler=sampler, cache=cache) == want
+        assert not cache.live_slots() and cache.free_pages() == 2
+    log = []
+    model = AheadModel(log)
+    generate(model, [a, b], cfg, sampler=AheadSampler(log, [eos]), cache=model.new_cache(128, max_slots=2))
+    assert ("step", None) in log[1:]  # the step that waited
+
+
+def test_what_needs_the_tokens_on_the_host_keeps_the_loop_that_waits():
+    class Reads(AheadSampler):
+        needs_histories = True
+
+    for kw, sampler_cls in ((dict(output_scores=True, return_dict_in_generate=True), AheadSampler), (dict(max_time=100.0), AheadSampler),
+                            (dict(), Reads)):
+        log = []
+        generate(AheadModel(log), [[1, 2], [3]], GenerationConfig(max_new_tokens=3, **kw), sampler=sampler_cls(log))
+        assert not any(what == "step from" for what, _ in log)
+    log = []
+    generate(AheadModel(log), [[1, 2], [3]], GenerationConfig(max_new_tokens=3), sampler=AheadSampler(log), streamer=lambda i, t: None)
+    assert not any(what == "step from" for what, _ in log)

@@ -245,6 +245,11 @@ def test_pair_ranges_are_timed_once_per_shape_and_kept():
         assert kept[2] in (1, 2) and 1 <= kept[0] <= 2 * rule[0] + 1 and 1 <= kept[1] <= 2 * rule[1] + 1
         assert ops.gemm_splitk_pair_parts(N1, K1, N2, K2) == kept[:2]
     p1, p2 = ops.gemm_splitk_pair_parts(N1, K1, N2, K2)
+    # (what follows is about the kernel that walks K in stages: where the timing has kept the launch with stationary
+    # activations for some class of rows, which has ranges of its own, that is set aside)
+    for cls in range(len(ops.STATIONARY_CLASS_ROWS)):
+        assert lib.pta_gemm_splitk_pair_fix_stationary(N1, K1, N2, K2, cls, 0, 0) == 0
+    y1, y2 = ops.gemm_splitk_pair_bf16(x1, w1, x2, w2)
     assert torch.equal(y1, ops.gemm_splitk_bf16(x1, w1, rt=1, parts=p1)) and torch.equal(y2, ops.gemm_splitk_bf16(x2, w2, rt=1, parts=p2))
     for y, x, w in ((y1, x1, w1), (y2, x2, w2)):
         want = (x.double() @ w.double().T).float()
@@ -265,7 +270,9 @@ def test_pair_ranges_are_timed_once_per_shape_and_kept():
         assert lib.pta_gemm_splitk_pair_fix(N1, K1, N2, K2, 1, 3, 3) == 1
     finally:
         assert lib.pta_gemm_splitk_pair_fix_parts(N1, K1, N2, K2, 0, 0) == 0
+        assert lib.pta_gemm_splitk_pair_fix_stationary(N1, K1, N2, K2, -1, 0, 0) == 0
         ops._pair_parts_tuned.pop(key, None)
+        ops._pair_stationary_tuned.pop(key, None)
     assert ops.gemm_splitk_pair_parts(N1, K1, N2, K2) == rule
 
 

@@ -414,6 +414,33 @@ def test_sampled_generation_equals_plain_fed_the_same_uniforms(folders):
     assert two == got
 
 
+def test_steps_ahead_of_the_host_choose_what_the_loop_that_waits_chooses(folders):
+    """Tiny B, six prompts of 3 to 64 ids in batches of four, 40 tokens, a stop token that ends some early: with every
+    step launched from the tokens on the device, and with a wait after every step (a streamer makes the loop wait)."""
+    from pytorch_transformers_amd import AutoModelForCausalLM, GenerationConfig
+
+    cfg, _ = P.read_model(folders["B"])
+    g = torch.Generator().manual_seed(5)
+    prompts = [torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for n in (3, 9, 1, 30, 17, 64)]
+    for dtype in ("float32", "bfloat16"):
+        model = AutoModelForCausalLM.from_pretrained(folders["B"], dtype=dtype)
+        assert model.steps_ahead
+        for kw in (dict(do_sample=False), dict(do_sample=True, temperature=0.9, top_k=50, top_p=0.95, seed=3)):
+            free_run = model.generate(prompts, GenerationConfig(max_new_tokens=40, eos_token_id=None, **kw), batch_size=4)
+            eos = free_run[1][len(prompts[1]) + 5]
+            gen = GenerationConfig(max_new_tokens=40, eos_token_id=eos, min_new_tokens=2, **kw)
+            cache = model.new_cache(4 * 128, max_slots=4)
+            ahead = model.generate(prompts, gen, batch_size=4, cache=cache)
+            assert not cache.live_slots() and cache.free_pages() == cache.num_pages
+            waits = model.generate(prompts, gen, batch_size=4, cache=cache, streamer=lambda i, t: None)
+            assert ahead == waits
+            ended_early = [len(a) - len(p) < 40 for a, p in zip(ahead, prompts)]
+            assert any(ended_early) and not all(ended_early), ended_early
+            for a, p in zip(ahead, prompts):  # the stop token is kept, nothing follows it, and it is not among the first two
+                new = a[len(p):]
+                assert eos not in new[:-1] and (len(new) == 40 or new[-1] == eos) and eos not in new[:2]
+
+
 def test_pipeline_entry(folders):
     from pytorch_transformers_amd import pipeline
 
