@@ -1,6 +1,6 @@
 // The residual sum and the LayerNorm that reads it, in one pass over bfloat16 rows.
 //
-//   v    = A + B + add1 + add2          (terms that are absent are skipped; at least one is given)
+//   v    = A + B + add1 + add2 + add3   (terms that are absent are skipped; at least one is given)
 //   x    = round(v)                     -> out_x, if wanted
 //   out1 = LN(x) * w1 + b1              -> if wanted; out2 with (w2, b2) likewise
 //
@@ -57,9 +57,9 @@ template <int CH>
 __global__ __launch_bounds__(NS_THREADS / CH) void layernorm_sum_kernel(
     bf16_t* __restrict__ out_x, bf16_t* __restrict__ out1, bf16_t* __restrict__ out2, const float* __restrict__ pa,
     int Pa, const float* __restrict__ bias_a, const float* __restrict__ pb, int Pb, const float* __restrict__ bias_b,
-    const bf16_t* __restrict__ add1, const bf16_t* __restrict__ add2, const int* __restrict__ rows,
-    const float* __restrict__ w1, const float* __restrict__ b1, const float* __restrict__ w2,
-    const float* __restrict__ b2, int M_in, int H, float eps) {
+    const bf16_t* __restrict__ add1, const bf16_t* __restrict__ add2, const bf16_t* __restrict__ add3,
+    const int* __restrict__ rows, const float* __restrict__ w1, const float* __restrict__ b1,
+    const float* __restrict__ w2, const float* __restrict__ b2, int M_in, int H, float eps) {
     __shared__ float red[16];
     const int m = blockIdx.x;
     const long src = rows ? (long)rows[m] : (long)m;
@@ -93,6 +93,13 @@ __global__ __launch_bounds__(NS_THREADS / CH) void layernorm_sum_kernel(
         if (add2) {
             float t[8];
             unpack8(*reinterpret_cast<const uint4*>(add2 + at), t);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[j][e] = any ? v[j][e] + t[e] : t[e];
+            any = true;
+        }
+        if (add3) {
+            float t[8];
+            unpack8(*reinterpret_cast<const uint4*>(add3 + at), t);
 #pragma unroll
             for (int e = 0; e < 8; ++e) v[j][e] = any ? v[j][e] + t[e] : t[e];
         }
@@ -138,18 +145,19 @@ __global__ __launch_bounds__(NS_THREADS / CH) void layernorm_sum_kernel(
 template <int MAXCH>
 __global__ __launch_bounds__(256) void layernorm_rows_kernel(
     bf16_t* __restrict__ out_x, bf16_t* __restrict__ out1, bf16_t* __restrict__ out2, const bf16_t* __restrict__ add1,
-    const bf16_t* __restrict__ add2, const float* __restrict__ w1, const float* __restrict__ b1,
-    const float* __restrict__ w2, const float* __restrict__ b2, int M, int H, float eps) {
+    const bf16_t* __restrict__ add2, const bf16_t* __restrict__ add3, const float* __restrict__ w1,
+    const float* __restrict__ b1, const float* __restrict__ w2, const float* __restrict__ b2, int M, int H, float eps) {
     const int lane = threadIdx.x & 63;
     const long m = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (m >= M) return;
     const int chunks = H / 8;
-    uint4 r1[MAXCH], r2[MAXCH];
+    uint4 r1[MAXCH], r2[MAXCH], r3[MAXCH];
 #pragma unroll
     for (int j = 0; j < MAXCH; ++j) {
         const int ch = min(lane + j * 64, chunks - 1);
         r1[j] = *reinterpret_cast<const uint4*>(add1 + m * H + ch * 8);
         if (add2) r2[j] = *reinterpret_cast<const uint4*>(add2 + m * H + ch * 8);
+        if (add3) r3[j] = *reinterpret_cast<const uint4*>(add3 + m * H + ch * 8);
     }
     float v[MAXCH][8];
     float s = 0.f;
@@ -157,11 +165,18 @@ __global__ __launch_bounds__(256) void layernorm_rows_kernel(
     for (int j = 0; j < MAXCH; ++j) {
         const bool live = lane + j * 64 < chunks;
         unpack8(r1[j], v[j]);
-        if (add2) {
+        if (add2) {  // the terms are added in 32-bit, in their order, and the sum is rounded once
             float t[8];
             unpack8(r2[j], t);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) v[j][e] = round_to_bf16(v[j][e] + t[e]);
+            for (int e = 0; e < 8; ++e) v[j][e] += t[e];
+            if (add3) {
+                unpack8(r3[j], t);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[j][e] += t[e];
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[j][e] = round_to_bf16(v[j][e]);
         }
 #pragma unroll
         for (int e = 0; e < 8; ++e) s += live ? v[j][e] : 0.f;
@@ -196,28 +211,32 @@ __global__ __launch_bounds__(256) void layernorm_rows_kernel(
 }
 
 template <int MAXCH>
-static void launch_rows(void* out_x, void* out1, void* out2, const void* add1, const void* add2, const float* w1,
-                        const float* b1, const float* w2, const float* b2, int M, int H, float eps, hipStream_t s) {
+static void launch_rows(void* out_x, void* out1, void* out2, const void* add1, const void* add2, const void* add3,
+                        const float* w1, const float* b1, const float* w2, const float* b2, int M, int H, float eps,
+                        hipStream_t s) {
     hipLaunchKernelGGL(layernorm_rows_kernel<MAXCH>, dim3((M + 3) / 4), dim3(256), 0, s, (bf16_t*)out_x, (bf16_t*)out1,
-                       (bf16_t*)out2, (const bf16_t*)add1, (const bf16_t*)add2, w1, b1, w2, b2, M, H, eps);
+                       (bf16_t*)out2, (const bf16_t*)add1, (const bf16_t*)add2, (const bf16_t*)add3, w1, b1, w2, b2, M, H, eps);
 }
 
 extern "C" int pta_layernorm_sum_ok(int H) { return H > 0 && H % 8 == 0 && H <= NS_MAX_H; }
 
+extern "C" int pta_layernorm_sum_rows_min(void) { return NS_ROWS_MIN; }
+
 extern "C" int pta_layernorm_sum(void* out_x, void* out1, void* out2, const float* pa, int Pa, const float* bias_a,
                                  const float* pb, int Pb, const float* bias_b, const void* add1, const void* add2,
-                                 const int* rows, const float* w1, const float* b1, const float* w2, const float* b2,
+                                 const void* add3, const int* rows, const float* w1, const float* b1, const float* w2, const float* b2,
                                  int M_in, int M, int H, float eps, void* stream) {
     PTA_REQUIRE(M > 0 && M_in > 0 && H > 0, "layernorm_sum: M=%d M_in=%d H=%d must be positive", M, M_in, H);
     PTA_REQUIRE(pta_layernorm_sum_ok(H), "layernorm_sum: H=%d must be a multiple of 8 up to %d", H,
                 NS_MAX_H);
-    PTA_REQUIRE(pa || pb || add1 || add2, "layernorm_sum: nothing to sum");
+    PTA_REQUIRE(pa || pb || add1 || add2 || add3, "layernorm_sum: nothing to sum");
+    PTA_REQUIRE(!add3 || (add1 && add2), "layernorm_sum: a third tensor comes after a first and a second");
     PTA_REQUIRE((!pa || Pa > 0) && (!pb || Pb > 0), "layernorm_sum: a product needs at least one part");
     PTA_REQUIRE(out_x || out1, "layernorm_sum: no output wanted");
     PTA_REQUIRE(!out1 || (w1 && b1), "layernorm_sum: the norm needs weight and bias");
     PTA_REQUIRE(!out2 || (out1 && w2 && b2), "layernorm_sum: a second output needs the first, and its own weight and bias");
     PTA_REQUIRE(rows || M == M_in, "layernorm_sum: without row selection M (%d) must equal M_in (%d)", M, M_in);
-    const void* ptrs[] = {out_x, out1, out2, pa, pb, add1, add2, bias_a, bias_b, w1, b1, w2, b2};
+    const void* ptrs[] = {out_x, out1, out2, pa, pb, add1, add2, add3, bias_a, bias_b, w1, b1, w2, b2};
     for (const void* p : ptrs) PTA_REQUIRE(((uintptr_t)p % 16) == 0, "layernorm_sum: pointers must be 16-byte aligned");
     // Many rows of plain tensors: a wave per row.  Measured at 2,048 rows of 4,544 against a workgroup per row:
     // 18 us against 27.  The two kernels add a row's squares in different orders, so a row's norm may differ in its
@@ -225,9 +244,9 @@ extern "C" int pta_layernorm_sum(void* out_x, void* out1, void* out2, const floa
     if (!pa && !pb && !rows && add1 && M >= NS_ROWS_MIN) {
         const int per_lane = (H / 8 + 63) / 64;
         hipStream_t s = (hipStream_t)stream;
-        if (per_lane <= 4) launch_rows<4>(out_x, out1, out2, add1, add2, w1, b1, w2, b2, M, H, eps, s);
-        else if (per_lane <= 9) launch_rows<9>(out_x, out1, out2, add1, add2, w1, b1, w2, b2, M, H, eps, s);
-        else launch_rows<16>(out_x, out1, out2, add1, add2, w1, b1, w2, b2, M, H, eps, s);
+        if (per_lane <= 4) launch_rows<4>(out_x, out1, out2, add1, add2, add3, w1, b1, w2, b2, M, H, eps, s);
+        else if (per_lane <= 9) launch_rows<9>(out_x, out1, out2, add1, add2, add3, w1, b1, w2, b2, M, H, eps, s);
+        else launch_rows<16>(out_x, out1, out2, add1, add2, add3, w1, b1, w2, b2, M, H, eps, s);
         return pta_check_launch("layernorm_sum");
     }
     // One chunk per thread for every row count.  Measured at 2,048 rows of 4,544: 1 chunk 26 us, 2 chunks 34 us,
@@ -235,6 +254,6 @@ extern "C" int pta_layernorm_sum(void* out_x, void* out1, void* out2, const floa
     const int chunks = H / 8;
     hipLaunchKernelGGL(layernorm_sum_kernel<1>, dim3(M), dim3((chunks + 63) / 64 * 64), 0, (hipStream_t)stream,
                        (bf16_t*)out_x, (bf16_t*)out1, (bf16_t*)out2, pa, Pa, bias_a, pb, Pb, bias_b, (const bf16_t*)add1,
-                       (const bf16_t*)add2, rows, w1, b1, w2, b2, M_in, H, eps);
+                       (const bf16_t*)add2, (const bf16_t*)add3, rows, w1, b1, w2, b2, M_in, H, eps);
     return pta_check_launch("layernorm_sum");
 }

@@ -14,7 +14,7 @@
 
 #include <stdint.h>
 
-#define PTA_ABI_VERSION 5
+#define PTA_ABI_VERSION 6
 
 #ifdef __cplusplus
 extern "C" {
@@ -31,14 +31,16 @@ int pta_embed(void* out, const void* table, const int* ids, int M, int H, int dt
 int pta_layernorm(void* out1, void* out2, const void* x, const int* rows, const float* w1, const float* b1,
                   const float* w2, const float* b2, int M, int H, float eps, int dtype, void* stream);
 
-// bfloat16 rows: x = round(A + B + add1 + add2) with A, B products left as 32-bit partial sums [P, M_in, H]
-// (summed in order, rounded, bias added and rounded); out_x = x, out1 = LN(x) * w1 + b1, out2 likewise, each
-// if not null; rows (may be null) selects the M source rows out of M_in
+// bfloat16 rows: x = round(A + B + add1 + add2 + add3) with A, B products left as 32-bit partial sums [P, M_in, H]
+// (summed in order, rounded, bias added and rounded) and up to three tensors (a third only after two); out_x = x,
+// out1 = LN(x) * w1 + b1, out2 likewise, each if not null; rows (may be null) selects the M source rows out of M_in
 int pta_layernorm_sum(void* out_x, void* out1, void* out2, const float* pa, int Pa, const float* bias_a,
                       const float* pb, int Pb, const float* bias_b, const void* add1, const void* add2,
-                      const int* rows, const float* w1, const float* b1, const float* w2, const float* b2, int M_in,
+                      const void* add3, const int* rows, const float* w1, const float* b1, const float* w2, const float* b2, int M_in,
                       int M, int H, float eps, void* stream);
 int pta_layernorm_sum_ok(int H);
+// rows from which tensors alone (no products, no row selection) are summed and normalised by a wave per row
+int pta_layernorm_sum_rows_min(void);
 
 // in place: y = act(round(y + bias)) + add1 + add2; bias, add1, add2 may be null
 int pta_epilogue(void* y, int ld_y, const float* bias, const void* add1, const void* add2, int M, int N, int act,

@@ -24,7 +24,7 @@ QKV_LAYOUT_CODES = {"grouped": 0, "tail": 1, "interleaved": 2}
 ACT_CODES = {None: 0, "none": 0, "linear": 0, "gelu": 1, "gelu_python": 1, "gelu_new": 2, "gelu_pytorch_tanh": 2,
              "gelu_fast": 2, "gelu_accurate": 2, "quick_gelu": 3, "relu": 4, "relu2": 5, "relu6": 6, "silu": 7, "swish": 7,
              "sigmoid": 8, "tanh": 9, "leaky_relu": 10, "mish": 11, "gelu_10": 12, "laplace": 13}
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 _lib = None
 _lock = threading.Lock()
@@ -145,7 +145,7 @@ def _entry_cost(name: str, a) -> tuple:
     if name == "pta_gemm_f32":
         return gemm(a[6], a[7], a[8], 4)
     if name == "pta_layernorm_sum":
-        return ((a[4] + a[7]) * float(a[16]) * a[18] * 4, 0.0)
+        return ((a[4] + a[7]) * float(a[17]) * a[19] * 4, 0.0)
     if name in ("pta_attn_mfma", "pta_attn_generic"):
         return (float(timing_hint.get("attn_bytes", 0)), float(timing_hint.get("attn_flops", 0)))
     return (0.0, 0.0)
@@ -1326,17 +1326,22 @@ def layernorm_sum_ok(H: int) -> bool:
     return bool(load_library().pta_layernorm_sum_ok(int(H)))
 
 
+def layernorm_sum_rows_min() -> int:
+    """Rows from which a sum of tensors alone is formed and normalised by a wave per row (the arrangement for prompts)."""
+    return int(load_library().pta_layernorm_sum_rows_min())
+
+
 def layernorm_sum(terms, H: int, *, w=None, b=None, eps: float = 0.0, w2=None, b2=None, rows=None,
                   want_x: bool = True):
     """The sum of ``terms`` rounded to bfloat16 and, with (w, b), its LayerNorm: ``(x, out1, out2)``.
 
     A term is a bfloat16 tensor [M, H] or a pair (partial sums [P, M, H] in 32-bit, bias or None) of a
-    product left unreduced; at most two of each, products first.  A product is valued as its own epilogue
-    would have stored it; the terms are added in the order given."""
+    product left unreduced; at most two products and three tensors, products first.  A product is valued as its
+    own epilogue would have stored it; the terms are added in 32-bit in the order given, and the sum is rounded."""
     prods = [t for t in terms if isinstance(t, tuple)]
     adds = [t for t in terms if not isinstance(t, tuple)]
-    if len(prods) > 2 or len(adds) > 2 or not terms:
-        raise KernelError(f"layernorm_sum takes one to four terms, at most two products and two tensors; got {len(terms)}")
+    if len(prods) > 2 or len(adds) > 3 or not terms:
+        raise KernelError(f"layernorm_sum takes one to five terms, at most two products and three tensors; got {len(terms)}")
     if any(isinstance(t, tuple) for t in terms[len(prods):]):
         raise KernelError("layernorm_sum: products must come before tensors in the list of terms")
     M_in = None
@@ -1377,8 +1382,9 @@ def layernorm_sum(terms, H: int, *, w=None, b=None, eps: float = 0.0, w2=None, b
     pa, ba = prods[1] if len(prods) > 1 else (None, None)
     a1 = adds[0] if adds else None
     a2 = adds[1] if len(adds) > 1 else None
+    a3 = adds[2] if len(adds) > 2 else None
     _call("pta_layernorm_sum", _ptr(out_x), _ptr(out1), _ptr(out2), _ptr(pa), 0 if pa is None else pa.shape[0], _ptr(ba),
-          _ptr(pb), 0 if pb is None else pb.shape[0], _ptr(bb), _ptr(a1), _ptr(a2), _ptr(rows), _ptr(w), _ptr(b),
+          _ptr(pb), 0 if pb is None else pb.shape[0], _ptr(bb), _ptr(a1), _ptr(a2), _ptr(a3), _ptr(rows), _ptr(w), _ptr(b),
           _ptr(w2), _ptr(b2), M_in, M, H, ctypes.c_float(eps), _stream())
     return out_x, out1, out2
 

@@ -45,12 +45,18 @@ def _sum_parallel(ffn_out: PendingProjection, mixer_out: PendingProjection, x: t
     p = ffn_out.partial()
     if p is not None:
         return ResidualSum([p, mixer_out.partial() or mixer_out.run(), x])
+    if ffn_out.additions_cost_a_pass():  # prompts: the next norm adds the three while it reads them
+        return ResidualSum([ffn_out.run(), mixer_out.run(), x])
     return ffn_out.run(add1=mixer_out.run(), add2=x)
 
 
 def _sum_sequential(out: PendingProjection, residual: torch.Tensor):
     p = out.partial()
-    return ResidualSum([p, residual]) if p is not None else out.run(add1=residual)
+    if p is not None:
+        return ResidualSum([p, residual])
+    if out.additions_cost_a_pass():
+        return ResidualSum([out.run(), residual])
+    return out.run(add1=residual)
 
 
 class ParallelBlock(Part):

@@ -184,6 +184,15 @@ class PendingProjection:
     def partial(self) -> Optional[PartialProduct]:
         return self.linear.partial(self.x)
 
+    def additions_cost_a_pass(self) -> bool:
+        """Whether tensors added to this product would be a pass of their own over the result: the vendor
+        library's product of many rows, which has no epilogue of ours, with no bias to add.  The norm that reads
+        the sum next can then form it while it reads (``ResidualSum``)."""
+        x, lin = self.x, self.linear
+        return (x.dtype == torch.bfloat16 and lin.bias is None and ops.layernorm_sum_ok(lin.out_features)
+                and x.shape[0] >= ops.layernorm_sum_rows_min()
+                and not ops.gemm_skinny_ok(x, lin.weight) and not ops.gemm_splitk_ok(x, lin.weight))
+
     @staticmethod
     def partial_pair(first: "PendingProjection", second: "PendingProjection"):
         """Both as partial sums from one launch, or None where that does not apply."""

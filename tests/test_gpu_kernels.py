@@ -168,7 +168,9 @@ def test_layernorm_sum_of_many_rows(H, M):
     ops = _ops()
     x1, x2 = _rand(M, H, seed=4, dtype=torch.bfloat16), _rand(M, H, seed=5, dtype=torch.bfloat16)
     w, b, w2, b2 = _rand(H, seed=6) + 1.0, _rand(H, seed=7), _rand(H, seed=8) + 1.0, _rand(H, seed=9)
-    for terms, want in (([x1], x1), ([x1, x2], (x1.float() + x2.float()).bfloat16())):
+    x3 = _rand(M, H, seed=11, dtype=torch.bfloat16)
+    for terms, want in (([x1], x1), ([x1, x2], (x1.float() + x2.float()).bfloat16()),
+                        ([x1, x2, x3], (x1.float() + x2.float() + x3.float()).bfloat16())):
         x, o1, o2 = ops.layernorm_sum(terms, H, w=w, b=b, eps=1e-5, w2=w2, b2=b2)
         assert torch.equal(x, want)
         for o, (ww, bb) in ((o1, (w, b)), (o2, (w2, b2))):
@@ -178,6 +180,15 @@ def test_layernorm_sum_of_many_rows(H, M):
         few = ops.layernorm_sum([t[:7] for t in terms], H, w=w, b=b, eps=1e-5)[1]  # a workgroup per row
         torch.testing.assert_close(o1[:7].float(), few.float(), rtol=1e-2, atol=1e-2)
     assert torch.equal(ops.layernorm_sum([x1, x2], H)[0], (x1.float() + x2.float()).bfloat16())
+    assert M >= ops.layernorm_sum_rows_min()
+    # three tensors are the sum that a product's epilogue with two additions stores; chosen rows of it (a workgroup per row)
+    y = x1.clone()
+    ops.epilogue_(y, None, None, x2, x3)
+    assert torch.equal(ops.layernorm_sum([x1, x2, x3], H)[0], y)
+    rows = torch.tensor([M - 1, 0, 5], dtype=torch.int32).cuda()
+    picked = ops.layernorm_sum([x1, x2, x3], H, w=w, b=b, eps=1e-5, rows=rows)
+    assert torch.equal(picked[0], y[rows.long()])
+    torch.testing.assert_close(picked[1].float(), F.layer_norm(y[rows.long()].float(), (H,), w, b, 1e-5), rtol=1e-2, atol=1e-2)
 
 
 def test_layernorm_sum_refuses_what_it_cannot_do():
