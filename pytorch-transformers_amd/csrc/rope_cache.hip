@@ -27,6 +27,36 @@ __global__ __launch_bounds__(RC_THREADS) void qkv_rope_cache_kernel(
     const int m = blockIdx.x, tid = threadIdx.x;
     const int g = nh / nkv, half = d >> 1;
     const int pos = token_pos[m];
+    const T* row = fused + (long)m * fused_ld;  // rows of the fused projection may lie apart
+    const int n_slots = write_cache ? nh + 2 * nkv : nh;  // queries, then keys, then values
+    // rotated items: (slot < nh + nkv, pair i < half); plain items: every element of a slot
+    const int rot_slots = inv_freq ? min(n_slots, nh + nkv) : 0;
+    // gridDim.y workgroups share a token's items (a decode step has few tokens and many heads)
+    const int stride = RC_THREADS * gridDim.y, first = tid + blockIdx.y * RC_THREADS;
+    // bfloat16 with halves that are multiples of eight: eight pairs per item, sixteen bytes per access
+    const bool wide = sizeof(T) == 2 && (d & 15) == 0;
+    const int h8 = half >> 3;
+    auto source_head = [&](int kind, int head) {
+        if (layout == PTA_QKV_GROUPED) return kind == 0 ? (head / g) * (g + 2) + (head % g) : head * (g + 2) + g;
+        if (layout == PTA_QKV_TAIL) return kind == 0 ? head : nh;
+        return head * 3 + kind;
+    };
+    // A thread's first two items are asked for before anything else, so that the table of angles is made and the
+    // page looked up while they are on their way: a token's row is read in one round trip to memory, not three.
+    constexpr int AHEAD = 2;
+    uint4 ra[AHEAD], rb[AHEAD];
+    if (wide) {
+#pragma unroll
+        for (int u = 0; u < AHEAD; ++u) {
+            const int item = first + u * stride;
+            if (item < rot_slots * h8) {
+                const int slot = item / h8, i = (item - slot * h8) * 8;
+                const bf16_t* src = (const bf16_t*)row + (long)source_head(slot < nh ? 0 : 1, slot < nh ? slot : slot - nh) * d;
+                ra[u] = *reinterpret_cast<const uint4*>(src + i);
+                rb[u] = *reinterpret_cast<const uint4*>(src + i + half);
+            }
+        }
+    }
     if (inv_freq) {
         // one table for all tokens, or one per sequence of the step (frequencies that follow a sequence's length)
         const float* freq = inv_freq + (inv_freq_ld ? (long)token_seq[m] * inv_freq_ld : 0L);
@@ -40,28 +70,15 @@ __global__ __launch_bounds__(RC_THREADS) void qkv_rope_cache_kernel(
     long page = 0;
     if (write_cache) page = block_table[(long)token_seq[m] * bt_stride + pos / PTA_PAGE];
     const int in_page = pos % PTA_PAGE;
-    const long qout = (long)(nh + 2 * nkv) * d;
-    const T* row = fused + (long)m * fused_ld;  // rows of the fused projection may lie apart
-    const int n_slots = write_cache ? nh + 2 * nkv : nh;  // queries, then keys, then values
 
-    // rotated items: (slot < nh + nkv, pair i < half); plain items: every element of a slot
-    const int rot_slots = inv_freq ? min(n_slots, nh + nkv) : 0;
-    // gridDim.y workgroups share a token's items (a decode step has few tokens and many heads)
-    const int stride = RC_THREADS * gridDim.y, first = tid + blockIdx.y * RC_THREADS;
-    if (sizeof(T) == 2 && (d & 15) == 0) {
-        // bfloat16 with halves that are multiples of eight: eight pairs per item, sixteen bytes per access
-        const int h8 = half >> 3;
-        for (int item = first; item < rot_slots * h8; item += stride) {
+    if (wide) {
+        auto rotate_item = [&](int item, const uint4& va, const uint4& vb) {
             const int slot = item / h8, i = (item - slot * h8) * 8;
             const int kind = slot < nh ? 0 : 1, head = slot < nh ? slot : slot - nh;
-            int src_head;
-            if (layout == PTA_QKV_GROUPED) src_head = kind == 0 ? (head / g) * (g + 2) + (head % g) : head * (g + 2) + g;
-            else if (layout == PTA_QKV_TAIL) src_head = kind == 0 ? head : nh;
-            else src_head = head * 3 + kind;
-            const bf16_t* src = (const bf16_t*)row + (long)src_head * d;
+            const int src_head = source_head(kind, head);
             float a[8], b[8], lo[8], hi[8];
-            unpack8(*reinterpret_cast<const uint4*>(src + i), a);
-            unpack8(*reinterpret_cast<const uint4*>(src + i + half), b);
+            unpack8(va, a);
+            unpack8(vb, b);
             if (bias) {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
@@ -79,6 +96,14 @@ __global__ __launch_bounds__(RC_THREADS) void qkv_rope_cache_kernel(
                                     : (bf16_t*)k_pool + ((page * nkv + head) * PTA_PAGE + in_page) * (long)d;
             *reinterpret_cast<uint4*>(dst + i) = pack8(lo);
             *reinterpret_cast<uint4*>(dst + i + half) = pack8(hi);
+        };
+#pragma unroll
+        for (int u = 0; u < AHEAD; ++u)
+            if (first + u * stride < rot_slots * h8) rotate_item(first + u * stride, ra[u], rb[u]);
+        for (int item = first + AHEAD * stride; item < rot_slots * h8; item += stride) {
+            const int slot = item / h8, i = (item - slot * h8) * 8;
+            const bf16_t* src = (const bf16_t*)row + (long)source_head(slot < nh ? 0 : 1, slot < nh ? slot : slot - nh) * d;
+            rotate_item(item, *reinterpret_cast<const uint4*>(src + i), *reinterpret_cast<const uint4*>(src + i + half));
         }
     } else {
     for (int item = first; item < rot_slots * half; item += stride) {
