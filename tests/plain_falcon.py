@@ -1,7 +1,7 @@
 """A plain, slow Falcon: whole sequences, no cache, one function per part.
 
-Written from the reference's formulas (each function cites file:line of the
-reference checkout); it imports nothing from the engine, reads ``config.json`` as
+Written from the reference's formulas (each function cites the reference's
+file:line); it imports nothing from the engine, reads ``config.json`` as
 a dict and the weights with safetensors' own loader.  Arithmetic is float64 by
 default, so what the 32-bit engine is compared with is closer to exact than the
 engine itself; the places where the reference rounds on purpose (ALiBi's
