@@ -441,6 +441,41 @@ def test_steps_ahead_of_the_host_choose_what_the_loop_that_waits_chooses(folders
                 assert eos not in new[:-1] and (len(new) == 40 or new[-1] == eos) and eos not in new[:2]
 
 
+def test_a_step_from_tokens_on_the_device_equals_the_step_from_the_same_tokens_on_the_host(folders):
+    """Tiny A in bfloat16: three sequences' next step from a ``TokensAhead`` (all rows, then two of them in another
+    order) against the step from the tokens as lists, with captured steps and, where there are none, after a wait."""
+    from pytorch_transformers_amd import AutoModelForCausalLM, GenerationConfig
+    from pytorch_transformers_amd.sampling import Sampler, TokensAhead
+
+    model = AutoModelForCausalLM.from_pretrained(folders["A"], dtype="bfloat16")
+    sampler = Sampler(GenerationConfig(do_sample=False), model.vocab_size, model.device)
+    prompts = [[5, 6, 7, 8], [9, 10], [11, 12, 13, 14, 15, 16]]
+
+    def start():
+        cache = model.new_cache(3 * 64, max_slots=3)
+        slots = [cache.alloc() for _ in prompts]
+        return cache, slots, model.step(cache, slots, prompts, "last")
+
+    for graphs in (True, False):
+        model.use_graphs = graphs
+        assert model.steps_ahead == graphs
+        (c1, s1, l1), (c2, s2, l2) = start(), start()
+        ahead, _ = sampler.sample(l1, rng_seq=[0, 1, 2], rng_step=[0, 0, 0], need_scores=False, ahead=True)
+        assert isinstance(ahead, TokensAhead) and len(ahead) == 3
+        host_tokens, _ = sampler.sample(l2, rng_seq=[0, 1, 2], rng_step=[0, 0, 0], need_scores=False)
+        a = model.step(c1, s1, ahead.take(None), "last", own_logits=False).clone()
+        b = model.step(c2, s2, [[t] for t in host_tokens], "last")
+        assert ahead.tolist() == host_tokens and torch.equal(a, b)
+        # two of the three rows, in another order
+        a = model.step(c1, [s1[2], s1[0]], ahead.take([2, 0]), "last", own_logits=False).clone()
+        b = model.step(c2, [s2[2], s2[0]], [[host_tokens[2]], [host_tokens[0]]], "last")
+        assert torch.equal(a, b)
+        if graphs:
+            with pytest.raises(Exception, match="tokens ahead for 2"):  # three sequences, two rows taken
+                model.step(c1, s1, ahead.take([2, 0]), "last")
+    model.use_graphs = True
+
+
 def test_pipeline_entry(folders):
     from pytorch_transformers_amd import pipeline
 
