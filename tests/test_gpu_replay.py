@@ -10,7 +10,7 @@ import torch
 
 import helpers
 from helpers import REL_BF16, REL_F32
-from tiny import TINY, write_model
+from tiny import TINY, write_config, write_model
 
 pytestmark = pytest.mark.gpu
 
@@ -132,6 +132,32 @@ def test_decoding_across_the_length_bound_of_a_captured_step(folders, dtype, rel
     got = helpers.run_schedule(rp, helpers.schedule_batches(reqs, 3, decode=(90, 40, 12)))
     for rid in reqs:
         helpers.assert_close(got[rid], want[rid], rel, f"D {dtype} across 1024 {rid}")
+
+
+@pytest.mark.parametrize("name", ["A", "C", "E", "B without bias"])
+def test_prompts_of_many_rows_in_one_step(folders, tmp_path, name):
+    """Prompts of 330, 270 and 60 tokens in one step of 660 rows, then a few tokens each: beyond 512 rows the matrix
+    products are the vendor library's, a wave normalises a row, and where no bias stands in the way the norm adds the
+    block's terms itself (bfloat16; both parallel arrangements, ALiBi, and the sequential one)."""
+    from pytorch_transformers_amd import ops
+
+    if name in TINY:
+        folder, vocab = folders[name], TINY[name]["vocab_size"]
+    else:
+        folder, vocab = write_config(dict(TINY["B"], bias=False), str(tmp_path), "B-no-bias", 6), TINY["B"]["vocab_size"]
+    reqs = helpers.make_requests(vocab, [333, 275, 64], seed=21)
+    want = helpers.plain_logits(folder, reqs)
+    rp = _replayer(folder, "bfloat16", max_tokens=3 * 384)
+    sums = []
+    real = ops.layernorm_sum
+    ops.layernorm_sum = lambda terms, H, **kw: (sums.append(len(terms)), real(terms, H, **kw))[1]
+    try:
+        got = helpers.run_schedule(rp, helpers.schedule_batches(reqs, 3, decode=(3, 5, 4)))
+    finally:
+        ops.layernorm_sum = real
+    for rid in reqs:
+        helpers.assert_close(got[rid], want[rid], REL_BF16, f"{name} many rows {rid}")
+    assert max(sums) == (2 if name.startswith("B") else 3), "the norm was handed the block's terms to add"
 
 
 @pytest.mark.parametrize("dtype,rel", [("float32", REL_F32), ("bfloat16", REL_BF16)])
