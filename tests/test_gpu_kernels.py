@@ -789,6 +789,20 @@ def test_attn_mfma_prefill_and_chunks(nh, nkv, d):
     _attn_case(ops, _mfma(ops), torch.bfloat16, nh, nkv, d, starts=[0, 63, 200, 0, 127, 31], news=[70, 1, 5, 1, 2, 40])
 
 
+@pytest.mark.parametrize("nh,nkv,d", [(71, 1, 64), (16, 2, 64), (8, 2, 128), (6, 1, 48)])
+def test_attn_mfma_long_prompts(nh, nkv, d):
+    """A prompt of 1,300 tokens and 500 new tokens over 900 cached ones in one launch: many stages of keys per
+    workgroup, column groups of every length, with one far key that stands out for the last query of each."""
+    ops = _ops()
+    _attn_case(ops, _mfma(ops), torch.bfloat16, nh, nkv, d, starts=[0, 900, 3], news=[1300, 500, 61], boost=[7, 1390, None])
+    slopes = None
+    if nh == 16:
+        from pytorch_transformers_amd.parts import AlibiPositions
+        slopes = AlibiPositions(nh).slopes.cuda()
+        _attn_case(ops, _mfma(ops), torch.bfloat16, nh, nkv, d, starts=[0, 700], news=[800, 300], slopes=slopes, seed=3)
+        _attn_case(ops, _mfma(ops), torch.bfloat16, nh, nkv, d, starts=[0, 700], news=[800, 300], window=200, seed=4)
+
+
 @pytest.mark.parametrize("nh,nkv,d", [(71, 1, 64), (6, 2, 32), (3, 3, 16), (8, 2, 128), (2, 1, 256)])
 @pytest.mark.parametrize("split", [64, 256])
 def test_attn_mfma_decode_split(nh, nkv, d, split):
