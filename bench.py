@@ -243,7 +243,9 @@ def main():
                     help="one batch of unequal prompts through generate(): 11b 16 x U[128,4096] + 256 new, "
                          "40b 32 x U[64,1536] + 512 new; prints its own record")
     ap.add_argument("--only-prefill", action="store_true",
-                    help="run the 2,048-token prefill alone and print its record (for profiling)")
+                    help="run the prefill alone and print its record (for profiling)")
+    ap.add_argument("--prefill-tokens", type=int, default=2048,
+                    help="with --only-prefill: the prompt's length (the default run's prefill is of 2,048 tokens)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -288,14 +290,16 @@ def main():
         return 0
     # the choices between kernels that are timed rather than ruled, once, for the shapes measured below; the timed
     # steps themselves time nothing
-    model.tune(prompt_lens=(2048,), batches=sorted({args.batch, 1, 64}),
-               contexts=sorted({args.prompt_len + 1, args.prompt_len + args.warmup + args.steps}))
     if args.only_prefill:
-        pt = run_prefill(model, 2048)
-        print(json.dumps({"prefill": {"value": round(2048 / pt, 1), "tokens": 2048, "ms": round(pt * 1e3, 3),
-                                      "frac": round(prefill_flops(cfg, 2048) / pt / (PEAK_TFLOPS[args.dtype] * 1e12), 4)},
+        T = args.prefill_tokens
+        model.tune(prompt_lens=(T,), batches=())
+        pt = run_prefill(model, T)
+        print(json.dumps({"prefill": {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3),
+                                      "frac": round(prefill_flops(cfg, T) / pt / (PEAK_TFLOPS[args.dtype] * 1e12), 4)},
                           "layers": args.layers, "dtype": args.dtype}))
         return 0
+    model.tune(prompt_lens=(2048,), batches=sorted({args.batch, 1, 64}),
+               contexts=sorted({args.prompt_len + 1, args.prompt_len + args.warmup + args.steps}))
 
     dt, mean_ctx = run_decode(model, Sampler, gen_cfg, args.batch, args.prompt_len, args.steps, args.warmup)
     ms = dt / args.steps * 1e3
