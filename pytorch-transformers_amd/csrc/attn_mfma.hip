@@ -654,11 +654,16 @@ static bool launch_decode(const AttnLaunch& a, int tiles) {
 // prompts: four waves of two column tiles share each stage of keys through LDS (head sizes up to 128;
 // beyond, one wave per workgroup).  Heads up to 64 fit four waves a SIMD (measured at 8,192 tokens, 71 heads
 // on one KV head of 64: as many registers as the compiler likes, three waves, 800 us a layer; four waves 760;
-// a third column tile, 256 registers, two waves, 817).
+// a third column tile, 256 registers, two waves, 817), and with many column groups eight waves share a stage
+// (`wide`: 256 columns a workgroup, half the staging for every wave).
+constexpr int prompt_columns(int dt, bool wide) { return dt <= 4 && wide ? 256 : dt <= 8 ? 128 : 16; }
+
 template <int DT>
-static void launch_prompt(const AttnLaunch& a) {
-    if constexpr (DT <= 4) launch_attn<DT, 2, 4, 1, 4>(a);
-    else if constexpr (DT <= 8) launch_attn<DT, 2, 4>(a);
+static void launch_prompt(const AttnLaunch& a, bool wide) {
+    if constexpr (DT <= 4) {
+        if (wide) launch_attn<DT, 2, 8, 1, 4>(a);
+        else launch_attn<DT, 2, 4, 1, 4>(a);
+    } else if constexpr (DT <= 8) launch_attn<DT, 2, 4>(a);
     else launch_attn<DT, 1, 1>(a);
 }
 
@@ -700,10 +705,19 @@ extern "C" int pta_attn_mfma(void* out, const void* q, const void* k_pool, const
     // paired; pairs win where the two are equal (32 heads on 8 KV heads of 128: 2,048 tokens 92 -> 77 us a layer,
     // 8,192 tokens 787 -> 657; 128 on 8 of 64: 123 -> 103 and 1,264 -> 1,214) and lose where they are not (71 on
     // 1 of 64: 68 -> 89, and 737 -> 766 where the two differ by 2 %).
+    // Eight waves a workgroup where that still leaves four workgroups and more for every compute unit (71 heads on
+    // 1 KV head of 64: 2,048 tokens 67 -> 72 us a layer, 4,096 the same, 8,192 712 -> 693, 16,384 2,542 -> 2,433;
+    // 128 on 8 of 64: 2,048 tokens 101 -> 94, 8,192 1,213 -> 1,151).
     static const int pair_env = getenv("PTA_ATTN_PAIR") ? atoi(getenv("PTA_ATTN_PAIR")) : -1;
+    const char* wide_set = getenv("PTA_ATTN_WIDE");  // looked up at every launch: tests switch it
+    const int wide_env = wide_set ? atoi(wide_set) : -1;
     int paired = 0;
+    bool wide = false;
     if (!narrow) {
-        const double wgs = std::ceil((double)M * (nh / nkv) / (d <= 128 ? 128 : 16)) * nkv, units = pta_compute_units();
+        const double units = pta_compute_units();
+        const double wide_wgs = std::ceil((double)M * (nh / nkv) / prompt_columns(d / 16, true)) * nkv;
+        wide = d <= 64 && (wide_env >= 0 ? wide_env != 0 : wide_wgs >= 4.0 * units);
+        const double wgs = std::ceil((double)M * (nh / nkv) / prompt_columns(d / 16, wide)) * nkv;
         paired = pair_env >= 0 ? pair_env : 2.0 * std::ceil(wgs / 2.0 / units) <= 1.01 * std::max(wgs / units, 2.0);
     }
     const int dct_most = std::min((nh / nkv + 15) / 16, pta_attn_decode_max_tiles(d));
@@ -719,7 +733,7 @@ extern "C" int pta_attn_mfma(void* out, const void* q, const void* k_pool, const
                        split_size, n_splits, window, paired, narrow ? decode_waves : 1, s};
 #define PTA_ATTN_CASE(DT_)                                        \
     case DT_:                                                     \
-        if (!narrow) launch_prompt<DT_>(a);                       \
+        if (!narrow) launch_prompt<DT_>(a, wide);                 \
         else if (!launch_decode<DT_>(a, dct))                     \
             return pta_fail("attn_mfma: no kernel for %d waves and %d column tiles at head size %d", decode_waves, dct, d); \
         break;

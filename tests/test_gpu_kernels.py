@@ -1,5 +1,6 @@
 """Each kernel alone against a plain torch computation, at sizes other than the tiny models' (GPU)."""
 import math
+import os
 
 import pytest
 import torch
@@ -795,6 +796,15 @@ def test_attn_mfma_long_prompts(nh, nkv, d):
     workgroup, column groups of every length, with one far key that stands out for the last query of each."""
     ops = _ops()
     _attn_case(ops, _mfma(ops), torch.bfloat16, nh, nkv, d, starts=[0, 900, 3], news=[1300, 500, 61], boost=[7, 1390, None])
+    if d <= 64:
+        # workgroups of eight waves, which launches with four such workgroups a compute unit and more choose by themselves
+        os.environ["PTA_ATTN_WIDE"] = "1"
+        try:
+            _attn_case(ops, _mfma(ops), torch.bfloat16, nh, nkv, d, starts=[0, 900, 3], news=[1300, 500, 61], boost=[7, 1390, None])
+            _attn_case(ops, _mfma(ops), torch.bfloat16, nh, nkv, d, starts=[0, 63, 200, 0, 127, 31], news=[70, 1, 5, 1, 2, 40])
+            _attn_case(ops, _mfma(ops), torch.bfloat16, nh, nkv, d, starts=[0, 700], news=[800, 300], window=200, seed=4)
+        finally:
+            del os.environ["PTA_ATTN_WIDE"]
     slopes = None
     if nh == 16:
         from pytorch_transformers_amd.parts import AlibiPositions
