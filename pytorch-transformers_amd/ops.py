@@ -1016,7 +1016,9 @@ def tune_pair_parts(w1: torch.Tensor, w2: torch.Tensor) -> None:
     apply, but the ranges do).  ``_pair_parts_tuned`` says what is in use: (ranges, ranges, row tiles per wave).
     Then, at 8, 32, 64 and 128 rows (one count per class of rows), the launch with stationary activations is timed
     against the winner with one to six ranges of the shorter K (and as many times more of the longer), each
-    charged for the partial sums that its ranges leave to be read: the fastest is fixed for the class, or the staged kernel where that is not beaten by 2 % (``_pair_stationary_tuned``)."""
+    with what reads its partial sums behind it (the norm that adds them, where the two products have one width; else
+    a charge for the ranges' bytes): the fastest is fixed for the class, or the staged kernel where that is not
+    beaten by 2 % (``_pair_stationary_tuned``)."""
     key = (tuple(w1.shape), tuple(w2.shape))
     if not PAIR_TUNE or key in _pair_parts_tuned or not _may_time():
         return
@@ -1035,6 +1037,7 @@ def tune_pair_parts(w1: torch.Tensor, w2: torch.Tensor) -> None:
     cands = [c for c in cands if fix(c) == 0]
     xs = {rows: [torch.randn((rows, K), dtype=torch.float32, device=w1.device).to(torch.bfloat16) for K in (K1, K2)]
           for rows in sorted({PAIR_TUNE_ROWS, 24, 8, 32, 64, 128})}
+    xs_bf16 = {rows: torch.zeros((rows, N1), dtype=torch.bfloat16, device=w1.device) for rows in xs}
     kmin = min(K1, K2)
     f1, f2 = max(1, (K1 + kmin // 2) // kmin), max(1, (K2 + kmin // 2) // kmin)
     st_cands = [(b * f1, b * f2) for b in (1, 2, 3, 4, 6) if b * f1 <= 16 and b * f2 <= 16 and fix_st(0, (b * f1, b * f2)) == 0]
@@ -1048,7 +1051,7 @@ def tune_pair_parts(w1: torch.Tensor, w2: torch.Tensor) -> None:
     n_copies = max(2, min(6, int(640e6 // copy_bytes) + 1))
     copies = [(w1, w2)] + [(w1.clone(), w2.clone()) for _ in range(n_copies - 1)]
 
-    def timed_ways(chosen, rows, rounds=3, fix=fix):
+    def timed_ways(chosen, rows, rounds=3, fix=fix, read=None):
         best = [float("inf")] * len(chosen)
         for r in range(rounds + 1):  # the first round warms up
             for j, c in enumerate(chosen):
@@ -1058,11 +1061,23 @@ def tune_pair_parts(w1: torch.Tensor, w2: torch.Tensor) -> None:
                 for a, b in copies:
                     _call("pta_gemm_splitk_pair_bf16", _ptr(parts[0]), _ptr(xs[rows][0]), _ptr(a), int(N1), int(K1),
                           _ptr(parts[1]), _ptr(xs[rows][1]), _ptr(b), int(N2), int(K2), rows, _stream())
+                    if read is not None:
+                        read(c, rows)
                 end.record()
                 end.synchronize()
                 if r > 0:
                     best[j] = min(best[j], start.elapsed_time(end) / len(copies))
         return best
+
+    # Two products of the same width are a block's last ones, and what reads their partial sums next is the norm
+    # that adds them: it is launched behind every timed launch of the comparison below, so that a launch pays for
+    # the ranges it leaves to be added and for how it leaves them (all at once at its end, or as it goes).
+    norm_w = (torch.ones(N1, dtype=torch.float32, device=w1.device)
+              if N1 == N2 and layernorm_sum_ok(N1) and os.environ.get("PTA_PAIR_TUNE_READER", "1") != "0" else None)
+
+    def read_sums(c, rows):
+        views = [parts[i].view(-1)[:int(c[-2 + i]) * rows * N].view(int(c[-2 + i]), rows, N) for i, N in enumerate((N1, N2))]
+        layernorm_sum([(views[1], None), (views[0], None), xs_bf16[rows]], N1, w=norm_w, b=norm_w, eps=1e-5)
 
     try:
         times = timed_ways(cands, PAIR_TUNE_ROWS)
@@ -1091,9 +1106,11 @@ def tune_pair_parts(w1: torch.Tensor, w2: torch.Tensor) -> None:
             fix_st(cls, (0, 0))
             # what reads the partial sums afterwards pays for every range (measured: some 8 TB/s worth of them), so
             # a launch is charged for its ranges' bytes at that rate on top of its own time
-            slices_ms = lambda c: (c[0] * N1 + c[1] * N2) * rows * 4 / 8e12 * 1e3
-            t_staged = timed_ways([chosen], rows)[0] + slices_ms(chosen)
-            t_st = timed_ways([(cls, c) for c in st_cands], rows, fix=lambda a: fix_st(a[0], a[1])) if st_cands else []
+            read = read_sums if norm_w is not None else None
+            slices_ms = (lambda c: 0.0) if read else (lambda c: (c[0] * N1 + c[1] * N2) * rows * 4 / 8e12 * 1e3)
+            t_staged = timed_ways([chosen[:2]], rows, fix=lambda c: None, read=read)[0] + slices_ms(chosen)
+            t_st = (timed_ways([(cls,) + c for c in st_cands], rows, fix=lambda a: fix_st(a[0], a[1:]), read=read)
+                    if st_cands else [])
             t_st = [t + slices_ms(c) for t, c in zip(t_st, st_cands)]
             best = min(range(len(st_cands)), key=lambda i: t_st[i]) if st_cands else -1
             keep = st_cands[best] if best >= 0 and t_st[best] < 0.98 * t_staged else (0, 0)
