@@ -539,41 +539,80 @@ __global__ __launch_bounds__(64 * W * KS, OCC) void attn_mfma_kernel(
     }  // pass
 }
 
-// out[row, :] = sum_s w_s po[row, s, :] / sum_s w_s pl[row, s], w_s = 2^(pm[row, s] - max_s pm), splits in
-// order.  A split whose maximum is -inf (a range past the row's keys) has weight zero and is not read.
-__global__ __launch_bounds__(64) void attn_combine_kernel(bf16_t* __restrict__ out, const float* __restrict__ po,
-                                                          const float* __restrict__ pm, const float* __restrict__ pl,
-                                                          int D, int n_splits) {
-    __shared__ float w_s[1024];
+// out[row, :] = sum_s w_s po[row, s, :] / sum_s w_s pl[row, s], w_s = 2^(pm[row, s] - max_s pm).  A split whose
+// maximum is -inf (a range past the row's keys) has weight zero and is not read.
+//
+// A row's splits are many short vectors, and a chain of loads one behind the other is what this kernel's time
+// would be: so LPS lanes (the next power of two from D/4) take one split's vector as float4 each, the 64/LPS
+// groups of a wave and the WAVES waves of the workgroup take every (64/LPS * WAVES)-th split, four of them in
+// flight per group; the groups' sums are added across the wave by lane exchange and across waves through LDS in
+// wave order.  The order of the additions depends on (n_splits, D, WAVES) alone.
+template <int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void attn_combine_kernel(bf16_t* __restrict__ out, const float* __restrict__ po,
+                                                                  const float* __restrict__ pm, const float* __restrict__ pl,
+                                                                  int D, int n_splits, int lps) {
+    __shared__ float part[WAVES][256 + 4];
     const long row = blockIdx.x;
-    const int lane = threadIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const float* m = pm + row * n_splits;
     const float* l = pl + row * n_splits;
     float mx = -INFINITY;
     for (int s = lane; s < n_splits; s += 64) mx = fmaxf(mx, m[s]);
     mx = wave_max(mx);
+    const int per_wave = 64 / lps, g = lane / lps, c = (lane % lps) * 4;
+    const bool active = c < D;
+    const int stride = per_wave * WAVES;
+    const float* p = po + row * (long)n_splits * D + c;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
     float L = 0.f;
-    int used = 0;
-    for (int s0 = 0; s0 < n_splits; s0 += 64) {  // lanes in order, chunks in order: a fixed summation order
-        const int s = s0 + lane;
-        float w = 0.f;
-        if (s < n_splits && m[s] != -INFINITY) { w = __builtin_amdgcn_exp2f(m[s] - mx); used = s + 1; }
-        if (s < n_splits) w_s[s] = w;
-        L += wave_sum(w * (s < n_splits ? l[s] : 0.f));
-    }
-    used = (int)wave_max((float)used);
-    __syncthreads();
-    const float inv = 1.0f / L;
-    for (int dd = lane; dd < D; dd += 64) {
-        float acc = 0.f;
-        const float* p = po + row * (long)n_splits * D + dd;
-        int s = 0;
-        for (; s + 4 <= used; s += 4) {
-            const float v0 = p[(long)s * D], v1 = p[(long)(s + 1) * D], v2 = p[(long)(s + 2) * D], v3 = p[(long)(s + 3) * D];
-            acc += w_s[s] * v0; acc += w_s[s + 1] * v1; acc += w_s[s + 2] * v2; acc += w_s[s + 3] * v3;
+    for (int s0 = wave * per_wave + g; s0 < n_splits; s0 += 4 * stride) {
+        float w[4], ll[4];
+        float4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int s = s0 + u * stride;
+            w[u] = 0.f; ll[u] = 0.f; v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (s < n_splits) {
+                const float ms = m[s];
+                if (ms != -INFINITY) {
+                    w[u] = __builtin_amdgcn_exp2f(ms - mx);
+                    ll[u] = l[s];
+                    if (active) v[u] = *reinterpret_cast<const float4*>(p + (long)s * D);
+                }
+            }
         }
-        for (; s < used; ++s) acc += w_s[s] * p[(long)s * D];
-        out[row * D + dd] = f32_to_bf16_bits(acc * inv);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            acc.x += w[u] * v[u].x; acc.y += w[u] * v[u].y; acc.z += w[u] * v[u].z; acc.w += w[u] * v[u].w;
+            L += w[u] * ll[u];
+        }
+    }
+    for (int off = lps; off < 64; off <<= 1) {
+        acc.x += __shfl_xor(acc.x, off); acc.y += __shfl_xor(acc.y, off);
+        acc.z += __shfl_xor(acc.z, off); acc.w += __shfl_xor(acc.w, off);
+        L += __shfl_xor(L, off);
+    }
+    if constexpr (WAVES > 1) {
+        if (g == 0 && active) *reinterpret_cast<float4*>(&part[wave][c]) = acc;
+        if (lane == 0) part[wave][256] = L;
+        __syncthreads();
+        if (wave != 0) return;
+        acc = make_float4(0.f, 0.f, 0.f, 0.f);
+        L = 0.f;
+        if (active) {
+#pragma unroll
+            for (int wv = 0; wv < WAVES; ++wv) {
+                const float4 a = *reinterpret_cast<const float4*>(&part[wv][c]);
+                acc.x += a.x; acc.y += a.y; acc.z += a.z; acc.w += a.w;
+                L += part[wv][256];
+            }
+        }
+    }
+    if (g == 0 && active) {
+        const float inv = 1.0f / L;
+        bf16_t r[4] = {f32_to_bf16_bits(acc.x * inv), f32_to_bf16_bits(acc.y * inv), f32_to_bf16_bits(acc.z * inv),
+                       f32_to_bf16_bits(acc.w * inv)};
+        *reinterpret_cast<uint2*>(out + row * D + c) = *reinterpret_cast<const uint2*>(r);
     }
 }
 
@@ -754,8 +793,13 @@ extern "C" int pta_attn_mfma(void* out, const void* q, const void* k_pool, const
     int rc = pta_check_launch("attn_mfma");
     if (rc) return rc;
     if (n_splits > 1) {
-        hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)((long)M * nh)), dim3(64), 0, s, (bf16_t*)out, po, pm, pl, d,
-                           n_splits);
+        int lps = 4;  // lanes that share a split's vector of d floats, a float4 each
+        while (lps * 4 < d) lps *= 2;
+        const dim3 rows((unsigned)((long)M * nh));
+        if (n_splits > 4 * (64 / lps))  // more splits than one wave has in flight at once
+            hipLaunchKernelGGL(attn_combine_kernel<4>, rows, dim3(256), 0, s, (bf16_t*)out, po, pm, pl, d, n_splits, lps);
+        else
+            hipLaunchKernelGGL(attn_combine_kernel<1>, rows, dim3(64), 0, s, (bf16_t*)out, po, pm, pl, d, n_splits, lps);
         rc = pta_check_launch("attn_combine");
     }
     return rc;
