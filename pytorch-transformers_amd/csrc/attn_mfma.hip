@@ -98,8 +98,9 @@ __device__ __forceinline__ void load_block(KvBlock<DT>& b, int kb, const int* __
 }
 
 // W = 1: a workgroup is one wave, which loads its keys and values straight from global memory.
-// W = 4 (prompts): four waves with neighbouring column groups walk the keys together and share every
-// block through LDS, so that a block crosses the vector memory path once for 64 * CT columns.
+// W > 1 (prompts; one token per sequence with many heads on a KV head): W waves with neighbouring column groups
+// walk the keys together and share every block through LDS, so that a block crosses the vector memory path once
+// for 16 * W * CT columns.
 // WIN: the launch has a window (a kernel of its own, so that launches without one pay nothing for it).
 // KS > 1 (one token per sequence): KS waves of a workgroup hold the same columns and take every KS-th block of the
 // workgroup's keys; their partial results meet in LDS, so that a context walked by KS waves needs no second launch.
@@ -706,6 +707,30 @@ static void launch_prompt(const AttnLaunch& a, bool wide) {
     else launch_attn<DT, 1, 1>(a);
 }
 
+// One token per sequence, the heads of a KV head on the waves of one workgroup, which share its keys through LDS
+// as a prompt's column groups do: a wave per tile of sixteen heads for four or five tiles (49 to 80 heads on a KV
+// head), four waves of two tiles for six to eight.  Built for head sizes 64 and 128.  Fewer heads on a KV head fit
+// the tiles of one wave (`launch_decode`), which reads the keys once as well.
+constexpr bool decode_shared_built(int dt, int tiles) { return (dt == 4 || dt == 8) && tiles >= 4 && tiles <= 8; }
+
+template <int DT>
+static bool launch_decode_shared(const AttnLaunch& a) {
+    if constexpr (DT == 4 || DT == 8) {
+        constexpr int OCC = DT <= 4 ? 4 : 1;
+        const int tiles = (a.nh / a.nkv + 15) / 16;
+        if (tiles == 4) launch_attn<DT, 1, 4, 1, OCC>(a);
+        else if (tiles == 5) launch_attn<DT, 1, 5, 1, OCC>(a);
+        else if (tiles >= 6 && tiles <= 8) launch_attn<DT, 2, 4, 1, OCC>(a);
+        else return false;
+        return true;
+    }
+    return false;
+}
+
+extern "C" int pta_attn_decode_shared_ok(int d, int heads_per_kv_head) {
+    return d % 16 == 0 && heads_per_kv_head > 0 && decode_shared_built(d / 16, (heads_per_kv_head + 15) / 16);
+}
+
 extern "C" int pta_attn_mfma_supported(int d) { return d % 16 == 0 && ((d >= 16 && d <= 128) || d == 256); }
 
 extern "C" int pta_attn_decode_max_tiles(int d) { return decode_max_tiles(d / 16); }
@@ -736,7 +761,16 @@ extern "C" int pta_attn_mfma(void* out, const void* q, const void* k_pool, const
     // tiles of its KV head (at most what the head size leaves registers for).  More tiles: the keys cross the memory
     // path fewer times; fewer: shorter waves, more of them (71 heads on one KV head, 2,048 keys: 64
     // sequences 39.5 us a layer with one tile, 27.5 us with five; 8 sequences 14.6 and 18.5 us).
-    const bool narrow = max_new == 1;
+    // `decode_waves` 0: the heads of a KV head on the waves of one workgroup, keys shared through LDS
+    // (`launch_decode_shared`; `decode_tiles` does not apply).  71 heads on one KV head of 64, with the merge of
+    // the ranges, after a flush of the caches: 64 sequences of 1,100 keys 12.6 us against 17.5 with the best cut
+    // of one-wave workgroups, of 2,100 keys 14.8 against 26.0; 8 sequences of 16,384 keys 19.8 against 24.8; 8
+    // sequences of 1,100 keys 11.4 against 9.8.
+    const bool shared = max_new == 1 && decode_waves == 0;
+    PTA_REQUIRE(!shared || pta_attn_decode_shared_ok(d, nh / nkv),
+                "attn_mfma: a decode launch with keys shared through LDS is not built for %d heads on a KV head of "
+                "size %d (49 to 128 heads, sizes 64 and 128)", nh / nkv, d);
+    const bool narrow = max_new == 1 && !shared;
     // Prompts: whether workgroups take a late and an early column group each.  Paired workgroups all do the
     // same work, which ends a launch evenly if their number fills the compute units evenly; unpaired ones are
     // twice as many and of all lengths, which the longest-first order spreads well over any number of units.
@@ -752,7 +786,7 @@ extern "C" int pta_attn_mfma(void* out, const void* q, const void* k_pool, const
     const int wide_env = wide_set ? atoi(wide_set) : -1;
     int paired = 0;
     bool wide = false;
-    if (!narrow) {
+    if (!narrow && !shared) {
         const double units = pta_compute_units();
         const double wide_wgs = std::ceil((double)M * (nh / nkv) / prompt_columns(d / 16, true)) * nkv;
         wide = d <= 64 && (wide_env >= 0 ? wide_env != 0 : wide_wgs >= 4.0 * units);
@@ -772,7 +806,9 @@ extern "C" int pta_attn_mfma(void* out, const void* q, const void* k_pool, const
                        split_size, n_splits, window, paired, narrow ? decode_waves : 1, s};
 #define PTA_ATTN_CASE(DT_)                                        \
     case DT_:                                                     \
-        if (!narrow) launch_prompt<DT_>(a, wide);                 \
+        if (shared) {                                             \
+            if (!launch_decode_shared<DT_>(a)) return pta_fail("attn_mfma: no kernel with shared keys at head size %d", d); \
+        } else if (!narrow) launch_prompt<DT_>(a, wide);          \
         else if (!launch_decode<DT_>(a, dct))                     \
             return pta_fail("attn_mfma: no kernel for %d waves and %d column tiles at head size %d", decode_waves, dct, d); \
         break;

@@ -14,7 +14,7 @@
 
 #include <stdint.h>
 
-#define PTA_ABI_VERSION 6
+#define PTA_ABI_VERSION 7
 
 #ifdef __cplusplus
 extern "C" {
@@ -77,6 +77,10 @@ int pta_attn_decode_max_tiles(int d);
 // decode_waves (max_new == 1): waves of a workgroup that take its range of keys block by block in turn and merge
 // their results in LDS (1, 4 or 8; pta_attn_decode_waves_ok says whether the combination with decode_tiles is built).
 int pta_attn_decode_waves_ok(int d, int tiles, int waves);
+// decode_waves 0 (max_new == 1): the heads of a KV head go to the waves of one workgroup, which share its range of
+// keys through LDS (decode_tiles does not apply); pta_attn_decode_shared_ok says whether that is built for this head
+// size and this many heads on a KV head.
+int pta_attn_decode_shared_ok(int d, int heads_per_kv_head);
 int pta_attn_mfma(void* out, const void* q, const void* k_pool, const void* v_pool, const int* block_table,
                   int bt_stride, const int* cu_tokens, const int* seq_start, const float* slopes, int alibi_exact,
                   int n_seqs, int max_new, int M, int nh, int nkv, int d, float scale, int split_size, int n_splits, float* po,

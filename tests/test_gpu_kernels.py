@@ -875,22 +875,60 @@ def test_attn_mfma_decode_waves_refusals():
         _attn_case(ops, _mfma(ops, None, 1, 2), torch.bfloat16, 71, 1, 64, starts=[5], news=[1])
 
 
+@pytest.mark.parametrize("nh,nkv,d", [(71, 1, 64), (64, 1, 64), (100, 1, 64), (130, 2, 128), (56, 1, 128), (128, 1, 128)])
+def test_attn_mfma_decode_shared_keys(nh, nkv, d):
+    """One token per sequence, the heads of a KV head on the waves of one workgroup that shares its keys through
+    LDS (four and five waves of one tile, four of two): the whole context in one workgroup and ranges of 128, 256
+    and 512 keys merged afterwards; contexts shorter than a stage, page edges, ALiBi, a window, and one far key
+    that must dominate in whichever range it lies."""
+    ops = _ops()
+    from pytorch_transformers_amd.parts import AlibiPositions
+    assert ops.attn_decode_shared_ok(d, nh // nkv)
+    starts = [0, 63, 64, 700, 255, 256, 1, 31, 32, 1500]
+    boost = [0, 40, None, 333, None, 17, None, None, 31, 1203]
+    shared = ops.SHARED_KEYS
+    for split in (None, 128, 256, 512):
+        _attn_case(ops, _mfma(ops, split, 0, shared), torch.bfloat16, nh, nkv, d, starts=starts, news=[1] * 10, boost=boost)
+    slopes = AlibiPositions(nh).slopes.cuda()
+    for split in (None, 256):
+        _attn_case(ops, _mfma(ops, split, 0, shared), torch.bfloat16, nh, nkv, d, starts=starts, news=[1] * 10, slopes=slopes)
+    for window in (33, 100):
+        for split in (None, 256):
+            _attn_case(ops, _mfma(ops, split, 0, shared), torch.bfloat16, nh, nkv, d, starts=starts, news=[1] * 10,
+                       window=window)
+
+
+def test_attn_mfma_decode_shared_keys_refusals():
+    ops = _ops()
+    assert ops.attn_decode_shared_ok(64, 71) and ops.attn_decode_shared_ok(128, 49) and ops.attn_decode_shared_ok(64, 128)
+    assert not ops.attn_decode_shared_ok(64, 48) and not ops.attn_decode_shared_ok(64, 129)
+    assert not ops.attn_decode_shared_ok(48, 71) and not ops.attn_decode_shared_ok(256, 71)
+    for nh, nkv, d in ((32, 8, 128), (71, 1, 48)):
+        with pytest.raises(ops.KernelError, match="keys shared through LDS is not built"):
+            _attn_case(ops, _mfma(ops, None, 0, ops.SHARED_KEYS), torch.bfloat16, nh, nkv, d, starts=[5], news=[1])
+
+
 def test_decode_plan():
     """The cut of a decode launch: whole tiles within what the head size allows, a range size that is a
     multiple of the page, the same for every batch and context of one captured step's bucket."""
     ops = _ops()
+    bucket_keys = lambda n, length: (1 << (n - 1).bit_length()) * ((length + 1023) // 1024 * 1024)
+    assert ops.decode_plan(64, 71, 1, 64, 1100)[2] == ops.SHARED_KEYS and ops.decode_plan(8, 71, 1, 64, 1100)[2] == 1
     for nh, nkv, d in ((71, 1, 64), (32, 8, 128), (128, 8, 64), (6, 2, 32), (2, 1, 256)):
         groups = (nh // nkv + 15) // 16
         for n in (1, 3, 8, 33, 64, 128, 300, 512):
             for length in (1, 100, 1024, 1025, 2049, 8192, 32768, 65536, 100000):
                 tiles, size, waves = ops.decode_plan(n, nh, nkv, d, length)
-                assert 1 <= tiles <= groups and size % 64 == 0 and size >= 128 and waves == 1  # the rule: one wave
+                # the rule: one wave a workgroup, or, with many heads on a KV head and keys enough, shared keys
+                assert 1 <= tiles <= groups and size % 64 == 0 and size >= 128
+                assert waves == 1 or (waves == ops.SHARED_KEYS and ops.attn_decode_shared_ok(d, nh // nkv)
+                                      and bucket_keys(n, length) >= 20000)
                 assert (length + size - 1) // size <= 1024
                 bucket_n = 1 << (n - 1).bit_length()
                 # the launch has one workgroup row per (sequence of the padded batch, range): the grid's limit
                 assert bucket_n * ((((length + 1023) // 1024 * 1024) + size - 1) // size) <= 65535
                 bucket_len = (length + 1023) // 1024 * 1024
-                assert (tiles, size, 1) == ops.decode_plan(bucket_n, nh, nkv, d, bucket_len)
+                assert (tiles, size, waves) == ops.decode_plan(bucket_n, nh, nkv, d, bucket_len)
                 for mean in (1, length // 3 + 1, length):
                     cut = ops.decode_plan(n, nh, nkv, d, length, mean)
                     assert cut == ops.decode_plan(bucket_n, nh, nkv, d, bucket_len, min(bucket_len, (mean + 511) // 512 * 512))
@@ -937,25 +975,28 @@ def test_decode_attention_as_planned(nh, nkv, d, n, lengths):
     far = v_pool[int(bt[0, 0]), :, :, 5].float().repeat_interleave(nh // nkv, 0).reshape(-1)
     assert float((got[0] - far).abs().max()) < 0.05, "the far key does not dominate"
     tiles, size, waves = ops.decode_plan(n, nh, nkv, d, ctx.max_len, ctx.mean_len)
-    assert 1 <= tiles <= (nh // nkv + 15) // 16 and size % 64 == 0 and waves == 1
+    assert 1 <= tiles <= (nh // nkv + 15) // 16 and size % 64 == 0 and waves in (1, ops.SHARED_KEYS)
     # the same launch with every other cut that may be timed against the rule's: the same result within rounding;
     # a fixed cut holds for the step's bucket and for no other, travels in the tuning table, and is forgotten with it
     key = ops._decode_key(n, nh, nkv, d, ctx.max_len, ctx.mean_len)
     cuts = ops.decode_plan_candidates(key)
-    assert cuts[0] == (tiles, size, 1) and len(set(cuts)) == len(cuts) > 3 and any(c[2] > 1 for c in cuts)
+    assert cuts[0] == (tiles, size, waves) and len(set(cuts)) == len(cuts) > 3 and any(c[2] > 1 for c in cuts)
+    assert any(c[2] == ops.SHARED_KEYS for c in cuts) == ops.attn_decode_shared_ok(d, nh // nkv)
     try:
         with ops.live_tuning():
             ops.take_decode_keys()
             ops.attention(q, k_pool, v_pool, bt.cuda(), ctx, None, scale)
             assert ops.take_decode_keys() == [key] and ops.take_decode_keys() == []
         for cut in cuts[1:]:
-            assert ops.load_library().pta_attn_decode_waves_ok(d, cut[0], cut[2]) and cut[1] % 64 == 0
+            assert cut[1] % 64 == 0 and (ops.attn_decode_shared_ok(d, nh // nkv) if cut[2] == ops.SHARED_KEYS
+                                         else ops.load_library().pta_attn_decode_waves_ok(d, cut[0], cut[2]))
             ops.set_decode_plan(key, cut)
             assert ops.decode_plan(n, nh, nkv, d, ctx.max_len, ctx.mean_len) == cut
             fixed = ops.attention(q, k_pool, v_pool, bt.cuda(), ctx, None, scale).float()
             assert float((fixed - want).abs().max()) <= 2e-2 * max(1.0, float(want.abs().max())), cut
             assert float((fixed[0] - far).abs().max()) < 0.05, cut
-        assert ops.decode_plan(n, nh, nkv, d, ctx.max_len + 2048, ctx.mean_len)[2] == 1  # another bucket: the rule
+        other = ops.decode_plan(n, nh, nkv, d, ctx.max_len + 2048, ctx.mean_len)  # another bucket: the rule
+        assert other == ops.decode_plan_candidates(ops._decode_key(n, nh, nkv, d, ctx.max_len + 2048, ctx.mean_len))[0]
         table = ops.tuning_table()
         assert table["decode_plans"][",".join(str(v) for v in key)] == list(cuts[-1])
         ops.clear_tuning()
