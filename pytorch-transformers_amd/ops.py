@@ -469,13 +469,14 @@ def _decode_key(n_seqs: int, n_heads: int, n_kv_heads: int, head_dim: int, max_l
 def decode_plan(n_seqs: int, n_heads: int, n_kv_heads: int, head_dim: int, max_len: int, mean_len: int = 0):
     """How a decode launch is cut: (column tiles per wave, keys per workgroup, waves per workgroup); a size that
     covers the context means one workgroup per sequence and head group, which writes the result itself.  The
-    waves of a workgroup take its keys block by block in turn and merge in LDS.
+    waves of a workgroup take its keys block by block in turn and merge in LDS; ``SHARED_KEYS`` in their place
+    means a wave per tile of heads, all on the same keys (``_shared_keys_rule``).
 
     The batch counts by its next power of two, the longest context by its next multiple of 1,024 and the
     mean context (``mean_len``; 0: as the longest) by its next multiple of 512, so that a captured step,
     which is sized for a padded batch and such bounds, is cut exactly as the same step run directly.
     A cut that was fixed for these counts (``set_decode_plan``; ``CausalLM.tune`` times whole steps with the cuts
-    of ``decode_plan_candidates``) goes before the rule, which has one wave per workgroup."""
+    of ``decode_plan_candidates``) goes before the rule, which has one wave per workgroup or shared keys."""
     key = _decode_key(n_seqs, n_heads, n_kv_heads, head_dim, max_len, mean_len)
     kept = _decode_plans.get(key)
     if kept is not None:
@@ -515,9 +516,9 @@ def take_decode_keys() -> list:
 
 
 def decode_plan_candidates(key) -> list:
-    """Cuts of the decode launch that ``key`` counts, the rule's first: its neighbours with one wave per
-    workgroup, and workgroups of four and eight waves over the whole context and over ranges of 512 and 1,024
-    keys.  A workgroup of several waves needs no second launch when it walks the whole context, but all its keys
+    """Cuts of the decode launch that ``key`` counts, the rule's first: the one-wave rule's neighbours,
+    workgroups of four and eight waves over the whole context and over ranges of 512 and 1,024 keys, and, where
+    they are built, workgroups that share their keys over ranges of 256 to 1,024 keys and the whole context.  A workgroup of several waves needs no second launch when it walks the whole context, but all its keys
     pass through one compute unit; which wins depends on how many sequences and KV heads there are to fill the
     chip.  Timed alone after a flush of the caches, these cuts rank differently than inside a step (the rule's
     cut at 64 sequences, 8 KV heads of 64 and 1,100 keys: 42 us alone, 31 us in a step, where a cut with four
