@@ -821,6 +821,18 @@ def test_attn_mfma_decode_split(nh, nkv, d, split):
     _attn_case(ops, _mfma(ops, split), torch.bfloat16, nh, nkv, d, starts=[0, 63, 64, 700, 255, 256, 1], news=[1] * 7)
 
 
+@pytest.mark.parametrize("nh,nkv,d", [(3, 3, 16), (6, 2, 32), (5, 5, 48), (7, 1, 64), (8, 2, 80), (2, 2, 112), (4, 2, 128),
+                                      (2, 1, 256)])
+def test_attn_mfma_many_ranges(nh, nkv, d):
+    """One token per sequence over contexts of up to 4,500 keys cut into ranges of 64: up to 71 partial results a
+    row, which four waves merge (groups of 4 to 64 lanes per result, some lanes idle where the head size is no
+    power of two), ranges past a shorter sequence's end, and a far key in a range of its own."""
+    ops = _ops()
+    starts = [4499, 130, 2100, 63, 1025]
+    _attn_case(ops, _mfma(ops, 64), torch.bfloat16, nh, nkv, d, starts=starts, news=[1] * 5, boost=[70, None, 2000, 5, None])
+    _attn_case(ops, _mfma(ops, 128), torch.bfloat16, nh, nkv, d, starts=starts, news=[1] * 5, boost=[4490, 129, None, None, 1])
+
+
 @pytest.mark.parametrize("nh,nkv,d,tiles", [(71, 1, 64, 1), (71, 1, 64, 2), (71, 1, 64, 3), (71, 1, 64, 5), (40, 1, 32, 3),
                                             (128, 2, 128, 4), (128, 2, 128, 3), (66, 2, 16, 2), (17, 1, 256, 1)])
 def test_attn_mfma_decode_tiles(nh, nkv, d, tiles):
