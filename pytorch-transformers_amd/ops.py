@@ -502,6 +502,8 @@ def _shared_keys_rule(n: int, n_heads: int, n_kv_heads: int, head_dim: int, boun
     if keys < 20_000:
         return None
     size = 256 if keys <= 100_000 else 512 if keys <= 300_000 else 1024
+    while size < bound and ((bound + size - 1) // size > 1024 or n * ((bound + size - 1) // size) > 65535):
+        size *= 2  # the launch's limits: ranges of a sequence, and sequences x ranges
     return (1, min(size, bound), SHARED_KEYS)
 
 
@@ -543,7 +545,8 @@ def decode_plan_candidates(key) -> list:
     if attn_decode_shared_ok(d, nh // nkv):
         for size in (256, 512, 1024, bound):
             cut = (1, min(size, bound), SHARED_KEYS)
-            if cut not in cuts and n * ((bound + cut[1] - 1) // cut[1]) <= 65535:
+            splits = (bound + cut[1] - 1) // cut[1]
+            if cut not in cuts and splits <= 1024 and n * splits <= 65535:
                 cuts.append(cut)
     return cuts
 

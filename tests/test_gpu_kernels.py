@@ -929,7 +929,7 @@ def test_decode_plan():
     for nh, nkv, d in ((71, 1, 64), (32, 8, 128), (128, 8, 64), (6, 2, 32), (2, 1, 256)):
         groups = (nh // nkv + 15) // 16
         for n in (1, 3, 8, 33, 64, 128, 300, 512):
-            for length in (1, 100, 1024, 1025, 2049, 8192, 32768, 65536, 100000):
+            for length in (1, 100, 1024, 1025, 2049, 8192, 32768, 65536, 100000, 300000):
                 tiles, size, waves = ops.decode_plan(n, nh, nkv, d, length)
                 # the rule: one wave a workgroup, or, with many heads on a KV head and keys enough, shared keys
                 assert 1 <= tiles <= groups and size % 64 == 0 and size >= 128
