@@ -3,16 +3,30 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 A step is one decode step of the batch (model step from the cache plus the greedy choice of the
-next token, fed back).  The default run: batch 8, prompts of 1,024 synthetic token ids, decoding
-towards a context of 2,048.  One JSON line is printed: decode tokens a second as ``value``, the
-prefill of 2,048 tokens under ``prefill``, the decode step's HBM roofline under ``roofline``,
-decode at batch 1 and 64 under ``points``, and under ``kernels`` the launches of a decode step at batch
-8 and 64 and of the prefill, each with its time (events around every launch of a step that is launched
-directly), the bytes it has to read or its arithmetic, and the fraction of the published peak.
+next token, fed back).  The default run: batch 8, prompts of 1,024 synthetic token ids, the timed steps
+right behind the prompt.  One JSON line is printed: decode tokens a second as ``value`` (all timed steps
+over their time; ``ms_per_step_median`` is the median step by events between the steps), the
+prefill of 2,048 tokens under ``prefill``, the decode step's HBM roofline under ``roofline``, and under
+``points`` (flat):
+
+* ``decode_b1`` / ``decode_b8`` / ``decode_b64``: tokens a second over the range of contexts that the
+  configuration names (1,024 -> 2,048), as the mean step time of runs at three contexts (1,030, 1,536, 2,040;
+  ``decode_b64_ctx1536`` and so on are the three), each with ``..._frac``, the fraction of the HBM roofline;
+* ``decode_b8_untuned``: the same step with the built-in choices between kernels, before ``model.tune()`` has
+  timed any (what a process runs that neither tunes nor loads a tuning table);
+* ``falcon11b_...`` / ``falcon40b_...``: decode at batch 8 and 64 and one batch of whole requests of unequal
+  lengths through ``generate()`` at the layer sizes of Falcon2-11B and Falcon-40B, each measured by a child
+  process with a time limit, so that a failure there costs those figures and nothing else.
+
+Under ``kernels``: the launches of a decode step at batch 8 and 64 and of the prefill, each with its time (events
+around every launch of a step that is launched directly), the bytes it has to read or its arithmetic, and the
+fraction of the published peak.
 """
 import argparse
 import json
 import os
+import statistics
+import subprocess
 import sys
 import time
 
@@ -71,17 +85,28 @@ def prefill_flops(cfg, T):
     return linear + attn + head
 
 
-def run_decode(model, sampler_cls, gen_cfg, batch, prompt_len, steps, warmup, seed=0):
-    """Prefill ``batch`` prompts, then time ``steps`` decode steps; returns (seconds, mean context)."""
+def run_decode(model, sampler_cls, gen_cfg, batch, prompt_len, steps, warmup, seed=0, start_ctx=None, per_step=False):
+    """Prefill ``batch`` prompts of ``prompt_len`` tokens, then time ``steps`` decode steps; returns (seconds, mean
+    context of the timed steps, median milliseconds of a step or None).  With ``start_ctx`` nothing is prefilled:
+    the sequences are set to that length (pages reserved, lengths committed; the keys and values there are
+    zeros) and decoding goes on from there, which puts the timed steps at any context at no cost.  ``per_step``:
+    an event is recorded behind every step, for the median."""
     import torch
 
     g = torch.Generator().manual_seed(seed)
-    prompts = torch.randint(0, model.vocab_size, (batch, prompt_len), generator=g).tolist()
-    total = prompt_len + warmup + steps + 1
-    cache = model.new_cache(batch * ((total + 63) // 64 * 64), max_slots=batch)
+    page = model.page_size
+    first = prompt_len if start_ctx is None else start_ctx
+    total = first + warmup + steps + 1
+    cache = model.new_cache(batch * ((total + page - 1) // page * page), max_slots=batch)
     sampler = sampler_cls(gen_cfg, model.vocab_size, model.device)
     slots = [cache.alloc() for _ in range(batch)]
-    logits = model.step(cache, slots, prompts, "last")
+    if start_ctx is None:
+        prompts = torch.randint(0, model.vocab_size, (batch, prompt_len), generator=g).tolist()
+        logits = model.step(cache, slots, prompts, "last")
+    else:
+        cache.reserve(slots, [start_ctx - 1] * batch)
+        cache.commit(slots, [start_ctx - 1] * batch)
+        logits = model.step(cache, slots, torch.randint(0, model.vocab_size, (batch, 1), generator=g).tolist(), "last")
     rng = list(range(batch))
     pending, _ = sampler.sample(logits, rng_seq=rng, rng_step=[0] * batch, need_scores=False, ahead=True)
 
@@ -94,18 +119,48 @@ def run_decode(model, sampler_cls, gen_cfg, batch, prompt_len, steps, warmup, se
 
     for k in range(warmup):
         one(k)
+    marks = []
+    if per_step:
+        marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
+    if per_step:
+        marks[0].record()
     for k in range(steps):
         one(warmup + k)
+        if per_step:
+            marks[k + 1].record()
     pending.tolist()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
-    mean_ctx = prompt_len + warmup + (steps + 1) / 2.0
+    median = statistics.median(marks[k].elapsed_time(marks[k + 1]) for k in range(steps)) if per_step else None
+    mean_ctx = first + warmup + (steps + 1) / 2.0
     for s in slots:
         cache.free(s)
     del cache
-    return dt, mean_ctx
+    return dt, mean_ctx, median
+
+
+RANGE_CONTEXTS = (1030, 1536, 2040)  # the start, the middle and the end of decoding from 1,024 towards 2,048 tokens
+
+
+def decode_over_range(model, sampler_cls, gen_cfg, cfg, elem, batch, steps=16, warmup=4, contexts=RANGE_CONTEXTS):
+    """Decode steps of ``batch`` sequences timed around each of ``contexts``; returns flat figures: tokens a second
+    and fraction of the HBM roofline at each context, and over the range (the mean of the step times)."""
+    out, ms_all, frac_all = {}, [], []
+    for c in contexts:
+        dt, mean_ctx, _ = run_decode(model, sampler_cls, gen_cfg, batch, 0, steps, warmup, seed=c,
+                                     start_ctx=max(1, c - warmup - steps // 2))
+        ms = dt / steps * 1e3
+        gbs = (weight_bytes(cfg, elem) + batch * mean_ctx * kv_bytes_per_token(cfg, elem)) / (ms * 1e-3) / 1e9
+        out[f"decode_b{batch}_ctx{c}"] = round(batch / ms * 1e3, 2)
+        out[f"decode_b{batch}_ctx{c}_frac"] = round(gbs / HBM_PEAK_GBS, 4)
+        ms_all.append(ms)
+        frac_all.append(gbs / HBM_PEAK_GBS)
+    mean_ms = sum(ms_all) / len(ms_all)
+    out[f"decode_b{batch}"] = round(batch / mean_ms * 1e3, 2)
+    out[f"decode_b{batch}_frac"] = round(sum(f * m for f, m in zip(frac_all, ms_all)) / sum(ms_all), 4)
+    return out
 
 
 def run_prefill(model, T, reps=3, seed=1):
@@ -227,6 +282,52 @@ def run_mixed(model, batch, lo, hi, new, seed=2):
     return dt, sum(lens)
 
 
+def mixed_record(model, ops, cfg, sizes, dtype, elem):
+    """One batch of whole requests of unequal lengths through ``generate()`` (prefill included), with the floor of
+    its arithmetic and bytes; the choices that are timed are timed first, for the shapes of this run."""
+    batch, lo, hi, new = MIXED[sizes]
+    with ops.live_tuning():  # the choices that are timed, for the shapes of this run; nothing of it is timed below
+        run_mixed(model, batch, lo, hi, 2)
+    ops.release_flush()
+    # ... and the decode attention's cut at the (longest, mean) contexts that the run passes through
+    lens = run_mixed.lens
+    model.tune(prompt_lens=(), batches=(batch,),
+               contexts=sorted({(max(lens) + k, sum(lens) // len(lens) + k) for k in range(1, new + 1, 64)}))
+    dt, prompt_tokens = run_mixed(model, batch, lo, hi, new)
+    # what the request has to do at the least: the prompts' arithmetic, and for every decode step all weights once
+    # and the live sequences' keys and values (a sequence of n prompt tokens is n + k long at step k)
+    flops = sum(prefill_flops(cfg, n) for n in run_mixed.lens)
+    kv = kv_bytes_per_token(cfg, elem)
+    decode_bytes = new * weight_bytes(cfg, elem) + sum(kv * (n * new + new * (new + 1) / 2) for n in run_mixed.lens)
+    floor = flops / (PEAK_TFLOPS[dtype] * 1e12) + decode_bytes / (HBM_PEAK_GBS * 1e9)
+    return {"metric": f"falcon{sizes}_mixed_generated_tokens_per_second",
+            "value": round(batch * new / dt, 1), "unit": "tokens/s", "seconds": round(dt, 3),
+            "batch": batch, "prompt_tokens": prompt_tokens, "new_tokens_each": new,
+            "prompt_lengths": f"U[{lo},{hi}]", "layers": cfg.num_hidden_layers, "dtype": dtype,
+            "roofline": {"bound": "prefill arithmetic + decode hbm", "prefill_tflop": round(flops / 1e12, 1),
+                         "decode_gb": round(decode_bytes / 1e9, 1), "floor_s": round(floor, 3),
+                         "frac": round(floor / dt, 4)},
+            "note": "whole requests, prefill included; greedy, no stop token"}
+
+
+EXTRA_SIZES = (("11b", 170), ("40b", 270))  # other layer sizes measured by a child process, and its time limit in seconds
+
+
+def extra_points(sizes, limit, dtype):
+    """Flat figures of ``--extra-record`` at ``sizes`` from a child process (the 7B model of this process keeps its
+    memory; both fit).  A child that fails or overruns its limit leaves an ``..._error`` entry and nothing else."""
+    tag = f"falcon{sizes}"
+    cmd = [sys.executable, os.path.abspath(__file__), "--sizes", sizes, "--dtype", dtype, "--extra-record"]
+    try:
+        done = subprocess.run(cmd, capture_output=True, text=True, timeout=limit, cwd=ROOT)
+    except subprocess.TimeoutExpired:
+        return {f"{tag}_error": f"not done within {limit} s"}
+    lines = [ln for ln in done.stdout.splitlines() if ln.startswith("{")]
+    if done.returncode != 0 or not lines:
+        return {f"{tag}_error": f"exit code {done.returncode}: {done.stderr.strip()[-200:]}"}
+    return {f"{tag}_{k}": v for k, v in json.loads(lines[-1]).items()}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -239,9 +340,13 @@ def main():
                     help="layer sizes: Falcon-7B (the default run), Falcon2-11B or Falcon-40B")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / batch 64 / prefill measurements")
+    ap.add_argument("--no-extra", action="store_true", help="skip the figures at Falcon2-11B and Falcon-40B layer sizes")
     ap.add_argument("--mixed", action="store_true",
                     help="one batch of unequal prompts through generate(): 11b 16 x U[128,4096] + 256 new, "
                          "40b 32 x U[64,1536] + 512 new; prints its own record")
+    ap.add_argument("--extra-record", action="store_true",
+                    help="decode at batch 8 and 64 over the range of contexts and the --mixed request, as one flat record "
+                         "(what the default run asks a child process for at the other layer sizes)")
     ap.add_argument("--only-prefill", action="store_true",
                     help="run the prefill alone and print its record (for profiling)")
     ap.add_argument("--prefill-tokens", type=int, default=2048,
@@ -264,29 +369,19 @@ def main():
     model = AutoModelForCausalLM.from_config(cfg, seed=0, dtype=dtype, device="cuda:0")
     gen_cfg = GenerationConfig(do_sample=False, eos_token_id=None)
     if args.mixed:
-        batch, lo, hi, new = MIXED[args.sizes]
-        with ops.live_tuning():  # the choices that are timed, for the shapes of this run; nothing of it is timed below
-            run_mixed(model, batch, lo, hi, 2)
-        ops.release_flush()
-        # ... and the decode attention's cut at the (longest, mean) contexts that the run passes through
-        lens = run_mixed.lens
-        model.tune(prompt_lens=(), batches=(batch,),
-                   contexts=sorted({(max(lens) + k, sum(lens) // len(lens) + k) for k in range(1, new + 1, 64)}))
-        dt, prompt_tokens = run_mixed(model, batch, lo, hi, new)
-        # what the request has to do at the least: the prompts' arithmetic, and for every decode step all weights once
-        # and the live sequences' keys and values (a sequence of n prompt tokens is n + k long at step k)
-        flops = sum(prefill_flops(cfg, n) for n in run_mixed.lens)
-        kv = kv_bytes_per_token(cfg, elem)
-        decode_bytes = new * weight_bytes(cfg, elem) + sum(kv * (n * new + new * (new + 1) / 2) for n in run_mixed.lens)
-        floor = flops / (PEAK_TFLOPS[args.dtype] * 1e12) + decode_bytes / (HBM_PEAK_GBS * 1e9)
-        print(json.dumps({"metric": f"falcon{args.sizes}_mixed_generated_tokens_per_second",
-                          "value": round(batch * new / dt, 1), "unit": "tokens/s", "seconds": round(dt, 3),
-                          "batch": batch, "prompt_tokens": prompt_tokens, "new_tokens_each": new,
-                          "prompt_lengths": f"U[{lo},{hi}]", "layers": args.layers, "dtype": args.dtype,
-                          "roofline": {"bound": "prefill arithmetic + decode hbm", "prefill_tflop": round(flops / 1e12, 1),
-                                       "decode_gb": round(decode_bytes / 1e9, 1), "floor_s": round(floor, 3),
-                                       "frac": round(floor / dt, 4)},
-                          "note": "whole requests, prefill included; greedy, no stop token"}))
+        print(json.dumps(mixed_record(model, ops, cfg, args.sizes, args.dtype, elem)))
+        return 0
+    if args.extra_record:
+        ends = (RANGE_CONTEXTS[0], RANGE_CONTEXTS[-1])
+        model.tune(prompt_lens=(), batches=(8, 64), contexts=RANGE_CONTEXTS)
+        rec = {}
+        for b in (8, 64):
+            rec.update(decode_over_range(model, Sampler, gen_cfg, cfg, elem, b, steps=12, warmup=3))
+        mixed = mixed_record(model, ops, cfg, args.sizes, args.dtype, elem)
+        rec.update({"mixed": mixed["value"], "mixed_seconds": mixed["seconds"], "mixed_frac": mixed["roofline"]["frac"],
+                    "mixed_batch": mixed["batch"], "mixed_new_tokens_each": mixed["new_tokens_each"],
+                    "mixed_prompt_lengths": mixed["prompt_lengths"], "layers": args.layers})
+        print(json.dumps(rec))
         return 0
     # the choices between kernels that are timed rather than ruled, once, for the shapes measured below; the timed
     # steps themselves time nothing
@@ -298,10 +393,15 @@ def main():
                                       "frac": round(prefill_flops(cfg, T) / pt / (PEAK_TFLOPS[args.dtype] * 1e12), 4)},
                           "layers": args.layers, "dtype": args.dtype}))
         return 0
+    points = {}
+    if not args.no_points:  # before anything is timed: the step as a process runs it that neither tunes nor loads a table
+        d, _, _ = run_decode(model, Sampler, gen_cfg, args.batch, args.prompt_len, 16, 4)
+        points[f"decode_b{args.batch}_untuned"] = round(args.batch * 16 / d, 2)
     model.tune(prompt_lens=(2048,), batches=sorted({args.batch, 1, 64}),
-               contexts=sorted({args.prompt_len + 1, args.prompt_len + args.warmup + args.steps}))
+               contexts=sorted({args.prompt_len + 1, args.prompt_len + args.warmup + args.steps, *RANGE_CONTEXTS}))
 
-    dt, mean_ctx = run_decode(model, Sampler, gen_cfg, args.batch, args.prompt_len, args.steps, args.warmup)
+    dt, mean_ctx, median_ms = run_decode(model, Sampler, gen_cfg, args.batch, args.prompt_len, args.steps, args.warmup,
+                                         per_step=True)
     ms = dt / args.steps * 1e3
     value = args.batch * args.steps / dt
     step_bytes = weight_bytes(cfg, elem) + args.batch * mean_ctx * kv_bytes_per_token(cfg, elem)
@@ -309,13 +409,16 @@ def main():
 
     out = {
         "metric": f"falcon{args.sizes}_decode_tokens_per_second", "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4), "ms_per_step_median": round(median_ms, 4),
+        "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
         "data": "synthetic token ids, random weights N(0, 0.02)",
         "config": {"model": f"falcon-{args.sizes} layer sizes", "layers": args.layers, "layers_of_config": full_layers,
                    "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.kv_heads,
                    "head_dim": cfg.head_dim, "ffn": cfg.ffn_hidden_size, "vocab": cfg.vocab_size,
                    "global_batch": args.batch, "prompt_len": args.prompt_len, "seq_len": 2048,
+                   "timed_ctx_from": args.prompt_len + args.warmup + 1,
+                   "timed_ctx_to": args.prompt_len + args.warmup + args.steps,
                    "decode": "greedy", "parallelism": "single"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
@@ -326,11 +429,8 @@ def main():
         flops = prefill_flops(cfg, T)
         out["prefill"] = {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3),
                           "frac": round(flops / pt / (PEAK_TFLOPS[args.dtype] * 1e12), 4)}
-        points = {}
-        for b in (1, 64):
-            steps_b = max(16, args.steps // 2)
-            d, _ = run_decode(model, Sampler, gen_cfg, b, args.prompt_len, steps_b, 8)
-            points[f"decode_b{b}"] = round(b * steps_b / d, 2)
+        for b in sorted({1, args.batch, 64}):
+            points.update(decode_over_range(model, Sampler, gen_cfg, cfg, elem, b))
         out["points"] = points
         if args.dtype == "bf16":
             out["kernels"] = {
@@ -338,6 +438,9 @@ def main():
                 "decode_b64": decode_kernels(model, ops, Sampler, gen_cfg, cfg, args.dtype, elem, 64, args.prompt_len),
                 "prefill_2048": prefill_kernels(model, ops, cfg, args.dtype, 2048),
             }
+        if args.sizes == "7b" and not args.no_extra:
+            for sizes, limit in EXTRA_SIZES:
+                points.update(extra_points(sizes, limit, args.dtype))
     print(json.dumps(out))
     return 0
 

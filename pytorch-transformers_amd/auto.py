@@ -10,10 +10,12 @@ from __future__ import annotations
 
 class AutoModelForCausalLM:
     @staticmethod
-    def from_pretrained(folder: str, dtype="bfloat16", device="cuda:0", strict: bool = True, torch_dtype=None):
+    def from_pretrained(folder: str, dtype="bfloat16", device="cuda:0", strict: bool = True, torch_dtype=None,
+                        tuning_table=None):
         from .engine.model import CausalLM
 
-        return CausalLM.from_pretrained(folder, dtype=torch_dtype or dtype, device=device, strict=strict)
+        return CausalLM.from_pretrained(folder, dtype=torch_dtype or dtype, device=device, strict=strict,
+                                        tuning_table=tuning_table)
 
     @staticmethod
     def from_config(config, seed: int = 0, dtype="bfloat16", device="cuda:0", torch_dtype=None, **kwargs):

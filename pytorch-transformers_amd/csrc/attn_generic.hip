@@ -77,6 +77,17 @@ __global__ void attn_generic_kernel(T* __restrict__ out, const T* __restrict__ q
     }
 }
 
+// Whether the attention kernels and the kernel that rotates queries and keys take these sizes (0), or why not
+// (pta_last_error): for a caller that wants to refuse a model before it reads a weight.  ``rotated``: queries and
+// keys are rotated by position (pairs of elements: an even head size).
+extern "C" int pta_attention_sizes_ok(int nh, int nkv, int d, int rotated) {
+    PTA_REQUIRE(nh > 0 && nkv > 0 && nh % nkv == 0, "attention: %d heads are no multiple of %d kv heads", nh, nkv);
+    PTA_REQUIRE(d > 0 && d <= 256, "attention: head size %d is outside 1..256, which is what the kernels take", d);
+    PTA_REQUIRE(nh <= 65535, "attention: at most 65535 heads, got %d", nh);
+    PTA_REQUIRE(!rotated || d % 2 == 0, "attention: rotation pairs elements and needs an even head size, got %d", d);
+    return 0;
+}
+
 extern "C" int pta_attn_generic(void* out, const void* q, const void* k_pool, const void* v_pool,
                                 const int* block_table, int bt_stride, const int* token_seq, const int* token_pos,
                                 const float* slopes, int alibi_exact, int M, int nh, int nkv, int d, float scale, int window, int dtype,

@@ -743,7 +743,7 @@ extern "C" int pta_attn_mfma(void* out, const void* q, const void* k_pool, const
                              int bt_stride, const int* cu_tokens, const int* seq_start, const float* slopes, int alibi_exact,
                              int n_seqs, int max_new, int M, int nh, int nkv, int d, float scale, int split_size, int n_splits,
                              float* po, float* pm, float* pl, int window, int decode_tiles, int decode_waves,
-                             void* stream) {
+                             int prompt_wide, void* stream) {
     PTA_REQUIRE(n_seqs > 0 && max_new > 0 && M > 0 && nh > 0 && nkv > 0, "attn_mfma: sizes must be positive");
     PTA_REQUIRE(nh % nkv == 0, "attn_mfma: heads (%d) must be a multiple of kv heads (%d)", nh, nkv);
     PTA_REQUIRE(pta_attn_mfma_supported(d), "attn_mfma: head size %d is not built (16..128 in steps of 16, or 256)", d);
@@ -782,14 +782,12 @@ extern "C" int pta_attn_mfma(void* out, const void* q, const void* k_pool, const
     // 1 KV head of 64: 2,048 tokens 67 -> 72 us a layer, 4,096 the same, 8,192 712 -> 693, 16,384 2,542 -> 2,433;
     // 128 on 8 of 64: 2,048 tokens 101 -> 94, 8,192 1,213 -> 1,151).
     static const int pair_env = getenv("PTA_ATTN_PAIR") ? atoi(getenv("PTA_ATTN_PAIR")) : -1;
-    const char* wide_set = getenv("PTA_ATTN_WIDE");  // looked up at every launch: tests switch it
-    const int wide_env = wide_set ? atoi(wide_set) : -1;
     int paired = 0;
     bool wide = false;
     if (!narrow && !shared) {
         const double units = pta_compute_units();
         const double wide_wgs = std::ceil((double)M * (nh / nkv) / prompt_columns(d / 16, true)) * nkv;
-        wide = d <= 64 && (wide_env >= 0 ? wide_env != 0 : wide_wgs >= 4.0 * units);
+        wide = d <= 64 && (prompt_wide >= 0 ? prompt_wide != 0 : wide_wgs >= 4.0 * units);
         const double wgs = std::ceil((double)M * (nh / nkv) / prompt_columns(d / 16, wide)) * nkv;
         paired = pair_env >= 0 ? pair_env : 2.0 * std::ceil(wgs / 2.0 / units) <= 1.01 * std::max(wgs / units, 2.0);
     }

@@ -336,7 +336,7 @@ static int clamp_parts(int P, int K) { return max(1, min(min(P, 16), max(1, K / 
 // with many row tiles the ranges may be longer: fewer partial sums for the same number of workgroups
 static int range_for(int groups) { return SK_RANGE * max(1, groups / 64); }
 
-// Among the counts near that rule's, the one with the least (rounds of workgroups on the chip's 256 compute units)
+// Among the counts near that rule's, the one with the least (rounds of workgroups on the chip's compute units)
 // x (a workgroup's fixed cost + the length of its range).  Measured at 32 to 128 rows: a launch just over a whole
 // number of rounds pays for the last one in full (N = 9,216 and K = 8,192, 144 row tiles: 4 ranges, 2.25 rounds, 81
 // us; 3 ranges, 1.69 rounds, 65 us; N = 4,672 and K = 4,544, 73 row tiles: 8 ranges 31.6 us, 7 ranges 27.6 us), and the fixed
@@ -345,7 +345,8 @@ static int range_for(int groups) { return SK_RANGE * max(1, groups / 64); }
 static int pick_parts(int N, int K, int rt) {
     const int groups = (N + 64 * rt - 1) / (64 * rt), range = range_for(groups);
     const int p0 = clamp_parts(max((splitk_target() + groups - 1) / groups, (K + range / 2) / range), K);
-    auto cost = [&](int p) { return (((long)groups * p + 255) / 256) * (SK_WG_FIXED + K / p); };
+    const long units = max(1, pta_compute_units());
+    auto cost = [&](int p) { return (((long)groups * p + units - 1) / units) * (SK_WG_FIXED + K / p); };
     static const bool balance = !getenv("PTA_SPLITK_BALANCE") || atoi(getenv("PTA_SPLITK_BALANCE")) != 0;
     int best = p0;
     for (int p = max(1, p0 - 2); balance && p <= p0 + 2; ++p) {

@@ -14,7 +14,7 @@
 
 #include <stdint.h>
 
-#define PTA_ABI_VERSION 7
+#define PTA_ABI_VERSION 8
 
 #ifdef __cplusplus
 extern "C" {
@@ -55,6 +55,10 @@ int pta_qkv_rope_cache(void* q_out, const void* fused, int fused_ld, const float
                        void* k_pool, void* v_pool, int M, int nh, int nkv, int d, int layout, int write_cache,
                        int dtype, void* stream);
 
+// 0 if the attention kernels (and, with ``rotated``, the kernel that rotates queries and keys) take these sizes, else
+// nonzero with the reason in pta_last_error; launches nothing
+int pta_attention_sizes_ok(int nh, int nkv, int d, int rotated);
+
 // causal attention of M tokens over their sequences' cache, 32-bit arithmetic
 // window: 0, or the number of last positions a token sees (itself included)
 // slopes (null: none): a bias slope[head] * key position / sqrt(d) on the scores; with alibi_exact = 0 the position
@@ -81,10 +85,12 @@ int pta_attn_decode_waves_ok(int d, int tiles, int waves);
 // keys through LDS (decode_tiles does not apply); pta_attn_decode_shared_ok says whether that is built for this head
 // size and this many heads on a KV head.
 int pta_attn_decode_shared_ok(int d, int heads_per_kv_head);
+// prompt_wide (max_new > 1, head sizes up to 64): 1 workgroups of eight waves, 0 of four, -1 eight where the launch
+// still has four workgroups and more for every compute unit.
 int pta_attn_mfma(void* out, const void* q, const void* k_pool, const void* v_pool, const int* block_table,
                   int bt_stride, const int* cu_tokens, const int* seq_start, const float* slopes, int alibi_exact,
                   int n_seqs, int max_new, int M, int nh, int nkv, int d, float scale, int split_size, int n_splits, float* po,
-                  float* pm, float* pl, int window, int decode_tiles, int decode_waves, void* stream);
+                  float* pm, float* pl, int window, int decode_tiles, int decode_waves, int prompt_wide, void* stream);
 
 // C = act(A . W^T + bias) + add1 + add2, all 32-bit, fixed summation order
 int pta_gemm_f32(float* C, const float* A, const float* W, const float* bias, const float* add1, const float* add2,
@@ -191,12 +197,17 @@ long pta_gemm_splitk_static_floats(void);
 // processors in the reference's order, then argmax (do_sample 0) or a draw; `work` [R, V] is scratch and,
 // with want_scores, receives the processed scores (without, its contents are unspecified);
 // typical_p 1, epsilon_cutoff 0 and eta_cutoff 0 switch those off; hist/hist_off (tokens seen, per row),
-// ban/ban_off (tokens a row may not take, per row), eos/suppress, uniforms may be null
+// ban/ban_off (tokens a row may not take, per row), eos/suppress, uniforms may be null.  bias_tok/bias_val/bias_off
+// (per row: tokens, each once, whose score gets a value added before anything else; null: none), forced/n_forced
+// (in this step every score goes but those of these tokens, which become 0; 0: nothing is forced), decay_on/decay_m
+// (the EOS tokens' scores gain |score| * decay_m after the removal of invalid values)
 int pta_sample(int* out_tok, float* work, const float* logits, int R, int V, int do_sample, float temperature,
                int top_k, float top_p, float min_p, float typical_p, float epsilon_cutoff, float eta_cutoff,
                float penalty, const int* hist, const int* hist_off, const int* ban, const int* ban_off,
                const int* eos, int n_eos, const int* suppress, int remove_invalid, int renorm, uint64_t seed,
-               const int* rng_seq, const int* rng_step, const float* uniforms, int want_scores, void* stream);
+               const int* rng_seq, const int* rng_step, const float* uniforms, int want_scores, const int* bias_tok,
+               const float* bias_val, const int* bias_off, const int* forced, int n_forced, int decay_on, float decay_m,
+               void* stream);
 
 // out_tok[r] = index of the largest of logits[r, :], lowest index among equals (greedy choice, no processors)
 int pta_argmax(int* out_tok, const float* logits, int R, int V, void* stream);

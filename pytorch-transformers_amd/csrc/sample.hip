@@ -1,10 +1,12 @@
 // Next-token choice on the GPU: the reference's logits processors in their order, then argmax or
 // a draw from the softmax, one workgroup per row of 32-bit logits.
 //
-// Order (src/transformers/generation/utils.py:926-1097): repetition penalty, EOS suppression
-// (minimum length), removal of invalid values, then for sampling temperature, top-k, top-p, min-p;
+// Order (src/transformers/generation/utils.py:898-1097): additive biases on tokens, repetition penalty, banned
+// tokens, EOS suppression (minimum length), a forced last token, removal of invalid values, the growing bonus on
+// EOS, then for sampling temperature, top-k, top-p, min-p;
 // then softmax and a draw (:3274-3279) or argmax.  Formulas: src/transformers/generation/logits_process.py
-// :337-343 (penalty), :144-151 (EOS), :1618-1626 (invalid), :286-289 (temperature), :505-518 (top-k),
+// :1112-1140 (biases), :337-343 (penalty), :144-151 (EOS), :1590-1596 (forced token), :1618-1626 (invalid),
+// :1716-1727 (bonus on EOS), :286-289 (temperature), :505-518 (top-k),
 // :452-465 (top-p), :578-595 (min-p), :1762-1764 (renormalise).
 //
 // Thresholds are found without sorting: the k-th largest score by a radix search on counts, the
@@ -261,9 +263,11 @@ __device__ __forceinline__ float key_value(uint32_t k) {
     return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
 }
 
-// The processed score of a token before the thresholds: repetition penalty (tokens seen before are marked in
-// a bitmap in LDS, so vocabularies up to 65,536), the row's banned tokens (a second bitmap), EOS suppression,
-// invalid values, temperature, in this order.
+// The processed score of a token before the thresholds: the row's additive biases (a short list of (token,
+// value), searched for every score), repetition penalty (tokens seen before are marked in a bitmap in LDS, so
+// vocabularies up to 65,536), the row's banned tokens (a second bitmap), EOS suppression, a forced token (every
+// other score gone, its own 0; a banned token stays gone), invalid values, the bonus |score| * decay_m on the EOS
+// tokens, temperature, in this order.
 struct Processed {
     const float* l;
     const uint32_t* seen;  // null: no penalty
@@ -272,17 +276,36 @@ struct Processed {
     int n_eos;  // 0: no suppression
     float penalty, temperature;
     int remove_invalid;
+    const int* bias_tok;  // this row's biased tokens, each once, and their values
+    const float* bias_val;
+    int n_bias;
+    const int* forced;
+    int n_forced;  // 0: nothing is forced in this step
+    int n_eos_all;  // the EOS tokens, whether suppressed or not
+    int decay_on;
+    float decay_m;
     __device__ __forceinline__ float operator()(int i) const { return of(i, l[i]); }
     __device__ __forceinline__ float of(int i, float x) const {
+        for (int t = 0; t < n_bias; ++t)
+            if (bias_tok[t] == i) x += bias_val[t];
         if (seen && ((seen[i >> 5] >> (i & 31)) & 1u)) x = x < 0.f ? x * penalty : x / penalty;
-        if (banned && ((banned[i >> 5] >> (i & 31)) & 1u)) x = -INFINITY;
+        const bool gone = banned && ((banned[i >> 5] >> (i & 31)) & 1u);
+        if (gone) x = -INFINITY;
         for (int e = 0; e < n_eos; ++e)
             if (eos[e] == i) x = -INFINITY;
+        if (n_forced) {
+            bool is = false;
+            for (int e = 0; e < n_forced; ++e) is = is || forced[e] == i;
+            x = is && !gone ? 0.f : -INFINITY;
+        }
         if (remove_invalid) {
             if (x != x) x = 0.f;
             else if (x == INFINITY) x = FLT_MAX;
             else if (x == -INFINITY) x = -FLT_MAX;
         }
+        if (decay_on)
+            for (int e = 0; e < n_eos_all; ++e)
+                if (eos[e] == i) { x += fabsf(x) * decay_m; break; }
         if (temperature != 1.0f) x = x / temperature;
         return x;
     }
@@ -469,7 +492,9 @@ __global__ __launch_bounds__(S_THREADS) void sample_kernel(
     float penalty, const int* __restrict__ hist, const int* __restrict__ hist_off, const int* __restrict__ ban,
     const int* __restrict__ ban_off, const int* __restrict__ eos, int n_eos, const int* __restrict__ suppress,
     int remove_invalid, int renorm, uint64_t seed, const int* __restrict__ rng_seq,
-    const int* __restrict__ rng_step, const float* __restrict__ uniforms, int want_scores) {
+    const int* __restrict__ rng_step, const float* __restrict__ uniforms, int want_scores,
+    const int* __restrict__ bias_tok, const float* __restrict__ bias_val, const int* __restrict__ bias_off,
+    const int* __restrict__ forced, int n_forced, int decay_on, float decay_m) {
     __shared__ SampleShared sh;
     float* const red = sh.red;
     int* const red_i = sh.red_i;
@@ -486,6 +511,7 @@ __global__ __launch_bounds__(S_THREADS) void sample_kernel(
     const float* l = logits + (long)row * V;
 
     const bool suppress_eos = suppress && suppress[row];
+    const int bias_lo = bias_off ? bias_off[row] : 0, n_bias = bias_off ? bias_off[row + 1] - bias_lo : 0;
     ArgBest first_best = {-INFINITY, 0x7fffffff};
     unsigned long long first_finite = 0ull;
     float first_max = -INFINITY;  // the largest of the scores this thread saw in the first pass
@@ -493,7 +519,8 @@ __global__ __launch_bounds__(S_THREADS) void sample_kernel(
     if (V <= 65536) {
         const Processed score{l, mark_seen(sh, row, V, penalty, hist, hist_off), mark_banned(sh, row, V, ban, ban_off), eos,
                               suppress_eos ? n_eos : 0, penalty,
-                              do_sample ? temperature : 1.0f, remove_invalid};
+                              do_sample ? temperature : 1.0f, remove_invalid, bias_tok + bias_lo, bias_val + bias_lo, n_bias,
+                              forced, n_forced, n_eos, decay_on, decay_m};
         const bool later_warpers = typical_p < 1.0f || epsilon_cutoff > 0.0f || eta_cutoff > 0.0f;  // the long way has them
         if (do_sample && top_k > 0 && top_k < V && top_k <= n_holding && top_k <= S_SHORT && !later_warpers) {
             const float u = uniforms ? uniforms[row] : uniform_of(seed, (uint32_t)rng_seq[row], (uint32_t)rng_step[row]);
@@ -517,11 +544,24 @@ __global__ __launch_bounds__(S_THREADS) void sample_kernel(
     } else {
         for (int i = tid; i < V; i += S_THREADS) w[i] = l[i];
         __syncthreads();
+        auto biased = [&](int tok) {  // the score with the row's bias for this token (a token is listed once)
+            float v = l[tok];
+            for (int t = 0; t < n_bias; ++t)
+                if (bias_tok[bias_lo + t] == tok) v += bias_val[bias_lo + t];
+            return v;
+        };
+        if (n_bias) {
+            for (int t = tid; t < n_bias; t += S_THREADS) {
+                const int tok = bias_tok[bias_lo + t];
+                if (tok >= 0 && tok < V) w[tok] = biased(tok);
+            }
+            __syncthreads();
+        }
         if (hist_off && penalty != 1.0f) {
             for (int t = hist_off[row] + tid; t < hist_off[row + 1]; t += S_THREADS) {
                 const int tok = hist[t];
                 if (tok >= 0 && tok < V) {
-                    const float v = l[tok];
+                    const float v = biased(tok);
                     w[tok] = v < 0.f ? v * penalty : v / penalty;
                 }
             }
@@ -537,6 +577,19 @@ __global__ __launch_bounds__(S_THREADS) void sample_kernel(
                 if (eos[e] >= 0 && eos[e] < V) w[eos[e]] = -INFINITY;
             __syncthreads();
         }
+        if (n_forced) {
+            for (int i = tid; i < V; i += S_THREADS) {
+                bool is = false;
+                for (int e = 0; e < n_forced; ++e) is = is || forced[e] == i;
+                w[i] = is ? 0.f : -INFINITY;
+            }
+            __syncthreads();
+            if (ban_off) {  // a banned token stays gone
+                for (int t = ban_off[row] + tid; t < ban_off[row + 1]; t += S_THREADS)
+                    if (ban[t] >= 0 && ban[t] < V) w[ban[t]] = -INFINITY;
+                __syncthreads();
+            }
+        }
         if (remove_invalid) {
             for (int i = tid; i < V; i += S_THREADS) {
                 float v = w[i];
@@ -545,6 +598,15 @@ __global__ __launch_bounds__(S_THREADS) void sample_kernel(
                 else if (v == -INFINITY) v = -FLT_MAX;
                 w[i] = v;
             }
+            __syncthreads();
+        }
+        if (decay_on) {
+            if (tid == 0)
+                for (int e = 0; e < n_eos; ++e) {
+                    bool again = false;  // an id listed twice counts once
+                    for (int o = 0; o < e; ++o) again = again || eos[o] == eos[e];
+                    if (!again && eos[e] >= 0 && eos[e] < V) w[eos[e]] += fabsf(w[eos[e]]) * decay_m;
+                }
             __syncthreads();
         }
         if (do_sample && temperature != 1.0f) {
@@ -897,7 +959,7 @@ __global__ __launch_bounds__(S_THREADS) void sample_kernel(
             }
         }
     }
-    if (!do_sample && tid == 0) out_tok[row] = chosen;
+    if (!do_sample && tid == 0) out_tok[row] = chosen < V ? chosen : 0;  // every score -inf: token 0, as an argmax gives
     if (renorm) {
         __syncthreads();
         const float lse = best.v + logf(Z);
@@ -911,7 +973,8 @@ extern "C" int pta_sample(int* out_tok, float* work, const float* logits, int R,
                           const int* hist_off, const int* ban, const int* ban_off, const int* eos, int n_eos,
                           const int* suppress, int remove_invalid,
                           int renorm, uint64_t seed, const int* rng_seq, const int* rng_step, const float* uniforms,
-                          int want_scores, void* stream) {
+                          int want_scores, const int* bias_tok, const float* bias_val, const int* bias_off,
+                          const int* forced, int n_forced, int decay_on, float decay_m, void* stream) {
     PTA_REQUIRE(R > 0 && V > 0, "sample: rows=%d vocab=%d must be positive", R, V);
     PTA_REQUIRE(out_tok && work && logits, "sample: null pointer");
     PTA_REQUIRE(!do_sample || temperature > 0.f, "sample: temperature must be > 0, got %g", (double)temperature);
@@ -925,9 +988,13 @@ extern "C" int pta_sample(int* out_tok, float* work, const float* logits, int R,
     PTA_REQUIRE(!do_sample || uniforms || (rng_seq && rng_step), "sample: sampling needs uniforms or rng counters");
     PTA_REQUIRE(n_eos == 0 || eos, "sample: eos ids missing");
     PTA_REQUIRE(!ban_off || ban, "sample: banned ids missing");
+    PTA_REQUIRE(!bias_off || (bias_tok && bias_val), "sample: biased ids or their values missing");
+    PTA_REQUIRE(n_forced == 0 || forced, "sample: forced ids missing");
+    PTA_REQUIRE(!decay_on || n_eos > 0, "sample: a bonus on the EOS tokens needs their ids");
     hipLaunchKernelGGL(sample_kernel, dim3(R), dim3(S_THREADS), 0, (hipStream_t)stream, out_tok, work, logits, V,
                        do_sample, temperature, top_k, top_p, min_p, typical_p, epsilon_cutoff, eta_cutoff, penalty, hist,
-                       hist_off, ban, ban_off, eos, n_eos, suppress, remove_invalid, renorm, seed, rng_seq, rng_step, uniforms, want_scores);
+                       hist_off, ban, ban_off, eos, n_eos, suppress, remove_invalid, renorm, seed, rng_seq, rng_step, uniforms, want_scores,
+                       bias_tok, bias_val, bias_off, forced, n_forced, decay_on, decay_m);
     return pta_check_launch("sample");
 }
 

@@ -34,6 +34,9 @@ class GenerateOutput:
     #: that goes on from there (the reference returns ``past_key_values`` for that, :3314-3322)
     cache: Optional[object] = None
     slots: Optional[List[int]] = None
+    #: with ``keep_slots``: per sequence, how many draws of its random stream are used up (``rng_step_start`` of the
+    #: call that goes on, so that it draws what one call over the whole length would have drawn)
+    rng_steps: Optional[List[int]] = None
 
 
 def _round_up(n: int, m: int) -> int:
@@ -63,7 +66,8 @@ def resolve_lengths(cfg: GenerationConfig, prompt_lens: Sequence[int]):
 def generate(model, prompts: Sequence[Sequence[int]], generation_config: Optional[GenerationConfig] = None, *,
              batch_size: Optional[int] = None, sampler=None, streamer=None, cache=None,
              rng_ids: Optional[Sequence[int]] = None, tokenizer=None, keep_slots: bool = False,
-             slots: Optional[Sequence[int]] = None, **kwargs) -> Union[List[List[int]], GenerateOutput]:
+             slots: Optional[Sequence[int]] = None, rng_step_start: Optional[Sequence[int]] = None,
+             **kwargs) -> Union[List[List[int]], GenerateOutput]:
     """Generate for every prompt (a list of token ids); returns prompt + new tokens per prompt.
 
     ``generation_config`` defaults to the model's; keyword arguments override its fields
@@ -79,7 +83,10 @@ def generate(model, prompts: Sequence[Sequence[int]], generation_config: Optiona
     cache, those ``slots`` and, as prompts, the whole sequences so far: only the tokens a slot does not hold yet
     are run (the reference continues from a returned cache the same way, src/transformers/generation/utils.py
     :349-481, tests/generation/test_utils.py:1775-1855).  Whoever keeps slots frees them (``cache.free``), or
-    hands them to a call without ``keep_slots``, which frees them when it ends.
+    hands them to a call without ``keep_slots``, which frees them when it ends.  A random stream is a sequence of
+    draws numbered from 0; ``rng_step_start`` says, per prompt, at which number this call starts (default 0).  A call
+    that goes on from kept slots passes the earlier result's ``rng_steps`` there and then samples the tokens that
+    one call over the whole length would have sampled.
     """
     cfg = generation_config or getattr(model, "generation_config", None) or GenerationConfig()
     if kwargs:
@@ -114,6 +121,10 @@ def generate(model, prompts: Sequence[Sequence[int]], generation_config: Optiona
         ids = [r * n_ret + j for r in rng_ids for j in range(n_ret)]
     if len(ids) != len(prompts):
         raise ValueError("rng_ids must name one stream per prompt")
+    first_draw = [int(v) for v in rng_step_start] if rng_step_start is not None else [0] * (len(prompts) // n_ret)
+    if len(first_draw) * n_ret != len(prompts) or any(v < 0 for v in first_draw):
+        raise ValueError("rng_step_start must give one number, 0 or more, per prompt")
+    first_draw = [v for v in first_draw for _ in range(n_ret)]
 
     batch_size = batch_size or len(prompts)
     batches = [list(range(b, min(b + batch_size, len(prompts)))) for b in range(0, len(prompts), batch_size)]
@@ -168,17 +179,17 @@ def generate(model, prompts: Sequence[Sequence[int]], generation_config: Optiona
         try:
             if ahead:
                 _decode_ahead(model, cache, sampler, cfg, eos, ids, batch, slot_of, feed, out_tokens, new_budget,
-                              padded_len, done_with)
+                              padded_len, done_with, first_draw)
                 live = []
             while live:
                 logits = model.step(cache, [slot_of[i] for i in live], [feed[i] for i in live], "last")
                 # EOS is masked while the minimum lengths are not reached (logits_process.py:144-151, :214-223)
                 too_short = (padded_len + step_no < (cfg.min_length or 0)) or (step_no < (cfg.min_new_tokens or 0))
                 tokens, scores = sampler.sample(
-                    logits, rng_seq=[ids[i] for i in live], rng_step=[step_no] * len(live),
+                    logits, rng_seq=[ids[i] for i in live], rng_step=[first_draw[i] + step_no for i in live],
                     histories=[prompts[i] + out_tokens[i] for i in live], suppress_eos=[too_short] * len(live),
                     new_counts=[len(out_tokens[i]) for i in live],
-                    need_scores=want_scores)
+                    need_scores=want_scores, **_step_extras(sampler, step_no, new_budget))
                 step_no += 1
                 timed_out = cfg.max_time is not None and (time.time() - t0) > cfg.max_time  # stopping_criteria.py:87-107
                 still = []
@@ -201,23 +212,31 @@ def generate(model, prompts: Sequence[Sequence[int]], generation_config: Optiona
         except BaseException:
             for i in list(slot_of):  # a step failed: nothing of this batch can be gone on from
                 cache.free(slot_of.pop(i))
-            for i in batch:
-                if kept[i] is not None:
-                    cache.free(kept[i])
+            for i, slot in enumerate(kept):  # nor of the earlier batches: the caller never learns their slots
+                if slot is not None:
+                    cache.free(slot)
                     kept[i] = None
             raise
     if streamer is not None and hasattr(streamer, "end"):
         streamer.end()
     sequences = [p + t for p, t in zip(prompts, out_tokens)]
     if keep_slots:
-        return GenerateOutput(sequences, out_scores, out_logits, cache=cache, slots=kept)
+        return GenerateOutput(sequences, out_scores, out_logits, cache=cache, slots=kept,
+                              rng_steps=[first_draw[i] + len(out_tokens[i]) for i in range(len(prompts))])
     if cfg.return_dict_in_generate:
         return GenerateOutput(sequences, out_scores, out_logits)
     return sequences
 
 
+def _step_extras(sampler, step: int, new_budget: int) -> dict:
+    """The processors that follow the step's number rather than its rows (a forced last token, the bonus on EOS that
+    grows with the length), for samplers that have them."""
+    extras = getattr(sampler, "step_extras", None)
+    return extras(step, new_budget) if extras is not None else {}
+
+
 def _decode_ahead(model, cache, sampler, cfg, eos, ids, batch, slot_of, feed, out_tokens, new_budget, padded_len,
-                  done_with) -> None:
+                  done_with, first_draw) -> None:
     """One batch, with every step launched before the host has seen the tokens of the step before it.
 
     The tokens of a step stay on the device (``sampler.sample(..., ahead=True)``) and the next step takes them
@@ -234,8 +253,9 @@ def _decode_ahead(model, cache, sampler, cfg, eos, ids, batch, slot_of, feed, ou
         return (padded_len + step < (cfg.min_length or 0)) or (step < (cfg.min_new_tokens or 0))
 
     def choose(logits, seqs, step):
-        return sampler.sample(logits, rng_seq=[ids[i] for i in seqs], rng_step=[step] * len(seqs),
-                              suppress_eos=[too_short(step)] * len(seqs), need_scores=False, ahead=True)[0]
+        return sampler.sample(logits, rng_seq=[ids[i] for i in seqs], rng_step=[first_draw[i] + step for i in seqs],
+                              suppress_eos=[too_short(step)] * len(seqs), need_scores=False, ahead=True,
+                              **_step_extras(sampler, step, new_budget))[0]
 
     step_no = 0  # the number of the token that `pending` holds for each of its sequences
     seqs = list(batch)

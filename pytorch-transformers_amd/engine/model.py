@@ -20,7 +20,7 @@ import weakref
 import numpy as np
 import torch
 
-from .. import host
+from .. import host, tuning
 from ..cache.paged import PagedCache
 from ..config.registry import AutoConfig, lookup
 from ..parts.base import ResidualSum, StepContext, as_tensor
@@ -218,6 +218,7 @@ class _DecodeGraph:
 class CausalLM:
     def __init__(self, spec: ModelSpec, tensors: Dict[str, torch.Tensor], dtype: torch.dtype, device):
         spec.validate()
+        spec.check_sizes()
         self.spec = spec
         self.config = spec.config
         self.dtype = dtype
@@ -230,6 +231,8 @@ class CausalLM:
                 part.after_load()
         self._move_constants()
         self.generation_config = None
+        #: the timed choices between kernels for this model's shapes (``tune``); active while this model steps
+        self.tuning = tuning.TuningTable()
         #: run steps in which every sequence brings one token as replays of a captured HIP graph
         self.use_graphs = bool(spec.supports_graphs)
         #: ``layer_hook(i, x)`` is called after entry ``i`` of the run order with the residual stream
@@ -254,7 +257,10 @@ class CausalLM:
 
     # construction ----------------------------------------------------------
     @classmethod
-    def from_pretrained(cls, folder: str, dtype="bfloat16", device="cuda:0", strict: bool = True) -> "CausalLM":
+    def from_pretrained(cls, folder: str, dtype="bfloat16", device="cuda:0", strict: bool = True,
+                        tuning_table=None) -> "CausalLM":
+        """``tuning_table``: choices between kernels that another process timed (``tune``), as the dict that
+        ``tune`` returns or the path of a JSON file that holds it."""
         from ..config.generation import GenerationConfig
 
         device = _require_gpu(device)
@@ -262,9 +268,13 @@ class CausalLM:
         dtype = auto_dtype(config, folder) if dtype == "auto" else resolve_dtype(dtype)
         _, builder = lookup(config.model_type)
         spec = builder(config)
+        spec.validate()
+        spec.check_sizes()  # a configuration that no kernel takes is refused before a weight is read
         tensors = load_weights(folder, spec.tensor_specs(), dtype, device, base_prefix=spec.base_prefix, strict=strict)
         model = cls(spec, tensors, dtype, device)
         model.generation_config = GenerationConfig.from_pretrained(folder, config)
+        if tuning_table is not None:
+            model.tune(table=tuning_table)
         return model
 
     @classmethod
@@ -277,6 +287,8 @@ class CausalLM:
         dtype = resolve_dtype(dtype)
         _, builder = lookup(config.model_type)
         spec = builder(config)
+        spec.validate()
+        spec.check_sizes()
         std = float(getattr(config, "initializer_range", 0.02) if std is None else std)
         specs = spec.tensor_specs()
         tensors = random_tensors(specs, seed, std, noise=noise, device=device, compute_dtype=dtype)
@@ -292,30 +304,34 @@ class CausalLM:
     def tune(self, prompt_lens: Sequence[int] = (2048,), batches: Sequence[int] = (8, 64), table=None,
              contexts: Sequence = ()) -> dict:
         """Time, once, the choices between kernels that no rule decides, for prompts of ``prompt_lens`` tokens and
-        decode steps of ``batches`` sequences, and keep them for every later step of this process; returns the
-        table (``ops.tuning_table``).  With ``contexts`` the decode steps are also run at these context lengths,
+        decode steps of ``batches`` sequences, and keep them in this model's table (``self.tuning``) for every
+        later step of this model; returns the table as plain data.  With ``contexts`` the decode steps are also run at these context lengths,
         each a number or a pair (longest, mean of the batch), over a cache that holds whatever it holds (only times
-        are taken): that is where the cut of the decode attention is timed.  With ``table`` given nothing is
-        timed: its choices are taken instead.
+        are taken): that is where the cut of the decode attention is timed.  With ``table`` given (such data, or
+        the path of a JSON file that holds it) nothing is timed: its choices are taken instead.
         Steps never time anything by themselves (unless PTA_TUNE=1 is set): untuned, they take the built-in
         choice, and logits are the same bits in every process."""
-        from .. import ops
-
+        tuning.activate(self.tuning)
         if table is not None:
-            ops.load_tuning(table)
-            return ops.tuning_table()
+            if isinstance(table, (str, os.PathLike)):
+                import json
+
+                with open(table) as f:
+                    table = json.load(f)
+            self.tuning.load(table)
+            return self.tuning.to_dict()
         if self.dtype != torch.bfloat16:
-            return ops.tuning_table()  # the 32-bit path has one kernel per operation
+            return self.tuning.to_dict()  # the 32-bit path has one kernel per operation
         graphs, self.use_graphs = self.use_graphs, False  # nothing can be timed inside a capture
         page = self.page_size
         pairs = sorted({(int(c), int(c)) if isinstance(c, int) else (int(c[0]), int(c[1])) for c in contexts})
         most = max([int(b) for b in batches] + [1])
-        need = max([int(t) for t in prompt_lens] + [0]) + 64 * most + 64
+        need = max([int(t) for t in prompt_lens] + [0]) + page * most + page
         need = max(need, most * ((max([c[0] for c in pairs] + [0]) + page) // page * page))
         cache = self.new_cache(need)
         timed: set = set()  # decode launches whose cuts have been timed in this call
         try:
-            with ops.live_tuning():
+            with tuning.live_tuning():
                 for T in prompt_lens:
                     slot = cache.alloc()
                     self.step(cache, [slot], [[0] * int(T)], "last")
@@ -331,7 +347,7 @@ class CausalLM:
                         if grow:
                             cache.reserve([s_ for s_, _ in grow], [n_ for _, n_ in grow])
                             cache.commit([s_ for s_, _ in grow], [n_ for _, n_ in grow])
-                        ops.take_decode_keys()
+                        tuning.take_decode_keys()
                         self.step(cache, slots, [[0]] * b, "last")
                         if longest > 1 and graphs and os.environ.get("PTA_DECODE_TUNE", "1") != "0":
                             self._time_decode_cuts(cache, slots, timed)
@@ -340,8 +356,8 @@ class CausalLM:
             torch.cuda.synchronize()
         finally:
             self.use_graphs = graphs
-            ops.release_flush()
-        return ops.tuning_table()
+            tuning.release_flush()
+        return self.tuning.to_dict()
 
     def _time_decode_cuts(self, cache: PagedCache, slots: Sequence[int], timed: set, replays: int = 8,
                           rounds: int = 3) -> None:
@@ -350,9 +366,7 @@ class CausalLM:
         the rule's by more than noise.  Whole steps are timed because a cut's time alone, after a flush of the
         caches, does not rank the cuts as a step does.  Nothing is committed: every replay writes the same
         position again."""
-        from .. import ops
-
-        keys = ops.take_decode_keys()
+        keys = tuning.take_decode_keys()
         if not keys:
             return
         b = len(slots)
@@ -381,18 +395,18 @@ class CausalLM:
             if key in timed:
                 continue
             timed.add(key)
-            cuts = ops.decode_plan_candidates(key)
+            cuts = tuning.decode_plan_candidates(key)
             times = []
             for cut in cuts:
-                ops.set_decode_plan(key, cut)
+                tuning.set_decode_plan(key, cut)
                 times.append(step_ms())
             best = min(range(len(cuts)), key=lambda i: times[i])
             chosen = cuts[best] if times[best] < 0.985 * times[0] else None
-            ops.set_decode_plan(key, chosen)
+            tuning.set_decode_plan(key, chosen)
             if os.environ.get("PTA_TUNE_VERBOSE"):
                 print(f"[pta tune] decode attention {key}: " + " ".join(f"{c}:{t:.3f}" for c, t in zip(cuts, times))
                       + f" ms a step -> {chosen or cuts[0]}", flush=True)
-        ops.take_decode_keys()  # the steps above asked too
+        tuning.take_decode_keys()  # the steps above asked too
 
     @property
     def steps_ahead(self) -> bool:
@@ -479,6 +493,7 @@ class CausalLM:
         """
         from ..sampling.ahead import TokensAhead
 
+        tuning.activate(self.tuning)
         graphs = self.use_graphs and self.layer_hook is None
         if isinstance(tokens, TokensAhead):
             if graphs and want == "last":

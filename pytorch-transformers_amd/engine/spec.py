@@ -102,6 +102,15 @@ class ModelSpec:
                 specs.append(s)
         return specs
 
+    def check_sizes(self) -> None:
+        """Every part's sizes against what the kernels take (``Part.check_sizes``): a configuration that cannot run
+        is refused here, before a weight is read."""
+        seen = set()
+        for p in self.parts():
+            if id(p) not in seen:
+                seen.add(id(p))
+                p.check_all_sizes()
+
     def validate(self) -> None:
         groups = {g.name: g for g in self.cache_groups}
         if len(groups) != len(self.cache_groups):

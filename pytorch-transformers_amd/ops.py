@@ -24,7 +24,7 @@ QKV_LAYOUT_CODES = {"grouped": 0, "tail": 1, "interleaved": 2}
 ACT_CODES = {None: 0, "none": 0, "linear": 0, "gelu": 1, "gelu_python": 1, "gelu_new": 2, "gelu_pytorch_tanh": 2,
              "gelu_fast": 2, "gelu_accurate": 2, "quick_gelu": 3, "relu": 4, "relu2": 5, "relu6": 6, "silu": 7, "swish": 7,
              "sigmoid": 8, "tanh": 9, "leaky_relu": 10, "mish": 11, "gelu_10": 12, "laplace": 13}
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 _lib = None
 _lock = threading.Lock()
@@ -32,6 +32,19 @@ _lock = threading.Lock()
 
 class KernelError(RuntimeError):
     pass
+
+
+from . import tuning  # noqa: E402  the timed choices; it calls the faces below back, so each refers to the other by module
+
+
+def __getattr__(name: str):
+    """Names of ``tuning`` (``decode_plan``, ``live_tuning``, ``tuning_table`` ...) are reachable here too."""
+    if name.startswith("__"):
+        raise AttributeError(name)
+    try:
+        return getattr(tuning, name)
+    except AttributeError:
+        raise AttributeError(f"module {__name__!r} has no attribute {name!r}") from None
 
 
 def _build_module():
@@ -308,6 +321,15 @@ def qkv_rope_cache(fused: torch.Tensor, bias, inv_freq, cs_scale: float, token_p
     return q
 
 
+def attention_sizes_problem(nh: int, nkv: int, d: int, rotated: bool) -> Optional[str]:
+    """None if the attention kernels take these head counts and this head size (``rotated``: queries and keys are
+    rotated by position), else the reason.  Launches nothing: for refusing a model before its weights are read."""
+    lib = load_library()
+    if lib.pta_attention_sizes_ok(int(nh), int(nkv), int(d), int(bool(rotated))) == 0:
+        return None
+    return lib.pta_last_error().decode("utf-8", "replace")
+
+
 def attn_generic(q: torch.Tensor, k_pool, v_pool, block_table, token_seq, token_pos, slopes, scale: float,
                  window: int = 0, alibi_exact: bool = False):
     """Causal attention of every token over its sequence's cache (the last ``window`` positions of it, itself
@@ -352,6 +374,7 @@ def gemm_f32(a: torch.Tensor, w: torch.Tensor, bias=None, act=None, add1=None, a
 ATTN_SPLIT_KEYS = 128
 ATTN_FORCE_SPLIT = int(os.environ.get("PTA_ATTN_SPLIT", "0"))
 ATTN_FORCE_TILES = int(os.environ.get("PTA_ATTN_TILES", "0"))
+ATTN_FORCE_WIDE = int(os.environ.get("PTA_ATTN_WIDE", "-1"))  # eight-wave workgroups for prompts: 1 always, 0 never
 
 def attn_mfma_ok(q: torch.Tensor) -> bool:
     """Whether the matrix-core attention kernel takes these queries (bfloat16, head size built)."""
@@ -368,7 +391,8 @@ def attn_decode_shared_ok(head_dim: int, heads_per_kv_head: int) -> bool:
 
 def attn_mfma(q: torch.Tensor, k_pool, v_pool, block_table, cu_tokens, seq_start, slopes, scale: float, *,
               max_new: int, n_splits: int = 1, split_size: int = ATTN_SPLIT_KEYS, window: int = 0,
-              decode_tiles: int = 0, decode_waves: int = 1, alibi_exact: bool = False) -> torch.Tensor:
+              decode_tiles: int = 0, decode_waves: int = 1, alibi_exact: bool = False,
+              prompt_wide: Optional[bool] = None) -> torch.Tensor:
     """Causal attention of a step's tokens over the cache on the matrix cores; out [M, nh*d].
 
     ``max_new`` bounds the new tokens of any sequence of the step; with ``n_splits > 1`` the keys
@@ -376,7 +400,8 @@ def attn_mfma(q: torch.Tensor, k_pool, v_pool, block_table, cu_tokens, seq_start
     ``decode_tiles``: groups of sixteen heads of one KV head that a wave holds when ``max_new`` is 1
     (0: as many as the head size allows).  ``decode_waves``: waves of a workgroup that divide its keys among
     them, or ``SHARED_KEYS``: the heads of a KV head on the waves of one workgroup, which share its keys through
-    LDS (``attn_decode_shared_ok``)."""
+    LDS (``attn_decode_shared_ok``).  ``prompt_wide``: workgroups of eight waves (True) or four (False) for prompts
+    with heads up to 64 (None: eight where the launch has workgroups enough)."""
     _need(q, "q", torch.bfloat16)
     M, nh, d = q.shape
     nkv = k_pool.shape[1]
@@ -397,166 +422,9 @@ def attn_mfma(q: torch.Tensor, k_pool, v_pool, block_table, cu_tokens, seq_start
           _ptr(cu_tokens), _ptr(seq_start), _ptr(slopes), int(bool(alibi_exact)), n_seqs, int(max_new), M, nh, nkv, d,
           ctypes.c_float(scale),
           int(split_size), int(n_splits), _ptr(po), _ptr(pm), _ptr(pl), int(window), int(decode_tiles), int(decode_waves),
-          _stream())
+          ATTN_FORCE_WIDE if prompt_wide is None else int(bool(prompt_wide)), _stream())
     return out
 
-
-@functools.lru_cache(maxsize=None)
-def _decode_plan(n: int, n_heads: int, n_kv_heads: int, head_dim: int, bound: int, mean: int, most_tiles: int):
-    """The cheapest cut of a decode launch of ``n`` sequences of up to ``bound`` keys, ``mean`` on average,
-    by a model of its time.
-
-    A wave holds ``t`` groups of sixteen heads of one KV head and walks ``size`` keys in blocks of 32.  In
-    microseconds, fitted to launches with cold caches at three head shapes (71 heads on 1 KV head of 64; 32 on
-    8 of 128; 128 on 8 of 64), 1 to 64 sequences of 1,100 to 8,192 keys, every cut (the model's choice is
-    within a tenth of the best measured cut nearly everywhere, and mostly equal to it):
-
-    - a wave takes 0.22 + 0.21 t + 0.15 (head_dim / 64 - 1) per block, and waves beyond what the chip
-      holds at once (1,024 SIMDs, as many waves each as 512 registers allow) wait for a whole round;
-    - the keys and values stream at 5.1 TB/s, and again at 7.2 TB/s for every further wave that shares
-      a KV head;
-    - the launch takes the 4.2-norm of those two times (the larger one, and more where they are close);
-    - ranges cost 2.2 + 0.1 per range, and their partial sums (32-bit, written and read) move at 3.5 TB/s.
-
-    The longest context of a step that is sized for ``bound`` lies in its last 1,024 and the mean in the 512
-    below ``mean``, so the longest wave's time is taken at ``bound - 512`` keys and the traffic at
-    ``mean - 256`` keys a sequence."""
-    groups = (n_heads // n_kv_heads + 15) // 16
-    dt = head_dim / 16.0
-    keys = bound - 512
-    mean_keys = min(keys, mean - 256)
-    kv_mb = n * mean_keys * n_kv_heads * head_dim * 4 / 1e6
-    best = None
-    for t in range(1, most_tiles + 1):
-        if ATTN_FORCE_TILES and t != min(ATTN_FORCE_TILES, most_tiles):
-            continue
-        sharing = (groups + t - 1) // t
-        resident = 1024 * max(1, int(512 // ((38 + 11.5 * dt) + (26 + 8 * dt) * t)))
-        block_us = 0.22 + 0.21 * t + 0.15 * (head_dim / 64.0 - 1.0)
-        size = min(ATTN_SPLIT_KEYS, ATTN_FORCE_SPLIT) if ATTN_FORCE_SPLIT else ATTN_SPLIT_KEYS
-        while True:
-            whole = size >= bound
-            if (bound + size - 1) // size <= 1024 and n * ((bound + size - 1) // size) <= 65535 and (not ATTN_FORCE_SPLIT or size == ATTN_FORCE_SPLIT or
-                                                       (whole and size < ATTN_FORCE_SPLIT)):
-                ranges = (mean_keys + size - 1) // size
-                waves = n * n_kv_heads * sharing * ranges
-                wave_us = min(size, keys) / 32 * block_us * ((waves + resident - 1) // resident)
-                stream_us = kv_mb / 5.1 + kv_mb * (sharing - 1) / 7.2
-                part_us = 0.0 if whole else 2.2 + 0.1 * ranges + n * n_heads * ranges * head_dim * 8 / 1e6 / 3.5
-                cost = (wave_us ** 4.2 + stream_us ** 4.2) ** (1 / 4.2) + part_us
-                if best is None or cost < best[0]:
-                    best = (cost, t, size)
-            if whole:
-                break
-            size *= 2
-    if best is None:
-        raise KernelError(f"no cut of a decode launch over {bound} keys with PTA_ATTN_SPLIT={ATTN_FORCE_SPLIT}")
-    return best[1], best[2]
-
-
-_decode_plans: dict = {}  # (batch, heads, KV heads, head size, longest, mean) as counted below -> a timed cut
-
-
-def _decode_key(n_seqs: int, n_heads: int, n_kv_heads: int, head_dim: int, max_len: int, mean_len: int):
-    n = 1
-    while n < n_seqs:
-        n *= 2
-    bound = (max_len + 1023) // 1024 * 1024
-    mean = min(bound, (mean_len + 511) // 512 * 512) if mean_len > 0 else bound
-    return (n, int(n_heads), int(n_kv_heads), int(head_dim), bound, mean)
-
-
-def decode_plan(n_seqs: int, n_heads: int, n_kv_heads: int, head_dim: int, max_len: int, mean_len: int = 0):
-    """How a decode launch is cut: (column tiles per wave, keys per workgroup, waves per workgroup); a size that
-    covers the context means one workgroup per sequence and head group, which writes the result itself.  The
-    waves of a workgroup take its keys block by block in turn and merge in LDS; ``SHARED_KEYS`` in their place
-    means a wave per tile of heads, all on the same keys (``_shared_keys_rule``).
-
-    The batch counts by its next power of two, the longest context by its next multiple of 1,024 and the
-    mean context (``mean_len``; 0: as the longest) by its next multiple of 512, so that a captured step,
-    which is sized for a padded batch and such bounds, is cut exactly as the same step run directly.
-    A cut that was fixed for these counts (``set_decode_plan``; ``CausalLM.tune`` times whole steps with the cuts
-    of ``decode_plan_candidates``) goes before the rule, which has one wave per workgroup or shared keys."""
-    key = _decode_key(n_seqs, n_heads, n_kv_heads, head_dim, max_len, mean_len)
-    kept = _decode_plans.get(key)
-    if kept is not None:
-        return kept
-    n, _, _, _, bound, mean = key
-    shared = _shared_keys_rule(n, n_heads, n_kv_heads, head_dim, bound, mean)
-    if shared is not None:
-        return shared
-    groups = (n_heads // n_kv_heads + 15) // 16
-    most = min(groups, int(load_library().pta_attn_decode_max_tiles(head_dim)))
-    return _decode_plan(n, n_heads, n_kv_heads, head_dim, bound, mean, most) + (1,)
-
-
-def _shared_keys_rule(n: int, n_heads: int, n_kv_heads: int, head_dim: int, bound: int, mean: int):
-    """The cut with keys shared through LDS where it is built (many heads on a KV head) and the launch walks keys
-    enough to fill the chip with such workgroups, else None.  Measured with 71 heads on one KV head of 64, launch
-    and merge after a flush of the caches, against the best cut of one-wave workgroups: 8 sequences of 1,100 keys
-    11.4 against 9.8 us; 32 of 1,100 10.3 against 15.4; 64 of 2,100 14.8 against 26.0; 8 of 16,384 19.8 against
-    24.8; 32 of 16,384 45.6 against 49.8.  Ranges of 256 keys up to 100 k keys in all, 512 up to 300 k, then 1,024."""
-    if ATTN_FORCE_SPLIT or ATTN_FORCE_TILES or not attn_decode_shared_ok(head_dim, n_heads // n_kv_heads):
-        return None
-    keys = n * n_kv_heads * mean
-    if keys < 20_000:
-        return None
-    size = 256 if keys <= 100_000 else 512 if keys <= 300_000 else 1024
-    while size < bound and ((bound + size - 1) // size > 1024 or n * ((bound + size - 1) // size) > 65535):
-        size *= 2  # the launch's limits: ranges of a sequence, and sequences x ranges
-    return (1, min(size, bound), SHARED_KEYS)
-
-
-_decode_keys_seen: set = set()  # what decode launches asked ``decode_plan`` for while timing was on
-
-
-def take_decode_keys() -> list:
-    """The (batch, head shape, context) counts of the decode launches since the last call, while timing was on."""
-    keys = sorted(_decode_keys_seen)
-    _decode_keys_seen.clear()
-    return keys
-
-
-def decode_plan_candidates(key) -> list:
-    """Cuts of the decode launch that ``key`` counts, the rule's first: the one-wave rule's neighbours,
-    workgroups of four and eight waves over the whole context and over ranges of 512 and 1,024 keys, and, where
-    they are built, workgroups that share their keys over ranges of 256 to 1,024 keys and the whole context.  A workgroup of several waves needs no second launch when it walks the whole context, but all its keys
-    pass through one compute unit; which wins depends on how many sequences and KV heads there are to fill the
-    chip.  Timed alone after a flush of the caches, these cuts rank differently than inside a step (the rule's
-    cut at 64 sequences, 8 KV heads of 64 and 1,100 keys: 42 us alone, 31 us in a step, where a cut with four
-    waves takes 34 us both times), so the caller times whole steps with each (``CausalLM.tune``)."""
-    n, nh, nkv, d, bound, mean = key
-    lib = load_library()
-    groups = (nh // nkv + 15) // 16
-    most = min(groups, int(lib.pta_attn_decode_max_tiles(d)))
-    rule = _decode_plan(n, nh, nkv, d, bound, mean, most) + (1,)
-    shared = _shared_keys_rule(n, nh, nkv, d, bound, mean)
-    cuts = [rule] if shared is None else [shared, rule]
-    want = [(rule[0], rule[1] * 2, 1), (rule[0], rule[1] // 2, 1), (max(1, rule[0] - 1), rule[1], 1),
-            (min(most, rule[0] + 1), rule[1], 1)]
-    want += [(t, size, w) for t in (1, min(2, most)) for w in (4, 8) for size in (bound, 1024, 512)]
-    for t, size, w in want:
-        size = min(size, bound)
-        splits = (bound + size - 1) // size
-        if (size < ATTN_SPLIT_KEYS or size % 64 or size // w < 64 or splits > 1024 or n * splits > 65535 or (t, size, w) in cuts
-                or not lib.pta_attn_decode_waves_ok(d, t, w)):
-            continue
-        cuts.append((t, size, w))
-    if attn_decode_shared_ok(d, nh // nkv):
-        for size in (256, 512, 1024, bound):
-            cut = (1, min(size, bound), SHARED_KEYS)
-            splits = (bound + cut[1] - 1) // cut[1]
-            if cut not in cuts and splits <= 1024 and n * splits <= 65535:
-                cuts.append(cut)
-    return cuts
-
-
-def set_decode_plan(key, cut=None) -> None:
-    """Fix the cut of the decode launches that ``key`` counts (None: back to the rule)."""
-    if cut is None:
-        _decode_plans.pop(tuple(key), None)
-    else:
-        _decode_plans[tuple(key)] = tuple(int(v) for v in cut)
 
 
 def attention(q: torch.Tensor, k_pool, v_pool, block_table, ctx, slopes, scale: float, window: int = 0,
@@ -569,11 +437,10 @@ def attention(q: torch.Tensor, k_pool, v_pool, block_table, ctx, slopes, scale: 
     if attn_mfma_ok(q):
         n_splits, size, tiles, waves = 1, ATTN_SPLIT_KEYS, 0, 1
         if ctx.is_decode:
-            if window == 0 and _may_time():
-                _decode_keys_seen.add(_decode_key(ctx.n_seqs, q.shape[1], k_pool.shape[1], q.shape[2], ctx.max_len,
-                                                  getattr(ctx, "mean_len", 0)))
-            tiles, size, waves = decode_plan(ctx.n_seqs, q.shape[1], k_pool.shape[1], q.shape[2], ctx.max_len,
-                                             getattr(ctx, "mean_len", 0))
+            shape = (ctx.n_seqs, q.shape[1], k_pool.shape[1], q.shape[2], ctx.max_len, getattr(ctx, "mean_len", 0))
+            if window == 0:
+                tuning.note_decode_launch(*shape)
+            tiles, size, waves = tuning.decode_plan(*shape)
             n_splits = (ctx.max_len + size - 1) // size
         return attn_mfma(q, k_pool, v_pool, block_table, ctx.cu_tokens, ctx.seq_start, slopes, scale,
                          max_new=max(ctx.new_tokens), n_splits=n_splits, split_size=size, window=window,
@@ -585,8 +452,14 @@ def sample(logits: torch.Tensor, *, do_sample: bool, temperature: float = 1.0, t
            min_p: float = 0.0, typical_p: float = 1.0, epsilon_cutoff: float = 0.0, eta_cutoff: float = 0.0,
            penalty: float = 1.0, hist=None, hist_off=None, ban=None, ban_off=None, eos=None, suppress=None,
            remove_invalid: bool = False, renorm: bool = False, seed: int = 0, rng_seq=None, rng_step=None,
-           uniforms=None, need_scores: bool = True):
+           uniforms=None, need_scores: bool = True, bias_tok=None, bias_val=None, bias_off=None, forced=None,
+           decay: Optional[float] = None):
     """Processors and choice for every row of ``logits`` [R, V] (32-bit); returns (tokens int32 [R], scores [R, V]).
+
+    ``bias_tok`` / ``bias_val`` / ``bias_off``: per row a list of tokens (each once) whose scores get a value added
+    before every other processor.  ``forced``: token ids of which one is forced in this step (every other score
+    goes, theirs become 0; a banned token stays gone).  ``decay``: the scores of the ``eos`` tokens gain
+    ``|score| * decay`` after the removal of invalid values.
 
     Without ``need_scores``, a greedy choice that no processor touches is a plain argmax and the scores
     come back as None."""
@@ -596,8 +469,10 @@ def sample(logits: torch.Tensor, *, do_sample: bool, temperature: float = 1.0, t
     R, V = logits.shape
     if ban is not None and ban.numel() == 0:
         ban = ban_off = None  # no row has a banned token
+    if bias_off is not None and (bias_tok is None or bias_tok.numel() == 0):
+        bias_tok = bias_val = bias_off = None  # no row has a biased token
     if (not need_scores and not do_sample and penalty == 1.0 and suppress is None and ban_off is None
-            and not remove_invalid and not renorm):
+            and not remove_invalid and not renorm and bias_off is None and forced is None and decay is None):
         out = torch.empty((R,), dtype=torch.int32, device=logits.device)
         _call("pta_argmax", _ptr(out), _ptr(logits), R, V, _stream())
         return out, None
@@ -615,6 +490,14 @@ def sample(logits: torch.Tensor, *, do_sample: bool, temperature: float = 1.0, t
         _need(eos, "eos", torch.int32)
     if uniforms is not None:
         _need(uniforms, "uniforms", torch.float32, (R,))
+    if bias_off is not None:
+        _need(bias_off, "bias_off", torch.int32, (R + 1,))
+        _need(bias_tok, "bias_tok", torch.int32)
+        _need(bias_val, "bias_val", torch.float32, tuple(bias_tok.shape))
+    if forced is not None:
+        _need(forced, "forced", torch.int32)
+    if decay is not None and (eos is None or eos.numel() == 0):
+        raise KernelError("a bonus on the EOS tokens needs their ids")
     work = torch.empty_like(logits)
     out = torch.empty((R,), dtype=torch.int32, device=logits.device)
     _call("pta_sample", _ptr(out), _ptr(work), _ptr(logits), R, V, int(bool(do_sample)), ctypes.c_float(temperature),
@@ -623,235 +506,22 @@ def sample(logits: torch.Tensor, *, do_sample: bool, temperature: float = 1.0, t
           _ptr(ban), _ptr(ban_off),
           _ptr(eos), 0 if eos is None else int(eos.numel()), _ptr(suppress), int(bool(remove_invalid)),
           int(bool(renorm)), ctypes.c_uint64(int(seed) & (2 ** 64 - 1)), _ptr(rng_seq), _ptr(rng_step), _ptr(uniforms),
-          int(bool(need_scores)), _stream())
+          int(bool(need_scores)), _ptr(bias_tok), _ptr(bias_val), _ptr(bias_off), _ptr(forced),
+          0 if forced is None else int(forced.numel()), int(decay is not None), ctypes.c_float(decay or 0.0), _stream())
     return out, (work if need_scores else None)
 
-
-# ---- choices that are timed, and when ---------------------------------------------------------------------
-# Some choices between two ways to the same product have no rule that holds across shapes (how many ranges of K
-# a pair launch is cut into, up to how many rows the decode batch kernel beats the vendor library, in which pieces
-# along M the library's product runs, whether two matrices of one input run as one product, whether K is cut into
-# a batch).  Each has a built-in default, and a table keyed by shape that overrides it.  The table is filled only
-# while timing is switched on: inside ``live_tuning()`` (``CausalLM.tune`` runs steps of given sizes in it), or in
-# every step with PTA_TUNE=1 in the environment.  With timing off (the default) a step allocates nothing for
-# measurements and times nothing, and its results depend on weights, tokens and schedule alone: two processes give
-# the same bits.  ``tuning_table()`` / ``load_tuning()`` carry a table from one process to another.
-TUNE_LIVE = os.environ.get("PTA_TUNE", "0") == "1"
-
-
-class live_tuning:
-    """Context in which choices that have no entry in the tuning table yet are timed at first use."""
-
-    def __enter__(self):
-        global TUNE_LIVE
-        self._old, TUNE_LIVE = TUNE_LIVE, True
-        return self
-
-    def __exit__(self, *exc):
-        global TUNE_LIVE
-        TUNE_LIVE = self._old
-        return False
-
-
-def _may_time() -> bool:
-    return TUNE_LIVE and not torch.cuda.is_current_stream_capturing()
-
-
-SKINNY_MAX_ROWS = 64
-# rows up to which the decode batch kernel (x shared through LDS, K split over workgroups) stands in for the
-# vendor library's product, whose choices for 65 to 128 rows leave most of the chip idle (K = 4,544 with N =
-# 4,672 and 18,176 in one product of 128 rows: 151 us, 1.4 TB/s of weights)
-SPLITK_MAX_ROWS = int(os.environ.get("PTA_SPLITK_MAX_ROWS", "256"))
-SPLITK_MARGIN = float(os.environ.get("PTA_SPLITK_MARGIN", "0.95"))
-SPLITK_SURE_ROWS = 128  # up to here the kernel won at every shape measured; beyond, by the weight's own timing
-_splitk_limits: dict = {}  # (N, K) -> rows up to which the batch kernel beats the library's product
-
-
-_flush = None  # half a gigabyte that is read between timed runs; held only while timing is on (``release_flush``)
-
-
-def release_flush() -> None:
-    global _flush
-    _flush = None
-
-
-def _time_ways_cold(ways, device, rounds: int = 3):
-    """Milliseconds of each of ``ways`` (callables), the fastest of ``rounds`` runs each, taken in turn; before
-    every run half a gigabyte is read, so that the weights come from memory as they do in a model (timed back
-    to back, a product finds its matrix in the memory-side cache and every way looks alike).  Read, not
-    written: after half a gigabyte of writes the caches are full of lines that must go back to memory before
-    anything else comes in, which no step of a model leaves behind, and a kernel that streams from memory then
-    measures at little more than half its speed (decode attention over 144 MB of keys and values: 55 us after
-    writes, 31 us in a step)."""
-    global _flush
-    if _flush is None or _flush.device != device:
-        _flush = torch.zeros(128 * 1024 * 1024, dtype=torch.float32, device=device)
-    flush = _flush
-    best = [float("inf")] * len(ways)
-    for run in ways:  # plans are made and the library set up before anything is timed
-        run()
-    for _ in range(rounds):
-        for i, run in enumerate(ways):
-            flush.sum()
-            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            start.record()
-            run()
-            end.record()
-            end.synchronize()
-            best[i] = min(best[i], start.elapsed_time(end))
-    return best
-
-
-def splitk_row_limit(*ws: torch.Tensor) -> int:
-    """Rows up to which the decode batch kernel is the faster way to the product with ``w`` (or, for two weights, to
-    the two products of a pair launch).  Up to 128 rows it always was (one chunk of rows per workgroup); with two
-    chunks it depends on how well the library does at the shape (at 256 rows it wins with K = 4,544, 9.5 against
-    11.4 ms a step of 32 layers, and loses with K = 4,096, 22.1 against 20.2 ms of 60 layers), so both are timed once
-    per shape at 192 and 256 rows, when timing is on; without an entry the kernel stops at 128 rows."""
-    if SPLITK_MAX_ROWS <= SPLITK_SURE_ROWS:
-        return SPLITK_MAX_ROWS
-    key = tuple(tuple(w.shape) for w in ws)
-    limit = _splitk_limits.get(key)
-    if limit is None:
-        if not _may_time():
-            return SPLITK_SURE_ROWS
-        dev = ws[0].device
-        xs = [torch.randn((256, w.shape[1]), dtype=torch.float32, device=dev).to(torch.bfloat16) for w in ws]
-        outs = [torch.empty((256, w.shape[0]), dtype=torch.bfloat16, device=dev) for w in ws]
-        limit = SPLITK_SURE_ROWS
-        for rows in (192, 256):
-            if rows > SPLITK_MAX_ROWS:
-                break
-            xr = [x[:rows] for x in xs]
-
-            def kernel():
-                if len(ws) == 1:
-                    gemm_splitk_bf16(xr[0], ws[0])
-                else:
-                    gemm_splitk_pair_bf16(xr[0], ws[0], xr[1], ws[1])
-
-            def library():
-                for x, w, out in zip(xr, ws, outs):
-                    torch.mm(x, w.t(), out=out[:rows])
-
-            best = _time_ways_cold((kernel, library), dev)
-            if best[0] < SPLITK_MARGIN * best[1]:
-                limit = rows
-            else:
-                break
-        _splitk_limits[key] = limit
-    return limit
-
-
-def _splitk_rows(x: torch.Tensor, *ws: torch.Tensor) -> bool:
-    return x.shape[0] <= SPLITK_SURE_ROWS or x.shape[0] <= splitk_row_limit(*ws)
-
-
-# ---- the vendor library's product for many rows, cut along M where that is faster -----------------------
-# The library picks a kernel per (M, N, K) from a table, and on this hardware its choices are uneven in M:
-# with K = 4,544 and N = 18,176, 2,048 rows take longer than 2,304, and 4,096 rows of the product with the
-# transposed shape almost as long as 8,192.  So, when timing is on, the product is timed once per weight shape at
-# a ladder of row counts, and a product of M rows then runs as the cheapest sequence of those pieces (each written
-# straight into its rows of the result); without an entry it runs whole.  PTA_MM_CHUNKS=0 switches this off.
-MM_LADDER = (256, 512, 768, 1024, 1536, 2048, 3072, 4096, 6144, 8192)
-MM_CHUNKS = os.environ.get("PTA_MM_CHUNKS", "1") != "0"
-MM_JOIN = os.environ.get("PTA_MM_JOIN", "1") != "0"  # one product for two matrices of one input where it is faster
-_mm_times: dict = {}  # (N, K) -> {rows: microseconds}
-_mm_plans: dict = {}  # (N, K, M) -> [rows, ...]
-_mm_costs: dict = {}  # (N, K, M) -> microseconds of that plan, as measured piece by piece
-_mm_joined: dict = {}  # (N1, N2, K, M) -> whether one product with both matrices beats the two
-
-
-def _mm_measure(x: torch.Tensor, w: torch.Tensor, rows: int, out: torch.Tensor) -> float:
-    """Microseconds of ``x[:rows] @ w.T``: the fastest of five runs, each timed on its own (a mean over two runs
-    right after the library's set-up misjudged products by a tenth, enough to choose the slower plan)."""
-    torch.mm(x[:rows], w.t(), out=out[:rows])  # the library's first call of a shape sets it up
-    best = float("inf")
-    for _ in range(5):
-        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        start.record()
-        torch.mm(x[:rows], w.t(), out=out[:rows])
-        end.record()
-        end.synchronize()
-        best = min(best, start.elapsed_time(end) * 1e3)
-    return best
-
-
-def _mm_plan(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor):
-    M, (N, K) = x.shape[0], w.shape
-    bucket = (M + 63) // 64  # row counts within 64 of each other share a plan: one timing of the whole product
-    plan = _mm_plans.get((N, K, bucket))
-    if plan is not None:
-        return plan[:-1] + [M - sum(plan[:-1])]
-    if not _may_time():
-        return [M]
-    times = _mm_times.setdefault((N, K), {})
-    for rows in MM_LADDER:
-        if rows <= M and rows not in times:
-            times[rows] = _mm_measure(x, w, rows, out)
-    whole = M <= MM_LADDER[-1]  # beyond the ladder the product always runs in pieces: timing it whole costs too much
-    if whole and M not in times:
-        times[M] = _mm_measure(x, w, M, out)  # the product as it is
-    # cheapest way to cover M rows with pieces of the ladder; what is left over rides on the last piece
-    units, rest = divmod(M, 256)
-    best = [(0.0, [])] + [None] * units
-    for u in range(1, units + 1):
-        for rows in MM_LADDER:
-            k = rows // 256
-            if k <= u and rows in times and best[u - k] is not None:
-                cand = best[u - k][0] + times[rows]
-                if best[u] is None or cand < best[u][0]:
-                    best[u] = (cand, best[u - k][1] + [rows])
-    cost, pieces = best[units]
-    if rest:
-        pieces = pieces[:-1] + [pieces[-1] + rest]
-        cost *= M / (M - rest)
-    plan = pieces if not whole or (len(pieces) > 1 and cost < 0.97 * times[M]) else [M]
-    _mm_plans[(N, K, bucket)] = plan
-    _mm_costs[(N, K, bucket)] = cost if plan is pieces else times[M]
-    return plan
-
-
-def joined_mm_pays(x: torch.Tensor, joined: torch.Tensor, n_first: int) -> bool:
-    """Whether ``x @ joined.T`` in one library product beats the products with its first ``n_first`` rows and
-    with the rest on their own.  The library's kernel choice decides, so both ways are timed once per shape when
-    timing is on (2,048 rows, K = 4,544, N = 4,672 + 18,176: 308 us against 87 + 286; K = 4,096, N = 6,144 + 16,384:
-    311 against 80 + 179); without an entry the two stay apart."""
-    M, (N, K) = x.shape[0], joined.shape
-    if not MM_JOIN or not MM_CHUNKS or M < 512:
-        return False
-    bucket = (M + 63) // 64
-    key = (n_first, N - n_first, K, bucket)
-    if key not in _mm_joined:
-        if not _may_time():
-            return False
-        first, rest = joined[:n_first], joined[n_first:]
-        ways = (lambda: library_mm(x, joined), lambda: (library_mm(x, first), library_mm(x, rest)))
-        best = [float("inf"), float("inf")]
-        for run in ways:  # plans are made and the library set up before anything is timed
-            run()
-        for _ in range(4):  # the two ways in turn, each run timed on its own; the fastest of each counts
-            for i, run in enumerate(ways):
-                start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                start.record()
-                run()
-                end.record()
-                end.synchronize()
-                best[i] = min(best[i], start.elapsed_time(end))
-        _mm_joined[key] = best[0] < 0.98 * best[1]
-    return _mm_joined[key]
 
 
 def library_mm(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     """``x @ w.T`` in bfloat16 through the vendor library, in the pieces along M that were measured fastest."""
     M, N = x.shape[0], w.shape[0]
     with timed("library_mm", float(w.numel()) * 2, 2.0 * M * N * w.shape[1]):
-        if not MM_CHUNKS or M < 512:
+        if not tuning.MM_CHUNKS or M < 512:
             return torch.mm(x, w.t())
-        if (N, w.shape[1], (M + 63) // 64) not in _mm_plans and not _may_time():
+        if (N, w.shape[1], (M + 63) // 64) not in tuning.active().mm_plans and not tuning.may_time():
             return torch.mm(x, w.t())
         out = torch.empty((M, N), dtype=x.dtype, device=x.device)
-        plan = _mm_plan(x, w, out)
+        plan = tuning.mm_plan(x, w, out)
         at = 0
         for rows in plan:
             torch.mm(x[at:at + rows], w.t(), out=out[at:at + rows])
@@ -868,7 +538,6 @@ def library_mm(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
 # timing is on; without an entry the plain product runs.
 MM_KSPLIT = os.environ.get("PTA_MM_KSPLIT", "1") != "0"
 MM_KSPLIT_MAX_ROWS = 1536  # at 2,048 rows the batch gained nothing alone and lost 3 % in a model (K = 32,768, N = 8,192)
-_mm_ksplit: dict = {}  # (N, K, row bucket) -> ranges of K (1: the plain product)
 
 
 def _k_batch(x: torch.Tensor, w: torch.Tensor, S: int) -> torch.Tensor:
@@ -882,19 +551,19 @@ def library_mm_ksplit(x: torch.Tensor, w: torch.Tensor, bias=None, act=None, add
     """``act(x @ w.T + bias) + add1 + add2`` through the library's batched product over ranges of K, where that
     was timed faster than its plain product (once per shape, by 64 rows); else None."""
     M, (N, K) = x.shape[0], w.shape
-    if (not MM_KSPLIT or K < 2 * N or not (SPLITK_MAX_ROWS < M <= MM_KSPLIT_MAX_ROWS) or K % 32 or x.stride(1) != 1
+    if (not MM_KSPLIT or K < 2 * N or not (tuning.SPLITK_MAX_ROWS < M <= MM_KSPLIT_MAX_ROWS) or K % 32 or x.stride(1) != 1
             or not w.is_contiguous()):
         return None
     key = (N, K, (M + 63) // 64)
-    S = _mm_ksplit.get(key)
+    S = tuning.active().mm_ksplit.get(key)
     if S is None:
-        if not _may_time():
+        if not tuning.may_time():
             return None
         ways = [(1, lambda: library_mm(x, w))] + [(s, (lambda s=s: _k_batch(x, w, s))) for s in (2, 4) if K % (s * 8) == 0]
-        best = _time_ways_cold([run for _, run in ways], x.device)
+        best = tuning.time_ways_cold([run for _, run in ways], x.device)
         pick = min(range(len(ways)), key=lambda i: best[i])
         S = ways[pick][0] if best[pick] < 0.9 * best[0] else 1
-        _mm_ksplit[key] = S
+        tuning.active().mm_ksplit[key] = S
     if S == 1:
         return None
     with timed("library_mm", float(w.numel()) * 2, 2.0 * M * N * K):
@@ -1035,215 +704,6 @@ def gemm_stationary_rule(N1: int, K1: int, N2: int, K2: int, cls: int):
     return q1.value, q2.value
 
 
-# Ranges of K for the pairs of a shape: the kernel library's rule gives a choice; when timing is on, its neighbours
-# are timed once per shape, at 64 rows, with cold caches, and one that is at least 3 % faster is kept for every
-# later launch (PTA_PAIR_TUNE=0 switches this off).
-PAIR_TUNE = os.environ.get("PTA_PAIR_TUNE", "1") != "0"
-PAIR_TUNE_MARGIN = 0.97
-PAIR_TUNE_ROWS = int(os.environ.get("PTA_PAIR_TUNE_ROWS", "64"))  # rows of the timed launches (17 to 128)
-_pair_parts_tuned: dict = {}  # (shape of w1, shape of w2) -> the counts in use
-_pair_stationary_tuned: dict = {}  # (shape of w1, shape of w2) -> per class of rows the (ranges, ranges) of the
-#                                    launch with stationary activations, (0, 0) where the staged kernel stays
-
-
-def tune_pair_parts(w1: torch.Tensor, w2: torch.Tensor) -> None:
-    """Once per pair of shapes, while timing is on: time the pair launch with the rule's ranges of K, with their
-    neighbours, and with workgroups of 128 rows of W (which load the activations half as often, have half as many
-    workgroups and so want more ranges), at 64 rows with cold caches; keep the fastest in the kernel library if it
-    beats the rule's by the margin and is no slower than the rule's at 24 rows (where the tile height does not
-    apply, but the ranges do).  ``_pair_parts_tuned`` says what is in use: (ranges, ranges, row tiles per wave).
-    Then, at 8, 32, 64 and 128 rows (one count per class of rows), the launch with stationary activations is timed
-    against the winner with one to six ranges of the shorter K (and as many times more of the longer), each
-    with what reads its partial sums behind it (the norm that adds them, where the two products have one width; else
-    a charge for the ranges' bytes): the fastest is fixed for the class, or the staged kernel where that is not
-    beaten by 2 % (``_pair_stationary_tuned``)."""
-    key = (tuple(w1.shape), tuple(w2.shape))
-    if not PAIR_TUNE or key in _pair_parts_tuned or not _may_time():
-        return
-    lib = load_library()
-    (N1, K1), (N2, K2) = w1.shape, w2.shape
-    a0, b0 = gemm_splitk_pair_parts(N1, K1, N2, K2)
-    fix = lambda c: lib.pta_gemm_splitk_pair_fix(int(N1), int(K1), int(N2), int(K2), int(c[0]), int(c[1]), int(c[2]))
-    forget = lambda: lib.pta_gemm_splitk_pair_fix(int(N1), int(K1), int(N2), int(K2), 0, 0, 1)
-    fix_st = lambda cls, c: lib.pta_gemm_splitk_pair_fix_stationary(int(N1), int(K1), int(N2), int(K2), int(cls), int(c[0]), int(c[1]))
-    for cls in range(len(STATIONARY_CLASS_ROWS)):
-        fix_st(cls, (0, 0))  # the launches timed first are the staged kernel's
-    cands = [(a0, b0, 1)] + [(a, b, 1) for a in range(max(1, a0 - 1), a0 + 3) for b in range(max(1, b0 - 2), b0 + 3)
-                             if (a, b) != (a0, b0)]
-    tall = lambda p: sorted({max(1, p - 1), p, p + 1, max(1, 2 * p - 1), 2 * p, 2 * p + 1})
-    cands += [(a, b, 2) for a in tall(a0) for b in tall(b0)]
-    cands = [c for c in cands if fix(c) == 0]
-    xs = {rows: [torch.randn((rows, K), dtype=torch.float32, device=w1.device).to(torch.bfloat16) for K in (K1, K2)]
-          for rows in sorted({PAIR_TUNE_ROWS, 24, 8, 32, 64, 128})}
-    xs_bf16 = {rows: torch.zeros((rows, N1), dtype=torch.bfloat16, device=w1.device) for rows in xs}
-    kmin = min(K1, K2)
-    f1, f2 = max(1, (K1 + kmin // 2) // kmin), max(1, (K2 + kmin // 2) // kmin)
-    st_cands = [(b * f1, b * f2) for b in (1, 2, 3, 4, 6) if b * f1 <= 16 and b * f2 <= 16 and fix_st(0, (b * f1, b * f2)) == 0]
-    fix_st(0, (0, 0))
-    most = [max([c[i] for c in cands] + [c[i] for c in st_cands] + [16]) for i in (0, 1)]
-    parts = [torch.empty((most[i], 128, N), dtype=torch.float32, device=w1.device) for i, N in enumerate((N1, N2))]
-    # A launch is timed over several copies of the matrices in turn (more bytes than the memory-side cache holds),
-    # back to back between two events: every launch reads its matrices from memory, as in a model, and no gap of
-    # the host's lies inside the timed span.
-    copy_bytes = (w1.numel() + w2.numel()) * 2
-    n_copies = max(2, min(6, int(640e6 // copy_bytes) + 1))
-    copies = [(w1, w2)] + [(w1.clone(), w2.clone()) for _ in range(n_copies - 1)]
-
-    def timed_ways(chosen, rows, rounds=3, fix=fix, read=None):
-        best = [float("inf")] * len(chosen)
-        for r in range(rounds + 1):  # the first round warms up
-            for j, c in enumerate(chosen):
-                fix(c)
-                start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                start.record()
-                for a, b in copies:
-                    _call("pta_gemm_splitk_pair_bf16", _ptr(parts[0]), _ptr(xs[rows][0]), _ptr(a), int(N1), int(K1),
-                          _ptr(parts[1]), _ptr(xs[rows][1]), _ptr(b), int(N2), int(K2), rows, _stream())
-                    if read is not None:
-                        read(c, rows)
-                end.record()
-                end.synchronize()
-                if r > 0:
-                    best[j] = min(best[j], start.elapsed_time(end) / len(copies))
-        return best
-
-    # Two products of the same width are a block's last ones, and what reads their partial sums next is the norm
-    # that adds them: it is launched behind every timed launch of the comparison below, so that a launch pays for
-    # the ranges it leaves to be added and for how it leaves them (all at once at its end, or as it goes).
-    norm_w = (torch.ones(N1, dtype=torch.float32, device=w1.device)
-              if N1 == N2 and layernorm_sum_ok(N1) and os.environ.get("PTA_PAIR_TUNE_READER", "1") != "0" else None)
-
-    def read_sums(c, rows):
-        views = [parts[i].view(-1)[:int(c[-2 + i]) * rows * N].view(int(c[-2 + i]), rows, N) for i, N in enumerate((N1, N2))]
-        layernorm_sum([(views[1], None), (views[0], None), xs_bf16[rows]], N1, w=norm_w, b=norm_w, eps=1e-5)
-
-    try:
-        times = timed_ways(cands, PAIR_TUNE_ROWS)
-        order = sorted(range(len(cands)), key=lambda i: times[i])
-        short = [0] + [i for i in order if i != 0 and times[i] < PAIR_TUNE_MARGIN * times[0]][:3]
-        small = timed_ways([cands[i] for i in short], 24) if len(short) > 1 else [0.0]
-    finally:
-        forget()
-    if os.environ.get("PTA_TUNE_VERBOSE"):
-        print(f"[pta tune] pair {key}: rule {cands[0]} {times[0] * 1e3:.1f} us at {PAIR_TUNE_ROWS} rows; fastest " +
-              ", ".join(f"{cands[i]} {times[i] * 1e3:.1f}" for i in order[:6]) +
-              (f"; at 24 rows {[round(t * 1e3, 1) for t in small]} for {[cands[i] for i in short]}" if len(short) > 1 else ""),
-              flush=True)
-    chosen = cands[0]
-    for i, t24 in zip(short[1:], small[1:]):  # fastest first
-        if t24 <= 1.03 * small[0]:
-            chosen = cands[i]
-            break
-    if chosen != cands[0]:
-        fix(chosen)
-    _pair_parts_tuned[key] = chosen
-    # the launch with stationary activations against that choice, per class of rows
-    chosen_st = []
-    try:
-        for cls, rows in enumerate((8, 32, 64, 128)):
-            fix_st(cls, (0, 0))
-            # what reads the partial sums afterwards pays for every range (measured: some 8 TB/s worth of them), so
-            # a launch is charged for its ranges' bytes at that rate on top of its own time
-            read = read_sums if norm_w is not None else None
-            slices_ms = (lambda c: 0.0) if read else (lambda c: (c[0] * N1 + c[1] * N2) * rows * 4 / 8e12 * 1e3)
-            t_staged = timed_ways([chosen[:2]], rows, fix=lambda c: None, read=read)[0] + slices_ms(chosen)
-            t_st = (timed_ways([(cls,) + c for c in st_cands], rows, fix=lambda a: fix_st(a[0], a[1:]), read=read)
-                    if st_cands else [])
-            t_st = [t + slices_ms(c) for t, c in zip(t_st, st_cands)]
-            best = min(range(len(st_cands)), key=lambda i: t_st[i]) if st_cands else -1
-            keep = st_cands[best] if best >= 0 and t_st[best] < 0.98 * t_staged else (0, 0)
-            chosen_st.append(keep)
-            if os.environ.get("PTA_TUNE_VERBOSE"):
-                print(f"[pta tune] pair {key} at {rows} rows (with the reading of the partial sums): staged {t_staged * 1e3:.1f} us; stationary " +
-                      ", ".join(f"{c} {t * 1e3:.1f}" for c, t in zip(st_cands, t_st)) + f" -> {keep}", flush=True)
-    finally:
-        while len(chosen_st) < len(STATIONARY_CLASS_ROWS):
-            chosen_st.append((0, 0))
-        for cls, c in enumerate(chosen_st):
-            fix_st(cls, c)
-    _pair_stationary_tuned[key] = tuple(chosen_st)
-
-
-def tuning_table() -> dict:
-    """What has been timed so far, as plain data (JSON-able): give it to ``load_tuning`` in another process and
-    that process makes the same choices, hence the same bits."""
-    key = lambda t: ",".join("x".join(str(int(v)) for v in (p if isinstance(p, tuple) else (p,))) for p in t)
-    return {
-        "pair_parts": {key(k): list(v) for k, v in _pair_parts_tuned.items()},  # ranges, ranges, row tiles per wave
-        "pair_stationary": {key(k): [list(c) for c in v] for k, v in _pair_stationary_tuned.items()},  # per class of rows
-        "splitk_rows": {key(k): int(v) for k, v in _splitk_limits.items()},
-        "mm_plans": {key(k): list(v) for k, v in _mm_plans.items()},
-        "mm_joined": {key(k): bool(v) for k, v in _mm_joined.items()},
-        "mm_ksplit": {key(k): int(v) for k, v in _mm_ksplit.items()},
-        "decode_plans": {key(k): list(v) for k, v in _decode_plans.items()},  # tiles, keys per workgroup, waves
-    }
-
-
-def clear_tuning() -> None:
-    """Back to the built-in defaults for every shape."""
-    lib = load_library()
-    for (s1, s2) in list(_pair_parts_tuned):
-        lib.pta_gemm_splitk_pair_fix(int(s1[0]), int(s1[1]), int(s2[0]), int(s2[1]), 0, 0, 1)
-    for (s1, s2) in list(_pair_stationary_tuned):
-        lib.pta_gemm_splitk_pair_fix_stationary(int(s1[0]), int(s1[1]), int(s2[0]), int(s2[1]), -1, 0, 0)
-    for d in (_pair_stationary_tuned, _pair_parts_tuned, _splitk_limits, _mm_plans, _mm_costs, _mm_times, _mm_joined, _mm_ksplit, _decode_plans):
-        d.clear()
-
-
-def load_tuning(table: dict) -> None:
-    """Take the choices of a table that ``tuning_table`` made (entries for other shapes stay as they are)."""
-    lib = load_library()
-    shapes = lambda k: tuple(tuple(int(v) for v in p.split("x")) for p in k.split(","))
-    flat = lambda k: tuple(int(p) for p in k.split(","))
-    for k, v in table.get("pair_parts", {}).items():
-        s1, s2 = shapes(k)
-        a, b, rt = int(v[0]), int(v[1]), int(v[2]) if len(v) > 2 else 1
-        rule = gemm_splitk_pair_parts_rule(s1[0], s1[1], s2[0], s2[1])
-        if (a, b, rt) != rule + (1,) and lib.pta_gemm_splitk_pair_fix(s1[0], s1[1], s2[0], s2[1], a, b, rt):
-            raise KernelError(f"tuning table: {a} and {b} ranges of K with {rt} row tiles are not valid for the pair {k}")
-        _pair_parts_tuned[(s1, s2)] = (a, b, rt)
-    for k, v in table.get("pair_stationary", {}).items():
-        s1, s2 = shapes(k)
-        for cls, c in enumerate(v):
-            if lib.pta_gemm_splitk_pair_fix_stationary(s1[0], s1[1], s2[0], s2[1], cls, int(c[0]), int(c[1])):
-                raise KernelError(f"tuning table: {list(c)} is not valid for the pair {k} with stationary activations")
-        _pair_stationary_tuned[(s1, s2)] = tuple((int(c[0]), int(c[1])) for c in v)
-    for k, v in table.get("splitk_rows", {}).items():
-        _splitk_limits[shapes(k)] = int(v)
-    for k, v in table.get("mm_plans", {}).items():
-        _mm_plans[flat(k)] = [int(r) for r in v]
-    for k, v in table.get("mm_joined", {}).items():
-        _mm_joined[flat(k)] = bool(v)
-    for k, v in table.get("mm_ksplit", {}).items():
-        _mm_ksplit[flat(k)] = int(v)
-    for k, v in table.get("decode_plans", {}).items():
-        _decode_plans[flat(k)] = tuple(int(p) for p in v)
-
-
-def gemm_splitk_pair_parts_rule(N1: int, K1: int, N2: int, K2: int):
-    """The ranges of K that the kernel library's own rule gives a pair, whatever has been fixed for the shape."""
-    lib = load_library()
-    kept = _pair_parts_tuned.get(((int(N1), int(K1)), (int(N2), int(K2))))
-    lib.pta_gemm_splitk_pair_fix(int(N1), int(K1), int(N2), int(K2), 0, 0, 1)
-    rule = gemm_splitk_pair_parts(N1, K1, N2, K2)
-    if kept is not None and tuple(kept) != rule + (1,):
-        lib.pta_gemm_splitk_pair_fix(int(N1), int(K1), int(N2), int(K2), int(kept[0]), int(kept[1]), int(kept[2]))
-    return rule
-
-
-# Elements of both matrices of a pair launch up to which it beats the two products on their own beyond 48 rows.
-# Measured in whole decode steps: pairs of 104 M elements (K = 4,544, N = 4,672 + 18,176) and of 92 M (K = 4,096, N
-# = 6,144 + 16,384) win at every row count; a pair of 344 M (K = 8,192, N = 9,216 + 32,768) wins up to 48 rows (32
-# rows: 20.8 against 23.0 ms a step) and loses beyond them to the vendor library's product for the longer matrix
-# (64 rows: 24.3 against 23.3 ms).
-PAIR_MAX_WEIGHTS = 160 * 1024 * 1024
-PAIR_SURE_ROWS = 48
-
-
-def pair_launch_pays(rows: int, w1: torch.Tensor, w2: torch.Tensor) -> bool:
-    """Whether two products of ``rows`` rows (17 and more) run as one launch of the decode batch kernels."""
-    return rows <= PAIR_SURE_ROWS or w1.numel() + w2.numel() <= PAIR_MAX_WEIGHTS
-
 
 def gemm_splitk_pair_partial(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tensor, w2: torch.Tensor):
     """(x1 @ w1.T, x2 @ w2.T), both left as 32-bit partial sums, in one launch; the products share M."""
@@ -1254,7 +714,7 @@ def gemm_splitk_pair_partial(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tenso
         raise KernelError(f"a pair shares M: x1 {tuple(x1.shape)}, w1 {tuple(w1.shape)}, x2 {tuple(x2.shape)}, "
                           f"w2 {tuple(w2.shape)}")
     (N1, K1), (N2, K2) = w1.shape, w2.shape
-    tune_pair_parts(w1, w2)
+    tuning.tune_pair_parts(w1, w2)
     p1, p2 = gemm_splitk_pair_parts(N1, K1, N2, K2, M)
     part1 = torch.empty((p1, M, N1), dtype=torch.float32, device=x1.device)
     part2 = torch.empty((p2, M, N2), dtype=torch.float32, device=x1.device)
@@ -1279,7 +739,7 @@ def gemm_splitk_pair_bf16(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tensor, 
         _need(bias1, "bias1", torch.float32, (N1,))
     if bias2 is not None:
         _need(bias2, "bias2", torch.float32, (N2,))
-    tune_pair_parts(w1, w2)
+    tuning.tune_pair_parts(w1, w2)
     p1, p2 = gemm_splitk_pair_parts(N1, K1, N2, K2, M)
     part1 = torch.empty((p1, M, N1), dtype=torch.float32, device=x1.device)
     part2 = torch.empty((p2, M, N2), dtype=torch.float32, device=x1.device)
@@ -1316,7 +776,7 @@ def gemm_splitk_pair_qkv(x1: torch.Tensor, w_qkv: torch.Tensor, bias_qkv, inv_fr
         raise KernelError("block_table must be [sequences, pages]")
     freq_ld = _freq_ld(inv_freq, d, block_table.shape[0])
     _need_pools(k_pool, v_pool, torch.bfloat16, nkv, d)
-    tune_pair_parts(w_qkv, w2)
+    tuning.tune_pair_parts(w_qkv, w2)
     p1, p2 = gemm_splitk_pair_parts(N1, K1, N2, K2, M)
     part1 = torch.empty((p1, M, N1), dtype=torch.float32, device=x1.device)
     part2 = torch.empty((p2, M, N2), dtype=torch.float32, device=x1.device)
@@ -1363,8 +823,8 @@ def gemm_splitk_qkv(x: torch.Tensor, w_qkv: torch.Tensor, bias_qkv, inv_freq, cs
 def gemm_partial_pair_ok(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tensor, w2: torch.Tensor) -> bool:
     """Whether two products onto the same features are best left as partial sums of one launch: up to 128
     rows each, and at least one of them worth leaving so on its own."""
-    return (_bf16_rows_ok(x1, w1) and _bf16_rows_ok(x2, w2) and 0 < x1.shape[0] == x2.shape[0] <= SPLITK_MAX_ROWS
-            and _splitk_rows(x1, w1, w2)
+    return (_bf16_rows_ok(x1, w1) and _bf16_rows_ok(x2, w2) and 0 < x1.shape[0] == x2.shape[0] <= tuning.SPLITK_MAX_ROWS
+            and tuning.splitk_rows_ok(x1, w1, w2)
             and w1.shape[0] == w2.shape[0] and w1.shape[0] % 8 == 0
             and (gemm_partial_ok(x1, w1) or gemm_partial_ok(x2, w2)))
 
@@ -1372,7 +832,7 @@ def gemm_partial_pair_ok(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tensor, w
 def gemm_partial_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
     """Whether leaving x @ w.T as partial sums for the next norm pays: up to 128 rows, and either K long against
     N (any batch: the kernel for few rows has too few row tiles there) or a batch past 16 rows."""
-    if not (_bf16_rows_ok(x, w) and 0 < x.shape[0] <= SPLITK_MAX_ROWS and w.shape[0] % 8 == 0 and _splitk_rows(x, w)):
+    if not (_bf16_rows_ok(x, w) and 0 < x.shape[0] <= tuning.SPLITK_MAX_ROWS and w.shape[0] % 8 == 0 and tuning.splitk_rows_ok(x, w)):
         return False
     return w.shape[1] >= 2 * w.shape[0] or (x.shape[0] > 16 and w.shape[0] < 2 * w.shape[1])
 
@@ -1458,16 +918,16 @@ def gemm_skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
 def gemm_splitk_pair_ok(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tensor, w2: torch.Tensor) -> bool:
     """Whether the two products run as a pair launch of the decode batch kernel (17 to 256 rows; beyond 128 only
     where the pair was timed faster than the library's two products)."""
-    return (_bf16_rows_ok(x1, w1) and _bf16_rows_ok(x2, w2) and 16 < x1.shape[0] == x2.shape[0] <= SPLITK_MAX_ROWS
-            and _splitk_rows(x1, w1, w2))
+    return (_bf16_rows_ok(x1, w1) and _bf16_rows_ok(x2, w2) and 16 < x1.shape[0] == x2.shape[0] <= tuning.SPLITK_MAX_ROWS
+            and tuning.splitk_rows_ok(x1, w1, w2))
 
 
 def gemm_splitk_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
     """Whether the kernel for a decode batch of 17 to 128 rows is the faster choice.  Measured at K = 4,544 and
     K = 18,176: it beats the vendor library except where N is long against K (the feed-forward's first matrix
     and the output head), which give the library enough row tiles to fill the chip."""
-    return (_bf16_rows_ok(x, w) and 16 < x.shape[0] <= SPLITK_MAX_ROWS and w.shape[0] < 2 * w.shape[1]
-            and _splitk_rows(x, w))
+    return (_bf16_rows_ok(x, w) and 16 < x.shape[0] <= tuning.SPLITK_MAX_ROWS and w.shape[0] < 2 * w.shape[1]
+            and tuning.splitk_rows_ok(x, w))
 
 
 def gemm_skinny_bf16(x: torch.Tensor, w: torch.Tensor, bias=None, act=None, add1=None, add2=None,

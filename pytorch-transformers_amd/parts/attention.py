@@ -47,6 +47,12 @@ class AttentionMixer(Part):
 
     can_defer = True
 
+    def check_sizes(self) -> None:
+        rotated = self.positions.rotation()[0] is not None or hasattr(self.positions, "rotation_for")
+        problem = ops.attention_sizes_problem(self.num_heads, self.kv_heads, self.head_dim, rotated)
+        if problem is not None:
+            raise ValueError(f"{self.name}: {problem}")
+
     def input_projection(self):
         """The first product of ``forward`` and how it is called: a block may run it together with another
         part's and hand the result back as ``projected``."""

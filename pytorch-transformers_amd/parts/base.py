@@ -94,6 +94,14 @@ class Part:
         for c in self.children():
             c.load_all(tensors)
 
+    def check_sizes(self) -> None:
+        """Raise ``ValueError`` if no kernel takes this part's sizes; called before a weight is read or drawn."""
+
+    def check_all_sizes(self) -> None:
+        self.check_sizes()
+        for c in self.children():
+            c.check_all_sizes()
+
 
 @dataclasses.dataclass
 class PartialProduct:

@@ -63,12 +63,17 @@ class TextGenerationPipeline:
 
 
 def pipeline(task: str = "text-generation", model: Optional[str] = None, dtype="bfloat16", device="cuda:0",
-             tokenizer=None, **kwargs) -> TextGenerationPipeline:
+             tokenizer=None, tuning_table=None, **kwargs) -> TextGenerationPipeline:
+    """``tuning_table``: timed choices between kernels for the model to take (``CausalLM.tune``'s result, or the
+    path of a JSON file that holds it)."""
     if task != "text-generation":
         raise ValueError(f"task {task!r} is not built; only 'text-generation'")
     if model is None:
         raise ValueError("pipeline needs model=<folder with config.json and model.safetensors>")
     if isinstance(model, str):
         tokenizer = tokenizer or load_tokenizer(model)
-        model = AutoModelForCausalLM.from_pretrained(model, dtype=kwargs.pop("torch_dtype", None) or dtype, device=device)
+        model = AutoModelForCausalLM.from_pretrained(model, dtype=kwargs.pop("torch_dtype", None) or dtype, device=device,
+                                                     tuning_table=tuning_table)
+    elif tuning_table is not None:
+        model.tune(table=tuning_table)
     return TextGenerationPipeline(model, tokenizer)

@@ -9,12 +9,16 @@ defaults and meanings: ``--model_type``, ``--model_name_or_path``, ``--prompt``,
 (``do_sample=True``, :408-417) and prints ``=== GENERATED SEQUENCE n ===`` before each result
 (:425-441).  Added here: ``--prompt_ids`` / ``--prompt_file`` (token ids, for folders without a
 tokenizer), ``--greedy``, ``--dtype``, ``--random_config`` with ``--random_seed`` (write a model
-folder with random weights first), ``--min_length``-style limits and ``--batch_size``.
+folder with random weights first), ``--min_length``-style limits and ``--batch_size``; ``--tune`` (time, once,
+the choices between kernels that no rule decides, for this run's prompt lengths and batch, before anything is
+generated) and ``--tuning_table FILE`` (such choices as a JSON file: read if it is there, written after ``--tune``),
+with which a run makes the choices of the run that was measured.
 """
 from __future__ import annotations
 
 import argparse
 import json
+import os
 import sys
 import tempfile
 
@@ -58,6 +62,10 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--device", default="cuda:0")
     ap.add_argument("--random_config", type=str, default=None, help="config.json to build a random-weights model from")
     ap.add_argument("--random_seed", type=int, default=0)
+    ap.add_argument("--tune", action="store_true",
+                    help="time the choices between kernels for this run's prompt lengths and batch before generating")
+    ap.add_argument("--tuning_table", type=str, default=None,
+                    help="JSON file of timed choices: taken if it exists; written after --tune")
     return ap
 
 
@@ -81,7 +89,8 @@ def main(argv=None) -> int:
     if args.model_type is not None and args.model_type != config.model_type:
         print(f"--model_type {args.model_type} but {folder} holds model_type {config.model_type}", file=sys.stderr)
         return 2
-    pipe = pipeline("text-generation", model=folder, dtype=args.dtype, device=args.device)
+    table = args.tuning_table if args.tuning_table and os.path.isfile(args.tuning_table) else None
+    pipe = pipeline("text-generation", model=folder, dtype=args.dtype, device=args.device, tuning_table=table)
 
     if args.prompt_file:
         with open(args.prompt_file) as f:
@@ -103,6 +112,16 @@ def main(argv=None) -> int:
     else:
         gen.update(do_sample=True, temperature=args.temperature, top_k=args.k, top_p=args.p, min_p=args.min_p)
     GenerationConfig(**{k: v for k, v in gen.items()})  # validate before the model runs
+    if args.tune:
+        lens = [len(pipe._encode(p, args.prefix)) for p in prompts]
+        rows = len(prompts) * (gen["num_return_sequences"] or 1)
+        batch = min(rows, args.batch_size) if args.batch_size else rows
+        mean = sum(lens) // len(lens)
+        timed = pipe.model.tune(prompt_lens=sorted(set(lens)), batches=(batch,),
+                                contexts=((max(lens) + 1, mean + 1), (max(lens) + length, mean + length)))
+        if args.tuning_table:
+            with open(args.tuning_table, "w") as f:
+                json.dump(timed, f)
     results = pipe(prompts, prefix=args.prefix, batch_size=args.batch_size, **gen)
     n = 0
     for records in results:

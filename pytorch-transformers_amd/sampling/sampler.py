@@ -17,7 +17,7 @@ import torch
 from .. import ops
 from ..config.generation import GenerationConfig
 from .ahead import TokensAhead
-from .bans import BanRules
+from .bans import BanRules, BiasRules
 
 
 class Sampler:
@@ -41,11 +41,29 @@ class Sampler:
         self.penalty = float(c.repetition_penalty) if c.repetition_penalty is not None else 1.0
         self.bans = BanRules(c.no_repeat_ngram_size, c.bad_words_ids, c.suppress_tokens, c.begin_suppress_tokens,
                              self.eos_ids)
+        self.biases = BiasRules(c.sequence_bias, vocab_size)
+        forced = c.forced_eos_token_ids
+        self._forced_dev = torch.tensor(forced, dtype=torch.int32, device=self.device) if forced else None
+        self.decay = c.exponential_decay_length_penalty  # (start index, factor) or None
+        if self.decay is not None and not self.eos_ids:
+            raise ValueError("`exponential_decay_length_penalty` raises the scores of the EOS tokens: set `eos_token_id`")
+
+    def step_extras(self, step: int, new_budget: int) -> dict:
+        """What ``sample`` needs to know of a step beyond its rows, from the step's number among the new tokens (0
+        for the first) and the number of new tokens allowed: whether the last token is forced now
+        (src/transformers/generation/logits_process.py:1590-1596: at ``max_length - 1``) and the factor of the
+        bonus on EOS (:1716-1727: ``factor ** (tokens past the start index) - 1``, from the token after it)."""
+        out = {}
+        if self._forced_dev is not None and step == new_budget - 1:
+            out["force"] = True
+        if self.decay is not None and step > int(self.decay[0]):
+            out["decay"] = float(self.decay[1]) ** (step - int(self.decay[0])) - 1.0
+        return out
 
     def sample(self, logits: torch.Tensor, *, rng_seq: Sequence[int], rng_step: Sequence[int],
                histories: Optional[Sequence[Sequence[int]]] = None, suppress_eos: Optional[Sequence[bool]] = None,
                uniforms: Optional[Sequence[float]] = None, new_counts: Optional[Sequence[int]] = None,
-               need_scores: bool = True, ahead: bool = False):
+               need_scores: bool = True, ahead: bool = False, force: bool = False, decay: Optional[float] = None):
         """Tokens for the rows of ``logits`` and the processed scores ``[rows, vocab]`` (None if not needed
         and the choice could be made without forming them).  ``histories`` are the rows' ids so far (prompt and
         new tokens) and ``new_counts`` how many of them are new; the repetition penalty and the options that forbid
@@ -56,15 +74,25 @@ class Sampler:
             raise ValueError("tokens ahead of the host cannot be chosen by options that read the tokens so far")
         suppress = self._eos_dev is not None and suppress_eos is not None and any(suppress_eos)
         ban_lists = None
+        force = bool(force) and self._forced_dev is not None
         if self.bans:
             if histories is None:
                 raise ValueError("options that forbid tokens by what was generated need the rows' histories")
             counts = new_counts if new_counts is not None else [1] * R
-            ban_lists = [self.bans.banned(h, n) for h, n in zip(histories, counts)]
+            if force:  # what the forced token overrides does not apply in this step
+                ban_lists = [self.bans.banned_after_force(n) for n in counts]
+            else:
+                ban_lists = [self.bans.banned(h, n) for h, n in zip(histories, counts)]
             if not any(ban_lists):
                 ban_lists = None
+        bias_lists = None
+        if self.biases:
+            if histories is None and self.biases.needs_history:
+                raise ValueError("a bias on sequences of several tokens needs the rows' histories")
+            bias_lists = [self.biases.biases(histories[r] if histories is not None else None) for r in range(R)]
         if (not need_scores and not self.do_sample and self.penalty == 1.0 and not suppress and ban_lists is None
-                and not self.config.remove_invalid_values and not self.config.renormalize_logits):
+                and not self.config.remove_invalid_values and not self.config.renormalize_logits
+                and bias_lists is None and not force and decay is None):
             # greedy with no processor in the way: nothing to upload, one argmax kernel
             chosen = ops.sample(logits, do_sample=False, need_scores=False)[0]
             return (TokensAhead(chosen) if ahead else chosen.tolist()), None
@@ -82,6 +110,12 @@ class Sampler:
             boff = np.zeros(R + 1, dtype=np.int32)
             boff[1:] = np.cumsum([len(b) for b in ban_lists])
             pieces += [boff, np.asarray([t for b in ban_lists for t in b], dtype=np.int32)]
+        n_bias_at = len(pieces)
+        if bias_lists is not None:  # offsets, tokens, and the values' bits as integers (one buffer, one copy)
+            voff = np.zeros(R + 1, dtype=np.int32)
+            voff[1:] = np.cumsum([len(b) for b in bias_lists])
+            pieces += [voff, np.asarray([t for b in bias_lists for t, _ in b], dtype=np.int32),
+                       np.asarray([v for b in bias_lists for _, v in b], dtype=np.float32).view(np.int32)]
         staged = torch.from_numpy(np.concatenate(pieces))
         # (ahead of the host nothing may wait for the stream: the copy starts from pinned memory and does not block)
         dev = staged.pin_memory().to(self.device, non_blocking=True) if ahead else staged.to(self.device)
@@ -100,13 +134,17 @@ class Sampler:
             ban_off=views[n_before] if ban_lists is not None else None, eos=self._eos_dev,
             suppress=views[2] if (self._eos_dev is not None and suppress_eos is not None and any(suppress_eos)) else None,
             remove_invalid=self.config.remove_invalid_values, renorm=self.config.renormalize_logits,
-            seed=self.config.seed, rng_seq=views[0], rng_step=views[1], uniforms=u, need_scores=need_scores)
+            seed=self.config.seed, rng_seq=views[0], rng_step=views[1], uniforms=u, need_scores=need_scores,
+            bias_off=views[n_bias_at] if bias_lists is not None else None,
+            bias_tok=views[n_bias_at + 1] if bias_lists is not None else None,
+            bias_val=views[n_bias_at + 2].view(torch.float32) if bias_lists is not None else None,
+            forced=self._forced_dev if force else None, decay=decay)
         return (TokensAhead(tokens) if ahead else tokens.tolist()), scores
 
     @property
     def needs_histories(self) -> bool:
         """Whether a choice reads the sequence's tokens so far (which the host then has to have seen)."""
-        return bool(self.bans) or self.penalty != 1.0
+        return bool(self.bans) or self.penalty != 1.0 or self.biases.needs_history
 
 
 def philox_uniform(seed: int, seq: int, step: int) -> float:

@@ -113,6 +113,17 @@ def plain_logits(folder: str, reqs: Dict[str, List[int]]) -> Dict[str, torch.Ten
     return {rid: plain.forward(cfg, w, toks).float() for rid, toks in reqs.items()}
 
 
+def plain_logits_on_gpu(folder: str, reqs: Dict[str, List[int]], last: int = 0) -> Dict[str, torch.Tensor]:
+    """The plain implementation's float64 logits (of the last ``last`` places; 0: all) with its tensors on the GPU:
+    the same functions as ``plain_logits``, plain torch, nothing of the engine, for sizes at which the CPU takes
+    minutes."""
+    cfg, w = plain.read_model(folder, device="cuda")
+    out = {rid: plain.forward(cfg, w, toks, last=last).float().cpu() for rid, toks in reqs.items()}
+    del w
+    torch.cuda.empty_cache()
+    return out
+
+
 def lengths_reached(reqs: Dict[str, List[int]], records: List[dict]) -> Dict[str, List[int]]:
     """For every token of every request, the length its request had after the step that brought the token: what
     frequencies that follow a sequence's length look at."""

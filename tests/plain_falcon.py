@@ -22,8 +22,9 @@ DT = torch.float64
 
 
 # --- files -----------------------------------------------------------------
-def read_model(folder: str, dtype=DT):
-    """config.json as a dict, tensors by name (src/transformers/modeling_utils.py:3680-3695, :493-560)."""
+def read_model(folder: str, dtype=DT, device=None):
+    """config.json as a dict, tensors by name (src/transformers/modeling_utils.py:3680-3695, :493-560).
+    ``device``: where the tensors are put (default: the CPU); every function below computes where its inputs lie."""
     from safetensors.torch import load_file
 
     with open(os.path.join(folder, "config.json")) as f:
@@ -37,7 +38,7 @@ def read_model(folder: str, dtype=DT):
         tensors = {}
         for shard in sorted(set(wm.values())):
             tensors.update(load_file(os.path.join(folder, shard)))
-    return cfg, {k: v.to(dtype) for k, v in tensors.items()}
+    return cfg, {k: v.to(device=device, dtype=dtype) for k, v in tensors.items()}
 
 
 def cfg_defaults(cfg: dict) -> dict:
@@ -153,7 +154,7 @@ def rope_parameters(c, seq_len: Optional[int] = None):
 def rope_cos_sin(positions, inv_freq, dtype=DT, scale=1.0):
     """angles = position * inv_freq in 32-bit, doubled along the last axis
     (src/transformers/models/falcon/modeling_falcon.py:155-164)."""
-    freqs = positions.float()[:, None] * inv_freq.float()[None, :]
+    freqs = positions.float()[:, None] * inv_freq.float().to(positions.device)[None, :]
     emb = torch.cat((freqs, freqs), dim=-1)
     return (emb.cos() * scale).to(dtype), (emb.sin() * scale).to(dtype)
 
@@ -218,7 +219,7 @@ def attention_scores_softmax(q, k, v, bias=None):
     nkv = k.shape[1]
     g = nh // nkv
     out = torch.empty_like(q)
-    mask = torch.full((T, T), float("-inf"), dtype=q.dtype).triu(1)
+    mask = torch.full((T, T), float("-inf"), dtype=q.dtype, device=q.device).triu(1)
     for h in range(nh):
         s = q[:, h] @ k[:, h // g].T / math.sqrt(d)
         if bias is not None:
@@ -239,7 +240,7 @@ def self_attention(x, w, prefix, c, positions, seq_lens=None):
     q, k, v = split_heads(fused, c)
     bias = None
     if c["alibi"]:
-        bias = alibi_bias(nh, x.shape[0], d, x.dtype, bool(c.get("alibi_bf16_compat", True)))
+        bias = alibi_bias(nh, x.shape[0], d, x.dtype, bool(c.get("alibi_bf16_compat", True))).to(x.device)
     elif seq_lens is None or (c.get("rope_scaling") or {}).get("rope_type", (c.get("rope_scaling") or {}).get("type")) != "dynamic":
         inv_freq, scale = rope_parameters(c, x.shape[0])
         cos, sin = rope_cos_sin(positions, inv_freq, x.dtype, scale)
@@ -247,7 +248,7 @@ def self_attention(x, w, prefix, c, positions, seq_lens=None):
     else:
         q, k = q.clone(), k.clone()
         for n in sorted(set(int(v) for v in seq_lens)):  # the tokens of one forward pass share its table
-            rows = torch.tensor([t for t, v in enumerate(seq_lens) if int(v) == n])
+            rows = torch.tensor([t for t, v in enumerate(seq_lens) if int(v) == n], device=x.device)
             inv_freq, scale = rope_parameters(c, n)
             cos, sin = rope_cos_sin(positions[rows], inv_freq, x.dtype, scale)
             q[rows], k[rows] = apply_rope(q[rows], cos, sin), apply_rope(k[rows], cos, sin)
@@ -311,21 +312,23 @@ def decoder_layer(x, w, i, c, positions, seq_lens=None):
 
 
 def forward(cfg: dict, w: Dict[str, torch.Tensor], token_ids: Sequence[int], seq_lens: Optional[Sequence[int]] = None,
-            hidden: Optional[list] = None):
+            hidden: Optional[list] = None, last: int = 0):
     """Logits [T, V] of one whole sequence (FalconModel.forward :864-1011, head :1230).  ``seq_lens``: see
     ``self_attention``; it says in which pieces the sequence was fed, for configurations that ask.  ``hidden``: a
-    list that receives the residual stream after every layer."""
+    list that receives the residual stream after every layer.  ``last``: the logits of the last ``last`` places only
+    (the reference's ``num_logits_to_keep``, :1230; 0: all)."""
     c = cfg_defaults(cfg)
-    ids = torch.as_tensor(list(token_ids), dtype=torch.long)
-    x = w["transformer.word_embeddings.weight"][ids]  # :895-896
-    positions = torch.arange(len(ids))
+    table = w["transformer.word_embeddings.weight"]
+    ids = torch.as_tensor(list(token_ids), dtype=torch.long, device=table.device)
+    x = table[ids]  # :895-896
+    positions = torch.arange(len(ids), device=table.device)
     for i in range(c["num_hidden_layers"]):
         x = decoder_layer(x, w, i, c, positions, seq_lens)
         if hidden is not None:
             hidden.append(x)
     x = layer_norm(x, w["transformer.ln_f.weight"], w["transformer.ln_f.bias"], c["layer_norm_epsilon"])  # :992
     head = w["lm_head.weight"] if "lm_head.weight" in w else w["transformer.word_embeddings.weight"]  # tied :1163
-    return x @ head.T
+    return x[-last:] @ head.T  # x[-0:] is all of x
 
 
 # --- generation ---------------------------------------------------------------
@@ -430,24 +433,65 @@ def no_repeat_ngram(scores, history, n):
 
 def no_bad_words(scores, history, bad_words, eos_ids=()):
     """logits_process.py:1110-1140, :1270-1286: -inf for the last token of an entry whose other tokens end the ids
-    so far (one-token entries always); an entry that is an EOS token alone does not count."""
+    so far (one-token entries always; an entry longer than the ids so far never applies, :1122); an entry that is an
+    EOS token alone does not count."""
     ids = list(history)
     gone = []
     for word in bad_words:
         if len(word) == 1 and word[0] in eos_ids:
             continue
-        if len(word) == 1 or (len(word) - 1 <= len(ids) and ids[len(ids) - (len(word) - 1):] == list(word[:-1])):
+        if len(word) == 1 or (len(word) <= len(ids) and ids[len(ids) - (len(word) - 1):] == list(word[:-1])):
             gone.append(word[-1])
     return suppress(scores, gone)
 
 
+def sequence_bias(scores, history, entries):
+    """logits_process.py:1112-1140: ``entries`` is {tuple of ids: bias}; an entry of one token adds its bias to that
+    token always, a longer one to its last token while the ids so far end in the tokens before it (an entry longer
+    than the ids so far never applies, :1122)."""
+    ids = list(history)
+    out = scores.clone()
+    for seq, bias in entries.items():
+        seq = tuple(seq)
+        if len(seq) == 1:
+            out[seq[0]] += bias
+        elif len(seq) <= len(ids) and tuple(ids[len(ids) - (len(seq) - 1):]) == seq[:-1]:
+            out[seq[-1]] += bias
+    return out
+
+
+def forced_eos(scores, cur_len, max_length, forced_ids):
+    """logits_process.py:1590-1596: with one token left before ``max_length`` every score becomes -inf and the
+    forced ids' become 0."""
+    if cur_len != max_length - 1:
+        return scores
+    out = torch.full_like(scores, float("-inf"))
+    out[torch.as_tensor(list(forced_ids), dtype=torch.long)] = 0
+    return out
+
+
+def exponential_decay(scores, cur_len, prompt_len, start_index, factor, eos_ids):
+    """logits_process.py:1699-1727: past ``start_index + prompt_len`` ids, the EOS scores gain
+    ``|score| * (factor ** (ids past that) - 1)``."""
+    start = start_index + prompt_len
+    if cur_len <= start:
+        return scores
+    out = scores.clone()
+    idx = torch.as_tensor(list(eos_ids), dtype=torch.long)
+    out[idx] = scores[idx] + torch.abs(scores[idx]) * (pow(factor, cur_len - start) - 1)
+    return out
+
+
 def process(scores, history, *, do_sample, temperature_=1.0, top_k_=0, top_p_=1.0, min_p_=None, typical_p_=None,
             epsilon_cutoff_=None, eta_cutoff_=None, repetition_penalty_=1.0, suppress_ids=(), no_repeat_ngram_size_=0,
-            bad_words_ids_=None, eos_ids_=()):
-    """Processors in the order the reference builds them (src/transformers/generation/utils.py:926-1097):
-    repetition penalty, no-repeat n-grams, bad words, minimum length, then (sampling only) temperature, top-k, top-p, min-p, typical-p,
-    epsilon and eta cut-offs."""
+            bad_words_ids_=None, eos_ids_=(), sequence_bias_=None, forced_eos_=None, exponential_decay_=None):
+    """Processors in the order the reference builds them (src/transformers/generation/utils.py:898-1097):
+    sequence bias, repetition penalty, no-repeat n-grams, bad words, minimum length, forced last token
+    (``forced_eos_``: (max_length, ids)), the growing bonus on EOS (``exponential_decay_``: (prompt length, start index,
+    factor)), then (sampling only) temperature, top-k, top-p, min-p, typical-p, epsilon and eta cut-offs."""
     s = scores
+    if sequence_bias_:
+        s = sequence_bias(s, history, sequence_bias_)
     if repetition_penalty_ is not None and repetition_penalty_ != 1.0:
         s = repetition_penalty(s, history, repetition_penalty_)
     if no_repeat_ngram_size_:
@@ -456,6 +500,10 @@ def process(scores, history, *, do_sample, temperature_=1.0, top_k_=0, top_p_=1.
         s = no_bad_words(s, history, bad_words_ids_, eos_ids_)
     if suppress_ids:
         s = suppress(s, suppress_ids)
+    if forced_eos_ is not None:
+        s = forced_eos(s, len(history), forced_eos_[0], forced_eos_[1])
+    if exponential_decay_ is not None:
+        s = exponential_decay(s, len(history), exponential_decay_[0], exponential_decay_[1], exponential_decay_[2], eos_ids_)
     if do_sample:
         if temperature_ is not None and temperature_ != 1.0:
             s = temperature(s, temperature_)
@@ -485,11 +533,17 @@ def pick(scores, u: Optional[float]):
 
 
 def generate(cfg, w, prompt: Sequence[int], max_new_tokens: int, *, eos_ids=(), min_new_tokens=0,
-             uniforms: Optional[Sequence[float]] = None, **proc) -> List[int]:
+             uniforms: Optional[Sequence[float]] = None, forced_eos_ids=None, exponential_decay_length_penalty=None,
+             **proc) -> List[int]:
     """One sequence, recomputed whole at every step (no cache); returns the new tokens, EOS included
     (loop of src/transformers/generation/utils.py:3220-3296, stop test stopping_criteria.py:446-467)."""
     seq = list(prompt)
     new = []
+    if forced_eos_ids is not None:  # max_length = prompt + new tokens (src/transformers/generation/utils.py:1461)
+        proc["forced_eos_"] = (len(prompt) + max_new_tokens, list(forced_eos_ids))
+    if exponential_decay_length_penalty is not None:
+        proc["exponential_decay_"] = (len(prompt), *exponential_decay_length_penalty)
+        proc.setdefault("eos_ids_", tuple(eos_ids))
     for step in range(max_new_tokens):
         logits = forward(cfg, w, seq)[-1].float()
         s = process(logits, seq, do_sample=uniforms is not None,

@@ -173,3 +173,53 @@ def test_generation_config_from_folder(tmp_path):
         {"eos_token_id": 2, "bos_token_id": 1, "do_sample": True, "temperature": 0.7, "transformers_version": "4.33"}))
     g = GenerationConfig.from_pretrained(str(tmp_path))
     assert (g.eos_token_id, g.do_sample, g.temperature) == (2, True, 0.7)
+
+
+def test_options_that_are_not_built_are_refused_by_name_and_the_rest_is_kept(tmp_path):
+    """A ``generation_config.json`` that names an option which would change the tokens and is not built raises with
+    the option's name and the file's; options that change nothing here are kept and written back."""
+    path = tmp_path / "generation_config.json"
+    harmless = {"eos_token_id": 2, "max_length": 30, "transformers_version": "4.33", "length_penalty": 2.0,
+                "early_stopping": True, "num_beam_groups": 1, "penalty_alpha": None, "_from_model_config": True}
+    path.write_text(json.dumps(harmless))
+    g = GenerationConfig.from_pretrained(str(tmp_path))
+    assert g.max_length == 30 and g.extra["length_penalty"] == 2.0 and g.extra["transformers_version"] == "4.33"
+    assert g.to_dict()["early_stopping"] is True and GenerationConfig.from_dict(g.to_dict()) == g
+    for bad in ({"forced_bos_token_id": 1}, {"penalty_alpha": 0.6, "top_k": 4}, {"num_beams": 4},
+                {"encoder_repetition_penalty": 1.3}, {"prompt_lookup_num_tokens": 3}, {"guidance_scale": 1.5},
+                {"watermarking_config": {"bias": 2.0}}, {"output_attentions": True}, {"diversity_penalty": 0.5}):
+        path.write_text(json.dumps(dict(harmless, **bad)))
+        name = next(k for k in bad if k != "top_k")
+        with pytest.raises(ValueError, match=f"(?s)generation_config.json.*not built.*{name}"):
+            GenerationConfig.from_pretrained(str(tmp_path))
+    with pytest.raises(ValueError, match="arguments of generate.*guidance_scale"):
+        g.updated(guidance_scale=2.0)
+    path.write_text(json.dumps({"do_sample": True, "temperature": 0.0}))
+    with pytest.raises(ValueError, match="generation_config.json.*temperature"):  # a bad value names its file too
+        GenerationConfig.from_pretrained(str(tmp_path))
+
+
+def test_bias_forced_token_and_decay_options():
+    from pytorch_transformers_amd.sampling.bans import BiasRules
+
+    g = GenerationConfig(sequence_bias={(5, 6): -2.0, (7,): 1.5}, forced_eos_token_id=3,
+                         exponential_decay_length_penalty=(4, 1.1))
+    assert g.sequence_bias == [[[5, 6], -2.0], [[7], 1.5]] and g.forced_eos_token_ids == [3]
+    assert g.exponential_decay_length_penalty == [4, 1.1] and GenerationConfig.from_dict(json.loads(json.dumps(g.to_dict()))) == g
+    for bad, match in (({"sequence_bias": []}, "non-empty"), ({"sequence_bias": [[[1, 2], 3]]}, "positive integers and float"),
+                       ({"sequence_bias": [[[], 1.0]]}, "positive integers and float"), ({"sequence_bias": {"a": 1.0}}, "tuples as keys"),
+                       ({"forced_eos_token_id": -1}, "positive integers"), ({"forced_eos_token_id": [2, 1.5]}, "positive integers"),
+                       ({"exponential_decay_length_penalty": [1.5, 2.0]}, "start_index"),
+                       ({"exponential_decay_length_penalty": [3, -1.0]}, "start_index")):
+        with pytest.raises(ValueError, match=match):
+            GenerationConfig(**bad)
+    # tests/generation/test_logits_process.py:604-629 on the host's rule
+    rules = BiasRules([[[1], 100.0], [[4], 100.0], [[1, 0], -100.0], [[0, 1, 2], -100.0], [[1, 3, 1, 3], -100.0],
+                       [[1, 3, 1, 3, 1, 3], -100.0]], vocab_size=5)
+    assert rules.biases([0, 1, 3, 1]) == [(0, -100.0), (1, 100.0), (3, -100.0), (4, 100.0)]
+    assert rules.biases([0, 1, 0, 1]) == [(0, -100.0), (1, 100.0), (2, -100.0), (4, 100.0)]
+    both = BiasRules([[[3, 1], 1.5], [[2, 3, 1], 2.0], [[1], 0.25]])
+    assert both.biases([9, 2, 3]) == [(1, 3.75)] and both.biases([2, 3]) == [(1, 1.75)] and both.needs_history
+    assert not BiasRules([[[1], 0.5]]).needs_history and BiasRules([[[1], 0.5]]).biases(None) == [(1, 0.5)] and not BiasRules()
+    with pytest.raises(ValueError, match="vocabulary size is 5"):
+        BiasRules([[[1, 7], 1.0]], vocab_size=5)

@@ -248,12 +248,12 @@ def test_pair_ranges_are_timed_once_per_shape_and_kept():
     rule = ops.gemm_splitk_pair_parts(N1, K1, N2, K2)
     key = ((N1, K1), (N2, K2))
     ops.gemm_splitk_pair_bf16(x1, w1, x2, w2)
-    assert ops.TUNE_LIVE or key not in ops._pair_parts_tuned, "a launch times nothing unless timing is switched on"
+    assert ops.TUNE_LIVE or key not in ops.active().pair_parts, "a launch times nothing unless timing is switched on"
     with ops.live_tuning():
         y1, y2 = ops.gemm_splitk_pair_bf16(x1, w1, x2, w2)
     ops.release_flush()
     if ops.PAIR_TUNE:
-        kept = ops._pair_parts_tuned[key]  # ranges, ranges, row tiles per wave
+        kept = ops.active().pair_parts[key]  # ranges, ranges, row tiles per wave
         assert kept[2] in (1, 2) and 1 <= kept[0] <= 2 * rule[0] + 1 and 1 <= kept[1] <= 2 * rule[1] + 1
         assert ops.gemm_splitk_pair_parts(N1, K1, N2, K2) == kept[:2]
     p1, p2 = ops.gemm_splitk_pair_parts(N1, K1, N2, K2)
@@ -283,8 +283,8 @@ def test_pair_ranges_are_timed_once_per_shape_and_kept():
     finally:
         assert lib.pta_gemm_splitk_pair_fix_parts(N1, K1, N2, K2, 0, 0) == 0
         assert lib.pta_gemm_splitk_pair_fix_stationary(N1, K1, N2, K2, -1, 0, 0) == 0
-        ops._pair_parts_tuned.pop(key, None)
-        ops._pair_stationary_tuned.pop(key, None)
+        ops.active().pair_parts.pop(key, None)
+        ops.active().pair_stationary.pop(key, None)
     assert ops.gemm_splitk_pair_parts(N1, K1, N2, K2) == rule
 
 
@@ -412,15 +412,15 @@ def test_library_mm_in_pieces():
     ops = _ops()
     N, K = 136, 264
     w = _rand(N, K, seed=1, dtype=torch.bfloat16, scale=0.05)
-    ops._mm_times[(N, K)] = {256: 1.0, 512: 50.0, 1000: 1e6, 1030: 1e6}  # pieces of 256 look cheapest
+    ops.active().mm_times[(N, K)] = {256: 1.0, 512: 50.0, 1000: 1e6, 1030: 1e6}  # pieces of 256 look cheapest
     try:
         for M in (1000, 1030, 700):
             x = _rand(M, K, seed=M, dtype=torch.bfloat16)
             ops.library_mm(x, w)
-            assert ops.TUNE_LIVE or (N, K, (M + 63) // 64) not in ops._mm_plans, "no plan is made unless timing is on"
+            assert ops.TUNE_LIVE or (N, K, (M + 63) // 64) not in ops.active().mm_plans, "no plan is made unless timing is on"
             with ops.live_tuning():
                 y = ops.library_mm(x, w)
-            plan = ops._mm_plans[(N, K, (M + 63) // 64)]
+            plan = ops.active().mm_plans[(N, K, (M + 63) // 64)]
             if M != 700:
                 assert len(plan) > 1 and sum(plan) == M and all(p >= 256 for p in plan), plan
             torch.testing.assert_close(y.float(), torch.mm(x, w.t()).float(), rtol=2e-2, atol=2e-2)
@@ -428,9 +428,9 @@ def test_library_mm_in_pieces():
         x = _rand(1001, K, seed=7, dtype=torch.bfloat16)
         torch.testing.assert_close(ops.library_mm(x, w).float(), torch.mm(x, w.t()).float(), rtol=2e-2, atol=2e-2)
     finally:
-        ops._mm_times.pop((N, K), None)
-        for key in [k for k in ops._mm_plans if k[:2] == (N, K)]:
-            ops._mm_plans.pop(key)
+        ops.active().mm_times.pop((N, K), None)
+        for key in [k for k in ops.active().mm_plans if k[:2] == (N, K)]:
+            ops.active().mm_plans.pop(key)
 
 
 def test_gemm_skinny_refuses_what_it_cannot_do():
@@ -769,7 +769,7 @@ def test_attn_generic_far_key_and_alibi(dtype):
         _attn_case(ops, _generic(ops), dtype, nh, nh, 16, starts=[0, 290], news=[40, 30], slopes=slopes)
 
 
-def _mfma(ops, n_splits_for=None, tiles=0, waves=1):
+def _mfma(ops, n_splits_for=None, tiles=0, waves=1, wide=None):
     def fn(q, k_pool, v_pool, bt, token_seq, token_pos, slopes, scale, starts, news, window=0):
         cu = torch.tensor([0] + list(torch.tensor(news).cumsum(0)), dtype=torch.int32).cuda()
         st = torch.tensor(starts, dtype=torch.int32).cuda()
@@ -777,7 +777,8 @@ def _mfma(ops, n_splits_for=None, tiles=0, waves=1):
         if n_splits_for is not None:
             n_splits = (max(s + n for s, n in zip(starts, news)) + n_splits_for - 1) // n_splits_for
         return ops.attn_mfma(q, k_pool, v_pool, bt, cu, st, slopes, scale, max_new=max(news), n_splits=n_splits,
-                             split_size=n_splits_for or 256, window=window, decode_tiles=tiles, decode_waves=waves)
+                             split_size=n_splits_for or 256, window=window, decode_tiles=tiles, decode_waves=waves,
+                             prompt_wide=wide)
     return fn
 
 
@@ -798,13 +799,10 @@ def test_attn_mfma_long_prompts(nh, nkv, d):
     _attn_case(ops, _mfma(ops), torch.bfloat16, nh, nkv, d, starts=[0, 900, 3], news=[1300, 500, 61], boost=[7, 1390, None])
     if d <= 64:
         # workgroups of eight waves, which launches with four such workgroups a compute unit and more choose by themselves
-        os.environ["PTA_ATTN_WIDE"] = "1"
-        try:
-            _attn_case(ops, _mfma(ops), torch.bfloat16, nh, nkv, d, starts=[0, 900, 3], news=[1300, 500, 61], boost=[7, 1390, None])
-            _attn_case(ops, _mfma(ops), torch.bfloat16, nh, nkv, d, starts=[0, 63, 200, 0, 127, 31], news=[70, 1, 5, 1, 2, 40])
-            _attn_case(ops, _mfma(ops), torch.bfloat16, nh, nkv, d, starts=[0, 700], news=[800, 300], window=200, seed=4)
-        finally:
-            del os.environ["PTA_ATTN_WIDE"]
+        eight = _mfma(ops, wide=True)
+        _attn_case(ops, eight, torch.bfloat16, nh, nkv, d, starts=[0, 900, 3], news=[1300, 500, 61], boost=[7, 1390, None])
+        _attn_case(ops, eight, torch.bfloat16, nh, nkv, d, starts=[0, 63, 200, 0, 127, 31], news=[70, 1, 5, 1, 2, 40])
+        _attn_case(ops, eight, torch.bfloat16, nh, nkv, d, starts=[0, 700], news=[800, 300], window=200, seed=4)
     slopes = None
     if nh == 16:
         from pytorch_transformers_amd.parts import AlibiPositions
@@ -951,7 +949,8 @@ def test_decode_plan():
 @pytest.mark.parametrize("n,lengths", [(8, "equal"), (64, "equal"), (16, "unequal"), (33, "unequal")])
 def test_decode_attention_as_planned(nh, nkv, d, n, lengths):
     """A decode step's attention the way the engine cuts it at the published models' head shapes (groups of
-    heads per wave, keys per wave, with and without partial sums), against the 32-bit-arithmetic kernel."""
+    heads per wave, keys per wave, with and without partial sums), against plain attention over each sequence's keys
+    and values as the pages hold them (float64, on the GPU)."""
     from types import SimpleNamespace
 
     from pytorch_transformers_amd.engine.model import _len_bound, mean_len_bound
@@ -982,7 +981,15 @@ def test_decode_attention_as_planned(nh, nkv, d, n, lengths):
                           token_pos=torch.tensor(starts, dtype=torch.int32).cuda())
     scale = 1.0 / math.sqrt(d)
     got = ops.attention(q, k_pool, v_pool, bt.cuda(), ctx, None, scale).float()
-    want = ops.attn_generic(q, k_pool, v_pool, bt.cuda(), ctx.token_seq, ctx.token_pos, None, scale).float()
+    rows = []
+    for i, L in enumerate(lens):
+        mine = bt[i, :pages[i]].long().cuda()
+        k = k_pool[mine].permute(0, 2, 1, 3).reshape(-1, nkv, d)[:L].double()  # [page, kv head, 64, d] -> [keys, kv head, d]
+        v = v_pool[mine].permute(0, 3, 1, 2).reshape(-1, nkv, d)[:L].double()  # [page, kv head, d, 64] -> the same
+        q_full = torch.zeros(L, nh, d, dtype=torch.float64, device="cuda")
+        q_full[-1] = q[i].double()  # plain attention wants a query per position: the last one is the step's
+        rows.append(P.attention_scores_softmax(q_full, k, v)[-1])
+    want = torch.stack(rows).float()
     assert float((got - want).abs().max()) <= 2e-2 * max(1.0, float(want.abs().max()))
     far = v_pool[int(bt[0, 0]), :, :, 5].float().repeat_interleave(nh // nkv, 0).reshape(-1)
     assert float((got[0] - far).abs().max()) < 0.05, "the far key does not dominate"
@@ -990,7 +997,7 @@ def test_decode_attention_as_planned(nh, nkv, d, n, lengths):
     assert 1 <= tiles <= (nh // nkv + 15) // 16 and size % 64 == 0 and waves in (1, ops.SHARED_KEYS)
     # the same launch with every other cut that may be timed against the rule's: the same result within rounding;
     # a fixed cut holds for the step's bucket and for no other, travels in the tuning table, and is forgotten with it
-    key = ops._decode_key(n, nh, nkv, d, ctx.max_len, ctx.mean_len)
+    key = ops.decode_key(n, nh, nkv, d, ctx.max_len, ctx.mean_len)
     cuts = ops.decode_plan_candidates(key)
     assert cuts[0] == (tiles, size, waves) and len(set(cuts)) == len(cuts) > 3 and any(c[2] > 1 for c in cuts)
     assert any(c[2] == ops.SHARED_KEYS for c in cuts) == ops.attn_decode_shared_ok(d, nh // nkv)
@@ -1008,7 +1015,7 @@ def test_decode_attention_as_planned(nh, nkv, d, n, lengths):
             assert float((fixed - want).abs().max()) <= 2e-2 * max(1.0, float(want.abs().max())), cut
             assert float((fixed[0] - far).abs().max()) < 0.05, cut
         other = ops.decode_plan(n, nh, nkv, d, ctx.max_len + 2048, ctx.mean_len)  # another bucket: the rule
-        assert other == ops.decode_plan_candidates(ops._decode_key(n, nh, nkv, d, ctx.max_len + 2048, ctx.mean_len))[0]
+        assert other == ops.decode_plan_candidates(ops.decode_key(n, nh, nkv, d, ctx.max_len + 2048, ctx.mean_len))[0]
         table = ops.tuning_table()
         assert table["decode_plans"][",".join(str(v) for v in key)] == list(cuts[-1])
         ops.clear_tuning()

@@ -132,7 +132,7 @@ def test_joined_matrices_give_one_product_for_many_rows(monkeypatch):
 def test_rows_beyond_one_chunk_take_the_way_that_was_timed_faster(monkeypatch):
     """129 to 256 rows: the decode batch kernel (two chunks of rows per launch) or the library's product, by a
     timing per weight shape; both ways give the plain result, alone and as a pair launch."""
-    from pytorch_transformers_amd import ops
+    from pytorch_transformers_amd import ops, tuning
     from pytorch_transformers_amd.parts import Linear
 
     if ops.SPLITK_MAX_ROWS < 256:
@@ -148,7 +148,7 @@ def test_rows_beyond_one_chunk_take_the_way_that_was_timed_faster(monkeypatch):
         assert ops.splitk_row_limit(first.weight) in (128, 192, 256)  # measured, whichever
     ops.release_flush()
     for limit in (256, 128):
-        monkeypatch.setattr(ops, "splitk_row_limit", lambda *ws: limit)
+        monkeypatch.setattr(tuning, "splitk_row_limit", lambda *ws: limit)
         assert ops.gemm_splitk_ok(x, first.weight) == (limit == 256)
         _close(first(x), want1, 2e-2, f"alone, limit {limit}")
         both = Linear.pair(first, x, {}, second, x, {"act": "gelu"})
@@ -157,7 +157,7 @@ def test_rows_beyond_one_chunk_take_the_way_that_was_timed_faster(monkeypatch):
             _close(both[0], want1, 2e-2, "first of the pair")
             _close(both[1], want2, 2e-2, "second of the pair")
     # at 128 rows and below nothing is timed: the kernel takes them
-    monkeypatch.setattr(ops, "splitk_row_limit", lambda *ws: 1 / 0)
+    monkeypatch.setattr(tuning, "splitk_row_limit", lambda *ws: 1 / 0)
     assert ops.gemm_splitk_ok(x[:128].contiguous(), first.weight)
 
 
@@ -180,19 +180,19 @@ def test_library_product_over_ranges_of_k():
     key = (N, K, (M + 63) // 64)
     try:
         for S in (2, 4, 1):
-            ops._mm_ksplit[key] = S
+            ops.active().mm_ksplit[key] = S
             got = ops.library_mm_ksplit(x, lin.weight, lin.bias, "gelu", a1, a2)
             assert (got is None) == (S == 1)
             _close(lin(x, act="gelu", add1=a1, add2=a2), want, 2e-2, f"{S} ranges of K")
     finally:
-        ops._mm_ksplit.pop(key, None)
+        ops.active().mm_ksplit.pop(key, None)
     assert ops.library_mm_ksplit(x[:64], lin.weight) is None  # few rows go to the decode kernels
     lin(x, act="gelu", add1=a1, add2=a2)
-    assert ops.TUNE_LIVE or key not in ops._mm_ksplit  # nothing is timed unless asked
+    assert ops.TUNE_LIVE or key not in ops.active().mm_ksplit  # nothing is timed unless asked
     with ops.live_tuning():
         lin(x, act="gelu", add1=a1, add2=a2)  # timed, whichever way
     ops.release_flush()
-    assert ops._mm_ksplit.pop(key) in (1, 2, 4)
+    assert ops.active().mm_ksplit.pop(key) in (1, 2, 4)
 
 
 def test_positions():

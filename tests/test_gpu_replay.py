@@ -334,6 +334,59 @@ def test_steps_time_nothing_unless_asked_and_a_table_carries_the_choices(folders
     helpers.assert_close(tuned, before, 2e-2, "tuned against untuned logits")
 
 
+def test_a_configuration_that_no_kernel_takes_is_refused_before_a_weight_is_read(tmp_path):
+    """Heads of 512 elements (1,024 wide, two heads): the folder holds a configuration and no weights at all, and the
+    error is about the head size, from the part that has it; the same from a configuration alone."""
+    from pytorch_transformers_amd import AutoModelForCausalLM
+    from pytorch_transformers_amd.config import AutoConfig
+
+    raw = dict(TINY["C"], hidden_size=1024, num_attention_heads=2, ffn_hidden_size=64)
+    (tmp_path / "config.json").write_text(json.dumps(raw))
+    for dtype in ("bfloat16", "float32"):
+        with pytest.raises(ValueError, match=r"transformer\.h\.0\.self_attention: attention: head size 512 is outside 1\.\.256"):
+            AutoModelForCausalLM.from_pretrained(str(tmp_path), dtype=dtype)
+    with pytest.raises(ValueError, match="head size 512"):
+        AutoModelForCausalLM.from_config(AutoConfig.from_dict(raw))
+
+
+def test_two_models_in_one_process_keep_their_own_timed_choices(folders):
+    """A model's table is its own: timing the choices of one model, or loading a table into it, changes neither
+    another model's table nor its bits, however their steps interleave; a table file given to ``from_pretrained``
+    makes the choices of the model that wrote it."""
+    import json as _json
+
+    from pytorch_transformers_amd import AutoModelForCausalLM, tuning
+
+    first = AutoModelForCausalLM.from_pretrained(folders["C"], dtype="bfloat16")
+    second = AutoModelForCausalLM.from_pretrained(folders["C"], dtype="bfloat16")
+    prompt = list(range(600))
+
+    def logits(model):
+        cache = model.new_cache(1024, max_slots=1)
+        slot = cache.alloc()
+        out = model.step(cache, [slot], [prompt], "last").clone()
+        more = model.step(cache, [slot], [[5]], "last").clone()
+        return torch.cat([out, more])
+
+    plain_bits = logits(second)
+    assert torch.equal(logits(first), plain_bits)
+    table = first.tune(prompt_lens=(600,), batches=(4, 40))
+    assert table["pair_parts"] and first.tuning.pair_parts and not any(second.tuning.to_dict().values())
+    tuned_bits = logits(first)
+    assert tuning.active() is first.tuning
+    assert torch.equal(logits(second), plain_bits), "another model's timed choices changed this model's bits"
+    assert tuning.active() is second.tuning
+    assert torch.equal(logits(first), tuned_bits) and torch.equal(logits(second), plain_bits)
+    path = os.path.join(os.path.dirname(folders["C"]), "tuning_table.json")
+    with open(path, "w") as f:
+        _json.dump(table, f)
+    third = AutoModelForCausalLM.from_pretrained(folders["C"], dtype="bfloat16", tuning_table=path)
+    assert third.tuning.to_dict() == table
+    assert torch.equal(logits(third), tuned_bits) and torch.equal(logits(second), plain_bits)
+    with pytest.raises(ValueError, match="sections"):
+        second.tune(table={"pair_ranges": {}})
+
+
 def test_tune_times_whole_steps_with_each_cut_of_the_decode_attention(folders):
     """``tune(contexts=...)`` replays captured decode steps at those contexts once per candidate cut of the attention
     and leaves every bucket either at the rule's cut or at a candidate.  Decoding with every candidate fixed by hand
@@ -356,7 +409,7 @@ def test_tune_times_whole_steps_with_each_cut_of_the_decode_attention(folders):
             assert tuple(cut) in ops.decode_plan_candidates(tuple(int(v) for v in k.split(",")))[1:]
         assert ops.take_decode_keys() == [] and ops._flush is None
         cfg = model.config
-        key = ops._decode_key(1, cfg.num_attention_heads, cfg.kv_heads, cfg.head_dim, 700, 700)
+        key = ops.decode_key(1, cfg.num_attention_heads, cfg.kv_heads, cfg.head_dim, 700, 700)
         cuts = ops.decode_plan_candidates(key)
         assert any(c[2] > 1 for c in cuts)
         for cut in cuts:

@@ -1,5 +1,6 @@
 """The sampling kernel against the plain processors, and generation through the entry point (GPU)."""
 import math
+import os
 
 import pytest
 import torch
@@ -291,6 +292,143 @@ def test_banned_tokens_per_row(V):
             assert int(tok[r]) not in bans[r] and keep_got[int(tok[r])]
 
 
+@pytest.mark.parametrize("V", [40, 65024, 70001])
+def test_bias_forced_token_and_bonus_on_eos_per_row(V):
+    """Additive biases on a list of tokens per row (before the repetition penalty), a token forced in this step
+    (over bans that come before it, under bans that come after it), and the bonus on the EOS scores (after the
+    removal of invalid values): scores and choices equal the plain processors', greedy and drawn, by the short way
+    and the long way, and by the path for vocabularies beyond the bitmaps."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(V + 1)
+    R = 4
+    logits = torch.randn(R, V, generator=g) * 2
+    best = logits.argmax(-1).tolist()
+    eos = [2, V - 3]
+    logits[:, eos[0]] = logits[:, eos[0]].abs() + 0.5  # one EOS score above zero, one below: the bonus raises both
+    logits[:, eos[1]] = -logits[:, eos[1]].abs() - 0.5
+    biases = [[(best[0], -50.0), (5, 3.0)], [], [(V - 1, 60.0)] + [(t, -1.0) for t in range(10, 30)], [(best[3], 0.5)]]
+    hist = [[best[r], 5, V - 1] + [1] * 7 for r in range(R)]  # ten ids so far
+    off = [0]
+    for b in biases:
+        off.append(off[-1] + len(b))
+    kw_bias = dict(bias_tok=_dev([t for b in biases for t, _ in b], torch.int32),
+                   bias_val=_dev([v for b in biases for _, v in b]), bias_off=_dev(off, torch.int32))
+    kw_hist = dict(hist=_dev([t for h in hist for t in h], torch.int32), hist_off=_dev([0, 10, 20, 30, 40], torch.int32))
+    entries = [{(t,): v for t, v in b} for b in biases]
+    # biases and the penalty, greedy: every score
+    tok, scores = ops.sample(_dev(logits), do_sample=False, penalty=1.5, **kw_hist, **kw_bias)
+    for r in range(R):
+        want = P.process(logits[r], hist[r], do_sample=False, sequence_bias_=entries[r], repetition_penalty_=1.5)
+        torch.testing.assert_close(scores[r].cpu(), want, rtol=1e-6, atol=1e-6)
+        assert int(tok[r]) == int(want.argmax())
+    assert int(tok[0]) != best[0] and int(tok[2]) == V - 1, "the biases decide these rows"
+    # the bonus on EOS with invalid values removed before it, and with biases
+    m = 1.1 ** 7 - 1
+    tok, scores = ops.sample(_dev(logits), do_sample=False, eos=_dev(eos, torch.int32), decay=m, **kw_bias)
+    for r in range(R):
+        want = P.process(logits[r], hist[r], do_sample=False, sequence_bias_=entries[r], eos_ids_=eos,
+                         exponential_decay_=(3, 0, 1.1))  # three ids of a prompt, start index 0: 10 - 3 = 7 ids past it
+        torch.testing.assert_close(scores[r].cpu(), want, rtol=1e-6, atol=1e-6)
+        assert float(want[eos[0]]) > float(logits[r, eos[0]]) and float(want[eos[1]]) > float(logits[r, eos[1]])
+    with pytest.raises(ops.KernelError, match="EOS"):
+        ops.sample(_dev(logits), do_sample=False, decay=m)
+    # a forced token: everything else goes, whatever was banned or suppressed before; a ban that comes after it stays
+    forced = [eos[0], 7]
+    bans = [[7], [], [eos[0], 7], [3]]
+    boff = [0, 1, 1, 3, 4]
+    tok, scores = ops.sample(_dev(logits), do_sample=False, forced=_dev(forced, torch.int32), eos=_dev(eos, torch.int32),
+                             suppress=_dev([1, 0, 0, 1], torch.int32), ban=_dev([t for b in bans for t in b], torch.int32),
+                             ban_off=_dev(boff, torch.int32), **kw_bias)
+    for r in range(R):
+        want = P.suppress(P.forced_eos(logits[r], 4, 5, forced), bans[r])
+        assert torch.equal(scores[r].cpu(), want)
+    assert tok.tolist() == [eos[0], eos[0], 0, eos[0]]  # (row 2: both forced tokens are banned afterwards, nothing is left)
+    # drawn, with the other processors around them (top-k: the short way; top-p alone: the long way)
+    u = torch.rand(R, generator=g)
+    for kw in (dict(top_k=5), dict(top_k=0, top_p=0.9), dict(top_k=20, temperature=0.7, penalty=1.3)):
+        tok, scores = ops.sample(_dev(logits), do_sample=True, uniforms=_dev(u), temperature=kw.get("temperature", 1.0),
+                                 top_k=kw["top_k"], top_p=kw.get("top_p", 1.0), penalty=kw.get("penalty", 1.0),
+                                 eos=_dev(eos, torch.int32), decay=m, **kw_hist, **kw_bias)
+        for r in range(R):
+            want = P.process(logits[r], hist[r], do_sample=True, temperature_=kw.get("temperature", 1.0), top_k_=kw["top_k"],
+                             top_p_=kw.get("top_p", 1.0), repetition_penalty_=kw.get("penalty", 1.0),
+                             sequence_bias_=entries[r], eos_ids_=eos, exponential_decay_=(3, 0, 1.1))
+            keep_want, keep_got = want != float("-inf"), _finite_mask(scores[r])
+            assert int((keep_want != keep_got).sum()) <= (1 if "top_p" in kw else 0), (V, kw, r)
+            both = keep_want & keep_got
+            torch.testing.assert_close(scores[r].cpu()[both], want[both], rtol=1e-5, atol=1e-5)
+            assert keep_got[int(tok[r])]
+
+
+def test_generation_with_bias_forced_last_token_and_bonus_on_eos_equals_plain(folders):
+    """Greedy and sampled generation with ``sequence_bias`` (entries of one and of several tokens), ``forced_eos_token_id``
+    and ``exponential_decay_length_penalty`` against the plain loop, in a batch of unequal prompts of one length class
+    each (the reference counts lengths on the padded batch: one prompt a call keeps both sides on the same count),
+    with steps ahead of the host where nothing reads the tokens so far."""
+    from pytorch_transformers_amd import AutoModelForCausalLM, GenerationConfig
+    from pytorch_transformers_amd.sampling import philox_uniform
+
+    cfg, w = P.read_model(folders["A"])
+    g = torch.Generator().manual_seed(6)
+    prompts = [torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for n in (4, 9)]
+    model = AutoModelForCausalLM.from_pretrained(folders["A"], dtype="float32")
+    free = [p + P.generate(cfg, w, p, 12) for p in prompts]
+    for i, p in enumerate(prompts):
+        new = free[i][len(p):]
+        bias = [[[new[1]], -30.0], [new[3:5], -30.0], [[new[0], new[1], new[2]], 5.0]]
+        as_dict = {tuple(e[0]): e[1] for e in bias}
+        eos = next(t for t in range(cfg["vocab_size"]) if t not in free[i])  # a token that does not come by itself
+        # the bias alone: the tokens change where it says
+        want = p + P.generate(cfg, w, p, 12, sequence_bias_=as_dict)
+        got = model.generate([p], GenerationConfig(max_new_tokens=12, do_sample=False, eos_token_id=None, sequence_bias=bias))
+        assert got == [want] and want != free[i]
+        # a forced last token, with and without a bias on single tokens (which lets steps run ahead of the host)
+        for sb in (None, [[[new[1]], -30.0]]):
+            want = p + P.generate(cfg, w, p, 6, eos_ids=(eos,), forced_eos_ids=[eos],
+                                  sequence_bias_={tuple(e[0]): e[1] for e in sb} if sb else None)
+            got = model.generate([p], GenerationConfig(max_new_tokens=6, do_sample=False, eos_token_id=eos,
+                                                       forced_eos_token_id=eos, sequence_bias=sb))
+            assert got == [want] and want[-1] == eos and len(want) == len(p) + 6
+        # the bonus on EOS: the sequence ends earlier than without it, and where the plain loop ends
+        late = p + P.generate(cfg, w, p, 40, eos_ids=(eos,), no_repeat_ngram_size_=2)
+        want = p + P.generate(cfg, w, p, 40, eos_ids=(eos,), no_repeat_ngram_size_=2, exponential_decay_length_penalty=(2, 1.6))
+        got = model.generate([p], GenerationConfig(max_new_tokens=40, do_sample=False, eos_token_id=eos,
+                                                   no_repeat_ngram_size=2, exponential_decay_length_penalty=(2, 1.6)))
+        assert got == [want] and len(want) < len(late) and want[-1] == eos
+        # sampled, with all three, from the same uniform numbers
+        us = [philox_uniform(3, 0, s) for s in range(10)]
+        want = p + P.generate(cfg, w, p, 10, uniforms=us, temperature_=0.9, eos_ids=(eos,), forced_eos_ids=[eos],
+                              sequence_bias_=as_dict, exponential_decay_length_penalty=(1, 1.2))
+        got = model.generate([p], GenerationConfig(max_new_tokens=10, do_sample=True, temperature=0.9, top_k=0, seed=3,
+                                                   eos_token_id=eos, forced_eos_token_id=eos, sequence_bias=bias,
+                                                   exponential_decay_length_penalty=(1, 1.2)))[0]
+        _same_or_a_draw_on_a_boundary(cfg, w, got, want, len(p), us, 0.9)
+    with pytest.raises(ValueError, match="eos_token_id"):
+        model.generate([prompts[0]], GenerationConfig(max_new_tokens=3, eos_token_id=None, exponential_decay_length_penalty=(1, 1.2)))
+
+
+def test_sampled_generation_goes_on_from_kept_slots_with_its_random_stream(folders):
+    """Five sampled tokens at once equal three and then two more from kept slots when the second call starts each
+    sequence's random stream where the first one stopped (``rng_step_start``); started at 0 again, it would draw
+    with the first call's numbers."""
+    from pytorch_transformers_amd import AutoModelForCausalLM
+
+    model = AutoModelForCausalLM.from_pretrained(folders["A"], dtype="float32")
+    prompts = [[3, 1, 4, 1, 5], [9, 2], [6, 5, 3, 5, 8, 9, 7]]
+    kw = dict(do_sample=True, temperature=1.5, top_k=0, seed=11, eos_token_id=None)
+    at_once = model.generate(prompts, max_new_tokens=5, **kw)
+    first = model.generate(prompts, max_new_tokens=3, keep_slots=True, **kw)
+    assert first.rng_steps == [3, 3, 3]
+    again = model.generate(first.sequences, max_new_tokens=2, cache=first.cache, slots=first.slots, **kw)  # from draw 0
+    assert not first.cache.live_slots()
+    first = model.generate(prompts, max_new_tokens=3, keep_slots=True, **kw)
+    more = model.generate(first.sequences, max_new_tokens=2, cache=first.cache, slots=first.slots,
+                          rng_step_start=first.rng_steps, **kw)
+    assert more == at_once
+    assert again != at_once, "the stream started anew gives other tokens: the test sees the counter"
+    assert not first.cache.live_slots()
+
+
 def test_generation_without_repeated_ngrams_equals_plain(folders):
     """Greedy generation with no_repeat_ngram_size and bad_words_ids against the plain loop: a tiny random model
     repeats itself soon, so the option decides tokens."""
@@ -558,6 +696,89 @@ def test_command_line_as_a_program(folders, tmp_path):
     folder = write_random_model(str(tmp_path / "same"), AutoConfig.from_dict(raw), 3)
     cfg_c, w_c = P.read_model(folder)
     assert got == [[9, 8, 7, 6] + P.generate(cfg_c, w_c, [9, 8, 7, 6], 5, eos_ids=(eos_default,))]
+
+
+WORDS = ["[UNK]", "the", "cat", "sat", "on", "a", "mat", "dog", "ran", "to", "its", "house", "and", "then", "slept", "all",
+         "day", "long", "while", "it", "rained", "outside", "again", "today"]
+
+
+def _folder_with_a_tokenizer(tmp_path):
+    """A tiny model whose vocabulary is ``WORDS``, with a word-level ``tokenizer.json`` beside its weights (written
+    with the ``tokenizers`` package: words split at spaces, joined by spaces again)."""
+    from tokenizers import Tokenizer
+    from tokenizers.models import WordLevel
+    from tokenizers.pre_tokenizers import Whitespace
+
+    from tiny import write_config
+
+    folder = write_config(dict(TINY["C"], vocab_size=len(WORDS)), str(tmp_path), "words", seed=8, std=LIVELY_STD)
+    tok = Tokenizer(WordLevel({w: i for i, w in enumerate(WORDS)}, unk_token="[UNK]"))
+    tok.pre_tokenizer = Whitespace()
+    tok.save(os.path.join(folder, "tokenizer.json"))
+    return folder
+
+
+def test_text_through_the_command_line_and_the_pipeline(tmp_path):
+    """The text path of both entry points (examples/pytorch/text-generation/run_generation.py:365-441,
+    src/transformers/pipelines/text_generation.py:349-449): ``--prompt``, ``--prefix`` and ``--stop_token`` of the
+    program, text in and out of the pipeline, ``stop_strings`` and ``return_full_text``.  Under the text the ids are
+    the plain loop's."""
+    import subprocess
+    import sys
+
+    from pytorch_transformers_amd import pipeline
+
+    folder = _folder_with_a_tokenizer(tmp_path)
+    cfg, w = P.read_model(folder)
+    ids_of = lambda text: [WORDS.index(t) if t in WORDS else 0 for t in text.split()]
+    text_of = lambda ids: " ".join(WORDS[t] for t in ids)
+    eos = 11  # FalconConfig's default, "house" here
+    prompt, prefix = "cat sat on zebra", "the "
+    ids = ids_of(prefix + prompt)
+    assert ids == [1, 2, 3, 4, 0]  # a word the vocabulary lacks becomes [UNK]
+    new = P.generate(cfg, w, ids, 10, eos_ids=(eos,))
+    assert len(set(new)) > 4, "tokens that keep changing carry the comparison"
+    whole = text_of(ids + new)
+
+    def program(*argv):
+        root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+        p = subprocess.run([sys.executable, "-m", "pytorch_transformers_amd.run_generation", "--model_name_or_path", folder,
+                            "--dtype", "float32", *argv], cwd=root, capture_output=True, text=True, timeout=300)
+        assert p.returncode == 0, p.stderr[-3000:]
+        lines = [ln for ln in p.stdout.splitlines() if ln.strip()]
+        assert lines[0] == "=== GENERATED SEQUENCE 1 ===", p.stdout
+        return lines[1:]
+
+    assert program("--prompt", prompt, "--prefix", prefix, "--length", "10", "--greedy") == [whole]
+    stop = WORDS[new[3]]  # a word that is generated: the printed text is cut in front of its first occurrence
+    assert whole.find(stop) > 0
+    assert program("--prompt", prompt, "--prefix", prefix, "--length", "10", "--greedy", "--stop_token", stop) == \
+        [whole[:whole.find(stop)]]
+    # the prompt read from standard input when none is given (run_generation.py:365)
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    p = subprocess.run([sys.executable, "-m", "pytorch_transformers_amd.run_generation", "--model_name_or_path", folder,
+                        "--dtype", "float32", "--length", "4", "--greedy"], cwd=root, input=prefix + prompt + "\n",
+                       capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0 and text_of(ids + new[:4]) in p.stdout, p.stderr[-2000:]
+
+    pipe = pipeline("text-generation", model=folder, dtype="float32")
+    out = pipe(prefix + prompt, max_new_tokens=10, do_sample=False)
+    assert out == [{"generated_text": whole}]
+    assert pipe(prompt, prefix=prefix, max_new_tokens=10, do_sample=False, return_full_text=False) == \
+        [{"generated_text": text_of(new)}]
+    # a stop string of two words, completed by the fourth new token: that token is kept, nothing follows it
+    stop_string = text_of(new[2:4])
+    cut = next(k for k in range(1, len(new) + 1) if stop_string in text_of(new[:k]))
+    assert cut < len(new)
+    out = pipe([prefix + prompt, "the dog"], max_new_tokens=10, do_sample=False, stop_strings=[stop_string])
+    assert out[0] == [{"generated_text": text_of(ids + new[:cut])}]
+    other = P.generate(cfg, w, ids_of("the dog"), 10, eos_ids=(eos,))
+    cut2 = next((k for k in range(1, len(other) + 1) if stop_string in text_of(other[:k])), len(other))
+    assert out[1] == [{"generated_text": text_of(ids_of("the dog") + other[:cut2])}]
+    # token ids through the same pipeline stay ids
+    assert pipe([ids], max_new_tokens=3, do_sample=False)[0] == [{"generated_token_ids": ids + new[:3]}]
+    with pytest.raises(ValueError, match="tokenizer"):
+        pipeline("text-generation", model=pipe.model)("the cat", max_new_tokens=2)
 
 
 def test_generation_goes_on_from_kept_slots(folders):

@@ -530,6 +530,46 @@ def test_processors_on_the_references_vectors():
     assert torch.isinf(P.suppress(torch.zeros(6), [2, 4])).tolist() == [False, False, True, False, True, False]
 
 
+def test_bias_forced_token_and_bonus_on_eos_on_the_references_vectors():
+    """tests/generation/test_logits_process.py: :604-629 sequence bias, :766-791 forced last token, :820-855 the bonus
+    on EOS that grows with the length."""
+    entries = {(1,): 100.0, (4,): 100.0, (1, 0): -100.0, (0, 1, 2): -100.0, (1, 3, 1, 3): -100.0,
+               (1, 3, 1, 3, 1, 3): -100.0}
+    flat = torch.zeros(5)
+    assert P.sequence_bias(flat, [0, 1, 3, 1], entries).tolist() == [-100.0, 100.0, 0.0, -100.0, 100.0]
+    assert P.sequence_bias(flat, [0, 1, 0, 1], entries).tolist() == [-100.0, 100.0, -100.0, 0.0, 100.0]
+    assert flat.abs().sum() == 0  # inputs are not changed in place
+    # two entries that end in one token add up; a one-token entry adds to whatever else the token gets
+    both = {(3, 1): 1.5, (2, 3, 1): 2.0, (1,): 0.25}
+    assert P.sequence_bias(flat, [9, 2, 3], both).tolist() == [0, 3.75, 0, 0, 0]
+    # an entry longer than the ids so far never applies, although the ids end in the tokens before its last (:1122)
+    assert P.sequence_bias(flat, [2, 3], both).tolist() == [0, 1.75, 0, 0, 0]
+    assert not torch.isinf(P.no_bad_words(flat, [2, 3], [[2, 3, 1]])).any()
+    assert torch.isinf(P.no_bad_words(flat, [9, 2, 3], [[2, 3, 1]])).tolist() == [False, True, False, False, False]
+
+    uniform = torch.full((20,), 1.0 / 20)
+    forced = P.forced_eos(uniform, 4, 5, [0])
+    assert float(forced[0]) == 0 and torch.isneginf(forced[1:]).all()
+    assert torch.equal(P.forced_eos(uniform, 3, 5, [0]), uniform)
+
+    # a prompt of 2 ids, start index 5, factor 1.1: nothing up to 7 ids, then |score| * (1.1 ** (ids - 7) - 1) on top
+    assert torch.equal(P.exponential_decay(uniform, 2, 2, 5, 1.1, [0]), uniform)
+    assert torch.equal(P.exponential_decay(uniform, 7, 2, 5, 1.1, [0]), uniform)
+    after = P.exponential_decay(uniform, 20, 2, 5, 1.1, [0])
+    assert float(after[0]) == pytest.approx(0.05 * 1.1 ** 13) and torch.equal(after[1:], uniform[1:])
+    negative = P.exponential_decay(-uniform, 20, 2, 5, 1.1, [0])
+    assert float(negative[0]) == pytest.approx(-0.05 + 0.05 * (1.1 ** 13 - 1)) and float(negative[0]) > -0.05
+
+    # their places in the order (generation/utils.py:898-1005): the bias before the penalty, the forced token over
+    # everything before it, the bonus after it
+    s = torch.tensor([2.0, 1.0, -1.0])
+    out = P.process(s, [0], do_sample=False, sequence_bias_={(0,): -4.0}, repetition_penalty_=2.0)
+    assert out.tolist() == [-4.0, 1.0, -1.0]  # (2 - 4) * 2; the penalty first would have given 2 / 2 - 4 = -3
+    out = P.process(s, [0, 1], do_sample=False, forced_eos_=(3, [2]), exponential_decay_=(1, 0, 2.0), eos_ids_=[2],
+                    suppress_ids=[2])
+    assert out.tolist() == [float("-inf"), float("-inf"), 0.0]  # the forced token undoes the suppression; |0| gains nothing
+
+
 def test_processing_order_and_pick():
     """Penalty before temperature, top-k before top-p (generation/utils.py:926-1097); argmax and
     inverse-CDF choice."""

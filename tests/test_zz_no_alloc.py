@@ -28,11 +28,19 @@ def _both_ways(lib, M, N, K, seed, with_tail_terms):
     rc = lib.pta_gemm_splitk_bf16(_ptr(want), _ptr(part), _ptr(x), _ptr(w), _ptr(bias), _ptr(add1), None, M, N, K, act, 0,
                                   0, 0, 0, 0, 1, stream)
     assert rc == 0, lib.pta_last_error().decode()
-    before = torch.cuda.memory_allocated()
+    # once to warm up (the first call on a device looks the array's address up, and the code object is loaded), then
+    # the call whose memory is watched: torch's own counter, and the driver's count of free device memory, which
+    # also sees an allocation that does not go through torch
     rc = lib.pta_gemm_splitk_bf16_static(_ptr(got), _ptr(x), _ptr(w), _ptr(bias), _ptr(add1), None, M, N, K, act, 0, stream)
     assert rc == 0, lib.pta_last_error().decode()
-    assert torch.cuda.memory_allocated() == before
     torch.cuda.synchronize()
+    got.fill_(float("nan"))
+    torch.cuda.synchronize()
+    before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
+    rc = lib.pta_gemm_splitk_bf16_static(_ptr(got), _ptr(x), _ptr(w), _ptr(bias), _ptr(add1), None, M, N, K, act, 0, stream)
+    assert rc == 0, lib.pta_last_error().decode()
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() == before and torch.cuda.mem_get_info()[0] == free_before
     ref = x.float() @ w.float().t()
     return got, want, ref, parts
 
