@@ -10,8 +10,8 @@ prefill of 2,048 tokens under ``prefill``, the decode step's HBM roofline under 
 ``points`` (flat):
 
 * ``decode_b1`` / ``decode_b8`` / ``decode_b64``: tokens a second over the range of contexts that the
-  configuration names (1,024 -> 2,048), as the mean step time of runs at three contexts (1,030, 1,536, 2,040;
-  ``decode_b64_ctx1536`` and so on are the three), each with ``..._frac``, the fraction of the HBM roofline;
+  configuration names, every decode step from 1,024 tokens to 2,048 in one run; ``decode_b64_ctx1568`` and so on
+  are short runs around three contexts of that range; each with ``..._frac``, the fraction of the HBM roofline;
 * ``decode_b8_untuned``: the same step with the built-in choices between kernels, before ``model.tune()`` has
   timed any (what a process runs that neither tunes nor loads a tuning table);
 * ``falcon11b_...`` / ``falcon40b_...``: decode at batch 8 and 64 and one batch of whole requests of unequal
@@ -141,7 +141,10 @@ def run_decode(model, sampler_cls, gen_cfg, batch, prompt_len, steps, warmup, se
     return dt, mean_ctx, median
 
 
-RANGE_CONTEXTS = (1030, 1536, 2040)  # the start, the middle and the end of decoding from 1,024 towards 2,048 tokens
+# Near the start, the middle and the end of decoding from 1,024 towards 2,048 tokens, each clear of the lengths at
+# which a captured decode step is exchanged for the next one (multiples of 512): a run of a few steps across such
+# a length would time the capture, which decoding meets twice in a thousand steps.
+RANGE_CONTEXTS = (1056, 1568, 2016)
 
 
 def decode_over_range(model, sampler_cls, gen_cfg, cfg, elem, batch, steps=16, warmup=4, contexts=RANGE_CONTEXTS):
@@ -161,6 +164,17 @@ def decode_over_range(model, sampler_cls, gen_cfg, cfg, elem, batch, steps=16, w
     out[f"decode_b{batch}"] = round(batch / mean_ms * 1e3, 2)
     out[f"decode_b{batch}_frac"] = round(sum(f * m for f, m in zip(frac_all, ms_all)) / sum(ms_all), 4)
     return out
+
+
+def decode_whole_range(model, sampler_cls, gen_cfg, cfg, elem, batch, first=1024, last=2048):
+    """Every decode step from a context of ``first`` tokens to one of ``last``, as one run (the captured steps that
+    are exchanged on the way included): tokens a second and the fraction of the HBM roofline over the run."""
+    steps = last - first - 1
+    dt, mean_ctx, _ = run_decode(model, sampler_cls, gen_cfg, batch, 0, steps, 1, start_ctx=first)
+    ms = dt / steps * 1e3
+    gbs = (weight_bytes(cfg, elem) + batch * mean_ctx * kv_bytes_per_token(cfg, elem)) / (ms * 1e-3) / 1e9
+    return {f"decode_b{batch}": round(batch / ms * 1e3, 2), f"decode_b{batch}_frac": round(gbs / HBM_PEAK_GBS, 4),
+            f"decode_b{batch}_steps": steps}
 
 
 def run_prefill(model, T, reps=3, seed=1):
@@ -372,7 +386,6 @@ def main():
         print(json.dumps(mixed_record(model, ops, cfg, args.sizes, args.dtype, elem)))
         return 0
     if args.extra_record:
-        ends = (RANGE_CONTEXTS[0], RANGE_CONTEXTS[-1])
         model.tune(prompt_lens=(), batches=(8, 64), contexts=RANGE_CONTEXTS)
         rec = {}
         for b in (8, 64):
@@ -431,6 +444,8 @@ def main():
                           "frac": round(flops / pt / (PEAK_TFLOPS[args.dtype] * 1e12), 4)}
         for b in sorted({1, args.batch, 64}):
             points.update(decode_over_range(model, Sampler, gen_cfg, cfg, elem, b))
+            # ... and what the metric names: every step from prompts of 1,024 tokens to 2,048, in place of the mean of three
+            points.update(decode_whole_range(model, Sampler, gen_cfg, cfg, elem, b, 1024, 2048))
         out["points"] = points
         if args.dtype == "bf16":
             out["kernels"] = {

@@ -5,20 +5,21 @@
 // batch.  This is the engine's 32-bit path and the fallback for sizes the MFMA
 // kernels refuse.
 //
-// score[j] = q . k_j / sqrt(d) + alibi_j, keys 0 .. pos (or the last `window` of them)
+// score[j] = q . k_j / sqrt(d) + bias_j, keys 0 .. pos (or the last `window` of them)
 // (src/transformers/models/falcon/modeling_falcon.py:371-386, :407-422).
-// alibi_j = bf16(bf16(slope_h) * bf16(j)) / sqrt(d): the reference forms slope x position in
-// bfloat16 even in a 32-bit model (:196-198) and divides by sqrt(d) when it folds the bias into
-// the mask (:1078-1085).  `slopes` holds the slopes already rounded to bfloat16.
+// The bias is data (PtaScoreBias, pta_kernels.h).  The reference's ALiBi is bf16(bf16(slope_h) * bf16(j)) / sqrt(d):
+// it forms slope x position in bfloat16 even in a 32-bit model (:196-198) and divides by sqrt(d) when it folds the
+// bias into the mask (:1078-1085); `slopes` then holds the slopes already rounded to bfloat16, and the scale 1 / sqrt(d).
 #include "common.h"
 #include "pta_kernels.h"
+#include "score_bias.h"
 
 template <typename T>
 __global__ void attn_generic_kernel(T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ k_pool,
                                     const T* __restrict__ v_pool, const int* __restrict__ block_table,
                                     int bt_stride, const int* __restrict__ token_seq,
-                                    const int* __restrict__ token_pos, const float* __restrict__ slopes, int alibi_exact, int nh,
-                                    int nkv, int d, float scale, float sqrt_d, int window) {
+                                    const int* __restrict__ token_pos, const float* __restrict__ slopes, int bias_mode, float bias_scale,
+                                    int nh, int nkv, int d, float scale, int window) {
     __shared__ float q_s[256];
     __shared__ float p_s[PTA_PAGE];
     const int m = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
@@ -47,7 +48,9 @@ __global__ void attn_generic_kernel(T* __restrict__ out, const T* __restrict__ q
             float dot = 0.f;
             for (int i = 0; i < d; ++i) dot += q_s[i] * Io<T>::ld(kr + i);
             s = dot * scale;
-            if (slopes) s += (alibi_exact ? slope * (float)j : round_to_bf16(slope * round_to_bf16((float)j))) / sqrt_d;
+            if (slopes)  // slope x key position as the reference rounds it (0), exact (1), or x the distance from the query (2)
+                s += (bias_mode == 0 ? round_to_bf16(slope * round_to_bf16((float)j))
+                                     : slope * (float)(bias_mode == 2 ? j - (nkeys - 1) : j)) * bias_scale;
         }
         const float m_new = fmaxf(m_run, wave_max(s));
         const float p = valid ? expf(s - m_new) : 0.f;
@@ -90,8 +93,12 @@ extern "C" int pta_attention_sizes_ok(int nh, int nkv, int d, int rotated) {
 
 extern "C" int pta_attn_generic(void* out, const void* q, const void* k_pool, const void* v_pool,
                                 const int* block_table, int bt_stride, const int* token_seq, const int* token_pos,
-                                const float* slopes, int alibi_exact, int M, int nh, int nkv, int d, float scale, int window, int dtype,
+                                const PtaScoreBias* score_bias, int M, int nh, int nkv, int d, float scale, int window, int dtype,
                                 void* stream) {
+    int bias_mode = 0;
+    if (pta_score_bias_mode("attn_generic", score_bias, &bias_mode)) return 1;
+    const float* slopes = score_bias ? score_bias->slopes : nullptr;
+    const float bias_scale = slopes ? score_bias->scale : 0.f;
     PTA_REQUIRE(M > 0 && nh > 0 && nkv > 0, "attn_generic: sizes must be positive (M=%d nh=%d nkv=%d)", M, nh, nkv);
     PTA_REQUIRE(nh % nkv == 0, "attn_generic: heads (%d) must be a multiple of kv heads (%d)", nh, nkv);
     PTA_REQUIRE(d > 0 && d <= 256, "attn_generic: head size %d is outside 1..256", d);
@@ -99,15 +106,14 @@ extern "C" int pta_attn_generic(void* out, const void* q, const void* k_pool, co
     PTA_REQUIRE(window >= 0, "attn_generic: window must be 0 (none) or positive, got %d", window);
     hipStream_t s = (hipStream_t)stream;
     dim3 grid(M, nh);
-    const float sqrt_d = sqrtf((float)d);
     if (dtype == PTA_F32)
         hipLaunchKernelGGL(attn_generic_kernel<float>, grid, dim3(PTA_WAVE), 0, s, (float*)out, (const float*)q,
                            (const float*)k_pool, (const float*)v_pool, block_table, bt_stride, token_seq, token_pos,
-                           slopes, alibi_exact, nh, nkv, d, scale, sqrt_d, window);
+                           slopes, bias_mode, bias_scale, nh, nkv, d, scale, window);
     else if (dtype == PTA_BF16)
         hipLaunchKernelGGL(attn_generic_kernel<bf16_t>, grid, dim3(PTA_WAVE), 0, s, (bf16_t*)out, (const bf16_t*)q,
                            (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_table, bt_stride, token_seq,
-                           token_pos, slopes, alibi_exact, nh, nkv, d, scale, sqrt_d, window);
+                           token_pos, slopes, bias_mode, bias_scale, nh, nkv, d, scale, window);
     else
         return pta_fail("attn_generic: unknown dtype %d", dtype);
     return pta_check_launch("attn_generic");

@@ -27,6 +27,7 @@
 // (src/transformers/models/falcon/modeling_falcon.py:371-386, :407-422, :196-198, :1078-1085).
 #include "common.h"
 #include "pta_kernels.h"
+#include "score_bias.h"
 
 #include <stdlib.h>
 
@@ -111,7 +112,7 @@ __global__ __launch_bounds__(64 * W * KS, OCC) void attn_mfma_kernel(
     bf16_t* __restrict__ out, float* __restrict__ po, float* __restrict__ pm, float* __restrict__ pl,
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
     const int* __restrict__ block_table, int bt_stride, const int* __restrict__ cu_tokens,
-    const int* __restrict__ seq_start, const float* __restrict__ slopes, int alibi_exact, int nh, int nkv, float scale,
+    const int* __restrict__ seq_start, const float* __restrict__ slopes, int bias_mode, int nh, int nkv, float scale,
     float alibi_mul,
     int split_size, int n_splits, int window_arg, int paired) {
     constexpr int D = DT * 16;
@@ -237,7 +238,10 @@ __global__ __launch_bounds__(64 * W * KS, OCC) void attn_mfma_kernel(
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                     const int key = kb + 8 * gq + j;  // j = 4*tt + e
-                    const float bias = alibi_exact ? slope[ct] * (float)key : round_to_bf16(slope[ct] * round_to_bf16((float)key));
+                    // the slope times the key's position, rounded as the reference rounds it (0) or exact (1), or
+                    // times the key's distance from the query (2)
+                    const float bias = bias_mode == 0 ? round_to_bf16(slope[ct] * round_to_bf16((float)key))
+                                                      : slope[ct] * (float)(bias_mode == 2 ? key - qpos[ct] : key);
                     sacc[j >> 2][ct][j & 3] = sacc[j >> 2][ct][j & 3] * scale + bias * alibi_mul;
                 }
             }
@@ -621,7 +625,7 @@ struct AttnLaunch {
     bf16_t* out; float *po, *pm, *pl;
     const bf16_t *q, *k_pool, *v_pool;
     const int* block_table; int bt_stride;
-    const int *cu_tokens, *seq_start; const float* slopes; int alibi_exact;
+    const int *cu_tokens, *seq_start; const float* slopes; int bias_mode; float bias_scale;
     int n_seqs, max_new, nh, nkv; float scale;
     int split_size, n_splits, window;
     int paired;  // workgroups take two column groups each, a late one and the early one that mirrors it
@@ -654,8 +658,8 @@ static void launch_attn(const AttnLaunch& a) {
         }
     }
     hipLaunchKernelGGL(kern, grid, dim3(64 * W * KS), lds, a.s, a.out, a.po, a.pm, a.pl, a.q, a.k_pool, a.v_pool,
-                       a.block_table, a.bt_stride, a.cu_tokens, a.seq_start, a.slopes, a.alibi_exact, a.nh, a.nkv,
-                       a.scale * PTA_LOG2E, PTA_LOG2E / sqrtf((float)(DT * 16)), a.split_size, a.n_splits, a.window, paired);
+                       a.block_table, a.bt_stride, a.cu_tokens, a.seq_start, a.slopes, a.bias_mode, a.nh, a.nkv,
+                       a.scale * PTA_LOG2E, PTA_LOG2E * a.bias_scale, a.split_size, a.n_splits, a.window, paired);
 }
 
 // column tiles (of sixteen query heads of one KV head) that one wave of a decode launch holds at most:
@@ -740,11 +744,15 @@ extern "C" int pta_attn_decode_waves_ok(int d, int tiles, int waves) {
 }
 
 extern "C" int pta_attn_mfma(void* out, const void* q, const void* k_pool, const void* v_pool, const int* block_table,
-                             int bt_stride, const int* cu_tokens, const int* seq_start, const float* slopes, int alibi_exact,
+                             int bt_stride, const int* cu_tokens, const int* seq_start, const PtaScoreBias* score_bias,
                              int n_seqs, int max_new, int M, int nh, int nkv, int d, float scale, int split_size, int n_splits,
                              float* po, float* pm, float* pl, int window, int decode_tiles, int decode_waves,
                              int prompt_wide, void* stream) {
     PTA_REQUIRE(n_seqs > 0 && max_new > 0 && M > 0 && nh > 0 && nkv > 0, "attn_mfma: sizes must be positive");
+    int bias_mode = 0;
+    if (pta_score_bias_mode("attn_mfma", score_bias, &bias_mode)) return 1;
+    const float* slopes = score_bias ? score_bias->slopes : nullptr;
+    const float bias_scale = slopes ? score_bias->scale : 0.f;
     PTA_REQUIRE(nh % nkv == 0, "attn_mfma: heads (%d) must be a multiple of kv heads (%d)", nh, nkv);
     PTA_REQUIRE(pta_attn_mfma_supported(d), "attn_mfma: head size %d is not built (16..128 in steps of 16, or 256)", d);
     PTA_REQUIRE(n_splits >= 1 && n_splits <= 1024, "attn_mfma: n_splits must be 1..1024, got %d", n_splits);
@@ -800,7 +808,7 @@ extern "C" int pta_attn_mfma(void* out, const void* q, const void* k_pool, const
                 "attn_mfma: %d waves on the keys of a workgroup with %d column tiles are not built for head size %d "
                 "(one wave, or four or eight with up to two tiles)", decode_waves, dct, d);
     const AttnLaunch a{(bf16_t*)out, po, pm, pl, (const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool,
-                       block_table, bt_stride, cu_tokens, seq_start, slopes, alibi_exact, n_seqs, max_new, nh, nkv, scale,
+                       block_table, bt_stride, cu_tokens, seq_start, slopes, bias_mode, bias_scale, n_seqs, max_new, nh, nkv, scale,
                        split_size, n_splits, window, paired, narrow ? decode_waves : 1, s};
 #define PTA_ATTN_CASE(DT_)                                        \
     case DT_:                                                     \

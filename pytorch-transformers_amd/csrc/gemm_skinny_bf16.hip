@@ -107,9 +107,11 @@ struct SkinnyProblem {
 };
 
 // With a QkvTail (qkv_tail.h) the first product's rows are not stored: they are split into heads, rotated and written
-// as queries and into the cache pages.  The rotation pairs feature i of a head with i + d/2, so a workgroup takes
-// sixteen features of a head's lower half as its first row tile and their partners as its second.
-template <int MT, int RT, int U, typename OutT, bool TAIL = false>
+// as queries and into the cache pages.  The rotation works on pairs of a head's elements, so a workgroup takes the
+// first elements of sixteen pairs as its first row tile and their partners as its second (TAIL 1: whole heads in
+// half-split pairs, or no rotation: pair p is elements p and p + d/2, and four pairs in a row are stored as eight
+// bytes; TAIL 2: any rotation that qkv_tail_pair_elements describes, stored element by element).
+template <int MT, int RT, int U, typename OutT, int TAIL = 0>
 __global__ __launch_bounds__(512) void gemm_skinny_kernel(SkinnyProblem pa, SkinnyProblem pb, int M, int K,
                                                           int rot_stride, QkvTail tail) {
     static_assert(!TAIL || (RT == 2 && MT == 1 && sizeof(OutT) == 2), "the query_key_value tail: two row tiles, sixteen rows of x");
@@ -129,11 +131,19 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(SkinnyProblem pa, Skin
     const int n0 = (int)((long)j * N / blocks), n1 = (int)((long)(j + 1) * N / blocks);
     const bf16_t* wrow[RT];
     const bool tailed = TAIL && !second;
-    // with the tail: workgroup j has features s16*16 .. +15 of segment seg (a head's q, k or v) and their partners
+    // with the tail: workgroup j has pairs s16*16 .. +15 of segment seg (a head's q, k or v)
     const int per_seg = TAIL ? tail.d / 32 : 1, seg = j / per_seg, s16 = j % per_seg;
+    int pair_e[2] = {0, 0};  // the two elements of this lane's pair
+    if (TAIL == 1) {
+        pair_e[0] = s16 * 16 + r;
+        pair_e[1] = pair_e[0] + (tail.d >> 1);
+    } else if (TAIL == 2) {
+        bool rotated;
+        qkv_tail_pair_elements(tail.rot, tail.d, s16 * 16 + r, pair_e[0], pair_e[1], rotated);
+    }
 #pragma unroll
     for (int t = 0; t < RT; ++t) {
-        const int row = tailed ? seg * tail.d + t * (tail.d >> 1) + s16 * 16 + r : min(n0 + t * 16 + r, n1 - 1);
+        const int row = tailed ? seg * tail.d + pair_e[t & 1] : min(n0 + t * 16 + r, n1 - 1);
         wrow[t] = W + (long)row * K;
     }
     // x through a buffer descriptor whose bounds are the M real rows (0x00020000: 32-bit raw data format)
@@ -183,6 +193,11 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(SkinnyProblem pa, Skin
                 const int m = ln & 15;
                 if (m >= M) continue;
                 const int d = tail.d, half = d >> 1, i0 = s16 * 16 + (ln >> 4) * 4;
+                if constexpr (TAIL == 2) {  // pairs i0 .. i0+3, wherever their elements lie
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) qkv_tail_pair(tail, bias, m, seg, i0 + e, round_to_bf16(lo[e]), round_to_bf16(hi[e]));
+                    continue;
+                }
                 int kind, head;  // 0 query, 1 key, 2 value
                 qkv_tail_segment(tail, seg, kind, head);
                 if (kind != 0 && !tail.write_cache) continue;
@@ -197,12 +212,12 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(SkinnyProblem pa, Skin
                         b[e] = round_to_bf16(b[e] + bias[seg * d + half + i0 + e]);
                     }
                 }
-                if (tail.inv_freq && kind != 2) {
+                if (tail.rot.inv_freq && kind != 2) {
                     const float* freq = qkv_tail_freq(tail, m);
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         const float ang = (float)pos * freq[i0 + e];
-                        const float c = cosf(ang) * tail.cs_scale, sn = sinf(ang) * tail.cs_scale;
+                        const float c = cosf(ang) * tail.rot.cs_scale, sn = sinf(ang) * tail.rot.cs_scale;
                         const float x0 = a[e], x1 = b[e];
                         a[e] = x0 * c - x1 * sn;
                         b[e] = x1 * c + x0 * sn;
@@ -363,8 +378,7 @@ extern "C" int pta_gemm_skinny_bf16(void* y, const void* x, const void* W, const
 // cache pages of their sequences, as pta_qkv_rope_cache would have left them.  Up to 16 rows, head sizes that are
 // multiples of 32.  The second product is y2 = act2(x2 . W2^T + bias2) as in the plain pair.
 extern "C" int pta_gemm_skinny_pair_qkv_bf16(void* q_out, const void* x1, const void* W1, const float* bias1,
-                                             const float* inv_freq, int inv_freq_ld, float cs_scale,
-                                             const int* token_pos,
+                                             const PtaRotation* rotation, const int* token_pos,
                                              const int* token_seq, const int* block_table, int bt_stride, void* k_pool,
                                              void* v_pool, int nh, int nkv, int d, int layout, int write_cache, void* y2,
                                              const void* x2, const void* W2, const float* bias2, int N2, int act2, int M,
@@ -379,13 +393,13 @@ extern "C" int pta_gemm_skinny_pair_qkv_bf16(void* q_out, const void* x1, const 
     PTA_REQUIRE(layout != PTA_QKV_TAIL || nkv == 1, "gemm_skinny_pair_qkv_bf16: the tail layout has one kv head, got %d", nkv);
     PTA_REQUIRE(layout != PTA_QKV_INTERLEAVED || nkv == nh, "gemm_skinny_pair_qkv_bf16: the interleaved layout needs kv heads == heads");
     PTA_REQUIRE(token_pos, "gemm_skinny_pair_qkv_bf16: null token positions");
-    PTA_REQUIRE(inv_freq_ld == 0 || (inv_freq && token_seq && inv_freq_ld >= d / 2),
-                "gemm_skinny_pair_qkv_bf16: a frequency table per sequence needs the tokens' sequences and rows of %d", d / 2);
+    const PtaRotation rot = pta_rotation_of(rotation);
+    if (pta_check_rotation("gemm_skinny_pair_qkv_bf16", rot, d, token_seq)) return 1;
     PTA_REQUIRE(!write_cache || (k_pool && v_pool && block_table && token_seq), "gemm_skinny_pair_qkv_bf16: null cache pointer");
     PTA_REQUIRE((((uintptr_t)q_out | (uintptr_t)k_pool) % 8) == 0, "gemm_skinny_pair_qkv_bf16: outputs must be 8-byte aligned");
     SkinnyProblem a{nullptr, (const bf16_t*)x1, (const bf16_t*)W1, bias1, nullptr, nullptr, N1, PTA_ACT_NONE, 0};
     SkinnyProblem b{y2, (const bf16_t*)x2, (const bf16_t*)W2, bias2, nullptr, nullptr, N2, in_kernel(act2) ? act2 : 0, 0};
-    const QkvTail tail{(bf16_t*)q_out, inv_freq, inv_freq_ld, cs_scale, token_pos, token_seq, block_table, bt_stride, (bf16_t*)k_pool,
+    const QkvTail tail{(bf16_t*)q_out, rot, token_pos, token_seq, block_table, bt_stride, (bf16_t*)k_pool,
                        (bf16_t*)v_pool, nh, nkv, d, layout, write_cache};
     // the first product's workgroups are bound to heads; the second one's fill the launch up to a whole number per unit
     a.blocks = (nh + 2 * nkv) * (d / 32);
@@ -395,8 +409,12 @@ extern "C" int pta_gemm_skinny_pair_qkv_bf16(void* q_out, const void* x1, const 
     const int S = pick_split(N1 + N2);
     static const int rot_env = getenv("PTA_SKINNY_ROT") ? atoi(getenv("PTA_SKINNY_ROT")) : -1;
     const int rot_stride = rot_env >= 0 ? rot_env : (K % 2048 == 0 ? 5 : 0);
-    hipLaunchKernelGGL((gemm_skinny_kernel<1, 2, 2, bf16_t, true>), dim3(a.blocks + b.blocks), dim3(S * 64),
-                       (size_t)S * 2 * 64 * sizeof(f32x4_t), (hipStream_t)stream, a, b, M, K, rot_stride, tail);
+    if (qkv_tail_plain_pairs(rot, d))
+        hipLaunchKernelGGL((gemm_skinny_kernel<1, 2, 2, bf16_t, 1>), dim3(a.blocks + b.blocks), dim3(S * 64),
+                           (size_t)S * 2 * 64 * sizeof(f32x4_t), (hipStream_t)stream, a, b, M, K, rot_stride, tail);
+    else
+        hipLaunchKernelGGL((gemm_skinny_kernel<1, 2, 2, bf16_t, 2>), dim3(a.blocks + b.blocks), dim3(S * 64),
+                           (size_t)S * 2 * 64 * sizeof(f32x4_t), (hipStream_t)stream, a, b, M, K, rot_stride, tail);
     if (pta_check_launch("gemm_skinny_pair_qkv_bf16")) return 1;
     if (!in_kernel(act2)) return pta_epilogue(y2, N2, nullptr, nullptr, nullptr, M, N2, act2, PTA_BF16, stream);
     return 0;

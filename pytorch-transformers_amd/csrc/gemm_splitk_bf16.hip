@@ -286,8 +286,8 @@ extern "C" int pta_gemm_reduce_parts(void* y, const float* part, const float* bi
 }
 
 // The reduction of a pair launch whose first product is a fused query_key_value projection: a thread adds the
-// partial sums of one rotation pair (feature i of a segment's lower half and i + d/2) and takes it to its end
-// (qkv_tail.h); the second product as in gemm_splitk_reduce2_kernel.
+// partial sums of one pair of a segment's elements (the two that are rotated together, or two that pass;
+// qkv_tail_pair_elements) and takes it to its end (qkv_tail.h); the second product as in gemm_splitk_reduce2_kernel.
 __global__ __launch_bounds__(256) void gemm_splitk_reduce2_qkv_kernel(QkvTail tail, const float* __restrict__ part1,
                                                                       const float* __restrict__ bias1, long MN1, int N1,
                                                                       int P1, bf16_t* __restrict__ y2,
@@ -299,7 +299,10 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce2_qkv_kernel(QkvTail ta
     if (o < pairs) {
         const int half = tail.d >> 1, per_row = N1 >> 1;
         const int m = (int)(o / per_row), p = (int)(o % per_row), seg = p / half, i = p % half;
-        const long lo = (long)m * N1 + (long)seg * tail.d + i, hi = lo + half;
+        int ea, eb;
+        bool rotated;
+        qkv_tail_pair_elements(tail.rot, tail.d, i, ea, eb, rotated);
+        const long lo = (long)m * N1 + (long)seg * tail.d + ea, hi = (long)m * N1 + (long)seg * tail.d + eb;
         float a = part1[lo], b = part1[hi];
         for (int q = 1; q < P1; ++q) { a += part1[(long)q * MN1 + lo]; b += part1[(long)q * MN1 + hi]; }
         qkv_tail_pair(tail, bias1, m, seg, i, round_to_bf16(a), round_to_bf16(b));
@@ -672,13 +675,12 @@ extern "C" int pta_gemm_splitk_pair_reduced_bf16(void* y1, float* part1, const v
 }
 
 // what the launches that take fused query_key_value rows to their end ask of their arguments
-static int check_qkv_tail(const char* what, const void* q_out, const float* inv_freq, int inv_freq_ld,
+static int check_qkv_tail(const char* what, const void* q_out, const PtaRotation& rot,
                           const int* token_pos, const int* token_seq,
                           const int* block_table, const void* k_pool, const void* v_pool, int nh, int nkv, int d,
                           int layout, int write_cache) {
-    PTA_REQUIRE(inv_freq_ld == 0 || (inv_freq && token_seq && inv_freq_ld >= d / 2),
-                "%s: a frequency table per sequence needs the tokens' sequences and rows of %d", what, d / 2);
     PTA_REQUIRE(nh > 0 && nkv > 0 && d > 0 && nh % nkv == 0, "%s: heads %d, kv heads %d, head size %d", what, nh, nkv, d);
+    if (pta_check_rotation(what, rot, d, token_seq)) return 1;
     PTA_REQUIRE(d % 2 == 0, "%s: head size %d must be even", what, d);
     PTA_REQUIRE(layout >= 0 && layout <= 2, "%s: unknown layout %d", what, layout);
     PTA_REQUIRE(layout != PTA_QKV_TAIL || nkv == 1, "%s: the tail layout has one kv head, got %d", what, nkv);
@@ -691,14 +693,14 @@ static int check_qkv_tail(const char* what, const void* q_out, const float* inv_
 // The same pair with the first product a fused query_key_value projection taken to its end: queries rotated in
 // q_out [M, heads, d], keys and values in the cache pages (as pta_qkv_rope_cache leaves them); even head sizes.
 extern "C" int pta_gemm_splitk_pair_reduced_qkv_bf16(void* q_out, float* part1, const void* x1, const void* W1,
-                                                     const float* bias1, int K1, const float* inv_freq, int inv_freq_ld,
-                                                     float cs_scale,
+                                                     const float* bias1, int K1, const PtaRotation* rotation,
                                                      const int* token_pos, const int* token_seq, const int* block_table,
                                                      int bt_stride, void* k_pool, void* v_pool, int nh, int nkv, int d,
                                                      int layout, int write_cache, void* y2, float* part2, const void* x2,
                                                      const void* W2, const float* bias2, int N2, int K2, int act2, int M,
                                                      void* stream) {
-    if (check_qkv_tail("gemm_splitk_pair_reduced_qkv_bf16", q_out, inv_freq, inv_freq_ld, token_pos, token_seq, block_table, k_pool, v_pool, nh,
+    const PtaRotation rot = pta_rotation_of(rotation);
+    if (check_qkv_tail("gemm_splitk_pair_reduced_qkv_bf16", q_out, rot, token_pos, token_seq, block_table, k_pool, v_pool, nh,
                        nkv, d, layout, write_cache))
         return 1;
     PTA_REQUIRE(y2, "gemm_splitk_pair_reduced_qkv_bf16: null pointer");
@@ -709,7 +711,7 @@ extern "C" int pta_gemm_splitk_pair_reduced_qkv_bf16(void* q_out, float* part1, 
     const long MN1 = (long)M * N1, MN2 = (long)M * N2;
     int P1, P2;
     pick_pair_parts_rows(N1, K1, N2, K2, M, &P1, &P2);
-    const QkvTail tail{(bf16_t*)q_out, inv_freq, inv_freq_ld, cs_scale, token_pos, token_seq, block_table, bt_stride, (bf16_t*)k_pool,
+    const QkvTail tail{(bf16_t*)q_out, rot, token_pos, token_seq, block_table, bt_stride, (bf16_t*)k_pool,
                        (bf16_t*)v_pool, nh, nkv, d, layout, write_cache};
     hipLaunchKernelGGL(gemm_splitk_reduce2_qkv_kernel, dim3((unsigned)((MN1 / 2 + MN2 + 255) / 256)), dim3(256), 0,
                        (hipStream_t)stream, tail, part1, bias1, MN1, N1, P1, (bf16_t*)y2, part2, bias2, MN2, N2, P2, act2);
@@ -719,12 +721,12 @@ extern "C" int pta_gemm_splitk_pair_reduced_qkv_bf16(void* q_out, float* part1, 
 // A fused query_key_value projection on its own (17 to 256 rows), taken to its end by the launch that adds its
 // partial sums: part [pta_gemm_splitk_parts(N, K, 0, 0), M, N] is the workspace, N = (nh + 2 nkv) d.
 extern "C" int pta_gemm_splitk_reduced_qkv_bf16(void* q_out, float* part, const void* x, const void* W,
-                                                const float* bias, int K, const float* inv_freq, int inv_freq_ld,
-                                                float cs_scale,
+                                                const float* bias, int K, const PtaRotation* rotation,
                                                 const int* token_pos, const int* token_seq, const int* block_table,
                                                 int bt_stride, void* k_pool, void* v_pool, int nh, int nkv, int d,
                                                 int layout, int write_cache, int M, void* stream) {
-    if (check_qkv_tail("gemm_splitk_reduced_qkv_bf16", q_out, inv_freq, inv_freq_ld, token_pos, token_seq, block_table, k_pool, v_pool, nh, nkv,
+    const PtaRotation rot = pta_rotation_of(rotation);
+    if (check_qkv_tail("gemm_splitk_reduced_qkv_bf16", q_out, rot, token_pos, token_seq, block_table, k_pool, v_pool, nh, nkv,
                        d, layout, write_cache))
         return 1;
     PTA_REQUIRE(part, "gemm_splitk_reduced_qkv_bf16: null workspace");
@@ -733,7 +735,7 @@ extern "C" int pta_gemm_splitk_reduced_qkv_bf16(void* q_out, float* part, const 
                                         0, 0, stream);
     if (rc) return rc;
     const long MN = (long)M * N;
-    const QkvTail tail{(bf16_t*)q_out, inv_freq, inv_freq_ld, cs_scale, token_pos, token_seq, block_table, bt_stride, (bf16_t*)k_pool,
+    const QkvTail tail{(bf16_t*)q_out, rot, token_pos, token_seq, block_table, bt_stride, (bf16_t*)k_pool,
                        (bf16_t*)v_pool, nh, nkv, d, layout, write_cache};
     hipLaunchKernelGGL(gemm_splitk_reduce2_qkv_kernel, dim3((unsigned)((MN / 2 + 255) / 256)), dim3(256), 0,
                        (hipStream_t)stream, tail, part, bias, MN, N, pta_gemm_splitk_parts(N, K, 0, 0), (bf16_t*)nullptr,

@@ -14,7 +14,7 @@
 
 #include <stdint.h>
 
-#define PTA_ABI_VERSION 8
+#define PTA_ABI_VERSION 9
 
 #ifdef __cplusplus
 extern "C" {
@@ -46,11 +46,35 @@ int pta_layernorm_sum_rows_min(void);
 int pta_epilogue(void* y, int ld_y, const float* bias, const void* add1, const void* add2, int M, int N, int act,
                  int dtype, void* stream);
 
-// split fused qkv rows, add bias, rotate q and k (inv_freq null: no rotation), write q and append k, v.
-// inv_freq_ld (here and in the three launches below that rotate): 0 for one table [d/2] for all tokens, else a
-// table per sequence of the step, [sequences, inv_freq_ld], found through token_seq
-int pta_qkv_rope_cache(void* q_out, const void* fused, int fused_ld, const float* bias, const float* inv_freq,
-                       int inv_freq_ld, float cs_scale,
+// How queries and keys are rotated by position, as data (here and in the three launches below that rotate).  The
+// first rotary_dim elements of a head are rotated, the rest pass; element pairs are (i, i + rotary_dim / 2)
+// (PTA_PAIR_HALF) or (2i, 2i + 1) (PTA_PAIR_INTERLEAVED), each by the angle position * inv_freq[i], cosines and
+// sines multiplied by cs_scale.  inv_freq_ld: 0 for one table [rotary_dim / 2] for all tokens, else a table per
+// sequence of the step, [sequences, inv_freq_ld], found through token_seq.  A null struct or null inv_freq: no rotation.
+enum PtaPairing { PTA_PAIR_HALF = 0, PTA_PAIR_INTERLEAVED = 1 };
+typedef struct PtaRotation {
+    const float* inv_freq;
+    int inv_freq_ld;
+    float cs_scale;
+    int rotary_dim;
+    int pairing;
+} PtaRotation;
+
+// A bias on attention scores, as data: slopes[head] * x * scale is added to the score of a query and a key, x being
+// the key's position (PTA_BIAS_KEY) or the key's position minus the query's (PTA_BIAS_DISTANCE: 0 for a token's own
+// key, negative before it); softmax makes the two equal up to rounding.  bf16 = 1 (PTA_BIAS_KEY only): the position
+// and the product are rounded to bfloat16 before the scale, as the reference rounds them
+// (src/transformers/models/falcon/modeling_falcon.py:196-198).  A null struct or null slopes: no bias.
+enum PtaBiasOf { PTA_BIAS_KEY = 0, PTA_BIAS_DISTANCE = 1 };
+typedef struct PtaScoreBias {
+    const float* slopes;
+    int of;
+    int bf16;
+    float scale;
+} PtaScoreBias;
+
+// split fused qkv rows, add bias, rotate q and k, write q and append k, v.
+int pta_qkv_rope_cache(void* q_out, const void* fused, int fused_ld, const float* bias, const PtaRotation* rotation,
                        const int* token_pos, const int* token_seq, const int* block_table, int bt_stride,
                        void* k_pool, void* v_pool, int M, int nh, int nkv, int d, int layout, int write_cache,
                        int dtype, void* stream);
@@ -61,11 +85,9 @@ int pta_attention_sizes_ok(int nh, int nkv, int d, int rotated);
 
 // causal attention of M tokens over their sequences' cache, 32-bit arithmetic
 // window: 0, or the number of last positions a token sees (itself included)
-// slopes (null: none): a bias slope[head] * key position / sqrt(d) on the scores; with alibi_exact = 0 the position
-// and the product are rounded to bfloat16 first, as the reference forms them, and the slopes given are expected
-// rounded too; with 1 nothing is rounded
+// score_bias (null: none): see PtaScoreBias above; with bf16 = 1 the slopes given are expected rounded to bfloat16 too
 int pta_attn_generic(void* out, const void* q, const void* k_pool, const void* v_pool, const int* block_table,
-                     int bt_stride, const int* token_seq, const int* token_pos, const float* slopes, int alibi_exact,
+                     int bt_stride, const int* token_seq, const int* token_pos, const PtaScoreBias* score_bias,
                      int M, int nh,
                      int nkv, int d, float scale, int window, int dtype, void* stream);
 
@@ -88,7 +110,7 @@ int pta_attn_decode_shared_ok(int d, int heads_per_kv_head);
 // prompt_wide (max_new > 1, head sizes up to 64): 1 workgroups of eight waves, 0 of four, -1 eight where the launch
 // still has four workgroups and more for every compute unit.
 int pta_attn_mfma(void* out, const void* q, const void* k_pool, const void* v_pool, const int* block_table,
-                  int bt_stride, const int* cu_tokens, const int* seq_start, const float* slopes, int alibi_exact,
+                  int bt_stride, const int* cu_tokens, const int* seq_start, const PtaScoreBias* score_bias,
                   int n_seqs, int max_new, int M, int nh, int nkv, int d, float scale, int split_size, int n_splits, float* po,
                   float* pm, float* pl, int window, int decode_tiles, int decode_waves, int prompt_wide, void* stream);
 
@@ -110,7 +132,7 @@ int pta_gemm_skinny_pair_bf16(void* y1, const void* x1, const void* W1, const fl
 // are split, rotated and written as queries [M, heads, d] and into the cache pages, as pta_qkv_rope_cache leaves
 // them; head sizes that are multiples of 32
 int pta_gemm_skinny_pair_qkv_bf16(void* q_out, const void* x1, const void* W1, const float* bias1,
-                                  const float* inv_freq, int inv_freq_ld, float cs_scale, const int* token_pos,
+                                  const PtaRotation* rotation, const int* token_pos,
                                   const int* token_seq,
                                   const int* block_table, int bt_stride, void* k_pool, void* v_pool, int nh, int nkv,
                                   int d, int layout, int write_cache, void* y2, const void* x2, const void* W2,
@@ -133,7 +155,7 @@ int pta_gemm_splitk_pair_parts(int N1, int K1, int N2, int K2, int M, int* parts
 // the pair run to the end with the first product a fused query_key_value projection (N1 = (nh + 2 nkv) d rows of
 // W1): queries rotated in q_out [M, nh, d], keys and values in the cache pages, as pta_qkv_rope_cache leaves them
 int pta_gemm_splitk_pair_reduced_qkv_bf16(void* q_out, float* part1, const void* x1, const void* W1, const float* bias1,
-                                          int K1, const float* inv_freq, int inv_freq_ld, float cs_scale,
+                                          int K1, const PtaRotation* rotation,
                                           const int* token_pos,
                                           const int* token_seq, const int* block_table, int bt_stride, void* k_pool,
                                           void* v_pool, int nh, int nkv, int d, int layout, int write_cache, void* y2,
@@ -141,7 +163,7 @@ int pta_gemm_splitk_pair_reduced_qkv_bf16(void* q_out, float* part1, const void*
                                           int act2, int M, void* stream);
 // such a projection on its own: part [pta_gemm_splitk_parts(N, K, 0, 0), M, N] is the workspace
 int pta_gemm_splitk_reduced_qkv_bf16(void* q_out, float* part, const void* x, const void* W, const float* bias, int K,
-                                     const float* inv_freq, int inv_freq_ld, float cs_scale, const int* token_pos,
+                                     const PtaRotation* rotation, const int* token_pos,
                                      const int* token_seq,
                                      const int* block_table, int bt_stride, void* k_pool, void* v_pool, int nh, int nkv,
                                      int d, int layout, int write_cache, int M, void* stream);

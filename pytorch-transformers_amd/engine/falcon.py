@@ -7,6 +7,8 @@ and forward (:599-612, :630-666); see ``config.falcon.FalconConfig.norm_scheme``
 """
 from __future__ import annotations
 
+import math
+
 from ..config.falcon import NORMS_DUAL, NORMS_SEQUENTIAL, FalconConfig
 from ..config.registry import register
 from ..parts import (AlibiPositions, AttentionMixer, DenseFeedForward, Embedding, LayerNorm, OutputHead,
@@ -46,7 +48,9 @@ def build_falcon(cfg: FalconConfig) -> ModelSpec:
     H, L, eps = cfg.hidden_size, cfg.num_hidden_layers, cfg.layer_norm_epsilon
     if cfg.alibi:
         # ``alibi_bf16_compat`` is this library's own key (default true: the reference's rounding of the bias)
-        positions = AlibiPositions(cfg.num_attention_heads, bf16_compat=bool(cfg.extra.get("alibi_bf16_compat", True)))
+        # (the bias is divided by the root of the head size when it is folded into the mask, modeling_falcon.py:1081)
+        positions = AlibiPositions(cfg.num_attention_heads, bf16_compat=bool(cfg.extra.get("alibi_bf16_compat", True)),
+                                   scale=1.0 / math.sqrt(cfg.head_dim))
     else:
         positions = rotary_positions(cfg)
     blocks = []

@@ -24,7 +24,18 @@ QKV_LAYOUT_CODES = {"grouped": 0, "tail": 1, "interleaved": 2}
 ACT_CODES = {None: 0, "none": 0, "linear": 0, "gelu": 1, "gelu_python": 1, "gelu_new": 2, "gelu_pytorch_tanh": 2,
              "gelu_fast": 2, "gelu_accurate": 2, "quick_gelu": 3, "relu": 4, "relu2": 5, "relu6": 6, "silu": 7, "swish": 7,
              "sigmoid": 8, "tanh": 9, "leaky_relu": 10, "mish": 11, "gelu_10": 12, "laplace": 13}
-ABI_VERSION = 8
+ABI_VERSION = 9
+PAIRING_CODES = {"half": 0, "interleaved": 1}  # PtaPairing: elements (i, i + rotary_dim / 2) or (2i, 2i + 1)
+BIAS_OF_CODES = {"key": 0, "distance": 1}  # PtaBiasOf: the slope times the key's position, or times key - query position
+
+
+class _PtaRotation(ctypes.Structure):
+    _fields_ = [("inv_freq", ctypes.c_void_p), ("inv_freq_ld", ctypes.c_int), ("cs_scale", ctypes.c_float),
+                ("rotary_dim", ctypes.c_int), ("pairing", ctypes.c_int)]
+
+
+class _PtaScoreBias(ctypes.Structure):
+    _fields_ = [("slopes", ctypes.c_void_p), ("of", ctypes.c_int), ("bf16", ctypes.c_int), ("scale", ctypes.c_float)]
 
 _lib = None
 _lock = threading.Lock()
@@ -144,7 +155,7 @@ def _entry_cost(name: str, a) -> tuple:
     if name == "pta_gemm_skinny_pair_bf16":
         return both(gemm(a[12], a[4], a[13]), gemm(a[12], a[10], a[13]))
     if name == "pta_gemm_skinny_pair_qkv_bf16":
-        return both(gemm(a[24], (a[13] + 2 * a[14]) * a[15], a[25]), gemm(a[24], a[22], a[25]))
+        return both(gemm(a[22], (a[11] + 2 * a[12]) * a[13], a[23]), gemm(a[22], a[20], a[23]))
     if name == "pta_gemm_splitk_bf16":
         return gemm(a[7], a[8], a[9])
     if name == "pta_gemm_splitk_pair_bf16":
@@ -152,9 +163,9 @@ def _entry_cost(name: str, a) -> tuple:
     if name == "pta_gemm_splitk_pair_reduced_bf16":
         return both(gemm(a[16], a[5], a[6]), gemm(a[16], a[13], a[14]))
     if name == "pta_gemm_splitk_pair_reduced_qkv_bf16":
-        return both(gemm(a[28], (a[15] + 2 * a[16]) * a[17], a[5]), gemm(a[28], a[25], a[26]))
+        return both(gemm(a[26], (a[13] + 2 * a[14]) * a[15], a[5]), gemm(a[26], a[23], a[24]))
     if name == "pta_gemm_splitk_reduced_qkv_bf16":
-        return gemm(a[20], (a[15] + 2 * a[16]) * a[17], a[5])
+        return gemm(a[18], (a[13] + 2 * a[14]) * a[15], a[5])
     if name == "pta_gemm_f32":
         return gemm(a[6], a[7], a[8], 4)
     if name == "pta_layernorm_sum":
@@ -270,17 +281,60 @@ def epilogue_(y: torch.Tensor, bias=None, act=None, add1=None, add2=None) -> tor
     return y
 
 
-def _freq_ld(inv_freq, d: int, n_seqs: Optional[int] = None) -> int:
-    """0 for one frequency table [d/2] for all tokens; for a table per sequence of the step, [sequences, d/2],
-    the distance between its rows."""
+def _rotation_arg(inv_freq, cs_scale: float, d: int, n_seqs: Optional[int] = None, rotary_dim: Optional[int] = None,
+                  pairing: str = "half"):
+    """The rotation of queries and keys as the kernels take it (a ``PtaRotation`` by reference; None: no rotation).
+    ``inv_freq`` is one table ``[rotary_dim / 2]`` for all tokens or one per sequence of the step, ``[sequences,
+    rotary_dim / 2]``; the first ``rotary_dim`` elements of a head (default: all of them) are rotated in pairs
+    ``(i, i + rotary_dim / 2)`` (``"half"``) or ``(2i, 2i + 1)`` (``"interleaved"``)."""
     if inv_freq is None:
-        return 0
+        return None
+    r = int(d if rotary_dim is None else rotary_dim)
+    problem = rotation_problem(d, rotary_dim, pairing)
+    if problem is not None:
+        raise KernelError(problem)
     _need(inv_freq, "inv_freq", torch.float32)
-    if inv_freq.dim() == 1 and inv_freq.shape[0] == d // 2:
-        return 0
-    if inv_freq.dim() == 2 and inv_freq.shape[1] == d // 2 and (n_seqs is None or inv_freq.shape[0] == n_seqs):
-        return d // 2
-    raise KernelError(f"inv_freq must be [{d // 2}] or [sequences, {d // 2}], got {tuple(inv_freq.shape)}")
+    if inv_freq.dim() == 1 and inv_freq.shape[0] == r // 2:
+        ld = 0
+    elif inv_freq.dim() == 2 and inv_freq.shape[1] == r // 2 and (n_seqs is None or inv_freq.shape[0] == n_seqs):
+        ld = r // 2
+    else:
+        raise KernelError(f"inv_freq must be [{r // 2}] or [sequences, {r // 2}], got {tuple(inv_freq.shape)}")
+    return ctypes.byref(_PtaRotation(inv_freq.data_ptr(), ld, float(cs_scale), r, PAIRING_CODES[pairing]))
+
+
+def rotation_problem(d: int, rotary_dim: Optional[int] = None, pairing: str = "half") -> Optional[str]:
+    """None if the launches that rotate take this arrangement, else why not (for refusing a model early)."""
+    r = int(d if rotary_dim is None else rotary_dim)
+    if pairing not in PAIRING_CODES:
+        return f"a rotation with pairing {pairing!r} is not built; built: {sorted(PAIRING_CODES)}"
+    if r < 2 or r % 2 or r > d:
+        return f"rotary_dim must be even, from 2 up to the head size {d}; got {r}"
+    return None
+
+
+def score_bias_problem(bias_of: str, bf16: bool) -> Optional[str]:
+    """None if the attention kernels form this bias on scores, else why not."""
+    if bias_of not in BIAS_OF_CODES:
+        return (f"a score bias of {bias_of!r} is not built; built: slopes per head times {sorted(BIAS_OF_CODES)} "
+                "(the key's position, or its distance from the query)")
+    if bf16 and bias_of != "key":
+        return "rounding to bfloat16 as the reference rounds is built for slopes times the key's position only"
+    return None
+
+
+def _score_bias_arg(slopes, nh: int, bias_of: str = "key", bias_bf16: bool = True, bias_scale: float = 1.0):
+    """A bias on attention scores as the kernels take it (a ``PtaScoreBias`` by reference; None: no bias):
+    ``slopes[head] * x * bias_scale`` with x the key's position (``"key"``; ``bias_bf16``: position and product
+    rounded to bfloat16 as the reference rounds them) or the key's position minus the query's (``"distance"``)."""
+    if slopes is None:
+        return None
+    problem = score_bias_problem(bias_of, False)
+    if problem is not None:
+        raise KernelError(problem)
+    _need(slopes, "slopes", torch.float32, (nh,))
+    return ctypes.byref(_PtaScoreBias(slopes.data_ptr(), BIAS_OF_CODES[bias_of], int(bool(bias_bf16) and bias_of == "key"),
+                                      float(bias_scale)))
 
 
 def rope_dynamic_table(seq_start: torch.Tensor, cu_tokens: torch.Tensor, d: int, theta: float, factor: float,
@@ -298,9 +352,10 @@ def rope_dynamic_table(seq_start: torch.Tensor, cu_tokens: torch.Tensor, d: int,
 
 
 def qkv_rope_cache(fused: torch.Tensor, bias, inv_freq, cs_scale: float, token_pos, token_seq, block_table,
-                   k_pool, v_pool, nh: int, nkv: int, d: int, layout: str, write_cache: bool = True) -> torch.Tensor:
+                   k_pool, v_pool, nh: int, nkv: int, d: int, layout: str, write_cache: bool = True,
+                   rotary_dim: Optional[int] = None, pairing: str = "half") -> torch.Tensor:
     """Queries [M, nh, d] from the fused rows (which may lie apart); keys and values go to the cache pages.
-    ``inv_freq`` is one table [d/2], or one per sequence of the step, [sequences, d/2]."""
+    ``inv_freq``, ``rotary_dim`` and ``pairing`` say how queries and keys are rotated (``_rotation_arg``)."""
     M = fused.shape[0]
     _need_rows(fused, "fused", None, (M, (nh + 2 * nkv) * d))
     dt = fused.dtype
@@ -311,11 +366,10 @@ def qkv_rope_cache(fused: torch.Tensor, bias, inv_freq, cs_scale: float, token_p
     _need(block_table, "block_table", torch.int32)
     if block_table.dim() != 2:
         raise KernelError("block_table must be [sequences, pages]")
-    freq_ld = _freq_ld(inv_freq, d, block_table.shape[0])
+    rot = _rotation_arg(inv_freq, cs_scale, d, block_table.shape[0], rotary_dim, pairing)
     _need_pools(k_pool, v_pool, dt, nkv, d)
     q = torch.empty((M, nh, d), dtype=dt, device=fused.device)
-    _call("pta_qkv_rope_cache", _ptr(q), _ptr(fused), int(fused.stride(0)), _ptr(bias), _ptr(inv_freq), freq_ld,
-          ctypes.c_float(cs_scale),
+    _call("pta_qkv_rope_cache", _ptr(q), _ptr(fused), int(fused.stride(0)), _ptr(bias), rot,
           _ptr(token_pos), _ptr(token_seq), _ptr(block_table), block_table.shape[1], _ptr(k_pool), _ptr(v_pool), M,
           nh, nkv, d, QKV_LAYOUT_CODES[layout], int(write_cache), dtype_code(dt), _stream())
     return q
@@ -331,9 +385,11 @@ def attention_sizes_problem(nh: int, nkv: int, d: int, rotated: bool) -> Optiona
 
 
 def attn_generic(q: torch.Tensor, k_pool, v_pool, block_table, token_seq, token_pos, slopes, scale: float,
-                 window: int = 0, alibi_exact: bool = False):
+                 window: int = 0, alibi_exact: bool = False, bias_of: str = "key", bias_scale: Optional[float] = None):
     """Causal attention of every token over its sequence's cache (the last ``window`` positions of it, itself
-    included, if ``window`` > 0); out [M, nh*d]."""
+    included, if ``window`` > 0); out [M, nh*d].  ``slopes`` (None: no bias), ``bias_of``, ``alibi_exact`` (no
+    rounding to bfloat16) and ``bias_scale`` (None: 1 / sqrt(head size), as the reference folds its bias into the
+    mask) describe a bias on the scores (``_score_bias_arg``)."""
     _need(q, "q")
     M, nh, d = q.shape
     nkv = k_pool.shape[1]
@@ -341,11 +397,10 @@ def attn_generic(q: torch.Tensor, k_pool, v_pool, block_table, token_seq, token_
     _need(block_table, "block_table", torch.int32)
     _need(token_seq, "token_seq", torch.int32, (M,))
     _need(token_pos, "token_pos", torch.int32, (M,))
-    if slopes is not None:
-        _need(slopes, "slopes", torch.float32, (nh,))
+    bias = _score_bias_arg(slopes, nh, bias_of, not alibi_exact, d ** -0.5 if bias_scale is None else bias_scale)
     out = torch.empty((M, nh * d), dtype=q.dtype, device=q.device)
     _call("pta_attn_generic", _ptr(out), _ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(block_table),
-          block_table.shape[1], _ptr(token_seq), _ptr(token_pos), _ptr(slopes), int(bool(alibi_exact)), M, nh, nkv, d,
+          block_table.shape[1], _ptr(token_seq), _ptr(token_pos), bias, M, nh, nkv, d,
           ctypes.c_float(scale), int(window), dtype_code(q.dtype), _stream())
     return out
 
@@ -392,7 +447,7 @@ def attn_decode_shared_ok(head_dim: int, heads_per_kv_head: int) -> bool:
 def attn_mfma(q: torch.Tensor, k_pool, v_pool, block_table, cu_tokens, seq_start, slopes, scale: float, *,
               max_new: int, n_splits: int = 1, split_size: int = ATTN_SPLIT_KEYS, window: int = 0,
               decode_tiles: int = 0, decode_waves: int = 1, alibi_exact: bool = False,
-              prompt_wide: Optional[bool] = None) -> torch.Tensor:
+              prompt_wide: Optional[bool] = None, bias_of: str = "key", bias_scale: Optional[float] = None) -> torch.Tensor:
     """Causal attention of a step's tokens over the cache on the matrix cores; out [M, nh*d].
 
     ``max_new`` bounds the new tokens of any sequence of the step; with ``n_splits > 1`` the keys
@@ -401,7 +456,8 @@ def attn_mfma(q: torch.Tensor, k_pool, v_pool, block_table, cu_tokens, seq_start
     (0: as many as the head size allows).  ``decode_waves``: waves of a workgroup that divide its keys among
     them, or ``SHARED_KEYS``: the heads of a KV head on the waves of one workgroup, which share its keys through
     LDS (``attn_decode_shared_ok``).  ``prompt_wide``: workgroups of eight waves (True) or four (False) for prompts
-    with heads up to 64 (None: eight where the launch has workgroups enough)."""
+    with heads up to 64 (None: eight where the launch has workgroups enough).  ``slopes``, ``alibi_exact``,
+    ``bias_of`` and ``bias_scale``: the bias on the scores, as in ``attn_generic``."""
     _need(q, "q", torch.bfloat16)
     M, nh, d = q.shape
     nkv = k_pool.shape[1]
@@ -410,8 +466,7 @@ def attn_mfma(q: torch.Tensor, k_pool, v_pool, block_table, cu_tokens, seq_start
     n_seqs = block_table.shape[0]
     _need(cu_tokens, "cu_tokens", torch.int32, (n_seqs + 1,))
     _need(seq_start, "seq_start", torch.int32, (n_seqs,))
-    if slopes is not None:
-        _need(slopes, "slopes", torch.float32, (nh,))
+    bias = _score_bias_arg(slopes, nh, bias_of, not alibi_exact, d ** -0.5 if bias_scale is None else bias_scale)
     out = torch.empty((M, nh * d), dtype=q.dtype, device=q.device)
     po = pm = pl = None
     if n_splits > 1:
@@ -419,7 +474,7 @@ def attn_mfma(q: torch.Tensor, k_pool, v_pool, block_table, cu_tokens, seq_start
         pm = torch.empty((M, nh, n_splits), dtype=torch.float32, device=q.device)
         pl = torch.empty((M, nh, n_splits), dtype=torch.float32, device=q.device)
     _call("pta_attn_mfma", _ptr(out), _ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(block_table), block_table.shape[1],
-          _ptr(cu_tokens), _ptr(seq_start), _ptr(slopes), int(bool(alibi_exact)), n_seqs, int(max_new), M, nh, nkv, d,
+          _ptr(cu_tokens), _ptr(seq_start), bias, n_seqs, int(max_new), M, nh, nkv, d,
           ctypes.c_float(scale),
           int(split_size), int(n_splits), _ptr(po), _ptr(pm), _ptr(pl), int(window), int(decode_tiles), int(decode_waves),
           ATTN_FORCE_WIDE if prompt_wide is None else int(bool(prompt_wide)), _stream())
@@ -428,7 +483,7 @@ def attn_mfma(q: torch.Tensor, k_pool, v_pool, block_table, cu_tokens, seq_start
 
 
 def attention(q: torch.Tensor, k_pool, v_pool, block_table, ctx, slopes, scale: float, window: int = 0,
-              alibi_exact: bool = False) -> torch.Tensor:
+              alibi_exact: bool = False, bias_of: str = "key", bias_scale: Optional[float] = None) -> torch.Tensor:
     """Attention of a step's tokens over the cache: picks the kernel for the step's shape and type.
 
     bfloat16 with a head size the matrix-core kernel is built for: that kernel, with the context
@@ -444,8 +499,10 @@ def attention(q: torch.Tensor, k_pool, v_pool, block_table, ctx, slopes, scale: 
             n_splits = (ctx.max_len + size - 1) // size
         return attn_mfma(q, k_pool, v_pool, block_table, ctx.cu_tokens, ctx.seq_start, slopes, scale,
                          max_new=max(ctx.new_tokens), n_splits=n_splits, split_size=size, window=window,
-                         decode_tiles=tiles, decode_waves=waves, alibi_exact=alibi_exact)
-    return attn_generic(q, k_pool, v_pool, block_table, ctx.token_seq, ctx.token_pos, slopes, scale, window, alibi_exact)
+                         decode_tiles=tiles, decode_waves=waves, alibi_exact=alibi_exact, bias_of=bias_of,
+                         bias_scale=bias_scale)
+    return attn_generic(q, k_pool, v_pool, block_table, ctx.token_seq, ctx.token_pos, slopes, scale, window, alibi_exact,
+                        bias_of, bias_scale)
 
 
 def sample(logits: torch.Tensor, *, do_sample: bool, temperature: float = 1.0, top_k: int = 0, top_p: float = 1.0,
@@ -613,7 +670,8 @@ QKV_TAIL = os.environ.get("PTA_QKV_TAIL", "1") != "0"
 
 def gemm_skinny_pair_qkv(x1: torch.Tensor, w_qkv: torch.Tensor, bias_qkv, inv_freq, cs_scale: float, token_pos,
                          token_seq, block_table, k_pool, v_pool, nh: int, nkv: int, d: int, layout: str,
-                         write_cache: bool, x2: torch.Tensor, w2: torch.Tensor, bias2=None, act2=None):
+                         write_cache: bool, x2: torch.Tensor, w2: torch.Tensor, bias2=None, act2=None,
+                         rotary_dim: Optional[int] = None, pairing: str = "half"):
     """One launch for a decode step's two input products, the first a fused query_key_value projection taken to
     its end: returns (queries [M, nh, d] rotated, act2(x2 @ w2.T + bias2)); keys and values are in the cache pages,
     as ``qkv_rope_cache`` would have left them."""
@@ -633,12 +691,11 @@ def gemm_skinny_pair_qkv(x1: torch.Tensor, w_qkv: torch.Tensor, bias_qkv, inv_fr
     _need(block_table, "block_table", torch.int32)
     if block_table.dim() != 2:
         raise KernelError("block_table must be [sequences, pages]")
-    freq_ld = _freq_ld(inv_freq, d, block_table.shape[0])
+    rot = _rotation_arg(inv_freq, cs_scale, d, block_table.shape[0], rotary_dim, pairing)
     _need_pools(k_pool, v_pool, torch.bfloat16, nkv, d)
     q = torch.empty((M, nh, d), dtype=torch.bfloat16, device=x1.device)
     y2 = torch.empty((M, N2), dtype=torch.bfloat16, device=x1.device)
-    _call("pta_gemm_skinny_pair_qkv_bf16", _ptr(q), _ptr(x1), _ptr(w_qkv), _ptr(bias_qkv), _ptr(inv_freq), freq_ld,
-          ctypes.c_float(cs_scale), _ptr(token_pos), _ptr(token_seq), _ptr(block_table), block_table.shape[1], _ptr(k_pool),
+    _call("pta_gemm_skinny_pair_qkv_bf16", _ptr(q), _ptr(x1), _ptr(w_qkv), _ptr(bias_qkv), rot, _ptr(token_pos), _ptr(token_seq), _ptr(block_table), block_table.shape[1], _ptr(k_pool),
           _ptr(v_pool), nh, nkv, d, QKV_LAYOUT_CODES[layout], int(write_cache), _ptr(y2), _ptr(x2), _ptr(w2), _ptr(bias2),
           N2, ACT_CODES[act2], M, K, _stream())
     return q, y2
@@ -752,7 +809,8 @@ def gemm_splitk_pair_bf16(x1: torch.Tensor, w1: torch.Tensor, x2: torch.Tensor, 
 
 def gemm_splitk_pair_qkv(x1: torch.Tensor, w_qkv: torch.Tensor, bias_qkv, inv_freq, cs_scale: float, token_pos,
                          token_seq, block_table, k_pool, v_pool, nh: int, nkv: int, d: int, layout: str,
-                         write_cache: bool, x2: torch.Tensor, w2: torch.Tensor, bias2=None, act2=None):
+                         write_cache: bool, x2: torch.Tensor, w2: torch.Tensor, bias2=None, act2=None,
+                         rotary_dim: Optional[int] = None, pairing: str = "half"):
     """The pair launch of a decode batch (17 to 256 rows) with its first product a fused query_key_value projection
     taken to its end by the launch that adds the partial sums: returns (queries [M, nh, d] rotated,
     act2(x2 @ w2.T + bias2)); keys and values are in the cache pages, as ``qkv_rope_cache`` leaves them."""
@@ -774,7 +832,7 @@ def gemm_splitk_pair_qkv(x1: torch.Tensor, w_qkv: torch.Tensor, bias_qkv, inv_fr
     _need(block_table, "block_table", torch.int32)
     if block_table.dim() != 2:
         raise KernelError("block_table must be [sequences, pages]")
-    freq_ld = _freq_ld(inv_freq, d, block_table.shape[0])
+    rot = _rotation_arg(inv_freq, cs_scale, d, block_table.shape[0], rotary_dim, pairing)
     _need_pools(k_pool, v_pool, torch.bfloat16, nkv, d)
     tuning.tune_pair_parts(w_qkv, w2)
     p1, p2 = gemm_splitk_pair_parts(N1, K1, N2, K2, M)
@@ -783,14 +841,15 @@ def gemm_splitk_pair_qkv(x1: torch.Tensor, w_qkv: torch.Tensor, bias_qkv, inv_fr
     q = torch.empty((M, nh, d), dtype=torch.bfloat16, device=x1.device)
     y2 = torch.empty((M, N2), dtype=torch.bfloat16, device=x1.device)
     _call("pta_gemm_splitk_pair_reduced_qkv_bf16", _ptr(q), _ptr(part1), _ptr(x1), _ptr(w_qkv), _ptr(bias_qkv), K1,
-          _ptr(inv_freq), freq_ld, ctypes.c_float(cs_scale), _ptr(token_pos), _ptr(token_seq), _ptr(block_table),
+          rot, _ptr(token_pos), _ptr(token_seq), _ptr(block_table),
           block_table.shape[1], _ptr(k_pool), _ptr(v_pool), nh, nkv, d, QKV_LAYOUT_CODES[layout], int(write_cache),
           _ptr(y2), _ptr(part2), _ptr(x2), _ptr(w2), _ptr(bias2), N2, K2, ACT_CODES[act2], M, _stream())
     return q, y2
 
 
 def gemm_splitk_qkv(x: torch.Tensor, w_qkv: torch.Tensor, bias_qkv, inv_freq, cs_scale: float, token_pos, token_seq,
-                    block_table, k_pool, v_pool, nh: int, nkv: int, d: int, layout: str, write_cache: bool):
+                    block_table, k_pool, v_pool, nh: int, nkv: int, d: int, layout: str, write_cache: bool,
+                    rotary_dim: Optional[int] = None, pairing: str = "half"):
     """A fused query_key_value projection of a decode batch (17 to 256 rows) on its own, taken to its end by the
     launch that adds its partial sums: returns the queries [M, nh, d] rotated; keys and values are in the cache
     pages, as ``qkv_rope_cache`` leaves them."""
@@ -809,12 +868,12 @@ def gemm_splitk_qkv(x: torch.Tensor, w_qkv: torch.Tensor, bias_qkv, inv_freq, cs
     _need(block_table, "block_table", torch.int32)
     if block_table.dim() != 2:
         raise KernelError("block_table must be [sequences, pages]")
-    freq_ld = _freq_ld(inv_freq, d, block_table.shape[0])
+    rot = _rotation_arg(inv_freq, cs_scale, d, block_table.shape[0], rotary_dim, pairing)
     _need_pools(k_pool, v_pool, torch.bfloat16, nkv, d)
     part = torch.empty((int(load_library().pta_gemm_splitk_parts(N, K, 0, 0)), M, N), dtype=torch.float32, device=x.device)
     q = torch.empty((M, nh, d), dtype=torch.bfloat16, device=x.device)
     _call("pta_gemm_splitk_reduced_qkv_bf16", _ptr(q), _ptr(part), _ptr(x), _ptr(w_qkv), _ptr(bias_qkv), K,
-          _ptr(inv_freq), freq_ld, ctypes.c_float(cs_scale), _ptr(token_pos), _ptr(token_seq), _ptr(block_table),
+          rot, _ptr(token_pos), _ptr(token_seq), _ptr(block_table),
           block_table.shape[1], _ptr(k_pool), _ptr(v_pool), nh, nkv, d, QKV_LAYOUT_CODES[layout], int(write_cache), M,
           _stream())
     return q

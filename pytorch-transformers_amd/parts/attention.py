@@ -18,6 +18,7 @@ import torch
 from .. import ops
 from .base import Part, StepContext, register_part
 from .linear import Linear, PendingProjection, QkvTail, TailDone
+from .positions import as_rotation, as_score_bias
 
 
 class AttentionMixer(Part):
@@ -48,8 +49,14 @@ class AttentionMixer(Part):
     can_defer = True
 
     def check_sizes(self) -> None:
-        rotated = self.positions.rotation()[0] is not None or hasattr(self.positions, "rotation_for")
-        problem = ops.attention_sizes_problem(self.num_heads, self.kv_heads, self.head_dim, rotated)
+        rot = as_rotation(self.positions.rotation())
+        problem = ops.attention_sizes_problem(self.num_heads, self.kv_heads, self.head_dim,
+                                              rot is not None or hasattr(self.positions, "rotation_for"))
+        if problem is None and rot is not None:
+            problem = ops.rotation_problem(self.head_dim, rot.rotary_dim, rot.pairing)
+        bias = as_score_bias(self.positions.score_bias(), self.head_dim)
+        if problem is None and bias is not None:
+            problem = ops.score_bias_problem(bias.of, bias.bf16)
         if problem is not None:
             raise ValueError(f"{self.name}: {problem}")
 
@@ -63,9 +70,9 @@ class AttentionMixer(Part):
         own may hand this to the launch (``Linear.pair``)."""
         k_pool, v_pool = ctx.cache.kv_layer(call.cache_group, call.cache_layer)
         # a position encoding whose rotation depends on the step (frequencies per sequence) offers rotation_for
-        inv_freq, cs_scale = (self.positions.rotation_for(ctx) if hasattr(self.positions, "rotation_for")
-                              else self.positions.rotation())
-        return QkvTail(self.qkv.bias, inv_freq, cs_scale, ctx.token_pos, ctx.token_seq, ctx.block_tables[call.cache_group],
+        rot = as_rotation(self.positions.rotation_for(ctx) if hasattr(self.positions, "rotation_for")
+                          else self.positions.rotation())
+        return QkvTail(self.qkv.bias, rot, ctx.token_pos, ctx.token_seq, ctx.block_tables[call.cache_group],
                        k_pool, v_pool, self.num_heads, self.kv_heads, self.head_dim, self.qkv_layout, call.write_cache)
 
     def forward(self, x: torch.Tensor, ctx: StepContext, call, residual: Optional[torch.Tensor] = None,
@@ -83,8 +90,12 @@ class AttentionMixer(Part):
         else:
             fused = projected if projected is not None else self.qkv(x, apply_bias=False)
             q = self.projection_tail(ctx, call).run(fused)
-        o = ops.attention(q, k_pool, v_pool, table, ctx, self.positions.score_bias(), self.scale, self.window,
-                          alibi_exact=bool(getattr(self.positions, "exact_bias", False)))
+        bias = as_score_bias(self.positions.score_bias(), self.head_dim)
+        if bias is None:
+            o = ops.attention(q, k_pool, v_pool, table, ctx, None, self.scale, self.window)
+        else:
+            o = ops.attention(q, k_pool, v_pool, table, ctx, bias.slopes, self.scale, self.window,
+                              alibi_exact=not bias.bf16, bias_of=bias.of, bias_scale=bias.scale)
         if defer:
             return PendingProjection(self.out, o)
         return self.out(o, add1=residual)

@@ -87,7 +87,8 @@ class Linear(Part):
             return None
         return TailDone(ops.gemm_splitk_qkv(
             x, self.weight, tail.bias, tail.inv_freq, tail.cs_scale, tail.token_pos, tail.token_seq, tail.table,
-            tail.k_pool, tail.v_pool, tail.num_heads, tail.kv_heads, tail.head_dim, tail.layout, tail.write_cache))
+            tail.k_pool, tail.v_pool, tail.num_heads, tail.kv_heads, tail.head_dim, tail.layout, tail.write_cache,
+            **tail.how))
 
     @staticmethod
     def pair(first: "Linear", x1: torch.Tensor, kw1: dict, second: "Linear", x2: torch.Tensor, kw2: dict, tail=None):
@@ -106,7 +107,7 @@ class Linear(Part):
             q, y2 = ops.gemm_skinny_pair_qkv(
                 x1, first.weight, tail.bias, tail.inv_freq, tail.cs_scale, tail.token_pos, tail.token_seq, tail.table,
                 tail.k_pool, tail.v_pool, tail.num_heads, tail.kv_heads, tail.head_dim, tail.layout, tail.write_cache,
-                x2, second.weight, b2, kw2.get("act"))
+                x2, second.weight, b2, kw2.get("act"), **tail.how)
             return TailDone(q), y2
         args = (x1, first.weight, x2, second.weight, b1, kw1.get("act"), b2, kw2.get("act"))
         if x1.shape == x2.shape and ops.gemm_skinny_ok(x1, first.weight) and ops.gemm_skinny_ok(x2, second.weight):
@@ -129,7 +130,7 @@ class Linear(Part):
                 q, y2 = ops.gemm_splitk_pair_qkv(
                     x1, first.weight, tail.bias, tail.inv_freq, tail.cs_scale, tail.token_pos, tail.token_seq, tail.table,
                     tail.k_pool, tail.v_pool, tail.num_heads, tail.kv_heads, tail.head_dim, tail.layout, tail.write_cache,
-                    x2, second.weight, b2, kw2.get("act"))
+                    x2, second.weight, b2, kw2.get("act"), **tail.how)
                 return TailDone(q), y2
             return ops.gemm_splitk_pair_bf16(*args)
         return None
@@ -149,9 +150,14 @@ class QkvTail:
     and values into the cache pages.  ``run`` does it as a kernel of its own; a pair launch that is given the tail
     may do it in its epilogue instead (``Linear.pair``)."""
 
-    def __init__(self, bias, inv_freq, cs_scale, token_pos, token_seq, table, k_pool, v_pool, num_heads: int,
+    def __init__(self, bias, rotation, token_pos, token_seq, table, k_pool, v_pool, num_heads: int,
                  kv_heads: int, head_dim: int, layout: str, write_cache: bool):
-        self.bias, self.inv_freq, self.cs_scale = bias, inv_freq, cs_scale
+        """``rotation``: a ``positions.Rotation`` or None."""
+        self.bias, self.rotation = bias, rotation
+        self.inv_freq = None if rotation is None else rotation.inv_freq
+        self.cs_scale = 1.0 if rotation is None else rotation.scale
+        #: how the rotation lies in a head, as keywords of the launches that rotate
+        self.how = {} if rotation is None else {"rotary_dim": rotation.rotary_dim, "pairing": rotation.pairing}
         self.token_pos, self.token_seq, self.table, self.k_pool, self.v_pool = token_pos, token_seq, table, k_pool, v_pool
         self.num_heads, self.kv_heads, self.head_dim, self.layout = num_heads, kv_heads, head_dim, layout
         self.write_cache = write_cache
@@ -159,7 +165,7 @@ class QkvTail:
     def run(self, fused: torch.Tensor) -> torch.Tensor:
         return ops.qkv_rope_cache(fused, self.bias, self.inv_freq, self.cs_scale, self.token_pos, self.token_seq,
                                   self.table, self.k_pool, self.v_pool, self.num_heads, self.kv_heads, self.head_dim,
-                                  self.layout, write_cache=self.write_cache)
+                                  self.layout, write_cache=self.write_cache, **self.how)
 
 
 class TailDone:

@@ -1,22 +1,72 @@
-"""Position encodings: what rotates queries and keys, and what is added to attention scores."""
+"""Position encodings: what rotates queries and keys, and what is added to attention scores.
+
+Both are data that the kernels take (``Rotation``, ``ScoreBias``); a position encoding is a part that hands them
+out.  Another scheme of either kind that the fields can say (a rotation of part of the head, interleaved pairs,
+other frequencies; slopes times the distance instead of the key's position, another scale) is a new part and no
+change to a kernel.
+"""
 from __future__ import annotations
 
+import dataclasses
 import math
-from typing import Optional, Tuple
+from typing import Optional, Tuple, Union
 
 import torch
 
 from .base import Part, register_part
 
 
+@dataclasses.dataclass
+class Rotation:
+    """Queries and keys are rotated by position: the first ``rotary_dim`` elements of a head (None: all) in pairs
+    ``(i, i + rotary_dim / 2)`` (``"half"``) or ``(2i, 2i + 1)`` (``"interleaved"``), pair i by the angle
+    ``position * inv_freq[i]``, cosines and sines multiplied by ``scale``.  ``inv_freq`` is ``[rotary_dim / 2]``, or
+    one such row per sequence of the step."""
+
+    inv_freq: torch.Tensor
+    scale: float = 1.0
+    rotary_dim: Optional[int] = None
+    pairing: str = "half"
+
+
+@dataclasses.dataclass
+class ScoreBias:
+    """``slopes[head] * x * scale`` is added to the score of a query and a key: x is the key's position (``of="key"``)
+    or the key's position minus the query's (``"distance"``).  ``bf16``: the position and the product are rounded to
+    bfloat16 before the scale, and the slopes are held rounded (what the reference does, ``"key"`` only)."""
+
+    slopes: torch.Tensor
+    of: str = "key"
+    bf16: bool = False
+    scale: float = 1.0
+
+
+def as_rotation(given) -> Optional[Rotation]:
+    """What a position encoding's ``rotation()`` may return, as a ``Rotation`` or None: a ``Rotation``, None, or the
+    pair ``(inv_freq or None, scale)`` of a rotation of whole heads in half-split pairs."""
+    if given is None or isinstance(given, Rotation):
+        return given
+    inv_freq, scale = given
+    return None if inv_freq is None else Rotation(inv_freq, float(scale))
+
+
+def as_score_bias(given, head_dim: int) -> Optional[ScoreBias]:
+    """What ``score_bias()`` may return, as a ``ScoreBias`` or None: a ``ScoreBias``, None, or a tensor of slopes per
+    head, which stands for the reference's ALiBi (times the key's position, rounded to bfloat16, divided by the root
+    of the head size; src/transformers/models/falcon/modeling_falcon.py:196-198, :1078-1085)."""
+    if given is None or isinstance(given, ScoreBias):
+        return given
+    return ScoreBias(given, "key", True, 1.0 / math.sqrt(head_dim))
+
+
 class NoPositions(Part):
     def to(self, device) -> None:
         pass
 
-    def rotation(self) -> Tuple[Optional[torch.Tensor], float]:
-        return None, 1.0
+    def rotation(self) -> Union[None, Rotation, Tuple[Optional[torch.Tensor], float]]:
+        return None
 
-    def score_bias(self) -> Optional[torch.Tensor]:
+    def score_bias(self) -> Union[None, ScoreBias, torch.Tensor]:
         return None
 
 
@@ -72,11 +122,11 @@ class RotaryPositions(NoPositions):
     def to(self, device) -> None:
         self.inv_freq = self.inv_freq.to(device)
 
-    def rotation(self):
-        return self.inv_freq, self.attention_scaling
+    def rotation(self) -> Rotation:
+        return Rotation(self.inv_freq, self.attention_scaling)
 
-    def rotation_for(self, ctx):
-        """The frequencies for one step: the table, or with dynamic scaling one table per sequence of the step,
+    def rotation_for(self, ctx) -> Rotation:
+        """The rotation for one step: the table, or with dynamic scaling one table per sequence of the step,
         ``[sequences, head_dim / 2]``, made once per step on the device from the step's own arrays (so a captured
         step makes it anew at every replay)."""
         if self.dynamic_factor is None:
@@ -88,7 +138,7 @@ class RotaryPositions(NoPositions):
         if table is None:
             table = ctx.extras[key] = ops.rope_dynamic_table(ctx.seq_start, ctx.cu_tokens, self.head_dim, self.theta,
                                                              self.dynamic_factor, self.trained_positions)
-        return table, self.attention_scaling
+        return Rotation(table, self.attention_scaling)
 
 
 def default_frequencies(head_dim: int, theta: float) -> torch.Tensor:
@@ -186,19 +236,22 @@ class AlibiPositions(NoPositions):
     #: False: slopes, positions and their product are rounded to bfloat16 as the reference rounds them
     exact_bias = False
 
-    def __init__(self, num_heads: int, bf16_compat: bool = True):
+    def __init__(self, num_heads: int, bf16_compat: bool = True, scale: float = 1.0):
         """``bf16_compat=False`` leaves the reference's numbers for the exact ``slope * position`` in 32-bit
-        (``alibi_bf16_compat: false`` in config.json); the default reproduces the reference."""
+        (``alibi_bf16_compat: false`` in config.json); the default reproduces the reference.  ``scale``: what the
+        bias is multiplied by when it joins the scores (the reference's Falcon: one over the root of the head size,
+        :1081)."""
         self.num_heads = num_heads
         self.exact_bias = not bf16_compat
+        self.scale = float(scale)
         slopes = alibi_slopes(num_heads)
         self.slopes = (slopes if self.exact_bias else slopes.bfloat16().float()).contiguous()
 
     def to(self, device) -> None:
         self.slopes = self.slopes.to(device)
 
-    def score_bias(self):
-        return self.slopes
+    def score_bias(self) -> ScoreBias:
+        return ScoreBias(self.slopes, "key", not self.exact_bias, self.scale)
 
 
 register_part("positions", "none", NoPositions)

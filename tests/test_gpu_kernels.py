@@ -675,6 +675,167 @@ def test_batch_launch_takes_the_fused_qkv_rows_to_their_end(layout, nh, nkv, d, 
         ops.gemm_splitk_qkv(x, w[:-8], b, inv, 1.0, token_pos, token_seq, bt, k1, v1, nh, nkv, d, layout, False)
 
 
+def _rotate_plain(x, pos, inv_freq, scale, rotary_dim, pairing):
+    """The rotation spelled out element by element: x [T, heads, d], the first ``rotary_dim`` elements of a head in
+    pairs (i, i + rotary_dim / 2) ("half") or (2i, 2i + 1) ("interleaved"), pair i by position * inv_freq[i] (the
+    angle in 32-bit); the other elements as they are."""
+    out = x.clone()
+    ang = pos.float()[:, None] * inv_freq.float()  # [T, rotary_dim / 2], one row of frequencies or one per token
+    cos, sin = (ang.cos() * scale).double()[:, None, :], (ang.sin() * scale).double()[:, None, :]
+    first = slice(0, rotary_dim, 2) if pairing == "interleaved" else slice(0, rotary_dim // 2)
+    second = slice(1, rotary_dim, 2) if pairing == "interleaved" else slice(rotary_dim // 2, rotary_dim)
+    a, b = x[..., first], x[..., second]
+    out[..., first] = a * cos - b * sin
+    out[..., second] = b * cos + a * sin
+    return out
+
+
+ARRANGEMENTS = [dict(rotary_dim=None, pairing="interleaved"), dict(rotary_dim=0.5, pairing="half"),
+                dict(rotary_dim=0.5, pairing="interleaved"), dict(rotary_dim=0.25, pairing="half"),
+                dict(rotary_dim=0.75, pairing="interleaved")]
+
+
+def _how(arrangement, d):
+    """Keywords of the launches that rotate, the table of frequencies' length, for a head size."""
+    r = d if arrangement["rotary_dim"] is None else max(2, int(d * arrangement["rotary_dim"]) // 2 * 2)
+    return dict(rotary_dim=r, pairing=arrangement["pairing"]), r
+
+
+def test_the_whole_head_in_half_split_pairs_is_what_the_reference_rotates():
+    """The spelling above with the whole head and half-split pairs is the reference's rotate_half form."""
+    x = torch.randn(5, 3, 16, dtype=torch.float64)
+    pos, inv = torch.tensor([0, 3, 9, 70, 71]), P.rope_inv_freq(16, 10000.0)
+    cos, sin = P.rope_cos_sin(pos, inv)
+    torch.testing.assert_close(_rotate_plain(x, pos, inv[None, :], 1.0, 16, "half"), P.apply_rope(x, cos, sin), rtol=1e-12, atol=1e-12)
+    # interleaved pairs are the same rotation of a head whose elements are laid out pair by pair
+    order = torch.stack([torch.arange(8), torch.arange(8) + 8], dim=1).reshape(-1)  # 0, 8, 1, 9, ...
+    torch.testing.assert_close(_rotate_plain(x[..., order], pos, inv[None, :], 1.0, 16, "interleaved"),
+                               P.apply_rope(x, cos, sin)[..., order], rtol=1e-12, atol=1e-12)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("layout,nh,nkv,d", [("grouped", 6, 2, 32), ("tail", 7, 1, 64), ("interleaved", 5, 5, 24),
+                                             ("grouped", 4, 1, 128)])
+@pytest.mark.parametrize("arrangement", ARRANGEMENTS)
+@pytest.mark.parametrize("rotary", [True, "per sequence"])
+def test_rotation_of_part_of_the_head_and_of_interleaved_pairs(dtype, layout, nh, nkv, d, arrangement, rotary):
+    """The kernel that splits, rotates and writes the cache with a rotation given as data: part of the head or all
+    of it, half-split or interleaved pairs, against the spelling above; what is not rotated passes as it is."""
+    ops = _ops()
+    how, r = _how(arrangement, d)
+    starts, news = [70, 0, 127], [3, 66, 1]
+    lens = [s + n for s, n in zip(starts, news)]
+    k_pool, v_pool, bt, lists = _cache_setup(3, lens, nkv, d, dtype)
+    M = sum(news)
+    fused = _rand(M, (nh + 2 * nkv) * d, dtype=dtype)
+    bias = _rand((nh + 2 * nkv) * d, seed=9)
+    token_seq = torch.tensor([i for i, n in enumerate(news) for _ in range(n)], dtype=torch.int32).cuda()
+    token_pos = torch.tensor([s + j for s, n in zip(starts, news) for j in range(n)], dtype=torch.int32).cuda()
+    inv = _freq(rotary, r, 3, 500042.0, 2.0)
+    q = ops.qkv_rope_cache(fused, bias, inv, 0.8, token_pos, token_seq, bt, k_pool, v_pool, nh, nkv, d, layout, **how)
+    c = dict(num_attention_heads=nh, hidden_size=nh * d, num_kv_heads=nkv,
+             new_decoder_architecture=layout == "grouped", multi_query=layout == "tail")
+    rnd = (lambda t: t) if dtype == torch.float32 else (lambda t: t.bfloat16().double())
+    wq, wk, wv = P.split_heads(rnd(fused.double().cpu() + bias.double().cpu()), c)
+    per_token = inv.cpu()[token_seq.cpu().long()] if rotary == "per sequence" else inv.cpu()[None, :]
+    wq, wk = (_rotate_plain(t, token_pos.cpu(), per_token, 0.8, r, how["pairing"]) for t in (wq, wk))
+    tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(q.double().cpu(), wq, **tol)
+    if r < d and dtype == torch.bfloat16:  # what lies past rotary_dim is the fused row's value (and bias), bit for bit
+        assert torch.equal(q[..., r:].double().cpu(), wq[..., r:])
+    at = 0
+    for i, (s_, n) in enumerate(zip(starts, news)):
+        gk, gv = _gather(k_pool, lists[i], lens[i]), _gather(v_pool, lists[i], lens[i], transposed=True)
+        torch.testing.assert_close(gk[s_:].double().cpu(), wk[at:at + n].contiguous(), **tol)
+        torch.testing.assert_close(gv[s_:].double().cpu(), wv[at:at + n].contiguous(), **tol)
+        at += n
+    for bad, match in ((dict(rotary_dim=d + 2), "rotary_dim"), (dict(rotary_dim=5), "rotary_dim"), (dict(pairing="thirds"), "pairing")):
+        with pytest.raises(ops.KernelError, match=match):
+            ops.qkv_rope_cache(fused, bias, inv, 1.0, token_pos, token_seq, bt, k_pool, v_pool, nh, nkv, d, layout, **bad)
+
+
+@pytest.mark.parametrize("layout,nh,nkv,d", [("grouped", 4, 2, 32), ("tail", 7, 1, 64), ("interleaved", 3, 3, 96), ("grouped", 8, 2, 128)])
+@pytest.mark.parametrize("arrangement", ARRANGEMENTS)
+def test_fused_launches_rotate_as_the_kernel_of_its_own_in_every_arrangement(layout, nh, nkv, d, arrangement):
+    """The three launches that take fused query_key_value rows to their end (the pair launch for few rows, the pair
+    launch of a decode batch, the batch product on its own) with a rotation of part of the head or of interleaved
+    pairs: queries and pages bit for bit those of the product followed by the kernel of its own."""
+    ops = _ops()
+    how, r = _how(arrangement, d)
+    K, N2 = 264, 200
+    N1 = (nh + 2 * nkv) * d
+    w1, w2 = _rand(N1, K, seed=1, dtype=torch.bfloat16, scale=0.05), _rand(N2, K, seed=2, dtype=torch.bfloat16, scale=0.05)
+    b1, b2 = _rand(N1, seed=3), _rand(N2, seed=4)
+    same = lambda a, b: torch.equal(torch.nan_to_num(a.float(), nan=-7.0), torch.nan_to_num(b.float(), nan=-7.0))
+    for M in (5, 40):
+        g = torch.Generator().manual_seed(M)
+        starts = torch.randint(0, 190, (M,), generator=g).tolist()
+        lens = [s_ + 1 for s_ in starts]
+        x = _rand(M, K, dtype=torch.bfloat16)
+        token_seq = torch.arange(M, dtype=torch.int32).cuda()
+        token_pos = torch.tensor(starts, dtype=torch.int32).cuda()
+        inv = _freq("per sequence", r, M)
+        results = {}
+        for way in ("own kernel", "pair") + (("single",) if M > 16 else ()):
+            k_pool, v_pool, bt, _ = _cache_setup(M, lens, nkv, d, torch.bfloat16, n_pages=3 * M + 8)
+            tail_args = (inv, 0.9, token_pos, token_seq, bt, k_pool, v_pool, nh, nkv, d, layout)
+            if way == "own kernel":
+                fused = (ops.gemm_skinny_pair_bf16 if M <= 16 else ops.gemm_splitk_pair_bf16)(x, w1, x, w2, None, None, b2, "gelu")[0]
+                q = ops.qkv_rope_cache(fused, b1, *tail_args, **how)
+            elif way == "pair":
+                fn = ops.gemm_skinny_pair_qkv if M <= 16 else ops.gemm_splitk_pair_qkv
+                q = fn(x, w1, b1, *tail_args, True, x, w2, b2, "gelu", **how)[0]
+            else:
+                q = ops.gemm_splitk_qkv(x, w1, b1, *tail_args, True, **how)
+            results[way] = (q, k_pool, v_pool)
+        q0, k0, v0 = results["own kernel"]
+        for way, (q, k_pool, v_pool) in results.items():
+            if way == "single":  # the product on its own cuts K by its own rule: its own bits, the same rotation
+                fused = ops.gemm_splitk_bf16(x, w1)
+                k_pool2, v_pool2, bt2, _ = _cache_setup(M, lens, nkv, d, torch.bfloat16, n_pages=3 * M + 8)
+                q0 = ops.qkv_rope_cache(fused, b1, inv, 0.9, token_pos, token_seq, bt2, k_pool2, v_pool2, nh, nkv, d, layout, **how)
+                k0, v0 = k_pool2, v_pool2
+            assert torch.equal(q, q0), (way, M)
+            assert same(k_pool, k0) and same(v_pool, v0), (way, M)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_score_bias_of_the_distance_and_with_another_scale(dtype):
+    """The bias on scores as data: slopes times the key's position or times its distance from the query (equal
+    under softmax), exact or rounded as the reference rounds, with any scale; prompts, chunks and decode steps of
+    both attention kernels against plain attention with the bias spelled out."""
+    ops = _ops()
+    nh, nkv, d = 6, 2, 32
+    slopes = (0.5 ** torch.arange(1, nh + 1).float()).cuda()
+    starts, news = [0, 63, 200, 0, 127], [70, 1, 5, 1, 2]
+
+    def case(fn, bias_scale, **kw):
+        def run(q, k_pool, v_pool, bt, token_seq, token_pos, slopes_, scale, starts_, news_, window=0):
+            return fn(q, k_pool, v_pool, bt, token_seq, token_pos, slopes_, scale, starts_, news_, bias_scale=bias_scale, **kw)
+        return run
+
+    def generic(q, k_pool, v_pool, bt, token_seq, token_pos, slopes_, scale, starts_, news_, **kw):
+        return ops.attn_generic(q, k_pool, v_pool, bt, token_seq, token_pos, slopes_, scale, 0, **kw)
+
+    def mfma(q, k_pool, v_pool, bt, token_seq, token_pos, slopes_, scale, starts_, news_, **kw):
+        cu = torch.tensor([0] + list(torch.tensor(news_).cumsum(0)), dtype=torch.int32).cuda()
+        st = torch.tensor(starts_, dtype=torch.int32).cuda()
+        return ops.attn_mfma(q, k_pool, v_pool, bt, cu, st, slopes_, scale, max_new=max(news_), **kw)
+
+    kernels = [generic] + ([mfma] if dtype == torch.bfloat16 else [])
+    for fn in kernels:
+        for bias_scale in (1.0, 0.3):
+            for kw in (dict(alibi_exact=True), dict(alibi_exact=True, bias_of="distance")):
+                _attn_case(ops, case(fn, bias_scale, **kw), dtype, nh, nkv, d, starts, news, slopes=slopes,
+                           plain_bias=lambda L: (slopes.cpu().double()[:, None] * torch.arange(L).double()[None, :]) * bias_scale)
+        # the reference's rounding (bfloat16 slopes, position and product), with the scale it has there
+        from pytorch_transformers_amd.parts import AlibiPositions
+        _attn_case(ops, case(fn, d ** -0.5), dtype, nh, nkv, d, starts, news, slopes=AlibiPositions(nh).slopes.cuda())
+    with pytest.raises(ops.KernelError, match="not built"):
+        ops._score_bias_arg(slopes, nh, "query")
+    assert ops.score_bias_problem("distance", True) and ops.score_bias_problem("key", True) is None
+
+
 def _windowed_attention(q, k, v, window):
     """Plain attention in which query t sees keys t - window + 1 .. t; q [T, nh, d], k, v [T, nkv, d]."""
     T, nh, d = q.shape
@@ -688,7 +849,7 @@ def _windowed_attention(q, k, v, window):
     return out.reshape(T, nh * d)
 
 
-def _attn_case(ops, fn, dtype, nh, nkv, d, starts, news, slopes=None, seed=0, boost=None, window=0):
+def _attn_case(ops, fn, dtype, nh, nkv, d, starts, news, slopes=None, seed=0, boost=None, window=0, plain_bias=None):
     """Fill a cache with random keys and values, run ``fn`` for the new tokens, compare with plain attention.
     With a window, the pages that lie wholly behind every new token's window hold NaN: they may be gone."""
     lens = [s + n for s, n in zip(starts, news)]
@@ -724,7 +885,9 @@ def _attn_case(ops, fn, dtype, nh, nkv, d, starts, news, slopes=None, seed=0, bo
     for i, (s, n) in enumerate(zip(starts, news)):
         L = lens[i]
         bias = None
-        if slopes is not None:
+        if plain_bias is not None:  # [heads, keys] for a sequence of L keys
+            bias = plain_bias(L)
+        elif slopes is not None:
             bias = P.alibi_bias(nh, L, d)
         # plain attention of the whole sequence needs a query per position: only the new rows are compared
         q_full = torch.zeros(L, nh, d, dtype=torch.float64)

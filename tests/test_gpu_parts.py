@@ -198,13 +198,24 @@ def test_library_product_over_ranges_of_k():
 def test_positions():
     from pytorch_transformers_amd.parts import AlibiPositions, NoPositions, RotaryPositions
 
+    from pytorch_transformers_amd.parts.positions import Rotation, ScoreBias, as_rotation, as_score_bias
+
     r = RotaryPositions(64, 500042.0, scaling_factor=4.0)
-    inv, scale = r.rotation()
-    assert torch.equal(inv, P.rope_inv_freq(64, 500042.0, 4.0)) and scale == 1.0 and r.score_bias() is None
+    rot = r.rotation()
+    assert torch.equal(rot.inv_freq, P.rope_inv_freq(64, 500042.0, 4.0)) and r.score_bias() is None
+    assert (rot.scale, rot.rotary_dim, rot.pairing) == (1.0, None, "half")  # the whole head, half-split pairs
     for nh in (6, 20, 64):
-        a = AlibiPositions(nh)
-        assert torch.equal(a.score_bias(), P.alibi_slopes(nh).bfloat16().float()) and a.rotation() == (None, 1.0)
-    assert NoPositions().rotation() == (None, 1.0) and NoPositions().score_bias() is None
+        a = AlibiPositions(nh, scale=0.125)
+        bias = a.score_bias()
+        assert torch.equal(bias.slopes, P.alibi_slopes(nh).bfloat16().float()) and a.rotation() is None
+        assert (bias.of, bias.bf16, bias.scale) == ("key", True, 0.125)
+        assert not AlibiPositions(nh, bf16_compat=False).score_bias().bf16
+    assert NoPositions().rotation() is None and NoPositions().score_bias() is None
+    # what a position encoding may hand out in place of the two classes: a pair for a rotation of whole heads, a
+    # tensor of slopes for the reference's bias
+    inv = torch.ones(8)
+    assert as_rotation((None, 1.0)) is None and as_rotation((inv, 0.5)) == Rotation(inv, 0.5)
+    assert as_score_bias(inv, 64) == ScoreBias(inv, "key", True, 0.125) and as_score_bias(None, 64) is None
 
 
 @pytest.mark.parametrize("dtype,rel", DTYPES)
@@ -219,7 +230,7 @@ def test_attention_mixer_and_blocks(dtype, rel, layout, nh, nkv, d, alibi, bias)
                                                 RotaryPositions, SequentialBlock)
 
     H, F, T = nh * d, 3 * nh * d + 8, 75
-    pos = AlibiPositions(nh) if alibi else RotaryPositions(d, 10000.0)
+    pos = AlibiPositions(nh, scale=d ** -0.5) if alibi else RotaryPositions(d, 10000.0)  # the scale of modeling_falcon.py:1081
     pos.to("cuda:0")
     mixer = AttentionMixer("transformer.h.0.self_attention", H, nh, nkv, d, layout, bias, pos)
     ffn = DenseFeedForward("transformer.h.0.mlp", H, F, bias)
@@ -710,3 +721,176 @@ def test_toy_architecture_with_a_window_layer(tmp_path, dtype, rel):
         cache.check_consistent()
     finally:
         unregister("toy-window")
+
+
+# --- a fourth toy: position encodings of its own, said in the data that the kernels take ---
+def _define_positions_toy():
+    from pytorch_transformers_amd.config.base import ModelConfig
+    from pytorch_transformers_amd.engine.spec import CACHE_FULL, CacheGroupSpec, LayerCall, ModelSpec
+    from pytorch_transformers_amd.parts import (AttentionMixer, DenseFeedForward, Embedding, LayerNorm, NoPositions,
+                                                OutputHead, ParallelBlock, Rotation, ScoreBias, SequentialBlock,
+                                                register_part)
+
+    @dataclasses.dataclass
+    class PositionsConfig(ModelConfig):
+        model_type = "toy-positions"
+        vocab_size: int = 157
+        width: int = 256
+        heads: int = 4
+        rotary_fraction: float = 0.5
+        theta: float = 1000.0
+        slope_base: float = 0.25
+
+    class PartialInterleavedRotary(NoPositions):
+        """Rotates the first part of every head only, in pairs of neighbouring elements (2i, 2i + 1): a rotation that
+        the framework's own position encoding does not have, said in the fields of ``Rotation``."""
+
+        def __init__(self, head_dim, fraction, theta):
+            self.rotary_dim = int(head_dim * fraction) // 2 * 2
+            self.inv_freq = (1.0 / theta ** (torch.arange(0, self.rotary_dim, 2, dtype=torch.float32) / self.rotary_dim)).contiguous()
+
+        def to(self, device):
+            self.inv_freq = self.inv_freq.to(device)
+
+        def rotation(self):
+            return Rotation(self.inv_freq, 1.0, rotary_dim=self.rotary_dim, pairing="interleaved")
+
+    class DistanceBias(NoPositions):
+        """A bias on the scores that falls with the distance between query and key, ``-slope_h * (t - j)``, exact and
+        with no further scale: another bias function of (head, query position, key position)."""
+
+        def __init__(self, heads, base):
+            self.slopes = (base ** torch.arange(1, heads + 1, dtype=torch.float32)).contiguous()
+
+        def to(self, device):
+            self.slopes = self.slopes.to(device)
+
+        def score_bias(self):
+            return ScoreBias(self.slopes, of="distance", bf16=False, scale=1.0)
+
+    register_part("positions", "partial-interleaved", PartialInterleavedRotary, exist_ok=True)
+    register_part("positions", "distance-bias", DistanceBias, exist_ok=True)
+
+    def build(cfg):
+        d = cfg.width // cfg.heads
+        rotary = PartialInterleavedRotary(d, cfg.rotary_fraction, cfg.theta)
+        blocks = [
+            # one norm, so that decode steps run the fused query_key_value rows through the pair launches' tails
+            ParallelBlock(AttentionMixer("t.h.0.attn", cfg.width, cfg.heads, 2, d, "grouped", True, rotary),
+                          DenseFeedForward("t.h.0.mlp", cfg.width, 2 * cfg.width, bias=False), LayerNorm("t.h.0.norm", cfg.width, 1e-5)),
+            SequentialBlock(AttentionMixer("t.h.1.attn", cfg.width, cfg.heads, 1, d, "tail", False, DistanceBias(cfg.heads, cfg.slope_base)),
+                            DenseFeedForward("t.h.1.mlp", cfg.width, 2 * cfg.width, bias=False), LayerNorm("t.h.1.n1", cfg.width, 1e-5),
+                            LayerNorm("t.h.1.n2", cfg.width, 1e-5)),
+        ]
+        return ModelSpec(config=cfg, embedding=Embedding("t.embed", cfg.vocab_size, cfg.width), blocks=blocks,
+                         order=[LayerCall(0, "two", 0), LayerCall(1, "one", 0)],
+                         final_norm=LayerNorm("t.final", cfg.width, 1e-5),
+                         head=OutputHead("t.head", cfg.vocab_size, cfg.width, "t.embed.weight"),
+                         cache_groups=[CacheGroupSpec("two", CACHE_FULL, 1, 2, d), CacheGroupSpec("one", CACHE_FULL, 1, 1, d)])
+
+    return PositionsConfig, build
+
+
+def _plain_positions_toy(cfg, w, ids):
+    T, H, nh = len(ids), cfg.width, cfg.heads
+    d = H // nh
+    r = int(d * cfg.rotary_fraction) // 2 * 2
+    x = w["t.embed.weight"][torch.as_tensor(ids)]
+    ln = lambda h, n: P.layer_norm(h, w[n + ".weight"], w[n + ".bias"], 1e-5)
+    ffn = lambda h, p: P.gelu(h @ w[p + ".dense_h_to_4h.weight"].T) @ w[p + ".dense_4h_to_h.weight"].T
+    pos = torch.arange(T)
+
+    def rotate(t):  # neighbouring elements of the first r of a head, pair i by pos * theta^(-2i/r); angles in 32-bit
+        inv = 1.0 / cfg.theta ** (torch.arange(0, r, 2, dtype=torch.float32) / r)
+        ang = pos.float()[:, None] * inv[None, :]
+        cos, sin = ang.cos().double()[:, None, :], ang.sin().double()[:, None, :]
+        out = t.clone()
+        a, b = t[..., 0:r:2], t[..., 1:r:2]
+        out[..., 0:r:2], out[..., 1:r:2] = a * cos - b * sin, b * cos + a * sin
+        return out
+
+    # layer 0: parallel, grouped rows (2 groups of 2 heads) with a bias, part of each head rotated in interleaved pairs
+    a = ln(x, "t.h.0.norm")
+    f = (a @ w["t.h.0.attn.query_key_value.weight"].T + w["t.h.0.attn.query_key_value.bias"]).view(T, 2, 4, d)
+    q, k, v = f[:, :, :2].reshape(T, nh, d), f[:, :, 2], f[:, :, 3]
+    o = P.attention_scores_softmax(rotate(q), rotate(k), v)
+    x = x + (ffn(a, "t.h.0.mlp") + (o @ w["t.h.0.attn.dense.weight"].T + w["t.h.0.attn.dense.bias"]))
+    # layer 1: sequential, one KV head at the tail, scores biased by -slope_h * (query position - key position)
+    a = ln(x, "t.h.1.n1")
+    f = (a @ w["t.h.1.attn.query_key_value.weight"].T).view(T, nh + 2, d)
+    slopes = (cfg.slope_base ** torch.arange(1, nh + 1, dtype=torch.float32)).double()
+    o = torch.empty(T, nh, d, dtype=x.dtype)
+    causal = pos[None, :] <= pos[:, None]
+    for h in range(nh):
+        s = f[:, h] @ f[:, nh].T / math.sqrt(d) + slopes[h] * (pos[None, :] - pos[:, None]).double()
+        o[:, h] = torch.softmax(s.masked_fill(~causal, float("-inf")), dim=-1) @ f[:, nh + 1]
+    rsd = x + o.reshape(T, H) @ w["t.h.1.attn.dense.weight"].T
+    x = rsd + ffn(ln(rsd, "t.h.1.n2"), "t.h.1.mlp")
+    return ln(x, "t.final") @ w["t.embed.weight"].T
+
+
+@pytest.mark.parametrize("dtype,rel", [("float32", 5e-5), ("bfloat16", helpers.REL_BF16)])
+def test_toy_architecture_with_positions_of_its_own(tmp_path, dtype, rel):
+    """A rotation of half of every head in interleaved pairs and a score bias by the distance between query and key,
+    both defined in this file as position parts that hand the kernels their data (``Rotation``, ``ScoreBias``):
+    registered, built and stepped through every schedule with no change to the framework's files; in bfloat16 also
+    as decode batches of 5 and of 20 sequences, whose fused rows are rotated in the matrix launches' own tails."""
+    from safetensors.torch import load_file
+
+    from pytorch_transformers_amd import AutoModelForCausalLM
+    from pytorch_transformers_amd.config import register, unregister
+    from pytorch_transformers_amd.engine.replay import Replayer
+    from pytorch_transformers_amd.parts import registered_parts
+    from pytorch_transformers_amd.weights import write_random_model
+
+    PositionsConfig, build = _define_positions_toy()
+    assert {"partial-interleaved", "distance-bias"} <= set(registered_parts("positions"))
+    register("toy-positions", PositionsConfig, build, exist_ok=True)
+    try:
+        cfg = PositionsConfig()
+        folder = write_random_model(str(tmp_path / "positions"), cfg, seed=12, std=0.1, noise=0.1)
+        w = {k: v.double() for k, v in load_file(f"{folder}/model.safetensors").items()}
+        model = AutoModelForCausalLM.from_pretrained(folder, dtype=dtype)
+        reqs = helpers.make_requests(cfg.vocab_size, [11, 40, 70, 5, 131], seed=4)
+        want = {rid: _plain_positions_toy(cfg, w, toks).float() for rid, toks in reqs.items()}
+        # the positions decide: the same tokens in another order give other logits at the last place
+        swapped = list(reqs["r1"])
+        swapped[3], swapped[17] = swapped[17], swapped[3]
+        assert float((_plain_positions_toy(cfg, w, swapped)[-1] - want["r1"][-1].double()).abs().max()) > 1e-3
+        rp = Replayer(model, 4096, max_slots=24)
+        for name, records in (("whole", helpers.schedule_whole(reqs)), ("tail", helpers.schedule_tail(reqs, 16)),
+                              ("batches", helpers.schedule_batches(reqs, 3)), ("one batch", helpers.schedule_batches(reqs, 5))):
+            got = helpers.run_schedule(rp, records)
+            for rid in reqs:
+                helpers.assert_close(got[rid], want[rid], rel, f"positions toy {dtype} {name} {rid}")
+        # twenty sequences at once: decode steps of 17 rows and more
+        many = helpers.make_requests(cfg.vocab_size, [20 + (7 * i) % 30 for i in range(20)], seed=5)
+        want = {rid: _plain_positions_toy(cfg, w, toks).float() for rid, toks in many.items()}
+        got = helpers.run_schedule(rp, helpers.schedule_batches(many, 20, decode=(6, 8, 7, 9)))
+        for rid in many:
+            helpers.assert_close(got[rid], want[rid], rel, f"positions toy {dtype} twenty at once {rid}")
+    finally:
+        unregister("toy-positions")
+
+
+def test_a_position_part_that_asks_for_what_no_kernel_has_is_refused_by_name():
+    """A rotation or a score bias that the fields cannot say is refused when the model is put together, by the part
+    that has it, with what is built."""
+    from pytorch_transformers_amd.parts import AttentionMixer, NoPositions, Rotation, ScoreBias
+
+    class Thirds(NoPositions):
+        def rotation(self):
+            return Rotation(torch.ones(8), 1.0, rotary_dim=16, pairing="thirds")
+
+    class QueryBias(NoPositions):
+        def score_bias(self):
+            return ScoreBias(torch.ones(4), of="query")
+
+    class TooWide(NoPositions):
+        def rotation(self):
+            return Rotation(torch.ones(40), 1.0, rotary_dim=80)
+
+    for positions, match in ((Thirds(), "pairing 'thirds' is not built"), (QueryBias(), "score bias of 'query' is not built"),
+                             (TooWide(), "rotary_dim must be even, from 2 up to the head size 64")):
+        with pytest.raises(ValueError, match=match):
+            AttentionMixer("m", 256, 4, 2, 64, "grouped", False, positions).check_sizes()
