@@ -33,7 +33,10 @@ def _normed(x, norm: Part, other: Optional[Part] = None):
         x = x.tensor()
     if other is None:
         return x, norm.forward(x), None
-    a, m = norm.forward_pair(x, other)
+    if hasattr(norm, "forward_pair"):  # two norms of one input in one pass, where the norm offers it
+        a, m = norm.forward_pair(x, other)
+    else:
+        a, m = norm.forward(x), other.forward(x)
     return x, a, m
 
 

@@ -894,3 +894,120 @@ def test_a_position_part_that_asks_for_what_no_kernel_has_is_refused_by_name():
                              (TooWide(), "rotary_dim must be even, from 2 up to the head size 64")):
         with pytest.raises(ValueError, match=match):
             AttentionMixer("m", 256, 4, 2, 64, "grouped", False, positions).check_sizes()
+
+
+# --- a fifth toy: a norm of its own (no mean, no bias), in every place a norm stands ---
+def _define_norm_toy():
+    from pytorch_transformers_amd.config.base import ModelConfig
+    from pytorch_transformers_amd.engine.spec import CACHE_FULL, INIT_ONE_NOISE, VECTOR, CacheGroupSpec, LayerCall, ModelSpec, TensorSpec
+    from pytorch_transformers_amd.parts import (AttentionMixer, DenseFeedForward, Embedding, OutputHead, ParallelBlock, Part,
+                                                RotaryPositions, SequentialBlock, register_part)
+
+    @dataclasses.dataclass
+    class NormConfig(ModelConfig):
+        model_type = "toy-norm"
+        vocab_size: int = 149
+        width: int = 96
+        heads: int = 3
+        eps: float = 1e-4
+
+    class RootMeanSquareNorm(Part):
+        """``x / sqrt(mean(x^2) + eps) * w``: no mean taken off, no bias; statistics in 32-bit.  It offers the plain
+        interface of a norm and none of the optional ones (no pair in one pass, no sum formed while it reads)."""
+
+        def __init__(self, name, width, eps):
+            self.name, self.width, self.eps = name, width, eps
+
+        def tensor_specs(self):
+            return [TensorSpec(self.name + ".weight", (self.width,), VECTOR, INIT_ONE_NOISE)]
+
+        def load(self, tensors):
+            self.weight = tensors[self.name + ".weight"]
+
+        def forward(self, x, rows=None):
+            if rows is not None:
+                x = x.index_select(0, rows.long())
+            h = x.float()
+            return (h * torch.rsqrt(h.pow(2).mean(-1, keepdim=True) + self.eps) * self.weight).to(x.dtype)
+
+    register_part("norm", "rms", RootMeanSquareNorm, exist_ok=True)
+
+    def build(cfg):
+        d, W = cfg.width // cfg.heads, cfg.width
+        rms = lambda name: RootMeanSquareNorm(name, W, cfg.eps)
+        pos = RotaryPositions(d, 10000.0)
+        blocks = [
+            ParallelBlock(AttentionMixer("t.h.0.attn", W, cfg.heads, 1, d, "tail", False, pos),
+                          DenseFeedForward("t.h.0.mlp", W, 2 * W, bias=True), rms("t.h.0.n_attn"), rms("t.h.0.n_mlp")),
+            SequentialBlock(AttentionMixer("t.h.1.attn", W, cfg.heads, cfg.heads, d, "interleaved", False, pos),
+                            DenseFeedForward("t.h.1.mlp", W, 2 * W, bias=False), rms("t.h.1.n1"), rms("t.h.1.n2")),
+            ParallelBlock(AttentionMixer("t.h.2.attn", W, cfg.heads, 1, d, "tail", False, pos),
+                          DenseFeedForward("t.h.2.mlp", W, 2 * W, bias=False), rms("t.h.2.n")),
+        ]
+        return ModelSpec(config=cfg, embedding=Embedding("t.embed", cfg.vocab_size, W), blocks=blocks,
+                         order=[LayerCall(0, "one", 0), LayerCall(1, "all", 0), LayerCall(2, "one", 1)],
+                         final_norm=rms("t.final"), head=OutputHead("t.head", cfg.vocab_size, W, "t.embed.weight"),
+                         cache_groups=[CacheGroupSpec("one", CACHE_FULL, 2, 1, d), CacheGroupSpec("all", CACHE_FULL, 1, cfg.heads, d)])
+
+    return NormConfig, build
+
+
+def _plain_norm_toy(cfg, w, ids):
+    T, W, nh = len(ids), cfg.width, cfg.heads
+    d = W // nh
+    x = w["t.embed.weight"][torch.as_tensor(ids)]
+    rms = lambda h, n: h / torch.sqrt((h * h).mean(-1, keepdim=True) + cfg.eps) * w[n + ".weight"]
+    cos, sin = P.rope_cos_sin(torch.arange(T), P.rope_inv_freq(d, 10000.0))
+
+    def attn(h, p, layout):
+        f = h @ w[p + ".query_key_value.weight"].T
+        if layout == "tail":
+            f = f.view(T, nh + 2, d)
+            q, k, v = f[:, :nh], f[:, nh:nh + 1], f[:, nh + 1:]
+        else:
+            f = f.view(T, nh, 3, d)
+            q, k, v = f[:, :, 0], f[:, :, 1], f[:, :, 2]
+        return P.attention_scores_softmax(P.apply_rope(q, cos, sin), P.apply_rope(k, cos, sin), v) @ w[p + ".dense.weight"].T
+
+    def ffn(h, p, bias):
+        u = h @ w[p + ".dense_h_to_4h.weight"].T + (w[p + ".dense_h_to_4h.bias"] if bias else 0)
+        return P.gelu(u) @ w[p + ".dense_4h_to_h.weight"].T + (w[p + ".dense_4h_to_h.bias"] if bias else 0)
+
+    x = x + (ffn(rms(x, "t.h.0.n_mlp"), "t.h.0.mlp", True) + attn(rms(x, "t.h.0.n_attn"), "t.h.0.attn", "tail"))
+    r = x + attn(rms(x, "t.h.1.n1"), "t.h.1.attn", "interleaved")
+    x = r + ffn(rms(r, "t.h.1.n2"), "t.h.1.mlp", False)
+    a = rms(x, "t.h.2.n")
+    x = x + (ffn(a, "t.h.2.mlp", False) + attn(a, "t.h.2.attn", "tail"))
+    return rms(x, "t.final") @ w["t.embed.weight"].T
+
+
+@pytest.mark.parametrize("dtype,rel", [("float32", 5e-5), ("bfloat16", helpers.REL_BF16)])
+def test_toy_architecture_with_a_norm_of_its_own(tmp_path, dtype, rel):
+    """A norm without mean and bias, defined in this file with the plain interface alone, in every place a norm
+    stands: the two norms of a parallel block, the one norm of another, both norms of a sequential block (whose
+    input may arrive as a sum that is not formed yet) and the final norm on the wanted rows."""
+    from safetensors.torch import load_file
+
+    from pytorch_transformers_amd import AutoModelForCausalLM
+    from pytorch_transformers_amd.config import register, unregister
+    from pytorch_transformers_amd.engine.replay import Replayer
+    from pytorch_transformers_amd.weights import write_random_model
+
+    NormConfig, build = _define_norm_toy()
+    register("toy-norm", NormConfig, build, exist_ok=True)
+    try:
+        cfg = NormConfig()
+        folder = write_random_model(str(tmp_path / "norm"), cfg, seed=14, std=0.15, noise=0.1)
+        w = {k: v.double() for k, v in load_file(f"{folder}/model.safetensors").items()}
+        assert "t.h.0.n_attn.weight" in w and "t.h.0.n_attn.bias" not in w
+        model = AutoModelForCausalLM.from_pretrained(folder, dtype=dtype)
+        reqs = helpers.make_requests(cfg.vocab_size, [11, 40, 70, 5], seed=4)
+        want = {rid: _plain_norm_toy(cfg, w, toks).float() for rid, toks in reqs.items()}
+        rp = Replayer(model, 1024, max_slots=4)
+        for name, records in (("whole", helpers.schedule_whole(reqs)), ("tail", helpers.schedule_tail(reqs, 16)),
+                              ("batches", helpers.schedule_batches(reqs, 3))):
+            got = helpers.run_schedule(rp, records)
+            for rid in reqs:
+                helpers.assert_close(got[rid], want[rid], rel, f"norm toy {dtype} {name} {rid}")
+    finally:
+        unregister("toy-norm")
