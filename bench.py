@@ -182,7 +182,8 @@ def run_prefill(model, T, reps=3, seed=1):
 
     g = torch.Generator().manual_seed(seed)
     prompt = torch.randint(0, model.vocab_size, (T,), generator=g).tolist()
-    cache = model.new_cache((T + 63) // 64 * 64, max_slots=1)
+    page = model.page_size
+    cache = model.new_cache((T + page - 1) // page * page, max_slots=1)
     best = None
     for r in range(reps + 1):
         slot = cache.alloc()
@@ -248,7 +249,8 @@ def decode_kernels(model, ops, sampler_cls, gen_cfg, cfg, dtype, elem, batch, pr
 
     g = torch.Generator().manual_seed(3)
     prompts = torch.randint(0, model.vocab_size, (batch, prompt_len), generator=g).tolist()
-    cache = model.new_cache(batch * ((prompt_len + 8 + 63) // 64 * 64), max_slots=batch)
+    page = model.page_size
+    cache = model.new_cache(batch * ((prompt_len + 8 + page - 1) // page * page), max_slots=batch)
     slots = [cache.alloc() for _ in range(batch)]
     model.step(cache, slots, prompts, "last")
     per_layer_kv = batch * (prompt_len + 1) * 2 * cfg.kv_heads * cfg.head_dim * elem
@@ -264,7 +266,8 @@ def prefill_kernels(model, ops, cfg, dtype, T):
 
     g = torch.Generator().manual_seed(4)
     prompt = torch.randint(0, model.vocab_size, (T,), generator=g).tolist()
-    cache = model.new_cache((T + 63) // 64 * 64 * 2, max_slots=2)
+    page = model.page_size
+    cache = model.new_cache((T + page - 1) // page * page * 2, max_slots=2)
 
     def step():
         slot = cache.alloc()
