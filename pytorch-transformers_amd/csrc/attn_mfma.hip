@@ -123,7 +123,12 @@ __global__ __launch_bounds__(64 * W * KS, OCC) void attn_mfma_kernel(
     const int lane = threadIdx.x & 63, c = lane & 15, gq = lane >> 4;
     const int wave = KS > 1 ? 0 : __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // which columns of the workgroup
     const int kw = KS > 1 ? threadIdx.x >> 6 : 0;     // which blocks of the keys
-    const int seq = blockIdx.z / n_splits, split = blockIdx.z % n_splits;
+    // Ranges of keys are handed out range-major: the first ranges of every sequence, which all of them have whole,
+    // start first, and the last ones, which are short or empty for most sequences, fill the launch's end.  (Sequence-
+    // major, 32 sequences of 16,405 keys in ranges of 1,024 left two whole ranges to start when the first ones ended:
+    // 45.8 us against 30.3 us at 16,384 keys.)
+    const int n_seqs_z = gridDim.z / n_splits;
+    const int seq = blockIdx.z % n_seqs_z, split = blockIdx.z / n_seqs_z;
     const int kvh = blockIdx.y, g = nh / nkv;
     const int t0 = cu_tokens[seq], n_new = cu_tokens[seq + 1] - t0, start = seq_start[seq];
     const int ncols = n_new * g, n_groups = (ncols + 16 * CT * W - 1) / (16 * CT * W);
