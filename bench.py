@@ -12,6 +12,8 @@ prefill of 2,048 tokens under ``prefill``, the decode step's HBM roofline under 
 * ``decode_b1`` / ``decode_b8`` / ``decode_b64``: tokens a second over the range of contexts that the
   configuration names, every decode step from 1,024 tokens to 2,048 in one run; ``decode_b64_ctx1568`` and so on
   are short runs around three contexts of that range; each with ``..._frac``, the fraction of the HBM roofline;
+* ``decode_b8_ctx4128`` ... ``decode_b32_ctx16416``: short runs at batch 8 and 32 around contexts of 4,128, 8,224 and
+  16,416 tokens, where the live sequences' keys and values weigh as much as the weights;
 * ``decode_b8_untuned``: the same step with the built-in choices between kernels, before ``model.tune()`` has
   timed any (what a process runs that neither tunes nor loads a tuning table);
 * ``falcon11b_...`` / ``falcon40b_...``: decode at batch 8 and 64 and one batch of whole requests of unequal
@@ -147,9 +149,17 @@ def run_decode(model, sampler_cls, gen_cfg, batch, prompt_len, steps, warmup, se
 RANGE_CONTEXTS = (1056, 1568, 2016)
 
 
-def decode_over_range(model, sampler_cls, gen_cfg, cfg, elem, batch, steps=16, warmup=4, contexts=RANGE_CONTEXTS):
+# Contexts past the metric's range (the configuration's own limit is 2,048 positions; rotation has no limit of its
+# own): where the keys and values of the live sequences weigh as much as the weights.  Clear of the captured steps'
+# exchanges, as above.
+LONG_CONTEXTS = (4128, 8224, 16416)
+LONG_BATCHES = (8, 32)
+
+
+def decode_over_range(model, sampler_cls, gen_cfg, cfg, elem, batch, steps=16, warmup=4, contexts=RANGE_CONTEXTS,
+                      mean=True):
     """Decode steps of ``batch`` sequences timed around each of ``contexts``; returns flat figures: tokens a second
-    and fraction of the HBM roofline at each context, and over the range (the mean of the step times)."""
+    and fraction of the HBM roofline at each context, and (``mean``) over the range (the mean of the step times)."""
     out, ms_all, frac_all = {}, [], []
     for c in contexts:
         dt, mean_ctx, _ = run_decode(model, sampler_cls, gen_cfg, batch, 0, steps, warmup, seed=c,
@@ -160,6 +170,8 @@ def decode_over_range(model, sampler_cls, gen_cfg, cfg, elem, batch, steps=16, w
         out[f"decode_b{batch}_ctx{c}_frac"] = round(gbs / HBM_PEAK_GBS, 4)
         ms_all.append(ms)
         frac_all.append(gbs / HBM_PEAK_GBS)
+    if not mean:
+        return out
     mean_ms = sum(ms_all) / len(ms_all)
     out[f"decode_b{batch}"] = round(batch / mean_ms * 1e3, 2)
     out[f"decode_b{batch}_frac"] = round(sum(f * m for f, m in zip(frac_all, ms_all)) / sum(ms_all), 4)
@@ -449,6 +461,11 @@ def main():
             points.update(decode_over_range(model, Sampler, gen_cfg, cfg, elem, b))
             # ... and what the metric names: every step from prompts of 1,024 tokens to 2,048, in place of the mean of three
             points.update(decode_whole_range(model, Sampler, gen_cfg, cfg, elem, b, 1024, 2048))
+        if args.sizes == "7b" and args.layers == full_layers:  # long contexts: decode_b8_ctx4128 ... decode_b32_ctx16416
+            model.tune(prompt_lens=(), batches=LONG_BATCHES, contexts=LONG_CONTEXTS)
+            for b in LONG_BATCHES:
+                points.update(decode_over_range(model, Sampler, gen_cfg, cfg, elem, b, steps=12, warmup=3,
+                                                contexts=LONG_CONTEXTS, mean=False))
         out["points"] = points
         if args.dtype == "bf16":
             out["kernels"] = {
