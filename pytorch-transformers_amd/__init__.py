@@ -5,7 +5,10 @@ from .config import AutoConfig, ConfigError, FalconConfig, GenerationConfig, reg
 from .engine import falcon as _falcon  # registers model_type "falcon"  # noqa: F401
 from .auto import AutoModelForCausalLM
 from .pipeline import TextGenerationPipeline, pipeline
+from .sampling.custom import LogitsProcessor, LogitsProcessorList, StoppingCriteria, StoppingCriteriaList
+from .streamers import BaseStreamer, TextIteratorStreamer, TextStreamer
 
 __version__ = "0.1.0"
-__all__ = ["AutoConfig", "AutoModelForCausalLM", "ConfigError", "FalconConfig", "GenerationConfig", "TextGenerationPipeline",
-           "pipeline", "register"]
+__all__ = ["AutoConfig", "AutoModelForCausalLM", "BaseStreamer", "ConfigError", "FalconConfig", "GenerationConfig",
+           "LogitsProcessor", "LogitsProcessorList", "StoppingCriteria", "StoppingCriteriaList", "TextGenerationPipeline",
+           "TextIteratorStreamer", "TextStreamer", "pipeline", "register"]

@@ -67,12 +67,19 @@ def generate(model, prompts: Sequence[Sequence[int]], generation_config: Optiona
              batch_size: Optional[int] = None, sampler=None, streamer=None, cache=None,
              rng_ids: Optional[Sequence[int]] = None, tokenizer=None, keep_slots: bool = False,
              slots: Optional[Sequence[int]] = None, rng_step_start: Optional[Sequence[int]] = None,
+             logits_processor: Optional[Sequence] = None, stopping_criteria: Optional[Sequence] = None,
              **kwargs) -> Union[List[List[int]], GenerateOutput]:
     """Generate for every prompt (a list of token ids); returns prompt + new tokens per prompt.
 
     ``generation_config`` defaults to the model's; keyword arguments override its fields
-    (:1543-1545).  ``streamer`` is called as ``streamer(index, token)`` for every new token and
-    ``streamer.end()`` if it has one.  ``rng_ids`` name each prompt's random stream (default: its
+    (:1543-1545).  ``streamer``: an object with ``put`` and ``end`` as the reference's streamers have them
+    (src/transformers/generation/streamers.py:23-39: ``put`` is given the prompt first and then every new token, one
+    prompt per call; src/transformers/generation/utils.py:2087, :3288, :3301-3302), or a callable ``streamer(index, token)`` for any number of prompts
+    (and ``streamer.end()`` if it has one).  ``logits_processor``: the caller's own processors, ``processor(input_ids,
+    scores) -> scores``, run behind those that the options switch on and in front of temperature and the top-k
+    family (:1038-1039); ``stopping_criteria``: ``criterion(input_ids, scores)`` gives a flag per row (or one for
+    all), and a row whose flag is set ends with the token just chosen (:1136, stopping_criteria.py:491-497).  Both
+    are handed the rows' ids so far as one int64 tensor, padded on the left with ``pad_token_id`` (0 if none).  ``rng_ids`` name each prompt's random stream (default: its
     index), so that a prompt draws the same tokens in any batch.  ``tokenizer`` (anything with
     ``decode(ids) -> str``) is needed for ``stop_strings`` only: a sequence ends with the token that
     completes one of them in the text of its new tokens (src/transformers/generation/utils.py:1118-1125,
@@ -148,6 +155,10 @@ def generate(model, prompts: Sequence[Sequence[int]], generation_config: Optiona
             "There are one or more stop strings, either in the arguments to `generate` or in the model's generation "
             "config, but we could not locate a tokenizer. When generating with stop strings, you must pass the model's "
             "tokenizer to the `tokenizer` argument of `generate`.")
+    logits_processor, stopping_criteria = list(logits_processor or []), list(stopping_criteria or [])
+    puts = streamer is not None and hasattr(streamer, "put")
+    if puts and len(prompts) != 1:
+        raise ValueError("TextStreamer only supports batch size 1")  # streamers.py:87-88
     want_scores, want_logits = bool(cfg.output_scores), bool(cfg.output_logits)
     out_tokens: List[List[int]] = [[] for _ in prompts]
     out_scores = [[] for _ in prompts] if want_scores else None
@@ -158,7 +169,11 @@ def generate(model, prompts: Sequence[Sequence[int]], generation_config: Optiona
     # step is launched from the tokens on the device before the host has read them.
     ahead = (bool(getattr(model, "steps_ahead", False)) and getattr(sampler, "needs_histories", True) is False
              and not want_scores and not want_logits and streamer is None and not stop_strings
-             and cfg.max_time is None and not keep_slots)
+             and cfg.max_time is None and not keep_slots and not logits_processor and not stopping_criteria)
+    pad = 0 if cfg.pad_token_id is None else int(cfg.pad_token_id)
+    custom = dict(extra_processors=logits_processor, pad_token_id=pad) if logits_processor else {}
+    if puts:
+        streamer.put(_ids_tensor(prompts[0]))
 
     def done_with(i: int, slot: int) -> None:
         if keep_slots:
@@ -189,21 +204,26 @@ def generate(model, prompts: Sequence[Sequence[int]], generation_config: Optiona
                     logits, rng_seq=[ids[i] for i in live], rng_step=[first_draw[i] + step_no for i in live],
                     histories=[prompts[i] + out_tokens[i] for i in live], suppress_eos=[too_short] * len(live),
                     new_counts=[len(out_tokens[i]) for i in live],
-                    need_scores=want_scores, **_step_extras(sampler, step_no, new_budget))
+                    need_scores=want_scores or bool(stopping_criteria), **custom,
+                    **_step_extras(sampler, step_no, new_budget))
                 step_no += 1
                 timed_out = cfg.max_time is not None and (time.time() - t0) > cfg.max_time  # stopping_criteria.py:87-107
                 still = []
                 for row, i in enumerate(live):
-                    tok = int(tokens[row])
-                    out_tokens[i].append(tok)
+                    out_tokens[i].append(int(tokens[row]))
+                halted = _criteria_flags(stopping_criteria, [prompts[i] + out_tokens[i] for i in live], scores, pad)
+                for row, i in enumerate(live):
+                    tok = out_tokens[i][-1]
                     if want_scores:
                         out_scores[i].append(scores[row].clone())
                     if want_logits:
                         out_logits[i].append(logits[row].clone())
-                    if streamer is not None:
+                    if puts:
+                        streamer.put(_ids_tensor([tok]))
+                    elif streamer is not None:
                         streamer(i, tok)
                     said_stop = bool(stop_strings) and _ends_with_stop(tokenizer, out_tokens[i], stop_strings)
-                    if tok in eos or step_no >= new_budget or timed_out or said_stop:
+                    if tok in eos or step_no >= new_budget or timed_out or said_stop or halted[row]:
                         done_with(i, slot_of.pop(i))
                     else:
                         feed[i] = [tok]
@@ -226,6 +246,35 @@ def generate(model, prompts: Sequence[Sequence[int]], generation_config: Optiona
     if cfg.return_dict_in_generate:
         return GenerateOutput(sequences, out_scores, out_logits)
     return sequences
+
+
+def _ids_tensor(ids: Sequence[int]):
+    import torch
+
+    return torch.tensor(list(ids), dtype=torch.long)
+
+
+def _criteria_flags(criteria: Sequence, sequences: Sequence[Sequence[int]], scores, pad: int) -> List[bool]:
+    """Which of the rows the caller's stopping criteria end now: each criterion is called with the rows' ids (the
+    token just chosen included) and the step's scores, and gives a flag per row or one for all rows; a row ends if
+    any criterion says so (src/transformers/generation/stopping_criteria.py:491-497)."""
+    flags = [False] * len(sequences)
+    if not criteria:
+        return flags
+    import torch
+
+    from ..sampling.sampler import left_padded
+
+    ids = left_padded(sequences, pad, scores.device if scores is not None else "cpu")
+    for criterion in criteria:
+        said = criterion(ids, scores)
+        said = said.reshape(-1).tolist() if isinstance(said, torch.Tensor) else [bool(said)]
+        if len(said) == 1:
+            said = said * len(sequences)
+        if len(said) != len(sequences):
+            raise ValueError(f"the stopping criterion {criterion!r} gave {len(said)} flags for {len(sequences)} rows")
+        flags = [a or bool(b) for a, b in zip(flags, said)]
+    return flags
 
 
 def _step_extras(sampler, step: int, new_budget: int) -> dict:

@@ -63,13 +63,25 @@ class Sampler:
     def sample(self, logits: torch.Tensor, *, rng_seq: Sequence[int], rng_step: Sequence[int],
                histories: Optional[Sequence[Sequence[int]]] = None, suppress_eos: Optional[Sequence[bool]] = None,
                uniforms: Optional[Sequence[float]] = None, new_counts: Optional[Sequence[int]] = None,
-               need_scores: bool = True, ahead: bool = False, force: bool = False, decay: Optional[float] = None):
+               need_scores: bool = True, ahead: bool = False, force: bool = False, decay: Optional[float] = None,
+               extra_processors: Optional[Sequence] = None, pad_token_id: Optional[int] = None):
         """Tokens for the rows of ``logits`` and the processed scores ``[rows, vocab]`` (None if not needed
         and the choice could be made without forming them).  ``histories`` are the rows' ids so far (prompt and
         new tokens) and ``new_counts`` how many of them are new; the repetition penalty and the options that forbid
         tokens read them.  ``ahead``: the tokens come back as a ``TokensAhead``, without a wait for the GPU
-        (only where ``needs_histories`` is false)."""
+        (only where ``needs_histories`` is false).
+
+        ``extra_processors``: the caller's own processors, each called as ``processor(input_ids, scores) -> scores``
+        with the rows' ids so far as one tensor, padded on the left with ``pad_token_id``, and the scores ``[rows,
+        vocab]`` in 32-bit on the device.  They run where the reference puts them: behind the processors that the
+        options switch on and in front of temperature, the top-k / top-p family and the renormalization
+        (src/transformers/generation/utils.py:1038-1039), which then takes two launches instead of one."""
         R = logits.shape[0]
+        if extra_processors:
+            if histories is None:
+                raise ValueError("the caller's processors are given the rows' ids so far: histories are needed")
+            if ahead:
+                raise ValueError("tokens ahead of the host cannot pass through the caller's processors")
         if ahead and self.needs_histories:
             raise ValueError("tokens ahead of the host cannot be chosen by options that read the tokens so far")
         suppress = self._eos_dev is not None and suppress_eos is not None and any(suppress_eos)
@@ -92,7 +104,7 @@ class Sampler:
             bias_lists = [self.biases.biases(histories[r] if histories is not None else None) for r in range(R)]
         if (not need_scores and not self.do_sample and self.penalty == 1.0 and not suppress and ban_lists is None
                 and not self.config.remove_invalid_values and not self.config.renormalize_logits
-                and bias_lists is None and not force and decay is None):
+                and bias_lists is None and not force and decay is None and not extra_processors):
             # greedy with no processor in the way: nothing to upload, one argmax kernel
             chosen = ops.sample(logits, do_sample=False, need_scores=False)[0]
             return (TokensAhead(chosen) if ahead else chosen.tolist()), None
@@ -126,25 +138,50 @@ class Sampler:
             u = torch.tensor(list(uniforms), dtype=torch.float32).pin_memory().to(self.device, non_blocking=True)
         else:
             u = torch.tensor(list(uniforms), dtype=torch.float32, device=self.device)
-        tokens, scores = ops.sample(
-            logits, do_sample=self.do_sample, temperature=self.temperature, top_k=self.top_k, top_p=self.top_p,
-            min_p=self.min_p, typical_p=self.typical_p, epsilon_cutoff=self.epsilon_cutoff, eta_cutoff=self.eta_cutoff,
+        warpers = dict(do_sample=self.do_sample, temperature=self.temperature, top_k=self.top_k, top_p=self.top_p,
+                       min_p=self.min_p, typical_p=self.typical_p, epsilon_cutoff=self.epsilon_cutoff,
+                       eta_cutoff=self.eta_cutoff, renorm=self.config.renormalize_logits)
+        draws = dict(seed=self.config.seed, rng_seq=views[0], rng_step=views[1], uniforms=u)
+        processors = dict(
             penalty=self.penalty, hist=views[4] if use_hist else None,
             hist_off=views[3] if use_hist else None, ban=views[n_before + 1] if ban_lists is not None else None,
             ban_off=views[n_before] if ban_lists is not None else None, eos=self._eos_dev,
             suppress=views[2] if (self._eos_dev is not None and suppress_eos is not None and any(suppress_eos)) else None,
-            remove_invalid=self.config.remove_invalid_values, renorm=self.config.renormalize_logits,
-            seed=self.config.seed, rng_seq=views[0], rng_step=views[1], uniforms=u, need_scores=need_scores,
+            remove_invalid=self.config.remove_invalid_values,
             bias_off=views[n_bias_at] if bias_lists is not None else None,
             bias_tok=views[n_bias_at + 1] if bias_lists is not None else None,
             bias_val=views[n_bias_at + 2].view(torch.float32) if bias_lists is not None else None,
             forced=self._forced_dev if force else None, decay=decay)
+        if not extra_processors:
+            tokens, scores = ops.sample(logits, need_scores=need_scores, **warpers, **draws, **processors)
+        else:
+            # the options' processors alone (the greedy form of the launch returns their scores untouched by any
+            # warper), the caller's on that tensor, then the warpers and the choice
+            _, scores = ops.sample(logits, do_sample=False, need_scores=True, **draws, **processors)
+            ids = left_padded(histories, 0 if pad_token_id is None else int(pad_token_id), self.device)
+            for proc in extra_processors:
+                scores = proc(ids, scores)
+                if not (isinstance(scores, torch.Tensor) and scores.shape == logits.shape):
+                    raise ValueError(f"the processor {proc!r} must return scores of shape {tuple(logits.shape)}")
+            scores = scores.to(device=self.device, dtype=torch.float32).contiguous()
+            tokens, scores = ops.sample(scores, need_scores=need_scores, **warpers, **draws)
         return (TokensAhead(tokens) if ahead else tokens.tolist()), scores
 
     @property
     def needs_histories(self) -> bool:
         """Whether a choice reads the sequence's tokens so far (which the host then has to have seen)."""
         return bool(self.bans) or self.penalty != 1.0 or self.biases.needs_history
+
+
+def left_padded(histories: Sequence[Sequence[int]], pad: int, device) -> torch.Tensor:
+    """The rows' ids as the reference's rectangular ``input_ids``: int64 ``[rows, longest]``, shorter rows padded on
+    the left."""
+    longest = max(len(h) for h in histories)
+    ids = np.full((len(histories), longest), int(pad), dtype=np.int64)
+    for r, h in enumerate(histories):
+        if len(h):
+            ids[r, longest - len(h):] = np.asarray(h, dtype=np.int64)
+    return torch.from_numpy(ids).to(device)
 
 
 def philox_uniform(seed: int, seq: int, step: int) -> float:

@@ -484,11 +484,13 @@ def exponential_decay(scores, cur_len, prompt_len, start_index, factor, eos_ids)
 
 def process(scores, history, *, do_sample, temperature_=1.0, top_k_=0, top_p_=1.0, min_p_=None, typical_p_=None,
             epsilon_cutoff_=None, eta_cutoff_=None, repetition_penalty_=1.0, suppress_ids=(), no_repeat_ngram_size_=0,
-            bad_words_ids_=None, eos_ids_=(), sequence_bias_=None, forced_eos_=None, exponential_decay_=None):
+            bad_words_ids_=None, eos_ids_=(), sequence_bias_=None, forced_eos_=None, exponential_decay_=None,
+            custom_=()):
     """Processors in the order the reference builds them (src/transformers/generation/utils.py:898-1097):
     sequence bias, repetition penalty, no-repeat n-grams, bad words, minimum length, forced last token
     (``forced_eos_``: (max_length, ids)), the growing bonus on EOS (``exponential_decay_``: (prompt length, start index,
-    factor)), then (sampling only) temperature, top-k, top-p, min-p, typical-p, epsilon and eta cut-offs."""
+    factor)), the caller's own processors (``custom_``: functions of (history, scores), :1038-1039), then (sampling
+    only) temperature, top-k, top-p, min-p, typical-p, epsilon and eta cut-offs."""
     s = scores
     if sequence_bias_:
         s = sequence_bias(s, history, sequence_bias_)
@@ -504,6 +506,8 @@ def process(scores, history, *, do_sample, temperature_=1.0, top_k_=0, top_p_=1.
         s = forced_eos(s, len(history), forced_eos_[0], forced_eos_[1])
     if exponential_decay_ is not None:
         s = exponential_decay(s, len(history), exponential_decay_[0], exponential_decay_[1], exponential_decay_[2], eos_ids_)
+    for fn in custom_:
+        s = fn(list(history), s)
     if do_sample:
         if temperature_ is not None and temperature_ != 1.0:
             s = temperature(s, temperature_)
@@ -534,7 +538,7 @@ def pick(scores, u: Optional[float]):
 
 def generate(cfg, w, prompt: Sequence[int], max_new_tokens: int, *, eos_ids=(), min_new_tokens=0,
              uniforms: Optional[Sequence[float]] = None, forced_eos_ids=None, exponential_decay_length_penalty=None,
-             **proc) -> List[int]:
+             stop_when=(), **proc) -> List[int]:
     """One sequence, recomputed whole at every step (no cache); returns the new tokens, EOS included
     (loop of src/transformers/generation/utils.py:3220-3296, stop test stopping_criteria.py:446-467)."""
     seq = list(prompt)
@@ -551,6 +555,6 @@ def generate(cfg, w, prompt: Sequence[int], max_new_tokens: int, *, eos_ids=(), 
         tok = pick(s, None if uniforms is None else uniforms[step])
         seq.append(tok)
         new.append(tok)
-        if tok in eos_ids:
+        if tok in eos_ids or any(fn(list(seq)) for fn in stop_when):  # the caller's criteria see the new token too
             break
     return new

@@ -365,3 +365,141 @@ def test_what_needs_the_tokens_on_the_host_keeps_the_loop_that_waits():
     log = []
     generate(AheadModel(log), [[1, 2], [3]], GenerationConfig(max_new_tokens=3), sampler=AheadSampler(log), streamer=lambda i, t: None)
     assert not any(what == "step from" for what, _ in log)
+
+
+# ---- the caller's own stopping criteria and streamers ------------------------------------------------------------
+
+def test_a_callers_stopping_criterion_ends_its_rows_only():
+    """A criterion is handed the rows' ids, the new token included, padded on the left, and the step's scores; the
+    rows it flags end with that token and give their slots back, the others go on."""
+    m = ScriptedModel()
+    prompts = [[1, 2, 3], [4], [5, 6]]
+    seen = []
+
+    def has_an_even_sum(input_ids, scores):
+        seen.append((input_ids.clone(), None if scores is None else tuple(scores.shape)))
+        return (input_ids.sum(-1) % 4 == 0)
+
+    out = generate(m, prompts, GenerationConfig(max_new_tokens=6, pad_token_id=0), sampler=ArgmaxSampler(),
+                   stopping_criteria=[has_an_even_sum])
+    for p, o in zip(prompts, out):
+        want = list(p)
+        for _ in range(6):
+            want.append(sum(want) % V)
+            if sum(want) % 4 == 0:
+                break
+        assert o == want
+    assert len({len(o) - len(p) for p, o in zip(prompts, out)}) > 1, "the case must end its rows at different steps"
+    first_ids, first_shape = seen[0]
+    assert first_ids.dtype == torch.long and first_ids.shape == (3, 4) and first_shape == (3, V)
+    assert first_ids[1].tolist() == [0, 0, 4, 4] and first_ids[0].tolist() == [1, 2, 3, 6]  # left-padded with pad_token_id
+    assert all(not c.live_slots() and c.free_pages() == c.num_pages for c in m.caches)
+    # one flag for all rows ends all of them
+    out = generate(ScriptedModel(), prompts, GenerationConfig(max_new_tokens=6), sampler=ArgmaxSampler(),
+                   stopping_criteria=[lambda ids, scores: ids.shape[1] >= 4])
+    assert [len(o) for o in out] == [4, 2, 3]
+    with pytest.raises(ValueError, match="gave 2 flags for 3 rows"):
+        generate(ScriptedModel(), prompts, GenerationConfig(max_new_tokens=2), sampler=ArgmaxSampler(),
+                 stopping_criteria=[lambda ids, scores: torch.tensor([True, False])])
+
+
+def test_the_callers_processors_reach_the_sampler_with_the_pad_id():
+    class Recording(ArgmaxSampler):
+        def sample(self, logits, *, extra_processors=None, pad_token_id=None, **kw):
+            self.extra = (extra_processors, pad_token_id)
+            return super().sample(logits, **kw)
+
+    s = Recording()
+    fn = lambda ids, scores: scores
+    generate(ScriptedModel(), [[1, 2]], GenerationConfig(max_new_tokens=1, pad_token_id=7), sampler=s, logits_processor=[fn])
+    assert s.extra == ([fn], 7)
+    s = ArgmaxSampler()  # without processors a sampler that knows nothing of them is called as before
+    generate(ScriptedModel(), [[1, 2]], GenerationConfig(max_new_tokens=1), sampler=s)
+
+
+class WordTokenizer:
+    """id -> a word; decoding joins with spaces, except that id 0 is a line break and ids from 40 on are CJK."""
+
+    def decode(self, ids, **kw):
+        self.kw = kw
+        out = ""
+        for t in ids:
+            if t == 0:
+                out += "\n"
+            elif t >= 40:
+                out += chr(0x4E00 + t)
+            else:
+                out += ("" if out == "" or out.endswith("\n") else " ") + f"w{t}"
+        return out
+
+
+def test_text_streamer_shows_whole_words_and_flushes_at_line_breaks(capsys):
+    from pytorch_transformers_amd import TextStreamer
+
+    st = TextStreamer(WordTokenizer(), skip_special_tokens=True)
+    st.put(torch.tensor([[1, 2]]))  # the prompt: "w1 w2" -> up to the last space
+    assert capsys.readouterr().out == "w1 "
+    st.put(torch.tensor([3]))
+    assert capsys.readouterr().out == "w2 "
+    st.put(torch.tensor([0]))  # a line break flushes, and decoding starts anew behind it
+    assert capsys.readouterr().out == "w3\n"
+    st.put(torch.tensor([4]))
+    assert capsys.readouterr().out == ""
+    st.put(torch.tensor([41]))  # a character of a script without spaces is shown at once, with what was held back
+    assert capsys.readouterr().out == "w4" + chr(0x4E00 + 41)
+    st.put(torch.tensor([5]))
+    st.end()
+    assert capsys.readouterr().out == " w5\n"
+    assert st.tokenizer.kw == {"skip_special_tokens": True}
+    with pytest.raises(ValueError, match="batch size 1"):
+        st.put(torch.tensor([[1], [2]]))
+    quiet = TextStreamer(WordTokenizer(), skip_prompt=True)
+    quiet.put(torch.tensor([1, 2]))
+    quiet.put(torch.tensor([3]))
+    quiet.put(torch.tensor([4]))
+    quiet.end()
+    assert capsys.readouterr().out == "w3 w4\n"
+    quiet.put(torch.tensor([9]))  # the next call's prompt is skipped again
+    quiet.put(torch.tensor([5]))
+    quiet.end()
+    assert capsys.readouterr().out == "w5\n"
+
+
+def test_generate_feeds_a_streamer_the_prompt_then_every_token_and_iterates_in_a_thread():
+    import threading
+
+    from pytorch_transformers_amd import TextIteratorStreamer
+
+    class Tape:
+        def __init__(self):
+            self.got, self.ended = [], 0
+
+        def put(self, value):
+            assert value.dtype == torch.long and value.dim() == 1
+            self.got.append(value.tolist())
+
+        def end(self):
+            self.ended += 1
+
+    tape = Tape()
+    out = generate(ScriptedModel(), [[1, 2, 3]], GenerationConfig(max_new_tokens=3), sampler=ArgmaxSampler(), streamer=tape)
+    assert tape.got == [[1, 2, 3]] + [[t] for t in out[0][3:]] and tape.ended == 1
+    with pytest.raises(ValueError, match="batch size 1"):
+        generate(ScriptedModel(), [[1], [2]], GenerationConfig(max_new_tokens=1), sampler=ArgmaxSampler(), streamer=Tape())
+    it = TextIteratorStreamer(WordTokenizer(), skip_prompt=True, timeout=30)
+    th = threading.Thread(target=generate, args=(ScriptedModel(), [[1, 2, 3]], GenerationConfig(max_new_tokens=4)),
+                          kwargs=dict(sampler=ArgmaxSampler(), streamer=it))
+    th.start()
+    text = "".join(piece for piece in it)
+    th.join()
+    assert text == WordTokenizer().decode(expected([1, 2, 3], 4)[3:])
+
+
+def test_processor_and_criteria_lists_are_callable():
+    from pytorch_transformers_amd import LogitsProcessorList, StoppingCriteriaList
+
+    ids, scores = torch.tensor([[1, 2], [3, 4]]), torch.zeros(2, 5)
+    procs = LogitsProcessorList([lambda i, s: s + 1.0, lambda i, s: s * i.sum(-1, keepdim=True)])
+    assert procs(ids, scores).tolist() == [[3.0] * 5, [7.0] * 5]
+    crit = StoppingCriteriaList([lambda i, s: i[:, -1] == 2, lambda i, s: False])
+    assert crit(ids, scores).tolist() == [True, False]

@@ -814,3 +814,58 @@ def test_greedy_without_scores_is_an_argmax():
         assert tok.tolist() == want
         full, _ = ops.sample(logits, do_sample=False)
         assert full.tolist() == want
+
+
+def test_the_callers_processors_and_criteria_through_generate_equal_plain(folders):
+    """Tiny B in 32-bit, prompts of 2 to 19 ids in one batch.  The caller's processor (here: odd ids are forbidden and
+    the id behind the last one is raised) runs behind the options' processors (a repetition penalty) and in front of
+    the warpers: with top-k 1 a draw can only take the token the processor has made the best, which a processor run
+    behind the warpers could not have made it.  A criterion ends its rows with the token that fulfils it."""
+    from pytorch_transformers_amd import AutoModelForCausalLM, GenerationConfig, LogitsProcessorList, StoppingCriteriaList
+
+    cfg, w = P.read_model(folders["B"])
+    V = cfg["vocab_size"]
+    g = torch.Generator().manual_seed(5)
+    prompts = [torch.randint(0, V, (n,), generator=g).tolist() for n in (2, 19, 7)]
+    model = AutoModelForCausalLM.from_pretrained(folders["B"], dtype="float32")
+    calls = []
+
+    def even_only(input_ids, scores):
+        assert input_ids.dtype == torch.long and input_ids.is_cuda and scores.dtype == torch.float32
+        assert scores.shape == (input_ids.shape[0], V)
+        calls.append(tuple(input_ids.shape))
+        out = scores.clone()
+        out[:, 1::2] = float("-inf")
+        return out
+
+    def even_only_plain(history, s):
+        s = s.clone()
+        s[1::2] = float("-inf")
+        return s
+
+    gen = GenerationConfig(max_new_tokens=12, do_sample=False, repetition_penalty=1.3, eos_token_id=None, pad_token_id=0)
+    got = model.generate(prompts, gen, logits_processor=LogitsProcessorList([even_only]))
+    for p, o in zip(prompts, got):
+        assert o == p + P.generate(cfg, w, p, 12, repetition_penalty_=1.3, custom_=[even_only_plain])
+        assert all(t % 2 == 0 for t in o[len(p):])
+    assert calls[0] == (3, 19) and calls[1] == (3, 20)  # the rows' ids so far, as one rectangle
+
+    def raise_the_next_id(input_ids, scores):
+        out = scores.clone()
+        out[torch.arange(out.shape[0]), (input_ids[:, -1] + 1) % V] += 1e4
+        return out
+
+    drawn = model.generate(prompts, GenerationConfig(max_new_tokens=6, do_sample=True, top_k=1, temperature=0.7, seed=3,
+                                                     eos_token_id=None), logits_processor=[raise_the_next_id])
+    for p, o in zip(prompts, drawn):
+        assert o[len(p):] == [(p[-1] + k) % V for k in range(1, 7)]
+
+    ends_on_a_multiple_of_five = lambda input_ids, scores: input_ids[:, -1] % 5 == 0
+    stopped = model.generate(prompts, GenerationConfig(max_new_tokens=30, do_sample=False, eos_token_id=None),
+                             stopping_criteria=StoppingCriteriaList([ends_on_a_multiple_of_five]))
+    lens = set()
+    for p, o in zip(prompts, stopped):
+        want = P.generate(cfg, w, p, 30, stop_when=[lambda seq: seq[-1] % 5 == 0])
+        assert o == p + want
+        lens.add(len(want))
+    assert len(lens) > 1 and min(lens) < 30, f"rows must end at different steps, some by the criterion: {lens}"
