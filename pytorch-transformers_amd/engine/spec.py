@@ -7,7 +7,7 @@ one builder this package ships.
 from __future__ import annotations
 
 import dataclasses
-from typing import Any, List, Optional, Sequence, Tuple
+from typing import Any, Callable, List, Optional, Sequence, Tuple
 
 # how a tensor is held on the device
 MATRIX = "matrix"  # operand of a matrix product or a lookup table of activations: held in the compute dtype
@@ -28,6 +28,12 @@ class TensorSpec:
     init: str = INIT_NORMAL
     #: if the file lacks this tensor, use that other tensor's storage instead (tied output head)
     tied_to: Optional[str] = None
+    #: A file may hold this tensor in pieces instead (a checkpoint with separate query, key and value matrices for
+    #: a model that runs them as one): (name, shape) of each piece.  ``assemble`` makes the tensor of the pieces,
+    #: given in this order (None: joined along the first dimension).  A file that holds the tensor under its own
+    #: name is read as before; random weights are drawn and written whole.
+    pieces: Tuple[Tuple[str, Tuple[int, ...]], ...] = ()
+    assemble: Optional[Callable[[Sequence[Any]], Any]] = None
 
 
 # kinds of per-sequence storage a group of layers can ask for

@@ -21,10 +21,31 @@ from .linear import Linear, PendingProjection, QkvTail, TailDone
 from .positions import as_rotation, as_score_bias
 
 
+def fused_rows(num_heads: int, kv_heads: int, head_dim: int, qkv_layout: str):
+    """A function that lays the rows of separate query, key and value projections (heads in order) out as the fused
+    projection's in ``qkv_layout`` (the row orders of src/transformers/models/falcon/modeling_falcon.py:264-294):
+    ``grouped``: per KV head its query heads, its key, its value; ``tail``: all query heads, the key, the value
+    (one KV head); ``interleaved``: per head query, key, value (as many KV heads as heads).  All three are the
+    grouped order at their head counts."""
+    if (qkv_layout == "tail" and kv_heads != 1) or (qkv_layout == "interleaved" and kv_heads != num_heads):
+        raise ValueError(f"the {qkv_layout} layout does not go with {num_heads} heads and {kv_heads} kv heads")
+
+    def assemble(parts):
+        q, k, v = parts
+        rest = tuple(q.shape[1:])
+        per = [t.reshape(kv_heads, -1, *rest) for t in (q, k, v)]  # [kv head, its rows, ...]
+        return torch.cat(per, dim=1).reshape(-1, *rest)
+
+    return assemble
+
+
 class AttentionMixer(Part):
     def __init__(self, name: str, hidden_size: int, num_heads: int, kv_heads: int, head_dim: int, qkv_layout: str,
                  bias: bool, positions: Part, qkv_name: str = "query_key_value", out_name: str = "dense",
-                 window: int = 0):
+                 window: int = 0, qkv_pieces: Optional[Sequence[str]] = None):
+        """``qkv_pieces``: the names of separate query, key and value projections (``("q_proj", "k_proj", "v_proj")``)
+        that a weight file may hold in place of the fused one; their rows, heads in order, are laid out in
+        ``qkv_layout`` when the weights are read, and the model runs the fused product either way."""
         if num_heads % kv_heads:
             raise ValueError(f"heads ({num_heads}) must be a multiple of kv heads ({kv_heads})")
         if qkv_layout not in ops.QKV_LAYOUT_CODES:
@@ -40,7 +61,13 @@ class AttentionMixer(Part):
         #: of kind ``window`` with the same number, and gives back the pages that fall behind
         self.window = int(window)
         self.scale = 1.0 / math.sqrt(head_dim)  # modeling_falcon.py:250
-        self.qkv = Linear(f"{name}.{qkv_name}", hidden_size, (num_heads + 2 * kv_heads) * head_dim, bias)
+        pieces = assemble = None
+        if qkv_pieces is not None:
+            if len(qkv_pieces) != 3:
+                raise ValueError(f"{name}: qkv_pieces names the query, key and value projections, got {qkv_pieces!r}")
+            pieces = [(f"{name}.{n}", rows * head_dim) for n, rows in zip(qkv_pieces, (num_heads, kv_heads, kv_heads))]
+            assemble = fused_rows(num_heads, kv_heads, head_dim, qkv_layout)
+        self.qkv = Linear(f"{name}.{qkv_name}", hidden_size, (num_heads + 2 * kv_heads) * head_dim, bias, pieces, assemble)
         self.out = Linear(f"{name}.{out_name}", num_heads * head_dim, hidden_size, bias)
 
     def children(self) -> Sequence[Part]:

@@ -23,18 +23,27 @@ from .base import PartialProduct, Part
 
 
 class Linear(Part):
-    def __init__(self, name: str, in_features: int, out_features: int, bias: bool):
+    def __init__(self, name: str, in_features: int, out_features: int, bias: bool, pieces=None, assemble=None):
+        """``pieces``: (name, rows) of the matrices that a weight file may hold instead of this one (their ``.weight``
+        and ``.bias`` under those names), which ``assemble`` (None: one after the other) makes into this one by
+        their rows; the same function is applied to the biases."""
         self.name = name
         self.in_features = in_features
         self.out_features = out_features
         self.has_bias = bias
+        self.pieces = tuple((str(n), int(rows)) for n, rows in (pieces or ()))
+        self.assemble = assemble
         self.weight: Optional[torch.Tensor] = None
         self.bias: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> List[TensorSpec]:
-        specs = [TensorSpec(self.name + ".weight", (self.out_features, self.in_features), MATRIX, INIT_NORMAL)]
+        specs = [TensorSpec(self.name + ".weight", (self.out_features, self.in_features), MATRIX, INIT_NORMAL,
+                            pieces=tuple((n + ".weight", (rows, self.in_features)) for n, rows in self.pieces),
+                            assemble=self.assemble)]
         if self.has_bias:
-            specs.append(TensorSpec(self.name + ".bias", (self.out_features,), VECTOR, INIT_ZERO_NOISE))
+            specs.append(TensorSpec(self.name + ".bias", (self.out_features,), VECTOR, INIT_ZERO_NOISE,
+                                    pieces=tuple((n + ".bias", (rows,)) for n, rows in self.pieces),
+                                    assemble=self.assemble))
         return specs
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:

@@ -138,8 +138,11 @@ def load_weights(folder: str, specs: Sequence[TensorSpec], compute_dtype: torch.
     # ties after it has loaded (src/transformers/modeling_utils.py:1858-1884 called from :4368), which overwrites a
     # head that a file of a tied model carries.  The file's copy is neither read nor unexpected.
     tied_in_file = {mapping.pop(s.name) for s in specs if s.tied_to is not None and s.name in mapping}
+    # A tensor that the file does not hold under its own name may lie there in pieces
+    in_pieces = {s.name: _strip_or_add_prefix(files.keys(), [n for n, _ in s.pieces], base_prefix)
+                 for s in specs if s.pieces and s.name not in mapping}
 
-    used_file_names = set(mapping.values())
+    used_file_names = set(mapping.values()) | {f for found in in_pieces.values() for f in found.values()}
     unexpected = sorted(k for k in files if k not in used_file_names and k not in tied_in_file
                         and not k.endswith(_IGNORED_SUFFIXES))
     missing = []
@@ -148,29 +151,47 @@ def load_weights(folder: str, specs: Sequence[TensorSpec], compute_dtype: torch.
             continue
         if s.tied_to is not None and s.tied_to in mapping:
             continue
-        missing.append(s.name)
+        if s.name in in_pieces and in_pieces[s.name]:  # some pieces are there: the others are what is missing
+            missing.extend(n for n, _ in s.pieces if n not in in_pieces[s.name])
+            continue
+        missing.append(s.name if not s.pieces else f"{s.name} (or its pieces {', '.join(n for n, _ in s.pieces)})")
 
     wrong_shape, wrong_type = [], []
     handles = {}
     out: Dict[str, torch.Tensor] = {}
+
+    def read(spec, name, fname, shape):
+        """The file tensor ``fname`` if it has ``shape`` and the kind of ``spec``; else None, with the problem noted."""
+        path = files[fname]
+        if path not in handles:
+            handles[path] = safe_open(path, framework="pt")
+            _check_metadata(path, handles[path].metadata())
+        got = tuple(handles[path].get_slice(fname).get_shape())
+        if got != tuple(shape):
+            wrong_shape.append((name, got, tuple(shape)))
+            return None
+        t = handles[path].get_tensor(fname)
+        if (spec.kind == INT) == (t.dtype in _FLOAT_DTYPES):
+            wrong_type.append((name, str(t.dtype).replace("torch.", ""), "integer" if spec.kind == INT else "floating point"))
+            return None
+        return t
+
     try:
         for s in specs:
             fname = mapping.get(s.name)
-            if fname is None:
+            if fname is not None:
+                t = read(s, s.name, fname, s.shape)
+            elif s.name in in_pieces and len(in_pieces[s.name]) == len(s.pieces):
+                parts = [read(s, n, in_pieces[s.name][n], shape) for n, shape in s.pieces]
+                if any(part is None for part in parts):
+                    continue
+                t = s.assemble(parts) if s.assemble is not None else torch.cat(parts, dim=0)
+                if tuple(t.shape) != tuple(s.shape):
+                    raise ValueError(f"the pieces of {s.name} make a tensor of shape {tuple(t.shape)}, the model needs "
+                                     f"{tuple(s.shape)}: the model's own description of its pieces is wrong")
+            else:
                 continue
-            path = files[fname]
-            if path not in handles:
-                handles[path] = safe_open(path, framework="pt")
-                _check_metadata(path, handles[path].metadata())
-            sl = handles[path].get_slice(fname)
-            shape = tuple(sl.get_shape())
-            if shape != tuple(s.shape):
-                wrong_shape.append((s.name, shape, s.shape))
-                continue
-            t = handles[path].get_tensor(fname)
-            is_float = t.dtype in _FLOAT_DTYPES
-            if (s.kind == INT) == is_float:
-                wrong_type.append((s.name, str(t.dtype).replace("torch.", ""), "integer" if s.kind == INT else "floating point"))
+            if t is None:
                 continue
             out[s.name] = place(s, t, compute_dtype, device)
             del t

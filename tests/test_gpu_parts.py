@@ -1011,3 +1011,100 @@ def test_toy_architecture_with_a_norm_of_its_own(tmp_path, dtype, rel):
                 helpers.assert_close(got[rid], want[rid], rel, f"norm toy {dtype} {name} {rid}")
     finally:
         unregister("toy-norm")
+
+
+# --- a sixth toy: its weight files hold query, key and value projections apart ---
+def _define_split_toy():
+    from pytorch_transformers_amd.config.base import ModelConfig
+    from pytorch_transformers_amd.engine.spec import CACHE_FULL, CacheGroupSpec, LayerCall, ModelSpec
+    from pytorch_transformers_amd.parts import (AttentionMixer, DenseFeedForward, Embedding, LayerNorm, OutputHead,
+                                                RotaryPositions, SequentialBlock)
+
+    @dataclasses.dataclass
+    class SplitConfig(ModelConfig):
+        model_type = "toy-split"
+        vocab_size: int = 131
+        width: int = 96
+        heads: int = 6
+        kv_heads: tuple = (2, 6, 1)  # per layer: grouped, one per head, one for all
+        eps: float = 1e-5
+
+    LAYOUTS = {2: "grouped", 6: "interleaved", 1: "tail"}
+
+    def build(cfg):
+        W, nh = cfg.width, cfg.heads
+        d = W // nh
+        pos = RotaryPositions(d, 10000.0)
+        norm = lambda n: LayerNorm(n, W, cfg.eps)
+        blocks = [SequentialBlock(AttentionMixer(f"s.h.{i}.attn", W, nh, nkv, d, LAYOUTS[nkv], True, pos, out_name="o_proj",
+                                                 qkv_pieces=("q_proj", "k_proj", "v_proj")),
+                                  DenseFeedForward(f"s.h.{i}.mlp", W, 2 * W, bias=False), norm(f"s.h.{i}.n1"), norm(f"s.h.{i}.n2"))
+                  for i, nkv in enumerate(cfg.kv_heads)]
+        return ModelSpec(config=cfg, embedding=Embedding("s.embed", cfg.vocab_size, W), blocks=blocks,
+                         order=[LayerCall(i, f"g{i}", 0) for i in range(len(blocks))], final_norm=norm("s.final"),
+                         head=OutputHead("s.head", cfg.vocab_size, W, "s.embed.weight"),
+                         cache_groups=[CacheGroupSpec(f"g{i}", CACHE_FULL, 1, nkv, d) for i, nkv in enumerate(cfg.kv_heads)])
+
+    return SplitConfig, build
+
+
+def _plain_split_toy(cfg, w, ids):
+    """Separate projections, heads in order; query head h reads KV head h // (heads / kv heads)."""
+    T, W, nh = len(ids), cfg.width, cfg.heads
+    d = W // nh
+    x = w["s.embed.weight"][torch.as_tensor(ids)]
+    ln = lambda h, n: P.layer_norm(h, w[n + ".weight"], w[n + ".bias"], cfg.eps)
+    cos, sin = P.rope_cos_sin(torch.arange(T), P.rope_inv_freq(d, 10000.0))
+    for i, nkv in enumerate(cfg.kv_heads):
+        a = ln(x, f"s.h.{i}.n1")
+        proj = lambda n, heads: (a @ w[f"s.h.{i}.attn.{n}.weight"].T + w[f"s.h.{i}.attn.{n}.bias"]).view(T, heads, d)
+        q, k, v = proj("q_proj", nh), proj("k_proj", nkv), proj("v_proj", nkv)
+        k, v = (t.repeat_interleave(nh // nkv, dim=1) for t in (k, v))
+        o = P.attention_scores_softmax(P.apply_rope(q, cos, sin), P.apply_rope(k, cos, sin), v)
+        x = x + o @ w[f"s.h.{i}.attn.o_proj.weight"].T + w[f"s.h.{i}.attn.o_proj.bias"]
+        m = ln(x, f"s.h.{i}.n2")
+        x = x + P.gelu(m @ w[f"s.h.{i}.mlp.dense_h_to_4h.weight"].T) @ w[f"s.h.{i}.mlp.dense_4h_to_h.weight"].T
+    return ln(x, "s.final") @ w["s.embed.weight"].T
+
+
+@pytest.mark.parametrize("dtype,rel", [("float32", 5e-5), ("bfloat16", helpers.REL_BF16)])
+def test_toy_architecture_whose_files_hold_query_key_and_value_apart(tmp_path, dtype, rel):
+    """The attention part runs one fused projection; this toy's weight files hold ``q_proj``, ``k_proj`` and
+    ``v_proj`` apart, with grouped heads, one KV head per head, and one for all, and the loader lays their rows out
+    as each layer's fused launch wants them.  The file is written by this test from matrices of its own; the plain
+    implementation multiplies by the separate matrices."""
+    from safetensors.torch import load_file, save_file
+
+    from pytorch_transformers_amd import AutoModelForCausalLM
+    from pytorch_transformers_amd.config import register, unregister
+    from pytorch_transformers_amd.engine.replay import Replayer
+    from pytorch_transformers_amd.weights import write_random_model
+
+    SplitConfig, build = _define_split_toy()
+    register("toy-split", SplitConfig, build, exist_ok=True)
+    try:
+        cfg = SplitConfig()
+        folder = write_random_model(str(tmp_path / "split"), cfg, seed=21, std=0.15, noise=0.1)
+        path = f"{folder}/model.safetensors"
+        tensors = load_file(path)
+        d = cfg.width // cfg.heads
+        g = torch.Generator().manual_seed(3)
+        for i, nkv in enumerate(cfg.kv_heads):  # the fused tensors go, separate ones of this test's making come
+            for kind in ("weight", "bias"):
+                fused = tensors.pop(f"s.h.{i}.attn.query_key_value.{kind}")
+                for n, heads in (("q_proj", cfg.heads), ("k_proj", nkv), ("v_proj", nkv)):
+                    shape = (heads * d, cfg.width) if kind == "weight" else (heads * d,)
+                    tensors[f"s.h.{i}.attn.{n}.{kind}"] = (torch.randn(shape, generator=g) * 0.15).to(fused.dtype)
+        save_file(tensors, path, metadata={"format": "pt"})
+        w = {k: v.double() for k, v in tensors.items()}
+        model = AutoModelForCausalLM.from_pretrained(folder, dtype=dtype)
+        reqs = helpers.make_requests(cfg.vocab_size, [9, 37, 66], seed=8)
+        want = {rid: _plain_split_toy(cfg, w, toks).float() for rid, toks in reqs.items()}
+        rp = Replayer(model, 1024, max_slots=3)
+        for name, records in (("whole", helpers.schedule_whole(reqs)), ("tail", helpers.schedule_tail(reqs, 16)),
+                              ("batches", helpers.schedule_batches(reqs, 2))):
+            got = helpers.run_schedule(rp, records)
+            for rid in reqs:
+                helpers.assert_close(got[rid], want[rid], rel, f"split toy {dtype} {name} {rid}")
+    finally:
+        unregister("toy-split")

@@ -170,3 +170,57 @@ def test_a_tied_head_in_the_file_is_not_read(tmp_path):
     specs_u = lookup("falcon")[1](cfg_u).tensor_specs()
     w = load_weights(f, specs_u, torch.float32, "cpu", base_prefix="transformer.")
     assert float(w["lm_head.weight"][0, 0]) == 7.0
+
+
+def test_a_tensor_may_lie_in_the_file_in_pieces(tmp_path):
+    """A model that runs query, key and value as one matrix reads a file that holds them apart: the pieces are
+    checked one by one (missing, wrong shape), laid out as the model says, and are not 'unexpected'; a file that
+    holds the matrix whole loads as before, and then stray pieces are unexpected."""
+    from safetensors.torch import save_file
+
+    from pytorch_transformers_amd.engine.spec import MATRIX, VECTOR, TensorSpec
+    from pytorch_transformers_amd.parts.attention import fused_rows
+
+    nh, nkv, d, W = 4, 2, 2, 6
+    lay = fused_rows(nh, nkv, d, "grouped")
+    names = ("a.q", "a.k", "a.v")
+    rows = (nh * d, nkv * d, nkv * d)
+    specs = [TensorSpec("a.qkv.weight", ((nh + 2 * nkv) * d, W), MATRIX,
+                        pieces=tuple((n + ".weight", (r, W)) for n, r in zip(names, rows)), assemble=lay),
+             TensorSpec("a.qkv.bias", ((nh + 2 * nkv) * d,), VECTOR,
+                        pieces=tuple((n + ".bias", (r,)) for n, r in zip(names, rows)), assemble=lay),
+             TensorSpec("a.out.weight", (W, nh * d), MATRIX)]
+    g = torch.Generator().manual_seed(0)
+    parts = {f"{n}.{kind}": torch.randn((r, W) if kind == "weight" else (r,), generator=g)
+             for n, r in zip(names, rows) for kind in ("weight", "bias")}
+    out_w = torch.randn(W, nh * d, generator=g)
+
+    def folder(name, tensors):
+        f = tmp_path / name
+        f.mkdir()
+        save_file({k: v.contiguous() for k, v in tensors.items()}, str(f / "model.safetensors"), metadata={"format": "pt"})
+        return str(f)
+
+    apart = folder("apart", {**parts, "a.out.weight": out_w})
+    w = load_weights(apart, specs, torch.float32, "cpu")
+    q, k, v = (parts[n + ".weight"] for n in names)
+    gq = nh // nkv
+    want = torch.cat([torch.cat([q[j * gq * d:(j + 1) * gq * d], k[j * d:(j + 1) * d], v[j * d:(j + 1) * d]]) for j in range(nkv)])
+    assert torch.equal(w["a.qkv.weight"], want)
+    assert torch.equal(w["a.qkv.bias"], lay([parts[n + ".bias"] for n in names])) and w["a.qkv.bias"].shape == (16,)
+    whole = folder("whole", {"a.qkv.weight": want, "a.qkv.bias": w["a.qkv.bias"], "a.out.weight": out_w})
+    assert torch.equal(load_weights(whole, specs, torch.float32, "cpu")["a.qkv.weight"], want)
+    # a piece is missing, another has the wrong shape: both are named, each under its own name
+    broken = dict(parts)
+    del broken["a.k.weight"]
+    broken["a.v.bias"] = torch.zeros(3)
+    with pytest.raises(WeightsError) as e:
+        load_weights(folder("broken", {**broken, "a.out.weight": out_w}), specs, torch.float32, "cpu")
+    assert e.value.missing == ["a.k.weight"] and [n for n, _, _ in e.value.wrong_shape] == ["a.v.bias"]
+    with pytest.raises(WeightsError) as e:  # nothing of it is there: the whole and the pieces are named
+        load_weights(folder("none", {"a.out.weight": out_w, "a.qkv.bias": w["a.qkv.bias"]}), specs, torch.float32, "cpu")
+    assert e.value.missing == ["a.qkv.weight (or its pieces a.q.weight, a.k.weight, a.v.weight)"]
+    with pytest.raises(WeightsError) as e:  # whole and in pieces: the pieces are not read
+        load_weights(folder("both", {**parts, "a.qkv.weight": want, "a.qkv.bias": w["a.qkv.bias"], "a.out.weight": out_w}),
+                     specs, torch.float32, "cpu")
+    assert sorted(e.value.unexpected) == sorted(parts)
