@@ -161,6 +161,34 @@ def test_layernorm_sum(H, case):
     assert x_none is None and torch.equal(o1b, o1)
 
 
+@pytest.mark.parametrize("H", [200, 4544, 5120, 5128, 8192])
+@pytest.mark.parametrize("Pb,Pa", [(8, 4), (9, 0), (12, 4), (13, 2), (16, 4), (16, 0), (17, 4), (3, 5)])
+def test_layernorm_sum_of_many_ranges(H, Pb, Pa):
+    """A decode step's sum with as many ranges of partial sums as the pair launches leave: up to 16 of the first
+    product and 4 of the second with every load in flight at once (rows of up to 5,120 features from 9 ranges on),
+    beyond that one after the other; the ranges are added in their order whichever kernel runs, so the sum is the
+    same bits as the additions one by one."""
+    ops = _ops()
+    M = 6
+    bf = lambda t: t.bfloat16()
+    pb, pa = _rand(Pb, M, H, seed=1), (_rand(Pa, M, H, seed=2) if Pa else None)
+    bb, ba = _rand(H, seed=3), _rand(H, seed=4)
+    x1 = bf(_rand(M, H, seed=5))
+    w, b = _rand(H, seed=6) + 1.0, _rand(H, seed=7)
+
+    def value(p, bias):
+        acc = p[0].clone()
+        for u in range(1, p.shape[0]):
+            acc = acc + p[u]
+        return bf(bf(acc).float() + bias).float()
+
+    terms = [(pb, bb)] + ([(pa, ba)] if Pa else []) + [x1]
+    want = bf(value(pb, bb) + (value(pa, ba) if Pa else 0.0) + x1.float())
+    x, o1, _ = ops.layernorm_sum(terms, H, w=w, b=b, eps=1e-5)
+    assert torch.equal(x, want), "the ranges are added in their order and the sum is rounded once"
+    torch.testing.assert_close(o1.float(), F.layer_norm(want.float(), (H,), w, b, 1e-5), rtol=1e-2, atol=1e-2)
+
+
 @pytest.mark.parametrize("H", [64, 200, 4544, 5000, 8192])
 @pytest.mark.parametrize("M", [512, 515, 1031])
 def test_layernorm_sum_of_many_rows(H, M):
