@@ -146,8 +146,8 @@ __global__ __launch_bounds__(NS_THREADS / CH) void layernorm_sum_kernel(
 // else is one trip.  The additions are the same, in the same order: the same bits.  Measured in whole decode steps
 // at 32 layers of 4,544 features, 8 rows: 3.416 -> 3.384 ms a step (a microsecond a layer; most of this kernel's nine
 // are what any kernel boundary costs).
-// TH: the most threads of a launch (what the registers of a thread are bounded by: 12 and 16 ranges in flight need
-// more than the 128 that 1,024 threads leave each).
+// TH: the most threads of a launch (what the registers of a thread are bounded by: 12 ranges in flight need more
+// than the 128 that 1,024 threads leave each).
 template <int NB, int NA, int TH = NS_THREADS>
 __global__ __launch_bounds__(TH) void layernorm_sum_ahead_kernel(
     bf16_t* __restrict__ out_x, bf16_t* __restrict__ out1, bf16_t* __restrict__ out2, const float* __restrict__ pa,
@@ -358,14 +358,14 @@ extern "C" int pta_layernorm_sum(void* out_x, void* out1, void* out2, const floa
         else launch_rows<16>(out_x, out1, out2, add1, add2, add3, w1, b1, w2, b2, M, H, eps, s);
         return pta_check_launch("layernorm_sum");
     }
-    // A decode step's usual sum (a first product of up to 16 ranges, a second of up to 4, tensors): every load at once.
+    // A decode step's usual sum (a first product of up to 12 ranges, a second of up to 4, tensors): every load at once
+    // (16 ranges at once, 168 registers and some spilled, took 11.3 us where one range after the other takes 9.1).
     static const bool ahead = !getenv("PTA_NORM_AHEAD") || atoi(getenv("PTA_NORM_AHEAD")) != 0;
     const int threads = (H / 8 + 63) / 64 * 64;
     constexpr int WIDE_THREADS = 640;  // rows of up to 5,120 features
-    if (ahead && pb && (Pb <= 8 || (Pb <= 16 && threads <= WIDE_THREADS)) && (!pa || Pa <= 4) && H <= NS_MAX_H) {
+    if (ahead && pb && (Pb <= 8 || (Pb <= 12 && threads <= WIDE_THREADS)) && (!pa || Pa <= 4) && H <= NS_MAX_H) {
         auto kern = pa ? layernorm_sum_ahead_kernel<8, 4> : layernorm_sum_ahead_kernel<8, 1>;
-        if (Pb > 12) kern = pa ? layernorm_sum_ahead_kernel<16, 4, WIDE_THREADS> : layernorm_sum_ahead_kernel<16, 1, WIDE_THREADS>;
-        else if (Pb > 8) kern = pa ? layernorm_sum_ahead_kernel<12, 4, WIDE_THREADS> : layernorm_sum_ahead_kernel<12, 1, WIDE_THREADS>;
+        if (Pb > 8) kern = pa ? layernorm_sum_ahead_kernel<12, 4, WIDE_THREADS> : layernorm_sum_ahead_kernel<12, 1, WIDE_THREADS>;
         hipLaunchKernelGGL(kern, dim3(M), dim3(threads), 0, (hipStream_t)stream,
                            (bf16_t*)out_x, (bf16_t*)out1, (bf16_t*)out2, pa, Pa, bias_a, pb, Pb, bias_b, (const bf16_t*)add1,
                            (const bf16_t*)add2, (const bf16_t*)add3, rows, w1, b1, w2, b2, M_in, H, eps);

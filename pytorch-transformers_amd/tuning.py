@@ -655,7 +655,10 @@ def tune_pair_parts(w1: torch.Tensor, w2: torch.Tensor) -> None:
             t_st = (timed_ways([(cls,) + c for c in st_cands], rows, fix=lambda a: fix_st(a[0], a[1:]), read=read)
                     if st_cands else [])
             t_st = [t + slices_ms(c) for t, c in zip(t_st, st_cands)]
-            best = min(range(len(st_cands)), key=lambda i: t_st[i]) if st_cands else -1
+            # the fewest ranges among those within 1.5 % of the fastest: what separates them is less than a box
+            # varies, and fewer ranges leave whatever reads them next less to read
+            best = (min((i for i in range(len(st_cands)) if t_st[i] <= 1.015 * min(t_st)), key=lambda i: st_cands[i])
+                    if st_cands else -1)
             keep = st_cands[best] if best >= 0 and t_st[best] < 0.98 * t_staged else (0, 0)
             chosen_st.append(keep)
             if os.environ.get("PTA_TUNE_VERBOSE"):
