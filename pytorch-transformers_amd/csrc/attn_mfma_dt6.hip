@@ -1,0 +1,4 @@
+// The attention on the matrix cores for heads of 96 elements (see attn_mfma_impl.h).
+#include "attn_mfma_impl.h"
+
+template int attn_launch_head<6>(const AttnLaunch&, bool, bool, bool, int);
