@@ -68,8 +68,15 @@ def generate(model, prompts: Sequence[Sequence[int]], generation_config: Optiona
              rng_ids: Optional[Sequence[int]] = None, tokenizer=None, keep_slots: bool = False,
              slots: Optional[Sequence[int]] = None, rng_step_start: Optional[Sequence[int]] = None,
              logits_processor: Optional[Sequence] = None, stopping_criteria: Optional[Sequence] = None,
-             **kwargs) -> Union[List[List[int]], GenerateOutput]:
+             attention_mask=None, **kwargs) -> Union[List[List[int]], GenerateOutput]:
     """Generate for every prompt (a list of token ids); returns prompt + new tokens per prompt.
+
+    ``prompts`` may also be the reference's rectangular ``input_ids``, an integer tensor ``[rows, longest]`` with
+    ``attention_mask`` (same shape; 0 where a row is padded, on the left as the reference asks of decoder-only
+    models, src/transformers/generation/utils.py:2036-2048): a row's prompt is then its ids where the mask is 1, and the
+    result is the reference's tensor, prompts padded on the left and finished rows on the right with
+    ``pad_token_id`` (the first ``eos_token_id`` if there is none, :1863-1871; ``sequences`` of a ``GenerateOutput``
+    likewise).
 
     ``generation_config`` defaults to the model's; keyword arguments override its fields
     (:1543-1545).  ``streamer``: an object with ``put`` and ``end`` as the reference's streamers have them
@@ -98,6 +105,13 @@ def generate(model, prompts: Sequence[Sequence[int]], generation_config: Optiona
     cfg = generation_config or getattr(model, "generation_config", None) or GenerationConfig()
     if kwargs:
         cfg = cfg.updated(**kwargs)
+    if hasattr(prompts, "dim"):  # a tensor: the reference's input_ids
+        return _generate_from_tensor(model, prompts, attention_mask, cfg, dict(
+            batch_size=batch_size, sampler=sampler, streamer=streamer, cache=cache, rng_ids=rng_ids, tokenizer=tokenizer,
+            keep_slots=keep_slots, slots=slots, rng_step_start=rng_step_start, logits_processor=logits_processor,
+            stopping_criteria=stopping_criteria))
+    if attention_mask is not None:
+        raise ValueError("an attention_mask goes with input_ids as a tensor; prompts given as lists have no padding")
     prompts = [list(map(int, p)) for p in prompts]
     if not prompts:
         return GenerateOutput([]) if cfg.return_dict_in_generate else []
@@ -246,6 +260,34 @@ def generate(model, prompts: Sequence[Sequence[int]], generation_config: Optiona
     if cfg.return_dict_in_generate:
         return GenerateOutput(sequences, out_scores, out_logits)
     return sequences
+
+
+def _generate_from_tensor(model, input_ids, attention_mask, cfg: GenerationConfig, how: dict):
+    """``generate`` for the reference's rectangular input: rows without their padding in, the reference's tensor out."""
+    import torch
+
+    if input_ids.dim() != 2 or input_ids.dtype not in (torch.int64, torch.int32):
+        raise ValueError(f"input_ids must be an integer tensor [rows, length], got {tuple(input_ids.shape)} {input_ids.dtype}")
+    ids = input_ids.detach().cpu()
+    if attention_mask is None:
+        rows = ids.tolist()
+    else:
+        mask = torch.as_tensor(attention_mask).detach().cpu()
+        if mask.shape != ids.shape:
+            raise ValueError(f"attention_mask {tuple(mask.shape)} must have the shape of input_ids {tuple(ids.shape)}")
+        rows = [r[m.bool()].tolist() for r, m in zip(ids, mask)]
+    out = generate(model, rows, cfg, **how)
+    pad = cfg.pad_token_id
+    if pad is None:
+        pad = cfg.eos_token_ids[0] if cfg.eos_token_ids else 0
+    n_ret = cfg.num_return_sequences
+    lens = [len(r) for r in rows for _ in range(n_ret)]
+    seqs = out.sequences if isinstance(out, GenerateOutput) else out
+    padded = pad_sequences(seqs, lens, pad).to(input_ids.device)
+    if isinstance(out, GenerateOutput):
+        out.sequences = padded
+        return out
+    return padded
 
 
 def _ids_tensor(ids: Sequence[int]):

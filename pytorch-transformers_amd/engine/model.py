@@ -542,7 +542,15 @@ class CausalLM:
         return logits
 
     # generation (see engine.generate) -----------------------------------------------
-    def generate(self, prompts, generation_config=None, **kwargs):
+    def generate(self, prompts=None, generation_config=None, *, input_ids=None, **kwargs):
+        """``engine.generate.generate`` for this model; ``input_ids=`` (with ``attention_mask=``) is the reference's
+        spelling of tensor prompts, so ``model.generate(**tokenizer(texts, return_tensors="pt", padding=True))`` works."""
         from .generate import generate
 
+        if prompts is None:
+            prompts = input_ids
+        elif input_ids is not None:
+            raise ValueError("prompts were given twice: positionally and as input_ids")
+        if prompts is None:
+            raise ValueError("generate needs prompts: lists of token ids, or input_ids as a tensor")
         return generate(self, prompts, generation_config, **kwargs)

@@ -503,3 +503,36 @@ def test_processor_and_criteria_lists_are_callable():
     assert procs(ids, scores).tolist() == [[3.0] * 5, [7.0] * 5]
     crit = StoppingCriteriaList([lambda i, s: i[:, -1] == 2, lambda i, s: False])
     assert crit(ids, scores).tolist() == [True, False]
+
+
+def test_rectangular_input_ids_with_a_mask_come_back_as_the_references_tensor():
+    """``input_ids`` padded on the left with an ``attention_mask``: each row generates from its own ids, and the result
+    is one tensor, prompts padded on the left, rows that ended early padded on the right with the pad token (the EOS
+    token if no pad token is set)."""
+    pad = 49
+    prompts = [[1, 2, 3], [4], [5, 6]]
+    ids = torch.tensor([[1, 2, 3], [pad, pad, 4], [pad, 5, 6]])
+    mask = torch.tensor([[1, 1, 1], [0, 0, 1], [0, 1, 1]])
+    want = [expected(p, 5, eos=(12,)) for p in prompts]
+    assert len({len(w) for w in want}) > 1, "the case must end a row early"
+    m = ScriptedModel()
+    out = generate(m, ids, GenerationConfig(max_new_tokens=5, eos_token_id=12, pad_token_id=pad), sampler=ArgmaxSampler(),
+                   attention_mask=mask)
+    assert isinstance(out, torch.Tensor) and out.dtype == torch.long
+    assert m.steps[0][1] == prompts  # no padding reaches the model
+    width = 3 + max(len(w) - len(p) for w, p in zip(want, prompts))
+    assert out.shape == (3, width)
+    for row, p, w in zip(out.tolist(), prompts, want):
+        assert row == [pad] * (3 - len(p)) + w + [pad] * (width - 3 - (len(w) - len(p)))
+    # no pad token set: the EOS token pads; return_dict keeps the tensor under `sequences`
+    res = generate(ScriptedModel(), ids, GenerationConfig(max_new_tokens=5, eos_token_id=12, return_dict_in_generate=True),
+                   sampler=ArgmaxSampler(), attention_mask=mask)
+    assert isinstance(res, GenerateOutput) and res.sequences.shape == (3, width)
+    assert res.sequences[1].tolist()[:3] == [12, 12, 4]
+    # without a mask every id of a row counts
+    out = generate(ScriptedModel(), torch.tensor([[1, 2, 3], [7, 8, 9]]), GenerationConfig(max_new_tokens=2), sampler=ArgmaxSampler())
+    assert out.tolist() == [expected([1, 2, 3], 2), expected([7, 8, 9], 2)]
+    with pytest.raises(ValueError, match="shape of input_ids"):
+        generate(ScriptedModel(), ids, GenerationConfig(max_new_tokens=1), sampler=ArgmaxSampler(), attention_mask=mask[:, :2])
+    with pytest.raises(ValueError, match="lists have no padding"):
+        generate(ScriptedModel(), prompts, GenerationConfig(max_new_tokens=1), sampler=ArgmaxSampler(), attention_mask=mask)

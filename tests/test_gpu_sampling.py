@@ -869,3 +869,24 @@ def test_the_callers_processors_and_criteria_through_generate_equal_plain(folder
         assert o == p + want
         lens.add(len(want))
     assert len(lens) > 1 and min(lens) < 30, f"rows must end at different steps, some by the criterion: {lens}"
+
+
+def test_tensor_prompts_in_the_references_spelling(folders):
+    """``model.generate(input_ids=..., attention_mask=...)`` with rows padded on the left gives, row by row, what the
+    same prompts give as lists, as one tensor padded as the reference pads it."""
+    from pytorch_transformers_amd import AutoModelForCausalLM, GenerationConfig
+
+    model = AutoModelForCausalLM.from_pretrained(folders["A"], dtype="float32")
+    g = torch.Generator().manual_seed(2)
+    prompts = [torch.randint(1, model.vocab_size, (n,), generator=g).tolist() for n in (9, 2, 5)]
+    ids = torch.zeros((3, 9), dtype=torch.long)
+    mask = torch.zeros((3, 9), dtype=torch.long)
+    for r, p in enumerate(prompts):
+        ids[r, 9 - len(p):] = torch.tensor(p)
+        mask[r, 9 - len(p):] = 1
+    gen = GenerationConfig(max_new_tokens=7, do_sample=False, eos_token_id=None, pad_token_id=0)
+    lists = model.generate(prompts, gen)
+    out = model.generate(input_ids=ids.cuda(), attention_mask=mask.cuda(), generation_config=gen)
+    assert out.is_cuda and out.shape == (3, 16)
+    for r, (p, want) in enumerate(zip(prompts, lists)):
+        assert out[r].tolist() == [0] * (9 - len(p)) + want
