@@ -60,6 +60,14 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--fp16", action="store_true", help="accepted for compatibility; the 16-bit type here is bfloat16")
     ap.add_argument("--device", default="cuda:0")
+    # options of the reference's example that have no counterpart here: accepted where they change nothing, refused where
+    # they would (examples/pytorch/text-generation/run_generation.py:316-332)
+    ap.add_argument("--padding_text", type=str, default="", help="Deprecated, the use of `--prefix` is preferred.")
+    ap.add_argument("--xlm_language", type=str, default="",
+                    help="the reference's language choice for XLM; must stay empty: Falcon has none")
+    ap.add_argument("--use_cpu", action="store_true", help="refused: the model runs on the GPU only")
+    ap.add_argument("--jit", action="store_true",
+                    help="accepted for compatibility: nothing is traced; decode steps are captured as HIP graphs anyway")
     ap.add_argument("--random_config", type=str, default=None, help="config.json to build a random-weights model from")
     ap.add_argument("--random_seed", type=int, default=0)
     ap.add_argument("--tune", action="store_true",
@@ -71,6 +79,15 @@ def build_parser() -> argparse.ArgumentParser:
 
 def main(argv=None) -> int:
     args = build_parser().parse_args(argv)
+    if args.use_cpu:
+        print("--use_cpu: there is no CPU path; the model runs on an AMD GPU (see --device)", file=sys.stderr)
+        return 2
+    if args.xlm_language:
+        print("--xlm_language belongs to another architecture of the reference's example and would change nothing here; "
+              "leave it out", file=sys.stderr)
+        return 2
+    if not args.prefix:  # the older name of the same option (run_generation.py:382)
+        args.prefix = args.padding_text
     from . import AutoConfig, GenerationConfig
     from .pipeline import pipeline
     from .weights import write_random_model

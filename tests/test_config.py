@@ -223,3 +223,14 @@ def test_bias_forced_token_and_decay_options():
     assert not BiasRules([[[1], 0.5]]).needs_history and BiasRules([[[1], 0.5]]).biases(None) == [(1, 0.5)] and not BiasRules()
     with pytest.raises(ValueError, match="vocabulary size is 5"):
         BiasRules([[[1, 7], 1.0]], vocab_size=5)
+
+
+def test_command_line_refuses_what_it_cannot_do_before_anything_is_loaded(capsys):
+    """``--use_cpu`` and ``--xlm_language`` of the reference's example (run_generation.py:319-330) are known and refused
+    with a reason, without a model or a GPU."""
+    from pytorch_transformers_amd.run_generation import main
+
+    assert main(["--use_cpu", "--prompt_ids", "1"]) == 2
+    assert "no CPU path" in capsys.readouterr().err
+    assert main(["--xlm_language", "en", "--prompt_ids", "1"]) == 2
+    assert "another architecture" in capsys.readouterr().err

@@ -750,6 +750,8 @@ def test_text_through_the_command_line_and_the_pipeline(tmp_path):
         return lines[1:]
 
     assert program("--prompt", prompt, "--prefix", prefix, "--length", "10", "--greedy") == [whole]
+    # the older name of --prefix, and the reference's --jit, which changes nothing here (run_generation.py:318, :382, :332)
+    assert program("--prompt", prompt, "--padding_text", prefix, "--length", "10", "--greedy", "--jit") == [whole]
     stop = WORDS[new[3]]  # a word that is generated: the printed text is cut in front of its first occurrence
     assert whole.find(stop) > 0
     assert program("--prompt", prompt, "--prefix", prefix, "--length", "10", "--greedy", "--stop_token", stop) == \
