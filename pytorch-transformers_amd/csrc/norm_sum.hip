@@ -162,10 +162,13 @@ __global__ __launch_bounds__(TH) void layernorm_sum_ahead_kernel(
     const int i = threadIdx.x * 8;
     const bool live = i < H;
     const long at = src * H + (live ? i : 0);
-    float tb[NB][8], ta[NA][8], v[8];
+    // of the first product's ranges at most FLY are on their way at once: a range past them is asked for into the
+    // registers of the range that was just added (16 at once need more registers than a wave has)
+    constexpr int FLY = NB < 12 ? NB : 12;
+    float tb[FLY][8], ta[NA][8], v[8];
     uint4 r1 = make_uint4(0u, 0u, 0u, 0u), r2 = r1, r3 = r1;
 #pragma unroll
-    for (int u = 0; u < NB; ++u) load8f(pb + (long)min(u, Pb - 1) * part_stride + at, tb[u]);
+    for (int u = 0; u < FLY; ++u) load8f(pb + (long)min(u, Pb - 1) * part_stride + at, tb[u]);
     if (pa) {
 #pragma unroll
         for (int u = 0; u < NA; ++u) load8f(pa + (long)min(u, Pa - 1) * part_stride + at, ta[u]);
@@ -176,9 +179,11 @@ __global__ __launch_bounds__(TH) void layernorm_sum_ahead_kernel(
     // the first product: its ranges in order, rounded, then its bias added and rounded
 #pragma unroll
     for (int u = 0; u < NB; ++u) {
-        if (u >= Pb) continue;
+        if (u < Pb) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = u == 0 ? tb[u][e] : v[e] + tb[u][e];
+            for (int e = 0; e < 8; ++e) v[e] = u == 0 ? tb[u % FLY][e] : v[e] + tb[u % FLY][e];
+        }
+        if (u + FLY < NB) load8f(pb + (long)min(u + FLY, Pb - 1) * part_stride + at, tb[u % FLY]);
     }
 #pragma unroll
     for (int e = 0; e < 8; ++e) v[e] = round_to_bf16(v[e]);
@@ -358,14 +363,16 @@ extern "C" int pta_layernorm_sum(void* out_x, void* out1, void* out2, const floa
         else launch_rows<16>(out_x, out1, out2, add1, add2, add3, w1, b1, w2, b2, M, H, eps, s);
         return pta_check_launch("layernorm_sum");
     }
-    // A decode step's usual sum (a first product of up to 12 ranges, a second of up to 4, tensors): every load at once
-    // (16 ranges at once, 168 registers and some spilled, took 11.3 us where one range after the other takes 9.1).
+    // A decode step's usual sum (a first product of up to 16 ranges, a second of up to 4, tensors): every load at once,
+    // or of 13 to 16 ranges twelve at once and the rest behind them (16 at once, 168 registers and some spilled, took
+    // 11.3 us where one range after the other takes 9.1).
     static const bool ahead = !getenv("PTA_NORM_AHEAD") || atoi(getenv("PTA_NORM_AHEAD")) != 0;
     const int threads = (H / 8 + 63) / 64 * 64;
     constexpr int WIDE_THREADS = 640;  // rows of up to 5,120 features
-    if (ahead && pb && (Pb <= 8 || (Pb <= 12 && threads <= WIDE_THREADS)) && (!pa || Pa <= 4) && H <= NS_MAX_H) {
+    if (ahead && pb && (Pb <= 8 || (Pb <= 16 && threads <= WIDE_THREADS)) && (!pa || Pa <= 4) && H <= NS_MAX_H) {
         auto kern = pa ? layernorm_sum_ahead_kernel<8, 4> : layernorm_sum_ahead_kernel<8, 1>;
-        if (Pb > 8) kern = pa ? layernorm_sum_ahead_kernel<12, 4, WIDE_THREADS> : layernorm_sum_ahead_kernel<12, 1, WIDE_THREADS>;
+        if (Pb > 12) kern = pa ? layernorm_sum_ahead_kernel<16, 4, WIDE_THREADS> : layernorm_sum_ahead_kernel<16, 1, WIDE_THREADS>;
+        else if (Pb > 8) kern = pa ? layernorm_sum_ahead_kernel<12, 4, WIDE_THREADS> : layernorm_sum_ahead_kernel<12, 1, WIDE_THREADS>;
         hipLaunchKernelGGL(kern, dim3(M), dim3(threads), 0, (hipStream_t)stream,
                            (bf16_t*)out_x, (bf16_t*)out1, (bf16_t*)out2, pa, Pa, bias_a, pb, Pb, bias_b, (const bf16_t*)add1,
                            (const bf16_t*)add2, (const bf16_t*)add3, rows, w1, b1, w2, b2, M_in, H, eps);

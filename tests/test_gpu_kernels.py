@@ -165,8 +165,8 @@ def test_layernorm_sum(H, case):
 @pytest.mark.parametrize("Pb,Pa", [(8, 4), (9, 0), (12, 4), (13, 2), (16, 4), (16, 0), (17, 4), (3, 5)])
 def test_layernorm_sum_of_many_ranges(H, Pb, Pa):
     """A decode step's sum with as many ranges of partial sums as the pair launches leave: up to 16 of the first
-    product and 4 of the second; up to 12 and 4 with every load in flight at once (rows of up to 5,120 features from
-    9 ranges on), beyond that one after the other; the ranges are added in their order whichever kernel runs, so the sum is the
+    product and 4 of the second with the loads in flight at once (at most twelve ranges of the first, the rest behind
+    them; rows of up to 5,120 features from 9 ranges on), beyond that one after the other; the ranges are added in their order whichever kernel runs, so the sum is the
     same bits as the additions one by one."""
     ops = _ops()
     M = 6
