@@ -779,6 +779,13 @@ def test_text_through_the_command_line_and_the_pipeline(tmp_path):
     assert out[1] == [{"generated_text": text_of(ids_of("the dog") + other[:cut2])}]
     # token ids through the same pipeline stay ids
     assert pipe([ids], max_new_tokens=3, do_sample=False)[0] == [{"generated_token_ids": ids + new[:3]}]
+    # a streamer sees the same text while it is generated, prompt included or not
+    from pytorch_transformers_amd import TextIteratorStreamer
+
+    for skip in (False, True):
+        it = TextIteratorStreamer(pipe.tokenizer, skip_prompt=skip, timeout=60)
+        assert pipe(prefix + prompt, max_new_tokens=10, do_sample=False, streamer=it) == [{"generated_text": whole}]
+        assert "".join(it) == (text_of(new) if skip else whole)
     with pytest.raises(ValueError, match="tokenizer"):
         pipeline("text-generation", model=pipe.model)("the cat", max_new_tokens=2)
 
