@@ -390,6 +390,26 @@ def _ends_with_stop(tokenizer, new_tokens: Sequence[int], stop_strings: Sequence
     return any(s and s in text and s not in before for s in stop_strings)
 
 
+def compute_transition_scores(output: "GenerateOutput", prompt_lens: Sequence[int], normalize_logits: bool = False):
+    """The score of every generated token: per sequence, ``scores[step][token chosen at that step]`` from a result
+    of ``generate(..., output_scores=True, return_dict_in_generate=True)`` (src/transformers/generation/utils.py
+    :1160-1283 without beams); with ``normalize_logits`` the log-softmax of the step's scores first.  Sequences are
+    ragged here (one that ended early has fewer steps), so the result is a list of 32-bit tensors, one per sequence."""
+    import torch
+
+    if output.scores is None:
+        raise ValueError("transition scores need the steps' scores: generate(..., output_scores=True)")
+    out = []
+    for seq, n, steps in zip(output.sequences, prompt_lens, output.scores):
+        new = [int(t) for t in (seq.tolist() if hasattr(seq, "tolist") else seq)][int(n):int(n) + len(steps)]
+        vals = []
+        for tok, s in zip(new, steps):
+            s = s.float()
+            vals.append((torch.log_softmax(s, -1) if normalize_logits else s)[tok])
+        out.append(torch.stack(vals) if vals else torch.zeros(0))
+    return out
+
+
 def pad_sequences(sequences: Sequence[Sequence[int]], prompt_lens: Sequence[int], pad_token_id: int):
     """The reference's rectangular return value: prompts padded on the left to the longest prompt, new
     tokens padded on the right after a row ended (src/transformers/generation/utils.py:3282-3286)."""

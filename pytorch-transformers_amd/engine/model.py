@@ -462,6 +462,12 @@ class CausalLM:
             h = norm.forward(x, rows=logit_rows) if norm is not None else x.index_select(0, logit_rows.long())
         return self.spec.head.forward(h)
 
+    def compute_transition_scores(self, output, prompt_lens, normalize_logits: bool = False):
+        """``engine.generate.compute_transition_scores`` (the reference's method of the same name, without beams)."""
+        from .generate import compute_transition_scores
+
+        return compute_transition_scores(output, prompt_lens, normalize_logits)
+
     # decode steps as HIP graphs ---------------------------------------------------------
     def _graph_for(self, cache: PagedCache, plan: StepPlan) -> "_DecodeGraph":
         return self._graph_for_sizes(cache, plan.n_seqs, plan.max_len, plan.total_len)

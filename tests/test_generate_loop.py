@@ -536,3 +536,18 @@ def test_rectangular_input_ids_with_a_mask_come_back_as_the_references_tensor():
         generate(ScriptedModel(), ids, GenerationConfig(max_new_tokens=1), sampler=ArgmaxSampler(), attention_mask=mask[:, :2])
     with pytest.raises(ValueError, match="lists have no padding"):
         generate(ScriptedModel(), prompts, GenerationConfig(max_new_tokens=1), sampler=ArgmaxSampler(), attention_mask=mask)
+
+
+def test_transition_scores_are_the_chosen_tokens_scores():
+    from pytorch_transformers_amd.engine.generate import compute_transition_scores
+
+    prompts = [[1, 2, 3], [4]]
+    out = generate(ScriptedModel(), prompts, GenerationConfig(max_new_tokens=3, output_scores=True, return_dict_in_generate=True),
+                   sampler=ArgmaxSampler())
+    raw = compute_transition_scores(out, [len(p) for p in prompts])
+    assert [r.tolist() for r in raw] == [[5.0] * 3, [5.0] * 3]  # the scripted model scores its next token 5, the rest 0
+    norm = compute_transition_scores(out, [len(p) for p in prompts], normalize_logits=True)
+    want = float(torch.log_softmax(torch.tensor([5.0] + [0.0] * (V - 1)), -1)[0])
+    assert all(abs(v - want) < 1e-6 for r in norm for v in r.tolist())
+    with pytest.raises(ValueError, match="output_scores"):
+        compute_transition_scores(GenerateOutput([[1, 2]]), [1])
