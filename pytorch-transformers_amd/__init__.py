@@ -6,7 +6,7 @@ from .engine import falcon as _falcon  # registers model_type "falcon"  # noqa: 
 from .auto import AutoModelForCausalLM
 from .pipeline import TextGenerationPipeline, pipeline
 from .sampling.custom import LogitsProcessor, LogitsProcessorList, StoppingCriteria, StoppingCriteriaList
-from .streamers import BaseStreamer, TextIteratorStreamer, TextStreamer
+from .streaming import BaseStreamer, TextIteratorStreamer, TextStreamer
 
 __version__ = "0.1.0"
 __all__ = ["AutoConfig", "AutoModelForCausalLM", "BaseStreamer", "ConfigError", "FalconConfig", "GenerationConfig",
